@@ -1,0 +1,443 @@
+"""CPU restatement of the reference's quantized MoE expert path.
+
+TEST INFRASTRUCTURE ONLY -- this file is the checker, never the product.  Only
+``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import it.
+
+Every function cites the reference lines (paths relative to the reference
+checkout) whose behaviour it restates.  Index/integer work is numpy; floating
+point work uses torch on the CPU because numpy has no bfloat16 / float8.
+
+How each function is pinned (see tests/test_oracle_*.py):
+
+  top_k, deepseek_routing, expert_group_mask
+      hand-computed case of tests/unit/moe_test.py:293-326; brute force.
+  calculate_load_balance_updates
+      hand-computed case of tests/unit/moe_test.py:328-341.
+  permute / unpermute
+      permutation invariants, brute-force loops, k*x identity.
+  gmm
+      per-expert python loop, E=1 == plain matmul, int8 path exact on
+      integer inputs, the [3,5]-group case of quantizations_test.py:607-653.
+  moe_layer (sparse path)
+      independent dense all-experts formulation (moe.py:2986-3040) and the
+      per-expert loop block of tests/unit/moe_test.py:344-411.
+  get_static_scale
+      quantizations_test.py:723-726 (224 -> 0.5 for e4m3fn).
+  unpack_int4 / dequantize_int4 / dequantize_fp8_blocks
+      tests/unit/dequantize_pack_quantized_int4_test.py:61-127 cases.
+
+PARITY UNPINNED (third-party arithmetic whose source is not in the reference
+tree, and which no reference test pins):
+  * quantize_* rounding mode and zero-scale handling (qwix.pallas.quantize,
+    qwix >= 0.1.8).  Adopted: scale = absmax / qmax, q = clip(rint(x / scale)),
+    zero absmax -> q = 0 (as pallas_mosaic_tpu_v2_gmm_kernel.py:537-540).
+    GEMM parity is therefore asserted on identical already-quantized operands.
+  * tie order of jax.lax.top_k and stability of jnp.argsort (jax >= 0.10.2).
+    Adopted: larger value first, lower index first on ties; stable sort.
+  * bf16 rounding of the norm_topk_prob renormalisation (moe.py:756).
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+FP8_E4M3_MAX = 448.0
+INT8_MAX = 127.0
+INT4_MAX = 7.0
+
+
+# --------------------------------------------------------------------------
+# Routing  (src/maxtext/layers/moe.py:717-839)
+# --------------------------------------------------------------------------
+
+
+def top_k(x: np.ndarray, k: int):
+  """jax.lax.top_k semantics as adopted here: descending values, lower index
+  first among equal values (moe.py:747, :834).  Brute force via stable sort."""
+  x = np.asarray(x)
+  idx = np.argsort(-x.astype(np.float64), axis=-1, kind="stable")[..., :k].astype(np.int32)
+  vals = np.take_along_axis(x, idx, axis=-1)
+  return vals, idx
+
+
+def expert_group_mask(gate_logits: np.ndarray, n_routing_groups: int, topk_routing_group: int) -> np.ndarray:
+  """moe.py:775-811: keep experts of the top groups; group score = sum of the
+  group's top-2 expert scores (f32)."""
+  e = gate_logits.shape[-1]
+  grouped = gate_logits.reshape(gate_logits.shape[:-1] + (n_routing_groups, e // n_routing_groups))
+  top2, _ = top_k(grouped, 2)
+  group_scores = top2.astype(np.float32).sum(-1)
+  _, group_idx = top_k(group_scores, topk_routing_group)
+  group_mask = np.zeros(group_scores.shape, np.float32)
+  np.put_along_axis(group_mask, group_idx, 1.0, axis=-1)
+  mask = np.repeat(group_mask, e // n_routing_groups, axis=-1)
+  return mask
+
+
+def deepseek_routing(gate_logits, pre_bias_logits, k, n_routing_groups=-1, topk_routing_group=-1):
+  """moe.py:813-839: select on post-bias scores (optionally group-limited),
+  return the pre-bias scores of the selected experts as weights."""
+  gate_logits = np.asarray(gate_logits)
+  if n_routing_groups == -1:
+    masked = gate_logits
+  else:
+    mask = expert_group_mask(gate_logits, n_routing_groups, topk_routing_group)
+    masked = np.where(mask > 0, gate_logits, -np.inf)
+  _, idx = top_k(masked, k)
+  weights = np.take_along_axis(np.asarray(pre_bias_logits), idx, axis=-1)
+  return weights, idx
+
+
+def _softmax_f32(x: np.ndarray) -> np.ndarray:
+  x = x.astype(np.float32)
+  m = x.max(-1, keepdims=True)
+  e = np.exp(x - m, dtype=np.float32)
+  return (e / e.sum(-1, keepdims=True, dtype=np.float32)).astype(np.float32)
+
+
+def _round_bf16(x: np.ndarray) -> np.ndarray:
+  return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch.bfloat16).to(torch.float32).numpy()
+
+
+def get_topk(
+    gate_logits,
+    pre_bias_logits=None,
+    *,
+    k: int,
+    mode: str = "softmax_topk",
+    norm_topk_prob: bool = False,
+    routed_scaling_factor: float = 1.0,
+    routed_score_func: str = "sigmoid",
+    n_routing_groups: int = -1,
+    topk_routing_group: int = -1,
+    weight_dtype: str = "bf16",
+):
+  """moe.py:717-765.  Returns (weights f32 ndarray holding values already
+  rounded to `weight_dtype`, indices int32).
+
+  mode "softmax_topk": lax.top_k -> softmax over the k values in f32 -> cast to
+  the layer dtype (:747, :753) -> optional renormalisation in that dtype (:756).
+  mode "deepseek": deepseek_routing (:744) then deepseek_scale_weights (:767-773);
+  weights keep the gate dtype (f32).
+  """
+  gate_logits = np.asarray(gate_logits)
+  if mode == "deepseek":
+    w, idx = deepseek_routing(gate_logits, pre_bias_logits, k, n_routing_groups, topk_routing_group)
+    w = w.astype(np.float32)
+    if routed_score_func in ("sigmoid", "sqrtsoftplus"):
+      w = w / (w.sum(-1, keepdims=True, dtype=np.float32) + np.float32(1e-20))
+    w = (w * np.float32(routed_scaling_factor)).astype(np.float32)
+    return w, idx
+  if mode != "softmax_topk":
+    raise ValueError(f"unknown routing mode {mode}")
+  vals, idx = top_k(gate_logits, k)
+  w = _softmax_f32(vals)
+  if weight_dtype == "bf16":
+    w = _round_bf16(w)
+  if norm_topk_prob:
+    s = w.sum(-1, keepdims=True, dtype=np.float32)
+    if weight_dtype == "bf16":
+      s = _round_bf16(s)
+      w = _round_bf16(w / s)
+    else:
+      w = (w / s).astype(np.float32)
+  return w, idx
+
+
+def calculate_load_balance_updates(top_k_indices, num_experts: int, rate: float):
+  """moe.py:215-236."""
+  flat = np.asarray(top_k_indices).ravel()
+  counts = np.bincount(flat, minlength=num_experts)
+  average = flat.size / num_experts
+  return np.sign(average - counts) * rate
+
+
+# --------------------------------------------------------------------------
+# Permute / unpermute  (moe.py:950-960, :986-991, :1039-1063)
+# --------------------------------------------------------------------------
+
+
+def permute(inputs_2d: torch.Tensor, selected_experts: np.ndarray, num_experts: int):
+  """moe.py:950-960, :986-991 (non-ragged branch).
+
+  Returns (sorted_inputs [M,d], sorted_selected_experts [M] int32 -- the stable
+  argsort of the flattened expert ids, group_size [E] int32, sorted_experts [M]).
+  Row i of sorted_inputs is token perm[i] // k (repeat(x, k)[perm])."""
+  t, k = selected_experts.shape
+  flat = np.asarray(selected_experts).reshape(-1)
+  perm = np.argsort(flat, kind="stable").astype(np.int32)
+  sorted_inputs = inputs_2d[torch.from_numpy((perm // k).astype(np.int64))]
+  group_size = np.bincount(flat, minlength=num_experts).astype(np.int32)
+  sorted_experts = np.repeat(np.arange(num_experts, dtype=np.int32), group_size)
+  return sorted_inputs, perm, group_size, sorted_experts
+
+
+def unpermute(intermediate: torch.Tensor, perm: np.ndarray, weights: np.ndarray, k: int, out_dtype=torch.bfloat16):
+  """moe.py:1039-1063 with float32_weight_sum=True: gather by argsort(perm),
+  reshape [T,k,d], f32 einsum "BKE,BK->BE", cast to the layer dtype."""
+  inv = np.argsort(perm, kind="stable")
+  un = intermediate[torch.from_numpy(inv.astype(np.int64))].to(torch.float32)
+  w = torch.from_numpy(np.ascontiguousarray(weights, dtype=np.float32)).reshape(-1, k)
+  un = un.reshape(w.shape[0], k, -1)
+  out = torch.einsum("bke,bk->be", un, w)
+  return out.to(out_dtype)
+
+
+def unroute_sum(tokens: torch.Tensor, selected_experts: np.ndarray):
+  """kernels/sort_activations.py:98-121: gather by argsort(argsort) and sum
+  over k without weights (batch-split DeepSeek variant)."""
+  t, k = selected_experts.shape
+  inds = np.argsort(np.argsort(selected_experts.reshape(-1), kind="stable"), kind="stable")
+  g = tokens[torch.from_numpy(inds.astype(np.int64))]
+  return g.reshape(t, k, -1).sum(1)
+
+
+# --------------------------------------------------------------------------
+# Activation  (moe.py:841-870; pallas_mosaic_tpu_v2_gmm_kernel.py:33-73)
+# --------------------------------------------------------------------------
+
+
+def apply_ffn_activation(h0: torch.Tensor, h1: torch.Tensor, kind: str = "silu", limit: float = 7.0, out_dtype=torch.bfloat16):
+  """kind "silu": silu(h0)*h1 (moe.py:868-869); "swigluoai": GPT-OSS clipped
+  variant (moe.py:844-853 == v2 kernel :33-40); "silu_clip": DeepSeek-V4
+  (moe.py:854-866).  Computed in f32, cast to the layer dtype (:870)."""
+  h0 = h0.to(torch.float32)
+  h1 = h1.to(torch.float32)
+  if kind == "silu":
+    out = torch.nn.functional.silu(h0) * h1
+  elif kind == "swigluoai":
+    g = torch.clamp(h0, max=limit)
+    u = torch.clamp(h1, min=-limit, max=limit)
+    out = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+  elif kind == "silu_clip":
+    g = torch.clamp(h0, max=limit)
+    u = torch.clamp(h1, min=-limit, max=limit)
+    out = torch.nn.functional.silu(g) * u
+  else:
+    raise ValueError(kind)
+  return out.to(out_dtype)
+
+
+# --------------------------------------------------------------------------
+# Grouped matmul
+#   tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:92-153 (reference_gmm),
+#   kernels/megablox/backend.py:316-333, moe.py:1450-1459 (per-expert scale)
+# --------------------------------------------------------------------------
+
+
+def _to_f(x: torch.Tensor, dt):
+  return x.to(dt)
+
+
+def gmm(
+    lhs: torch.Tensor,  # [m, k]  bf16 / int8 / float8_e4m3fn
+    rhs: torch.Tensor,  # [g, k, n] (or [g, n, k] with transpose_rhs)
+    group_sizes,  # [G_total] int32
+    *,
+    rhs_scale: torch.Tensor | None = None,  # [g, nb, 1, n] f32 (v2 format) or [g, n]
+    lhs_scale: torch.Tensor | None = None,  # [m] / [m,1] per row, or [m, nb] per K-block
+    rhs_bias: torch.Tensor | None = None,  # [g, 1, n]
+    partial_sum: torch.Tensor | None = None,  # [m, n]
+    group_offset: int = 0,
+    quant_block: int | None = None,  # K-block size when scales are block-wise (ragged tail allowed)
+    transpose_rhs: bool = False,
+    out_dtype=torch.bfloat16,
+    acc_dtype=torch.float64,
+) -> torch.Tensor:
+  """out[rows of group g] = lhs[rows] @ rhs[g - group_offset], accumulating
+  per K-block and applying the block's scales to the partial sum
+  (reference_gmm :121-135); rows of non-local groups and rows past
+  sum(group_sizes) are zero (:139-141; v2 kernel :753-826)."""
+  if transpose_rhs:
+    rhs = rhs.transpose(1, 2)
+  m, k = lhs.shape
+  g, k2, n = rhs.shape
+  assert k == k2
+  group_sizes = np.asarray(group_sizes, dtype=np.int64)
+  out = torch.zeros((m, n), dtype=acc_dtype)
+
+  if rhs_scale is not None and rhs_scale.dim() == 2:
+    rhs_scale = rhs_scale[:, None, None, :]
+  nb_r = rhs_scale.shape[1] if rhs_scale is not None else 1
+  if lhs_scale is not None and lhs_scale.dim() == 1:
+    lhs_scale = lhs_scale[:, None]
+  nb_l = lhs_scale.shape[1] if lhs_scale is not None else 1
+  nb = max(nb_r, nb_l)
+  if nb > 1:
+    qb = quant_block if quant_block is not None else k // nb
+    assert math.ceil(k / qb) == nb, (k, qb, nb)
+  else:
+    qb = k
+
+  start = 0
+  for gg in range(group_sizes.size):
+    end = min(start + int(group_sizes[gg]), m)
+    loc = gg - group_offset
+    if 0 <= loc < g and end > start:
+      acc = torch.zeros((end - start, n), dtype=acc_dtype)
+      for b in range(nb):
+        ks, ke = b * qb, min((b + 1) * qb, k)
+        part = lhs[start:end, ks:ke].to(acc_dtype) @ rhs[loc, ks:ke, :].to(acc_dtype)
+        if rhs_scale is not None:
+          part = part * rhs_scale[loc, b if nb_r > 1 else 0].to(acc_dtype)
+        if lhs_scale is not None:
+          part = part * lhs_scale[start:end, (b if nb_l > 1 else 0)].to(acc_dtype)[:, None]
+        acc += part
+      if rhs_bias is not None:
+        acc = acc + rhs_bias[loc].to(acc_dtype)
+      if partial_sum is not None:
+        acc = acc + partial_sum[start:end].to(acc_dtype)
+      out[start:end] = acc
+    start = end
+  return out.to(out_dtype)
+
+
+# --------------------------------------------------------------------------
+# Quantisers and storage formats
+# --------------------------------------------------------------------------
+
+
+def get_static_scale(qmax: float, calibration_method: str) -> float:
+  """layers/quantizations.py:928-958 with qmax = symmetric bound of the dtype
+  (448 for float8_e4m3fn, pinned by quantizations_test.py:723-726)."""
+  if calibration_method is None or not calibration_method.lower().startswith("fixed"):
+    raise ValueError(f"Only static scale quantization is supported, got {calibration_method}")
+  args = [float(a) for a in calibration_method.split(",")[1:]]
+  if len(args) == 1:
+    args = [-args[0], args[0]]
+  if len(args) != 2 or args[0] + args[1] != 0 or args[1] <= 0:
+    raise ValueError(f"Expected format: 'fixed,max' or 'fixed,-max,max'. Got: {calibration_method}")
+  scale = args[1] / qmax
+  if scale < np.finfo(np.float32).tiny ** 0.5:
+    scale = 1.0
+  return scale
+
+
+def _absmax_scale(x: torch.Tensor, dim, qmax: float):
+  absmax = x.abs().to(torch.float32).amax(dim=dim, keepdim=True)
+  return absmax / qmax
+
+
+def _quant_int(x: torch.Tensor, scale: torch.Tensor, qmin: float, qmax: float):
+  x = x.to(torch.float32)
+  q = torch.where(scale == 0, torch.zeros_like(x), torch.round(x / scale))  # torch.round = half-to-even
+  return q.clamp(qmin, qmax)
+
+
+def quantize_rows_int8(x: torch.Tensor):
+  """Per-row (per-token) symmetric int8, scale [m] f32 (ops.py:241-248:
+  channelwise_axes=[0]; rounding unpinned, see module docstring)."""
+  scale = _absmax_scale(x, -1, INT8_MAX)
+  q = _quant_int(x, scale, -INT8_MAX, INT8_MAX).to(torch.int8)
+  return q, scale.squeeze(-1)
+
+
+def quantize_weight_int8(w: torch.Tensor, per_expert: bool = True):
+  """w [g, k, n] -> int8 [g,k,n], scale [g, n] f32.  per_expert=True is the
+  serve-mode layout gathered per row at moe.py:1450-1459; per_expert=False
+  shares one [n] scale across experts and K (ops.py:250-260)."""
+  if per_expert:
+    scale = _absmax_scale(w, 1, INT8_MAX)  # [g,1,n]
+  else:
+    scale = _absmax_scale(w, (0, 1), INT8_MAX).expand(w.shape[0], 1, w.shape[2])
+  q = _quant_int(w, scale, -INT8_MAX, INT8_MAX).to(torch.int8)
+  return q, scale.squeeze(1).contiguous()
+
+
+def quantize_fp8_blocks(x: torch.Tensor, block_rows: int, block_cols: int):
+  """Symmetric float8_e4m3fn with one f32 scale per [block_rows, block_cols]
+  block of the last two dims (ragged edge blocks allowed).  1x128 for
+  activations, 128x128 for weights (DeepSeek-V3 recipe; storage format follows
+  checkpoint_conversion/standalone_scripts/deepseek_dequantize.py:42-68).
+  Returns (q float8_e4m3fn same shape, scale [..., ceil(r/br), ceil(c/bc)])."""
+  *lead, r, c = x.shape
+  nr, nc = math.ceil(r / block_rows), math.ceil(c / block_cols)
+  xp = torch.zeros(*lead, nr * block_rows, nc * block_cols, dtype=torch.float32)
+  xp[..., :r, :c] = x.to(torch.float32)
+  xb = xp.reshape(*lead, nr, block_rows, nc, block_cols)
+  absmax = xb.abs().amax(dim=(-3, -1), keepdim=True)
+  scale = absmax / FP8_E4M3_MAX
+  q = torch.where(scale == 0, torch.zeros_like(xb), xb / scale).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX)
+  q = q.reshape(*lead, nr * block_rows, nc * block_cols)[..., :r, :c].to(torch.float8_e4m3fn)
+  return q.contiguous(), scale.reshape(*lead, nr, nc).contiguous()
+
+
+def dequantize_fp8_blocks(q: torch.Tensor, scale: torch.Tensor, block: int = 128) -> torch.Tensor:
+  """deepseek_dequantize.py:42-68 (float scale branch): x * repeat(scale) -> bf16."""
+  r, c = q.shape[-2:]
+  s = torch.repeat_interleave(torch.repeat_interleave(scale.to(torch.float32), block, dim=-2), block, dim=-1)
+  return (q.to(torch.float32) * s[..., :r, :c]).to(torch.bfloat16)
+
+
+def quantize_int4_groups(w: torch.Tensor, group: int = 128):
+  """Symmetric int4 with one scale per `group` consecutive elements of the
+  last (contraction) axis; restates _quantize_per_group of
+  tests/unit/dequantize_pack_quantized_int4_test.py:46-53 (scale clamped at
+  1e-12, round, clamp [-8, 7]) and allows a ragged last group.
+  Returns (int8 values in [-8,7] same shape, scale [..., ceil(K/group)] f32)."""
+  *lead, kdim = w.shape
+  ng = math.ceil(kdim / group)
+  wp = torch.zeros(*lead, ng * group, dtype=torch.float32)
+  wp[..., :kdim] = w.to(torch.float32)
+  wg = wp.reshape(*lead, ng, group)
+  scale = (wg.abs().amax(-1, keepdim=True) / INT4_MAX).clamp(min=1e-12)
+  q = torch.round(wg / scale).clamp(-8, 7).to(torch.int8).reshape(*lead, ng * group)[..., :kdim]
+  return q.contiguous(), scale.squeeze(-1).contiguous()
+
+
+def pack_int4(q: torch.Tensor) -> torch.Tensor:
+  """Two values per byte along the last axis, first value in the low nibble,
+  stored as value + 8 -- byte-identical (little endian) to the int32 layout
+  described at convert_deepseek_family_ckpt.py:62-66 (weight k in bits
+  [4k, 4k+4))."""
+  assert q.shape[-1] % 2 == 0
+  u = (q.to(torch.int16) + 8).to(torch.uint8)
+  return (u[..., 0::2] | (u[..., 1::2] << 4)).contiguous()
+
+
+def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
+  """Inverse of pack_int4 (convert_deepseek_family_ckpt.py:72-74: nibble - 8)."""
+  lo = (packed & 0xF).to(torch.int8) - 8
+  hi = (packed >> 4).to(torch.int8) - 8
+  return torch.stack([lo, hi], dim=-1).reshape(*packed.shape[:-1], packed.shape[-1] * 2)
+
+
+def dequantize_int4(packed: torch.Tensor, scale: torch.Tensor, group: int = 128) -> torch.Tensor:
+  """convert_deepseek_family_ckpt.py:56-84: (nibble-8) * scale per group -> bf16."""
+  q = unpack_int4(packed).to(torch.float32)
+  kdim = q.shape[-1]
+  s = torch.repeat_interleave(scale.to(torch.float32), group, dim=-1)[..., :kdim]
+  return (q * s).to(torch.bfloat16)
+
+
+# --------------------------------------------------------------------------
+# Whole layer: sparse path (moe.py:2186-2294) and two independent restatements
+# --------------------------------------------------------------------------
+
+
+def moe_layer_sparse(x: torch.Tensor, weights: np.ndarray, idx: np.ndarray, num_experts: int, expert_fn):
+  """permute -> expert_fn(sorted_inputs, group_sizes) -> unpermute.
+  expert_fn maps the sorted [M,d] rows to [M,d] outputs (gmm x3 + activation)."""
+  k = idx.shape[-1]
+  sorted_inputs, perm, group_size, _ = permute(x, idx, num_experts)
+  inter = expert_fn(sorted_inputs, group_size)
+  return unpermute(inter, perm, weights, k, out_dtype=x.dtype)
+
+
+def moe_layer_loop(x: torch.Tensor, weights: np.ndarray, idx: np.ndarray, num_experts: int, mlp_fn):
+  """Per-expert masked loop, the ground truth of tests/unit/moe_test.py:344-411
+  (MoeLoopBlock): out = sum_e mask_e * w * MLP_e(x).  mlp_fn(e, rows)->[r,d]."""
+  t, d = x.shape
+  out = torch.zeros((t, d), dtype=torch.float32)
+  w = torch.from_numpy(np.ascontiguousarray(weights, dtype=np.float32))
+  for e in range(num_experts):
+    tok, slot = np.nonzero(idx == e)
+    if tok.size == 0:
+      continue
+    y = mlp_fn(e, x[torch.from_numpy(tok)]).to(torch.float32)
+    out.index_add_(0, torch.from_numpy(tok), y * w[torch.from_numpy(tok), torch.from_numpy(slot)][:, None])
+  return out.to(x.dtype)

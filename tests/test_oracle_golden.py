@@ -1,0 +1,317 @@
+"""Pins the CPU oracle against the reference's own known answers and against
+independent formulations (brute force, closed forms, second code paths)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+
+# ---- known answers held by the reference's tests ---------------------------
+
+
+def test_deepseek_group_routing_known_answer():
+  # tests/unit/moe_test.py:293-326 (16 experts, 4 groups, top-2 groups, top-4)
+  gate = np.array(
+      [[[0.20, 0.10, 0.05, 0.10, 0.10, 0.60, 0.30, 0.10, 0.80, 0.01, 0.01, 0.01, 0.05, 0.80, 0.20, 0.10],
+        [0.68, 0.20, 0.06, 0.03, 0.32, 0.10, 0.05, 0.02, 0.65, 0.20, 0.04, 0.01, 0.32, 0.10, 0.05, 0.02]]],
+      dtype=np.float32)
+  pre = gate - 0.5
+  w, idx = O.deepseek_routing(gate, pre, 4, n_routing_groups=4, topk_routing_group=2)
+  expect = np.array([[[13, 5, 6, 14], [0, 8, 1, 9]]])
+  np.testing.assert_array_equal(idx, expect)
+  np.testing.assert_allclose(w, np.take_along_axis(pre, expect, -1), rtol=1e-5, atol=1e-5)
+
+
+def test_load_balance_updates_known_answer():
+  # tests/unit/moe_test.py:328-341
+  idx = np.array([[[0, 1], [3, 0], [3, 1], [1, 0]], [[0, 3], [2, 0], [1, 2], [2, 3]]])
+  np.testing.assert_allclose(O.calculate_load_balance_updates(idx, 4, 0.01), [-0.01, 0.0, 0.01, 0.0])
+
+
+def test_static_scale_known_answer():
+  # tests/unit/quantizations_test.py:723-743
+  assert abs(O.get_static_scale(O.FP8_E4M3_MAX, "fixed,224.0") - 0.5) < 1e-6
+  assert abs(O.get_static_scale(O.FP8_E4M3_MAX, "fixed,-224,224") - 0.5) < 1e-6
+  for bad in ("fixed,1,2,3", "fixed,-200.0,224.0", "fixed", "absmax"):
+    with pytest.raises(ValueError):
+      O.get_static_scale(O.FP8_E4M3_MAX, bad)
+  assert float(torch.finfo(torch.float8_e4m3fn).max) == O.FP8_E4M3_MAX
+
+
+def test_int4_pack_format_known_answers():
+  # tests/unit/dequantize_pack_quantized_int4_test.py:61-127 (cases restated:
+  # pack_to_int32 of compressed_tensors is not installed; its layout is
+  # "weight k in bits [4k,4k+4) of the int32", i.e. low nibble first).
+  torch.manual_seed(0)
+  w = torch.randn(64, 128) * 0.1
+  q, scale = O.quantize_int4_groups(w, group=32)
+  packed = O.pack_int4(q)
+  assert packed.shape == (64, 64)
+  # int32 view: weight k lives in bits [4k, 4k+4)
+  as_i32 = packed.contiguous().view(torch.int32)
+  shifts = torch.arange(8, dtype=torch.int32) * 4
+  nib = ((as_i32.unsqueeze(-1) >> shifts) & 0xF) - 8
+  assert torch.equal(nib.reshape(64, 128).to(torch.int8), q)
+  assert torch.equal(O.unpack_int4(packed), q)
+  # full dequant == (int * bf16 scale).bf16 bit for bit
+  sb = scale.to(torch.bfloat16)
+  ref = (q.reshape(64, 4, 32).float() * sb.float().unsqueeze(-1)).reshape(64, 128).to(torch.bfloat16)
+  assert torch.equal(O.dequantize_int4(packed, sb, group=32), ref)
+  # boundary values and zero groups
+  ones = torch.ones(16, 2, dtype=torch.bfloat16)
+  for v in (-8, 7):
+    p = O.pack_int4(torch.full((16, 64), v, dtype=torch.int8))
+    assert torch.all(O.dequantize_int4(p, ones, group=32).float() == float(v))
+  p = O.pack_int4(torch.zeros(8, 64, dtype=torch.int8))
+  assert torch.all(O.dequantize_int4(p, torch.full((8, 2), 0.123, dtype=torch.bfloat16), group=32) == 0)
+
+
+def test_fp8_block_dequant_formula():
+  # deepseek_dequantize.py:42-68: reshape/broadcast branch vs element loop
+  torch.manual_seed(1)
+  x = (torch.randn(256, 384) * 3).to(torch.float8_e4m3fn)
+  s = torch.rand(2, 3) + 0.5
+  got = O.dequantize_fp8_blocks(x, s, 128)
+  for (i, j) in [(0, 0), (127, 127), (128, 128), (255, 383), (200, 130)]:
+    assert got[i, j] == (x[i, j].float() * s[i // 128, j // 128]).to(torch.bfloat16)
+  # ragged shape branch (:57-62)
+  xr = x[:200, :300]
+  gr = O.dequantize_fp8_blocks(xr, s, 128)
+  assert torch.equal(gr, got[:200, :300])
+
+
+def test_gmm_int8_small_known_tolerance():
+  # tests/unit/quantizations_test.py:607-653: groups [3,5], k=6, n=4, int8 on
+  # both sides, mean relative error below 0.2 versus the unquantised product.
+  g = torch.Generator().manual_seed(0)
+  gs = np.array([3, 5], np.int32)
+  lhs = torch.randn(8, 6, generator=g)
+  rhs = torch.randn(2, 6, 4, generator=g)
+  base = O.gmm(lhs, rhs, gs, out_dtype=torch.float32)
+  ql, sl = O.quantize_rows_int8(lhs)
+  qr, sr = O.quantize_weight_int8(rhs, per_expert=False)
+  quant = O.gmm(ql, qr, gs, lhs_scale=sl, rhs_scale=sr, out_dtype=torch.float32)
+  assert (quant - base).abs().mean() / base.abs().mean() < 0.2
+
+
+# ---- brute force / invariants / independent second paths -------------------
+
+
+def test_top_k_brute_force_and_ties():
+  rng = np.random.default_rng(0)
+  x = rng.standard_normal((50, 37)).astype(np.float32)
+  vals, idx = O.top_k(x, 5)
+  for r in range(50):
+    row = list(x[r])
+    picked = []
+    for _ in range(5):
+      best = max(range(37), key=lambda j: (row[j], -j) if j not in picked else (-np.inf, -j))
+      picked.append(best)
+    assert picked == list(idx[r])
+    assert np.all(np.diff(vals[r]) <= 0)
+  # ties: lower index first
+  t = np.array([[1.0, 3.0, 3.0, 2.0, 3.0]], np.float32)
+  assert list(O.top_k(t, 4)[1][0]) == [1, 2, 4, 3]
+
+
+def test_softmax_topk_weights_closed_form():
+  rng = np.random.default_rng(1)
+  x = rng.standard_normal((64, 8)).astype(np.float32)
+  w, idx = O.get_topk(x, k=2, weight_dtype="f32")
+  a = np.take_along_axis(x, idx, -1).astype(np.float64)
+  # two-way softmax == logistic of the difference
+  np.testing.assert_allclose(w[:, 0], 1 / (1 + np.exp(a[:, 1] - a[:, 0])), rtol=1e-6)
+  np.testing.assert_allclose(w.sum(-1), 1.0, rtol=1e-6)
+  wb, _ = O.get_topk(x, k=2)
+  assert np.max(np.abs(wb - w) / w) <= 2.0**-8
+  wn, _ = O.get_topk(x, k=2, norm_topk_prob=True)
+  np.testing.assert_allclose(wn.sum(-1), 1.0, atol=2e-2)
+
+
+def test_deepseek_weights_closed_form():
+  rng = np.random.default_rng(2)
+  logits = rng.standard_normal((32, 64)).astype(np.float32)
+  scores = (1 / (1 + np.exp(-logits))).astype(np.float32)
+  bias = (rng.standard_normal(64) * 0.1).astype(np.float32)
+  w, idx = O.get_topk(scores + bias, scores, k=8, mode="deepseek", routed_scaling_factor=2.5)
+  np.testing.assert_allclose(w.sum(-1), 2.5, rtol=1e-5)
+  # selection uses biased scores, weights use unbiased ones
+  sel = np.argsort(-(scores + bias), -1, kind="stable")[:, :8]
+  np.testing.assert_array_equal(idx, sel)
+  raw = np.take_along_axis(scores, idx, -1)
+  np.testing.assert_allclose(w, raw / raw.sum(-1, keepdims=True) * 2.5, rtol=1e-5)
+
+
+def test_permute_invariants_and_bruteforce():
+  rng = np.random.default_rng(3)
+  t, k, e, d = 97, 3, 11, 16
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  sel[sel == 7] = 6  # leave expert 7 empty, duplicates across tokens only
+  x = torch.randn(t, d).to(torch.bfloat16)
+  sx, perm, gs, se = O.permute(x, sel, e)
+  flat = sel.reshape(-1)
+  assert sorted(perm.tolist()) == list(range(t * k))
+  assert np.all(np.diff(flat[perm]) >= 0)
+  for i in range(1, t * k):
+    if flat[perm[i]] == flat[perm[i - 1]]:
+      assert perm[i] > perm[i - 1]
+  assert gs.sum() == t * k and gs[7] == 0
+  for ee in range(e):
+    assert gs[ee] == int((flat == ee).sum())
+  np.testing.assert_array_equal(se, flat[perm])
+  for i in range(t * k):
+    assert torch.equal(sx[i], x[perm[i] // k])
+
+
+def test_unpermute_bruteforce_and_identity():
+  rng = np.random.default_rng(4)
+  t, k, e, d = 40, 4, 9, 8
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  x = torch.randn(t, d).to(torch.bfloat16)
+  sx, perm, _, _ = O.permute(x, sel, e)
+  # identity experts, weights one: output == k * x
+  out = O.unpermute(sx, perm, np.ones((t, k), np.float32), k)
+  assert torch.equal(out, (x.float() * k).to(torch.bfloat16))
+  # brute force with random weights and random intermediate
+  inter = torch.randn(t * k, d).to(torch.bfloat16)
+  w = rng.random((t, k)).astype(np.float32)
+  out = O.unpermute(inter, perm, w, k, out_dtype=torch.float32)
+  pos = {int(p): i for i, p in enumerate(perm)}
+  for tt in range(t):
+    acc = np.zeros(d, np.float64)
+    for s in range(k):
+      acc += float(w[tt, s]) * inter[pos[tt * k + s]].double().numpy()
+    np.testing.assert_allclose(out[tt].numpy(), acc, rtol=1e-5, atol=1e-6)
+  # unweighted unroute (sort_activations.py:98-121)
+  un = O.unroute_sum(inter.float(), sel)
+  np.testing.assert_allclose(un.numpy(), O.unpermute(inter, perm, np.ones((t, k), np.float32), k, torch.float32).numpy(), rtol=1e-6)
+
+
+def test_gmm_special_cases():
+  g = torch.Generator().manual_seed(5)
+  m, k, n, e = 64, 48, 40, 5
+  lhs = torch.randn(m, k, generator=g)
+  rhs = torch.randn(e, k, n, generator=g)
+  # one group holds everything -> plain matmul
+  gs = np.array([0, 0, m, 0, 0], np.int32)
+  np.testing.assert_allclose(O.gmm(lhs, rhs, gs, out_dtype=torch.float32), lhs @ rhs[2], rtol=1e-5, atol=1e-5)
+  # ragged groups with an empty one, rows past the sum are zero
+  gs = np.array([7, 0, 20, 1, 30], np.int32)
+  out = O.gmm(lhs, rhs, gs, out_dtype=torch.float32)
+  off = np.concatenate([[0], np.cumsum(gs)])
+  for ee in range(e):
+    np.testing.assert_allclose(out[off[ee]:off[ee + 1]], lhs[off[ee]:off[ee + 1]] @ rhs[ee], rtol=1e-5, atol=1e-5)
+  assert torch.all(out[off[-1]:] == 0)
+  # transpose_rhs
+  np.testing.assert_allclose(O.gmm(lhs, rhs.transpose(1, 2).contiguous(), gs, transpose_rhs=True, out_dtype=torch.float32), out)
+  # group_offset: only local groups computed, others zero (reference_gmm :111-141)
+  out2 = O.gmm(lhs, rhs[2:4], gs, group_offset=2, out_dtype=torch.float32)
+  assert torch.all(out2[:off[2]] == 0) and torch.all(out2[off[4]:] == 0)
+  np.testing.assert_allclose(out2[off[2]:off[4]], out[off[2]:off[4]])
+  # bias + partial_sum
+  bias = torch.randn(e, 1, n, generator=g)
+  ps = torch.randn(m, n, generator=g)
+  out3 = O.gmm(lhs, rhs, gs, rhs_bias=bias, partial_sum=ps, out_dtype=torch.float32)
+  np.testing.assert_allclose(out3[:7], lhs[:7] @ rhs[0] + bias[0] + ps[:7], rtol=1e-5, atol=1e-5)
+
+
+def test_gmm_int8_exact_on_integers():
+  g = torch.Generator().manual_seed(6)
+  m, k, n, e = 33, 512, 24, 3
+  lq = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8)
+  rq = torch.randint(-127, 128, (e, k, n), generator=g, dtype=torch.int8)
+  gs = np.array([10, 3, 20], np.int32)
+  out = O.gmm(lq, rq, gs, out_dtype=torch.float64)
+  off = [0, 10, 13, 33]
+  for ee in range(e):
+    want = lq[off[ee]:off[ee + 1]].to(torch.int64) @ rq[ee].to(torch.int64)
+    assert torch.equal(out[off[ee]:off[ee + 1]].to(torch.int64), want)
+
+
+def test_gmm_block_scales_equal_dequantised_matmul():
+  g = torch.Generator().manual_seed(7)
+  m, k, n, e = 24, 384, 256, 2
+  a = torch.randn(m, k, generator=g)
+  w = torch.randn(e, n, k, generator=g) * 0.02  # [g, n, k]
+  aq, asc = O.quantize_fp8_blocks(a, 1, 128)
+  wq, wsc = O.quantize_fp8_blocks(w, 128, 128)  # scale [e, n/128, k/128]
+  gs = np.array([10, 14], np.int32)
+  rhs_scale = torch.repeat_interleave(wsc.permute(0, 2, 1), 128, dim=2)[:, :, None, :]  # v2 format [g, nb, 1, n]
+  out = O.gmm(aq, wq, gs, lhs_scale=asc, rhs_scale=rhs_scale, transpose_rhs=True, quant_block=128, out_dtype=torch.float32)
+  a_deq = aq.float() * torch.repeat_interleave(asc, 128, dim=1)
+  w_deq = wq.float() * torch.repeat_interleave(torch.repeat_interleave(wsc, 128, 1), 128, 2)
+  want = torch.cat([a_deq[:10] @ w_deq[0].T, a_deq[10:] @ w_deq[1].T])
+  np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-5)
+  # quantisation error itself is small
+  full = torch.cat([a[:10] @ w[0].T, a[10:] @ w[1].T])
+  assert (out - full).norm() / full.norm() < 0.06
+
+
+def test_quantisers_closed_form():
+  x = torch.tensor([[0.0, 0.0, 0.0, 0.0], [1.0, -2.0, 0.5, 127.0], [-254.0, 1.0, 3.0, 5.0]])
+  q, s = O.quantize_rows_int8(x)
+  assert s.tolist() == [0.0, 1.0, 2.0]
+  assert q.tolist() == [[0, 0, 0, 0], [1, -2, 0, 127], [-127, 0, 2, 2]]  # 0.5->0, 1.5->2, 2.5->2 (half to even)
+  w = torch.randn(3, 16, 5)
+  qw, sw = O.quantize_weight_int8(w)
+  assert sw.shape == (3, 5) and torch.allclose(sw, w.abs().amax(1) / 127)
+  assert (qw.float() * sw[:, None, :] - w).abs().max() <= sw.max() * 0.5 + 1e-7
+  qs, ss = O.quantize_weight_int8(w, per_expert=False)
+  assert torch.all(ss == ss[0])
+  q4, s4 = O.quantize_int4_groups(torch.randn(4, 2880), group=128)
+  assert s4.shape == (4, 23) and q4.min() >= -8 and q4.max() <= 7
+
+
+def test_activation_closed_forms():
+  h0 = torch.tensor([-3.0, 0.0, 2.0, 9.0])
+  h1 = torch.tensor([1.0, 2.0, -8.0, 0.5])
+  a = O.apply_ffn_activation(h0, h1, "silu", out_dtype=torch.float32)
+  np.testing.assert_allclose(a, (h0 / (1 + torch.exp(-h0))) * h1, rtol=1e-6)
+  b = O.apply_ffn_activation(h0, h1, "swigluoai", out_dtype=torch.float32)
+  g = torch.tensor([-3.0, 0.0, 2.0, 7.0])
+  u = torch.tensor([1.0, 2.0, -7.0, 0.5])
+  np.testing.assert_allclose(b, g / (1 + torch.exp(-1.702 * g)) * (u + 1), rtol=1e-6)
+
+
+def _layer_fixture(seed=8, t=60, d=32, f=48, e=6, k=2):
+  g = torch.Generator().manual_seed(seed)
+  x = torch.randn(t, d, generator=g).to(torch.bfloat16)
+  w0 = (torch.randn(e, d, f, generator=g) * 0.1).to(torch.bfloat16)
+  w1 = (torch.randn(e, d, f, generator=g) * 0.1).to(torch.bfloat16)
+  wo = (torch.randn(e, f, d, generator=g) * 0.1).to(torch.bfloat16)
+  logits = torch.randn(t, e, generator=g).numpy()
+  return x, w0, w1, wo, logits
+
+
+def test_sparse_layer_equals_loop_and_dense():
+  x, w0, w1, wo, logits = _layer_fixture()
+  e, k = 6, 2
+  wts, idx = O.get_topk(logits, k=k)
+
+  def expert_fn(rows, gs):
+    h0 = O.gmm(rows, w0, gs)
+    h1 = O.gmm(rows, w1, gs)
+    return O.gmm(O.apply_ffn_activation(h0, h1), wo, gs)
+
+  sparse = O.moe_layer_sparse(x, wts, idx, e, expert_fn)
+
+  def mlp(ee, rows):
+    h0 = (rows.double() @ w0[ee].double()).to(torch.bfloat16)
+    h1 = (rows.double() @ w1[ee].double()).to(torch.bfloat16)
+    a = O.apply_ffn_activation(h0, h1)
+    return (a.double() @ wo[ee].double()).to(torch.bfloat16)
+
+  loop = O.moe_layer_loop(x, wts, idx, e, mlp)
+  assert (sparse.float() - loop.float()).abs().max() <= 2e-2 * loop.float().abs().max()
+  # dense all-experts formulation (moe.py:2996-3039): "BSM,EMH->BSEH" then
+  # "BSEM,BSE->BSM" with a scattered weight matrix
+  dense_w = torch.zeros(x.shape[0], e)
+  dense_w.scatter_(1, torch.from_numpy(idx.astype(np.int64)), torch.from_numpy(wts))
+  h0 = torch.einsum("tm,emh->teh", x.float(), w0.float()).to(torch.bfloat16)
+  h1 = torch.einsum("tm,emh->teh", x.float(), w1.float()).to(torch.bfloat16)
+  a = O.apply_ffn_activation(h0, h1)
+  y = torch.einsum("teh,ehm->tem", a.float(), wo.float()).to(torch.bfloat16)
+  dense = torch.einsum("tem,te->tm", y.float(), dense_w).to(torch.bfloat16)
+  assert (sparse.float() - dense.float()).abs().max() <= 2e-2 * dense.float().abs().max()
