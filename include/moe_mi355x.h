@@ -1,0 +1,207 @@
+/*
+ * moe_mi355x.h -- C ABI of libmoe_mi355x.so: the quantized MoE expert path
+ * (routing -> permute -> grouped GEMM with fused SwiGLU -> unpermute+combine)
+ * as hand-written gfx950 HIP kernels.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the parameter name ends in _host;
+ *   - every call is asynchronous on `stream` (a hipStream_t passed as void*; NULL =
+ *     the default stream), allocates nothing, never synchronises and never throws;
+ *   - the return value is a moe_status (0 = ok, negative = the call enqueued nothing);
+ *   - `group_sizes` stays on the device: no entry point reads it on the host;
+ *   - inputs are never written; outputs are fully defined (rows that belong to no
+ *     local group are written as zeros), so buffers need no pre-clearing;
+ *   - no global mutable state: calls on different streams with disjoint buffers
+ *     may overlap.
+ *
+ * Paths in the citations are relative to the reference (AI-Hypercomputer/maxtext).
+ */
+#ifndef MOE_MI355X_H_
+#define MOE_MI355X_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Exported from the shared library (everything else is built with hidden visibility). */
+#define MOE_API __attribute__((visibility("default")))
+
+typedef enum {
+  MOE_OK = 0,
+  MOE_ERR_INVALID_ARG = -1, /* NULL pointer, non-positive size, bad enum            */
+  MOE_ERR_UNSUPPORTED = -2, /* valid request the kernels do not cover (see below)   */
+  MOE_ERR_WORKSPACE = -3,   /* workspace_bytes smaller than *_workspace_bytes()     */
+  MOE_ERR_LAUNCH = -4       /* hipGetLastError() != hipSuccess after a launch       */
+} moe_status;
+
+typedef enum {
+  MOE_BF16 = 0,
+  MOE_INT8 = 1,
+  MOE_FP8_E4M3 = 2, /* OCP float8_e4m3fn (max 448), layers/quantizations.py:237      */
+  MOE_INT4 = 3,     /* 2 per byte along K, first value in the low nibble, stored +8  */
+  MOE_F32 = 4
+} moe_dtype;
+
+typedef enum {
+  MOE_ROUTE_SOFTMAX_TOPK = 0, /* lax.top_k -> softmax over the k values, moe.py:747-753 */
+  MOE_ROUTE_DEEPSEEK = 1      /* deepseek_routing + deepseek_scale_weights, moe.py:767-839 */
+} moe_route_mode;
+
+typedef enum {
+  MOE_ACT_NONE = 0,
+  MOE_ACT_SILU = 1,      /* silu(gate) * up, moe.py:868-869; v2 kernel "silu" :64-65   */
+  MOE_ACT_SWIGLUOAI = 2, /* GPT-OSS clipped variant, moe.py:844-853; v2 kernel :33-40   */
+  MOE_ACT_SILU_CLIP = 3  /* DeepSeek-V4 clipped SwiGLU, moe.py:854-866                  */
+} moe_act;
+
+/* Text for the last non-zero status returned on the calling thread. */
+MOE_API const char* moe_last_error(void);
+/* ABI version; bumped when a struct below changes. */
+MOE_API int moe_abi_version(void);
+
+/* ---------------------------------------------------------------------------
+ * Routing.  Replaces RoutedMoE.get_topk (src/maxtext/layers/moe.py:717-765),
+ * deepseek_routing (:813-839), expert_group_mask (:775-811) and
+ * deepseek_scale_weights (:767-773).
+ *
+ *   gate_logits      [T, E] f32   scores the selection runs on (post-bias for DeepSeek)
+ *   pre_bias_logits  [T, E] f32   DeepSeek only: scores the weights are read from
+ *   topk_weights     [T, k] f32   out; SOFTMAX_TOPK rounds them to bf16 when
+ *                                 weights_round_bf16 != 0 (the cast at moe.py:753)
+ *   topk_idx         [T, k] i32   out; descending score, lower index first on ties
+ *
+ * norm_topk_prob: SOFTMAX_TOPK: divide by the sum of the k weights (moe.py:756);
+ *   DEEPSEEK: w /= sum(w) + 1e-20, the sigmoid / sqrtsoftplus branch of moe.py:770-771.
+ *   DEEPSEEK always multiplies by routed_scaling_factor (moe.py:772).
+ * n_routing_groups / topk_routing_group: DeepSeek group-limited routing; -1 disables.
+ * Limits: 1 <= k <= 16, k <= E <= 512, n_routing_groups <= 64 and divides E.
+ */
+MOE_API int moe_route_topk(const float* gate_logits, const float* pre_bias_logits, int T, int E, int k,
+                   int mode, int norm_topk_prob, int weights_round_bf16,
+                   float routed_scaling_factor, int n_routing_groups, int topk_routing_group,
+                   float* topk_weights, int32_t* topk_idx, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Sort by expert.  Replaces the index half of RoutedMoE.permute
+ * (moe.py:950-954, :960, :986-991): jnp.argsort (stable) of the flattened
+ * expert ids, jnp.bincount, and repeat(arange(E), group_size).
+ *
+ *   topk_idx        [T, k] i32   in
+ *   perm            [M] i32      out, M = T*k; == sorted_selected_experts
+ *   inv_perm        [M] i32      out (may be NULL); inv_perm[perm[i]] = i == argsort(perm)
+ *   group_sizes     [E] i32      out
+ *   sorted_experts  [M] i32      out (may be NULL)
+ * Limits: E <= 512.
+ */
+MOE_API size_t moe_sort_workspace_bytes(int T, int k, int E);
+MOE_API int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,
+                       int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Row gather with optional quantisation.  Replaces the data half of permute
+ * (moe.py:956-959: repeat(x, k)[perm]) fused with the activation quantiser of
+ * the grouped GEMM (kernels/megablox/ops.py:241-248, per-row scale;
+ * pallas_mosaic_tpu_v2_gmm_kernel.py:534-542, per-K-block scale).
+ *
+ *   x        [R_in, d] bf16
+ *   row_idx  [R_out] i32 or NULL; output row i reads input row row_idx[i] / idx_div
+ *            (NULL: row i).  permute passes row_idx = perm, idx_div = k.
+ *   out      [R_out, d] of out_dtype: MOE_BF16 (copy), MOE_INT8, MOE_FP8_E4M3
+ *   scale    f32; block_k == 0: [R_out] one scale per row; else [R_out, ceil(d/block_k)]
+ *            (block_k must be 128).  scale = absmax / qmax, q = rint(x / scale)
+ *            clipped to +-qmax (127 / 448); zero absmax gives q = 0, scale = 0.
+ * Limits: d % 8 == 0, d <= 16384.
+ */
+MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_out, int d,
+                    int out_dtype, int block_k, void* out, float* scale, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Grouped matmul.  Replaces gmm(lhs, rhs, group_sizes, ...)
+ * (src/maxtext/kernels/megablox/ops.py:46-129; backend.gmm backend.py:304-562;
+ * gmm_v2 pallas_mosaic_tpu_v2_gmm_kernel.py:1297-1481) and the fused
+ * "gmm, gmm, activation" of gmm_up + apply_ffn_activation (moe.py:1932-1986, :841-870).
+ *
+ *   out[rows of group g, :] = act( lhs[rows] @ rhs[g - group_offset]^T ... )
+ *
+ * for every g in [group_offset, group_offset + num_groups_local); all other rows of
+ * `out` (non-local groups, rows past sum(group_sizes)) are written as zeros
+ * (reference_gmm, tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:139-141).
+ *
+ * Operand layouts in HBM
+ *   lhs        [M, K] row-major, lhs_dtype in {BF16, INT8, FP8_E4M3}
+ *   lhs_scale  f32: NULL (bf16 lhs) | [M] per row (lhs_scale_block_k == 0)
+ *              | [M, ceil(K/128)] (lhs_scale_block_k == 128)
+ *   rhs        [G_local, N, K], K contiguous ("transpose_rhs" layout, ops.py:52),
+ *              rhs_dtype in {BF16, INT8, FP8_E4M3, INT4}; INT4 rows hold K/2 bytes
+ *   rhs_scale  NULL (bf16 rhs) | [G_local, ceil(N/bn), nkb] with
+ *              bn = rhs_scale_block_n (1 = per output channel, 128 = DeepSeek 128x128 blocks),
+ *              nkb = 1 when rhs_scale_block_k == 0 (per channel over all of K), else
+ *              ceil(K / rhs_scale_block_k) (must be 128); f32, or bf16 for INT4
+ *   rhs_up / rhs_up_scale   second projection (wi_1) with the same layout; when non-NULL
+ *              the kernel computes act(lhs@rhs^T) * (lhs@rhs_up^T) in one pass
+ *   out        [M, N] bf16
+ *
+ * Supported operand combinations (others return MOE_ERR_UNSUPPORTED):
+ *   BF16 x BF16 | BF16 x INT8 (per-channel) | BF16 x INT4 (bn=1, bk=128)
+ *   INT8 (per-row) x INT8 (per-channel) | FP8 (1x128) x FP8 (128x128 blocks)
+ * Alignment: K % 32 == 0 (INT4), K % 16 == 0 otherwise; N % 8 == 0; pointers 16-byte aligned.
+ */
+typedef struct {
+  size_t struct_size; /* sizeof(moe_gmm_args), checked */
+  const void* lhs;
+  const float* lhs_scale;
+  const void* rhs;
+  const void* rhs_scale;
+  const void* rhs_up;
+  const void* rhs_up_scale;
+  const int32_t* group_sizes; /* [num_groups_total] i32, device */
+  void* out;
+  void* workspace;
+  size_t workspace_bytes;
+  int32_t M, K, N;
+  int32_t num_groups_total; /* length of group_sizes                       */
+  int32_t num_groups_local; /* leading dim of rhs                          */
+  int32_t group_offset;     /* first global group held by rhs (backend.py:340-347) */
+  int32_t lhs_dtype, rhs_dtype;
+  int32_t lhs_scale_block_k;
+  int32_t rhs_scale_block_n, rhs_scale_block_k;
+  int32_t act;     /* moe_act; must be MOE_ACT_NONE when rhs_up == NULL      */
+  float act_limit; /* clip for SWIGLUOAI / SILU_CLIP                        */
+  int32_t reserved[4];
+} moe_gmm_args;
+
+MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
+MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);
+
+/* One-time weight re-layout [G, K, N] -> [G, N, K] (1-byte or 2-byte elements), for
+ * callers that hold the reference's default rhs layout (ops.py:47, transpose_rhs=False). */
+MOE_API int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem_bytes, void* rhs_gnk,
+                      void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Unpermute + top-k weighted combine.  Replaces RoutedMoE.unpermute
+ * (moe.py:1039-1063, float32_weight_sum=True) and the fused gather-reduce
+ * fallback (kernels/ragged/ragged_gather_reduce_v2.py:170-182):
+ *
+ *   out[t, :] = bf16( sum_s weights[t, s] * f32(y[inv_perm[t*k + s], :]) )
+ *
+ *   y        [M, d] bf16     expert outputs in sorted order
+ *   perm     [M] i32         sorted_selected_experts; used only when inv_perm == NULL,
+ *                            then inv_perm is rebuilt into `workspace` (M * 4 bytes)
+ *   weights  [T, k] f32, or NULL for an unweighted sum
+ *            (kernels/sort_activations.py:98-121)
+ *   out      [T, d] bf16
+ * Limits: d % 8 == 0, k <= 16.
+ */
+MOE_API int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv_perm,
+                          const float* weights, int T, int k, int d, void* out, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_MI355X_H_ */

@@ -1,0 +1,106 @@
+"""ctypes binding of libmoe_mi355x.so (declared in include/moe_mi355x.h).
+
+There is no fallback: if the library has not been built, or a call reports an error, a
+RuntimeError is raised.  torch is used only for device memory and the current stream.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libmoe_mi355x.so")
+
+# enums of include/moe_mi355x.h
+MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32 = 0, 1, 2, 3, 4
+MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK = 0, 1
+MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
+
+ACT_BY_NAME = {None: MOE_ACT_NONE, "silu": MOE_ACT_SILU, "swigluoai": MOE_ACT_SWIGLUOAI, "silu_clip": MOE_ACT_SILU_CLIP}
+
+c_void_p, c_int, c_float, c_size_t = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+
+
+class GmmArgs(ctypes.Structure):
+  """moe_gmm_args."""
+
+  _fields_ = [
+      ("struct_size", c_size_t),
+      ("lhs", c_void_p),
+      ("lhs_scale", c_void_p),
+      ("rhs", c_void_p),
+      ("rhs_scale", c_void_p),
+      ("rhs_up", c_void_p),
+      ("rhs_up_scale", c_void_p),
+      ("group_sizes", c_void_p),
+      ("out", c_void_p),
+      ("workspace", c_void_p),
+      ("workspace_bytes", c_size_t),
+      ("M", ctypes.c_int32),
+      ("K", ctypes.c_int32),
+      ("N", ctypes.c_int32),
+      ("num_groups_total", ctypes.c_int32),
+      ("num_groups_local", ctypes.c_int32),
+      ("group_offset", ctypes.c_int32),
+      ("lhs_dtype", ctypes.c_int32),
+      ("rhs_dtype", ctypes.c_int32),
+      ("lhs_scale_block_k", ctypes.c_int32),
+      ("rhs_scale_block_n", ctypes.c_int32),
+      ("rhs_scale_block_k", ctypes.c_int32),
+      ("act", ctypes.c_int32),
+      ("act_limit", c_float),
+      ("reserved", ctypes.c_int32 * 4),
+  ]
+
+
+SIGNATURES = {
+    "moe_last_error": (ctypes.c_char_p, []),
+    "moe_abi_version": (c_int, []),
+    "moe_route_topk": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "moe_sort_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "moe_sort_by_expert": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "moe_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "moe_gmm_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "moe_gmm": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
+    "moe_transpose_rhs": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "moe_unpermute_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+}
+
+_lib = None
+
+
+def load():
+  """Loads the shared library once; raises if it has not been built."""
+  global _lib
+  if _lib is not None:
+    return _lib
+  if not os.path.exists(LIB_PATH):
+    raise RuntimeError(
+        f"{LIB_PATH} is missing: build it with `python -m maxtext_amd.build` "
+        "(there is no non-HIP fallback for the MoE expert path)"
+    )
+  lib = ctypes.CDLL(LIB_PATH)
+  for name, (res, args) in SIGNATURES.items():
+    fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+    fn.restype = res
+    fn.argtypes = args
+  _lib = lib
+  return lib
+
+
+def check(status: int, what: str):
+  if status != 0:
+    msg = load().moe_last_error().decode("utf-8", "replace")
+    raise RuntimeError(f"{what} failed with status {status}: {msg}")
+
+
+def ptr(t):
+  """Device pointer of a torch tensor (None -> NULL)."""
+  return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def current_stream():
+  import torch
+
+  return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)

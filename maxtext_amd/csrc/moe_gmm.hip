@@ -1,0 +1,652 @@
+// Grouped matmul for gfx950.
+//
+//   tile_map_kernel   group_sizes (device) -> list of (group, first row, rows) m-tiles that never
+//                     straddle a group boundary, plus zero-fill tiles for non-local / tail rows.
+//   gmm_tiled_kernel  LDS-staged, double-buffered MFMA GEMM over that tile list.  Weights are the
+//                     MFMA "A" operand (32 output channels per tile), activations the "B" operand
+//                     (32 rows), so each lane ends up with 4 consecutive output channels of one
+//                     row per accumulator quad and stores 8 bytes.  bf16 x {bf16, int8, int4}
+//                     weights run on v_mfma_f32_32x32x16_bf16 (weights are widened to bf16 while
+//                     they are copied into LDS), int8 x int8 on v_mfma_i32_32x32x32_i8.
+//   gmm_fp8_skinny_kernel  block-scaled fp8 for few rows per expert (decode): no LDS, every wave
+//                     streams 16 weight rows through v_mfma_f32_16x16x128_f8f6f4 and applies the
+//                     per-128 K-block scales to the f32 partial sums.
+
+#include <type_traits>
+
+#include "moe_common.h"
+
+namespace moe {
+
+struct TileInfo {
+  int32_t group;  // local group id, or -1: write zeros
+  int32_t row0;
+  int32_t nrows;
+  int32_t pad;
+};
+
+// workspace: int32 header[4] (header[0] = number of tiles) | TileInfo tiles[max_tiles]
+static inline int max_tiles_for(int M, int G, int bm) { return cdiv(M, bm) + G + 1; }
+
+constexpr int kMapThreads = 256;
+
+__device__ __forceinline__ int block_exclusive_scan(int v, int* s_buf, int* total) {
+  const int tid = threadIdx.x;
+  s_buf[tid] = v;
+  __syncthreads();
+  for (int o = 1; o < kMapThreads; o <<= 1) {
+    int add = tid >= o ? s_buf[tid - o] : 0;
+    __syncthreads();
+    s_buf[tid] += add;
+    __syncthreads();
+  }
+  int incl = s_buf[tid];
+  *total = s_buf[kMapThreads - 1];
+  __syncthreads();
+  return incl - v;
+}
+
+__global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
+    const int32_t* __restrict__ group_sizes, int G_total, int group_offset, int G_local, int M,
+    int BM, int32_t* __restrict__ header, TileInfo* __restrict__ tiles) {
+  __shared__ int s_buf[kMapThreads];
+  const int tid = threadIdx.x;
+  const int per = (G_total + kMapThreads - 1) / kMapThreads;
+  const int g0 = min(tid * per, G_total), g1 = min(g0 + per, G_total);
+  long long rows = 0;
+  for (int g = g0; g < g1; g++) rows += max(group_sizes[g], 0);
+  int total_rows;
+  int row_prefix = block_exclusive_scan((int)min(rows, (long long)M), s_buf, &total_rows);
+  // clipped extents (reference_gmm: end = min(start + size, m)) and tile counts
+  int ntiles = 0;
+  {
+    long long start = row_prefix;
+    for (int g = g0; g < g1; g++) {
+      long long end = start + max(group_sizes[g], 0);
+      int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
+      ntiles += (e - s + BM - 1) / BM;
+      start = end;
+    }
+  }
+  int total_tiles;
+  int tile_prefix = block_exclusive_scan(ntiles, s_buf, &total_tiles);
+  {
+    long long start = row_prefix;
+    int ti = tile_prefix;
+    for (int g = g0; g < g1; g++) {
+      long long end = start + max(group_sizes[g], 0);
+      int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
+      int local = g - group_offset;
+      int kind = (local >= 0 && local < G_local) ? local : -1;
+      for (int r = s; r < e; r += BM) {
+        TileInfo t;
+        t.group = kind;
+        t.row0 = r;
+        t.nrows = min(BM, e - r);
+        t.pad = 0;
+        tiles[ti++] = t;
+      }
+      start = end;
+    }
+  }
+  const int covered = min(total_rows, M);
+  const int tail = (M - covered + BM - 1) / BM;
+  for (int i = tid; i < tail; i += kMapThreads) {
+    TileInfo t;
+    t.group = -1;
+    t.row0 = covered + i * BM;
+    t.nrows = min(BM, M - t.row0);
+    t.pad = 0;
+    tiles[total_tiles + i] = t;
+  }
+  if (tid == 0) header[0] = total_tiles + tail;
+}
+
+// ---------------------------------------------------------------------------------------
+// Tiled MFMA kernel
+// ---------------------------------------------------------------------------------------
+
+enum { OP_BF16 = 0, OP_I8 = 1 };                 // MFMA operand type (= LDS element type)
+enum { BSRC_SAME = 0, BSRC_I8 = 1, BSRC_I4 = 2 };  // weight format in HBM
+
+struct TiledParams {
+  const uint8_t* lhs;        // [M, K] elements of the MFMA operand type
+  const float* lhs_scale;    // [M] or NULL
+  const uint8_t* rhs;        // [G, N, K] (INT4: K/2 bytes per row)
+  const uint8_t* rhs_up;     // same, or NULL
+  const void* rhs_scale;     // f32 [G, N] (per channel) | bf16 [G, N, nkg] (INT4)
+  const void* rhs_up_scale;
+  const int32_t* header;
+  const TileInfo* tiles;
+  uint16_t* out;  // [M, N] bf16
+  int M, K, N;
+  int max_m_tiles, tiles_n;
+  int act;
+  float act_limit;
+};
+
+__device__ __forceinline__ uint32_t i8x2_to_bf16x2(int lo, int hi) {
+  // |value| <= 128 is exact in bf16, so truncating the f32 is the conversion
+  return (__float_as_uint((float)lo) >> 16) | (__float_as_uint((float)hi) & 0xffff0000u);
+}
+
+template <int OP_, int BSRC_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, bool GLU_>
+struct TiledCfg {
+  static constexpr int OP = OP_, BSRC = BSRC_, BM = BM_, BN = BN_, BKB = BKB_;
+  static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+  static constexpr bool GLU = GLU_;
+  static constexpr int THREADS = WAVES_M * WAVES_N * kWave;
+  static constexpr int ESZ = OP == OP_I8 ? 1 : 2;
+  static constexpr int BK = BKB / ESZ;
+  static constexpr int LDR = BKB + 16;  // LDS row stride in bytes (pad keeps b128 reads conflict free)
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int KSUB = BKB / 32;  // MFMA steps per stage (32 bytes of K per row each)
+  static constexpr int A_CPR = BKB / 16;
+  static constexpr int A_CH = BM * A_CPR / THREADS;
+  static constexpr int B_CHE = BSRC == BSRC_SAME ? 16 / ESZ : (BSRC == BSRC_I8 ? 16 : 32);  // elems per 16B
+  static constexpr int B_CPR = BK / B_CHE;
+  static constexpr int B_CH = BN * B_CPR / THREADS;
+  static constexpr int STAGE = (BM + BN) * LDR;
+  static constexpr int LDS_BYTES = 2 * STAGE;
+  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tiling");
+  static_assert(!GLU || TN % 2 == 0, "GLU needs gate and up tiles in every wave");
+  static_assert(BM * A_CPR % THREADS == 0 && A_CH >= 1, "A chunks");
+  static_assert(BN * B_CPR % THREADS == 0 && B_CH >= 1, "B chunks");
+  static_assert(BSRC == BSRC_SAME || OP == OP_BF16, "weight-only formats feed the bf16 MFMA");
+};
+
+template <typename C>
+__global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  constexpr int OP = C::OP;
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
+
+  // ---- block -> (m-tile, n-tile): contiguous ids per XCD, then GSM x tiles_n super-rows ----
+  int m_idx, n_idx;
+  {
+    const int nb = gridDim.x, pid = blockIdx.x;
+    const int q = nb / 8, rem = nb % 8, xcd = pid % 8, loc = pid / 8;
+    const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+    constexpr int GSM = 4;
+    const int width = GSM * p.tiles_n;
+    const int sg = logical / width, first_m = sg * GSM;
+    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    m_idx = first_m + (logical % width) % gsz;
+    n_idx = (logical % width) / gsz;
+  }
+  if (m_idx >= p.header[0]) return;
+  const TileInfo tile = p.tiles[m_idx];
+  const int n0 = n_idx * C::OUT_BN;
+  const int N = p.N, K = p.K;
+
+  if (tile.group < 0) {  // rows of no local group: zeros
+    constexpr int QPR = C::OUT_BN / 4;
+    for (int i = tid; i < tile.nrows * QPR; i += C::THREADS) {
+      int r = i / QPR, c = n0 + (i % QPR) * 4;
+      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  // ---- global -> register staging -------------------------------------------------------
+  const size_t a_row_bytes = (size_t)K * C::ESZ;
+  const size_t b_row_bytes = C::BSRC == BSRC_I4 ? (size_t)K / 2 : (size_t)K * (C::BSRC == BSRC_I8 ? 1 : C::ESZ);
+  const uint8_t* a_ptr[C::A_CH];
+  int a_k[C::A_CH], a_lds[C::A_CH];
+#pragma unroll
+  for (int i = 0; i < C::A_CH; i++) {
+    int c = tid + i * C::THREADS;
+    int r = c / C::A_CPR, col = c % C::A_CPR;
+    int gr = tile.row0 + min(r, tile.nrows - 1);
+    a_ptr[i] = p.lhs + (size_t)gr * a_row_bytes + col * 16;
+    a_k[i] = col * (16 / C::ESZ);
+    a_lds[i] = r * C::LDR + col * 16;
+  }
+  const uint8_t* b_ptr[C::B_CH];
+  int b_k[C::B_CH], b_lds[C::B_CH], b_n[C::B_CH];
+  bool b_up[C::B_CH];
+#pragma unroll
+  for (int i = 0; i < C::B_CH; i++) {
+    int c = tid + i * C::THREADS;
+    int vr = c / C::B_CPR, col = c % C::B_CPR;
+    bool up = C::GLU && vr >= C::BN / 2;
+    int n = n0 + (up ? vr - C::BN / 2 : vr);
+    n = min(n, N - 1);
+    const uint8_t* base = up ? p.rhs_up : p.rhs;
+    b_ptr[i] = base + ((size_t)tile.group * N + n) * b_row_bytes + col * 16;
+    b_k[i] = col * C::B_CHE;
+    b_lds[i] = C::BM * C::LDR + vr * C::LDR + col * C::B_CHE * C::ESZ;
+    b_n[i] = n;
+    b_up[i] = up;
+  }
+
+  uint4 a_reg[C::A_CH], b_reg[C::B_CH];
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+  auto load_stage = [&](int kt) {
+    const int k0 = kt * C::BK;
+#pragma unroll
+    for (int i = 0; i < C::A_CH; i++)
+      a_reg[i] = (k0 + a_k[i] < K) ? *(const uint4*)(a_ptr[i] + (size_t)k0 * C::ESZ) : zero4;
+#pragma unroll
+    for (int i = 0; i < C::B_CH; i++) {
+      const size_t off = C::BSRC == BSRC_I4 ? (size_t)k0 / 2 : (size_t)k0 * (C::BSRC == BSRC_I8 ? 1 : C::ESZ);
+      b_reg[i] = (k0 + b_k[i] < K) ? *(const uint4*)(b_ptr[i] + off) : zero4;
+    }
+  };
+
+  auto store_stage = [&](int buf, int kt) {
+    uint8_t* s = smem + buf * C::STAGE;
+#pragma unroll
+    for (int i = 0; i < C::A_CH; i++) *(uint4*)(s + a_lds[i]) = a_reg[i];
+#pragma unroll
+    for (int i = 0; i < C::B_CH; i++) {
+      if (C::BSRC == BSRC_SAME) {
+        *(uint4*)(s + b_lds[i]) = b_reg[i];
+      } else if (C::BSRC == BSRC_I8) {
+        const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
+        uint32_t o[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          int v = (int)w[j];
+          o[2 * j] = i8x2_to_bf16x2((v << 24) >> 24, (v << 16) >> 24);
+          o[2 * j + 1] = i8x2_to_bf16x2((v << 8) >> 24, v >> 24);
+        }
+        *(uint4*)(s + b_lds[i]) = make_uint4(o[0], o[1], o[2], o[3]);
+        *(uint4*)(s + b_lds[i] + 16) = make_uint4(o[4], o[5], o[6], o[7]);
+      } else {  // BSRC_I4: 32 values of one 128-wide scale group
+        const int kk = kt * C::BK + b_k[i];
+        const int nkg = (K + 127) / 128;
+        const uint16_t* sc = (const uint16_t*)(b_up[i] ? p.rhs_up_scale : p.rhs_scale);
+        const float scale = kk < K ? bf16_bits_to_f32(sc[((size_t)tile.group * N + b_n[i]) * nkg + kk / 128]) : 0.f;
+        const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
+        uint32_t o[16];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+          for (int h = 0; h < 4; h++) {
+            int lo = (int)((w[j] >> (8 * h)) & 0xf) - 8;
+            int hi = (int)((w[j] >> (8 * h + 4)) & 0xf) - 8;
+            o[4 * j + h] = pack_bf16x2((float)lo * scale, (float)hi * scale);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          *(uint4*)(s + b_lds[i] + 16 * j) = make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+      }
+    }
+  };
+
+  // ---- accumulators ---------------------------------------------------------------------
+  typedef typename std::conditional<OP == OP_I8, v16i, v16f>::type acc_t;
+  acc_t acc[C::TN][C::TM];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++)
+#pragma unroll
+    for (int i = 0; i < C::TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
+
+  // LDS row of the wave's j-th weight tile: with GLU the first TN/2 tiles are gate channels,
+  // the rest the matching up channels.
+  int b_row[C::TN];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++) {
+    if (C::GLU) {
+      constexpr int H = C::TN / 2;
+      int jj = j < H ? j : j - H;
+      b_row[j] = (j < H ? 0 : C::BN / 2) + wn * (C::WN / 2) + jj * 32;
+    } else {
+      b_row[j] = wn * C::WN + j * 32;
+    }
+  }
+  const int frag_off = (lane % 32) * C::LDR + (lane / 32) * 16;
+
+  auto compute_stage = [&](int buf) {
+    const uint8_t* sa = smem + buf * C::STAGE + (wm * C::WM) * C::LDR + frag_off;
+    const uint8_t* sb = smem + buf * C::STAGE + C::BM * C::LDR + frag_off;
+#pragma unroll
+    for (int ks = 0; ks < C::KSUB; ks++) {
+      v4i af[C::TM], bf[C::TN];
+#pragma unroll
+      for (int i = 0; i < C::TM; i++) af[i] = *(const v4i*)(sa + i * 32 * C::LDR + ks * 32);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) bf[j] = *(const v4i*)(sb + b_row[j] * C::LDR + ks * 32);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int i = 0; i < C::TM; i++) {
+          if constexpr (OP == OP_I8) {
+            acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
+          } else {
+            acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(v8bf, bf[j]), __builtin_bit_cast(v8bf, af[i]), acc[j][i], 0, 0, 0);
+          }
+        }
+    }
+  };
+
+  // ---- main loop: one barrier per stage --------------------------------------------------
+  const int nk = (K + C::BK - 1) / C::BK;
+  load_stage(0);
+  store_stage(0, 0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt++) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) load_stage(kt + 1);
+    compute_stage(cur);
+    if (kt + 1 < nk) store_stage(cur ^ 1, kt + 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: scales, activation, bf16 store ------------------------------------------
+  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
+  const int half = lane / 32;
+#pragma unroll
+  for (int i = 0; i < C::TM; i++) {
+    const int lr = wm * C::WM + i * 32 + (lane % 32);
+    const bool row_ok = lr < tile.nrows;
+    const int gr = tile.row0 + (row_ok ? lr : 0);
+    const float sa = p.lhs_scale ? p.lhs_scale[gr] : 1.0f;
+#pragma unroll
+    for (int j = 0; j < NT_OUT; j++) {
+      const int nbase = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN) + j * 32;
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = nbase + 8 * q + 4 * half;
+        if (!row_ok || n >= N) continue;
+        float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
+        if (C::BSRC != BSRC_I4 && p.rhs_scale) {
+          const float4 t = *(const float4*)((const float*)p.rhs_scale + (size_t)tile.group * N + n);
+          sg[0] = t.x; sg[1] = t.y; sg[2] = t.z; sg[3] = t.w;
+          if (C::GLU) {
+            const float4 u = *(const float4*)((const float*)p.rhs_up_scale + (size_t)tile.group * N + n);
+            su[0] = u.x; su[1] = u.y; su[2] = u.z; su[3] = u.w;
+          }
+        }
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          float g = (float)acc[j][i][4 * q + r] * (sa * sg[r]);
+          if (C::GLU) {
+            float u = (float)acc[j + NT_OUT][i][4 * q + r] * (sa * su[r]);
+            v[r] = glu_act(g, u, p.act, p.act_limit);
+          } else {
+            v[r] = g;
+          }
+        }
+        *(uint2*)(p.out + (size_t)gr * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Block-scaled fp8 for few rows per expert.  One wave = 16 output channels x (16*MT) rows x all K.
+// Weights and activations are read straight from global memory (activations hit in L2: every
+// wave of a tile reads the same rows); nothing is shared between waves, so there are no barriers.
+// ---------------------------------------------------------------------------------------
+
+struct SkinnyParams {
+  const uint8_t* lhs;      // [M, K] fp8
+  const float* lhs_scale;  // [M, K/128]
+  const uint8_t* rhs;      // [G, N, K] fp8
+  const uint8_t* rhs_up;
+  const float* rhs_scale;  // [G, ceil(N/128), K/128]
+  const float* rhs_up_scale;
+  const int32_t* header;
+  const TileInfo* tiles;
+  uint16_t* out;
+  int M, K, N;
+  int n_blocks;  // blocks along N (64 channels each)
+  int act;
+  float act_limit;
+};
+
+__device__ __forceinline__ v8i load32(const uint8_t* p) {
+  const uint4 a = *(const uint4*)p, b = *(const uint4*)(p + 16);
+  v8i r;
+  r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
+  r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+  return r;
+}
+
+template <int MT, bool GLU>
+__global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams p) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int j = lane % 16, kq = lane / 16;
+  const int m_idx = blockIdx.x / p.n_blocks;
+  if (m_idx >= p.header[0]) return;
+  const TileInfo tile = p.tiles[m_idx];
+  const int N = p.N, K = p.K;
+  const int n16 = (blockIdx.x % p.n_blocks) * 64 + wave * 16;
+  if (n16 >= N) return;
+
+  if (tile.group < 0) {
+    for (int i = lane; i < tile.nrows * 4; i += kWave) {
+      int r = i / 4, c = n16 + (i % 4) * 4;
+      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  const int nkb = K / 128;
+  const int nnb = (N + 127) / 128;
+  const int nw = min(n16 + j, N - 1);
+  const size_t wrow = ((size_t)tile.group * N + nw) * K + kq * 32;
+  const uint8_t* wp = p.rhs + wrow;
+  const uint8_t* up = GLU ? p.rhs_up + wrow : nullptr;
+  const size_t srow = ((size_t)tile.group * nnb + n16 / 128) * nkb;
+  const float* wsp = p.rhs_scale + srow;
+  const float* usp = GLU ? p.rhs_up_scale + srow : nullptr;
+  const uint8_t* ap[MT];
+  const float* asp[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int gr = tile.row0 + min(mt * 16 + j, tile.nrows - 1);
+    ap[mt] = p.lhs + (size_t)gr * K + kq * 32;
+    asp[mt] = p.lhs_scale + (size_t)gr * nkb;
+  }
+  v4f acc_g[MT], acc_u[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    acc_g[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+    acc_u[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+  }
+  const v4f zero = {0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 4
+  for (int kb = 0; kb < nkb; kb++) {
+    const v8i wf = load32(wp + (size_t)kb * 128);
+    const float ws = wsp[kb];
+    v8i uf;
+    float us = 0.f;
+    if (GLU) {
+      uf = load32(up + (size_t)kb * 128);
+      us = usp[kb];
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      const v8i af = load32(ap[mt] + (size_t)kb * 128);
+      const float as = asp[mt][kb];
+      const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, zero, 0, 0, 0, 127, 0, 127);
+      const float sg = as * ws;
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc_g[mt][r] = fmaf(pg[r], sg, acc_g[mt][r]);
+      if (GLU) {
+        const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf, af, zero, 0, 0, 0, 127, 0, 127);
+        const float su = as * us;
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc_u[mt][r] = fmaf(pu[r], su, acc_u[mt][r]);
+      }
+    }
+  }
+
+  const int n = n16 + 4 * kq;
+  if (n >= N) return;
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int lr = mt * 16 + j;
+    if (lr >= tile.nrows) continue;
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) v[r] = GLU ? glu_act(acc_g[mt][r], acc_u[mt][r], p.act, p.act_limit) : acc_g[mt][r];
+    *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+
+template <typename C>
+static int launch_tiled(const TiledParams& p0, int M, int G_total, hipStream_t s) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gmm_tiled_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "gmm: cannot reserve %d bytes of LDS: %s", C::LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  TiledParams p = p0;
+  p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
+  p.tiles_n = cdiv(p.N, C::OUT_BN);
+  const long long blocks = (long long)p.max_m_tiles * p.tiles_n;
+  if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  gmm_tiled_kernel<C><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
+  return check_launch("gmm_tiled_kernel");
+}
+
+template <int OP, int BSRC, bool GLU>
+static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* bm_out, bool dry, hipStream_t s) {
+  // rows per expert on average decides the m-tile: full 256-row tiles for prefill, 64 otherwise
+  const bool big = (long long)M >= 128LL * G_total;
+  *bm_out = big ? 256 : 64;
+  if (dry) return MOE_OK;
+  if (big) return launch_tiled<TiledCfg<OP, BSRC, 256, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
+  return launch_tiled<TiledCfg<OP, BSRC, 64, 256, 128, 1, 4, GLU>>(p, M, G_total, s);
+}
+
+template <int OP, int BSRC>
+static int launch_tiled_glu(const TiledParams& p, bool glu, int M, int G_total, int* bm_out, bool dry, hipStream_t s) {
+  return glu ? launch_tiled_by_rows<OP, BSRC, true>(p, M, G_total, bm_out, dry, s)
+             : launch_tiled_by_rows<OP, BSRC, false>(p, M, G_total, bm_out, dry, s);
+}
+
+template <int MT>
+static int launch_skinny(const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s) {
+  const long long blocks = (long long)max_tiles * p.n_blocks;
+  if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  if (glu)
+    gmm_fp8_skinny_kernel<MT, true><<<(unsigned)blocks, 256, 0, s>>>(p);
+  else
+    gmm_fp8_skinny_kernel<MT, false><<<(unsigned)blocks, 256, 0, s>>>(p);
+  return check_launch("gmm_fp8_skinny_kernel");
+}
+
+}  // namespace moe
+
+using namespace moe;
+
+extern "C" {
+
+size_t moe_gmm_workspace_bytes(int M, int num_groups_total) {
+  if (M < 0 || num_groups_total <= 0) return 0;
+  return 16 + (size_t)max_tiles_for(M, num_groups_total, 16) * sizeof(TileInfo);
+}
+
+int moe_gmm(const moe_gmm_args* a, void* stream) {
+  if (!a) return fail(MOE_ERR_INVALID_ARG, "gmm: NULL args");
+  if (a->struct_size != sizeof(moe_gmm_args)) return fail(MOE_ERR_INVALID_ARG, "gmm: struct_size %zu != %zu", a->struct_size, sizeof(moe_gmm_args));
+  if (!a->lhs || !a->rhs || !a->group_sizes || !a->out || !a->workspace) return fail(MOE_ERR_INVALID_ARG, "gmm: NULL pointer");
+  if (a->M < 0 || a->K <= 0 || a->N <= 0 || a->num_groups_total <= 0 || a->num_groups_local <= 0 || a->group_offset < 0)
+    return fail(MOE_ERR_INVALID_ARG, "gmm: bad sizes M=%d K=%d N=%d G=%d/%d", a->M, a->K, a->N, a->num_groups_local, a->num_groups_total);
+  if (a->workspace_bytes < moe_gmm_workspace_bytes(a->M, a->num_groups_total)) return fail(MOE_ERR_WORKSPACE, "gmm: workspace too small");
+  const bool glu = a->rhs_up != nullptr;
+  if (glu && a->act == MOE_ACT_NONE) return fail(MOE_ERR_INVALID_ARG, "gmm: rhs_up needs an activation");
+  if (!glu && a->act != MOE_ACT_NONE) return fail(MOE_ERR_INVALID_ARG, "gmm: activation needs rhs_up");
+  if (a->act < MOE_ACT_NONE || a->act > MOE_ACT_SILU_CLIP) return fail(MOE_ERR_INVALID_ARG, "gmm: bad act %d", a->act);
+  if (a->N % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: N %% 8 != 0 (N=%d)", a->N);
+  if (a->M == 0) return MOE_OK;
+  const uintptr_t align = (uintptr_t)a->lhs | (uintptr_t)a->rhs | (uintptr_t)a->rhs_up | (uintptr_t)a->out |
+                          (uintptr_t)a->rhs_scale | (uintptr_t)a->rhs_up_scale;
+  if (align & 15) return fail(MOE_ERR_UNSUPPORTED, "gmm: pointers must be 16-byte aligned");
+
+  hipStream_t s = (hipStream_t)stream;
+  int32_t* header = (int32_t*)a->workspace;
+  TileInfo* tiles = (TileInfo*)((uint8_t*)a->workspace + 16);
+
+  const int L = a->lhs_dtype, R = a->rhs_dtype;
+  int bm = 0;
+
+  if (L == MOE_FP8_E4M3 && R == MOE_FP8_E4M3) {
+    if (a->lhs_scale_block_k != 128 || a->rhs_scale_block_k != 128 || a->rhs_scale_block_n != 128 || !a->lhs_scale || !a->rhs_scale || (glu && !a->rhs_up_scale))
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs 1x128 lhs scales and 128x128 rhs scales");
+    if (a->K % 128 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs K %% 128 == 0 (K=%d)", a->K);
+    const long long avg = (long long)a->M / a->num_groups_total;
+    const int mt = avg <= 16 ? 1 : (avg <= 32 ? 2 : 4);
+    bm = 16 * mt;
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, header, tiles);
+    SkinnyParams p;
+    p.lhs = (const uint8_t*)a->lhs; p.lhs_scale = a->lhs_scale;
+    p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
+    p.rhs_scale = (const float*)a->rhs_scale; p.rhs_up_scale = (const float*)a->rhs_up_scale;
+    p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
+    p.M = a->M; p.K = a->K; p.N = a->N; p.n_blocks = cdiv(a->N, 64);
+    p.act = a->act; p.act_limit = a->act_limit;
+    const int mx = max_tiles_for(a->M, a->num_groups_total, bm);
+    if (mt == 1) return launch_skinny<1>(p, glu, mx, s);
+    if (mt == 2) return launch_skinny<2>(p, glu, mx, s);
+    return launch_skinny<4>(p, glu, mx, s);
+  }
+
+  TiledParams p;
+  p.lhs = (const uint8_t*)a->lhs; p.lhs_scale = nullptr;
+  p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
+  p.rhs_scale = a->rhs_scale; p.rhs_up_scale = a->rhs_up_scale;
+  p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
+  p.M = a->M; p.K = a->K; p.N = a->N; p.max_m_tiles = 0; p.tiles_n = 0;
+  p.act = a->act; p.act_limit = a->act_limit;
+
+  enum { V_NONE, V_BF16, V_W8, V_W4, V_I8 } variant = V_NONE;
+  if (L == MOE_BF16 && R == MOE_BF16) {
+    if (a->K % 8) return fail(MOE_ERR_UNSUPPORTED, "gmm: bf16 needs K %% 8 == 0");
+    p.rhs_scale = p.rhs_up_scale = nullptr;
+    variant = V_BF16;
+  } else if (L == MOE_BF16 && R == MOE_INT8) {
+    if (!a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || a->rhs_scale_block_k != 0)
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: int8 weights need per-channel f32 scales [G, N]");
+    if (a->K % 16) return fail(MOE_ERR_UNSUPPORTED, "gmm: int8 weights need K %% 16 == 0");
+    variant = V_W8;
+  } else if (L == MOE_BF16 && R == MOE_INT4) {
+    if (!a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || a->rhs_scale_block_k != 128)
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need bf16 group-128 scales [G, N, ceil(K/128)]");
+    if (a->K % 32) return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need K %% 32 == 0");
+    variant = V_W4;
+  } else if (L == MOE_INT8 && R == MOE_INT8) {
+    if (!a->lhs_scale || a->lhs_scale_block_k != 0 || !a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || a->rhs_scale_block_k != 0)
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: int8 x int8 needs per-row lhs scales [M] and per-channel rhs scales [G, N]");
+    if (a->K % 16) return fail(MOE_ERR_UNSUPPORTED, "gmm: int8 needs K %% 16 == 0");
+    p.lhs_scale = a->lhs_scale;
+    variant = V_I8;
+  } else {
+    return fail(MOE_ERR_UNSUPPORTED, "gmm: lhs_dtype %d x rhs_dtype %d", L, R);
+  }
+
+  // dry run to learn the m-tile, then build the tile list and launch
+  const int M = a->M, G = a->num_groups_total;
+  launch_tiled_by_rows<OP_BF16, BSRC_SAME, false>(p, M, G, &bm, true, s);
+  tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
+  switch (variant) {
+    case V_BF16: return launch_tiled_glu<OP_BF16, BSRC_SAME>(p, glu, M, G, &bm, false, s);
+    case V_W8: return launch_tiled_glu<OP_BF16, BSRC_I8>(p, glu, M, G, &bm, false, s);
+    case V_W4: return launch_tiled_glu<OP_BF16, BSRC_I4>(p, glu, M, G, &bm, false, s);
+    case V_I8: return launch_tiled_glu<OP_I8, BSRC_SAME>(p, glu, M, G, &bm, false, s);
+    default: break;
+  }
+  return fail(MOE_ERR_UNSUPPORTED, "gmm: no kernel");
+}
+
+}  // extern "C"

@@ -1,0 +1,571 @@
+// Routing, sort-by-expert, row gather (+ activation quantisation), unpermute+combine.
+// All of these are HBM/latency-bound integer and byte work: one wavefront per token for
+// top-k, a three-launch stable counting sort for the permutation, 16-byte coalesced
+// row copies for the gathers.
+
+#include <limits.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "moe_common.h"
+
+namespace moe {
+
+static thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return MOE_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// Top-k routing: one wavefront per token, lane l owns experts l, l+64, ...
+// ---------------------------------------------------------------------------------------
+
+constexpr int kRouteMaxE = 512;
+constexpr int kRouteVpl = kRouteMaxE / kWave;  // values per lane
+constexpr int kRouteWaves = 4;
+
+// (value, index) order of lax.top_k as adopted here: larger value first, lower index first.
+__device__ __forceinline__ bool better(float av, int ai, float bv, int bi) {
+  return av > bv || (av == bv && ai < bi);
+}
+
+__device__ __forceinline__ void wave_argmax(float& bv, int& bi) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ov = __shfl_xor(bv, o);
+    int oi = __shfl_xor(bi, o);
+    if (better(ov, oi, bv, bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
+    const float* __restrict__ logits, const float* __restrict__ pre_bias, int T, int E, int k,
+    int mode, int norm, int round_bf16, float scaling, int n_groups, int topk_groups,
+    float* __restrict__ w_out, int32_t* __restrict__ idx_out) {
+  __shared__ float s_row[kRouteWaves][kRouteMaxE];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int t_raw = blockIdx.x * kRouteWaves + wave;
+  const bool active = t_raw < T;
+  const int t = active ? t_raw : T - 1;
+  const float* row = logits + (size_t)t * E;
+
+  float v[kRouteVpl];
+  unsigned taken = 0;
+#pragma unroll
+  for (int j = 0; j < kRouteVpl; j++) {
+    int e = lane + kWave * j;
+    v[j] = e < E ? row[e] : -INFINITY;
+    if (e >= E) taken |= 1u << j;
+  }
+
+  if (n_groups > 0) {
+    // expert_group_mask: group score = sum of the group's two best scores; keep the best
+    // topk_groups groups, everything else becomes -inf (still selectable, as in jnp.where).
+    const int gs = E / n_groups;
+#pragma unroll
+    for (int j = 0; j < kRouteVpl; j++) {
+      int e = lane + kWave * j;
+      if (e < E) s_row[wave][e] = v[j];
+    }
+    __syncthreads();
+    float score = -INFINITY;
+    int gi = INT_MAX;
+    if (lane < n_groups) {
+      float b1 = -INFINITY, b2 = -INFINITY;
+      for (int i = 0; i < gs; i++) {
+        float x = s_row[wave][lane * gs + i];
+        if (x > b1) {
+          b2 = b1;
+          b1 = x;
+        } else if (x > b2) {
+          b2 = x;
+        }
+      }
+      score = b1 + b2;
+      gi = lane;
+    }
+    unsigned long long sel = 0;
+    bool mine_taken = lane >= n_groups;
+    for (int r = 0; r < topk_groups; r++) {
+      float bv = mine_taken ? -INFINITY : score;
+      int bi = mine_taken ? INT_MAX : gi;
+      wave_argmax(bv, bi);
+      if (bi < n_groups) sel |= 1ull << bi;
+      if (bi == lane) mine_taken = true;
+    }
+#pragma unroll
+    for (int j = 0; j < kRouteVpl; j++) {
+      int e = lane + kWave * j;
+      if (e < E && !((sel >> (e / gs)) & 1ull)) v[j] = -INFINITY;
+    }
+  }
+
+  float myv = 0.f;
+  int myi = 0;
+  for (int r = 0; r < k; r++) {
+    float bv = -INFINITY;
+    int bi = INT_MAX;
+#pragma unroll
+    for (int j = 0; j < kRouteVpl; j++) {
+      if (!((taken >> j) & 1u)) {
+        int e = lane + kWave * j;
+        if (better(v[j], e, bv, bi)) {
+          bv = v[j];
+          bi = e;
+        }
+      }
+    }
+    wave_argmax(bv, bi);
+    if (bi == INT_MAX) bi = 0;  // only reachable with NaN scores
+    if (lane == r) {
+      myv = bv;
+      myi = bi;
+    }
+    if ((bi & (kWave - 1)) == lane) taken |= 1u << (bi >> 6);
+  }
+
+  float w;
+  if (mode == MOE_ROUTE_DEEPSEEK) {
+    w = lane < k ? pre_bias[(size_t)t * E + myi] : 0.f;
+    if (norm) {
+      float s = wave_sum(w);
+      w = w / (s + 1e-20f);
+    }
+    w *= scaling;
+  } else {
+    float mx = __shfl(myv, 0);
+    float ex = lane < k ? expf(myv - mx) : 0.f;
+    float s = wave_sum(ex);
+    w = ex / s;
+    if (round_bf16) w = round_bf16_fn(w);
+    if (norm) {
+      float s2 = wave_sum(lane < k ? w : 0.f);
+      if (round_bf16) s2 = round_bf16_fn(s2);
+      w = w / s2;
+      if (round_bf16) w = round_bf16_fn(w);
+    }
+  }
+  if (active && lane < k) {
+    w_out[(size_t)t * k + lane] = w;
+    idx_out[(size_t)t * k + lane] = myi;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Stable counting sort of the flattened expert ids.
+//   pass 1: per-wave-segment histograms; pass 2: exclusive scan over segments and experts;
+//   pass 3: each wave re-reads its segment and ranks equal ids with ballots, in index order.
+// ---------------------------------------------------------------------------------------
+
+constexpr int kSortWaves = 4;
+constexpr int kSortRounds = 4;
+constexpr int kSortSeg = kSortRounds * kWave;    // entries per wave
+constexpr int kSortChunk = kSortSeg * kSortWaves;  // entries per block
+constexpr int kSortMaxE = 512;
+
+__device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
+
+__global__ __launch_bounds__(kSortWaves* kWave) void sort_hist_kernel(
+    const int32_t* __restrict__ flat, int M, int E, int32_t* __restrict__ seg_hist) {
+  __shared__ int cnt[kSortWaves][kSortMaxE];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  for (int e = lane; e < E; e += kWave) cnt[wave][e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kSortChunk + wave * kSortSeg;
+#pragma unroll
+  for (int r = 0; r < kSortRounds; r++) {
+    int i = base + r * kWave + lane;
+    if (i < M) atomicAdd(&cnt[wave][clamp_expert(flat[i], E)], 1);
+  }
+  __syncthreads();
+  int32_t* dst = seg_hist + (size_t)(blockIdx.x * kSortWaves + wave) * E;
+  for (int e = lane; e < E; e += kWave) dst[e] = cnt[wave][e];
+}
+
+__global__ __launch_bounds__(kSortMaxE) void sort_scan_kernel(int32_t* __restrict__ seg_hist,
+                                                              int nseg, int E,
+                                                              int32_t* __restrict__ group_sizes,
+                                                              int32_t* __restrict__ expert_off) {
+  __shared__ int tot[kSortMaxE];
+  const int e = threadIdx.x;
+  int running = 0;
+  if (e < E) {
+    for (int s = 0; s < nseg; s++) {
+      int c = seg_hist[(size_t)s * E + e];
+      seg_hist[(size_t)s * E + e] = running;
+      running += c;
+    }
+    group_sizes[e] = running;
+  }
+  tot[e] = e < E ? running : 0;
+  __syncthreads();
+  // inclusive Hillis-Steele scan over experts
+  for (int o = 1; o < kSortMaxE; o <<= 1) {
+    int add = e >= o ? tot[e - o] : 0;
+    __syncthreads();
+    tot[e] += add;
+    __syncthreads();
+  }
+  if (e < E) expert_off[e] = tot[e] - running;
+}
+
+__global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
+    const int32_t* __restrict__ flat, int M, int E, int ebits,
+    const int32_t* __restrict__ seg_hist, const int32_t* __restrict__ expert_off,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
+    int32_t* __restrict__ sorted_experts) {
+  __shared__ int run[kSortWaves][kSortMaxE];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int32_t* seg = seg_hist + (size_t)(blockIdx.x * kSortWaves + wave) * E;
+  for (int e = lane; e < E; e += kWave) run[wave][e] = expert_off[e] + seg[e];
+  __syncthreads();
+  const int base = blockIdx.x * kSortChunk + wave * kSortSeg;
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  for (int r = 0; r < kSortRounds; r++) {
+    const int i = base + r * kWave + lane;
+    const bool valid = i < M;
+    const int e = valid ? clamp_expert(flat[i], E) : 0;
+    unsigned long long mask = __ballot(valid);
+    for (int b = 0; b < ebits; b++) {
+      const bool bit = (e >> b) & 1;
+      const unsigned long long bal = __ballot(valid && bit);
+      mask &= bit ? bal : ~bal;
+    }
+    const int rank = __popcll(mask & lt);
+    const int cnt = __popcll(mask);
+    const int start = valid ? run[wave][e] : 0;
+    __builtin_amdgcn_wave_barrier();
+    if (valid && rank == cnt - 1) run[wave][e] = start + cnt;
+    __builtin_amdgcn_wave_barrier();
+    if (valid) {
+      const int dest = start + rank;
+      perm[dest] = i;
+      if (inv_perm) inv_perm[i] = dest;
+      if (sorted_experts) sorted_experts[dest] = e;
+    }
+  }
+}
+
+__global__ void invert_perm_kernel(const int32_t* __restrict__ perm, int M,
+                                   int32_t* __restrict__ inv) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < M) {
+    int p = perm[i];
+    if (p >= 0 && p < M) inv[p] = i;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Row gather with optional quantisation: one 256-thread block per output row, the row is
+// held in registers between the absmax pass and the quantise pass (one HBM read).
+// ---------------------------------------------------------------------------------------
+
+constexpr int kGqThreads = 256;
+constexpr int kGqMaxChunks = 8;  // 16-byte chunks per thread -> d <= 256*8*8
+
+enum { GQ_COPY = 0, GQ_INT8_ROW = 1, GQ_FP8_BLK128 = 2 };
+
+__device__ __forceinline__ void unpack8(const uint4& u, float f[8]) {
+  f[0] = bf16_bits_to_f32(u.x & 0xffffu);
+  f[1] = bf16_bits_to_f32(u.x >> 16);
+  f[2] = bf16_bits_to_f32(u.y & 0xffffu);
+  f[3] = bf16_bits_to_f32(u.y >> 16);
+  f[4] = bf16_bits_to_f32(u.z & 0xffffu);
+  f[5] = bf16_bits_to_f32(u.z >> 16);
+  f[6] = bf16_bits_to_f32(u.w & 0xffffu);
+  f[7] = bf16_bits_to_f32(u.w >> 16);
+}
+
+__device__ __forceinline__ float absmax8(const uint4& u) {
+  float f[8];
+  unpack8(u, f);
+  float m = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(f[i]));
+  return m;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(kGqThreads) void gather_rows_kernel(
+    const uint4* __restrict__ x, const int32_t* __restrict__ row_idx, int idx_div, int d,
+    void* __restrict__ out, float* __restrict__ scale) {
+  __shared__ float s_red[kGqThreads / kWave];
+  const int r = blockIdx.x;
+  const int src = row_idx ? row_idx[r] / idx_div : r;
+  const int nch = d / 8;
+  const uint4* xrow = x + (size_t)src * nch;
+  uint4 regs[kGqMaxChunks];
+#pragma unroll
+  for (int c = 0; c < kGqMaxChunks; c++) {
+    int ci = threadIdx.x + c * kGqThreads;
+    regs[c] = ci < nch ? xrow[ci] : make_uint4(0, 0, 0, 0);
+  }
+
+  if (MODE == GQ_COPY) {
+    uint4* orow = (uint4*)out + (size_t)r * nch;
+#pragma unroll
+    for (int c = 0; c < kGqMaxChunks; c++) {
+      int ci = threadIdx.x + c * kGqThreads;
+      if (ci < nch) orow[ci] = regs[c];
+    }
+    return;
+  }
+
+  if (MODE == GQ_INT8_ROW) {
+    float m = 0.f;
+#pragma unroll
+    for (int c = 0; c < kGqMaxChunks; c++) m = fmaxf(m, absmax8(regs[c]));
+    m = wave_max(m);
+    if (threadIdx.x % kWave == 0) s_red[threadIdx.x / kWave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float sc = m / 127.0f;
+    if (threadIdx.x == 0) scale[r] = sc;
+    uint2* orow = (uint2*)out + (size_t)r * nch;
+#pragma unroll
+    for (int c = 0; c < kGqMaxChunks; c++) {
+      int ci = threadIdx.x + c * kGqThreads;
+      if (ci < nch) {
+        float f[8];
+        unpack8(regs[c], f);
+        uint32_t b[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          float q = sc == 0.f ? 0.f : rintf(f[i] / sc);
+          q = fminf(fmaxf(q, -127.f), 127.f);
+          b[i] = (uint32_t)((int)q) & 0xffu;
+        }
+        uint2 o;
+        o.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        o.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+        orow[ci] = o;
+      }
+    }
+    return;
+  }
+
+  if (MODE == GQ_FP8_BLK128) {
+    // a 128-element block is 16 consecutive chunks == 16 consecutive lanes
+    const int nkb = (d + 127) / 128;
+    uint2* orow = (uint2*)out + (size_t)r * nch;
+#pragma unroll
+    for (int c = 0; c < kGqMaxChunks; c++) {
+      int ci = threadIdx.x + c * kGqThreads;
+      float m = absmax8(regs[c]);
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      const float sc = m / 448.0f;
+      if (ci < nch) {
+        if ((threadIdx.x & 15) == 0) scale[(size_t)r * nkb + ci / 16] = sc;
+        float f[8];
+        unpack8(regs[c], f);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          float q = sc == 0.f ? 0.f : f[i] / sc;
+          f[i] = fminf(fmaxf(q, -448.f), 448.f);
+        }
+        int lo = 0, hi = 0;
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+        orow[ci] = make_uint2((uint32_t)lo, (uint32_t)hi);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Unpermute + weighted combine: one block per token, f32 accumulation over the k rows.
+// ---------------------------------------------------------------------------------------
+
+constexpr int kCombineMaxK = 16;
+
+__global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ y,
+                                                      const int32_t* __restrict__ inv_perm,
+                                                      const float* __restrict__ weights, int k,
+                                                      int d, uint4* __restrict__ out) {
+  __shared__ int s_row[kCombineMaxK];
+  __shared__ float s_w[kCombineMaxK];
+  const int t = blockIdx.x;
+  if (threadIdx.x < k) {
+    s_row[threadIdx.x] = inv_perm[(size_t)t * k + threadIdx.x];
+    s_w[threadIdx.x] = weights ? weights[(size_t)t * k + threadIdx.x] : 1.0f;
+  }
+  __syncthreads();
+  const int nch = d / 8;
+  for (int ci = threadIdx.x; ci < nch; ci += blockDim.x) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < k; s++) {
+      uint4 u = y[(size_t)s_row[s] * nch + ci];
+      float f[8];
+      unpack8(u, f);
+      const float w = s_w[s];
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] = fmaf(w, f[i], acc[i]);
+    }
+    uint4 o;
+    o.x = pack_bf16x2(acc[0], acc[1]);
+    o.y = pack_bf16x2(acc[2], acc[3]);
+    o.z = pack_bf16x2(acc[4], acc[5]);
+    o.w = pack_bf16x2(acc[6], acc[7]);
+    out[(size_t)t * nch + ci] = o;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// [G, K, N] -> [G, N, K] re-layout through a padded LDS tile.
+// ---------------------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in, int K, int N,
+                                                        T* __restrict__ out) {
+  __shared__ T tile[64][65];
+  const size_t g = blockIdx.z;
+  const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+  for (int i = ty; i < 64; i += 4) {
+    int kk = k0 + i, nn = n0 + tx;
+    if (kk < K && nn < N) tile[i][tx] = in[(g * K + kk) * N + nn];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int nn = n0 + i, kk = k0 + tx;
+    if (kk < K && nn < N) out[(g * N + nn) * K + kk] = tile[tx][i];
+  }
+}
+
+}  // namespace moe
+
+using namespace moe;
+
+extern "C" {
+
+const char* moe_last_error(void) { return g_err; }
+int moe_abi_version(void) { return 1; }
+
+int moe_route_topk(const float* gate_logits, const float* pre_bias_logits, int T, int E, int k,
+                   int mode, int norm_topk_prob, int weights_round_bf16,
+                   float routed_scaling_factor, int n_routing_groups, int topk_routing_group,
+                   float* topk_weights, int32_t* topk_idx, void* stream) {
+  if (!gate_logits || !topk_weights || !topk_idx) return fail(MOE_ERR_INVALID_ARG, "route: NULL pointer");
+  if (T < 0 || E <= 0 || k <= 0) return fail(MOE_ERR_INVALID_ARG, "route: bad sizes T=%d E=%d k=%d", T, E, k);
+  if (E > kRouteMaxE || k > 16 || k > E) return fail(MOE_ERR_UNSUPPORTED, "route: need k<=16, k<=E<=512 (E=%d k=%d)", E, k);
+  if (mode != MOE_ROUTE_SOFTMAX_TOPK && mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "route: bad mode %d", mode);
+  if (mode == MOE_ROUTE_DEEPSEEK && !pre_bias_logits) return fail(MOE_ERR_INVALID_ARG, "route: DeepSeek mode needs pre_bias_logits");
+  int ng = n_routing_groups > 0 ? n_routing_groups : 0;
+  if (ng > 0) {
+    if (mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "route: routing groups need DeepSeek mode");
+    if (ng > kWave || E % ng != 0 || E / ng < 2 || topk_routing_group <= 0 || topk_routing_group > ng)
+      return fail(MOE_ERR_UNSUPPORTED, "route: bad routing groups %d/%d for E=%d", ng, topk_routing_group, E);
+  }
+  if (T == 0) return MOE_OK;
+  route_topk_kernel<<<cdiv(T, kRouteWaves), kRouteWaves * kWave, 0, (hipStream_t)stream>>>(
+      gate_logits, pre_bias_logits, T, E, k, mode, norm_topk_prob, weights_round_bf16,
+      routed_scaling_factor, ng, topk_routing_group, topk_weights, topk_idx);
+  return check_launch("route_topk_kernel");
+}
+
+size_t moe_sort_workspace_bytes(int T, int k, int E) {
+  if (T < 0 || k <= 0 || E <= 0) return 0;
+  size_t M = (size_t)T * k;
+  size_t nseg = (size_t)cdiv((int)M, kSortChunk) * kSortWaves;
+  return (nseg * E + E) * sizeof(int32_t) + 256;
+}
+
+int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,
+                       int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  if (!topk_idx || !perm || !group_sizes || !workspace) return fail(MOE_ERR_INVALID_ARG, "sort: NULL pointer");
+  if (T < 0 || k <= 0 || E <= 0) return fail(MOE_ERR_INVALID_ARG, "sort: bad sizes");
+  if (E > kSortMaxE) return fail(MOE_ERR_UNSUPPORTED, "sort: E=%d > %d", E, kSortMaxE);
+  if ((long long)T * k > INT_MAX / 2) return fail(MOE_ERR_UNSUPPORTED, "sort: T*k too large");
+  if (workspace_bytes < moe_sort_workspace_bytes(T, k, E)) return fail(MOE_ERR_WORKSPACE, "sort: workspace too small");
+  const int M = T * k;
+  const int nblk = cdiv(M, kSortChunk);
+  const int nseg = nblk * kSortWaves;
+  int32_t* seg_hist = (int32_t*)workspace;
+  int32_t* expert_off = seg_hist + (size_t)nseg * E;
+  hipStream_t s = (hipStream_t)stream;
+  int ebits = 0;
+  while ((1 << ebits) < E) ebits++;
+  if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, seg_hist);
+  sort_scan_kernel<<<1, kSortMaxE, 0, s>>>(seg_hist, nseg, E, group_sizes, expert_off);
+  if (nblk > 0)
+    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, seg_hist, expert_off,
+                                                          perm, inv_perm, sorted_experts);
+  return check_launch("sort_by_expert");
+}
+
+int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_out, int d,
+                    int out_dtype, int block_k, void* out, float* scale, void* stream) {
+  if (!x || !out) return fail(MOE_ERR_INVALID_ARG, "gather: NULL pointer");
+  if (R_out < 0 || d <= 0 || idx_div <= 0) return fail(MOE_ERR_INVALID_ARG, "gather: bad sizes");
+  if (d % 8 != 0 || d > kGqThreads * kGqMaxChunks * 8) return fail(MOE_ERR_UNSUPPORTED, "gather: need d%%8==0 and d<=16384 (d=%d)", d);
+  if (R_out == 0) return MOE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const uint4* xs = (const uint4*)x;
+  if (out_dtype == MOE_BF16) {
+    gather_rows_kernel<GQ_COPY><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, d, out, scale);
+  } else if (out_dtype == MOE_INT8) {
+    if (!scale || block_k != 0) return fail(MOE_ERR_UNSUPPORTED, "gather: int8 needs per-row scale (block_k=0)");
+    gather_rows_kernel<GQ_INT8_ROW><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, d, out, scale);
+  } else if (out_dtype == MOE_FP8_E4M3) {
+    if (!scale || block_k != 128) return fail(MOE_ERR_UNSUPPORTED, "gather: fp8 needs block_k=128 scales");
+    gather_rows_kernel<GQ_FP8_BLK128><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, d, out, scale);
+  } else {
+    return fail(MOE_ERR_UNSUPPORTED, "gather: out_dtype %d", out_dtype);
+  }
+  return check_launch("gather_rows_kernel");
+}
+
+int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv_perm,
+                          const float* weights, int T, int k, int d, void* out, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  if (!y || !out || (!perm && !inv_perm)) return fail(MOE_ERR_INVALID_ARG, "combine: NULL pointer");
+  if (T < 0 || k <= 0 || d <= 0) return fail(MOE_ERR_INVALID_ARG, "combine: bad sizes");
+  if (k > kCombineMaxK || d % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "combine: need k<=16, d%%8==0");
+  if (T == 0) return MOE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const int M = T * k;
+  if (!inv_perm) {
+    if (!workspace || workspace_bytes < (size_t)M * sizeof(int32_t)) return fail(MOE_ERR_WORKSPACE, "combine: workspace too small");
+    invert_perm_kernel<<<cdiv(M, 256), 256, 0, s>>>(perm, M, (int32_t*)workspace);
+    inv_perm = (const int32_t*)workspace;
+  }
+  combine_kernel<<<T, 256, 0, s>>>((const uint4*)y, inv_perm, weights, k, d, (uint4*)out);
+  return check_launch("combine_kernel");
+}
+
+int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem_bytes, void* rhs_gnk,
+                      void* stream) {
+  if (!rhs_gkn || !rhs_gnk) return fail(MOE_ERR_INVALID_ARG, "transpose: NULL pointer");
+  if (G <= 0 || K <= 0 || N <= 0) return fail(MOE_ERR_INVALID_ARG, "transpose: bad sizes");
+  if (G > 65535 || cdiv(K, 64) > 65535) return fail(MOE_ERR_UNSUPPORTED, "transpose: grid too large");
+  dim3 grid(cdiv(N, 64), cdiv(K, 64), G);
+  hipStream_t s = (hipStream_t)stream;
+  if (elem_bytes == 1)
+    transpose_kernel<uint8_t><<<grid, 256, 0, s>>>((const uint8_t*)rhs_gkn, K, N, (uint8_t*)rhs_gnk);
+  else if (elem_bytes == 2)
+    transpose_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)rhs_gkn, K, N, (uint16_t*)rhs_gnk);
+  else
+    return fail(MOE_ERR_UNSUPPORTED, "transpose: elem_bytes %d", elem_bytes);
+  return check_launch("transpose_kernel");
+}
+
+}  // extern "C"

@@ -1,0 +1,201 @@
+"""Thin torch-tensor wrappers over the C ABI (one function per entry point).
+
+Each wrapper checks device, dtype, contiguity and shapes on the host before the launch,
+allocates outputs/workspaces with torch and enqueues on torch's current stream.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from maxtext_amd import _lib
+from maxtext_amd._lib import (MOE_BF16, MOE_FP8_E4M3, MOE_INT4, MOE_INT8, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_SOFTMAX_TOPK)
+
+_DTYPE_CODE = {torch.bfloat16: MOE_BF16, torch.int8: MOE_INT8, torch.float8_e4m3fn: MOE_FP8_E4M3}
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, ndim=None):
+  if not isinstance(t, torch.Tensor):
+    raise TypeError(f"{name} must be a torch.Tensor")
+  if not t.is_cuda:
+    raise ValueError(f"{name} must live on the GPU (the MoE path has no CPU implementation)")
+  if not t.is_contiguous():
+    raise ValueError(f"{name} must be contiguous")
+  if dtype is not None and t.dtype != dtype:
+    raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+  if ndim is not None and t.dim() != ndim:
+    raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+
+
+def route_topk(gate_logits, pre_bias_logits=None, *, k, mode="softmax_topk", norm_topk_prob=False,
+               weights_round_bf16=True, routed_scaling_factor=1.0, n_routing_groups=-1, topk_routing_group=-1):
+  """-> (weights [T,k] f32, indices [T,k] int32)."""
+  _need(gate_logits, "gate_logits", torch.float32, 2)
+  t, e = gate_logits.shape
+  if mode == "deepseek":
+    _need(pre_bias_logits, "pre_bias_logits", torch.float32, 2)
+    if pre_bias_logits.shape != gate_logits.shape:
+      raise ValueError("pre_bias_logits must match gate_logits")
+    code = MOE_ROUTE_DEEPSEEK
+  elif mode == "softmax_topk":
+    code = MOE_ROUTE_SOFTMAX_TOPK
+  else:
+    raise ValueError(f"unknown routing mode {mode!r}")
+  w = torch.empty((t, k), dtype=torch.float32, device=gate_logits.device)
+  idx = torch.empty((t, k), dtype=torch.int32, device=gate_logits.device)
+  lib = _lib.load()
+  st = lib.moe_route_topk(_lib.ptr(gate_logits), _lib.ptr(pre_bias_logits) if mode == "deepseek" else None, t, e, k, code,
+                          int(bool(norm_topk_prob)), int(bool(weights_round_bf16)), float(routed_scaling_factor),
+                          int(n_routing_groups), int(topk_routing_group), _lib.ptr(w), _lib.ptr(idx), _lib.current_stream())
+  _lib.check(st, "moe_route_topk")
+  return w, idx
+
+
+def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True):
+  """-> (perm [M], inv_perm [M], group_sizes [E], sorted_experts [M] or None), all int32."""
+  _need(topk_idx, "topk_idx", torch.int32, 2)
+  t, k = topk_idx.shape
+  m = t * k
+  dev = topk_idx.device
+  lib = _lib.load()
+  perm = torch.empty((m,), dtype=torch.int32, device=dev)
+  inv = torch.empty((m,), dtype=torch.int32, device=dev)
+  gs = torch.empty((num_experts,), dtype=torch.int32, device=dev)
+  se = torch.empty((m,), dtype=torch.int32, device=dev) if want_sorted_experts else None
+  nbytes = lib.moe_sort_workspace_bytes(t, k, num_experts)
+  ws = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=dev)
+  st = lib.moe_sort_by_expert(_lib.ptr(topk_idx), t, k, num_experts, _lib.ptr(perm), _lib.ptr(inv), _lib.ptr(gs),
+                              _lib.ptr(se), _lib.ptr(ws), ws.numel(), _lib.current_stream())
+  _lib.check(st, "moe_sort_by_expert")
+  return perm, inv, gs, se
+
+
+def gather_rows(x, row_idx=None, idx_div=1, *, out_dtype=torch.bfloat16, block_k=0, num_rows=None):
+  """Row gather (+ per-row int8 / 1x128 fp8 quantisation).  -> out or (q, scale)."""
+  _need(x, "x", torch.bfloat16, 2)
+  d = x.shape[1]
+  if row_idx is not None:
+    _need(row_idx, "row_idx", torch.int32, 1)
+    r_out = row_idx.shape[0]
+  else:
+    r_out = x.shape[0] if num_rows is None else num_rows
+  out = torch.empty((r_out, d), dtype=out_dtype, device=x.device)
+  scale = None
+  if out_dtype == torch.int8:
+    scale = torch.empty((r_out,), dtype=torch.float32, device=x.device)
+  elif out_dtype == torch.float8_e4m3fn:
+    scale = torch.empty((r_out, (d + block_k - 1) // block_k), dtype=torch.float32, device=x.device)
+  lib = _lib.load()
+  st = lib.moe_gather_rows(_lib.ptr(x), _lib.ptr(row_idx), int(idx_div), r_out, d, _DTYPE_CODE[out_dtype], int(block_k),
+                           _lib.ptr(out), _lib.ptr(scale), _lib.current_stream())
+  _lib.check(st, "moe_gather_rows")
+  return out if scale is None else (out, scale)
+
+
+def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None):
+  """out[t] = sum_s weights[t,s] * y[inv_perm[t*k+s]]  (f32 accumulate, bf16 out)."""
+  _need(y, "y", torch.bfloat16, 2)
+  m, d = y.shape
+  if m % k:
+    raise ValueError("rows of y must be a multiple of k")
+  t = m // k
+  if weights is not None:
+    _need(weights, "weights", torch.float32)
+    if weights.numel() != m:
+      raise ValueError("weights must have T*k elements")
+  ws = None
+  if inv_perm is None:
+    _need(perm, "perm", torch.int32, 1)
+    if perm.numel() != m:
+      raise ValueError("perm must have T*k elements")
+    ws = torch.empty((m,), dtype=torch.int32, device=y.device)
+  else:
+    _need(inv_perm, "inv_perm", torch.int32, 1)
+    if inv_perm.numel() != m:
+      raise ValueError("inv_perm must have T*k elements")
+  out = torch.empty((t, d), dtype=torch.bfloat16, device=y.device)
+  lib = _lib.load()
+  st = lib.moe_unpermute_combine(_lib.ptr(y), _lib.ptr(perm), _lib.ptr(inv_perm), _lib.ptr(weights), t, k, d, _lib.ptr(out),
+                                 _lib.ptr(ws), 0 if ws is None else ws.numel() * 4, _lib.current_stream())
+  _lib.check(st, "moe_unpermute_combine")
+  return out
+
+
+def transpose_rhs(rhs_gkn):
+  """[G, K, N] -> [G, N, K] for 1- or 2-byte element types."""
+  _need(rhs_gkn, "rhs", None, 3)
+  g, k, n = rhs_gkn.shape
+  out = torch.empty((g, n, k), dtype=rhs_gkn.dtype, device=rhs_gkn.device)
+  lib = _lib.load()
+  st = lib.moe_transpose_rhs(_lib.ptr(rhs_gkn), g, k, n, rhs_gkn.element_size(), _lib.ptr(out), _lib.current_stream())
+  _lib.check(st, "moe_transpose_rhs")
+  return out
+
+
+def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
+            rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
+            group_offset=0, out=None):
+  """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4: uint8 [G,N,K/2])."""
+  _need(lhs, "lhs", None, 2)
+  _need(rhs, "rhs", None, 3)
+  _need(group_sizes, "group_sizes", torch.int32, 1)
+  m, kdim = lhs.shape
+  g_local, n, kr = rhs.shape
+  if lhs.dtype not in _DTYPE_CODE:
+    raise TypeError(f"lhs dtype {lhs.dtype} not supported")
+  if rhs_dtype is None:
+    if rhs.dtype not in _DTYPE_CODE:
+      raise TypeError(f"rhs dtype {rhs.dtype} needs an explicit rhs_dtype")
+    rhs_dtype = _DTYPE_CODE[rhs.dtype]
+  if rhs_dtype == MOE_INT4:
+    if rhs.dtype != torch.uint8 or kr * 2 != kdim:
+      raise ValueError("INT4 rhs must be uint8 [G, N, K/2]")
+  elif kr != kdim:
+    raise ValueError(f"rhs K {kr} != lhs K {kdim}")
+  for name, t in (("rhs_up", rhs_up),):
+    if t is not None:
+      _need(t, name, rhs.dtype, 3)
+      if t.shape != rhs.shape:
+        raise ValueError("rhs_up must match rhs")
+  nkb_r = 1 if rhs_scale_block_k == 0 else (kdim + rhs_scale_block_k - 1) // rhs_scale_block_k
+  nnb = (n + rhs_scale_block_n - 1) // rhs_scale_block_n
+  for name, t in (("rhs_scale", rhs_scale), ("rhs_up_scale", rhs_up_scale)):
+    if t is not None:
+      _need(t, name)
+      want = torch.bfloat16 if rhs_dtype == MOE_INT4 else torch.float32
+      if t.dtype != want or t.numel() != g_local * nnb * nkb_r:
+        raise ValueError(f"{name} must be {want} with {g_local}x{nnb}x{nkb_r} elements, got {t.dtype} {tuple(t.shape)}")
+  if lhs_scale is not None:
+    _need(lhs_scale, "lhs_scale", torch.float32)
+    nkb_l = 1 if lhs_scale_block_k == 0 else (kdim + lhs_scale_block_k - 1) // lhs_scale_block_k
+    if lhs_scale.numel() != m * nkb_l:
+      raise ValueError(f"lhs_scale must have {m}x{nkb_l} elements")
+  if out is None:
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=lhs.device)
+  else:
+    _need(out, "out", torch.bfloat16, 2)
+    if out.shape != (m, n):
+      raise ValueError("out must be [M, N]")
+  lib = _lib.load()
+  g_total = group_sizes.numel()
+  wsb = lib.moe_gmm_workspace_bytes(m, g_total)
+  ws = torch.empty((max(wsb, 16),), dtype=torch.uint8, device=lhs.device)
+  a = _lib.GmmArgs()
+  a.struct_size = ctypes.sizeof(_lib.GmmArgs)
+  a.lhs, a.lhs_scale = lhs.data_ptr(), (lhs_scale.data_ptr() if lhs_scale is not None else None)
+  a.rhs, a.rhs_scale = rhs.data_ptr(), (rhs_scale.data_ptr() if rhs_scale is not None else None)
+  a.rhs_up = rhs_up.data_ptr() if rhs_up is not None else None
+  a.rhs_up_scale = rhs_up_scale.data_ptr() if rhs_up_scale is not None else None
+  a.group_sizes, a.out = group_sizes.data_ptr(), out.data_ptr()
+  a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+  a.M, a.K, a.N = m, kdim, n
+  a.num_groups_total, a.num_groups_local, a.group_offset = g_total, g_local, int(group_offset)
+  a.lhs_dtype, a.rhs_dtype = _DTYPE_CODE[lhs.dtype], rhs_dtype
+  a.lhs_scale_block_k, a.rhs_scale_block_n, a.rhs_scale_block_k = int(lhs_scale_block_k), int(rhs_scale_block_n), int(rhs_scale_block_k)
+  a.act = _lib.ACT_BY_NAME[act]
+  a.act_limit = float(act_limit)
+  st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
+  _lib.check(st, "moe_gmm")
+  return out

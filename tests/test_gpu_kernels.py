@@ -1,0 +1,343 @@
+"""GPU parity: every C-ABI entry point against the CPU oracle on identical seeded inputs.
+
+Index outputs (top-k indices, perm, group_sizes, sorted_experts, quantised values) are compared
+bit-exactly; floating-point outputs with max|got-want| / max|want| <= 1e-2 (bf16 outputs, f32
+accumulation), the tolerance BASELINE.json states.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def relerr(got: torch.Tensor, want: torch.Tensor) -> float:
+  got, want = got.detach().float().cpu(), want.detach().float().cpu()
+  return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+@pytest.fixture(scope="module")
+def K():
+  from maxtext_amd import kernels
+
+  assert torch.cuda.is_available()
+  return kernels
+
+
+def cuda(x):
+  if isinstance(x, np.ndarray):
+    x = torch.from_numpy(x)
+  return x.cuda().contiguous()
+
+
+# ---------------------------------------------------------------- routing
+
+
+@pytest.mark.parametrize("t,e,k", [(1, 8, 2), (257, 8, 2), (100, 128, 8), (64, 256, 8), (33, 32, 4), (5, 512, 16), (19, 60, 6)])
+def test_route_softmax_topk(K, t, e, k):
+  rng = np.random.default_rng(t * 1000 + e)
+  logits = rng.standard_normal((t, e)).astype(np.float32)
+  for norm in (False, True):
+    w, idx = K.route_topk(cuda(logits), k=k, norm_topk_prob=norm)
+    ow, oidx = O.get_topk(logits, k=k, norm_topk_prob=norm)
+    np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+    # weights are bf16-rounded: a 1-ulp f32 difference in exp may move a value by one bf16 ulp
+    np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=2.0**-7, atol=1e-6)
+
+
+def test_route_ties_lower_index_first(K):
+  logits = np.zeros((4, 16), np.float32)
+  logits[1, [3, 9, 12]] = 2.0
+  logits[2] = -np.inf
+  logits[3, 5] = np.inf
+  w, idx = K.route_topk(cuda(logits), k=4)
+  _, oidx = O.get_topk(logits, k=4)
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+  assert idx[0].tolist() == [0, 1, 2, 3] and idx[1].tolist() == [3, 9, 12, 0]
+
+
+@pytest.mark.parametrize("t,e,k,groups,topg", [(256, 256, 8, -1, -1), (64, 64, 6, 8, 3), (2, 16, 4, 4, 2)])
+def test_route_deepseek(K, t, e, k, groups, topg):
+  rng = np.random.default_rng(7 + e)
+  raw = rng.standard_normal((t, e)).astype(np.float32)
+  scores = (1.0 / (1.0 + np.exp(-raw))).astype(np.float32)
+  bias = (rng.standard_normal(e) * 0.1).astype(np.float32)
+  gate = (scores + bias).astype(np.float32)
+  w, idx = K.route_topk(cuda(gate), cuda(scores), k=k, mode="deepseek", norm_topk_prob=True, routed_scaling_factor=2.5,
+                        n_routing_groups=groups, topk_routing_group=topg)
+  ow, oidx = O.get_topk(gate, scores, k=k, mode="deepseek", routed_scaling_factor=2.5, n_routing_groups=groups,
+                        topk_routing_group=topg)
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+  np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=1e-5)
+
+
+def test_route_deepseek_reference_known_answer(K):
+  # tests/unit/moe_test.py:293-326
+  gate = np.array(
+      [[0.20, 0.10, 0.05, 0.10, 0.10, 0.60, 0.30, 0.10, 0.80, 0.01, 0.01, 0.01, 0.05, 0.80, 0.20, 0.10],
+       [0.68, 0.20, 0.06, 0.03, 0.32, 0.10, 0.05, 0.02, 0.65, 0.20, 0.04, 0.01, 0.32, 0.10, 0.05, 0.02]], np.float32)
+  pre = gate - 0.5
+  w, idx = K.route_topk(cuda(gate), cuda(pre), k=4, mode="deepseek", norm_topk_prob=False, routed_scaling_factor=1.0,
+                        n_routing_groups=4, topk_routing_group=2)
+  expect = np.array([[13, 5, 6, 14], [0, 8, 1, 9]])
+  np.testing.assert_array_equal(idx.cpu().numpy(), expect)
+  np.testing.assert_allclose(w.cpu().numpy(), np.take_along_axis(pre, expect, -1), rtol=1e-6)
+
+
+# ---------------------------------------------------------------- sort / permute
+
+
+def _zipf_selection(rng, t, e, k, s=1.2):
+  logits = rng.standard_normal((t, e)) - s * np.log(np.arange(1, e + 1)) * 3.0
+  return np.argsort(-logits, -1, kind="stable")[:, :k].astype(np.int32)
+
+
+@pytest.mark.parametrize("t,e,k", [(1, 8, 2), (7, 8, 2), (128, 8, 2), (1000, 128, 8), (4099, 256, 8), (2048, 32, 4), (513, 512, 3)])
+def test_sort_by_expert_bit_exact(K, t, e, k):
+  rng = np.random.default_rng(e + t)
+  sel = _zipf_selection(rng, t, e, k) if e >= 32 else np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  perm, inv, gs, se = K.sort_by_expert(cuda(sel), e)
+  x = torch.zeros(t, 8, dtype=torch.bfloat16)
+  _, operm, ogs, ose = O.permute(x, sel, e)
+  np.testing.assert_array_equal(perm.cpu().numpy(), operm)
+  np.testing.assert_array_equal(gs.cpu().numpy(), ogs)
+  np.testing.assert_array_equal(se.cpu().numpy(), ose)
+  np.testing.assert_array_equal(inv.cpu().numpy(), np.argsort(operm, kind="stable").astype(np.int32))
+  if e >= 128:
+    assert (ogs == 0).any()  # the skewed selection leaves experts empty
+
+
+@pytest.mark.parametrize("d", [8, 512, 2048, 4096, 7168, 14336])
+def test_gather_rows_copy_bit_exact(K, d):
+  rng = np.random.default_rng(d)
+  t, k, e = 50, 4, 16
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  x = torch.randn(t, d, generator=torch.Generator().manual_seed(d)).to(torch.bfloat16)
+  perm, _, _, _ = K.sort_by_expert(cuda(sel), e)
+  got = K.gather_rows(cuda(x), perm, k)
+  want, _, _, _ = O.permute(x, sel, e)
+  assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("d", [64, 512, 4096, 14336])
+def test_gather_rows_int8_quant(K, d):
+  g = torch.Generator().manual_seed(d + 1)
+  x = torch.randn(37, d, generator=g).to(torch.bfloat16)
+  x[3] = 0
+  idx = torch.randint(0, 37, (80,), generator=g).to(torch.int32)
+  q, s = K.gather_rows(cuda(x), cuda(idx), 1, out_dtype=torch.int8)
+  oq, os_ = O.quantize_rows_int8(x[idx.long()])
+  assert torch.equal(s.cpu(), os_)
+  assert torch.equal(q.cpu(), oq)
+
+
+@pytest.mark.parametrize("d", [128, 2048, 7168, 2880])
+def test_gather_rows_fp8_block_quant(K, d):
+  g = torch.Generator().manual_seed(d + 2)
+  x = (torch.randn(29, d, generator=g) * 3).to(torch.bfloat16)
+  x[5, 128:256] = 0 if d > 256 else x[5, 128:256]
+  q, s = K.gather_rows(cuda(x), None, 1, out_dtype=torch.float8_e4m3fn, block_k=128)
+  oq, os_ = O.quantize_fp8_blocks(x, 1, 128)
+  assert torch.equal(s.cpu(), os_)
+  assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8))
+
+
+@pytest.mark.parametrize("t,k,d", [(1, 2, 512), (300, 2, 4096), (64, 8, 7168), (100, 4, 2880), (33, 9, 64)])
+def test_unpermute_combine(K, t, k, d):
+  rng = np.random.default_rng(t + d)
+  e = 16
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  y = torch.randn(t * k, d, generator=torch.Generator().manual_seed(t)).to(torch.bfloat16)
+  w = rng.random((t, k)).astype(np.float32)
+  perm, inv, _, _ = K.sort_by_expert(cuda(sel), e)
+  want = O.unpermute(y, perm.cpu().numpy(), w, k)
+  got = K.unpermute_combine(cuda(y), cuda(w), k=k, inv_perm=inv)
+  assert relerr(got, want) <= 2.0**-8
+  got2 = K.unpermute_combine(cuda(y), cuda(w), k=k, perm=perm)  # inverse rebuilt from perm
+  assert torch.equal(got, got2)
+  # unweighted sum (sort_activations.py:98-121)
+  got3 = K.unpermute_combine(cuda(y), None, k=k, inv_perm=inv)
+  assert relerr(got3, O.unroute_sum(y.float(), sel)) <= 2.0**-8
+
+
+def test_combine_exact_on_integers(K):
+  # integer-valued bf16 inputs make the f32 accumulation exact (trick of tests/gather_reduce_sc_test.py:68)
+  rng = np.random.default_rng(0)
+  t, k, d, e = 200, 8, 256, 64
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  y = torch.from_numpy(rng.integers(-8, 9, (t * k, d)).astype(np.float32)).to(torch.bfloat16)
+  w = rng.integers(0, 3, (t, k)).astype(np.float32)
+  perm, inv, _, _ = K.sort_by_expert(cuda(sel), e)
+  got = K.unpermute_combine(cuda(y), cuda(w), k=k, inv_perm=inv)
+  assert torch.equal(got.cpu(), O.unpermute(y, perm.cpu().numpy(), w, k))
+
+
+def test_transpose_rhs(K):
+  w = torch.randint(-128, 128, (3, 200, 136), dtype=torch.int8)
+  assert torch.equal(K.transpose_rhs(cuda(w)).cpu(), w.transpose(1, 2).contiguous())
+  wb = torch.randn(2, 70, 264).to(torch.bfloat16)
+  assert torch.equal(K.transpose_rhs(cuda(wb)).cpu(), wb.transpose(1, 2).contiguous())
+
+
+# ---------------------------------------------------------------- grouped matmul
+
+# (M, K, N, group_sizes): small-tile (rows/expert < 128) and big-tile (>= 128) dispatch, empty groups,
+# ragged boundaries, rows past the sum, K and N that are not multiples of the tile.
+GMM_SHAPES = [
+    (300, 256, 128, [7, 0, 120, 1, 100, 60]),
+    (64, 512, 264, [64]),
+    (1024, 320, 200, [300, 0, 500, 200]),
+    (1500, 1024, 512, [256, 257, 255, 700]),
+    (520, 2880, 96, [500, 20]),
+]
+
+
+def _gmm_inputs(m, k, n, gs, seed):
+  g = torch.Generator().manual_seed(seed)
+  e = len(gs)
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w = torch.randn(e, k, n, generator=g) * 0.05  # [g, k, n] f32
+  w_up = torch.randn(e, k, n, generator=g) * 0.05
+  return lhs, w, w_up, np.asarray(gs, np.int32)
+
+
+def native(w_gkn):
+  return w_gkn.transpose(1, 2).contiguous()
+
+
+@pytest.mark.parametrize("m,k,n,gs", GMM_SHAPES)
+def test_gmm_bf16(K, m, k, n, gs):
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 1)
+  wb, ub = w.to(torch.bfloat16), w_up.to(torch.bfloat16)
+  got = K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs))
+  want = O.gmm(lhs, wb, gs)
+  assert relerr(got, want) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  got = K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), rhs_up=cuda(native(ub)), act="silu")
+  want = O.apply_ffn_activation(O.gmm(lhs, wb, gs, out_dtype=torch.float32), O.gmm(lhs, ub, gs, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
+@pytest.mark.parametrize("m,k,n,gs", GMM_SHAPES)
+def test_gmm_int8_weight_only(K, m, k, n, gs):
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 2)
+  q, s = O.quantize_weight_int8(w)
+  qu, su = O.quantize_weight_int8(w_up)
+  got = K.gmm_raw(cuda(lhs), cuda(native(q)), cuda(gs), rhs_scale=cuda(s))
+  want = O.gmm(lhs, q, gs, rhs_scale=s)
+  assert relerr(got, want) <= TOL
+  got = K.gmm_raw(cuda(lhs), cuda(native(q)), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(native(qu)), rhs_up_scale=cuda(su), act="silu")
+  want = O.apply_ffn_activation(O.gmm(lhs, q, gs, rhs_scale=s, out_dtype=torch.float32), O.gmm(lhs, qu, gs, rhs_scale=su, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
+@pytest.mark.parametrize("m,k,n,gs", GMM_SHAPES)
+def test_gmm_int8_int8(K, m, k, n, gs):
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 3)
+  q, s = O.quantize_weight_int8(w)
+  qu, su = O.quantize_weight_int8(w_up)
+  lq, ls = O.quantize_rows_int8(lhs)
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s))
+  want = O.gmm(lq, q, gs, lhs_scale=ls, rhs_scale=s)
+  assert relerr(got, want) <= TOL
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s), rhs_up=cuda(native(qu)),
+                  rhs_up_scale=cuda(su), act="silu")
+  want = O.apply_ffn_activation(O.gmm(lq, q, gs, lhs_scale=ls, rhs_scale=s, out_dtype=torch.float32),
+                                O.gmm(lq, qu, gs, lhs_scale=ls, rhs_scale=su, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
+def test_gmm_int8_exact_with_unit_scales(K):
+  # integer operands, unit scales, |sum| < 256: the bf16 output must equal the integer product exactly
+  g = torch.Generator().manual_seed(4)
+  m, k, n = 400, 64, 128
+  gs = np.array([100, 0, 300], np.int32)
+  lq = torch.randint(-1, 2, (m, k), generator=g, dtype=torch.int8)
+  q = torch.randint(-2, 3, (3, k, n), generator=g, dtype=torch.int8)
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(torch.ones(m)), rhs_scale=cuda(torch.ones(3, n)))
+  want = O.gmm(lq, q, gs, out_dtype=torch.float32)
+  assert want.abs().max() < 256
+  assert torch.equal(got.float().cpu(), want)
+
+
+@pytest.mark.parametrize("m,k,n,gs", [(300, 256, 128, [7, 0, 120, 1, 100, 60]), (520, 2880, 96, [500, 20]), (1024, 320 + 64, 200, [300, 0, 500, 200])])
+def test_gmm_int4_weight_only(K, m, k, n, gs):
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 5)
+  q, s = O.quantize_int4_groups(native(w), 128)  # along K: q [g,n,k], scale [g,n,ceil(k/128)]
+  qu, su = O.quantize_int4_groups(native(w_up), 128)
+  s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
+  from maxtext_amd._lib import MOE_INT4
+  got = K.gmm_raw(cuda(lhs), cuda(O.pack_int4(q)), cuda(gs), rhs_scale=cuda(s), rhs_dtype=MOE_INT4, rhs_scale_block_k=128)
+  rhs_scale_v2 = s.float().permute(0, 2, 1)[:, :, None, :]  # [g, nb, 1, n]
+  want = O.gmm(lhs, q.transpose(1, 2), gs, rhs_scale=rhs_scale_v2, quant_block=128)
+  assert relerr(got, want) <= TOL
+  got = K.gmm_raw(cuda(lhs), cuda(O.pack_int4(q)), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(O.pack_int4(qu)), rhs_up_scale=cuda(su),
+                  rhs_dtype=MOE_INT4, rhs_scale_block_k=128, act="silu")
+  up_scale_v2 = su.float().permute(0, 2, 1)[:, :, None, :]
+  want = O.apply_ffn_activation(O.gmm(lhs, q.transpose(1, 2), gs, rhs_scale=rhs_scale_v2, quant_block=128, out_dtype=torch.float32),
+                                O.gmm(lhs, qu.transpose(1, 2), gs, rhs_scale=up_scale_v2, quant_block=128, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
+FP8_SHAPES = [
+    (40, 256, 128, [7, 0, 12, 1, 20]),
+    (256, 1024, 384, [8] * 32),
+    (200, 512, 200, [100, 60, 40]),
+    (300, 384, 256, [5, 290]),
+]
+
+
+@pytest.mark.parametrize("m,k,n,gs", FP8_SHAPES)
+def test_gmm_fp8_block_scaled(K, m, k, n, gs):
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 6)
+  aq, asc = O.quantize_fp8_blocks(lhs, 1, 128)
+  wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)  # [g, n, k], scale [g, n/128, k/128]
+  uq, usc = O.quantize_fp8_blocks(native(w_up), 128, 128)
+
+  def v2(sc):  # -> [g, nb, 1, n]
+    return torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
+
+  got = K.gmm_raw(cuda(aq), cuda(wq), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc), lhs_scale_block_k=128,
+                  rhs_scale_block_n=128, rhs_scale_block_k=128)
+  want = O.gmm(aq, wq, gs, lhs_scale=asc, rhs_scale=v2(wsc), transpose_rhs=True, quant_block=128)
+  assert relerr(got, want) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  got = K.gmm_raw(cuda(aq), cuda(wq), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc), rhs_up=cuda(uq), rhs_up_scale=cuda(usc),
+                  lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128, act="silu")
+  want = O.apply_ffn_activation(
+      O.gmm(aq, wq, gs, lhs_scale=asc, rhs_scale=v2(wsc), transpose_rhs=True, quant_block=128, out_dtype=torch.float32),
+      O.gmm(aq, uq, gs, lhs_scale=asc, rhs_scale=v2(usc), transpose_rhs=True, quant_block=128, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
+def test_gmm_group_offset_and_nan_isolation(K):
+  # non-local groups produce zeros (v2 kernel test :939); a NaN row must not leak into other experts' rows (:592)
+  lhs, w, _, gs = _gmm_inputs(600, 256, 128, [100, 200, 150, 100], 8)
+  wb = w.to(torch.bfloat16)
+  got = K.gmm_raw(cuda(lhs), cuda(native(wb[1:3])), cuda(gs), group_offset=1)
+  want = O.gmm(lhs, wb[1:3], gs, group_offset=1)
+  assert relerr(got, want) <= TOL
+  assert torch.all(got[:100] == 0) and torch.all(got[450:] == 0)
+  lhs_nan = lhs.clone()
+  lhs_nan[100:300] = float("nan")
+  clean = K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs))
+  dirty = K.gmm_raw(cuda(lhs_nan), cuda(native(wb)), cuda(gs))
+  assert torch.equal(clean[:100], dirty[:100]) and torch.equal(clean[300:], dirty[300:])
+  assert torch.isnan(dirty[100:300].float()).all()
+
+
+def test_gmm_argument_errors(K):
+  lhs = torch.zeros(16, 64, dtype=torch.bfloat16).cuda()
+  rhs = torch.zeros(2, 24, 64, dtype=torch.bfloat16).cuda()
+  gs = torch.tensor([8, 8], dtype=torch.int32).cuda()
+  with pytest.raises(RuntimeError):
+    K.gmm_raw(lhs, rhs[:, :20].contiguous(), gs)  # N % 8 != 0
+  with pytest.raises(RuntimeError):
+    K.gmm_raw(lhs, rhs, gs, act="silu")  # activation without rhs_up
+  with pytest.raises(ValueError):
+    K.gmm_raw(lhs.cpu(), rhs, gs)
