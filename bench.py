@@ -1,0 +1,190 @@
+"""Benchmark of the quantized MoE expert path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+
+One step = one pass of the hot path (top-k routing -> sort/permute with activation quantisation
+-> fused wi_0/wi_1 grouped GEMM + SwiGLU -> activation quantisation -> wo grouped GEMM ->
+unpermute + weighted combine) over one batch of synthetic input that is already resident in HBM.
+The default workload is the Mixtral-8x7B-shape int8 prefill layer (8192 tokens, d 4096, f 14336,
+8 experts, top-2).  Prints ONE JSON line.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"int8": 5000.0, "fp8": 5000.0, "bf16": 2500.0}  # dense MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=20)
+  ap.add_argument("--warmup", type=int, default=5)
+  ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+  ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
+  ap.add_argument("--cpu-sample-tokens", type=int, default=None)
+  ap.add_argument("--no-cpu-baseline", action="store_true")
+  return ap.parse_args()
+
+
+def dominant_kernel_model(wl, group_sizes):
+  """Algorithmic work of one launch of the dominant kernel: the fused wi_0/wi_1 grouped GEMM."""
+  cfg = wl.cfg
+  d, f = cfg.emb_dim, cfg.moe_mlp_dim
+  rows = int(group_sizes.sum())
+  nonempty = int((group_sizes > 0).sum())
+  flops = 4.0 * rows * d * f
+  if wl.weight_quant == "fp8":
+    # HBM bound (decode): weights of the non-empty experts + block scales + activations in + out
+    w_bytes = nonempty * 2.0 * d * f
+    s_bytes = nonempty * 2.0 * (d / 128) * (f / 128) * 4 + rows * (d / 128) * 4
+    io_bytes = rows * d * 1.0 + rows * f * 2.0
+    return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
+                name="gmm_fp8_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")
+  op = "int8" if cfg.act_quant == "int8" else "bf16"
+  return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
+              name="gmm_tiled_kernel (wi_0|wi_1 + SwiGLU)", dtype=op)
+
+
+def cpu_baseline(wl, layer, sample_tokens):
+  """The oracle's layer (torch CPU, f32 accumulation) on the first `sample_tokens` tokens of the same
+  workload with the same quantised weights: a reported baseline, timed on this host's cores."""
+  import torch
+
+  from maxtext_amd import synthetic
+  from oracle.layer import oracle_layer
+
+  cfg = wl.cfg
+  t = min(sample_tokens, wl.tokens)
+  trip = lambda qa: (qa.qvalue.cpu(), qa.scale.cpu(), qa.qtype)
+  x = layer["x"][:, :t].cpu()
+  logits = layer["gate_logits"][:, :t].cpu()
+  pre = None if layer["pre_bias_logits"] is None else layer["pre_bias_logits"][:, :t].cpu()
+  w0, w1, wo = trip(layer["wi_0"]), trip(layer["wi_1"]), trip(layer["wo"])
+  torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))))
+  t0 = time.perf_counter()
+  oracle_layer(x, logits, pre, w0, w1, wo, num_experts=cfg.num_experts, k=cfg.num_experts_per_tok, emb_dim=cfg.emb_dim,
+               mlp_dim=cfg.moe_mlp_dim, deepseek=cfg.is_deepseek, routed_scaling_factor=cfg.routed_scaling_factor,
+               norm_topk_prob=cfg.norm_topk_prob, shared_experts=cfg.shared_experts, act_quant=cfg.act_quant,
+               activation=cfg.activation, acc_dtype=torch.float32)
+  dt = time.perf_counter() - t0
+  import dataclasses
+
+  flops = synthetic.layer_flops(dataclasses.replace(wl, tokens=t))
+  return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+              sample=f"first {t} of {wl.tokens} tokens, all experts, same d/f and quantised weights; {dt:.1f} s wall",
+              seconds=dt)
+
+
+def main():
+  args = parse()
+  if args.gpus != 1:
+    print("bench.py measures one GPU: every box of this build has a single MI355X and the expert path has no "
+          "multi-GPU code; run with --gpus 1", file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+
+  from maxtext_amd import _lib, moe, synthetic
+
+  _lib.load()
+  if not torch.cuda.is_available():
+    print("bench.py needs a GPU", file=sys.stderr)
+    sys.exit(2)
+  torch.cuda.set_device(0)
+
+  wl = synthetic.workload(args.workload, args.tokens)
+  cfg = wl.cfg
+  layer = synthetic.make_layer(wl, device="cuda")
+  cls = moe.RoutedAndSharedMoE if cfg.shared_experts else moe.RoutedMoE
+  block = cls(cfg, layer["wi_0"], layer["wi_1"], layer["wo"])
+  routed = block.routed if cfg.shared_experts else block
+  x, logits, pre = layer["x"], layer["gate_logits"], layer["pre_bias_logits"]
+
+  def step():
+    if cfg.shared_experts:
+      return block.sparse_matmul(x, logits, pre)[0]
+    return block.sparse_matmul(x, logits, pre, layer["wi_0"], layer["wi_1"], layer["wo"])[0]
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+
+  routed.profile_events = []
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    out = step()
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+  events = routed.profile_events
+  routed.profile_events = None
+  ms_per_step = elapsed * 1e3 / args.steps
+
+  # group sizes of this batch (read back after the timed region) for the algorithmic work model
+  _, sel = routed.get_topk(logits, pre)
+  gs = torch.bincount(sel.reshape(-1).long(), minlength=cfg.num_experts)
+  if cfg.shared_experts:
+    gs = torch.cat([gs, torch.tensor([wl.tokens], device=gs.device)])
+  gs = gs.cpu().numpy()
+
+  model = dominant_kernel_model(wl, gs)
+  stage_ms = {}
+  for name in ("wi_glu", "wo"):
+    ts = [a.elapsed_time(b) for (n, a, b) in events if n == name]
+    if ts:
+      stage_ms[name] = sum(ts) / len(ts)
+  dom_ms = stage_ms.get("wi_glu")
+  achieved = model["work"] / (dom_ms * 1e-3) / model["scale"] if dom_ms else None
+  roofline = dict(bound=model["bound"], achieved=achieved, peak=model["peak"], unit=model["unit"],
+                  frac=(achieved / model["peak"]) if achieved else None, traffic=None, kernel=model["name"],
+                  kernel_ms=dom_ms)
+
+  flops = synthetic.layer_flops(wl)
+  value = flops / (elapsed / args.steps) / 1e12
+  result = {
+      "metric": "moe_quant_gmm_layer_tflops",
+      "value": value,
+      "unit": "TFLOP/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": ms_per_step,
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": model["dtype"],
+      "data": "synthetic",
+      "config": {
+          "workload": f"{wl.name}: MoE expert layer, {wl.tokens} tokens, d_model {cfg.emb_dim}, d_ff {cfg.moe_mlp_dim}, "
+                      f"{cfg.num_experts} experts top-{cfg.num_experts_per_tok}"
+                      f"{' + 1 shared' if cfg.shared_experts else ''}, {wl.weight_quant} weights, "
+                      f"{cfg.act_quant or 'bf16'} activations, SwiGLU",
+          "tokens": wl.tokens, "d_model": cfg.emb_dim, "d_ff": cfg.moe_mlp_dim, "experts": cfg.num_experts,
+          "top_k": cfg.num_experts_per_tok, "parallelism": "single GPU",
+      },
+      "roofline": roofline,
+      "stage_ms": stage_ms,
+      "layer_gbps": None,
+  }
+  # whole-layer minimum HBM traffic (weights of non-empty experts + activations in/out), for HBM-bound shapes
+  nonempty = int((gs > 0).sum())
+  min_bytes = nonempty * synthetic.weight_bytes_per_expert(wl) + wl.tokens * cfg.emb_dim * 2 * 2
+  result["layer_gbps"] = min_bytes / (elapsed / args.steps) / 1e9
+
+  if not args.no_cpu_baseline:
+    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 256, "c3": 16, "c4": 1024, "c5": 256}[wl.name]
+    del out
+    result["cpu_baseline"] = cpu_baseline(wl, layer, sample)
+  print(json.dumps(result))
+
+
+if __name__ == "__main__":
+  main()

@@ -1,0 +1,232 @@
+"""Host-side mirror of the reference's sparse MoE expert path, driving the HIP kernels.
+
+Mirrors the method surface of RoutedMoE in src/maxtext/layers/moe.py: get_topk (:717),
+permute (:872), unpermute (:1004), apply_ffn_activation (:841, fused into the first GEMM),
+sparse_matmul (:1403) and __call__ (:3143), plus RoutedAndSharedMoE (:3259).  Only the
+single-device dropless `sparse_matmul=True` branch exists here; arrays are torch CUDA tensors.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import torch
+
+from maxtext_amd import kernels, megablox
+from maxtext_amd.quantizations import QArray
+
+
+@dataclasses.dataclass
+class MoEConfig:
+  """The MoE keys of src/maxtext/configs/base.yml:212-298 that the expert path reads."""
+
+  num_experts: int
+  num_experts_per_tok: int
+  emb_dim: int
+  moe_mlp_dim: int
+  model_name: str = "mixtral-8x7b"  # "deepseek3-*" selects DeepSeek routing (moe.py:744)
+  decoder_block: str = "mixtral"  # "gpt_oss" selects the clipped activation (moe.py:844)
+  norm_topk_prob: bool = False
+  routed_scaling_factor: float = 1.0
+  routed_score_func: str = ""  # "sigmoid" for DeepSeek-V3
+  routed_bias: bool = False
+  n_routing_groups: int = -1
+  topk_routing_group: int = -1
+  mlp_activations_limit: float = -1.0
+  float32_weight_sum: bool = True
+  float32_gate_logits: bool = True
+  shared_experts: int = 0
+  # activation quantisation for the grouped GEMMs: None | "int8" | "fp8"
+  act_quant: Optional[str] = None
+
+  @property
+  def is_deepseek(self) -> bool:
+    return self.model_name.startswith(("deepseek3", "deepseek4"))
+
+  @property
+  def activation(self) -> str:
+    if self.decoder_block == "gpt_oss":
+      return "swigluoai"
+    if self.is_deepseek and self.mlp_activations_limit > 0.0:
+      return "silu_clip"
+    return "silu"
+
+
+class RoutedMoE:
+  """Routed experts: top-k routing, permute, three grouped GEMMs with fused SwiGLU, combine.
+
+  Expert weights are held in the kernels' layout [E, N, K] (K contiguous): `wi_0`, `wi_1` are
+  [E, moe_mlp_dim, emb_dim] and `wo` is [E, emb_dim, moe_mlp_dim], each a bf16 tensor or a
+  quantizations.QArray.  `gate_kernel` is [emb_dim, E] (GateLogit, moe.py:247); `gate_bias` [E].
+  """
+
+  def __init__(self, config: MoEConfig, wi_0, wi_1, wo, gate_kernel=None, gate_bias=None):
+    self.config = config
+    self.num_experts = config.num_experts
+    self.num_experts_per_tok = config.num_experts_per_tok
+    self.wi_0, self.wi_1, self.wo = wi_0, wi_1, wo
+    self.gate_kernel, self.gate_bias = gate_kernel, gate_bias
+    # when set to a list, _experts appends (stage, start_event, end_event) recorded on the launch stream
+    self.profile_events = None
+
+  # -- GateLogit.__call__ (moe.py:353-392): upstream of the kernels' boundary -----------------
+  def gate(self, inputs_2d: torch.Tensor):
+    cfg = self.config
+    x = inputs_2d.float() if cfg.float32_gate_logits else inputs_2d
+    out = (x @ self.gate_kernel.to(x.dtype)).float()
+    if cfg.routed_score_func == "sigmoid":
+      out = torch.sigmoid(out)
+    elif cfg.routed_score_func:
+      raise NotImplementedError(cfg.routed_score_func)
+    pre_bias = out if cfg.is_deepseek else None
+    if self.gate_bias is not None:
+      out = out + self.gate_bias.float()
+    return out.contiguous(), pre_bias
+
+  # -- get_topk (moe.py:717-765) ------------------------------------------------------------
+  def get_topk(self, gate_logits: torch.Tensor, pre_bias_logits: Optional[torch.Tensor] = None):
+    cfg = self.config
+    shape = gate_logits.shape[:-1]
+    g2 = gate_logits.reshape(-1, gate_logits.shape[-1]).float().contiguous()
+    if cfg.is_deepseek:
+      p2 = pre_bias_logits.reshape(g2.shape).float().contiguous()
+      w, idx = kernels.route_topk(
+          g2, p2, k=self.num_experts_per_tok, mode="deepseek",
+          norm_topk_prob=cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"),
+          routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups,
+          topk_routing_group=cfg.topk_routing_group)
+    else:
+      w, idx = kernels.route_topk(g2, k=self.num_experts_per_tok, norm_topk_prob=cfg.norm_topk_prob)
+    k = self.num_experts_per_tok
+    return w.reshape(*shape, k), idx.reshape(*shape, k)
+
+  # -- permute (moe.py:872-1002), non-ragged branch -----------------------------------------
+  def permute(self, inputs, gate_logits, pre_bias_logits=None, use_custom_sort_vjp=True, rngs=None,
+              roll_to_expert_id=None, input_ids=None):
+    """-> (sorted_inputs, sorted_selected_experts, weights, group_size, sorted_experts,
+    lb_loss, bias_updates, local_group_size), as moe.py:993-1002."""
+    if roll_to_expert_id is not None or input_ids is not None:
+      raise NotImplementedError("ring-of-experts roll and hash routing are multi-device / DeepSeek-V4 features")
+    b, s, d = inputs.shape
+    x2d = inputs.reshape(b * s, d).contiguous()
+    weights, selected = self.get_topk(gate_logits, pre_bias_logits)
+    sel2d = selected.reshape(b * s, -1).contiguous()
+    perm, inv, group_size, sorted_experts = kernels.sort_by_expert(sel2d, self.num_experts)
+    sorted_inputs = kernels.gather_rows(x2d, perm, self.num_experts_per_tok)
+    self._last_inv_perm = inv
+    return sorted_inputs, perm, weights, group_size, sorted_experts, None, None, None
+
+  # -- unpermute (moe.py:1004-1063), non-ragged branch --------------------------------------
+  def unpermute(self, intermediate, sorted_selected_experts, weights, batch_size, sequence_length,
+                use_custom_sort_vjp=True, group_sizes=None, inv_perm=None):
+    if not self.config.float32_weight_sum:
+      raise NotImplementedError("only float32_weight_sum=True is implemented")
+    k = self.num_experts_per_tok
+    w = weights.reshape(-1, k).float().contiguous()
+    out = kernels.unpermute_combine(intermediate.contiguous(), w, k=k,
+                                    perm=None if inv_perm is not None else sorted_selected_experts,
+                                    inv_perm=inv_perm)
+    return out.reshape(batch_size, sequence_length, -1)
+
+  # -- the three grouped GEMMs: gmm_up + apply_ffn_activation + wo (moe.py:1932-1986, :841, :2226)
+  def _experts(self, sorted_inputs, group_size, w0, w1, wo):
+    cfg = self.config
+    act, limit = cfg.activation, (cfg.mlp_activations_limit if cfg.mlp_activations_limit > 0 else 7.0)
+    ev = self.profile_events
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if ev is not None else None
+    if marks:
+      marks[0].record()
+    inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit)
+    if marks:
+      marks[1].record()
+    if cfg.act_quant is not None:
+      inter = megablox.quantize_lhs(inter, cfg.act_quant)
+    if marks:
+      marks[2].record()
+    out = megablox.gmm(inter, wo, group_size, transpose_rhs=True)
+    if marks:
+      marks[3].record()
+      ev.append(("wi_glu", marks[0], marks[1]))
+      ev.append(("wo", marks[2], marks[3]))
+    return out
+
+  # -- sparse_matmul (moe.py:1403), single device -------------------------------------------
+  def sparse_matmul(self, inputs, gate_logits, pre_bias_logits, w0_kernel, w1_kernel, wo_kernel,
+                    w0_bias=None, w1_bias=None, wo_bias=None, input_ids=None):
+    """-> (output [B,S,d], lb_loss, bias_updates)."""
+    if w0_bias is not None or w1_bias is not None or wo_bias is not None:
+      raise NotImplementedError("mlp_bias is not implemented")
+    cfg = self.config
+    b, s, d = inputs.shape
+    k = self.num_experts_per_tok
+    x2d = inputs.reshape(b * s, d).contiguous()
+    weights, selected = self.get_topk(gate_logits, pre_bias_logits)
+    perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
+                                                      want_sorted_experts=False)
+    # permute fused with the activation quantiser of the first GEMM
+    if cfg.act_quant == "int8":
+      q, sc = kernels.gather_rows(x2d, perm, k, out_dtype=torch.int8)
+      sorted_inputs = QArray(q, sc, "int8")
+    elif cfg.act_quant == "fp8":
+      q, sc = kernels.gather_rows(x2d, perm, k, out_dtype=torch.float8_e4m3fn, block_k=128)
+      sorted_inputs = QArray(q, sc, "fp8")
+    else:
+      sorted_inputs = kernels.gather_rows(x2d, perm, k)
+    inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel)
+    out = self.unpermute(inter, perm, weights, b, s, inv_perm=inv)
+    return out, None, None
+
+  def __call__(self, inputs, input_ids=None, gate_inputs=None, out_sharding=None):
+    """-> (output, lb_loss, bias_updates), as moe.py:3143."""
+    b, s, d = inputs.shape
+    routing_inputs = inputs if gate_inputs is None else gate_inputs
+    gate_logits, pre_bias = self.gate(routing_inputs.reshape(b * s, -1))
+    gate_logits = gate_logits.reshape(b, s, -1)
+    pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
+    return self.sparse_matmul(inputs, gate_logits, pre_bias, self.wi_0, self.wi_1, self.wo)
+
+
+class RoutedAndSharedMoE:
+  """Routed experts plus always-on shared experts (moe.py:3259-3371).
+
+  The shared expert is one more group that owns every token: its weights are stored as expert
+  index E of the stacked [E+1, N, K] tensors, every token gets it as a (k+1)-th selection with
+  combine weight 1, and the whole layer runs through the same three grouped-GEMM launches.
+  """
+
+  def __init__(self, config: MoEConfig, wi_0, wi_1, wo, gate_kernel=None, gate_bias=None):
+    if config.shared_experts < 1:
+      raise ValueError("RoutedAndSharedMoE needs shared_experts >= 1")
+    self.config = config
+    self.routed = RoutedMoE(config, wi_0, wi_1, wo, gate_kernel, gate_bias)
+    n_stacked = (wi_0.qvalue if isinstance(wi_0, QArray) else wi_0).shape[0]
+    if n_stacked != config.num_experts + 1:
+      raise ValueError("expert tensors must hold num_experts routed experts followed by the shared expert")
+
+  def sparse_matmul(self, inputs, gate_logits, pre_bias_logits):
+    cfg, r = self.config, self.routed
+    b, s, d = inputs.shape
+    t, k, e = b * s, cfg.num_experts_per_tok, cfg.num_experts
+    x2d = inputs.reshape(t, d).contiguous()
+    w, sel = r.get_topk(gate_logits, pre_bias_logits)
+    sel = torch.cat([sel.reshape(t, k), torch.full((t, 1), e, dtype=torch.int32, device=sel.device)], 1).contiguous()
+    w = torch.cat([w.reshape(t, k), torch.ones((t, 1), dtype=torch.float32, device=w.device)], 1).contiguous()
+    perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + 1, want_sorted_experts=False)
+    if cfg.act_quant == "int8":
+      q, sc = kernels.gather_rows(x2d, perm, k + 1, out_dtype=torch.int8)
+      rows = QArray(q, sc, "int8")
+    elif cfg.act_quant == "fp8":
+      q, sc = kernels.gather_rows(x2d, perm, k + 1, out_dtype=torch.float8_e4m3fn, block_k=128)
+      rows = QArray(q, sc, "fp8")
+    else:
+      rows = kernels.gather_rows(x2d, perm, k + 1)
+    inter = r._experts(rows, group_size, r.wi_0, r.wi_1, r.wo)
+    out = kernels.unpermute_combine(inter, w, k=k + 1, inv_perm=inv)
+    return out.reshape(b, s, d), None, None
+
+  def __call__(self, inputs, input_ids=None, gate_inputs=None, out_sharding=None):
+    b, s, d = inputs.shape
+    gate_logits, pre_bias = self.routed.gate(inputs.reshape(b * s, -1))
+    pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
+    return self.sparse_matmul(inputs, gate_logits.reshape(b, s, -1), pre_bias)

@@ -1,0 +1,102 @@
+"""Weight-side quantisers and storage formats (offline preparation, torch ops on any device).
+
+Activations are quantised by the HIP kernels (kernels.gather_rows); the functions here prepare
+expert weights once, at load time, in the layouts the grouped GEMM reads:
+
+  int8   per-output-channel, per expert:  q [G, N, K] int8,  scale [G, N] f32
+         (serve-mode layout gathered per row at src/maxtext/layers/moe.py:1450-1459;
+          share_across_experts=True gives the [1,1,n] scale of kernels/megablox/ops.py:250-260)
+  fp8    e4m3fn, 128x128 blocks:          q [G, N, K] fp8,   scale [G, ceil(N/128), ceil(K/128)] f32
+         (storage format of checkpoint_conversion/standalone_scripts/deepseek_dequantize.py:42-68)
+  int4   symmetric, groups of 128 along K: q [G, N, K/2] uint8 (two per byte, first value in the
+         low nibble, stored +8 -- convert_deepseek_family_ckpt.py:56-84), scale [G, N, ceil(K/128)] bf16
+
+Rounding: scale = absmax / qmax, q = round-half-even(x / scale) clipped; a zero absmax gives q = 0.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+
+import torch
+
+FP8_E4M3_MAX = 448.0
+
+
+@dataclasses.dataclass
+class QArray:
+  """Quantised tensor: values plus scales (the role qwix.pallas.QArray plays in ops.py:232-267).
+
+  For expert weights `qvalue` is [G, N, K] (K contiguous; INT4: uint8 [G, N, K/2]) and `scale`
+  has the layout described in the module docstring; `qtype` is "int8" | "fp8" | "int4".
+  For activations `qvalue` is [M, K] and `scale` is [M] (int8) or [M, ceil(K/128)] (fp8).
+  """
+
+  qvalue: torch.Tensor
+  scale: torch.Tensor
+  qtype: str
+
+  @property
+  def shape(self):
+    return self.qvalue.shape
+
+
+def get_static_scale(qmax: float, calibration_method: str) -> float:
+  """Static symmetric scale from "fixed,max" / "fixed,-max,max" (layers/quantizations.py:928-958)."""
+  if calibration_method is None or not calibration_method.lower().startswith("fixed"):
+    raise ValueError(f"Only static scale quantization is supported, got {calibration_method}")
+  args = [float(a) for a in calibration_method.split(",")[1:]]
+  if len(args) == 1:
+    args = [-args[0], args[0]]
+  if len(args) != 2 or args[0] + args[1] != 0 or args[1] <= 0:
+    raise ValueError(f"Expected format: 'fixed,max' or 'fixed,-max,max'. Got: {calibration_method}")
+  scale = args[1] / qmax
+  if scale < torch.finfo(torch.float32).tiny ** 0.5:
+    scale = 1.0
+  return scale
+
+
+def _rint_div(x, scale):
+  return torch.where(scale == 0, torch.zeros_like(x), torch.round(x / scale))
+
+
+def quantize_weight_int8(w_gnk: torch.Tensor, share_across_experts: bool = False) -> QArray:
+  """w [G, N, K] -> int8 per output channel."""
+  w = w_gnk.to(torch.float32)
+  if share_across_experts:
+    absmax = w.abs().amax(dim=(0, 2), keepdim=True).expand(w.shape[0], w.shape[1], 1)
+  else:
+    absmax = w.abs().amax(dim=2, keepdim=True)
+  scale = absmax / 127.0
+  q = _rint_div(w, scale).clamp(-127, 127).to(torch.int8)
+  return QArray(q.contiguous(), scale.squeeze(-1).contiguous(), "int8")
+
+
+def quantize_weight_fp8_blocks(w_gnk: torch.Tensor, block: int = 128) -> QArray:
+  """w [G, N, K] -> float8_e4m3fn with one f32 scale per block x block tile."""
+  g, n, k = w_gnk.shape
+  nb, kb = math.ceil(n / block), math.ceil(k / block)
+  wp = torch.zeros((g, nb * block, kb * block), dtype=torch.float32, device=w_gnk.device)
+  wp[:, :n, :k] = w_gnk
+  wb = wp.view(g, nb, block, kb, block)
+  scale = wb.abs().amax(dim=(2, 4), keepdim=True) / FP8_E4M3_MAX
+  q = torch.where(scale == 0, torch.zeros_like(wb), wb / scale).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX)
+  q = q.view(g, nb * block, kb * block)[:, :n, :k].to(torch.float8_e4m3fn)
+  return QArray(q.contiguous(), scale.view(g, nb, kb).contiguous(), "fp8")
+
+
+def quantize_weight_int4(w_gnk: torch.Tensor, group: int = 128) -> QArray:
+  """w [G, N, K] -> packed int4 with bf16 scales per `group` values of K (ragged last group allowed)."""
+  g, n, k = w_gnk.shape
+  if k % 2:
+    raise ValueError("K must be even to pack two int4 values per byte")
+  ng = math.ceil(k / group)
+  wp = torch.zeros((g, n, ng * group), dtype=torch.float32, device=w_gnk.device)
+  wp[:, :, :k] = w_gnk
+  wg = wp.view(g, n, ng, group)
+  scale = (wg.abs().amax(-1, keepdim=True) / 7.0).clamp(min=1e-12).to(torch.bfloat16)
+  q = torch.round(wg / scale.to(torch.float32)).clamp(-8, 7).to(torch.int16).view(g, n, ng * group)[:, :, :k]
+  u = (q + 8).to(torch.uint8)
+  packed = (u[..., 0::2] | (u[..., 1::2] << 4)).contiguous()
+  return QArray(packed, scale.squeeze(-1).contiguous(), "int4")

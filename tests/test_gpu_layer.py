@@ -1,0 +1,151 @@
+"""GPU parity of the whole expert path (route -> permute -> gmm x3 + SwiGLU -> combine) against
+the oracle, on the benchmark configurations (C1 at full size, C2..C5 at reduced dims so the
+CPU oracle finishes in seconds) plus size-independent properties at larger sizes.
+
+Routing indices, perm and group sizes must match bit-exactly; outputs within
+max|got-want| / max|want| <= 1e-2.
+"""
+
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def relerr(got, want):
+  got, want = got.detach().float().cpu(), want.detach().float().cpu()
+  return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def _small(name, tokens, **dims):
+  from maxtext_amd import synthetic
+
+  wl = synthetic.workload(name, tokens)
+  return dataclasses.replace(wl, cfg=dataclasses.replace(wl.cfg, **dims))
+
+
+def oracle_layer(wl, layer):
+  """The same pipeline with oracle functions, consuming the identical quantised weights."""
+  from oracle.layer import oracle_layer as run
+
+  cfg = wl.cfg
+  trip = lambda qa: (qa.qvalue, qa.scale, qa.qtype)
+  return run(layer["x"], layer["gate_logits"], layer["pre_bias_logits"], trip(layer["wi_0"]), trip(layer["wi_1"]), trip(layer["wo"]),
+             num_experts=cfg.num_experts, k=cfg.num_experts_per_tok, emb_dim=cfg.emb_dim, mlp_dim=cfg.moe_mlp_dim,
+             deepseek=cfg.is_deepseek, routed_scaling_factor=cfg.routed_scaling_factor, norm_topk_prob=cfg.norm_topk_prob,
+             shared_experts=cfg.shared_experts, act_quant=cfg.act_quant, activation=cfg.activation)
+
+
+def run_gpu(wl, layer_cpu):
+  from maxtext_amd import moe
+  from maxtext_amd.quantizations import QArray
+
+  def dev(v):
+    if isinstance(v, QArray):
+      return QArray(v.qvalue.cuda(), v.scale.cuda(), v.qtype)
+    return None if v is None else v.cuda()
+
+  L = {k: dev(v) for k, v in layer_cpu.items()}
+  cls = moe.RoutedAndSharedMoE if wl.cfg.shared_experts else moe.RoutedMoE
+  block = cls(wl.cfg, L["wi_0"], L["wi_1"], L["wo"])
+  if wl.cfg.shared_experts:
+    out, _, _ = block.sparse_matmul(L["x"], L["gate_logits"], L["pre_bias_logits"])
+  else:
+    out, _, _ = block.sparse_matmul(L["x"], L["gate_logits"], L["pre_bias_logits"], L["wi_0"], L["wi_1"], L["wo"])
+  return out, block, L
+
+
+CASES = {
+    "c1_full": lambda: _small("c1", 2048),
+    "c2_small": lambda: _small("c2", 1024, emb_dim=1024, moe_mlp_dim=2048),
+    "c3_small": lambda: _small("c3", 64, emb_dim=1024, moe_mlp_dim=512, num_experts=32),
+    "c4_small": lambda: _small("c4", 2048, emb_dim=512, moe_mlp_dim=256),
+    "c5_t1": lambda: _small("c5", 1, num_experts=8),
+    "c5_t16": lambda: _small("c5", 16, num_experts=8),
+    "c5_t128": lambda: _small("c5", 128, num_experts=8),
+    "c5_t1024": lambda: _small("c5", 1024, num_experts=4, moe_mlp_dim=1024),
+}
+
+
+@pytest.mark.parametrize("case", list(CASES))
+def test_layer_matches_oracle(case):
+  from maxtext_amd import synthetic
+
+  wl = CASES[case]()
+  layer = synthetic.make_layer(wl, device="cpu")
+  want, oidx, operm, ogs = oracle_layer(wl, layer)
+  got, block, L = run_gpu(wl, layer)
+  # the integer half of the path, bit-exact
+  r = block.routed if wl.cfg.shared_experts else block
+  _, idx = r.get_topk(L["gate_logits"], L["pre_bias_logits"])
+  k = wl.cfg.num_experts_per_tok
+  np.testing.assert_array_equal(idx.reshape(-1, k).cpu().numpy(), oidx[:, :k])
+  if not wl.cfg.shared_experts:
+    _, perm, _, gs, _, _, _, _ = r.permute(L["x"], L["gate_logits"], L["pre_bias_logits"])
+    np.testing.assert_array_equal(perm.cpu().numpy(), operm)
+    np.testing.assert_array_equal(gs.cpu().numpy(), ogs)
+  assert got.shape == layer["x"].shape and got.dtype == torch.bfloat16
+  assert relerr(got.reshape(want.shape), want) <= TOL
+
+
+def test_permute_unpermute_api_roundtrip():
+  # unpermute(permute(x)) with unit weights returns k*x exactly (property, any size)
+  from maxtext_amd import moe
+
+  t, d, e, k = 4096, 1024, 64, 4
+  cfg = moe.MoEConfig(e, k, d, 128)
+  block = moe.RoutedMoE(cfg, None, None, None)
+  g = torch.Generator(device="cuda").manual_seed(3)
+  x = torch.randn((1, t, d), generator=g, device="cuda").to(torch.bfloat16)
+  logits = torch.randn((1, t, e), generator=g, device="cuda")
+  sorted_inputs, perm, weights, group_size, sorted_experts, _, _, _ = block.permute(x, logits)
+  assert int(group_size.sum()) == t * k
+  assert torch.equal(torch.sort(perm.long())[0], torch.arange(t * k, device="cuda"))
+  assert torch.all(sorted_experts[1:] >= sorted_experts[:-1])
+  assert torch.equal(torch.bincount(sorted_experts.long(), minlength=e).int(), group_size)
+  out = block.unpermute(sorted_inputs, perm, torch.ones_like(weights), 1, t)
+  assert torch.equal(out, (x.float() * k).to(torch.bfloat16))
+
+
+def test_megablox_gmm_api():
+  from maxtext_amd import megablox
+
+  g = torch.Generator().manual_seed(11)
+  m, kd, n, e = 512, 256, 384, 4
+  lhs = torch.randn(m, kd, generator=g).to(torch.bfloat16)
+  rhs = (torch.randn(e, kd, n, generator=g) * 0.05).to(torch.bfloat16)  # reference default layout [g, k, n]
+  gs = np.array([100, 0, 312, 100], np.int32)
+  want = O.gmm(lhs, rhs, gs)
+  got = megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda())
+  assert relerr(got, want) <= TOL
+  got_t = megablox.gmm(lhs.cuda(), rhs.transpose(1, 2).contiguous().cuda(), torch.from_numpy(gs).cuda(), transpose_rhs=True)
+  assert torch.equal(got, got_t)
+  # dynamic int8 on both sides (ops.py:232-267): close to the unquantised product (quantizations_test.py:653: < 0.2)
+  got_q = megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda(), lhs_quantize_dtype="int8", rhs_quantize_dtype="int8")
+  assert (got_q.float().cpu() - want.float()).abs().mean() / want.float().abs().mean() < 0.2
+  with pytest.raises(ValueError):
+    megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs.astype(np.int64)).cuda())
+  with pytest.raises(ValueError):
+    megablox.gmm(lhs.cuda()[None], rhs.cuda(), torch.from_numpy(gs).cuda())
+
+
+def test_layer_linearity_at_benchmark_width():
+  # property at C2's real width (d 4096, f 14336): with bf16 activations and int8 weights the layer is
+  # positively homogeneous in the wo weights' scales: doubling wo's scales doubles the output exactly.
+  from maxtext_amd import moe, synthetic
+  from maxtext_amd.quantizations import QArray
+
+  wl = _small("c2", 512, act_quant=None)
+  layer = synthetic.make_layer(wl, device="cuda")
+  block = moe.RoutedMoE(wl.cfg, layer["wi_0"], layer["wi_1"], layer["wo"])
+  out1, _, _ = block.sparse_matmul(layer["x"], layer["gate_logits"], None, layer["wi_0"], layer["wi_1"], layer["wo"])
+  wo2 = QArray(layer["wo"].qvalue, layer["wo"].scale * 2, "int8")
+  out2, _, _ = block.sparse_matmul(layer["x"], layer["gate_logits"], None, layer["wi_0"], layer["wi_1"], wo2)
+  assert torch.isfinite(out1.float()).all()
+  assert torch.equal(out2.float(), out1.float() * 2)
