@@ -224,17 +224,33 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
   }
 
   uint4 a_reg[C::A_CH], b_reg[C::B_CH];
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+  constexpr int B_GSZ = C::BSRC == BSRC_I4 ? 1 : (C::BSRC == BSRC_I8 ? 2 : 2 * C::ESZ);  // half-bytes per element in HBM
 
+  // Every chunk of a full stage is in range: plain loads that stay in flight during the MFMAs.
   auto load_stage = [&](int kt) {
+    const size_t k0 = (size_t)kt * C::BK;
+#pragma unroll
+    for (int i = 0; i < C::A_CH; i++) a_reg[i] = *(const uint4*)(a_ptr[i] + k0 * C::ESZ);
+#pragma unroll
+    for (int i = 0; i < C::B_CH; i++) b_reg[i] = *(const uint4*)(b_ptr[i] + k0 * B_GSZ / 2);
+  };
+  // Last stage when K is not a multiple of BK: chunks past K read offset 0 and are zeroed by value.
+  auto load_stage_tail = [&](int kt) {
     const int k0 = kt * C::BK;
 #pragma unroll
-    for (int i = 0; i < C::A_CH; i++)
-      a_reg[i] = (k0 + a_k[i] < K) ? *(const uint4*)(a_ptr[i] + (size_t)k0 * C::ESZ) : zero4;
+    for (int i = 0; i < C::A_CH; i++) {
+      const bool ok = k0 + a_k[i] < K;
+      const uint4 v = *(const uint4*)(a_ptr[i] + (ok ? (size_t)k0 * C::ESZ : 0));
+      const uint32_t m = ok ? 0xffffffffu : 0u;
+      a_reg[i] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+    }
 #pragma unroll
     for (int i = 0; i < C::B_CH; i++) {
-      const size_t off = C::BSRC == BSRC_I4 ? (size_t)k0 / 2 : (size_t)k0 * (C::BSRC == BSRC_I8 ? 1 : C::ESZ);
-      b_reg[i] = (k0 + b_k[i] < K) ? *(const uint4*)(b_ptr[i] + off) : zero4;
+      const bool ok = k0 + b_k[i] < K;
+      const uint4 v = *(const uint4*)(b_ptr[i] + (ok ? (size_t)k0 * B_GSZ / 2 : 0));
+      // INT4 stores value+8: a zero weight is the nibble 8
+      const uint32_t z = C::BSRC == BSRC_I4 ? 0x88888888u : 0u;
+      b_reg[i] = ok ? v : make_uint4(z, z, z, z);
     }
   };
 
@@ -331,14 +347,18 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
 
   // ---- main loop: one barrier per stage --------------------------------------------------
   const int nk = (K + C::BK - 1) / C::BK;
-  load_stage(0);
+  const bool k_tail = (K % C::BK) != 0;
+  if (nk == 1 && k_tail) load_stage_tail(0); else load_stage(0);
   store_stage(0, 0);
   __syncthreads();
   for (int kt = 0; kt < nk; kt++) {
     const int cur = kt & 1;
-    if (kt + 1 < nk) load_stage(kt + 1);
+    const bool more = kt + 1 < nk;
+    if (more) {
+      if (k_tail && kt + 2 == nk) load_stage_tail(kt + 1); else load_stage(kt + 1);
+    }
     compute_stage(cur);
-    if (kt + 1 < nk) store_stage(cur ^ 1, kt + 1);
+    if (more) store_stage(cur ^ 1, kt + 1);
     __syncthreads();
   }
 
@@ -529,6 +549,25 @@ static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* b
   return launch_tiled<TiledCfg<OP, BSRC, 64, 256, 128, 1, 4, GLU>>(p, M, G_total, s);
 }
 
+// Tile variants of the int8 kernel that reserved[0] can force (tuning aid); returns the m-tile.
+template <bool GLU>
+static int launch_i8_variant(int id, const TiledParams& p, int M, int G_total, int* bm_out, bool dry, hipStream_t s) {
+#define MOE_VARIANT(ID, BM, BN, BKB, WM, WN)                                                        \
+  if (id == ID) {                                                                                   \
+    *bm_out = BM;                                                                                   \
+    if (dry) return MOE_OK;                                                                         \
+    return launch_tiled<TiledCfg<OP_I8, BSRC_SAME, BM, BN, BKB, WM, WN, GLU>>(p, M, G_total, s);    \
+  }
+  MOE_VARIANT(3, 256, 256, 64, 2, 4)
+  MOE_VARIANT(4, 256, 256, 64, 2, 2)
+  MOE_VARIANT(5, 256, 256, 128, 2, 2)
+  MOE_VARIANT(6, 128, 256, 128, 2, 2)
+  MOE_VARIANT(7, 128, 128, 128, 2, 2)
+  MOE_VARIANT(8, 128, 256, 64, 2, 2)
+#undef MOE_VARIANT
+  return fail(MOE_ERR_INVALID_ARG, "gmm: unknown tile variant %d", id);
+}
+
 template <int OP, int BSRC>
 static int launch_tiled_glu(const TiledParams& p, bool glu, int M, int G_total, int* bm_out, bool dry, hipStream_t s) {
   return glu ? launch_tiled_by_rows<OP, BSRC, true>(p, M, G_total, bm_out, dry, s)
@@ -637,6 +676,13 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
 
   // dry run to learn the m-tile, then build the tile list and launch
   const int M = a->M, G = a->num_groups_total;
+  const int forced = a->reserved[0];
+  if (forced >= 3 && variant == V_I8) {
+    int st = glu ? launch_i8_variant<true>(forced, p, M, G, &bm, true, s) : launch_i8_variant<false>(forced, p, M, G, &bm, true, s);
+    if (st != MOE_OK) return st;
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
+    return glu ? launch_i8_variant<true>(forced, p, M, G, &bm, false, s) : launch_i8_variant<false>(forced, p, M, G, &bm, false, s);
+  }
   launch_tiled_by_rows<OP_BF16, BSRC_SAME, false>(p, M, G, &bm, true, s);
   tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
   switch (variant) {
