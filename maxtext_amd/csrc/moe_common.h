@@ -34,8 +34,13 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 
 __device__ __forceinline__ float round_bf16_fn(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// Two f32 -> packed bf16 (round to nearest even) in one v_cvt_pk_bf16_f32.
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -50,7 +55,10 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// 1 / (1 + 2^(-x log2 e)) on the hardware exp2 / rcp units (about 1 ulp each): five instructions.
+__device__ __forceinline__ float sigmoidf_(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
 
 // gate/up -> activation, computed in f32 (moe.py:841-870).
 __device__ __forceinline__ float glu_act(float g, float u, int act, float limit) {

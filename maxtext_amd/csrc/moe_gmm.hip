@@ -123,11 +123,76 @@ struct TiledParams {
   int max_m_tiles, tiles_n;
   int act;
   float act_limit;
+  int dbg;  // timing experiments only: 1 = no barrier/wait, 2 = no loads in the loop
 };
 
 __device__ __forceinline__ uint32_t i8x2_to_bf16x2(int lo, int hi) {
   // |value| <= 128 is exact in bf16, so truncating the f32 is the conversion
   return (__float_as_uint((float)lo) >> 16) | (__float_as_uint((float)hi) & 0xffff0000u);
+}
+
+// Per-lane scales of the epilogue, fetched before the K loop so their latency hides behind it.  With
+// weights as the MFMA "A" operand a lane owns row (lane % 32) of each 32-row tile and, per accumulator
+// quad q, the 4 consecutive output channels 8*q + 4*(lane / 32) .. +3 of each 32-channel tile.
+template <int TM, int NT_OUT, bool GLU>
+struct EpilogueScales {
+  float sa[TM];
+  float4 sg[NT_OUT][4], su[NT_OUT][4];
+};
+
+template <int TM, int NT_OUT, bool GLU, bool CHANNEL_SCALES>
+__device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, GLU>& e, const TiledParams& p, const TileInfo& tile,
+                                                     int row_base, int n_base, int lane) {
+  const float4 one = make_float4(1.f, 1.f, 1.f, 1.f);
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int lr = row_base + i * 32 + (lane % 32);
+    e.sa[i] = p.lhs_scale ? p.lhs_scale[tile.row0 + (lr < tile.nrows ? lr : 0)] : 1.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int n = n_base + j * 32 + 8 * q + 4 * (lane / 32);
+      e.sg[j][q] = one;
+      e.su[j][q] = one;
+      if (CHANNEL_SCALES && p.rhs_scale && n < p.N) {
+        e.sg[j][q] = *(const float4*)((const float*)p.rhs_scale + (size_t)tile.group * p.N + n);
+        if (GLU) e.su[j][q] = *(const float4*)((const float*)p.rhs_up_scale + (size_t)tile.group * p.N + n);
+      }
+    }
+}
+
+template <int TM, int TN, int NT_OUT, bool GLU, typename acc_t>
+__device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
+                                               const TiledParams& p, const TileInfo& tile, int row_base, int n_base, int lane) {
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int lr = row_base + i * 32 + (lane % 32);
+    if (lr >= tile.nrows) continue;
+    uint16_t* orow = p.out + (size_t)(tile.row0 + lr) * p.N;
+#pragma unroll
+    for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n_base + j * 32 + 8 * q + 4 * (lane / 32);
+        if (n >= p.N) continue;
+        const float sg[4] = {e.sg[j][q].x, e.sg[j][q].y, e.sg[j][q].z, e.sg[j][q].w};
+        const float su[4] = {e.su[j][q].x, e.su[j][q].y, e.su[j][q].z, e.su[j][q].w};
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float g = (float)acc[j][i][4 * q + r] * (e.sa[i] * sg[r]);
+          if (GLU) {
+            const float u = (float)acc[j + NT_OUT][i][4 * q + r] * (e.sa[i] * su[r]);
+            v[r] = glu_act(g, u, p.act, p.act_limit);
+          } else {
+            v[r] = g;
+          }
+        }
+        *(uint2*)(orow + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
+  }
 }
 
 template <int OP_, int BSRC_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, bool GLU_>
@@ -346,62 +411,243 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
   };
 
   // ---- main loop: one barrier per stage --------------------------------------------------
+  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
+  const int n_out0 = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+  EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+  load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC != BSRC_I4>(esc, p, tile, wm * C::WM, n_out0, lane);
+
+  // The steady-state loop only ever issues full-stage loads; the stage that may hold the K tail is
+  // loaded in a peeled iteration so its masking code never merges into the loop body.
   const int nk = (K + C::BK - 1) / C::BK;
   const bool k_tail = (K % C::BK) != 0;
   if (nk == 1 && k_tail) load_stage_tail(0); else load_stage(0);
   store_stage(0, 0);
   __syncthreads();
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < nk;
-    if (more) {
-      if (k_tail && kt + 2 == nk) load_stage_tail(kt + 1); else load_stage(kt + 1);
-    }
-    compute_stage(cur);
-    if (more) store_stage(cur ^ 1, kt + 1);
+  int kt = 0;
+  for (; kt + 2 < nk; kt++) {
+    load_stage(kt + 1);
+    __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the MFMAs: it needs their time to land
+    compute_stage(kt & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    store_stage((kt & 1) ^ 1, kt + 1);
     __syncthreads();
   }
+  if (kt + 1 < nk) {
+    if (k_tail) load_stage_tail(kt + 1); else load_stage(kt + 1);
+    compute_stage(kt & 1);
+    store_stage((kt & 1) ^ 1, kt + 1);
+    __syncthreads();
+    kt++;
+  }
+  compute_stage(kt & 1);
 
-  // ---- epilogue: scales, activation, bf16 store ------------------------------------------
-  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
-  const int half = lane / 32;
+  store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, tile, wm * C::WM, n_out0, lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// Direct-to-LDS variant of the tiled kernel for operands that need no conversion (int8 x int8,
+// bf16 x bf16) and K * elem_size % BKB == 0.  global_load_lds_dwordx4 copies 16 bytes per lane
+// straight into LDS (1 KB per wave instruction, no staging registers, no ds_write), NSTAGE
+// buffers are kept in flight, and there is one barrier per K stage.  LDS rows are unpadded; the
+// 16-byte chunk q of row r is stored at slot q ^ f(r), chosen so that the b128 fragment reads of
+// 16 consecutive rows hit 16 different bank groups.  The permutation is applied on the global
+// address side, because the LDS side of the instruction is fixed (base + 16 * lane).
+// ---------------------------------------------------------------------------------------
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+template <int OP_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, int NSTAGE_, bool GLU_>
+struct DlCfg {
+  static constexpr int OP = OP_, BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
+  static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NWAVES = WAVES_M_ * WAVES_N_;
+  static constexpr bool GLU = GLU_;
+  static constexpr int THREADS = NWAVES * kWave;
+  static constexpr int ESZ = OP == OP_I8 ? 1 : 2;
+  static constexpr int BK = BKB / ESZ;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int KSUB = BKB / 32;
+  static constexpr int CPR = BKB / 16;         // 16-byte chunks per row
+  static constexpr int RPI = 1024 / BKB;       // rows per wave instruction
+  static constexpr int A_IPW = BM / RPI / NWAVES, B_IPW = BN / RPI / NWAVES;  // instructions per wave per stage
+  static constexpr int LPS = A_IPW + B_IPW;
+  static constexpr int STAGE = (BM + BN) * BKB;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE;
+  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static_assert(BKB == 64 || BKB == 128, "row swizzle is defined for 64 and 128 byte rows");
+  static_assert(BM % (RPI * NWAVES) == 0 && BN % (RPI * NWAVES) == 0, "load split");
+  static_assert(!GLU || ((BN / 2) % RPI == 0 && TN % 2 == 0), "GLU halves");
+  static_assert((NSTAGE - 1) * LPS < 64, "vmcnt range");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+  __device__ static __forceinline__ int swz(int row) { return BKB == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
+};
+
+// s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <typename C>
+__global__ __launch_bounds__(C::THREADS) void gmm_dl_kernel(const TiledParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int OP = C::OP;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
+
+  int m_idx, n_idx;
+  {
+    const int nb = gridDim.x, pid = blockIdx.x;
+    const int q = nb / 8, rem = nb % 8, xcd = pid % 8, loc = pid / 8;
+    const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+    constexpr int GSM = 4;
+    const int width = GSM * p.tiles_n;
+    const int sg = logical / width, first_m = sg * GSM;
+    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    m_idx = first_m + (logical % width) % gsz;
+    n_idx = (logical % width) / gsz;
+  }
+  if (m_idx >= p.header[0]) return;
+  const TileInfo tile = p.tiles[m_idx];
+  const int n0 = n_idx * C::OUT_BN;
+  const int N = p.N, K = p.K;
+
+  if (tile.group < 0) {
+    constexpr int QPR = C::OUT_BN / 4;
+    for (int i = tid; i < tile.nrows * QPR; i += C::THREADS) {
+      int r = i / QPR, c = n0 + (i % QPR) * 4;
+      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  // ---- per-lane source addresses of this wave's load instructions ---------------------------
+  const size_t row_bytes = (size_t)K * C::ESZ;
+  const uint8_t* a_src[C::A_IPW];
+  const uint8_t* b_src[C::B_IPW];
 #pragma unroll
-  for (int i = 0; i < C::TM; i++) {
-    const int lr = wm * C::WM + i * 32 + (lane % 32);
-    const bool row_ok = lr < tile.nrows;
-    const int gr = tile.row0 + (row_ok ? lr : 0);
-    const float sa = p.lhs_scale ? p.lhs_scale[gr] : 1.0f;
+  for (int i = 0; i < C::A_IPW; i++) {
+    const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
+    const int q = (lane % C::CPR) ^ C::swz(r);
+    a_src[i] = p.lhs + (size_t)(tile.row0 + min(r, tile.nrows - 1)) * row_bytes + q * 16;
+  }
 #pragma unroll
-    for (int j = 0; j < NT_OUT; j++) {
-      const int nbase = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN) + j * 32;
+  for (int i = 0; i < C::B_IPW; i++) {
+    const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
+    const int q = (lane % C::CPR) ^ C::swz(vr);
+    const bool up = C::GLU && vr >= C::BN / 2;
+    const int n = min(n0 + (up ? vr - C::BN / 2 : vr), N - 1);
+    b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)tile.group * N + n) * row_bytes + q * 16;
+  }
+
+  auto issue_stage = [&](int kt, int buf) {
+    const size_t koff = (size_t)kt * C::BKB;
+    uint8_t* s = smem + buf * C::STAGE;
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int n = nbase + 8 * q + 4 * half;
-        if (!row_ok || n >= N) continue;
-        float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
-        if (C::BSRC != BSRC_I4 && p.rhs_scale) {
-          const float4 t = *(const float4*)((const float*)p.rhs_scale + (size_t)tile.group * N + n);
-          sg[0] = t.x; sg[1] = t.y; sg[2] = t.z; sg[3] = t.w;
-          if (C::GLU) {
-            const float4 u = *(const float4*)((const float*)p.rhs_up_scale + (size_t)tile.group * N + n);
-            su[0] = u.x; su[1] = u.y; su[2] = u.z; su[3] = u.w;
-          }
-        }
-        float v[4];
+    for (int i = 0; i < C::A_IPW; i++)
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[i] + koff), (lds_ptr_t)(s + (wave * C::A_IPW + i) * 1024), 16, 0, 0);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          float g = (float)acc[j][i][4 * q + r] * (sa * sg[r]);
-          if (C::GLU) {
-            float u = (float)acc[j + NT_OUT][i][4 * q + r] * (sa * su[r]);
-            v[r] = glu_act(g, u, p.act, p.act_limit);
-          } else {
-            v[r] = g;
-          }
-        }
-        *(uint2*)(p.out + (size_t)gr * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-      }
+    for (int i = 0; i < C::B_IPW; i++)
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
+                                       (lds_ptr_t)(s + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+  };
+
+  typedef typename std::conditional<OP == OP_I8, v16i, v16f>::type acc_t;
+  acc_t acc[C::TN][C::TM];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++)
+#pragma unroll
+    for (int i = 0; i < C::TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
+
+  int b_row[C::TN];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++) {
+    if (C::GLU) {
+      constexpr int H = C::TN / 2;
+      b_row[j] = (j < H ? 0 : C::BN / 2) + wn * (C::WN / 2) + (j < H ? j : j - H) * 32;
+    } else {
+      b_row[j] = wn * C::WN + j * 32;
     }
   }
+  // fragment of k-step ks: row (lane % 32), chunk q = 2*ks + lane/32, stored at slot q ^ swz(row)
+  const int lrow = lane % 32;
+  const int t16 = ((lane / 32) ^ C::swz(lrow)) * 16;
+  const int row_off = lrow * C::BKB;
+
+  // Fragments are double-buffered in registers: while the MFMAs of k-step ks run, the b128 reads of the
+  // next k-step (possibly the first one of the next stage) are already in flight.
+  v4i fa[2][C::TM], fb[2][C::TN];
+  auto load_frags = [&](int buf, int ks, int set) {
+    const uint8_t* sa = smem + buf * C::STAGE + (wm * C::WM) * C::BKB + row_off;
+    const uint8_t* sb = smem + buf * C::STAGE + C::BM * C::BKB + row_off;
+    const int koff = t16 ^ (ks * 32);
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) fa[set][i] = *(const v4i*)(sa + i * 32 * C::BKB + koff);
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) fb[set][j] = *(const v4i*)(sb + b_row[j] * C::BKB + koff);
+  };
+  auto mfma_frags = [&](int set) {
+#pragma unroll
+    for (int j = 0; j < C::TN; j++)
+#pragma unroll
+      for (int i = 0; i < C::TM; i++) {
+        if constexpr (OP == OP_I8) {
+          acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
+        } else {
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              __builtin_bit_cast(v8bf, fb[set][j]), __builtin_bit_cast(v8bf, fa[set][i]), acc[j][i], 0, 0, 0);
+        }
+      }
+  };
+
+  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
+  const int n_out0 = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+  EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+
+  // ---- pipeline -----------------------------------------------------------------------------------
+  // Stages 0..NSTAGE-2 are requested up front.  In iteration kt, just before the last k-step's MFMAs,
+  // the wave waits for its own loads of stage kt+1, meets the others at a bare barrier (stage kt+1 is
+  // then complete in LDS and nobody reads stage kt-1's buffer any more), requests stage kt+NSTAGE-1
+  // into that free buffer, and prefetches stage kt+1's first fragments.  __syncthreads() is not used:
+  // its fence would drain vmcnt to 0 and with it the loads that are meant to stay in flight.
+  static_assert(C::KSUB % 2 == 0 && C::NSTAGE >= 3, "pipeline shape");
+  const int nk = K / C::BK;
+  // (issued before the first stage so that the vmcnt bookkeeping below only ever counts stage loads)
+  load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, tile, wm * C::WM, n_out0, lane);
+#pragma unroll
+  for (int s = 0; s < C::NSTAGE - 1; s++)
+    if (s < nk) issue_stage(s, s);
+  if (nk >= C::NSTAGE - 1) wait_vmcnt<(C::NSTAGE - 2) * C::LPS>(); else wait_vmcnt<0>();
+  asm volatile("s_barrier" ::: "memory");
+  load_frags(0, 0, 0);
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
+  for (int kt = 0; kt < nk; kt++) {
+    const int buf = kt % C::NSTAGE;
+#pragma unroll
+    for (int ks = 0; ks < C::KSUB; ks++) {
+      if (ks + 1 < C::KSUB) {
+        load_frags(buf, ks + 1, (ks + 1) & 1);
+      } else if (kt + 1 < nk) {
+        if (kt + C::NSTAGE - 1 <= nk) wait_vmcnt<(C::NSTAGE - 3) * C::LPS>(); else wait_vmcnt<0>();
+        asm volatile("s_barrier" ::: "memory");
+        if (kt + C::NSTAGE - 1 < nk) issue_stage(kt + C::NSTAGE - 1, (kt + C::NSTAGE - 1) % C::NSTAGE);
+        load_frags((kt + 1) % C::NSTAGE, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_frags(ks & 1);
+      // By the time the last of these MFMAs has issued, the prefetched fragments have long arrived; waiting
+      // for them here (and not at the top of the next k-step) keeps that k-step's MFMAs free of LDS waits.
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, tile, wm * C::WM, n_out0, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -539,12 +785,34 @@ static int launch_tiled(const TiledParams& p0, int M, int G_total, hipStream_t s
   return check_launch("gmm_tiled_kernel");
 }
 
+template <typename C>
+static int launch_dl(const TiledParams& p0, int M, int G_total, hipStream_t s) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gmm_dl_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "gmm: cannot reserve %d bytes of LDS: %s", C::LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  TiledParams p = p0;
+  p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
+  p.tiles_n = cdiv(p.N, C::OUT_BN);
+  const long long blocks = (long long)p.max_m_tiles * p.tiles_n;
+  if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  gmm_dl_kernel<C><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
+  return check_launch("gmm_dl_kernel");
+}
+
 template <int OP, int BSRC, bool GLU>
 static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* bm_out, bool dry, hipStream_t s) {
   // rows per expert on average decides the m-tile: full 256-row tiles for prefill, 64 otherwise
   const bool big = (long long)M >= 128LL * G_total;
   *bm_out = big ? 256 : 64;
   if (dry) return MOE_OK;
+  if constexpr (BSRC == BSRC_SAME) {
+    // operands that need no conversion stream straight into LDS when every stage is a full 64-byte row slice
+    constexpr int ESZ = OP == OP_I8 ? 1 : 2;
+    if (big && (p.K * ESZ) % 64 == 0) return launch_dl<DlCfg<OP, 256, 256, 64, 2, 4, 4, GLU>>(p, M, G_total, s);
+  }
   if (big) return launch_tiled<TiledCfg<OP, BSRC, 256, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
   return launch_tiled<TiledCfg<OP, BSRC, 64, 256, 128, 1, 4, GLU>>(p, M, G_total, s);
 }
@@ -565,6 +833,21 @@ static int launch_i8_variant(int id, const TiledParams& p, int M, int G_total, i
   MOE_VARIANT(7, 128, 128, 128, 2, 2)
   MOE_VARIANT(8, 128, 256, 64, 2, 2)
 #undef MOE_VARIANT
+#define MOE_DL_VARIANT(ID, BM, BN, BKB, WM, WN, NS)                                                 \
+  if (id == ID) {                                                                                   \
+    *bm_out = BM;                                                                                   \
+    if (dry) return MOE_OK;                                                                         \
+    if (p.K % BKB) return fail(MOE_ERR_UNSUPPORTED, "gmm: variant needs K %% %d == 0", BKB);        \
+    return launch_dl<DlCfg<OP_I8, BM, BN, BKB, WM, WN, NS, GLU>>(p, M, G_total, s);                 \
+  }
+  MOE_DL_VARIANT(10, 256, 256, 64, 2, 4, 5)
+  MOE_DL_VARIANT(11, 256, 256, 64, 2, 4, 3)
+  MOE_DL_VARIANT(12, 256, 256, 64, 2, 4, 4)
+  MOE_DL_VARIANT(13, 256, 256, 64, 2, 2, 3)
+  MOE_DL_VARIANT(14, 256, 256, 64, 2, 2, 4)
+  MOE_DL_VARIANT(15, 128, 256, 64, 2, 2, 4)
+  MOE_DL_VARIANT(16, 256, 128, 64, 2, 2, 4)
+#undef MOE_DL_VARIANT
   return fail(MOE_ERR_INVALID_ARG, "gmm: unknown tile variant %d", id);
 }
 
@@ -647,7 +930,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   p.rhs_scale = a->rhs_scale; p.rhs_up_scale = a->rhs_up_scale;
   p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
   p.M = a->M; p.K = a->K; p.N = a->N; p.max_m_tiles = 0; p.tiles_n = 0;
-  p.act = a->act; p.act_limit = a->act_limit;
+  p.act = a->act; p.act_limit = a->act_limit; p.dbg = a->reserved[1];
 
   enum { V_NONE, V_BF16, V_W8, V_W4, V_I8 } variant = V_NONE;
   if (L == MOE_BF16 && R == MOE_BF16) {

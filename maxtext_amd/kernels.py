@@ -197,6 +197,7 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.act = _lib.ACT_BY_NAME[act]
   a.act_limit = float(act_limit)
   a.reserved[0] = int(tile_variant)
+  a.reserved[1] = int(__import__("os").environ.get("MOE_DBG", "0"))
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
   _lib.check(st, "moe_gmm")
   return out
