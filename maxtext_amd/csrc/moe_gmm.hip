@@ -667,7 +667,8 @@ struct SkinnyParams {
   const TileInfo* tiles;
   uint16_t* out;
   int M, K, N;
-  int n_blocks;  // blocks along N (64 channels each)
+  int n_blocks;  // blocks along N
+  int min_rows, max_rows;  // only tiles with min_rows <= nrows <= max_rows are computed by this launch
   int act;
   float act_limit;
 };
@@ -680,20 +681,24 @@ __device__ __forceinline__ v8i load32(const uint8_t* p) {
   return r;
 }
 
-template <int MT, bool GLU>
+// One wave owns NT tiles of 16 output channels (x2 with GLU) and MT tiles of 16 rows, and walks K in
+// steps of U 128-byte blocks whose loads are all issued before the first MFMA of the step.
+template <int MT, int NT, int U, bool GLU>
 __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams p) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int j = lane % 16, kq = lane / 16;
   const int m_idx = blockIdx.x / p.n_blocks;
   if (m_idx >= p.header[0]) return;
   const TileInfo tile = p.tiles[m_idx];
+  if (tile.group >= 0 ? (tile.nrows < p.min_rows || tile.nrows > p.max_rows) : p.min_rows > 1) return;
   const int N = p.N, K = p.K;
-  const int n16 = (blockIdx.x % p.n_blocks) * 64 + wave * 16;
-  if (n16 >= N) return;
+  constexpr int WN = 16 * NT;  // channels per wave
+  const int n_w = (blockIdx.x % p.n_blocks) * (4 * WN) + wave * WN;
+  if (n_w >= N) return;
 
   if (tile.group < 0) {
-    for (int i = lane; i < tile.nrows * 4; i += kWave) {
-      int r = i / 4, c = n16 + (i % 4) * 4;
+    for (int i = lane; i < tile.nrows * (WN / 4); i += kWave) {
+      int r = i / (WN / 4), c = n_w + (i % (WN / 4)) * 4;
       if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
     }
     return;
@@ -701,13 +706,21 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 
   const int nkb = K / 128;
   const int nnb = (N + 127) / 128;
-  const int nw = min(n16 + j, N - 1);
-  const size_t wrow = ((size_t)tile.group * N + nw) * K + kq * 32;
-  const uint8_t* wp = p.rhs + wrow;
-  const uint8_t* up = GLU ? p.rhs_up + wrow : nullptr;
-  const size_t srow = ((size_t)tile.group * nnb + n16 / 128) * nkb;
-  const float* wsp = p.rhs_scale + srow;
-  const float* usp = GLU ? p.rhs_up_scale + srow : nullptr;
+  const uint8_t* wp[NT];
+  const uint8_t* up[NT];
+  const float* wsp[NT];
+  const float* usp[NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const int n16 = n_w + t * 16;
+    const int nw = min(n16 + j, N - 1);
+    const size_t wrow = ((size_t)tile.group * N + nw) * K + kq * 32;
+    wp[t] = p.rhs + wrow;
+    up[t] = GLU ? p.rhs_up + wrow : nullptr;
+    const size_t srow = ((size_t)tile.group * nnb + min(n16, N - 1) / 128) * nkb;
+    wsp[t] = p.rhs_scale + srow;
+    usp[t] = GLU ? p.rhs_up_scale + srow : nullptr;
+  }
   const uint8_t* ap[MT];
   const float* asp[MT];
 #pragma unroll
@@ -716,51 +729,77 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
     ap[mt] = p.lhs + (size_t)gr * K + kq * 32;
     asp[mt] = p.lhs_scale + (size_t)gr * nkb;
   }
-  v4f acc_g[MT], acc_u[MT];
+  v4f acc_g[NT][MT], acc_u[NT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; mt++) {
-    acc_g[mt] = v4f{0.f, 0.f, 0.f, 0.f};
-    acc_u[mt] = v4f{0.f, 0.f, 0.f, 0.f};
-  }
-  const v4f zero = {0.f, 0.f, 0.f, 0.f};
-
-#pragma unroll 4
-  for (int kb = 0; kb < nkb; kb++) {
-    const v8i wf = load32(wp + (size_t)kb * 128);
-    const float ws = wsp[kb];
-    v8i uf;
-    float us = 0.f;
-    if (GLU) {
-      uf = load32(up + (size_t)kb * 128);
-      us = usp[kb];
-    }
+  for (int t = 0; t < NT; t++)
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-      const v8i af = load32(ap[mt] + (size_t)kb * 128);
-      const float as = asp[mt][kb];
-      const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, zero, 0, 0, 0, 127, 0, 127);
-      const float sg = as * ws;
-#pragma unroll
-      for (int r = 0; r < 4; r++) acc_g[mt][r] = fmaf(pg[r], sg, acc_g[mt][r]);
-      if (GLU) {
-        const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf, af, zero, 0, 0, 0, 127, 0, 127);
-        const float su = as * us;
-#pragma unroll
-        for (int r = 0; r < 4; r++) acc_u[mt][r] = fmaf(pu[r], su, acc_u[mt][r]);
-      }
+      acc_g[t][mt] = v4f{0.f, 0.f, 0.f, 0.f};
+      acc_u[t][mt] = v4f{0.f, 0.f, 0.f, 0.f};
     }
-  }
+  const v4f zero = {0.f, 0.f, 0.f, 0.f};
 
-  const int n = n16 + 4 * kq;
-  if (n >= N) return;
+  auto step = [&](int kb0, auto ucount) {
+    constexpr int UC = decltype(ucount)::value;
+    v8i wf[UC][NT], uf[UC][NT], af[UC][MT];
+    float ws[UC][NT], us[UC][NT], as[UC][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; mt++) {
-    const int lr = mt * 16 + j;
-    if (lr >= tile.nrows) continue;
-    float v[4];
+    for (int u = 0; u < UC; u++) {
+      const size_t off = (size_t)(kb0 + u) * 128;
 #pragma unroll
-    for (int r = 0; r < 4; r++) v[r] = GLU ? glu_act(acc_g[mt][r], acc_u[mt][r], p.act, p.act_limit) : acc_g[mt][r];
-    *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      for (int t = 0; t < NT; t++) {
+        wf[u][t] = load32(wp[t] + off);
+        if (GLU) uf[u][t] = load32(up[t] + off);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) af[u][mt] = load32(ap[mt] + off);
+    }
+#pragma unroll
+    for (int u = 0; u < UC; u++) {
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        ws[u][t] = wsp[t][kb0 + u];
+        us[u][t] = GLU ? usp[t][kb0 + u] : 0.f;
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) as[u][mt] = asp[mt][kb0 + u];
+    }
+#pragma unroll
+    for (int u = 0; u < UC; u++)
+#pragma unroll
+      for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+          const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[u][t], af[u][mt], zero, 0, 0, 0, 127, 0, 127);
+          const float sg = as[u][mt] * ws[u][t];
+#pragma unroll
+          for (int r = 0; r < 4; r++) acc_g[t][mt][r] = fmaf(pg[r], sg, acc_g[t][mt][r]);
+          if (GLU) {
+            const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf[u][t], af[u][mt], zero, 0, 0, 0, 127, 0, 127);
+            const float su = as[u][mt] * us[u][t];
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc_u[t][mt][r] = fmaf(pu[r], su, acc_u[t][mt][r]);
+          }
+        }
+  };
+
+  int kb = 0;
+  for (; kb + U <= nkb; kb += U) step(kb, std::integral_constant<int, U>{});
+  for (; kb < nkb; kb++) step(kb, std::integral_constant<int, 1>{});
+
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const int n = n_w + t * 16 + 4 * kq;
+    if (n >= N) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      const int lr = mt * 16 + j;
+      if (lr >= tile.nrows) continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) v[r] = GLU ? glu_act(acc_g[t][mt][r], acc_u[t][mt][r], p.act, p.act_limit) : acc_g[t][mt][r];
+      *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    }
   }
 }
 
@@ -857,15 +896,33 @@ static int launch_tiled_glu(const TiledParams& p, bool glu, int M, int G_total, 
              : launch_tiled_by_rows<OP, BSRC, false>(p, M, G_total, bm_out, dry, s);
 }
 
-template <int MT>
-static int launch_skinny(const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s) {
+template <int MT, int NT, int U>
+static int launch_skinny(SkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
+  p.n_blocks = cdiv(p.N, 64 * NT);
   const long long blocks = (long long)max_tiles * p.n_blocks;
   if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
   if (glu)
-    gmm_fp8_skinny_kernel<MT, true><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_fp8_skinny_kernel<MT, NT, U, true><<<(unsigned)blocks, 256, 0, s>>>(p);
   else
-    gmm_fp8_skinny_kernel<MT, false><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_fp8_skinny_kernel<MT, NT, U, false><<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_launch("gmm_fp8_skinny_kernel");
+}
+
+// reserved[0] can force (NT, U) of the fp8 kernel: id = 100 + 10 * NT + U (tuning aid); 0 picks the default.
+template <int MT>
+static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s) {
+  if (id == 0) id = MT > 1 ? 121 : (glu ? 141 : 124);
+  switch (id) {
+    case 111: return launch_skinny<MT, 1, 1>(p, glu, max_tiles, s);
+    case 112: return launch_skinny<MT, 1, 2>(p, glu, max_tiles, s);
+    case 114: return launch_skinny<MT, 1, 4>(p, glu, max_tiles, s);
+    case 121: return launch_skinny<MT, 2, 1>(p, glu, max_tiles, s);
+    case 122: return launch_skinny<MT, 2, 2>(p, glu, max_tiles, s);
+    case 124: return launch_skinny<MT, 2, 4>(p, glu, max_tiles, s);
+    case 141: return launch_skinny<MT, 4, 1>(p, glu, max_tiles, s);
+    case 142: return launch_skinny<MT, 4, 2>(p, glu, max_tiles, s);
+    default: return fail(MOE_ERR_INVALID_ARG, "gmm: unknown fp8 variant %d", id);
+  }
 }
 
 }  // namespace moe
@@ -907,21 +964,23 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     if (a->lhs_scale_block_k != 128 || a->rhs_scale_block_k != 128 || a->rhs_scale_block_n != 128 || !a->lhs_scale || !a->rhs_scale || (glu && !a->rhs_up_scale))
       return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs 1x128 lhs scales and 128x128 rhs scales");
     if (a->K % 128 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs K %% 128 == 0 (K=%d)", a->K);
-    const long long avg = (long long)a->M / a->num_groups_total;
-    const int mt = avg <= 16 ? 1 : (avg <= 32 ? 2 : 4);
-    bm = 16 * mt;
+    // Few rows per expert (decode): 16-row tiles, one MFMA row tile per wave.  A group with more rows
+    // simply gets several tiles; they are adjacent in the grid, run at the same time and share the group's
+    // weights through L2.  Many rows per expert: 64-row tiles.
+    const bool few_rows = (long long)a->M <= 16LL * a->num_groups_total;
+    bm = few_rows ? 16 : 64;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, header, tiles);
     SkinnyParams p;
     p.lhs = (const uint8_t*)a->lhs; p.lhs_scale = a->lhs_scale;
     p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
     p.rhs_scale = (const float*)a->rhs_scale; p.rhs_up_scale = (const float*)a->rhs_up_scale;
     p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
-    p.M = a->M; p.K = a->K; p.N = a->N; p.n_blocks = cdiv(a->N, 64);
+    p.M = a->M; p.K = a->K; p.N = a->N; p.n_blocks = 0;
     p.act = a->act; p.act_limit = a->act_limit;
     const int mx = max_tiles_for(a->M, a->num_groups_total, bm);
-    if (mt == 1) return launch_skinny<1>(p, glu, mx, s);
-    if (mt == 2) return launch_skinny<2>(p, glu, mx, s);
-    return launch_skinny<4>(p, glu, mx, s);
+    p.min_rows = 1; p.max_rows = bm;
+    if (few_rows) return launch_skinny_variant<1>(a->reserved[0], p, glu, mx, s);
+    return launch_skinny_variant<4>(a->reserved[0], p, glu, mx, s);
   }
 
   TiledParams p;
