@@ -22,6 +22,13 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"int8": 5000.0, "fp8": 5000.0, "bf16": 2500.0}  # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+# scaled by a 1 GiB copy dispatch of the same run (profiles/pmc_traffic_*.md); None where not measured.
+MEASURED_TRAFFIC_BYTES = {
+    "c2": (1962366 * 2.0 + 458788 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
+    "c3": (3805940 * 2.0 + 9245 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
+}
+
 
 def parse():
   ap = argparse.ArgumentParser()
@@ -32,6 +39,8 @@ def parse():
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--calibrate-copy", action="store_true",
+                  help="also run one plain 1 GiB device copy (reference dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   return ap.parse_args()
 
 
@@ -51,7 +60,7 @@ def dominant_kernel_model(wl, group_sizes):
                 name="gmm_fp8_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")
   op = "int8" if cfg.act_quant == "int8" else "bf16"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
-              name="gmm_tiled_kernel (wi_0|wi_1 + SwiGLU)", dtype=op)
+              name=("gmm_dl_kernel" if cfg.act_quant == "int8" else "gmm_tiled_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype=op)
 
 
 def cpu_baseline(wl, layer, sample_tokens):
@@ -144,7 +153,7 @@ def main():
   dom_ms = stage_ms.get("wi_glu")
   achieved = model["work"] / (dom_ms * 1e-3) / model["scale"] if dom_ms else None
   roofline = dict(bound=model["bound"], achieved=achieved, peak=model["peak"], unit=model["unit"],
-                  frac=(achieved / model["peak"]) if achieved else None, traffic=None, kernel=model["name"],
+                  frac=(achieved / model["peak"]) if achieved else None, traffic=MEASURED_TRAFFIC_BYTES.get(wl.name), kernel=model["name"],
                   kernel_ms=dom_ms)
 
   flops = synthetic.layer_flops(wl)
@@ -179,8 +188,15 @@ def main():
   min_bytes = nonempty * synthetic.weight_bytes_per_expert(wl) + wl.tokens * cfg.emb_dim * 2 * 2
   result["layer_gbps"] = min_bytes / (elapsed / args.steps) / 1e9
 
+  if args.calibrate_copy:
+    src = torch.ones((1 << 28,), dtype=torch.int32, device="cuda")
+    dst = torch.empty_like(src)
+    torch.add(src, 1, out=dst)  # reads 1 GiB, writes 1 GiB
+    torch.cuda.synchronize()
+    del src, dst
+
   if not args.no_cpu_baseline:
-    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 256, "c3": 16, "c4": 1024, "c5": 256}[wl.name]
+    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048}[wl.name]
     del out
     result["cpu_baseline"] = cpu_baseline(wl, layer, sample)
   print(json.dumps(result))
