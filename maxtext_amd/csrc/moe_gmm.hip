@@ -579,73 +579,100 @@ __global__ __launch_bounds__(C::THREADS) void gmm_dl_kernel(const TiledParams p)
   const int row_off = lrow * C::BKB;
 
   // Fragments are double-buffered in registers: while the MFMAs of k-step ks run, the b128 reads of the
-  // next k-step (possibly the first one of the next stage) are already in flight.
+  // next k-step (possibly the first one of the next stage) are in flight.  LDS reads and global->LDS
+  // requests are issued one at a time between MFMAs: a wave issues in order, so a burst of 4 loads + 6 reads
+  // from all 8 waves right after the barrier would park every wave behind the address queues while the
+  // MFMA pipes run dry.
   v4i fa[2][C::TM], fb[2][C::TN];
-  auto load_frags = [&](int buf, int ks, int set) {
-    const uint8_t* sa = smem + buf * C::STAGE + (wm * C::WM) * C::BKB + row_off;
-    const uint8_t* sb = smem + buf * C::STAGE + C::BM * C::BKB + row_off;
+  auto read_frag = [&](int buf, int ks, int set, int f) {
     const int koff = t16 ^ (ks * 32);
-#pragma unroll
-    for (int i = 0; i < C::TM; i++) fa[set][i] = *(const v4i*)(sa + i * 32 * C::BKB + koff);
-#pragma unroll
-    for (int j = 0; j < C::TN; j++) fb[set][j] = *(const v4i*)(sb + b_row[j] * C::BKB + koff);
+    if (f < C::TM) {
+      fa[set][f] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + f * 32) * C::BKB + row_off + koff);
+    } else {
+      fb[set][f - C::TM] = *(const v4i*)(smem + buf * C::STAGE + (C::BM + b_row[f - C::TM]) * C::BKB + row_off + koff);
+    }
   };
-  auto mfma_frags = [&](int set) {
-#pragma unroll
-    for (int j = 0; j < C::TN; j++)
-#pragma unroll
-      for (int i = 0; i < C::TM; i++) {
-        if constexpr (OP == OP_I8) {
-          acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
-        } else {
-          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              __builtin_bit_cast(v8bf, fb[set][j]), __builtin_bit_cast(v8bf, fa[set][i]), acc[j][i], 0, 0, 0);
-        }
-      }
+  auto issue_one = [&](int kt, int buf, int idx) {
+    const size_t koff = (size_t)kt * C::BKB;
+    uint8_t* s = smem + buf * C::STAGE;
+    if (idx < C::A_IPW) {
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[idx] + koff), (lds_ptr_t)(s + (wave * C::A_IPW + idx) * 1024), 16, 0, 0);
+    } else {
+      const int i = idx - C::A_IPW;
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
+                                       (lds_ptr_t)(s + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+    }
   };
+  auto mfma_one = [&](int set, int idx) {
+    const int j = idx / C::TM, i = idx % C::TM;
+    if constexpr (OP == OP_I8) {
+      acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
+    } else {
+      acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+          __builtin_bit_cast(v8bf, fb[set][j]), __builtin_bit_cast(v8bf, fa[set][i]), acc[j][i], 0, 0, 0);
+    }
+  };
+  constexpr int NMFMA = C::TM * C::TN, NFRAG = C::TM + C::TN;
+  constexpr int HALF = C::LPS / 2;  // a stage's requests are split over two k-steps
+  static_assert(NFRAG <= NMFMA && C::LPS % 2 == 0 && HALF <= NMFMA / 2, "interleave shape");
+  // One k-step: MFMAs on register set SET with, slotted between them, the fragment reads of the next
+  // k-step (RD) and HALF of a stage's requests (LD).  SET / RD / LD are compile-time so that the body is
+  // straight-line code.
+  auto kstep = [&](auto set_c, auto rd_c, auto ld_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf, int ld_first) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
+#pragma unroll
+    for (int idx = 0; idx < NMFMA; idx++) {
+      mfma_one(SET, idx);
+      if (RD && idx < NFRAG) read_frag(rd_buf, rd_ks, SET ^ 1, idx);
+      if (LD && (idx & 1) && idx / 2 < HALF) issue_one(ld_kt, ld_buf, ld_first + idx / 2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): long satisfied by the time the last MFMA has issued
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
 
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
   const int n_out0 = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
   EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
 
   // ---- pipeline -----------------------------------------------------------------------------------
-  // Stages 0..NSTAGE-2 are requested up front.  In iteration kt, just before the last k-step's MFMAs,
-  // the wave waits for its own loads of stage kt+1, meets the others at a bare barrier (stage kt+1 is
-  // then complete in LDS and nobody reads stage kt-1's buffer any more), requests stage kt+NSTAGE-1
-  // into that free buffer, and prefetches stage kt+1's first fragments.  __syncthreads() is not used:
-  // its fence would drain vmcnt to 0 and with it the loads that are meant to stay in flight.
-  static_assert(C::KSUB % 2 == 0 && C::NSTAGE >= 3, "pipeline shape");
+  // A stage's requests are issued in two halves: the first during the last k-step of iteration kt (right
+  // after the barrier that proves buffer (kt-1) % NSTAGE free), the second during the first k-step of
+  // iteration kt+1.  Before the last k-step of iteration kt the wave waits for its own loads of stage
+  // kt+1 and meets the others at a bare barrier: stage kt+1 is then complete in LDS and nobody reads stage
+  // kt-1's buffer any more.  __syncthreads() is not used: its fence would drain vmcnt to 0 and with it the
+  // loads that are meant to stay in flight.  Requests past the last stage re-read the last stage into a
+  // buffer nobody reads again, which keeps the vmcnt bookkeeping uniform.
+  static_assert(C::KSUB == 2 && C::NSTAGE >= 3, "pipeline shape");
   const int nk = K / C::BK;
   // (issued before the first stage so that the vmcnt bookkeeping below only ever counts stage loads)
   load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, tile, wm * C::WM, n_out0, lane);
 #pragma unroll
-  for (int s = 0; s < C::NSTAGE - 1; s++)
-    if (s < nk) issue_stage(s, s);
-  if (nk >= C::NSTAGE - 1) wait_vmcnt<(C::NSTAGE - 2) * C::LPS>(); else wait_vmcnt<0>();
-  asm volatile("s_barrier" ::: "memory");
-  load_frags(0, 0, 0);
-  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
-  for (int kt = 0; kt < nk; kt++) {
-    const int buf = kt % C::NSTAGE;
+  for (int s = 0; s < C::NSTAGE - 2; s++) issue_stage(min(s, nk - 1), s);
 #pragma unroll
-    for (int ks = 0; ks < C::KSUB; ks++) {
-      if (ks + 1 < C::KSUB) {
-        load_frags(buf, ks + 1, (ks + 1) & 1);
-      } else if (kt + 1 < nk) {
-        if (kt + C::NSTAGE - 1 <= nk) wait_vmcnt<(C::NSTAGE - 3) * C::LPS>(); else wait_vmcnt<0>();
-        asm volatile("s_barrier" ::: "memory");
-        if (kt + C::NSTAGE - 1 < nk) issue_stage(kt + C::NSTAGE - 1, (kt + C::NSTAGE - 1) % C::NSTAGE);
-        load_frags((kt + 1) % C::NSTAGE, 0, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_frags(ks & 1);
-      // By the time the last of these MFMAs has issued, the prefetched fragments have long arrived; waiting
-      // for them here (and not at the top of the next k-step) keeps that k-step's MFMAs free of LDS waits.
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-      __builtin_amdgcn_sched_barrier(0);
-    }
+  for (int i = 0; i < HALF; i++) issue_one(min(C::NSTAGE - 2, nk - 1), C::NSTAGE - 2, i);
+  wait_vmcnt<(C::NSTAGE - 3) * C::LPS + HALF>();
+  asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+  for (int f = 0; f < NFRAG; f++) read_frag(0, 0, 0, f);
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
+  int kt = 0;
+  for (; kt + 1 < nk; kt++) {
+    const int buf = kt % C::NSTAGE;
+    const int kb = kt + C::NSTAGE - 2, ka = kt + C::NSTAGE - 1;
+    kstep(S0{}, T_{}, T_{}, buf, 1, min(kb, nk - 1), kb % C::NSTAGE, HALF);
+    wait_vmcnt<(C::NSTAGE - 3) * C::LPS>();
+    asm volatile("s_barrier" ::: "memory");
+    kstep(S1{}, T_{}, T_{}, (kt + 1) % C::NSTAGE, 0, min(ka, nk - 1), ka % C::NSTAGE, 0);
   }
+  kstep(S0{}, T_{}, F_{}, kt % C::NSTAGE, 1, 0, 0, 0);
+  kstep(S1{}, F_{}, F_{}, 0, 0, 0, 0, 0);
+  wait_vmcnt<0>();  // no request of this block may still be writing LDS when the block retires
 
   store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, tile, wm * C::WM, n_out0, lane);
 }
