@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "moe_mi355x.h"
 
 namespace moe {
@@ -60,20 +62,31 @@ __device__ __forceinline__ float sigmoidf_(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
-// gate/up -> activation, computed in f32 (moe.py:841-870).
-__device__ __forceinline__ float glu_act(float g, float u, int act, float limit) {
-  if (act == MOE_ACT_SILU) return g * sigmoidf_(g) * u;
-  if (act == MOE_ACT_SWIGLUOAI) {
+// gate/up -> activation, computed in f32 (moe.py:841-870).  ACT is a compile-time moe_act so that the
+// epilogues stay straight-line code.
+template <int ACT>
+__device__ __forceinline__ float glu_act(float g, float u, float limit) {
+  if (ACT == MOE_ACT_SILU) return g * sigmoidf_(g) * u;
+  if (ACT == MOE_ACT_SWIGLUOAI) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
     return g * sigmoidf_(1.702f * g) * (u + 1.0f);
   }
-  if (act == MOE_ACT_SILU_CLIP) {
+  if (ACT == MOE_ACT_SILU_CLIP) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
     return g * sigmoidf_(g) * u;
   }
   return g;
+}
+
+// Calls f(std::integral_constant<int, act>) with the runtime activation turned into a constant.
+template <typename F>
+__device__ __forceinline__ void dispatch_act(int act, F&& f) {
+  if (act == MOE_ACT_SILU) f(std::integral_constant<int, MOE_ACT_SILU>{});
+  else if (act == MOE_ACT_SWIGLUOAI) f(std::integral_constant<int, MOE_ACT_SWIGLUOAI>{});
+  else if (act == MOE_ACT_SILU_CLIP) f(std::integral_constant<int, MOE_ACT_SILU_CLIP>{});
+  else f(std::integral_constant<int, MOE_ACT_NONE>{});
 }
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }

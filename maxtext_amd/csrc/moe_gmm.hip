@@ -166,6 +166,8 @@ __device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, 
 template <int TM, int TN, int NT_OUT, bool GLU, typename acc_t>
 __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
                                                const TiledParams& p, const TileInfo& tile, int row_base, int n_base, int lane) {
+  dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
+  constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
   for (int i = 0; i < TM; i++) {
     const int lr = row_base + i * 32 + (lane % 32);
@@ -185,7 +187,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
           const float g = (float)acc[j][i][4 * q + r] * (e.sa[i] * sg[r]);
           if (GLU) {
             const float u = (float)acc[j + NT_OUT][i][4 * q + r] * (e.sa[i] * su[r]);
-            v[r] = glu_act(g, u, p.act, p.act_limit);
+            v[r] = glu_act<ACT>(g, u, p.act_limit);
           } else {
             v[r] = g;
           }
@@ -193,6 +195,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
         *(uint2*)(orow + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
       }
   }
+  });
 }
 
 template <int OP_, int BSRC_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, bool GLU_>
@@ -814,20 +817,23 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
   for (; kb + U <= nkb; kb += U) step(kb, std::integral_constant<int, U>{});
   for (; kb < nkb; kb++) step(kb, std::integral_constant<int, 1>{});
 
+  dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
-  for (int t = 0; t < NT; t++) {
-    const int n = n_w + t * 16 + 4 * kq;
-    if (n >= N) continue;
+    for (int t = 0; t < NT; t++) {
+      const int n = n_w + t * 16 + 4 * kq;
+      if (n >= N) continue;
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-      const int lr = mt * 16 + j;
-      if (lr >= tile.nrows) continue;
-      float v[4];
+      for (int mt = 0; mt < MT; mt++) {
+        const int lr = mt * 16 + j;
+        if (lr >= tile.nrows) continue;
+        float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; r++) v[r] = GLU ? glu_act(acc_g[t][mt][r], acc_u[t][mt][r], p.act, p.act_limit) : acc_g[t][mt][r];
-      *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        for (int r = 0; r < 4; r++) v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r], acc_u[t][mt][r], p.act_limit) : acc_g[t][mt][r];
+        *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
     }
-  }
+  });
 }
 
 // ---------------------------------------------------------------------------------------
