@@ -837,6 +837,175 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 }
 
 // ---------------------------------------------------------------------------------------
+// Weight-only int8 / int4 for few rows per expert (decode): bf16 activations, weights widened to bf16 in
+// registers, v_mfma_f32_16x16x32_bf16.  Same streaming structure as the fp8 kernel: no LDS, one wave owns
+// 16*NT output channels and walks K in 128-element blocks; lane (n = lane%16, kq = lane/16) holds the 32
+// consecutive k values kq*32.. of the block for its channel (one 16-byte load for int4, two for int8) and
+// the matching 64 bytes of its activation row.  int4 weights are multiplied by their group-128 scale while
+// they are widened; the int8 per-channel scale is applied once at the end.
+// ---------------------------------------------------------------------------------------
+
+struct WqSkinnyParams {
+  const uint8_t* lhs;       // [M, K] bf16
+  const uint8_t* rhs;       // [G, N, K] int8 or [G, N, K/2] packed int4
+  const uint8_t* rhs_up;
+  const void* rhs_scale;    // int8: f32 [G, N]; int4: bf16 [G, N, ceil(K/128)]
+  const void* rhs_up_scale;
+  const int32_t* header;
+  const TileInfo* tiles;
+  uint16_t* out;
+  int M, K, N;
+  int n_blocks;
+  int act;
+  float act_limit;
+};
+
+template <bool INT4>
+__device__ __forceinline__ void widen32(const uint8_t* p, float scale, v8bf (&w)[4]) {
+  if (INT4) {
+    const uint4 q = *(const uint4*)p;
+    const uint32_t x[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      uint32_t o[4];
+#pragma unroll
+      for (int h = 0; h < 4; h++) {
+        const int lo = (int)((x[s] >> (8 * h)) & 0xf) - 8, hi = (int)((x[s] >> (8 * h + 4)) & 0xf) - 8;
+        o[h] = pack_bf16x2((float)lo * scale, (float)hi * scale);
+      }
+      w[s] = __builtin_bit_cast(v8bf, make_uint4(o[0], o[1], o[2], o[3]));
+    }
+  } else {
+    const uint4 q0 = *(const uint4*)p, q1 = *(const uint4*)(p + 16);
+    const uint32_t x[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      uint32_t o[4];
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int v = (int)x[2 * s + h];
+        o[2 * h] = i8x2_to_bf16x2((v << 24) >> 24, (v << 16) >> 24);
+        o[2 * h + 1] = i8x2_to_bf16x2((v << 8) >> 24, v >> 24);
+      }
+      w[s] = __builtin_bit_cast(v8bf, make_uint4(o[0], o[1], o[2], o[3]));
+    }
+  }
+}
+
+template <bool INT4, int MT, int NT, bool GLU>
+__global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams p) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int j = lane % 16, kq = lane / 16;
+  const int m_idx = blockIdx.x / p.n_blocks;
+  if (m_idx >= p.header[0]) return;
+  const TileInfo tile = p.tiles[m_idx];
+  const int N = p.N, K = p.K;
+  constexpr int WN = 16 * NT;
+  const int n_w = (blockIdx.x % p.n_blocks) * (4 * WN) + wave * WN;
+  if (n_w >= N) return;
+
+  if (tile.group < 0) {
+    for (int i = lane; i < tile.nrows * (WN / 4); i += kWave) {
+      int r = i / (WN / 4), c = n_w + (i % (WN / 4)) * 4;
+      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  const int nkb = (K + 127) / 128;  // the last block may be partial (K % 32 == 0)
+  const size_t wrow_bytes = INT4 ? (size_t)K / 2 : (size_t)K;
+  const uint8_t* wp[NT];
+  const uint8_t* up[NT];
+  const uint16_t* wsp[NT];
+  const uint16_t* usp[NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const int nw = min(n_w + t * 16 + j, N - 1);
+    const size_t row = (size_t)tile.group * N + nw;
+    wp[t] = p.rhs + row * wrow_bytes + kq * (INT4 ? 16 : 32);
+    up[t] = GLU ? p.rhs_up + row * wrow_bytes + kq * (INT4 ? 16 : 32) : nullptr;
+    wsp[t] = INT4 ? (const uint16_t*)p.rhs_scale + row * nkb : nullptr;
+    usp[t] = INT4 && GLU ? (const uint16_t*)p.rhs_up_scale + row * nkb : nullptr;
+  }
+  const uint8_t* ap[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int gr = tile.row0 + min(mt * 16 + j, tile.nrows - 1);
+    ap[mt] = p.lhs + ((size_t)gr * K + kq * 32) * 2;
+  }
+  v4f acc_g[NT][MT], acc_u[NT][MT];
+#pragma unroll
+  for (int t = 0; t < NT; t++)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      acc_g[t][mt] = v4f{0.f, 0.f, 0.f, 0.f};
+      acc_u[t][mt] = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+
+  for (int kb = 0; kb < nkb; kb++) {
+    // this lane's 32 k values exist unless the block is the partial tail
+    const bool live = kb * 128 + kq * 32 < K;
+    const size_t woff = live ? (size_t)kb * (INT4 ? 64 : 128) : 0;
+    v8bf af[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      const uint8_t* a = ap[mt] + (live ? (size_t)kb * 256 : 0);
+#pragma unroll
+      for (int s = 0; s < 4; s++) {
+        uint4 v = *(const uint4*)(a + s * 16);
+        if (!live) v = make_uint4(0, 0, 0, 0);
+        af[mt][s] = __builtin_bit_cast(v8bf, v);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      v8bf wf[4], uf[4];
+      const float ws = INT4 ? bf16_bits_to_f32(wsp[t][kb]) : 1.0f;
+      widen32<INT4>(wp[t] + woff, ws, wf);
+      if (GLU) {
+        const float us = INT4 ? bf16_bits_to_f32(usp[t][kb]) : 1.0f;
+        widen32<INT4>(up[t] + woff, us, uf);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          acc_g[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af[mt][s], acc_g[t][mt], 0, 0, 0);
+          if (GLU) acc_u[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[s], af[mt][s], acc_u[t][mt], 0, 0, 0);
+        }
+    }
+  }
+
+  dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      const int n = n_w + t * 16 + 4 * kq;
+      if (n >= N) continue;
+      float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
+      if (!INT4) {
+        const float4 a = *(const float4*)((const float*)p.rhs_scale + (size_t)tile.group * N + n);
+        sg[0] = a.x; sg[1] = a.y; sg[2] = a.z; sg[3] = a.w;
+        if (GLU) {
+          const float4 b = *(const float4*)((const float*)p.rhs_up_scale + (size_t)tile.group * N + n);
+          su[0] = b.x; su[1] = b.y; su[2] = b.z; su[3] = b.w;
+        }
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int lr = mt * 16 + j;
+        if (lr >= tile.nrows) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r] * sg[r], acc_u[t][mt][r] * su[r], p.act_limit) : acc_g[t][mt][r] * sg[r];
+        *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
+    }
+  });
+}
+
+// ---------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------
 
@@ -958,6 +1127,19 @@ static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int ma
   }
 }
 
+template <bool INT4, int MT>
+static int launch_wq_skinny(WqSkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
+  constexpr int NT = 2;
+  p.n_blocks = cdiv(p.N, 64 * NT);
+  const long long blocks = (long long)max_tiles * p.n_blocks;
+  if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  if (glu)
+    gmm_wq_skinny_kernel<INT4, MT, NT, true><<<(unsigned)blocks, 256, 0, s>>>(p);
+  else
+    gmm_wq_skinny_kernel<INT4, MT, NT, false><<<(unsigned)blocks, 256, 0, s>>>(p);
+  return check_launch("gmm_wq_skinny_kernel");
+}
+
 }  // namespace moe
 
 using namespace moe;
@@ -1049,8 +1231,22 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     return fail(MOE_ERR_UNSUPPORTED, "gmm: lhs_dtype %d x rhs_dtype %d", L, R);
   }
 
-  // dry run to learn the m-tile, then build the tile list and launch
   const int M = a->M, G = a->num_groups_total;
+  // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
+  if ((variant == V_W8 || variant == V_W4) && (long long)M <= 32LL * G && a->reserved[0] != 1) {
+    const bool one = (long long)M <= 16LL * G;
+    bm = one ? 16 : 32;
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
+    WqSkinnyParams q;
+    q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
+    q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
+    q.header = header; q.tiles = tiles; q.out = (uint16_t*)a->out;
+    q.M = M; q.K = a->K; q.N = a->N; q.n_blocks = 0; q.act = a->act; q.act_limit = a->act_limit;
+    const int mx = max_tiles_for(M, G, bm);
+    if (variant == V_W4) return one ? launch_wq_skinny<true, 1>(q, glu, mx, s) : launch_wq_skinny<true, 2>(q, glu, mx, s);
+    return one ? launch_wq_skinny<false, 1>(q, glu, mx, s) : launch_wq_skinny<false, 2>(q, glu, mx, s);
+  }
+  // dry run to learn the m-tile, then build the tile list and launch
   const int forced = a->reserved[0];
   if (forced >= 3 && variant == V_I8) {
     int st = glu ? launch_i8_variant<true>(forced, p, M, G, &bm, true, s) : launch_i8_variant<false>(forced, p, M, G, &bm, true, s);
