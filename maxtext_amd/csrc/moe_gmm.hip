@@ -493,78 +493,86 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 template <typename C>
-__global__ __launch_bounds__(C::THREADS) void gmm_dl_kernel(const TiledParams p) {
+__global__ __launch_bounds__(C::THREADS, 2) void gmm_dl_kernel(const TiledParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   constexpr int OP = C::OP;
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
+  const int N = p.N, K = p.K;
+  const size_t row_bytes = (size_t)K * C::ESZ;
+  const int num_tiles = p.header[0];
+  const int total = p.max_m_tiles * p.tiles_n;
 
-  int m_idx, n_idx;
-  {
-    const int nb = gridDim.x, pid = blockIdx.x;
-    const int q = nb / 8, rem = nb % 8, xcd = pid % 8, loc = pid / 8;
+  // Persistent blocks: block b works on tile ids b, b + gridDim.x, ...  A tile id is turned into (m-tile,
+  // n-tile) so that ids that run at the same time on one XCD (ids congruent mod 8 go to the same XCD) form
+  // a GSM x (32 / GSM) patch sharing activation and weight panels in that XCD's L2.
+  struct Tile {
+    TileInfo info;
+    int n0;
+  };
+  auto locate = [&](int id, Tile& t) -> bool {
+    const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
-    constexpr int GSM = 4;
+    const int GSM = p.dbg > 0 ? p.dbg : 8;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
     const int gsz = min(p.max_m_tiles - first_m, GSM);
-    m_idx = first_m + (logical % width) % gsz;
-    n_idx = (logical % width) / gsz;
-  }
-  if (m_idx >= p.header[0]) return;
-  const TileInfo tile = p.tiles[m_idx];
-  const int n0 = n_idx * C::OUT_BN;
-  const int N = p.N, K = p.K;
-
-  if (tile.group < 0) {
-    constexpr int QPR = C::OUT_BN / 4;
-    for (int i = tid; i < tile.nrows * QPR; i += C::THREADS) {
-      int r = i / QPR, c = n0 + (i % QPR) * 4;
-      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    const int m_idx = first_m + (logical % width) % gsz;
+    if (m_idx >= num_tiles) return false;
+    t.info = p.tiles[m_idx];
+    t.n0 = ((logical % width) / gsz) * C::OUT_BN;
+    return true;
+  };
+  // Advances `id` to this block's next tile that needs the matmul; tiles of rows that belong to no local
+  // group are written as zeros on the way.
+  auto next_compute_tile = [&](int& id, Tile& t) -> bool {
+    for (; id < total; id += gridDim.x) {
+      if (!locate(id, t)) continue;
+      if (t.info.group >= 0) return true;
+      constexpr int QPR = C::OUT_BN / 4;
+      for (int i = tid; i < t.info.nrows * QPR; i += C::THREADS) {
+        int r = i / QPR, c = t.n0 + (i % QPR) * 4;
+        if (c < N) *(uint2*)(p.out + (size_t)(t.info.row0 + r) * N + c) = make_uint2(0, 0);
+      }
     }
-    return;
-  }
+    return false;
+  };
 
   // ---- per-lane source addresses of this wave's load instructions ---------------------------
-  const size_t row_bytes = (size_t)K * C::ESZ;
   const uint8_t* a_src[C::A_IPW];
   const uint8_t* b_src[C::B_IPW];
+  auto set_sources = [&](const Tile& t) {
 #pragma unroll
-  for (int i = 0; i < C::A_IPW; i++) {
-    const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
-    const int q = (lane % C::CPR) ^ C::swz(r);
-    a_src[i] = p.lhs + (size_t)(tile.row0 + min(r, tile.nrows - 1)) * row_bytes + q * 16;
-  }
+    for (int i = 0; i < C::A_IPW; i++) {
+      const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
+      const int q = (lane % C::CPR) ^ C::swz(r);
+      a_src[i] = p.lhs + (size_t)(t.info.row0 + min(r, t.info.nrows - 1)) * row_bytes + q * 16;
+    }
 #pragma unroll
-  for (int i = 0; i < C::B_IPW; i++) {
-    const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
-    const int q = (lane % C::CPR) ^ C::swz(vr);
-    const bool up = C::GLU && vr >= C::BN / 2;
-    const int n = min(n0 + (up ? vr - C::BN / 2 : vr), N - 1);
-    b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)tile.group * N + n) * row_bytes + q * 16;
-  }
+    for (int i = 0; i < C::B_IPW; i++) {
+      const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
+      const int q = (lane % C::CPR) ^ C::swz(vr);
+      const bool up = C::GLU && vr >= C::BN / 2;
+      const int n = min(t.n0 + (up ? vr - C::BN / 2 : vr), N - 1);
+      b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)t.info.group * N + n) * row_bytes + q * 16;
+    }
+  };
 
-  auto issue_stage = [&](int kt, int buf) {
+  auto issue_one = [&](int kt, int buf, int idx) {
     const size_t koff = (size_t)kt * C::BKB;
     uint8_t* s = smem + buf * C::STAGE;
-#pragma unroll
-    for (int i = 0; i < C::A_IPW; i++)
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[i] + koff), (lds_ptr_t)(s + (wave * C::A_IPW + i) * 1024), 16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < C::B_IPW; i++)
+    if (idx < C::A_IPW) {
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[idx] + koff), (lds_ptr_t)(s + (wave * C::A_IPW + idx) * 1024), 16, 0, 0);
+    } else {
+      const int i = idx - C::A_IPW;
       __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
                                        (lds_ptr_t)(s + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+    }
   };
 
   typedef typename std::conditional<OP == OP_I8, v16i, v16f>::type acc_t;
   acc_t acc[C::TN][C::TM];
-#pragma unroll
-  for (int j = 0; j < C::TN; j++)
-#pragma unroll
-    for (int i = 0; i < C::TM; i++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
 
   int b_row[C::TN];
 #pragma unroll
@@ -593,17 +601,6 @@ __global__ __launch_bounds__(C::THREADS) void gmm_dl_kernel(const TiledParams p)
       fa[set][f] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + f * 32) * C::BKB + row_off + koff);
     } else {
       fb[set][f - C::TM] = *(const v4i*)(smem + buf * C::STAGE + (C::BM + b_row[f - C::TM]) * C::BKB + row_off + koff);
-    }
-  };
-  auto issue_one = [&](int kt, int buf, int idx) {
-    const size_t koff = (size_t)kt * C::BKB;
-    uint8_t* s = smem + buf * C::STAGE;
-    if (idx < C::A_IPW) {
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[idx] + koff), (lds_ptr_t)(s + (wave * C::A_IPW + idx) * 1024), 16, 0, 0);
-    } else {
-      const int i = idx - C::A_IPW;
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
-                                       (lds_ptr_t)(s + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
     }
   };
   auto mfma_one = [&](int set, int idx) {
@@ -640,8 +637,18 @@ __global__ __launch_bounds__(C::THREADS) void gmm_dl_kernel(const TiledParams p)
   using S1 = std::integral_constant<int, 1>;
 
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
-  const int n_out0 = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
-  EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+  static_assert(C::KSUB == 2 && C::NSTAGE >= 3, "pipeline shape");
+  const int nk = K / C::BK;
+
+  // Requests of a tile's first stages: stages 0..NSTAGE-3 in full and the first half of stage NSTAGE-2.
+  auto issue_prologue = [&]() {
+#pragma unroll
+    for (int s = 0; s < C::NSTAGE - 2; s++)
+#pragma unroll
+      for (int i = 0; i < C::LPS; i++) issue_one(min(s, nk - 1), s, i);
+#pragma unroll
+    for (int i = 0; i < HALF; i++) issue_one(min(C::NSTAGE - 2, nk - 1), C::NSTAGE - 2, i);
+  };
 
   // ---- pipeline -----------------------------------------------------------------------------------
   // A stage's requests are issued in two halves: the first during the last k-step of iteration kt (right
@@ -651,33 +658,57 @@ __global__ __launch_bounds__(C::THREADS) void gmm_dl_kernel(const TiledParams p)
   // kt-1's buffer any more.  __syncthreads() is not used: its fence would drain vmcnt to 0 and with it the
   // loads that are meant to stay in flight.  Requests past the last stage re-read the last stage into a
   // buffer nobody reads again, which keeps the vmcnt bookkeeping uniform.
-  static_assert(C::KSUB == 2 && C::NSTAGE >= 3, "pipeline shape");
-  const int nk = K / C::BK;
-  // (issued before the first stage so that the vmcnt bookkeeping below only ever counts stage loads)
-  load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, tile, wm * C::WM, n_out0, lane);
-#pragma unroll
-  for (int s = 0; s < C::NSTAGE - 2; s++) issue_stage(min(s, nk - 1), s);
-#pragma unroll
-  for (int i = 0; i < HALF; i++) issue_one(min(C::NSTAGE - 2, nk - 1), C::NSTAGE - 2, i);
-  wait_vmcnt<(C::NSTAGE - 3) * C::LPS + HALF>();
-  asm volatile("s_barrier" ::: "memory");
-#pragma unroll
-  for (int f = 0; f < NFRAG; f++) read_frag(0, 0, 0, f);
-  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
-  int kt = 0;
-  for (; kt + 1 < nk; kt++) {
-    const int buf = kt % C::NSTAGE;
-    const int kb = kt + C::NSTAGE - 2, ka = kt + C::NSTAGE - 1;
-    kstep(S0{}, T_{}, T_{}, buf, 1, min(kb, nk - 1), kb % C::NSTAGE, HALF);
-    wait_vmcnt<(C::NSTAGE - 3) * C::LPS>();
-    asm volatile("s_barrier" ::: "memory");
-    kstep(S1{}, T_{}, T_{}, (kt + 1) % C::NSTAGE, 0, min(ka, nk - 1), ka % C::NSTAGE, 0);
+  // Across tiles: once a tile's last k-step has been issued, the first stages of the block's next tile are
+  // requested, so they travel while the epilogue of the finished tile runs.
+  int id = blockIdx.x;
+  Tile cur;
+  bool have = next_compute_tile(id, cur);
+  if (have) {
+    set_sources(cur);
+    issue_prologue();
   }
-  kstep(S0{}, T_{}, F_{}, kt % C::NSTAGE, 1, 0, 0, 0);
-  kstep(S1{}, F_{}, F_{}, 0, 0, 0, 0, 0);
-  wait_vmcnt<0>();  // no request of this block may still be writing LDS when the block retires
-
-  store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, tile, wm * C::WM, n_out0, lane);
+  while (have) {
+#pragma unroll
+    for (int j = 0; j < C::TN; j++)
+#pragma unroll
+      for (int i = 0; i < C::TM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
+    // every request of the prologue (and every store of the previous epilogue) has completed
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+    for (int f = 0; f < NFRAG; f++) read_frag(0, 0, 0, f);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
+    int kt = 0;
+    for (; kt + 1 < nk; kt++) {
+      const int buf = kt % C::NSTAGE;
+      const int kb = kt + C::NSTAGE - 2, ka = kt + C::NSTAGE - 1;
+      kstep(S0{}, T_{}, T_{}, buf, 1, min(kb, nk - 1), kb % C::NSTAGE, HALF);
+      wait_vmcnt<(C::NSTAGE - 3) * C::LPS>();
+      asm volatile("s_barrier" ::: "memory");
+      kstep(S1{}, T_{}, T_{}, (kt + 1) % C::NSTAGE, 0, min(ka, nk - 1), ka % C::NSTAGE, 0);
+    }
+    // the epilogue's scales are fetched behind the last two k-steps
+    const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+    EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+    load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, cur.info, wm * C::WM, n_out0, lane);
+    kstep(S0{}, T_{}, F_{}, kt % C::NSTAGE, 1, 0, 0, 0);
+    kstep(S1{}, F_{}, F_{}, 0, 0, 0, 0, 0);
+    // all LDS reads of this tile are done in every wave and no request is still writing LDS: the buffers
+    // can take the next tile's first stages
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    const Tile done = cur;
+    id += gridDim.x;
+    have = next_compute_tile(id, cur);
+    if (have) {
+      set_sources(cur);
+      issue_prologue();
+    }
+    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, done.info, wm * C::WM, n_out0, lane);
+  }
+  wait_vmcnt<0>();
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1037,8 +1068,19 @@ static int launch_dl(const TiledParams& p0, int M, int G_total, hipStream_t s) {
   TiledParams p = p0;
   p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
   p.tiles_n = cdiv(p.N, C::OUT_BN);
-  const long long blocks = (long long)p.max_m_tiles * p.tiles_n;
-  if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  const long long tiles = (long long)p.max_m_tiles * p.tiles_n;
+  if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  // one persistent block per CU (the LDS footprint allows no more); a multiple of 8 keeps "tile id mod 8"
+  // equal to the XCD a block runs on
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return fail(MOE_ERR_LAUNCH, "gmm: cannot query the CU count");
+    num_cus = n;
+  }
+  long long blocks = tiles < num_cus ? tiles : num_cus;
+  if (blocks >= 8) blocks -= blocks % 8;
   gmm_dl_kernel<C><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
   return check_launch("gmm_dl_kernel");
 }
@@ -1084,10 +1126,8 @@ static int launch_i8_variant(int id, const TiledParams& p, int M, int G_total, i
   MOE_DL_VARIANT(10, 256, 256, 64, 2, 4, 5)
   MOE_DL_VARIANT(11, 256, 256, 64, 2, 4, 3)
   MOE_DL_VARIANT(12, 256, 256, 64, 2, 4, 4)
-  MOE_DL_VARIANT(13, 256, 256, 64, 2, 2, 3)
-  MOE_DL_VARIANT(14, 256, 256, 64, 2, 2, 4)
-  MOE_DL_VARIANT(15, 128, 256, 64, 2, 2, 4)
-  MOE_DL_VARIANT(16, 256, 128, 64, 2, 2, 4)
+  MOE_DL_VARIANT(17, 256, 128, 64, 2, 2, 3)
+  MOE_DL_VARIANT(18, 128, 256, 64, 2, 2, 3)
 #undef MOE_DL_VARIANT
   return fail(MOE_ERR_INVALID_ARG, "gmm: unknown tile variant %d", id);
 }
