@@ -493,7 +493,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 template <typename C>
-__global__ __launch_bounds__(C::THREADS, 2) void gmm_dl_kernel(const TiledParams p) {
+__global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_kernel(const TiledParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   constexpr int OP = C::OP;
   const int tid = threadIdx.x, lane = tid % kWave;
@@ -1126,8 +1126,8 @@ static int launch_i8_variant(int id, const TiledParams& p, int M, int G_total, i
   MOE_DL_VARIANT(10, 256, 256, 64, 2, 4, 5)
   MOE_DL_VARIANT(11, 256, 256, 64, 2, 4, 3)
   MOE_DL_VARIANT(12, 256, 256, 64, 2, 4, 4)
-  MOE_DL_VARIANT(17, 256, 128, 64, 2, 2, 3)
-  MOE_DL_VARIANT(18, 128, 256, 64, 2, 2, 3)
+  MOE_DL_VARIANT(14, 256, 256, 64, 2, 2, 4)
+  MOE_DL_VARIANT(15, 256, 256, 64, 2, 2, 5)
 #undef MOE_DL_VARIANT
   return fail(MOE_ERR_INVALID_ARG, "gmm: unknown tile variant %d", id);
 }

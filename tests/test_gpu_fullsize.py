@@ -1,0 +1,188 @@
+"""GPU parity at the full sizes of the benchmark configurations.
+
+The integer half of the path (top-k indices, perm, group_sizes) is compared bit-exactly against the
+oracle over ALL tokens.  The floating-point half is too large for a CPU oracle in full, so it is
+checked (a) on a random sample of sorted rows, each recomputed by the oracle's formula from the same
+quantised operands (per-row matmul against its expert's weights), and (b) through size-independent
+properties of the whole output (finite, routing round trip, zero rows stay zero).
+Tolerance for sampled rows: max|got-want| / max|want| <= 1e-2.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+N_SAMPLE = 40
+
+
+def _routing(wl, L):
+  from maxtext_amd import moe
+
+  cfg = wl.cfg
+  r = moe.RoutedMoE(cfg, L["wi_0"], L["wi_1"], L["wo"])
+  w, idx = r.get_topk(L["gate_logits"], L["pre_bias_logits"])
+  k, e = cfg.num_experts_per_tok, cfg.num_experts
+  logits = L["gate_logits"].cpu().numpy().reshape(-1, e)
+  if cfg.is_deepseek:
+    pre = L["pre_bias_logits"].cpu().numpy().reshape(-1, e)
+    ow, oidx = O.get_topk(logits, pre, k=k, mode="deepseek", routed_scaling_factor=cfg.routed_scaling_factor)
+    np.testing.assert_allclose(w.reshape(-1, k).cpu().numpy(), ow, rtol=1e-5)
+  else:
+    ow, oidx = O.get_topk(logits, k=k, norm_topk_prob=cfg.norm_topk_prob)
+    np.testing.assert_allclose(w.reshape(-1, k).cpu().numpy(), ow, rtol=2.0**-6, atol=1e-6)
+  np.testing.assert_array_equal(idx.reshape(-1, k).cpu().numpy(), oidx)
+  return r, w, idx, oidx
+
+
+def _dequant_rows(qa, expert, n_rows=None):
+  """Rows [N, K] of one expert's weights as f64 with scales applied where they are not separable."""
+  q = qa.qvalue[expert].cpu()
+  if qa.qtype == "int8":
+    return q.double(), qa.scale[expert].cpu().double()  # per-channel scale applied after the dot
+  if qa.qtype == "int4":
+    w = O.unpack_int4(q).double()
+    s = torch.repeat_interleave(qa.scale[expert].cpu().double(), 128, dim=-1)[:, : w.shape[1]]
+    return w * s, None
+  raise ValueError(qa.qtype)
+
+
+def _check_sampled_rows(wl, L, rows_q, rows_scale, inter, y, group_sizes, act_quant):
+  """Recomputes `inter` (after wi_0/wi_1 + SwiGLU) and `y` (after wo) for a sample of sorted rows."""
+  gs = group_sizes.cpu().numpy()
+  offs = np.concatenate([[0], np.cumsum(gs)])
+  m = int(offs[-1])
+  rng = np.random.default_rng(0)
+  bounds = np.concatenate([offs[:-1][gs > 0][:4], offs[1:][gs > 0][:4] - 1])  # first / last rows of groups
+  picks = np.unique(np.concatenate([bounds, rng.integers(0, m, N_SAMPLE)]))[:N_SAMPLE]
+  experts = np.searchsorted(offs, picks, side="right") - 1
+  got_i, want_i, got_y, want_y = [], [], [], []
+  cache = {}
+  for r, e in zip(picks, experts):
+    if e not in cache:
+      if len(cache) >= 4:
+        continue
+      cache[e] = (_dequant_rows(L["wi_0"], e), _dequant_rows(L["wi_1"], e), _dequant_rows(L["wo"], e))
+    (w0, s0), (w1, s1), (wo, so) = cache[e]
+    a = rows_q[r].cpu().double()
+    a_s = 1.0 if rows_scale is None else float(rows_scale[r])
+    h0 = (w0 @ a) * a_s * (s0 if s0 is not None else 1.0)
+    h1 = (w1 @ a) * a_s * (s1 if s1 is not None else 1.0)
+    want_i.append(O.apply_ffn_activation(h0.float(), h1.float(), wl.cfg.activation))
+    got_i.append(inter[r].cpu())
+    # the second matmul consumes the GPU's own intermediate row (re-quantised as the path does)
+    b = inter[r].cpu()
+    if act_quant == "int8":
+      bq, bs = O.quantize_rows_int8(b[None].float())
+      b, b_s = bq[0].double(), float(bs[0])
+    else:
+      b, b_s = b.double(), 1.0
+    want_y.append(((wo @ b) * b_s * (so if so is not None else 1.0)).to(torch.bfloat16))
+    got_y.append(y[r].cpu())
+  gi, wi = torch.stack(got_i).float(), torch.stack(want_i).float()
+  gy, wy = torch.stack(got_y).float(), torch.stack(want_y).float()
+  assert float((gi - wi).abs().max() / wi.abs().max()) <= TOL
+  assert float((gy - wy).abs().max() / wy.abs().max()) <= TOL
+  return len(got_i)
+
+
+@pytest.mark.parametrize("name", ["c2", "c4", "c5"])
+def test_fullsize_int_weight_layers(name):
+  from maxtext_amd import kernels, megablox, synthetic
+  from maxtext_amd.quantizations import QArray
+
+  wl = synthetic.workload(name)
+  cfg = wl.cfg
+  L = synthetic.make_layer(wl, device="cuda")
+  r, w, idx, oidx = _routing(wl, L)
+  k, e, d = cfg.num_experts_per_tok, cfg.num_experts, cfg.emb_dim
+  t = wl.tokens
+  # perm / group_sizes over all M rows, bit-exact against the stable argsort
+  perm, inv, gs, se = kernels.sort_by_expert(idx.reshape(t, k).contiguous(), e)
+  flat = oidx.reshape(-1)
+  operm = np.argsort(flat, kind="stable").astype(np.int32)
+  np.testing.assert_array_equal(perm.cpu().numpy(), operm)
+  np.testing.assert_array_equal(gs.cpu().numpy(), np.bincount(flat, minlength=e).astype(np.int32))
+  np.testing.assert_array_equal(se.cpu().numpy(), flat[operm])
+  if name == "c4":
+    assert (gs == 0).any().item(), "the Zipf workload must leave experts empty"
+  x2d = L["x"].reshape(t, d)
+  if cfg.act_quant == "int8":
+    q, sc = kernels.gather_rows(x2d, perm, k, out_dtype=torch.int8)
+    oq, osc = O.quantize_rows_int8(x2d.cpu()[torch.from_numpy(operm[:4096].astype(np.int64) // k)])
+    assert torch.equal(q[:4096].cpu(), oq) and torch.equal(sc[:4096].cpu(), osc)
+    rows, rows_q, rows_scale = QArray(q, sc, "int8"), q, sc.cpu().numpy()
+  else:
+    rows = kernels.gather_rows(x2d, perm, k)
+    assert torch.equal(rows[:4096].cpu(), x2d.cpu()[torch.from_numpy(operm[:4096].astype(np.int64) // k)])
+    rows_q, rows_scale = rows, None
+  inter = megablox.gmm(rows, L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act=cfg.activation)
+  inter_in = megablox.quantize_lhs(inter, "int8") if cfg.act_quant == "int8" else inter
+  y = megablox.gmm(inter_in, L["wo"], gs, transpose_rhs=True)
+  assert torch.isfinite(inter.float()).all() and torch.isfinite(y.float()).all()
+  n = _check_sampled_rows(wl, L, rows_q, rows_scale, inter, y, gs, cfg.act_quant)
+  assert n >= 16
+  # combine: with unit weights and y := sorted inputs the layer returns k * x (routing round trip)
+  back = kernels.unpermute_combine(kernels.gather_rows(x2d, perm, k), torch.ones((t, k), device="cuda"), k=k, inv_perm=inv)
+  assert torch.equal(back, (x2d.float() * k).to(torch.bfloat16))
+  # and the real combine equals the f32 weighted sum of the rows it gathers, on a sample of tokens
+  out = kernels.unpermute_combine(y, w.reshape(t, k).contiguous(), k=k, inv_perm=inv)
+  toks = np.random.default_rng(1).integers(0, t, 64)
+  invc, wc = inv.cpu().numpy().reshape(t, k), w.reshape(t, k).cpu().numpy()
+  for tok in toks:
+    want = sum(float(wc[tok, s]) * y[int(invc[tok, s])].float().cpu() for s in range(k)).to(torch.bfloat16)
+    assert float((out[tok].float().cpu() - want.float()).abs().max()) <= 2.0**-7 * float(want.float().abs().max()) + 1e-6
+
+
+def test_fullsize_deepseek_fp8_decode():
+  """C3 at full size: 256 routed experts + shared expert resident, fp8 128x128 weights."""
+  from maxtext_amd import kernels, megablox, synthetic
+  from maxtext_amd.quantizations import QArray
+
+  wl = synthetic.workload("c3")
+  cfg = wl.cfg
+  L = synthetic.make_layer(wl, device="cuda")
+  r, w, idx, oidx = _routing(wl, L)
+  k, e, d, f, t = cfg.num_experts_per_tok, cfg.num_experts, cfg.emb_dim, cfg.moe_mlp_dim, wl.tokens
+  sel = torch.cat([idx.reshape(t, k), torch.full((t, 1), e, dtype=torch.int32, device="cuda")], 1).contiguous()
+  perm, inv, gs, _ = kernels.sort_by_expert(sel, e + 1)
+  flat = np.concatenate([oidx, np.full((t, 1), e, np.int32)], 1).reshape(-1)
+  operm = np.argsort(flat, kind="stable").astype(np.int32)
+  np.testing.assert_array_equal(perm.cpu().numpy(), operm)
+  np.testing.assert_array_equal(gs.cpu().numpy(), np.bincount(flat, minlength=e + 1).astype(np.int32))
+  x2d = L["x"].reshape(t, d)
+  q, sc = kernels.gather_rows(x2d, perm, k + 1, out_dtype=torch.float8_e4m3fn, block_k=128)
+  oq, osc = O.quantize_fp8_blocks(x2d.cpu()[torch.from_numpy(operm.astype(np.int64) // (k + 1))], 1, 128)
+  assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(sc.cpu(), osc)
+  inter = megablox.gmm(QArray(q, sc, "fp8"), L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act="silu")
+  y = megablox.gmm(megablox.quantize_lhs(inter, "fp8"), L["wo"], gs, transpose_rhs=True)
+  assert torch.isfinite(y.float()).all()
+  # sampled rows against the oracle's block-scaled formula (including rows of the shared expert)
+  gsn = gs.cpu().numpy()
+  offs = np.concatenate([[0], np.cumsum(gsn)])
+  rng = np.random.default_rng(2)
+  picks = np.concatenate([rng.integers(0, offs[-2], 24), rng.integers(offs[-2], offs[-1], 8)])
+  got, want = [], []
+  for rr in picks:
+    ex = int(np.searchsorted(offs, rr, side="right") - 1)
+    a = q[rr].cpu()[None]
+    a_s = sc[rr].cpu()[None]
+    one = np.array([1], np.int32)
+
+    def proj(qa, lhs, lhs_s):
+      wq = qa.qvalue[ex].cpu()[None]  # [1, n, k]
+      n = wq.shape[1]
+      ws = torch.repeat_interleave(qa.scale[ex].cpu()[None].permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
+      return O.gmm(lhs, wq, one, lhs_scale=lhs_s, rhs_scale=ws, transpose_rhs=True, quant_block=128, out_dtype=torch.float32)
+
+    it = O.apply_ffn_activation(proj(L["wi_0"], a, a_s), proj(L["wi_1"], a, a_s))
+    got.append(inter[rr].cpu().float())
+    want.append(it[0].float())
+    bq, bs = O.quantize_fp8_blocks(inter[rr].cpu()[None], 1, 128)
+    got.append(y[rr].cpu().float())
+    want.append(proj(L["wo"], bq, bs)[0].to(torch.bfloat16).float())
+  for g_, w_ in zip(got, want):
+    assert float((g_ - w_).abs().max() / w_.abs().max().clamp_min(1e-30)) <= TOL
