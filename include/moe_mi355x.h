@@ -183,6 +183,23 @@ MOE_API int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem
                       void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Transposed grouped matmul (weight gradient of gmm).  Replaces tgmm(lhs^T, dout, group_sizes, ...)
+ * (src/maxtext/kernels/megablox/backend.py:575-816; called from _gmm_bwd, ops.py:766) for bf16 operands:
+ *
+ *   out[g - group_offset, n, k] = sum over the rows m of group g of dout[m, n] * lhs[m, k]
+ *
+ *   lhs   [M, K] bf16   forward activations (the caller does NOT transpose them)
+ *   dout  [M, N] bf16   gradient of the forward output
+ *   out   [G_local, N, K] bf16 or f32 (out_dtype): the layout of the forward weights; groups with no
+ *         rows are written as zeros (reference_tgmm, tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:156-186)
+ * The gradient of lhs needs no entry point of its own: it is moe_gmm(dout, rhs re-laid out as [G, K, N]).
+ * Limits: K % 8 == 0, N % 8 == 0.
+ */
+MOE_API int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
+                     int num_groups_total, int num_groups_local, int group_offset, int out_dtype, void* out,
+                     void* stream);
+
+/* ---------------------------------------------------------------------------
  * Unpermute + top-k weighted combine.  Replaces RoutedMoE.unpermute
  * (moe.py:1039-1063, float32_weight_sum=True) and the fused gather-reduce
  * fallback (kernels/ragged/ragged_gather_reduce_v2.py:170-182):

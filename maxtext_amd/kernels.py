@@ -201,3 +201,24 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
   _lib.check(st, "moe_gmm")
   return out
+
+
+def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16):
+  """Weight gradient: out[g, n, k] = sum over rows m of group g of dout[m, n] * lhs[m, k]  ->  [G_local, N, K]."""
+  _need(lhs, "lhs", torch.bfloat16, 2)
+  _need(dout, "dout", torch.bfloat16, 2)
+  _need(group_sizes, "group_sizes", torch.int32, 1)
+  m, k = lhs.shape
+  if dout.shape[0] != m:
+    raise ValueError("lhs and dout must have the same number of rows")
+  n = dout.shape[1]
+  g_total = group_sizes.numel()
+  g_local = g_total - int(group_offset) if num_groups_local is None else int(num_groups_local)
+  if out_dtype not in (torch.bfloat16, torch.float32):
+    raise TypeError("out_dtype must be bfloat16 or float32")
+  out = torch.empty((g_local, n, k), dtype=out_dtype, device=lhs.device)
+  lib = _lib.load()
+  st = lib.moe_tgmm(_lib.ptr(lhs), _lib.ptr(dout), _lib.ptr(group_sizes), m, k, n, g_total, g_local, int(group_offset),
+                    _lib.MOE_BF16 if out_dtype == torch.bfloat16 else _lib.MOE_F32, _lib.ptr(out), _lib.current_stream())
+  _lib.check(st, "moe_tgmm")
+  return out

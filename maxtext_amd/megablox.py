@@ -121,6 +121,9 @@ def gmm(
     else:
       offset = int(group_offset)
 
+  if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up)):
+    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit)
+
   rhs_n = _native_rhs(rhs, transpose_rhs)
   up_n = _native_rhs(rhs_up, transpose_rhs) if rhs_up is not None else None
   if not isinstance(rhs_n, QArray) and rhs_quantize_dtype is not None:
@@ -157,3 +160,102 @@ def gmm(
     if up_n is not None:
       kw["rhs_up"] = up_n
   return kernels.gmm_raw(lhs_t, rhs_t, group_sizes, **kw)
+
+
+def tgmm(
+    lhs,
+    rhs,
+    group_sizes,
+    preferred_element_type=torch.float32,
+    tiling=(128, 128, 128),
+    group_offset=None,
+    num_actual_groups=None,
+    existing_out=None,
+    interpret=False,
+    varying_axes=(),
+):
+  """Transposed grouped matmul out[g] = lhs[:, rows of g] @ rhs[rows of g, :] (backend.py:575-816).
+
+  lhs: [k, m] bf16 (the reference passes the forward activation swapped, ops.py:889-899; a
+  `.t()` view of a contiguous [m, k] tensor is consumed without a copy); rhs: [m, n] bf16 (the
+  incoming gradient); returns [num_actual_groups, k, n] as a transposed view of the [G, N, K]
+  buffer the kernel writes, which is the layout moe_gmm takes weights in.
+  """
+  del tiling, interpret, varying_axes
+  if lhs.dim() != 2 or rhs.dim() != 2:
+    raise ValueError("Expected 2-tensors for 'lhs' and 'rhs'.")
+  if group_sizes.dtype != torch.int32:
+    raise ValueError(f"Expected 32-bit integer 'group_sizes' but got {group_sizes.dtype}.")
+  if lhs.shape[1] != rhs.shape[0]:
+    raise ValueError(f"Expected lhs [k, m] and rhs [m, n] to share m, got {tuple(lhs.shape)} and {tuple(rhs.shape)}.")
+  if existing_out is not None:
+    raise NotImplementedError("existing_out is not implemented")
+  if preferred_element_type not in (torch.float32, torch.bfloat16):
+    raise NotImplementedError("tgmm outputs are float32 or bfloat16")
+  offset = 0 if group_offset is None else int(group_offset)
+  lhs_mk = lhs.t()
+  if not lhs_mk.is_contiguous():
+    lhs_mk = lhs_mk.contiguous()
+  out = kernels.tgmm(
+      lhs_mk, rhs.contiguous(), group_sizes, num_groups_local=num_actual_groups, group_offset=offset, out_dtype=preferred_element_type
+  )
+  return out.transpose(1, 2)
+
+
+class _GmmFn(torch.autograd.Function):
+  """Differentiable gmm for bf16 operands (custom VJP of ops.py:137-230 / :438-527).
+
+  Forward may quantise its operands on the fly; backward differentiates through the quantisers
+  as identities and uses the bf16 residuals: dlhs = gmm(dout, rhs^T) (ops.py:612-642) and
+  drhs = tgmm(lhs^T, dout) (ops.py:766-796), both without quantisation of the gradient.
+  """
+
+  @staticmethod
+  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q):
+    ctx.save_for_backward(lhs, rhs, group_sizes)
+    ctx.offset, ctx.transpose_rhs = offset, transpose_rhs
+    with torch.no_grad():
+      return gmm(lhs, rhs, group_sizes, group_offset=offset, transpose_rhs=transpose_rhs, lhs_quantize_dtype=lhs_q, rhs_quantize_dtype=rhs_q)
+
+  @staticmethod
+  def backward(ctx, dout):
+    lhs, rhs, group_sizes = ctx.saved_tensors
+    dout = dout.contiguous()
+    dlhs = drhs = None
+    with torch.no_grad():
+      if ctx.needs_input_grad[0]:
+        # dout [m, n] @ rhs[g]^T: the kernel's weight layout [G, out, in] is here [G, k, n]
+        dlhs = gmm(dout, rhs, group_sizes, group_offset=ctx.offset, transpose_rhs=not ctx.transpose_rhs)
+        # rows of groups outside [offset, offset + G_local) are zero in the forward output
+      if ctx.needs_input_grad[1]:
+        d = tgmm(lhs.t(), dout, group_sizes, rhs.dtype, group_offset=ctx.offset, num_actual_groups=rhs.shape[0])
+        drhs = d.transpose(1, 2) if ctx.transpose_rhs else d.contiguous()
+    return dlhs, drhs, None, None, None, None, None
+
+
+def _glu_torch(h0, h1, kind, limit):
+  """apply_ffn_activation of the expert MLP (moe.py:1288-1306) in differentiable torch ops."""
+  h0, h1 = h0.float(), h1.float()
+  if kind == "silu":
+    return (torch.nn.functional.silu(h0) * h1).to(torch.bfloat16)
+  if kind == "swigluoai":
+    g, u = h0.clamp(max=limit), h1.clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(torch.bfloat16)
+  if kind == "silu_clip":
+    return (torch.nn.functional.silu(h0.clamp(max=limit)) * h1.clamp(-limit, limit)).to(torch.bfloat16)
+  raise ValueError(f"unknown activation {kind}")
+
+
+def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit):
+  for name, t in (("lhs", lhs), ("rhs", rhs), ("rhs_up", rhs_up)):
+    if t is not None and not isinstance(t, torch.Tensor):
+      raise NotImplementedError(f"gradients need bf16 tensors; {name} is already quantised")
+  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q)
+  if rhs_up is None:
+    if fuse_act is not None:
+      raise ValueError("fuse_act needs rhs_up")
+    return h0
+  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q)
+  if fuse_act is None:
+    raise ValueError("rhs_up needs fuse_act")
+  return _glu_torch(h0, h1, fuse_act, act_limit)

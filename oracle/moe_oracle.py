@@ -16,6 +16,8 @@ How each function is pinned (see tests/test_oracle_*.py):
       hand-computed case of tests/unit/moe_test.py:328-341.
   permute / unpermute
       permutation invariants, brute-force loops, k*x identity.
+  tgmm
+      per-group python loop; autograd of the gmm oracle (d/d rhs of sum(gmm * dout)).
   gmm
       per-expert python loop, E=1 == plain matmul, int8 path exact on
       integer inputs, the [3,5]-group case of quantizations_test.py:607-653.
@@ -294,6 +296,26 @@ def gmm(
       out[start:end] = acc
     start = end
   return out.to(out_dtype)
+
+
+def tgmm(lhs: torch.Tensor, dout: torch.Tensor, group_sizes, *, num_actual_groups=None, group_offset: int = 0,
+         out_dtype=torch.bfloat16) -> torch.Tensor:
+  """Transposed grouped matmul, the weight gradient of gmm
+  (tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:156-186 reference_tgmm; backend.py:587):
+  out[g] = lhs[rows of group g]^T @ dout[rows of group g], shape [groups, k, n]; only the
+  num_actual_groups groups starting at group_offset are produced."""
+  group_sizes = np.asarray(group_sizes, dtype=np.int64)
+  m = lhs.shape[0]
+  g = group_sizes.size - group_offset if num_actual_groups is None else num_actual_groups
+  outs = []
+  start = 0
+  for gg in range(group_sizes.size):
+    end = min(start + int(group_sizes[gg]), m)
+    loc = gg - group_offset
+    if 0 <= loc < g:
+      outs.append((lhs[start:end].double().T @ dout[start:end].double()).to(out_dtype))
+    start = end
+  return torch.stack(outs)
 
 
 # --------------------------------------------------------------------------

@@ -383,3 +383,117 @@ def test_gmm_argument_errors(K):
     K.gmm_raw(lhs, rhs, gs, act="silu")  # activation without rhs_up
   with pytest.raises(ValueError):
     K.gmm_raw(lhs.cpu(), rhs, gs)
+
+
+# ---------------------------------------------------------------- backward: tgmm, dlhs, autograd
+
+TGMM_SHAPES = [
+    (300, 128, 128, [100, 0, 150, 50]),
+    (1000, 256, 384, [1, 31, 32, 33, 400, 0, 503]),
+    (520, 200, 72, [500, 20]),  # K, N not multiples of the 128 tile
+    (64, 2880, 96, [7, 57]),
+    (700, 128, 256, [300, 200]),  # rows past sum(group_sizes) belong to no group
+]
+
+
+@pytest.mark.parametrize("m,k,n,gs", TGMM_SHAPES)
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_tgmm(K, m, k, n, gs, out_dtype):
+  g = torch.Generator().manual_seed(5)
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  gs = np.asarray(gs, np.int32)
+  got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=out_dtype)  # [G, N, K]
+  want = O.tgmm(lhs, dout, gs, out_dtype=out_dtype).transpose(1, 2)
+  assert got.shape == want.shape and got.dtype == out_dtype
+  assert relerr(got, want) <= TOL
+  for i, sz in enumerate(gs):
+    if sz == 0:
+      assert torch.all(got[i] == 0)
+    else:  # per-group bound too, so a small group next to a big one is not hidden by the global max
+      assert relerr(got[i], want[i]) <= TOL
+
+
+def test_tgmm_exact_on_small_integers_and_group_window(K):
+  rng = np.random.default_rng(3)
+  m, k, n = 333, 136, 264
+  gs = np.array([40, 0, 100, 93, 100], np.int32)
+  lhs = torch.from_numpy(rng.integers(-3, 4, (m, k)).astype(np.float32)).to(torch.bfloat16)
+  dout = torch.from_numpy(rng.integers(-3, 4, (m, n)).astype(np.float32)).to(torch.bfloat16)
+  want = O.tgmm(lhs, dout, gs, out_dtype=torch.float32).transpose(1, 2)
+  got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=torch.float32)
+  assert torch.equal(got.cpu(), want)  # sums of at most 100 products of magnitude <= 9 are exact in f32
+  win = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), num_groups_local=3, group_offset=1, out_dtype=torch.float32)
+  assert torch.equal(win.cpu(), want[1:4])
+  # NaN rows outside the window must not leak into it
+  lhs_nan = lhs.clone()
+  lhs_nan[:40] = float("nan")
+  win = K.tgmm(cuda(lhs_nan), cuda(dout), cuda(gs), num_groups_local=3, group_offset=1, out_dtype=torch.float32)
+  assert torch.equal(win.cpu(), want[1:4])
+
+
+def test_tgmm_argument_errors(K):
+  a = torch.zeros(16, 64, dtype=torch.bfloat16, device="cuda")
+  gs = torch.tensor([16], dtype=torch.int32, device="cuda")
+  with pytest.raises(ValueError):
+    K.tgmm(a, torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda"), gs)
+  with pytest.raises(RuntimeError, match="multiples of 8"):
+    K.tgmm(a, torch.zeros(16, 12, dtype=torch.bfloat16, device="cuda"), gs)
+  with pytest.raises(TypeError):
+    K.tgmm(a.float(), a, gs)
+
+
+@pytest.mark.parametrize("transpose_rhs", [False, True])
+def test_gmm_autograd_matches_torch_autograd(transpose_rhs):
+  """dlhs and drhs of megablox.gmm against torch autograd through a per-group f64 matmul (the custom
+  VJP of ops.py:438-527: dlhs = gmm(dout, rhs^T), drhs = tgmm(lhs^T, dout))."""
+  from maxtext_amd import megablox
+
+  g = torch.Generator().manual_seed(9)
+  m, k, n = 450, 256, 192
+  gs = np.array([200, 0, 70, 150], np.int32)  # 30 trailing rows in no group
+  e = len(gs)
+  lhs = (torch.randn(m, k, generator=g)).to(torch.bfloat16)
+  w = (torch.randn(e, k, n, generator=g) * 0.05).to(torch.bfloat16)  # [g, k, n]
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  lhs64 = lhs.double().requires_grad_()
+  w64 = w.double().requires_grad_()
+  off = np.concatenate([[0], np.cumsum(gs)])
+  ref = torch.cat([lhs64[off[i] : off[i + 1]] @ w64[i] for i in range(e)] + [torch.zeros(m - off[-1], n, dtype=torch.float64)])
+  (ref * dout.double()).sum().backward()
+
+  lhs_g = cuda(lhs).requires_grad_()
+  rhs_g = cuda(w.transpose(1, 2) if transpose_rhs else w).requires_grad_()
+  out = megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs)
+  assert relerr(out, ref) <= TOL
+  out.backward(cuda(dout))
+  assert lhs_g.grad.shape == lhs.shape and rhs_g.grad.shape == rhs_g.shape
+  assert relerr(lhs_g.grad, lhs64.grad) <= TOL
+  assert torch.all(lhs_g.grad[int(off[-1]) :] == 0)
+  want_drhs = w64.grad.transpose(1, 2) if transpose_rhs else w64.grad
+  assert relerr(rhs_g.grad, want_drhs) <= TOL
+  assert torch.all(rhs_g.grad[1] == 0)
+
+
+def test_gmm_autograd_through_fused_activation():
+  from maxtext_amd import megablox
+
+  g = torch.Generator().manual_seed(10)
+  m, k, n = 256, 128, 128
+  gs = np.array([100, 156], np.int32)
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w0 = (torch.randn(2, n, k, generator=g) * 0.1).to(torch.bfloat16)
+  w1 = (torch.randn(2, n, k, generator=g) * 0.1).to(torch.bfloat16)
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  a, b0, b1 = lhs.double().requires_grad_(), w0.double().requires_grad_(), w1.double().requires_grad_()
+  off = [0, 100, 256]
+  h0 = torch.cat([a[off[i] : off[i + 1]] @ b0[i].T for i in range(2)])
+  h1 = torch.cat([a[off[i] : off[i + 1]] @ b1[i].T for i in range(2)])
+  (torch.nn.functional.silu(h0) * h1 * dout.double()).sum().backward()
+  la, r0, r1 = cuda(lhs).requires_grad_(), cuda(w0).requires_grad_(), cuda(w1).requires_grad_()
+  out = megablox.gmm(la, r0, cuda(gs), transpose_rhs=True, rhs_up=r1, fuse_act="silu")
+  out.backward(cuda(dout))
+  # bf16 intermediates (h0, h1 and their gradients are rounded to bf16) -> 2e-2 on the gradients
+  assert relerr(la.grad, a.grad) <= 2e-2
+  assert relerr(r0.grad, b0.grad) <= 2e-2
+  assert relerr(r1.grad, b1.grad) <= 2e-2

@@ -315,3 +315,28 @@ def test_sparse_layer_equals_loop_and_dense():
   y = torch.einsum("teh,ehm->tem", a.float(), wo.float()).to(torch.bfloat16)
   dense = torch.einsum("tem,te->tm", y.float(), dense_w).to(torch.bfloat16)
   assert (sparse.float() - dense.float()).abs().max() <= 2e-2 * dense.float().abs().max()
+
+
+def test_tgmm_equals_autograd_of_grouped_matmul_and_hand_case():
+  """tgmm is the weight gradient of gmm: d/d rhs of sum(gmm(lhs, rhs) * dout), here taken by torch
+  autograd through an independent per-group matmul; plus a hand-computed 2-group case and the
+  group_offset / num_actual_groups window."""
+  g = torch.Generator().manual_seed(0)
+  m, k, n, e = 50, 16, 24, 4
+  lhs = torch.randn(m, k, generator=g, dtype=torch.float64)
+  rhs = torch.randn(e, k, n, generator=g, dtype=torch.float64, requires_grad=True)
+  dout = torch.randn(m, n, generator=g, dtype=torch.float64)
+  gs = np.array([10, 0, 25, 15], np.int32)
+  off = np.concatenate([[0], np.cumsum(gs)])
+  out = torch.cat([lhs[off[i] : off[i + 1]] @ rhs[i] for i in range(e)])
+  (out * dout).sum().backward()
+  got = O.tgmm(lhs, dout, gs, out_dtype=torch.float64)
+  assert torch.allclose(got, rhs.grad, rtol=1e-12, atol=1e-12)
+  assert torch.all(got[1] == 0)  # empty group -> zero gradient
+  win = O.tgmm(lhs, dout, gs, num_actual_groups=2, group_offset=2, out_dtype=torch.float64)
+  assert torch.equal(win, got[2:4])
+  # hand case: rows [1,2],[3,4] | [5,6];  dout rows [1],[10] | [100]
+  lhs2 = torch.tensor([[1.0, 2.0], [3.0, 4.0], [5.0, 6.0]])
+  d2 = torch.tensor([[1.0], [10.0], [100.0]])
+  t2 = O.tgmm(lhs2, d2, np.array([2, 1], np.int32), out_dtype=torch.float32)
+  assert t2.tolist() == [[[31.0], [42.0]], [[500.0], [600.0]]]
