@@ -218,6 +218,24 @@ MOE_API int moe_unpermute_combine(const void* y, const int32_t* perm, const int3
                           const float* weights, int T, int k, int d, void* out, void* workspace,
                           size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Gradient of moe_unpermute_combine with respect to y and to the weights (the VJP that JAX derives for
+ * the gather + einsum of moe.py:1041-1062; its hand-written counterpart for the fused kernel is
+ * kernels/sort_activations.py:85-121):
+ *
+ *   dy[inv_perm[t*k + s], :] = bf16( weights[t, s] * f32(dout[t, :]) )
+ *   dweights[t, s]           = sum_d f32(y[inv_perm[t*k + s], d]) * f32(dout[t, d])
+ *
+ *   dout [T, d] bf16; y [M, d] bf16 (forward input; may be NULL when dweights is NULL);
+ *   weights [T, k] f32 or NULL (ones); dy [M, d] bf16 (every row is written: inv_perm is a permutation);
+ *   dweights [T, k] f32 or NULL.
+ * The gradient of the row gather (moe_gather_rows in copy mode; _sort_activations_custom_bwd,
+ * moe.py:165-171) is moe_unpermute_combine itself with weights == NULL.
+ * Limits: d % 8 == 0, k <= 16.
+ */
+MOE_API int moe_unpermute_combine_bwd(const void* dout, const void* y, const int32_t* inv_perm, const float* weights,
+                                      int T, int k, int d, void* dy, float* dweights, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -428,6 +428,59 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ 
   }
 }
 
+// Gradient of the combine: one block per token.  dy[row_s] = bf16(w_s * dout[t]) for the k rows the token
+// gathered, dw[t, s] = sum_d f32(y[row_s, d]) * f32(dout[t, d]).
+__global__ __launch_bounds__(256) void combine_bwd_kernel(const uint4* __restrict__ dout, const uint4* __restrict__ y,
+                                                          const int32_t* __restrict__ inv_perm,
+                                                          const float* __restrict__ weights, int k, int d,
+                                                          uint4* __restrict__ dy, float* __restrict__ dw) {
+  __shared__ int s_row[kCombineMaxK];
+  __shared__ float s_w[kCombineMaxK];
+  __shared__ float s_part[kCombineMaxK][4];
+  const int t = blockIdx.x;
+  if (threadIdx.x < k) {
+    s_row[threadIdx.x] = inv_perm[(size_t)t * k + threadIdx.x];
+    s_w[threadIdx.x] = weights ? weights[(size_t)t * k + threadIdx.x] : 1.0f;
+  }
+  __syncthreads();
+  const int nch = d / 8;
+  float dot[kCombineMaxK];
+#pragma unroll
+  for (int s = 0; s < kCombineMaxK; s++) dot[s] = 0.f;
+  for (int ci = threadIdx.x; ci < nch; ci += blockDim.x) {
+    float g[8];
+    unpack8(dout[(size_t)t * nch + ci], g);
+#pragma unroll
+    for (int s = 0; s < kCombineMaxK; s++) {
+      if (s >= k) break;
+      const size_t at = (size_t)s_row[s] * nch + ci;
+      const float w = s_w[s];
+      uint4 o;
+      o.x = pack_bf16x2(w * g[0], w * g[1]);
+      o.y = pack_bf16x2(w * g[2], w * g[3]);
+      o.z = pack_bf16x2(w * g[4], w * g[5]);
+      o.w = pack_bf16x2(w * g[6], w * g[7]);
+      dy[at] = o;
+      if (dw) {
+        float f[8];
+        unpack8(y[at], f);
+#pragma unroll
+        for (int i = 0; i < 8; i++) dot[s] = fmaf(f[i], g[i], dot[s]);
+      }
+    }
+  }
+  if (!dw) return;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int s = 0; s < kCombineMaxK; s++) {
+    if (s >= k) break;
+    const float v = wave_sum(dot[s]);
+    if (lane == 0) s_part[s][wave] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < k) dw[(size_t)t * k + threadIdx.x] = s_part[threadIdx.x][0] + s_part[threadIdx.x][1] + s_part[threadIdx.x][2] + s_part[threadIdx.x][3];
+}
+
 // ---------------------------------------------------------------------------------------
 // [G, K, N] -> [G, N, K] re-layout through a padded LDS tile.
 // ---------------------------------------------------------------------------------------
@@ -550,6 +603,17 @@ int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv
   }
   combine_kernel<<<T, 256, 0, s>>>((const uint4*)y, inv_perm, weights, k, d, (uint4*)out);
   return check_launch("combine_kernel");
+}
+
+int moe_unpermute_combine_bwd(const void* dout, const void* y, const int32_t* inv_perm, const float* weights,
+                              int T, int k, int d, void* dy, float* dweights, void* stream) {
+  if (!dout || !inv_perm || !dy || (dweights && !y)) return fail(MOE_ERR_INVALID_ARG, "combine_bwd: NULL pointer");
+  if (T < 0 || k <= 0 || d <= 0) return fail(MOE_ERR_INVALID_ARG, "combine_bwd: bad sizes");
+  if (k > kCombineMaxK || d % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "combine_bwd: need k<=16, d%%8==0");
+  if (T == 0) return MOE_OK;
+  combine_bwd_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const uint4*)dout, (const uint4*)y, inv_perm, weights, k, d,
+                                                         (uint4*)dy, dweights);
+  return check_launch("combine_bwd_kernel");
 }
 
 int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem_bytes, void* rhs_gnk,

@@ -123,6 +123,32 @@ def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None):
   return out
 
 
+def unpermute_combine_bwd(dout, y, weights, *, k, inv_perm, need_dweights=True):
+  """Gradient of unpermute_combine: -> (dy [M, d] bf16, dweights [T, k] f32 or None)."""
+  _need(dout, "dout", torch.bfloat16, 2)
+  _need(inv_perm, "inv_perm", torch.int32, 1)
+  t, d = dout.shape
+  m = t * k
+  if inv_perm.numel() != m:
+    raise ValueError("inv_perm must have T*k elements")
+  if weights is not None:
+    _need(weights, "weights", torch.float32)
+    if weights.numel() != m:
+      raise ValueError("weights must have T*k elements")
+  dw = None
+  if need_dweights:
+    _need(y, "y", torch.bfloat16, 2)
+    if y.shape != (m, d):
+      raise ValueError("y must be [T*k, d]")
+    dw = torch.empty((t, k), dtype=torch.float32, device=dout.device)
+  dy = torch.empty((m, d), dtype=torch.bfloat16, device=dout.device)
+  lib = _lib.load()
+  st = lib.moe_unpermute_combine_bwd(_lib.ptr(dout), _lib.ptr(y) if need_dweights else None, _lib.ptr(inv_perm), _lib.ptr(weights),
+                                     t, k, d, _lib.ptr(dy), _lib.ptr(dw), _lib.current_stream())
+  _lib.check(st, "moe_unpermute_combine_bwd")
+  return dy, dw
+
+
 def transpose_rhs(rhs_gkn):
   """[G, K, N] -> [G, N, K] for 1- or 2-byte element types."""
   _need(rhs_gkn, "rhs", None, 3)

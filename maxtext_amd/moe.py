@@ -53,6 +53,39 @@ class MoEConfig:
     return "silu"
 
 
+class _GatherRowsFn(torch.autograd.Function):
+  """Row gather sorted[i] = x[perm[i] // k] with the custom VJP of moe.py:154-171: the gradient of a
+  token is the sum of the gradients of its k copies, gathered through the inverse permutation."""
+
+  @staticmethod
+  def forward(ctx, x2d, perm, inv_perm, k):
+    ctx.save_for_backward(inv_perm)
+    ctx.k = k
+    return kernels.gather_rows(x2d, perm, k)
+
+  @staticmethod
+  def backward(ctx, dsorted):
+    (inv_perm,) = ctx.saved_tensors
+    return kernels.unpermute_combine(dsorted.contiguous(), None, k=ctx.k, inv_perm=inv_perm), None, None, None
+
+
+class _CombineFn(torch.autograd.Function):
+  """unpermute + weighted sum (moe.py:1039-1062) with gradients for the expert outputs and the weights."""
+
+  @staticmethod
+  def forward(ctx, y, weights, inv_perm, k):
+    ctx.save_for_backward(y, weights, inv_perm)
+    ctx.k = k
+    return kernels.unpermute_combine(y, weights, k=k, inv_perm=inv_perm)
+
+  @staticmethod
+  def backward(ctx, dout):
+    y, weights, inv_perm = ctx.saved_tensors
+    dy, dw = kernels.unpermute_combine_bwd(dout.contiguous(), y, weights, k=ctx.k, inv_perm=inv_perm,
+                                           need_dweights=ctx.needs_input_grad[1])
+    return dy, dw, None, None
+
+
 class RoutedMoE:
   """Routed experts: top-k routing, permute, three grouped GEMMs with fused SwiGLU, combine.
 
@@ -99,7 +132,24 @@ class RoutedMoE:
     else:
       w, idx = kernels.route_topk(g2, k=self.num_experts_per_tok, norm_topk_prob=cfg.norm_topk_prob)
     k = self.num_experts_per_tok
+    if torch.is_grad_enabled() and (gate_logits.requires_grad or (pre_bias_logits is not None and pre_bias_logits.requires_grad)):
+      w = self._weights_with_grad(gate_logits, pre_bias_logits, idx.reshape(*shape, k))
     return w.reshape(*shape, k), idx.reshape(*shape, k)
+
+  def _weights_with_grad(self, gate_logits, pre_bias_logits, idx):
+    """The weight half of get_topk in differentiable torch ops, on the indices the kernel selected
+    (moe.py:747-756 and :767-773, :838); top-k indices carry no gradient."""
+    cfg = self.config
+    gi = idx.long()
+    if cfg.is_deepseek:
+      w = torch.gather(pre_bias_logits.float(), -1, gi)
+      if cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"):
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+      return w * cfg.routed_scaling_factor
+    w = torch.softmax(torch.gather(gate_logits.float(), -1, gi), -1).to(torch.bfloat16)
+    if cfg.norm_topk_prob:
+      w = w / w.sum(-1, keepdim=True)
+    return w.float()
 
   # -- permute (moe.py:872-1002), non-ragged branch -----------------------------------------
   def permute(self, inputs, gate_logits, pre_bias_logits=None, use_custom_sort_vjp=True, rngs=None,
@@ -113,7 +163,10 @@ class RoutedMoE:
     weights, selected = self.get_topk(gate_logits, pre_bias_logits)
     sel2d = selected.reshape(b * s, -1).contiguous()
     perm, inv, group_size, sorted_experts = kernels.sort_by_expert(sel2d, self.num_experts)
-    sorted_inputs = kernels.gather_rows(x2d, perm, self.num_experts_per_tok)
+    if torch.is_grad_enabled() and x2d.requires_grad:
+      sorted_inputs = _GatherRowsFn.apply(x2d, perm, inv, self.num_experts_per_tok)
+    else:
+      sorted_inputs = kernels.gather_rows(x2d, perm, self.num_experts_per_tok)
     self._last_inv_perm = inv
     return sorted_inputs, perm, weights, group_size, sorted_experts, None, None, None
 
@@ -124,9 +177,15 @@ class RoutedMoE:
       raise NotImplementedError("only float32_weight_sum=True is implemented")
     k = self.num_experts_per_tok
     w = weights.reshape(-1, k).float().contiguous()
-    out = kernels.unpermute_combine(intermediate.contiguous(), w, k=k,
-                                    perm=None if inv_perm is not None else sorted_selected_experts,
-                                    inv_perm=inv_perm)
+    if torch.is_grad_enabled() and (intermediate.requires_grad or w.requires_grad):
+      if inv_perm is None:
+        inv_perm = torch.empty_like(sorted_selected_experts)
+        inv_perm[sorted_selected_experts.long()] = torch.arange(inv_perm.numel(), dtype=torch.int32, device=inv_perm.device)
+      out = _CombineFn.apply(intermediate.contiguous(), w, inv_perm, k)
+    else:
+      out = kernels.unpermute_combine(intermediate.contiguous(), w, k=k,
+                                      perm=None if inv_perm is not None else sorted_selected_experts,
+                                      inv_perm=inv_perm)
     return out.reshape(batch_size, sequence_length, -1)
 
   # -- the three grouped GEMMs: gmm_up + apply_ffn_activation + wo (moe.py:1932-1986, :841, :2226)
@@ -137,6 +196,17 @@ class RoutedMoE:
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if ev is not None else None
     if marks:
       marks[0].record()
+    training = torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (sorted_inputs, w0, w1, wo))
+    if training:
+      # differentiable path: bf16 operands; with act_quant both operands of each GEMM are quantised
+      # inside its forward (ops.py:232-267) and gradients pass through the quantisers unchanged; the
+      # activation is applied unfused so that its inputs are kept for the backward pass
+      if any(isinstance(t, QArray) for t in (sorted_inputs, w0, w1, wo)):
+        raise NotImplementedError("gradients need bf16 weights; QArray weights are an inference format")
+      q = cfg.act_quant
+      inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit, lhs_quantize_dtype=q,
+                           rhs_quantize_dtype=q)
+      return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q)
     inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit)
     if marks:
       marks[1].record()
@@ -164,8 +234,12 @@ class RoutedMoE:
     weights, selected = self.get_topk(gate_logits, pre_bias_logits)
     perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
                                                       want_sorted_experts=False)
+    training = torch.is_grad_enabled() and any(
+        isinstance(t, torch.Tensor) and t.requires_grad for t in (x2d, weights, w0_kernel, w1_kernel, wo_kernel))
     # permute fused with the activation quantiser of the first GEMM
-    if cfg.act_quant == "int8":
+    if training:
+      sorted_inputs = _GatherRowsFn.apply(x2d, perm, inv, k) if x2d.requires_grad else kernels.gather_rows(x2d, perm, k)
+    elif cfg.act_quant == "int8":
       q, sc = kernels.gather_rows(x2d, perm, k, out_dtype=torch.int8)
       sorted_inputs = QArray(q, sc, "int8")
     elif cfg.act_quant == "fp8":

@@ -149,3 +149,102 @@ def test_layer_linearity_at_benchmark_width():
   out2, _, _ = block.sparse_matmul(layer["x"], layer["gate_logits"], None, layer["wi_0"], layer["wi_1"], wo2)
   assert torch.isfinite(out1.float()).all()
   assert torch.equal(out2.float(), out1.float() * 2)
+
+
+# ---------------------------------------------------------------- training: gradients of the whole layer
+
+
+def test_combine_bwd_matches_bruteforce():
+  from maxtext_amd import kernels
+
+  g = torch.Generator().manual_seed(4)
+  t, k, d = 37, 3, 264
+  y = torch.randn(t * k, d, generator=g).to(torch.bfloat16)
+  dout = torch.randn(t, d, generator=g).to(torch.bfloat16)
+  w = torch.rand(t, k, generator=g)
+  inv = torch.randperm(t * k, generator=g).to(torch.int32)
+  dy, dw = kernels.unpermute_combine_bwd(dout.cuda(), y.cuda(), w.cuda(), k=k, inv_perm=inv.cuda())
+  rows = inv.long().reshape(t, k)
+  want_dy = torch.zeros(t * k, d)
+  want_dy[rows.reshape(-1)] = (w[:, :, None] * dout.float()[:, None, :]).reshape(t * k, d)
+  want_dw = (y.float()[rows] * dout.float()[:, None, :]).sum(-1)
+  assert torch.equal(dy.cpu(), want_dy.to(torch.bfloat16))  # one rounding of an exact f32 product
+  assert relerr(dw, want_dw) <= 1e-5
+  dy1, none = kernels.unpermute_combine_bwd(dout.cuda(), None, None, k=k, inv_perm=inv.cuda(), need_dweights=False)
+  assert none is None
+  want1 = torch.zeros(t * k, d, dtype=torch.bfloat16)
+  want1[rows.reshape(-1)] = dout[:, None, :].expand(t, k, d).reshape(t * k, d)
+  assert torch.equal(dy1.cpu(), want1)
+
+
+@pytest.mark.parametrize("norm_topk_prob", [False, True])
+def test_layer_gradients_match_torch_autograd(norm_topk_prob):
+  """Forward + backward of RoutedMoE with bf16 weights (gate -> top-k -> permute -> gmm x3 -> combine)
+  against torch autograd through the per-token formulation of tests/unit/moe_test.py:344-411
+  (sum over the selected experts of weight * MLP_e(x)) in f64, on the indices the GPU selected."""
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(21)
+  t, d, f, e, k = 192, 128, 256, 4, 2
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  wg = (torch.randn(d, e, generator=g) * 0.1)
+  w0 = (torch.randn(e, f, d, generator=g) * 0.08).to(torch.bfloat16)
+  w1 = (torch.randn(e, f, d, generator=g) * 0.08).to(torch.bfloat16)
+  wo = (torch.randn(e, d, f, generator=g) * 0.08).to(torch.bfloat16)
+  dout = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, norm_topk_prob=norm_topk_prob)
+  leaves = [v.cuda().requires_grad_() for v in (x, wg, w0, w1, wo)]
+  xg, wgg, w0g, w1g, wog = leaves
+  block = moe.RoutedMoE(cfg, w0g, w1g, wog, gate_kernel=wgg)
+  out, _, _ = block(xg)
+  out.backward(dout.cuda())
+  # the indices the kernel chose (no gradient flows through them)
+  with torch.no_grad():
+    logits, _ = block.gate(xg.reshape(t, d))
+    _, idx = block.get_topk(logits)
+  idx = idx.reshape(t, k).cpu().long()
+
+  r = [v.double().requires_grad_() for v in (x, wg, w0, w1, wo)]
+  xr, wgr, w0r, w1r, wor = r
+  x2 = xr.reshape(t, d)
+  lg = x2 @ wgr
+  wts = torch.softmax(torch.gather(lg, -1, idx), -1)
+  if norm_topk_prob:
+    wts = wts / wts.sum(-1, keepdim=True)
+  ref = torch.zeros(t, d, dtype=torch.float64)
+  for s in range(k):
+    ex = idx[:, s]
+    h0 = torch.einsum("td,tfd->tf", x2, w0r[ex])
+    h1 = torch.einsum("td,tfd->tf", x2, w1r[ex])
+    y = torch.einsum("tf,tdf->td", torch.nn.functional.silu(h0) * h1, wor[ex])
+    ref = ref + wts[:, s : s + 1] * y
+  (ref * dout.double().reshape(t, d)).sum().backward()
+  assert relerr(out.reshape(t, d), ref) <= 2e-2
+  # bf16 intermediates on the way back (dy, d inter, d h0/h1 are each rounded to bf16): 3e-2 of the max
+  for got, want, name in zip(leaves, r, ("x", "gate", "wi_0", "wi_1", "wo")):
+    assert got.grad is not None and got.grad.shape == got.shape, name
+    assert relerr(got.grad, want.grad) <= 3e-2, name
+
+
+def test_layer_gradients_with_int8_quantised_forward():
+  """With act_quant the forward quantises both operands of each GEMM and the backward treats the
+  quantisers as identities: gradients stay within the quantisation noise of the bf16 run."""
+  import dataclasses as dc
+
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(22)
+  t, d, f, e, k = 128, 128, 128, 4, 2
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  logits = torch.randn(1, t, e, generator=g)
+  ws = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
+  grads = {}
+  for q in (None, "int8"):
+    leaves = [v.cuda().requires_grad_() for v in [x] + ws]
+    block = moe.RoutedMoE(dc.replace(cfg, act_quant=q), *leaves[1:])
+    out, _, _ = block.sparse_matmul(leaves[0], logits.cuda(), None, *leaves[1:])
+    out.float().square().sum().backward()
+    grads[q] = [v.grad for v in leaves]
+  for a, b in zip(grads[None], grads["int8"]):
+    assert relerr(b, a) <= 5e-2
