@@ -39,6 +39,8 @@ def parse():
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--train", action="store_true",
+                  help="forward + backward of the layer with bf16 weights of the workload's shape (weight and input gradients)")
   ap.add_argument("--calibrate-copy", action="store_true",
                   help="also run one plain 1 GiB device copy (reference dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   return ap.parse_args()
@@ -93,6 +95,105 @@ def cpu_baseline(wl, layer, sample_tokens):
               seconds=dt)
 
 
+def train_cpu_baseline(wl, sample_tokens):
+  """Forward + backward of the three grouped GEMMs with the oracle's gmm / tgmm (torch CPU, f32 results)
+  on `sample_tokens` tokens spread evenly over the experts: a reported baseline."""
+  import numpy as np
+  import torch
+
+  from oracle import moe_oracle as O
+
+  cfg = wl.cfg
+  e, d, f = cfg.num_experts, cfg.emb_dim, cfg.moe_mlp_dim
+  m = sample_tokens * cfg.num_experts_per_tok
+  gs = np.full((e,), m // e, np.int32)
+  m = int(gs.sum())
+  g = torch.Generator().manual_seed(0)
+  x = torch.randn(m, d, generator=g).to(torch.bfloat16)
+  w0, w1 = [(torch.randn(e, d, f, generator=g) * 0.02).to(torch.bfloat16) for _ in range(2)]
+  wo = (torch.randn(e, f, d, generator=g) * 0.02).to(torch.bfloat16)
+  dy = torch.randn(m, d, generator=g).to(torch.bfloat16)
+  torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))))
+  t0 = time.perf_counter()
+  h0 = O.gmm(x, w0, gs, out_dtype=torch.float32, acc_dtype=torch.float32)
+  h1 = O.gmm(x, w1, gs, out_dtype=torch.float32, acc_dtype=torch.float32)
+  a = O.apply_ffn_activation(h0, h1, cfg.activation)
+  O.gmm(a, wo, gs, out_dtype=torch.float32, acc_dtype=torch.float32)
+  da = O.gmm(dy, wo.transpose(1, 2).contiguous(), gs, out_dtype=torch.bfloat16, acc_dtype=torch.float32)
+  O.tgmm(a.float(), dy.float(), gs, out_dtype=torch.float32)
+  for w in (w0, w1):
+    O.gmm(da, w.transpose(1, 2).contiguous(), gs, out_dtype=torch.bfloat16, acc_dtype=torch.float32)
+    O.tgmm(x.float(), da.float(), gs, out_dtype=torch.float32)
+  dt = time.perf_counter() - t0
+  return dict(value=18.0 * m * d * f / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+              sample=f"{m} routed rows spread evenly over {e} experts, same d/f, bf16 weights, the nine grouped matmuls of "
+                     f"forward + backward (activation derivative not included); {dt:.1f} s wall", seconds=dt)
+
+
+def train_main(args):
+  """Forward + backward of the routed layer with bf16 weights: 3 forward GEMMs, 3 input-gradient GEMMs
+  (moe_gmm on re-laid-out weights) and 3 weight-gradient launches (moe_tgmm) per step."""
+  import torch
+
+  from maxtext_amd import _lib, megablox, moe, synthetic
+
+  _lib.load()
+  torch.cuda.set_device(0)
+  wl = synthetic.workload(args.workload, args.tokens)
+  import dataclasses
+
+  cfg = dataclasses.replace(wl.cfg, act_quant=None, shared_experts=0)
+  e, d, f, k, t = cfg.num_experts, cfg.emb_dim, cfg.moe_mlp_dim, cfg.num_experts_per_tok, wl.tokens
+  g = torch.Generator(device="cuda").manual_seed(0)
+  mk = lambda *shape: (torch.randn(*shape, device="cuda", generator=g) * 0.02).to(torch.bfloat16).requires_grad_()
+  w0, w1, wo = mk(e, f, d), mk(e, f, d), mk(e, d, f)
+  x = torch.randn(1, t, d, device="cuda", generator=g).to(torch.bfloat16).requires_grad_()
+  dout = torch.randn(1, t, d, device="cuda", generator=g).to(torch.bfloat16)
+  logits = torch.randn(1, t, e, device="cuda", generator=g)
+  pre = torch.sigmoid(logits) if cfg.is_deepseek else None
+  block = moe.RoutedMoE(cfg, w0, w1, wo)
+
+  def step():
+    for v in (x, w0, w1, wo):
+      v.grad = None
+    out = block.sparse_matmul(x, logits, pre, w0, w1, wo)[0]
+    out.backward(dout)
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  megablox.PROFILE_EVENTS = []
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+  events, megablox.PROFILE_EVENTS = megablox.PROFILE_EVENTS, None
+  stage_ms = {}
+  for name in sorted({n for n, _, _ in events}):
+    ts = [a.elapsed_time(b) for n, a, b in events if n == name]
+    stage_ms[name] = sum(ts) / len(ts)
+  m = t * k
+  dom = f"tgmm_k{d}_n{f}"  # weight gradient of wi_0 / wi_1: [E, f, d] from x [M, d] and d h [M, f]
+  dom_ms = stage_ms[dom]
+  achieved = 2.0 * m * d * f / (dom_ms * 1e-3) / 1e12
+  flops = 18.0 * m * d * f
+  result = {
+      "metric": "moe_bf16_layer_fwd_bwd_tflops", "value": flops / (elapsed / args.steps) / 1e12, "unit": "TFLOP/s",
+      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": f"{wl.name} shape, training: forward + backward of the MoE expert layer, {t} tokens, d_model {d}, "
+                             f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU",
+                 "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
+      "roofline": dict(bound="mfma", achieved=achieved, peak=PEAK_TFLOPS["bf16"], unit="TFLOP/s", frac=achieved / PEAK_TFLOPS["bf16"],
+                       traffic=None, kernel="tgmm_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
+      "stage_ms": stage_ms,
+  }
+  if not args.no_cpu_baseline:
+    result["cpu_baseline"] = train_cpu_baseline(wl, args.cpu_sample_tokens or 1024)
+  print(json.dumps(result))
+
+
 def main():
   args = parse()
   if args.gpus != 1:
@@ -109,6 +210,8 @@ def main():
     print("bench.py needs a GPU", file=sys.stderr)
     sys.exit(2)
   torch.cuda.set_device(0)
+  if args.train:
+    return train_main(args)
 
   wl = synthetic.workload(args.workload, args.tokens)
   cfg = wl.cfg

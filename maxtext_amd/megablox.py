@@ -19,6 +19,9 @@ from maxtext_amd import kernels, quantizations
 from maxtext_amd._lib import MOE_INT4
 from maxtext_amd.quantizations import QArray
 
+# When set to a list, the backward pass of gmm appends (stage, start_event, end_event) recorded on the launch stream.
+PROFILE_EVENTS = None
+
 _INT8_NAMES = ("int8", torch.int8)
 _FP8_NAMES = ("fp8", "float8_e4m3fn", torch.float8_e4m3fn)
 _INT4_NAMES = ("int4",)
@@ -222,14 +225,25 @@ class _GmmFn(torch.autograd.Function):
     lhs, rhs, group_sizes = ctx.saved_tensors
     dout = dout.contiguous()
     dlhs = drhs = None
+    ev = PROFILE_EVENTS
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(3)] if ev is not None else None
     with torch.no_grad():
+      if marks:
+        marks[0].record()
       if ctx.needs_input_grad[0]:
         # dout [m, n] @ rhs[g]^T: the kernel's weight layout [G, out, in] is here [G, k, n]
         dlhs = gmm(dout, rhs, group_sizes, group_offset=ctx.offset, transpose_rhs=not ctx.transpose_rhs)
         # rows of groups outside [offset, offset + G_local) are zero in the forward output
+      if marks:
+        marks[1].record()
       if ctx.needs_input_grad[1]:
         d = tgmm(lhs.t(), dout, group_sizes, rhs.dtype, group_offset=ctx.offset, num_actual_groups=rhs.shape[0])
         drhs = d.transpose(1, 2) if ctx.transpose_rhs else d.contiguous()
+      if marks:
+        marks[2].record()
+        shape = f"k{lhs.shape[1]}_n{dout.shape[1]}"
+        ev.append(("dlhs_" + shape, marks[0], marks[1]))
+        ev.append(("tgmm_" + shape, marks[1], marks[2]))
     return dlhs, drhs, None, None, None, None, None
 
 
