@@ -27,6 +27,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "c2": (2335090 * 2.0 + 459081 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
     "c3": (3829460 * 2.0 + 9218 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
+    "c2_train": (3100853 * 2.0 + 917551 * 1.0) * 1024,  # profiles/tgmm_kernel_bf16_mixtral_shape_train.md
 }
 
 
@@ -186,7 +187,8 @@ def train_main(args):
                              f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU",
                  "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
       "roofline": dict(bound="mfma", achieved=achieved, peak=PEAK_TFLOPS["bf16"], unit="TFLOP/s", frac=achieved / PEAK_TFLOPS["bf16"],
-                       traffic=None, kernel="tgmm_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
+                       traffic=MEASURED_TRAFFIC_BYTES.get(wl.name + "_train") if args.tokens is None else None,
+                       kernel="tgmm_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
       "stage_ms": stage_ms,
   }
   if not args.no_cpu_baseline:
