@@ -40,6 +40,7 @@ def parse():
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--graph", action="store_true", help="replay the layer as one captured HIP graph (launch-bound shapes)")
   ap.add_argument("--train", action="store_true",
                   help="forward + backward of the layer with bf16 weights of the workload's shape (weight and input gradients)")
   ap.add_argument("--calibrate-copy", action="store_true",
@@ -228,6 +229,14 @@ def main():
       return block.sparse_matmul(x, logits, pre)[0]
     return block.sparse_matmul(x, logits, pre, layer["wi_0"], layer["wi_1"], layer["wo"])[0]
 
+  if args.graph:
+    from maxtext_amd import graph as graph_mod
+
+    graphed = graph_mod.GraphedLayer(block, x, logits, pre)
+    gx, gl, gp = graphed.inputs
+    eager_step = step
+    step = lambda: graphed(gx, gl, gp)
+
   for _ in range(args.warmup):
     step()
   torch.cuda.synchronize()
@@ -238,6 +247,10 @@ def main():
     out = step()
   torch.cuda.synchronize()
   elapsed = time.perf_counter() - t0
+  if args.graph:  # per-kernel events cannot be recorded inside a replay: time the same kernels in a few eager steps
+    for _ in range(3):
+      eager_step()
+    torch.cuda.synchronize()
   events = routed.profile_events
   routed.profile_events = None
   ms_per_step = elapsed * 1e3 / args.steps
@@ -286,6 +299,7 @@ def main():
       },
       "roofline": roofline,
       "stage_ms": stage_ms,
+      "graph": bool(args.graph),
       "layer_gbps": None,
   }
   # whole-layer minimum HBM traffic (weights of non-empty experts + activations in/out), for HBM-bound shapes

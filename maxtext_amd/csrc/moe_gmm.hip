@@ -891,11 +891,24 @@ struct WqSkinnyParams {
   float act_limit;
 };
 
+// Raw weight bytes of one lane for one 128-wide k block: 32 values = 16 bytes (int4) or 32 bytes (int8).
 template <bool INT4>
-__device__ __forceinline__ void widen32(const uint8_t* p, float scale, v8bf (&w)[4]) {
+struct WqRaw {
+  uint4 q0, q1;
+};
+
+template <bool INT4>
+__device__ __forceinline__ WqRaw<INT4> wq_load(const uint8_t* p) {
+  WqRaw<INT4> r;
+  r.q0 = *(const uint4*)p;
+  r.q1 = INT4 ? make_uint4(0, 0, 0, 0) : *(const uint4*)(p + 16);
+  return r;
+}
+
+template <bool INT4>
+__device__ __forceinline__ void widen32(const WqRaw<INT4>& raw, float scale, v8bf (&w)[4]) {
   if (INT4) {
-    const uint4 q = *(const uint4*)p;
-    const uint32_t x[4] = {q.x, q.y, q.z, q.w};
+    const uint32_t x[4] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w};
 #pragma unroll
     for (int s = 0; s < 4; s++) {
       uint32_t o[4];
@@ -907,8 +920,7 @@ __device__ __forceinline__ void widen32(const uint8_t* p, float scale, v8bf (&w)
       w[s] = __builtin_bit_cast(v8bf, make_uint4(o[0], o[1], o[2], o[3]));
     }
   } else {
-    const uint4 q0 = *(const uint4*)p, q1 = *(const uint4*)(p + 16);
-    const uint32_t x[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const uint32_t x[8] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w, raw.q1.x, raw.q1.y, raw.q1.z, raw.q1.w};
 #pragma unroll
     for (int s = 0; s < 4; s++) {
       uint32_t o[4];
@@ -923,20 +935,26 @@ __device__ __forceinline__ void widen32(const uint8_t* p, float scale, v8bf (&w)
   }
 }
 
-template <bool INT4, int MT, int NT, bool GLU>
+// A block owns 16*NT output channels of one m-tile; its 4 waves split K into 4 contiguous ranges of
+// 128-wide blocks and add their partial sums through LDS at the end (decode has few tiles, and a single
+// wave walking all of K is bound by the latency of its dependent loads, not by bandwidth).  Within its
+// range a wave issues the loads of U blocks before it converts and multiplies the first one.
+template <bool INT4, int MT, int NT, bool GLU, int U>
 __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams p) {
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  constexpr int NACC = NT * MT * 4 * (GLU ? 2 : 1);
+  __shared__ float red[3 * NACC * kWave];
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int j = lane % 16, kq = lane / 16;
   const int m_idx = blockIdx.x / p.n_blocks;
   if (m_idx >= p.header[0]) return;
   const TileInfo tile = p.tiles[m_idx];
   const int N = p.N, K = p.K;
   constexpr int WN = 16 * NT;
-  const int n_w = (blockIdx.x % p.n_blocks) * (4 * WN) + wave * WN;
-  if (n_w >= N) return;
+  const int n_w = (blockIdx.x % p.n_blocks) * WN;
 
   if (tile.group < 0) {
-    for (int i = lane; i < tile.nrows * (WN / 4); i += kWave) {
+    for (int i = threadIdx.x; i < tile.nrows * (WN / 4); i += 256) {
       int r = i / (WN / 4), c = n_w + (i % (WN / 4)) * 4;
       if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
     }
@@ -973,38 +991,152 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
       acc_u[t][mt] = v4f{0.f, 0.f, 0.f, 0.f};
     }
 
-  for (int kb = 0; kb < nkb; kb++) {
-    // this lane's 32 k values exist unless the block is the partial tail
-    const bool live = kb * 128 + kq * 32 < K;
-    const size_t woff = live ? (size_t)kb * (INT4 ? 64 : 128) : 0;
-    v8bf af[MT][4];
+  auto step = [&](int kb0, auto ucount) {
+    constexpr int UC = decltype(ucount)::value;
+    uint4 araw[UC][MT][4];
+    WqRaw<INT4> wraw[UC][NT], uraw[UC][NT];
+    uint16_t wsc[UC][NT], usc[UC][NT];
+    bool live[UC];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-      const uint8_t* a = ap[mt] + (live ? (size_t)kb * 256 : 0);
+    for (int u = 0; u < UC; u++) {
+      const int kb = kb0 + u;
+      // this lane's 32 k values exist unless the block is the partial tail
+      live[u] = kb * 128 + kq * 32 < K;
+      const size_t woff = live[u] ? (size_t)kb * (INT4 ? 64 : 128) : 0;
 #pragma unroll
-      for (int s = 0; s < 4; s++) {
-        uint4 v = *(const uint4*)(a + s * 16);
-        if (!live) v = make_uint4(0, 0, 0, 0);
-        af[mt][s] = __builtin_bit_cast(v8bf, v);
+      for (int t = 0; t < NT; t++) {
+        wraw[u][t] = wq_load<INT4>(wp[t] + woff);
+        if (GLU) uraw[u][t] = wq_load<INT4>(up[t] + woff);
+        if (INT4) {
+          wsc[u][t] = wsp[t][kb];
+          if (GLU) usc[u][t] = usp[t][kb];
+        }
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const uint8_t* a = ap[mt] + (live[u] ? (size_t)kb * 256 : 0);
+#pragma unroll
+        for (int s = 0; s < 4; s++) araw[u][mt][s] = *(const uint4*)(a + s * 16);
       }
     }
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-      v8bf wf[4], uf[4];
-      const float ws = INT4 ? bf16_bits_to_f32(wsp[t][kb]) : 1.0f;
-      widen32<INT4>(wp[t] + woff, ws, wf);
-      if (GLU) {
-        const float us = INT4 ? bf16_bits_to_f32(usp[t][kb]) : 1.0f;
-        widen32<INT4>(up[t] + woff, us, uf);
+    for (int u = 0; u < UC; u++) {
+      if constexpr (INT4) {
+        // A nibble n (stored value + 8) becomes the bf16 number 128 + n by OR-ing it into the mantissa of
+        // 128.0 (0x4300): one AND-OR per pair of values, pairs (k, k+4) of each 8-nibble word.  The MFMA then
+        // yields P = sum (128 + n_k) a_k; with SA = sum a_k from one more MFMA against a row of ones, the block's
+        // contribution is scale * (P - 136 * SA), applied in f32.  The activations are permuted to the same
+        // k order (k0,k4,k1,k5,k2,k6,k3,k7) with byte permutes.
+        v8bf af[MT][4];
+        v4f sa[MT];
+        const v8bf ones = __builtin_bit_cast(v8bf, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+          sa[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            const uint4 a = live[u] ? araw[u][mt][s] : make_uint4(0, 0, 0, 0);
+            const uint4 q = make_uint4(__builtin_amdgcn_perm(a.z, a.x, 0x05040100u), __builtin_amdgcn_perm(a.z, a.x, 0x07060302u),
+                                       __builtin_amdgcn_perm(a.w, a.y, 0x05040100u), __builtin_amdgcn_perm(a.w, a.y, 0x07060302u));
+            af[mt][s] = __builtin_bit_cast(v8bf, q);
+            sa[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, af[mt][s], sa[mt], 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+          // scales of the 4 channels this lane holds in the accumulator layout: channel 4*kq + r lives in lane 4*kq + r
+          const uint32_t mine = (uint32_t)wsc[u][t] | (GLU ? (uint32_t)usc[u][t] << 16 : 0u);
+          float sg[4], su[4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const uint32_t v = (uint32_t)__builtin_amdgcn_ds_bpermute((4 * kq + r) * 4, (int)mine);
+            sg[r] = __uint_as_float(v << 16);
+            su[r] = __uint_as_float(v & 0xffff0000u);
+          }
+          const uint32_t xw[4] = {wraw[u][t].q0.x, wraw[u][t].q0.y, wraw[u][t].q0.z, wraw[u][t].q0.w};
+          const uint32_t xu[4] = {uraw[u][t].q0.x, uraw[u][t].q0.y, uraw[u][t].q0.z, uraw[u][t].q0.w};
+          constexpr uint32_t M4 = 0x000f000fu, C = 0x43004300u;
+          v8bf wf[4], uf[4];
+#pragma unroll
+          for (int s = 0; s < 4; s++) {
+            wf[s] = __builtin_bit_cast(v8bf, make_uint4((xw[s] & M4) | C, ((xw[s] >> 4) & M4) | C, ((xw[s] >> 8) & M4) | C, ((xw[s] >> 12) & M4) | C));
+            if (GLU)
+              uf[s] = __builtin_bit_cast(v8bf, make_uint4((xu[s] & M4) | C, ((xu[s] >> 4) & M4) | C, ((xu[s] >> 8) & M4) | C, ((xu[s] >> 12) & M4) | C));
+          }
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++) {
+            v4f pg = {0.f, 0.f, 0.f, 0.f}, pu = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+              pg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af[mt][s], pg, 0, 0, 0);
+              if (GLU) pu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[s], af[mt][s], pu, 0, 0, 0);
+            }
+            const float off = 136.0f * sa[mt][0];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              acc_g[t][mt][r] = fmaf(sg[r], pg[r] - off, acc_g[t][mt][r]);
+              if (GLU) acc_u[t][mt][r] = fmaf(su[r], pu[r] - off, acc_u[t][mt][r]);
+            }
+          }
+        }
+      } else {
+        v8bf af[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+          for (int s = 0; s < 4; s++) af[mt][s] = __builtin_bit_cast(v8bf, live[u] ? araw[u][mt][s] : make_uint4(0, 0, 0, 0));
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+          v8bf wf[4], uf[4];
+          widen32<INT4>(wraw[u][t], 1.0f, wf);
+          if (GLU) widen32<INT4>(uraw[u][t], 1.0f, uf);
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+              acc_g[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af[mt][s], acc_g[t][mt], 0, 0, 0);
+              if (GLU) acc_u[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[s], af[mt][s], acc_u[t][mt], 0, 0, 0);
+            }
+        }
       }
+    }
+  };
+
+  const int chunk = (nkb + 3) / 4;
+  int kb = wave * chunk;
+  const int kb_end = min(nkb, kb + chunk);
+  for (; kb + U <= kb_end; kb += U) step(kb, std::integral_constant<int, U>{});
+  for (; kb < kb_end; kb++) step(kb, std::integral_constant<int, 1>{});
+
+  // partial sums of waves 1..3 -> LDS -> wave 0
+  if (wave > 0) {
+    float* r = red + (size_t)(wave - 1) * NACC * kWave + lane;
+    int i = 0;
+#pragma unroll
+    for (int t = 0; t < NT; t++)
 #pragma unroll
       for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-          acc_g[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s], af[mt][s], acc_g[t][mt], 0, 0, 0);
-          if (GLU) acc_u[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[s], af[mt][s], acc_u[t][mt], 0, 0, 0);
+        for (int c = 0; c < 4; c++) {
+          r[(i++) * kWave] = acc_g[t][mt][c];
+          if (GLU) r[(i++) * kWave] = acc_u[t][mt][c];
         }
-    }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; w++) {
+    const float* r = red + (size_t)w * NACC * kWave + lane;
+    int i = 0;
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          acc_g[t][mt][c] += r[(i++) * kWave];
+          if (GLU) acc_u[t][mt][c] += r[(i++) * kWave];
+        }
   }
 
   dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
@@ -1170,13 +1302,14 @@ static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int ma
 template <bool INT4, int MT>
 static int launch_wq_skinny(WqSkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
   constexpr int NT = 2;
-  p.n_blocks = cdiv(p.N, 64 * NT);
+  constexpr int U = MT == 1 ? 3 : 2;
+  p.n_blocks = cdiv(p.N, 16 * NT);
   const long long blocks = (long long)max_tiles * p.n_blocks;
   if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
   if (glu)
-    gmm_wq_skinny_kernel<INT4, MT, NT, true><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<INT4, MT, NT, true, U><<<(unsigned)blocks, 256, 0, s>>>(p);
   else
-    gmm_wq_skinny_kernel<INT4, MT, NT, false><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<INT4, MT, NT, false, U><<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_launch("gmm_wq_skinny_kernel");
 }
 
