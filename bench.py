@@ -40,6 +40,8 @@ def parse():
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--gate", action="store_true",
+                  help="include the router in the step: gate matmul + top-k from x (moe_gate_route) instead of given logits")
   ap.add_argument("--graph", action="store_true", help="replay the layer as one captured HIP graph (launch-bound shapes)")
   ap.add_argument("--train", action="store_true",
                   help="forward + backward of the layer with bf16 weights of the workload's shape (weight and input gradients)")
@@ -224,7 +226,15 @@ def main():
   routed = block.routed if cfg.shared_experts else block
   x, logits, pre = layer["x"], layer["gate_logits"], layer["pre_bias_logits"]
 
+  if args.gate:
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    routed.gate_kernel = torch.randn(cfg.emb_dim, cfg.num_experts, device="cuda", generator=gen) * 0.02
+    if cfg.is_deepseek:
+      routed.gate_bias = torch.randn(cfg.num_experts, device="cuda", generator=gen) * 0.01
+
   def step():
+    if args.gate:
+      return block(x)[0]
     if cfg.shared_experts:
       return block.sparse_matmul(x, logits, pre)[0]
     return block.sparse_matmul(x, logits, pre, layer["wi_0"], layer["wi_1"], layer["wo"])[0]
@@ -232,7 +242,7 @@ def main():
   if args.graph:
     from maxtext_amd import graph as graph_mod
 
-    graphed = graph_mod.GraphedLayer(block, x, logits, pre)
+    graphed = graph_mod.GraphedLayer(block, x, None if args.gate else logits, None if args.gate else pre)
     gx, gl, gp = graphed.inputs
     eager_step = step
     step = lambda: graphed(gx, gl, gp)
@@ -256,7 +266,7 @@ def main():
   ms_per_step = elapsed * 1e3 / args.steps
 
   # group sizes of this batch (read back after the timed region) for the algorithmic work model
-  _, sel = routed.get_topk(logits, pre)
+  _, sel = routed.gate_and_route(x.reshape(-1, cfg.emb_dim)) if args.gate else routed.get_topk(logits, pre)
   gs = torch.bincount(sel.reshape(-1).long(), minlength=cfg.num_experts)
   if cfg.shared_experts:
     gs = torch.cat([gs, torch.tensor([wl.tokens], device=gs.device)])
@@ -300,6 +310,7 @@ def main():
       "roofline": roofline,
       "stage_ms": stage_ms,
       "graph": bool(args.graph),
+      "gate_in_step": bool(args.gate),
       "layer_gbps": None,
   }
   # whole-layer minimum HBM traffic (weights of non-empty experts + activations in/out), for HBM-bound shapes

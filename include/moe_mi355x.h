@@ -85,6 +85,32 @@ MOE_API int moe_route_topk(const float* gate_logits, const float* pre_bias_logit
                    float* topk_weights, int32_t* topk_idx, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Router: gate matmul + score function + bias + top-k through one call.  Replaces GateLogit.__call__
+ * (src/maxtext/layers/moe.py:353-392) followed by RoutedMoE.get_topk (moe.py:717-765):
+ *
+ *   logits   = x @ Wg                       (f32 accumulation)
+ *   scores   = sigmoid(logits) if score_func == 1 else logits;   pre_bias = scores   (moe.py:382-386)
+ *   scores  += gate_bias                                                              (moe.py:388-390)
+ *   (topk_weights, topk_idx) = moe_route_topk(scores, pre_bias, ...)
+ *
+ *   x                  [T, d] bf16
+ *   gate_kernel_terms  [num_terms, E, d] bf16: Wg^T written as a sum of bf16 terms.  num_terms == 3
+ *                      (hi, mid, lo; hi = bf16(w), mid = bf16(w - hi), lo = bf16(w - hi - mid)) reproduces
+ *                      the f32 gate (float32_gate_logits, moe.py:494-495): every product is exact in f32;
+ *                      num_terms == 1 with gate_round_bf16 = 1 is the bf16 gate.
+ *   gate_bias          [E] f32 or NULL
+ *   gate_logits_out, pre_bias_logits_out   [T, E] f32 or NULL (the two values GateLogit returns)
+ *   workspace          moe_gate_route_workspace_bytes(T, d, E) bytes (K-split partial sums, added in a fixed order)
+ * The remaining arguments are those of moe_route_topk.  Limits: d % 64 == 0, E % 4 == 0, E <= 512, k <= 16.
+ */
+MOE_API size_t moe_gate_route_workspace_bytes(int T, int d, int E);
+MOE_API int moe_gate_route(const void* x, const void* gate_kernel_terms, int num_terms, const float* gate_bias, int T,
+                           int d, int E, int k, int score_func, int gate_round_bf16, int mode, int norm_topk_prob,
+                           int weights_round_bf16, float routed_scaling_factor, int n_routing_groups,
+                           int topk_routing_group, float* topk_weights, int32_t* topk_idx, float* gate_logits_out,
+                           float* pre_bias_logits_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Sort by expert.  Replaces the index half of RoutedMoE.permute
  * (moe.py:950-954, :960, :986-991): jnp.argsort (stable) of the flattened
  * expert ids, jnp.bincount, and repeat(arange(E), group_size).

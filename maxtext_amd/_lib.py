@@ -58,6 +58,9 @@ SIGNATURES = {
     "moe_last_error": (ctypes.c_char_p, []),
     "moe_abi_version": (c_int, []),
     "moe_route_topk": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "moe_gate_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "moe_gate_route": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                               c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_sort_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_sort_by_expert": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),

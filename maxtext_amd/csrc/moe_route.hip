@@ -53,11 +53,27 @@ __device__ __forceinline__ void wave_argmax(float& bv, int& bi) {
   }
 }
 
+// With GATE the scores are built here from the partial sums of the gate matmul (GateLogit.__call__,
+// moe.py:353-392): logits = sum of the K-split partials (in split order, so the result does not depend on
+// scheduling), optional bf16 rounding (gate computed in bf16), score function, pre_bias = scores,
+// scores += bias.
+struct GateEpilogue {
+  const float* partials;  // [num_partials, T, E]
+  const float* bias;      // [E] or NULL
+  float* logits_out;      // [T, E] or NULL
+  float* pre_bias_out;    // [T, E] or NULL
+  int num_partials;
+  int score_func;         // 0 none, 1 sigmoid
+  int round_bf16;         // round the matmul result to bf16 first
+};
+
+template <bool GATE>
 __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
     const float* __restrict__ logits, const float* __restrict__ pre_bias, int T, int E, int k,
     int mode, int norm, int round_bf16, float scaling, int n_groups, int topk_groups,
-    float* __restrict__ w_out, int32_t* __restrict__ idx_out) {
+    float* __restrict__ w_out, int32_t* __restrict__ idx_out, const GateEpilogue g) {
   __shared__ float s_row[kRouteWaves][kRouteMaxE];
+  __shared__ float s_pre[GATE ? kRouteWaves : 1][GATE ? kRouteMaxE : 1];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int t_raw = blockIdx.x * kRouteWaves + wave;
   const bool active = t_raw < T;
@@ -69,7 +85,22 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
 #pragma unroll
   for (int j = 0; j < kRouteVpl; j++) {
     int e = lane + kWave * j;
-    v[j] = e < E ? row[e] : -INFINITY;
+    if (GATE) {
+      float x = -INFINITY;
+      if (e < E) {
+        x = 0.f;
+        for (int s = 0; s < g.num_partials; s++) x += g.partials[((size_t)s * T + t) * E + e];
+        if (g.round_bf16) x = round_bf16_fn(x);
+        if (g.score_func == 1) x = 1.0f / (1.0f + expf(-x));
+        s_pre[wave][e] = x;
+        if (active && g.pre_bias_out) g.pre_bias_out[(size_t)t * E + e] = x;
+        if (g.bias) x += g.bias[e];
+        if (active && g.logits_out) g.logits_out[(size_t)t * E + e] = x;
+      }
+      v[j] = x;
+    } else {
+      v[j] = e < E ? row[e] : -INFINITY;
+    }
     if (e >= E) taken |= 1u << j;
   }
 
@@ -141,7 +172,10 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
 
   float w;
   if (mode == MOE_ROUTE_DEEPSEEK) {
-    w = lane < k ? pre_bias[(size_t)t * E + myi] : 0.f;
+    if (GATE)
+      w = lane < k ? s_pre[wave][myi] : 0.f;  // written by this wave's own lanes above
+    else
+      w = lane < k ? pre_bias[(size_t)t * E + myi] : 0.f;
     if (norm) {
       float s = wave_sum(w);
       w = w / (s + 1e-20f);
@@ -163,6 +197,102 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
   if (active && lane < k) {
     w_out[(size_t)t * k + lane] = w;
     idx_out[(size_t)t * k + lane] = myi;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Gate matmul x [T, d] bf16  @  Wg [d, E] f32 -> partial logits f32, Wg given as a sum of S bf16 terms
+// [S, E, d] (S = 3 reproduces f32 products: 3 x 8 mantissa bits; S = 1 is the bf16 gate).  A block owns
+// 32 tokens x 32 experts and one slice of K; its 4 waves split the slice further and add through LDS.
+// Operands go straight from global memory into MFMA fragments: within a 64-element chunk of K, lanes
+// 0-31 take elements 0-31 of their row and lanes 32-63 elements 32-63 (64 contiguous bytes each), the
+// same for both operands, so the contraction order is a fixed permutation of K.
+// ---------------------------------------------------------------------------------------
+
+struct GateGemmParams {
+  const uint16_t* x;   // [T, d] bf16
+  const uint16_t* wg;  // [S, E, d] bf16
+  float* partial;      // [KS, T, E]
+  int T, d, E, S;
+  int chunks_per_block;  // 64-element chunks of K per block (grid.z slices)
+};
+
+template <int S>
+__global__ __launch_bounds__(256) void gate_gemm_kernel(const GateGemmParams p) {
+  __shared__ float red[3 * 16 * kWave];
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int r = lane % 32, g = lane / 32;
+  const int t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
+  const int nchunks = p.d / 64;
+  const int c_begin = blockIdx.z * p.chunks_per_block;
+  const int c_end = min(nchunks, c_begin + p.chunks_per_block);
+  const int per_wave = (c_end - c_begin + 3) / 4;
+  int c = c_begin + wave * per_wave;
+  const int c_stop = min(c_end, c + per_wave);
+
+  const uint8_t* xp = (const uint8_t*)(p.x + (size_t)min(t0 + r, p.T - 1) * p.d) + g * 64;
+  const uint8_t* wp[S];
+#pragma unroll
+  for (int s = 0; s < S; s++) wp[s] = (const uint8_t*)(p.wg + ((size_t)s * p.E + min(e0 + r, p.E - 1)) * p.d) + g * 64;
+
+  v16f acc[S];
+#pragma unroll
+  for (int s = 0; s < S; s++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[s][i] = 0.f;
+
+  auto step = [&](int c0, auto ucount) {
+    constexpr int UC = decltype(ucount)::value;
+    uint4 xr[UC][4], wr[UC][S][4];
+#pragma unroll
+    for (int u = 0; u < UC; u++) {
+      const size_t off = (size_t)(c0 + u) * 128;
+#pragma unroll
+      for (int q = 0; q < 4; q++) xr[u][q] = *(const uint4*)(xp + off + q * 16);
+#pragma unroll
+      for (int s = 0; s < S; s++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) wr[u][s][q] = *(const uint4*)(wp[s] + off + q * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < UC; u++)
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int s = 0; s < S; s++)
+          acc[s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wr[u][s][q]), __builtin_bit_cast(v8bf, xr[u][q]),
+                                                           acc[s], 0, 0, 0);
+  };
+  for (; c + 2 <= c_stop; c += 2) step(c, std::integral_constant<int, 2>{});
+  for (; c < c_stop; c++) step(c, std::integral_constant<int, 1>{});
+
+  // smallest term first, as one would add a float's low bits
+  v16f sum = acc[S - 1];
+#pragma unroll
+  for (int s = S - 2; s >= 0; s--)
+#pragma unroll
+    for (int i = 0; i < 16; i++) sum[i] += acc[s][i];
+
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) red[((wave - 1) * 16 + i) * kWave + lane] = sum[i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; w++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) sum[i] += red[(w * 16 + i) * kWave + lane];
+
+  // D[i = expert][j = token]: lane holds token r and experts 8*q + 4*g + 0..3
+  const int t = t0 + r;
+  if (t >= p.T) return;
+  float* out = p.partial + ((size_t)blockIdx.z * p.T + t) * p.E;
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    const int e = e0 + 8 * q + 4 * g;
+    if (e < p.E) *(float4*)(out + e) = make_float4(sum[4 * q], sum[4 * q + 1], sum[4 * q + 2], sum[4 * q + 3]);
   }
 }
 
@@ -528,10 +658,64 @@ int moe_route_topk(const float* gate_logits, const float* pre_bias_logits, int T
       return fail(MOE_ERR_UNSUPPORTED, "route: bad routing groups %d/%d for E=%d", ng, topk_routing_group, E);
   }
   if (T == 0) return MOE_OK;
-  route_topk_kernel<<<cdiv(T, kRouteWaves), kRouteWaves * kWave, 0, (hipStream_t)stream>>>(
+  route_topk_kernel<false><<<cdiv(T, kRouteWaves), kRouteWaves * kWave, 0, (hipStream_t)stream>>>(
       gate_logits, pre_bias_logits, T, E, k, mode, norm_topk_prob, weights_round_bf16,
-      routed_scaling_factor, ng, topk_routing_group, topk_weights, topk_idx);
+      routed_scaling_factor, ng, topk_routing_group, topk_weights, topk_idx, GateEpilogue{});
   return check_launch("route_topk_kernel");
+}
+
+static int gate_k_splits(int T, int d, int E) {
+  const int tiles = cdiv(T, 32) * cdiv(E, 32), nchunks = d / 64;
+  int ks = 256 / tiles;
+  ks = ks < 1 ? 1 : ks;
+  const int cap = nchunks / 8 < 1 ? 1 : nchunks / 8;  // at least 8 chunks (2 per wave) per block
+  ks = ks > cap ? cap : ks;
+  return ks > 16 ? 16 : ks;
+}
+
+size_t moe_gate_route_workspace_bytes(int T, int d, int E) {
+  if (T < 0 || d <= 0 || E <= 0) return 0;
+  return (size_t)gate_k_splits(T, d, E) * T * E * sizeof(float) + 16;
+}
+
+int moe_gate_route(const void* x, const void* gate_kernel_terms, int num_terms, const float* gate_bias, int T, int d,
+                   int E, int k, int score_func, int gate_round_bf16, int mode, int norm_topk_prob,
+                   int weights_round_bf16, float routed_scaling_factor, int n_routing_groups, int topk_routing_group,
+                   float* topk_weights, int32_t* topk_idx, float* gate_logits_out, float* pre_bias_logits_out,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !gate_kernel_terms || !topk_weights || !topk_idx || !workspace) return fail(MOE_ERR_INVALID_ARG, "gate_route: NULL pointer");
+  if (T < 0 || d <= 0 || E <= 0 || k <= 0) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad sizes T=%d d=%d E=%d k=%d", T, d, E, k);
+  if (num_terms != 1 && num_terms != 3) return fail(MOE_ERR_INVALID_ARG, "gate_route: num_terms must be 1 or 3");
+  if (d % 64 != 0 || E % 4 != 0) return fail(MOE_ERR_UNSUPPORTED, "gate_route: need d %% 64 == 0 and E %% 4 == 0 (d=%d E=%d)", d, E);
+  if (E > kRouteMaxE || k > 16 || k > E) return fail(MOE_ERR_UNSUPPORTED, "gate_route: need k<=16, k<=E<=512 (E=%d k=%d)", E, k);
+  if (score_func != 0 && score_func != 1) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad score_func %d", score_func);
+  if (mode != MOE_ROUTE_SOFTMAX_TOPK && mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad mode %d", mode);
+  int ng = n_routing_groups > 0 ? n_routing_groups : 0;
+  if (ng > 0) {
+    if (mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "gate_route: routing groups need DeepSeek mode");
+    if (ng > kWave || E % ng != 0 || E / ng < 2 || topk_routing_group <= 0 || topk_routing_group > ng)
+      return fail(MOE_ERR_UNSUPPORTED, "gate_route: bad routing groups %d/%d for E=%d", ng, topk_routing_group, E);
+  }
+  if (workspace_bytes < moe_gate_route_workspace_bytes(T, d, E)) return fail(MOE_ERR_WORKSPACE, "gate_route: workspace too small");
+  if (((uintptr_t)x | (uintptr_t)gate_kernel_terms | (uintptr_t)workspace) & 15) return fail(MOE_ERR_UNSUPPORTED, "gate_route: pointers must be 16-byte aligned");
+  if (T == 0) return MOE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const int ks = gate_k_splits(T, d, E);
+  GateGemmParams gp;
+  gp.x = (const uint16_t*)x; gp.wg = (const uint16_t*)gate_kernel_terms; gp.partial = (float*)workspace;
+  gp.T = T; gp.d = d; gp.E = E; gp.S = num_terms; gp.chunks_per_block = cdiv(d / 64, ks);
+  dim3 grid(cdiv(T, 32), cdiv(E, 32), ks);
+  if (num_terms == 3)
+    gate_gemm_kernel<3><<<grid, 256, 0, s>>>(gp);
+  else
+    gate_gemm_kernel<1><<<grid, 256, 0, s>>>(gp);
+  GateEpilogue ge;
+  ge.partials = (const float*)workspace; ge.bias = gate_bias; ge.logits_out = gate_logits_out; ge.pre_bias_out = pre_bias_logits_out;
+  ge.num_partials = ks; ge.score_func = score_func; ge.round_bf16 = gate_round_bf16;
+  route_topk_kernel<true><<<cdiv(T, kRouteWaves), kRouteWaves * kWave, 0, s>>>(
+      nullptr, nullptr, T, E, k, mode, norm_topk_prob, weights_round_bf16, routed_scaling_factor, ng, topk_routing_group,
+      topk_weights, topk_idx, ge);
+  return check_launch("gate_route");
 }
 
 size_t moe_sort_workspace_bytes(int T, int k, int E) {

@@ -15,13 +15,14 @@ class GraphedLayer:
   """Captures `block.sparse_matmul` for fixed input shapes.
 
   block: moe.RoutedMoE or moe.RoutedAndSharedMoE (weights are captured by reference: updating them in
-  place is seen by later replays).  x: [B, S, d] bf16; gate_logits / pre_bias_logits: [B, S, E] f32.
+  place is seen by later replays).  x: [B, S, d] bf16; gate_logits / pre_bias_logits: [B, S, E] f32, or
+  gate_logits=None to capture `block(x)` with the router (gate matmul + top-k) inside the graph.
   """
 
-  def __init__(self, block, x, gate_logits, pre_bias_logits=None, warmup: int = 2):
+  def __init__(self, block, x, gate_logits=None, pre_bias_logits=None, warmup: int = 2):
     self.block = block
     self._x = x.clone()
-    self._logits = gate_logits.clone()
+    self._logits = None if gate_logits is None else gate_logits.clone()
     self._pre = None if pre_bias_logits is None else pre_bias_logits.clone()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -36,18 +37,22 @@ class GraphedLayer:
 
   def _run(self):
     b = self.block
+    if self._logits is None:
+      return b(self._x)[0]
     if getattr(b, "routed", None) is not None:
       return b.sparse_matmul(self._x, self._logits, self._pre)[0]
     return b.sparse_matmul(self._x, self._logits, self._pre, b.wi_0, b.wi_1, b.wo)[0]
 
-  def __call__(self, x, gate_logits, pre_bias_logits=None):
-    if x.shape != self._x.shape or gate_logits.shape != self._logits.shape:
-      raise ValueError(f"captured for x {tuple(self._x.shape)} / logits {tuple(self._logits.shape)}")
-    if (pre_bias_logits is None) != (self._pre is None):
-      raise ValueError("pre_bias_logits must be given exactly when it was given at capture")
+  def __call__(self, x, gate_logits=None, pre_bias_logits=None):
+    if x.shape != self._x.shape:
+      raise ValueError(f"captured for x {tuple(self._x.shape)}")
+    if (gate_logits is None) != (self._logits is None) or (pre_bias_logits is None) != (self._pre is None):
+      raise ValueError("gate_logits / pre_bias_logits must be given exactly when they were given at capture")
+    if gate_logits is not None and gate_logits.shape != self._logits.shape:
+      raise ValueError(f"captured for logits {tuple(self._logits.shape)}")
     if x.data_ptr() != self._x.data_ptr():
       self._x.copy_(x)
-    if gate_logits.data_ptr() != self._logits.data_ptr():
+    if gate_logits is not None and gate_logits.data_ptr() != self._logits.data_ptr():
       self._logits.copy_(gate_logits)
     if self._pre is not None and pre_bias_logits.data_ptr() != self._pre.data_ptr():
       self._pre.copy_(pre_bias_logits)

@@ -53,6 +53,42 @@ def route_topk(gate_logits, pre_bias_logits=None, *, k, mode="softmax_topk", nor
   return w, idx
 
 
+def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_round_bf16=False, mode="softmax_topk",
+               norm_topk_prob=False, weights_round_bf16=True, routed_scaling_factor=1.0, n_routing_groups=-1,
+               topk_routing_group=-1, return_logits=False):
+  """Gate matmul + score function + bias + top-k.  x [T, d] bf16; gate_kernel_terms [S, E, d] bf16 (S = 1 or 3).
+  -> (weights [T,k] f32, indices [T,k] int32[, gate_logits [T,E] f32, pre_bias_logits [T,E] f32])."""
+  _need(x, "x", torch.bfloat16, 2)
+  _need(gate_kernel_terms, "gate_kernel_terms", torch.bfloat16, 3)
+  t, d = x.shape
+  s_, e, d2 = gate_kernel_terms.shape
+  if d2 != d:
+    raise ValueError(f"gate kernel has d={d2}, x has d={d}")
+  if gate_bias is not None:
+    _need(gate_bias, "gate_bias", torch.float32, 1)
+    if gate_bias.numel() != e:
+      raise ValueError("gate_bias must have E elements")
+  if score_func not in ("", "sigmoid"):
+    raise NotImplementedError(f"score_func {score_func!r}")
+  if mode not in ("softmax_topk", "deepseek"):
+    raise ValueError(f"unknown routing mode {mode!r}")
+  dev = x.device
+  w = torch.empty((t, k), dtype=torch.float32, device=dev)
+  idx = torch.empty((t, k), dtype=torch.int32, device=dev)
+  logits = torch.empty((t, e), dtype=torch.float32, device=dev) if return_logits else None
+  pre = torch.empty((t, e), dtype=torch.float32, device=dev) if return_logits else None
+  lib = _lib.load()
+  ws = torch.empty((max(lib.moe_gate_route_workspace_bytes(t, d, e), 16),), dtype=torch.uint8, device=dev)
+  st = lib.moe_gate_route(_lib.ptr(x), _lib.ptr(gate_kernel_terms), s_, _lib.ptr(gate_bias), t, d, e, k,
+                          1 if score_func == "sigmoid" else 0, int(bool(gate_round_bf16)),
+                          MOE_ROUTE_DEEPSEEK if mode == "deepseek" else MOE_ROUTE_SOFTMAX_TOPK, int(bool(norm_topk_prob)),
+                          int(bool(weights_round_bf16)), float(routed_scaling_factor), int(n_routing_groups),
+                          int(topk_routing_group), _lib.ptr(w), _lib.ptr(idx), _lib.ptr(logits), _lib.ptr(pre), _lib.ptr(ws),
+                          ws.numel(), _lib.current_stream())
+  _lib.check(st, "moe_gate_route")
+  return (w, idx, logits, pre) if return_logits else (w, idx)
+
+
 def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True):
   """-> (perm [M], inv_perm [M], group_sizes [E], sorted_experts [M] or None), all int32."""
   _need(topk_idx, "topk_idx", torch.int32, 2)

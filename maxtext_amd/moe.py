@@ -100,6 +100,7 @@ class RoutedMoE:
     self.num_experts_per_tok = config.num_experts_per_tok
     self.wi_0, self.wi_1, self.wo = wi_0, wi_1, wo
     self.gate_kernel, self.gate_bias = gate_kernel, gate_bias
+    self._gate_terms = None  # [S, E, d] bf16 form of gate_kernel for moe_gate_route, built on first use
     # when set to a list, _experts appends (stage, start_event, end_event) recorded on the launch stream
     self.profile_events = None
 
@@ -116,6 +117,27 @@ class RoutedMoE:
     if self.gate_bias is not None:
       out = out + self.gate_bias.float()
     return out.contiguous(), pre_bias
+
+  # -- GateLogit.__call__ + get_topk through one entry point (no [T, E] round trip through torch) ---------
+  def gate_and_route(self, inputs_2d: torch.Tensor, return_logits: bool = False):
+    """-> (weights [T,k] f32, indices [T,k] int32[, gate_logits, pre_bias_logits])."""
+    cfg = self.config
+    if cfg.routed_score_func not in ("", "sigmoid"):
+      raise NotImplementedError(cfg.routed_score_func)
+    if self._gate_terms is None or self._gate_terms.device != inputs_2d.device:
+      from maxtext_amd.quantizations import split_gate_kernel
+
+      self._gate_terms = split_gate_kernel(self.gate_kernel, 3 if cfg.float32_gate_logits else 1).to(inputs_2d.device)
+    bias = None if self.gate_bias is None else self.gate_bias.float().contiguous()
+    common = dict(k=self.num_experts_per_tok, score_func=cfg.routed_score_func, gate_round_bf16=not cfg.float32_gate_logits,
+                  return_logits=return_logits)
+    x = inputs_2d.to(torch.bfloat16).contiguous()
+    if cfg.is_deepseek:
+      return kernels.gate_route(x, self._gate_terms, bias, mode="deepseek",
+                                norm_topk_prob=cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"),
+                                routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups,
+                                topk_routing_group=cfg.topk_routing_group, **common)
+    return kernels.gate_route(x, self._gate_terms, bias, norm_topk_prob=cfg.norm_topk_prob, **common)
 
   # -- get_topk (moe.py:717-765) ------------------------------------------------------------
   def get_topk(self, gate_logits: torch.Tensor, pre_bias_logits: Optional[torch.Tensor] = None):
@@ -223,15 +245,15 @@ class RoutedMoE:
 
   # -- sparse_matmul (moe.py:1403), single device -------------------------------------------
   def sparse_matmul(self, inputs, gate_logits, pre_bias_logits, w0_kernel, w1_kernel, wo_kernel,
-                    w0_bias=None, w1_bias=None, wo_bias=None, input_ids=None):
-    """-> (output [B,S,d], lb_loss, bias_updates)."""
+                    w0_bias=None, w1_bias=None, wo_bias=None, input_ids=None, routing=None):
+    """-> (output [B,S,d], lb_loss, bias_updates).  `routing` = (weights, indices) skips get_topk."""
     if w0_bias is not None or w1_bias is not None or wo_bias is not None:
       raise NotImplementedError("mlp_bias is not implemented")
     cfg = self.config
     b, s, d = inputs.shape
     k = self.num_experts_per_tok
     x2d = inputs.reshape(b * s, d).contiguous()
-    weights, selected = self.get_topk(gate_logits, pre_bias_logits)
+    weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits)
     perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
                                                       want_sorted_experts=False)
     training = torch.is_grad_enabled() and any(
@@ -255,6 +277,11 @@ class RoutedMoE:
     """-> (output, lb_loss, bias_updates), as moe.py:3143."""
     b, s, d = inputs.shape
     routing_inputs = inputs if gate_inputs is None else gate_inputs
+    needs_grad = torch.is_grad_enabled() and any(
+        isinstance(t, torch.Tensor) and t.requires_grad for t in (routing_inputs, self.gate_kernel, self.gate_bias))
+    if not needs_grad and routing_inputs.dtype == torch.bfloat16 and routing_inputs.shape[-1] % 64 == 0 and self.num_experts % 4 == 0:
+      routing = self.gate_and_route(routing_inputs.reshape(b * s, -1))
+      return self.sparse_matmul(inputs, None, None, self.wi_0, self.wi_1, self.wo, routing=routing)
     gate_logits, pre_bias = self.gate(routing_inputs.reshape(b * s, -1))
     gate_logits = gate_logits.reshape(b, s, -1)
     pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
@@ -278,12 +305,12 @@ class RoutedAndSharedMoE:
     if n_stacked != config.num_experts + 1:
       raise ValueError("expert tensors must hold num_experts routed experts followed by the shared expert")
 
-  def sparse_matmul(self, inputs, gate_logits, pre_bias_logits):
+  def sparse_matmul(self, inputs, gate_logits, pre_bias_logits, routing=None):
     cfg, r = self.config, self.routed
     b, s, d = inputs.shape
     t, k, e = b * s, cfg.num_experts_per_tok, cfg.num_experts
     x2d = inputs.reshape(t, d).contiguous()
-    w, sel = r.get_topk(gate_logits, pre_bias_logits)
+    w, sel = routing if routing is not None else r.get_topk(gate_logits, pre_bias_logits)
     sel = torch.cat([sel.reshape(t, k), torch.full((t, 1), e, dtype=torch.int32, device=sel.device)], 1).contiguous()
     w = torch.cat([w.reshape(t, k), torch.ones((t, 1), dtype=torch.float32, device=w.device)], 1).contiguous()
     perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + 1, want_sorted_experts=False)
@@ -301,6 +328,13 @@ class RoutedAndSharedMoE:
 
   def __call__(self, inputs, input_ids=None, gate_inputs=None, out_sharding=None):
     b, s, d = inputs.shape
+    if inputs.dtype == torch.bfloat16 and d % 64 == 0 and cfg_ok(self.config):
+      return self.sparse_matmul(inputs, None, None, routing=self.routed.gate_and_route(inputs.reshape(b * s, -1)))
     gate_logits, pre_bias = self.routed.gate(inputs.reshape(b * s, -1))
     pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
     return self.sparse_matmul(inputs, gate_logits.reshape(b, s, -1), pre_bias)
+
+
+def cfg_ok(cfg: MoEConfig) -> bool:
+  """Whether moe_gate_route covers this configuration's router."""
+  return cfg.num_experts % 4 == 0 and cfg.routed_score_func in ("", "sigmoid")

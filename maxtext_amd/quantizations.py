@@ -100,3 +100,18 @@ def quantize_weight_int4(w_gnk: torch.Tensor, group: int = 128) -> QArray:
   u = (q + 8).to(torch.uint8)
   packed = (u[..., 0::2] | (u[..., 1::2] << 4)).contiguous()
   return QArray(packed, scale.squeeze(-1).contiguous(), "int4")
+
+
+def split_gate_kernel(kernel_de: torch.Tensor, terms: int = 3) -> torch.Tensor:
+  """GateLogit kernel [d, E] (f32, moe.py:247-318) -> [terms, E, d] bf16 with sum(terms) == kernel to 24
+  mantissa bits for terms == 3 (hi, mid, lo), the form moe_gate_route consumes; terms == 1 is the bf16 cast
+  the reference applies when the gate runs in bf16 (moe.py:366)."""
+  if terms not in (1, 3):
+    raise ValueError("terms must be 1 or 3")
+  w = kernel_de.detach().float().t().contiguous()
+  out, rest = [], w
+  for _ in range(terms):
+    piece = rest.to(torch.bfloat16)
+    out.append(piece)
+    rest = rest - piece.float()
+  return torch.stack(out).contiguous()

@@ -10,6 +10,8 @@ point work uses torch on the CPU because numpy has no bfloat16 / float8.
 
 How each function is pinned (see tests/test_oracle_*.py):
 
+  gate_logits
+      zero kernel -> sigmoid(0) = 0.5 (+ bias); one-hot kernel columns copy input features.
   top_k, deepseek_routing, expert_group_mask
       hand-computed case of tests/unit/moe_test.py:293-326; brute force.
   calculate_load_balance_updates
@@ -92,6 +94,26 @@ def deepseek_routing(gate_logits, pre_bias_logits, k, n_routing_groups=-1, topk_
   _, idx = top_k(masked, k)
   weights = np.take_along_axis(np.asarray(pre_bias_logits), idx, axis=-1)
   return weights, idx
+
+
+def gate_logits(x: torch.Tensor, kernel: torch.Tensor, bias=None, *, score_func: str = "", deepseek: bool = False,
+                float32_gate_logits: bool = True):
+  """GateLogit.__call__ (moe.py:353-392): inputs and kernel cast to the gate dtype (f32 when
+  float32_gate_logits, moe.py:494), output = inputs @ kernel [d, E], optional score function, pre_bias_logits =
+  output for DeepSeek-V3/V4 (:385-386), output += bias (:388-390).  Returns float32 ndarrays (logits, pre_bias
+  or None).  The f32 matmul is carried in f64 and rounded once."""
+  if float32_gate_logits:
+    out = (x.double() @ kernel.double()).float()
+  else:
+    out = (x.to(torch.bfloat16).double() @ kernel.to(torch.bfloat16).double()).to(torch.bfloat16).float()
+  if score_func == "sigmoid":
+    out = torch.sigmoid(out)
+  elif score_func:
+    raise ValueError(score_func)
+  pre = out.clone() if deepseek else None
+  if bias is not None:
+    out = out + bias.float()
+  return out.numpy(), None if pre is None else pre.numpy()
 
 
 def _softmax_f32(x: np.ndarray) -> np.ndarray:

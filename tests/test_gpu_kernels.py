@@ -497,3 +497,95 @@ def test_gmm_autograd_through_fused_activation():
   assert relerr(la.grad, a.grad) <= 2e-2
   assert relerr(r0.grad, b0.grad) <= 2e-2
   assert relerr(r1.grad, b1.grad) <= 2e-2
+
+
+# ---------------------------------------------------------------- router: gate matmul + top-k in one call
+
+
+def _margin_ok(scores, k, eps):
+  """Tokens whose k+1 best scores are pairwise separated by more than eps (ties are where a different
+  summation order may legitimately pick another expert)."""
+  s = np.sort(scores.astype(np.float64), axis=-1)[:, ::-1][:, : k + 1]
+  return np.all(s[:, :-1] - s[:, 1:] > eps, axis=-1)
+
+
+@pytest.mark.parametrize("t,d,e,k", [(2048, 4096, 8, 2), (256, 7168, 256, 8), (3, 7168, 256, 8), (1, 2880 // 64 * 64, 32, 4), (77, 512, 128, 8)])
+def test_gate_route_softmax_f32(K, t, d, e, k):
+  from maxtext_amd.quantizations import split_gate_kernel
+
+  g = torch.Generator().manual_seed(31)
+  x = torch.randn(t, d, generator=g).to(torch.bfloat16)
+  wg = torch.randn(d, e, generator=g) * 0.02
+  w, idx, logits, pre = K.gate_route(cuda(x), cuda(split_gate_kernel(wg)), k=k, return_logits=True)
+  want_logits, _ = O.gate_logits(x, wg)
+  scale = np.abs(want_logits).max()
+  assert np.abs(logits.cpu().numpy() - want_logits).max() <= 2e-6 * scale  # f32 products, f32 accumulation over d
+  assert torch.equal(pre, logits)
+  ow, oidx = O.get_topk(want_logits, k=k)
+  ok = _margin_ok(want_logits, k, 1e-5 * scale)
+  assert ok.mean() > 0.9
+  np.testing.assert_array_equal(idx.cpu().numpy()[ok], oidx[ok])
+  np.testing.assert_allclose(w.cpu().numpy()[ok], ow[ok], rtol=2.0**-7, atol=1e-6)
+  # and bit-exact against the top-k of the logits the kernel itself produced, ties included
+  ow2, oidx2 = O.get_topk(logits.cpu().numpy(), k=k)
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx2)
+  np.testing.assert_array_equal(w.cpu().numpy(), ow2)
+
+
+def test_gate_route_exact_on_integers(K):
+  """Small-integer activations and gate weights make every partial sum exact in f32, so logits and indices
+  must match the oracle bit for bit whatever the summation order (and the mid / lo terms are zero)."""
+  from maxtext_amd.quantizations import split_gate_kernel
+
+  rng = np.random.default_rng(7)
+  t, d, e, k = 513, 1024, 64, 6
+  x = torch.from_numpy(rng.integers(-4, 5, (t, d)).astype(np.float32)).to(torch.bfloat16)
+  wg = torch.from_numpy(rng.integers(-8, 9, (d, e)).astype(np.float32)) / 16.0
+  terms = split_gate_kernel(wg)
+  assert torch.all(terms[1] == 0) and torch.all(terms[2] == 0)
+  w, idx, logits, _ = K.gate_route(cuda(x), cuda(terms), k=k, norm_topk_prob=True, return_logits=True)
+  want_logits, _ = O.gate_logits(x, wg)
+  np.testing.assert_array_equal(logits.cpu().numpy(), want_logits)
+  ow, oidx = O.get_topk(want_logits, k=k, norm_topk_prob=True)
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx)  # integer logits: many exact ties, lower index first
+  np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=2.0**-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("groups", [(-1, -1), (8, 4)])
+def test_gate_route_deepseek_sigmoid_bias(K, groups):
+  from maxtext_amd.quantizations import split_gate_kernel
+
+  g = torch.Generator().manual_seed(33)
+  t, d, e, k = 200, 1024, 256, 8
+  x = torch.randn(t, d, generator=g).to(torch.bfloat16)
+  wg = torch.randn(d, e, generator=g) * 0.05
+  bias = torch.randn(e, generator=g) * 0.1
+  w, idx, logits, pre = K.gate_route(cuda(x), cuda(split_gate_kernel(wg)), cuda(bias), k=k, score_func="sigmoid", mode="deepseek",
+                                     norm_topk_prob=True, routed_scaling_factor=2.5, n_routing_groups=groups[0],
+                                     topk_routing_group=groups[1], return_logits=True)
+  want_logits, want_pre = O.gate_logits(x, wg, bias, score_func="sigmoid", deepseek=True)
+  assert np.abs(pre.cpu().numpy() - want_pre).max() <= 1e-6
+  assert np.abs(logits.cpu().numpy() - want_logits).max() <= 1e-6
+  # routing on the kernel's own scores must equal the oracle's routing on the same scores, bit for bit
+  ow, oidx = O.get_topk(logits.cpu().numpy(), pre.cpu().numpy(), k=k, mode="deepseek", routed_scaling_factor=2.5,
+                        n_routing_groups=groups[0], topk_routing_group=groups[1])
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+  np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=1e-5)
+
+
+def test_gate_route_bf16_gate_and_errors(K):
+  from maxtext_amd.quantizations import split_gate_kernel
+
+  g = torch.Generator().manual_seed(34)
+  t, d, e, k = 100, 512, 16, 2
+  x = torch.randn(t, d, generator=g).to(torch.bfloat16)
+  wg = torch.randn(d, e, generator=g) * 0.05
+  w, idx, logits, _ = K.gate_route(cuda(x), cuda(split_gate_kernel(wg, 1)), k=k, gate_round_bf16=True, return_logits=True)
+  want, _ = O.gate_logits(x, wg, float32_gate_logits=False)
+  got = logits.cpu().numpy()
+  # f32 accumulation order may move a sum across a bf16 rounding boundary: allow one bf16 ulp on a few values
+  assert np.mean(got != want) < 0.02 and np.abs(got - want).max() <= 2.0**-7 * np.abs(want).max()
+  with pytest.raises(RuntimeError, match="d % 64"):
+    K.gate_route(cuda(x[:, :72].contiguous()), cuda(split_gate_kernel(wg[:72], 1)), k=k)
+  with pytest.raises(ValueError):
+    K.gate_route(cuda(x), cuda(split_gate_kernel(wg[:256], 1)), k=k)

@@ -280,3 +280,37 @@ def test_graph_replay_equals_eager(case):
     torch.cuda.synchronize()
     assert torch.equal(got, want), f"replay {it}"
     _ = (xi.float() @ xi.float().transpose(-1, -2)).sum().item()  # unrelated eager work between replays
+
+
+# ---------------------------------------------------------------- router inside the layer call
+
+
+@pytest.mark.parametrize("deepseek", [False, True])
+def test_layer_call_routes_through_gate_route(deepseek):
+  """block(x) computes the gate inside the HIP path; it must equal sparse_matmul fed with the logits that
+  the same entry point reports (identical routing by construction), and the torch gate within tolerance."""
+  from maxtext_amd import moe, quantizations
+
+  g = torch.Generator().manual_seed(40)
+  t, d, f, e, k = 300, 256, 512, 16, 4
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16).cuda()
+  wg = (torch.randn(d, e, generator=g) * 0.1).cuda()
+  bias = (torch.randn(e, generator=g) * 0.1).cuda() if deepseek else None
+  ws = [(torch.randn(e + (1 if deepseek else 0), n_, k_, generator=g) * 0.05).to(torch.bfloat16).cuda() for n_, k_ in ((f, d), (f, d), (d, f))]
+  if deepseek:
+    cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek3-test",
+                        routed_score_func="sigmoid", routed_bias=True, routed_scaling_factor=2.5, shared_experts=1)
+    block = moe.RoutedAndSharedMoE(cfg, *ws, gate_kernel=wg, gate_bias=bias)
+    routed = block.routed
+  else:
+    cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
+    block = routed = moe.RoutedMoE(cfg, *ws, gate_kernel=wg)
+  out, _, _ = block(x)
+  w, idx, logits, pre = routed.gate_and_route(x.reshape(t, d), return_logits=True)
+  if deepseek:
+    want, _, _ = block.sparse_matmul(x, logits.reshape(1, t, e), pre.reshape(1, t, e))
+  else:
+    want, _, _ = block.sparse_matmul(x, logits.reshape(1, t, e), None, *ws)
+  assert torch.equal(out, want)
+  tl, tp = routed.gate(x.reshape(t, d))
+  assert float((tl - logits).abs().max()) <= 1e-4 * float(tl.abs().max())

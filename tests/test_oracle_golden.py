@@ -340,3 +340,22 @@ def test_tgmm_equals_autograd_of_grouped_matmul_and_hand_case():
   d2 = torch.tensor([[1.0], [10.0], [100.0]])
   t2 = O.tgmm(lhs2, d2, np.array([2, 1], np.int32), out_dtype=torch.float32)
   assert t2.tolist() == [[[31.0], [42.0]], [[500.0], [600.0]]]
+
+
+def test_gate_logits_special_cases():
+  """GateLogit: a zero kernel gives sigmoid(0) = 0.5 everywhere (+ bias, with pre_bias untouched); a kernel
+  whose columns are unit vectors copies input features; the bf16 gate rounds once at the end."""
+  g = torch.Generator().manual_seed(1)
+  x = torch.randn(5, 8, generator=g).to(torch.bfloat16)
+  bias = torch.tensor([0.25, -1.0, 0.0, 2.0])
+  out, pre = O.gate_logits(x, torch.zeros(8, 4), bias, score_func="sigmoid", deepseek=True)
+  assert np.all(pre == 0.5) and np.array_equal(out, np.broadcast_to(0.5 + bias.numpy(), (5, 4)))
+  sel = torch.zeros(8, 4)
+  for e, f in enumerate((6, 0, 3, 3)):
+    sel[f, e] = 1.0
+  out, pre = O.gate_logits(x, sel)
+  assert pre is None and np.array_equal(out, x.float().numpy()[:, [6, 0, 3, 3]])
+  w = torch.randn(8, 4, generator=g)
+  out16, _ = O.gate_logits(x, w, float32_gate_logits=False)
+  want = (x.double() @ w.to(torch.bfloat16).double()).to(torch.bfloat16).float().numpy()
+  assert np.array_equal(out16, want)
