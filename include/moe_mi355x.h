@@ -169,6 +169,7 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  *              ceil(K / rhs_scale_block_k) (must be 128); f32, or bf16 for INT4
  *   rhs_up / rhs_up_scale   second projection (wi_1) with the same layout; when non-NULL
  *              the kernel computes act(lhs@rhs^T) * (lhs@rhs_up^T) in one pass
+ *   rhs_bias / rhs_up_bias   [G_local, N] f32 or NULL, see the end of the struct
  *   out        [M, N] bf16
  *
  * Supported operand combinations (others return MOE_ERR_UNSUPPORTED):
@@ -198,6 +199,11 @@ typedef struct {
   int32_t act;     /* moe_act; must be MOE_ACT_NONE when rhs_up == NULL      */
   float act_limit; /* clip for SWIGLUOAI / SILU_CLIP                        */
   int32_t reserved[4];
+  /* per-expert bias [G_local, N] f32 added to lhs@rhs^T (and to lhs@rhs_up^T) before the activation:
+   * w0_bias / w1_bias / wo_bias of mlp_bias models (moe.py:1952-1981, :2239-2241; rhs_bias of
+   * pallas_mosaic_tpu_v2_gmm_kernel.py:573).  NULL = no bias.  Rows that are written as zeros stay zero. */
+  const float* rhs_bias;
+  const float* rhs_up_bias;
 } moe_gmm_args;
 
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);

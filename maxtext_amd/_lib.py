@@ -51,6 +51,8 @@ class GmmArgs(ctypes.Structure):
       ("act", ctypes.c_int32),
       ("act_limit", c_float),
       ("reserved", ctypes.c_int32 * 4),
+      ("rhs_bias", c_void_p),
+      ("rhs_up_bias", c_void_p),
   ]
 
 

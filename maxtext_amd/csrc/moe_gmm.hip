@@ -116,6 +116,8 @@ struct TiledParams {
   const uint8_t* rhs_up;     // same, or NULL
   const void* rhs_scale;     // f32 [G, N] (per channel) | bf16 [G, N, nkg] (INT4)
   const void* rhs_up_scale;
+  const float* rhs_bias;     // [G, N] f32 or NULL, added before the activation
+  const float* rhs_up_bias;
   const int32_t* header;
   const TileInfo* tiles;
   uint16_t* out;  // [M, N] bf16
@@ -129,6 +131,15 @@ struct TiledParams {
 __device__ __forceinline__ uint32_t i8x2_to_bf16x2(int lo, int hi) {
   // |value| <= 128 is exact in bf16, so truncating the f32 is the conversion
   return (__float_as_uint((float)lo) >> 16) | (__float_as_uint((float)hi) & 0xffff0000u);
+}
+
+// Bias of 4 consecutive output channels of one group (zeros without a bias).
+__device__ __forceinline__ void load_bias4(const float* bias, int group, int N, int n, float (&b)[4]) {
+  b[0] = b[1] = b[2] = b[3] = 0.f;
+  if (bias) {
+    const float4 v = *(const float4*)(bias + (size_t)group * N + n);
+    b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
+  }
 }
 
 // Per-lane scales of the epilogue, fetched before the K loop so their latency hides behind it.  With
@@ -181,12 +192,15 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
         if (n >= p.N) continue;
         const float sg[4] = {e.sg[j][q].x, e.sg[j][q].y, e.sg[j][q].z, e.sg[j][q].w};
         const float su[4] = {e.su[j][q].x, e.su[j][q].y, e.su[j][q].z, e.su[j][q].w};
+        float bg[4], bu[4];
+        load_bias4(p.rhs_bias, tile.group, p.N, n, bg);
+        load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, p.N, n, bu);
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float g = (float)acc[j][i][4 * q + r] * (e.sa[i] * sg[r]);
+          const float g = fmaf((float)acc[j][i][4 * q + r], e.sa[i] * sg[r], bg[r]);
           if (GLU) {
-            const float u = (float)acc[j + NT_OUT][i][4 * q + r] * (e.sa[i] * su[r]);
+            const float u = fmaf((float)acc[j + NT_OUT][i][4 * q + r], e.sa[i] * su[r], bu[r]);
             v[r] = glu_act<ACT>(g, u, p.act_limit);
           } else {
             v[r] = g;
@@ -724,6 +738,8 @@ struct SkinnyParams {
   const uint8_t* rhs_up;
   const float* rhs_scale;  // [G, ceil(N/128), K/128]
   const float* rhs_up_scale;
+  const float* rhs_bias;   // [G, N] f32 or NULL
+  const float* rhs_up_bias;
   const int32_t* header;
   const TileInfo* tiles;
   uint16_t* out;
@@ -854,13 +870,17 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
     for (int t = 0; t < NT; t++) {
       const int n = n_w + t * 16 + 4 * kq;
       if (n >= N) continue;
+      float bg[4], bu[4];
+      load_bias4(p.rhs_bias, tile.group, N, n, bg);
+      load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, N, n, bu);
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
         const int lr = mt * 16 + j;
         if (lr >= tile.nrows) continue;
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r], acc_u[t][mt][r], p.act_limit) : acc_g[t][mt][r];
+        for (int r = 0; r < 4; r++)
+          v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r] + bg[r], acc_u[t][mt][r] + bu[r], p.act_limit) : acc_g[t][mt][r] + bg[r];
         *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
       }
     }
@@ -882,6 +902,8 @@ struct WqSkinnyParams {
   const uint8_t* rhs_up;
   const void* rhs_scale;    // int8: f32 [G, N]; int4: bf16 [G, N, ceil(K/128)]
   const void* rhs_up_scale;
+  const float* rhs_bias;    // [G, N] f32 or NULL
+  const float* rhs_up_bias;
   const int32_t* header;
   const TileInfo* tiles;
   uint16_t* out;
@@ -1146,6 +1168,9 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
       const int n = n_w + t * 16 + 4 * kq;
       if (n >= N) continue;
       float sg[4] = {1.f, 1.f, 1.f, 1.f}, su[4] = {1.f, 1.f, 1.f, 1.f};
+      float bg[4], bu[4];
+      load_bias4(p.rhs_bias, tile.group, N, n, bg);
+      load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, N, n, bu);
       if (!INT4) {
         const float4 a = *(const float4*)((const float*)p.rhs_scale + (size_t)tile.group * N + n);
         sg[0] = a.x; sg[1] = a.y; sg[2] = a.z; sg[3] = a.w;
@@ -1161,7 +1186,8 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r] * sg[r], acc_u[t][mt][r] * su[r], p.act_limit) : acc_g[t][mt][r] * sg[r];
+          v[r] = GLU ? glu_act<ACT>(fmaf(acc_g[t][mt][r], sg[r], bg[r]), fmaf(acc_u[t][mt][r], su[r], bu[r]), p.act_limit)
+                     : fmaf(acc_g[t][mt][r], sg[r], bg[r]);
         *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
       }
     }
@@ -1336,6 +1362,8 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   if (!glu && a->act != MOE_ACT_NONE) return fail(MOE_ERR_INVALID_ARG, "gmm: activation needs rhs_up");
   if (a->act < MOE_ACT_NONE || a->act > MOE_ACT_SILU_CLIP) return fail(MOE_ERR_INVALID_ARG, "gmm: bad act %d", a->act);
   if (a->N % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: N %% 8 != 0 (N=%d)", a->N);
+  if (a->rhs_up_bias && !glu) return fail(MOE_ERR_INVALID_ARG, "gmm: rhs_up_bias needs rhs_up");
+  if (((uintptr_t)a->rhs_bias | (uintptr_t)a->rhs_up_bias) & 15) return fail(MOE_ERR_UNSUPPORTED, "gmm: bias pointers must be 16-byte aligned");
   if (a->M == 0) return MOE_OK;
   const uintptr_t align = (uintptr_t)a->lhs | (uintptr_t)a->rhs | (uintptr_t)a->rhs_up | (uintptr_t)a->out |
                           (uintptr_t)a->rhs_scale | (uintptr_t)a->rhs_up_scale;
@@ -1362,6 +1390,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     p.lhs = (const uint8_t*)a->lhs; p.lhs_scale = a->lhs_scale;
     p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
     p.rhs_scale = (const float*)a->rhs_scale; p.rhs_up_scale = (const float*)a->rhs_up_scale;
+    p.rhs_bias = a->rhs_bias; p.rhs_up_bias = a->rhs_up_bias;
     p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
     p.M = a->M; p.K = a->K; p.N = a->N; p.n_blocks = 0;
     p.act = a->act; p.act_limit = a->act_limit;
@@ -1375,6 +1404,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   p.lhs = (const uint8_t*)a->lhs; p.lhs_scale = nullptr;
   p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
   p.rhs_scale = a->rhs_scale; p.rhs_up_scale = a->rhs_up_scale;
+  p.rhs_bias = a->rhs_bias; p.rhs_up_bias = a->rhs_up_bias;
   p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
   p.M = a->M; p.K = a->K; p.N = a->N; p.max_m_tiles = 0; p.tiles_n = 0;
   p.act = a->act; p.act_limit = a->act_limit; p.dbg = a->reserved[1];
@@ -1413,6 +1443,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     WqSkinnyParams q;
     q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
     q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
+    q.rhs_bias = a->rhs_bias; q.rhs_up_bias = a->rhs_up_bias;
     q.header = header; q.tiles = tiles; q.out = (uint16_t*)a->out;
     q.M = M; q.K = a->K; q.N = a->N; q.n_blocks = 0; q.act = a->act; q.act_limit = a->act_limit;
     const int mx = max_tiles_for(M, G, bm);

@@ -198,7 +198,7 @@ def transpose_rhs(rhs_gkn):
 
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
-            group_offset=0, out=None, tile_variant=0):
+            group_offset=0, out=None, tile_variant=0, rhs_bias=None, rhs_up_bias=None):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4: uint8 [G,N,K/2])."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
@@ -229,6 +229,13 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
       want = torch.bfloat16 if rhs_dtype == MOE_INT4 else torch.float32
       if t.dtype != want or t.numel() != g_local * nnb * nkb_r:
         raise ValueError(f"{name} must be {want} with {g_local}x{nnb}x{nkb_r} elements, got {t.dtype} {tuple(t.shape)}")
+  for name, t in (("rhs_bias", rhs_bias), ("rhs_up_bias", rhs_up_bias)):
+    if t is not None:
+      _need(t, name, torch.float32, 2)
+      if t.shape != (g_local, n):
+        raise ValueError(f"{name} must be [{g_local}, {n}] f32")
+  if rhs_up_bias is not None and rhs_up is None:
+    raise ValueError("rhs_up_bias needs rhs_up")
   if lhs_scale is not None:
     _need(lhs_scale, "lhs_scale", torch.float32)
     nkb_l = 1 if lhs_scale_block_k == 0 else (kdim + lhs_scale_block_k - 1) // lhs_scale_block_k
@@ -258,6 +265,8 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.lhs_scale_block_k, a.rhs_scale_block_n, a.rhs_scale_block_k = int(lhs_scale_block_k), int(rhs_scale_block_n), int(rhs_scale_block_k)
   a.act = _lib.ACT_BY_NAME[act]
   a.act_limit = float(act_limit)
+  a.rhs_bias = rhs_bias.data_ptr() if rhs_bias is not None else None
+  a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
   a.reserved[0] = int(tile_variant)
   a.reserved[1] = int(__import__("os").environ.get("MOE_DBG", "0"))
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())

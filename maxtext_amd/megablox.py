@@ -8,7 +8,8 @@ lhs_quantize_dtype / rhs_quantize_dtype ask for it.
 
 Extra keyword arguments the quantised expert path needs (they follow gmm_v2,
 pallas_mosaic_tpu_v2_gmm_kernel.py:1297-1315): `rhs_up` (second projection, fused
-act(lhs@rhs) * (lhs@rhs_up)) and `fuse_act`.
+act(lhs@rhs) * (lhs@rhs_up)), `fuse_act`, and `rhs_bias` / `rhs_up_bias` ([G, N] per-expert biases
+added before the activation).
 """
 
 from __future__ import annotations
@@ -97,6 +98,8 @@ def gmm(
     rhs_up=None,
     fuse_act=None,
     act_limit=7.0,
+    rhs_bias=None,
+    rhs_up_bias=None,
 ):
   """Grouped matmul: out[rows of group g] = lhs[rows] @ rhs[g] (ops.py:46).
 
@@ -124,7 +127,9 @@ def gmm(
     else:
       offset = int(group_offset)
 
-  if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up)):
+  if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
+    if rhs_bias is not None or rhs_up_bias is not None:
+      raise NotImplementedError("gradients with rhs_bias are not implemented")
     return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit)
 
   rhs_n = _native_rhs(rhs, transpose_rhs)
@@ -137,6 +142,10 @@ def gmm(
     lhs = quantize_lhs(lhs.contiguous(), lhs_quantize_dtype)
 
   kw = dict(act=fuse_act, act_limit=act_limit, group_offset=offset)
+  if rhs_bias is not None:
+    kw["rhs_bias"] = rhs_bias.float().contiguous()  # [G, N] (rhs_bias [G, 1, N] of the v2 kernel, :573)
+  if rhs_up_bias is not None:
+    kw["rhs_up_bias"] = rhs_up_bias.float().contiguous()
   if isinstance(lhs, QArray):
     kw["lhs_scale"] = lhs.scale
     kw["lhs_scale_block_k"] = 128 if lhs.qtype == "fp8" else 0

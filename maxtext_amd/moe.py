@@ -211,7 +211,7 @@ class RoutedMoE:
     return out.reshape(batch_size, sequence_length, -1)
 
   # -- the three grouped GEMMs: gmm_up + apply_ffn_activation + wo (moe.py:1932-1986, :841, :2226)
-  def _experts(self, sorted_inputs, group_size, w0, w1, wo):
+  def _experts(self, sorted_inputs, group_size, w0, w1, wo, w0_bias=None, w1_bias=None, wo_bias=None):
     cfg = self.config
     act, limit = cfg.activation, (cfg.mlp_activations_limit if cfg.mlp_activations_limit > 0 else 7.0)
     ev = self.profile_events
@@ -225,18 +225,21 @@ class RoutedMoE:
       # activation is applied unfused so that its inputs are kept for the backward pass
       if any(isinstance(t, QArray) for t in (sorted_inputs, w0, w1, wo)):
         raise NotImplementedError("gradients need bf16 weights; QArray weights are an inference format")
+      if w0_bias is not None or w1_bias is not None or wo_bias is not None:
+        raise NotImplementedError("gradients with mlp_bias are not implemented")
       q = cfg.act_quant
       inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit, lhs_quantize_dtype=q,
                            rhs_quantize_dtype=q)
       return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q)
-    inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit)
+    inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
+                         rhs_bias=w0_bias, rhs_up_bias=w1_bias)
     if marks:
       marks[1].record()
     if cfg.act_quant is not None:
       inter = megablox.quantize_lhs(inter, cfg.act_quant)
     if marks:
       marks[2].record()
-    out = megablox.gmm(inter, wo, group_size, transpose_rhs=True)
+    out = megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias)
     if marks:
       marks[3].record()
       ev.append(("wi_glu", marks[0], marks[1]))
@@ -246,9 +249,9 @@ class RoutedMoE:
   # -- sparse_matmul (moe.py:1403), single device -------------------------------------------
   def sparse_matmul(self, inputs, gate_logits, pre_bias_logits, w0_kernel, w1_kernel, wo_kernel,
                     w0_bias=None, w1_bias=None, wo_bias=None, input_ids=None, routing=None):
-    """-> (output [B,S,d], lb_loss, bias_updates).  `routing` = (weights, indices) skips get_topk."""
-    if w0_bias is not None or w1_bias is not None or wo_bias is not None:
-      raise NotImplementedError("mlp_bias is not implemented")
+    """-> (output [B,S,d], lb_loss, bias_updates).  `routing` = (weights, indices) skips get_topk.
+    w0_bias / w1_bias [E, moe_mlp_dim] and wo_bias [E, emb_dim] are the per-expert biases of mlp_bias models
+    (moe.py:617-637): every routed row gets the bias of its expert (transform_bias, moe.py:1363)."""
     cfg = self.config
     b, s, d = inputs.shape
     k = self.num_experts_per_tok
@@ -269,7 +272,7 @@ class RoutedMoE:
       sorted_inputs = QArray(q, sc, "fp8")
     else:
       sorted_inputs = kernels.gather_rows(x2d, perm, k)
-    inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel)
+    inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias)
     out = self.unpermute(inter, perm, weights, b, s, inv_perm=inv)
     return out, None, None
 

@@ -589,3 +589,72 @@ def test_gate_route_bf16_gate_and_errors(K):
     K.gate_route(cuda(x[:, :72].contiguous()), cuda(split_gate_kernel(wg[:72], 1)), k=k)
   with pytest.raises(ValueError):
     K.gate_route(cuda(x), cuda(split_gate_kernel(wg[:256], 1)), k=k)
+
+
+# ---------------------------------------------------------------- per-expert bias (mlp_bias models)
+
+
+def _bias(e, n, seed):
+  g = torch.Generator().manual_seed(seed)
+  return torch.randn(e, n, generator=g) * 0.5, torch.randn(e, n, generator=g) * 0.5
+
+
+@pytest.mark.parametrize("m,k,n,gs", [GMM_SHAPES[0], GMM_SHAPES[3], DECODE_SHAPES[0], DECODE_SHAPES[2]])
+def test_gmm_bias_every_kernel_family(K, m, k, n, gs):
+  """rhs_bias / rhs_up_bias through each kernel family: bf16 tiles (small / large), int8 x int8, weight-only int8
+  (tiled or streaming by shape), int4, block-scaled fp8.  Bias enters before the activation (moe.py:1952-1981)
+  and rows that belong to no group stay zero."""
+  from maxtext_amd._lib import MOE_INT4
+
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 17)
+  e = len(gs)
+  b0, b1 = _bias(e, n, 18)
+  ob0, ob1 = b0[:, None, :], b1[:, None, :]
+  act = lambda h0, h1: O.apply_ffn_activation(h0, h1, "swigluoai")
+  used = int(gs.sum())
+
+  def check(got, want):
+    assert relerr(got, want) <= TOL
+    assert torch.all(got[used:] == 0)
+
+  # bf16 x bf16
+  wb, ub = w.to(torch.bfloat16), w_up.to(torch.bfloat16)
+  check(K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), rhs_bias=cuda(b0)), O.gmm(lhs, wb, gs, rhs_bias=ob0))
+  check(K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), rhs_up=cuda(native(ub)), act="swigluoai", rhs_bias=cuda(b0), rhs_up_bias=cuda(b1)),
+        act(O.gmm(lhs, wb, gs, rhs_bias=ob0, out_dtype=torch.float32), O.gmm(lhs, ub, gs, rhs_bias=ob1, out_dtype=torch.float32)))
+  # weight-only int8 and int8 x int8
+  q, s = O.quantize_weight_int8(w)
+  qu, su = O.quantize_weight_int8(w_up)
+  want_glu = act(O.gmm(lhs, q, gs, rhs_scale=s, rhs_bias=ob0, out_dtype=torch.float32), O.gmm(lhs, qu, gs, rhs_scale=su, rhs_bias=ob1, out_dtype=torch.float32))
+  check(K.gmm_raw(cuda(lhs), cuda(native(q)), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(native(qu)), rhs_up_scale=cuda(su), act="swigluoai",
+                  rhs_bias=cuda(b0), rhs_up_bias=cuda(b1)), want_glu)
+  aq, asc = O.quantize_rows_int8(lhs.float())
+  check(K.gmm_raw(cuda(aq), cuda(native(q)), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(s), rhs_bias=cuda(b0)),
+        O.gmm(aq, q, gs, lhs_scale=asc[:, None], rhs_scale=s, rhs_bias=ob0))
+  # int4
+  if k % 32 == 0:
+    q4, s4 = O.quantize_int4_groups(native(w), 128)
+    s4 = s4.to(torch.bfloat16)
+    v2 = lambda sc: sc.float().permute(0, 2, 1)[:, :, None, :]
+    check(K.gmm_raw(cuda(lhs), cuda(O.pack_int4(q4)), cuda(gs), rhs_scale=cuda(s4), rhs_dtype=MOE_INT4, rhs_scale_block_k=128, rhs_bias=cuda(b0)),
+          O.gmm(lhs, q4.transpose(1, 2), gs, rhs_scale=v2(s4), quant_block=128, rhs_bias=ob0))
+  # fp8 block scaled
+  if k % 128 == 0:
+    fq, fsc = O.quantize_fp8_blocks(lhs, 1, 128)
+    wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)
+    uq, usc = O.quantize_fp8_blocks(native(w_up), 128, 128)
+    v2f = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
+    fkw = dict(lhs_scale=cuda(fsc), lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128)
+    okw = dict(lhs_scale=fsc, transpose_rhs=True, quant_block=128, out_dtype=torch.float32)
+    check(K.gmm_raw(cuda(fq), cuda(wq), cuda(gs), rhs_scale=cuda(wsc), rhs_up=cuda(uq), rhs_up_scale=cuda(usc), act="swigluoai",
+                    rhs_bias=cuda(b0), rhs_up_bias=cuda(b1), **fkw),
+          act(O.gmm(fq, wq, gs, rhs_scale=v2f(wsc), rhs_bias=ob0, **okw), O.gmm(fq, uq, gs, rhs_scale=v2f(usc), rhs_bias=ob1, **okw)))
+
+
+def test_gmm_bias_argument_errors(K):
+  lhs, w, _, gs = _gmm_inputs(64, 128, 64, [64], 19)
+  wb = cuda(native(w.to(torch.bfloat16)))
+  with pytest.raises(ValueError):
+    K.gmm_raw(cuda(lhs), wb, cuda(gs), rhs_bias=torch.zeros(1, 32, device="cuda"))
+  with pytest.raises(ValueError):
+    K.gmm_raw(cuda(lhs), wb, cuda(gs), rhs_up_bias=torch.zeros(1, 64, device="cuda"))

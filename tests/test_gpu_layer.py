@@ -314,3 +314,31 @@ def test_layer_call_routes_through_gate_route(deepseek):
   assert torch.equal(out, want)
   tl, tp = routed.gate(x.reshape(t, d))
   assert float((tl - logits).abs().max()) <= 1e-4 * float(tl.abs().max())
+
+
+def test_gpt_oss_style_layer_with_mlp_bias():
+  """GPT-OSS variant (gpt-oss-20b.yml:44-49): clipped swigluoai activation and per-expert biases on all three
+  projections, against the per-token loop formulation in f64 on the GPU's own routing."""
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(50)
+  t, d, f, e, k = 160, 192, 320, 8, 4
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  logits = torch.randn(1, t, e, generator=g)
+  w0, w1 = [(torch.randn(e, f, d, generator=g) * 0.1).to(torch.bfloat16) for _ in range(2)]
+  wo = (torch.randn(e, d, f, generator=g) * 0.1).to(torch.bfloat16)
+  b0, b1, bo = torch.randn(e, f, generator=g) * 0.3, torch.randn(e, f, generator=g) * 0.3, torch.randn(e, d, generator=g) * 0.3
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, decoder_block="gpt_oss", mlp_activations_limit=7.0)
+  block = moe.RoutedMoE(cfg, w0.cuda(), w1.cuda(), wo.cuda())
+  out, _, _ = block.sparse_matmul(x.cuda(), logits.cuda(), None, w0.cuda(), w1.cuda(), wo.cuda(), b0.cuda(), b1.cuda(), bo.cuda())
+  w, idx = block.get_topk(logits.cuda())
+  w, idx = w.reshape(t, k).cpu().double(), idx.reshape(t, k).cpu().long()
+  x2 = x.reshape(t, d).double()
+  want = torch.zeros(t, d, dtype=torch.float64)
+  for s_ in range(k):
+    ex = idx[:, s_]
+    h0 = torch.einsum("td,tfd->tf", x2, w0.double()[ex]) + b0.double()[ex]
+    h1 = torch.einsum("td,tfd->tf", x2, w1.double()[ex]) + b1.double()[ex]
+    a = O.apply_ffn_activation(h0.float(), h1.float(), "swigluoai", 7.0).double()
+    want += w[:, s_ : s_ + 1] * (torch.einsum("tf,tdf->td", a, wo.double()[ex]) + bo.double()[ex])
+  assert relerr(out.reshape(t, d), want) <= TOL
