@@ -268,6 +268,20 @@ MOE_API int moe_unpermute_combine(const void* y, const int32_t* perm, const int3
 MOE_API int moe_unpermute_combine_bwd(const void* dout, const void* y, const int32_t* inv_perm, const float* weights,
                                       int T, int k, int d, void* dy, float* dweights, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Gated activation as a stand-alone pass and its gradient, for training, where both projections are kept
+ * for the backward pass (apply_ffn_activation, moe.py:841-870, and the VJP JAX derives for it):
+ *
+ *   out = act(h0, h1)                 (as the fused epilogue of moe_gmm computes it, f32 math, bf16 result)
+ *   dh0, dh1 = d out / d (h0, h1) * dout; clipped inputs (SWIGLUOAI, SILU_CLIP) pass no gradient outside
+ *   their clip range.
+ *
+ * All tensors are bf16 with n elements (n % 8 == 0), 16-byte aligned.
+ */
+MOE_API int moe_glu_act(const void* h0, const void* h1, size_t n, int act, float act_limit, void* out, void* stream);
+MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, size_t n, int act, float act_limit,
+                            void* dh0, void* dh1, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -612,6 +612,52 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const uint4* __restric
 }
 
 // ---------------------------------------------------------------------------------------
+// Gated activation on its own (training keeps both projections for the backward pass) and its gradient.
+// 8 bf16 values per thread; all math in f32.
+// ---------------------------------------------------------------------------------------
+
+template <int ACT>
+__global__ __launch_bounds__(256) void glu_fwd_kernel(const uint4* __restrict__ h0, const uint4* __restrict__ h1, size_t nvec,
+                                                      float limit, uint4* __restrict__ out) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
+    float g[8], u[8], y[8];
+    unpack8(h0[i], g);
+    unpack8(h1[i], u);
+#pragma unroll
+    for (int j = 0; j < 8; j++) y[j] = glu_act<ACT>(g[j], u[j], limit);
+    out[i] = make_uint4(pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]), pack_bf16x2(y[6], y[7]));
+  }
+}
+
+// y = gc * sigmoid(a * gc) * (uc + b) with gc = min(g, L), uc = clamp(u, -L, L) (no clipping for plain SiLU):
+// dy/dg = [g <= L] (uc + b) s (1 + a gc (1 - s)),  dy/du = [-L <= u <= L] gc s,  s = sigmoid(a gc).
+template <int ACT>
+__global__ __launch_bounds__(256) void glu_bwd_kernel(const uint4* __restrict__ h0, const uint4* __restrict__ h1,
+                                                      const uint4* __restrict__ dy, size_t nvec, float limit,
+                                                      uint4* __restrict__ dh0, uint4* __restrict__ dh1) {
+  constexpr bool CLIP = ACT != MOE_ACT_SILU;
+  constexpr float a = ACT == MOE_ACT_SWIGLUOAI ? 1.702f : 1.0f;
+  constexpr float b = ACT == MOE_ACT_SWIGLUOAI ? 1.0f : 0.0f;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
+    float g[8], u[8], d[8], dg[8], du[8];
+    unpack8(h0[i], g);
+    unpack8(h1[i], u);
+    unpack8(dy[i], d);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float gc = CLIP ? fminf(g[j], limit) : g[j];
+      const float uc = CLIP ? fminf(fmaxf(u[j], -limit), limit) : u[j];
+      const float s = 1.0f / (1.0f + expf(-a * gc));
+      const bool g_in = !CLIP || g[j] <= limit, u_in = !CLIP || (u[j] >= -limit && u[j] <= limit);
+      dg[j] = g_in ? d[j] * (uc + b) * s * (1.0f + a * gc * (1.0f - s)) : 0.f;
+      du[j] = u_in ? d[j] * gc * s : 0.f;
+    }
+    dh0[i] = make_uint4(pack_bf16x2(dg[0], dg[1]), pack_bf16x2(dg[2], dg[3]), pack_bf16x2(dg[4], dg[5]), pack_bf16x2(dg[6], dg[7]));
+    dh1[i] = make_uint4(pack_bf16x2(du[0], du[1]), pack_bf16x2(du[2], du[3]), pack_bf16x2(du[4], du[5]), pack_bf16x2(du[6], du[7]));
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // [G, K, N] -> [G, N, K] re-layout through a padded LDS tile.
 // ---------------------------------------------------------------------------------------
 
@@ -798,6 +844,37 @@ int moe_unpermute_combine_bwd(const void* dout, const void* y, const int32_t* in
   combine_bwd_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const uint4*)dout, (const uint4*)y, inv_perm, weights, k, d,
                                                          (uint4*)dy, dweights);
   return check_launch("combine_bwd_kernel");
+}
+
+int moe_glu_act(const void* h0, const void* h1, size_t n, int act, float act_limit, void* out, void* stream) {
+  if (!h0 || !h1 || !out) return fail(MOE_ERR_INVALID_ARG, "glu_act: NULL pointer");
+  if (act < MOE_ACT_SILU || act > MOE_ACT_SILU_CLIP) return fail(MOE_ERR_INVALID_ARG, "glu_act: bad act %d", act);
+  if (n % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "glu_act: element count must be a multiple of 8");
+  if (n == 0) return MOE_OK;
+  const size_t nvec = n / 8;
+  const unsigned blocks = (unsigned)(nvec / 256 + 1 < 8192 ? nvec / 256 + 1 : 8192);
+  hipStream_t s = (hipStream_t)stream;
+  if (act == MOE_ACT_SILU) glu_fwd_kernel<MOE_ACT_SILU><<<blocks, 256, 0, s>>>((const uint4*)h0, (const uint4*)h1, nvec, act_limit, (uint4*)out);
+  else if (act == MOE_ACT_SWIGLUOAI) glu_fwd_kernel<MOE_ACT_SWIGLUOAI><<<blocks, 256, 0, s>>>((const uint4*)h0, (const uint4*)h1, nvec, act_limit, (uint4*)out);
+  else glu_fwd_kernel<MOE_ACT_SILU_CLIP><<<blocks, 256, 0, s>>>((const uint4*)h0, (const uint4*)h1, nvec, act_limit, (uint4*)out);
+  return check_launch("glu_fwd_kernel");
+}
+
+int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, size_t n, int act, float act_limit, void* dh0,
+                    void* dh1, void* stream) {
+  if (!h0 || !h1 || !dout || !dh0 || !dh1) return fail(MOE_ERR_INVALID_ARG, "glu_act_bwd: NULL pointer");
+  if (act < MOE_ACT_SILU || act > MOE_ACT_SILU_CLIP) return fail(MOE_ERR_INVALID_ARG, "glu_act_bwd: bad act %d", act);
+  if (n % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "glu_act_bwd: element count must be a multiple of 8");
+  if (n == 0) return MOE_OK;
+  const size_t nvec = n / 8;
+  const unsigned blocks = (unsigned)(nvec / 256 + 1 < 8192 ? nvec / 256 + 1 : 8192);
+  hipStream_t s = (hipStream_t)stream;
+#define MOE_GLU_BWD(A) glu_bwd_kernel<A><<<blocks, 256, 0, s>>>((const uint4*)h0, (const uint4*)h1, (const uint4*)dout, nvec, act_limit, (uint4*)dh0, (uint4*)dh1)
+  if (act == MOE_ACT_SILU) MOE_GLU_BWD(MOE_ACT_SILU);
+  else if (act == MOE_ACT_SWIGLUOAI) MOE_GLU_BWD(MOE_ACT_SWIGLUOAI);
+  else MOE_GLU_BWD(MOE_ACT_SILU_CLIP);
+#undef MOE_GLU_BWD
+  return check_launch("glu_bwd_kernel");
 }
 
 int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem_bytes, void* rhs_gnk,

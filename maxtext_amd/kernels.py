@@ -185,6 +185,32 @@ def unpermute_combine_bwd(dout, y, weights, *, k, inv_perm, need_dweights=True):
   return dy, dw
 
 
+def glu_act(h0, h1, act="silu", act_limit=7.0):
+  """act(h0, h1) elementwise on bf16 tensors of one shape -> bf16."""
+  _need(h0, "h0", torch.bfloat16)
+  _need(h1, "h1", torch.bfloat16)
+  if h0.shape != h1.shape:
+    raise ValueError("h0 and h1 must have one shape")
+  out = torch.empty_like(h0)
+  st = _lib.load().moe_glu_act(_lib.ptr(h0), _lib.ptr(h1), h0.numel(), _lib.ACT_BY_NAME[act], float(act_limit), _lib.ptr(out),
+                               _lib.current_stream())
+  _lib.check(st, "moe_glu_act")
+  return out
+
+
+def glu_act_bwd(h0, h1, dout, act="silu", act_limit=7.0):
+  """-> (dh0, dh1), the gradient of glu_act."""
+  for name, t in (("h0", h0), ("h1", h1), ("dout", dout)):
+    _need(t, name, torch.bfloat16)
+  if h0.shape != h1.shape or h0.shape != dout.shape:
+    raise ValueError("h0, h1 and dout must have one shape")
+  dh0, dh1 = torch.empty_like(h0), torch.empty_like(h0)
+  st = _lib.load().moe_glu_act_bwd(_lib.ptr(h0), _lib.ptr(h1), _lib.ptr(dout), h0.numel(), _lib.ACT_BY_NAME[act], float(act_limit),
+                                   _lib.ptr(dh0), _lib.ptr(dh1), _lib.current_stream())
+  _lib.check(st, "moe_glu_act_bwd")
+  return dh0, dh1
+
+
 def transpose_rhs(rhs_gkn):
   """[G, K, N] -> [G, N, K] for 1- or 2-byte element types."""
   _need(rhs_gkn, "rhs", None, 3)

@@ -256,17 +256,20 @@ class _GmmFn(torch.autograd.Function):
     return dlhs, drhs, None, None, None, None, None
 
 
-def _glu_torch(h0, h1, kind, limit):
-  """apply_ffn_activation of the expert MLP (moe.py:1288-1306) in differentiable torch ops."""
-  h0, h1 = h0.float(), h1.float()
-  if kind == "silu":
-    return (torch.nn.functional.silu(h0) * h1).to(torch.bfloat16)
-  if kind == "swigluoai":
-    g, u = h0.clamp(max=limit), h1.clamp(-limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(torch.bfloat16)
-  if kind == "silu_clip":
-    return (torch.nn.functional.silu(h0.clamp(max=limit)) * h1.clamp(-limit, limit)).to(torch.bfloat16)
-  raise ValueError(f"unknown activation {kind}")
+class _GluFn(torch.autograd.Function):
+  """apply_ffn_activation of the expert MLP (moe.py:841-870) on kept projections, with its gradient."""
+
+  @staticmethod
+  def forward(ctx, h0, h1, kind, limit):
+    ctx.save_for_backward(h0, h1)
+    ctx.kind, ctx.limit = kind, limit
+    return kernels.glu_act(h0, h1, kind, limit)
+
+  @staticmethod
+  def backward(ctx, dout):
+    h0, h1 = ctx.saved_tensors
+    dh0, dh1 = kernels.glu_act_bwd(h0, h1, dout.contiguous(), ctx.kind, ctx.limit)
+    return dh0, dh1, None, None
 
 
 def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit):
@@ -281,4 +284,6 @@ def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, 
   h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q)
   if fuse_act is None:
     raise ValueError("rhs_up needs fuse_act")
-  return _glu_torch(h0, h1, fuse_act, act_limit)
+  if fuse_act not in ("silu", "swigluoai", "silu_clip"):
+    raise ValueError(f"unknown activation {fuse_act}")
+  return _GluFn.apply(h0.contiguous(), h1.contiguous(), fuse_act, act_limit)

@@ -658,3 +658,31 @@ def test_gmm_bias_argument_errors(K):
     K.gmm_raw(cuda(lhs), wb, cuda(gs), rhs_bias=torch.zeros(1, 32, device="cuda"))
   with pytest.raises(ValueError):
     K.gmm_raw(cuda(lhs), wb, cuda(gs), rhs_up_bias=torch.zeros(1, 64, device="cuda"))
+
+
+# ---------------------------------------------------------------- stand-alone gated activation and its gradient
+
+
+@pytest.mark.parametrize("act", ["silu", "swigluoai", "silu_clip"])
+def test_glu_act_forward_and_gradient(K, act):
+  g = torch.Generator().manual_seed(60)
+  h0 = (torch.randn(300, 264, generator=g) * 4).to(torch.bfloat16)  # |x| reaches past the clip limit of 7
+  h1 = (torch.randn(300, 264, generator=g) * 4).to(torch.bfloat16)
+  dy = torch.randn(300, 264, generator=g).to(torch.bfloat16)
+  got = K.glu_act(cuda(h0), cuda(h1), act, 7.0)
+  want = O.apply_ffn_activation(h0, h1, act, 7.0)
+  assert relerr(got, want) <= 2.0**-7
+  a, b = h0.double().requires_grad_(), h1.double().requires_grad_()
+  if act == "silu":
+    y = torch.nn.functional.silu(a) * b
+  elif act == "swigluoai":
+    gc, uc = a.clamp(max=7.0), b.clamp(-7.0, 7.0)
+    y = gc * torch.sigmoid(1.702 * gc) * (uc + 1.0)
+  else:
+    y = torch.nn.functional.silu(a.clamp(max=7.0)) * b.clamp(-7.0, 7.0)
+  (y * dy.double()).sum().backward()
+  d0, d1 = K.glu_act_bwd(cuda(h0), cuda(h1), cuda(dy), act, 7.0)
+  assert relerr(d0, a.grad) <= 2.0**-7 and relerr(d1, b.grad) <= 2.0**-7
+  if act != "silu":  # no gradient outside the clip range
+    assert torch.all(d0.cpu()[h0.float() > 7.0] == 0) and torch.all(d1.cpu()[h1.float().abs() > 7.0] == 0)
+    assert (h0.float() > 7.0).any() and (h1.float().abs() > 7.0).any()
