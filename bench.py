@@ -36,7 +36,7 @@ def parse():
   ap.add_argument("--gpus", type=int, default=1)
   ap.add_argument("--steps", type=int, default=20)
   ap.add_argument("--warmup", type=int, default=5)
-  ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+  ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c5mx"])
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
   ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -326,7 +326,7 @@ def main():
     del src, dst
 
   if not args.no_cpu_baseline:
-    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048}[wl.name]
+    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048, "c5mx": 2048}[wl.name]
     del out
     result["cpu_baseline"] = cpu_baseline(wl, layer, sample)
   print(json.dumps(result))

@@ -42,7 +42,9 @@ typedef enum {
   MOE_INT8 = 1,
   MOE_FP8_E4M3 = 2, /* OCP float8_e4m3fn (max 448), layers/quantizations.py:237      */
   MOE_INT4 = 3,     /* 2 per byte along K, first value in the low nibble, stored +8  */
-  MOE_F32 = 4
+  MOE_F32 = 4,
+  MOE_MXFP4 = 5    /* OCP MX fp4: e2m1 values, 2 per byte along K (first in the low nibble), one e8m0 scale
+                      byte 2^(s-127) per 32 values (dequantize_mxfp4.py:46-72) */
 } moe_dtype;
 
 typedef enum {
@@ -166,16 +168,17 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  *   rhs_scale  NULL (bf16 rhs) | [G_local, ceil(N/bn), nkb] with
  *              bn = rhs_scale_block_n (1 = per output channel, 128 = DeepSeek 128x128 blocks),
  *              nkb = 1 when rhs_scale_block_k == 0 (per channel over all of K), else
- *              ceil(K / rhs_scale_block_k) (must be 128); f32, or bf16 for INT4
+ *              ceil(K / rhs_scale_block_k) (must be 128); f32, or bf16 for INT4;
+ *              MXFP4: bytes [G_local, N, K/32] (rhs_scale_block_n = 1, rhs_scale_block_k = 32)
  *   rhs_up / rhs_up_scale   second projection (wi_1) with the same layout; when non-NULL
  *              the kernel computes act(lhs@rhs^T) * (lhs@rhs_up^T) in one pass
  *   rhs_bias / rhs_up_bias   [G_local, N] f32 or NULL, see the end of the struct
  *   out        [M, N] bf16
  *
  * Supported operand combinations (others return MOE_ERR_UNSUPPORTED):
- *   BF16 x BF16 | BF16 x INT8 (per-channel) | BF16 x INT4 (bn=1, bk=128)
+ *   BF16 x BF16 | BF16 x INT8 (per-channel) | BF16 x INT4 (bn=1, bk=128) | BF16 x MXFP4 (bn=1, bk=32)
  *   INT8 (per-row) x INT8 (per-channel) | FP8 (1x128) x FP8 (128x128 blocks)
- * Alignment: K % 32 == 0 (INT4), K % 16 == 0 otherwise; N % 8 == 0; pointers 16-byte aligned.
+ * Alignment: K % 32 == 0 (INT4, MXFP4), K % 16 == 0 otherwise; N % 8 == 0; pointers 16-byte aligned.
  */
 typedef struct {
   size_t struct_size; /* sizeof(moe_gmm_args), checked */

@@ -13,7 +13,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libmoe_mi355x.so")
 
 # enums of include/moe_mi355x.h
-MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32 = 0, 1, 2, 3, 4
+MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32, MOE_MXFP4 = 0, 1, 2, 3, 4, 5
 MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK = 0, 1
 MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
 

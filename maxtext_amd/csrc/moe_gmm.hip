@@ -107,14 +107,14 @@ __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
 // ---------------------------------------------------------------------------------------
 
 enum { OP_BF16 = 0, OP_I8 = 1 };                 // MFMA operand type (= LDS element type)
-enum { BSRC_SAME = 0, BSRC_I8 = 1, BSRC_I4 = 2 };  // weight format in HBM
+enum { BSRC_SAME = 0, BSRC_I8 = 1, BSRC_I4 = 2, BSRC_MX4 = 3 };  // weight format in HBM
 
 struct TiledParams {
   const uint8_t* lhs;        // [M, K] elements of the MFMA operand type
   const float* lhs_scale;    // [M] or NULL
   const uint8_t* rhs;        // [G, N, K] (INT4: K/2 bytes per row)
   const uint8_t* rhs_up;     // same, or NULL
-  const void* rhs_scale;     // f32 [G, N] (per channel) | bf16 [G, N, nkg] (INT4)
+  const void* rhs_scale;     // f32 [G, N] (per channel) | bf16 [G, N, nkg] (INT4) | e8m0 bytes [G, N, K/32] (MXFP4)
   const void* rhs_up_scale;
   const float* rhs_bias;     // [G, N] f32 or NULL, added before the activation
   const float* rhs_up_bias;
@@ -226,6 +226,7 @@ struct TiledCfg {
   static constexpr int KSUB = BKB / 32;  // MFMA steps per stage (32 bytes of K per row each)
   static constexpr int A_CPR = BKB / 16;
   static constexpr int A_CH = BM * A_CPR / THREADS;
+  static constexpr bool NIBBLES = BSRC == BSRC_I4 || BSRC == BSRC_MX4;  // two weights per byte
   static constexpr int B_CHE = BSRC == BSRC_SAME ? 16 / ESZ : (BSRC == BSRC_I8 ? 16 : 32);  // elems per 16B
   static constexpr int B_CPR = BK / B_CHE;
   static constexpr int B_CH = BN * B_CPR / THREADS;
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
 
   // ---- global -> register staging -------------------------------------------------------
   const size_t a_row_bytes = (size_t)K * C::ESZ;
-  const size_t b_row_bytes = C::BSRC == BSRC_I4 ? (size_t)K / 2 : (size_t)K * (C::BSRC == BSRC_I8 ? 1 : C::ESZ);
+  const size_t b_row_bytes = C::NIBBLES ? (size_t)K / 2 : (size_t)K * (C::BSRC == BSRC_I8 ? 1 : C::ESZ);
   const uint8_t* a_ptr[C::A_CH];
   int a_k[C::A_CH], a_lds[C::A_CH];
 #pragma unroll
@@ -306,7 +307,7 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
   }
 
   uint4 a_reg[C::A_CH], b_reg[C::B_CH];
-  constexpr int B_GSZ = C::BSRC == BSRC_I4 ? 1 : (C::BSRC == BSRC_I8 ? 2 : 2 * C::ESZ);  // half-bytes per element in HBM
+  constexpr int B_GSZ = C::NIBBLES ? 1 : (C::BSRC == BSRC_I8 ? 2 : 2 * C::ESZ);  // half-bytes per element in HBM
 
   // Every chunk of a full stage is in range: plain loads that stay in flight during the MFMAs.
   auto load_stage = [&](int kt) {
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
     for (int i = 0; i < C::B_CH; i++) {
       const bool ok = k0 + b_k[i] < K;
       const uint4 v = *(const uint4*)(b_ptr[i] + (ok ? (size_t)k0 * B_GSZ / 2 : 0));
-      // INT4 stores value+8: a zero weight is the nibble 8
+      // INT4 stores value+8: a zero weight is the nibble 8 (MXFP4: nibble 0 is +0.0)
       const uint32_t z = C::BSRC == BSRC_I4 ? 0x88888888u : 0u;
       b_reg[i] = ok ? v : make_uint4(z, z, z, z);
     }
@@ -355,6 +356,19 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
         }
         *(uint4*)(s + b_lds[i]) = make_uint4(o[0], o[1], o[2], o[3]);
         *(uint4*)(s + b_lds[i] + 16) = make_uint4(o[4], o[5], o[6], o[7]);
+      } else if (C::BSRC == BSRC_MX4) {  // 32 e2m1 values = one MX block with its e8m0 scale 2^(s - 127)
+        const int kk = kt * C::BK + b_k[i];
+        const uint8_t* sc = (const uint8_t*)(b_up[i] ? p.rhs_up_scale : p.rhs_scale);
+        const uint32_t sbyte = kk < K ? sc[((size_t)tile.group * N + b_n[i]) * (K / 32) + kk / 32] : 127u;
+        const float scale = __uint_as_float(sbyte << 23);
+        const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          *(uint4*)(s + b_lds[i] + 16 * j) = make_uint4(
+              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 0)),
+              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 1)),
+              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 2)),
+              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 3)));
       } else {  // BSRC_I4: 32 values of one 128-wide scale group
         const int kk = kt * C::BK + b_k[i];
         const int nkg = (K + 127) / 128;
@@ -431,7 +445,7 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
   const int n_out0 = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
   EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
-  load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC != BSRC_I4>(esc, p, tile, wm * C::WM, n_out0, lane);
+  load_epilogue_scales<C::TM, NT_OUT, C::GLU, !C::NIBBLES>(esc, p, tile, wm * C::WM, n_out0, lane);
 
   // The steady-state loop only ever issues full-stage loads; the stage that may hold the K tail is
   // loaded in a peeled iteration so its masking code never merges into the loop body.
@@ -914,22 +928,32 @@ struct WqSkinnyParams {
 };
 
 // Raw weight bytes of one lane for one 128-wide k block: 32 values = 16 bytes (int4) or 32 bytes (int8).
-template <bool INT4>
+enum { WQ_I8 = 0, WQ_I4 = 1, WQ_MX4 = 2 };  // weight formats of the streaming kernel
+
+template <int FMT>
 struct WqRaw {
   uint4 q0, q1;
 };
 
-template <bool INT4>
-__device__ __forceinline__ WqRaw<INT4> wq_load(const uint8_t* p) {
-  WqRaw<INT4> r;
+template <int FMT>
+__device__ __forceinline__ WqRaw<FMT> wq_load(const uint8_t* p) {
+  WqRaw<FMT> r;
   r.q0 = *(const uint4*)p;
-  r.q1 = INT4 ? make_uint4(0, 0, 0, 0) : *(const uint4*)(p + 16);
+  r.q1 = FMT != WQ_I8 ? make_uint4(0, 0, 0, 0) : *(const uint4*)(p + 16);
   return r;
 }
 
-template <bool INT4>
-__device__ __forceinline__ void widen32(const WqRaw<INT4>& raw, float scale, v8bf (&w)[4]) {
-  if (INT4) {
+template <int FMT>
+__device__ __forceinline__ void widen32(const WqRaw<FMT>& raw, float scale, v8bf (&w)[4]) {
+  if (FMT == WQ_MX4) {  // e2m1 pairs -> bf16 pairs times the block scale, one instruction per byte
+    const uint32_t x[4] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w};
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+      w[s] = __builtin_bit_cast(v8bf, make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 0)),
+                                                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 1)),
+                                                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 2)),
+                                                 __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 3))));
+  } else if (FMT == WQ_I4) {
     const uint32_t x[4] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w};
 #pragma unroll
     for (int s = 0; s < 4; s++) {
@@ -957,46 +981,59 @@ __device__ __forceinline__ void widen32(const WqRaw<INT4>& raw, float scale, v8b
   }
 }
 
-// A block owns 16*NT output channels of one m-tile; its 4 waves split K into 4 contiguous ranges of
-// 128-wide blocks and add their partial sums through LDS at the end (decode has few tiles, and a single
-// wave walking all of K is bound by the latency of its dependent loads, not by bandwidth).  Within its
-// range a wave issues the loads of U blocks before it converts and multiplies the first one.
-template <bool INT4, int MT, int NT, bool GLU, int U>
+// A block of 4 waves owns (4 / KSPLIT) * 16*NT output channels of one m-tile; KSPLIT waves share a channel
+// group, split K into contiguous ranges of 128-wide blocks and add their partial sums through LDS at the
+// end (with few tiles, a wave walking all of K alone leaves the memory system idle: KSPLIT = 4 for a handful
+// of tokens, 1 once there are enough blocks).  Within its range a wave works in rounds of U blocks whose loads
+// are all issued before the first block is converted and multiplied; other resident waves cover the rest of the
+// latency (holding two rounds in registers halves the occupancy and measures slower).
+template <int FMT, int MT, int NT, bool GLU, int U, int KSPLIT>
 __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams p) {
+  constexpr bool INT4 = FMT == WQ_I4, MX4 = FMT == WQ_MX4, NIB = FMT != WQ_I8;
   constexpr int NACC = NT * MT * 4 * (GLU ? 2 : 1);
-  __shared__ float red[3 * NACC * kWave];
+  constexpr int NSUB = 4 / KSPLIT;  // channel groups per block
+  __shared__ float red[KSPLIT > 1 ? NSUB * (KSPLIT - 1) * NACC * kWave : 1];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int ksub = wave % KSPLIT, nsub = wave / KSPLIT;
   const int j = lane % 16, kq = lane / 16;
   const int m_idx = blockIdx.x / p.n_blocks;
   if (m_idx >= p.header[0]) return;
   const TileInfo tile = p.tiles[m_idx];
   const int N = p.N, K = p.K;
   constexpr int WN = 16 * NT;
-  const int n_w = (blockIdx.x % p.n_blocks) * WN;
+  const int n_b = (blockIdx.x % p.n_blocks) * (NSUB * WN);
+  const int n_w = n_b + nsub * WN;
 
   if (tile.group < 0) {
-    for (int i = threadIdx.x; i < tile.nrows * (WN / 4); i += 256) {
-      int r = i / (WN / 4), c = n_w + (i % (WN / 4)) * 4;
+    for (int i = threadIdx.x; i < tile.nrows * (NSUB * WN / 4); i += 256) {
+      int r = i / (NSUB * WN / 4), c = n_b + (i % (NSUB * WN / 4)) * 4;
       if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
     }
     return;
   }
+  // a channel group past N has nothing to do, but its waves still meet the others at the barrier below
+  const bool idle = n_w >= N;
 
   const int nkb = (K + 127) / 128;  // the last block may be partial (K % 32 == 0)
-  const size_t wrow_bytes = INT4 ? (size_t)K / 2 : (size_t)K;
+  const size_t wrow_bytes = NIB ? (size_t)K / 2 : (size_t)K;
   const uint8_t* wp[NT];
   const uint8_t* up[NT];
   const uint16_t* wsp[NT];
   const uint16_t* usp[NT];
+  const uint8_t* wmx[NT];
+  const uint8_t* umx[NT];
 #pragma unroll
   for (int t = 0; t < NT; t++) {
     const int nw = min(n_w + t * 16 + j, N - 1);
     const size_t row = (size_t)tile.group * N + nw;
-    wp[t] = p.rhs + row * wrow_bytes + kq * (INT4 ? 16 : 32);
-    up[t] = GLU ? p.rhs_up + row * wrow_bytes + kq * (INT4 ? 16 : 32) : nullptr;
+    wp[t] = p.rhs + row * wrow_bytes + kq * (NIB ? 16 : 32);
+    up[t] = GLU ? p.rhs_up + row * wrow_bytes + kq * (NIB ? 16 : 32) : nullptr;
     wsp[t] = INT4 ? (const uint16_t*)p.rhs_scale + row * nkb : nullptr;
     usp[t] = INT4 && GLU ? (const uint16_t*)p.rhs_up_scale + row * nkb : nullptr;
+    // MXFP4: one e8m0 byte per 32 values = per lane and k block
+    wmx[t] = MX4 ? (const uint8_t*)p.rhs_scale + row * (size_t)(K / 32) + kq : nullptr;
+    umx[t] = MX4 && GLU ? (const uint8_t*)p.rhs_up_scale + row * (size_t)(K / 32) + kq : nullptr;
   }
   const uint8_t* ap[MT];
 #pragma unroll
@@ -1013,36 +1050,59 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
       acc_u[t][mt] = v4f{0.f, 0.f, 0.f, 0.f};
     }
 
-  auto step = [&](int kb0, auto ucount) {
-    constexpr int UC = decltype(ucount)::value;
-    uint4 araw[UC][MT][4];
-    WqRaw<INT4> wraw[UC][NT], uraw[UC][NT];
-    uint16_t wsc[UC][NT], usc[UC][NT];
-    bool live[UC];
+  // One round = U k-blocks held as raw bytes.
+  struct Round {
+    uint4 araw[U][MT][4];
+    WqRaw<FMT> wraw[U][NT], uraw[U][NT];
+    uint16_t wsc[U][NT], usc[U][NT];
+    bool live[U];
+  };
+  const int chunk = (nkb + KSPLIT - 1) / KSPLIT;
+  const int kb_begin = ksub * chunk;
+  const int kb_end = idle ? kb_begin : min(nkb, kb_begin + chunk);
+
+  // Blocks past the end of the range are loaded from the range's last block and flagged dead (their activations
+  // are zeroed before use), so every round has the same instruction stream.
+  auto load_round = [&](Round& r, int kb0) {
 #pragma unroll
-    for (int u = 0; u < UC; u++) {
-      const int kb = kb0 + u;
+    for (int u = 0; u < U; u++) {
+      const bool in_range = kb0 + u < kb_end;
+      const int kb = in_range ? kb0 + u : max(kb_end - 1, 0);
       // this lane's 32 k values exist unless the block is the partial tail
-      live[u] = kb * 128 + kq * 32 < K;
-      const size_t woff = live[u] ? (size_t)kb * (INT4 ? 64 : 128) : 0;
+      r.live[u] = in_range && kb * 128 + kq * 32 < K;
+      const bool addr_ok = kb * 128 + kq * 32 < K;
+      const size_t woff = addr_ok ? (size_t)kb * (NIB ? 64 : 128) : 0;
 #pragma unroll
       for (int t = 0; t < NT; t++) {
-        wraw[u][t] = wq_load<INT4>(wp[t] + woff);
-        if (GLU) uraw[u][t] = wq_load<INT4>(up[t] + woff);
+        r.wraw[u][t] = wq_load<FMT>(wp[t] + woff);
+        if (GLU) r.uraw[u][t] = wq_load<FMT>(up[t] + woff);
         if (INT4) {
-          wsc[u][t] = wsp[t][kb];
-          if (GLU) usc[u][t] = usp[t][kb];
+          r.wsc[u][t] = wsp[t][kb];
+          if (GLU) r.usc[u][t] = usp[t][kb];
+        }
+        if (MX4) {
+          r.wsc[u][t] = addr_ok ? wmx[t][kb * 4] : (uint16_t)127;
+          if (GLU) r.usc[u][t] = addr_ok ? umx[t][kb * 4] : (uint16_t)127;
         }
       }
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
-        const uint8_t* a = ap[mt] + (live[u] ? (size_t)kb * 256 : 0);
+        const uint8_t* a = ap[mt] + (addr_ok ? (size_t)kb * 256 : 0);
 #pragma unroll
-        for (int s = 0; s < 4; s++) araw[u][mt][s] = *(const uint4*)(a + s * 16);
+        for (int s = 0; s < 4; s++) r.araw[u][mt][s] = *(const uint4*)(a + s * 16);
       }
     }
+  };
+
+  auto compute_round = [&](const Round& r) {
+    const auto& araw = r.araw;
+    const auto& wraw = r.wraw;
+    const auto& uraw = r.uraw;
+    const auto& wsc = r.wsc;
+    const auto& usc = r.usc;
+    const auto& live = r.live;
 #pragma unroll
-    for (int u = 0; u < UC; u++) {
+    for (int u = 0; u < U; u++) {
       if constexpr (INT4) {
         // A nibble n (stored value + 8) becomes the bf16 number 128 + n by OR-ing it into the mantissa of
         // 128.0 (0x4300): one AND-OR per pair of values, pairs (k, k+4) of each 8-nibble word.  The MFMA then
@@ -1110,8 +1170,8 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 #pragma unroll
         for (int t = 0; t < NT; t++) {
           v8bf wf[4], uf[4];
-          widen32<INT4>(wraw[u][t], 1.0f, wf);
-          if (GLU) widen32<INT4>(uraw[u][t], 1.0f, uf);
+          widen32<FMT>(wraw[u][t], MX4 ? __uint_as_float((uint32_t)wsc[u][t] << 23) : 1.0f, wf);
+          if (GLU) widen32<FMT>(uraw[u][t], MX4 ? __uint_as_float((uint32_t)usc[u][t] << 23) : 1.0f, uf);
 #pragma unroll
           for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -1124,42 +1184,47 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
     }
   };
 
-  const int chunk = (nkb + 3) / 4;
-  int kb = wave * chunk;
-  const int kb_end = min(nkb, kb + chunk);
-  for (; kb + U <= kb_end; kb += U) step(kb, std::integral_constant<int, U>{});
-  for (; kb < kb_end; kb++) step(kb, std::integral_constant<int, 1>{});
+  {
+    Round r;
+    for (int kb = kb_begin; kb < kb_end; kb += U) {
+      load_round(r, kb);
+      compute_round(r);
+    }
+  }
 
-  // partial sums of waves 1..3 -> LDS -> wave 0
-  if (wave > 0) {
-    float* r = red + (size_t)(wave - 1) * NACC * kWave + lane;
-    int i = 0;
+  if constexpr (KSPLIT > 1) {
+    // partial sums of the group's waves 1..KSPLIT-1 -> LDS -> its wave 0
+    if (ksub > 0) {
+      float* r = red + (size_t)(nsub * (KSPLIT - 1) + ksub - 1) * NACC * kWave + lane;
+      int i = 0;
 #pragma unroll
-    for (int t = 0; t < NT; t++)
+      for (int t = 0; t < NT; t++)
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++)
+        for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-          r[(i++) * kWave] = acc_g[t][mt][c];
-          if (GLU) r[(i++) * kWave] = acc_u[t][mt][c];
-        }
+          for (int c = 0; c < 4; c++) {
+            r[(i++) * kWave] = acc_g[t][mt][c];
+            if (GLU) r[(i++) * kWave] = acc_u[t][mt][c];
+          }
+    }
+    __syncthreads();
+    if (ksub > 0) return;
+#pragma unroll
+    for (int w = 0; w < KSPLIT - 1; w++) {
+      const float* r = red + (size_t)(nsub * (KSPLIT - 1) + w) * NACC * kWave + lane;
+      int i = 0;
+#pragma unroll
+      for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            acc_g[t][mt][c] += r[(i++) * kWave];
+            if (GLU) acc_u[t][mt][c] += r[(i++) * kWave];
+          }
+    }
   }
-  __syncthreads();
-  if (wave > 0) return;
-#pragma unroll
-  for (int w = 0; w < 3; w++) {
-    const float* r = red + (size_t)w * NACC * kWave + lane;
-    int i = 0;
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-#pragma unroll
-      for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          acc_g[t][mt][c] += r[(i++) * kWave];
-          if (GLU) acc_u[t][mt][c] += r[(i++) * kWave];
-        }
-  }
+  if (idle) return;
 
   dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
@@ -1171,7 +1236,7 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
       float bg[4], bu[4];
       load_bias4(p.rhs_bias, tile.group, N, n, bg);
       load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, N, n, bu);
-      if (!INT4) {
+      if (FMT == WQ_I8) {
         const float4 a = *(const float4*)((const float*)p.rhs_scale + (size_t)tile.group * N + n);
         sg[0] = a.x; sg[1] = a.y; sg[2] = a.z; sg[3] = a.w;
         if (GLU) {
@@ -1325,18 +1390,25 @@ static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int ma
   }
 }
 
-template <bool INT4, int MT>
-static int launch_wq_skinny(WqSkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
-  constexpr int NT = 2;
-  constexpr int U = MT == 1 ? 3 : 2;
-  p.n_blocks = cdiv(p.N, 16 * NT);
+template <int FMT, int MT, int KSPLIT, int NT, int U>
+static int launch_wq_skinny_k(WqSkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
+  p.n_blocks = cdiv(p.N, (4 / KSPLIT) * 16 * NT);
   const long long blocks = (long long)max_tiles * p.n_blocks;
   if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
   if (glu)
-    gmm_wq_skinny_kernel<INT4, MT, NT, true, U><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<FMT, MT, NT, true, U, KSPLIT><<<(unsigned)blocks, 256, 0, s>>>(p);
   else
-    gmm_wq_skinny_kernel<INT4, MT, NT, false, U><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<FMT, MT, NT, false, U, KSPLIT><<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_launch("gmm_wq_skinny_kernel");
+}
+
+// K is split over the 4 waves of a block; `tune` == 1 (reserved[1] of the arguments) gives every wave all of K
+// instead (measured slower up to 32 rows per expert; kept as a tuning aid).
+template <int FMT, int MT>
+static int launch_wq_skinny(const WqSkinnyParams& p, bool glu, int max_tiles, int tune, hipStream_t s) {
+  constexpr int U = MT == 1 ? 3 : 2;  // k-blocks per round
+  if (tune == 1) return launch_wq_skinny_k<FMT, MT, 1, 2, U>(p, glu, max_tiles, s);
+  return launch_wq_skinny_k<FMT, MT, 4, 2, U>(p, glu, max_tiles, s);
 }
 
 }  // namespace moe
@@ -1409,7 +1481,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   p.M = a->M; p.K = a->K; p.N = a->N; p.max_m_tiles = 0; p.tiles_n = 0;
   p.act = a->act; p.act_limit = a->act_limit; p.dbg = a->reserved[1];
 
-  enum { V_NONE, V_BF16, V_W8, V_W4, V_I8 } variant = V_NONE;
+  enum { V_NONE, V_BF16, V_W8, V_W4, V_I8, V_MX4 } variant = V_NONE;
   if (L == MOE_BF16 && R == MOE_BF16) {
     if (a->K % 8) return fail(MOE_ERR_UNSUPPORTED, "gmm: bf16 needs K %% 8 == 0");
     p.rhs_scale = p.rhs_up_scale = nullptr;
@@ -1424,6 +1496,11 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
       return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need bf16 group-128 scales [G, N, ceil(K/128)]");
     if (a->K % 32) return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need K %% 32 == 0");
     variant = V_W4;
+  } else if (L == MOE_BF16 && R == MOE_MXFP4) {
+    if (!a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || a->rhs_scale_block_k != 32)
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: mxfp4 weights need e8m0 block-32 scales [G, N, K/32]");
+    if (a->K % 32) return fail(MOE_ERR_UNSUPPORTED, "gmm: mxfp4 weights need K %% 32 == 0");
+    variant = V_MX4;
   } else if (L == MOE_INT8 && R == MOE_INT8) {
     if (!a->lhs_scale || a->lhs_scale_block_k != 0 || !a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || a->rhs_scale_block_k != 0)
       return fail(MOE_ERR_UNSUPPORTED, "gmm: int8 x int8 needs per-row lhs scales [M] and per-channel rhs scales [G, N]");
@@ -1436,7 +1513,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
 
   const int M = a->M, G = a->num_groups_total;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
-  if ((variant == V_W8 || variant == V_W4) && (long long)M <= 32LL * G && a->reserved[0] != 1) {
+  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->reserved[0] != 1) {
     const bool one = (long long)M <= 16LL * G;
     bm = one ? 16 : 32;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
@@ -1447,8 +1524,10 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     q.header = header; q.tiles = tiles; q.out = (uint16_t*)a->out;
     q.M = M; q.K = a->K; q.N = a->N; q.n_blocks = 0; q.act = a->act; q.act_limit = a->act_limit;
     const int mx = max_tiles_for(M, G, bm);
-    if (variant == V_W4) return one ? launch_wq_skinny<true, 1>(q, glu, mx, s) : launch_wq_skinny<true, 2>(q, glu, mx, s);
-    return one ? launch_wq_skinny<false, 1>(q, glu, mx, s) : launch_wq_skinny<false, 2>(q, glu, mx, s);
+    const int kso = a->reserved[1];
+    if (variant == V_W4) return one ? launch_wq_skinny<WQ_I4, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_I4, 2>(q, glu, mx, kso, s);
+    if (variant == V_MX4) return one ? launch_wq_skinny<WQ_MX4, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_MX4, 2>(q, glu, mx, kso, s);
+    return one ? launch_wq_skinny<WQ_I8, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_I8, 2>(q, glu, mx, kso, s);
   }
   // dry run to learn the m-tile, then build the tile list and launch
   const int forced = a->reserved[0];
@@ -1464,6 +1543,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     case V_BF16: return launch_tiled_glu<OP_BF16, BSRC_SAME>(p, glu, M, G, &bm, false, s);
     case V_W8: return launch_tiled_glu<OP_BF16, BSRC_I8>(p, glu, M, G, &bm, false, s);
     case V_W4: return launch_tiled_glu<OP_BF16, BSRC_I4>(p, glu, M, G, &bm, false, s);
+    case V_MX4: return launch_tiled_glu<OP_BF16, BSRC_MX4>(p, glu, M, G, &bm, false, s);
     case V_I8: return launch_tiled_glu<OP_I8, BSRC_SAME>(p, glu, M, G, &bm, false, s);
     default: break;
   }

@@ -11,7 +11,7 @@ import ctypes
 import torch
 
 from maxtext_amd import _lib
-from maxtext_amd._lib import (MOE_BF16, MOE_FP8_E4M3, MOE_INT4, MOE_INT8, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_SOFTMAX_TOPK)
+from maxtext_amd._lib import (MOE_BF16, MOE_FP8_E4M3, MOE_INT4, MOE_INT8, MOE_MXFP4, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_SOFTMAX_TOPK)
 
 _DTYPE_CODE = {torch.bfloat16: MOE_BF16, torch.int8: MOE_INT8, torch.float8_e4m3fn: MOE_FP8_E4M3}
 
@@ -225,7 +225,7 @@ def transpose_rhs(rhs_gkn):
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
             group_offset=0, out=None, tile_variant=0, rhs_bias=None, rhs_up_bias=None):
-  """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4: uint8 [G,N,K/2])."""
+  """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2])."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
   _need(group_sizes, "group_sizes", torch.int32, 1)
@@ -237,9 +237,9 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
     if rhs.dtype not in _DTYPE_CODE:
       raise TypeError(f"rhs dtype {rhs.dtype} needs an explicit rhs_dtype")
     rhs_dtype = _DTYPE_CODE[rhs.dtype]
-  if rhs_dtype == MOE_INT4:
+  if rhs_dtype in (MOE_INT4, MOE_MXFP4):
     if rhs.dtype != torch.uint8 or kr * 2 != kdim:
-      raise ValueError("INT4 rhs must be uint8 [G, N, K/2]")
+      raise ValueError("INT4 / MXFP4 rhs must be uint8 [G, N, K/2]")
   elif kr != kdim:
     raise ValueError(f"rhs K {kr} != lhs K {kdim}")
   for name, t in (("rhs_up", rhs_up),):
@@ -252,7 +252,7 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   for name, t in (("rhs_scale", rhs_scale), ("rhs_up_scale", rhs_up_scale)):
     if t is not None:
       _need(t, name)
-      want = torch.bfloat16 if rhs_dtype == MOE_INT4 else torch.float32
+      want = torch.bfloat16 if rhs_dtype == MOE_INT4 else (torch.uint8 if rhs_dtype == MOE_MXFP4 else torch.float32)
       if t.dtype != want or t.numel() != g_local * nnb * nkb_r:
         raise ValueError(f"{name} must be {want} with {g_local}x{nnb}x{nkb_r} elements, got {t.dtype} {tuple(t.shape)}")
   for name, t in (("rhs_bias", rhs_bias), ("rhs_up_bias", rhs_up_bias)):

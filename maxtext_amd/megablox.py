@@ -17,7 +17,7 @@ from __future__ import annotations
 import torch
 
 from maxtext_amd import kernels, quantizations
-from maxtext_amd._lib import MOE_INT4
+from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
 from maxtext_amd.quantizations import QArray
 
 # When set to a list, the backward pass of gmm appends (stage, start_event, end_event) recorded on the launch stream.
@@ -164,6 +164,8 @@ def gmm(
       kw.update(rhs_scale_block_n=128, rhs_scale_block_k=128)
     elif rhs_n.qtype == "int4":
       kw.update(rhs_scale_block_n=1, rhs_scale_block_k=128, rhs_dtype=MOE_INT4)
+    elif rhs_n.qtype == "mxfp4":
+      kw.update(rhs_scale_block_n=1, rhs_scale_block_k=32, rhs_dtype=MOE_MXFP4)
     else:
       raise ValueError(f"unknown qtype {rhs_n.qtype}")
     rhs_t = rhs_n.qvalue

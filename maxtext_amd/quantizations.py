@@ -29,7 +29,8 @@ class QArray:
   """Quantised tensor: values plus scales (the role qwix.pallas.QArray plays in ops.py:232-267).
 
   For expert weights `qvalue` is [G, N, K] (K contiguous; INT4: uint8 [G, N, K/2]) and `scale`
-  has the layout described in the module docstring; `qtype` is "int8" | "fp8" | "int4".
+  has the layout described in the module docstring; `qtype` is "int8" | "fp8" | "int4" | "mxfp4"
+  (mxfp4: uint8 [G, N, K/2] e2m1 pairs and uint8 [G, N, K/32] e8m0 block scales).
   For activations `qvalue` is [M, K] and `scale` is [M] (int8) or [M, ceil(K/128)] (fp8).
   """
 
@@ -100,6 +101,27 @@ def quantize_weight_int4(w_gnk: torch.Tensor, group: int = 128) -> QArray:
   u = (q + 8).to(torch.uint8)
   packed = (u[..., 0::2] | (u[..., 1::2] << 4)).contiguous()
   return QArray(packed, scale.squeeze(-1).contiguous(), "int4")
+
+
+def quantize_weight_mxfp4(w_gnk: torch.Tensor) -> QArray:
+  """w [G, N, K] -> OCP MX fp4: e2m1 values (two per byte along K, first in the low nibble) with one e8m0 scale per
+  32 values, the storage format of GPT-OSS checkpoints (dequantize_mxfp4.py:46-72).  Shared exponent =
+  floor(log2(absmax of the block)) - 2, values rounded to the nearest e2m1 point, saturating at +-6."""
+  g, n, k = w_gnk.shape
+  if k % 32:
+    raise ValueError("K must be a multiple of 32")
+  x = w_gnk.float().reshape(g, n, k // 32, 32)
+  amax = x.abs().amax(-1, keepdim=True)
+  exp = torch.where(amax > 0, torch.floor(torch.log2(amax.clamp_min(1e-38))) - 2.0, torch.zeros_like(amax)).clamp(-127, 127)
+  y = (x / torch.exp2(exp)).clamp(-6.0, 6.0)
+  a = y.abs()
+  # e2m1 magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6 -> codes 0..7; thresholds are the midpoints (ties to the even code)
+  code = ((a > 0.25).to(torch.uint8) + (a >= 0.75).to(torch.uint8) + (a > 1.25).to(torch.uint8) + (a >= 1.75).to(torch.uint8)
+          + (a > 2.5).to(torch.uint8) + (a >= 3.5).to(torch.uint8) + (a > 5.0).to(torch.uint8))
+  code = code | ((y < 0).to(torch.uint8) << 3)
+  packed = (code[..., 0::2] | (code[..., 1::2] << 4)).reshape(g, n, k // 2).contiguous()
+  scale = (exp.squeeze(-1) + 127.0).to(torch.uint8).contiguous()
+  return QArray(packed, scale, "mxfp4")
 
 
 def split_gate_kernel(kernel_de: torch.Tensor, terms: int = 3) -> torch.Tensor:

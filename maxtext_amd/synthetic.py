@@ -31,7 +31,7 @@ class Workload:
   name: str
   tokens: int
   cfg: MoEConfig
-  weight_quant: str  # "int8" | "fp8" | "int4"
+  weight_quant: str  # "int8" | "fp8" | "int4" | "mxfp4"
   seed: int
   zipf_s: float = 0.0
   router_from_weights: bool = False
@@ -55,6 +55,9 @@ def workload(name: str, tokens: Optional[int] = None) -> Workload:
   if name == "c5":
     cfg = MoEConfig(32, 4, 2880, 2880, model_name="gpt-oss-20b", decoder_block="mixtral")
     return Workload("c5", tokens or 4096, cfg, "int4", 1239)
+  if name == "c5mx":  # the C5 shape with the weights in the format GPT-OSS checkpoints are stored in
+    cfg = MoEConfig(32, 4, 2880, 2880, model_name="gpt-oss-20b", decoder_block="mixtral")
+    return Workload("c5mx", tokens or 4096, cfg, "mxfp4", 1240)
   raise ValueError(f"unknown workload {name}")
 
 
@@ -65,6 +68,8 @@ def _quantize(w_gnk: torch.Tensor, kind: str) -> Q.QArray:
     return Q.quantize_weight_fp8_blocks(w_gnk)
   if kind == "int4":
     return Q.quantize_weight_int4(w_gnk)
+  if kind == "mxfp4":
+    return Q.quantize_weight_mxfp4(w_gnk)
   raise ValueError(kind)
 
 
@@ -119,5 +124,5 @@ def layer_flops(wl: Workload) -> float:
 
 
 def weight_bytes_per_expert(wl: Workload) -> float:
-  per = {"int8": 1.0, "fp8": 1.0, "int4": 0.5}[wl.weight_quant]
+  per = {"int8": 1.0, "fp8": 1.0, "int4": 0.5, "mxfp4": 0.5}[wl.weight_quant]
   return 3.0 * wl.cfg.emb_dim * wl.cfg.moe_mlp_dim * per

@@ -25,6 +25,10 @@ def oracle_rhs(qvalue: torch.Tensor, scale: torch.Tensor, qtype: str, n: int):
     return qv.transpose(1, 2), s, 128
   if qtype == "int4":
     return O.unpack_int4(qv).transpose(1, 2), sc.float().permute(0, 2, 1)[:, :, None, :], 128
+  if qtype == "mxfp4":
+    g, nn, kb = qv.shape
+    deq = O.dequantize_mxfp4(qv.reshape(g, nn, kb // 16, 16), sc).to(torch.bfloat16)  # exact: e2m1 * 2^e fits bf16
+    return deq.transpose(1, 2), None, None
   raise ValueError(qtype)
 
 

@@ -30,6 +30,10 @@ How each function is pinned (see tests/test_oracle_*.py):
       quantizations_test.py:723-726 (224 -> 0.5 for e4m3fn).
   unpack_int4 / dequantize_int4 / dequantize_fp8_blocks
       tests/unit/dequantize_pack_quantized_int4_test.py:61-127 cases.
+  dequantize_mxfp4
+      the 16 e2m1 code points of the OCP MX specification (0, 0.5, 1, 1.5, 2, 3, 4, 6 and negatives), the
+      nibble order and 2^(s-127) scaling on hand-made blocks; quantize_mxfp4 (a test-data generator only) by
+      dequantize(quantize(x)) == x on representable inputs.
 
 PARITY UNPINNED (third-party arithmetic whose source is not in the reference
 tree, and which no reference test pins):
@@ -485,3 +489,45 @@ def moe_layer_loop(x: torch.Tensor, weights: np.ndarray, idx: np.ndarray, num_ex
     y = mlp_fn(e, x[torch.from_numpy(tok)]).to(torch.float32)
     out.index_add_(0, torch.from_numpy(tok), y * w[torch.from_numpy(tok), torch.from_numpy(slot)][:, None])
   return out.to(x.dtype)
+
+
+# --------------------------------------------------------------------------
+# MXFP4 (OCP microscaling fp4, the GPT-OSS checkpoint format)
+# --------------------------------------------------------------------------
+
+# e2m1 code -> value: bit 3 sign, bits 2..1 exponent (bias 1), bit 0 mantissa; exponent 0 is subnormal
+# (src/maxtext/checkpoint_conversion/standalone_scripts/dequantize_mxfp4.py:46-59).
+E2M1_VALUES = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0], np.float32)
+
+
+def dequantize_mxfp4(blocks: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+  """dequantize_mxfp4.py:62-72: blocks uint8 [..., G, 16] hold 32 e2m1 values each, first value in the low nibble;
+  scales uint8 [..., G] are e8m0 exponents, value = e2m1 * 2^(scale - 127).  -> float32 [..., G * 32]."""
+  b = blocks.to(torch.int64)
+  table = torch.from_numpy(E2M1_VALUES)
+  vals = torch.stack([table[b & 0xF], table[b >> 4]], -1)  # [..., G, 16, 2]
+  factor = torch.exp2(scales.to(torch.float32) - 127.0)[..., None, None]
+  out = vals * factor
+  return out.reshape(out.shape[:-3] + (-1,))
+
+
+def quantize_mxfp4(w: torch.Tensor):
+  """Test-data generator (no counterpart in the reference): [..., K] f32 -> (blocks uint8 [..., K/32, 16], scales
+  uint8 [..., K/32]) by the OCP MX rule: shared exponent = floor(log2(absmax of the block)) - 2 (2 = exponent of
+  the largest e2m1 normal, 6 = 1.5 * 2^2), elements rounded to the nearest e2m1 value (ties to the even code),
+  saturating at +-6."""
+  k = w.shape[-1]
+  assert k % 32 == 0
+  x = w.float().reshape(w.shape[:-1] + (k // 32, 32))
+  amax = x.abs().amax(-1, keepdim=True)
+  exp = torch.where(amax > 0, torch.floor(torch.log2(amax.clamp_min(1e-38))) - 2.0, torch.zeros_like(amax)).clamp(-127, 127)
+  y = (x / torch.exp2(exp)).clamp(-6.0, 6.0)
+  grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+  d = (y.abs()[..., None] - grid).abs()
+  # nearest grid point; on a tie prefer the even code (codes 0, 2, 4, 6 have mantissa bit 0)
+  tie_break = torch.tensor([0.0, 1e-6, 0.0, 1e-6, 0.0, 1e-6, 0.0, 1e-6])
+  code = torch.argmin(d + tie_break, dim=-1)
+  code = code + 8 * (y < 0).long()
+  blocks = (code[..., 0::2] | (code[..., 1::2] << 4)).to(torch.uint8)
+  scales = (exp.squeeze(-1) + 127.0).to(torch.uint8)
+  return blocks, scales

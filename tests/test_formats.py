@@ -1,0 +1,89 @@
+"""Checkpoint-format adapters (host logic, CPU): the bytes they hand to the kernels must dequantise, by the oracle's
+restatement of the reference's converters, to what the reference's converters produce from the checkpoint tensors."""
+
+import numpy as np
+import pytest
+import torch
+
+from maxtext_amd import formats
+from oracle import moe_oracle as O
+
+
+def test_deepseek_fp8_is_zero_copy_and_matches_block_dequant():
+  g = torch.Generator().manual_seed(0)
+  n, k, e = 256, 384, 3
+  ws = [(torch.randn(n, k, generator=g)).to(torch.float8_e4m3fn) for _ in range(e)]
+  ss = [torch.rand(n // 128, k // 128, generator=g) * 0.01 + 1e-3 for _ in range(e)]
+  qa = formats.deepseek_fp8_experts(ws, ss)
+  assert qa.qtype == "fp8" and qa.qvalue.shape == (e, n, k) and qa.scale.shape == (e, 2, 3)
+  for i in range(e):
+    # deepseek_dequantize.py:62-68: q reshaped into 128x128 blocks times the block's scale
+    want = (ws[i].float().reshape(2, 128, 3, 128) * ss[i].reshape(2, 1, 3, 1)).reshape(n, k)
+    got = O.dequantize_fp8_blocks(qa.qvalue[i], qa.scale[i], 128)
+    assert torch.equal(got, want.to(torch.bfloat16))
+  state = {}
+  for i in range(e):
+    for proj in ("gate_proj", "up_proj", "down_proj"):
+      state[f"model.layers.4.mlp.experts.{i}.{proj}.weight"] = ws[i]
+      state[f"model.layers.4.mlp.experts.{i}.{proj}.weight_scale_inv"] = ss[i]
+  w0, w1, wo = formats.deepseek_fp8_layer(state, 4, e)
+  assert torch.equal(w0.qvalue.view(torch.uint8), qa.qvalue.view(torch.uint8)) and torch.equal(wo.scale, qa.scale)
+  # e8m0 scales
+  qa8 = formats.deepseek_fp8_experts(ws[:1], [torch.tensor([[127, 126, 128], [120, 127, 130]], dtype=torch.uint8)])
+  assert qa8.scale[0].tolist() == [[1.0, 0.5, 2.0], [2.0**-7, 1.0, 8.0]]
+  with pytest.raises(ValueError):
+    formats.deepseek_fp8_experts(ws[:1], [torch.ones(3, 3)])
+
+
+def test_compressed_int4_bytes_are_the_kernel_packing():
+  """The reference's own vectors (tests/unit/dequantize_pack_quantized_int4_test.py:61-100): nibble k of the int32
+  is weight k, value = nibble - 8; viewed as bytes that is low-nibble-first pairs."""
+  n, k = 4, 256
+  rng = np.random.default_rng(0)
+  w = rng.integers(-8, 8, (n, k))
+  words = np.zeros((n, k // 8), np.int64)
+  for j in range(8):
+    words |= ((w[:, j::8] + 8) & 0xF) << (4 * j)
+  packed = torch.from_numpy(words.astype(np.uint32).view(np.int32).reshape(n, k // 8))
+  scale = torch.tensor(rng.random((n, k // 128)) + 0.5, dtype=torch.bfloat16)
+  qa = formats.compressed_int4_experts([packed], [scale], [(n, k)])
+  assert qa.qtype == "int4" and qa.qvalue.shape == (1, n, k // 2)
+  assert np.array_equal(O.unpack_int4(qa.qvalue[0]).numpy(), w)
+  want = torch.from_numpy(w).float().reshape(n, k // 128, 128) * scale.float()[..., None]
+  assert torch.equal(O.dequantize_int4(qa.qvalue[0], qa.scale[0], 128), want.reshape(n, k).to(torch.bfloat16))
+  # the all-ones word of the reference test: nibbles 0xF -> +7 everywhere; zero word -> -8
+  ones = torch.full((1, 4), -1, dtype=torch.int32)
+  assert torch.all(O.unpack_int4(formats.compressed_int4_experts([ones], [torch.ones(1, 1)], [(1, 32)]).qvalue[0]) == 7)
+  with pytest.raises(NotImplementedError):
+    formats.compressed_int4_experts([packed], [scale], [(n, k)], group_size=32)
+
+
+def test_gpt_oss_mxfp4_deinterleave_matches_dequantised_split():
+  g = torch.Generator().manual_seed(1)
+  e, f, d = 2, 24, 64
+  blocks = torch.randint(0, 256, (e, 2 * f, d // 32, 16), generator=g, dtype=torch.uint8)
+  scales = torch.randint(120, 132, (e, 2 * f, d // 32), generator=g, dtype=torch.uint8)
+  dblocks = torch.randint(0, 256, (e, d, f * 2 // 32 + 1, 16), generator=g, dtype=torch.uint8)
+  dscales = torch.randint(120, 132, (e, d, f * 2 // 32 + 1), generator=g, dtype=torch.uint8)
+  bias = torch.randn(e, 2 * f, generator=g)
+  wi_0, wi_1, wo, (b0, b1, bo) = formats.gpt_oss_mxfp4_layer(blocks, scales, dblocks, dscales, bias, None)
+  full = O.dequantize_mxfp4(blocks, scales)  # [e, 2f, d]: what dequantize_mxfp4.py produces before the split
+  deq = lambda qa: O.dequantize_mxfp4(qa.qvalue.reshape(qa.qvalue.shape[0], qa.qvalue.shape[1], -1, 16), qa.scale)
+  assert torch.equal(deq(wi_0), full[:, 0::2]) and torch.equal(deq(wi_1), full[:, 1::2])  # convert_gpt_oss_ckpt.py:270-271
+  assert torch.equal(deq(wo), O.dequantize_mxfp4(dblocks, dscales))
+  assert torch.equal(b0, bias[:, 0::2]) and torch.equal(b1, bias[:, 1::2]) and bo is None
+  assert wi_0.qtype == "mxfp4" and wi_0.qvalue.shape == (e, f, d // 2) and wi_0.scale.shape == (e, f, d // 32)
+
+
+def test_aqt_int8_relayout():
+  g = torch.Generator().manual_seed(2)
+  q = torch.randint(-127, 128, (3, 16, 8), generator=g, dtype=torch.int8)
+  s = torch.rand(3, 1, 8, generator=g)
+  qa = formats.aqt_int8_experts(q, s)
+  assert qa.qvalue.shape == (3, 8, 16) and qa.scale.shape == (3, 8)
+  # moe.py:1450-1459: out = ragged_dot(x, qvalue) * scale[expert] per output channel
+  x = torch.randn(5, 16, generator=g)
+  for ex in range(3):
+    want = (x @ q[ex].float()) * s[ex, 0]
+    got = (x @ qa.qvalue[ex].float().T) * qa.scale[ex]
+    assert torch.allclose(got, want)

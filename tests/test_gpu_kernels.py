@@ -686,3 +686,54 @@ def test_glu_act_forward_and_gradient(K, act):
   if act != "silu":  # no gradient outside the clip range
     assert torch.all(d0.cpu()[h0.float() > 7.0] == 0) and torch.all(d1.cpu()[h1.float().abs() > 7.0] == 0)
     assert (h0.float() > 7.0).any() and (h1.float().abs() > 7.0).any()
+
+
+# ---------------------------------------------------------------- MXFP4 weights (GPT-OSS checkpoint format)
+
+
+@pytest.mark.parametrize("m,k,n,gs", DECODE_SHAPES + [GMM_SHAPES[0], GMM_SHAPES[3], (520, 2880, 96, [500, 20])])
+def test_gmm_mxfp4_weight_only(K, m, k, n, gs):
+  """bf16 activations x MXFP4 weights consumed as stored (e2m1 pairs + e8m0 block scales): the dequantised
+  weights are exact in bf16, so the oracle is its plain bf16 gmm on dequantize_mxfp4 of the same bytes."""
+  from maxtext_amd._lib import MOE_MXFP4
+
+  if k % 32:
+    pytest.skip("MXFP4 blocks hold 32 values")
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 70)
+  blocks, scales = O.quantize_mxfp4(native(w))  # [g, n, k/32, 16], [g, n, k/32]
+  ublocks, uscales = O.quantize_mxfp4(native(w_up))
+  deq = O.dequantize_mxfp4(blocks, scales).to(torch.bfloat16)  # [g, n, k]
+  udeq = O.dequantize_mxfp4(ublocks, uscales).to(torch.bfloat16)
+  assert torch.equal(deq.float(), O.dequantize_mxfp4(blocks, scales))  # exact in bf16
+  e = len(gs)
+  q = blocks.reshape(e, n, k // 2)
+  uq = ublocks.reshape(e, n, k // 2)
+  kw = dict(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+  got = K.gmm_raw(cuda(lhs), cuda(q), cuda(gs), rhs_scale=cuda(scales), **kw)
+  want = O.gmm(lhs, deq, gs, transpose_rhs=True)
+  assert relerr(got, want) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  got = K.gmm_raw(cuda(lhs), cuda(q), cuda(gs), rhs_scale=cuda(scales), rhs_up=cuda(uq), rhs_up_scale=cuda(uscales), act="swigluoai", **kw)
+  want = O.apply_ffn_activation(O.gmm(lhs, deq, gs, transpose_rhs=True, out_dtype=torch.float32),
+                                O.gmm(lhs, udeq, gs, transpose_rhs=True, out_dtype=torch.float32), "swigluoai")
+  assert relerr(got, want) <= TOL
+  # tiled and streaming kernels agree on the same operands
+  tiled = K.gmm_raw(cuda(lhs), cuda(q), cuda(gs), rhs_scale=cuda(scales), rhs_up=cuda(uq), rhs_up_scale=cuda(uscales), act="swigluoai",
+                    tile_variant=1, **kw)
+  assert relerr(tiled, want) <= TOL
+
+
+def test_gmm_mxfp4_exact_on_small_integers(K):
+  """Integer activations and weights from the e2m1 grid with power-of-two scales: every product and partial sum
+  is exact in f32, so the result must equal the oracle bit for bit (catches a swapped nibble or a scale off by one)."""
+  from maxtext_amd._lib import MOE_MXFP4
+
+  rng = np.random.default_rng(11)
+  m, k, n, gs = 48, 256, 64, np.array([20, 0, 28], np.int32)
+  lhs = torch.from_numpy(rng.integers(-3, 4, (m, k)).astype(np.float32)).to(torch.bfloat16)
+  blocks = torch.from_numpy(rng.integers(0, 256, (3, n, k // 32, 16)).astype(np.uint8))
+  scales = torch.from_numpy(rng.integers(124, 131, (3, n, k // 32)).astype(np.uint8))
+  deq = O.dequantize_mxfp4(blocks, scales).to(torch.bfloat16)
+  got = K.gmm_raw(cuda(lhs), cuda(blocks.reshape(3, n, k // 2)), cuda(gs), rhs_scale=cuda(scales), rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+  want = O.gmm(lhs, deq, gs, transpose_rhs=True)
+  assert torch.equal(got.cpu(), want)

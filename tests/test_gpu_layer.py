@@ -70,6 +70,8 @@ CASES = {
     "c5_t16": lambda: _small("c5", 16, num_experts=8),
     "c5_t128": lambda: _small("c5", 128, num_experts=8),
     "c5_t1024": lambda: _small("c5", 1024, num_experts=4, moe_mlp_dim=1024),
+    "c5mx_t16": lambda: _small("c5mx", 16, num_experts=8),
+    "c5mx_t1024": lambda: _small("c5mx", 1024, num_experts=4, moe_mlp_dim=1024),
 }
 
 

@@ -359,3 +359,44 @@ def test_gate_logits_special_cases():
   out16, _ = O.gate_logits(x, w, float32_gate_logits=False)
   want = (x.double() @ w.to(torch.bfloat16).double()).to(torch.bfloat16).float().numpy()
   assert np.array_equal(out16, want)
+
+
+def test_mxfp4_dequantize_code_points_and_layout():
+  """MXFP4: every e2m1 code against the OCP MX value table (restated independently from the bit fields:
+  sign, 2-bit exponent with bias 1, 1 mantissa bit, subnormal 0.5), low nibble first, scale 2^(s-127)."""
+  want = []
+  for code in range(16):
+    sign = -1.0 if code & 8 else 1.0
+    e, m = (code >> 1) & 3, code & 1
+    want.append(sign * (0.5 * m if e == 0 else (1.0 + 0.5 * m) * 2.0 ** (e - 1)))
+  assert np.array_equal(O.E2M1_VALUES, np.array(want, np.float32))
+  blocks = torch.zeros(1, 2, 16, dtype=torch.uint8)
+  blocks[0, 0, 0] = 0x52  # first value code 2 (1.0), second value code 5 (3.0)
+  blocks[0, 0, 15] = 0xF7  # 31st value code 7 (6.0), 32nd code 15 (-6.0)
+  blocks[0, 1, 1] = 0x0B  # block 1: third value code 11 (-1.5)
+  scales = torch.tensor([[127, 124]], dtype=torch.uint8)  # 2^0, 2^-3
+  out = O.dequantize_mxfp4(blocks, scales)
+  assert out.shape == (1, 64)
+  assert out[0, 0] == 1.0 and out[0, 1] == 3.0 and out[0, 30] == 6.0 and out[0, 31] == -6.0
+  assert out[0, 34] == -1.5 / 8 and out[0, 35] == 0.0
+  # quantise -> dequantise is the identity on representable inputs
+  g = torch.Generator().manual_seed(3)
+  codes = torch.randint(0, 16, (4, 96), generator=g)
+  exps = torch.randint(-6, 5, (4, 3), generator=g).float()
+  x = torch.from_numpy(O.E2M1_VALUES)[codes].reshape(4, 3, 32) * torch.exp2(exps)[..., None]
+  x[:, :, 0] = 6.0 * torch.exp2(exps)  # pin the block maximum so the shared exponent is the one used above
+  b, s_ = O.quantize_mxfp4(x.reshape(4, 96))
+  assert torch.equal(O.dequantize_mxfp4(b, s_), x.reshape(4, 96))
+
+
+def test_product_mxfp4_quantiser_agrees_with_oracle_generator():
+  """The package's mxfp4 quantiser (used for synthetic weights) and the oracle's test-data generator are written
+  independently (threshold chain vs nearest-grid search); they must produce the same bytes."""
+  from maxtext_amd import quantizations as Q
+
+  g = torch.Generator().manual_seed(5)
+  w = torch.randn(2, 6, 96, generator=g) * 0.02
+  w[0, 0, :32] = 0.0  # an all-zero block
+  qa = Q.quantize_weight_mxfp4(w)
+  blocks, scales = O.quantize_mxfp4(w)
+  assert torch.equal(qa.qvalue.reshape(2, 6, 3, 16), blocks) and torch.equal(qa.scale, scales)
