@@ -11,6 +11,7 @@ The default workload is the Mixtral-8x7B-shape int8 prefill layer (8192 tokens, 
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -64,6 +65,13 @@ def dominant_kernel_model(wl, group_sizes):
     io_bytes = rows * d * 1.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name="gmm_fp8_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")
+  if wl.weight_quant in ("int4", "mxfp4") and rows <= 32 * cfg.num_experts:
+    # weight-only 4-bit decode: bound by streaming the weights of the experts that were hit
+    w_bytes = nonempty * 2.0 * d * f * 0.5
+    s_bytes = nonempty * 2.0 * f * (math.ceil(d / 128) * 2 if wl.weight_quant == "int4" else d / 32)
+    io_bytes = rows * d * 2.0 + rows * f * 2.0
+    return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
+                name="gmm_wq_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="bf16")
   op = "int8" if cfg.act_quant == "int8" else "bf16"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
               name=("gmm_dl_kernel" if cfg.act_quant == "int8" else "gmm_tiled_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype=op)
@@ -281,7 +289,8 @@ def main():
   dom_ms = stage_ms.get("wi_glu")
   achieved = model["work"] / (dom_ms * 1e-3) / model["scale"] if dom_ms else None
   roofline = dict(bound=model["bound"], achieved=achieved, peak=model["peak"], unit=model["unit"],
-                  frac=(achieved / model["peak"]) if achieved else None, traffic=MEASURED_TRAFFIC_BYTES.get(wl.name), kernel=model["name"],
+                  frac=(achieved / model["peak"]) if achieved else None,
+                  traffic=MEASURED_TRAFFIC_BYTES.get(wl.name) if args.tokens is None else None, kernel=model["name"],
                   kernel_ms=dom_ms)
 
   flops = synthetic.layer_flops(wl)
