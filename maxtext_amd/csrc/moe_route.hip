@@ -679,6 +679,44 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in
   }
 }
 
+// 2-byte elements with K % 8 == 0 and N % 8 == 0: 16-byte loads along N into LDS, then ds_read_b64_tr_b16 (the
+// transposing LDS load: 16 lanes read a 4 x 16 block and lane L receives column L) twice per lane, which yields 8
+// consecutive K values of one output row as one 16-byte store.
+typedef short tr_v4s __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) tr_v4s* tr_lds_ptr;
+
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* __restrict__ in, int K, int N,
+                                                          uint16_t* __restrict__ out) {
+  constexpr int kPitch = 64 * 2 + 16;  // bytes per LDS row
+  __shared__ __attribute__((aligned(16))) uint8_t tile[64 * kPitch];
+  const size_t g = blockIdx.z;
+  const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int r = h * 32 + tid / 8, c8 = tid % 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (k0 + r < K && n0 + c8 * 8 < N) v = *(const uint4*)(in + (g * K + k0 + r) * N + n0 + c8 * 8);
+    *(uint4*)(tile + r * kPitch + c8 * 16) = v;
+  }
+  __syncthreads();
+  const int s = tid % 16, grp = tid / 16;  // 16 lane groups
+  const int n16 = grp % 4;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int k8 = grp / 4 + h * 4;
+    const uint8_t* p = tile + (k8 * 8 + s / 4) * kPitch + (n16 * 16 + 4 * (s % 4)) * 2;
+    const tr_v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_lds_ptr)p);
+    const tr_v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_lds_ptr)(p + 4 * kPitch));
+    const int n = n0 + n16 * 16 + s, k = k0 + k8 * 8;
+    if (n < N && k < K) {
+      typedef short v8s __attribute__((ext_vector_type(8)));
+      const v8s v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      *(uint4*)(out + (g * N + n) * K + k) = __builtin_bit_cast(uint4, v);
+    }
+  }
+}
+
 }  // namespace moe
 
 using namespace moe;
@@ -886,6 +924,8 @@ int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem_bytes, 
   hipStream_t s = (hipStream_t)stream;
   if (elem_bytes == 1)
     transpose_kernel<uint8_t><<<grid, 256, 0, s>>>((const uint8_t*)rhs_gkn, K, N, (uint8_t*)rhs_gnk);
+  else if (elem_bytes == 2 && K % 8 == 0 && N % 8 == 0 && (((uintptr_t)rhs_gkn | (uintptr_t)rhs_gnk) & 15) == 0)
+    transpose16_kernel<<<grid, 256, 0, s>>>((const uint16_t*)rhs_gkn, K, N, (uint16_t*)rhs_gnk);
   else if (elem_bytes == 2)
     transpose_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)rhs_gkn, K, N, (uint16_t*)rhs_gnk);
   else

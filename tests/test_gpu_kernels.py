@@ -180,8 +180,11 @@ def test_combine_exact_on_integers(K):
 def test_transpose_rhs(K):
   w = torch.randint(-128, 128, (3, 200, 136), dtype=torch.int8)
   assert torch.equal(K.transpose_rhs(cuda(w)).cpu(), w.transpose(1, 2).contiguous())
-  wb = torch.randn(2, 70, 264).to(torch.bfloat16)
+  wb = torch.randn(2, 70, 264).to(torch.bfloat16)  # K % 8 != 0: element-wise kernel
   assert torch.equal(K.transpose_rhs(cuda(wb)).cpu(), wb.transpose(1, 2).contiguous())
+  for shape in ((2, 72, 264), (3, 128, 64), (1, 200, 136), (2, 8, 8), (1, 1024, 520)):  # 16-byte path, ragged tiles
+    wb = torch.randn(*shape).to(torch.bfloat16)
+    assert torch.equal(K.transpose_rhs(cuda(wb)).cpu(), wb.transpose(1, 2).contiguous()), shape
 
 
 # ---------------------------------------------------------------- grouped matmul
