@@ -1263,14 +1263,31 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 // Host side
 // ---------------------------------------------------------------------------------------
 
+// Per-device launch state: the attribute that lets a kernel use more than 64 KB of dynamic LDS belongs to a
+// device's code object, and the CU count to the device, so both are kept per device ordinal.  A race between two
+// host threads only repeats an idempotent call.
+constexpr int kMaxDevices = 64;
+
+static int current_device(int* dev) {
+  if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= kMaxDevices) return fail(MOE_ERR_LAUNCH, "gmm: cannot identify the current device");
+  return MOE_OK;
+}
+
+template <typename K>
+static int reserve_lds(K kernel, int bytes, bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  if (int st = current_device(&dev)) return st;
+  if (done[dev]) return MOE_OK;
+  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "gmm: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+  done[dev] = true;
+  return MOE_OK;
+}
+
 template <typename C>
 static int launch_tiled(const TiledParams& p0, int M, int G_total, hipStream_t s) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gmm_tiled_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "gmm: cannot reserve %d bytes of LDS: %s", C::LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static bool attr_set[kMaxDevices] = {};
+  if (int st = reserve_lds(gmm_tiled_kernel<C>, C::LDS_BYTES, attr_set)) return st;
   TiledParams p = p0;
   p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
   p.tiles_n = cdiv(p.N, C::OUT_BN);
@@ -1282,12 +1299,8 @@ static int launch_tiled(const TiledParams& p0, int M, int G_total, hipStream_t s
 
 template <typename C>
 static int launch_dl(const TiledParams& p0, int M, int G_total, hipStream_t s) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gmm_dl_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "gmm: cannot reserve %d bytes of LDS: %s", C::LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static bool attr_set[kMaxDevices] = {};
+  if (int st = reserve_lds(gmm_dl_kernel<C>, C::LDS_BYTES, attr_set)) return st;
   TiledParams p = p0;
   p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
   p.tiles_n = cdiv(p.N, C::OUT_BN);
@@ -1295,13 +1308,16 @@ static int launch_dl(const TiledParams& p0, int M, int G_total, hipStream_t s) {
   if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
   // one persistent block per CU (the LDS footprint allows no more); a multiple of 8 keeps "tile id mod 8"
   // equal to the XCD a block runs on
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+  static int cus_of[kMaxDevices] = {};
+  int dev = 0;
+  if (int st = current_device(&dev)) return st;
+  if (cus_of[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
       return fail(MOE_ERR_LAUNCH, "gmm: cannot query the CU count");
-    num_cus = n;
+    cus_of[dev] = n;
   }
+  const int num_cus = cus_of[dev];
   long long blocks = tiles < num_cus ? tiles : num_cus;
   if (blocks >= 8) blocks -= blocks % 8;
   gmm_dl_kernel<C><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
@@ -1513,7 +1529,8 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
 
   const int M = a->M, G = a->num_groups_total;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
-  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->reserved[0] != 1) {
+  // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
+  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->K % 32 == 0 && a->reserved[0] != 1) {
     const bool one = (long long)M <= 16LL * G;
     bm = one ? 16 : 32;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);

@@ -740,3 +740,145 @@ def test_gmm_mxfp4_exact_on_small_integers(K):
   got = K.gmm_raw(cuda(lhs), cuda(blocks.reshape(3, n, k // 2)), cuda(gs), rhs_scale=cuda(scales), rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
   want = O.gmm(lhs, deq, gs, transpose_rhs=True)
   assert torch.equal(got.cpu(), want)
+
+
+# ---------------------------------------------------------------- randomised shapes, every operand family
+
+
+def _random_case(rng, k_mult):
+  e = int(rng.integers(1, 9))
+  k = int(rng.integers(1, 9)) * k_mult
+  n = int(rng.integers(1, 40)) * 8
+  regime = rng.integers(0, 3)  # few rows per expert (streaming kernels), medium, many (256-row tiles)
+  hi = (12, 90, 400)[regime]
+  gs = rng.integers(0, hi, e)
+  gs[rng.integers(0, e)] = 0 if e > 1 and rng.random() < 0.5 else gs[rng.integers(0, e)]
+  m = int(gs.sum()) + int(rng.integers(0, 20))  # trailing rows that belong to no group
+  return max(m, 1), k, n, gs.astype(np.int32)
+
+
+@pytest.mark.parametrize("family", ["bf16", "w8", "i8", "int4", "mxfp4", "fp8"])
+def test_gmm_random_shapes(K, family):
+  """20 random (M, K, N, group_sizes) per operand family against the oracle: ragged groups, empty groups, rows
+  past the last group, K and N at every supported granularity, with and without the fused activation and bias."""
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
+
+  rng = np.random.default_rng({"bf16": 1, "w8": 2, "i8": 3, "int4": 4, "mxfp4": 5, "fp8": 6}[family])
+  k_mult = {"bf16": 8, "w8": 16, "i8": 16, "int4": 32, "mxfp4": 32, "fp8": 128}[family]
+  for case in range(20):
+    m, k, n, gs = _random_case(rng, k_mult)
+    lhs, w, w_up, _ = _gmm_inputs(m, k, n, list(gs), 1000 + case)
+    e = len(gs)
+    glu = bool(case % 2)
+    bias = _bias(e, n, case) if case % 3 == 0 else (None, None)
+    kw, okw, lhs_g, lhs_o = {}, {}, lhs, lhs
+    if family == "bf16":
+      wq, uq = w.to(torch.bfloat16), w_up.to(torch.bfloat16)
+      rhs, rhs_up, orhs, orhs_up = native(wq), native(uq), wq, uq
+    elif family in ("w8", "i8"):
+      (q, s), (qu, su) = O.quantize_weight_int8(w), O.quantize_weight_int8(w_up)
+      rhs, rhs_up, orhs, orhs_up = native(q), native(qu), q, qu
+      kw.update(rhs_scale=cuda(s), rhs_up_scale=cuda(su))
+      okw.update(rhs_scale=s)
+      oup = dict(rhs_scale=su)
+      if family == "i8":
+        aq, asc = O.quantize_rows_int8(lhs.float())
+        lhs_g, lhs_o = aq, aq
+        kw.update(lhs_scale=cuda(asc))
+        okw.update(lhs_scale=asc[:, None])
+        oup.update(lhs_scale=asc[:, None])
+    elif family == "int4":
+      (q, s), (qu, su) = O.quantize_int4_groups(native(w), 128), O.quantize_int4_groups(native(w_up), 128)
+      s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
+      v2 = lambda sc: sc.float().permute(0, 2, 1)[:, :, None, :]
+      rhs, rhs_up, orhs, orhs_up = O.pack_int4(q), O.pack_int4(qu), q.transpose(1, 2), qu.transpose(1, 2)
+      kw.update(rhs_scale=cuda(s), rhs_up_scale=cuda(su), rhs_dtype=MOE_INT4, rhs_scale_block_k=128)
+      okw.update(rhs_scale=v2(s), quant_block=128)
+      oup = dict(rhs_scale=v2(su), quant_block=128)
+    elif family == "mxfp4":
+      (b, s), (bu, su) = O.quantize_mxfp4(native(w)), O.quantize_mxfp4(native(w_up))
+      rhs, rhs_up = b.reshape(e, n, k // 2), bu.reshape(e, n, k // 2)
+      orhs = O.dequantize_mxfp4(b, s).to(torch.bfloat16).transpose(1, 2)
+      orhs_up = O.dequantize_mxfp4(bu, su).to(torch.bfloat16).transpose(1, 2)
+      kw.update(rhs_scale=cuda(s), rhs_up_scale=cuda(su), rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+    else:  # fp8 block scaled
+      aq, asc = O.quantize_fp8_blocks(lhs, 1, 128)
+      (q, s), (qu, su) = O.quantize_fp8_blocks(native(w), 128, 128), O.quantize_fp8_blocks(native(w_up), 128, 128)
+      v2f = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
+      lhs_g, lhs_o = aq, aq
+      rhs, rhs_up, orhs, orhs_up = q, qu, q.transpose(1, 2), qu.transpose(1, 2)
+      kw.update(lhs_scale=cuda(asc), rhs_scale=cuda(s), rhs_up_scale=cuda(su), lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128)
+      okw.update(lhs_scale=asc, rhs_scale=v2f(s), quant_block=128)
+      oup = dict(lhs_scale=asc, rhs_scale=v2f(su), quant_block=128)
+    if family in ("bf16", "mxfp4"):
+      oup = {}
+    if not glu:
+      kw.pop("rhs_up_scale", None)
+    ob0 = None if bias[0] is None else bias[0][:, None, :]
+    ob1 = None if bias[1] is None else bias[1][:, None, :]
+    tag = f"{family} case {case}: m={m} k={k} n={n} gs={list(gs)} glu={glu} bias={bias[0] is not None}"
+    if glu:
+      got = K.gmm_raw(cuda(lhs_g), cuda(rhs), cuda(gs), rhs_up=cuda(rhs_up), act="silu", rhs_bias=None if bias[0] is None else cuda(bias[0]),
+                      rhs_up_bias=None if bias[1] is None else cuda(bias[1]), **kw)
+      want = O.apply_ffn_activation(O.gmm(lhs_o, orhs, gs, out_dtype=torch.float32, rhs_bias=ob0, **okw),
+                                    O.gmm(lhs_o, orhs_up, gs, out_dtype=torch.float32, rhs_bias=ob1, **{**okw, **oup}))
+    else:
+      got = K.gmm_raw(cuda(lhs_g), cuda(rhs), cuda(gs), rhs_bias=None if bias[0] is None else cuda(bias[0]), **kw)
+      want = O.gmm(lhs_o, orhs, gs, rhs_bias=ob0, **okw)
+    used = int(gs.sum())
+    assert torch.isfinite(got.float()).all(), tag
+    assert torch.all(got[used:] == 0), tag
+    if used:
+      assert relerr(got, want) <= TOL, tag
+
+
+def test_route_sort_gather_combine_random_sizes(K):
+  """Random (T, E, k, d): the integer half of the path bit-exact against numpy, gathers and the weighted combine
+  against brute force, for sizes around the kernels' internal chunk boundaries."""
+  rng = np.random.default_rng(77)
+  for case in range(24):
+    e = int(rng.choice([1, 2, 7, 8, 32, 60, 64, 65, 128, 200, 256, 384, 512]))
+    k = int(rng.integers(1, min(e, 8) + 1))
+    t = int(rng.choice([1, 2, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 4097, 9000]))
+    d = int(rng.integers(1, 40)) * 8
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    if case % 4 == 0:
+      logits = np.round(logits * 2) / 2  # many exact ties
+    w, idx = K.route_topk(cuda(logits), k=k, norm_topk_prob=bool(case % 2))
+    ow, oidx = O.get_topk(logits, k=k, norm_topk_prob=bool(case % 2))
+    tag = f"case {case}: t={t} e={e} k={k} d={d}"
+    np.testing.assert_array_equal(idx.cpu().numpy(), oidx, err_msg=tag)
+    np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=2.0**-6, atol=1e-6, err_msg=tag)
+    perm, inv, gs, se = K.sort_by_expert(idx, e)
+    flat = oidx.reshape(-1)
+    operm = np.argsort(flat, kind="stable").astype(np.int32)
+    np.testing.assert_array_equal(perm.cpu().numpy(), operm, err_msg=tag)
+    np.testing.assert_array_equal(gs.cpu().numpy(), np.bincount(flat, minlength=e), err_msg=tag)
+    np.testing.assert_array_equal(se.cpu().numpy(), flat[operm], err_msg=tag)
+    np.testing.assert_array_equal(inv.cpu().numpy()[operm], np.arange(t * k), err_msg=tag)
+    x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(torch.bfloat16)
+    rows = K.gather_rows(cuda(x), perm, k)
+    assert torch.equal(rows.cpu(), x[torch.from_numpy(operm.astype(np.int64) // k)]), tag
+    out = K.unpermute_combine(rows, w, k=k, inv_perm=inv)
+    want = (x.float() * torch.from_numpy(ow).sum(-1, keepdim=True)).to(torch.bfloat16)  # every copy of a token is the token itself
+    assert relerr(out, want) <= 2.0**-7, tag
+
+
+def test_tgmm_random_shapes(K):
+  rng = np.random.default_rng(78)
+  for case in range(16):
+    e = int(rng.integers(1, 7))
+    k, n = int(rng.integers(1, 50)) * 8, int(rng.integers(1, 50)) * 8
+    gs = rng.integers(0, (5, 40, 300)[case % 3], e).astype(np.int32)
+    m = max(int(gs.sum()) + int(rng.integers(0, 10)), 1)
+    g = torch.Generator().manual_seed(case)
+    lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=torch.float32)
+    want = O.tgmm(lhs, dout, gs, out_dtype=torch.float32).transpose(1, 2)
+    tag = f"case {case}: m={m} k={k} n={n} gs={list(gs)}"
+    for i, sz in enumerate(gs):
+      if sz == 0:
+        assert torch.all(got[i] == 0), tag
+      else:
+        assert relerr(got[i], want[i]) <= TOL, tag
