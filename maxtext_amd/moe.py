@@ -39,6 +39,8 @@ class MoEConfig:
   shared_experts: int = 0
   # activation quantisation for the grouped GEMMs: None | "int8" | "fp8"
   act_quant: Optional[str] = None
+  load_balance_loss_weight: float = 0.0  # > 0: permute / sparse_matmul return the auxiliary loss (moe.py:888-891)
+  routed_bias_update_rate: float = 0.0  # > 0 with routed_bias: return the loss-free balancing update (moe.py:893-898)
 
   @property
   def is_deepseek(self) -> bool:
@@ -51,6 +53,13 @@ class MoEConfig:
     if self.is_deepseek and self.mlp_activations_limit > 0.0:
       return "silu_clip"
     return "silu"
+
+
+def calculate_load_balance_updates(top_k_indices: torch.Tensor, num_experts: int, rate: float) -> torch.Tensor:
+  """Bias adjustment sign(average_load - expert_load) * rate, shape [num_experts] (moe.py:215-236)."""
+  flat = top_k_indices.reshape(-1).long()
+  counts = torch.bincount(flat, minlength=num_experts).float()
+  return torch.sign(flat.numel() / num_experts - counts) * rate
 
 
 class _GatherRowsFn(torch.autograd.Function):
@@ -139,6 +148,29 @@ class RoutedMoE:
                                 topk_routing_group=cfg.topk_routing_group, **common)
     return kernels.gate_route(x, self._gate_terms, bias, norm_topk_prob=cfg.norm_topk_prob, **common)
 
+  # -- auxiliary outputs of permute (moe.py:886-900) ------------------------------------------
+  def load_balance_loss(self, top_k_indices: torch.Tensor, probs: torch.Tensor) -> torch.Tensor:
+    """Sequence-wise load-balance loss (moe.py:2662-2687): per sequence, token density per expert times mean
+    routing probability per expert, averaged, times E^2 * load_balance_loss_weight.  top_k_indices [B,S,k],
+    probs [B,S,E]."""
+    e = self.num_experts
+    b, s_, k = top_k_indices.shape
+    counts = torch.zeros((b, e), dtype=torch.float32, device=probs.device)
+    counts.scatter_add_(1, top_k_indices.reshape(b, s_ * k).long(), torch.ones((b, s_ * k), dtype=torch.float32, device=probs.device))
+    density = counts / s_
+    density_prob = probs.float().mean(dim=1)
+    return (density * density_prob).mean() * (e**2) * self.config.load_balance_loss_weight
+
+  def _aux_outputs(self, gate_logits, selected):
+    cfg = self.config
+    lb_loss = bias_updates = None
+    if cfg.load_balance_loss_weight > 0.0 and gate_logits is not None:
+      probs = torch.softmax(gate_logits.float(), dim=-1).to(torch.bfloat16)
+      lb_loss = self.load_balance_loss(selected, probs)
+    if cfg.routed_bias and cfg.routed_bias_update_rate > 0.0:
+      bias_updates = calculate_load_balance_updates(selected, self.num_experts, cfg.routed_bias_update_rate)
+    return lb_loss, bias_updates
+
   # -- get_topk (moe.py:717-765) ------------------------------------------------------------
   def get_topk(self, gate_logits: torch.Tensor, pre_bias_logits: Optional[torch.Tensor] = None):
     cfg = self.config
@@ -190,7 +222,8 @@ class RoutedMoE:
     else:
       sorted_inputs = kernels.gather_rows(x2d, perm, self.num_experts_per_tok)
     self._last_inv_perm = inv
-    return sorted_inputs, perm, weights, group_size, sorted_experts, None, None, None
+    lb_loss, bias_updates = self._aux_outputs(gate_logits, selected)
+    return sorted_inputs, perm, weights, group_size, sorted_experts, lb_loss, bias_updates, None
 
   # -- unpermute (moe.py:1004-1063), non-ragged branch --------------------------------------
   def unpermute(self, intermediate, sorted_selected_experts, weights, batch_size, sequence_length,
@@ -274,7 +307,8 @@ class RoutedMoE:
       sorted_inputs = kernels.gather_rows(x2d, perm, k)
     inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias)
     out = self.unpermute(inter, perm, weights, b, s, inv_perm=inv)
-    return out, None, None
+    lb_loss, bias_updates = self._aux_outputs(gate_logits, selected.reshape(b, s, k))
+    return out, lb_loss, bias_updates
 
   def __call__(self, inputs, input_ids=None, gate_inputs=None, out_sharding=None):
     """-> (output, lb_loss, bias_updates), as moe.py:3143."""
@@ -283,8 +317,10 @@ class RoutedMoE:
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (routing_inputs, self.gate_kernel, self.gate_bias))
     if not needs_grad and routing_inputs.dtype == torch.bfloat16 and routing_inputs.shape[-1] % 64 == 0 and self.num_experts % 4 == 0:
-      routing = self.gate_and_route(routing_inputs.reshape(b * s, -1))
-      return self.sparse_matmul(inputs, None, None, self.wi_0, self.wi_1, self.wo, routing=routing)
+      want_logits = self.config.load_balance_loss_weight > 0.0  # the auxiliary loss needs the full distribution
+      r = self.gate_and_route(routing_inputs.reshape(b * s, -1), return_logits=want_logits)
+      logits = r[2].reshape(b, s, -1) if want_logits else None
+      return self.sparse_matmul(inputs, logits, None, self.wi_0, self.wi_1, self.wo, routing=(r[0], r[1]))
     gate_logits, pre_bias = self.gate(routing_inputs.reshape(b * s, -1))
     gate_logits = gate_logits.reshape(b, s, -1)
     pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)

@@ -344,3 +344,41 @@ def test_gpt_oss_style_layer_with_mlp_bias():
     a = O.apply_ffn_activation(h0.float(), h1.float(), "swigluoai", 7.0).double()
     want += w[:, s_ : s_ + 1] * (torch.einsum("tf,tdf->td", a, wo.double()[ex]) + bo.double()[ex])
   assert relerr(out.reshape(t, d), want) <= TOL
+
+
+def test_auxiliary_outputs_match_reference_formulas():
+  """lb_loss (moe.py:2662-2687) and bias_updates (moe.py:215-236, known answer of tests/unit/moe_test.py:328-341)
+  as returned by sparse_matmul / __call__."""
+  import dataclasses as dc
+
+  from maxtext_amd import moe
+
+  # the reference's own vector: 4 experts, indices [[0,1],[0,2],[0,3]] -> sign(1.5 - [3,1,1,1]) * rate
+  upd = moe.calculate_load_balance_updates(torch.tensor([[[0, 1], [0, 2], [0, 3]]]), 4, 0.1)
+  assert torch.allclose(upd, torch.tensor([-0.1, 0.1, 0.1, 0.1]))
+  assert np.allclose(O.calculate_load_balance_updates(np.array([[[0, 1], [0, 2], [0, 3]]]), 4, 0.1), upd.numpy())
+
+  g = torch.Generator().manual_seed(61)
+  b, s_, d, f, e, k = 2, 96, 128, 128, 8, 2
+  x = torch.randn(b, s_, d, generator=g).to(torch.bfloat16).cuda()
+  logits = torch.randn(b, s_, e, generator=g).cuda()
+  ws = [(torch.randn(e, n_, k_, generator=g) * 0.05).to(torch.bfloat16).cuda() for n_, k_ in ((f, d), (f, d), (d, f))]
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, load_balance_loss_weight=0.01,
+                      routed_bias=True, routed_bias_update_rate=0.001)
+  block = moe.RoutedMoE(cfg, *ws)
+  out, lb, upd = block.sparse_matmul(x, logits, None, *ws)
+  _, idx = block.get_topk(logits)
+  idx = idx.cpu().long()
+  # brute force per sequence
+  probs = torch.softmax(logits.cpu().float(), -1).to(torch.bfloat16).float()
+  want = 0.0
+  for bi in range(b):
+    dens = torch.bincount(idx[bi].reshape(-1), minlength=e).float() / s_
+    want += float((dens * probs[bi].mean(0)).mean())
+  want = want / b * e * e * 0.01
+  assert abs(float(lb) - want) <= 1e-4 * abs(want)
+  cnt = torch.bincount(idx.reshape(-1), minlength=e).float()
+  assert torch.equal(upd.cpu(), torch.sign(b * s_ * k / e - cnt) * 0.001)
+  # without the config keys nothing is returned
+  _, lb0, upd0 = moe.RoutedMoE(dc.replace(cfg, load_balance_loss_weight=0.0, routed_bias_update_rate=0.0), *ws).sparse_matmul(x, logits, None, *ws)
+  assert lb0 is None and upd0 is None
