@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void gate_gemm_kernel(const GateGemmParams p) 
 
 // ---------------------------------------------------------------------------------------
 // Stable counting sort of the flattened expert ids.
-//   pass 1: per-wave-segment histograms; pass 2: exclusive scan over segments and experts;
+//   pass 1: per-wave-segment histograms; pass 2: exclusive scan over segments (one wave per expert);
 //   pass 3: each wave re-reads its segment and ranks equal ids with ballots, in index order.
 // ---------------------------------------------------------------------------------------
 
@@ -327,42 +327,54 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_hist_kernel(
   for (int e = lane; e < E; e += kWave) dst[e] = cnt[wave][e];
 }
 
-__global__ __launch_bounds__(kSortMaxE) void sort_scan_kernel(int32_t* __restrict__ seg_hist,
-                                                              int nseg, int E,
-                                                              int32_t* __restrict__ group_sizes,
-                                                              int32_t* __restrict__ expert_off) {
-  __shared__ int tot[kSortMaxE];
-  const int e = threadIdx.x;
+// pass 2: one wave per expert turns its column of segment counts into exclusive prefixes (64 segments per step,
+// a shuffle scan inside the wave) and writes the expert's total to group_sizes.
+__global__ __launch_bounds__(kSortWaves* kWave) void sort_scan_kernel(int32_t* __restrict__ seg_hist, int nseg, int E,
+                                                                     int32_t* __restrict__ group_sizes) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int e = blockIdx.x * kSortWaves + wave;
+  if (e >= E) return;
   int running = 0;
-  if (e < E) {
-    for (int s = 0; s < nseg; s++) {
-      int c = seg_hist[(size_t)s * E + e];
-      seg_hist[(size_t)s * E + e] = running;
-      running += c;
+  for (int s0 = 0; s0 < nseg; s0 += kWave) {
+    const int s = s0 + lane;
+    const int c = s < nseg ? seg_hist[(size_t)s * E + e] : 0;
+    int incl = c;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const int up = __shfl_up(incl, o);
+      if (lane >= o) incl += up;
     }
-    group_sizes[e] = running;
+    if (s < nseg) seg_hist[(size_t)s * E + e] = running + incl - c;
+    running += __shfl(incl, kWave - 1);
   }
-  tot[e] = e < E ? running : 0;
-  __syncthreads();
-  // inclusive Hillis-Steele scan over experts
-  for (int o = 1; o < kSortMaxE; o <<= 1) {
-    int add = e >= o ? tot[e - o] : 0;
-    __syncthreads();
-    tot[e] += add;
-    __syncthreads();
-  }
-  if (e < E) expert_off[e] = tot[e] - running;
+  if (lane == 0) group_sizes[e] = running;
 }
 
 __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
     const int32_t* __restrict__ flat, int M, int E, int ebits,
-    const int32_t* __restrict__ seg_hist, const int32_t* __restrict__ expert_off,
+    const int32_t* __restrict__ seg_hist, const int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
     int32_t* __restrict__ sorted_experts) {
   __shared__ int run[kSortWaves][kSortMaxE];
+  __shared__ int off[kSortMaxE];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  // first row of every expert = exclusive scan of group_sizes, rebuilt by each block (E <= 512 values)
+  for (int e = threadIdx.x; e < kSortMaxE; e += kSortWaves * kWave) off[e] = e < E ? group_sizes[e] : 0;
+  __syncthreads();
+  for (int o = 1; o < kSortMaxE; o <<= 1) {
+    int add[kSortMaxE / (kSortWaves * kWave)];
+#pragma unroll
+    for (int q = 0; q < kSortMaxE / (kSortWaves * kWave); q++) {
+      const int e = threadIdx.x + q * kSortWaves * kWave;
+      add[q] = e >= o ? off[e - o] : 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kSortMaxE / (kSortWaves * kWave); q++) off[threadIdx.x + q * kSortWaves * kWave] += add[q];
+    __syncthreads();
+  }
   const int32_t* seg = seg_hist + (size_t)(blockIdx.x * kSortWaves + wave) * E;
-  for (int e = lane; e < E; e += kWave) run[wave][e] = expert_off[e] + seg[e];
+  for (int e = lane; e < E; e += kWave) run[wave][e] = (e > 0 ? off[e - 1] : 0) + seg[e];
   __syncthreads();
   const int base = blockIdx.x * kSortChunk + wave * kSortSeg;
   const unsigned long long lt = (1ull << lane) - 1ull;
@@ -821,14 +833,13 @@ int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* pe
   const int nblk = cdiv(M, kSortChunk);
   const int nseg = nblk * kSortWaves;
   int32_t* seg_hist = (int32_t*)workspace;
-  int32_t* expert_off = seg_hist + (size_t)nseg * E;
   hipStream_t s = (hipStream_t)stream;
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
   if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, seg_hist);
-  sort_scan_kernel<<<1, kSortMaxE, 0, s>>>(seg_hist, nseg, E, group_sizes, expert_off);
+  sort_scan_kernel<<<cdiv(E, kSortWaves), kSortWaves * kWave, 0, s>>>(seg_hist, nseg, E, group_sizes);
   if (nblk > 0)
-    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, seg_hist, expert_off,
+    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, seg_hist, group_sizes,
                                                           perm, inv_perm, sorted_experts);
   return check_launch("sort_by_expert");
 }
