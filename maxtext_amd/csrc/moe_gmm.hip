@@ -1326,8 +1326,10 @@ static int launch_dl(const TiledParams& p0, int M, int G_total, hipStream_t s) {
 
 template <int OP, int BSRC, bool GLU>
 static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* bm_out, bool dry, hipStream_t s) {
-  // rows per expert on average decides the m-tile: full 256-row tiles for prefill, 64 otherwise
-  const bool big = (long long)M >= 128LL * G_total;
+  // rows per expert on average decides the m-tile: full 256-row tiles for prefill, 64 otherwise; a problem with
+  // fewer 256 x 256 tiles than half the CUs of the chip also takes the 64-row tiles, which quadruples its blocks
+  const long long tiles_big = (long long)max_tiles_for(M, G_total, 256) * cdiv(p.N, GLU ? 128 : 256);
+  const bool big = (long long)M >= 128LL * G_total && tiles_big >= 128;
   *bm_out = big ? 256 : 64;
   if (dry) return MOE_OK;
   if constexpr (BSRC == BSRC_SAME) {
@@ -1554,7 +1556,10 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
     return glu ? launch_i8_variant<true>(forced, p, M, G, &bm, false, s) : launch_i8_variant<false>(forced, p, M, G, &bm, false, s);
   }
-  launch_tiled_by_rows<OP_BF16, BSRC_SAME, false>(p, M, G, &bm, true, s);
+  if (glu)
+    launch_tiled_by_rows<OP_BF16, BSRC_SAME, true>(p, M, G, &bm, true, s);
+  else
+    launch_tiled_by_rows<OP_BF16, BSRC_SAME, false>(p, M, G, &bm, true, s);
   tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
   switch (variant) {
     case V_BF16: return launch_tiled_glu<OP_BF16, BSRC_SAME>(p, glu, M, G, &bm, false, s);
