@@ -168,7 +168,7 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  *   rhs_scale  NULL (bf16 rhs) | [G_local, ceil(N/bn), nkb] with
  *              bn = rhs_scale_block_n (1 = per output channel, 128 = DeepSeek 128x128 blocks),
  *              nkb = 1 when rhs_scale_block_k == 0 (per channel over all of K), else
- *              ceil(K / rhs_scale_block_k) (must be 128); f32, or bf16 for INT4;
+ *              ceil(K / rhs_scale_block_k) (128; INT4 also 32, the Kimi-K2 group size); f32, or bf16 for INT4;
  *              MXFP4: bytes [G_local, N, K/32] (rhs_scale_block_n = 1, rhs_scale_block_k = 32)
  *   rhs_up / rhs_up_scale   second projection (wi_1) with the same layout; when non-NULL
  *              the kernel computes act(lhs@rhs^T) * (lhs@rhs_up^T) in one pass
@@ -176,7 +176,7 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  *   out        [M, N] bf16
  *
  * Supported operand combinations (others return MOE_ERR_UNSUPPORTED):
- *   BF16 x BF16 | BF16 x INT8 (per-channel) | BF16 x INT4 (bn=1, bk=128) | BF16 x MXFP4 (bn=1, bk=32)
+ *   BF16 x BF16 | BF16 x INT8 (per-channel) | BF16 x INT4 (bn=1, bk=128 or 32) | BF16 x MXFP4 (bn=1, bk=32)
  *   INT8 (per-row) x INT8 (per-channel) | FP8 (1x128) x FP8 (128x128 blocks)
  * Alignment: K % 32 == 0 (INT4, MXFP4), K % 16 == 0 otherwise; N % 8 == 0; pointers 16-byte aligned.
  */
@@ -201,7 +201,7 @@ typedef struct {
   int32_t rhs_scale_block_n, rhs_scale_block_k;
   int32_t act;     /* moe_act; must be MOE_ACT_NONE when rhs_up == NULL      */
   float act_limit; /* clip for SWIGLUOAI / SILU_CLIP                        */
-  int32_t reserved[4];
+  int32_t reserved[4]; /* zero.  [0] and [1] select experimental kernel shapes (tuning aids of the benchmarks) */
   /* per-expert bias [G_local, N] f32 added to lhs@rhs^T (and to lhs@rhs_up^T) before the activation:
    * w0_bias / w1_bias / wo_bias of mlp_bias models (moe.py:1952-1981, :2239-2241; rhs_bias of
    * pallas_mosaic_tpu_v2_gmm_kernel.py:573).  NULL = no bias.  Rows that are written as zeros stay zero. */

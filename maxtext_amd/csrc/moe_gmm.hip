@@ -8,9 +8,14 @@
 //                     row per accumulator quad and stores 8 bytes.  bf16 x {bf16, int8, int4}
 //                     weights run on v_mfma_f32_32x32x16_bf16 (weights are widened to bf16 while
 //                     they are copied into LDS), int8 x int8 on v_mfma_i32_32x32x32_i8.
+//                     Used for weight-only formats, small problems and K tails.
+//   gmm_dl_kernel     the prefill kernel for int8 x int8 and bf16 x bf16: persistent blocks, operands
+//                     copied global -> LDS without passing through registers, 4 stages in flight.
 //   gmm_fp8_skinny_kernel  block-scaled fp8 for few rows per expert (decode): no LDS, every wave
 //                     streams 16 weight rows through v_mfma_f32_16x16x128_f8f6f4 and applies the
 //                     per-128 K-block scales to the f32 partial sums.
+//   gmm_wq_skinny_kernel   the same streaming design for bf16 activations x int8 / int4 / mxfp4 weights,
+//                     with K split over the waves of a block.
 
 #include <type_traits>
 
@@ -125,7 +130,8 @@ struct TiledParams {
   int max_m_tiles, tiles_n;
   int act;
   float act_limit;
-  int dbg;  // timing experiments only: 1 = no barrier/wait, 2 = no loads in the loop
+  int tune;  // > 0: m-tiles per raster super-row of the persistent kernel (tuning aid; 0 = default)
+  int i4_group;  // values of K per int4 scale: 128 or 32
 };
 
 __device__ __forceinline__ uint32_t i8x2_to_bf16x2(int lo, int hi) {
@@ -260,8 +266,10 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
     m_idx = first_m + (logical % width) % gsz;
     n_idx = (logical % width) / gsz;
   }
-  if (m_idx >= p.header[0]) return;
+  // the slot exists even when the tile does not (the list is sized for the worst case): both loads go out
+  // together instead of one after the other
   const TileInfo tile = p.tiles[m_idx];
+  if (m_idx >= p.header[0]) return;
   const int n0 = n_idx * C::OUT_BN;
   const int N = p.N, K = p.K;
 
@@ -371,9 +379,9 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
               __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 3)));
       } else {  // BSRC_I4: 32 values of one 128-wide scale group
         const int kk = kt * C::BK + b_k[i];
-        const int nkg = (K + 127) / 128;
+        const int nkg = (K + p.i4_group - 1) / p.i4_group;
         const uint16_t* sc = (const uint16_t*)(b_up[i] ? p.rhs_up_scale : p.rhs_scale);
-        const float scale = kk < K ? bf16_bits_to_f32(sc[((size_t)tile.group * N + b_n[i]) * nkg + kk / 128]) : 0.f;
+        const float scale = kk < K ? bf16_bits_to_f32(sc[((size_t)tile.group * N + b_n[i]) * nkg + kk / p.i4_group]) : 0.f;
         const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
         uint32_t o[16];
 #pragma unroll
@@ -542,7 +550,7 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   auto locate = [&](int id, Tile& t) -> bool {
     const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
-    const int GSM = p.dbg > 0 ? p.dbg : 8;
+    const int GSM = p.tune > 0 ? p.tune : 8;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
     const int gsz = min(p.max_m_tiles - first_m, GSM);
@@ -779,8 +787,10 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int j = lane % 16, kq = lane / 16;
   const int m_idx = blockIdx.x / p.n_blocks;
-  if (m_idx >= p.header[0]) return;
+  // the slot exists even when the tile does not (the list is sized for the worst case): both loads go out
+  // together instead of one after the other
   const TileInfo tile = p.tiles[m_idx];
+  if (m_idx >= p.header[0]) return;
   if (tile.group >= 0 ? (tile.nrows < p.min_rows || tile.nrows > p.max_rows) : p.min_rows > 1) return;
   const int N = p.N, K = p.K;
   constexpr int WN = 16 * NT;  // channels per wave
@@ -928,7 +938,7 @@ struct WqSkinnyParams {
 };
 
 // Raw weight bytes of one lane for one 128-wide k block: 32 values = 16 bytes (int4) or 32 bytes (int8).
-enum { WQ_I8 = 0, WQ_I4 = 1, WQ_MX4 = 2 };  // weight formats of the streaming kernel
+enum { WQ_I8 = 0, WQ_I4 = 1, WQ_MX4 = 2, WQ_I4G32 = 3 };  // weight formats of the streaming kernel (int4: group 128 / 32)
 
 template <int FMT>
 struct WqRaw {
@@ -953,7 +963,7 @@ __device__ __forceinline__ void widen32(const WqRaw<FMT>& raw, float scale, v8bf
                                                  __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 1)),
                                                  __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 2)),
                                                  __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(x[s], scale, 3))));
-  } else if (FMT == WQ_I4) {
+  } else if (FMT == WQ_I4 || FMT == WQ_I4G32) {  // (nibble - 8) * scale rounded to bf16, as the reference dequantises
     const uint32_t x[4] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w};
 #pragma unroll
     for (int s = 0; s < 4; s++) {
@@ -989,7 +999,7 @@ __device__ __forceinline__ void widen32(const WqRaw<FMT>& raw, float scale, v8bf
 // latency (holding two rounds in registers halves the occupancy and measures slower).
 template <int FMT, int MT, int NT, bool GLU, int U, int KSPLIT>
 __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams p) {
-  constexpr bool INT4 = FMT == WQ_I4, MX4 = FMT == WQ_MX4, NIB = FMT != WQ_I8;
+  constexpr bool INT4 = FMT == WQ_I4, MX4 = FMT == WQ_MX4, G32 = FMT == WQ_I4G32, NIB = FMT != WQ_I8;
   constexpr int NACC = NT * MT * 4 * (GLU ? 2 : 1);
   constexpr int NSUB = 4 / KSPLIT;  // channel groups per block
   __shared__ float red[KSPLIT > 1 ? NSUB * (KSPLIT - 1) * NACC * kWave : 1];
@@ -998,8 +1008,10 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
   const int ksub = wave % KSPLIT, nsub = wave / KSPLIT;
   const int j = lane % 16, kq = lane / 16;
   const int m_idx = blockIdx.x / p.n_blocks;
-  if (m_idx >= p.header[0]) return;
+  // the slot exists even when the tile does not (the list is sized for the worst case): both loads go out
+  // together instead of one after the other
   const TileInfo tile = p.tiles[m_idx];
+  if (m_idx >= p.header[0]) return;
   const int N = p.N, K = p.K;
   constexpr int WN = 16 * NT;
   const int n_b = (blockIdx.x % p.n_blocks) * (NSUB * WN);
@@ -1034,6 +1046,11 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
     // MXFP4: one e8m0 byte per 32 values = per lane and k block
     wmx[t] = MX4 ? (const uint8_t*)p.rhs_scale + row * (size_t)(K / 32) + kq : nullptr;
     umx[t] = MX4 && GLU ? (const uint8_t*)p.rhs_up_scale + row * (size_t)(K / 32) + kq : nullptr;
+    // int4 with group 32: one bf16 scale per lane and k block, indexed like the MXFP4 byte
+    if (G32) {
+      wsp[t] = (const uint16_t*)p.rhs_scale + row * (size_t)(K / 32) + kq;
+      usp[t] = GLU ? (const uint16_t*)p.rhs_up_scale + row * (size_t)(K / 32) + kq : nullptr;
+    }
   }
   const uint8_t* ap[MT];
 #pragma unroll
@@ -1083,6 +1100,10 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
         if (MX4) {
           r.wsc[u][t] = addr_ok ? wmx[t][kb * 4] : (uint16_t)127;
           if (GLU) r.usc[u][t] = addr_ok ? umx[t][kb * 4] : (uint16_t)127;
+        }
+        if (G32) {
+          r.wsc[u][t] = addr_ok ? wsp[t][kb * 4] : (uint16_t)0;
+          if (GLU) r.usc[u][t] = addr_ok ? usp[t][kb * 4] : (uint16_t)0;
         }
       }
 #pragma unroll
@@ -1170,8 +1191,8 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 #pragma unroll
         for (int t = 0; t < NT; t++) {
           v8bf wf[4], uf[4];
-          widen32<FMT>(wraw[u][t], MX4 ? __uint_as_float((uint32_t)wsc[u][t] << 23) : 1.0f, wf);
-          if (GLU) widen32<FMT>(uraw[u][t], MX4 ? __uint_as_float((uint32_t)usc[u][t] << 23) : 1.0f, uf);
+          widen32<FMT>(wraw[u][t], MX4 ? __uint_as_float((uint32_t)wsc[u][t] << 23) : (G32 ? bf16_bits_to_f32(wsc[u][t]) : 1.0f), wf);
+          if (GLU) widen32<FMT>(uraw[u][t], MX4 ? __uint_as_float((uint32_t)usc[u][t] << 23) : (G32 ? bf16_bits_to_f32(usc[u][t]) : 1.0f), uf);
 #pragma unroll
           for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -1497,7 +1518,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   p.rhs_bias = a->rhs_bias; p.rhs_up_bias = a->rhs_up_bias;
   p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
   p.M = a->M; p.K = a->K; p.N = a->N; p.max_m_tiles = 0; p.tiles_n = 0;
-  p.act = a->act; p.act_limit = a->act_limit; p.dbg = a->reserved[1];
+  p.act = a->act; p.act_limit = a->act_limit; p.tune = a->reserved[1]; p.i4_group = a->rhs_scale_block_k == 32 ? 32 : 128;
 
   enum { V_NONE, V_BF16, V_W8, V_W4, V_I8, V_MX4 } variant = V_NONE;
   if (L == MOE_BF16 && R == MOE_BF16) {
@@ -1510,8 +1531,8 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     if (a->K % 16) return fail(MOE_ERR_UNSUPPORTED, "gmm: int8 weights need K %% 16 == 0");
     variant = V_W8;
   } else if (L == MOE_BF16 && R == MOE_INT4) {
-    if (!a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || a->rhs_scale_block_k != 128)
-      return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need bf16 group-128 scales [G, N, ceil(K/128)]");
+    if (!a->rhs_scale || (glu && !a->rhs_up_scale) || a->rhs_scale_block_n != 1 || (a->rhs_scale_block_k != 128 && a->rhs_scale_block_k != 32))
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need bf16 group scales [G, N, ceil(K/group)] with group 128 or 32");
     if (a->K % 32) return fail(MOE_ERR_UNSUPPORTED, "gmm: int4 weights need K %% 32 == 0");
     variant = V_W4;
   } else if (L == MOE_BF16 && R == MOE_MXFP4) {
@@ -1544,6 +1565,8 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     q.M = M; q.K = a->K; q.N = a->N; q.n_blocks = 0; q.act = a->act; q.act_limit = a->act_limit;
     const int mx = max_tiles_for(M, G, bm);
     const int kso = a->reserved[1];
+    if (variant == V_W4 && a->rhs_scale_block_k == 32)
+      return one ? launch_wq_skinny<WQ_I4G32, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_I4G32, 2>(q, glu, mx, kso, s);
     if (variant == V_W4) return one ? launch_wq_skinny<WQ_I4, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_I4, 2>(q, glu, mx, kso, s);
     if (variant == V_MX4) return one ? launch_wq_skinny<WQ_MX4, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_MX4, 2>(q, glu, mx, kso, s);
     return one ? launch_wq_skinny<WQ_I8, 1>(q, glu, mx, kso, s) : launch_wq_skinny<WQ_I8, 2>(q, glu, mx, kso, s);

@@ -54,10 +54,9 @@ def compressed_int4_experts(packed: Sequence[torch.Tensor], scales: Sequence[tor
   """compressed-tensors pack-quantized int4: int32 [N, K/8], weight k of a word in bits [4k, 4k+4), stored value + 8,
   symmetric group scales [N, K/group] (convert_deepseek_family_ckpt.py:56-84).  Read as little-endian bytes this is
   the kernels' packing (two values per byte, first in the low nibble), so the values are a view; the scales are
-  cast to bf16.  Only group_size 128 matches the kernels' scale granularity."""
-  if group_size != 128:
-    raise NotImplementedError(f"int4 group size {group_size}: the kernels apply one scale per 128 values of K "
-                              "(group 32 checkpoints need their scales regrouped, which is not lossless)")
+  cast to bf16.  group_size 128 or 32 (INT4_GROUP_SIZE of the Kimi-K2 variants, convert_deepseek_family_ckpt.py:51-53)."""
+  if group_size not in (32, 128):
+    raise NotImplementedError(f"int4 group size {group_size}: the kernels apply one scale per 32 or 128 values of K")
   qs, ss = [], []
   for p, s, shape in zip(packed, scales, shapes):
     n, k = int(shape[0]), int(shape[1])
@@ -65,11 +64,11 @@ def compressed_int4_experts(packed: Sequence[torch.Tensor], scales: Sequence[tor
       raise ValueError(f"weight_packed must be int32 [{n}, {(k + 7) // 8}], got {p.dtype} {tuple(p.shape)}")
     if k % 32:
       raise ValueError("K must be a multiple of 32")
-    if tuple(s.shape) != (n, (k + 127) // 128):
-      raise ValueError(f"weight_scale must be [{n}, {(k + 127) // 128}]")
+    if tuple(s.shape) != (n, (k + group_size - 1) // group_size):
+      raise ValueError(f"weight_scale must be [{n}, {(k + group_size - 1) // group_size}]")
     qs.append(p.contiguous().view(torch.uint8)[:, : k // 2])
     ss.append(s.to(torch.bfloat16))
-  return QArray(torch.stack(qs).contiguous(), torch.stack(ss).contiguous(), "int4")
+  return QArray(torch.stack(qs).contiguous(), torch.stack(ss).contiguous(), "int4" if group_size == 128 else "int4g32")
 
 
 def mxfp4_experts(blocks: torch.Tensor, scales: torch.Tensor) -> QArray:

@@ -224,7 +224,7 @@ def transpose_rhs(rhs_gkn):
 
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
-            group_offset=0, out=None, tile_variant=0, rhs_bias=None, rhs_up_bias=None):
+            group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2])."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
@@ -294,7 +294,7 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.rhs_bias = rhs_bias.data_ptr() if rhs_bias is not None else None
   a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
   a.reserved[0] = int(tile_variant)
-  a.reserved[1] = int(__import__("os").environ.get("MOE_DBG", "0"))
+  a.reserved[1] = int(tune)
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
   _lib.check(st, "moe_gmm")
   return out

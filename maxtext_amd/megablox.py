@@ -164,6 +164,8 @@ def gmm(
       kw.update(rhs_scale_block_n=128, rhs_scale_block_k=128)
     elif rhs_n.qtype == "int4":
       kw.update(rhs_scale_block_n=1, rhs_scale_block_k=128, rhs_dtype=MOE_INT4)
+    elif rhs_n.qtype == "int4g32":
+      kw.update(rhs_scale_block_n=1, rhs_scale_block_k=32, rhs_dtype=MOE_INT4)
     elif rhs_n.qtype == "mxfp4":
       kw.update(rhs_scale_block_n=1, rhs_scale_block_k=32, rhs_dtype=MOE_MXFP4)
     else:

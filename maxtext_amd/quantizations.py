@@ -29,7 +29,7 @@ class QArray:
   """Quantised tensor: values plus scales (the role qwix.pallas.QArray plays in ops.py:232-267).
 
   For expert weights `qvalue` is [G, N, K] (K contiguous; INT4: uint8 [G, N, K/2]) and `scale`
-  has the layout described in the module docstring; `qtype` is "int8" | "fp8" | "int4" | "mxfp4"
+  has the layout described in the module docstring; `qtype` is "int8" | "fp8" | "int4" | "int4g32" | "mxfp4"
   (mxfp4: uint8 [G, N, K/2] e2m1 pairs and uint8 [G, N, K/32] e8m0 block scales).
   For activations `qvalue` is [M, K] and `scale` is [M] (int8) or [M, ceil(K/128)] (fp8).
   """
@@ -100,7 +100,7 @@ def quantize_weight_int4(w_gnk: torch.Tensor, group: int = 128) -> QArray:
   q = torch.round(wg / scale.to(torch.float32)).clamp(-8, 7).to(torch.int16).view(g, n, ng * group)[:, :, :k]
   u = (q + 8).to(torch.uint8)
   packed = (u[..., 0::2] | (u[..., 1::2] << 4)).contiguous()
-  return QArray(packed, scale.squeeze(-1).contiguous(), "int4")
+  return QArray(packed, scale.squeeze(-1).contiguous(), "int4" if group == 128 else f"int4g{group}")
 
 
 def quantize_weight_mxfp4(w_gnk: torch.Tensor) -> QArray:

@@ -55,7 +55,13 @@ def test_compressed_int4_bytes_are_the_kernel_packing():
   ones = torch.full((1, 4), -1, dtype=torch.int32)
   assert torch.all(O.unpack_int4(formats.compressed_int4_experts([ones], [torch.ones(1, 1)], [(1, 32)]).qvalue[0]) == 7)
   with pytest.raises(NotImplementedError):
-    formats.compressed_int4_experts([packed], [scale], [(n, k)], group_size=32)
+    formats.compressed_int4_experts([packed], [scale], [(n, k)], group_size=64)
+  # group 32 (INT4_GROUP_SIZE of the Kimi-K2 variants, convert_deepseek_family_ckpt.py:51-53)
+  scale32 = torch.tensor(rng.random((n, k // 32)) + 0.5, dtype=torch.bfloat16)
+  qa32 = formats.compressed_int4_experts([packed], [scale32], [(n, k)], group_size=32)
+  assert qa32.qtype == "int4g32" and qa32.scale.shape == (1, n, k // 32)
+  want32 = torch.from_numpy(w).float().reshape(n, k // 32, 32) * scale32.float()[..., None]
+  assert torch.equal(O.dequantize_int4(qa32.qvalue[0], qa32.scale[0], 32), want32.reshape(n, k).to(torch.bfloat16))
 
 
 def test_gpt_oss_mxfp4_deinterleave_matches_dequantised_split():

@@ -882,3 +882,27 @@ def test_tgmm_random_shapes(K):
         assert torch.all(got[i] == 0), tag
       else:
         assert relerr(got[i], want[i]) <= TOL, tag
+
+
+@pytest.mark.parametrize("m,k,n,gs", DECODE_SHAPES + [GMM_SHAPES[0], GMM_SHAPES[3]])
+def test_gmm_int4_group32(K, m, k, n, gs):
+  """int4 with one scale per 32 values (Kimi-K2 checkpoints): the reference dequantises to bf16 first
+  (convert_deepseek_family_ckpt.py:56-84), so the oracle is its bf16 gmm on dequantize_int4(..., 32)."""
+  from maxtext_amd._lib import MOE_INT4
+
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 80)
+  q, s = O.quantize_int4_groups(native(w), 32)
+  qu, su = O.quantize_int4_groups(native(w_up), 32)
+  s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
+  pq, pu = O.pack_int4(q), O.pack_int4(qu)
+  deq, udeq = O.dequantize_int4(pq, s, 32), O.dequantize_int4(pu, su, 32)  # [g, n, k] bf16
+  kw = dict(rhs_dtype=MOE_INT4, rhs_scale_block_k=32)
+  got = K.gmm_raw(cuda(lhs), cuda(pq), cuda(gs), rhs_scale=cuda(s), **kw)
+  assert relerr(got, O.gmm(lhs, deq, gs, transpose_rhs=True)) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  want = O.apply_ffn_activation(O.gmm(lhs, deq, gs, transpose_rhs=True, out_dtype=torch.float32),
+                                O.gmm(lhs, udeq, gs, transpose_rhs=True, out_dtype=torch.float32))
+  got = K.gmm_raw(cuda(lhs), cuda(pq), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(pu), rhs_up_scale=cuda(su), act="silu", **kw)
+  assert relerr(got, want) <= TOL
+  tiled = K.gmm_raw(cuda(lhs), cuda(pq), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(pu), rhs_up_scale=cuda(su), act="silu", tile_variant=1, **kw)
+  assert relerr(tiled, want) <= TOL
