@@ -107,6 +107,47 @@ def cpu_baseline(wl, layer, sample_tokens):
               seconds=dt)
 
 
+def calibration(dtype_name):
+  """What this machine sustains on the two roofs, measured with the library's calibration kernels: a register-only
+  MFMA loop (operands constant / changing every instruction: changing data draws more power and lowers the clock)
+  and a plain streaming read of 2 GiB.  Reported beside the roofline, whose `peak` stays the published figure."""
+  import torch
+
+  from maxtext_amd import _lib
+
+  lib = _lib.load()
+  stream = _lib.current_stream()
+  scratch = torch.empty((lib.moe_calib_scratch_bytes(),), dtype=torch.uint8, device="cuda")
+
+  def best_ms(fn, reps=3):
+    fn()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(reps):
+      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      a.record()
+      fn()
+      b.record()
+      torch.cuda.synchronize()
+      out.append(a.elapsed_time(b))
+    return min(out)
+
+  res = {}
+  code = _lib.MOE_INT8 if dtype_name in ("int8", "fp8") else _lib.MOE_BF16
+  iters = 4000
+  ops = lib.moe_calib_mfma_ops(code, iters)
+  for key, rnd in (("mfma_constant_operands", 0), ("mfma_changing_operands", 1)):
+    ms = best_ms(lambda: _lib.check(lib.moe_calib_mfma(code, rnd, iters, _lib.ptr(scratch), stream), "moe_calib_mfma"))
+    res[key] = ops / ms / 1e9
+  res["mfma_unit"] = "TOP/s int8 (v_mfma_i32_32x32x32_i8)" if code == _lib.MOE_INT8 else "TFLOP/s bf16 (v_mfma_f32_32x32x16_bf16)"
+  buf = torch.empty((1 << 31,), dtype=torch.uint8, device="cuda")
+  buf.fill_(1)
+  ms = best_ms(lambda: _lib.check(lib.moe_calib_read(_lib.ptr(buf), buf.numel(), _lib.ptr(scratch), stream), "moe_calib_read"))
+  res["hbm_read_gbs"] = buf.numel() / ms / 1e6
+  del buf
+  return res
+
+
 def train_cpu_baseline(wl, sample_tokens):
   """Forward + backward of the three grouped GEMMs with the oracle's gmm / tgmm (torch CPU, f32 results)
   on `sample_tokens` tokens spread evenly over the experts: a reported baseline."""
@@ -202,6 +243,7 @@ def train_main(args):
                        kernel="tgmm_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
       "stage_ms": stage_ms,
   }
+  result["calibration"] = calibration("bf16")
   if not args.no_cpu_baseline:
     result["cpu_baseline"] = train_cpu_baseline(wl, args.cpu_sample_tokens or 1024)
   print(json.dumps(result))
@@ -334,6 +376,7 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
+  result["calibration"] = calibration(model["dtype"])
   if not args.no_cpu_baseline:
     sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048, "c5mx": 2048}[wl.name]
     del out

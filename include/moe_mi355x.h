@@ -285,6 +285,19 @@ MOE_API int moe_glu_act(const void* h0, const void* h1, size_t n, int act, float
 MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, size_t n, int act, float act_limit,
                             void* dh0, void* dh1, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Calibration (no counterpart in the reference; used by the benchmark): what this machine sustains with a
+ * register-only MFMA loop, with constant operands or operands that change every instruction (random data makes
+ * the chip draw more power and lower its clock), and with a plain streaming read.  The caller times the launches.
+ *   moe_calib_mfma: dtype MOE_INT8 (v_mfma_i32_32x32x32_i8) or MOE_BF16 (v_mfma_f32_32x32x16_bf16); the launch
+ *   performs moe_calib_mfma_ops(dtype, iters) operations.  scratch: moe_calib_scratch_bytes() bytes.
+ *   moe_calib_read: reads `bytes` (16-byte aligned, >= 64 KiB) once.
+ */
+MOE_API size_t moe_calib_scratch_bytes(void);
+MOE_API double moe_calib_mfma_ops(int dtype, int iters);
+MOE_API int moe_calib_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream);
+MOE_API int moe_calib_read(const void* src, size_t bytes, void* scratch, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
