@@ -345,59 +345,88 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
     }
   };
 
-  auto store_stage = [&](int buf, int kt) {
+  // single-chunk versions: MODE 1 = full stage, 2 = the stage that holds the K tail
+  auto load_a_chunk = [&](int kt, int i, auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
+    const int k0 = kt * C::BK;
+    if constexpr (MODE == 1) {
+      a_reg[i] = *(const uint4*)(a_ptr[i] + (size_t)k0 * C::ESZ);
+    } else {
+      const bool ok = k0 + a_k[i] < K;
+      const uint4 v = *(const uint4*)(a_ptr[i] + (ok ? (size_t)k0 * C::ESZ : 0));
+      const uint32_t m = ok ? 0xffffffffu : 0u;
+      a_reg[i] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+    }
+  };
+  auto load_b_chunk = [&](int kt, int i, auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
+    const int k0 = kt * C::BK;
+    if constexpr (MODE == 1) {
+      b_reg[i] = *(const uint4*)(b_ptr[i] + (size_t)k0 * B_GSZ / 2);
+    } else {
+      const bool ok = k0 + b_k[i] < K;
+      const uint4 v = *(const uint4*)(b_ptr[i] + (ok ? (size_t)k0 * B_GSZ / 2 : 0));
+      const uint32_t z = C::BSRC == BSRC_I4 ? 0x88888888u : 0u;
+      b_reg[i] = ok ? v : make_uint4(z, z, z, z);
+    }
+  };
+
+  auto store_a_chunk = [&](int buf, int i) {
     uint8_t* s = smem + buf * C::STAGE;
-#pragma unroll
-    for (int i = 0; i < C::A_CH; i++) *(uint4*)(s + a_lds[i]) = a_reg[i];
-#pragma unroll
-    for (int i = 0; i < C::B_CH; i++) {
-      if (C::BSRC == BSRC_SAME) {
-        *(uint4*)(s + b_lds[i]) = b_reg[i];
-      } else if (C::BSRC == BSRC_I8) {
-        const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
-        uint32_t o[8];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          int v = (int)w[j];
-          o[2 * j] = i8x2_to_bf16x2((v << 24) >> 24, (v << 16) >> 24);
-          o[2 * j + 1] = i8x2_to_bf16x2((v << 8) >> 24, v >> 24);
-        }
-        *(uint4*)(s + b_lds[i]) = make_uint4(o[0], o[1], o[2], o[3]);
-        *(uint4*)(s + b_lds[i] + 16) = make_uint4(o[4], o[5], o[6], o[7]);
-      } else if (C::BSRC == BSRC_MX4) {  // 32 e2m1 values = one MX block with its e8m0 scale 2^(s - 127)
+    *(uint4*)(s + a_lds[i]) = a_reg[i];
+  };
+  // A weight chunk is converted and stored in 4 parts (one 32-bit word of the staged register each), so that the
+  // conversions can be spread over the k sub-steps of a stage.  The chunk's scale is fetched with part 0.
+  float b_scale[C::B_CH];
+  auto store_b_part = [&](int buf, int kt, int i, int part) {
+    uint8_t* s = smem + buf * C::STAGE;
+    const uint32_t w4[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
+    const uint32_t w = w4[part];
+    if (C::BSRC == BSRC_SAME) {  // nothing to convert: one 16-byte store with the last part
+      if (part == 3) *(uint4*)(s + b_lds[i]) = b_reg[i];
+    } else if (C::BSRC == BSRC_I8) {  // 4 int8 -> 4 bf16
+      const int v = (int)w;
+      *(uint2*)(s + b_lds[i] + 8 * part) = make_uint2(i8x2_to_bf16x2((v << 24) >> 24, (v << 16) >> 24), i8x2_to_bf16x2((v << 8) >> 24, v >> 24));
+    } else if (C::BSRC == BSRC_MX4) {  // 8 e2m1 values of an MX block with its e8m0 scale 2^(s - 127)
+      if (part == 0) {
         const int kk = kt * C::BK + b_k[i];
         const uint8_t* sc = (const uint8_t*)(b_up[i] ? p.rhs_up_scale : p.rhs_scale);
         const uint32_t sbyte = kk < K ? sc[((size_t)tile.group * N + b_n[i]) * (K / 32) + kk / 32] : 127u;
-        const float scale = __uint_as_float(sbyte << 23);
-        const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-          *(uint4*)(s + b_lds[i] + 16 * j) = make_uint4(
-              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 0)),
-              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 1)),
-              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 2)),
-              __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[j], scale, 3)));
-      } else {  // BSRC_I4: 32 values of one 128-wide scale group
+        b_scale[i] = __uint_as_float(sbyte << 23);
+      }
+      const float scale = b_scale[i];
+      *(uint4*)(s + b_lds[i] + 16 * part) = make_uint4(
+          __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 0)),
+          __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 1)),
+          __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 2)),
+          __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 3)));
+    } else {  // BSRC_I4: 8 values of one scale group (128 or 32 wide)
+      if (part == 0) {
         const int kk = kt * C::BK + b_k[i];
         const int nkg = (K + p.i4_group - 1) / p.i4_group;
         const uint16_t* sc = (const uint16_t*)(b_up[i] ? p.rhs_up_scale : p.rhs_scale);
-        const float scale = kk < K ? bf16_bits_to_f32(sc[((size_t)tile.group * N + b_n[i]) * nkg + kk / p.i4_group]) : 0.f;
-        const uint32_t w[4] = {b_reg[i].x, b_reg[i].y, b_reg[i].z, b_reg[i].w};
-        uint32_t o[16];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-#pragma unroll
-          for (int h = 0; h < 4; h++) {
-            int lo = (int)((w[j] >> (8 * h)) & 0xf) - 8;
-            int hi = (int)((w[j] >> (8 * h + 4)) & 0xf) - 8;
-            o[4 * j + h] = pack_bf16x2((float)lo * scale, (float)hi * scale);
-          }
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-          *(uint4*)(s + b_lds[i] + 16 * j) = make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+        b_scale[i] = kk < K ? bf16_bits_to_f32(sc[((size_t)tile.group * N + b_n[i]) * nkg + kk / p.i4_group]) : 0.f;
       }
+      const float scale = b_scale[i];
+      uint32_t o[4];
+#pragma unroll
+      for (int h = 0; h < 4; h++) {
+        const int lo = (int)((w >> (8 * h)) & 0xf) - 8;
+        const int hi = (int)((w >> (8 * h + 4)) & 0xf) - 8;
+        o[h] = pack_bf16x2((float)lo * scale, (float)hi * scale);
+      }
+      *(uint4*)(s + b_lds[i] + 16 * part) = make_uint4(o[0], o[1], o[2], o[3]);
     }
+  };
+  auto store_b_chunk = [&](int buf, int kt, int i) {
+#pragma unroll
+    for (int part = 0; part < 4; part++) store_b_part(buf, kt, i, part);
+  };
+  auto store_stage = [&](int buf, int kt) {
+#pragma unroll
+    for (int i = 0; i < C::A_CH; i++) store_a_chunk(buf, i);
+#pragma unroll
+    for (int i = 0; i < C::B_CH; i++) store_b_chunk(buf, kt, i);
   };
 
   // ---- accumulators ---------------------------------------------------------------------
@@ -449,6 +478,59 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
     }
   };
 
+  // MFMAs of the stage in `buf` with, after each k sub-step, a share of the register -> LDS stores (and weight
+  // conversions) of stage kt_store into the other buffer; every register is refilled right after its store with
+  // the same chunk of the stage after that (LOAD: 0 none, 1 full stage, 2 the stage holding the K tail), so a
+  // load has a whole stage of MFMAs to land and the stores ride in the shadow of the MFMAs instead of forming a
+  // phase of their own before the barrier.
+  auto compute_and_store = [&](int buf, int kt_store, auto store_c, auto load_c) {
+    constexpr bool STORE = decltype(store_c)::value;
+    constexpr int LOAD = decltype(load_c)::value;
+    const uint8_t* sa = smem + buf * C::STAGE + (wm * C::WM) * C::LDR + frag_off;
+    const uint8_t* sb = smem + buf * C::STAGE + C::BM * C::LDR + frag_off;
+    constexpr int A_PER = (C::A_CH + C::KSUB - 1) / C::KSUB;
+#pragma unroll
+    for (int ks = 0; ks < C::KSUB; ks++) {
+      v4i af[C::TM], bf[C::TN];
+#pragma unroll
+      for (int i = 0; i < C::TM; i++) af[i] = *(const v4i*)(sa + i * 32 * C::LDR + ks * 32);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) bf[j] = *(const v4i*)(sb + b_row[j] * C::LDR + ks * 32);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int i = 0; i < C::TM; i++) {
+          if constexpr (OP == OP_I8) {
+            acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
+          } else {
+            acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(v8bf, bf[j]), __builtin_bit_cast(v8bf, af[i]), acc[j][i], 0, 0, 0);
+          }
+        }
+      if constexpr (STORE) {
+#pragma unroll
+        for (int c = 0; c < A_PER; c++) {
+          const int i = ks * A_PER + c;
+          if (i < C::A_CH) {
+            store_a_chunk(buf ^ 1, i);
+            if constexpr (LOAD != 0) load_a_chunk(kt_store + 1, i, load_c);
+          }
+        }
+        // part ks of every weight chunk; the register is refilled after its last part
+        static_assert(C::KSUB == 4 || C::KSUB == 2, "weight chunks are stored in KSUB or 2 * KSUB parts");
+#pragma unroll
+        for (int i = 0; i < C::B_CH; i++) {
+#pragma unroll
+          for (int q = 0; q < 4 / C::KSUB; q++) store_b_part(buf ^ 1, kt_store, i, ks * (4 / C::KSUB) + q);
+          if (ks == C::KSUB - 1) {
+            if constexpr (LOAD != 0) load_b_chunk(kt_store + 1, i, load_c);
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
   // ---- main loop: one barrier per stage --------------------------------------------------
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
   const int n_out0 = n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
@@ -459,22 +541,29 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
   // loaded in a peeled iteration so its masking code never merges into the loop body.
   const int nk = (K + C::BK - 1) / C::BK;
   const bool k_tail = (K % C::BK) != 0;
+  const int full = k_tail ? nk - 1 : nk;  // stages 0 .. full-1 need no masking
+  using L0 = std::integral_constant<int, 0>;
+  using L1 = std::integral_constant<int, 1>;
+  using L2 = std::integral_constant<int, 2>;
   if (nk == 1 && k_tail) load_stage_tail(0); else load_stage(0);
   store_stage(0, 0);
+  if (nk > 1) {
+    if (nk == 2 && k_tail) load_stage_tail(1); else load_stage(1);
+  }
   __syncthreads();
+  // Steady state: stage kt is computed, stage kt+1 moves from registers to LDS, stage kt+2 (a full one) is requested.
   int kt = 0;
-  for (; kt + 2 < nk; kt++) {
-    load_stage(kt + 1);
-    __builtin_amdgcn_sched_barrier(0);  // keep the prefetch above the MFMAs: it needs their time to land
-    compute_stage(kt & 1);
-    __builtin_amdgcn_sched_barrier(0);
-    store_stage((kt & 1) ^ 1, kt + 1);
+  for (; kt + 2 < full; kt++) {
+    compute_and_store(kt & 1, kt + 1, std::true_type{}, L1{});
     __syncthreads();
   }
+  if (kt + 2 < nk) {  // the stage after next is the one with the K tail
+    compute_and_store(kt & 1, kt + 1, std::true_type{}, L2{});
+    __syncthreads();
+    kt++;
+  }
   if (kt + 1 < nk) {
-    if (k_tail) load_stage_tail(kt + 1); else load_stage(kt + 1);
-    compute_stage(kt & 1);
-    store_stage((kt & 1) ^ 1, kt + 1);
+    compute_and_store(kt & 1, kt + 1, std::true_type{}, L0{});
     __syncthreads();
     kt++;
   }
