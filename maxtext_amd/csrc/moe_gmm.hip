@@ -551,20 +551,23 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
     if (nk == 2 && k_tail) load_stage_tail(1); else load_stage(1);
   }
   __syncthreads();
+  // LDS writes of this wave done, then the barrier; not __syncthreads(), whose fence would also wait for the global
+  // loads that were just issued for the stage after next
+  auto stage_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
   // Steady state: stage kt is computed, stage kt+1 moves from registers to LDS, stage kt+2 (a full one) is requested.
   int kt = 0;
   for (; kt + 2 < full; kt++) {
     compute_and_store(kt & 1, kt + 1, std::true_type{}, L1{});
-    __syncthreads();
+    stage_barrier();
   }
   if (kt + 2 < nk) {  // the stage after next is the one with the K tail
     compute_and_store(kt & 1, kt + 1, std::true_type{}, L2{});
-    __syncthreads();
+    stage_barrier();
     kt++;
   }
   if (kt + 1 < nk) {
     compute_and_store(kt & 1, kt + 1, std::true_type{}, L0{});
-    __syncthreads();
+    stage_barrier();
     kt++;
   }
   compute_stage(kt & 1);
