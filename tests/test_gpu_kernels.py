@@ -2,7 +2,7 @@
 
 Index outputs (top-k indices, perm, group_sizes, sorted_experts, quantised values) are compared
 bit-exactly; floating-point outputs with max|got-want| / max|want| <= 1e-2 (bf16 outputs, f32
-accumulation), the tolerance BASELINE.json states.
+accumulation), the tolerance this path is specified to.
 """
 
 import numpy as np
