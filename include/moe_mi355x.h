@@ -207,6 +207,11 @@ typedef struct {
    * pallas_mosaic_tpu_v2_gmm_kernel.py:573).  NULL = no bias.  Rows that are written as zeros stay zero. */
   const float* rhs_bias;
   const float* rhs_up_bias;
+  /* [M, N] bf16 or NULL: added to lhs@rhs^T (to lhs@rhs_up^T) after the bias and before the activation, for rows
+   * of local groups only: partial_sum of ops.py:77 / pallas_mosaic_tpu_v2_gmm_kernel.py:576-578, used by the
+   * embedding-chunked expert MLP (moe.py:1962-1980).  Must not alias `out`. */
+  const void* partial_sum;
+  const void* partial_sum_up;
 } moe_gmm_args;
 
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);

@@ -53,6 +53,8 @@ class GmmArgs(ctypes.Structure):
       ("reserved", ctypes.c_int32 * 4),
       ("rhs_bias", c_void_p),
       ("rhs_up_bias", c_void_p),
+      ("partial_sum", c_void_p),
+      ("partial_sum_up", c_void_p),
   ]
 
 

@@ -123,6 +123,8 @@ struct TiledParams {
   const void* rhs_up_scale;
   const float* rhs_bias;     // [G, N] f32 or NULL, added before the activation
   const float* rhs_up_bias;
+  const uint16_t* partial_sum;     // [M, N] bf16 or NULL, added like the bias
+  const uint16_t* partial_sum_up;
   const int32_t* header;
   const TileInfo* tiles;
   uint16_t* out;  // [M, N] bf16
@@ -145,6 +147,17 @@ __device__ __forceinline__ void load_bias4(const float* bias, int group, int N, 
   if (bias) {
     const float4 v = *(const float4*)(bias + (size_t)group * N + n);
     b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
+  }
+}
+
+// b += 4 consecutive bf16 values of row `row` of a [M, N] partial-sum matrix (nothing without one).
+__device__ __forceinline__ void add_partial4(const uint16_t* ps, size_t row, int N, int n, float (&b)[4]) {
+  if (ps) {
+    const uint2 v = *(const uint2*)(ps + row * N + n);
+    b[0] += bf16_bits_to_f32((uint16_t)(v.x & 0xffff));
+    b[1] += bf16_bits_to_f32((uint16_t)(v.x >> 16));
+    b[2] += bf16_bits_to_f32((uint16_t)(v.y & 0xffff));
+    b[3] += bf16_bits_to_f32((uint16_t)(v.y >> 16));
   }
 }
 
@@ -201,6 +214,8 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
         float bg[4], bu[4];
         load_bias4(p.rhs_bias, tile.group, p.N, n, bg);
         load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, p.N, n, bu);
+        add_partial4(p.partial_sum, (size_t)(tile.row0 + lr), p.N, n, bg);
+        add_partial4(GLU ? p.partial_sum_up : nullptr, (size_t)(tile.row0 + lr), p.N, n, bu);
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -854,6 +869,8 @@ struct SkinnyParams {
   const float* rhs_up_scale;
   const float* rhs_bias;   // [G, N] f32 or NULL
   const float* rhs_up_bias;
+  const uint16_t* partial_sum;     // [M, N] bf16 or NULL, added like the bias
+  const uint16_t* partial_sum_up;
   const int32_t* header;
   const TileInfo* tiles;
   uint16_t* out;
@@ -993,10 +1010,13 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
       for (int mt = 0; mt < MT; mt++) {
         const int lr = mt * 16 + j;
         if (lr >= tile.nrows) continue;
+        float pg[4] = {bg[0], bg[1], bg[2], bg[3]}, pu[4] = {bu[0], bu[1], bu[2], bu[3]};
+        add_partial4(p.partial_sum, (size_t)(tile.row0 + lr), N, n, pg);
+        add_partial4(GLU ? p.partial_sum_up : nullptr, (size_t)(tile.row0 + lr), N, n, pu);
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r] + bg[r], acc_u[t][mt][r] + bu[r], p.act_limit) : acc_g[t][mt][r] + bg[r];
+          v[r] = GLU ? glu_act<ACT>(acc_g[t][mt][r] + pg[r], acc_u[t][mt][r] + pu[r], p.act_limit) : acc_g[t][mt][r] + pg[r];
         *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
       }
     }
@@ -1020,6 +1040,8 @@ struct WqSkinnyParams {
   const void* rhs_up_scale;
   const float* rhs_bias;    // [G, N] f32 or NULL
   const float* rhs_up_bias;
+  const uint16_t* partial_sum;     // [M, N] bf16 or NULL, added like the bias
+  const uint16_t* partial_sum_up;
   const int32_t* header;
   const TileInfo* tiles;
   uint16_t* out;
@@ -1361,11 +1383,14 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
       for (int mt = 0; mt < MT; mt++) {
         const int lr = mt * 16 + j;
         if (lr >= tile.nrows) continue;
+        float pg[4] = {bg[0], bg[1], bg[2], bg[3]}, pu[4] = {bu[0], bu[1], bu[2], bu[3]};
+        add_partial4(p.partial_sum, (size_t)(tile.row0 + lr), N, n, pg);
+        add_partial4(GLU ? p.partial_sum_up : nullptr, (size_t)(tile.row0 + lr), N, n, pu);
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++)
-          v[r] = GLU ? glu_act<ACT>(fmaf(acc_g[t][mt][r], sg[r], bg[r]), fmaf(acc_u[t][mt][r], su[r], bu[r]), p.act_limit)
-                     : fmaf(acc_g[t][mt][r], sg[r], bg[r]);
+          v[r] = GLU ? glu_act<ACT>(fmaf(acc_g[t][mt][r], sg[r], pg[r]), fmaf(acc_u[t][mt][r], su[r], pu[r]), p.act_limit)
+                     : fmaf(acc_g[t][mt][r], sg[r], pg[r]);
         *(uint2*)(p.out + (size_t)(tile.row0 + lr) * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
       }
     }
@@ -1566,6 +1591,9 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   if (a->act < MOE_ACT_NONE || a->act > MOE_ACT_SILU_CLIP) return fail(MOE_ERR_INVALID_ARG, "gmm: bad act %d", a->act);
   if (a->N % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: N %% 8 != 0 (N=%d)", a->N);
   if (a->rhs_up_bias && !glu) return fail(MOE_ERR_INVALID_ARG, "gmm: rhs_up_bias needs rhs_up");
+  if (a->partial_sum_up && !glu) return fail(MOE_ERR_INVALID_ARG, "gmm: partial_sum_up needs rhs_up");
+  if (((uintptr_t)a->partial_sum | (uintptr_t)a->partial_sum_up) & 7) return fail(MOE_ERR_UNSUPPORTED, "gmm: partial sums must be 8-byte aligned");
+  if (a->partial_sum == a->out || a->partial_sum_up == a->out) return fail(MOE_ERR_INVALID_ARG, "gmm: partial sums must not alias out");
   if (((uintptr_t)a->rhs_bias | (uintptr_t)a->rhs_up_bias) & 15) return fail(MOE_ERR_UNSUPPORTED, "gmm: bias pointers must be 16-byte aligned");
   if (a->M == 0) return MOE_OK;
   const uintptr_t align = (uintptr_t)a->lhs | (uintptr_t)a->rhs | (uintptr_t)a->rhs_up | (uintptr_t)a->out |
@@ -1594,6 +1622,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
     p.rhs_scale = (const float*)a->rhs_scale; p.rhs_up_scale = (const float*)a->rhs_up_scale;
     p.rhs_bias = a->rhs_bias; p.rhs_up_bias = a->rhs_up_bias;
+    p.partial_sum = (const uint16_t*)a->partial_sum; p.partial_sum_up = (const uint16_t*)a->partial_sum_up;
     p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
     p.M = a->M; p.K = a->K; p.N = a->N; p.n_blocks = 0;
     p.act = a->act; p.act_limit = a->act_limit;
@@ -1608,6 +1637,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
   p.rhs_scale = a->rhs_scale; p.rhs_up_scale = a->rhs_up_scale;
   p.rhs_bias = a->rhs_bias; p.rhs_up_bias = a->rhs_up_bias;
+  p.partial_sum = (const uint16_t*)a->partial_sum; p.partial_sum_up = (const uint16_t*)a->partial_sum_up;
   p.header = header; p.tiles = tiles; p.out = (uint16_t*)a->out;
   p.M = a->M; p.K = a->K; p.N = a->N; p.max_m_tiles = 0; p.tiles_n = 0;
   p.act = a->act; p.act_limit = a->act_limit; p.tune = a->reserved[1]; p.i4_group = a->rhs_scale_block_k == 32 ? 32 : 128;
@@ -1653,6 +1683,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
     q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
     q.rhs_bias = a->rhs_bias; q.rhs_up_bias = a->rhs_up_bias;
+    q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
     q.header = header; q.tiles = tiles; q.out = (uint16_t*)a->out;
     q.M = M; q.K = a->K; q.N = a->N; q.n_blocks = 0; q.act = a->act; q.act_limit = a->act_limit;
     const int mx = max_tiles_for(M, G, bm);

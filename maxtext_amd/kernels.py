@@ -224,7 +224,7 @@ def transpose_rhs(rhs_gkn):
 
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
-            group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None):
+            group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2])."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
@@ -262,6 +262,13 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
         raise ValueError(f"{name} must be [{g_local}, {n}] f32")
   if rhs_up_bias is not None and rhs_up is None:
     raise ValueError("rhs_up_bias needs rhs_up")
+  for name, t in (("partial_sum", partial_sum), ("partial_sum_up", partial_sum_up)):
+    if t is not None:
+      _need(t, name, torch.bfloat16, 2)
+      if t.shape != (m, n):
+        raise ValueError(f"{name} must be [{m}, {n}] bf16")
+  if partial_sum_up is not None and rhs_up is None:
+    raise ValueError("partial_sum_up needs rhs_up")
   if lhs_scale is not None:
     _need(lhs_scale, "lhs_scale", torch.float32)
     nkb_l = 1 if lhs_scale_block_k == 0 else (kdim + lhs_scale_block_k - 1) // lhs_scale_block_k
@@ -293,6 +300,8 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.act_limit = float(act_limit)
   a.rhs_bias = rhs_bias.data_ptr() if rhs_bias is not None else None
   a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
+  a.partial_sum = partial_sum.data_ptr() if partial_sum is not None else None
+  a.partial_sum_up = partial_sum_up.data_ptr() if partial_sum_up is not None else None
   a.reserved[0] = int(tile_variant)
   a.reserved[1] = int(tune)
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())

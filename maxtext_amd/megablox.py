@@ -9,7 +9,8 @@ lhs_quantize_dtype / rhs_quantize_dtype ask for it.
 Extra keyword arguments the quantised expert path needs (they follow gmm_v2,
 pallas_mosaic_tpu_v2_gmm_kernel.py:1297-1315): `rhs_up` (second projection, fused
 act(lhs@rhs) * (lhs@rhs_up)), `fuse_act`, and `rhs_bias` / `rhs_up_bias` ([G, N] per-expert biases
-added before the activation).
+added before the activation) and `partial_sum_up` (the partial sum of the second projection; `partial_sum` is the
+reference's own argument).
 """
 
 from __future__ import annotations
@@ -100,6 +101,7 @@ def gmm(
     act_limit=7.0,
     rhs_bias=None,
     rhs_up_bias=None,
+    partial_sum_up=None,
 ):
   """Grouped matmul: out[rows of group g] = lhs[rows] @ rhs[g] (ops.py:46).
 
@@ -113,8 +115,8 @@ def gmm(
   _validate_args(lhs, rhs, group_sizes)
   if preferred_element_type != torch.bfloat16:
     raise NotImplementedError("only bfloat16 outputs are implemented")
-  if existing_out is not None or partial_sum is not None:
-    raise NotImplementedError("existing_out / partial_sum are not implemented")
+  if existing_out is not None:
+    raise NotImplementedError("existing_out is not implemented")
   if weight_gather_axes:
     raise NotImplementedError("weight all-gather belongs to the multi-device path")
   if group_offset is None:
@@ -128,8 +130,8 @@ def gmm(
       offset = int(group_offset)
 
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
-    if rhs_bias is not None or rhs_up_bias is not None:
-      raise NotImplementedError("gradients with rhs_bias are not implemented")
+    if rhs_bias is not None or rhs_up_bias is not None or partial_sum is not None or partial_sum_up is not None:
+      raise NotImplementedError("gradients with rhs_bias / partial_sum are not implemented")
     return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit)
 
   rhs_n = _native_rhs(rhs, transpose_rhs)
@@ -146,6 +148,10 @@ def gmm(
     kw["rhs_bias"] = rhs_bias.float().contiguous()  # [G, N] (rhs_bias [G, 1, N] of the v2 kernel, :573)
   if rhs_up_bias is not None:
     kw["rhs_up_bias"] = rhs_up_bias.float().contiguous()
+  if partial_sum is not None:  # [m, n], added to the product before the activation (ops.py:77)
+    kw["partial_sum"] = partial_sum.to(torch.bfloat16).contiguous()
+  if partial_sum_up is not None:
+    kw["partial_sum_up"] = partial_sum_up.to(torch.bfloat16).contiguous()
   if isinstance(lhs, QArray):
     kw["lhs_scale"] = lhs.scale
     kw["lhs_scale_block_k"] = 128 if lhs.qtype == "fp8" else 0

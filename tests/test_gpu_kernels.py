@@ -906,3 +906,58 @@ def test_gmm_int4_group32(K, m, k, n, gs):
   assert relerr(got, want) <= TOL
   tiled = K.gmm_raw(cuda(lhs), cuda(pq), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(pu), rhs_up_scale=cuda(su), act="silu", tile_variant=1, **kw)
   assert relerr(tiled, want) <= TOL
+
+
+@pytest.mark.parametrize("m,k,n,gs", [GMM_SHAPES[0], GMM_SHAPES[3], DECODE_SHAPES[0]])
+def test_gmm_partial_sum_every_kernel_family(K, m, k, n, gs):
+  """partial_sum (ops.py:77; v2 kernel :576-578): added after the bias and before the activation, only to rows of
+  local groups; rows that belong to no group stay zero.  Exercised with bf16 (tiled / direct-to-LDS), int8 x int8,
+  weight-only int8 (tiled or streaming by shape) and block-scaled fp8."""
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 90)
+  g = torch.Generator().manual_seed(91)
+  ps = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  ps_up = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  used = int(gs.sum())
+  act = lambda h0, h1: O.apply_ffn_activation(h0, h1, "silu")
+
+  def check(got, want):
+    assert relerr(got, want) <= TOL
+    assert torch.all(got[used:] == 0)
+
+  wb, ub = w.to(torch.bfloat16), w_up.to(torch.bfloat16)
+  check(K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), partial_sum=cuda(ps)), O.gmm(lhs, wb, gs, partial_sum=ps))
+  check(K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), rhs_up=cuda(native(ub)), act="silu", partial_sum=cuda(ps), partial_sum_up=cuda(ps_up)),
+        act(O.gmm(lhs, wb, gs, partial_sum=ps, out_dtype=torch.float32), O.gmm(lhs, ub, gs, partial_sum=ps_up, out_dtype=torch.float32)))
+  q, s = O.quantize_weight_int8(w)
+  qu, su = O.quantize_weight_int8(w_up)
+  check(K.gmm_raw(cuda(lhs), cuda(native(q)), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(native(qu)), rhs_up_scale=cuda(su), act="silu",
+                  partial_sum=cuda(ps), partial_sum_up=cuda(ps_up)),
+        act(O.gmm(lhs, q, gs, rhs_scale=s, partial_sum=ps, out_dtype=torch.float32), O.gmm(lhs, qu, gs, rhs_scale=su, partial_sum=ps_up, out_dtype=torch.float32)))
+  aq, asc = O.quantize_rows_int8(lhs.float())
+  check(K.gmm_raw(cuda(aq), cuda(native(q)), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(s), partial_sum=cuda(ps)),
+        O.gmm(aq, q, gs, lhs_scale=asc[:, None], rhs_scale=s, partial_sum=ps))
+  if k % 128 == 0:
+    fq, fsc = O.quantize_fp8_blocks(lhs, 1, 128)
+    wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)
+    v2f = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
+    check(K.gmm_raw(cuda(fq), cuda(wq), cuda(gs), lhs_scale=cuda(fsc), rhs_scale=cuda(wsc), lhs_scale_block_k=128, rhs_scale_block_n=128,
+                    rhs_scale_block_k=128, partial_sum=cuda(ps)),
+          O.gmm(fq, wq, gs, lhs_scale=fsc, rhs_scale=v2f(wsc), transpose_rhs=True, quant_block=128, partial_sum=ps))
+  with pytest.raises(ValueError):
+    K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), partial_sum_up=cuda(ps_up))
+
+
+def test_megablox_gmm_partial_sum_accumulates_k_chunks():
+  """The way the reference uses partial_sum (moe.py:1962-1980): the contraction is split into chunks of the embedding
+  dimension and each call adds the previous chunks' result; the chunked result must match the one-shot call."""
+  from maxtext_amd import megablox
+
+  lhs, w, _, gs = _gmm_inputs(600, 512, 256, [100, 0, 300, 200], 92)
+  wb = cuda(w.to(torch.bfloat16))  # [g, k, n]
+  lhs_d, gs_d = cuda(lhs), cuda(gs)
+  acc = None
+  for c in range(4):
+    sl = slice(c * 128, (c + 1) * 128)
+    acc = megablox.gmm(lhs_d[:, sl].contiguous(), wb[:, sl].contiguous(), gs_d, partial_sum=acc)
+  full = megablox.gmm(lhs_d, wb, gs_d)
+  assert relerr(acc, full) <= 2e-2  # three extra bf16 roundings of the running sum
