@@ -212,7 +212,14 @@ typedef struct {
    * embedding-chunked expert MLP (moe.py:1962-1980).  Must not alias `out`. */
   const void* partial_sum;
   const void* partial_sum_up;
+  int32_t flags; /* MOE_GMM_* bits */
+  int32_t pad_;
 } moe_gmm_args;
+
+/* flags: rows that belong to no local group are left as `out` holds them instead of being written as zeros:
+ * the existing_out argument of gmm (ops.py:51, backend.py:493-501), where a caller accumulates the shards' rows
+ * in one buffer. */
+#define MOE_GMM_KEEP_OTHER_ROWS 1
 
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
 MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libmoe_mi355x.so")
 MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32, MOE_MXFP4 = 0, 1, 2, 3, 4, 5
 MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK = 0, 1
 MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
+MOE_GMM_KEEP_OTHER_ROWS = 1
 
 ACT_BY_NAME = {None: MOE_ACT_NONE, "silu": MOE_ACT_SILU, "swigluoai": MOE_ACT_SWIGLUOAI, "silu_clip": MOE_ACT_SILU_CLIP}
 
@@ -55,6 +56,8 @@ class GmmArgs(ctypes.Structure):
       ("rhs_up_bias", c_void_p),
       ("partial_sum", c_void_p),
       ("partial_sum_up", c_void_p),
+      ("flags", ctypes.c_int32),
+      ("pad_", ctypes.c_int32),
   ]
 
 

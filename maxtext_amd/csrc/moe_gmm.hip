@@ -53,7 +53,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* s_buf, int* tota
 
 __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
     const int32_t* __restrict__ group_sizes, int G_total, int group_offset, int G_local, int M,
-    int BM, int32_t* __restrict__ header, TileInfo* __restrict__ tiles) {
+    int BM, int zero_fill, int32_t* __restrict__ header, TileInfo* __restrict__ tiles) {
   __shared__ int s_buf[kMapThreads];
   const int tid = threadIdx.x;
   const int per = (G_total + kMapThreads - 1) / kMapThreads;
@@ -69,7 +69,9 @@ __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
     for (int g = g0; g < g1; g++) {
       long long end = start + max(group_sizes[g], 0);
       int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
-      ntiles += (e - s + BM - 1) / BM;
+      const int local = g - group_offset;
+      // rows of groups held elsewhere get zero-fill tiles, or none at all when the caller keeps what `out` holds
+      if (zero_fill || (local >= 0 && local < G_local)) ntiles += (e - s + BM - 1) / BM;
       start = end;
     }
   }
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
       int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
       int local = g - group_offset;
       int kind = (local >= 0 && local < G_local) ? local : -1;
-      for (int r = s; r < e; r += BM) {
+      for (int r = s; r < e && (zero_fill || kind >= 0); r += BM) {
         TileInfo t;
         t.group = kind;
         t.row0 = r;
@@ -95,7 +97,7 @@ __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
     }
   }
   const int covered = min(total_rows, M);
-  const int tail = (M - covered + BM - 1) / BM;
+  const int tail = zero_fill ? (M - covered + BM - 1) / BM : 0;
   for (int i = tid; i < tail; i += kMapThreads) {
     TileInfo t;
     t.group = -1;
@@ -1601,6 +1603,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   if (align & 15) return fail(MOE_ERR_UNSUPPORTED, "gmm: pointers must be 16-byte aligned");
 
   hipStream_t s = (hipStream_t)stream;
+  const int zero_fill = (a->flags & MOE_GMM_KEEP_OTHER_ROWS) ? 0 : 1;
   int32_t* header = (int32_t*)a->workspace;
   TileInfo* tiles = (TileInfo*)((uint8_t*)a->workspace + 16);
 
@@ -1616,7 +1619,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     // weights through L2.  Many rows per expert: 64-row tiles.
     const bool few_rows = (long long)a->M <= 16LL * a->num_groups_total;
     bm = few_rows ? 16 : 64;
-    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, header, tiles);
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);
     SkinnyParams p;
     p.lhs = (const uint8_t*)a->lhs; p.lhs_scale = a->lhs_scale;
     p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
@@ -1678,7 +1681,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->K % 32 == 0 && a->reserved[0] != 1) {
     const bool one = (long long)M <= 16LL * G;
     bm = one ? 16 : 32;
-    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
     WqSkinnyParams q;
     q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
     q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
@@ -1699,14 +1702,14 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   if (forced >= 3 && variant == V_I8) {
     int st = glu ? launch_i8_variant<true>(forced, p, M, G, &bm, true, s) : launch_i8_variant<false>(forced, p, M, G, &bm, true, s);
     if (st != MOE_OK) return st;
-    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
     return glu ? launch_i8_variant<true>(forced, p, M, G, &bm, false, s) : launch_i8_variant<false>(forced, p, M, G, &bm, false, s);
   }
   if (glu)
     launch_tiled_by_rows<OP_BF16, BSRC_SAME, true>(p, M, G, &bm, true, s);
   else
     launch_tiled_by_rows<OP_BF16, BSRC_SAME, false>(p, M, G, &bm, true, s);
-  tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, header, tiles);
+  tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
   switch (variant) {
     case V_BF16: return launch_tiled_glu<OP_BF16, BSRC_SAME>(p, glu, M, G, &bm, false, s);
     case V_W8: return launch_tiled_glu<OP_BF16, BSRC_I8>(p, glu, M, G, &bm, false, s);

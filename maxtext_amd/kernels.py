@@ -224,7 +224,8 @@ def transpose_rhs(rhs_gkn):
 
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
-            group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None):
+            group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None,
+            keep_other_rows=False):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2])."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
@@ -302,6 +303,7 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
   a.partial_sum = partial_sum.data_ptr() if partial_sum is not None else None
   a.partial_sum_up = partial_sum_up.data_ptr() if partial_sum_up is not None else None
+  a.flags = _lib.MOE_GMM_KEEP_OTHER_ROWS if keep_other_rows else 0
   a.reserved[0] = int(tile_variant)
   a.reserved[1] = int(tune)
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())

@@ -116,7 +116,9 @@ def gmm(
   if preferred_element_type != torch.bfloat16:
     raise NotImplementedError("only bfloat16 outputs are implemented")
   if existing_out is not None:
-    raise NotImplementedError("existing_out is not implemented")
+    # rows of local groups are written into the caller's buffer, all other rows keep their contents (backend.py:493-501)
+    if existing_out.dtype != torch.bfloat16 or not existing_out.is_contiguous():
+      raise ValueError("existing_out must be a contiguous bfloat16 tensor")
   if weight_gather_axes:
     raise NotImplementedError("weight all-gather belongs to the multi-device path")
   if group_offset is None:
@@ -130,8 +132,8 @@ def gmm(
       offset = int(group_offset)
 
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
-    if rhs_bias is not None or rhs_up_bias is not None or partial_sum is not None or partial_sum_up is not None:
-      raise NotImplementedError("gradients with rhs_bias / partial_sum are not implemented")
+    if rhs_bias is not None or rhs_up_bias is not None or partial_sum is not None or partial_sum_up is not None or existing_out is not None:
+      raise NotImplementedError("gradients with rhs_bias / partial_sum / existing_out are not implemented")
     return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit)
 
   rhs_n = _native_rhs(rhs, transpose_rhs)
@@ -181,6 +183,8 @@ def gmm(
     rhs_t = rhs_n
     if up_n is not None:
       kw["rhs_up"] = up_n
+  if existing_out is not None:
+    kw.update(out=existing_out, keep_other_rows=True)
   return kernels.gmm_raw(lhs_t, rhs_t, group_sizes, **kw)
 
 
@@ -211,7 +215,9 @@ def tgmm(
   if lhs.shape[1] != rhs.shape[0]:
     raise ValueError(f"Expected lhs [k, m] and rhs [m, n] to share m, got {tuple(lhs.shape)} and {tuple(rhs.shape)}.")
   if existing_out is not None:
-    raise NotImplementedError("existing_out is not implemented")
+    # rows of local groups are written into the caller's buffer, all other rows keep their contents (backend.py:493-501)
+    if existing_out.dtype != torch.bfloat16 or not existing_out.is_contiguous():
+      raise ValueError("existing_out must be a contiguous bfloat16 tensor")
   if preferred_element_type not in (torch.float32, torch.bfloat16):
     raise NotImplementedError("tgmm outputs are float32 or bfloat16")
   offset = 0 if group_offset is None else int(group_offset)

@@ -961,3 +961,30 @@ def test_megablox_gmm_partial_sum_accumulates_k_chunks():
     acc = megablox.gmm(lhs_d[:, sl].contiguous(), wb[:, sl].contiguous(), gs_d, partial_sum=acc)
   full = megablox.gmm(lhs_d, wb, gs_d)
   assert relerr(acc, full) <= 2e-2  # three extra bf16 roundings of the running sum
+
+
+def test_gmm_existing_out_keeps_rows_of_other_groups():
+  """existing_out (ops.py:51): two calls, each holding half of the groups, fill one buffer; rows of the other
+  half and rows past the last group keep what the buffer held (here a sentinel), bit for bit."""
+  from maxtext_amd import megablox
+
+  lhs, w, _, gs = _gmm_inputs(700, 256, 128, [150, 0, 250, 100, 120], 95)  # 80 trailing rows in no group
+  wb = w.to(torch.bfloat16)
+  full = O.gmm(lhs, wb, gs)
+  buf = torch.full((700, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+  out = megablox.gmm(cuda(lhs), cuda(wb[:2]), cuda(gs), existing_out=buf, group_offset=0)
+  assert out.data_ptr() == buf.data_ptr()
+  assert torch.all(buf[150:] == 7.0) and relerr(buf[:150], full[:150]) <= TOL
+  megablox.gmm(cuda(lhs), cuda(wb[2:]), cuda(gs), existing_out=buf, group_offset=2)
+  assert relerr(buf[:620], full[:620]) <= TOL and torch.all(buf[620:] == 7.0)
+  # without existing_out the same call zeroes the rows it does not own
+  plain = megablox.gmm(cuda(lhs), cuda(wb[2:]), cuda(gs), group_offset=2)
+  assert torch.all(plain[:150] == 0) and torch.all(plain[620:] == 0)
+  # the few-rows (streaming) kernels take the same tile list
+  lhs2, w2, _, gs2 = _gmm_inputs(60, 256, 128, [10, 20, 5, 15], 96)
+  q, s = O.quantize_weight_int8(w2)
+  buf2 = torch.full((60, 128), -3.0, dtype=torch.bfloat16, device="cuda")
+  K = __import__("maxtext_amd.kernels", fromlist=["x"])
+  K.gmm_raw(cuda(lhs2), cuda(native(q[1:3])), cuda(gs2), rhs_scale=cuda(s[1:3]), group_offset=1, out=buf2, keep_other_rows=True)
+  want = O.gmm(lhs2, q, gs2, rhs_scale=s)
+  assert torch.all(buf2[:10] == -3.0) and torch.all(buf2[35:] == -3.0) and relerr(buf2[10:35], want[10:35]) <= TOL
