@@ -49,7 +49,9 @@ typedef enum {
 
 typedef enum {
   MOE_ROUTE_SOFTMAX_TOPK = 0, /* lax.top_k -> softmax over the k values, moe.py:747-753 */
-  MOE_ROUTE_DEEPSEEK = 1      /* deepseek_routing + deepseek_scale_weights, moe.py:767-839 */
+  MOE_ROUTE_DEEPSEEK = 1,     /* deepseek_routing + deepseek_scale_weights, moe.py:767-839 */
+  MOE_ROUTE_TOPK_RAW = 2,     /* Llama4: the top-k logits themselves are the weights, moe.py:747, :753 skipped */
+  MOE_ROUTE_SOFTMAX_ALL = 3   /* Gemma4: softmax over all experts, read at the top-k indices, moe.py:742-745 */
 } moe_route_mode;
 
 typedef enum {
@@ -75,7 +77,7 @@ MOE_API int moe_abi_version(void);
  *                                 weights_round_bf16 != 0 (the cast at moe.py:753)
  *   topk_idx         [T, k] i32   out; descending score, lower index first on ties
  *
- * norm_topk_prob: SOFTMAX_TOPK: divide by the sum of the k weights (moe.py:756);
+ * norm_topk_prob: SOFTMAX_TOPK, TOPK_RAW, SOFTMAX_ALL: divide by the sum of the k weights (moe.py:756);
  *   DEEPSEEK: w /= sum(w) + 1e-20, the sigmoid / sqrtsoftplus branch of moe.py:770-771.
  *   DEEPSEEK always multiplies by routed_scaling_factor (moe.py:772).
  * n_routing_groups / topk_routing_group: DeepSeek group-limited routing; -1 disables.

@@ -14,7 +14,8 @@ LIB_PATH = os.path.join(_PKG, "lib", "libmoe_mi355x.so")
 
 # enums of include/moe_mi355x.h
 MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32, MOE_MXFP4 = 0, 1, 2, 3, 4, 5
-MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK = 0, 1
+MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_TOPK_RAW, MOE_ROUTE_SOFTMAX_ALL = 0, 1, 2, 3
+ROUTE_BY_NAME = {"softmax_topk": 0, "deepseek": 1, "topk_raw": 2, "softmax_all": 3}
 MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
 MOE_GMM_KEEP_OTHER_ROWS = 1
 

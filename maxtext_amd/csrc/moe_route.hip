@@ -183,9 +183,21 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
     w *= scaling;
   } else {
     float mx = __shfl(myv, 0);
-    float ex = lane < k ? expf(myv - mx) : 0.f;
-    float s = wave_sum(ex);
-    w = ex / s;
+    if (mode == MOE_ROUTE_TOPK_RAW) {
+      w = lane < k ? myv : 0.f;
+    } else if (mode == MOE_ROUTE_SOFTMAX_ALL) {
+      // softmax over every expert (the best score is the first selected one), read at the selected experts
+      float part = 0.f;
+#pragma unroll
+      for (int j = 0; j < kRouteVpl; j++)
+        if (lane + kWave * j < E) part += expf(v[j] - mx);
+      const float s = wave_sum(part);
+      w = lane < k ? expf(myv - mx) / s : 0.f;
+    } else {
+      float ex = lane < k ? expf(myv - mx) : 0.f;
+      float s = wave_sum(ex);
+      w = ex / s;
+    }
     if (round_bf16) w = round_bf16_fn(w);
     if (norm) {
       float s2 = wave_sum(lane < k ? w : 0.f);
@@ -745,7 +757,7 @@ int moe_route_topk(const float* gate_logits, const float* pre_bias_logits, int T
   if (!gate_logits || !topk_weights || !topk_idx) return fail(MOE_ERR_INVALID_ARG, "route: NULL pointer");
   if (T < 0 || E <= 0 || k <= 0) return fail(MOE_ERR_INVALID_ARG, "route: bad sizes T=%d E=%d k=%d", T, E, k);
   if (E > kRouteMaxE || k > 16 || k > E) return fail(MOE_ERR_UNSUPPORTED, "route: need k<=16, k<=E<=512 (E=%d k=%d)", E, k);
-  if (mode != MOE_ROUTE_SOFTMAX_TOPK && mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "route: bad mode %d", mode);
+  if (mode < MOE_ROUTE_SOFTMAX_TOPK || mode > MOE_ROUTE_SOFTMAX_ALL) return fail(MOE_ERR_INVALID_ARG, "route: bad mode %d", mode);
   if (mode == MOE_ROUTE_DEEPSEEK && !pre_bias_logits) return fail(MOE_ERR_INVALID_ARG, "route: DeepSeek mode needs pre_bias_logits");
   int ng = n_routing_groups > 0 ? n_routing_groups : 0;
   if (ng > 0) {
@@ -785,7 +797,7 @@ int moe_gate_route(const void* x, const void* gate_kernel_terms, int num_terms, 
   if (d % 64 != 0 || E % 4 != 0) return fail(MOE_ERR_UNSUPPORTED, "gate_route: need d %% 64 == 0 and E %% 4 == 0 (d=%d E=%d)", d, E);
   if (E > kRouteMaxE || k > 16 || k > E) return fail(MOE_ERR_UNSUPPORTED, "gate_route: need k<=16, k<=E<=512 (E=%d k=%d)", E, k);
   if (score_func != 0 && score_func != 1) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad score_func %d", score_func);
-  if (mode != MOE_ROUTE_SOFTMAX_TOPK && mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad mode %d", mode);
+  if (mode < MOE_ROUTE_SOFTMAX_TOPK || mode > MOE_ROUTE_SOFTMAX_ALL) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad mode %d", mode);
   int ng = n_routing_groups > 0 ? n_routing_groups : 0;
   if (ng > 0) {
     if (mode != MOE_ROUTE_DEEPSEEK) return fail(MOE_ERR_INVALID_ARG, "gate_route: routing groups need DeepSeek mode");

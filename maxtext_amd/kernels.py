@@ -34,15 +34,13 @@ def route_topk(gate_logits, pre_bias_logits=None, *, k, mode="softmax_topk", nor
   """-> (weights [T,k] f32, indices [T,k] int32)."""
   _need(gate_logits, "gate_logits", torch.float32, 2)
   t, e = gate_logits.shape
+  if mode not in _lib.ROUTE_BY_NAME:
+    raise ValueError(f"unknown routing mode {mode!r}")
+  code = _lib.ROUTE_BY_NAME[mode]
   if mode == "deepseek":
     _need(pre_bias_logits, "pre_bias_logits", torch.float32, 2)
     if pre_bias_logits.shape != gate_logits.shape:
       raise ValueError("pre_bias_logits must match gate_logits")
-    code = MOE_ROUTE_DEEPSEEK
-  elif mode == "softmax_topk":
-    code = MOE_ROUTE_SOFTMAX_TOPK
-  else:
-    raise ValueError(f"unknown routing mode {mode!r}")
   w = torch.empty((t, k), dtype=torch.float32, device=gate_logits.device)
   idx = torch.empty((t, k), dtype=torch.int32, device=gate_logits.device)
   lib = _lib.load()
@@ -70,7 +68,7 @@ def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_r
       raise ValueError("gate_bias must have E elements")
   if score_func not in ("", "sigmoid"):
     raise NotImplementedError(f"score_func {score_func!r}")
-  if mode not in ("softmax_topk", "deepseek"):
+  if mode not in _lib.ROUTE_BY_NAME:
     raise ValueError(f"unknown routing mode {mode!r}")
   dev = x.device
   w = torch.empty((t, k), dtype=torch.float32, device=dev)
@@ -81,7 +79,7 @@ def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_r
   ws = torch.empty((max(lib.moe_gate_route_workspace_bytes(t, d, e), 16),), dtype=torch.uint8, device=dev)
   st = lib.moe_gate_route(_lib.ptr(x), _lib.ptr(gate_kernel_terms), s_, _lib.ptr(gate_bias), t, d, e, k,
                           1 if score_func == "sigmoid" else 0, int(bool(gate_round_bf16)),
-                          MOE_ROUTE_DEEPSEEK if mode == "deepseek" else MOE_ROUTE_SOFTMAX_TOPK, int(bool(norm_topk_prob)),
+                          _lib.ROUTE_BY_NAME[mode], int(bool(norm_topk_prob)),
                           int(bool(weights_round_bf16)), float(routed_scaling_factor), int(n_routing_groups),
                           int(topk_routing_group), _lib.ptr(w), _lib.ptr(idx), _lib.ptr(logits), _lib.ptr(pre), _lib.ptr(ws),
                           ws.numel(), _lib.current_stream())

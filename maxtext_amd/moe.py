@@ -47,6 +47,17 @@ class MoEConfig:
     return self.model_name.startswith(("deepseek3", "deepseek4"))
 
   @property
+  def route_mode(self) -> str:
+    """Weight rule of get_topk (moe.py:738-756)."""
+    if self.is_deepseek:
+      return "deepseek"
+    if self.decoder_block == "llama4":
+      return "topk_raw"  # raw top-k logits; sigmoid of them scales the inputs in permute (moe.py:902-906)
+    if self.decoder_block == "gemma4":
+      return "softmax_all"  # softmax over all experts read at the top-k indices (moe.py:742-745)
+    return "softmax_topk"
+
+  @property
   def activation(self) -> str:
     if self.decoder_block == "gpt_oss":
       return "swigluoai"
@@ -110,6 +121,7 @@ class RoutedMoE:
     self.wi_0, self.wi_1, self.wo = wi_0, wi_1, wo
     self.gate_kernel, self.gate_bias = gate_kernel, gate_bias
     self._gate_terms = None  # [S, E, d] bf16 form of gate_kernel for moe_gate_route, built on first use
+    self.per_expert_scale = None  # [E] f32, Gemma4: multiplies the routing weights (moe.py:758-763)
     # when set to a list, _experts appends (stage, start_event, end_event) recorded on the launch stream
     self.profile_events = None
 
@@ -146,7 +158,13 @@ class RoutedMoE:
                                 norm_topk_prob=cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"),
                                 routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups,
                                 topk_routing_group=cfg.topk_routing_group, **common)
-    return kernels.gate_route(x, self._gate_terms, bias, norm_topk_prob=cfg.norm_topk_prob, **common)
+    r = kernels.gate_route(x, self._gate_terms, bias, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob, **common)
+    return (self._scale_per_expert(r[0], r[1]),) + tuple(r[1:])
+
+  def _scale_per_expert(self, w, idx):
+    if self.per_expert_scale is None:
+      return w
+    return w * self.per_expert_scale.float()[idx.long()]
 
   # -- auxiliary outputs of permute (moe.py:886-900) ------------------------------------------
   def load_balance_loss(self, top_k_indices: torch.Tensor, probs: torch.Tensor) -> torch.Tensor:
@@ -184,7 +202,8 @@ class RoutedMoE:
           routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups,
           topk_routing_group=cfg.topk_routing_group)
     else:
-      w, idx = kernels.route_topk(g2, k=self.num_experts_per_tok, norm_topk_prob=cfg.norm_topk_prob)
+      w, idx = kernels.route_topk(g2, k=self.num_experts_per_tok, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob)
+      w = self._scale_per_expert(w, idx)
     k = self.num_experts_per_tok
     if torch.is_grad_enabled() and (gate_logits.requires_grad or (pre_bias_logits is not None and pre_bias_logits.requires_grad)):
       w = self._weights_with_grad(gate_logits, pre_bias_logits, idx.reshape(*shape, k))
@@ -200,10 +219,26 @@ class RoutedMoE:
       if cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"):
         w = w / (w.sum(-1, keepdim=True) + 1e-20)
       return w * cfg.routed_scaling_factor
-    w = torch.softmax(torch.gather(gate_logits.float(), -1, gi), -1).to(torch.bfloat16)
+    if cfg.route_mode == "topk_raw":
+      w = torch.gather(gate_logits.float(), -1, gi).to(torch.bfloat16)
+    elif cfg.route_mode == "softmax_all":
+      w = torch.gather(torch.softmax(gate_logits.float(), -1), -1, gi).to(torch.bfloat16)
+    else:
+      w = torch.softmax(torch.gather(gate_logits.float(), -1, gi), -1).to(torch.bfloat16)
     if cfg.norm_topk_prob:
       w = w / w.sum(-1, keepdim=True)
+    if self.per_expert_scale is not None:
+      w = w * self.per_expert_scale.to(w.dtype)[gi]
     return w.float()
+
+  def _scale_inputs_by_router_score(self, x2d, weights):
+    """Llama4 scales each token by sigmoid(router score) before the experts (moe.py:902-906); the reference's
+    broadcast of [T, d] * [T, k] only exists for top-1."""
+    if self.config.decoder_block != "llama4":
+      return x2d
+    if self.num_experts_per_tok != 1:
+      raise NotImplementedError("Llama4 routing scales the token by its single router score (num_experts_per_tok == 1)")
+    return (x2d.float() * torch.sigmoid(weights.reshape(-1, 1).float())).to(x2d.dtype)
 
   # -- permute (moe.py:872-1002), non-ragged branch -----------------------------------------
   def permute(self, inputs, gate_logits, pre_bias_logits=None, use_custom_sort_vjp=True, rngs=None,
@@ -215,6 +250,7 @@ class RoutedMoE:
     b, s, d = inputs.shape
     x2d = inputs.reshape(b * s, d).contiguous()
     weights, selected = self.get_topk(gate_logits, pre_bias_logits)
+    x2d = self._scale_inputs_by_router_score(x2d, weights)
     sel2d = selected.reshape(b * s, -1).contiguous()
     perm, inv, group_size, sorted_experts = kernels.sort_by_expert(sel2d, self.num_experts)
     if torch.is_grad_enabled() and x2d.requires_grad:
@@ -232,6 +268,8 @@ class RoutedMoE:
       raise NotImplementedError("only float32_weight_sum=True is implemented")
     k = self.num_experts_per_tok
     w = weights.reshape(-1, k).float().contiguous()
+    if self.config.decoder_block == "llama4":
+      w = torch.ones_like(w)  # the router score already scaled the inputs (moe.py:1051-1052)
     if torch.is_grad_enabled() and (intermediate.requires_grad or w.requires_grad):
       if inv_perm is None:
         inv_perm = torch.empty_like(sorted_selected_experts)
@@ -290,6 +328,7 @@ class RoutedMoE:
     k = self.num_experts_per_tok
     x2d = inputs.reshape(b * s, d).contiguous()
     weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits)
+    x2d = self._scale_inputs_by_router_score(x2d, weights)
     perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
                                                       want_sorted_experts=False)
     training = torch.is_grad_enabled() and any(

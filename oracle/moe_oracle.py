@@ -160,10 +160,15 @@ def get_topk(
       w = w / (w.sum(-1, keepdims=True, dtype=np.float32) + np.float32(1e-20))
     w = (w * np.float32(routed_scaling_factor)).astype(np.float32)
     return w, idx
-  if mode != "softmax_topk":
+  if mode not in ("softmax_topk", "topk_raw", "softmax_all"):
     raise ValueError(f"unknown routing mode {mode}")
   vals, idx = top_k(gate_logits, k)
-  w = _softmax_f32(vals)
+  if mode == "topk_raw":  # Llama4: no softmax over the selected logits (moe.py:753 is skipped for LLAMA4)
+    w = vals.astype(np.float32)
+  elif mode == "softmax_all":  # Gemma4: softmax over all experts, gathered at the indices (moe.py:742-745)
+    w = np.take_along_axis(_softmax_f32(gate_logits), idx, axis=-1)
+  else:
+    w = _softmax_f32(vals)
   if weight_dtype == "bf16":
     w = _round_bf16(w)
   if norm_topk_prob:

@@ -988,3 +988,26 @@ def test_gmm_existing_out_keeps_rows_of_other_groups():
   K.gmm_raw(cuda(lhs2), cuda(native(q[1:3])), cuda(gs2), rhs_scale=cuda(s[1:3]), group_offset=1, out=buf2, keep_other_rows=True)
   want = O.gmm(lhs2, q, gs2, rhs_scale=s)
   assert torch.all(buf2[:10] == -3.0) and torch.all(buf2[35:] == -3.0) and relerr(buf2[10:35], want[10:35]) <= TOL
+
+
+@pytest.mark.parametrize("mode", ["topk_raw", "softmax_all"])
+@pytest.mark.parametrize("t,e,k", [(300, 16, 1), (1000, 128, 8), (77, 200, 4)])
+def test_route_llama4_and_gemma4_weight_rules(K, mode, t, e, k):
+  """Llama4 keeps the selected logits as weights; Gemma4 reads a softmax over all experts at the selected
+  indices (moe.py:742-753).  Indices bit-exact, weights against the closed forms."""
+  rng = np.random.default_rng(8)
+  logits = rng.standard_normal((t, e)).astype(np.float32) * 2
+  for norm in (False, True):
+    w, idx = K.route_topk(cuda(logits), k=k, mode=mode, norm_topk_prob=norm)
+    ow, oidx = O.get_topk(logits, k=k, mode=mode, norm_topk_prob=norm)
+    np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+    np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=2.0**-6, atol=1e-6)
+  # independent closed forms in f64
+  w, idx = K.route_topk(cuda(logits), k=k, mode=mode, weights_round_bf16=False)
+  sel = np.take_along_axis(logits.astype(np.float64), idx.cpu().numpy().astype(np.int64), -1)
+  if mode == "topk_raw":
+    want = sel
+  else:
+    z = np.exp(logits.astype(np.float64) - logits.max(-1, keepdims=True))
+    want = np.exp(sel - logits.max(-1, keepdims=True)) / z.sum(-1, keepdims=True)
+  np.testing.assert_allclose(w.cpu().numpy(), want, rtol=1e-5, atol=1e-7)

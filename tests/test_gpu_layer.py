@@ -382,3 +382,46 @@ def test_auxiliary_outputs_match_reference_formulas():
   # without the config keys nothing is returned
   _, lb0, upd0 = moe.RoutedMoE(dc.replace(cfg, load_balance_loss_weight=0.0, routed_bias_update_rate=0.0), *ws).sparse_matmul(x, logits, None, *ws)
   assert lb0 is None and upd0 is None
+
+
+def test_llama4_and_gemma4_style_layers():
+  """Llama4: top-1, token scaled by sigmoid(router logit) before the expert, combine with ones (moe.py:902-906, :1051).
+  Gemma4: weights = softmax over all experts at the top-k, renormalised, times a per-expert scale (moe.py:742-763).
+  Both against the per-token loop in f64 on the GPU's routing."""
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(70)
+  t, d, f, e = 200, 128, 256, 8
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  logits = torch.randn(1, t, e, generator=g)
+  ws = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
+  scale = torch.rand(e, generator=g) + 0.5
+
+  def expert(xrow, ex):
+    h0 = torch.einsum("td,tfd->tf", xrow, ws[0].double()[ex])
+    h1 = torch.einsum("td,tfd->tf", xrow, ws[1].double()[ex])
+    return torch.einsum("tf,tdf->td", torch.nn.functional.silu(h0) * h1, ws[2].double()[ex])
+
+  # Llama4
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=1, emb_dim=d, moe_mlp_dim=f, decoder_block="llama4")
+  block = moe.RoutedMoE(cfg, *[w.cuda() for w in ws])
+  out, _, _ = block.sparse_matmul(x.cuda(), logits.cuda(), None, *[w.cuda() for w in ws])
+  top = logits.reshape(t, e).max(-1)
+  xs = (x.reshape(t, d).float() * torch.sigmoid(top.values.float())[:, None]).to(torch.bfloat16).double()
+  want = expert(xs, top.indices)
+  assert relerr(out.reshape(t, d), want) <= TOL
+  # Gemma4
+  k = 2
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, decoder_block="gemma4", norm_topk_prob=True)
+  block = moe.RoutedMoE(cfg, *[w.cuda() for w in ws])
+  block.per_expert_scale = scale.cuda()
+  out, _, _ = block.sparse_matmul(x.cuda(), logits.cuda(), None, *[w.cuda() for w in ws])
+  w_gpu, idx = block.get_topk(logits.cuda())
+  idx = idx.reshape(t, k).cpu().long()
+  probs = torch.softmax(logits.reshape(t, e).double(), -1)
+  wsel = torch.gather(probs, -1, idx)
+  wsel = wsel / wsel.sum(-1, keepdim=True) * scale.double()[idx]  # normalised first, then scaled (moe.py:755-763)
+  assert relerr(w_gpu.reshape(t, k), wsel) <= 2.0**-6
+  x2 = x.reshape(t, d).double()
+  want = sum(wsel[:, s_ : s_ + 1] * expert(x2, idx[:, s_]) for s_ in range(k))
+  assert relerr(out.reshape(t, d), want) <= 2e-2

@@ -130,6 +130,26 @@ def test_softmax_topk_weights_closed_form():
   np.testing.assert_allclose(wn.sum(-1), 1.0, atol=2e-2)
 
 
+def test_llama4_and_gemma4_weight_rules_closed_form():
+  """moe.py:742-753: Gemma4 reads softmax(all experts) at the top-k indices, Llama4 keeps the logits themselves."""
+  rng = np.random.default_rng(11)
+  x = rng.standard_normal((50, 12)).astype(np.float32)
+  w, idx = O.get_topk(x, k=3, mode="topk_raw", weight_dtype="f32")
+  np.testing.assert_array_equal(w, -np.sort(-x, axis=-1)[:, :3])
+  w, idx2 = O.get_topk(x, k=3, mode="softmax_all", weight_dtype="f32")
+  np.testing.assert_array_equal(idx, idx2)
+  # with k == E the rule is the plain softmax, which sums to one; the selected ones are its largest entries
+  wall, iall = O.get_topk(x, k=12, mode="softmax_all", weight_dtype="f32")
+  np.testing.assert_allclose(wall.sum(-1), 1.0, rtol=1e-6)
+  np.testing.assert_allclose(w, wall[:, :3], rtol=1e-6)
+  # ratio of two entries == exp of the logit difference (fails for a softmax over the top-k only if k changes it: it does not,
+  # so also check the absolute value against f64)
+  z = np.exp(x.astype(np.float64))
+  np.testing.assert_allclose(w, np.take_along_axis(z / z.sum(-1, keepdims=True), idx, -1), rtol=1e-5)
+  wn, _ = O.get_topk(x, k=3, mode="softmax_all", norm_topk_prob=True, weight_dtype="f32")
+  np.testing.assert_allclose(wn.sum(-1), 1.0, rtol=1e-5)
+
+
 def test_deepseek_weights_closed_form():
   rng = np.random.default_rng(2)
   logits = rng.standard_normal((32, 64)).astype(np.float32)
