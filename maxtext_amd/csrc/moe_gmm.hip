@@ -883,11 +883,50 @@ struct SkinnyParams {
   float act_limit;
 };
 
-__device__ __forceinline__ v8i load32(const uint8_t* p) {
-  const uint4 a = *(const uint4*)p, b = *(const uint4*)(p + 16);
+// Activation fragment of one 128-byte k-block: lane (j, kq) takes bytes kq*16.. and 64+kq*16.. of its row,
+// the k order load_w128 leaves the weights in.
+__device__ __forceinline__ v8i load_a128(const uint8_t* p) {
+  const uint4 a = *(const uint4*)p, b = *(const uint4*)(p + 64);
   v8i r;
   r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
   r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+  return r;
+}
+
+// Weight fragment of one 128-byte k-block for 16 channels.  Each of the two requests covers whole 128-byte
+// lines (8 channels x 128 B: lane (i, kq) asks for bytes (i/8)*64 + kq*16.. of channel i%8, then of channel
+// i%8 + 8) and is non-temporal: weights are read once, and a streamed read that owns its lines runs about
+// 12 % faster than one that leaves half of each line to the next request (STREAM = false keeps the lines
+// cached, for tiles that share weights).  A rotation by 8 inside each row of 16 lanes then hands every lane
+// the two 16-byte pieces of its own channel i.
+template <bool STREAM>
+__device__ __forceinline__ v4i load_w16(const uint8_t* p) {
+  return STREAM ? __builtin_nontemporal_load((const v4i*)p) : *(const v4i*)p;
+}
+
+// a = request for channels i%8, b = request for channels i%8 + 8, each lane holding piece i/8 (the first or second
+// 64 bytes of the 128-byte unit).  Returns in `first` / `second` the two pieces of the lane's own channel i.
+__device__ __forceinline__ void own_channel_pieces(const v4i& a, const v4i& b, v4i& first, v4i& second) {
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    // lanes 8..15 of a row: the first piece of their channel sits in `b` of lane i-8; lanes 0..7 keep their `a`
+    first[c] = __builtin_amdgcn_update_dpp(a[c], b[c], 0x128, 0xf, 0xc, false);
+    // lanes 0..7: the second piece of their channel sits in `a` of lane i+8; lanes 8..15 keep their `b`
+    second[c] = __builtin_amdgcn_update_dpp(b[c], a[c], 0x128, 0xf, 0x3, false);
+  }
+}
+
+template <bool STREAM>
+__device__ __forceinline__ v8i load_w128(const uint8_t* lo_rows, const uint8_t* hi_rows) {
+  const v4i a = load_w16<STREAM>(lo_rows), b = load_w16<STREAM>(hi_rows);
+  v4i x, y;
+  own_channel_pieces(a, b, x, y);
+  v8i r;
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    r[c] = x[c];
+    r[4 + c] = y[c];
+  }
   return r;
 }
 
@@ -918,17 +957,18 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 
   const int nkb = K / 128;
   const int nnb = (N + 127) / 128;
-  const uint8_t* wp[NT];
-  const uint8_t* up[NT];
+  // offsets inside the expert's [N, K] matrix (the host checks N * K < 2^31), shared by rhs and rhs_up
+  const uint8_t* wbase = p.rhs + (size_t)tile.group * N * K;
+  const uint8_t* ubase = GLU ? p.rhs_up + (size_t)tile.group * N * K : nullptr;
+  uint32_t wlo[NT], whi[NT];
   const float* wsp[NT];
   const float* usp[NT];
 #pragma unroll
   for (int t = 0; t < NT; t++) {
     const int n16 = n_w + t * 16;
-    const int nw = min(n16 + j, N - 1);
-    const size_t wrow = ((size_t)tile.group * N + nw) * K + kq * 32;
-    wp[t] = p.rhs + wrow;
-    up[t] = GLU ? p.rhs_up + wrow : nullptr;
+    const uint32_t in_line = (uint32_t)((j / 8) * 64 + kq * 16);
+    wlo[t] = (uint32_t)min(n16 + j % 8, N - 1) * (uint32_t)K + in_line;
+    whi[t] = (uint32_t)min(n16 + j % 8 + 8, N - 1) * (uint32_t)K + in_line;
     const size_t srow = ((size_t)tile.group * nnb + min(n16, N - 1) / 128) * nkb;
     wsp[t] = p.rhs_scale + srow;
     usp[t] = GLU ? p.rhs_up_scale + srow : nullptr;
@@ -938,7 +978,7 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 #pragma unroll
   for (int mt = 0; mt < MT; mt++) {
     const int gr = tile.row0 + min(mt * 16 + j, tile.nrows - 1);
-    ap[mt] = p.lhs + (size_t)gr * K + kq * 32;
+    ap[mt] = p.lhs + (size_t)gr * K + kq * 16;
     asp[mt] = p.lhs_scale + (size_t)gr * nkb;
   }
   v4f acc_g[NT][MT], acc_u[NT][MT];
@@ -960,11 +1000,11 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
       const size_t off = (size_t)(kb0 + u) * 128;
 #pragma unroll
       for (int t = 0; t < NT; t++) {
-        wf[u][t] = load32(wp[t] + off);
-        if (GLU) uf[u][t] = load32(up[t] + off);
+        wf[u][t] = load_w128<MT == 1>(wbase + wlo[t] + off, wbase + whi[t] + off);
+        if (GLU) uf[u][t] = load_w128<MT == 1>(ubase + wlo[t] + off, ubase + whi[t] + off);
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) af[u][mt] = load32(ap[mt] + off);
+      for (int mt = 0; mt < MT; mt++) af[u][mt] = load_a128(ap[mt] + off);
     }
 #pragma unroll
     for (int u = 0; u < UC; u++) {
@@ -1028,9 +1068,9 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 // ---------------------------------------------------------------------------------------
 // Weight-only int8 / int4 for few rows per expert (decode): bf16 activations, weights widened to bf16 in
 // registers, v_mfma_f32_16x16x32_bf16.  Same streaming structure as the fp8 kernel: no LDS, one wave owns
-// 16*NT output channels and walks K in 128-element blocks; lane (n = lane%16, kq = lane/16) holds the 32
-// consecutive k values kq*32.. of the block for its channel (one 16-byte load for int4, two for int8) and
-// the matching 64 bytes of its activation row.  int4 weights are multiplied by their group-128 scale while
+// 16*NT output channels and walks K in 128-element blocks; lane (n = lane%16, kq = lane/16) holds 32 k values
+// of the block for its channel (4-bit: kq*32.. ; int8: kq*16.. and 64 + kq*16..) and the matching 64 bytes of
+// its activation row.  int4 weights are multiplied by their group-128 scale while
 // they are widened; the int8 per-channel scale is applied once at the end.
 // ---------------------------------------------------------------------------------------
 
@@ -1060,14 +1100,6 @@ template <int FMT>
 struct WqRaw {
   uint4 q0, q1;
 };
-
-template <int FMT>
-__device__ __forceinline__ WqRaw<FMT> wq_load(const uint8_t* p) {
-  WqRaw<FMT> r;
-  r.q0 = *(const uint4*)p;
-  r.q1 = FMT != WQ_I8 ? make_uint4(0, 0, 0, 0) : *(const uint4*)(p + 16);
-  return r;
-}
 
 template <int FMT>
 __device__ __forceinline__ void widen32(const WqRaw<FMT>& raw, float scale, v8bf (&w)[4]) {
@@ -1113,9 +1145,16 @@ __device__ __forceinline__ void widen32(const WqRaw<FMT>& raw, float scale, v8bf
 // of tokens, 1 once there are enough blocks).  Within its range a wave works in rounds of U blocks whose loads
 // are all issued before the first block is converted and multiplied; other resident waves cover the rest of the
 // latency (holding two rounds in registers halves the occupancy and measures slower).
-template <int FMT, int MT, int NT, bool GLU, int U, int KSPLIT>
+//
+// Weight requests cover 128 contiguous bytes of 8 channels each (one k-block of int8, two of a 4-bit format), two
+// requests per 16 channels, like load_w128 of the fp8 kernel; 4-bit formats therefore walk K in pairs of blocks
+// (U even) and keep the k order inside a block, int8 gets the order (kq*16.., 64 + kq*16..) inside its block and
+// reads its activations to match.
+template <int FMT, int MT, int NT, bool GLU, int U, int KSPLIT, bool STREAM>
 __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams p) {
   constexpr bool INT4 = FMT == WQ_I4, MX4 = FMT == WQ_MX4, G32 = FMT == WQ_I4G32, NIB = FMT != WQ_I8;
+  constexpr int UB = NIB ? 2 : 1;  // k-blocks per 128-byte unit of a weight row
+  static_assert(U % UB == 0, "4-bit formats are loaded in pairs of k-blocks");
   constexpr int NACC = NT * MT * 4 * (GLU ? 2 : 1);
   constexpr int NSUB = 4 / KSPLIT;  // channel groups per block
   __shared__ float red[KSPLIT > 1 ? NSUB * (KSPLIT - 1) * NACC * kWave : 1];
@@ -1145,8 +1184,11 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 
   const int nkb = (K + 127) / 128;  // the last block may be partial (K % 32 == 0)
   const size_t wrow_bytes = NIB ? (size_t)K / 2 : (size_t)K;
-  const uint8_t* wp[NT];
-  const uint8_t* up[NT];
+  // the expert's matrix (the host checks N * K < 2^31) and, inside it, the rows of this lane's two requests
+  const uint8_t* wbase = p.rhs + (size_t)tile.group * N * wrow_bytes;
+  const uint8_t* ubase = GLU ? p.rhs_up + (size_t)tile.group * N * wrow_bytes : nullptr;
+  const int piece = j / 8;
+  uint32_t wlo[NT], whi[NT];
   const uint16_t* wsp[NT];
   const uint16_t* usp[NT];
   const uint8_t* wmx[NT];
@@ -1155,8 +1197,8 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
   for (int t = 0; t < NT; t++) {
     const int nw = min(n_w + t * 16 + j, N - 1);
     const size_t row = (size_t)tile.group * N + nw;
-    wp[t] = p.rhs + row * wrow_bytes + kq * (NIB ? 16 : 32);
-    up[t] = GLU ? p.rhs_up + row * wrow_bytes + kq * (NIB ? 16 : 32) : nullptr;
+    wlo[t] = (uint32_t)min(n_w + t * 16 + j % 8, N - 1) * (uint32_t)wrow_bytes;
+    whi[t] = (uint32_t)min(n_w + t * 16 + j % 8 + 8, N - 1) * (uint32_t)wrow_bytes;
     wsp[t] = INT4 ? (const uint16_t*)p.rhs_scale + row * nkb : nullptr;
     usp[t] = INT4 && GLU ? (const uint16_t*)p.rhs_up_scale + row * nkb : nullptr;
     // MXFP4: one e8m0 byte per 32 values = per lane and k block
@@ -1172,7 +1214,7 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 #pragma unroll
   for (int mt = 0; mt < MT; mt++) {
     const int gr = tile.row0 + min(mt * 16 + j, tile.nrows - 1);
-    ap[mt] = p.lhs + ((size_t)gr * K + kq * 32) * 2;
+    ap[mt] = p.lhs + (size_t)gr * K * 2;  // row start
   }
   v4f acc_g[NT][MT], acc_u[NT][MT];
 #pragma unroll
@@ -1186,29 +1228,47 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
   // One round = U k-blocks held as raw bytes.
   struct Round {
     uint4 araw[U][MT][4];
-    WqRaw<FMT> wraw[U][NT], uraw[U][NT];
+    v4i wa[U / UB][NT], wb[U / UB][NT], ua[U / UB][NT], ub[U / UB][NT];  // the two requests of each unit
     uint16_t wsc[U][NT], usc[U][NT];
-    bool live[U];
+    bool live[U][2];  // first / second 16 k values of the lane (int8; one flag for the 4-bit formats)
   };
-  const int chunk = (nkb + KSPLIT - 1) / KSPLIT;
+  const int chunk = (nkb + KSPLIT * UB - 1) / (KSPLIT * UB) * UB;  // whole units
   const int kb_begin = ksub * chunk;
   const int kb_end = idle ? kb_begin : min(nkb, kb_begin + chunk);
 
   // Blocks past the end of the range are loaded from the range's last block and flagged dead (their activations
   // are zeroed before use), so every round has the same instruction stream.
+  // k index of a block's first value for this lane, or of one of its two 16-value pieces with int8
+  auto lane_k = [&](int kb, int half) { return NIB ? kb * 128 + kq * 32 : kb * 128 + half * 64 + kq * 16; };
   auto load_round = [&](Round& r, int kb0) {
+#pragma unroll
+    for (int un = 0; un < U / UB; un++) {
+      // the piece of the unit this lane asks for: a whole block of a 4-bit format, half a block of int8
+      const int kbp_raw = kb0 + un * UB + (NIB ? piece : 0);
+      const int kbp = kbp_raw < kb_end ? kbp_raw : max(kb_end - 1, 0);
+      const int kp = lane_k(kbp, piece);
+      const uint32_t woff = kp < K ? (uint32_t)(NIB ? kp / 2 : kp) : 0u;
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        r.wa[un][t] = load_w16<STREAM>(wbase + wlo[t] + woff);
+        r.wb[un][t] = load_w16<STREAM>(wbase + whi[t] + woff);
+        if (GLU) {
+          r.ua[un][t] = load_w16<STREAM>(ubase + wlo[t] + woff);
+          r.ub[un][t] = load_w16<STREAM>(ubase + whi[t] + woff);
+        }
+      }
+    }
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const bool in_range = kb0 + u < kb_end;
       const int kb = in_range ? kb0 + u : max(kb_end - 1, 0);
-      // this lane's 32 k values exist unless the block is the partial tail
-      r.live[u] = in_range && kb * 128 + kq * 32 < K;
-      const bool addr_ok = kb * 128 + kq * 32 < K;
-      const size_t woff = addr_ok ? (size_t)kb * (NIB ? 64 : 128) : 0;
+      // this lane's k values exist unless the block is the partial tail
+      const bool ok0 = lane_k(kb, 0) < K, ok1 = lane_k(kb, 1) < K;
+      r.live[u][0] = in_range && ok0;
+      r.live[u][1] = in_range && ok1;
+      const bool addr_ok = ok0;
 #pragma unroll
       for (int t = 0; t < NT; t++) {
-        r.wraw[u][t] = wq_load<FMT>(wp[t] + woff);
-        if (GLU) r.uraw[u][t] = wq_load<FMT>(up[t] + woff);
         if (INT4) {
           r.wsc[u][t] = wsp[t][kb];
           if (GLU) r.usc[u][t] = usp[t][kb];
@@ -1224,20 +1284,37 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
       }
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
-        const uint8_t* a = ap[mt] + (addr_ok ? (size_t)kb * 256 : 0);
-#pragma unroll
-        for (int s = 0; s < 4; s++) r.araw[u][mt][s] = *(const uint4*)(a + s * 16);
+        // 4-bit formats: 64 contiguous bytes; int8: 32 bytes for each of the two pieces.  A piece past K reads the row start.
+        const uint8_t* a0 = ap[mt] + (ok0 ? (size_t)lane_k(kb, 0) * 2 : 0);
+        const uint8_t* a1 = NIB ? a0 + 32 : ap[mt] + (ok1 ? (size_t)lane_k(kb, 1) * 2 : 0);
+        r.araw[u][mt][0] = *(const uint4*)a0;
+        r.araw[u][mt][1] = *(const uint4*)(a0 + 16);
+        r.araw[u][mt][2] = *(const uint4*)a1;
+        r.araw[u][mt][3] = *(const uint4*)(a1 + 16);
       }
     }
   };
 
   auto compute_round = [&](const Round& r) {
     const auto& araw = r.araw;
-    const auto& wraw = r.wraw;
-    const auto& uraw = r.uraw;
     const auto& wsc = r.wsc;
     const auto& usc = r.usc;
     const auto& live = r.live;
+    WqRaw<FMT> wraw[U][NT], uraw[U][NT];
+#pragma unroll
+    for (int un = 0; un < U / UB; un++)
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        v4i x, y;
+        own_channel_pieces(r.wa[un][t], r.wb[un][t], x, y);
+        wraw[un * UB][t].q0 = __builtin_bit_cast(uint4, x);
+        (NIB ? wraw[un * UB + UB - 1][t].q0 : wraw[un][t].q1) = __builtin_bit_cast(uint4, y);
+        if (GLU) {
+          own_channel_pieces(r.ua[un][t], r.ub[un][t], x, y);
+          uraw[un * UB][t].q0 = __builtin_bit_cast(uint4, x);
+          (NIB ? uraw[un * UB + UB - 1][t].q0 : uraw[un][t].q1) = __builtin_bit_cast(uint4, y);
+        }
+      }
 #pragma unroll
     for (int u = 0; u < U; u++) {
       if constexpr (INT4) {
@@ -1254,7 +1331,7 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
           sa[mt] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < 4; s++) {
-            const uint4 a = live[u] ? araw[u][mt][s] : make_uint4(0, 0, 0, 0);
+            const uint4 a = live[u][0] ? araw[u][mt][s] : make_uint4(0, 0, 0, 0);
             const uint4 q = make_uint4(__builtin_amdgcn_perm(a.z, a.x, 0x05040100u), __builtin_amdgcn_perm(a.z, a.x, 0x07060302u),
                                        __builtin_amdgcn_perm(a.w, a.y, 0x05040100u), __builtin_amdgcn_perm(a.w, a.y, 0x07060302u));
             af[mt][s] = __builtin_bit_cast(v8bf, q);
@@ -1303,7 +1380,7 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-          for (int s = 0; s < 4; s++) af[mt][s] = __builtin_bit_cast(v8bf, live[u] ? araw[u][mt][s] : make_uint4(0, 0, 0, 0));
+          for (int s = 0; s < 4; s++) af[mt][s] = __builtin_bit_cast(v8bf, live[u][NIB ? 0 : s / 2] ? araw[u][mt][s] : make_uint4(0, 0, 0, 0));
 #pragma unroll
         for (int t = 0; t < NT; t++) {
           v8bf wf[4], uf[4];
@@ -1548,15 +1625,15 @@ static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int ma
   }
 }
 
-template <int FMT, int MT, int KSPLIT, int NT, int U>
+template <int FMT, int MT, int KSPLIT, int NT, int U, bool STREAM>
 static int launch_wq_skinny_k(WqSkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
   p.n_blocks = cdiv(p.N, (4 / KSPLIT) * 16 * NT);
   const long long blocks = (long long)max_tiles * p.n_blocks;
   if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
   if (glu)
-    gmm_wq_skinny_kernel<FMT, MT, NT, true, U, KSPLIT><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<FMT, MT, NT, true, U, KSPLIT, STREAM><<<(unsigned)blocks, 256, 0, s>>>(p);
   else
-    gmm_wq_skinny_kernel<FMT, MT, NT, false, U, KSPLIT><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<FMT, MT, NT, false, U, KSPLIT, STREAM><<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_launch("gmm_wq_skinny_kernel");
 }
 
@@ -1564,9 +1641,13 @@ static int launch_wq_skinny_k(WqSkinnyParams p, bool glu, int max_tiles, hipStre
 // instead (measured slower up to 32 rows per expert; kept as a tuning aid).
 template <int FMT, int MT>
 static int launch_wq_skinny(const WqSkinnyParams& p, bool glu, int max_tiles, int tune, hipStream_t s) {
-  constexpr int U = MT == 1 ? 3 : 2;  // k-blocks per round
-  if (tune == 1) return launch_wq_skinny_k<FMT, MT, 1, 2, U>(p, glu, max_tiles, s);
-  return launch_wq_skinny_k<FMT, MT, 4, 2, U>(p, glu, max_tiles, s);
+  // k-blocks per round: 2.  More raw bytes in flight per wave cost registers, and the occupancy lost with them costs
+  // more than the longer rounds gain (4 measured 30-50 % slower on the 4-bit formats).  Weights are requested as
+  // ordinary loads: at decode sizes of a few hundred MB part of them is served by the last-level cache on the next
+  // call, which a non-temporal request gives up; past those sizes the two measure the same.
+  constexpr int U = 2;
+  if (tune == 1) return launch_wq_skinny_k<FMT, MT, 1, 2, U, false>(p, glu, max_tiles, s);
+  return launch_wq_skinny_k<FMT, MT, 4, 2, U, false>(p, glu, max_tiles, s);
 }
 
 }  // namespace moe
@@ -1614,6 +1695,7 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     if (a->lhs_scale_block_k != 128 || a->rhs_scale_block_k != 128 || a->rhs_scale_block_n != 128 || !a->lhs_scale || !a->rhs_scale || (glu && !a->rhs_up_scale))
       return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs 1x128 lhs scales and 128x128 rhs scales");
     if (a->K % 128 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs K %% 128 == 0 (K=%d)", a->K);
+    if ((long long)a->N * a->K >= (1LL << 31)) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs N * K < 2^31");
     // Few rows per expert (decode): 16-row tiles, one MFMA row tile per wave.  A group with more rows
     // simply gets several tiles; they are adjacent in the grid, run at the same time and share the group's
     // weights through L2.  Many rows per expert: 64-row tiles.
@@ -1678,7 +1760,8 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   const int M = a->M, G = a->num_groups_total;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
-  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->K % 32 == 0 && a->reserved[0] != 1) {
+  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->K % 32 == 0 && a->reserved[0] != 1 &&
+      (long long)a->N * a->K < (1LL << 31)) {
     const bool one = (long long)M <= 16LL * G;
     bm = one ? 16 : 32;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
