@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 # scaled by a 1 GiB copy dispatch of the same run (profiles/pmc_traffic_*.md); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
     "c2": (2335090 * 2.0 + 459081 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
-    "c3": (3829460 * 2.0 + 9218 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
+    "c3": (3852849 * 2.0 + 9236 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
     "c2_train": (3100853 * 2.0 + 917551 * 1.0) * 1024,  # profiles/tgmm_kernel_bf16_mixtral_shape_train.md
 }
 

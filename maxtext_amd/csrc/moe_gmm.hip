@@ -1150,10 +1150,14 @@ __device__ __forceinline__ void widen32(const WqRaw<FMT>& raw, float scale, v8bf
 // requests per 16 channels, like load_w128 of the fp8 kernel; 4-bit formats therefore walk K in pairs of blocks
 // (U even) and keep the k order inside a block, int8 gets the order (kq*16.., 64 + kq*16..) inside its block and
 // reads its activations to match.
-template <int FMT, int MT, int NT, bool GLU, int U, int KSPLIT, bool STREAM, bool PREFETCH>
+//
+// LINE = false (4-bit formats only) is the plain form: one 16-byte request per lane and k-block, 64 bytes per
+// channel per request, no exchange, any U.
+template <int FMT, int MT, int NT, bool GLU, int U, int KSPLIT, bool STREAM, bool PREFETCH, bool LINE>
 __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams p) {
   constexpr bool INT4 = FMT == WQ_I4, MX4 = FMT == WQ_MX4, G32 = FMT == WQ_I4G32, NIB = FMT != WQ_I8;
-  constexpr int UB = NIB ? 2 : 1;  // k-blocks per 128-byte unit of a weight row
+  static_assert(LINE || NIB, "int8 always uses whole-line requests");
+  constexpr int UB = NIB && LINE ? 2 : 1;  // k-blocks per weight request pair
   static_assert(U % UB == 0, "4-bit formats are loaded in pairs of k-blocks");
   constexpr int NACC = NT * MT * 4 * (GLU ? 2 : 1);
   constexpr int NSUB = 4 / KSPLIT;  // channel groups per block
@@ -1197,7 +1201,7 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
   for (int t = 0; t < NT; t++) {
     const int nw = min(n_w + t * 16 + j, N - 1);
     const size_t row = (size_t)tile.group * N + nw;
-    wlo[t] = (uint32_t)min(n_w + t * 16 + j % 8, N - 1) * (uint32_t)wrow_bytes;
+    wlo[t] = (uint32_t)min(n_w + t * 16 + (LINE ? j % 8 : j), N - 1) * (uint32_t)wrow_bytes;
     whi[t] = (uint32_t)min(n_w + t * 16 + j % 8 + 8, N - 1) * (uint32_t)wrow_bytes;
     wsp[t] = INT4 ? (const uint16_t*)p.rhs_scale + row * nkb : nullptr;
     usp[t] = INT4 && GLU ? (const uint16_t*)p.rhs_up_scale + row * nkb : nullptr;
@@ -1246,17 +1250,17 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
 #pragma unroll
     for (int un = 0; un < U / UB; un++) {
       // the piece of the unit this lane asks for: a whole block of a 4-bit format, half a block of int8
-      const int kbp_raw = kb0 + un * UB + (NIB ? piece : 0);
+      const int kbp_raw = kb0 + un * UB + (NIB && LINE ? piece : 0);
       const int kbp = kbp_raw < kb_end ? kbp_raw : max(kb_end - 1, 0);
-      const int kp = lane_k(kbp, piece);
+      const int kp = lane_k(kbp, LINE ? piece : 0);
       const uint32_t woff = kp < K ? (uint32_t)(NIB ? kp / 2 : kp) : 0u;
 #pragma unroll
       for (int t = 0; t < NT; t++) {
         r.wa[un][t] = load_w16<STREAM>(wbase + wlo[t] + woff);
-        r.wb[un][t] = load_w16<STREAM>(wbase + whi[t] + woff);
+        if (LINE) r.wb[un][t] = load_w16<STREAM>(wbase + whi[t] + woff);
         if (GLU) {
           r.ua[un][t] = load_w16<STREAM>(ubase + wlo[t] + woff);
-          r.ub[un][t] = load_w16<STREAM>(ubase + whi[t] + woff);
+          if (LINE) r.ub[un][t] = load_w16<STREAM>(ubase + whi[t] + woff);
         }
       }
     }
@@ -1314,14 +1318,19 @@ __global__ __launch_bounds__(256) void gmm_wq_skinny_kernel(const WqSkinnyParams
     for (int un = 0; un < U / UB; un++)
 #pragma unroll
       for (int t = 0; t < NT; t++) {
-        v4i x, y;
-        own_channel_pieces(r.wa[un][t], r.wb[un][t], x, y);
-        wraw[un * UB][t].q0 = __builtin_bit_cast(uint4, x);
-        (NIB ? wraw[un * UB + UB - 1][t].q0 : wraw[un][t].q1) = __builtin_bit_cast(uint4, y);
-        if (GLU) {
-          own_channel_pieces(r.ua[un][t], r.ub[un][t], x, y);
-          uraw[un * UB][t].q0 = __builtin_bit_cast(uint4, x);
-          (NIB ? uraw[un * UB + UB - 1][t].q0 : uraw[un][t].q1) = __builtin_bit_cast(uint4, y);
+        if constexpr (!LINE) {
+          wraw[un][t].q0 = __builtin_bit_cast(uint4, r.wa[un][t]);
+          if (GLU) uraw[un][t].q0 = __builtin_bit_cast(uint4, r.ua[un][t]);
+        } else {
+          v4i x, y;
+          own_channel_pieces(r.wa[un][t], r.wb[un][t], x, y);
+          wraw[un * UB][t].q0 = __builtin_bit_cast(uint4, x);
+          (NIB ? wraw[un * UB + UB - 1][t].q0 : wraw[un][t].q1) = __builtin_bit_cast(uint4, y);
+          if (GLU) {
+            own_channel_pieces(r.ua[un][t], r.ub[un][t], x, y);
+            uraw[un * UB][t].q0 = __builtin_bit_cast(uint4, x);
+            (NIB ? uraw[un * UB + UB - 1][t].q0 : uraw[un][t].q1) = __builtin_bit_cast(uint4, y);
+          }
         }
       }
 #pragma unroll
@@ -1651,20 +1660,23 @@ static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int ma
   }
 }
 
-template <int FMT, int MT, int KSPLIT, int NT, int U, bool STREAM>
+template <int FMT, int MT, int KSPLIT, int NT, int U, bool LINE = true>
 static int launch_wq_skinny_k(WqSkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
   p.n_blocks = cdiv(p.N, (4 / KSPLIT) * 16 * NT);
   const long long blocks = (long long)max_tiles * p.n_blocks;
   if (blocks > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  // Weights are requested as ordinary loads: at decode sizes of a few hundred MB part of them is served by the
+  // last-level cache on the next call, which a non-temporal request gives up; past those sizes the two measure the same.
+  constexpr bool STREAM = false;
   // Requesting the next round's weights early pays where the extra registers leave the occupancy as it is
   // (measured: MXFP4 and group-32 int4 8 % faster, group-128 int4 without GLU 10 %; with GLU it drops to one wave
   // per SIMD and runs 25 % slower, int8 10 % slower).
-  constexpr bool PF_GLU = MT == 1 && (FMT == WQ_MX4 || FMT == WQ_I4G32);
-  constexpr bool PF_PLAIN = MT == 1 && FMT != WQ_I8;
+  constexpr bool PF_GLU = LINE && MT == 1 && (FMT == WQ_MX4 || FMT == WQ_I4G32);
+  constexpr bool PF_PLAIN = LINE && MT == 1 && FMT != WQ_I8;
   if (glu)
-    gmm_wq_skinny_kernel<FMT, MT, NT, true, U, KSPLIT, STREAM, PF_GLU><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<FMT, MT, NT, true, U, KSPLIT, STREAM, PF_GLU, LINE><<<(unsigned)blocks, 256, 0, s>>>(p);
   else
-    gmm_wq_skinny_kernel<FMT, MT, NT, false, U, KSPLIT, STREAM, PF_PLAIN><<<(unsigned)blocks, 256, 0, s>>>(p);
+    gmm_wq_skinny_kernel<FMT, MT, NT, false, U, KSPLIT, STREAM, PF_PLAIN, LINE><<<(unsigned)blocks, 256, 0, s>>>(p);
   return check_launch("gmm_wq_skinny_kernel");
 }
 
@@ -1673,12 +1685,16 @@ static int launch_wq_skinny_k(WqSkinnyParams p, bool glu, int max_tiles, hipStre
 template <int FMT, int MT>
 static int launch_wq_skinny(const WqSkinnyParams& p, bool glu, int max_tiles, int tune, hipStream_t s) {
   // k-blocks per round: 2.  More raw bytes in flight per wave cost registers, and the occupancy lost with them costs
-  // more than the longer rounds gain (4 measured 30-50 % slower on the 4-bit formats).  Weights are requested as
-  // ordinary loads: at decode sizes of a few hundred MB part of them is served by the last-level cache on the next
-  // call, which a non-temporal request gives up; past those sizes the two measure the same.
+  // more than the longer rounds gain (4 measured 30-50 % slower on the 4-bit formats).
   constexpr int U = 2;
-  if (tune == 1) return launch_wq_skinny_k<FMT, MT, 1, 2, U, false>(p, glu, max_tiles, s);
-  return launch_wq_skinny_k<FMT, MT, 4, 2, U, false>(p, glu, max_tiles, s);
+  if (tune == 1) return launch_wq_skinny_k<FMT, MT, 1, 2, U>(p, glu, max_tiles, s);
+  if constexpr (FMT == WQ_I4 && MT == 1) {
+    // Group-128 int4 with fused GLU holds the most registers of all variants and cannot afford the early request.
+    // When the rows of the matrix do not start on 128-byte lines anyway (GPT-OSS: 1440-byte rows), rounds of three
+    // k-blocks with plain 64-byte requests measure 8 % faster than rounds of two with request pairs.
+    if (glu && (p.K / 2) % 128 != 0) return launch_wq_skinny_k<FMT, MT, 4, 2, 3, false>(p, glu, max_tiles, s);
+  }
+  return launch_wq_skinny_k<FMT, MT, 4, 2, U>(p, glu, max_tiles, s);
 }
 
 }  // namespace moe
