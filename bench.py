@@ -44,6 +44,8 @@ def parse():
   ap.add_argument("--gate", action="store_true",
                   help="include the router in the step: gate matmul + top-k from x (moe_gate_route) instead of given logits")
   ap.add_argument("--graph", action="store_true", help="replay the layer as one captured HIP graph (launch-bound shapes)")
+  ap.add_argument("--cold", action="store_true",
+                  help="overwrite 1 GiB between steps so that no weights survive in the last-level cache (decode sizes)")
   ap.add_argument("--train", action="store_true",
                   help="forward + backward of the layer with bf16 weights of the workload's shape (weight and input gradients)")
   ap.add_argument("--calibrate-copy", action="store_true",
@@ -302,13 +304,28 @@ def main():
   torch.cuda.synchronize()
 
   routed.profile_events = []
-  t0 = time.perf_counter()
-  for _ in range(args.steps):
-    out = step()
-  torch.cuda.synchronize()
-  elapsed = time.perf_counter() - t0
+  if args.cold:
+    # decode-sized weights (C5: 0.4 GB) partly survive in the 256 MB last-level cache from one step to the next;
+    # overwriting 1 GiB between steps makes every step start cold.  Steps are timed one by one with events.
+    scratch = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in marks:
+      scratch.add_(1)
+      a.record()
+      out = step()
+      b.record()
+    torch.cuda.synchronize()
+    elapsed = sum(a.elapsed_time(b) for a, b in marks) * 1e-3
+  else:
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      out = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
   if args.graph:  # per-kernel events cannot be recorded inside a replay: time the same kernels in a few eager steps
     for _ in range(3):
+      if args.cold:
+        scratch.add_(1)
       eager_step()
     torch.cuda.synchronize()
   events = routed.profile_events
@@ -361,6 +378,7 @@ def main():
       "roofline": roofline,
       "stage_ms": stage_ms,
       "graph": bool(args.graph),
+      "cold_cache": bool(args.cold),
       "gate_in_step": bool(args.gate),
       "layer_gbps": None,
   }
