@@ -109,7 +109,7 @@ def cpu_baseline(wl, layer, sample_tokens):
               seconds=dt)
 
 
-def calibration(dtype_name):
+def calibration(dtype_name, vendor_gemm_shape=None):
   """What this machine sustains on the two roofs, measured with the library's calibration kernels: a register-only
   MFMA loop (operands constant / changing every instruction: changing data draws more power and lowers the clock)
   and a plain streaming read of 2 GiB.  Reported beside the roofline, whose `peak` stays the published figure."""
@@ -147,6 +147,18 @@ def calibration(dtype_name):
   ms = best_ms(lambda: _lib.check(lib.moe_calib_read(_lib.ptr(buf), buf.numel(), _lib.ptr(scratch), stream), "moe_calib_read"))
   res["hbm_read_gbs"] = buf.numel() / ms / 1e6
   del buf
+  if vendor_gemm_shape is not None and code == _lib.MOE_INT8:
+    # The vendor library's dense int8 GEMM (hipBLASLt behind torch._int_mm) at the shape of the dominant launch, with no
+    # grouping, scales or activation: what a tuned kernel sustains on this box under the same power limit.
+    m, k, n = vendor_gemm_shape
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    a = torch.randint(-127, 128, (m, k), device="cuda", dtype=torch.int8, generator=gen)
+    b = torch.randint(-127, 128, (n, k), device="cuda", dtype=torch.int8, generator=gen)
+    try:
+      ms = best_ms(lambda: torch._int_mm(a, b.t()))
+      res["vendor_int8_gemm"] = {"tops": 2.0 * m * k * n / ms / 1e9, "shape_mkn": [m, k, n]}
+    except Exception as exc:  # the library may lack a solution for a shape; the figure is only a reference point
+      res["vendor_int8_gemm"] = {"error": str(exc)[:120]}
   return res
 
 
@@ -394,10 +406,12 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
-  result["calibration"] = calibration(model["dtype"])
+  vendor_shape = (int(gs.sum()), cfg.emb_dim, 2 * cfg.moe_mlp_dim) if model["dtype"] == "int8" and model["bound"] == "mfma" else None
+  del out
+  torch.cuda.empty_cache()
+  result["calibration"] = calibration(model["dtype"], vendor_shape)
   if not args.no_cpu_baseline:
     sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048, "c5mx": 2048}[wl.name]
-    del out
     result["cpu_baseline"] = cpu_baseline(wl, layer, sample)
   print(json.dumps(result))
 

@@ -305,7 +305,8 @@ MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, si
  * the chip draw more power and lower its clock), and with a plain streaming read.  The caller times the launches.
  *   moe_calib_mfma: dtype MOE_INT8 (v_mfma_i32_32x32x32_i8) or MOE_BF16 (v_mfma_f32_32x32x16_bf16); the launch
  *   performs moe_calib_mfma_ops(dtype, iters) operations.  scratch: moe_calib_scratch_bytes() bytes.
- *   moe_calib_read: reads `bytes` (16-byte aligned, >= 64 KiB) once.
+ *   moe_calib_read: reads `bytes` (16-byte aligned, >= 64 KiB) once, with non-temporal requests that each cover
+ *   whole 128-byte lines (the fastest streaming read on this part).
  */
 MOE_API size_t moe_calib_scratch_bytes(void);
 MOE_API double moe_calib_mfma_ops(int dtype, int iters);

@@ -63,20 +63,20 @@ __global__ __launch_bounds__(256) void calib_mfma_bf16_kernel(int iters, int see
   sink[blockIdx.x * 256 + threadIdx.x] = (int)s;
 }
 
-// every wave reads 4 KB per step, the grid strides over the buffer once
-__global__ __launch_bounds__(256) void calib_read_kernel(const uint4* __restrict__ src, size_t nvec, int* __restrict__ sink) {
-  const size_t stride = (size_t)gridDim.x * 256 * 4;
-  uint4 s = make_uint4(0, 0, 0, 0);
-  for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x / kWave * kWave) * 4 + threadIdx.x % kWave; i + 3 * kWave < nvec; i += stride) {
-    uint4 v[4];
+// every wave reads 8 KB per step with non-temporal requests of 1 KB (whole 128-byte lines: the request shape that
+// streams fastest on this part), the grid strides over the buffer once
+__global__ __launch_bounds__(256) void calib_read_kernel(const v4i* __restrict__ src, size_t nvec, int* __restrict__ sink) {
+  constexpr int U = 8;
+  const size_t stride = (size_t)gridDim.x * 256 * U;
+  v4i s = {0, 0, 0, 0};
+  for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x / kWave * kWave) * U + threadIdx.x % kWave; i + (U - 1) * kWave < nvec; i += stride) {
+    v4i v[U];
 #pragma unroll
-    for (int j = 0; j < 4; j++) v[j] = src[i + j * kWave];
+    for (int j = 0; j < U; j++) v[j] = __builtin_nontemporal_load(src + i + j * kWave);
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      s.x ^= v[j].x; s.y ^= v[j].y; s.z ^= v[j].z; s.w ^= v[j].w;
-    }
+    for (int j = 0; j < U; j++) s ^= v[j];
   }
-  if ((s.x ^ s.y ^ s.z ^ s.w) == 0x12345678u) sink[0] = 1;
+  if ((s[0] ^ s[1] ^ s[2] ^ s[3]) == 0x12345678) sink[0] = 1;
 }
 
 constexpr int kCalibBlocks = 256 * 8;  // 2 waves per SIMD on 256 CUs
@@ -112,7 +112,7 @@ int moe_calib_mfma(int dtype, int random_operands, int iters, void* scratch, voi
 
 int moe_calib_read(const void* src, size_t bytes, void* scratch, void* stream) {
   if (!src || !scratch || bytes < 65536 || ((uintptr_t)src & 15)) return fail(MOE_ERR_INVALID_ARG, "calib_read: bad arguments");
-  calib_read_kernel<<<kCalibBlocks, 256, 0, (hipStream_t)stream>>>((const uint4*)src, bytes / 16, (int*)scratch);
+  calib_read_kernel<<<kCalibBlocks, 256, 0, (hipStream_t)stream>>>((const v4i*)src, bytes / 16, (int*)scratch);
   return check_launch("calib_read_kernel");
 }
 
