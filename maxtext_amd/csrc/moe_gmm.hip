@@ -1066,6 +1066,204 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 }
 
 // ---------------------------------------------------------------------------------------
+// Block-scaled fp8 for many rows per expert (prefill, training batches).  A block owns BM rows x 128 weight
+// rows (with GLU: 64 gate + 64 up channels) and walks K in stages of one 128-wide scale block.  Operands go
+// global -> LDS with global_load_lds_dwordx4 (8 rows x 128 bytes per wave instruction, the 16-byte chunk q of
+// row r stored at slot q ^ ((r >> 1) & 7) so that fragment reads are conflict free), NSTAGE buffers deep.
+// A wave owns 64 rows x 64 weight rows: per stage and 32 x 32 tile two chained v_mfma_f32_32x32x64_f8f6f4
+// produce the block's partial sum, which is multiplied by a_scale[row, kb] * w_scale[n / 128, kb] and added to
+// the f32 result: with weights as the "A" operand a lane holds one row of the tile, so the factor is one
+// scalar per lane and tile.  Two waves per SIMD take turns on the matrix pipe, which hides the scaling FMAs
+// of one behind the MFMAs of the other.
+// ---------------------------------------------------------------------------------------
+
+struct Fp8TiledParams {
+  TiledParams base;        // lhs / rhs / rhs_up fp8; its scale pointers stay NULL (the epilogue applies none)
+  const float* a_scale;    // [M, K/128]
+  const float* w_scale;    // [G, ceil(N/128), K/128]
+  const float* u_scale;
+};
+
+template <int BM_, bool GLU_>
+struct F8Cfg {
+  static constexpr int BM = BM_, BN = 128, BKB = 128;
+  static constexpr bool GLU = GLU_;
+  static constexpr int WAVES_M = BM / 64, WAVES_N = 2, NWAVES = WAVES_M * WAVES_N, THREADS = NWAVES * kWave;
+  static constexpr int NSTAGE = BM == 256 ? 3 : 2;  // 256 rows: one block per CU; 128 rows: two blocks of 64 KB
+  static constexpr int TM = 2, TN = 2;
+  static constexpr int A_IPW = BM / 8 / NWAVES, B_IPW = BN / 8 / NWAVES, LPS = A_IPW + B_IPW;
+  static constexpr int STAGE = (BM + BN) * BKB;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE;
+  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static_assert(BM == 128 || BM == 256, "row tile");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+template <typename C>
+__global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8TiledParams P) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const TiledParams& p = P.base;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
+  const int N = p.N, K = p.K;
+  const int nk = K / 128;
+
+  // block -> (m-tile, n-tile): ids that run at the same time on one XCD (ids congruent mod 8) form a patch of
+  // 4 m-tiles x 8 n-tiles that shares activation and weight panels in that XCD's L2
+  const int total = p.max_m_tiles * p.tiles_n;
+  TileInfo tile;
+  int n0;
+  {
+    const int id = blockIdx.x;
+    const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
+    const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+    constexpr int GSM = 4;
+    const int width = GSM * p.tiles_n;
+    const int sg = logical / width, first_m = sg * GSM;
+    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int m_idx = first_m + (logical % width) % gsz;
+    n0 = ((logical % width) / gsz) * C::OUT_BN;
+    tile = p.tiles[m_idx];  // the slot exists even when the tile does not
+    if (m_idx >= p.header[0]) return;
+  }
+  if (tile.group < 0) {
+    constexpr int QPR = C::OUT_BN / 4;
+    for (int i = tid; i < tile.nrows * QPR; i += C::THREADS) {
+      const int r = i / QPR, c = n0 + (i % QPR) * 4;
+      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  // ---- per-lane sources of this wave's requests: lane l asks for row l / 8, chunk (l % 8) ^ swz(row) -------
+  const uint8_t* a_src[C::A_IPW];
+  const uint8_t* b_src[C::B_IPW];
+#pragma unroll
+  for (int i = 0; i < C::A_IPW; i++) {
+    const int r = (wave * C::A_IPW + i) * 8 + lane / 8;
+    const int q = (lane % 8) ^ ((r >> 1) & 7);
+    a_src[i] = p.lhs + (size_t)(tile.row0 + min(r, tile.nrows - 1)) * K + q * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < C::B_IPW; i++) {
+    const int vr = (wave * C::B_IPW + i) * 8 + lane / 8;
+    const int q = (lane % 8) ^ ((vr >> 1) & 7);
+    const bool up = C::GLU && vr >= C::BN / 2;
+    const int n = min(n0 + (up ? vr - C::BN / 2 : vr), N - 1);
+    b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)tile.group * N + n) * K + q * 16;
+  }
+  auto issue_stage = [&](int kt, int buf) {
+    const size_t koff = (size_t)kt * 128;
+    uint8_t* st = smem + buf * C::STAGE;
+#pragma unroll
+    for (int i = 0; i < C::A_IPW; i++)
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[i] + koff), (lds_ptr_t)(st + (wave * C::A_IPW + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < C::B_IPW; i++)
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
+                                       (lds_ptr_t)(st + C::BM * 128 + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+  };
+
+  // ---- fragments: lane (row = lane % 32, kq = lane / 32) takes chunks 4h + 2kq, 4h + 2kq + 1 of half h ------
+  const int lrow = lane % 32, kq = lane / 32, sw = (lrow >> 1) & 7;
+  int choff[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int e = 0; e < 2; e++) choff[h][e] = lrow * 128 + (((4 * h + 2 * kq + e) ^ sw) * 16);
+  int w_row[2];  // first LDS row of this wave's two weight tiles
+  if (C::GLU) {
+    w_row[0] = wn * 32;
+    w_row[1] = C::BN / 2 + wn * 32;
+  } else {
+    w_row[0] = wn * 64;
+    w_row[1] = wn * 64 + 32;
+  }
+  auto frag = [&](const uint8_t* base, int h) {
+    const v4i a = *(const v4i*)(base + choff[h][0]), b = *(const v4i*)(base + choff[h][1]);
+    v8i r;
+    r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+    r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+    return r;
+  };
+
+  // ---- block scales ---------------------------------------------------------------------------------------
+  const float* as_ptr[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int lr = wm * 64 + i * 32 + lrow;
+    as_ptr[i] = P.a_scale + (size_t)(tile.row0 + min(lr, tile.nrows - 1)) * nk;
+  }
+  const int nnb = (N + 127) / 128;
+  const int n_out0 = n0 + (C::GLU ? wn * 32 : wn * 64);
+  // both weight tiles of a wave lie in one 128-channel block (gate and up have tensors of their own)
+  const float* ws_ptr[2];
+  ws_ptr[0] = P.w_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nk;
+  ws_ptr[1] = C::GLU ? P.u_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nk
+                     : P.w_scale + ((size_t)tile.group * nnb + min(n_out0 + 32, N - 1) / 128) * nk;
+
+  v16f fin[2][2];
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) fin[j][i][r] = 0.f;
+  const v16f zero = fin[0][0];
+
+  // ---- pipeline: stage kt is multiplied while stages kt+1 .. kt+NSTAGE-1 travel ---------------------------
+  float as_cur[2] = {as_ptr[0][0], as_ptr[1][0]};
+#pragma unroll
+  for (int s = 0; s < C::NSTAGE - 1; s++) issue_stage(min(s, nk - 1), s);
+  for (int kt = 0; kt < nk; kt++) {
+    const int buf = kt % C::NSTAGE;
+    // own requests of stage kt have landed (the newest NSTAGE-2 stages may still travel), then everybody's have,
+    // and nobody reads stage kt-1 any more
+    wait_vmcnt<(C::NSTAGE - 2) * C::LPS>();
+    asm volatile("s_barrier" ::: "memory");
+    float as_next[2];
+    const int kn = min(kt + 1, nk - 1);
+    as_next[0] = as_ptr[0][kn];
+    as_next[1] = as_ptr[1][kn];
+    const float ws0 = ws_ptr[0][kt], ws1 = ws_ptr[1][kt];
+    // (whatever order the compiler gives these loads and the requests below, stage kt+1 is older than the newest
+    // LPS operations when the next iteration waits)
+    const int kl = kt + C::NSTAGE - 1;
+    issue_stage(min(kl, nk - 1), kl % C::NSTAGE);
+
+    const uint8_t* st = smem + buf * C::STAGE;
+    v8i tf[2][2], wf[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) tf[i][h] = frag(st + (wm * 64 + i * 32) * 128, h);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) wf[j][h] = frag(st + (C::BM + w_row[j]) * 128, h);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], tf[i][0], zero, 0, 0, 0, 127, 0, 127);
+        t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], tf[i][1], t, 0, 0, 0, 127, 0, 127);
+        const float sc = as_cur[i] * (j == 0 ? ws0 : ws1);
+#pragma unroll
+        for (int r = 0; r < 16; r++) fin[j][i][r] = fmaf(t[r], sc, fin[j][i][r]);
+      }
+    as_cur[0] = as_next[0];
+    as_cur[1] = as_next[1];
+  }
+  wait_vmcnt<0>();  // the last requests re-read the final stage into a buffer nobody reads
+
+  constexpr int NT_OUT = C::GLU ? 1 : 2;
+  EpilogueScales<2, NT_OUT, C::GLU> esc;
+  load_epilogue_scales<2, NT_OUT, C::GLU, false>(esc, p, tile, wm * 64, n_out0, lane);
+  store_epilogue<2, 2, NT_OUT, C::GLU>(fin, esc, p, tile, wm * 64, n_out0, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Weight-only int8 / int4 for few rows per expert (decode): bf16 activations, weights widened to bf16 in
 // registers, v_mfma_f32_16x16x32_bf16.  Same streaming structure as the fp8 kernel: no LDS, one wave owns
 // 16*NT output channels and walks K in 128-element blocks; lane (n = lane%16, kq = lane/16) holds 32 k values
@@ -1631,6 +1829,19 @@ static int launch_tiled_glu(const TiledParams& p, bool glu, int M, int G_total, 
              : launch_tiled_by_rows<OP, BSRC, false>(p, M, G_total, bm_out, dry, s);
 }
 
+template <int BM, bool GLU>
+static int launch_fp8_tiled(Fp8TiledParams P, int M, int G_total, hipStream_t s) {
+  using C = F8Cfg<BM, GLU>;
+  static bool attr_set[kMaxDevices] = {};
+  if (int st = reserve_lds(gmm_fp8_tiled_kernel<C>, C::LDS_BYTES, attr_set)) return st;
+  P.base.max_m_tiles = max_tiles_for(M, G_total, BM);
+  P.base.tiles_n = cdiv(P.base.N, C::OUT_BN);
+  const long long tiles = (long long)P.base.max_m_tiles * P.base.tiles_n;
+  if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  gmm_fp8_tiled_kernel<C><<<(unsigned)tiles, C::THREADS, C::LDS_BYTES, s>>>(P);
+  return check_launch("gmm_fp8_tiled_kernel");
+}
+
 template <int MT, int NT, int U>
 static int launch_skinny(SkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
   p.n_blocks = cdiv(p.N, 64 * NT);
@@ -1743,10 +1954,32 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
       return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs 1x128 lhs scales and 128x128 rhs scales");
     if (a->K % 128 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs K %% 128 == 0 (K=%d)", a->K);
     if ((long long)a->N * a->K >= (1LL << 31)) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs N * K < 2^31");
-    // Few rows per expert (decode): 16-row tiles, one MFMA row tile per wave.  A group with more rows
-    // simply gets several tiles; they are adjacent in the grid, run at the same time and share the group's
-    // weights through L2.  Many rows per expert: 64-row tiles.
+    // Up to 16 rows per expert on average (decode): the streaming kernel with 16-row tiles, one MFMA row tile per
+    // wave; a group with more rows simply gets several tiles, which are adjacent in the grid, run at the same time
+    // and share the group's weights through L2.  Beyond that the LDS-tiled kernel (measured crossover at 16 rows
+    // per expert on 256 experts of 7168 x 2048; 128-row tiles with two blocks per CU beat 256-row tiles with one
+    // at every size measured).  reserved[0] = 1 / 2 / 3 forces the streaming kernel (64-row tiles past 16 rows per
+    // expert) / 128-row tiles / 256-row tiles (tuning aid).
+    const int forced = a->reserved[0] >= 1 && a->reserved[0] <= 3 ? a->reserved[0] : 0;
     const bool few_rows = (long long)a->M <= 16LL * a->num_groups_total;
+    const bool tiled = forced ? forced >= 2 : !few_rows;
+    if (tiled) {
+      bm = forced == 3 ? 256 : 128;
+      tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);
+      Fp8TiledParams P;
+      TiledParams& q = P.base;
+      q.lhs = (const uint8_t*)a->lhs; q.lhs_scale = nullptr;
+      q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
+      q.rhs_scale = nullptr; q.rhs_up_scale = nullptr;
+      q.rhs_bias = a->rhs_bias; q.rhs_up_bias = a->rhs_up_bias;
+      q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
+      q.header = header; q.tiles = tiles; q.out = (uint16_t*)a->out;
+      q.M = a->M; q.K = a->K; q.N = a->N; q.max_m_tiles = 0; q.tiles_n = 0;
+      q.act = a->act; q.act_limit = a->act_limit; q.tune = 0; q.i4_group = 0;
+      P.a_scale = a->lhs_scale; P.w_scale = (const float*)a->rhs_scale; P.u_scale = (const float*)a->rhs_up_scale;
+      if (bm == 256) return glu ? launch_fp8_tiled<256, true>(P, a->M, a->num_groups_total, s) : launch_fp8_tiled<256, false>(P, a->M, a->num_groups_total, s);
+      return glu ? launch_fp8_tiled<128, true>(P, a->M, a->num_groups_total, s) : launch_fp8_tiled<128, false>(P, a->M, a->num_groups_total, s);
+    }
     bm = few_rows ? 16 : 64;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);
     SkinnyParams p;
@@ -1760,8 +1993,9 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     p.act = a->act; p.act_limit = a->act_limit;
     const int mx = max_tiles_for(a->M, a->num_groups_total, bm);
     p.min_rows = 1; p.max_rows = bm;
-    if (few_rows) return launch_skinny_variant<1>(a->reserved[0], p, glu, mx, s);
-    return launch_skinny_variant<4>(a->reserved[0], p, glu, mx, s);
+    const int variant = a->reserved[0] > 100 ? a->reserved[0] : 0;
+    if (few_rows) return launch_skinny_variant<1>(variant, p, glu, mx, s);
+    return launch_skinny_variant<4>(variant, p, glu, mx, s);
   }
 
   TiledParams p;

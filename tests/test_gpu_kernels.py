@@ -334,11 +334,14 @@ FP8_SHAPES = [
     (256, 1024, 384, [8] * 32),
     (200, 512, 200, [100, 60, 40]),
     (300, 384, 256, [5, 290]),
+    (1500, 640, 456, [700, 0, 333, 300, 1, 166]),
 ]
 
 
+# 0: the kernel the library picks for the shape; 1: streaming kernel; 2 / 3: LDS-tiled kernel with 128 / 256 row tiles
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("m,k,n,gs", FP8_SHAPES)
-def test_gmm_fp8_block_scaled(K, m, k, n, gs):
+def test_gmm_fp8_block_scaled(K, m, k, n, gs, variant):
   lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 6)
   aq, asc = O.quantize_fp8_blocks(lhs, 1, 128)
   wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)  # [g, n, k], scale [g, n/128, k/128]
@@ -348,12 +351,12 @@ def test_gmm_fp8_block_scaled(K, m, k, n, gs):
     return torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
 
   got = K.gmm_raw(cuda(aq), cuda(wq), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc), lhs_scale_block_k=128,
-                  rhs_scale_block_n=128, rhs_scale_block_k=128)
+                  rhs_scale_block_n=128, rhs_scale_block_k=128, tile_variant=variant)
   want = O.gmm(aq, wq, gs, lhs_scale=asc, rhs_scale=v2(wsc), transpose_rhs=True, quant_block=128)
   assert relerr(got, want) <= TOL
   assert torch.all(got[int(gs.sum()):] == 0)
   got = K.gmm_raw(cuda(aq), cuda(wq), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc), rhs_up=cuda(uq), rhs_up_scale=cuda(usc),
-                  lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128, act="silu")
+                  lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128, act="silu", tile_variant=variant)
   want = O.apply_ffn_activation(
       O.gmm(aq, wq, gs, lhs_scale=asc, rhs_scale=v2(wsc), transpose_rhs=True, quant_block=128, out_dtype=torch.float32),
       O.gmm(aq, uq, gs, lhs_scale=asc, rhs_scale=v2(usc), transpose_rhs=True, quant_block=128, out_dtype=torch.float32))
