@@ -14,6 +14,8 @@
 //   gmm_fp8_skinny_kernel  block-scaled fp8 for few rows per expert (decode): no LDS, every wave
 //                     streams 16 weight rows through v_mfma_f32_16x16x128_f8f6f4 and applies the
 //                     per-128 K-block scales to the f32 partial sums.
+//   gmm_fp8_tiled_kernel   block-scaled fp8 for many rows per expert (prefill): 128 x 128 tiles through LDS,
+//                     v_mfma_f32_32x32x64_f8f6f4, one scaled accumulation per 128-wide K block.
 //   gmm_wq_skinny_kernel   the same streaming design for bf16 activations x int8 / int4 / mxfp4 weights,
 //                     with K split over the waves of a block.
 
@@ -1213,6 +1215,17 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
   const v16f zero = fin[0][0];
 
   // ---- pipeline: stage kt is multiplied while stages kt+1 .. kt+NSTAGE-1 travel ---------------------------
+  // The partial sums of a stage stay in `part` until the next stage: each tile's scaling FMAs are issued right
+  // before that tile's next pair of MFMAs, so they run in the shadow of the previous tile's MFMAs.
+  v16f part[2][2];
+  float sc[2][2];
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      part[j][i] = zero;
+      sc[j][i] = 0.f;
+    }
   float as_cur[2] = {as_ptr[0][0], as_ptr[1][0]};
 #pragma unroll
   for (int s = 0; s < C::NSTAGE - 1; s++) issue_stage(min(s, nk - 1), s);
@@ -1226,7 +1239,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
     const int kn = min(kt + 1, nk - 1);
     as_next[0] = as_ptr[0][kn];
     as_next[1] = as_ptr[1][kn];
-    const float ws0 = ws_ptr[0][kt], ws1 = ws_ptr[1][kt];
+    const float ws[2] = {ws_ptr[0][kt], ws_ptr[1][kt]};
     // (whatever order the compiler gives these loads and the requests below, stage kt+1 is older than the newest
     // LPS operations when the next iteration waits)
     const int kl = kt + C::NSTAGE - 1;
@@ -1246,15 +1259,21 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int i = 0; i < 2; i++) {
-        v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], tf[i][0], zero, 0, 0, 0, 127, 0, 127);
-        t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], tf[i][1], t, 0, 0, 0, 127, 0, 127);
-        const float sc = as_cur[i] * (j == 0 ? ws0 : ws1);
 #pragma unroll
-        for (int r = 0; r < 16; r++) fin[j][i][r] = fmaf(t[r], sc, fin[j][i][r]);
+        for (int r = 0; r < 16; r++) fin[j][i][r] = fmaf(part[j][i][r], sc[j][i], fin[j][i][r]);
+        v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], tf[i][0], zero, 0, 0, 0, 127, 0, 127);
+        part[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], tf[i][1], t, 0, 0, 0, 127, 0, 127);
+        sc[j][i] = as_cur[i] * ws[j];
       }
     as_cur[0] = as_next[0];
     as_cur[1] = as_next[1];
   }
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) fin[j][i][r] = fmaf(part[j][i][r], sc[j][i], fin[j][i][r]);
   wait_vmcnt<0>();  // the last requests re-read the final stage into a buffer nobody reads
 
   constexpr int NT_OUT = C::GLU ? 1 : 2;
