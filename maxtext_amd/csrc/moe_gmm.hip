@@ -1086,19 +1086,24 @@ struct Fp8TiledParams {
   const float* u_scale;
 };
 
-template <int BM_, bool GLU_>
+template <int BM_, int BKB_, int NSTAGE_, bool GLU_>
 struct F8Cfg {
-  static constexpr int BM = BM_, BN = 128, BKB = 128;
+  static constexpr int BM = BM_, BN = 128, BKB = BKB_, NSTAGE = NSTAGE_;
   static constexpr bool GLU = GLU_;
   static constexpr int WAVES_M = BM / 64, WAVES_N = 2, NWAVES = WAVES_M * WAVES_N, THREADS = NWAVES * kWave;
-  static constexpr int NSTAGE = BM == 256 ? 3 : 2;  // 256 rows: one block per CU; 128 rows: two blocks of 64 KB
   static constexpr int TM = 2, TN = 2;
-  static constexpr int A_IPW = BM / 8 / NWAVES, B_IPW = BN / 8 / NWAVES, LPS = A_IPW + B_IPW;
+  static constexpr int CPR = BKB / 16;     // 16-byte chunks per LDS row
+  static constexpr int RPI = 1024 / BKB;   // rows per wave instruction
+  static constexpr int SUBS = BKB / 64;    // MFMA k-steps (64 bytes of K) per stage
+  static constexpr int A_IPW = BM / RPI / NWAVES, B_IPW = BN / RPI / NWAVES, LPS = A_IPW + B_IPW;
   static constexpr int STAGE = (BM + BN) * BKB;
   static constexpr int LDS_BYTES = NSTAGE * STAGE;
   static constexpr int OUT_BN = GLU ? BN / 2 : BN;
   static_assert(BM == 128 || BM == 256, "row tile");
+  static_assert(BKB == 64 || BKB == 128, "stage depth");
+  static_assert(NSTAGE >= 2 && (NSTAGE - 2) * LPS < 64, "vmcnt range");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+  __device__ static __forceinline__ int swz(int row) { return BKB == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
 };
 
 template <typename C>
@@ -1109,7 +1114,8 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
   const int N = p.N, K = p.K;
-  const int nk = K / 128;
+  const int nkb = K / 128;          // scale blocks
+  const int nst = K / C::BKB;       // stages
 
   // block -> (m-tile, n-tile): ids that run at the same time on one XCD (ids congruent mod 8) form a patch of
   // 4 m-tiles x 8 n-tiles that shares activation and weight panels in that XCD's L2
@@ -1120,7 +1126,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
     const int id = blockIdx.x;
     const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
-    constexpr int GSM = 4;
+    const int GSM = p.tune > 0 ? p.tune : 4;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
     const int gsz = min(p.max_m_tiles - first_m, GSM);
@@ -1138,25 +1144,25 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
     return;
   }
 
-  // ---- per-lane sources of this wave's requests: lane l asks for row l / 8, chunk (l % 8) ^ swz(row) -------
+  // ---- per-lane sources of this wave's requests: lane l asks for row l / CPR, chunk (l % CPR) ^ swz(row) ----
   const uint8_t* a_src[C::A_IPW];
   const uint8_t* b_src[C::B_IPW];
 #pragma unroll
   for (int i = 0; i < C::A_IPW; i++) {
-    const int r = (wave * C::A_IPW + i) * 8 + lane / 8;
-    const int q = (lane % 8) ^ ((r >> 1) & 7);
+    const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
+    const int q = (lane % C::CPR) ^ C::swz(r);
     a_src[i] = p.lhs + (size_t)(tile.row0 + min(r, tile.nrows - 1)) * K + q * 16;
   }
 #pragma unroll
   for (int i = 0; i < C::B_IPW; i++) {
-    const int vr = (wave * C::B_IPW + i) * 8 + lane / 8;
-    const int q = (lane % 8) ^ ((vr >> 1) & 7);
+    const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
+    const int q = (lane % C::CPR) ^ C::swz(vr);
     const bool up = C::GLU && vr >= C::BN / 2;
     const int n = min(n0 + (up ? vr - C::BN / 2 : vr), N - 1);
     b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)tile.group * N + n) * K + q * 16;
   }
   auto issue_stage = [&](int kt, int buf) {
-    const size_t koff = (size_t)kt * 128;
+    const size_t koff = (size_t)kt * C::BKB;
     uint8_t* st = smem + buf * C::STAGE;
 #pragma unroll
     for (int i = 0; i < C::A_IPW; i++)
@@ -1164,16 +1170,16 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
 #pragma unroll
     for (int i = 0; i < C::B_IPW; i++)
       __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
-                                       (lds_ptr_t)(st + C::BM * 128 + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+                                       (lds_ptr_t)(st + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
   };
 
-  // ---- fragments: lane (row = lane % 32, kq = lane / 32) takes chunks 4h + 2kq, 4h + 2kq + 1 of half h ------
-  const int lrow = lane % 32, kq = lane / 32, sw = (lrow >> 1) & 7;
-  int choff[2][2];
+  // ---- fragments: lane (row = lane % 32, kq = lane / 32) takes chunks 4h + 2kq, 4h + 2kq + 1 of k-step h ----
+  const int lrow = lane % 32, kq = lane / 32, sw = C::swz(lrow);
+  int choff[C::SUBS][2];
 #pragma unroll
-  for (int h = 0; h < 2; h++)
+  for (int h = 0; h < C::SUBS; h++)
 #pragma unroll
-    for (int e = 0; e < 2; e++) choff[h][e] = lrow * 128 + (((4 * h + 2 * kq + e) ^ sw) * 16);
+    for (int e = 0; e < 2; e++) choff[h][e] = lrow * C::BKB + (((4 * h + 2 * kq + e) ^ sw) * 16);
   int w_row[2];  // first LDS row of this wave's two weight tiles
   if (C::GLU) {
     w_row[0] = wn * 32;
@@ -1195,15 +1201,15 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int lr = wm * 64 + i * 32 + lrow;
-    as_ptr[i] = P.a_scale + (size_t)(tile.row0 + min(lr, tile.nrows - 1)) * nk;
+    as_ptr[i] = P.a_scale + (size_t)(tile.row0 + min(lr, tile.nrows - 1)) * nkb;
   }
   const int nnb = (N + 127) / 128;
   const int n_out0 = n0 + (C::GLU ? wn * 32 : wn * 64);
   // both weight tiles of a wave lie in one 128-channel block (gate and up have tensors of their own)
   const float* ws_ptr[2];
-  ws_ptr[0] = P.w_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nk;
-  ws_ptr[1] = C::GLU ? P.u_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nk
-                     : P.w_scale + ((size_t)tile.group * nnb + min(n_out0 + 32, N - 1) / 128) * nk;
+  ws_ptr[0] = P.w_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nkb;
+  ws_ptr[1] = C::GLU ? P.u_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nkb
+                     : P.w_scale + ((size_t)tile.group * nnb + min(n_out0 + 32, N - 1) / 128) * nkb;
 
   v16f fin[2][2];
 #pragma unroll
@@ -1215,8 +1221,9 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
   const v16f zero = fin[0][0];
 
   // ---- pipeline: stage kt is multiplied while stages kt+1 .. kt+NSTAGE-1 travel ---------------------------
-  // The partial sums of a stage stay in `part` until the next stage: each tile's scaling FMAs are issued right
-  // before that tile's next pair of MFMAs, so they run in the shadow of the previous tile's MFMAs.
+  // The partial sum of a 128-wide K block (two k-steps) stays in `part` until the next block starts: each
+  // tile's scaling FMAs are issued right before that tile's first MFMA of the next block, so they run in the
+  // shadow of the previous tile's MFMAs.
   v16f part[2][2];
   float sc[2][2];
 #pragma unroll
@@ -1227,46 +1234,66 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
       sc[j][i] = 0.f;
     }
   float as_cur[2] = {as_ptr[0][0], as_ptr[1][0]};
+  float ws_cur[2] = {ws_ptr[0][0], ws_ptr[1][0]};
 #pragma unroll
-  for (int s = 0; s < C::NSTAGE - 1; s++) issue_stage(min(s, nk - 1), s);
-  for (int kt = 0; kt < nk; kt++) {
-    const int buf = kt % C::NSTAGE;
-    // own requests of stage kt have landed (the newest NSTAGE-2 stages may still travel), then everybody's have,
-    // and nobody reads stage kt-1 any more
+  for (int s = 0; s < C::NSTAGE - 1; s++) issue_stage(min(s, nst - 1), s);
+
+  // Opening stage kt: own requests of stage kt have landed (the newest NSTAGE-2 stages may still travel), then
+  // everybody's have, and nobody reads stage kt-1 any more, so its buffer takes stage kt+NSTAGE-1.  The scales of
+  // the NEXT K block are requested between the barrier and those requests: in vmcnt order they are then older than
+  // the requests that stay in flight, so neither the wait of the next stage nor the compiler's wait for the scale
+  // registers has to drain a stage that is still travelling.
+  float as_next[2], ws_next[2];
+  auto open_stage = [&](int kt, int next_kb) {
     wait_vmcnt<(C::NSTAGE - 2) * C::LPS>();
     asm volatile("s_barrier" ::: "memory");
-    float as_next[2];
-    const int kn = min(kt + 1, nk - 1);
-    as_next[0] = as_ptr[0][kn];
-    as_next[1] = as_ptr[1][kn];
-    const float ws[2] = {ws_ptr[0][kt], ws_ptr[1][kt]};
-    // (whatever order the compiler gives these loads and the requests below, stage kt+1 is older than the newest
-    // LPS operations when the next iteration waits)
+    if (next_kb >= 0) {
+      as_next[0] = as_ptr[0][next_kb];
+      as_next[1] = as_ptr[1][next_kb];
+      ws_next[0] = ws_ptr[0][next_kb];
+      ws_next[1] = ws_ptr[1][next_kb];
+    }
+    asm volatile("" ::: "memory");
     const int kl = kt + C::NSTAGE - 1;
-    issue_stage(min(kl, nk - 1), kl % C::NSTAGE);
-
-    const uint8_t* st = smem + buf * C::STAGE;
-    v8i tf[2][2], wf[2][2];
+    issue_stage(min(kl, nst - 1), kl % C::NSTAGE);
+  };
+  // one k-step (64 bytes of K) of all four tiles; FIRST: it opens a scale block
+  auto kstep = [&](const uint8_t* st, int h, auto first_c) {
+    constexpr bool FIRST = decltype(first_c)::value;
+    v8i tf[2], wf[2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 2; i++) tf[i] = frag(st + (wm * 64 + i * 32) * C::BKB, h);
 #pragma unroll
-      for (int h = 0; h < 2; h++) tf[i][h] = frag(st + (wm * 64 + i * 32) * 128, h);
-#pragma unroll
-    for (int j = 0; j < 2; j++)
-#pragma unroll
-      for (int h = 0; h < 2; h++) wf[j][h] = frag(st + (C::BM + w_row[j]) * 128, h);
+    for (int j = 0; j < 2; j++) wf[j] = frag(st + (C::BM + w_row[j]) * C::BKB, h);
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int i = 0; i < 2; i++) {
+        if (FIRST) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) fin[j][i][r] = fmaf(part[j][i][r], sc[j][i], fin[j][i][r]);
-        v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], tf[i][0], zero, 0, 0, 0, 127, 0, 127);
-        part[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], tf[i][1], t, 0, 0, 0, 127, 0, 127);
-        sc[j][i] = as_cur[i] * ws[j];
+          for (int r = 0; r < 16; r++) fin[j][i][r] = fmaf(part[j][i][r], sc[j][i], fin[j][i][r]);
+          sc[j][i] = as_cur[i] * ws_cur[j];
+        }
+        part[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j], tf[i], FIRST ? zero : part[j][i], 0, 0, 0, 127, 0, 127);
       }
+  };
+  for (int kb = 0; kb < nkb; kb++) {
+    const int kn = min(kb + 1, nkb - 1);
+    if constexpr (C::SUBS == 2) {
+      open_stage(kb, kn);
+      const uint8_t* st = smem + (kb % C::NSTAGE) * C::STAGE;
+      kstep(st, 0, std::true_type{});
+      kstep(st, 1, std::false_type{});
+    } else {
+      open_stage(2 * kb, kn);
+      kstep(smem + ((2 * kb) % C::NSTAGE) * C::STAGE, 0, std::true_type{});
+      open_stage(2 * kb + 1, -1);
+      kstep(smem + ((2 * kb + 1) % C::NSTAGE) * C::STAGE, 0, std::false_type{});
+    }
     as_cur[0] = as_next[0];
     as_cur[1] = as_next[1];
+    ws_cur[0] = ws_next[0];
+    ws_cur[1] = ws_next[1];
   }
 #pragma unroll
   for (int j = 0; j < 2; j++)
@@ -1848,9 +1875,9 @@ static int launch_tiled_glu(const TiledParams& p, bool glu, int M, int G_total, 
              : launch_tiled_by_rows<OP, BSRC, false>(p, M, G_total, bm_out, dry, s);
 }
 
-template <int BM, bool GLU>
+template <int BM, int BKB, int NSTAGE, bool GLU>
 static int launch_fp8_tiled(Fp8TiledParams P, int M, int G_total, hipStream_t s) {
-  using C = F8Cfg<BM, GLU>;
+  using C = F8Cfg<BM, BKB, NSTAGE, GLU>;
   static bool attr_set[kMaxDevices] = {};
   if (int st = reserve_lds(gmm_fp8_tiled_kernel<C>, C::LDS_BYTES, attr_set)) return st;
   P.base.max_m_tiles = max_tiles_for(M, G_total, BM);
@@ -1994,10 +2021,11 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
       q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
       q.header = header; q.tiles = tiles; q.out = (uint16_t*)a->out;
       q.M = a->M; q.K = a->K; q.N = a->N; q.max_m_tiles = 0; q.tiles_n = 0;
-      q.act = a->act; q.act_limit = a->act_limit; q.tune = 0; q.i4_group = 0;
+      q.act = a->act; q.act_limit = a->act_limit; q.tune = a->reserved[1]; q.i4_group = 0;
       P.a_scale = a->lhs_scale; P.w_scale = (const float*)a->rhs_scale; P.u_scale = (const float*)a->rhs_up_scale;
-      if (bm == 256) return glu ? launch_fp8_tiled<256, true>(P, a->M, a->num_groups_total, s) : launch_fp8_tiled<256, false>(P, a->M, a->num_groups_total, s);
-      return glu ? launch_fp8_tiled<128, true>(P, a->M, a->num_groups_total, s) : launch_fp8_tiled<128, false>(P, a->M, a->num_groups_total, s);
+      const int G = a->num_groups_total;
+      if (bm == 256) return glu ? launch_fp8_tiled<256, 128, 3, true>(P, a->M, G, s) : launch_fp8_tiled<256, 128, 3, false>(P, a->M, G, s);
+      return glu ? launch_fp8_tiled<128, 128, 2, true>(P, a->M, G, s) : launch_fp8_tiled<128, 128, 2, false>(P, a->M, G, s);
     }
     bm = few_rows ? 16 : 64;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);

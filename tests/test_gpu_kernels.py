@@ -652,9 +652,10 @@ def test_gmm_bias_every_kernel_family(K, m, k, n, gs):
     v2f = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
     fkw = dict(lhs_scale=cuda(fsc), lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128)
     okw = dict(lhs_scale=fsc, transpose_rhs=True, quant_block=128, out_dtype=torch.float32)
-    check(K.gmm_raw(cuda(fq), cuda(wq), cuda(gs), rhs_scale=cuda(wsc), rhs_up=cuda(uq), rhs_up_scale=cuda(usc), act="swigluoai",
-                    rhs_bias=cuda(b0), rhs_up_bias=cuda(b1), **fkw),
-          act(O.gmm(fq, wq, gs, rhs_scale=v2f(wsc), rhs_bias=ob0, **okw), O.gmm(fq, uq, gs, rhs_scale=v2f(usc), rhs_bias=ob1, **okw)))
+    for variant in (0, 1, 2, 3):  # picked by shape / streaming / LDS-tiled with 128- and 256-row tiles
+      check(K.gmm_raw(cuda(fq), cuda(wq), cuda(gs), rhs_scale=cuda(wsc), rhs_up=cuda(uq), rhs_up_scale=cuda(usc), act="swigluoai",
+                      rhs_bias=cuda(b0), rhs_up_bias=cuda(b1), tile_variant=variant, **fkw),
+            act(O.gmm(fq, wq, gs, rhs_scale=v2f(wsc), rhs_bias=ob0, **okw), O.gmm(fq, uq, gs, rhs_scale=v2f(usc), rhs_bias=ob1, **okw)))
 
 
 def test_gmm_bias_argument_errors(K):
@@ -943,9 +944,10 @@ def test_gmm_partial_sum_every_kernel_family(K, m, k, n, gs):
     fq, fsc = O.quantize_fp8_blocks(lhs, 1, 128)
     wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)
     v2f = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
-    check(K.gmm_raw(cuda(fq), cuda(wq), cuda(gs), lhs_scale=cuda(fsc), rhs_scale=cuda(wsc), lhs_scale_block_k=128, rhs_scale_block_n=128,
-                    rhs_scale_block_k=128, partial_sum=cuda(ps)),
-          O.gmm(fq, wq, gs, lhs_scale=fsc, rhs_scale=v2f(wsc), transpose_rhs=True, quant_block=128, partial_sum=ps))
+    for variant in (0, 1, 2, 3):
+      check(K.gmm_raw(cuda(fq), cuda(wq), cuda(gs), lhs_scale=cuda(fsc), rhs_scale=cuda(wsc), lhs_scale_block_k=128, rhs_scale_block_n=128,
+                      rhs_scale_block_k=128, partial_sum=cuda(ps), tile_variant=variant),
+            O.gmm(fq, wq, gs, lhs_scale=fsc, rhs_scale=v2f(wsc), transpose_rhs=True, quant_block=128, partial_sum=ps))
   with pytest.raises(ValueError):
     K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), partial_sum_up=cuda(ps_up))
 
@@ -1014,3 +1016,22 @@ def test_route_llama4_and_gemma4_weight_rules(K, mode, t, e, k):
     z = np.exp(logits.astype(np.float64) - logits.max(-1, keepdims=True))
     want = np.exp(sel - logits.max(-1, keepdims=True)) / z.sum(-1, keepdims=True)
   np.testing.assert_allclose(w.cpu().numpy(), want, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+def test_gmm_fp8_group_offset_and_kept_rows(K, variant):
+  """Block-scaled fp8 with a shard of the experts (group_offset, ops.py:50): rows of other groups are zero-filled, or keep
+  the buffer's contents with existing_out, in the streaming and in the LDS-tiled kernel."""
+  lhs, w, _, gs = _gmm_inputs(900, 384, 200, [130, 300, 0, 270, 150], 33)
+  aq, asc = O.quantize_fp8_blocks(lhs, 1, 128)
+  wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)
+  v2 = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :200]
+  kw = dict(lhs_scale=cuda(asc), lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128, tile_variant=variant)
+  got = K.gmm_raw(cuda(aq), cuda(wq[1:4]), cuda(gs), rhs_scale=cuda(wsc[1:4]), group_offset=1, **kw)
+  want = O.gmm(aq, wq[1:4], gs, lhs_scale=asc, rhs_scale=v2(wsc[1:4]), transpose_rhs=True, quant_block=128, group_offset=1)
+  assert relerr(got, want) <= TOL
+  assert torch.all(got[:130] == 0) and torch.all(got[700:] == 0)
+  buf = torch.full((900, 200), 3.0, dtype=torch.bfloat16, device="cuda")
+  K.gmm_raw(cuda(aq), cuda(wq[1:4]), cuda(gs), rhs_scale=cuda(wsc[1:4]), group_offset=1, out=buf, keep_other_rows=True, **kw)
+  assert torch.all(buf[:130] == 3.0) and torch.all(buf[700:] == 3.0)
+  assert torch.equal(buf[130:700], got[130:700])
