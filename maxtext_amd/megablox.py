@@ -27,6 +27,7 @@ PROFILE_EVENTS = None
 _INT8_NAMES = ("int8", torch.int8)
 _FP8_NAMES = ("fp8", "float8_e4m3fn", torch.float8_e4m3fn)
 _INT4_NAMES = ("int4",)
+_E5M2_NAMES = ("e5m2", "float8_e5m2", torch.float8_e5m2)
 
 
 def _validate_args(lhs, rhs, group_sizes, expected_rhs_dims=3):
@@ -102,8 +103,12 @@ def gmm(
     rhs_bias=None,
     rhs_up_bias=None,
     partial_sum_up=None,
+    bwd_quantize_dtype=None,
 ):
   """Grouped matmul: out[rows of group g] = lhs[rows] @ rhs[g] (ops.py:46).
+
+  bwd_quantize_dtype: the `bwd_qtype` of the reference's qwix rule (ops.py:97-103, :583-604): "float8_e5m2" quantises
+  the incoming gradient of an int8 x int8 forward per row (for dlhs) and per column (for drhs); None leaves it as is.
 
   lhs: [m, k] bf16 tensor or QArray; rhs: [g, k, n] bf16 ([g, n, k] with transpose_rhs) or a
   QArray holding [G, N, K]; group_sizes: int32 [G_total] on the device.  `tiling`, `interpret`,
@@ -134,7 +139,8 @@ def gmm(
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
     if rhs_bias is not None or rhs_up_bias is not None or partial_sum is not None or partial_sum_up is not None or existing_out is not None:
       raise NotImplementedError("gradients with rhs_bias / partial_sum / existing_out are not implemented")
-    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit)
+    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit,
+                          bwd_quantize_dtype)
 
   rhs_n = _native_rhs(rhs, transpose_rhs)
   up_n = _native_rhs(rhs_up, transpose_rhs) if rhs_up is not None else None
@@ -230,25 +236,93 @@ def tgmm(
   return out.transpose(1, 2)
 
 
+E5M2_MAX = 57344.0  # largest finite float8_e5m2
+
+
+def _quantize_e5m2(x: torch.Tensor, dim: int):
+  """Symmetric absmax float8_e5m2 along `dim` (the gradient quantiser of ops.py:583-604): returns the values on the
+  e5m2 grid as bf16 (exact) and the f32 scale with `dim` kept."""
+  xf = x.float()
+  # the quotient is taken in f64 and rounded once: the device's f32 division is not correctly rounded, and one ulp of
+  # scale moves values across e5m2 rounding boundaries
+  scale = (xf.abs().amax(dim=dim, keepdim=True).double() / E5M2_MAX).float()
+  q = torch.where(scale == 0, torch.zeros_like(xf), xf / scale).to(torch.float8_e5m2).to(torch.bfloat16)
+  return q, scale
+
+
 class _GmmFn(torch.autograd.Function):
   """Differentiable gmm for bf16 operands (custom VJP of ops.py:137-230 / :438-527).
 
-  Forward may quantise its operands on the fly; backward differentiates through the quantisers
-  as identities and uses the bf16 residuals: dlhs = gmm(dout, rhs^T) (ops.py:612-642) and
-  drhs = tgmm(lhs^T, dout) (ops.py:766-796), both without quantisation of the gradient.
+  Unquantised or fp8 forward: backward uses the bf16 residuals, dlhs = gmm(dout, rhs^T) (ops.py:612-642) and
+  drhs = tgmm(lhs^T, dout) (ops.py:766-796); fp8 block scales run along the contracted axis of both products and
+  cannot be folded into the gradient, so the fp8 quantisers are differentiated as identities.
+
+  int8 x int8 forward (channelwise scales): the residuals are the quantised operands and the backward is the
+  reference's (_bwd_prepare_inputs ops.py:530-580): the scale of the axis that disappears goes onto the gradient,
+  dlhs = gmm(dout * rhs_scale[n], rhs_q^T), drhs = tgmm(lhs_q^T, dout * lhs_scale[m]); with bwd_q the two scaled
+  gradients are first quantised to float8_e5m2 per row / per column (_bwd_quantize_gradient ops.py:583-604).  The
+  int8 and e5m2 values are exact in bf16, so both products run on the bf16 MFMA kernels.
   """
 
   @staticmethod
-  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q):
-    ctx.save_for_backward(lhs, rhs, group_sizes)
-    ctx.offset, ctx.transpose_rhs = offset, transpose_rhs
+  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q):
+    ctx.offset, ctx.transpose_rhs, ctx.bwd_q = offset, transpose_rhs, bwd_q
+    ctx.quantized = lhs_q in _INT8_NAMES and rhs_q in _INT8_NAMES
+    if bwd_q is not None and not ctx.quantized:
+      raise NotImplementedError("bwd_quantize_dtype needs the int8 x int8 forward (channelwise scales)")
+    if bwd_q is not None and bwd_q not in _E5M2_NAMES:
+      raise ValueError(f"unsupported bwd_quantize_dtype {bwd_q}")
     with torch.no_grad():
+      if ctx.quantized:
+        lq = quantize_lhs(lhs.contiguous(), lhs_q)
+        rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q)
+        ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes)
+        ctx.rhs_dtype = rhs.dtype
+        return gmm(lq, rq, group_sizes, group_offset=offset, transpose_rhs=True)
+      ctx.save_for_backward(lhs, rhs, group_sizes)
       return gmm(lhs, rhs, group_sizes, group_offset=offset, transpose_rhs=transpose_rhs, lhs_quantize_dtype=lhs_q, rhs_quantize_dtype=rhs_q)
 
   @staticmethod
+  def _backward_quantized(ctx, dout):
+    lq, ls, rq, rs, group_sizes = ctx.saved_tensors  # lq [m,k] i8, ls [m], rq [g,n,k] i8, rs [g,n]
+    m, n = dout.shape
+    g_local = rq.shape[0]
+    dlhs = drhs = None
+    if ctx.needs_input_grad[0]:
+      # expert of every row (rows past the last group take the last expert; their gradient rows are zero anyway)
+      ends = torch.cumsum(group_sizes, 0)
+      row_group = torch.searchsorted(ends, torch.arange(m, device=dout.device, dtype=ends.dtype), right=True)
+      local = (row_group - ctx.offset).clamp_(0, g_local - 1)
+      d = dout * rs.to(dout.dtype)[local]
+      s_row = None
+      if ctx.bwd_q is not None:
+        d, s_row = _quantize_e5m2(d, dim=1)
+      w_t = kernels.transpose_rhs(rq)  # [g, n, k] -> [g, k, n]: the layout with k as the output axis
+      ones = torch.ones((g_local, w_t.shape[1]), dtype=torch.float32, device=dout.device)
+      dlhs = kernels.gmm_raw(d.contiguous(), w_t, group_sizes, rhs_scale=ones, rhs_scale_block_n=1, group_offset=ctx.offset)
+      if s_row is not None:
+        dlhs = (dlhs.float() * s_row).to(torch.bfloat16)
+    if ctx.needs_input_grad[1]:
+      d = dout * ls.to(dout.dtype)[:, None]
+      s_col = None
+      if ctx.bwd_q is not None:
+        d, s_col = _quantize_e5m2(d, dim=0)
+      w = kernels.tgmm(lq.to(torch.bfloat16), d.contiguous(), group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
+                       out_dtype=torch.float32)  # [g, n, k]
+      if s_col is not None:
+        w = w * s_col.reshape(1, n, 1)
+      w = w.to(ctx.rhs_dtype)
+      drhs = w if ctx.transpose_rhs else w.transpose(1, 2)
+    return dlhs, drhs
+
+  @staticmethod
   def backward(ctx, dout):
-    lhs, rhs, group_sizes = ctx.saved_tensors
     dout = dout.contiguous()
+    if ctx.quantized:
+      with torch.no_grad():
+        dlhs, drhs = _GmmFn._backward_quantized(ctx, dout)
+      return dlhs, drhs, None, None, None, None, None, None
+    lhs, rhs, group_sizes = ctx.saved_tensors
     dlhs = drhs = None
     ev = PROFILE_EVENTS
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(3)] if ev is not None else None
@@ -269,7 +343,7 @@ class _GmmFn(torch.autograd.Function):
         shape = f"k{lhs.shape[1]}_n{dout.shape[1]}"
         ev.append(("dlhs_" + shape, marks[0], marks[1]))
         ev.append(("tgmm_" + shape, marks[1], marks[2]))
-    return dlhs, drhs, None, None, None, None, None
+    return dlhs, drhs, None, None, None, None, None, None
 
 
 class _GluFn(torch.autograd.Function):
@@ -288,16 +362,16 @@ class _GluFn(torch.autograd.Function):
     return dh0, dh1, None, None
 
 
-def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit):
+def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit, bwd_q=None):
   for name, t in (("lhs", lhs), ("rhs", rhs), ("rhs_up", rhs_up)):
     if t is not None and not isinstance(t, torch.Tensor):
       raise NotImplementedError(f"gradients need bf16 tensors; {name} is already quantised")
-  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q)
+  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q)
   if rhs_up is None:
     if fuse_act is not None:
       raise ValueError("fuse_act needs rhs_up")
     return h0
-  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q)
+  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q)
   if fuse_act is None:
     raise ValueError("rhs_up needs fuse_act")
   if fuse_act not in ("silu", "swigluoai", "silu_clip"):

@@ -1035,3 +1035,38 @@ def test_gmm_fp8_group_offset_and_kept_rows(K, variant):
   K.gmm_raw(cuda(aq), cuda(wq[1:4]), cuda(gs), rhs_scale=cuda(wsc[1:4]), group_offset=1, out=buf, keep_other_rows=True, **kw)
   assert torch.all(buf[:130] == 3.0) and torch.all(buf[700:] == 3.0)
   assert torch.equal(buf[130:700], got[130:700])
+
+
+@pytest.mark.parametrize("bwd_q", [None, "float8_e5m2"])
+@pytest.mark.parametrize("transpose_rhs", [False, True])
+def test_gmm_quantized_backward(transpose_rhs, bwd_q):
+  """int8 x int8 forward with the reference's backward (ops.py:530-604): quantised residuals, the scale of the
+  contracted axis folded into the gradient, optional e5m2 quantisation of the gradient per row / per column.
+  Compared with the oracle on the oracle's own quantised operands."""
+  from maxtext_amd import megablox
+
+  g = torch.Generator().manual_seed(12)
+  m, k, n = 450, 256, 192
+  gs = np.array([200, 0, 70, 150], np.int32)  # an empty group and 30 trailing rows in no group
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w = (torch.randn(4, k, n, generator=g) * 0.05).to(torch.bfloat16)  # [g, k, n]
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  lq, ls = O.quantize_rows_int8(lhs.float())
+  rq, rs = O.quantize_weight_int8(w.float(), per_expert=False)  # one [n] scale shared by the experts (ops.py:250-260)
+  want_dl, want_dr = O.gmm_bwd_quantized(dout, lq, ls, rq, rs[0], gs, bwd_qtype=None if bwd_q is None else "e5m2")
+  want_out = O.gmm(lq, rq, gs, lhs_scale=ls[:, None], rhs_scale=rs)
+
+  lhs_g = cuda(lhs).requires_grad_()
+  rhs_g = cuda(w.transpose(1, 2).contiguous() if transpose_rhs else w).requires_grad_()
+  out = megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, lhs_quantize_dtype="int8", rhs_quantize_dtype="int8",
+                     bwd_quantize_dtype=bwd_q)
+  assert relerr(out, want_out) <= TOL
+  out.backward(cuda(dout))
+  tol = TOL if bwd_q is None else 2e-2  # a gradient value next to an e5m2 rounding boundary may land on either side
+  assert relerr(lhs_g.grad, want_dl) <= tol
+  assert torch.all(lhs_g.grad[420:] == 0)
+  got_dr = rhs_g.grad.transpose(1, 2) if transpose_rhs else rhs_g.grad
+  assert got_dr.shape == want_dr.shape and relerr(got_dr, want_dr) <= tol
+  assert torch.all(got_dr[1] == 0)
+  with pytest.raises(NotImplementedError):
+    megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, bwd_quantize_dtype="float8_e5m2")

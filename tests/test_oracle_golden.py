@@ -420,3 +420,33 @@ def test_product_mxfp4_quantiser_agrees_with_oracle_generator():
   qa = Q.quantize_weight_mxfp4(w)
   blocks, scales = O.quantize_mxfp4(w)
   assert torch.equal(qa.qvalue.reshape(2, 6, 3, 16), blocks) and torch.equal(qa.scale, scales)
+
+
+def test_quantized_backward_equals_autograd_through_dequantised_operands():
+  """ops.py:530-604: folding the scale of the contracted axis into the gradient is exact algebra, so without
+  gradient quantisation the result equals autograd through the dequantised operands; the e5m2 quantiser keeps
+  one absmax scale per row / column and its values lie on the e5m2 grid."""
+  g = torch.Generator().manual_seed(4)
+  m, k, n, gs = 50, 16, 24, [20, 0, 30]
+  lhs_q = torch.randint(-127, 128, (m, k), generator=g).to(torch.int8)
+  rhs_q = torch.randint(-127, 128, (3, k, n), generator=g).to(torch.int8)
+  ls, rs = torch.rand(m, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
+  grad = torch.randn(m, n, generator=g)
+  dl, dr = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs, gs, grad_dtype=torch.float64)
+  L = (lhs_q.double() * ls.double()[:, None]).requires_grad_(True)
+  R = (rhs_q.double() * rs.double()[None, None, :]).requires_grad_(True)
+  torch.cat([L[:20] @ R[0], L[20:] @ R[2]]).backward(grad.double())
+  # d/dL of sum(grad * L R) = grad R^T: the reference's dlhs.  drhs is the gradient w.r.t. the value lhs_scale * lhs_q
+  # multiplies, i.e. R.grad with L replaced by lhs_q * lhs_scale: the same thing.
+  assert float((dl - L.grad).abs().max()) <= 1e-3
+  assert float((dr - R.grad).abs().max()) <= 1e-3 and float(dr[1].abs().max()) == 0.0
+  # per-expert scales [g, n] reduce to the shared case when all rows are equal
+  dl2, dr2 = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs[None].expand(3, n).contiguous(), gs, grad_dtype=torch.float64)
+  assert torch.equal(dl, dl2) and torch.equal(dr, dr2)
+  # e5m2 quantiser: closed-form scale, grid membership, and a backward that stays within the format's 2^-3 steps
+  q, s = O.quantize_e5m2(grad, dim=1)
+  np.testing.assert_allclose(s[:, 0].numpy(), grad.abs().amax(1).numpy() / 57344.0, rtol=1e-6)
+  assert torch.equal(q, q.to(torch.float8_e5m2).to(torch.float32)) and float(q.abs().max()) == 57344.0
+  assert float(((q * s) - grad).abs().max() / grad.abs().max()) <= 2.0**-3
+  dlq, drq = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs, gs, bwd_qtype="e5m2", grad_dtype=torch.float64)
+  assert float((dlq - dl).abs().max() / dl.abs().max()) <= 0.1 and float((drq - dr).abs().max() / dr.abs().max()) <= 0.1
