@@ -137,10 +137,10 @@ def gmm(
       offset = int(group_offset)
 
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
-    if rhs_bias is not None or rhs_up_bias is not None or partial_sum is not None or partial_sum_up is not None or existing_out is not None:
-      raise NotImplementedError("gradients with rhs_bias / partial_sum / existing_out are not implemented")
+    if partial_sum is not None or partial_sum_up is not None or existing_out is not None:
+      raise NotImplementedError("gradients with partial_sum / existing_out are not implemented")
     return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit,
-                          bwd_quantize_dtype)
+                          bwd_quantize_dtype, rhs_bias, rhs_up_bias)
 
   rhs_n = _native_rhs(rhs, transpose_rhs)
   up_n = _native_rhs(rhs_up, transpose_rhs) if rhs_up is not None else None
@@ -362,16 +362,50 @@ class _GluFn(torch.autograd.Function):
     return dh0, dh1, None, None
 
 
-def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit, bwd_q=None):
+class _BiasFn(torch.autograd.Function):
+  """h + bias[expert of the row] for the differentiable path (the per-expert `mlp_bias` of moe.py:1952-1957, :2239-2242;
+  the inference path adds it in the GEMM epilogue).  Rows of groups outside the local shard and rows past the last
+  group stay as they are (zero).  The bias gradient is the per-group column sum of the incoming gradient."""
+
+  @staticmethod
+  def forward(ctx, h, bias, group_sizes, offset):
+    m = h.shape[0]
+    g_local = bias.shape[0]
+    ends = torch.cumsum(group_sizes, 0)
+    row_group = torch.searchsorted(ends, torch.arange(m, device=h.device, dtype=ends.dtype), right=True)
+    local = row_group - offset
+    owned = (local >= 0) & (local < g_local) & (row_group < group_sizes.numel())
+    ctx.save_for_backward(group_sizes)
+    ctx.offset, ctx.g_local, ctx.bias_dtype = offset, g_local, bias.dtype
+    add = bias.float()[local.clamp(0, g_local - 1)] * owned[:, None]
+    return (h.float() + add).to(h.dtype)
+
+  @staticmethod
+  def backward(ctx, dout):
+    (group_sizes,) = ctx.saved_tensors
+    m = dout.shape[0]
+    # segment sums over the rows of each group (the remainder past the last group is one more segment), in a fixed order
+    lengths = torch.cat([group_sizes.long(), (m - group_sizes.sum()).reshape(1).long()])
+    sums = torch.segment_reduce(dout.float(), "sum", lengths=lengths, axis=0, unsafe=True)
+    dbias = sums[ctx.offset : ctx.offset + ctx.g_local].to(ctx.bias_dtype)
+    return dout, dbias, None, None
+
+
+def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit, bwd_q=None,
+                   rhs_bias=None, rhs_up_bias=None):
   for name, t in (("lhs", lhs), ("rhs", rhs), ("rhs_up", rhs_up)):
     if t is not None and not isinstance(t, torch.Tensor):
       raise NotImplementedError(f"gradients need bf16 tensors; {name} is already quantised")
   h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q)
+  if rhs_bias is not None:
+    h0 = _BiasFn.apply(h0, rhs_bias, group_sizes, offset)
   if rhs_up is None:
     if fuse_act is not None:
       raise ValueError("fuse_act needs rhs_up")
     return h0
   h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q)
+  if rhs_up_bias is not None:
+    h1 = _BiasFn.apply(h1, rhs_up_bias, group_sizes, offset)
   if fuse_act is None:
     raise ValueError("rhs_up needs fuse_act")
   if fuse_act not in ("silu", "swigluoai", "silu_clip"):

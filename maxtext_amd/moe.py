@@ -292,16 +292,15 @@ class RoutedMoE:
     training = torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (sorted_inputs, w0, w1, wo))
     if training:
       # differentiable path: bf16 operands; with act_quant both operands of each GEMM are quantised
-      # inside its forward (ops.py:232-267) and gradients pass through the quantisers unchanged; the
-      # activation is applied unfused so that its inputs are kept for the backward pass
+      # inside its forward (ops.py:232-267); the backward of the int8 path is the reference's quantised one, an fp8
+      # forward is differentiated through its quantisers unchanged; the activation is applied unfused so that its
+      # inputs are kept for the backward pass; per-expert biases are added (and differentiated) after each GEMM
       if any(isinstance(t, QArray) for t in (sorted_inputs, w0, w1, wo)):
         raise NotImplementedError("gradients need bf16 weights; QArray weights are an inference format")
-      if w0_bias is not None or w1_bias is not None or wo_bias is not None:
-        raise NotImplementedError("gradients with mlp_bias are not implemented")
       q = cfg.act_quant
       inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit, lhs_quantize_dtype=q,
-                           rhs_quantize_dtype=q)
-      return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q)
+                           rhs_quantize_dtype=q, rhs_bias=w0_bias, rhs_up_bias=w1_bias)
+      return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q, rhs_bias=wo_bias)
     inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
                          rhs_bias=w0_bias, rhs_up_bias=w1_bias)
     if marks:

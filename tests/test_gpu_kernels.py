@@ -1070,3 +1070,34 @@ def test_gmm_quantized_backward(transpose_rhs, bwd_q):
   assert torch.all(got_dr[1] == 0)
   with pytest.raises(NotImplementedError):
     megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, bwd_quantize_dtype="float8_e5m2")
+
+
+def test_gmm_autograd_with_expert_bias():
+  """Per-expert mlp_bias on the differentiable path (moe.py:1952-1957): forward equals the epilogue bias of the
+  inference path; gradients of lhs, both weights and both biases against torch autograd in f64."""
+  from maxtext_amd import megablox
+
+  g = torch.Generator().manual_seed(14)
+  m, k, n = 300, 128, 128
+  gs = np.array([100, 0, 156], np.int32)  # 44 trailing rows
+  off = [0, 100, 100, 256]
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w0 = (torch.randn(3, n, k, generator=g) * 0.1).to(torch.bfloat16)
+  w1 = (torch.randn(3, n, k, generator=g) * 0.1).to(torch.bfloat16)
+  b0, b1 = torch.randn(3, n, generator=g), torch.randn(3, n, generator=g)
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  a, r0, r1, c0, c1 = (t.double().requires_grad_() for t in (lhs, w0, w1, b0, b1))
+  h0 = torch.cat([a[off[i] : off[i + 1]] @ r0[i].T + c0[i] for i in range(3)])
+  h1 = torch.cat([a[off[i] : off[i + 1]] @ r1[i].T + c1[i] for i in range(3)])
+  ref = torch.cat([torch.nn.functional.silu(h0) * h1, torch.zeros(44, n, dtype=torch.float64)])
+  (ref * dout.double()).sum().backward()
+  la, q0, q1, d0, d1 = (cuda(t).requires_grad_() for t in (lhs, w0, w1, b0, b1))
+  out = megablox.gmm(la, q0, cuda(gs), transpose_rhs=True, rhs_up=q1, fuse_act="silu", rhs_bias=d0, rhs_up_bias=d1)
+  with torch.no_grad():
+    fused = megablox.gmm(cuda(lhs), cuda(w0), cuda(gs), transpose_rhs=True, rhs_up=cuda(w1), fuse_act="silu", rhs_bias=cuda(b0), rhs_up_bias=cuda(b1))
+  assert relerr(out, ref) <= 2e-2 and relerr(out, fused) <= 2e-2 and torch.all(out[256:] == 0)
+  out.backward(cuda(dout))
+  assert relerr(la.grad, a.grad) <= 2e-2
+  assert relerr(q0.grad, r0.grad) <= 2e-2 and relerr(q1.grad, r1.grad) <= 2e-2
+  assert relerr(d0.grad, c0.grad) <= 2e-2 and relerr(d1.grad, c1.grad) <= 2e-2
+  assert torch.all(d0.grad[1] == 0)

@@ -229,8 +229,9 @@ def test_layer_gradients_match_torch_autograd(norm_topk_prob):
 
 
 def test_layer_gradients_with_int8_quantised_forward():
-  """With act_quant the forward quantises both operands of each GEMM and the backward treats the
-  quantisers as identities: gradients stay within the quantisation noise of the bf16 run."""
+  """With act_quant="int8" the forward quantises both operands of each GEMM and the backward runs on the quantised
+  residuals with the scales folded into the gradient (ops.py:530-580): gradients stay within the quantisation
+  noise of the bf16 run."""
   import dataclasses as dc
 
   from maxtext_amd import moe
@@ -250,6 +251,42 @@ def test_layer_gradients_with_int8_quantised_forward():
     grads[q] = [v.grad for v in leaves]
   for a, b in zip(grads[None], grads["int8"]):
     assert relerr(b, a) <= 5e-2
+
+
+def test_layer_gradients_with_expert_biases():
+  """mlp_bias layer (GPT-OSS, moe.py:617-637): gradients of the inputs, the three weights and the three per-expert
+  biases against torch autograd through the per-token loop in f64, on the GPU's routing."""
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(23)
+  t, d, f, e, k = 160, 128, 128, 4, 2
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  logits = torch.randn(1, t, e, generator=g)
+  w0, w1, wo = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
+  b0, b1, bo = torch.randn(e, f, generator=g) * 0.5, torch.randn(e, f, generator=g) * 0.5, torch.randn(e, d, generator=g) * 0.5
+  dout = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
+  leaves = [v.cuda().requires_grad_() for v in (x, w0, w1, wo, b0, b1, bo)]
+  block = moe.RoutedMoE(cfg, *leaves[1:4])
+  out, _, _ = block.sparse_matmul(leaves[0], logits.cuda(), None, *leaves[1:4], *leaves[4:])
+  out.backward(dout.cuda())
+  with torch.no_grad():
+    wts, idx = block.get_topk(logits.cuda())
+  idx, wts = idx.reshape(t, k).cpu().long(), wts.reshape(t, k).cpu().double()
+  r = [v.double().requires_grad_() for v in (x, w0, w1, wo, b0, b1, bo)]
+  xr, w0r, w1r, wor, b0r, b1r, bor = r
+  x2 = xr.reshape(t, d)
+  ref = torch.zeros(t, d, dtype=torch.float64)
+  for s_ in range(k):
+    ex = idx[:, s_]
+    h0 = torch.einsum("td,tfd->tf", x2, w0r[ex]) + b0r[ex]
+    h1 = torch.einsum("td,tfd->tf", x2, w1r[ex]) + b1r[ex]
+    ref = ref + wts[:, s_ : s_ + 1] * (torch.einsum("tf,tdf->td", torch.nn.functional.silu(h0) * h1, wor[ex]) + bor[ex])
+  (ref * dout.double().reshape(t, d)).sum().backward()
+  assert relerr(out.reshape(t, d), ref) <= 2e-2
+  for got, want, name in zip(leaves, r, ("x", "wi_0", "wi_1", "wo", "b0", "b1", "bo")):
+    assert got.grad is not None and got.grad.shape == got.shape, name
+    assert relerr(got.grad, want.grad) <= 3e-2, name
 
 
 # ---------------------------------------------------------------- graph replay
