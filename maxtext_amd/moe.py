@@ -122,6 +122,7 @@ class RoutedMoE:
     self.gate_kernel, self.gate_bias = gate_kernel, gate_bias
     self._gate_terms = None  # [S, E, d] bf16 form of gate_kernel for moe_gate_route, built on first use
     self.per_expert_scale = None  # [E] f32, Gemma4: multiplies the routing weights (moe.py:758-763)
+    self.tid2eid = None  # [vocab, k] token id -> expert ids: DeepSeek-V4 hash routing (moe.py:443-454, :729-738)
     # when set to a list, _experts appends (stage, start_event, end_event) recorded on the launch stream
     self.profile_events = None
 
@@ -132,10 +133,12 @@ class RoutedMoE:
     out = (x @ self.gate_kernel.to(x.dtype)).float()
     if cfg.routed_score_func == "sigmoid":
       out = torch.sigmoid(out)
+    elif cfg.routed_score_func == "sqrtsoftplus":  # DeepSeek-V4 router (linears.py:51-53)
+      out = torch.sqrt(torch.nn.functional.softplus(out))
     elif cfg.routed_score_func:
       raise NotImplementedError(cfg.routed_score_func)
     pre_bias = out if cfg.is_deepseek else None
-    if self.gate_bias is not None:
+    if self.gate_bias is not None and self.tid2eid is None:  # a hash-routed layer has no gate bias (moe.py:499)
       out = out + self.gate_bias.float()
     return out.contiguous(), pre_bias
 
@@ -190,8 +193,10 @@ class RoutedMoE:
     return lb_loss, bias_updates
 
   # -- get_topk (moe.py:717-765) ------------------------------------------------------------
-  def get_topk(self, gate_logits: torch.Tensor, pre_bias_logits: Optional[torch.Tensor] = None):
+  def get_topk(self, gate_logits: torch.Tensor, pre_bias_logits: Optional[torch.Tensor] = None, input_ids=None):
     cfg = self.config
+    if self.tid2eid is not None:
+      return self._hash_routing(pre_bias_logits if pre_bias_logits is not None else gate_logits, input_ids)
     shape = gate_logits.shape[:-1]
     g2 = gate_logits.reshape(-1, gate_logits.shape[-1]).float().contiguous()
     if cfg.is_deepseek:
@@ -208,6 +213,25 @@ class RoutedMoE:
     if torch.is_grad_enabled() and (gate_logits.requires_grad or (pre_bias_logits is not None and pre_bias_logits.requires_grad)):
       w = self._weights_with_grad(gate_logits, pre_bias_logits, idx.reshape(*shape, k))
     return w.reshape(*shape, k), idx.reshape(*shape, k)
+
+  def _hash_routing(self, scores, input_ids):
+    """Hash routing (moe.py:729-738): the experts of a token are read from a table indexed by its id, the weights are
+    the scores at those experts, scaled as for DeepSeek (moe.py:767-773).  A table lookup and a gather: torch ops,
+    differentiable in the scores."""
+    cfg = self.config
+    if input_ids is None:
+      raise ValueError("input_ids cannot be None when is_hash_routing is True")
+    idx = self.tid2eid.to(torch.int32)[input_ids.long()]  # [..., k]
+    w = torch.gather(scores.float(), -1, idx.long())
+    if cfg.is_deepseek:
+      if cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"):
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+      w = w * cfg.routed_scaling_factor
+    else:
+      w = torch.softmax(w, -1).to(torch.bfloat16).float()
+      if cfg.norm_topk_prob:
+        w = w / w.sum(-1, keepdim=True)
+    return w, idx.contiguous()
 
   def _weights_with_grad(self, gate_logits, pre_bias_logits, idx):
     """The weight half of get_topk in differentiable torch ops, on the indices the kernel selected
@@ -245,11 +269,11 @@ class RoutedMoE:
               roll_to_expert_id=None, input_ids=None):
     """-> (sorted_inputs, sorted_selected_experts, weights, group_size, sorted_experts,
     lb_loss, bias_updates, local_group_size), as moe.py:993-1002."""
-    if roll_to_expert_id is not None or input_ids is not None:
-      raise NotImplementedError("ring-of-experts roll and hash routing are multi-device / DeepSeek-V4 features")
+    if roll_to_expert_id is not None:
+      raise NotImplementedError("the ring-of-experts roll is a multi-device feature")
     b, s, d = inputs.shape
     x2d = inputs.reshape(b * s, d).contiguous()
-    weights, selected = self.get_topk(gate_logits, pre_bias_logits)
+    weights, selected = self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
     x2d = self._scale_inputs_by_router_score(x2d, weights)
     sel2d = selected.reshape(b * s, -1).contiguous()
     perm, inv, group_size, sorted_experts = kernels.sort_by_expert(sel2d, self.num_experts)
@@ -326,7 +350,7 @@ class RoutedMoE:
     b, s, d = inputs.shape
     k = self.num_experts_per_tok
     x2d = inputs.reshape(b * s, d).contiguous()
-    weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits)
+    weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
     x2d = self._scale_inputs_by_router_score(x2d, weights)
     perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
                                                       want_sorted_experts=False)
@@ -354,7 +378,8 @@ class RoutedMoE:
     routing_inputs = inputs if gate_inputs is None else gate_inputs
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (routing_inputs, self.gate_kernel, self.gate_bias))
-    if not needs_grad and routing_inputs.dtype == torch.bfloat16 and routing_inputs.shape[-1] % 64 == 0 and self.num_experts % 4 == 0:
+    fused_router = self.tid2eid is None and self.config.routed_score_func in ("", "sigmoid")
+    if fused_router and not needs_grad and routing_inputs.dtype == torch.bfloat16 and routing_inputs.shape[-1] % 64 == 0 and self.num_experts % 4 == 0:
       want_logits = self.config.load_balance_loss_weight > 0.0  # the auxiliary loss needs the full distribution
       r = self.gate_and_route(routing_inputs.reshape(b * s, -1), return_logits=want_logits)
       logits = r[2].reshape(b, s, -1) if want_logits else None
@@ -362,7 +387,7 @@ class RoutedMoE:
     gate_logits, pre_bias = self.gate(routing_inputs.reshape(b * s, -1))
     gate_logits = gate_logits.reshape(b, s, -1)
     pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
-    return self.sparse_matmul(inputs, gate_logits, pre_bias, self.wi_0, self.wi_1, self.wo)
+    return self.sparse_matmul(inputs, gate_logits, pre_bias, self.wi_0, self.wi_1, self.wo, input_ids=input_ids)
 
 
 class RoutedAndSharedMoE:

@@ -181,6 +181,19 @@ def get_topk(
   return w, idx
 
 
+def hash_routing(scores: np.ndarray, tid2eid: np.ndarray, input_ids: np.ndarray, *, deepseek: bool = True,
+                 routed_score_func: str = "sigmoid", routed_scaling_factor: float = 1.0):
+  """DeepSeek-V4 hash routing (moe.py:729-738 then :749-751, :767-773): indices = tid2eid[input_ids]
+  (the table is stored as f32 and cast to int32), weights = scores at those indices, divided by their sum
+  (+1e-20) for the sigmoid / sqrtsoftplus score functions and multiplied by routed_scaling_factor."""
+  assert deepseek, "only DeepSeek-V4 layers are hash routed"
+  idx = np.asarray(tid2eid).astype(np.int32)[np.asarray(input_ids).astype(np.int32)]
+  w = np.take_along_axis(np.asarray(scores, np.float32), idx.astype(np.int64), axis=-1)
+  if routed_score_func in ("sigmoid", "sqrtsoftplus"):
+    w = w / (w.sum(-1, keepdims=True) + np.float32(1e-20))
+  return (w * np.float32(routed_scaling_factor)).astype(np.float32), idx
+
+
 def calculate_load_balance_updates(top_k_indices, num_experts: int, rate: float):
   """moe.py:215-236."""
   flat = np.asarray(top_k_indices).ravel()

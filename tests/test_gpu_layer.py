@@ -462,3 +462,36 @@ def test_llama4_and_gemma4_style_layers():
   x2 = x.reshape(t, d).double()
   want = sum(wsel[:, s_ : s_ + 1] * expert(x2, idx[:, s_]) for s_ in range(k))
   assert relerr(out.reshape(t, d), want) <= 2e-2
+
+
+def test_hash_routed_layer():
+  """DeepSeek-V4 hash routing (moe.py:729-738) with the sqrtsoftplus router score (linears.py:51-53): experts come from
+  the token-id table, weights from the scores at those experts; the layer output against the per-token loop in f64."""
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(71)
+  t, d, f, e, k, vocab = 96, 128, 128, 8, 2, 50
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  wg = torch.randn(d, e, generator=g) * 0.1
+  ws = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
+  table = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(vocab)]).float()
+  ids = torch.randint(0, vocab, (1, t), generator=g)
+  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek4", decoder_block="deepseek4",
+                      routed_score_func="sqrtsoftplus", routed_scaling_factor=1.5)
+  assert cfg.is_deepseek
+  block = moe.RoutedMoE(cfg, *[w.cuda() for w in ws], gate_kernel=wg.cuda())
+  block.tid2eid = table.cuda()
+  out, _, _ = block(x.cuda(), input_ids=ids.cuda())
+  scores = torch.sqrt(torch.nn.functional.softplus(x.reshape(t, d).float() @ wg))
+  ow, oidx = O.hash_routing(scores.numpy(), table.numpy(), ids.reshape(t).numpy(), routed_score_func="sqrtsoftplus", routed_scaling_factor=1.5)
+  w_gpu, idx_gpu = block.get_topk(scores.reshape(1, t, e).cuda(), scores.reshape(1, t, e).cuda(), input_ids=ids.cuda())
+  np.testing.assert_array_equal(idx_gpu.reshape(t, k).cpu().numpy(), oidx)
+  np.testing.assert_allclose(w_gpu.reshape(t, k).cpu().numpy(), ow, rtol=1e-5)
+  x2 = x.reshape(t, d).double()
+  want = torch.zeros(t, d, dtype=torch.float64)
+  for s_ in range(k):
+    ex = torch.as_tensor(oidx[:, s_]).long()
+    h0 = torch.einsum("td,tfd->tf", x2, ws[0].double()[ex])
+    h1 = torch.einsum("td,tfd->tf", x2, ws[1].double()[ex])
+    want += torch.as_tensor(ow[:, s_ : s_ + 1]).double() * torch.einsum("tf,tdf->td", torch.nn.functional.silu(h0) * h1, ws[2].double()[ex])
+  assert relerr(out.reshape(t, d), want) <= 2e-2

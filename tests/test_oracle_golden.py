@@ -450,3 +450,14 @@ def test_quantized_backward_equals_autograd_through_dequantised_operands():
   assert float(((q * s) - grad).abs().max() / grad.abs().max()) <= 2.0**-3
   dlq, drq = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs, gs, bwd_qtype="e5m2", grad_dtype=torch.float64)
   assert float((dlq - dl).abs().max() / dl.abs().max()) <= 0.1 and float((drq - dr).abs().max() / dr.abs().max()) <= 0.1
+
+
+def test_hash_routing_is_a_table_lookup():
+  """moe.py:729-738: a hand case (two tokens, k = 2) and the invariants of the scaling (moe.py:767-773)."""
+  scores = np.array([[0.1, 0.2, 0.3, 0.4], [0.4, 0.3, 0.2, 0.1]], np.float32)
+  table = np.array([[0, 1], [2, 3], [3, 0]], np.float32)  # stored as f32 (moe.py:448-454)
+  w, idx = O.hash_routing(scores, table, np.array([2, 1]), routed_scaling_factor=2.0)
+  np.testing.assert_array_equal(idx, [[3, 0], [2, 3]])
+  np.testing.assert_allclose(w, [[2 * 0.4 / 0.5, 2 * 0.1 / 0.5], [2 * 0.2 / 0.3, 2 * 0.1 / 0.3]], rtol=1e-6)
+  w2, _ = O.hash_routing(scores, table, np.array([2, 1]), routed_score_func="", routed_scaling_factor=1.0)
+  np.testing.assert_allclose(w2, [[0.4, 0.1], [0.2, 0.1]], rtol=1e-7)
