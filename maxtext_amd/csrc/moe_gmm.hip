@@ -14,8 +14,10 @@
 //   gmm_fp8_skinny_kernel  block-scaled fp8 for few rows per expert (decode): no LDS, every wave
 //                     streams 16 weight rows through v_mfma_f32_16x16x128_f8f6f4 and applies the
 //                     per-128 K-block scales to the f32 partial sums.
-//   gmm_fp8_tiled_kernel   block-scaled fp8 for many rows per expert (prefill): 128 x 128 tiles through LDS,
+//   gmm_fp8_tiled_kernel   block-scaled fp8 for 16 to 128 rows per expert: 128 x 128 tiles through LDS,
 //                     v_mfma_f32_32x32x64_f8f6f4, one scaled accumulation per 128-wide K block.
+//   gmm_fp8_big_kernel     block-scaled fp8 from 128 rows per expert (prefill): 256 x 256 tiles, one set of
+//                     accumulators kept in units of the current K block's scale.
 //   gmm_wq_skinny_kernel   the same streaming design for bf16 activations x int8 / int4 / mxfp4 weights,
 //                     with K split over the waves of a block.
 
@@ -1310,6 +1312,249 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
 }
 
 // ---------------------------------------------------------------------------------------
+// Block-scaled fp8, 256 x 256 tiles: half the operand bytes per flop of the 128 x 128 kernel above, which is
+// what bounds that kernel.  A second set of accumulators for the per-block partial sums does not fit (a wave's
+// 128 x 64 share of the tile is 128 registers), so there is ONE set, kept in units of the current block's scale:
+// when K block kb starts the accumulators are multiplied by s[kb-1] / s[kb] (s = a_scale[row, kb] * w_scale[n/128, kb],
+// one scalar per lane and tile) and the MFMAs of the block accumulate straight into them; the epilogue multiplies
+// by the last block's scale.  sum_kb s[kb] P[kb] is unchanged, each block costs one more f32 rounding.  A block
+// whose scale is zero (all-zero operands, so P = 0) keeps the previous unit.
+// 8 waves (2 x 4), stages of one 128-byte scale block (the L1 keeps a fixed number of line requests in flight, so
+// a request should carry a whole line), 2 buffers (128 KB), one block per CU; weights are the MFMA "A" operand.
+// ---------------------------------------------------------------------------------------
+
+template <bool GLU_, bool VEC4_>
+struct F8BigCfg {
+  static constexpr int BM = 256, BN = 256, BKB = 128, NSTAGE = 2;  // a stage is one scale block: 128-byte requests
+  static constexpr bool GLU = GLU_, VEC4 = VEC4_;
+  static constexpr int WAVES_M = 2, WAVES_N = 4, NWAVES = 8, THREADS = NWAVES * kWave;
+  static constexpr int TM = 4, TN = 2;             // 32-row tiles of a wave: 128 rows x 64 weight rows
+  static constexpr int CPR = BKB / 16, RPI = 1024 / BKB;
+  static constexpr int A_IPW = BM / RPI / NWAVES, B_IPW = BN / RPI / NWAVES, LPS = A_IPW + B_IPW;
+  static constexpr int STAGE = (BM + BN) * BKB;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE;
+  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+  __device__ static __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+};
+
+template <typename C>
+__global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_big_kernel(const Fp8TiledParams P) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const TiledParams& p = P.base;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
+  const int N = p.N, K = p.K;
+  const int nkb = K / 128, nst = K / C::BKB;
+
+  // block -> (m-tile, n-tile): contiguous ids per XCD, super-rows of GSM m-tiles
+  const int total = p.max_m_tiles * p.tiles_n;
+  TileInfo tile;
+  int n0;
+  {
+    const int id = blockIdx.x;
+    const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
+    const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+    const int GSM = p.tune > 0 ? p.tune : 4;
+    const int width = GSM * p.tiles_n;
+    const int sg = logical / width, first_m = sg * GSM;
+    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int m_idx = first_m + (logical % width) % gsz;
+    n0 = ((logical % width) / gsz) * C::OUT_BN;
+    tile = p.tiles[m_idx];
+    if (m_idx >= p.header[0]) return;
+  }
+  if (tile.group < 0) {
+    constexpr int QPR = C::OUT_BN / 4;
+    for (int i = tid; i < tile.nrows * QPR; i += C::THREADS) {
+      const int r = i / QPR, c = n0 + (i % QPR) * 4;
+      if (c < N) *(uint2*)(p.out + (size_t)(tile.row0 + r) * N + c) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  const uint8_t* a_src[C::A_IPW];
+  const uint8_t* b_src[C::B_IPW];
+#pragma unroll
+  for (int i = 0; i < C::A_IPW; i++) {
+    const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
+    const int q = (lane % C::CPR) ^ C::swz(r);
+    a_src[i] = p.lhs + (size_t)(tile.row0 + min(r, tile.nrows - 1)) * K + q * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < C::B_IPW; i++) {
+    const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
+    const int q = (lane % C::CPR) ^ C::swz(vr);
+    const bool up = C::GLU && vr >= C::BN / 2;
+    const int n = min(n0 + (up ? vr - C::BN / 2 : vr), N - 1);
+    b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)tile.group * N + n) * K + q * 16;
+  }
+  auto issue_stage = [&](int kt, int buf) {
+    const size_t koff = (size_t)kt * C::BKB;
+    uint8_t* st = smem + buf * C::STAGE;
+#pragma unroll
+    for (int i = 0; i < C::A_IPW; i++)
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[i] + koff), (lds_ptr_t)(st + (wave * C::A_IPW + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < C::B_IPW; i++)
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
+                                       (lds_ptr_t)(st + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+  };
+
+  // fragment of a 32-row tile for k-step h (64 bytes of the 128-byte row): lane (row = lane % 32, kq = lane / 32)
+  // takes chunks 4h + 2kq, 4h + 2kq + 1
+  const int lrow = lane % 32, kq = lane / 32, sw = C::swz(lrow);
+  int choff[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int e = 0; e < 2; e++) choff[h][e] = lrow * C::BKB + (((4 * h + 2 * kq + e) ^ sw) * 16);
+  auto frag = [&](const uint8_t* base, int h) {
+    const v4i a = *(const v4i*)(base + choff[h][0]), b = *(const v4i*)(base + choff[h][1]);
+    v8i r;
+    r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+    r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+    return r;
+  };
+  int w_row[2];
+  if (C::GLU) {
+    w_row[0] = wn * 32;
+    w_row[1] = C::BN / 2 + wn * 32;
+  } else {
+    w_row[0] = wn * 64;
+    w_row[1] = wn * 64 + 32;
+  }
+
+  // ---- block scales: a_scale per lane and row tile, w_scale per weight tile -----------------------------------
+  const float* as_ptr[C::TM];
+#pragma unroll
+  for (int i = 0; i < C::TM; i++) {
+    const int lr = wm * 128 + i * 32 + lrow;
+    as_ptr[i] = P.a_scale + (size_t)(tile.row0 + min(lr, tile.nrows - 1)) * nkb;
+  }
+  const int nnb = (N + 127) / 128;
+  const int n_out0 = n0 + (C::GLU ? wn * 32 : wn * 64);
+  const float* ws_ptr[2];
+  ws_ptr[0] = P.w_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nkb;
+  ws_ptr[1] = C::GLU ? P.u_scale + ((size_t)tile.group * nnb + min(n_out0, N - 1) / 128) * nkb
+                     : P.w_scale + ((size_t)tile.group * nnb + min(n_out0 + 32, N - 1) / 128) * nkb;
+
+  v16f acc[C::TN][C::TM];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++)
+#pragma unroll
+    for (int i = 0; i < C::TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[j][i][r] = 0.f;
+
+  // unit of the accumulators (the scale of the last block that had one) per row tile / weight tile
+  float ua[C::TM], uw[2];
+#pragma unroll
+  for (int i = 0; i < C::TM; i++) ua[i] = 1.0f;
+  uw[0] = uw[1] = 1.0f;
+#pragma unroll
+  for (int s = 0; s < C::NSTAGE - 1; s++) issue_stage(min(s, nst - 1), s);
+
+  // a_scale is read four K blocks at a time: a lane's row differs from its neighbours', so every such load touches
+  // 32 lines whatever its width, and the wide load cuts their number by four (VEC4: K / 128 is a multiple of 4, which
+  // also makes the 16-byte loads aligned).  The next group is requested between a barrier and the stage requests
+  // that follow it: in vmcnt order it is then older than everything that stays in flight.
+  constexpr int GRP = C::VEC4 ? 4 : 1;
+  float as_next[C::TM][GRP];  // one buffer: the next group is requested once the last value of this one has been read
+  float ws_next[2];
+  auto load_a_scales = [&](float (&dst)[C::TM][GRP], int kb) {
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) {
+      if constexpr (C::VEC4) {
+        const float4 v = *(const float4*)(as_ptr[i] + kb);
+        dst[i][0] = v.x; dst[i][1] = v.y; dst[i][2] = v.z; dst[i][3] = v.w;
+      } else {
+        dst[i][0] = as_ptr[i][kb];
+      }
+    }
+  };
+  load_a_scales(as_next, 0);
+  ws_next[0] = ws_ptr[0][0];
+  ws_next[1] = ws_ptr[1][0];
+
+  auto open_stage = [&](int kt, int next_group_kb, int next_kb) {
+    wait_vmcnt<(C::NSTAGE - 2) * C::LPS>();
+    asm volatile("s_barrier" ::: "memory");
+    if (next_group_kb >= 0) load_a_scales(as_next, next_group_kb);
+    if (next_kb >= 0) {
+      ws_next[0] = ws_ptr[0][next_kb];
+      ws_next[1] = ws_ptr[1][next_kb];
+    }
+    asm volatile("" ::: "memory");
+    const int kl = kt + C::NSTAGE - 1;
+    issue_stage(min(kl, nst - 1), kl % C::NSTAGE);
+  };
+  auto kstep = [&](int kt, int h) {
+    const uint8_t* st = smem + (kt % C::NSTAGE) * C::STAGE;
+    v8i tf[C::TM], wf[C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) tf[i] = frag(st + (wm * 128 + i * 32) * C::BKB, h);
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) wf[j] = frag(st + (C::BM + w_row[j]) * C::BKB, h);
+#pragma unroll
+    for (int j = 0; j < C::TN; j++)
+#pragma unroll
+      for (int i = 0; i < C::TM; i++)
+        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j], tf[i], acc[j][i], 0, 0, 0, 127, 0, 127);
+  };
+  for (int kb = 0; kb < nkb; kb++) {
+    const int c = C::VEC4 ? (kb & 3) : 0;  // uniform: which of the group's values this block uses
+    // scales of this block; a zero scale keeps the unit
+    float ra[C::TM], rw[2];
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) {
+      float sc = as_next[i][0];
+      if constexpr (C::VEC4) sc = c == 0 ? as_next[i][0] : (c == 1 ? as_next[i][1] : (c == 2 ? as_next[i][2] : as_next[i][3]));
+      const float nu = sc != 0.f ? sc : ua[i];
+      ra[i] = ua[i] / nu;
+      ua[i] = nu;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const float sc = ws_next[j];
+      const float nu = sc != 0.f ? sc : uw[j];
+      rw[j] = uw[j] / nu;
+      uw[j] = nu;
+    }
+    // the group's last value has been read above: its buffer takes the next group
+    open_stage(kb, c == GRP - 1 ? min(kb + 1, nkb - GRP) : -1, min(kb + 1, nkb - 1));
+    if (kb > 0) {
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int i = 0; i < C::TM; i++) {
+          const float r_ = ra[i] * rw[j];
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[j][i][r] *= r_;
+        }
+    }
+    kstep(kb, 0);
+    kstep(kb, 1);
+  }
+  wait_vmcnt<0>();  // the last requests re-read the final stage into a buffer nobody reads
+
+  // the epilogue's row and channel scales are the accumulators' unit
+  constexpr int NT_OUT = C::GLU ? 1 : 2;
+  EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+#pragma unroll
+  for (int i = 0; i < C::TM; i++) esc.sa[i] = ua[i];
+#pragma unroll
+  for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      esc.sg[j][q] = make_float4(uw[C::GLU ? 0 : j], uw[C::GLU ? 0 : j], uw[C::GLU ? 0 : j], uw[C::GLU ? 0 : j]);
+      esc.su[j][q] = make_float4(uw[1], uw[1], uw[1], uw[1]);
+    }
+  store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, tile, wm * 128, n_out0, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Weight-only int8 / int4 for few rows per expert (decode): bf16 activations, weights widened to bf16 in
 // registers, v_mfma_f32_16x16x32_bf16.  Same streaming structure as the fp8 kernel: no LDS, one wave owns
 // 16*NT output channels and walks K in 128-element blocks; lane (n = lane%16, kq = lane/16) holds 32 k values
@@ -1888,6 +2133,19 @@ static int launch_fp8_tiled(Fp8TiledParams P, int M, int G_total, hipStream_t s)
   return check_launch("gmm_fp8_tiled_kernel");
 }
 
+template <bool GLU, bool VEC4>
+static int launch_fp8_big(Fp8TiledParams P, int M, int G_total, hipStream_t s) {
+  using C = F8BigCfg<GLU, VEC4>;
+  static bool attr_set[kMaxDevices] = {};
+  if (int st = reserve_lds(gmm_fp8_big_kernel<C>, C::LDS_BYTES, attr_set)) return st;
+  P.base.max_m_tiles = max_tiles_for(M, G_total, C::BM);
+  P.base.tiles_n = cdiv(P.base.N, C::OUT_BN);
+  const long long tiles = (long long)P.base.max_m_tiles * P.base.tiles_n;
+  if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  gmm_fp8_big_kernel<C><<<(unsigned)tiles, C::THREADS, C::LDS_BYTES, s>>>(P);
+  return check_launch("gmm_fp8_big_kernel");
+}
+
 template <int MT, int NT, int U>
 static int launch_skinny(SkinnyParams p, bool glu, int max_tiles, hipStream_t s) {
   p.n_blocks = cdiv(p.N, 64 * NT);
@@ -2002,15 +2260,16 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     if ((long long)a->N * a->K >= (1LL << 31)) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs N * K < 2^31");
     // Up to 16 rows per expert on average (decode): the streaming kernel with 16-row tiles, one MFMA row tile per
     // wave; a group with more rows simply gets several tiles, which are adjacent in the grid, run at the same time
-    // and share the group's weights through L2.  Beyond that the LDS-tiled kernel (measured crossover at 16 rows
-    // per expert on 256 experts of 7168 x 2048; 128-row tiles with two blocks per CU beat 256-row tiles with one
-    // at every size measured).  reserved[0] = 1 / 2 / 3 forces the streaming kernel (64-row tiles past 16 rows per
-    // expert) / 128-row tiles / 256-row tiles (tuning aid).
+    // and share the group's weights through L2.  Beyond that the LDS-tiled kernels: 128 x 128 tiles, and from 128
+    // rows per expert 256 x 256 tiles (measured on 256 experts of 7168 x 2048: crossovers at 16 and at 128 rows per
+    // expert).  reserved[0] = 1 / 2 / 3 forces the streaming kernel (64-row tiles past 16 rows per expert) /
+    // 128-row tiles / 256-row tiles (tuning aid).
     const int forced = a->reserved[0] >= 1 && a->reserved[0] <= 3 ? a->reserved[0] : 0;
     const bool few_rows = (long long)a->M <= 16LL * a->num_groups_total;
     const bool tiled = forced ? forced >= 2 : !few_rows;
     if (tiled) {
-      bm = forced == 3 ? 256 : 128;
+      const bool big = forced ? forced == 3 : (long long)a->M >= 128LL * a->num_groups_total;
+      bm = big ? 256 : 128;
       tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);
       Fp8TiledParams P;
       TiledParams& q = P.base;
@@ -2024,7 +2283,11 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
       q.act = a->act; q.act_limit = a->act_limit; q.tune = a->reserved[1]; q.i4_group = 0;
       P.a_scale = a->lhs_scale; P.w_scale = (const float*)a->rhs_scale; P.u_scale = (const float*)a->rhs_up_scale;
       const int G = a->num_groups_total;
-      if (bm == 256) return glu ? launch_fp8_tiled<256, 128, 3, true>(P, a->M, G, s) : launch_fp8_tiled<256, 128, 3, false>(P, a->M, G, s);
+      if (big) {
+        const bool vec4 = (a->K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
+        if (vec4) return glu ? launch_fp8_big<true, true>(P, a->M, G, s) : launch_fp8_big<false, true>(P, a->M, G, s);
+        return glu ? launch_fp8_big<true, false>(P, a->M, G, s) : launch_fp8_big<false, false>(P, a->M, G, s);
+      }
       return glu ? launch_fp8_tiled<128, 128, 2, true>(P, a->M, G, s) : launch_fp8_tiled<128, 128, 2, false>(P, a->M, G, s);
     }
     bm = few_rows ? 16 : 64;

@@ -338,7 +338,7 @@ FP8_SHAPES = [
 ]
 
 
-# 0: the kernel the library picks for the shape; 1: streaming kernel; 2 / 3: LDS-tiled kernel with 128 / 256 row tiles
+# 0: the kernel the library picks for the shape; 1: streaming kernel; 2 / 3: LDS-tiled kernels with 128 x 128 / 256 x 256 tiles
 @pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("m,k,n,gs", FP8_SHAPES)
 def test_gmm_fp8_block_scaled(K, m, k, n, gs, variant):
