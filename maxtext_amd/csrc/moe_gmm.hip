@@ -1088,10 +1088,10 @@ struct Fp8TiledParams {
   const float* u_scale;
 };
 
-template <int BM_, int BKB_, int NSTAGE_, bool GLU_>
+template <int BM_, int BKB_, int NSTAGE_, bool GLU_, bool VEC4_>
 struct F8Cfg {
   static constexpr int BM = BM_, BN = 128, BKB = BKB_, NSTAGE = NSTAGE_;
-  static constexpr bool GLU = GLU_;
+  static constexpr bool GLU = GLU_, VEC4 = VEC4_;  // VEC4: a_scale is read four K blocks per load (K / 128 % 4 == 0)
   static constexpr int WAVES_M = BM / 64, WAVES_N = 2, NWAVES = WAVES_M * WAVES_N, THREADS = NWAVES * kWave;
   static constexpr int TM = 2, TN = 2;
   static constexpr int CPR = BKB / 16;     // 16-byte chunks per LDS row
@@ -1235,7 +1235,23 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
       part[j][i] = zero;
       sc[j][i] = 0.f;
     }
-  float as_cur[2] = {as_ptr[0][0], as_ptr[1][0]};
+  // a_scale: a lane's row differs from its neighbours', so a load touches 32 lines whatever its width; reading four K
+  // blocks per load cuts the number of these loads by four.  The group buffer is refilled once its last value is taken.
+  constexpr int GRP = C::VEC4 ? 4 : 1;
+  float as_grp[2][GRP];
+  auto load_a_scales = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      if constexpr (C::VEC4) {
+        const float4 v = *(const float4*)(as_ptr[i] + kb);
+        as_grp[i][0] = v.x; as_grp[i][1] = v.y; as_grp[i][2] = v.z; as_grp[i][3] = v.w;
+      } else {
+        as_grp[i][0] = as_ptr[i][kb];
+      }
+    }
+  };
+  load_a_scales(0);
+  float as_cur[2];
   float ws_cur[2] = {ws_ptr[0][0], ws_ptr[1][0]};
 #pragma unroll
   for (int s = 0; s < C::NSTAGE - 1; s++) issue_stage(min(s, nst - 1), s);
@@ -1245,13 +1261,12 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
   // the NEXT K block are requested between the barrier and those requests: in vmcnt order they are then older than
   // the requests that stay in flight, so neither the wait of the next stage nor the compiler's wait for the scale
   // registers has to drain a stage that is still travelling.
-  float as_next[2], ws_next[2];
-  auto open_stage = [&](int kt, int next_kb) {
+  float ws_next[2];
+  auto open_stage = [&](int kt, int next_kb, int next_group_kb) {
     wait_vmcnt<(C::NSTAGE - 2) * C::LPS>();
     asm volatile("s_barrier" ::: "memory");
+    if (next_group_kb >= 0) load_a_scales(next_group_kb);
     if (next_kb >= 0) {
-      as_next[0] = as_ptr[0][next_kb];
-      as_next[1] = as_ptr[1][next_kb];
       ws_next[0] = ws_ptr[0][next_kb];
       ws_next[1] = ws_ptr[1][next_kb];
     }
@@ -1279,21 +1294,19 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
         part[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j], tf[i], FIRST ? zero : part[j][i], 0, 0, 0, 127, 0, 127);
       }
   };
+  static_assert(C::SUBS == 2, "a stage is one scale block");
   for (int kb = 0; kb < nkb; kb++) {
     const int kn = min(kb + 1, nkb - 1);
-    if constexpr (C::SUBS == 2) {
-      open_stage(kb, kn);
-      const uint8_t* st = smem + (kb % C::NSTAGE) * C::STAGE;
-      kstep(st, 0, std::true_type{});
-      kstep(st, 1, std::false_type{});
-    } else {
-      open_stage(2 * kb, kn);
-      kstep(smem + ((2 * kb) % C::NSTAGE) * C::STAGE, 0, std::true_type{});
-      open_stage(2 * kb + 1, -1);
-      kstep(smem + ((2 * kb + 1) % C::NSTAGE) * C::STAGE, 0, std::false_type{});
+    const int c = C::VEC4 ? (kb & 3) : 0;  // uniform: which value of the group this block uses
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      as_cur[i] = as_grp[i][0];
+      if constexpr (C::VEC4) as_cur[i] = c == 0 ? as_grp[i][0] : (c == 1 ? as_grp[i][1] : (c == 2 ? as_grp[i][2] : as_grp[i][3]));
     }
-    as_cur[0] = as_next[0];
-    as_cur[1] = as_next[1];
+    open_stage(kb, kn, c == GRP - 1 ? min(kb + 1, nkb - GRP) : -1);
+    const uint8_t* st = smem + (kb % C::NSTAGE) * C::STAGE;
+    kstep(st, 0, std::true_type{});
+    kstep(st, 1, std::false_type{});
     ws_cur[0] = ws_next[0];
     ws_cur[1] = ws_next[1];
   }
@@ -2120,9 +2133,9 @@ static int launch_tiled_glu(const TiledParams& p, bool glu, int M, int G_total, 
              : launch_tiled_by_rows<OP, BSRC, false>(p, M, G_total, bm_out, dry, s);
 }
 
-template <int BM, int BKB, int NSTAGE, bool GLU>
+template <int BM, int BKB, int NSTAGE, bool GLU, bool VEC4>
 static int launch_fp8_tiled(Fp8TiledParams P, int M, int G_total, hipStream_t s) {
-  using C = F8Cfg<BM, BKB, NSTAGE, GLU>;
+  using C = F8Cfg<BM, BKB, NSTAGE, GLU, VEC4>;
   static bool attr_set[kMaxDevices] = {};
   if (int st = reserve_lds(gmm_fp8_tiled_kernel<C>, C::LDS_BYTES, attr_set)) return st;
   P.base.max_m_tiles = max_tiles_for(M, G_total, BM);
@@ -2260,15 +2273,15 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     if ((long long)a->N * a->K >= (1LL << 31)) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs N * K < 2^31");
     // Up to 16 rows per expert on average (decode): the streaming kernel with 16-row tiles, one MFMA row tile per
     // wave; a group with more rows simply gets several tiles, which are adjacent in the grid, run at the same time
-    // and share the group's weights through L2.  Beyond that the LDS-tiled kernels: 128 x 128 tiles, and from 128
-    // rows per expert 256 x 256 tiles (measured on 256 experts of 7168 x 2048: crossovers at 16 and at 128 rows per
-    // expert).  reserved[0] = 1 / 2 / 3 forces the streaming kernel (64-row tiles past 16 rows per expert) /
-    // 128-row tiles / 256-row tiles (tuning aid).
+    // and share the group's weights through L2.  Beyond that the LDS-tiled kernel with 128 x 128 tiles (measured on
+    // 256 experts of 7168 x 2048: crossover at 16 rows per expert; the 256 x 256 kernel is within 5 % of it from 128
+    // rows per expert on and behind it below, so it is not picked by default).  reserved[0] = 1 / 2 / 3 forces the
+    // streaming kernel (64-row tiles past 16 rows per expert) / 128 x 128 tiles / 256 x 256 tiles (tuning aid).
     const int forced = a->reserved[0] >= 1 && a->reserved[0] <= 3 ? a->reserved[0] : 0;
     const bool few_rows = (long long)a->M <= 16LL * a->num_groups_total;
     const bool tiled = forced ? forced >= 2 : !few_rows;
     if (tiled) {
-      const bool big = forced ? forced == 3 : (long long)a->M >= 128LL * a->num_groups_total;
+      const bool big = forced == 3;
       bm = big ? 256 : 128;
       tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);
       Fp8TiledParams P;
@@ -2283,12 +2296,13 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
       q.act = a->act; q.act_limit = a->act_limit; q.tune = a->reserved[1]; q.i4_group = 0;
       P.a_scale = a->lhs_scale; P.w_scale = (const float*)a->rhs_scale; P.u_scale = (const float*)a->rhs_up_scale;
       const int G = a->num_groups_total;
+      const bool vec4 = (a->K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
       if (big) {
-        const bool vec4 = (a->K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
         if (vec4) return glu ? launch_fp8_big<true, true>(P, a->M, G, s) : launch_fp8_big<false, true>(P, a->M, G, s);
         return glu ? launch_fp8_big<true, false>(P, a->M, G, s) : launch_fp8_big<false, false>(P, a->M, G, s);
       }
-      return glu ? launch_fp8_tiled<128, 128, 2, true>(P, a->M, G, s) : launch_fp8_tiled<128, 128, 2, false>(P, a->M, G, s);
+      if (vec4) return glu ? launch_fp8_tiled<128, 128, 2, true, true>(P, a->M, G, s) : launch_fp8_tiled<128, 128, 2, false, true>(P, a->M, G, s);
+      return glu ? launch_fp8_tiled<128, 128, 2, true, false>(P, a->M, G, s) : launch_fp8_tiled<128, 128, 2, false, false>(P, a->M, G, s);
     }
     bm = few_rows ? 16 : 64;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, a->num_groups_total, a->group_offset, a->num_groups_local, a->M, bm, zero_fill, header, tiles);
