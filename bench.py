@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "c2": (2335090 * 2.0 + 459081 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
     "c3": (3852849 * 2.0 + 9236 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
-    "c2_train": (3100853 * 2.0 + 917551 * 1.0) * 1024,  # profiles/tgmm_kernel_bf16_mixtral_shape_train.md
+    "c2_train": (3105239 * 2.0 + 917553 * 1.0) * 1024,  # profiles/tgmm_kernel_bf16_mixtral_shape_train.md
 }
 
 
