@@ -762,8 +762,8 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     }
   };
   constexpr int NMFMA = C::TM * C::TN, NFRAG = C::TM + C::TN;
-  constexpr int HALF = C::LPS / 2;  // a stage's requests are split over two k-steps
-  static_assert(NFRAG <= NMFMA && C::LPS % 2 == 0 && HALF <= NMFMA / 2, "interleave shape");
+  constexpr int HALF = C::LPS / 2;  // 64-byte stages: a stage's requests are split over two k-steps
+  static_assert(NFRAG <= NMFMA && C::LPS % 2 == 0 && (C::KSUB == 4 ? C::LPS <= NMFMA : HALF <= NMFMA / 2), "interleave shape");
   // One k-step: MFMAs on register set SET with, slotted between them, the fragment reads of the next
   // k-step (RD) and HALF of a stage's requests (LD).  SET / RD / LD are compile-time so that the body is
   // straight-line code.
@@ -780,17 +780,38 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): long satisfied by the time the last MFMA has issued
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The same for 128-byte stages (four k-steps): all LPS requests of a stage go out during ONE k-step, one per MFMA.
+  auto kstep4 = [&](auto set_c, auto rd_c, auto ld_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
+#pragma unroll
+    for (int idx = 0; idx < NMFMA; idx++) {
+      mfma_one(SET, idx);
+      if (RD && idx < NFRAG) read_frag(rd_buf, rd_ks, SET ^ 1, idx);
+      if (LD && idx < C::LPS) issue_one(ld_kt, ld_buf, idx);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+  };
   using T_ = std::true_type;
   using F_ = std::false_type;
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
 
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
-  static_assert(C::KSUB == 2 && C::NSTAGE >= 3, "pipeline shape");
+  static_assert((C::KSUB == 2 && C::NSTAGE >= 3) || (C::KSUB == 4 && C::NSTAGE == 2), "pipeline shape");
   const int nk = K / C::BK;
 
   // Requests of a tile's first stages: stages 0..NSTAGE-3 in full and the first half of stage NSTAGE-2.
   auto issue_prologue = [&]() {
+    if constexpr (C::KSUB == 4) {  // two buffers: both of the tile's first stages
+#pragma unroll
+      for (int s = 0; s < 2; s++)
+#pragma unroll
+        for (int i = 0; i < C::LPS; i++) issue_one(min(s, nk - 1), s, i);
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < C::NSTAGE - 2; s++)
 #pragma unroll
@@ -830,6 +851,29 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     for (int f = 0; f < NFRAG; f++) read_frag(0, 0, 0, f);
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
     int kt = 0;
+    const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+    EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+    if constexpr (C::KSUB == 4) {
+      // 128-byte stages, two buffers.  By the end of the third k-step a wave holds the whole of stage kt in
+      // registers (or has used it), so the barrier before the fourth proves stage kt's buffer free, and the requests
+      // of stage kt+2 go out during that k-step while the fragments of stage kt+1 (whose requests were waited for
+      // just before the barrier) are read.  A request carries a whole 128-byte line: the L1 keeps a fixed number
+      // of requests in flight whatever their size.
+      for (; kt + 1 < nk; kt++) {
+        const int buf = kt % 2;
+        kstep4(S0{}, T_{}, F_{}, buf, 1, 0, 0);
+        kstep4(S1{}, T_{}, F_{}, buf, 2, 0, 0);
+        kstep4(S0{}, T_{}, F_{}, buf, 3, 0, 0);
+        wait_vmcnt<0>();
+        asm volatile("s_barrier" ::: "memory");
+        kstep4(S1{}, T_{}, T_{}, buf ^ 1, 0, min(kt + 2, nk - 1), buf);
+      }
+      load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, cur.info, wm * C::WM, n_out0, lane);
+      kstep4(S0{}, T_{}, F_{}, kt % 2, 1, 0, 0);
+      kstep4(S1{}, T_{}, F_{}, kt % 2, 2, 0, 0);
+      kstep4(S0{}, T_{}, F_{}, kt % 2, 3, 0, 0);
+      kstep4(S1{}, F_{}, F_{}, 0, 0, 0, 0);
+    } else {
     for (; kt + 1 < nk; kt++) {
       const int buf = kt % C::NSTAGE;
       const int kb = kt + C::NSTAGE - 2, ka = kt + C::NSTAGE - 1;
@@ -839,11 +883,10 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
       kstep(S1{}, T_{}, T_{}, (kt + 1) % C::NSTAGE, 0, min(ka, nk - 1), ka % C::NSTAGE, 0);
     }
     // the epilogue's scales are fetched behind the last two k-steps
-    const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
-    EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
     load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, cur.info, wm * C::WM, n_out0, lane);
     kstep(S0{}, T_{}, F_{}, kt % C::NSTAGE, 1, 0, 0, 0);
     kstep(S1{}, F_{}, F_{}, 0, 0, 0, 0, 0);
+    }
     // all LDS reads of this tile are done in every wave and no request is still writing LDS: the buffers
     // can take the next tile's first stages
     wait_vmcnt<0>();
@@ -2089,6 +2132,9 @@ static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* b
   if constexpr (BSRC == BSRC_SAME) {
     // operands that need no conversion stream straight into LDS when every stage is a full 64-byte row slice
     constexpr int ESZ = OP == OP_I8 ? 1 : 2;
+    // 128-byte stages (two buffers) when the rows allow it: 3-7 % faster than 64-byte stages (four buffers) on the
+    // Mixtral shape (tile variant 12 of the int8 path is the 64-byte pipeline, for comparison)
+    if (big && (p.K * ESZ) % 128 == 0) return launch_dl<DlCfg<OP, 256, 256, 128, 2, 4, 2, GLU>>(p, M, G_total, s);
     if (big && (p.K * ESZ) % 64 == 0) return launch_dl<DlCfg<OP, 256, 256, 64, 2, 4, 4, GLU>>(p, M, G_total, s);
   }
   if (big) return launch_tiled<TiledCfg<OP, BSRC, 256, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
