@@ -1101,3 +1101,44 @@ def test_gmm_autograd_with_expert_bias():
   assert relerr(q0.grad, r0.grad) <= 2e-2 and relerr(q1.grad, r1.grad) <= 2e-2
   assert relerr(d0.grad, c0.grad) <= 2e-2 and relerr(d1.grad, c1.grad) <= 2e-2
   assert torch.all(d0.grad[1] == 0)
+
+
+# Shapes large enough for the persistent direct-to-LDS kernel (at least 128 tiles of 256 x 256, 128 rows per
+# expert): K = 128 (one stage), 384 (three 128-byte stages), 320 and 192 (K * elem only a multiple of 64: the
+# 64-byte pipeline for int8; for bf16 both are multiples of 128 bytes), ragged groups with an empty one and
+# trailing rows that belong to no group.
+DL_SHAPES = [(4200, 128, 2048), (4200, 384, 2048), (4200, 320, 2048), (4200, 192, 2304)]
+
+
+@pytest.mark.parametrize("m,k,n", DL_SHAPES)
+def test_gmm_direct_to_lds_pipelines_int8(K, m, k, n):
+  gs = np.array([1000, 0, 2000, 1096], np.int32)
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 41)
+  q, s = O.quantize_weight_int8(w)
+  qu, su = O.quantize_weight_int8(w_up)
+  lq, ls = O.quantize_rows_int8(lhs)
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s), rhs_up=cuda(native(qu)),
+                  rhs_up_scale=cuda(su), act="silu")
+  want = O.apply_ffn_activation(O.gmm(lq, q, gs, lhs_scale=ls, rhs_scale=s, out_dtype=torch.float32, acc_dtype=torch.float32),
+                                O.gmm(lq, qu, gs, lhs_scale=ls, rhs_scale=su, out_dtype=torch.float32, acc_dtype=torch.float32))
+  assert relerr(got, want) <= TOL and torch.all(got[4096:] == 0)
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s))
+  want = O.gmm(lq, q, gs, lhs_scale=ls, rhs_scale=s, acc_dtype=torch.float32)
+  assert relerr(got, want) <= TOL and torch.all(got[4096:] == 0)
+  # the 64-byte pipeline on the same operands (tile variant 12) agrees bit for bit: integer accumulation
+  if k % 128 == 0:
+    other = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s), tile_variant=12)
+    assert torch.equal(got, other)
+
+
+@pytest.mark.parametrize("m,k,n", DL_SHAPES[:3])
+def test_gmm_direct_to_lds_pipelines_bf16(K, m, k, n):
+  gs = np.array([1000, 0, 2000, 1096], np.int32)
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 42)
+  wb, ub = w.to(torch.bfloat16), w_up.to(torch.bfloat16)
+  got = K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs), rhs_up=cuda(native(ub)), act="silu")
+  want = O.apply_ffn_activation(O.gmm(lhs, wb, gs, out_dtype=torch.float32, acc_dtype=torch.float32),
+                                O.gmm(lhs, ub, gs, out_dtype=torch.float32, acc_dtype=torch.float32))
+  assert relerr(got, want) <= TOL and torch.all(got[4096:] == 0)
+  got = K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs))
+  assert relerr(got, O.gmm(lhs, wb, gs, acc_dtype=torch.float32)) <= TOL
