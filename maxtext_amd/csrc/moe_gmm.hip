@@ -2150,12 +2150,7 @@ static int launch_i8_variant(int id, const TiledParams& p, int M, int G_total, i
     if (dry) return MOE_OK;                                                                         \
     return launch_tiled<TiledCfg<OP_I8, BSRC_SAME, BM, BN, BKB, WM, WN, GLU>>(p, M, G_total, s);    \
   }
-  MOE_VARIANT(3, 256, 256, 64, 2, 4)
-  MOE_VARIANT(4, 256, 256, 64, 2, 2)
-  MOE_VARIANT(5, 256, 256, 128, 2, 2)
-  MOE_VARIANT(6, 128, 256, 128, 2, 2)
-  MOE_VARIANT(7, 128, 128, 128, 2, 2)
-  MOE_VARIANT(8, 128, 256, 64, 2, 2)
+  MOE_VARIANT(3, 256, 256, 64, 2, 4)  // the register-staged kernel on int8 x int8
 #undef MOE_VARIANT
 #define MOE_DL_VARIANT(ID, BM, BN, BKB, WM, WN, NS)                                                 \
   if (id == ID) {                                                                                   \
@@ -2164,11 +2159,7 @@ static int launch_i8_variant(int id, const TiledParams& p, int M, int G_total, i
     if (p.K % BKB) return fail(MOE_ERR_UNSUPPORTED, "gmm: variant needs K %% %d == 0", BKB);        \
     return launch_dl<DlCfg<OP_I8, BM, BN, BKB, WM, WN, NS, GLU>>(p, M, G_total, s);                 \
   }
-  MOE_DL_VARIANT(10, 256, 256, 64, 2, 4, 5)
-  MOE_DL_VARIANT(11, 256, 256, 64, 2, 4, 3)
-  MOE_DL_VARIANT(12, 256, 256, 64, 2, 4, 4)
-  MOE_DL_VARIANT(14, 256, 256, 64, 2, 2, 4)
-  MOE_DL_VARIANT(15, 256, 256, 64, 2, 2, 5)
+  MOE_DL_VARIANT(12, 256, 256, 64, 2, 4, 4)  // the 64-byte-stage pipeline where the default is the 128-byte one
 #undef MOE_DL_VARIANT
   return fail(MOE_ERR_INVALID_ARG, "gmm: unknown tile variant %d", id);
 }
@@ -2217,21 +2208,13 @@ static int launch_skinny(SkinnyParams p, bool glu, int max_tiles, hipStream_t s)
   return check_launch("gmm_fp8_skinny_kernel");
 }
 
-// reserved[0] can force (NT, U) of the fp8 kernel: id = 100 + 10 * NT + U (tuning aid); 0 picks the default.
+// (NT, U) of the fp8 streaming kernel, from sweeps over NT in {1, 2, 4} and U in {1, 2, 4} on the DeepSeek-V3 shapes:
+// 16-row tiles take 4 channel tiles per wave and one K block per step with fused GLU, 2 tiles and 4 blocks without;
+// 64-row tiles take 2 tiles and one block.
 template <int MT>
-static int launch_skinny_variant(int id, const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s) {
-  if (id == 0) id = MT > 1 ? 121 : (glu ? 141 : 124);
-  switch (id) {
-    case 111: return launch_skinny<MT, 1, 1>(p, glu, max_tiles, s);
-    case 112: return launch_skinny<MT, 1, 2>(p, glu, max_tiles, s);
-    case 114: return launch_skinny<MT, 1, 4>(p, glu, max_tiles, s);
-    case 121: return launch_skinny<MT, 2, 1>(p, glu, max_tiles, s);
-    case 122: return launch_skinny<MT, 2, 2>(p, glu, max_tiles, s);
-    case 124: return launch_skinny<MT, 2, 4>(p, glu, max_tiles, s);
-    case 141: return launch_skinny<MT, 4, 1>(p, glu, max_tiles, s);
-    case 142: return launch_skinny<MT, 4, 2>(p, glu, max_tiles, s);
-    default: return fail(MOE_ERR_INVALID_ARG, "gmm: unknown fp8 variant %d", id);
-  }
+static int launch_skinny_default(const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s) {
+  if (MT > 1) return launch_skinny<MT, 2, 1>(p, glu, max_tiles, s);
+  return glu ? launch_skinny<MT, 4, 1>(p, glu, max_tiles, s) : launch_skinny<MT, 2, 4>(p, glu, max_tiles, s);
 }
 
 template <int FMT, int MT, int KSPLIT, int NT, int U, bool LINE = true>
@@ -2363,9 +2346,8 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     p.act = a->act; p.act_limit = a->act_limit;
     const int mx = max_tiles_for(a->M, a->num_groups_total, bm);
     p.min_rows = 1; p.max_rows = bm;
-    const int variant = a->reserved[0] > 100 ? a->reserved[0] : 0;
-    if (few_rows) return launch_skinny_variant<1>(variant, p, glu, mx, s);
-    return launch_skinny_variant<4>(variant, p, glu, mx, s);
+    if (few_rows) return launch_skinny_default<1>(p, glu, mx, s);
+    return launch_skinny_default<4>(p, glu, mx, s);
   }
 
   TiledParams p;
