@@ -169,27 +169,34 @@ __device__ __forceinline__ void add_partial4(const uint16_t* ps, size_t row, int
 
 // Per-lane scales of the epilogue, fetched before the K loop so their latency hides behind it.  With
 // weights as the MFMA "A" operand a lane owns row (lane % 32) of each 32-row tile and, per accumulator
-// quad q, the 4 consecutive output channels 8*q + 4*(lane / 32) .. +3 of each 32-channel tile.
+// quad q, the 4 consecutive output channels 8*q + 4*(lane / 32) .. +3 of each 32-channel tile.  With the
+// 16 x 16 instructions (MI = 16) it owns row (lane % 16) of each 16-row tile and the one quad of channels
+// 4*(lane / 16) .. +3 of each 16-channel tile (only entry [.][0] of sg / su is used).
+template <int MI>
+__device__ __forceinline__ int epilogue_channel(int j, int q, int lane) {
+  return MI == 32 ? j * 32 + 8 * q + 4 * (lane / 32) : j * 16 + 4 * (lane / 16);
+}
+
 template <int TM, int NT_OUT, bool GLU>
 struct EpilogueScales {
   float sa[TM];
   float4 sg[NT_OUT][4], su[NT_OUT][4];
 };
 
-template <int TM, int NT_OUT, bool GLU, bool CHANNEL_SCALES>
+template <int TM, int NT_OUT, bool GLU, bool CHANNEL_SCALES, int MI = 32>
 __device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, GLU>& e, const TiledParams& p, const TileInfo& tile,
                                                      int row_base, int n_base, int lane) {
   const float4 one = make_float4(1.f, 1.f, 1.f, 1.f);
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-    const int lr = row_base + i * 32 + (lane % 32);
+    const int lr = row_base + i * MI + (lane % MI);
     e.sa[i] = p.lhs_scale ? p.lhs_scale[tile.row0 + (lr < tile.nrows ? lr : 0)] : 1.0f;
   }
 #pragma unroll
   for (int j = 0; j < NT_OUT; j++)
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const int n = n_base + j * 32 + 8 * q + 4 * (lane / 32);
+    for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+      const int n = n_base + epilogue_channel<MI>(j, q, lane);
       e.sg[j][q] = one;
       e.su[j][q] = one;
       if (CHANNEL_SCALES && p.rhs_scale && n < p.N) {
@@ -202,18 +209,19 @@ __device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, 
 template <int TM, int TN, int NT_OUT, bool GLU, typename acc_t>
 __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
                                                const TiledParams& p, const TileInfo& tile, int row_base, int n_base, int lane) {
+  constexpr int MI = sizeof(acc_t) == 16 ? 16 : 32;  // 4 accumulator registers per tile: the 16 x 16 instructions
   dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
   constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-    const int lr = row_base + i * 32 + (lane % 32);
+    const int lr = row_base + i * MI + (lane % MI);
     if (lr >= tile.nrows) continue;
     uint16_t* orow = p.out + (size_t)(tile.row0 + lr) * p.N;
 #pragma unroll
     for (int j = 0; j < NT_OUT; j++)
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int n = n_base + j * 32 + 8 * q + 4 * (lane / 32);
+      for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+        const int n = n_base + epilogue_channel<MI>(j, q, lane);
         if (n >= p.N) continue;
         const float sg[4] = {e.sg[j][q].x, e.sg[j][q].y, e.sg[j][q].z, e.sg[j][q].w};
         const float su[4] = {e.su[j][q].x, e.su[j][q].y, e.su[j][q].z, e.su[j][q].w};
@@ -612,13 +620,16 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 template <int OP_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, int NSTAGE_, bool GLU_>
 struct DlCfg {
   static constexpr int OP = OP_, BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
+  // rows (= columns) of the MFMA tile: 128-byte stages feed the 16 x 16 instructions (16x16x64 i8 / 16x16x32 bf16: 64
+  // bytes of K per row), 64-byte stages the 32 x 32 ones (32x32x32 i8 / 32x32x16 bf16: 32 bytes of K per row)
+  static constexpr int MI = BKB == 128 ? 16 : 32;
   static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NWAVES = WAVES_M_ * WAVES_N_;
   static constexpr bool GLU = GLU_;
   static constexpr int THREADS = NWAVES * kWave;
   static constexpr int ESZ = OP == OP_I8 ? 1 : 2;
   static constexpr int BK = BKB / ESZ;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  static constexpr int TM = WM / 32, TN = WN / 32;
+  static constexpr int TM = WM / MI, TN = WN / MI;
   static constexpr int KSUB = BKB / 32;
   static constexpr int CPR = BKB / 16;         // 16-byte chunks per row
   static constexpr int RPI = 1024 / BKB;       // rows per wave instruction
@@ -631,6 +642,7 @@ struct DlCfg {
   static_assert(BM % (RPI * NWAVES) == 0 && BN % (RPI * NWAVES) == 0, "load split");
   static_assert(!GLU || ((BN / 2) % RPI == 0 && TN % 2 == 0), "GLU halves");
   static_assert((NSTAGE - 1) * LPS < 64, "vmcnt range");
+  static_assert(MI == 32 || (NSTAGE == 2 && TM >= TN && TM * TN >= LPS), "16 x 16 pipeline shape");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS");
   __device__ static __forceinline__ int swz(int row) { return BKB == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
 };
@@ -720,7 +732,10 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     }
   };
 
-  typedef typename std::conditional<OP == OP_I8, v16i, v16f>::type acc_t;
+  typedef typename std::conditional<OP == OP_I8, v16i, v16f>::type acc32_t;
+  typedef typename std::conditional<OP == OP_I8, v4i, v4f>::type acc16_t;
+  typedef typename std::conditional<C::MI == 32, acc32_t, acc16_t>::type acc_t;
+  constexpr int ACC_REGS = C::MI == 32 ? 16 : 4;
   acc_t acc[C::TN][C::TM];
 
   int b_row[C::TN];
@@ -728,9 +743,9 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   for (int j = 0; j < C::TN; j++) {
     if (C::GLU) {
       constexpr int H = C::TN / 2;
-      b_row[j] = (j < H ? 0 : C::BN / 2) + wn * (C::WN / 2) + (j < H ? j : j - H) * 32;
+      b_row[j] = (j < H ? 0 : C::BN / 2) + wn * (C::WN / 2) + (j < H ? j : j - H) * C::MI;
     } else {
-      b_row[j] = wn * C::WN + j * 32;
+      b_row[j] = wn * C::WN + j * C::MI;
     }
   }
   // fragment of k-step ks: row (lane % 32), chunk q = 2*ks + lane/32, stored at slot q ^ swz(row)
@@ -754,7 +769,9 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   };
   auto mfma_one = [&](int set, int idx) {
     const int j = idx / C::TM, i = idx % C::TM;
-    if constexpr (OP == OP_I8) {
+    if constexpr (C::MI != 32) {
+      return;  // the 16 x 16 pipeline has its own k-step below
+    } else if constexpr (OP == OP_I8) {
       acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[set][j], fa[set][i], acc[j][i], 0, 0, 0);
     } else {
       acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -763,7 +780,7 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   };
   constexpr int NMFMA = C::TM * C::TN, NFRAG = C::TM + C::TN;
   constexpr int HALF = C::LPS / 2;  // 64-byte stages: a stage's requests are split over two k-steps
-  static_assert(NFRAG <= NMFMA && C::LPS % 2 == 0 && (C::KSUB == 4 ? C::LPS <= NMFMA : HALF <= NMFMA / 2), "interleave shape");
+  static_assert(NFRAG <= NMFMA && C::LPS % 2 == 0 && (C::MI == 16 || HALF <= NMFMA / 2), "interleave shape");
   // One k-step: MFMAs on register set SET with, slotted between them, the fragment reads of the next
   // k-step (RD) and HALF of a stage's requests (LD).  SET / RD / LD are compile-time so that the body is
   // straight-line code.
@@ -780,32 +797,59 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): long satisfied by the time the last MFMA has issued
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The same for 128-byte stages (four k-steps): all LPS requests of a stage go out during ONE k-step, one per MFMA.
-  auto kstep4 = [&](auto set_c, auto rd_c, auto ld_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
-    constexpr int SET = decltype(set_c)::value;
-    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
-#pragma unroll
-    for (int idx = 0; idx < NMFMA; idx++) {
-      mfma_one(SET, idx);
-      if (RD && idx < NFRAG) read_frag(rd_buf, rd_ks, SET ^ 1, idx);
-      if (LD && idx < C::LPS) issue_one(ld_kt, ld_buf, idx);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    __builtin_amdgcn_sched_barrier(0);
-  };
   using T_ = std::true_type;
   using F_ = std::false_type;
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
 
+  // ---- the 16 x 16 instructions (16x16x64 i8, 16x16x32 bf16): 64 bytes of K per row and k-step, two k-steps per
+  // 128-byte stage.  On changing operands the chip sustains about a fifth more of these than of the 32 x 32 ones
+  // (a quarter of the accumulator registers read and written per instruction at half the work: the matrix pipes run
+  // against the power limit, not the issue rate).  A wave's 128 x 64 tile takes 8 activation and 4 weight fragments
+  // per k-step for 32 MFMAs.  The weight fragments are double-buffered; an activation fragment is reloaded for the
+  // next k-step right after the four MFMAs that use it, so 12 fragments stay in registers instead of 24.
+  // fragment of k-step ks: row (lane % 16), chunk q = 4*ks + lane/16, stored at slot q ^ swz(row)
+  const int t16m = ((lane / 16) ^ C::swz(lane % 16)) * 16;
+  const int row_off_m = (lane % 16) * C::BKB;
+  v4i ga[C::TM], gb[2][C::TN];
+  auto read_a16 = [&](int buf, int ks, int i) {
+    ga[i] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
+  };
+  auto read_b16 = [&](int buf, int ks, int set, int j) {
+    gb[set][j] = *(const v4i*)(smem + buf * C::STAGE + (C::BM + b_row[j]) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
+  };
+  auto kstep16 = [&](auto set_c, auto rd_c, auto ld_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
+    if constexpr (C::MI == 16) {
+#pragma unroll
+      for (int i = 0; i < C::TM; i++) {
+#pragma unroll
+        for (int j = 0; j < C::TN; j++) {
+          if constexpr (OP == OP_I8) {
+            acc[j][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(gb[SET][j], ga[i], acc[j][i], 0, 0, 0);
+          } else {
+            acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(v8bf, gb[SET][j]), __builtin_bit_cast(v8bf, ga[i]), acc[j][i], 0, 0, 0);
+          }
+          // the stage's requests go out one per MFMA from the start of the k-step: they have until the middle of the
+          // next stage to land, and spreading them over the whole k-step measured 5 % slower
+          if (LD && i * C::TN + j < C::LPS) issue_one(ld_kt, ld_buf, i * C::TN + j);
+          if (RD && j == 1 && i < C::TN) read_b16(rd_buf, rd_ks, SET ^ 1, i);
+          if (RD && j == C::TN - 1) read_a16(rd_buf, rd_ks, i);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  };
+
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
-  static_assert((C::KSUB == 2 && C::NSTAGE >= 3) || (C::KSUB == 4 && C::NSTAGE == 2), "pipeline shape");
+  static_assert((C::MI == 32 && C::NSTAGE >= 3) || (C::MI == 16 && C::NSTAGE == 2), "pipeline shape");
   const int nk = K / C::BK;
 
   // Requests of a tile's first stages: stages 0..NSTAGE-3 in full and the first half of stage NSTAGE-2.
   auto issue_prologue = [&]() {
-    if constexpr (C::KSUB == 4) {  // two buffers: both of the tile's first stages
+    if constexpr (C::MI == 16) {  // two buffers: both of the tile's first stages
 #pragma unroll
       for (int s = 0; s < 2; s++)
 #pragma unroll
@@ -843,36 +887,41 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
 #pragma unroll
       for (int i = 0; i < C::TM; i++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
+        for (int r = 0; r < ACC_REGS; r++) acc[j][i][r] = 0;
     // every request of the prologue (and every store of the previous epilogue) has completed
     wait_vmcnt<0>();
     asm volatile("s_barrier" ::: "memory");
+    if constexpr (C::MI == 16) {
 #pragma unroll
-    for (int f = 0; f < NFRAG; f++) read_frag(0, 0, 0, f);
+      for (int i = 0; i < C::TM; i++) read_a16(0, 0, i);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) read_b16(0, 0, 0, j);
+    } else {
+#pragma unroll
+      for (int f = 0; f < NFRAG; f++) read_frag(0, 0, 0, f);
+    }
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the loop is entered with no LDS read pending
     int kt = 0;
     const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
     EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
-    if constexpr (C::KSUB == 4) {
-      // 128-byte stages, two buffers.  By the end of the third k-step a wave holds the whole of stage kt in
-      // registers (or has used it), so the barrier before the fourth proves stage kt's buffer free, and the requests
-      // of stage kt+2 go out during that k-step while the fragments of stage kt+1 (whose requests were waited for
-      // just before the barrier) are read.  A request carries a whole 128-byte line: the L1 keeps a fixed number
-      // of requests in flight whatever their size.
+    if constexpr (C::MI == 16) {
+      // 128-byte stages, two buffers, stage kt in buffer kt % 2.  During a stage's first k-step the fragments of its
+      // second one are read, after which no wave needs the buffer any more: once every wave has seen its own reads
+      // return and its requests of stage kt+1 land, the block meets, and during the second k-step the fragments of
+      // stage kt+1 are read from the other buffer while stage kt+2 is requested into this one.  A request carries a
+      // whole 128-byte line: the L1 keeps a fixed number of requests in flight whatever their size.  The loop is cut
+      // at the meeting point, where no LDS read may be pending anyway.
+      kstep16(S0{}, T_{}, F_{}, 0, 1, 0, 0);
       for (; kt + 1 < nk; kt++) {
         const int buf = kt % 2;
-        kstep4(S0{}, T_{}, F_{}, buf, 1, 0, 0);
-        kstep4(S1{}, T_{}, F_{}, buf, 2, 0, 0);
-        kstep4(S0{}, T_{}, F_{}, buf, 3, 0, 0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
         wait_vmcnt<0>();
         asm volatile("s_barrier" ::: "memory");
-        kstep4(S1{}, T_{}, T_{}, buf ^ 1, 0, min(kt + 2, nk - 1), buf);
+        kstep16(S1{}, T_{}, T_{}, buf ^ 1, 0, min(kt + 2, nk - 1), buf);
+        kstep16(S0{}, T_{}, F_{}, buf ^ 1, 1, 0, 0);
       }
-      load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, cur.info, wm * C::WM, n_out0, lane);
-      kstep4(S0{}, T_{}, F_{}, kt % 2, 1, 0, 0);
-      kstep4(S1{}, T_{}, F_{}, kt % 2, 2, 0, 0);
-      kstep4(S0{}, T_{}, F_{}, kt % 2, 3, 0, 0);
-      kstep4(S1{}, F_{}, F_{}, 0, 0, 0, 0);
+      load_epilogue_scales<C::TM, NT_OUT, C::GLU, true, C::MI>(esc, p, cur.info, wm * C::WM, n_out0, lane);
+      kstep16(S1{}, F_{}, F_{}, 0, 0, 0, 0);
     } else {
     for (; kt + 1 < nk; kt++) {
       const int buf = kt % C::NSTAGE;
@@ -883,7 +932,7 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
       kstep(S1{}, T_{}, T_{}, (kt + 1) % C::NSTAGE, 0, min(ka, nk - 1), ka % C::NSTAGE, 0);
     }
     // the epilogue's scales are fetched behind the last two k-steps
-    load_epilogue_scales<C::TM, NT_OUT, C::GLU, true>(esc, p, cur.info, wm * C::WM, n_out0, lane);
+    load_epilogue_scales<C::TM, NT_OUT, C::GLU, true, C::MI>(esc, p, cur.info, wm * C::WM, n_out0, lane);
     kstep(S0{}, T_{}, F_{}, kt % C::NSTAGE, 1, 0, 0, 0);
     kstep(S1{}, F_{}, F_{}, 0, 0, 0, 0, 0);
     }
@@ -2132,8 +2181,9 @@ static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* b
   if constexpr (BSRC == BSRC_SAME) {
     // operands that need no conversion stream straight into LDS when every stage is a full 64-byte row slice
     constexpr int ESZ = OP == OP_I8 ? 1 : 2;
-    // 128-byte stages (two buffers) when the rows allow it: 3-7 % faster than 64-byte stages (four buffers) on the
-    // Mixtral shape (tile variant 12 of the int8 path is the 64-byte pipeline, for comparison)
+    // 128-byte stages (two buffers, 16 x 16 MFMAs) when the rows allow it: 6-10 % faster than 64-byte stages (four
+    // buffers, 32 x 32 MFMAs) on the Mixtral shape (tile variant 12 of the int8 path is the 64-byte pipeline, for
+    // comparison)
     if (big && (p.K * ESZ) % 128 == 0) return launch_dl<DlCfg<OP, 256, 256, 128, 2, 4, 2, GLU>>(p, M, G_total, s);
     if (big && (p.K * ESZ) % 64 == 0) return launch_dl<DlCfg<OP, 256, 256, 64, 2, 4, 4, GLU>>(p, M, G_total, s);
   }
