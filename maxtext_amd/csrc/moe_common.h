@@ -91,4 +91,14 @@ __device__ __forceinline__ void dispatch_act(int act, F&& f) {
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 
+// Operands of global_load_lds (global -> LDS copy without staging registers).
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+// s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
 }  // namespace moe

@@ -614,9 +614,6 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
 // address side, because the LDS side of the instruction is fixed (base + 16 * lane).
 // ---------------------------------------------------------------------------------------
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
-
 template <int OP_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, int NSTAGE_, bool GLU_>
 struct DlCfg {
   static constexpr int OP = OP_, BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
@@ -646,12 +643,6 @@ struct DlCfg {
   static_assert(LDS_BYTES <= 160 * 1024, "LDS");
   __device__ static __forceinline__ int swz(int row) { return BKB == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
 };
-
-// s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]).
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
 
 template <typename C>
 __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_kernel(const TiledParams p) {

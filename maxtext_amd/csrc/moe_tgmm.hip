@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kTgThreads) void tgmm_kernel(const TgmmParams p) {
 
   // rows of group g: [start, start + size), clipped to M (sum of the sizes of the groups before it)
   long long part = 0;
-  for (int i = tid; i < g; i += kTgThreads) part += max(p.group_sizes[i], 0);
+  for (int i = tid; i < min(g, p.G_total); i += kTgThreads) part += max(p.group_sizes[i], 0);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o);
   if (lane == 0) s_red[wave] = (int)min(part, (long long)p.M);
@@ -145,6 +145,229 @@ __global__ __launch_bounds__(kTgThreads) void tgmm_kernel(const TgmmParams p) {
   }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// 256 (n) x 256 (k) output tiles for groups of many rows, on the pipeline of the direct-to-LDS GEMM: a stage is
+// 64 contraction rows of both operands (64 x 512 bytes each), copied by global_load_lds_dwordx4 (a wave
+// instruction moves two rows of 512 bytes: whole 128-byte lines) into two buffers of 64 KB; 8 waves of
+// 64 (k) x 128 (n) on v_mfma_f32_16x16x32_bf16, two k-steps of 32 MFMAs per stage; the 4 lhs fragments of a wave
+// are double-buffered in registers, each of its 8 dout fragments is reloaded for the next k-step right after the four
+// MFMAs that use it.  Fragments come out of the row-major stage through ds_read_b64_tr_b16 as in tgmm_kernel.  LDS
+// rows are unpadded, so the 16-byte chunk q of row r is stored at slot q ^ f(r), f(r) = 4 * (r % 4) ^ 2 * ((r / 8) % 2):
+// the 4 rows x 32 bytes that 16 lanes of a transposing read address, and those of the next 16 lanes (8 rows further),
+// then fall into 8 different 32-byte bank groups.  The permutation is applied on the global side (the LDS side of
+// the copy is fixed at base + 16 * lane) and stays inside a row's 512 bytes, so every request still covers whole
+// lines.  Rows past the end of the group are copied from a row of zeros.
+// ---------------------------------------------------------------------------------------
+
+constexpr int kTdTile = 256, kTdBM = 64;       // output tile edge, contraction rows per stage
+constexpr int kTdThreads = 512, kTdWaves = 8;
+constexpr int kTdRow = kTdTile * 2;            // bytes of one operand row in a stage
+constexpr int kTdOperand = kTdBM * kTdRow;     // 32 KB
+constexpr int kTdStage = 2 * kTdOperand;       // lhs rows | dout rows
+constexpr int kTdLds = 2 * kTdStage;           // two buffers
+constexpr int kTdIpw = kTdOperand / 1024 / kTdWaves;  // requests per wave, operand and stage
+constexpr int kTdLps = 2 * kTdIpw;
+
+__device__ __attribute__((aligned(512))) uint8_t tg_zero_row[kTdRow];
+
+__device__ __forceinline__ int td_swz(int row) { return ((row & 3) << 2) ^ (((row >> 3) & 1) << 1); }
+
+__device__ __forceinline__ v8bf td_read_frag(const uint8_t* p) {
+  // p: this lane's 8 bytes of row (4 * group + lane % 16 / 4) of the 16-column block; the second read is 4 rows down
+  const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)p);
+  const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)(p + 4 * kTdRow));
+  typedef short v8s __attribute__((ext_vector_type(8)));
+  const v8s v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(v8bf, v);
+}
+
+__global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t td_smem[];
+  __shared__ int s_red[kTdWaves];
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wk = wave % 4, wn = wave / 4;  // wave tile: 64 k x 128 n
+  const int N = p.N, K = p.K;
+
+  // Blocks b, b + 8, .. run on one XCD: give each XCD a contiguous range of tiles, walked in patches of 8 n-tiles x
+  // 4 k-tiles of one group, so that the 32 blocks an XCD runs at a time share 8 dout and 4 lhs panels in its L2.
+  const int tiles_k = K / kTdTile, tiles_n = N / kTdTile, per_group = tiles_k * tiles_n;
+  const int total = per_group * p.G_local;
+  const int q8 = total / 8, rem = total % 8, xcd = blockIdx.x % 8, loc = blockIdx.x / 8;
+  const int logical = xcd < rem ? xcd * (q8 + 1) + loc : rem * (q8 + 1) + (xcd - rem) * q8 + loc;
+  const int g_local = logical / per_group, t = logical % per_group, g = g_local + p.group_offset;
+  constexpr int GSM = 8;
+  const int width = GSM * tiles_k, first_n = (t / width) * GSM, gsz = min(tiles_n - first_n, GSM);
+  const int n0 = (first_n + (t % width) % gsz) * kTdTile, k0 = ((t % width) / gsz) * kTdTile;
+
+  // rows of group g: [start, start + size), clipped to M
+  long long part = 0;
+  for (int i = tid; i < min(g, p.G_total); i += kTdThreads) part += max(p.group_sizes[i], 0);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o);
+  if (lane == 0) s_red[wave] = (int)min(part, (long long)p.M);
+  __syncthreads();
+  long long start_ll = 0;
+  for (int w = 0; w < kTdWaves; w++) start_ll += s_red[w];
+  // (uniform by construction; saying so lets the requests below use a scalar base address)
+  const int start = __builtin_amdgcn_readfirstlane((int)min(start_ll, (long long)p.M));
+  const int size = __builtin_amdgcn_readfirstlane(g < p.G_total ? min(max(p.group_sizes[g], 0), p.M - start) : 0);
+
+  const int s16 = lane % 16, gq = lane / 16;
+  if (size == 0) {  // an empty group's gradient is zero
+    for (int i = tid; i < kTdTile * (kTdTile / 4); i += kTdThreads) {
+      const size_t off = ((size_t)g_local * N + n0 + i / (kTdTile / 4)) * K + k0 + (i % (kTdTile / 4)) * 4;
+      if (p.out_f32) *(float4*)((float*)p.out + off) = make_float4(0.f, 0.f, 0.f, 0.f);
+      else *(uint2*)((uint16_t*)p.out + off) = make_uint2(0, 0);
+    }
+    return;
+  }
+
+  // ---- sources of this wave's requests: request i of an operand covers stage rows 2 * (4 * wave + i) + {0, 1}.  A
+  // stage's first row is a scalar base, the lane adds a 32-bit offset.  Only a group's last stage can hold rows past its
+  // end: requests of full stages (FULL) need no check, the others pick the row of zeros per lane, without a branch.
+  // Requests i and i + 2 of a wave are 4 rows apart, which leaves the swizzle as it is: two per-lane offsets per operand.
+  uint32_t a_off[2], b_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = 2 * (wave * kTdIpw + i) + lane / 32;
+    const int chunk = (lane % 32) ^ td_swz(r);
+    a_off[i] = (uint32_t)r * K * 2 + chunk * 16;
+    b_off[i] = (uint32_t)r * N * 2 + chunk * 16;
+  }
+  static_assert(kTdIpw == 4, "request i + 2 is request i four rows further down");
+  const uint8_t* const a_base = (const uint8_t*)p.lhs + ((size_t)start * K + k0) * 2;
+  const uint8_t* const b_base = (const uint8_t*)p.dout + ((size_t)start * N + n0) * 2;
+  const size_t a_step = (size_t)kTdBM * K * 2, b_step = (size_t)kTdBM * N * 2;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)td_smem;
+  auto issue_one = [&](auto full_c, int kt, int buf, int idx) {
+    constexpr bool FULL = decltype(full_c)::value;
+    const int i = idx % kTdIpw;
+    const bool is_a = idx < kTdIpw;
+    const uint8_t* src = is_a ? a_base + (kt * a_step + (size_t)(i / 2) * 8 * K) + a_off[i % 2]
+                              : b_base + (kt * b_step + (size_t)(i / 2) * 8 * N) + b_off[i % 2];
+    if constexpr (!FULL) {
+      int l = lane;
+      asm volatile("" : "+v"(l));  // keeps what follows inside the (short) loops that need it, out of the steady state's registers
+      const int r = 2 * (wave * kTdIpw + i) + l / 32;
+      const uint64_t keep = kt * kTdBM + r < size ? ~0ull : 0ull;
+      const uint64_t zero = (uint64_t)(tg_zero_row + ((l % 32) ^ td_swz(r)) * 16);
+      src = (const uint8_t*)(((uint64_t)src & keep) | (zero & ~keep));
+    }
+    // The request is written as asm: the compiler orders every ds_read_b64_tr_b16 behind the global->LDS copies it
+    // knows of (s_waitcnt vmcnt(0) before the read: a full memory latency, four times per stage).  Which buffer a copy
+    // writes and a read reads is settled by the explicit vmcnt waits and barriers below.
+    const uint32_t dst = lds_base + buf * kTdStage + (is_a ? 0 : kTdOperand) + (wave * kTdIpw + i) * 1024;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+  };
+
+  // ---- fragments: lane (group gq, s16) addresses row 8 * gq + s16 / 4 (+ 4) of the k-step's 32 rows and the 8 bytes
+  // 8 * (s16 % 4) of the fragment's 32-byte row slice; fragment f of an operand is 32 * f bytes further along the row
+  // before the swizzle, which turns the step into an XOR of address bits 5..7.
+  const int xmask = ((s16 / 4) << 2) ^ ((gq & 1) << 1);
+  const int row_part = (gq * 8 + s16 / 4) * kTdRow, piece = s16 % 4;
+  const int k_base = row_part + ((((8 * wk + piece / 2) ^ xmask) << 4) | ((piece & 1) << 3));
+  const int n_base = row_part + ((((16 * wn + piece / 2) ^ xmask) << 4) | ((piece & 1) << 3));
+  v8bf fk[2][4], fn[8];
+  // (the two bases pass through an empty asm so that the 12 fragment addresses are formed where they are used, an XOR
+  // and an add each, instead of living in 12 registers across the loop: the kernel has none to spare)
+  auto read_k = [&](int buf, int ks, int set, int f) {
+    int base = k_base;
+    asm volatile("" : "+v"(base));
+    fk[set][f] = td_read_frag(td_smem + buf * kTdStage + ks * 32 * kTdRow + (base ^ (32 * f)));
+  };
+  auto read_n = [&](int buf, int ks, int f) {
+    int base = n_base;
+    asm volatile("" : "+v"(base));
+    fn[f] = td_read_frag(td_smem + buf * kTdStage + kTdOperand + ks * 32 * kTdRow + (base ^ (32 * f)));
+  };
+
+  v4f acc[4][8];  // [k fragment][n fragment]
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[j][i][r] = 0.f;
+
+  // One k-step: 32 MFMAs on lhs fragment set SET with, slotted between them, the fragment reads of the next k-step
+  // (RD) and the requests of a stage (LD, one per MFMA from the start of the k-step).
+  auto kstep = [&](auto set_c, auto rd_c, auto ld_c, auto full_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fk[SET][j], fn[i], acc[j][i], 0, 0, 0);
+        if (LD && i * 4 + j < kTdLps) issue_one(full_c, ld_kt, ld_buf, i * 4 + j);
+        if (RD && j == 1 && i < 4) read_k(rd_buf, rd_ks, SET ^ 1, i);
+        if (RD && j == 3) read_n(rd_buf, rd_ks, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+
+  // Stage kt sits in buffer kt % 2.  During a stage's first k-step the fragments of its second one are read, after
+  // which no wave needs the buffer any more: once every wave has seen its own reads return and its requests of stage
+  // kt+1 land, the block meets, and during the second k-step the fragments of stage kt+1 are read from the other
+  // buffer while stage kt+2 is requested into this one (past the last stage the last one is requested again, into a
+  // buffer nobody reads any more, which keeps the bookkeeping uniform).
+  const int nk = (size + kTdBM - 1) / kTdBM;
+#pragma unroll
+  for (int s = 0; s < 2; s++)
+#pragma unroll
+    for (int i = 0; i < kTdLps; i++) issue_one(F_{}, min(s, nk - 1), s, i);
+  wait_vmcnt<0>();
+  __syncthreads();
+#pragma unroll
+  for (int f = 0; f < 8; f++) read_n(0, 0, f);
+#pragma unroll
+  for (int f = 0; f < 4; f++) read_k(0, 0, 0, f);
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  kstep(S0{}, T_{}, F_{}, F_{}, 0, 1, 0, 0);
+  int kt = 0;
+  const int nfull = size / kTdBM;  // stages 0 .. nfull-1 hold 64 rows of the group
+  for (; kt + 2 < nfull; kt++) {   // steady state: the stage requested is a full one
+    const int buf = kt % 2;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    kstep(S1{}, T_{}, T_{}, T_{}, buf ^ 1, 0, kt + 2, buf);
+    kstep(S0{}, T_{}, F_{}, F_{}, buf ^ 1, 1, 0, 0);
+  }
+  for (; kt + 1 < nk; kt++) {
+    const int buf = kt % 2;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    kstep(S1{}, T_{}, T_{}, F_{}, buf ^ 1, 0, min(kt + 2, nk - 1), buf);
+    kstep(S0{}, T_{}, F_{}, F_{}, buf ^ 1, 1, 0, 0);
+  }
+  kstep(S1{}, F_{}, F_{}, F_{}, 0, 0, 0, 0);
+  wait_vmcnt<0>();  // no request may still be writing LDS when the block ends
+
+  // D[k][n]: the lane holds n = s16 and k = 4 * gq + r of each 16 x 16 tile
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int n = n0 + wn * 128 + i * 16 + s16;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int k = k0 + wk * 64 + j * 16 + 4 * gq;
+      const size_t off = ((size_t)g_local * N + n) * K + k;
+      if (p.out_f32)
+        *(float4*)((float*)p.out + off) = make_float4(acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]);
+      else
+        *(uint2*)((uint16_t*)p.out + off) = make_uint2(pack_bf16x2(acc[j][i][0], acc[j][i][1]), pack_bf16x2(acc[j][i][2], acc[j][i][3]));
+    }
+  }
+}
+
 }  // namespace moe
 
 using namespace moe;
@@ -163,6 +386,20 @@ extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_
   p.lhs = (const uint16_t*)lhs; p.dout = (const uint16_t*)dout; p.group_sizes = group_sizes; p.out = out;
   p.M = M; p.K = K; p.N = N; p.G_total = num_groups_total; p.G_local = num_groups_local; p.group_offset = group_offset;
   p.out_f32 = out_dtype == MOE_F32;
+  // groups of 128 rows and more on average take the 256 x 256 tiles when the shape allows it
+  const long long tiles = (long long)(K / kTdTile) * (N / kTdTile) * num_groups_local;
+  if (K % kTdTile == 0 && N % kTdTile == 0 && K < (1 << 24) && N < (1 << 24) && (long long)M >= 128LL * num_groups_total && tiles >= 128 && tiles <= 0x7fffffffLL) {
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(MOE_ERR_LAUNCH, "tgmm: cannot identify the current device");
+    if (!attr_set[dev]) {  // a race between two host threads only repeats an idempotent call
+      hipError_t e = hipFuncSetAttribute((const void*)tgmm_dl_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kTdLds);
+      if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "tgmm: cannot reserve %d bytes of LDS: %s", kTdLds, hipGetErrorString(e));
+      attr_set[dev] = true;
+    }
+    tgmm_dl_kernel<<<(unsigned)tiles, kTdThreads, kTdLds, (hipStream_t)stream>>>(p);
+    return check_launch("tgmm_dl_kernel");
+  }
   dim3 grid(cdiv(K, kTgBK), cdiv(N, kTgBN), num_groups_local);
   tgmm_kernel<<<grid, kTgThreads, 0, (hipStream_t)stream>>>(p);
   return check_launch("tgmm_kernel");

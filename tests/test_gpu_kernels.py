@@ -399,6 +399,9 @@ TGMM_SHAPES = [
     (520, 200, 72, [500, 20]),  # K, N not multiples of the 128 tile
     (64, 2880, 96, [7, 57]),
     (700, 128, 256, [300, 200]),  # rows past sum(group_sizes) belong to no group
+    # 256 x 256 tiles on the direct-to-LDS pipeline (K, N multiples of 256, 128 rows per group on average, 128 tiles):
+    (1065, 1024, 2048, [300, 0, 700, 65]),  # ragged last stages (44 and 1 rows), an empty group
+    (2100, 512, 4096, [1000, 500, 436, 64]),  # a group of exactly one stage; 100 rows belong to no group
 ]
 
 
@@ -436,6 +439,25 @@ def test_tgmm_exact_on_small_integers_and_group_window(K):
   lhs_nan[:40] = float("nan")
   win = K.tgmm(cuda(lhs_nan), cuda(dout), cuda(gs), num_groups_local=3, group_offset=1, out_dtype=torch.float32)
   assert torch.equal(win.cpu(), want[1:4])
+
+
+def test_tgmm_big_tiles_exact_on_small_integers_and_group_window(K):
+  """The same on a shape that takes the 256 x 256 kernel, whose rows past a group's end come from a row of zeros."""
+  rng = np.random.default_rng(4)
+  m, k, n = 700, 1024, 3072
+  gs = np.array([140, 0, 199, 193, 100], np.int32)  # 68 rows belong to no group
+  lhs = torch.from_numpy(rng.integers(-3, 4, (m, k)).astype(np.float32)).to(torch.bfloat16)
+  dout = torch.from_numpy(rng.integers(-3, 4, (m, n)).astype(np.float32)).to(torch.bfloat16)
+  want = O.tgmm(lhs, dout, gs, out_dtype=torch.float32).transpose(1, 2)
+  got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=torch.float32)
+  assert torch.equal(got.cpu(), want)  # sums of at most 199 products of magnitude <= 9 are exact in f32
+  lhs_nan = lhs.clone()
+  lhs_nan[:140] = float("nan")
+  lhs_nan[632:] = float("nan")
+  win = K.tgmm(cuda(lhs_nan), cuda(dout), cuda(gs), num_groups_local=3, group_offset=1, out_dtype=torch.float32)
+  assert torch.equal(win.cpu(), want[1:4])  # NaN rows of other groups and of no group do not leak into the window
+  got16 = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=torch.bfloat16)
+  assert torch.equal(got16.cpu(), want.to(torch.bfloat16))
 
 
 def test_tgmm_argument_errors(K):
