@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "c2": (2573804 * 2.0 + 473766 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
     "c3": (3852849 * 2.0 + 9236 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
-    "c2_train": (3105239 * 2.0 + 917553 * 1.0) * 1024,  # profiles/tgmm_kernel_bf16_mixtral_shape_train.md
+    "c2_train": (1382444 * 2.0 + 925383 * 1.0) * 1024,  # profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md
 }
 
 
@@ -258,7 +258,7 @@ def train_main(args):
                  "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
       "roofline": dict(bound="mfma", achieved=achieved, peak=PEAK_TFLOPS["bf16"], unit="TFLOP/s", frac=achieved / PEAK_TFLOPS["bf16"],
                        traffic=MEASURED_TRAFFIC_BYTES.get(wl.name + "_train") if args.tokens is None else None,
-                       kernel="tgmm_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
+                       kernel="tgmm_dl_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
       "stage_ms": stage_ms,
   }
   result["calibration"] = calibration("bf16")
