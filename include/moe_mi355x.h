@@ -222,7 +222,16 @@ typedef struct {
  * the existing_out argument of gmm (ops.py:51, backend.py:493-501), where a caller accumulates the shards' rows
  * in one buffer. */
 #define MOE_GMM_KEEP_OTHER_ROWS 1
+/* flags: rhs is [G_local, K, N] with N contiguous, the reference's default layout (transpose_rhs=False, ops.py:47-52),
+ * read as it is: no re-layout pass.  This is how the backward computes dlhs = gmm(dout, rhs, transpose_rhs=True)
+ * (ops.py:470-485) from the forward's [G, N, K] weights, whose roles of K and N are then swapped.  BF16 x BF16 without
+ * rhs_up, on shapes moe_gmm_rhs_kn_supported() accepts (others return MOE_ERR_UNSUPPORTED: re-lay the weights out with
+ * moe_transpose_rhs and call without the flag). */
+#define MOE_GMM_RHS_KN 2
 
+/* 1 when moe_gmm takes MOE_GMM_RHS_KN for this shape (K % 64 == 0, N % 256 == 0, 128 rows per group on average and
+ * enough 256 x 256 tiles to fill the chip), else 0. */
+MOE_API int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total);
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
 MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);
 

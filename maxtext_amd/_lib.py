@@ -18,6 +18,7 @@ MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_TOPK_RAW, MOE_ROUTE_SOFTMA
 ROUTE_BY_NAME = {"softmax_topk": 0, "deepseek": 1, "topk_raw": 2, "softmax_all": 3}
 MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
 MOE_GMM_KEEP_OTHER_ROWS = 1
+MOE_GMM_RHS_KN = 2
 
 ACT_BY_NAME = {None: MOE_ACT_NONE, "silu": MOE_ACT_SILU, "swigluoai": MOE_ACT_SWIGLUOAI, "silu_clip": MOE_ACT_SILU_CLIP}
 
@@ -73,6 +74,7 @@ SIGNATURES = {
     "moe_sort_by_expert": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "moe_gmm_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "moe_gmm_rhs_kn_supported": (c_int, [c_int, c_int, c_int, c_int]),
     "moe_gmm": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
     "moe_tgmm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moe_calib_scratch_bytes": (c_size_t, []),

@@ -95,6 +95,33 @@ inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
+// ds_read_b64_tr_b16, gfx950's transposing LDS load: within 16 lanes, lane L receives the L-th 16-bit column of a
+// 4 x 16 block whose rows are addressed by lanes 0-3, 4-7, ... (8 bytes each).  Two such reads, 4 rows apart, give a
+// lane the 8 contraction values of its channel that a 16 x 16 x 32 (or 32 x 32 x 16) bf16 MFMA fragment holds when the
+// tile is stored with the contraction index as the ROW index.  p: the lane's 8 bytes of the first block.
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4s* lds_v4s_t;
+__device__ __forceinline__ v8bf tr_read_frag(const uint8_t* p, int row_stride) {
+  const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)p);
+  const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)(p + 4 * row_stride));
+  typedef short v8s __attribute__((ext_vector_type(8)));
+  const v8s v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(v8bf, v);
+}
+
+// Swizzle of unpadded 512-byte rows (256 bf16 channels) that are read that way: the 16-byte chunk q of row r is stored
+// at slot q ^ tr_swz(r), so that the 4 rows x 32 bytes which 16 lanes address, and those of the next 16 lanes (8 rows
+// further down), fall into 8 different 32-byte bank groups.  The permutation stays inside aligned 256 bytes of a row.
+__device__ __forceinline__ int tr_swz(int row) { return ((row & 3) << 2) ^ (((row >> 3) & 1) << 1); }
+
+// global -> LDS copy of 16 bytes per lane (1 KB per wave at lds_addr, a wave-uniform LDS byte address) written as asm.
+// For kernels that use the transposing read: the compiler puts s_waitcnt vmcnt(0) before every such read that follows a
+// copy it knows of, a full memory latency several times per stage.  Which buffer a copy writes and a read reads must
+// then be settled by explicit vmcnt waits and barriers.
+__device__ __forceinline__ void dma16_untracked(const void* src, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory", "m0");
+}
+
 // s_waitcnt with only vmcnt constrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]).
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

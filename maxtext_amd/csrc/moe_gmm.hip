@@ -614,9 +614,13 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
 // address side, because the LDS side of the instruction is fixed (base + 16 * lane).
 // ---------------------------------------------------------------------------------------
 
-template <int OP_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, int NSTAGE_, bool GLU_>
+template <int OP_, int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_, int NSTAGE_, bool GLU_, bool RHS_KN_ = false>
 struct DlCfg {
   static constexpr int OP = OP_, BM = BM_, BN = BN_, BKB = BKB_, NSTAGE = NSTAGE_;
+  // RHS_KN: the weights are given as [G, K, N] with N contiguous (the contraction index is the row).  A stage then
+  // holds BK weight rows of BN channels instead of BN rows of BK values, and the weight fragments come out of it
+  // through the transposing LDS read (ds_read_b64_tr_b16), as in the weight-gradient kernel.
+  static constexpr bool RHS_KN = RHS_KN_;
   // rows (= columns) of the MFMA tile: 128-byte stages feed the 16 x 16 instructions (16x16x64 i8 / 16x16x32 bf16: 64
   // bytes of K per row), 64-byte stages the 32 x 32 ones (32x32x32 i8 / 32x32x16 bf16: 32 bytes of K per row)
   static constexpr int MI = BKB == 128 ? 16 : 32;
@@ -640,6 +644,7 @@ struct DlCfg {
   static_assert(!GLU || ((BN / 2) % RPI == 0 && TN % 2 == 0), "GLU halves");
   static_assert((NSTAGE - 1) * LPS < 64, "vmcnt range");
   static_assert(MI == 32 || (NSTAGE == 2 && TM >= TN && TM * TN >= LPS), "16 x 16 pipeline shape");
+  static_assert(!RHS_KN || (OP == 0 && MI == 16 && !GLU && BN == 256 && BK * BN * 2 == BN * BKB), "[G, K, N] weights: bf16, 256 channels");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS");
   __device__ static __forceinline__ int swz(int row) { return BKB == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
 };
@@ -703,23 +708,31 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     }
 #pragma unroll
     for (int i = 0; i < C::B_IPW; i++) {
-      const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
-      const int q = (lane % C::CPR) ^ C::swz(vr);
-      const bool up = C::GLU && vr >= C::BN / 2;
-      const int n = min(t.n0 + (up ? vr - C::BN / 2 : vr), N - 1);
-      b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)t.info.group * N + n) * row_bytes + q * 16;
+      if constexpr (C::RHS_KN) {
+        // a request covers two weight rows (contraction index) of the tile's 256 channels: 2 x 512 bytes
+        const int r = 2 * (wave * C::B_IPW + i) + lane / 32;
+        const int q = (lane % 32) ^ tr_swz(r);
+        b_src[i] = p.rhs + (((size_t)t.info.group * K + r) * N + t.n0) * 2 + q * 16;
+      } else {
+        const int vr = (wave * C::B_IPW + i) * C::RPI + lane / C::CPR;
+        const int q = (lane % C::CPR) ^ C::swz(vr);
+        const bool up = C::GLU && vr >= C::BN / 2;
+        const int n = min(t.n0 + (up ? vr - C::BN / 2 : vr), N - 1);
+        b_src[i] = (up ? p.rhs_up : p.rhs) + ((size_t)t.info.group * N + n) * row_bytes + q * 16;
+      }
     }
   };
 
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
   auto issue_one = [&](int kt, int buf, int idx) {
     const size_t koff = (size_t)kt * C::BKB;
-    uint8_t* s = smem + buf * C::STAGE;
-    if (idx < C::A_IPW) {
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[idx] + koff), (lds_ptr_t)(s + (wave * C::A_IPW + idx) * 1024), 16, 0, 0);
+    const int i = idx < C::A_IPW ? idx : idx - C::A_IPW;
+    const uint8_t* src = idx < C::A_IPW ? a_src[i] + koff : b_src[i] + (C::RHS_KN ? (size_t)kt * C::BK * N * 2 : koff);
+    const int off = buf * C::STAGE + (idx < C::A_IPW ? (wave * C::A_IPW + i) * 1024 : C::BM * C::BKB + (wave * C::B_IPW + i) * 1024);
+    if constexpr (C::RHS_KN) {
+      dma16_untracked(src, lds_base + off);  // the transposing reads below must not wait for the copies in flight
     } else {
-      const int i = idx - C::A_IPW;
-      __builtin_amdgcn_global_load_lds((gbl_ptr_t)(b_src[i] + koff),
-                                       (lds_ptr_t)(s + C::BM * C::BKB + (wave * C::B_IPW + i) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(smem + off), 16, 0, 0);
     }
   };
 
@@ -806,8 +819,20 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   auto read_a16 = [&](int buf, int ks, int i) {
     ga[i] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
   };
+  // [G, K, N] weights: the stage holds 64 rows of 512 bytes; lane (group gq, s16) addresses row 8 * gq + s16 / 4 (+ 4)
+  // of the k-step's 32 rows and the 8 bytes 8 * (s16 % 4) of the fragment's 32-byte row slice; fragment j of the wave is
+  // 32 * j bytes further along the row before the swizzle, which turns the step into an XOR of address bits 5 and 6
+  const int kn_gq = lane / 16, kn_s16 = lane % 16;
+  const int kn_base = (kn_gq * 8 + kn_s16 / 4) * (C::BN * 2) +
+                      ((((8 * wn + (kn_s16 % 4) / 2) ^ (((kn_s16 / 4) << 2) ^ ((kn_gq & 1) << 1))) << 4) | ((kn_s16 & 1) << 3));
   auto read_b16 = [&](int buf, int ks, int set, int j) {
-    gb[set][j] = *(const v4i*)(smem + buf * C::STAGE + (C::BM + b_row[j]) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
+    if constexpr (C::RHS_KN) {
+      int base = kn_base;
+      asm volatile("" : "+v"(base));  // the address is formed here, not kept in a register across the loop
+      gb[set][j] = __builtin_bit_cast(v4i, tr_read_frag(smem + buf * C::STAGE + C::BM * C::BKB + ks * 32 * (C::BN * 2) + (base ^ (32 * j)), C::BN * 2));
+    } else {
+      gb[set][j] = *(const v4i*)(smem + buf * C::STAGE + (C::BM + b_row[j]) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
+    }
   };
   auto kstep16 = [&](auto set_c, auto rd_c, auto ld_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
     constexpr int SET = decltype(set_c)::value;
@@ -2301,6 +2326,14 @@ using namespace moe;
 
 extern "C" {
 
+int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total) {
+  // the 256 x 256 direct-to-LDS kernel is the only one that reads [G, K, N]: whole 64-row stages of 256 channels, groups of
+  // 128 rows and more on average, enough tiles for the chip (the rule by which moe_gmm picks that kernel for [G, N, K] too)
+  if (M <= 0 || K <= 0 || N <= 0 || num_groups_total <= 0) return 0;
+  if (K % 64 != 0 || N % 256 != 0 || (long long)M < 128LL * num_groups_total) return 0;
+  return (long long)max_tiles_for(M, num_groups_total, 256) * (N / 256) >= 128 ? 1 : 0;
+}
+
 size_t moe_gmm_workspace_bytes(int M, int num_groups_total) {
   if (M < 0 || num_groups_total <= 0) return 0;
   return 16 + (size_t)max_tiles_for(M, num_groups_total, 16) * sizeof(TileInfo);
@@ -2432,6 +2465,12 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   }
 
   const int M = a->M, G = a->num_groups_total;
+  if (a->flags & MOE_GMM_RHS_KN) {
+    if (variant != V_BF16 || glu || !moe_gmm_rhs_kn_supported(M, a->K, a->N, G))
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: [G, K, N] weights need bf16 x bf16 without rhs_up and a shape moe_gmm_rhs_kn_supported accepts");
+    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, 256, zero_fill, header, tiles);
+    return launch_dl<DlCfg<OP_BF16, 256, 256, 128, 2, 4, 2, false, true>>(p, M, G, s);
+  }
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
   if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->K % 32 == 0 && a->reserved[0] != 1 &&

@@ -11,9 +11,6 @@
 
 namespace moe {
 
-typedef short v4s __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) v4s* lds_v4s_t;
-
 constexpr int kTgBN = 128, kTgBK = 128, kTgBM = 32;  // output tile [BN x BK], contraction chunk BM rows
 constexpr int kTgThreads = 256;
 constexpr int kTgLdr = kTgBN * 2 + 32;  // LDS row stride in bytes (the pad spreads the 4 rows of a transposing read over the banks)
@@ -171,17 +168,6 @@ constexpr int kTdLps = 2 * kTdIpw;
 
 __device__ __attribute__((aligned(512))) uint8_t tg_zero_row[kTdRow];
 
-__device__ __forceinline__ int td_swz(int row) { return ((row & 3) << 2) ^ (((row >> 3) & 1) << 1); }
-
-__device__ __forceinline__ v8bf td_read_frag(const uint8_t* p) {
-  // p: this lane's 8 bytes of row (4 * group + lane % 16 / 4) of the 16-column block; the second read is 4 rows down
-  const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)p);
-  const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_t)(p + 4 * kTdRow));
-  typedef short v8s __attribute__((ext_vector_type(8)));
-  const v8s v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  return __builtin_bit_cast(v8bf, v);
-}
-
 __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t td_smem[];
   __shared__ int s_red[kTdWaves];
@@ -232,7 +218,7 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int r = 2 * (wave * kTdIpw + i) + lane / 32;
-    const int chunk = (lane % 32) ^ td_swz(r);
+    const int chunk = (lane % 32) ^ tr_swz(r);
     a_off[i] = (uint32_t)r * K * 2 + chunk * 16;
     b_off[i] = (uint32_t)r * N * 2 + chunk * 16;
   }
@@ -252,14 +238,11 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
       asm volatile("" : "+v"(l));  // keeps what follows inside the (short) loops that need it, out of the steady state's registers
       const int r = 2 * (wave * kTdIpw + i) + l / 32;
       const uint64_t keep = kt * kTdBM + r < size ? ~0ull : 0ull;
-      const uint64_t zero = (uint64_t)(tg_zero_row + ((l % 32) ^ td_swz(r)) * 16);
+      const uint64_t zero = (uint64_t)(tg_zero_row + ((l % 32) ^ tr_swz(r)) * 16);
       src = (const uint8_t*)(((uint64_t)src & keep) | (zero & ~keep));
     }
-    // The request is written as asm: the compiler orders every ds_read_b64_tr_b16 behind the global->LDS copies it
-    // knows of (s_waitcnt vmcnt(0) before the read: a full memory latency, four times per stage).  Which buffer a copy
-    // writes and a read reads is settled by the explicit vmcnt waits and barriers below.
-    const uint32_t dst = lds_base + buf * kTdStage + (is_a ? 0 : kTdOperand) + (wave * kTdIpw + i) * 1024;
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+    // (untracked: which buffer a copy writes and a read reads is settled by the explicit vmcnt waits and barriers below)
+    dma16_untracked(src, lds_base + buf * kTdStage + (is_a ? 0 : kTdOperand) + (wave * kTdIpw + i) * 1024);
   };
 
   // ---- fragments: lane (group gq, s16) addresses row 8 * gq + s16 / 4 (+ 4) of the k-step's 32 rows and the 8 bytes
@@ -275,12 +258,12 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
   auto read_k = [&](int buf, int ks, int set, int f) {
     int base = k_base;
     asm volatile("" : "+v"(base));
-    fk[set][f] = td_read_frag(td_smem + buf * kTdStage + ks * 32 * kTdRow + (base ^ (32 * f)));
+    fk[set][f] = tr_read_frag(td_smem + buf * kTdStage + ks * 32 * kTdRow + (base ^ (32 * f)), kTdRow);
   };
   auto read_n = [&](int buf, int ks, int f) {
     int base = n_base;
     asm volatile("" : "+v"(base));
-    fn[f] = td_read_frag(td_smem + buf * kTdStage + kTdOperand + ks * 32 * kTdRow + (base ^ (32 * f)));
+    fn[f] = tr_read_frag(td_smem + buf * kTdStage + kTdOperand + ks * 32 * kTdRow + (base ^ (32 * f)), kTdRow);
   };
 
   v4f acc[4][8];  // [k fragment][n fragment]

@@ -223,13 +223,17 @@ def transpose_rhs(rhs_gkn):
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
             group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None,
-            keep_other_rows=False):
-  """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2])."""
+            keep_other_rows=False, rhs_kn=False):
+  """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2]).
+  rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 without rhs_up, on shapes `gmm_rhs_kn_supported` accepts)."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
   _need(group_sizes, "group_sizes", torch.int32, 1)
   m, kdim = lhs.shape
-  g_local, n, kr = rhs.shape
+  if rhs_kn:
+    g_local, kr, n = rhs.shape
+  else:
+    g_local, n, kr = rhs.shape
   if lhs.dtype not in _DTYPE_CODE:
     raise TypeError(f"lhs dtype {lhs.dtype} not supported")
   if rhs_dtype is None:
@@ -301,12 +305,17 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
   a.partial_sum = partial_sum.data_ptr() if partial_sum is not None else None
   a.partial_sum_up = partial_sum_up.data_ptr() if partial_sum_up is not None else None
-  a.flags = _lib.MOE_GMM_KEEP_OTHER_ROWS if keep_other_rows else 0
+  a.flags = (_lib.MOE_GMM_KEEP_OTHER_ROWS if keep_other_rows else 0) | (_lib.MOE_GMM_RHS_KN if rhs_kn else 0)
   a.reserved[0] = int(tile_variant)
   a.reserved[1] = int(tune)
   st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
   _lib.check(st, "moe_gmm")
   return out
+
+
+def gmm_rhs_kn_supported(m, k, n, num_groups_total):
+  """True when `gmm_raw(..., rhs_kn=True)` takes [G, K, N] bf16 weights of this shape as they are."""
+  return bool(_lib.load().moe_gmm_rhs_kn_supported(int(m), int(k), int(n), int(num_groups_total)))
 
 
 def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16):

@@ -142,6 +142,20 @@ def gmm(
     return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit,
                           bwd_quantize_dtype, rhs_bias, rhs_up_bias)
 
+  # [g, k, n] bf16 weights are read as they are where the kernel allows it (this is dlhs of a transpose_rhs=True layer:
+  # ops.py:470-485), instead of being re-laid out for every call
+  if (not transpose_rhs and rhs_up is None and rhs_quantize_dtype is None and lhs_quantize_dtype is None
+      and not isinstance(rhs, QArray) and not isinstance(lhs, QArray) and rhs.dtype == torch.bfloat16 and lhs.dtype == torch.bfloat16
+      and fuse_act is None and kernels.gmm_rhs_kn_supported(lhs.shape[0], rhs.shape[1], rhs.shape[2], group_sizes.numel())):
+    kw = dict(group_offset=offset, rhs_kn=True)
+    if rhs_bias is not None:
+      kw["rhs_bias"] = rhs_bias.float().contiguous()
+    if partial_sum is not None:
+      kw["partial_sum"] = partial_sum.to(torch.bfloat16).contiguous()
+    if existing_out is not None:
+      kw["out"], kw["keep_other_rows"] = existing_out, True
+    return kernels.gmm_raw(lhs.contiguous(), rhs.contiguous(), group_sizes, **kw)
+
   rhs_n = _native_rhs(rhs, transpose_rhs)
   up_n = _native_rhs(rhs_up, transpose_rhs) if rhs_up is not None else None
   if not isinstance(rhs_n, QArray) and rhs_quantize_dtype is not None:

@@ -20,7 +20,7 @@ def _declared_symbols():
 def test_header_declares_the_expected_entry_points():
   names = _declared_symbols()
   for must in ("moe_route_topk", "moe_sort_by_expert", "moe_gather_rows", "moe_gmm", "moe_unpermute_combine",
-               "moe_gmm_workspace_bytes", "moe_sort_workspace_bytes", "moe_transpose_rhs", "moe_last_error"):
+               "moe_gmm_workspace_bytes", "moe_gmm_rhs_kn_supported", "moe_sort_workspace_bytes", "moe_transpose_rhs", "moe_last_error"):
     assert must in names
 
 

@@ -226,6 +226,43 @@ def test_gmm_bf16(K, m, k, n, gs):
   assert relerr(got, want) <= TOL
 
 
+RHS_KN_SHAPES = [
+    (1065, 192, 3328, [300, 0, 700, 65]),  # three k stages, an empty group, ragged m-tiles
+    (2100, 1024, 2560, [1000, 500, 436, 64]),  # 100 rows belong to no group
+]
+
+
+@pytest.mark.parametrize("m,k,n,gs", RHS_KN_SHAPES)
+def test_gmm_bf16_rhs_kn(K, m, k, n, gs):
+  """[G, K, N] weights (the reference's default layout, ops.py:47-52) read as they are against the oracle and against
+  the same product on re-laid-out [G, N, K] weights, whole and through a window of local groups."""
+  lhs, w, _, gs = _gmm_inputs(m, k, n, gs, 1)
+  wb = w.to(torch.bfloat16)
+  assert K.gmm_rhs_kn_supported(m, k, n, len(gs))
+  got = K.gmm_raw(cuda(lhs), cuda(wb), cuda(gs), rhs_kn=True)
+  want = O.gmm(lhs, wb, gs)
+  assert relerr(got, want) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  assert torch.equal(got, K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs)))  # the same k order in both kernels
+  win = K.gmm_raw(cuda(lhs), cuda(wb[1:3].contiguous()), cuda(gs), rhs_kn=True, group_offset=1)
+  lo, hi = int(gs[0]), int(gs[:3].sum())
+  assert torch.equal(win[lo:hi], got[lo:hi]) and torch.all(win[:lo] == 0) and torch.all(win[hi:] == 0)
+
+
+def test_gmm_rhs_kn_rejects_other_shapes_and_formats(K):
+  gs = torch.tensor([64, 64], dtype=torch.int32, device="cuda")
+  lhs = torch.zeros(128, 64, dtype=torch.bfloat16, device="cuda")
+  assert not K.gmm_rhs_kn_supported(128, 64, 256, 2)  # too few rows per group
+  assert not K.gmm_rhs_kn_supported(4096, 96, 4096, 2) and not K.gmm_rhs_kn_supported(4096, 128, 4224, 2)
+  with pytest.raises(RuntimeError, match="moe_gmm_rhs_kn_supported"):
+    K.gmm_raw(lhs, torch.zeros(2, 64, 256, dtype=torch.bfloat16, device="cuda"), gs, rhs_kn=True)
+  big = torch.zeros(4096, 128, dtype=torch.int8, device="cuda")
+  gs2 = torch.tensor([2048, 2048], dtype=torch.int32, device="cuda")
+  with pytest.raises(RuntimeError, match="moe_gmm_rhs_kn_supported"):
+    K.gmm_raw(big, torch.zeros(2, 128, 4096, dtype=torch.int8, device="cuda"), gs2, rhs_kn=True,
+              lhs_scale=torch.ones(4096, device="cuda"), rhs_scale=torch.ones(2, 4096, device="cuda"))
+
+
 @pytest.mark.parametrize("m,k,n,gs", GMM_SHAPES)
 def test_gmm_int8_weight_only(K, m, k, n, gs):
   lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 2)
@@ -471,15 +508,17 @@ def test_tgmm_argument_errors(K):
     K.tgmm(a.float(), a, gs)
 
 
+# the second shape is large enough for the 256 x 256 kernels: [g, k, n] weights read as they are (the forward of
+# transpose_rhs=False, dlhs of transpose_rhs=True) and the big-tile weight gradient
+@pytest.mark.parametrize("m,k,n,gs", [(450, 256, 192, [200, 0, 70, 150]), (1100, 3328, 3328, [500, 0, 170, 400])])
 @pytest.mark.parametrize("transpose_rhs", [False, True])
-def test_gmm_autograd_matches_torch_autograd(transpose_rhs):
+def test_gmm_autograd_matches_torch_autograd(transpose_rhs, m, k, n, gs):
   """dlhs and drhs of megablox.gmm against torch autograd through a per-group f64 matmul (the custom
   VJP of ops.py:438-527: dlhs = gmm(dout, rhs^T), drhs = tgmm(lhs^T, dout))."""
   from maxtext_amd import megablox
 
   g = torch.Generator().manual_seed(9)
-  m, k, n = 450, 256, 192
-  gs = np.array([200, 0, 70, 150], np.int32)  # 30 trailing rows in no group
+  gs = np.array(gs, np.int32)  # 30 trailing rows in no group
   e = len(gs)
   lhs = (torch.randn(m, k, generator=g)).to(torch.bfloat16)
   w = (torch.randn(e, k, n, generator=g) * 0.05).to(torch.bfloat16)  # [g, k, n]
@@ -908,6 +947,38 @@ def test_tgmm_random_shapes(K):
         assert torch.all(got[i] == 0), tag
       else:
         assert relerr(got[i], want[i]) <= TOL, tag
+
+
+def test_tgmm_random_shapes_big_tiles(K):
+  """Random group sizes on shapes that take the 256 x 256 kernel (K, N multiples of 256, 128 rows per group on average,
+  at least 128 tiles): empty groups, groups shorter than one 64-row stage, ragged last stages, rows of no group, windows."""
+  rng = np.random.default_rng(79)
+  for case in range(6):
+    e = int(rng.integers(2, 7))
+    off = int(rng.integers(0, 2))
+    loc = e - off if case % 2 == 0 else max(1, e - off - 1)
+    tk, tn = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+    while tk * tn * loc < 128:
+      tk, tn = (tk + 1, tn) if tk <= tn else (tk, tn + 1)
+    k, n = tk * 256, tn * 256
+    gs = rng.integers(0, 520, e).astype(np.int32)
+    gs[int(rng.integers(0, e))] = (0, 1, 63, 64, 65, 129)[case]
+    need = 128 * e - int(gs.sum())
+    if need > 0:
+      gs[int(np.argmax(gs))] += need
+    m = int(gs.sum()) + int(rng.integers(0, 70))
+    g = torch.Generator().manual_seed(100 + case)
+    lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    want = O.tgmm(lhs, dout, gs, out_dtype=torch.float32).transpose(1, 2)
+    got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), num_groups_local=loc, group_offset=off, out_dtype=torch.float32)
+    tag = f"case {case}: m={m} k={k} n={n} gs={list(gs)} window=({off},{loc})"
+    assert got.shape == (loc, n, k), tag
+    for i in range(loc):
+      if gs[off + i] == 0:
+        assert torch.all(got[i] == 0), tag
+      else:
+        assert relerr(got[i], want[off + i]) <= TOL, tag
 
 
 @pytest.mark.parametrize("m,k,n,gs", DECODE_SHAPES + [GMM_SHAPES[0], GMM_SHAPES[3]])
