@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     "c2": (2573804 * 2.0 + 473766 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
     "c3": (3852849 * 2.0 + 9236 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
-    "c2_train": (1382444 * 2.0 + 925383 * 1.0) * 1024,  # profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md
+    "c2_train": (1376652 * 2.0 + 924637 * 1.0) * 1024,  # profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md
 }
 
 
