@@ -145,7 +145,7 @@ def calibration(dtype_name, vendor_gemm_shape=None):
   for key, rnd in (("mfma_constant_operands", 0), ("mfma_changing_operands", 1)):
     ms = best_ms(lambda: _lib.check(lib.moe_calib_mfma(code, rnd, iters, _lib.ptr(scratch), stream), "moe_calib_mfma"))
     res[key] = ops / ms / 1e9
-  res["mfma_unit"] = "TOP/s int8 (v_mfma_i32_32x32x32_i8)" if code == _lib.MOE_INT8 else "TFLOP/s bf16 (v_mfma_f32_32x32x16_bf16)"
+  res["mfma_unit"] = "TOP/s int8 (v_mfma_i32_16x16x64_i8)" if code == _lib.MOE_INT8 else "TFLOP/s bf16 (v_mfma_f32_16x16x32_bf16)"
   buf = torch.empty((1 << 31,), dtype=torch.uint8, device="cuda")
   buf.fill_(1)
   ms = best_ms(lambda: _lib.check(lib.moe_calib_read(_lib.ptr(buf), buf.numel(), _lib.ptr(scratch), stream), "moe_calib_read"))

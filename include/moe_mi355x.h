@@ -312,7 +312,8 @@ MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, si
  * Calibration (no counterpart in the reference; used by the benchmark): what this machine sustains with a
  * register-only MFMA loop, with constant operands or operands that change every instruction (random data makes
  * the chip draw more power and lower its clock), and with a plain streaming read.  The caller times the launches.
- *   moe_calib_mfma: dtype MOE_INT8 (v_mfma_i32_32x32x32_i8) or MOE_BF16 (v_mfma_f32_32x32x16_bf16); the launch
+ *   moe_calib_mfma: dtype MOE_INT8 (v_mfma_i32_16x16x64_i8) or MOE_BF16 (v_mfma_f32_16x16x32_bf16), the shapes of
+ *   the GEMM kernels (under the power limit they sustain about a fifth more than the 32 x 32 shapes); the launch
  *   performs moe_calib_mfma_ops(dtype, iters) operations.  scratch: moe_calib_scratch_bytes() bytes.
  *   moe_calib_read: reads `bytes` (16-byte aligned, >= 64 KiB) once, with non-temporal requests that each cover
  *   whole 128-byte lines (the fastest streaming read on this part).

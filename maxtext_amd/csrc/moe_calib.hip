@@ -7,60 +7,49 @@
 
 namespace moe {
 
-constexpr int kCalibAcc = 4;  // independent accumulators per wave: back-to-back MFMAs without dependency stalls
+constexpr int kCalibAcc = 16;   // independent accumulators per wave: back-to-back MFMAs without dependency stalls
+constexpr int kCalibFrag = 8;   // operand fragments per wave that the loop rotates through
 
-template <bool RANDOM>
-__global__ __launch_bounds__(256) void calib_mfma_i8_kernel(int iters, int seed, int* __restrict__ sink) {
-  v4i a = {seed + (int)threadIdx.x, seed * 3, seed * 5 + (int)threadIdx.x * 7, seed * 11};
-  v4i b = {seed * 13, (int)threadIdx.x * 17, seed, seed * 23};
-  v16i acc[kCalibAcc];
+// The 16 x 16 instructions of the GEMM kernels (16x16x64 i8, 16x16x32 bf16).  CHANGING: every MFMA takes another pair
+// of the 8 + 8 fragments a lane holds (random bits, drawn before the loop: no VALU work inside it), so the operand
+// buses toggle as they do on real data; otherwise all fragments are equal.  BF16: the random bits are confined to sign
+// and mantissa of values in +-[0.5, 1).
+template <bool BF16, bool CHANGING>
+__global__ __launch_bounds__(256) void calib_mfma_kernel(int iters, int seed, int* __restrict__ sink) {
+  unsigned s = seed * 7919u + threadIdx.x * 104729u + blockIdx.x * 1299709u;
+  v4i fa[kCalibFrag], fb[kCalibFrag];
+#pragma unroll
+  for (int i = 0; i < kCalibFrag; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      unsigned x = 0x01010101u, y = 0x01010101u;
+      if (CHANGING) {
+        s = s * 1664525u + 1013904223u; x = s ^ (s >> 15);
+        s = s * 1664525u + 1013904223u; y = s ^ (s >> 15);
+      }
+      if (BF16) { x = (x & 0x807f807fu) | 0x3f003f00u; y = (y & 0x807f807fu) | 0x3f003f00u; }
+      fa[i][c] = x; fb[i][c] = y;
+    }
+  typedef typename std::conditional<BF16, v4f, v4i>::type acc_t;
+  acc_t acc[kCalibAcc];
 #pragma unroll
   for (int i = 0; i < kCalibAcc; i++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[i][r] = 0;
+    for (int r = 0; r < 4; r++) acc[i][r] = 0;
   for (int it = 0; it < iters; it++) {
 #pragma unroll
     for (int i = 0; i < kCalibAcc; i++) {
-      if (RANDOM) {  // one word of each operand moves every instruction (a linear congruential step)
-        a[i & 3] = a[i & 3] * 1664525 + 1013904223;
-        b[i & 3] = b[i & 3] * 22695477 + 1;
-      }
-      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i], 0, 0, 0);
+      const int ia = i % kCalibFrag, ib = (i / 2 + 3 * (i & 1)) % kCalibFrag;
+      if constexpr (BF16) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, fa[ia]), __builtin_bit_cast(v8bf, fb[ib]), acc[i], 0, 0, 0);
+      else acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[ia], fb[ib], acc[i], 0, 0, 0);
     }
   }
-  int s = 0;
+  int sum = 0;
 #pragma unroll
   for (int i = 0; i < kCalibAcc; i++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) s += acc[i][r];
-  sink[blockIdx.x * 256 + threadIdx.x] = s;
-}
-
-template <bool RANDOM>
-__global__ __launch_bounds__(256) void calib_mfma_bf16_kernel(int iters, int seed, int* __restrict__ sink) {
-  v4i a = {0x3f803f80 + seed, 0x3f003f80, 0x40003f00 + (int)threadIdx.x, 0x3f803f00};
-  v4i b = {0x3f003f80, 0x3f803f80 + (int)threadIdx.x, 0x3f803f00, 0x40003f80};
-  v16f acc[kCalibAcc];
-#pragma unroll
-  for (int i = 0; i < kCalibAcc; i++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
-  for (int it = 0; it < iters; it++) {
-#pragma unroll
-    for (int i = 0; i < kCalibAcc; i++) {
-      if (RANDOM) {  // mantissa and low exponent bits move, the values stay finite and of order one
-        a[i & 3] = (a[i & 3] * 1664525 + 1013904223) & 0x00ff00ff | 0x3f003f00;
-        b[i & 3] = (b[i & 3] * 22695477 + 1) & 0x00ff00ff | 0x3f003f00;
-      }
-      acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc[i], 0, 0, 0);
-    }
-  }
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < kCalibAcc; i++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) s += acc[i][r];
-  sink[blockIdx.x * 256 + threadIdx.x] = (int)s;
+    for (int r = 0; r < 4; r++) sum += (int)acc[i][r];
+  sink[blockIdx.x * 256 + threadIdx.x] = sum;
 }
 
 // every wave reads 8 KB per step with non-temporal requests of 1 KB (whole 128-byte lines: the request shape that
@@ -90,7 +79,7 @@ extern "C" {
 size_t moe_calib_scratch_bytes(void) { return (size_t)kCalibBlocks * 256 * sizeof(int); }
 
 double moe_calib_mfma_ops(int dtype, int iters) {
-  const double per_mfma = dtype == MOE_INT8 ? 2.0 * 32 * 32 * 32 : 2.0 * 32 * 32 * 16;
+  const double per_mfma = dtype == MOE_INT8 ? 2.0 * 16 * 16 * 64 : 2.0 * 16 * 16 * 32;
   return (double)kCalibBlocks * 4 * (double)iters * kCalibAcc * per_mfma;
 }
 
@@ -99,11 +88,11 @@ int moe_calib_mfma(int dtype, int random_operands, int iters, void* scratch, voi
   hipStream_t s = (hipStream_t)stream;
   int* sink = (int*)scratch;
   if (dtype == MOE_INT8) {
-    if (random_operands) calib_mfma_i8_kernel<true><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
-    else calib_mfma_i8_kernel<false><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
+    if (random_operands) calib_mfma_kernel<false, true><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
+    else calib_mfma_kernel<false, false><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
   } else if (dtype == MOE_BF16) {
-    if (random_operands) calib_mfma_bf16_kernel<true><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
-    else calib_mfma_bf16_kernel<false><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
+    if (random_operands) calib_mfma_kernel<true, true><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
+    else calib_mfma_kernel<true, false><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
   } else {
     return fail(MOE_ERR_UNSUPPORTED, "calib_mfma: dtype %d", dtype);
   }
