@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by a 1 GiB copy dispatch of the same run (profiles/pmc_traffic_*.md); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "c2": (2573804 * 2.0 + 473766 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
+    "c2": (2590968 * 2.0 + 473766 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
     "c3": (3852849 * 2.0 + 9236 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
     "c2_train": (1376652 * 2.0 + 924637 * 1.0) * 1024,  # profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md
 }
