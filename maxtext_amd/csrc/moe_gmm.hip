@@ -2196,20 +2196,26 @@ static int launch_tiled_by_rows(const TiledParams& p, int M, int G_total, int* b
   // 128-row tiles.  Measured against the 64-row tiles on the Mixtral, Qwen3 and GPT-OSS shapes they are 15-35 % faster
   // from 32 rows per expert on (one weight conversion / tile fetch serves twice the rows), and 256-row tiles would be
   // half empty; below 32 rows per expert the 64-row tiles stay.
-  const bool mid = (long long)M >= 32LL * G_total && (long long)M < (BSRC == BSRC_SAME ? 128LL : 144LL) * G_total;
-  *bm_out = mid ? 128 : big ? 256 : 64;
+  const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
+  const bool mid_wq = BSRC != BSRC_SAME && (long long)M >= 32LL * G_total && (long long)M < 144LL * G_total;
+  // one decision for the tile map (bm_out, on the dry run) and for the launch
+  constexpr int ESZ = OP == OP_I8 ? 1 : 2;
+  enum { K_T64, K_T128, K_T256, K_DL128, K_DL64 } kind = K_T64;
+  if (mid || mid_wq) kind = K_T128;
+  else if (big && BSRC == BSRC_SAME && (p.K * ESZ) % 128 == 0) kind = K_DL128;
+  else if (big && BSRC == BSRC_SAME && (p.K * ESZ) % 64 == 0) kind = K_DL64;
+  else if (big) kind = K_T256;
+  *bm_out = kind == K_T64 ? 64 : kind == K_T128 ? 128 : 256;
   if (dry) return MOE_OK;
   if constexpr (BSRC == BSRC_SAME) {
-    // operands that need no conversion stream straight into LDS when every stage is a full 64-byte row slice
-    constexpr int ESZ = OP == OP_I8 ? 1 : 2;
-    // 128-byte stages (two buffers, 16 x 16 MFMAs) when the rows allow it: 6-10 % faster than 64-byte stages (four
-    // buffers, 32 x 32 MFMAs) on the Mixtral shape (tile variant 12 of the int8 path is the 64-byte pipeline, for
-    // comparison)
-    if (big && (p.K * ESZ) % 128 == 0) return launch_dl<DlCfg<OP, 256, 256, 128, 2, 4, 2, GLU>>(p, M, G_total, s);
-    if (big && (p.K * ESZ) % 64 == 0) return launch_dl<DlCfg<OP, 256, 256, 64, 2, 4, 4, GLU>>(p, M, G_total, s);
+    // operands that need no conversion stream straight into LDS when every stage is a full row slice: 128-byte stages
+    // (two buffers, 16 x 16 MFMAs) when the rows allow it, 6-10 % faster than 64-byte stages (four buffers, 32 x 32 MFMAs)
+    // on the Mixtral shape (tile variant 12 of the int8 path is the 64-byte pipeline, for comparison)
+    if (kind == K_DL128) return launch_dl<DlCfg<OP, 256, 256, 128, 2, 4, 2, GLU>>(p, M, G_total, s);
+    if (kind == K_DL64) return launch_dl<DlCfg<OP, 256, 256, 64, 2, 4, 4, GLU>>(p, M, G_total, s);
   }
-  if (mid) return launch_tiled<TiledCfg<OP, BSRC, 128, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
-  if (big) return launch_tiled<TiledCfg<OP, BSRC, 256, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
+  if (kind == K_T128) return launch_tiled<TiledCfg<OP, BSRC, 128, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
+  if (kind == K_T256) return launch_tiled<TiledCfg<OP, BSRC, 256, 256, 128, 2, 4, GLU>>(p, M, G_total, s);
   return launch_tiled<TiledCfg<OP, BSRC, 64, 256, 128, 1, 4, GLU>>(p, M, G_total, s);
 }
 

@@ -197,6 +197,7 @@ GMM_SHAPES = [
     (1024, 320, 200, [300, 0, 500, 200]),
     (1500, 1024, 512, [256, 257, 255, 700]),
     (520, 2880, 96, [500, 20]),
+    (1010, 256, 264, [300, 20, 0, 130, 250, 40, 160, 100, 0, 10]),  # 128-row tiles, groups of one to three tiles
 ]
 
 
