@@ -2484,14 +2484,16 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, 256, zero_fill, header, tiles);
     return launch_dl<DlCfg<OP_BF16, 256, 256, 128, 2, 4, 2, false, true>>(p, M, G, s);
   }
+  const bool int4_g128 = variant == V_W4 && a->rhs_scale_block_k != 32;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
-  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= 32LL * G && a->K % 32 == 0 && a->reserved[0] != 1 &&
+  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= (int4_g128 ? 56LL : 32LL) * G && a->K % 32 == 0 && a->reserved[0] != 1 &&
       (long long)a->N * a->K < (1LL << 31)) {
     // 16-row tiles up to 16 rows per expert on average, 32-row tiles above; group-128 int4 keeps the 16-row tiles over the
     // whole range (its 32-row variant runs at two waves per SIMD: 0.36 against 0.44 ms on the GPT-OSS shape at 256 tokens)
-    const long long one_hi = (variant == V_W4 && a->rhs_scale_block_k != 32) ? 32 : 16;
-    const bool one = (long long)M <= one_hi * G;
+    // and stays on this kernel up to 56 rows per expert (0.43 / 0.48 ms at 320 / 384 tokens against 0.52 / 0.58 ms on
+    // the 128-row tiles of the register-staged kernel; level at 512 tokens)
+    const bool one = int4_g128 || (long long)M <= 16LL * G;
     bm = one ? 16 : 32;
     tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
     WqSkinnyParams q;

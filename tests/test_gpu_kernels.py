@@ -198,6 +198,7 @@ GMM_SHAPES = [
     (1500, 1024, 512, [256, 257, 255, 700]),
     (520, 2880, 96, [500, 20]),
     (1010, 256, 264, [300, 20, 0, 130, 250, 40, 160, 100, 0, 10]),  # 128-row tiles, groups of one to three tiles
+    (400, 256, 264, [90, 0, 30, 45, 17, 60, 33, 50, 75]),  # 44 rows per group: group-128 int4 streams with up to six 16-row tiles per group
 ]
 
 
