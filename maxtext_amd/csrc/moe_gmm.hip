@@ -2485,9 +2485,13 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
     return launch_dl<DlCfg<OP_BF16, 256, 256, 128, 2, 4, 2, false, true>>(p, M, G, s);
   }
   const bool int4_g128 = variant == V_W4 && a->rhs_scale_block_k != 32;
+  // rows per expert up to which the streaming kernel beats the register-staged one (measured on the GPT-OSS and Qwen3
+  // shapes): 56 for group-128 int4, 64 for MXFP4 (0.38 / 0.41 / 0.49 ms at 320 / 384 / 512 tokens against 0.46 / 0.51 /
+  // 0.53 ms), 32 for int8 and group-32 int4
+  const long long stream_rows_hi = int4_g128 ? 56 : variant == V_MX4 ? 64 : 32;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
-  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= (int4_g128 ? 56LL : 32LL) * G && a->K % 32 == 0 && a->reserved[0] != 1 &&
+  if ((variant == V_W8 || variant == V_W4 || variant == V_MX4) && (long long)M <= stream_rows_hi * G && a->K % 32 == 0 && a->reserved[0] != 1 &&
       (long long)a->N * a->K < (1LL << 31)) {
     // 16-row tiles up to 16 rows per expert on average, 32-row tiles above; group-128 int4 keeps the 16-row tiles over the
     // whole range (its 32-row variant runs at two waves per SIMD: 0.36 against 0.44 ms on the GPT-OSS shape at 256 tokens)
