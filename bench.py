@@ -60,7 +60,7 @@ def dominant_kernel_model(wl, group_sizes):
   rows = int(group_sizes.sum())
   nonempty = int((group_sizes > 0).sum())
   flops = 4.0 * rows * d * f
-  if wl.weight_quant == "fp8" and rows > 16 * len(group_sizes):
+  if wl.weight_quant == "fp8" and rows > 14 * len(group_sizes):
     # many rows per expert (prefill): the LDS-tiled kernel, bound by the fp8 MFMA rate
     return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS["fp8"], scale=1e12,
                 name="gmm_fp8_tiled_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")

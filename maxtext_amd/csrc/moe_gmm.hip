@@ -2387,15 +2387,16 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
       return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs 1x128 lhs scales and 128x128 rhs scales");
     if (a->K % 128 != 0) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs K %% 128 == 0 (K=%d)", a->K);
     if ((long long)a->N * a->K >= (1LL << 31)) return fail(MOE_ERR_UNSUPPORTED, "gmm: fp8 needs N * K < 2^31");
-    // Up to 16 rows per expert on average (decode): the streaming kernel with 16-row tiles, one MFMA row tile per
+    // Up to 14 rows per expert on average (decode): the streaming kernel with 16-row tiles, one MFMA row tile per
     // wave; a group with more rows simply gets several tiles, which are adjacent in the grid, run at the same time
     // and share the group's weights through L2.  Beyond that the LDS-tiled kernel with 128 x 128 tiles (measured on
-    // 256 experts of 7168 x 2048: crossover at 16 rows per expert; the 256 x 256 kernel is within 5 % of it from 128
+    // 256 experts of 7168 x 2048: at 12 rows per expert 1.27 against 1.52 ms, at 16, where half of the experts need a
+    // second 16-row tile, 1.66 against 1.54 ms; the 256 x 256 kernel is within 5 % of it from 128
     // rows per expert on and behind it below, so it is not picked by default).  reserved[0] = 1 / 2 / 3 forces the
     // streaming kernel (64-row tiles past 16 rows per expert) / 128 x 128 tiles / 256 x 256 tiles (tuning aid).
     const int forced = a->reserved[0] >= 1 && a->reserved[0] <= 3 ? a->reserved[0] : 0;
     const bool few_rows = (long long)a->M <= 16LL * a->num_groups_total;
-    const bool tiled = forced ? forced >= 2 : !few_rows;
+    const bool tiled = forced ? forced >= 2 : (long long)a->M > 14LL * a->num_groups_total;
     if (tiled) {
       const bool big = forced == 3;
       bm = big ? 256 : 128;
