@@ -415,6 +415,76 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
   }
 }
 
+// All three passes in one block for at most kSortChunk entries (decode: a launch costs as much as a pass): per-wave
+// histograms in LDS, the prefixes over the four segments and over the experts, then the same in-order ranking.
+__global__ __launch_bounds__(kSortWaves* kWave) void sort_small_kernel(
+    const int32_t* __restrict__ flat, int M, int E, int ebits, int32_t* __restrict__ group_sizes,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts) {
+  __shared__ int run[kSortWaves][kSortMaxE];
+  __shared__ int off[kSortMaxE];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  for (int e = threadIdx.x; e < kSortWaves * kSortMaxE; e += kSortWaves * kWave) run[e / kSortMaxE][e % kSortMaxE] = 0;
+  __syncthreads();
+  const int base = wave * kSortSeg;
+#pragma unroll
+  for (int r = 0; r < kSortRounds; r++) {
+    const int i = base + r * kWave + lane;
+    if (i < M) atomicAdd(&run[wave][clamp_expert(flat[i], E)], 1);
+  }
+  __syncthreads();
+  // counts of the segments -> exclusive prefixes over the segments; the expert's total goes to group_sizes and to off
+  for (int e = threadIdx.x; e < kSortMaxE; e += kSortWaves * kWave) {
+    int running = 0;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; w++) {
+      const int c = run[w][e];
+      run[w][e] = running;
+      running += c;
+    }
+    off[e] = running;
+    if (e < E) group_sizes[e] = running;
+  }
+  __syncthreads();
+  for (int o = 1; o < kSortMaxE; o <<= 1) {  // inclusive scan of the totals
+    int add[kSortMaxE / (kSortWaves * kWave)];
+#pragma unroll
+    for (int q = 0; q < kSortMaxE / (kSortWaves * kWave); q++) {
+      const int e = threadIdx.x + q * kSortWaves * kWave;
+      add[q] = e >= o ? off[e - o] : 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < kSortMaxE / (kSortWaves * kWave); q++) off[threadIdx.x + q * kSortWaves * kWave] += add[q];
+    __syncthreads();
+  }
+  for (int e = lane; e < E; e += kWave) run[wave][e] += e > 0 ? off[e - 1] : 0;
+  __syncthreads();
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  for (int r = 0; r < kSortRounds; r++) {
+    const int i = base + r * kWave + lane;
+    const bool valid = i < M;
+    const int e = valid ? clamp_expert(flat[i], E) : 0;
+    unsigned long long mask = __ballot(valid);
+    for (int b = 0; b < ebits; b++) {
+      const bool bit = (e >> b) & 1;
+      const unsigned long long bal = __ballot(valid && bit);
+      mask &= bit ? bal : ~bal;
+    }
+    const int rank = __popcll(mask & lt);
+    const int cnt = __popcll(mask);
+    const int start = valid ? run[wave][e] : 0;
+    __builtin_amdgcn_wave_barrier();
+    if (valid && rank == cnt - 1) run[wave][e] = start + cnt;
+    __builtin_amdgcn_wave_barrier();
+    if (valid) {
+      const int dest = start + rank;
+      perm[dest] = i;
+      if (inv_perm) inv_perm[i] = dest;
+      if (sorted_experts) sorted_experts[dest] = e;
+    }
+  }
+}
+
 __global__ void invert_perm_kernel(const int32_t* __restrict__ perm, int M,
                                    int32_t* __restrict__ inv) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -848,6 +918,10 @@ int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* pe
   hipStream_t s = (hipStream_t)stream;
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
+  if (nblk <= 1) {  // also M == 0: group_sizes are all zero
+    sort_small_kernel<<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    return check_launch("sort_by_expert");
+  }
   if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, seg_hist);
   sort_scan_kernel<<<cdiv(E, kSortWaves), kSortWaves * kWave, 0, s>>>(seg_hist, nseg, E, group_sizes);
   if (nblk > 0)

@@ -97,7 +97,7 @@ def _zipf_selection(rng, t, e, k, s=1.2):
   return np.argsort(-logits, -1, kind="stable")[:, :k].astype(np.int32)
 
 
-@pytest.mark.parametrize("t,e,k", [(1, 8, 2), (7, 8, 2), (128, 8, 2), (1000, 128, 8), (4099, 256, 8), (2048, 32, 4), (513, 512, 3)])
+@pytest.mark.parametrize("t,e,k", [(1, 8, 2), (7, 8, 2), (128, 8, 2), (512, 8, 2), (128, 256, 8), (341, 512, 3), (1000, 128, 8), (4099, 256, 8), (2048, 32, 4), (513, 512, 3)])
 def test_sort_by_expert_bit_exact(K, t, e, k):
   rng = np.random.default_rng(e + t)
   sel = _zipf_selection(rng, t, e, k) if e >= 32 else np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
