@@ -11,8 +11,9 @@
  *   - `group_sizes` stays on the device: no entry point reads it on the host;
  *   - inputs are never written; outputs are fully defined (rows that belong to no
  *     local group are written as zeros), so buffers need no pre-clearing;
- *   - no global mutable state: calls on different streams with disjoint buffers
- *     may overlap.
+ *   - calls on different streams with disjoint buffers may overlap; the only state the library keeps is per device
+ *     and written once (the CU count and "this kernel may use more than 64 KB of LDS"), set up on the first call
+ *     that needs it or ahead of time by moe_init().
  *
  * Paths in the citations are relative to the reference (AI-Hypercomputer/maxtext).
  */
@@ -134,20 +135,35 @@ MOE_API int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int
 /* ---------------------------------------------------------------------------
  * Row gather with optional quantisation.  Replaces the data half of permute
  * (moe.py:956-959: repeat(x, k)[perm]) fused with the activation quantiser of
- * the grouped GEMM (kernels/megablox/ops.py:241-248, per-row scale;
- * pallas_mosaic_tpu_v2_gmm_kernel.py:534-542, per-K-block scale).
+ * the grouped GEMM.  Two quantisation rules (moe_quant_rule):
+ *
+ *   MOE_QUANT_RINT_DIV  scale = absmax / qmax, q = rint(x / scale) clipped to +-qmax, in f32; zero absmax gives
+ *                       q = 0, scale = 0.  Serves the v1 path, kernels/megablox/ops.py:241-248 (one scale per row,
+ *                       channelwise_axes=[0]); its quantiser is third-party (qwix.pallas.quantize), so the rounding
+ *                       rule is this library's choice, not a restatement.
+ *   MOE_QUANT_V2        the quantiser inside gmm_v2, pallas_mosaic_tpu_v2_gmm_kernel.py:528-542, op by op in the
+ *                       activation dtype (bf16): scale = bf16(absmax / qmax); inv = scale == 0 ? 0 : bf16(1 / scale);
+ *                       q = bf16(x * inv) cast as `.astype` does: truncated toward zero for int8, rounded to nearest
+ *                       even for fp8.  With static_scale (the per-tensor (1, 1) lhs_scale of :528-531, ops.py:333-360):
+ *                       s = bf16(*static_scale), inv = bf16(1 / s), q = clip(bf16(x * inv), +-qmax) cast the same way.
  *
  *   x        [R_in, d] bf16
  *   row_idx  [R_out] i32 or NULL; output row i reads input row row_idx[i] / idx_div
- *            (NULL: row i).  permute passes row_idx = perm, idx_div = k.
- *   out      [R_out, d] of out_dtype: MOE_BF16 (copy), MOE_INT8, MOE_FP8_E4M3
- *   scale    f32; block_k == 0: [R_out] one scale per row; else [R_out, ceil(d/block_k)]
- *            (block_k must be 128).  scale = absmax / qmax, q = rint(x / scale)
- *            clipped to +-qmax (127 / 448); zero absmax gives q = 0, scale = 0.
+ *            (NULL: row i).  permute passes row_idx = perm, idx_div = k.  An index outside [0, R_in) yields a row of zeros.
+ *   out      [R_out, d] of out_dtype: MOE_BF16 (copy), MOE_INT8, MOE_FP8_E4M3 (qmax 127 / 448)
+ *   scale    f32 out; block_k == 0: [R_out] one scale per row; block_k in {128, 256, 512}: [R_out, ceil(d/block_k)]
+ *            (gmm_v2 uses 512, :1231; the DeepSeek recipe 1 x 128).  Not written when static_scale is given.
+ *   static_scale  [1] f32 on the device, or NULL for dynamic (absmax) scales
+ *   row_weight    [R_out] f32 or NULL: the gathered row is multiplied by its weight first (x[indices] * weights[:, None],
+ *                 the weighted ragged_gather of kernels/ragged/ragged_gather.py:310-320; product rounded to bf16)
+ *   row_range     [2] i32 (start, end) on the device, or NULL: output rows outside [start, end) are written as zeros
+ *                 (ragged_gather.py:357-376 leaves them unspecified)
  * Limits: d % 8 == 0, d <= 16384.
  */
-MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_out, int d,
-                    int out_dtype, int block_k, void* out, float* scale, void* stream);
+typedef enum { MOE_QUANT_RINT_DIV = 0, MOE_QUANT_V2 = 1 } moe_quant_rule;
+MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_in, int R_out, int d,
+                    int out_dtype, int block_k, int rule, const float* static_scale, const float* row_weight,
+                    const int32_t* row_range, void* out, float* scale, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Grouped matmul.  Replaces gmm(lhs, rhs, group_sizes, ...)
@@ -162,26 +178,43 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  * (reference_gmm, tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:139-141).
  *
  * Operand layouts in HBM
- *   lhs        [M, K] row-major, lhs_dtype in {BF16, INT8, FP8_E4M3}
- *   lhs_scale  f32: NULL (bf16 lhs) | [M] per row (lhs_scale_block_k == 0)
- *              | [M, ceil(K/128)] (lhs_scale_block_k == 128)
+ *   lhs        [M, K] row-major ([lhs_rows, K] with lhs_row_idx), lhs_dtype in {BF16, INT8, FP8_E4M3}
+ *   lhs_scale  f32: NULL (bf16 lhs) | [M] one per row (lhs_scale_block_k == 0; qpl.quantize channelwise_axes=[0],
+ *              ops.py:241-248) | [1] one for the tensor (lhs_scale_block_k == MOE_SCALE_PER_TENSOR; the static (1, 1)
+ *              lhs_scale of gmm_v2, ops.py:333-360) | [M, ceil(K / b)] one per row and b values of K
+ *              (lhs_scale_block_k == b: 128 for the DeepSeek 1 x 128 recipe, 512 for gmm_v2's in-kernel quantiser,
+ *              pallas_mosaic_tpu_v2_gmm_kernel.py:1231; any multiple of 128)
  *   rhs        [G_local, N, K], K contiguous ("transpose_rhs" layout, ops.py:52),
- *              rhs_dtype in {BF16, INT8, FP8_E4M3, INT4}; INT4 rows hold K/2 bytes
- *   rhs_scale  NULL (bf16 rhs) | [G_local, ceil(N/bn), nkb] with
- *              bn = rhs_scale_block_n (1 = per output channel, 128 = DeepSeek 128x128 blocks),
- *              nkb = 1 when rhs_scale_block_k == 0 (per channel over all of K), else
- *              ceil(K / rhs_scale_block_k) (128; INT4 also 32, the Kimi-K2 group size); f32, or bf16 for INT4;
- *              MXFP4: bytes [G_local, N, K/32] (rhs_scale_block_n = 1, rhs_scale_block_k = 32)
+ *              rhs_dtype in {BF16, INT8, FP8_E4M3, INT4, MXFP4}; INT4 / MXFP4 rows hold K/2 bytes
+ *   rhs_scale  NULL (bf16 rhs), else scales over blocks of bn = rhs_scale_block_n output channels (1 = per channel,
+ *              128 = DeepSeek 128 x 128 blocks, MOE_SCALE_PER_TENSOR = one for all channels) and bk = rhs_scale_block_k
+ *              values of K (0 = all of K).  With nnb = ceil(N / bn) and nkb = ceil(K / bk) the layout is
+ *                [G_local, nnb, nkb]                     by default (DeepSeek fp8 checkpoints, int4 group scales), or
+ *                [G_local, nkb, nnb]                     with MOE_GMM_RHS_SCALE_KMAJOR: gmm_v2's [G, nb, 1, N]
+ *                                                        (ops.py:310-331; bn == 1, bk a multiple of 128, for INT8 / FP8
+ *                                                        lhs; a multiple of 32 for weight-only INT8 / INT4);
+ *              MOE_GMM_RHS_SCALE_SHARED drops the leading dimension: one set of scales for all experts (the
+ *              [1, 1, n] scale qpl.quantize yields for channelwise_axes=[2], ops.py:250-260, and the per-tensor scale
+ *              of manual_quantize, layers/quantizations.py:961-991).  f32; bf16 for INT4 in the default layout;
+ *              MXFP4: e8m0 bytes [G_local, N, K/32] (bn = 1, bk = 32)
  *   rhs_up / rhs_up_scale   second projection (wi_1) with the same layout; when non-NULL
  *              the kernel computes act(lhs@rhs^T) * (lhs@rhs_up^T) in one pass
  *   rhs_bias / rhs_up_bias   [G_local, N] f32 or NULL, see the end of the struct
- *   out        [M, N] bf16
+ *   out        [M, N] bf16, or f32 (out_dtype == MOE_F32: preferred_element_type of ops.py:50)
  *
  * Supported operand combinations (others return MOE_ERR_UNSUPPORTED):
- *   BF16 x BF16 | BF16 x INT8 (per-channel) | BF16 x INT4 (bn=1, bk=128 or 32) | BF16 x MXFP4 (bn=1, bk=32)
- *   INT8 (per-row) x INT8 (per-channel) | FP8 (1x128) x FP8 (128x128 blocks)
+ *   BF16 x BF16
+ *   BF16 x INT8   per channel or per tensor (bk = 0), or KMAJOR [G, nkb, N]
+ *   BF16 x INT4   bf16 [G, N, ceil(K/bk)] with bk = 128 or 32, or f32 KMAJOR [G, nkb, N]
+ *   BF16 x MXFP4
+ *   INT8 x INT8, FP8 x FP8:
+ *     lhs per row or per tensor  x  rhs per channel or per tensor over all of K (what gmm() quantises to, ops.py:232-267)
+ *     lhs per row / per tensor / [M, K/b]  x  rhs KMAJOR per channel [G, nkb, N] (gmm_v2's layouts; K % 128 == 0)
+ *     FP8 only: lhs [M, K/128]  x  rhs 128 x 128 blocks [G, N/128, K/128] (DeepSeek-V3 checkpoints)
  * Alignment: K % 32 == 0 (INT4, MXFP4), K % 16 == 0 otherwise; N % 8 == 0; pointers 16-byte aligned.
  */
+#define MOE_SCALE_PER_TENSOR (-1)
+
 typedef struct {
   size_t struct_size; /* sizeof(moe_gmm_args), checked */
   const void* lhs;
@@ -203,7 +236,10 @@ typedef struct {
   int32_t rhs_scale_block_n, rhs_scale_block_k;
   int32_t act;     /* moe_act; must be MOE_ACT_NONE when rhs_up == NULL      */
   float act_limit; /* clip for SWIGLUOAI / SILU_CLIP                        */
-  int32_t reserved[4]; /* zero.  [0] and [1] select experimental kernel shapes (tuning aids of the benchmarks) */
+  int32_t out_dtype;       /* MOE_BF16 (= 0) or MOE_F32                                        */
+  int32_t lhs_row_idx_div; /* see lhs_row_idx; values < 1 are read as 1                        */
+  int32_t lhs_rows;        /* rows of lhs when lhs_row_idx is given (indices are clamped to it) */
+  int32_t reserved;        /* zero */
   /* per-expert bias [G_local, N] f32 added to lhs@rhs^T (and to lhs@rhs_up^T) before the activation:
    * w0_bias / w1_bias / wo_bias of mlp_bias models (moe.py:1952-1981, :2239-2241; rhs_bias of
    * pallas_mosaic_tpu_v2_gmm_kernel.py:573).  NULL = no bias.  Rows that are written as zeros stay zero. */
@@ -216,6 +252,15 @@ typedef struct {
   const void* partial_sum_up;
   int32_t flags; /* MOE_GMM_* bits */
   int32_t pad_;
+  /* [M] i32 or NULL: row i of the product reads lhs row lhs_row_idx[i] / lhs_row_idx_div, and that row's scales, instead
+   * of row i: the permute (moe.py:956-959: repeat(x, k)[perm]; kernels/ragged/ragged_gather.py:310-320) fused into the
+   * matmul, so that the [M, K] gathered copy is never written and T token rows are quantised instead of M = T * k copies.
+   * permute passes lhs_row_idx = perm, lhs_row_idx_div = k, lhs_rows = T. */
+  const int32_t* lhs_row_idx;
+  /* [M] f32 or NULL: row i of the result is multiplied by out_row_scale[i] after the activation and before the rounding
+   * to out_dtype: the routing weights applied between the activation and wo
+   * (models/deepseek_batchsplit_fp8.py:1049, intermediate_layer *= weights[:, None]). */
+  const float* out_row_scale;
 } moe_gmm_args;
 
 /* flags: rows that belong to no local group are left as `out` holds them instead of being written as zeros:
@@ -228,12 +273,32 @@ typedef struct {
  * rhs_up, on shapes moe_gmm_rhs_kn_supported() accepts (others return MOE_ERR_UNSUPPORTED: re-lay the weights out with
  * moe_transpose_rhs and call without the flag). */
 #define MOE_GMM_RHS_KN 2
+/* flags: layout of rhs_scale / rhs_up_scale, see "Operand layouts" above. */
+#define MOE_GMM_RHS_SCALE_KMAJOR 4
+#define MOE_GMM_RHS_SCALE_SHARED 8
 
 /* 1 when moe_gmm takes MOE_GMM_RHS_KN for this shape (K % 64 == 0, N % 256 == 0, 128 rows per group on average and
  * enough 256 x 256 tiles to fill the chip), else 0. */
 MOE_API int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total);
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
 MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);
+
+/* Per-device set-up, for the device that is current: the CU count and the raised LDS limit of every kernel.  Optional: each entry point does its share on first use.  No counterpart in the reference. */
+MOE_API int moe_init(void);
+
+/* moe_gmm with the kernel family and the tile raster chosen by the caller instead of by the shape: a tuning and test
+ * aid (no counterpart in the reference; the parity tests use it to run every kernel family on small shapes).
+ * kernel: MOE_GMM_KERNEL_*; a family that does not take the operands returns MOE_ERR_UNSUPPORTED.
+ * raster: > 0 = m-tiles per super-row of the tile order (persistent and fp8 LDS kernels); 0 = default. */
+typedef enum {
+  MOE_GMM_KERNEL_AUTO = 0,
+  MOE_GMM_KERNEL_STREAM = 1,    /* streaming kernels without LDS tiles (fp8 block-scaled, weight-only formats)        */
+  MOE_GMM_KERNEL_TILED = 2,     /* LDS-tiled kernels with the m-tile chosen by rows per expert (fp8: 128 x 128)       */
+  MOE_GMM_KERNEL_BIG = 3,       /* 256 x 256 tiles: fp8 block-scaled big kernel; int8 x int8 register-staged kernel   */
+  MOE_GMM_KERNEL_DL64 = 4,      /* direct-to-LDS persistent kernel with 64-byte stages (int8 x int8, bf16 x bf16)     */
+  MOE_GMM_KERNEL_STREAM_NOSPLIT = 5 /* weight-only streaming kernel with every wave walking all of K                   */
+} moe_gmm_kernel;
+MOE_API int moe_gmm_tuned(const moe_gmm_args* args, int kernel, int raster, void* stream);
 
 /* One-time weight re-layout [G, K, N] -> [G, N, K] (1-byte or 2-byte elements), for
  * callers that hold the reference's default rhs layout (ops.py:47, transpose_rhs=False). */

@@ -19,6 +19,12 @@ ROUTE_BY_NAME = {"softmax_topk": 0, "deepseek": 1, "topk_raw": 2, "softmax_all":
 MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
 MOE_GMM_KEEP_OTHER_ROWS = 1
 MOE_GMM_RHS_KN = 2
+MOE_GMM_RHS_SCALE_KMAJOR = 4
+MOE_GMM_RHS_SCALE_SHARED = 8
+MOE_SCALE_PER_TENSOR = -1
+GMM_KERNEL_BY_NAME = {None: 0, "auto": 0, "stream": 1, "tiled": 2, "big": 3, "dl64": 4, "stream_nosplit": 5}
+MOE_QUANT_RINT_DIV, MOE_QUANT_V2 = 0, 1
+QUANT_RULE_BY_NAME = {"rint_div": MOE_QUANT_RINT_DIV, "v2": MOE_QUANT_V2}
 
 ACT_BY_NAME = {None: MOE_ACT_NONE, "silu": MOE_ACT_SILU, "swigluoai": MOE_ACT_SWIGLUOAI, "silu_clip": MOE_ACT_SILU_CLIP}
 
@@ -53,13 +59,18 @@ class GmmArgs(ctypes.Structure):
       ("rhs_scale_block_k", ctypes.c_int32),
       ("act", ctypes.c_int32),
       ("act_limit", c_float),
-      ("reserved", ctypes.c_int32 * 4),
+      ("out_dtype", ctypes.c_int32),
+      ("lhs_row_idx_div", ctypes.c_int32),
+      ("lhs_rows", ctypes.c_int32),
+      ("reserved", ctypes.c_int32),
       ("rhs_bias", c_void_p),
       ("rhs_up_bias", c_void_p),
       ("partial_sum", c_void_p),
       ("partial_sum_up", c_void_p),
       ("flags", ctypes.c_int32),
       ("pad_", ctypes.c_int32),
+      ("lhs_row_idx", c_void_p),
+      ("out_row_scale", c_void_p),
   ]
 
 
@@ -72,10 +83,13 @@ SIGNATURES = {
                                c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_sort_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_sort_by_expert": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
-    "moe_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "moe_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                c_void_p]),
     "moe_gmm_workspace_bytes": (c_size_t, [c_int, c_int]),
     "moe_gmm_rhs_kn_supported": (c_int, [c_int, c_int, c_int, c_int]),
     "moe_gmm": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
+    "moe_gmm_tuned": (c_int, [ctypes.POINTER(GmmArgs), c_int, c_int, c_void_p]),
+    "moe_init": (c_int, []),
     "moe_tgmm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moe_calib_scratch_bytes": (c_size_t, []),
     "moe_calib_mfma_ops": (ctypes.c_double, [c_int, c_int]),

@@ -1,0 +1,344 @@
+// Shared pieces of the grouped-matmul kernels: the m-tile list, the parameter blocks, the epilogue, and the
+// launchers each translation unit exports to the dispatcher (moe_gmm.hip).
+#pragma once
+
+#include <type_traits>
+
+#include "moe_common.h"
+
+namespace moe {
+
+struct TileInfo {
+  int32_t group;  // local group id, or -1: write zeros
+  int32_t row0;
+  int32_t nrows;
+  int32_t pad;
+};
+
+// workspace: int32 header[4] (header[0] = number of tiles) | TileInfo tiles[max_tiles]
+static inline int max_tiles_for(int M, int G, int bm) { return cdiv(M, bm) + G + 1; }
+
+enum { OP_BF16 = 0, OP_I8 = 1, OP_F8 = 2 };      // MFMA operand type (= LDS element type)
+enum { BSRC_SAME = 0, BSRC_I8 = 1, BSRC_I4 = 2, BSRC_MX4 = 3 };  // weight format in HBM
+
+// Options every kernel family honours: activation rows read through an index (the permute of moe.py:956-959 fused into
+// the matmul: row r of the product reads lhs row row_idx[r] / idx_div, and that row's scales), a factor per output row
+// applied after the activation (routing weights before wo, models/deepseek_batchsplit_fp8.py:1049), f32 output.
+struct RowOpts {
+  const int32_t* row_idx;  // [M] or NULL
+  int idx_div;
+  int lhs_rows;            // rows of lhs; indices are clamped into [0, lhs_rows)
+  int out_f32;             // out is [M, N] f32 instead of bf16
+  const float* row_scale;  // [M] or NULL
+};
+
+__device__ __forceinline__ int lhs_row_of(const RowOpts& o, int r) {
+  if (!o.row_idx) return r;
+  const int s = o.row_idx[r] / o.idx_div;
+  return min(max(s, 0), o.lhs_rows - 1);
+}
+
+// Four consecutive output values of one row: multiplied by the row's factor, then stored as bf16 (8 bytes) or f32.
+__device__ __forceinline__ void store_out4(void* out, const RowOpts& o, size_t row, int N, int n, float (&v)[4]) {
+  if (o.row_scale) {
+    const float w = o.row_scale[row];
+#pragma unroll
+    for (int r = 0; r < 4; r++) v[r] *= w;
+  }
+  if (o.out_f32)
+    *(float4*)((float*)out + row * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+  else
+    *(uint2*)((uint16_t*)out + row * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+}
+
+// Zeros for the `width` channels from n0 on of a tile's rows (rows of no local group).
+__device__ __forceinline__ void zero_fill_tile(void* out, const RowOpts& o, int row0, int nrows, int n0, int width, int N, int tid,
+                                               int nthreads) {
+  const int qpr = width / 4;
+  for (int i = tid; i < nrows * qpr; i += nthreads) {
+    const int r = i / qpr, c = n0 + (i % qpr) * 4;
+    if (c >= N) continue;
+    if (o.out_f32)
+      *(float4*)((float*)out + (size_t)(row0 + r) * N + c) = make_float4(0.f, 0.f, 0.f, 0.f);
+    else
+      *(uint2*)((uint16_t*)out + (size_t)(row0 + r) * N + c) = make_uint2(0, 0);
+  }
+}
+
+struct TiledParams {
+  const uint8_t* lhs;        // [M, K] elements of the MFMA operand type
+  const float* lhs_scale;    // epilogue scale of the activations: [M] (stride 1) or one value (stride 0), or NULL
+  const uint8_t* rhs;        // [G, N, K] (INT4: K/2 bytes per row)
+  const uint8_t* rhs_up;     // same, or NULL
+  const void* rhs_scale;     // f32 [G, N] (per channel) | bf16 [G, N, nkg] (INT4) | e8m0 bytes [G, N, K/32] (MXFP4)
+  const void* rhs_up_scale;  //   (f32 per channel: element (g, n) at g * rhs_scale_gstride + n * rhs_scale_nstride)
+  const float* rhs_bias;     // [G, N] f32 or NULL, added before the activation
+  const float* rhs_up_bias;
+  const uint16_t* partial_sum;     // [M, N] bf16 or NULL, added like the bias
+  const uint16_t* partial_sum_up;
+  const int32_t* header;
+  const TileInfo* tiles;
+  void* out;  // [M, N] bf16 (f32 with ro.out_f32)
+  int M, K, N;
+  int max_m_tiles, tiles_n;
+  int act;
+  float act_limit;
+  int tune;  // > 0: m-tiles per raster super-row of the persistent kernel (tuning aid; 0 = default)
+  int i4_group;  // values of K per int4 scale: 128 or 32
+  int lhs_scale_stride;   // 1: one epilogue scale per row; 0: one for the tensor (static per-tensor scale)
+  int rhs_scale_gstride;  // N: scales per expert; 0: one set shared by all experts ([1, 1, n], ops.py:250-260)
+  int rhs_scale_nstride;  // 1: per output channel; 0: one per expert / tensor
+  // K-block scales applied to the partial sums (block-scaled kernel; gmm_v2's layout): lhs_bs [M, lhs_nb] with one value
+  // per lhs_qb values of K, rhs_bs [G, rhs_nb, N] (element (g, b, n) at g * rhs_bs_gstride + b * N + n) per rhs_qb values.
+  // A side whose count is 1 has its scale in the epilogue fields above instead and a NULL pointer here.
+  const float* lhs_bs;
+  const float* rhs_bs;
+  const float* rhs_up_bs;
+  int lhs_nb, lhs_qb, rhs_nb, rhs_qb, rhs_bs_gstride;
+  // weight-only int8 / int4 with K-major block scales [G, nb, N] (f32), multiplied in while the weights are widened
+  int wq_kmajor;
+  RowOpts ro;
+};
+
+__device__ __forceinline__ uint32_t i8x2_to_bf16x2(int lo, int hi) {
+  // |value| <= 128 is exact in bf16, so truncating the f32 is the conversion
+  return (__float_as_uint((float)lo) >> 16) | (__float_as_uint((float)hi) & 0xffff0000u);
+}
+
+// Bias of 4 consecutive output channels of one group (zeros without a bias).
+__device__ __forceinline__ void load_bias4(const float* bias, int group, int N, int n, float (&b)[4]) {
+  b[0] = b[1] = b[2] = b[3] = 0.f;
+  if (bias) {
+    const float4 v = *(const float4*)(bias + (size_t)group * N + n);
+    b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
+  }
+}
+
+// b += 4 consecutive bf16 values of row `row` of a [M, N] partial-sum matrix (nothing without one).
+__device__ __forceinline__ void add_partial4(const uint16_t* ps, size_t row, int N, int n, float (&b)[4]) {
+  if (ps) {
+    const uint2 v = *(const uint2*)(ps + row * N + n);
+    b[0] += bf16_bits_to_f32((uint16_t)(v.x & 0xffff));
+    b[1] += bf16_bits_to_f32((uint16_t)(v.x >> 16));
+    b[2] += bf16_bits_to_f32((uint16_t)(v.y & 0xffff));
+    b[3] += bf16_bits_to_f32((uint16_t)(v.y >> 16));
+  }
+}
+
+// Per-lane scales of the epilogue, fetched before the K loop so their latency hides behind it.  With
+// weights as the MFMA "A" operand a lane owns row (lane % 32) of each 32-row tile and, per accumulator
+// quad q, the 4 consecutive output channels 8*q + 4*(lane / 32) .. +3 of each 32-channel tile.  With the
+// 16 x 16 instructions (MI = 16) it owns row (lane % 16) of each 16-row tile and the one quad of channels
+// 4*(lane / 16) .. +3 of each 16-channel tile (only entry [.][0] of sg / su is used).
+template <int MI>
+__device__ __forceinline__ int epilogue_channel(int j, int q, int lane) {
+  return MI == 32 ? j * 32 + 8 * q + 4 * (lane / 32) : j * 16 + 4 * (lane / 16);
+}
+
+template <int TM, int NT_OUT, bool GLU>
+struct EpilogueScales {
+  float sa[TM];
+  float4 sg[NT_OUT][4], su[NT_OUT][4];
+};
+
+template <int TM, int NT_OUT, bool GLU, bool CHANNEL_SCALES, int MI = 32>
+__device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, GLU>& e, const TiledParams& p, const TileInfo& tile,
+                                                     int row_base, int n_base, int lane) {
+  const float4 one = make_float4(1.f, 1.f, 1.f, 1.f);
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int lr = row_base + i * MI + (lane % MI);
+    e.sa[i] = p.lhs_scale ? p.lhs_scale[(size_t)lhs_row_of(p.ro, tile.row0 + (lr < tile.nrows ? lr : 0)) * p.lhs_scale_stride] : 1.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+    for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+      const int n = n_base + epilogue_channel<MI>(j, q, lane);
+      e.sg[j][q] = one;
+      e.su[j][q] = one;
+      if (CHANNEL_SCALES && p.rhs_scale && !p.wq_kmajor && n < p.N) {  // (K-major block scales went in with the weights)
+        const float* sg = (const float*)p.rhs_scale + (size_t)tile.group * p.rhs_scale_gstride;
+        const float* su = GLU ? (const float*)p.rhs_up_scale + (size_t)tile.group * p.rhs_scale_gstride : nullptr;
+        if (p.rhs_scale_nstride) {
+          e.sg[j][q] = *(const float4*)(sg + n);
+          if (GLU) e.su[j][q] = *(const float4*)(su + n);
+        } else {
+          e.sg[j][q] = make_float4(sg[0], sg[0], sg[0], sg[0]);
+          if (GLU) e.su[j][q] = make_float4(su[0], su[0], su[0], su[0]);
+        }
+      }
+    }
+}
+
+template <int TM, int TN, int NT_OUT, bool GLU, typename acc_t>
+__device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
+                                               const TiledParams& p, const TileInfo& tile, int row_base, int n_base, int lane) {
+  constexpr int MI = sizeof(acc_t) == 16 ? 16 : 32;  // 4 accumulator registers per tile: the 16 x 16 instructions
+  dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
+  constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int lr = row_base + i * MI + (lane % MI);
+    if (lr >= tile.nrows) continue;
+#pragma unroll
+    for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+      for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+        const int n = n_base + epilogue_channel<MI>(j, q, lane);
+        if (n >= p.N) continue;
+        const float sg[4] = {e.sg[j][q].x, e.sg[j][q].y, e.sg[j][q].z, e.sg[j][q].w};
+        const float su[4] = {e.su[j][q].x, e.su[j][q].y, e.su[j][q].z, e.su[j][q].w};
+        float bg[4], bu[4];
+        load_bias4(p.rhs_bias, tile.group, p.N, n, bg);
+        load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, p.N, n, bu);
+        add_partial4(p.partial_sum, (size_t)(tile.row0 + lr), p.N, n, bg);
+        add_partial4(GLU ? p.partial_sum_up : nullptr, (size_t)(tile.row0 + lr), p.N, n, bu);
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float g = fmaf((float)acc[j][i][4 * q + r], e.sa[i] * sg[r], bg[r]);
+          if (GLU) {
+            const float u = fmaf((float)acc[j + NT_OUT][i][4 * q + r], e.sa[i] * su[r], bu[r]);
+            v[r] = glu_act<ACT>(g, u, p.act_limit);
+          } else {
+            v[r] = g;
+          }
+        }
+        store_out4(p.out, p.ro, (size_t)(tile.row0 + lr), p.N, n, v);
+      }
+  }
+  });
+}
+
+// ---- whole-line weight requests of the streaming kernels ----
+
+// Weight fragment of one 128-byte k-block for 16 channels.  Each of the two requests covers whole 128-byte
+// lines (8 channels x 128 B: lane (i, kq) asks for bytes (i/8)*64 + kq*16.. of channel i%8, then of channel
+// i%8 + 8) and is non-temporal: weights are read once, and a streamed read that owns its lines runs about
+// 12 % faster than one that leaves half of each line to the next request (STREAM = false keeps the lines
+// cached, for tiles that share weights).  A rotation by 8 inside each row of 16 lanes then hands every lane
+// the two 16-byte pieces of its own channel i.
+template <bool STREAM>
+__device__ __forceinline__ v4i load_w16(const uint8_t* p) {
+  return STREAM ? __builtin_nontemporal_load((const v4i*)p) : *(const v4i*)p;
+}
+
+// a = request for channels i%8, b = request for channels i%8 + 8, each lane holding piece i/8 (the first or second
+// 64 bytes of the 128-byte unit).  Returns in `first` / `second` the two pieces of the lane's own channel i.
+__device__ __forceinline__ void own_channel_pieces(const v4i& a, const v4i& b, v4i& first, v4i& second) {
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    // lanes 8..15 of a row: the first piece of their channel sits in `b` of lane i-8; lanes 0..7 keep their `a`
+    first[c] = __builtin_amdgcn_update_dpp(a[c], b[c], 0x128, 0xf, 0xc, false);
+    // lanes 0..7: the second piece of their channel sits in `a` of lane i+8; lanes 8..15 keep their `b`
+    second[c] = __builtin_amdgcn_update_dpp(b[c], a[c], 0x128, 0xf, 0x3, false);
+  }
+}
+
+struct SkinnyParams {
+  const uint8_t* lhs;      // [M, K] fp8
+  const float* lhs_scale;  // [M, K/128]
+  const uint8_t* rhs;      // [G, N, K] fp8
+  const uint8_t* rhs_up;
+  const float* rhs_scale;  // [G, ceil(N/128), K/128]
+  const float* rhs_up_scale;
+  const float* rhs_bias;   // [G, N] f32 or NULL
+  const float* rhs_up_bias;
+  const uint16_t* partial_sum;     // [M, N] bf16 or NULL, added like the bias
+  const uint16_t* partial_sum_up;
+  const int32_t* header;
+  const TileInfo* tiles;
+  void* out;
+  int M, K, N;
+  int n_blocks;  // blocks along N
+  int min_rows, max_rows;  // only tiles with min_rows <= nrows <= max_rows are computed by this launch
+  int act;
+  float act_limit;
+  // per-row x per-channel scales (ops.py:241-260: lhs [m, 1], rhs [1, 1, n]) instead of blocks: the block scales above
+  // are NULL (taken as 1) and these are applied once to the finished sums
+  const float* row_scale_lhs;  // [M] (stride 1) or one value (stride 0), or NULL
+  const float* ch_scale;       // f32, element (g, n) at g * ch_gstride + n * ch_nstride, or NULL
+  const float* ch_scale_up;
+  int row_scale_lhs_stride, ch_gstride, ch_nstride;
+  RowOpts ro;
+};
+
+struct Fp8TiledParams {
+  TiledParams base;        // lhs / rhs / rhs_up fp8; its epilogue scales are NULL for block-scaled operands
+  const float* a_scale;    // [M, K/128], or NULL: no block scales (per-row x per-channel scales sit in `base`)
+  const float* w_scale;    // [G, ceil(N/128), K/128]
+  const float* u_scale;
+};
+
+struct WqSkinnyParams {
+  const uint8_t* lhs;       // [M, K] bf16
+  const uint8_t* rhs;       // [G, N, K] int8 or [G, N, K/2] packed int4
+  const uint8_t* rhs_up;
+  const void* rhs_scale;    // int8: f32 [G, N]; int4: bf16 [G, N, ceil(K/128)]
+  const void* rhs_up_scale;
+  const float* rhs_bias;    // [G, N] f32 or NULL
+  const float* rhs_up_bias;
+  const uint16_t* partial_sum;     // [M, N] bf16 or NULL, added like the bias
+  const uint16_t* partial_sum_up;
+  const int32_t* header;
+  const TileInfo* tiles;
+  void* out;
+  int M, K, N;
+  int n_blocks;
+  int act;
+  float act_limit;
+  int ch_gstride, ch_nstride;  // int8 per-channel scales: element (g, n) at g * ch_gstride + n * ch_nstride
+  RowOpts ro;
+};
+
+// ---------------------------------------------------------------------------------------
+// Host side shared by the launchers
+// ---------------------------------------------------------------------------------------
+
+// Per-device launch state: the attribute that lets a kernel use more than 64 KB of dynamic LDS belongs to a
+// device's code object, and the CU count to the device, so both are kept per device ordinal.  A race between two
+// host threads only repeats an idempotent call.
+constexpr int kMaxDevices = 64;
+
+int current_device(int* dev);
+int device_cu_count(int* cus);
+
+template <typename K>
+static int reserve_lds(K kernel, int bytes, bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  if (int st = current_device(&dev)) return st;
+  if (done[dev]) return MOE_OK;
+  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "gmm: cannot reserve %d bytes of LDS: %s", bytes, hipGetErrorString(e));
+  done[dev] = true;
+  return MOE_OK;
+}
+
+// One "LDS limit raised" flag per device for each kernel instantiation.
+template <typename Tag>
+static bool (&lds_flags())[kMaxDevices] {
+  static bool flags[kMaxDevices] = {};
+  return flags;
+}
+
+// Raise the LDS limit of every instantiation of a family on the current device (moe_init: callers that must not
+// touch function attributes later, e.g. while a stream is being captured, do it up front).
+int prepare_tiled();
+int prepare_dl();
+int prepare_fp8();
+
+// ---- launchers (one translation unit per kernel family) ----
+// moe_gmm_tiled.hip: register-staged kernel, m-tile bm in {64, 128, 256}; block_scaled: int8 x int8 / fp8 x fp8 with K-block
+// scales applied to the partial sums (bm 64 or 128)
+int launch_tiled_bm(int op, int bsrc, bool glu, int bm, bool block_scaled, const TiledParams& p, int M, int G_total, hipStream_t s);
+// moe_gmm_dl.hip: direct-to-LDS persistent kernel, 256 x 256 tiles; stage_bytes 128 or 64; rhs_kn: [G, K, N] bf16 weights
+int launch_dl(int op, bool glu, int stage_bytes, bool rhs_kn, const TiledParams& p, int M, int G_total, hipStream_t s);
+// moe_gmm_fp8.hip
+int launch_fp8_tiled(bool big, bool glu, bool vec4, const Fp8TiledParams& P, int M, int G_total, hipStream_t s);
+int launch_fp8_skinny(bool few_rows, const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s);
+// moe_gmm_wq.hip: fmt is one of WQ_*; one_tile: 16-row tiles (else 32)
+enum { WQ_I8 = 0, WQ_I4 = 1, WQ_MX4 = 2, WQ_I4G32 = 3 };  // weight formats of the streaming kernel (int4: group 128 / 32)
+int launch_wq(int fmt, bool one_tile, const WqSkinnyParams& q, bool glu, int max_tiles, int tune, hipStream_t s);
+
+}  // namespace moe

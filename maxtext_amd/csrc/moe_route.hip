@@ -502,7 +502,7 @@ __global__ void invert_perm_kernel(const int32_t* __restrict__ perm, int M,
 constexpr int kGqThreads = 256;
 constexpr int kGqMaxChunks = 8;  // 16-byte chunks per thread -> d <= 256*8*8
 
-enum { GQ_COPY = 0, GQ_INT8_ROW = 1, GQ_FP8_BLK128 = 2 };
+enum { GQ_COPY = 0, GQ_INT8 = 1, GQ_FP8 = 2 };
 
 __device__ __forceinline__ void unpack8(const uint4& u, float f[8]) {
   f[0] = bf16_bits_to_f32(u.x & 0xffffu);
@@ -524,20 +524,77 @@ __device__ __forceinline__ float absmax8(const uint4& u) {
   return m;
 }
 
+// Quantisation rules (moe_quant_rule).  RINT_DIV: scale = absmax / qmax, q = rint(x / scale) clipped, all in f32 (the
+// rule adopted for the v1 path's third-party quantiser).  V2: the in-kernel quantiser of the reference's gmm_v2
+// (pallas_mosaic_tpu_v2_gmm_kernel.py:528-542), whose every operation is carried out in the activation dtype, bf16:
+// scale = bf16(absmax / qmax), inv = scale == 0 ? 0 : bf16(1 / scale), y = bf16(x * inv), then the cast of
+// `.astype`: truncation toward zero for int8, round-to-nearest-even for fp8.  A bf16 op is an f32 op (correctly
+// rounded, the default of hipcc for division) followed by a rounding to bf16, as XLA computes it.
+struct QuantCfg {
+  int rule;                   // moe_quant_rule
+  int block_lanes;            // lanes that share a scale: 16 / 32 / 64 (K blocks of 128 / 256 / 512), 0 = the whole row
+  int nkb;                    // scales per row
+  const float* static_scale;  // [1] or NULL
+  const float* row_weight;    // [R_out] or NULL: the gathered row is multiplied by its weight (rounded to bf16) first
+  const int32_t* row_range;   // [2] (start, end) on the device or NULL: output rows outside [start, end) are zeros
+};
+
+template <int MODE>
+__device__ __forceinline__ void quant_scale(float m, int rule, float& sc, float& inv) {
+  const float qmax = MODE == GQ_INT8 ? 127.0f : 448.0f;
+  if (rule == MOE_QUANT_V2) {
+    sc = round_bf16_fn(m / qmax);
+    inv = sc == 0.f ? 0.f : round_bf16_fn(1.0f / sc);
+  } else {
+    sc = m / qmax;
+    inv = 0.f;  // unused: this rule divides
+  }
+}
+
+template <int MODE>
+__device__ __forceinline__ float quant_value(float f, float sc, float inv, int rule, bool is_static) {
+  const float qmax = MODE == GQ_INT8 ? 127.0f : 448.0f;
+  if (rule == MOE_QUANT_V2) {
+    float y = round_bf16_fn(f * inv);
+    // dynamic scales keep |y| <= 127.5 (450 for fp8), which the cast itself brings to qmax; the static branch
+    // clips before the cast (:531)
+    y = fminf(fmaxf(y, -qmax), qmax);
+    (void)is_static;
+    return MODE == GQ_INT8 ? truncf(y) : y;
+  }
+  float q = sc == 0.f ? 0.f : f / sc;
+  if (MODE == GQ_INT8) q = rintf(q);
+  return fminf(fmaxf(q, -qmax), qmax);
+}
+
 template <int MODE>
 __global__ __launch_bounds__(kGqThreads) void gather_rows_kernel(
-    const uint4* __restrict__ x, const int32_t* __restrict__ row_idx, int idx_div, int d,
-    void* __restrict__ out, float* __restrict__ scale) {
+    const uint4* __restrict__ x, const int32_t* __restrict__ row_idx, int idx_div, int R_in, int d,
+    void* __restrict__ out, float* __restrict__ scale, const QuantCfg qc) {
   __shared__ float s_red[kGqThreads / kWave];
   const int r = blockIdx.x;
   const int src = row_idx ? row_idx[r] / idx_div : r;
   const int nch = d / 8;
-  const uint4* xrow = x + (size_t)src * nch;
+  // an index outside the input (a malformed row_idx) reads nothing and yields a row of zeros, and so does an output
+  // row outside the requested range (ragged_gather's [start, end), kernels/ragged/ragged_gather.py:357-376)
+  bool in_range = src >= 0 && src < R_in;
+  if (qc.row_range) in_range = in_range && r >= qc.row_range[0] && r < qc.row_range[1];
+  const uint4* xrow = x + (size_t)(in_range ? src : 0) * nch;
   uint4 regs[kGqMaxChunks];
 #pragma unroll
   for (int c = 0; c < kGqMaxChunks; c++) {
     int ci = threadIdx.x + c * kGqThreads;
-    regs[c] = ci < nch ? xrow[ci] : make_uint4(0, 0, 0, 0);
+    regs[c] = ci < nch && in_range ? xrow[ci] : make_uint4(0, 0, 0, 0);
+  }
+  if (qc.row_weight) {  // x[indices] * weights[:, None] (ragged_gather.py:316-319), product rounded to bf16
+    const float w = qc.row_weight[r];
+#pragma unroll
+    for (int c = 0; c < kGqMaxChunks; c++) {
+      float f[8];
+      unpack8(regs[c], f);
+      regs[c] = make_uint4(pack_bf16x2(f[0] * w, f[1] * w), pack_bf16x2(f[2] * w, f[3] * w), pack_bf16x2(f[4] * w, f[5] * w),
+                           pack_bf16x2(f[6] * w, f[7] * w));
+    }
   }
 
   if (MODE == GQ_COPY) {
@@ -550,7 +607,14 @@ __global__ __launch_bounds__(kGqThreads) void gather_rows_kernel(
     return;
   }
 
-  if (MODE == GQ_INT8_ROW) {
+  const bool is_static = qc.static_scale != nullptr;
+  float row_sc = 0.f, row_inv = 0.f;
+  if (is_static) {
+    // one scale for the whole tensor: bf16(scale) and its bf16 inverse for the v2 rule (:528-529), the value itself otherwise
+    const float s = *qc.static_scale;
+    row_sc = qc.rule == MOE_QUANT_V2 ? round_bf16_fn(s) : s;
+    row_inv = qc.rule == MOE_QUANT_V2 ? round_bf16_fn(1.0f / row_sc) : 0.f;
+  } else if (qc.block_lanes == 0) {
     float m = 0.f;
 #pragma unroll
     for (int c = 0; c < kGqMaxChunks; c++) m = fmaxf(m, absmax8(regs[c]));
@@ -558,51 +622,32 @@ __global__ __launch_bounds__(kGqThreads) void gather_rows_kernel(
     if (threadIdx.x % kWave == 0) s_red[threadIdx.x / kWave] = m;
     __syncthreads();
     m = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    const float sc = m / 127.0f;
-    if (threadIdx.x == 0) scale[r] = sc;
-    uint2* orow = (uint2*)out + (size_t)r * nch;
+    quant_scale<MODE>(m, qc.rule, row_sc, row_inv);
+    if (threadIdx.x == 0) scale[r] = row_sc;
+  }
+  uint2* orow = (uint2*)out + (size_t)r * nch;
 #pragma unroll
-    for (int c = 0; c < kGqMaxChunks; c++) {
-      int ci = threadIdx.x + c * kGqThreads;
-      if (ci < nch) {
-        float f[8];
-        unpack8(regs[c], f);
+  for (int c = 0; c < kGqMaxChunks; c++) {
+    int ci = threadIdx.x + c * kGqThreads;
+    float sc = row_sc, inv = row_inv;
+    if (!is_static && qc.block_lanes != 0) {
+      // a K block is block_lanes consecutive 16-byte chunks == consecutive lanes of one wave
+      float m = absmax8(regs[c]);
+      for (int o = qc.block_lanes / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      quant_scale<MODE>(m, qc.rule, sc, inv);
+      if (ci < nch && (threadIdx.x & (qc.block_lanes - 1)) == 0) scale[(size_t)r * qc.nkb + ci / qc.block_lanes] = sc;
+    }
+    if (ci < nch) {
+      float f[8];
+      unpack8(regs[c], f);
+#pragma unroll
+      for (int i = 0; i < 8; i++) f[i] = quant_value<MODE>(f[i], sc, inv, qc.rule, is_static);
+      if (MODE == GQ_INT8) {
         uint32_t b[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-          float q = sc == 0.f ? 0.f : rintf(f[i] / sc);
-          q = fminf(fmaxf(q, -127.f), 127.f);
-          b[i] = (uint32_t)((int)q) & 0xffu;
-        }
-        uint2 o;
-        o.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
-        o.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
-        orow[ci] = o;
-      }
-    }
-    return;
-  }
-
-  if (MODE == GQ_FP8_BLK128) {
-    // a 128-element block is 16 consecutive chunks == 16 consecutive lanes
-    const int nkb = (d + 127) / 128;
-    uint2* orow = (uint2*)out + (size_t)r * nch;
-#pragma unroll
-    for (int c = 0; c < kGqMaxChunks; c++) {
-      int ci = threadIdx.x + c * kGqThreads;
-      float m = absmax8(regs[c]);
-#pragma unroll
-      for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-      const float sc = m / 448.0f;
-      if (ci < nch) {
-        if ((threadIdx.x & 15) == 0) scale[(size_t)r * nkb + ci / 16] = sc;
-        float f[8];
-        unpack8(regs[c], f);
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-          float q = sc == 0.f ? 0.f : f[i] / sc;
-          f[i] = fminf(fmaxf(q, -448.f), 448.f);
-        }
+        for (int i = 0; i < 8; i++) b[i] = (uint32_t)((int)f[i]) & 0xffu;
+        orow[ci] = make_uint2(b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24), b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24));
+      } else {
         int lo = 0, hi = 0;
         lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
         lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
@@ -628,7 +673,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ 
   __shared__ float s_w[kCombineMaxK];
   const int t = blockIdx.x;
   if (threadIdx.x < k) {
-    s_row[threadIdx.x] = inv_perm[(size_t)t * k + threadIdx.x];
+    // an index outside [0, M) (a malformed inv_perm) contributes nothing instead of reading out of bounds
+    const int row = inv_perm[(size_t)t * k + threadIdx.x];
+    const bool ok = row >= 0 && row < (int)gridDim.x * k;
+    s_row[threadIdx.x] = ok ? row : -1;
     s_w[threadIdx.x] = weights ? weights[(size_t)t * k + threadIdx.x] : 1.0f;
   }
   __syncthreads();
@@ -636,6 +684,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ 
   for (int ci = threadIdx.x; ci < nch; ci += blockDim.x) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < k; s++) {
+      if (s_row[s] < 0) continue;
       uint4 u = y[(size_t)s_row[s] * nch + ci];
       float f[8];
       unpack8(u, f);
@@ -663,7 +712,8 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const uint4* __restric
   __shared__ float s_part[kCombineMaxK][4];
   const int t = blockIdx.x;
   if (threadIdx.x < k) {
-    s_row[threadIdx.x] = inv_perm[(size_t)t * k + threadIdx.x];
+    const int row = inv_perm[(size_t)t * k + threadIdx.x];
+    s_row[threadIdx.x] = row >= 0 && row < (int)gridDim.x * k ? row : -1;  // malformed index: no row is written
     s_w[threadIdx.x] = weights ? weights[(size_t)t * k + threadIdx.x] : 1.0f;
   }
   __syncthreads();
@@ -677,6 +727,7 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const uint4* __restric
 #pragma unroll
     for (int s = 0; s < kCombineMaxK; s++) {
       if (s >= k) break;
+      if (s_row[s] < 0) continue;
       const size_t at = (size_t)s_row[s] * nch + ci;
       const float w = s_w[s];
       uint4 o;
@@ -818,7 +869,7 @@ using namespace moe;
 extern "C" {
 
 const char* moe_last_error(void) { return g_err; }
-int moe_abi_version(void) { return 1; }
+int moe_abi_version(void) { return 2; }
 
 int moe_route_topk(const float* gate_logits, const float* pre_bias_logits, int T, int E, int k,
                    int mode, int norm_topk_prob, int weights_round_bf16,
@@ -930,25 +981,37 @@ int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* pe
   return check_launch("sort_by_expert");
 }
 
-int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_out, int d,
-                    int out_dtype, int block_k, void* out, float* scale, void* stream) {
+int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_in, int R_out, int d,
+                    int out_dtype, int block_k, int rule, const float* static_scale, const float* row_weight,
+                    const int32_t* row_range, void* out, float* scale, void* stream) {
   if (!x || !out) return fail(MOE_ERR_INVALID_ARG, "gather: NULL pointer");
-  if (R_out < 0 || d <= 0 || idx_div <= 0) return fail(MOE_ERR_INVALID_ARG, "gather: bad sizes");
+  if (R_in <= 0 || R_out < 0 || d <= 0 || idx_div <= 0 || block_k < 0) return fail(MOE_ERR_INVALID_ARG, "gather: bad sizes");
+  if (!row_idx && R_out > R_in) return fail(MOE_ERR_INVALID_ARG, "gather: R_out > R_in without row_idx");
   if (d % 8 != 0 || d > kGqThreads * kGqMaxChunks * 8) return fail(MOE_ERR_UNSUPPORTED, "gather: need d%%8==0 and d<=16384 (d=%d)", d);
+  if (rule != MOE_QUANT_RINT_DIV && rule != MOE_QUANT_V2) return fail(MOE_ERR_INVALID_ARG, "gather: bad rule %d", rule);
   if (R_out == 0) return MOE_OK;
   hipStream_t s = (hipStream_t)stream;
   const uint4* xs = (const uint4*)x;
+  QuantCfg qc;
+  qc.rule = rule; qc.block_lanes = 0; qc.nkb = 1; qc.static_scale = nullptr; qc.row_weight = row_weight; qc.row_range = row_range;
   if (out_dtype == MOE_BF16) {
-    gather_rows_kernel<GQ_COPY><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, d, out, scale);
-  } else if (out_dtype == MOE_INT8) {
-    if (!scale || block_k != 0) return fail(MOE_ERR_UNSUPPORTED, "gather: int8 needs per-row scale (block_k=0)");
-    gather_rows_kernel<GQ_INT8_ROW><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, d, out, scale);
-  } else if (out_dtype == MOE_FP8_E4M3) {
-    if (!scale || block_k != 128) return fail(MOE_ERR_UNSUPPORTED, "gather: fp8 needs block_k=128 scales");
-    gather_rows_kernel<GQ_FP8_BLK128><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, d, out, scale);
-  } else {
-    return fail(MOE_ERR_UNSUPPORTED, "gather: out_dtype %d", out_dtype);
+    gather_rows_kernel<GQ_COPY><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, R_in, d, out, scale, qc);
+    return check_launch("gather_rows_kernel");
   }
+  if (out_dtype != MOE_INT8 && out_dtype != MOE_FP8_E4M3) return fail(MOE_ERR_UNSUPPORTED, "gather: out_dtype %d", out_dtype);
+  if (static_scale) {
+    qc.static_scale = static_scale;  // one scale for the tensor: block_k is not used and `scale` is not written
+  } else {
+    if (!scale) return fail(MOE_ERR_INVALID_ARG, "gather: quantised output needs a scale buffer");
+    if (block_k != 0 && block_k != 128 && block_k != 256 && block_k != 512)
+      return fail(MOE_ERR_UNSUPPORTED, "gather: block_k must be 0 (one scale per row), 128, 256 or 512 (block_k=%d)", block_k);
+    qc.block_lanes = block_k / 8;
+    qc.nkb = block_k ? cdiv(d, block_k) : 1;
+  }
+  if (out_dtype == MOE_INT8)
+    gather_rows_kernel<GQ_INT8><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, R_in, d, out, scale, qc);
+  else
+    gather_rows_kernel<GQ_FP8><<<R_out, kGqThreads, 0, s>>>(xs, row_idx, idx_div, R_in, d, out, scale, qc);
   return check_launch("gather_rows_kernel");
 }
 

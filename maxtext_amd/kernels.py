@@ -106,26 +106,49 @@ def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True):
   return perm, inv, gs, se
 
 
-def gather_rows(x, row_idx=None, idx_div=1, *, out_dtype=torch.bfloat16, block_k=0, num_rows=None):
-  """Row gather (+ per-row int8 / 1x128 fp8 quantisation).  -> out or (q, scale)."""
+def gather_rows(x, row_idx=None, idx_div=1, *, out_dtype=torch.bfloat16, block_k=0, num_rows=None, rule="rint_div", static_scale=None,
+                row_weight=None, row_range=None):
+  """Row gather (+ int8 / fp8 quantisation, one scale per row or per `block_k` values of a row, or one static scale).
+  rule: "rint_div" (v1 path) or "v2" (the in-kernel quantiser of gmm_v2).  row_weight [R_out] f32 multiplies each
+  gathered row; row_range int32 [2] (start, end) on the device zeroes the output rows outside it.  -> out or (q, scale)."""
   _need(x, "x", torch.bfloat16, 2)
-  d = x.shape[1]
+  r_in, d = x.shape
   if row_idx is not None:
     _need(row_idx, "row_idx", torch.int32, 1)
     r_out = row_idx.shape[0]
   else:
-    r_out = x.shape[0] if num_rows is None else num_rows
+    r_out = r_in if num_rows is None else num_rows
+  if rule not in _lib.QUANT_RULE_BY_NAME:
+    raise ValueError(f"unknown quantisation rule {rule!r}")
+  quantised = out_dtype in (torch.int8, torch.float8_e4m3fn)
+  if not quantised and out_dtype != torch.bfloat16:
+    raise TypeError(f"out_dtype {out_dtype} not supported")
+  if quantised and static_scale is None and block_k not in (0, 128, 256, 512):
+    raise ValueError(f"block_k must be 0 (one scale per row), 128, 256 or 512, got {block_k}")
   out = torch.empty((r_out, d), dtype=out_dtype, device=x.device)
   scale = None
-  if out_dtype == torch.int8:
-    scale = torch.empty((r_out,), dtype=torch.float32, device=x.device)
-  elif out_dtype == torch.float8_e4m3fn:
-    scale = torch.empty((r_out, (d + block_k - 1) // block_k), dtype=torch.float32, device=x.device)
+  if quantised and static_scale is not None:
+    _need(static_scale, "static_scale", torch.float32)
+    if static_scale.numel() != 1:
+      raise ValueError("static_scale must hold one value")
+  elif quantised:
+    scale = torch.empty((r_out,) if block_k == 0 else (r_out, (d + block_k - 1) // block_k), dtype=torch.float32, device=x.device)
+  if row_weight is not None:
+    _need(row_weight, "row_weight", torch.float32, 1)
+    if row_weight.numel() != r_out:
+      raise ValueError("row_weight must have one value per output row")
+  if row_range is not None:
+    _need(row_range, "row_range", torch.int32, 1)
+    if row_range.numel() != 2:
+      raise ValueError("row_range must hold (start, end)")
   lib = _lib.load()
-  st = lib.moe_gather_rows(_lib.ptr(x), _lib.ptr(row_idx), int(idx_div), r_out, d, _DTYPE_CODE[out_dtype], int(block_k),
-                           _lib.ptr(out), _lib.ptr(scale), _lib.current_stream())
+  st = lib.moe_gather_rows(_lib.ptr(x), _lib.ptr(row_idx), int(idx_div), r_in, r_out, d, _DTYPE_CODE[out_dtype], int(block_k),
+                           _lib.QUANT_RULE_BY_NAME[rule], _lib.ptr(static_scale) if quantised else None, _lib.ptr(row_weight),
+                           _lib.ptr(row_range), _lib.ptr(out), _lib.ptr(scale), _lib.current_stream())
   _lib.check(st, "moe_gather_rows")
-  return out if scale is None else (out, scale)
+  if not quantised:
+    return out
+  return out, (static_scale if static_scale is not None else scale)
 
 
 def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None):
@@ -222,14 +245,27 @@ def transpose_rhs(rhs_gkn):
 
 def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=None, rhs_up_scale=None,
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
-            group_offset=0, out=None, tile_variant=0, tune=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None,
-            keep_other_rows=False, rhs_kn=False):
+            group_offset=0, out=None, kernel=None, raster=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None,
+            keep_other_rows=False, rhs_kn=False, rhs_scale_kmajor=False, rhs_scale_shared=False, out_dtype=torch.bfloat16,
+            lhs_row_idx=None, lhs_row_idx_div=1, out_row_scale=None, num_rows=None, workspace=None):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2]).
-  rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 without rhs_up, on shapes `gmm_rhs_kn_supported` accepts)."""
+  rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 without rhs_up, on shapes `gmm_rhs_kn_supported` accepts).
+  Scale layouts follow include/moe_mi355x.h: lhs_scale_block_k 0 = [M], -1 = [1] (per tensor), b = [M, ceil(K/b)];
+  rhs scales [G, ceil(N/bn), ceil(K/bk)], or [G, ceil(K/bk), N] with rhs_scale_kmajor, without the leading G with
+  rhs_scale_shared; bn = -1: one scale for all channels.
+  lhs_row_idx [M] int32: row i of the product reads lhs row lhs_row_idx[i] // lhs_row_idx_div (lhs then has any number of
+  rows); out_row_scale [M] f32 multiplies the result rows.  kernel / raster select a kernel family (moe_gmm_tuned)."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
   _need(group_sizes, "group_sizes", torch.int32, 1)
-  m, kdim = lhs.shape
+  lhs_rows, kdim = lhs.shape
+  if lhs_row_idx is not None:
+    _need(lhs_row_idx, "lhs_row_idx", torch.int32, 1)
+    m = lhs_row_idx.numel()
+  else:
+    m = lhs_rows if num_rows is None else int(num_rows)
+    if m > lhs_rows:
+      raise ValueError("num_rows exceeds the rows of lhs")
   if rhs_kn:
     g_local, kr, n = rhs.shape
   else:
@@ -251,13 +287,14 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
       if t.shape != rhs.shape:
         raise ValueError("rhs_up must match rhs")
   nkb_r = 1 if rhs_scale_block_k == 0 else (kdim + rhs_scale_block_k - 1) // rhs_scale_block_k
-  nnb = (n + rhs_scale_block_n - 1) // rhs_scale_block_n
+  nnb = 1 if rhs_scale_block_n == _lib.MOE_SCALE_PER_TENSOR else (n + rhs_scale_block_n - 1) // rhs_scale_block_n
   for name, t in (("rhs_scale", rhs_scale), ("rhs_up_scale", rhs_up_scale)):
     if t is not None:
       _need(t, name)
-      want = torch.bfloat16 if rhs_dtype == MOE_INT4 else (torch.uint8 if rhs_dtype == MOE_MXFP4 else torch.float32)
-      if t.dtype != want or t.numel() != g_local * nnb * nkb_r:
-        raise ValueError(f"{name} must be {want} with {g_local}x{nnb}x{nkb_r} elements, got {t.dtype} {tuple(t.shape)}")
+      want = torch.bfloat16 if rhs_dtype == MOE_INT4 and not rhs_scale_kmajor else (torch.uint8 if rhs_dtype == MOE_MXFP4 else torch.float32)
+      count = (1 if rhs_scale_shared else g_local) * nnb * nkb_r
+      if t.dtype != want or t.numel() != count:
+        raise ValueError(f"{name} must be {want} with {count} elements, got {t.dtype} {tuple(t.shape)}")
   for name, t in (("rhs_bias", rhs_bias), ("rhs_up_bias", rhs_up_bias)):
     if t is not None:
       _need(t, name, torch.float32, 2)
@@ -274,19 +311,30 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
     raise ValueError("partial_sum_up needs rhs_up")
   if lhs_scale is not None:
     _need(lhs_scale, "lhs_scale", torch.float32)
-    nkb_l = 1 if lhs_scale_block_k == 0 else (kdim + lhs_scale_block_k - 1) // lhs_scale_block_k
-    if lhs_scale.numel() != m * nkb_l:
-      raise ValueError(f"lhs_scale must have {m}x{nkb_l} elements")
+    if lhs_scale_block_k == _lib.MOE_SCALE_PER_TENSOR:
+      count = 1
+    else:
+      count = lhs_rows * (1 if lhs_scale_block_k == 0 else (kdim + lhs_scale_block_k - 1) // lhs_scale_block_k)
+    if lhs_scale.numel() != count:
+      raise ValueError(f"lhs_scale must have {count} elements, got {lhs_scale.numel()}")
+  if out_row_scale is not None:
+    _need(out_row_scale, "out_row_scale", torch.float32, 1)
+    if out_row_scale.numel() != m:
+      raise ValueError("out_row_scale must have one value per row of the product")
+  if out_dtype not in (torch.bfloat16, torch.float32):
+    raise TypeError("out_dtype must be bfloat16 or float32")
   if out is None:
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=lhs.device)
+    out = torch.empty((m, n), dtype=out_dtype, device=lhs.device)
   else:
-    _need(out, "out", torch.bfloat16, 2)
+    _need(out, "out", out_dtype, 2)
     if out.shape != (m, n):
       raise ValueError("out must be [M, N]")
+  if kernel not in _lib.GMM_KERNEL_BY_NAME:
+    raise ValueError(f"unknown kernel family {kernel!r}")
   lib = _lib.load()
   g_total = group_sizes.numel()
   wsb = lib.moe_gmm_workspace_bytes(m, g_total)
-  ws = torch.empty((max(wsb, 16),), dtype=torch.uint8, device=lhs.device)
+  ws = workspace if workspace is not None else torch.empty((max(wsb, 16),), dtype=torch.uint8, device=lhs.device)
   a = _lib.GmmArgs()
   a.struct_size = ctypes.sizeof(_lib.GmmArgs)
   a.lhs, a.lhs_scale = lhs.data_ptr(), (lhs_scale.data_ptr() if lhs_scale is not None else None)
@@ -294,21 +342,28 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.rhs_up = rhs_up.data_ptr() if rhs_up is not None else None
   a.rhs_up_scale = rhs_up_scale.data_ptr() if rhs_up_scale is not None else None
   a.group_sizes, a.out = group_sizes.data_ptr(), out.data_ptr()
-  a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+  a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
   a.M, a.K, a.N = m, kdim, n
   a.num_groups_total, a.num_groups_local, a.group_offset = g_total, g_local, int(group_offset)
   a.lhs_dtype, a.rhs_dtype = _DTYPE_CODE[lhs.dtype], rhs_dtype
   a.lhs_scale_block_k, a.rhs_scale_block_n, a.rhs_scale_block_k = int(lhs_scale_block_k), int(rhs_scale_block_n), int(rhs_scale_block_k)
   a.act = _lib.ACT_BY_NAME[act]
   a.act_limit = float(act_limit)
+  a.out_dtype = _lib.MOE_BF16 if out_dtype == torch.bfloat16 else _lib.MOE_F32
+  a.lhs_row_idx = lhs_row_idx.data_ptr() if lhs_row_idx is not None else None
+  a.lhs_row_idx_div, a.lhs_rows = int(lhs_row_idx_div), lhs_rows
+  a.out_row_scale = out_row_scale.data_ptr() if out_row_scale is not None else None
   a.rhs_bias = rhs_bias.data_ptr() if rhs_bias is not None else None
   a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
   a.partial_sum = partial_sum.data_ptr() if partial_sum is not None else None
   a.partial_sum_up = partial_sum_up.data_ptr() if partial_sum_up is not None else None
-  a.flags = (_lib.MOE_GMM_KEEP_OTHER_ROWS if keep_other_rows else 0) | (_lib.MOE_GMM_RHS_KN if rhs_kn else 0)
-  a.reserved[0] = int(tile_variant)
-  a.reserved[1] = int(tune)
-  st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
+  a.flags = ((_lib.MOE_GMM_KEEP_OTHER_ROWS if keep_other_rows else 0) | (_lib.MOE_GMM_RHS_KN if rhs_kn else 0)
+             | (_lib.MOE_GMM_RHS_SCALE_KMAJOR if rhs_scale_kmajor else 0) | (_lib.MOE_GMM_RHS_SCALE_SHARED if rhs_scale_shared else 0))
+  code = _lib.GMM_KERNEL_BY_NAME[kernel]
+  if code or raster:
+    st = lib.moe_gmm_tuned(ctypes.byref(a), code, int(raster), _lib.current_stream())
+  else:
+    st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
   _lib.check(st, "moe_gmm")
   return out
 

@@ -42,28 +42,61 @@ def _validate_args(lhs, rhs, group_sizes, expected_rhs_dims=3):
     raise ValueError(f"Expected 32-bit integer 'group_sizes' but got {group_sizes.dtype}.")
 
 
-def quantize_lhs(lhs: torch.Tensor, qdtype) -> QArray:
-  """Activation quantiser: int8 per row (ops.py:241-248) or fp8 per row per 128 values of K
-  (the per-block dynamic scale of pallas_mosaic_tpu_v2_gmm_kernel.py:534-542, block 128)."""
+def _qname(qdtype):
   if qdtype in _INT8_NAMES:
-    q, s = kernels.gather_rows(lhs, out_dtype=torch.int8)
-    return QArray(q, s, "int8")
+    return "int8"
   if qdtype in _FP8_NAMES:
-    q, s = kernels.gather_rows(lhs, out_dtype=torch.float8_e4m3fn, block_k=128)
-    return QArray(q, s, "fp8")
-  raise ValueError(f"unsupported lhs_quantize_dtype {qdtype}")
-
-
-def quantize_rhs(rhs_gnk: torch.Tensor, qdtype, share_across_experts=True) -> QArray:
-  """Weight quantiser for rhs in [G, N, K] layout.  share_across_experts=True reproduces the
-  [1,1,n] scale of ops.py:250-260 (channelwise over the output axis only)."""
-  if qdtype in _INT8_NAMES:
-    return quantizations.quantize_weight_int8(rhs_gnk, share_across_experts=share_across_experts)
-  if qdtype in _FP8_NAMES:
-    return quantizations.quantize_weight_fp8_blocks(rhs_gnk)
+    return "fp8"
   if qdtype in _INT4_NAMES:
-    return quantizations.quantize_weight_int4(rhs_gnk)
-  raise ValueError(f"unsupported rhs_quantize_dtype {qdtype}")
+    return "int4"
+  raise ValueError(f"unsupported quantisation dtype {qdtype}")
+
+
+_TORCH_Q = {"int8": torch.int8, "fp8": torch.float8_e4m3fn}
+_QMAX = {"int8": 127.0, "fp8": quantizations.FP8_E4M3_MAX}
+
+
+def _static_scale_tensor(qname, calibration_method, device):
+  return torch.tensor([quantizations.get_static_scale(_QMAX[qname], calibration_method)], dtype=torch.float32, device=device)
+
+
+def quantize_lhs(lhs: torch.Tensor, qdtype, *, calibration_method="absmax", blocks=None, v2=False) -> QArray:
+  """Activation quantiser.
+
+  v2=False: the v1 path, qpl.quantize(lhs, act_qtype, channelwise_axes=[0], calibration_method) (ops.py:241-248):
+  one scale per row, for int8 and for fp8; "fixed,..." gives one static scale for the tensor.  blocks=128 keeps the
+  DeepSeek recipe's one scale per row and 128 values of K.
+  v2=True: the quantiser inside gmm_v2 (pallas_mosaic_tpu_v2_gmm_kernel.py:528-542): one scale per row and 512 values
+  of K (:1231), or the static (1, 1) scale of ops.py:333-360."""
+  qname = _qname(qdtype)
+  if qname not in _TORCH_Q:
+    raise ValueError(f"unsupported lhs_quantize_dtype {qdtype}")
+  rule = "v2" if v2 else "rint_div"
+  if calibration_method is not None and calibration_method.lower().startswith("fixed"):
+    st = _static_scale_tensor(qname, calibration_method, lhs.device)
+    q, s = kernels.gather_rows(lhs, out_dtype=_TORCH_Q[qname], rule=rule, static_scale=st)
+    return QArray(q, s, qname, block_k=-1)
+  block_k = 512 if v2 and blocks is None else (blocks or 0)
+  q, s = kernels.gather_rows(lhs, out_dtype=_TORCH_Q[qname], block_k=block_k, rule=rule)
+  return QArray(q, s, qname, block_k=block_k)
+
+
+def quantize_rhs(rhs_gnk: torch.Tensor, qdtype, share_across_experts=True, *, calibration_method="absmax", manual=False,
+                 fp8_blocks=False) -> QArray:
+  """Weight quantiser for rhs in [G, N, K] layout: one scale per output channel shared by the experts, the [1, 1, n]
+  scale of qpl.quantize(rhs, channelwise_axes=[2]) (ops.py:250-260), for int8 and fp8; manual=True is
+  quantizations.manual_quantize (per tensor, static, ops.py:262-266); fp8_blocks=True the 128 x 128 blocks of DeepSeek
+  checkpoints."""
+  qname = _qname(qdtype)
+  if manual:
+    return quantizations.manual_quantize_weight(rhs_gnk, qname, calibration_method)
+  if qname == "int8":
+    return quantizations.quantize_weight_int8(rhs_gnk, share_across_experts=share_across_experts)
+  if qname == "fp8":
+    if fp8_blocks:
+      return quantizations.quantize_weight_fp8_blocks(rhs_gnk)
+    return quantizations.quantize_weight_fp8_channel(rhs_gnk, share_across_experts=share_across_experts)
+  return quantizations.quantize_weight_int4(rhs_gnk)
 
 
 def _native_rhs(rhs, transpose_rhs):
@@ -73,6 +106,26 @@ def _native_rhs(rhs, transpose_rhs):
   if transpose_rhs:
     return rhs if rhs.is_contiguous() else rhs.contiguous()
   return kernels.transpose_rhs(rhs.contiguous())
+
+
+def _rhs_layout(q: QArray) -> dict:
+  """moe_gmm's scale arguments for a weight QArray."""
+  defaults = {"int8": (1, 0), "fp8": (128, 128), "int4": (1, 128), "int4g32": (1, 32), "mxfp4": (1, 32)}
+  if q.qtype not in defaults:
+    raise ValueError(f"unknown qtype {q.qtype}")
+  bn, bk = defaults[q.qtype]
+  kw = dict(rhs_scale_block_n=bn if q.block_n is None else q.block_n, rhs_scale_block_k=bk if q.block_k is None else q.block_k,
+            rhs_scale_kmajor=q.kmajor, rhs_scale_shared=q.shared)
+  if q.qtype.startswith("int4"):
+    kw["rhs_dtype"] = MOE_INT4
+  elif q.qtype == "mxfp4":
+    kw["rhs_dtype"] = MOE_MXFP4
+  return kw
+
+
+def _lhs_layout(q: QArray) -> dict:
+  bk = q.block_k if q.block_k is not None else (128 if q.qtype == "fp8" else 0)
+  return dict(lhs_scale=q.scale, lhs_scale_block_k=bk)
 
 
 def gmm(
@@ -104,6 +157,9 @@ def gmm(
     rhs_up_bias=None,
     partial_sum_up=None,
     bwd_quantize_dtype=None,
+    lhs_row_idx=None,
+    lhs_row_idx_div=1,
+    out_row_scale=None,
 ):
   """Grouped matmul: out[rows of group g] = lhs[rows] @ rhs[g] (ops.py:46).
 
@@ -112,18 +168,27 @@ def gmm(
 
   lhs: [m, k] bf16 tensor or QArray; rhs: [g, k, n] bf16 ([g, n, k] with transpose_rhs) or a
   QArray holding [G, N, K]; group_sizes: int32 [G_total] on the device.  `tiling`, `interpret`,
-  the vma axes and the backend switches only select TPU code paths in the reference and are
+  the vma axes and `use_tokamax_backend` only select TPU code paths in the reference and are
   accepted and ignored; the tile shape is chosen from rows-per-expert inside moe_gmm.
+
+  Quantisation follows ops.py:87-103 and _fwd_quantize_activation_and_weight (:232-267): with use_qwix_quantization
+  the rule is `qwix_rule` (a quantizations.QtRule), otherwise one is made from lhs / rhs_quantize_dtype with "absmax"
+  calibration.  Activations get one scale per row ([m, 1]), weights one per output channel shared by the experts
+  ([1, 1, n]); use_manual_quantization quantises the weights per tensor with the rule's static range; "fixed,..."
+  calibration gives static per-tensor scales.  With use_gmm_v2 the activations are quantised by gmm_v2's own rule
+  (per row and 512 values of K, or the static (1, 1) scale, ops.py:333-360) to the type the weights ask for
+  (pallas_mosaic_tpu_v2_gmm_kernel.py:1208-1223: int8 weights -> int8, fp8 weights -> fp8; int4 weights stay
+  weight-only here).  preferred_element_type: bfloat16 or float32.
+  lhs_row_idx / lhs_row_idx_div / out_row_scale: see kernels.gmm_raw (the permute and the routing weights fused in).
   """
-  del tiling, interpret, lhs_vma_axes, rhs_vma_axes, use_tokamax_backend, use_gmm_v2, use_qwix_quantization, qwix_rule
-  del use_manual_quantization
+  del tiling, interpret, lhs_vma_axes, rhs_vma_axes, use_tokamax_backend
   _validate_args(lhs, rhs, group_sizes)
-  if preferred_element_type != torch.bfloat16:
-    raise NotImplementedError("only bfloat16 outputs are implemented")
+  if preferred_element_type not in (torch.bfloat16, torch.float32):
+    raise NotImplementedError("outputs are bfloat16 or float32")
   if existing_out is not None:
     # rows of local groups are written into the caller's buffer, all other rows keep their contents (backend.py:493-501)
-    if existing_out.dtype != torch.bfloat16 or not existing_out.is_contiguous():
-      raise ValueError("existing_out must be a contiguous bfloat16 tensor")
+    if existing_out.dtype != preferred_element_type or not existing_out.is_contiguous():
+      raise ValueError("existing_out must be a contiguous tensor of preferred_element_type")
   if weight_gather_axes:
     raise NotImplementedError("weight all-gather belongs to the multi-device path")
   if group_offset is None:
@@ -136,75 +201,82 @@ def gmm(
     else:
       offset = int(group_offset)
 
+  # ops.py:87-103
+  rule = None
+  if use_qwix_quantization:
+    rule = qwix_rule
+    if not isinstance(rule, quantizations.QtRule):
+      raise ValueError(f"Expect a QtRule for quantized training. But get quantization_rule={rule} for gmm.")
+  elif lhs_quantize_dtype or rhs_quantize_dtype:
+    rule = quantizations.QtRule(weight_qtype=rhs_quantize_dtype, act_qtype=lhs_quantize_dtype, bwd_qtype=bwd_quantize_dtype)
+
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
-    if partial_sum is not None or partial_sum_up is not None or existing_out is not None:
-      raise NotImplementedError("gradients with partial_sum / existing_out are not implemented")
-    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_quantize_dtype, rhs_quantize_dtype, fuse_act, act_limit,
-                          bwd_quantize_dtype, rhs_bias, rhs_up_bias)
+    if partial_sum is not None or partial_sum_up is not None or existing_out is not None or lhs_row_idx is not None or out_row_scale is not None:
+      raise NotImplementedError("gradients with partial_sum / existing_out / lhs_row_idx / out_row_scale are not implemented")
+    if preferred_element_type != torch.bfloat16 or use_gmm_v2 or use_manual_quantization or (rule and rule.act_calibration_method != "absmax"):
+      raise NotImplementedError("the differentiable path takes bfloat16 outputs and dynamic (absmax) v1 quantisation")
+    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule.act_qtype if rule else None,
+                          rule.weight_qtype if rule else None, fuse_act, act_limit, rule.bwd_qtype if rule else bwd_quantize_dtype,
+                          rhs_bias, rhs_up_bias)
+
+  common = dict(group_offset=offset, out_dtype=preferred_element_type, lhs_row_idx=lhs_row_idx, lhs_row_idx_div=lhs_row_idx_div,
+                out_row_scale=out_row_scale)
+  if rhs_bias is not None:
+    common["rhs_bias"] = rhs_bias.float().contiguous()  # [G, N] (rhs_bias [G, 1, N] of the v2 kernel, :573)
+  if partial_sum is not None:  # [m, n], added to the product before the activation (ops.py:77)
+    common["partial_sum"] = partial_sum.to(torch.bfloat16).contiguous()
+  if existing_out is not None:
+    common.update(out=existing_out, keep_other_rows=True)
 
   # [g, k, n] bf16 weights are read as they are where the kernel allows it (this is dlhs of a transpose_rhs=True layer:
   # ops.py:470-485), instead of being re-laid out for every call
-  if (not transpose_rhs and rhs_up is None and rhs_quantize_dtype is None and lhs_quantize_dtype is None
-      and not isinstance(rhs, QArray) and not isinstance(lhs, QArray) and rhs.dtype == torch.bfloat16 and lhs.dtype == torch.bfloat16
-      and fuse_act is None and kernels.gmm_rhs_kn_supported(lhs.shape[0], rhs.shape[1], rhs.shape[2], group_sizes.numel())):
-    kw = dict(group_offset=offset, rhs_kn=True)
-    if rhs_bias is not None:
-      kw["rhs_bias"] = rhs_bias.float().contiguous()
-    if partial_sum is not None:
-      kw["partial_sum"] = partial_sum.to(torch.bfloat16).contiguous()
-    if existing_out is not None:
-      kw["out"], kw["keep_other_rows"] = existing_out, True
-    return kernels.gmm_raw(lhs.contiguous(), rhs.contiguous(), group_sizes, **kw)
+  if (not transpose_rhs and rhs_up is None and rule is None and not isinstance(rhs, QArray) and not isinstance(lhs, QArray)
+      and rhs.dtype == torch.bfloat16 and lhs.dtype == torch.bfloat16 and fuse_act is None and lhs_row_idx is None
+      and kernels.gmm_rhs_kn_supported(lhs.shape[0], rhs.shape[1], rhs.shape[2], group_sizes.numel())):
+    return kernels.gmm_raw(lhs.contiguous(), rhs.contiguous(), group_sizes, rhs_kn=True, **common)
 
   rhs_n = _native_rhs(rhs, transpose_rhs)
   up_n = _native_rhs(rhs_up, transpose_rhs) if rhs_up is not None else None
-  if not isinstance(rhs_n, QArray) and rhs_quantize_dtype is not None:
-    rhs_n = quantize_rhs(rhs_n, rhs_quantize_dtype)
+  if rule is not None and rule.weight_qtype and not isinstance(rhs_n, QArray):
+    if rule.disable_channelwise_axes and not use_manual_quantization:
+      raise NotImplementedError("dynamic per-tensor weight scales (disable_channelwise_axes) are not implemented")
+    qkw = dict(calibration_method=rule.weight_calibration_method, manual=use_manual_quantization)
+    rhs_n = quantize_rhs(rhs_n, rule.weight_qtype, **qkw)
     if up_n is not None:
-      up_n = quantize_rhs(up_n, rhs_quantize_dtype)
-  if not isinstance(lhs, QArray) and lhs_quantize_dtype is not None:
-    lhs = quantize_lhs(lhs.contiguous(), lhs_quantize_dtype)
+      up_n = quantize_rhs(up_n, rule.weight_qtype, **qkw)
+  if rule is not None and rule.act_qtype and not isinstance(lhs, QArray):
+    if rule.disable_channelwise_axes and not (rule.act_calibration_method or "").lower().startswith("fixed"):
+      raise NotImplementedError("dynamic per-tensor activation scales (disable_channelwise_axes) are not implemented")
+    if not use_gmm_v2:
+      lhs = quantize_lhs(lhs.contiguous(), rule.act_qtype, calibration_method=rule.act_calibration_method)
+  if use_gmm_v2 and isinstance(rhs_n, QArray) and not isinstance(lhs, QArray) and rhs_n.qtype in ("int8", "fp8"):
+    # gmm_v2 quantises the activations itself, to the type the weights ask for (:1208-1223), statically when the rule
+    # carries a fixed range (ops.py:333-360)
+    method = rule.act_calibration_method if rule is not None and rule.act_qtype else "absmax"
+    lhs = quantize_lhs(lhs.contiguous(), rhs_n.qtype, calibration_method=method, v2=True)
 
-  kw = dict(act=fuse_act, act_limit=act_limit, group_offset=offset)
-  if rhs_bias is not None:
-    kw["rhs_bias"] = rhs_bias.float().contiguous()  # [G, N] (rhs_bias [G, 1, N] of the v2 kernel, :573)
+  kw = dict(act=fuse_act, act_limit=act_limit, **common)
   if rhs_up_bias is not None:
     kw["rhs_up_bias"] = rhs_up_bias.float().contiguous()
-  if partial_sum is not None:  # [m, n], added to the product before the activation (ops.py:77)
-    kw["partial_sum"] = partial_sum.to(torch.bfloat16).contiguous()
   if partial_sum_up is not None:
     kw["partial_sum_up"] = partial_sum_up.to(torch.bfloat16).contiguous()
   if isinstance(lhs, QArray):
-    kw["lhs_scale"] = lhs.scale
-    kw["lhs_scale_block_k"] = 128 if lhs.qtype == "fp8" else 0
+    kw.update(_lhs_layout(lhs))
     lhs_t = lhs.qvalue
   else:
     lhs_t = lhs.contiguous()
   if isinstance(rhs_n, QArray):
     kw["rhs_scale"] = rhs_n.scale
+    kw.update(_rhs_layout(rhs_n))
     if up_n is not None:
       if not isinstance(up_n, QArray) or up_n.qtype != rhs_n.qtype:
         raise ValueError("rhs_up must be quantised like rhs")
       kw["rhs_up"], kw["rhs_up_scale"] = up_n.qvalue, up_n.scale
-    if rhs_n.qtype == "int8":
-      kw.update(rhs_scale_block_n=1, rhs_scale_block_k=0)
-    elif rhs_n.qtype == "fp8":
-      kw.update(rhs_scale_block_n=128, rhs_scale_block_k=128)
-    elif rhs_n.qtype == "int4":
-      kw.update(rhs_scale_block_n=1, rhs_scale_block_k=128, rhs_dtype=MOE_INT4)
-    elif rhs_n.qtype == "int4g32":
-      kw.update(rhs_scale_block_n=1, rhs_scale_block_k=32, rhs_dtype=MOE_INT4)
-    elif rhs_n.qtype == "mxfp4":
-      kw.update(rhs_scale_block_n=1, rhs_scale_block_k=32, rhs_dtype=MOE_MXFP4)
-    else:
-      raise ValueError(f"unknown qtype {rhs_n.qtype}")
     rhs_t = rhs_n.qvalue
   else:
     rhs_t = rhs_n
     if up_n is not None:
       kw["rhs_up"] = up_n
-  if existing_out is not None:
-    kw.update(out=existing_out, keep_other_rows=True)
   return kernels.gmm_raw(lhs_t, rhs_t, group_sizes, **kw)
 
 

@@ -330,7 +330,8 @@ class RoutedMoE:
     if marks:
       marks[1].record()
     if cfg.act_quant is not None:
-      inter = megablox.quantize_lhs(inter, cfg.act_quant)
+      # the layer's fp8 configuration is the DeepSeek recipe: 128 x 128 weight blocks with 1 x 128 activation scales
+      inter = megablox.quantize_lhs(inter, cfg.act_quant, blocks=128 if cfg.act_quant == "fp8" else None)
     if marks:
       marks[2].record()
     out = megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias)

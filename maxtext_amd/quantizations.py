@@ -32,15 +32,36 @@ class QArray:
   has the layout described in the module docstring; `qtype` is "int8" | "fp8" | "int4" | "int4g32" | "mxfp4"
   (mxfp4: uint8 [G, N, K/2] e2m1 pairs and uint8 [G, N, K/32] e8m0 block scales).
   For activations `qvalue` is [M, K] and `scale` is [M] (int8) or [M, ceil(K/128)] (fp8).
+
+  The optional fields override the layout a qtype implies (they mirror the scale arguments of moe_gmm):
+  block_n / block_k: output channels / values of K per scale (block_n -1: one scale for all channels; block_k 0: all
+  of K; for activations block_k -1: one scale for the tensor), kmajor: weight scales stored [G, K/block_k, N]
+  (gmm_v2's [G, nb, 1, N]), shared: weight scales without the leading expert dimension.
   """
 
   qvalue: torch.Tensor
   scale: torch.Tensor
   qtype: str
+  block_n: int | None = None
+  block_k: int | None = None
+  kmajor: bool = False
+  shared: bool = False
 
   @property
   def shape(self):
     return self.qvalue.shape
+
+
+@dataclasses.dataclass
+class QtRule:
+  """The fields of qwix.QtRule that gmm reads (ops.py:97-103, :241-266, :583-604)."""
+
+  weight_qtype: object = None
+  act_qtype: object = None
+  bwd_qtype: object = None
+  weight_calibration_method: str = "absmax"
+  act_calibration_method: str = "absmax"
+  disable_channelwise_axes: bool = False
 
 
 def get_static_scale(qmax: float, calibration_method: str) -> float:
@@ -72,6 +93,36 @@ def quantize_weight_int8(w_gnk: torch.Tensor, share_across_experts: bool = False
   scale = absmax / 127.0
   q = _rint_div(w, scale).clamp(-127, 127).to(torch.int8)
   return QArray(q.contiguous(), scale.squeeze(-1).contiguous(), "int8")
+
+
+def quantize_weight_fp8_channel(w_gnk: torch.Tensor, share_across_experts: bool = True) -> QArray:
+  """w [G, N, K] -> float8_e4m3fn with one f32 scale per output channel: shared by the experts ([1, 1, n], what
+  qpl.quantize(rhs, channelwise_axes=[2]) yields, ops.py:250-260) or per expert.  The rounding of the third-party
+  quantiser is not pinned; this uses scale = absmax / 448 and the round-to-nearest-even cast."""
+  w = w_gnk.to(torch.float32)
+  absmax = w.abs().amax(dim=(0, 2) if share_across_experts else 2, keepdim=True)
+  scale = absmax / FP8_E4M3_MAX
+  q = torch.where(scale == 0, torch.zeros_like(w), w / scale).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+  sc = scale.reshape(1, -1) if share_across_experts else scale.squeeze(-1)
+  return QArray(q.contiguous(), sc.contiguous(), "fp8", block_n=1, block_k=0, shared=share_across_experts)
+
+
+def manual_quantize_weight(w_gnk: torch.Tensor, qtype: str, calibration_method: str) -> QArray:
+  """Per-tensor static weight quantisation, layers/quantizations.py:961-991 (manual_quantize):
+  q = clip(w / scale, -qmax, qmax).astype(qtype) with scale and bounds held as bf16 tensors (:923-925), so the
+  division runs in promote(w.dtype, bf16); the QArray's scale is the python float in w's dtype.  int8 truncates
+  toward zero, fp8 rounds to nearest even, as `.astype` does."""
+  qmax = 127.0 if qtype == "int8" else FP8_E4M3_MAX
+  scale = get_static_scale(qmax, calibration_method)
+  s_bf = torch.tensor(scale, dtype=torch.float32).to(torch.bfloat16).float()
+  y = w_gnk.float() / s_bf.to(w_gnk.device)
+  if w_gnk.dtype == torch.bfloat16:
+    y = y.to(torch.bfloat16).float()
+  bound = float(torch.tensor(qmax).to(torch.bfloat16))
+  y = y.clamp(-bound, bound)
+  q = torch.trunc(y).clamp(-128, 127).to(torch.int8) if qtype == "int8" else y.to(torch.float8_e4m3fn)
+  sc = torch.tensor([scale], dtype=torch.float32).to(w_gnk.dtype).float().to(w_gnk.device)
+  return QArray(q.contiguous(), sc, qtype, block_n=-1, block_k=0, shared=True)
 
 
 def quantize_weight_fp8_blocks(w_gnk: torch.Tensor, block: int = 128) -> QArray:

@@ -35,15 +35,24 @@ How each function is pinned (see tests/test_oracle_*.py):
       nibble order and 2^(s-127) scaling on hand-made blocks; quantize_mxfp4 (a test-data generator only) by
       dequantize(quantize(x)) == x on representable inputs.
 
+  quantize_lhs_v2 / manual_quantize (the quantisers whose source IS in the reference tree)
+      hand cases worked out in exact rational arithmetic (python Fractions with an explicit round-to-nearest-even
+      to the 8-bit / 24-bit significand) that separate truncation from round-half-even and round-half-away,
+      x * (1 / scale) from x / scale, and bf16 from f32 intermediate arithmetic; the closed forms
+      q * scale == x on inputs that are exact multiples of the scale; zero rows.
+
 PARITY UNPINNED (third-party arithmetic whose source is not in the reference
 tree, and which no reference test pins):
-  * quantize_* rounding mode and zero-scale handling (qwix.pallas.quantize,
-    qwix >= 0.1.8).  Adopted: scale = absmax / qmax, q = clip(rint(x / scale)),
-    zero absmax -> q = 0 (as pallas_mosaic_tpu_v2_gmm_kernel.py:537-540).
-    GEMM parity is therefore asserted on identical already-quantized operands.
+  * quantize_rows_int8 / quantize_weight_int8 / quantize_fp8_blocks / quantize_e5m2: rounding mode and
+    zero-scale handling of qwix.pallas.quantize (qwix >= 0.1.8), the quantiser of the v1 path
+    (ops.py:241-260, :563-571, :590-603).  Adopted: scale = absmax / qmax, q = clip(rint(x / scale)),
+    zero absmax -> q = 0.  GEMM parity is therefore asserted on identical already-quantized operands.
+    (The v2 path's in-kernel quantiser and manual_quantize are restated exactly, see above.)
   * tie order of jax.lax.top_k and stability of jnp.argsort (jax >= 0.10.2).
     Adopted: larger value first, lower index first on ties; stable sort.
   * bf16 rounding of the norm_topk_prob renormalisation (moe.py:756).
+  * the value an out-of-range float -> int8 conversion yields in XLA (implementation defined); unreachable from
+    quantize_lhs_v2 (|x * inv| <= 127.5 before truncation), clamped here.
 """
 
 from __future__ import annotations
@@ -284,12 +293,12 @@ def gmm(
     rhs: torch.Tensor,  # [g, k, n] (or [g, n, k] with transpose_rhs)
     group_sizes,  # [G_total] int32
     *,
-    rhs_scale: torch.Tensor | None = None,  # [g, nb, 1, n] f32 (v2 format) or [g, n]
-    lhs_scale: torch.Tensor | None = None,  # [m] / [m,1] per row, or [m, nb] per K-block
+    rhs_scale: torch.Tensor | None = None,  # [g, nb, 1, n] f32 (v2 format) or [g, n]; g may be 1 (shared by all experts)
+    lhs_scale: torch.Tensor | None = None,  # [m] / [m,1] per row, [m, nb] per K-block, or [1, 1] (static per-tensor)
     rhs_bias: torch.Tensor | None = None,  # [g, 1, n]
     partial_sum: torch.Tensor | None = None,  # [m, n]
     group_offset: int = 0,
-    quant_block: int | None = None,  # K-block size when scales are block-wise (ragged tail allowed)
+    quant_block=None,  # K-block size when scales are block-wise (ragged tail allowed); (lhs_block, rhs_block) when they differ
     transpose_rhs: bool = False,
     out_dtype=torch.bfloat16,
     acc_dtype=torch.float64,
@@ -312,12 +321,17 @@ def gmm(
   if lhs_scale is not None and lhs_scale.dim() == 1:
     lhs_scale = lhs_scale[:, None]
   nb_l = lhs_scale.shape[1] if lhs_scale is not None else 1
-  nb = max(nb_r, nb_l)
-  if nb > 1:
-    qb = quant_block if quant_block is not None else k // nb
-    assert math.ceil(k / qb) == nb, (k, qb, nb)
+  # K-block of each side's scales (quant_block: the common one, or a (lhs, rhs) pair when they differ, as in gmm_v2
+  # where the activation block is 512 and the weight block comes with the checkpoint); the sum runs over the common
+  # refinement of the two grids
+  if isinstance(quant_block, (tuple, list)):
+    qb_l, qb_r = quant_block
   else:
-    qb = k
+    qb_l = qb_r = quant_block
+  qb_l = k if nb_l == 1 else (qb_l if qb_l is not None else k // nb_l)
+  qb_r = k if nb_r == 1 else (qb_r if qb_r is not None else k // nb_r)
+  assert math.ceil(k / qb_l) == nb_l and math.ceil(k / qb_r) == nb_r, (k, qb_l, nb_l, qb_r, nb_r)
+  cuts = sorted(set(range(0, k, qb_l)) | set(range(0, k, qb_r)) | {k})
 
   start = 0
   for gg in range(group_sizes.size):
@@ -325,13 +339,13 @@ def gmm(
     loc = gg - group_offset
     if 0 <= loc < g and end > start:
       acc = torch.zeros((end - start, n), dtype=acc_dtype)
-      for b in range(nb):
-        ks, ke = b * qb, min((b + 1) * qb, k)
+      for ks, ke in zip(cuts[:-1], cuts[1:]):
         part = lhs[start:end, ks:ke].to(acc_dtype) @ rhs[loc, ks:ke, :].to(acc_dtype)
         if rhs_scale is not None:
-          part = part * rhs_scale[loc, b if nb_r > 1 else 0].to(acc_dtype)
+          part = part * rhs_scale[loc if rhs_scale.shape[0] > 1 else 0, ks // qb_r].to(acc_dtype)
         if lhs_scale is not None:
-          part = part * lhs_scale[start:end, (b if nb_l > 1 else 0)].to(acc_dtype)[:, None]
+          rows = slice(start, end) if lhs_scale.shape[0] > 1 else slice(0, 1)  # [1, 1]: one static scale for all rows
+          part = part * lhs_scale[rows, ks // qb_l].to(acc_dtype)[:, None]
         acc += part
       if rhs_bias is not None:
         acc = acc + rhs_bias[loc].to(acc_dtype)
@@ -428,6 +442,79 @@ def get_static_scale(qmax: float, calibration_method: str) -> float:
   if scale < np.finfo(np.float32).tiny ** 0.5:
     scale = 1.0
   return scale
+
+
+def _round_to(x: torch.Tensor, dtype) -> torch.Tensor:
+  """f32 values rounded (nearest even) to `dtype`'s grid, returned as f32: one JAX op in that dtype."""
+  return x if dtype == torch.float32 else x.to(dtype).to(torch.float32)
+
+
+def _astype_q(y: torch.Tensor, qdtype) -> torch.Tensor:
+  """jnp `.astype(qdtype)` of float values: integers truncate toward zero (XLA ConvertElementType; out-of-range values
+  are clamped here), float8_e4m3fn rounds to nearest even (values above 464 become NaN: e4m3fn has no infinity)."""
+  if qdtype == torch.int8:
+    return torch.trunc(y).clamp(-128, 127).to(torch.int8)
+  if qdtype == torch.float8_e4m3fn:
+    return y.to(torch.float8_e4m3fn)
+  raise ValueError(qdtype)
+
+
+def qdtype_max(qdtype) -> float:
+  """jnp.iinfo(int8).max / jnp.finfo(float8_e4m3fn).max (pallas_mosaic_tpu_v2_gmm_kernel.py:496-501)."""
+  return {torch.int8: 127.0, torch.float8_e4m3fn: 448.0}[qdtype]
+
+
+def quantize_lhs_v2(x: torch.Tensor, qdtype, quant_block: int = 512, static_scale=None, acc_dtype=torch.bfloat16):
+  """The activation quantiser inside gmm_v2 (pallas_mosaic_tpu_v2_gmm_kernel.py:489-542), restated op by op.
+
+  Dynamic (static_scale None, :533-542), per row and per `quant_block` values of K, every op in x's dtype (the
+  python scalars dtype_max, 0 and 1 are weakly typed, so a bf16 input keeps the arithmetic in bf16):
+      block_abs_max   = max |x|                                  (exact)
+      block_scale     = block_abs_max / dtype_max
+      block_scale_inv = where(block_scale == 0, 0, 1 / block_scale)
+      q               = (x * block_scale_inv).astype(qdtype)     (int8: truncation; fp8: nearest even)
+  Static (:528-531, scale from get_static_scale as a (1, 1) array, ops.py:333-360): lhs_scale is cast to the
+  accumulator dtype (bf16 unless the caller asks otherwise, :1247-1254), lhs_scale_inv = 1.0 / lhs_scale in that
+  dtype, q = clip(x * lhs_scale_inv, -dtype_max, dtype_max).astype(qdtype) in the promoted dtype.
+
+  The last block may be ragged (K % quant_block != 0 is rejected by the reference's tiling; allowed here).
+  Returns (q [m, k] qdtype, scale f32 [m, ceil(k / quant_block)] holding the values of x's dtype; static: [1, 1])."""
+  dt = x.dtype
+  assert dt in (torch.bfloat16, torch.float32)
+  xf = x.to(torch.float32)
+  m, k = xf.shape
+  qmax = qdtype_max(qdtype)
+  if static_scale is not None:
+    wide = torch.float32 if torch.float32 in (dt, acc_dtype) else torch.bfloat16  # jnp promotion of x * lhs_scale_inv
+    s = _round_to(torch.tensor([[float(static_scale)]], dtype=torch.float32), acc_dtype)
+    inv = _round_to(1.0 / s, acc_dtype)
+    y = _round_to(xf * inv, wide).clamp(-qmax, qmax)
+    return _astype_q(y, qdtype), s
+  nb = math.ceil(k / quant_block)
+  q = torch.empty((m, k), dtype=qdtype)
+  scale = torch.empty((m, nb), dtype=torch.float32)
+  for b in range(nb):
+    blk = xf[:, b * quant_block : (b + 1) * quant_block]
+    amax = blk.abs().amax(dim=1, keepdim=True)
+    s = _round_to(amax / qmax, dt)
+    inv = torch.where(s == 0, torch.zeros_like(s), _round_to(1.0 / s, dt))
+    q[:, b * quant_block : (b + 1) * quant_block] = _astype_q(_round_to(blk * inv, dt), qdtype)
+    scale[:, b] = s[:, 0]
+  return q, scale
+
+
+def manual_quantize(w: torch.Tensor, qdtype, calibration_method: str):
+  """layers/quantizations.py:961-991: per-tensor static quantisation of a weight,
+  q = clip(w / scale, -qmax, qmax).astype(qdtype) with scale, qmax as bf16 tensors (_make_scale_tensor :923-925:
+  dtype=jnp.bfloat16), so w / scale is computed in promote(w.dtype, bf16); the QArray's scale is the python
+  float cast to w's dtype, shape [1] * ndim.  Returns (q, scale f32 scalar tensor holding that value)."""
+  qmax = qdtype_max(qdtype)
+  scale = get_static_scale(qmax, calibration_method)
+  s_bf = _round_to(torch.tensor(float(scale)), torch.bfloat16)
+  y = _round_to(w.to(torch.float32) / s_bf, w.dtype)
+  bound = float(_round_to(torch.tensor(qmax), torch.bfloat16))
+  q = _astype_q(y.clamp(-bound, bound), qdtype)
+  return q, _round_to(torch.tensor(float(scale)), w.dtype)
 
 
 def _absmax_scale(x: torch.Tensor, dim, qmax: float):

@@ -20,7 +20,7 @@ def _declared_symbols():
 def test_header_declares_the_expected_entry_points():
   names = _declared_symbols()
   for must in ("moe_route_topk", "moe_sort_by_expert", "moe_gather_rows", "moe_gmm", "moe_unpermute_combine",
-               "moe_gmm_workspace_bytes", "moe_gmm_rhs_kn_supported", "moe_sort_workspace_bytes", "moe_transpose_rhs", "moe_last_error"):
+               "moe_gmm_workspace_bytes", "moe_gmm_rhs_kn_supported", "moe_gmm_tuned", "moe_sort_workspace_bytes", "moe_transpose_rhs", "moe_last_error"):
     assert must in names
 
 
@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_size_queries_and_struct_layout_without_gpu():
   lib = _lib.load()
-  assert lib.moe_abi_version() == 1
+  assert lib.moe_abi_version() == 2
   assert lib.moe_sort_workspace_bytes(2048, 2, 8) >= (4 * 4 * 8 + 8) * 4
   assert lib.moe_gmm_workspace_bytes(4096, 8) >= 16 + (4096 // 16 + 9) * 16
 
@@ -44,13 +44,15 @@ def test_struct_layout_matches_the_header(tmp_path):
   # the C compiler's view of moe_gmm_args (size and a few offsets) must equal the ctypes mirror
   src = tmp_path / "layout.c"
   src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "moe_mi355x.h"\n'
-                 'int main(void){printf("%zu %zu %zu %zu %zu\\n", sizeof(moe_gmm_args), offsetof(moe_gmm_args, workspace_bytes),'
-                 ' offsetof(moe_gmm_args, M), offsetof(moe_gmm_args, act), offsetof(moe_gmm_args, act_limit));return 0;}\n')
+                 'int main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(moe_gmm_args), offsetof(moe_gmm_args, workspace_bytes),'
+                 ' offsetof(moe_gmm_args, M), offsetof(moe_gmm_args, act), offsetof(moe_gmm_args, act_limit),'
+                 ' offsetof(moe_gmm_args, out_dtype), offsetof(moe_gmm_args, rhs_bias), offsetof(moe_gmm_args, out_row_scale));return 0;}\n')
   exe = tmp_path / "layout"
   subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
   got = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
   g = _lib.GmmArgs
-  assert got == [ctypes.sizeof(g), g.workspace_bytes.offset, g.M.offset, g.act.offset, g.act_limit.offset]
+  assert got == [ctypes.sizeof(g), g.workspace_bytes.offset, g.M.offset, g.act.offset, g.act_limit.offset, g.out_dtype.offset,
+                 g.rhs_bias.offset, g.out_row_scale.offset]
 
 
 def test_argument_errors_are_reported_not_launched():

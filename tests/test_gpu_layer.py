@@ -18,9 +18,12 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def relerr(got, want):
-  got, want = got.detach().float().cpu(), want.detach().float().cpu()
-  return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+import functools
+
+import tolerances
+
+# whole layers are chains of three matmuls with bf16 (or re-quantised) intermediates
+relerr = functools.partial(tolerances.relerr, atol_rms=tolerances.ELEM_ATOL_RMS_CHAINED)
 
 
 def _small(name, tokens, **dims):
@@ -225,7 +228,8 @@ def test_layer_gradients_match_torch_autograd(norm_topk_prob):
   # bf16 intermediates on the way back (dy, d inter, d h0/h1 are each rounded to bf16): 3e-2 of the max
   for got, want, name in zip(leaves, r, ("x", "gate", "wi_0", "wi_1", "wo")):
     assert got.grad is not None and got.grad.shape == got.shape, name
-    assert relerr(got.grad, want.grad) <= 3e-2, name
+    # (each gradient is a sum of products of values that were rounded to bf16 two or three times on the way back)
+    assert relerr(got.grad, want.grad, atol_rms=5e-2) <= 3e-2, name
 
 
 def test_layer_gradients_with_int8_quantised_forward():
@@ -250,7 +254,8 @@ def test_layer_gradients_with_int8_quantised_forward():
     out.float().square().sum().backward()
     grads[q] = [v.grad for v in leaves]
   for a, b in zip(grads[None], grads["int8"]):
-    assert relerr(b, a) <= 5e-2
+    # two different computations (quantised against unquantised forward): only the max-norm criterion applies
+    assert relerr(b, a, elementwise=False) <= 5e-2
 
 
 def test_layer_gradients_with_expert_biases():
@@ -286,7 +291,8 @@ def test_layer_gradients_with_expert_biases():
   assert relerr(out.reshape(t, d), ref) <= 2e-2
   for got, want, name in zip(leaves, r, ("x", "wi_0", "wi_1", "wo", "b0", "b1", "bo")):
     assert got.grad is not None and got.grad.shape == got.shape, name
-    assert relerr(got.grad, want.grad) <= 3e-2, name
+    # (each gradient is a sum of products of values that were rounded to bf16 two or three times on the way back)
+    assert relerr(got.grad, want.grad, atol_rms=5e-2) <= 3e-2, name
 
 
 # ---------------------------------------------------------------- graph replay

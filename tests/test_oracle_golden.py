@@ -461,3 +461,187 @@ def test_hash_routing_is_a_table_lookup():
   np.testing.assert_allclose(w, [[2 * 0.4 / 0.5, 2 * 0.1 / 0.5], [2 * 0.2 / 0.3, 2 * 0.1 / 0.3]], rtol=1e-6)
   w2, _ = O.hash_routing(scores, table, np.array([2, 1]), routed_score_func="", routed_scaling_factor=1.0)
   np.testing.assert_allclose(w2, [[0.4, 0.1], [0.2, 0.1]], rtol=1e-7)
+
+
+# ---- the in-tree quantisers (gmm_v2's activation quantiser, manual_quantize), pinned in exact arithmetic ----
+#
+# The helpers below do IEEE arithmetic with python Fractions: every operation is carried out exactly and then
+# rounded (nearest, ties to even) to a significand of `p` bits (24 = float32, 8 = bfloat16).  They share no code
+# with the oracle (no torch, no numpy float types).
+
+
+def _rne(x, p):
+  from fractions import Fraction
+
+  x = Fraction(x)
+  if x == 0:
+    return x
+  sign = -1 if x < 0 else 1
+  a = abs(x)
+  e = 0
+  while a >= 2:
+    a /= 2
+    e += 1
+  while a < 1:
+    a *= 2
+    e -= 1
+  scaled = a * 2 ** (p - 1)  # in [2^(p-1), 2^p)
+  n = int(scaled)  # floor
+  rem = scaled - n
+  if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+    n += 1
+  return sign * Fraction(n, 2 ** (p - 1)) * Fraction(2) ** e
+
+
+def _op(x, dt):
+  """One JAX op whose result has dtype dt: float32 rounds once; bfloat16 is carried in float32 and rounded again."""
+  return _rne(x, 24) if dt == "f32" else _rne(_rne(x, 24), 8)
+
+
+def _trunc(x):
+  return int(x) if x >= 0 else -int(-x)
+
+
+def _v2_int8_row(row, dt):
+  """pallas_mosaic_tpu_v2_gmm_kernel.py:533-542 on one row (= one quant block) with Fractions."""
+  from fractions import Fraction
+
+  row = [Fraction(v) for v in row]
+  amax = max(abs(v) for v in row)
+  scale = _op(amax / 127, dt)
+  inv = Fraction(0) if scale == 0 else _op(1 / scale, dt)
+  return [_trunc(_op(v * inv, dt)) for v in row], scale
+
+
+def _bf16_exact(vals):
+  t = torch.tensor(vals, dtype=torch.float32)
+  assert torch.equal(t, t.to(torch.bfloat16).float()), "test inputs must be exact in bf16"
+  return t
+
+
+def test_v2_quantiser_int8_matches_exact_arithmetic():
+  # rows chosen so that the rule's ingredients matter: fractions of the scale, negative values, an all-zero row
+  rows = [[1.0, 0.703125, -0.5, 0.25, 0.00390625, -0.99609375, 0.33203125, 0.66796875],
+          [1.5, -1.4921875, 0.75, 0.375, 0.01171875, 1.0, -0.1875, 0.5],
+          [3.0, 2.984375, -2.96875, 1.0, 0.5, 0.25, -3.0, 0.0234375],
+          [0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0],
+          [100.0, 99.5, -37.25, 12.125, 0.78125, -100.0, 50.0, 25.0]]
+  for dt, tdt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+    x = _bf16_exact(rows).to(tdt)
+    q, s = O.quantize_lhs_v2(x, torch.int8, quant_block=8)
+    for r, row in enumerate(rows):
+      want_q, want_s = _v2_int8_row(row, dt)
+      assert q[r].tolist() == want_q, (dt, r)
+      assert float(s[r, 0]) == float(want_s), (dt, r)
+  # zero row: scale 0, inverse forced to 0 (:537-540), q = 0
+  assert q[3].abs().max() == 0 and float(s[3, 0]) == 0.0
+
+
+def test_v2_quantiser_hand_cases_separate_the_alternatives():
+  from fractions import Fraction as F
+
+  # (1) truncation vs rounding.  f32 row [1, 0.703125]: scale = f32(1/127), inv = f32(1/scale) = 127 exactly
+  #     (1/127 rounds to 0x3C010204 = 0.007874015718698502; its reciprocal is 127.0000000486, which rounds to 127),
+  #     0.703125 * 127 = 89.296875 -> truncation gives 89, and 0.99609375 * 127 = 126.50390625 -> 126 (rounding: 127).
+  x = torch.tensor([[1.0, 0.703125, 0.99609375, -0.99609375]], dtype=torch.float32)
+  q, s = O.quantize_lhs_v2(x, torch.int8, quant_block=4)
+  assert float(s[0, 0]) == float(_rne(F(1, 127), 24)) == 0.007874015718698502
+  assert q[0].tolist() == [127, 89, 126, -126]
+  assert torch.round(x * 127.0)[0].tolist() == [127.0, 89.0, 127.0, -127.0]  # what any rounding rule would give
+  # (2) half-even vs half-away cannot be told apart once truncation is in place; the product rule (rint) is pinned
+  #     separately in test_quantisers_closed_form.  What can be told apart is x * (1/scale) from x / scale:
+  #     bf16 row with absmax 1.5: scale = bf16(f32(1.5/127)) = 0.0118408203125 (1.515625 * 2^-7),
+  #     inv = bf16(84.4536...) = 84.5; 1.4921875 * 84.5 = 126.08984375 -> bf16 126.0 -> 126, while
+  #     1.4921875 / 0.0118408203125 = 126.02 -> 126 too, but 0.75 * 84.5 = 63.375 -> bf16 63.5 -> 63 against
+  #     0.75 / scale = 63.34 -> bf16 63.25 -> 63; the separating element is 1.5 itself:
+  #     1.5 * 84.5 = 126.75 -> bf16 (tie between 126.5 and 127.0, even significand) 127.0 -> 127, and
+  #     1.5 / scale = 126.68 -> bf16 126.5 -> 126.
+  xb = torch.tensor([[1.5, 1.4921875, 0.75]], dtype=torch.bfloat16)
+  q, s = O.quantize_lhs_v2(xb, torch.int8, quant_block=3)
+  assert float(s[0, 0]) == 0.0118408203125
+  assert q[0].tolist() == [127, 126, 63]
+  div = [_trunc(_op(F(v) / F(0.0118408203125), "bf16")) for v in (1.5, 1.4921875, 0.75)]
+  assert div == [126, 126, 63]  # the x / scale rule differs on the first element
+  # (3) bf16 vs f32 intermediate arithmetic: the same values as f32 input give scale = f32(1.5/127) and
+  #     inv = f32(84.666...): 1.4921875 * inv = 126.338... -> 126, 0.75 * inv = 63.4999... -> 63, 1.5 * inv -> 126 or 127
+  q32, s32 = O.quantize_lhs_v2(xb.float(), torch.int8, quant_block=3)
+  assert float(s32[0, 0]) == float(_rne(F(3, 2) / 127, 24)) != float(s[0, 0])
+  assert q32[0].tolist() == _v2_int8_row([1.5, 1.4921875, 0.75], "f32")[0]
+  # (4) per-block scales: two blocks of one row are quantised independently
+  x2 = torch.tensor([[1.0, 0.5, 8.0, 4.0]], dtype=torch.bfloat16)
+  q, s = O.quantize_lhs_v2(x2, torch.int8, quant_block=2)
+  assert s.shape == (1, 2) and q[0].tolist() == _v2_int8_row([1.0, 0.5], "bf16")[0] + _v2_int8_row([8.0, 4.0], "bf16")[0]
+
+
+def test_v2_quantiser_fp8_and_static_scale():
+  from fractions import Fraction as F
+
+  # e4m3fn grid near the top: 448 = max, spacing 32 above 256, 16 in [128, 256)
+  # dynamic, f32 row [448, 300, 17, -1.0625]: scale = 1, inv = 1 -> q = RNE to e4m3: 448, 288|320 -> 300 is 288 + 12 -> 288,
+  # 17 -> 16|18 (spacing 2 in [16,32)) tie -> even significand: 16 = 1.000b * 2^4, 18 = 1.001b * 2^4 -> 16;
+  # -1.0625 -> spacing 0.125 in [1,2): tie between -1.0 and -1.125 -> -1.0
+  x = torch.tensor([[448.0, 300.0, 17.0, -1.0625]], dtype=torch.float32)
+  q, s = O.quantize_lhs_v2(x, torch.float8_e4m3fn, quant_block=4)
+  assert float(s[0, 0]) == 1.0 and q[0].float().tolist() == [448.0, 288.0, 16.0, -1.0]
+  # static scale of tests/integration/tokamax_test.py:113-114 ("fixed,-224,224" -> 0.5, quantizations_test.py:723):
+  # inv = 2 exactly, values beyond +-224 are clipped to +-448 BEFORE the cast (no NaN), :531
+  st = O.get_static_scale(448.0, "fixed,-224,224")
+  x = torch.tensor([[1.0, 223.0, 224.0, 300.0, -1000.0, 0.51171875]], dtype=torch.bfloat16)
+  q, s = O.quantize_lhs_v2(x, torch.float8_e4m3fn, static_scale=st)
+  assert s.shape == (1, 1) and float(s) == 0.5
+  # 1.0234375 -> e4m3 spacing 0.125 in [1, 2) -> 1.0
+  assert q[0].float().tolist() == [2.0, 448.0, 448.0, 448.0, -448.0, 1.0]
+  # a static int8 scale that is not a power of two: "fixed,3" -> 3/127; bf16(3/127) = 0.0236816..., inverse in bf16
+  st = O.get_static_scale(127.0, "fixed,3")
+  sb = _op(F(st), "bf16")
+  inv = _op(1 / sb, "bf16")
+  vals = [3.0, 2.984375, -1.0, 0.01171875, 10.0, -10.0]
+  q, s = O.quantize_lhs_v2(_bf16_exact([vals]).to(torch.bfloat16), torch.int8, static_scale=st)
+  want = [_trunc(max(F(-127), min(F(127), _op(F(v) * inv, "bf16")))) for v in vals]
+  assert q[0].tolist() == want and float(s) == float(sb)
+  assert want[4] == 127 and want[5] == -127  # clipped, then cast
+  # with an f32 accumulator dtype the inverse and the product are f32 (promotion of bf16 * f32)
+  q32, s32 = O.quantize_lhs_v2(_bf16_exact([vals]).to(torch.bfloat16), torch.int8, static_scale=st, acc_dtype=torch.float32)
+  inv32 = _op(1 / _op(F(st), "f32"), "f32")
+  assert q32[0].tolist() == [_trunc(max(F(-127), min(F(127), _op(F(v) * inv32, "f32")))) for v in vals]
+
+
+def test_manual_quantize_matches_exact_arithmetic():
+  from fractions import Fraction as F
+
+  # layers/quantizations.py:961-991 with "fixed,-224,224" (scale 0.5, exact in bf16): q = clip(w / 0.5).astype(e4m3)
+  w = torch.tensor([[0.25, -0.28125, 300.0, 1.0625]], dtype=torch.bfloat16)
+  q, s = O.manual_quantize(w, torch.float8_e4m3fn, "fixed,-224,224")
+  assert float(s) == 0.5 and q[0].float().tolist() == [0.5, -0.5625, 448.0, 2.0]  # 2.125 -> tie 2.0|2.25 -> 2.0
+  # a scale that bf16 cannot hold: "fixed,3" for int8: the division uses the bf16-rounded scale tensor
+  wv = [3.0, -2.984375, 1.0, 0.01171875]
+  q, s = O.manual_quantize(_bf16_exact([wv]).to(torch.bfloat16), torch.int8, "fixed,3")
+  sb = _op(F(3, 127), "bf16")
+  assert q[0].tolist() == [_trunc(max(F(-127), min(F(127), _op(F(v) / sb, "bf16")))) for v in wv]
+  assert float(s) == float(sb)
+
+
+def test_gmm_with_v2_scale_layouts_equals_dequantised_matmul():
+  # lhs scales per row per 512-block (in-kernel quantiser), rhs scales [g, nb, 1, n] with another block size, a scale
+  # shared by all experts ([1, 1, 1, n], ops.py:250-260) and a static [1, 1] lhs scale: all equal the plain matmul of the
+  # dequantised operands, group by group
+  g0 = torch.Generator().manual_seed(11)
+  m, k, n, g = 24, 1024, 16, 3
+  gs = np.array([7, 0, 17], np.int32)
+  lq = torch.randint(-127, 128, (m, k), generator=g0).to(torch.int8)
+  rq = torch.randint(-127, 128, (g, k, n), generator=g0).to(torch.int8)
+  ls = torch.rand((m, 2), generator=g0) + 0.5
+  rs = torch.rand((g, 4, 1, n), generator=g0) + 0.5
+  ld = lq.double() * torch.repeat_interleave(ls.double(), 512, dim=1)
+  rd = rq.double() * torch.repeat_interleave(rs[:, :, 0, :].double(), 256, dim=1)
+  want = torch.zeros((m, n), dtype=torch.float64)
+  want[:7] = ld[:7] @ rd[0]
+  want[7:] = ld[7:] @ rd[2]
+  got = O.gmm(lq, rq, gs, lhs_scale=ls, rhs_scale=rs, quant_block=(512, 256), out_dtype=torch.float64)
+  torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-9)
+  shared = rs[:1, :1]
+  got = O.gmm(lq, rq, gs, lhs_scale=torch.tensor([[0.25]]), rhs_scale=shared, out_dtype=torch.float64)
+  want = torch.zeros((m, n), dtype=torch.float64)
+  want[:7] = lq[:7].double() @ rq[0].double()
+  want[7:] = lq[7:].double() @ rq[2].double()
+  torch.testing.assert_close(got, want * 0.25 * shared[0, 0].double(), rtol=1e-12, atol=1e-9)
