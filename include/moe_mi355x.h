@@ -283,7 +283,20 @@ MOE_API int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total);
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
 MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);
 
-/* Per-device set-up, for the device that is current: the CU count and the raised LDS limit of every kernel.  Optional: each entry point does its share on first use.  No counterpart in the reference. */
+/* moe_gmm for callers that cannot allocate device memory for the workspace (code under HIP graph capture, serving
+ * loops and harnesses that forbid hipMalloc): no counterpart in the reference.  args->workspace / workspace_bytes are
+ * ignored; the m-tile list goes into an array the library holds in device memory (one per GPU, 1 MiB =
+ * moe_gmm_static_ws_capacity(), kept until the process ends).  The call allocates nothing.  Requests whose tile list
+ * does not fit (moe_gmm_workspace_bytes(M, num_groups_total) above the capacity: about a million rows) return
+ * MOE_ERR_WORKSPACE.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls in stream order are safe, because each call rewrites the part of the list it reads.
+ * The first call on a device looks the array's address up and raises the LDS limit of the kernel it launches;
+ * moe_init() does both ahead of time for every kernel. */
+MOE_API size_t moe_gmm_static_ws_capacity(void);
+MOE_API int moe_gmm_static_ws(const moe_gmm_args* args, void* stream);
+
+/* Per-device set-up, for the device that is current: the CU count, the address of the static workspace and the raised
+ * LDS limit of every kernel.  Optional: each entry point does its share on first use.  No counterpart in the reference. */
 MOE_API int moe_init(void);
 
 /* moe_gmm with the kernel family and the tile raster chosen by the caller instead of by the shape: a tuning and test

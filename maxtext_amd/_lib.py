@@ -89,6 +89,8 @@ SIGNATURES = {
     "moe_gmm_rhs_kn_supported": (c_int, [c_int, c_int, c_int, c_int]),
     "moe_gmm": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
     "moe_gmm_tuned": (c_int, [ctypes.POINTER(GmmArgs), c_int, c_int, c_void_p]),
+    "moe_gmm_static_ws": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
+    "moe_gmm_static_ws_capacity": (c_size_t, []),
     "moe_init": (c_int, []),
     "moe_tgmm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moe_calib_scratch_bytes": (c_size_t, []),

@@ -102,6 +102,12 @@ __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
   if (tid == 0) header[0] = total_tiles + tail;
 }
 
+// Tile list of moe_gmm_static_ws: one array per device, held until the process ends.  Its name is a host-side handle,
+// not a device address: the address is looked up once per device (scratch_of) and passed to the kernels like any
+// caller-supplied workspace.
+constexpr size_t kStaticWsBytes = 1u << 20;
+static __device__ __align__(256) uint8_t g_static_ws[kStaticWsBytes];
+
 int current_device(int* dev) {
   if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= kMaxDevices) return fail(MOE_ERR_LAUNCH, "gmm: cannot identify the current device");
   return MOE_OK;
@@ -118,6 +124,20 @@ int device_cu_count(int* cus) {
     cus_of[dev] = n;
   }
   *cus = cus_of[dev];
+  return MOE_OK;
+}
+
+static int scratch_of(void** ptr) {
+  static void* ptr_of[kMaxDevices] = {};
+  int dev = 0;
+  if (int st = current_device(&dev)) return st;
+  if (!ptr_of[dev]) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_ws));
+    if (e != hipSuccess || !p) return fail(MOE_ERR_LAUNCH, "gmm: cannot locate the static workspace: %s", hipGetErrorString(e));
+    ptr_of[dev] = p;
+  }
+  *ptr = ptr_of[dev];
   return MOE_OK;
 }
 
@@ -445,9 +465,23 @@ int moe_gmm(const moe_gmm_args* a, void* stream) {
   return gmm_impl(a, a->workspace, a->workspace_bytes, MOE_GMM_KERNEL_AUTO, 0, stream);
 }
 
+size_t moe_gmm_static_ws_capacity(void) { return kStaticWsBytes; }
+
+int moe_gmm_static_ws(const moe_gmm_args* a, void* stream) {
+  if (!a) return fail(MOE_ERR_INVALID_ARG, "gmm: NULL args");
+  if (a->M < 0 || a->num_groups_total <= 0 || moe_gmm_workspace_bytes(a->M, a->num_groups_total) > kStaticWsBytes)
+    return fail(MOE_ERR_WORKSPACE, "gmm: M = %d rows in %d groups need a tile list of more than the %zu bytes of the static workspace", a->M,
+                a->num_groups_total, kStaticWsBytes);
+  void* ws = nullptr;
+  if (int st = scratch_of(&ws)) return st;
+  return gmm_impl(a, ws, kStaticWsBytes, MOE_GMM_KERNEL_AUTO, 0, stream);
+}
+
 int moe_init(void) {
   int cus = 0;
+  void* ws = nullptr;
   if (int st = device_cu_count(&cus)) return st;
+  if (int st = scratch_of(&ws)) return st;
   if (int st = prepare_tiled()) return st;
   if (int st = prepare_dl()) return st;
   return prepare_fp8();
