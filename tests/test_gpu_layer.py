@@ -69,10 +69,12 @@ CASES = {
     "c2_small": lambda: _small("c2", 1024, emb_dim=1024, moe_mlp_dim=2048),
     "c3_small": lambda: _small("c3", 64, emb_dim=1024, moe_mlp_dim=512, num_experts=32),
     "c4_small": lambda: _small("c4", 2048, emb_dim=512, moe_mlp_dim=256),
-    "c5_t1": lambda: _small("c5", 1, num_experts=8),
-    "c5_t16": lambda: _small("c5", 16, num_experts=8),
-    "c5_t128": lambda: _small("c5", 128, num_experts=8),
-    "c5_t1024": lambda: _small("c5", 1024, num_experts=4, moe_mlp_dim=1024),
+    # the GPT-OSS shape at its full dimensions (32 experts, d = f = 2880) over the token sweep; 4096 tokens run in
+    # tests/test_gpu_fullsize.py
+    "c5_t1": lambda: _small("c5", 1),
+    "c5_t16": lambda: _small("c5", 16),
+    "c5_t128": lambda: _small("c5", 128),
+    "c5_t1024": lambda: _small("c5", 1024),
     "c5mx_t16": lambda: _small("c5mx", 16, num_experts=8),
     "c5mx_t1024": lambda: _small("c5mx", 1024, num_experts=4, moe_mlp_dim=1024),
 }
