@@ -143,9 +143,9 @@ static int scratch_of(void** ptr) {
 
 // Which kernel family takes a shape (rows per expert on average decide the m-tile) and its m-tile: one decision for the
 // tile map and for the launch.
-enum TiledKind { K_T64, K_T128, K_T256, K_DL128, K_DL64 };
+enum TiledKind { K_T64, K_T128, K_T256, K_DL128, K_DL64, K_DLW };
 
-static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N, int G_total) {
+static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N, int G_total, bool wq_kmajor = false) {
   // full 256-row tiles for prefill, 64 otherwise; a problem with fewer 256 x 256 tiles than half the CUs of the chip also
   // takes the 64-row tiles, which quadruples its blocks
   const long long tiles_big = (long long)max_tiles_for(M, G_total, 256) * cdiv(N, glu ? 128 : 256);
@@ -156,9 +156,13 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // from 32 rows per expert on (one weight conversion / tile fetch serves twice the rows), and 256-row tiles would be
   // half empty; below 32 rows per expert the 64-row tiles stay.
   const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
-  const bool mid_wq = bsrc != BSRC_SAME && (long long)M >= 32LL * G_total && (long long)M < 200LL * G_total;
+  // weight-only formats on shapes their direct-to-LDS kernel does not take (K % 64 != 0, K-major scales) stay on the
+  // register-staged kernel, whose 128-row tiles are ahead of its 256-row tiles up to 200 rows per expert
+  const bool dlw_ok = bsrc != BSRC_SAME && K % 64 == 0 && !wq_kmajor;
+  const bool mid_wq = bsrc != BSRC_SAME && !dlw_ok && (long long)M >= 32LL * G_total && (long long)M < 200LL * G_total;
   const int esz = op == OP_I8 ? 1 : 2;
   if (mid || mid_wq) return K_T128;
+  if (big && dlw_ok) return K_DLW;
   // operands that need no conversion stream straight into LDS when every stage is a full row slice
   if (big && bsrc == BSRC_SAME && (K * esz) % 128 == 0) return K_DL128;
   if (big && bsrc == BSRC_SAME && (K * esz) % 64 == 0) return K_DL64;
@@ -166,11 +170,12 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   return K_T64;
 }
 
-static int tiled_kind_bm(TiledKind k) { return k == K_T64 ? 64 : k == K_T128 ? 128 : 256; }
+static int tiled_kind_bm(TiledKind k) { return k == K_T64 ? 64 : k == K_T128 ? 128 : 256; }  // (every direct-to-LDS kernel: 256)
 
 static int launch_tiled_kind(TiledKind kind, int op, int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
   if (kind == K_DL128) return launch_dl(op, glu, 128, false, p, M, G_total, s);
   if (kind == K_DL64) return launch_dl(op, glu, 64, false, p, M, G_total, s);
+  if (kind == K_DLW) return launch_dlw(bsrc, glu, p, M, G_total, s);
   return launch_tiled_bm(op, bsrc, glu, tiled_kind_bm(kind), false, p, M, G_total, s);
 }
 
@@ -454,8 +459,8 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     map_tiles(256);
     return launch_dl(op, glu, 64, false, p, M, G, s);
   }
-  TiledKind kind = kernel == MOE_GMM_KERNEL_BIG ? K_T256 : pick_tiled_kind(op, bsrc, glu, M, K, N, G);
-  if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64)) kind = K_T256;
+  TiledKind kind = kernel == MOE_GMM_KERNEL_BIG ? K_T256 : pick_tiled_kind(op, bsrc, glu, M, K, N, G, wq_kmajor);
+  if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64 || kind == K_DLW)) kind = K_T256;
   map_tiles(tiled_kind_bm(kind));
   return launch_tiled_kind(kind, op, bsrc, glu, p, M, G, s);
 }
@@ -484,6 +489,7 @@ int moe_init(void) {
   if (int st = scratch_of(&ws)) return st;
   if (int st = prepare_tiled()) return st;
   if (int st = prepare_dl()) return st;
+  if (int st = prepare_dlw()) return st;
   return prepare_fp8();
 }
 

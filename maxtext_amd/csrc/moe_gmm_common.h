@@ -38,6 +38,19 @@ __device__ __forceinline__ int lhs_row_of(const RowOpts& o, int r) {
   return min(max(s, 0), o.lhs_rows - 1);
 }
 
+// The same for a batch of rows: one uniform branch, the index loads issued back to back (a branch per row would put a
+// full memory round trip between consecutive loads).
+template <int NR>
+__device__ __forceinline__ void lhs_rows_of(const RowOpts& o, int (&r)[NR]) {
+  if (o.row_idx) {
+    int s[NR];
+#pragma unroll
+    for (int i = 0; i < NR; i++) s[i] = o.row_idx[r[i]];
+#pragma unroll
+    for (int i = 0; i < NR; i++) r[i] = min(max(s[i] / o.idx_div, 0), o.lhs_rows - 1);
+  }
+}
+
 // Four consecutive output values of one row: multiplied by the row's factor, then stored as bf16 (8 bytes) or f32.
 __device__ __forceinline__ void store_out4(void* out, const RowOpts& o, size_t row, int N, int n, float (&v)[4]) {
   if (o.row_scale) {
@@ -45,10 +58,11 @@ __device__ __forceinline__ void store_out4(void* out, const RowOpts& o, size_t r
 #pragma unroll
     for (int r = 0; r < 4; r++) v[r] *= w;
   }
-  if (o.out_f32)
+  if (o.out_f32) {
     *(float4*)((float*)out + row * N + n) = make_float4(v[0], v[1], v[2], v[3]);
-  else
+  } else {
     *(uint2*)((uint16_t*)out + row * N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+  }
 }
 
 // Zeros for the `width` channels from n0 on of a tile's rows (rows of no local group).
@@ -144,70 +158,122 @@ struct EpilogueScales {
 template <int TM, int NT_OUT, bool GLU, bool CHANNEL_SCALES, int MI = 32>
 __device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, GLU>& e, const TiledParams& p, const TileInfo& tile,
                                                      int row_base, int n_base, int lane) {
+  // every decision is uniform and taken once, so that the loads of a kind go out back to back
   const float4 one = make_float4(1.f, 1.f, 1.f, 1.f);
 #pragma unroll
-  for (int i = 0; i < TM; i++) {
-    const int lr = row_base + i * MI + (lane % MI);
-    e.sa[i] = p.lhs_scale ? p.lhs_scale[(size_t)lhs_row_of(p.ro, tile.row0 + (lr < tile.nrows ? lr : 0)) * p.lhs_scale_stride] : 1.0f;
+  for (int i = 0; i < TM; i++) e.sa[i] = 1.0f;
+  if (p.lhs_scale) {
+    int rows[TM];
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int lr = row_base + i * MI + (lane % MI);
+      rows[i] = tile.row0 + (lr < tile.nrows ? lr : 0);
+    }
+    lhs_rows_of<TM>(p.ro, rows);
+#pragma unroll
+    for (int i = 0; i < TM; i++) e.sa[i] = p.lhs_scale[(size_t)rows[i] * p.lhs_scale_stride];
   }
 #pragma unroll
   for (int j = 0; j < NT_OUT; j++)
 #pragma unroll
     for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
-      const int n = n_base + epilogue_channel<MI>(j, q, lane);
       e.sg[j][q] = one;
       e.su[j][q] = one;
-      if (CHANNEL_SCALES && p.rhs_scale && !p.wq_kmajor && n < p.N) {  // (K-major block scales went in with the weights)
-        const float* sg = (const float*)p.rhs_scale + (size_t)tile.group * p.rhs_scale_gstride;
-        const float* su = GLU ? (const float*)p.rhs_up_scale + (size_t)tile.group * p.rhs_scale_gstride : nullptr;
-        if (p.rhs_scale_nstride) {
+    }
+  if (CHANNEL_SCALES && p.rhs_scale && !p.wq_kmajor) {  // (K-major block scales went in with the weights)
+    const float* sg = (const float*)p.rhs_scale + (size_t)tile.group * p.rhs_scale_gstride;
+    const float* su = GLU ? (const float*)p.rhs_up_scale + (size_t)tile.group * p.rhs_scale_gstride : nullptr;
+    if (p.rhs_scale_nstride) {
+#pragma unroll
+      for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+        for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+          // channels past N (the last n-tile of a ragged N) read the scales of channel N - 4: they are never stored
+          const int n = min(n_base + epilogue_channel<MI>(j, q, lane), p.N - 4);
           e.sg[j][q] = *(const float4*)(sg + n);
           if (GLU) e.su[j][q] = *(const float4*)(su + n);
-        } else {
-          e.sg[j][q] = make_float4(sg[0], sg[0], sg[0], sg[0]);
-          if (GLU) e.su[j][q] = make_float4(su[0], su[0], su[0], su[0]);
         }
-      }
+    } else {
+      const float g1 = sg[0], u1 = GLU ? su[0] : 1.0f;
+#pragma unroll
+      for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+        for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+          e.sg[j][q] = make_float4(g1, g1, g1, g1);
+          e.su[j][q] = make_float4(u1, u1, u1, u1);
+        }
     }
+  }
 }
 
+// Writes a wave's results.  The MFMA leaves lane l with 4 consecutive channels of row l % MI: 8-byte stores, neighbouring
+// lanes in different rows.  (Passing each row tile through LDS so that consecutive lanes store consecutive 16 bytes was
+// measured and is slower: the epilogue is bound by what stands between the stores, not by the stores.)
 template <int TM, int TN, int NT_OUT, bool GLU, typename acc_t>
 __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
                                                const TiledParams& p, const TileInfo& tile, int row_base, int n_base, int lane) {
   constexpr int MI = sizeof(acc_t) == 16 ? 16 : 32;  // 4 accumulator registers per tile: the 16 x 16 instructions
-  dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
-  constexpr int ACT = decltype(act_c)::value;
+  // Everything that needs a load is decided and loaded up front, by uniform branches, and the variants of the body are
+  // separate straight-line instantiations: a branch or a load between two stores makes the compiler wait for ALL memory
+  // operations in flight, the stores included, i.e. one memory round trip per store (measured on 256 x 256 tiles: 18 us
+  // per tile, as much as ten K stages, against 6 us now).
+  float rw[TM];
 #pragma unroll
-  for (int i = 0; i < TM; i++) {
-    const int lr = row_base + i * MI + (lane % MI);
-    if (lr >= tile.nrows) continue;
+  for (int i = 0; i < TM; i++) rw[i] = 1.0f;
+  if (p.ro.row_scale) {
 #pragma unroll
-    for (int j = 0; j < NT_OUT; j++)
+    for (int i = 0; i < TM; i++) {
+      const int lr = row_base + i * MI + (lane % MI);
+      rw[i] = p.ro.row_scale[tile.row0 + (lr < tile.nrows ? lr : 0)];
+    }
+  }
+  // GENERAL: bias, partial sums, f32 output; otherwise bf16 results straight to memory
+  auto body = [&](auto act_c, auto general_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    constexpr bool GENERAL = decltype(general_c)::value;
 #pragma unroll
-      for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
-        const int n = n_base + epilogue_channel<MI>(j, q, lane);
-        if (n >= p.N) continue;
-        const float sg[4] = {e.sg[j][q].x, e.sg[j][q].y, e.sg[j][q].z, e.sg[j][q].w};
-        const float su[4] = {e.su[j][q].x, e.su[j][q].y, e.su[j][q].z, e.su[j][q].w};
-        float bg[4], bu[4];
-        load_bias4(p.rhs_bias, tile.group, p.N, n, bg);
-        load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, p.N, n, bu);
-        add_partial4(p.partial_sum, (size_t)(tile.row0 + lr), p.N, n, bg);
-        add_partial4(GLU ? p.partial_sum_up : nullptr, (size_t)(tile.row0 + lr), p.N, n, bu);
-        float v[4];
+    for (int i = 0; i < TM; i++) {
+      const int lr = row_base + i * MI + (lane % MI);
+      const bool row_ok = lr < tile.nrows;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const float g = fmaf((float)acc[j][i][4 * q + r], e.sa[i] * sg[r], bg[r]);
-          if (GLU) {
-            const float u = fmaf((float)acc[j + NT_OUT][i][4 * q + r], e.sa[i] * su[r], bu[r]);
-            v[r] = glu_act<ACT>(g, u, p.act_limit);
-          } else {
-            v[r] = g;
+      for (int j = 0; j < NT_OUT; j++)
+#pragma unroll
+        for (int q = 0; q < (MI == 32 ? 4 : 1); q++) {
+          const int n = n_base + epilogue_channel<MI>(j, q, lane);
+          const bool ok = row_ok && n < p.N;
+          const float sg[4] = {e.sg[j][q].x, e.sg[j][q].y, e.sg[j][q].z, e.sg[j][q].w};
+          const float su[4] = {e.su[j][q].x, e.su[j][q].y, e.su[j][q].z, e.su[j][q].w};
+          float bg[4] = {0.f, 0.f, 0.f, 0.f}, bu[4] = {0.f, 0.f, 0.f, 0.f};
+          if (GENERAL && ok) {
+            load_bias4(p.rhs_bias, tile.group, p.N, n, bg);
+            load_bias4(GLU ? p.rhs_up_bias : nullptr, tile.group, p.N, n, bu);
+            add_partial4(p.partial_sum, (size_t)(tile.row0 + lr), p.N, n, bg);
+            add_partial4(GLU ? p.partial_sum_up : nullptr, (size_t)(tile.row0 + lr), p.N, n, bu);
+          }
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const float g = fmaf((float)acc[j][i][4 * q + r], e.sa[i] * sg[r], bg[r]);
+            if (GLU) {
+              const float u = fmaf((float)acc[j + NT_OUT][i][4 * q + r], e.sa[i] * su[r], bu[r]);
+              v[r] = glu_act<ACT>(g, u, p.act_limit) * rw[i];
+            } else {
+              v[r] = g * rw[i];
+            }
+          }
+          if (ok) {
+            if (GENERAL && p.ro.out_f32)
+              *(float4*)((float*)p.out + (size_t)(tile.row0 + lr) * p.N + n) = make_float4(v[0], v[1], v[2], v[3]);
+            else
+              *(uint2*)((uint16_t*)p.out + (size_t)(tile.row0 + lr) * p.N + n) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
           }
         }
-        store_out4(p.out, p.ro, (size_t)(tile.row0 + lr), p.N, n, v);
-      }
-  }
+    }
+  };
+  const bool general = p.rhs_bias || p.rhs_up_bias || p.partial_sum || p.partial_sum_up || p.ro.out_f32;
+  dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
+    if (general) body(act_c, std::true_type{});
+    else body(act_c, std::false_type{});
   });
 }
 
@@ -327,6 +393,7 @@ static bool (&lds_flags())[kMaxDevices] {
 int prepare_tiled();
 int prepare_dl();
 int prepare_fp8();
+int prepare_dlw();
 
 // ---- launchers (one translation unit per kernel family) ----
 // moe_gmm_tiled.hip: register-staged kernel, m-tile bm in {64, 128, 256}; block_scaled: int8 x int8 / fp8 x fp8 with K-block
@@ -334,6 +401,8 @@ int prepare_fp8();
 int launch_tiled_bm(int op, int bsrc, bool glu, int bm, bool block_scaled, const TiledParams& p, int M, int G_total, hipStream_t s);
 // moe_gmm_dl.hip: direct-to-LDS persistent kernel, 256 x 256 tiles; stage_bytes 128 or 64; rhs_kn: [G, K, N] bf16 weights
 int launch_dl(int op, bool glu, int stage_bytes, bool rhs_kn, const TiledParams& p, int M, int G_total, hipStream_t s);
+// moe_gmm_dlw.hip: the same pipeline for bf16 activations x int8 / int4 / mxfp4 weights (K % 64 == 0, default scale layouts)
+int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
 // moe_gmm_fp8.hip
 int launch_fp8_tiled(bool big, bool glu, bool vec4, const Fp8TiledParams& P, int M, int G_total, hipStream_t s);
 int launch_fp8_skinny(bool few_rows, const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s);

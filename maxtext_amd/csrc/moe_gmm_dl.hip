@@ -77,8 +77,13 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     const int gsz = min(p.max_m_tiles - first_m, GSM);
     const int m_idx = first_m + (logical % width) % gsz;
     if (m_idx >= num_tiles) return false;
-    t.info = p.tiles[m_idx];
-    t.n0 = ((logical % width) / gsz) * C::OUT_BN;
+    // (uniform values: kept in scalar registers, so that a tile looked up ahead of time costs no vector registers)
+    const TileInfo ti = p.tiles[m_idx];
+    t.info.group = __builtin_amdgcn_readfirstlane(ti.group);
+    t.info.row0 = __builtin_amdgcn_readfirstlane(ti.row0);
+    t.info.nrows = __builtin_amdgcn_readfirstlane(ti.nrows);
+    t.info.pad = 0;
+    t.n0 = __builtin_amdgcn_readfirstlane(((logical % width) / gsz) * C::OUT_BN);
     return true;
   };
   // Advances `id` to this block's next tile that needs the matmul; tiles of rows that belong to no local
@@ -96,11 +101,15 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   const uint8_t* a_src[C::A_IPW];
   const uint8_t* b_src[C::B_IPW];
   auto set_sources = [&](const Tile& t) {
+    int a_rows[C::A_IPW];
+#pragma unroll
+    for (int i = 0; i < C::A_IPW; i++) a_rows[i] = t.info.row0 + min((wave * C::A_IPW + i) * C::RPI + lane / C::CPR, t.info.nrows - 1);
+    lhs_rows_of<C::A_IPW>(p.ro, a_rows);
 #pragma unroll
     for (int i = 0; i < C::A_IPW; i++) {
       const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
       const int q = (lane % C::CPR) ^ C::swz(r);
-      a_src[i] = p.lhs + (size_t)lhs_row_of(p.ro, t.info.row0 + min(r, t.info.nrows - 1)) * row_bytes + q * 16;
+      a_src[i] = p.lhs + (size_t)a_rows[i] * row_bytes + q * 16;
     }
 #pragma unroll
     for (int i = 0; i < C::B_IPW; i++) {
@@ -350,16 +359,20 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     }
     // all LDS reads of this tile are done in every wave and no request is still writing LDS: the buffers
     // can take the next tile's first stages
+    // The results are stored before anything of the next tile is looked up: the accumulators are then dead across the
+    // tile-boundary code.  (Requesting the next tile's first stages ahead of the stores, with the tile looked up before the
+    // main loop, was measured 3 % slower: any code between the last k-step and the stores makes the compiler push
+    // accumulators out to scratch memory and reload them between the stores, one memory round trip each.)
+    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, cur.info, wm * C::WM, n_out0, lane);
+    // all LDS reads of this tile are done in every wave and no request is still writing LDS: the buffers can take the next tile
     wait_vmcnt<0>();
     asm volatile("s_barrier" ::: "memory");
-    const Tile done = cur;
     id += gridDim.x;
     have = next_compute_tile(id, cur);
     if (have) {
       set_sources(cur);
       issue_prologue();
     }
-    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, done.info, wm * C::WM, n_out0, lane);
   }
   wait_vmcnt<0>();
 }

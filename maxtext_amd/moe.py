@@ -306,7 +306,9 @@ class RoutedMoE:
     return out.reshape(batch_size, sequence_length, -1)
 
   # -- the three grouped GEMMs: gmm_up + apply_ffn_activation + wo (moe.py:1932-1986, :841, :2226)
-  def _experts(self, sorted_inputs, group_size, w0, w1, wo, w0_bias=None, w1_bias=None, wo_bias=None):
+  def _experts(self, sorted_inputs, group_size, w0, w1, wo, w0_bias=None, w1_bias=None, wo_bias=None, row_idx=None, row_idx_div=1):
+    """row_idx / row_idx_div: `sorted_inputs` holds the T token rows (plain or quantised) and row i of the first product
+    reads row row_idx[i] // row_idx_div of it: the permute fused into the matmul, no [M, d] copy."""
     cfg = self.config
     act, limit = cfg.activation, (cfg.mlp_activations_limit if cfg.mlp_activations_limit > 0 else 7.0)
     ev = self.profile_events
@@ -326,7 +328,7 @@ class RoutedMoE:
                            rhs_quantize_dtype=q, rhs_bias=w0_bias, rhs_up_bias=w1_bias)
       return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q, rhs_bias=wo_bias)
     inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
-                         rhs_bias=w0_bias, rhs_up_bias=w1_bias)
+                         rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div)
     if marks:
       marks[1].record()
     if cfg.act_quant is not None:
@@ -357,18 +359,14 @@ class RoutedMoE:
                                                       want_sorted_experts=False)
     training = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (x2d, weights, w0_kernel, w1_kernel, wo_kernel))
-    # permute fused with the activation quantiser of the first GEMM
     if training:
       sorted_inputs = _GatherRowsFn.apply(x2d, perm, inv, k) if x2d.requires_grad else kernels.gather_rows(x2d, perm, k)
-    elif cfg.act_quant == "int8":
-      q, sc = kernels.gather_rows(x2d, perm, k, out_dtype=torch.int8)
-      sorted_inputs = QArray(q, sc, "int8")
-    elif cfg.act_quant == "fp8":
-      q, sc = kernels.gather_rows(x2d, perm, k, out_dtype=torch.float8_e4m3fn, block_k=128)
-      sorted_inputs = QArray(q, sc, "fp8")
+      inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias)
     else:
-      sorted_inputs = kernels.gather_rows(x2d, perm, k)
-    inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias)
+      # the permute is fused into the first grouped matmul: the T token rows are quantised once (not their M = T * k
+      # copies) and the matmul reads row perm[i] // k for its row i, so the [M, d] gathered copy is never written
+      inter = self._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias,
+                            row_idx=perm, row_idx_div=k)
     out = self.unpermute(inter, perm, weights, b, s, inv_perm=inv)
     lb_loss, bias_updates = self._aux_outputs(gate_logits, selected.reshape(b, s, k))
     return out, lb_loss, bias_updates
@@ -389,6 +387,18 @@ class RoutedMoE:
     gate_logits = gate_logits.reshape(b, s, -1)
     pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
     return self.sparse_matmul(inputs, gate_logits, pre_bias, self.wi_0, self.wi_1, self.wo, input_ids=input_ids)
+
+
+def _quantize_tokens(x2d, act_quant):
+  """The activation quantiser of the first grouped matmul on the token rows: int8 with one scale per row, or fp8 with
+  one scale per row and 128 values (the DeepSeek recipe); None leaves the bf16 rows as they are."""
+  if act_quant == "int8":
+    q, sc = kernels.gather_rows(x2d, out_dtype=torch.int8)
+    return QArray(q, sc, "int8")
+  if act_quant == "fp8":
+    q, sc = kernels.gather_rows(x2d, out_dtype=torch.float8_e4m3fn, block_k=128)
+    return QArray(q, sc, "fp8")
+  return x2d
 
 
 class RoutedAndSharedMoE:
@@ -417,15 +427,7 @@ class RoutedAndSharedMoE:
     sel = torch.cat([sel.reshape(t, k), torch.full((t, 1), e, dtype=torch.int32, device=sel.device)], 1).contiguous()
     w = torch.cat([w.reshape(t, k), torch.ones((t, 1), dtype=torch.float32, device=w.device)], 1).contiguous()
     perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + 1, want_sorted_experts=False)
-    if cfg.act_quant == "int8":
-      q, sc = kernels.gather_rows(x2d, perm, k + 1, out_dtype=torch.int8)
-      rows = QArray(q, sc, "int8")
-    elif cfg.act_quant == "fp8":
-      q, sc = kernels.gather_rows(x2d, perm, k + 1, out_dtype=torch.float8_e4m3fn, block_k=128)
-      rows = QArray(q, sc, "fp8")
-    else:
-      rows = kernels.gather_rows(x2d, perm, k + 1)
-    inter = r._experts(rows, group_size, r.wi_0, r.wi_1, r.wo)
+    inter = r._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, r.wi_0, r.wi_1, r.wo, row_idx=perm, row_idx_div=k + 1)
     out = kernels.unpermute_combine(inter, w, k=k + 1, inv_perm=inv)
     return out.reshape(b, s, d), None, None
 
