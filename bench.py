@@ -23,13 +23,53 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"int8": 5000.0, "fp8": 5000.0, "bf16": 2500.0}  # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
-# scaled by a 1 GiB copy dispatch of the same run (profiles/pmc_traffic_*.md); None where not measured.
-MEASURED_TRAFFIC_BYTES = {
-    "c2": (2590968 * 2.0 + 473766 * 1.0) * 1024,  # profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md
-    "c3": (3852849 * 2.0 + 9236 * 1.0) * 1024,  # profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md
-    "c2_train": (1376652 * 2.0 + 924637 * 1.0) * 1024,  # profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md
+# HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs that are made
+# offline and summarised in profiles/*.md.  Each summary carries two machine-readable lines,
+#   traffic_bytes_per_launch: <bytes>
+#   kernel_source_sha256: <hash of the kernel's source files when the counters were read>
+# and the figure is reported only while the sources still hash to that value: a kernel that changed since has no
+# measured traffic until its profile is refreshed.
+PROFILE_OF = {
+    "c2": ("profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md", ["moe_gmm_dl.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c3": ("profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md", ["moe_gmm_fp8.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c4": ("profiles/gmm_dlw_kernel_int8w_qwen3_prefill_c4.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c5": ("profiles/gmm_dlw_kernel_int4w_gptoss_prefill_c5_t4096.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c2_train": ("profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md", ["moe_tgmm.hip", "moe_common.h"]),
 }
+
+
+def kernel_source_hash(files):
+  import hashlib
+
+  h = hashlib.sha256()
+  for name in files:
+    with open(os.path.join(ROOT, "maxtext_amd", "csrc", name), "rb") as fh:
+      h.update(name.encode() + b"\0" + fh.read())
+  return h.hexdigest()
+
+
+def measured_traffic(key):
+  """(bytes or None, provenance) for the dominant kernel of workload `key` at its default size."""
+  import re
+
+  if key not in PROFILE_OF:
+    return None, None
+  rel, files = PROFILE_OF[key]
+  now = kernel_source_hash(files)
+  src = {"profile": rel, "kernel_sources": files, "source_sha256_now": now}
+  try:
+    with open(os.path.join(ROOT, rel)) as fh:
+      text = fh.read()
+  except OSError:
+    return None, dict(src, status="no profile for this kernel")
+  m_bytes = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
+  m_hash = re.search(r"^kernel_source_sha256:\s*([0-9a-f]{64})", text, re.M)
+  if not m_bytes or not m_hash:
+    return None, dict(src, status="profile carries no traffic figure")
+  src["source_sha256_profiled"] = m_hash.group(1)
+  if m_hash.group(1) != now:
+    return None, dict(src, status="kernel source changed since the counters were read")
+  return float(m_bytes.group(1)), dict(src, status="counters read on this kernel source")
 
 
 def parse():
@@ -37,7 +77,9 @@ def parse():
   ap.add_argument("--gpus", type=int, default=1)
   ap.add_argument("--steps", type=int, default=20)
   ap.add_argument("--warmup", type=int, default=5)
-  ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c5mx"])
+  ap.add_argument("--workload", default=None, choices=["c1", "c2", "c3", "c4", "c5", "c5mx"],
+                  help="one workload; by default c2 (the headline line) and then c3 (reported under \"secondary\")")
+  ap.add_argument("--source-hash", action="store_true", help="print the kernel source hash that a profile summary of --workload records")
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
   ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -79,8 +121,13 @@ def dominant_kernel_model(wl, group_sizes):
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name="gmm_wq_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="bf16")
   op = "int8" if cfg.act_quant == "int8" else "bf16"
+  big = rows >= 128 * len(group_sizes)  # the dispatch rule of moe_gmm for its persistent 256 x 256 kernels
+  if cfg.act_quant == "int8" or wl.weight_quant in (None, "bf16"):
+    kernel = "gmm_dl_kernel" if big else "gmm_tiled_kernel"
+  else:
+    kernel = "gmm_dlw_kernel" if big and d % 64 == 0 else "gmm_tiled_kernel"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
-              name=("gmm_dl_kernel" if cfg.act_quant == "int8" else "gmm_tiled_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype=op)
+              name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype=op)
 
 
 def cpu_baseline(wl, layer, sample_tokens):
@@ -119,11 +166,25 @@ def calibration(dtype_name, vendor_gemm_shape=None):
   and a plain streaming read of 2 GiB.  Reported beside the roofline, whose `peak` stays the published figure."""
   import torch
 
-  from maxtext_amd import _lib
+  import ctypes
 
-  lib = _lib.load()
+  from maxtext_amd import _lib, build
+
+  # the calibration loops live in a library of their own: they are a benchmark aid, not part of the MoE path's ABI
+  if not os.path.exists(build.CALIB_LIB_PATH):
+    raise RuntimeError(f"{build.CALIB_LIB_PATH} is missing: run `python -m maxtext_amd.build`")
+  lib = ctypes.CDLL(build.CALIB_LIB_PATH)
+  lib.calib_scratch_bytes.restype = ctypes.c_size_t
+  lib.calib_mfma_ops.restype, lib.calib_mfma_ops.argtypes = ctypes.c_double, [ctypes.c_int, ctypes.c_int]
+  lib.calib_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+  lib.calib_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p]
+
+  def ok(status, what):
+    if status != 0:
+      raise RuntimeError(f"{what}: hip error {status}")
+
   stream = _lib.current_stream()
-  scratch = torch.empty((lib.moe_calib_scratch_bytes(),), dtype=torch.uint8, device="cuda")
+  scratch = torch.empty((lib.calib_scratch_bytes(),), dtype=torch.uint8, device="cuda")
 
   def best_ms(fn, reps=3):
     fn()
@@ -141,14 +202,14 @@ def calibration(dtype_name, vendor_gemm_shape=None):
   res = {}
   code = _lib.MOE_INT8 if dtype_name in ("int8", "fp8") else _lib.MOE_BF16
   iters = 4000
-  ops = lib.moe_calib_mfma_ops(code, iters)
+  ops = lib.calib_mfma_ops(code, iters)
   for key, rnd in (("mfma_constant_operands", 0), ("mfma_changing_operands", 1)):
-    ms = best_ms(lambda: _lib.check(lib.moe_calib_mfma(code, rnd, iters, _lib.ptr(scratch), stream), "moe_calib_mfma"))
+    ms = best_ms(lambda: ok(lib.calib_mfma(code, rnd, iters, _lib.ptr(scratch), stream), "calib_mfma"))
     res[key] = ops / ms / 1e9
   res["mfma_unit"] = "TOP/s int8 (v_mfma_i32_16x16x64_i8)" if code == _lib.MOE_INT8 else "TFLOP/s bf16 (v_mfma_f32_16x16x32_bf16)"
   buf = torch.empty((1 << 31,), dtype=torch.uint8, device="cuda")
   buf.fill_(1)
-  ms = best_ms(lambda: _lib.check(lib.moe_calib_read(_lib.ptr(buf), buf.numel(), _lib.ptr(scratch), stream), "moe_calib_read"))
+  ms = best_ms(lambda: ok(lib.calib_read(_lib.ptr(buf), buf.numel(), _lib.ptr(scratch), stream), "calib_read"))
   res["hbm_read_gbs"] = buf.numel() / ms / 1e6
   del buf
   if vendor_gemm_shape is not None and code == _lib.MOE_INT8:
@@ -249,6 +310,7 @@ def train_main(args):
   dom_ms = stage_ms[dom]
   achieved = 2.0 * m * d * f / (dom_ms * 1e-3) / 1e12
   flops = 18.0 * m * d * f
+  traffic, traffic_source = measured_traffic(wl.name + "_train") if args.tokens is None else (None, None)
   result = {
       "metric": "moe_bf16_layer_fwd_bwd_tflops", "value": flops / (elapsed / args.steps) / 1e12, "unit": "TFLOP/s",
       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps,
@@ -257,7 +319,7 @@ def train_main(args):
                              f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU",
                  "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
       "roofline": dict(bound="mfma", achieved=achieved, peak=PEAK_TFLOPS["bf16"], unit="TFLOP/s", frac=achieved / PEAK_TFLOPS["bf16"],
-                       traffic=MEASURED_TRAFFIC_BYTES.get(wl.name + "_train") if args.tokens is None else None,
+                       traffic=traffic, traffic_source=traffic_source,
                        kernel="tgmm_dl_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
       "stage_ms": stage_ms,
   }
@@ -267,26 +329,13 @@ def train_main(args):
   print(json.dumps(result))
 
 
-def main():
-  args = parse()
-  if args.gpus != 1:
-    print("bench.py measures one GPU: every box of this build has a single MI355X and the expert path has no "
-          "multi-GPU code; run with --gpus 1", file=sys.stderr)
-    sys.exit(2)
-
+def run_workload(args, name, tokens=None):
+  """Builds workload `name`, times args.steps steps after args.warmup, returns the fields of its result line."""
   import torch
 
-  from maxtext_amd import _lib, moe, synthetic
+  from maxtext_amd import moe, synthetic
 
-  _lib.load()
-  if not torch.cuda.is_available():
-    print("bench.py needs a GPU", file=sys.stderr)
-    sys.exit(2)
-  torch.cuda.set_device(0)
-  if args.train:
-    return train_main(args)
-
-  wl = synthetic.workload(args.workload, args.tokens)
+  wl = synthetic.workload(name, tokens)
   cfg = wl.cfg
   layer = synthetic.make_layer(wl, device="cuda")
   cls = moe.RoutedAndSharedMoE if cfg.shared_experts else moe.RoutedMoE
@@ -357,32 +406,25 @@ def main():
 
   model = dominant_kernel_model(wl, gs)
   stage_ms = {}
-  for name in ("wi_glu", "wo"):
-    ts = [a.elapsed_time(b) for (n, a, b) in events if n == name]
+  for stage in ("wi_glu", "wo"):
+    ts = [a.elapsed_time(b) for (n, a, b) in events if n == stage]
     if ts:
-      stage_ms[name] = sum(ts) / len(ts)
+      stage_ms[stage] = sum(ts) / len(ts)
   dom_ms = stage_ms.get("wi_glu")
   achieved = model["work"] / (dom_ms * 1e-3) / model["scale"] if dom_ms else None
+  traffic, traffic_source = measured_traffic(wl.name) if tokens is None else (None, None)
   roofline = dict(bound=model["bound"], achieved=achieved, peak=model["peak"], unit=model["unit"],
-                  frac=(achieved / model["peak"]) if achieved else None,
-                  traffic=MEASURED_TRAFFIC_BYTES.get(wl.name) if args.tokens is None else None, kernel=model["name"],
-                  kernel_ms=dom_ms)
+                  frac=(achieved / model["peak"]) if achieved else None, traffic=traffic, traffic_source=traffic_source,
+                  kernel=model["name"], kernel_ms=dom_ms)
 
-  flops = synthetic.layer_flops(wl)
-  value = flops / (elapsed / args.steps) / 1e12
-  result = {
-      "metric": "moe_quant_gmm_layer_tflops",
-      "value": value,
+  # whole-layer minimum HBM traffic (weights of non-empty experts + activations in/out), for HBM-bound shapes
+  nonempty = int((gs > 0).sum())
+  min_bytes = nonempty * synthetic.weight_bytes_per_expert(wl) + wl.tokens * cfg.emb_dim * 2 * 2
+  res = {
+      "value": synthetic.layer_flops(wl) / (elapsed / args.steps) / 1e12,
       "unit": "TFLOP/s",
-      "n_gpus": 1,
-      "steps": args.steps,
-      "warmup": args.warmup,
       "ms_per_step": ms_per_step,
-      "higher_is_better": True,
-      "scaling": "weak",
-      "vs_baseline": None,
       "dtype": model["dtype"],
-      "data": "synthetic",
       "config": {
           "workload": f"{wl.name}: MoE expert layer, {wl.tokens} tokens, d_model {cfg.emb_dim}, d_ff {cfg.moe_mlp_dim}, "
                       f"{cfg.num_experts} experts top-{cfg.num_experts_per_tok}"
@@ -393,15 +435,61 @@ def main():
       },
       "roofline": roofline,
       "stage_ms": stage_ms,
+      "layer_gbps": min_bytes / (elapsed / args.steps) / 1e9,
+  }
+  vendor_shape = (int(gs.sum()), cfg.emb_dim, 2 * cfg.moe_mlp_dim) if model["dtype"] == "int8" and model["bound"] == "mfma" else None
+  return res, wl, layer, model, vendor_shape
+
+
+def main():
+  args = parse()
+  if args.source_hash:
+    key = (args.workload or "c2") + ("_train" if args.train else "")
+    print(kernel_source_hash(PROFILE_OF[key][1]))
+    return
+  if args.gpus != 1:
+    print("bench.py measures one GPU: every box of this build has a single MI355X and the expert path has no "
+          "multi-GPU code; run with --gpus 1", file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+
+  from maxtext_amd import _lib
+
+  _lib.load()
+  if not torch.cuda.is_available():
+    print("bench.py needs a GPU", file=sys.stderr)
+    sys.exit(2)
+  torch.cuda.set_device(0)
+  if args.train:
+    args.workload = args.workload or "c2"
+    return train_main(args)
+
+  # BASELINE's metric names two workloads: the int8 prefill layer (its MFMA half, the headline value) and the fp8
+  # decode layer (its HBM half).  With no --workload both run, one after the other, in this process.
+  both = args.workload is None
+  res, wl, layer, model, vendor_shape = run_workload(args, args.workload or "c2", args.tokens)
+  result = {
+      "metric": "moe_quant_gmm_layer_tflops",
+      "value": res["value"],
+      "unit": res["unit"],
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": res["ms_per_step"],
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": res["dtype"],
+      "data": "synthetic",
+      "config": res["config"],
+      "roofline": res["roofline"],
+      "stage_ms": res["stage_ms"],
       "graph": bool(args.graph),
       "cold_cache": bool(args.cold),
       "gate_in_step": bool(args.gate),
-      "layer_gbps": None,
+      "layer_gbps": res["layer_gbps"],
   }
-  # whole-layer minimum HBM traffic (weights of non-empty experts + activations in/out), for HBM-bound shapes
-  nonempty = int((gs > 0).sum())
-  min_bytes = nonempty * synthetic.weight_bytes_per_expert(wl) + wl.tokens * cfg.emb_dim * 2 * 2
-  result["layer_gbps"] = min_bytes / (elapsed / args.steps) / 1e9
 
   if args.calibrate_copy:
     src = torch.ones((1 << 28,), dtype=torch.int32, device="cuda")
@@ -410,13 +498,21 @@ def main():
     torch.cuda.synchronize()
     del src, dst
 
-  vendor_shape = (int(gs.sum()), cfg.emb_dim, 2 * cfg.moe_mlp_dim) if model["dtype"] == "int8" and model["bound"] == "mfma" else None
-  del out
   torch.cuda.empty_cache()
   result["calibration"] = calibration(model["dtype"], vendor_shape)
   if not args.no_cpu_baseline:
     sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048, "c5mx": 2048}[wl.name]
     result["cpu_baseline"] = cpu_baseline(wl, layer, sample)
+  del layer
+  torch.cuda.empty_cache()
+  if both:
+    sec, swl, slayer, smodel, _ = run_workload(args, "c3")
+    del slayer
+    result["secondary"] = {
+        "workload": sec["config"]["workload"], "metric": "moe_quant_gmm_layer_tflops", "value": sec["value"], "unit": sec["unit"],
+        "ms_per_step": sec["ms_per_step"], "steps": args.steps, "warmup": args.warmup, "dtype": sec["dtype"],
+        "config": sec["config"], "roofline": sec["roofline"], "stage_ms": sec["stage_ms"], "layer_gbps": sec["layer_gbps"],
+    }
   print(json.dumps(result))
 
 

@@ -326,14 +326,18 @@ MOE_API int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem
  *
  *   lhs   [M, K] bf16   forward activations (the caller does NOT transpose them)
  *   dout  [M, N] bf16   gradient of the forward output
+ *   existing_out  NULL, or [G_local, N, K] bf16 or f32 (existing_dtype) added to the f32 products before the
+ *         one rounding to out_dtype (backend.py:733-734).  It may be `out` itself when the element types agree
+ *         (the reference aliases the two buffers, backend.py:761-766).
  *   out   [G_local, N, K] bf16 or f32 (out_dtype): the layout of the forward weights; groups with no
- *         rows are written as zeros (reference_tgmm, tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:156-186)
+ *         rows are written as zeros plus existing_out (reference_tgmm,
+ *         tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:156-186)
  * The gradient of lhs needs no entry point of its own: it is moe_gmm(dout, rhs re-laid out as [G, K, N]).
  * Limits: K % 8 == 0, N % 8 == 0.
  */
 MOE_API int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
-                     int num_groups_total, int num_groups_local, int group_offset, int out_dtype, void* out,
-                     void* stream);
+                     int num_groups_total, int num_groups_local, int group_offset, const void* existing_out,
+                     int existing_dtype, int out_dtype, void* out, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Unpermute + top-k weighted combine.  Replaces RoutedMoE.unpermute
@@ -385,21 +389,6 @@ MOE_API int moe_unpermute_combine_bwd(const void* dout, const void* y, const int
 MOE_API int moe_glu_act(const void* h0, const void* h1, size_t n, int act, float act_limit, void* out, void* stream);
 MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, size_t n, int act, float act_limit,
                             void* dh0, void* dh1, void* stream);
-
-/* ---------------------------------------------------------------------------
- * Calibration (no counterpart in the reference; used by the benchmark): what this machine sustains with a
- * register-only MFMA loop, with constant operands or operands that change every instruction (random data makes
- * the chip draw more power and lower its clock), and with a plain streaming read.  The caller times the launches.
- *   moe_calib_mfma: dtype MOE_INT8 (v_mfma_i32_16x16x64_i8) or MOE_BF16 (v_mfma_f32_16x16x32_bf16), the shapes of
- *   the GEMM kernels (under the power limit they sustain about a fifth more than the 32 x 32 shapes); the launch
- *   performs moe_calib_mfma_ops(dtype, iters) operations.  scratch: moe_calib_scratch_bytes() bytes.
- *   moe_calib_read: reads `bytes` (16-byte aligned, >= 64 KiB) once, with non-temporal requests that each cover
- *   whole 128-byte lines (the fastest streaming read on this part).
- */
-MOE_API size_t moe_calib_scratch_bytes(void);
-MOE_API double moe_calib_mfma_ops(int dtype, int iters);
-MOE_API int moe_calib_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream);
-MOE_API int moe_calib_read(const void* src, size_t bytes, void* scratch, void* stream);
 
 #ifdef __cplusplus
 }

@@ -92,11 +92,7 @@ SIGNATURES = {
     "moe_gmm_static_ws": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
     "moe_gmm_static_ws_capacity": (c_size_t, []),
     "moe_init": (c_int, []),
-    "moe_tgmm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "moe_calib_scratch_bytes": (c_size_t, []),
-    "moe_calib_mfma_ops": (ctypes.c_double, [c_int, c_int]),
-    "moe_calib_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p]),
-    "moe_calib_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
+    "moe_tgmm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "moe_transpose_rhs": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moe_unpermute_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_glu_act": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_float, c_void_p, c_void_p]),

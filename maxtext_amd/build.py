@@ -11,7 +11,10 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "lib", "libmoe_mi355x.so")
-SOURCES = ["moe_route.hip", "moe_gmm.hip", "moe_gmm_tiled.hip", "moe_gmm_dl.hip", "moe_gmm_dlw.hip", "moe_gmm_fp8.hip", "moe_gmm_wq.hip", "moe_tgmm.hip", "moe_calib.hip"]
+SOURCES = ["moe_route.hip", "moe_gmm.hip", "moe_gmm_tiled.hip", "moe_gmm_dl.hip", "moe_gmm_dlw.hip", "moe_gmm_fp8.hip", "moe_gmm_wq.hip", "moe_tgmm.hip"]
+# benchmark-only helpers (machine calibration loops), linked into a library of their own
+CALIB_LIB_PATH = os.path.join(PKG_DIR, "lib", "libbench_calib.so")
+CALIB_SOURCE = "bench_calib.hip"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -48,7 +51,8 @@ def build_library(verbose: bool = True) -> str:
   flags = [f for f in HIPCC_FLAGS if f != "-shared"]
   objs = [os.path.join(obj_dir, s.replace(".hip", ".o")) for s in SOURCES]
   cmds = [[hipcc] + flags + ["-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
-  with ThreadPoolExecutor(max_workers=min(len(cmds), 8)) as pool:
+  cmds.append([hipcc] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC, os.path.join(CSRC, CALIB_SOURCE), "-o", CALIB_LIB_PATH])
+  with ThreadPoolExecutor(max_workers=8) as pool:
     errs = list(pool.map(lambda c: _run(c, verbose), cmds))
   errs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden"] + objs + ["-o", LIB_PATH], verbose))
   if verbose:

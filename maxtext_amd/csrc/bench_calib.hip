@@ -1,3 +1,4 @@
+// Benchmark-only library (libbench_calib.so), not part of the product ABI: nothing in the MoE path calls it.
 // Calibration kernels: what the machine delivers with no memory system in the way (a register-only MFMA loop,
 // with operands that stay constant or change every instruction) and with nothing but the memory system (a plain
 // streaming read).  The benchmark reports them beside the roofline fractions of the real kernels, whose peaks are
@@ -76,15 +77,18 @@ using namespace moe;
 
 extern "C" {
 
-size_t moe_calib_scratch_bytes(void) { return (size_t)kCalibBlocks * 256 * sizeof(int); }
+// Every function returns 0 or a hipError_t value; the caller times the launches.
+#define CALIB_API __attribute__((visibility("default")))
 
-double moe_calib_mfma_ops(int dtype, int iters) {
+CALIB_API size_t calib_scratch_bytes(void) { return (size_t)kCalibBlocks * 256 * sizeof(int); }
+
+CALIB_API double calib_mfma_ops(int dtype, int iters) {
   const double per_mfma = dtype == MOE_INT8 ? 2.0 * 16 * 16 * 64 : 2.0 * 16 * 16 * 32;
   return (double)kCalibBlocks * 4 * (double)iters * kCalibAcc * per_mfma;
 }
 
-int moe_calib_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream) {
-  if (!scratch || iters <= 0) return fail(MOE_ERR_INVALID_ARG, "calib_mfma: bad arguments");
+CALIB_API int calib_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream) {
+  if (!scratch || iters <= 0) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
   int* sink = (int*)scratch;
   if (dtype == MOE_INT8) {
@@ -94,15 +98,15 @@ int moe_calib_mfma(int dtype, int random_operands, int iters, void* scratch, voi
     if (random_operands) calib_mfma_kernel<true, true><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
     else calib_mfma_kernel<true, false><<<kCalibBlocks, 256, 0, s>>>(iters, 12345, sink);
   } else {
-    return fail(MOE_ERR_UNSUPPORTED, "calib_mfma: dtype %d", dtype);
+    return (int)hipErrorInvalidValue;
   }
-  return check_launch("calib_mfma_kernel");
+  return (int)hipGetLastError();
 }
 
-int moe_calib_read(const void* src, size_t bytes, void* scratch, void* stream) {
-  if (!src || !scratch || bytes < 65536 || ((uintptr_t)src & 15)) return fail(MOE_ERR_INVALID_ARG, "calib_read: bad arguments");
+CALIB_API int calib_read(const void* src, size_t bytes, void* scratch, void* stream) {
+  if (!src || !scratch || bytes < 65536 || ((uintptr_t)src & 15)) return (int)hipErrorInvalidValue;
   calib_read_kernel<<<kCalibBlocks, 256, 0, (hipStream_t)stream>>>((const v4i*)src, bytes / 16, (int*)scratch);
-  return check_launch("calib_read_kernel");
+  return (int)hipGetLastError();
 }
 
 }  // extern "C"

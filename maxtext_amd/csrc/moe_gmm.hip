@@ -490,6 +490,7 @@ int moe_init(void) {
   if (int st = prepare_tiled()) return st;
   if (int st = prepare_dl()) return st;
   if (int st = prepare_dlw()) return st;
+  if (int st = prepare_tgmm()) return st;
   return prepare_fp8();
 }
 

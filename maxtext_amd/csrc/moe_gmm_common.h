@@ -394,6 +394,7 @@ int prepare_tiled();
 int prepare_dl();
 int prepare_fp8();
 int prepare_dlw();
+int prepare_tgmm();
 
 // ---- launchers (one translation unit per kernel family) ----
 // moe_gmm_tiled.hip: register-staged kernel, m-tile bm in {64, 128, 256}; block_scaled: int8 x int8 / fp8 x fp8 with K-block

@@ -7,7 +7,7 @@
 // the "B" operand (32 n channels), so a lane ends up with 4 consecutive k of one n: contiguous stores into
 // the [G, N, K] weight layout.
 
-#include "moe_common.h"
+#include "moe_gmm_common.h"
 
 namespace moe {
 
@@ -20,10 +20,28 @@ struct TgmmParams {
   const uint16_t* dout;  // [M, N] bf16
   const int32_t* group_sizes;
   void* out;  // [G_local, N, K] bf16 or f32
+  const void* existing;  // NULL, or [G_local, N, K] values added to the products before the store (may be `out` itself)
   int M, K, N;
   int G_total, G_local, group_offset;
-  int out_f32;
+  int out_f32, existing_f32;
 };
+
+// out[off .. off+3] = v + existing[off .. off+3].  A lane reads the four values it is about to overwrite, so `existing`
+// may be the output buffer.
+__device__ __forceinline__ void tgmm_store4(const TgmmParams& p, size_t off, float v0, float v1, float v2, float v3) {
+  if (p.existing) {
+    if (p.existing_f32) {
+      const float4 e = *(const float4*)((const float*)p.existing + off);
+      v0 += e.x; v1 += e.y; v2 += e.z; v3 += e.w;
+    } else {
+      const uint2 e = *(const uint2*)((const uint16_t*)p.existing + off);
+      v0 += bf16_bits_to_f32(e.x & 0xffffu); v1 += bf16_bits_to_f32(e.x >> 16);
+      v2 += bf16_bits_to_f32(e.y & 0xffffu); v3 += bf16_bits_to_f32(e.y >> 16);
+    }
+  }
+  if (p.out_f32) *(float4*)((float*)p.out + off) = make_float4(v0, v1, v2, v3);
+  else *(uint2*)((uint16_t*)p.out + off) = make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+}
 
 __device__ __forceinline__ v8bf read_tr_frag(const uint8_t* tile, int row0, int col0, int lane) {
   // 8 contraction values (rows row0 + 8*(lane/32) .. +7) of column col0 + lane%32
@@ -133,11 +151,7 @@ __global__ __launch_bounds__(kTgThreads) void tgmm_kernel(const TgmmParams p) {
         const int k = k0 + wk * 64 + i * 32 + 8 * q + 4 * (lane / 32);
         if (k >= K) continue;
         const size_t off = ((size_t)g_local * N + n) * K + k;
-        const float v0 = acc[j][i][4 * q], v1 = acc[j][i][4 * q + 1], v2 = acc[j][i][4 * q + 2], v3 = acc[j][i][4 * q + 3];
-        if (p.out_f32)
-          *(float4*)((float*)p.out + off) = make_float4(v0, v1, v2, v3);
-        else
-          *(uint2*)((uint16_t*)p.out + off) = make_uint2(pack_bf16x2(v0, v1), pack_bf16x2(v2, v3));
+        tgmm_store4(p, off, acc[j][i][4 * q], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]);
       }
   }
 }
@@ -204,8 +218,7 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
   if (size == 0) {  // an empty group's gradient is zero
     for (int i = tid; i < kTdTile * (kTdTile / 4); i += kTdThreads) {
       const size_t off = ((size_t)g_local * N + n0 + i / (kTdTile / 4)) * K + k0 + (i % (kTdTile / 4)) * 4;
-      if (p.out_f32) *(float4*)((float*)p.out + off) = make_float4(0.f, 0.f, 0.f, 0.f);
-      else *(uint2*)((uint16_t*)p.out + off) = make_uint2(0, 0);
+      tgmm_store4(p, off, 0.f, 0.f, 0.f, 0.f);
     }
     return;
   }
@@ -343,10 +356,7 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
     for (int j = 0; j < 4; j++) {
       const int k = k0 + wk * 64 + j * 16 + 4 * gq;
       const size_t off = ((size_t)g_local * N + n) * K + k;
-      if (p.out_f32)
-        *(float4*)((float*)p.out + off) = make_float4(acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]);
-      else
-        *(uint2*)((uint16_t*)p.out + off) = make_uint2(pack_bf16x2(acc[j][i][0], acc[j][i][1]), pack_bf16x2(acc[j][i][2], acc[j][i][3]));
+      tgmm_store4(p, off, acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]);
     }
   }
 }
@@ -355,9 +365,13 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
 
 using namespace moe;
 
+namespace moe {
+int prepare_tgmm() { return reserve_lds(tgmm_dl_kernel, kTdLds, lds_flags<TgmmParams>()); }
+}  // namespace moe
+
 extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
-                        int num_groups_total, int num_groups_local, int group_offset, int out_dtype, void* out,
-                        void* stream) {
+                        int num_groups_total, int num_groups_local, int group_offset, const void* existing_out,
+                        int existing_dtype, int out_dtype, void* out, void* stream) {
   if (!lhs || !dout || !group_sizes || !out) return fail(MOE_ERR_INVALID_ARG, "tgmm: NULL pointer");
   if (M < 0 || K <= 0 || N <= 0 || num_groups_total <= 0 || num_groups_local <= 0 || group_offset < 0)
     return fail(MOE_ERR_INVALID_ARG, "tgmm: bad sizes");
@@ -369,17 +383,16 @@ extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_
   p.lhs = (const uint16_t*)lhs; p.dout = (const uint16_t*)dout; p.group_sizes = group_sizes; p.out = out;
   p.M = M; p.K = K; p.N = N; p.G_total = num_groups_total; p.G_local = num_groups_local; p.group_offset = group_offset;
   p.out_f32 = out_dtype == MOE_F32;
+  if (existing_out && existing_dtype != MOE_BF16 && existing_dtype != MOE_F32)
+    return fail(MOE_ERR_UNSUPPORTED, "tgmm: existing_dtype %d", existing_dtype);
+  if ((uintptr_t)existing_out & 15) return fail(MOE_ERR_UNSUPPORTED, "tgmm: pointers must be 16-byte aligned");
+  if (existing_out == out && existing_dtype != out_dtype)
+    return fail(MOE_ERR_INVALID_ARG, "tgmm: existing_out aliases out with another element type");
+  p.existing = existing_out; p.existing_f32 = existing_dtype == MOE_F32;
   // groups of 128 rows and more on average take the 256 x 256 tiles when the shape allows it
   const long long tiles = (long long)(K / kTdTile) * (N / kTdTile) * num_groups_local;
   if (K % kTdTile == 0 && N % kTdTile == 0 && K < (1 << 24) && N < (1 << 24) && (long long)M >= 128LL * num_groups_total && tiles >= 128 && tiles <= 0x7fffffffLL) {
-    static bool attr_set[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(MOE_ERR_LAUNCH, "tgmm: cannot identify the current device");
-    if (!attr_set[dev]) {  // a race between two host threads only repeats an idempotent call
-      hipError_t e = hipFuncSetAttribute((const void*)tgmm_dl_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kTdLds);
-      if (e != hipSuccess) return fail(MOE_ERR_LAUNCH, "tgmm: cannot reserve %d bytes of LDS: %s", kTdLds, hipGetErrorString(e));
-      attr_set[dev] = true;
-    }
+    if (int st = prepare_tgmm()) return st;
     tgmm_dl_kernel<<<(unsigned)tiles, kTdThreads, kTdLds, (hipStream_t)stream>>>(p);
     return check_launch("tgmm_dl_kernel");
   }

@@ -373,8 +373,10 @@ def gmm_rhs_kn_supported(m, k, n, num_groups_total):
   return bool(_lib.load().moe_gmm_rhs_kn_supported(int(m), int(k), int(n), int(num_groups_total)))
 
 
-def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16):
-  """Weight gradient: out[g, n, k] = sum over rows m of group g of dout[m, n] * lhs[m, k]  ->  [G_local, N, K]."""
+def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16, existing_out=None):
+  """Weight gradient: out[g, n, k] = sum over rows m of group g of dout[m, n] * lhs[m, k]  ->  [G_local, N, K].
+
+  existing_out: [G_local, N, K] bf16 or f32, added to the f32 products before the rounding to out_dtype."""
   _need(lhs, "lhs", torch.bfloat16, 2)
   _need(dout, "dout", torch.bfloat16, 2)
   _need(group_sizes, "group_sizes", torch.int32, 1)
@@ -387,8 +389,16 @@ def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_d
   if out_dtype not in (torch.bfloat16, torch.float32):
     raise TypeError("out_dtype must be bfloat16 or float32")
   out = torch.empty((g_local, n, k), dtype=out_dtype, device=lhs.device)
+  code = {torch.bfloat16: _lib.MOE_BF16, torch.float32: _lib.MOE_F32}
+  if existing_out is not None:
+    if existing_out.dtype not in code:
+      raise TypeError("existing_out must be bfloat16 or float32")
+    _need(existing_out, "existing_out", existing_out.dtype, 3)
+    if tuple(existing_out.shape) != (g_local, n, k):
+      raise ValueError(f"existing_out must be [{g_local}, {n}, {k}], got {tuple(existing_out.shape)}")
   lib = _lib.load()
   st = lib.moe_tgmm(_lib.ptr(lhs), _lib.ptr(dout), _lib.ptr(group_sizes), m, k, n, g_total, g_local, int(group_offset),
-                    _lib.MOE_BF16 if out_dtype == torch.bfloat16 else _lib.MOE_F32, _lib.ptr(out), _lib.current_stream())
+                    None if existing_out is None else _lib.ptr(existing_out), 0 if existing_out is None else code[existing_out.dtype],
+                    code[out_dtype], _lib.ptr(out), _lib.current_stream())
   _lib.check(st, "moe_tgmm")
   return out

@@ -297,7 +297,8 @@ def tgmm(
   lhs: [k, m] bf16 (the reference passes the forward activation swapped, ops.py:889-899; a
   `.t()` view of a contiguous [m, k] tensor is consumed without a copy); rhs: [m, n] bf16 (the
   incoming gradient); returns [num_actual_groups, k, n] as a transposed view of the [G, N, K]
-  buffer the kernel writes, which is the layout moe_gmm takes weights in.
+  buffer the kernel writes, which is the layout moe_gmm takes weights in.  existing_out
+  ([num_actual_groups, k, n], float32 or bfloat16) is added in before the output is rounded.
   """
   del tiling, interpret, varying_axes
   if lhs.dim() != 2 or rhs.dim() != 2:
@@ -306,18 +307,26 @@ def tgmm(
     raise ValueError(f"Expected 32-bit integer 'group_sizes' but got {group_sizes.dtype}.")
   if lhs.shape[1] != rhs.shape[0]:
     raise ValueError(f"Expected lhs [k, m] and rhs [m, n] to share m, got {tuple(lhs.shape)} and {tuple(rhs.shape)}.")
-  if existing_out is not None:
-    # rows of local groups are written into the caller's buffer, all other rows keep their contents (backend.py:493-501)
-    if existing_out.dtype != torch.bfloat16 or not existing_out.is_contiguous():
-      raise ValueError("existing_out must be a contiguous bfloat16 tensor")
   if preferred_element_type not in (torch.float32, torch.bfloat16):
     raise NotImplementedError("tgmm outputs are float32 or bfloat16")
+  existing_nk = None
+  if existing_out is not None:
+    # added to the f32 accumulator before the one rounding to the output type (backend.py:733-734)
+    g_local = group_sizes.numel() - (0 if group_offset is None else int(group_offset)) if num_actual_groups is None else int(num_actual_groups)
+    if tuple(existing_out.shape) != (g_local, lhs.shape[0], rhs.shape[1]):
+      raise ValueError(f"existing_out must be [{g_local}, {lhs.shape[0]}, {rhs.shape[1]}], got {tuple(existing_out.shape)}")
+    if existing_out.dtype not in (torch.float32, torch.bfloat16):
+      raise NotImplementedError("existing_out is float32 or bfloat16")
+    existing_nk = existing_out.transpose(1, 2)  # the kernel's [G, N, K] layout; a view when the caller kept a result of tgmm
+    if not existing_nk.is_contiguous():
+      existing_nk = existing_nk.contiguous()
   offset = 0 if group_offset is None else int(group_offset)
   lhs_mk = lhs.t()
   if not lhs_mk.is_contiguous():
     lhs_mk = lhs_mk.contiguous()
   out = kernels.tgmm(
-      lhs_mk, rhs.contiguous(), group_sizes, num_groups_local=num_actual_groups, group_offset=offset, out_dtype=preferred_element_type
+      lhs_mk, rhs.contiguous(), group_sizes, num_groups_local=num_actual_groups, group_offset=offset, out_dtype=preferred_element_type,
+      existing_out=existing_nk,
   )
   return out.transpose(1, 2)
 

@@ -357,11 +357,12 @@ def gmm(
 
 
 def tgmm(lhs: torch.Tensor, dout: torch.Tensor, group_sizes, *, num_actual_groups=None, group_offset: int = 0,
-         out_dtype=torch.bfloat16) -> torch.Tensor:
+         out_dtype=torch.bfloat16, existing_out=None) -> torch.Tensor:
   """Transposed grouped matmul, the weight gradient of gmm
   (tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:156-186 reference_tgmm; backend.py:587):
   out[g] = lhs[rows of group g]^T @ dout[rows of group g], shape [groups, k, n]; only the
-  num_actual_groups groups starting at group_offset are produced."""
+  num_actual_groups groups starting at group_offset are produced.  existing_out ([groups, k, n]) joins the
+  accumulator before the rounding to out_dtype (backend.py:731-735)."""
   group_sizes = np.asarray(group_sizes, dtype=np.int64)
   m = lhs.shape[0]
   g = group_sizes.size - group_offset if num_actual_groups is None else num_actual_groups
@@ -371,7 +372,10 @@ def tgmm(lhs: torch.Tensor, dout: torch.Tensor, group_sizes, *, num_actual_group
     end = min(start + int(group_sizes[gg]), m)
     loc = gg - group_offset
     if 0 <= loc < g:
-      outs.append((lhs[start:end].double().T @ dout[start:end].double()).to(out_dtype))
+      acc = lhs[start:end].double().T @ dout[start:end].double()
+      if existing_out is not None:
+        acc = acc + existing_out[loc].double()
+      outs.append(acc.to(out_dtype))
     start = end
   return torch.stack(outs)
 

@@ -556,6 +556,33 @@ def test_tgmm_big_tiles_exact_on_small_integers_and_group_window(K):
   assert torch.equal(got16.cpu(), want.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("m,k,n,gs", [(333, 136, 264, [40, 0, 100, 93, 100]), (700, 1024, 3072, [140, 0, 199, 193, 100])])
+@pytest.mark.parametrize("existing_dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_tgmm_existing_out_is_added_before_rounding(K, m, k, n, gs, existing_dtype, out_dtype):
+  """existing_out joins the f32 accumulator (backend.py:733-734), also for groups without rows, also when it is the
+  output buffer's own dtype; integer data keeps every sum exact, so the comparison is bit for bit."""
+  from maxtext_amd import megablox
+
+  rng = np.random.default_rng(31)
+  gs = np.array(gs, np.int32)
+  lhs = torch.from_numpy(rng.integers(-3, 4, (m, k)).astype(np.float32)).to(torch.bfloat16)
+  dout = torch.from_numpy(rng.integers(-3, 4, (m, n)).astype(np.float32)).to(torch.bfloat16)
+  # halves make the bf16 output round: rounding the products first and adding afterwards would give other bits
+  existing = torch.from_numpy(rng.integers(-9, 10, (3, k, n)).astype(np.float32) * 0.5).to(existing_dtype)
+  want = O.tgmm(lhs, dout, gs, num_actual_groups=3, group_offset=1, out_dtype=out_dtype, existing_out=existing)
+  got = megablox.tgmm(cuda(lhs).t(), cuda(dout), cuda(gs), preferred_element_type=out_dtype, group_offset=1, num_actual_groups=3,
+                      existing_out=cuda(existing))
+  assert got.shape == want.shape and got.dtype == out_dtype
+  assert torch.equal(got.cpu(), want)
+  assert torch.equal(got[0].cpu(), existing[0].to(out_dtype))  # group 1 has no rows: its slice is existing_out alone
+  # accumulating in place: the kernel's [G, N, K] result of one call is the existing_out of the next
+  first = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=torch.float32)
+  twice = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_dtype=torch.float32, existing_out=first)
+  assert torch.equal(twice, 2 * first)
+  with pytest.raises(ValueError):
+    megablox.tgmm(cuda(lhs).t(), cuda(dout), cuda(gs), existing_out=cuda(existing))  # 3 groups given, 5 expected
+
+
 def test_tgmm_argument_errors(K):
   a = torch.zeros(16, 64, dtype=torch.bfloat16, device="cuda")
   gs = torch.tensor([16], dtype=torch.int32, device="cuda")

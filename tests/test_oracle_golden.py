@@ -360,6 +360,12 @@ def test_tgmm_equals_autograd_of_grouped_matmul_and_hand_case():
   d2 = torch.tensor([[1.0], [10.0], [100.0]])
   t2 = O.tgmm(lhs2, d2, np.array([2, 1], np.int32), out_dtype=torch.float32)
   assert t2.tolist() == [[[31.0], [42.0]], [[500.0], [600.0]]]
+  # existing_out joins the accumulator before the one rounding (backend.py:733-734): 256 + 1 + 0.5 rounds to 258 in
+  # bf16 (8 bits of mantissa: spacing 2 above 256), while bf16(256 + 1) + 0.5 would have stayed at 256
+  lhs3, d3 = torch.tensor([[16.0], [1.0]]), torch.tensor([[16.0], [1.0]])
+  ex = torch.tensor([[[0.5]]])
+  assert O.tgmm(lhs3, d3, np.array([2], np.int32), out_dtype=torch.bfloat16, existing_out=ex).tolist() == [[[258.0]]]
+  assert O.tgmm(lhs3, d3, np.array([0, 2], np.int32), out_dtype=torch.float32, existing_out=torch.tensor([[[0.5]], [[1.0]]])).tolist() == [[[0.5]], [[258.0]]]
 
 
 def test_gate_logits_special_cases():
