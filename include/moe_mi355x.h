@@ -94,7 +94,8 @@ MOE_API int moe_route_topk(const float* gate_logits, const float* pre_bias_logit
  * (src/maxtext/layers/moe.py:353-392) followed by RoutedMoE.get_topk (moe.py:717-765):
  *
  *   logits   = x @ Wg                       (f32 accumulation)
- *   scores   = sigmoid(logits) if score_func == 1 else logits;   pre_bias = scores   (moe.py:382-386)
+ *   scores   = sigmoid(logits) if score_func == 1, sqrt(softplus(logits)) if score_func == 2 (the DeepSeek-V4 router,
+ *              layers/linears.py:51-53), else logits;   pre_bias = scores   (moe.py:382-386)
  *   scores  += gate_bias                                                              (moe.py:388-390)
  *   (topk_weights, topk_idx) = moe_route_topk(scores, pre_bias, ...)
  *
@@ -344,19 +345,22 @@ MOE_API int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_siz
  * (moe.py:1039-1063, float32_weight_sum=True) and the fused gather-reduce
  * fallback (kernels/ragged/ragged_gather_reduce_v2.py:170-182):
  *
- *   out[t, :] = bf16( sum_s weights[t, s] * f32(y[inv_perm[t*k + s], :]) )
+ *   out[t, :] = bf16( sum over the valid s of weights[t, s] * f32(y[inv_perm[t*k + s], :]) )
  *
  *   y        [M, d] bf16     expert outputs in sorted order
  *   perm     [M] i32         sorted_selected_experts; used only when inv_perm == NULL,
  *                            then inv_perm is rebuilt into `workspace` (M * 4 bytes)
  *   weights  [T, k] f32, or NULL for an unweighted sum
  *            (kernels/sort_activations.py:98-121)
+ *   valid_rows_mask  [T, k] bytes, or NULL for "all valid": a zero byte takes gathered row (t, s) out of the sum
+ *            (valid_rows_mask of ragged_gather_reduce, kernels/ragged/ragged_gather_reduce_v2.py:637-659; the row
+ *            is not read, so a NaN in it does not reach the output)
  *   out      [T, d] bf16
  * Limits: d % 8 == 0, k <= 16.
  */
 MOE_API int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv_perm,
-                          const float* weights, int T, int k, int d, void* out, void* workspace,
-                          size_t workspace_bytes, void* stream);
+                          const float* weights, const uint8_t* valid_rows_mask, int T, int k, int d, void* out,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Gradient of moe_unpermute_combine with respect to y and to the weights (the VJP that JAX derives for
@@ -368,13 +372,15 @@ MOE_API int moe_unpermute_combine(const void* y, const int32_t* perm, const int3
  *
  *   dout [T, d] bf16; y [M, d] bf16 (forward input; may be NULL when dweights is NULL);
  *   weights [T, k] f32 or NULL (ones); dy [M, d] bf16 (every row is written: inv_perm is a permutation);
- *   dweights [T, k] f32 or NULL.
+ *   dweights [T, k] f32 or NULL; valid_rows_mask as in the forward pass: a masked (t, s) gets a zero row of dy
+ *   and a zero dweights entry.
  * The gradient of the row gather (moe_gather_rows in copy mode; _sort_activations_custom_bwd,
  * moe.py:165-171) is moe_unpermute_combine itself with weights == NULL.
  * Limits: d % 8 == 0, k <= 16.
  */
 MOE_API int moe_unpermute_combine_bwd(const void* dout, const void* y, const int32_t* inv_perm, const float* weights,
-                                      int T, int k, int d, void* dy, float* dweights, void* stream);
+                                      const uint8_t* valid_rows_mask, int T, int k, int d, void* dy, float* dweights,
+                                      void* stream);
 
 /* ---------------------------------------------------------------------------
  * Gated activation as a stand-alone pass and its gradient, for training, where both projections are kept

@@ -54,9 +54,11 @@ __device__ __forceinline__ void lhs_rows_of(const RowOpts& o, int (&r)[NR]) {
 // Four consecutive output values of one row: multiplied by the row's factor, then stored as bf16 (8 bytes) or f32.
 __device__ __forceinline__ void store_out4(void* out, const RowOpts& o, size_t row, int N, int n, float (&v)[4]) {
   if (o.row_scale) {
+    // the reference multiplies the finished result of the output type (models/deepseek_batchsplit_fp8.py:1048-1049):
+    // a bf16 result is rounded before the multiplication and again after it
     const float w = o.row_scale[row];
 #pragma unroll
-    for (int r = 0; r < 4; r++) v[r] *= w;
+    for (int r = 0; r < 4; r++) v[r] = (o.out_f32 ? v[r] : round_bf16_fn(v[r])) * w;
   }
   if (o.out_f32) {
     *(float4*)((float*)out + row * N + n) = make_float4(v[0], v[1], v[2], v[3]);
@@ -218,6 +220,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
   // operations in flight, the stores included, i.e. one memory round trip per store (measured on 256 x 256 tiles: 18 us
   // per tile, as much as ten K stages, against 6 us now).
   float rw[TM];
+  const bool round_first = p.ro.row_scale && !p.ro.out_f32;
 #pragma unroll
   for (int i = 0; i < TM; i++) rw[i] = 1.0f;
   if (p.ro.row_scale) {
@@ -227,7 +230,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
       rw[i] = p.ro.row_scale[tile.row0 + (lr < tile.nrows ? lr : 0)];
     }
   }
-  // GENERAL: bias, partial sums, f32 output; otherwise bf16 results straight to memory
+  // GENERAL: bias, partial sums, row factors, f32 output; otherwise bf16 results straight to memory
   auto body = [&](auto act_c, auto general_c) {
     constexpr int ACT = decltype(act_c)::value;
     constexpr bool GENERAL = decltype(general_c)::value;
@@ -254,12 +257,14 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             const float g = fmaf((float)acc[j][i][4 * q + r], e.sa[i] * sg[r], bg[r]);
+            float a = g;
             if (GLU) {
               const float u = fmaf((float)acc[j + NT_OUT][i][4 * q + r], e.sa[i] * su[r], bu[r]);
-              v[r] = glu_act<ACT>(g, u, p.act_limit) * rw[i];
-            } else {
-              v[r] = g * rw[i];
+              a = glu_act<ACT>(g, u, p.act_limit);
             }
+            // a row factor multiplies the finished result of the output type (store_out4 states the rule)
+            if (GENERAL) a = (round_first ? round_bf16_fn(a) : a) * rw[i];
+            v[r] = a;
           }
           if (ok) {
             if (GENERAL && p.ro.out_f32)
@@ -270,7 +275,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
         }
     }
   };
-  const bool general = p.rhs_bias || p.rhs_up_bias || p.partial_sum || p.partial_sum_up || p.ro.out_f32;
+  const bool general = p.rhs_bias || p.rhs_up_bias || p.partial_sum || p.partial_sum_up || p.ro.out_f32 || p.ro.row_scale;
   dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
     if (general) body(act_c, std::true_type{});
     else body(act_c, std::false_type{});

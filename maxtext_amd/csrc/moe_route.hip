@@ -63,7 +63,7 @@ struct GateEpilogue {
   float* logits_out;      // [T, E] or NULL
   float* pre_bias_out;    // [T, E] or NULL
   int num_partials;
-  int score_func;         // 0 none, 1 sigmoid
+  int score_func;         // 0 none, 1 sigmoid, 2 sqrt(softplus)
   int round_bf16;         // round the matmul result to bf16 first
 };
 
@@ -92,6 +92,8 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
         for (int s = 0; s < g.num_partials; s++) x += g.partials[((size_t)s * T + t) * E + e];
         if (g.round_bf16) x = round_bf16_fn(x);
         if (g.score_func == 1) x = 1.0f / (1.0f + expf(-x));
+        // sqrt(softplus(x)), softplus as logaddexp(x, 0) = max(x, 0) + log1p(exp(-|x|)) (linears.py:51-53)
+        if (g.score_func == 2) x = sqrtf(fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))));
         s_pre[wave][e] = x;
         if (active && g.pre_bias_out) g.pre_bias_out[(size_t)t * E + e] = x;
         if (g.bias) x += g.bias[e];
@@ -667,15 +669,17 @@ constexpr int kCombineMaxK = 16;
 
 __global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ y,
                                                       const int32_t* __restrict__ inv_perm,
-                                                      const float* __restrict__ weights, int k,
+                                                      const float* __restrict__ weights,
+                                                      const uint8_t* __restrict__ valid, int k,
                                                       int d, uint4* __restrict__ out) {
   __shared__ int s_row[kCombineMaxK];
   __shared__ float s_w[kCombineMaxK];
   const int t = blockIdx.x;
   if (threadIdx.x < k) {
-    // an index outside [0, M) (a malformed inv_perm) contributes nothing instead of reading out of bounds
+    // an index outside [0, M) (a malformed inv_perm) contributes nothing instead of reading out of bounds, and so does
+    // a row that the caller masked out
     const int row = inv_perm[(size_t)t * k + threadIdx.x];
-    const bool ok = row >= 0 && row < (int)gridDim.x * k;
+    const bool ok = row >= 0 && row < (int)gridDim.x * k && (!valid || valid[(size_t)t * k + threadIdx.x]);
     s_row[threadIdx.x] = ok ? row : -1;
     s_w[threadIdx.x] = weights ? weights[(size_t)t * k + threadIdx.x] : 1.0f;
   }
@@ -705,16 +709,19 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ 
 // gathered, dw[t, s] = sum_d f32(y[row_s, d]) * f32(dout[t, d]).
 __global__ __launch_bounds__(256) void combine_bwd_kernel(const uint4* __restrict__ dout, const uint4* __restrict__ y,
                                                           const int32_t* __restrict__ inv_perm,
-                                                          const float* __restrict__ weights, int k, int d,
+                                                          const float* __restrict__ weights,
+                                                          const uint8_t* __restrict__ valid, int k, int d,
                                                           uint4* __restrict__ dy, float* __restrict__ dw) {
   __shared__ int s_row[kCombineMaxK];
   __shared__ float s_w[kCombineMaxK];
+  __shared__ bool s_masked[kCombineMaxK];
   __shared__ float s_part[kCombineMaxK][4];
   const int t = blockIdx.x;
   if (threadIdx.x < k) {
     const int row = inv_perm[(size_t)t * k + threadIdx.x];
     s_row[threadIdx.x] = row >= 0 && row < (int)gridDim.x * k ? row : -1;  // malformed index: no row is written
     s_w[threadIdx.x] = weights ? weights[(size_t)t * k + threadIdx.x] : 1.0f;
+    s_masked[threadIdx.x] = valid && !valid[(size_t)t * k + threadIdx.x];  // a masked row took no part: zero gradients
   }
   __syncthreads();
   const int nch = d / 8;
@@ -729,6 +736,10 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const uint4* __restric
       if (s >= k) break;
       if (s_row[s] < 0) continue;
       const size_t at = (size_t)s_row[s] * nch + ci;
+      if (s_masked[s]) {
+        dy[at] = make_uint4(0, 0, 0, 0);
+        continue;
+      }
       const float w = s_w[s];
       uint4 o;
       o.x = pack_bf16x2(w * g[0], w * g[1]);
@@ -917,7 +928,7 @@ int moe_gate_route(const void* x, const void* gate_kernel_terms, int num_terms, 
   if (num_terms != 1 && num_terms != 3) return fail(MOE_ERR_INVALID_ARG, "gate_route: num_terms must be 1 or 3");
   if (d % 64 != 0 || E % 4 != 0) return fail(MOE_ERR_UNSUPPORTED, "gate_route: need d %% 64 == 0 and E %% 4 == 0 (d=%d E=%d)", d, E);
   if (E > kRouteMaxE || k > 16 || k > E) return fail(MOE_ERR_UNSUPPORTED, "gate_route: need k<=16, k<=E<=512 (E=%d k=%d)", E, k);
-  if (score_func != 0 && score_func != 1) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad score_func %d", score_func);
+  if (score_func < 0 || score_func > 2) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad score_func %d", score_func);
   if (mode < MOE_ROUTE_SOFTMAX_TOPK || mode > MOE_ROUTE_SOFTMAX_ALL) return fail(MOE_ERR_INVALID_ARG, "gate_route: bad mode %d", mode);
   int ng = n_routing_groups > 0 ? n_routing_groups : 0;
   if (ng > 0) {
@@ -1016,8 +1027,8 @@ int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_in
 }
 
 int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv_perm,
-                          const float* weights, int T, int k, int d, void* out, void* workspace,
-                          size_t workspace_bytes, void* stream) {
+                          const float* weights, const uint8_t* valid_rows_mask, int T, int k, int d, void* out,
+                          void* workspace, size_t workspace_bytes, void* stream) {
   if (!y || !out || (!perm && !inv_perm)) return fail(MOE_ERR_INVALID_ARG, "combine: NULL pointer");
   if (T < 0 || k <= 0 || d <= 0) return fail(MOE_ERR_INVALID_ARG, "combine: bad sizes");
   if (k > kCombineMaxK || d % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "combine: need k<=16, d%%8==0");
@@ -1029,18 +1040,19 @@ int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv
     invert_perm_kernel<<<cdiv(M, 256), 256, 0, s>>>(perm, M, (int32_t*)workspace);
     inv_perm = (const int32_t*)workspace;
   }
-  combine_kernel<<<T, 256, 0, s>>>((const uint4*)y, inv_perm, weights, k, d, (uint4*)out);
+  combine_kernel<<<T, 256, 0, s>>>((const uint4*)y, inv_perm, weights, valid_rows_mask, k, d, (uint4*)out);
   return check_launch("combine_kernel");
 }
 
 int moe_unpermute_combine_bwd(const void* dout, const void* y, const int32_t* inv_perm, const float* weights,
-                              int T, int k, int d, void* dy, float* dweights, void* stream) {
+                              const uint8_t* valid_rows_mask, int T, int k, int d, void* dy, float* dweights,
+                              void* stream) {
   if (!dout || !inv_perm || !dy || (dweights && !y)) return fail(MOE_ERR_INVALID_ARG, "combine_bwd: NULL pointer");
   if (T < 0 || k <= 0 || d <= 0) return fail(MOE_ERR_INVALID_ARG, "combine_bwd: bad sizes");
   if (k > kCombineMaxK || d % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "combine_bwd: need k<=16, d%%8==0");
   if (T == 0) return MOE_OK;
-  combine_bwd_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const uint4*)dout, (const uint4*)y, inv_perm, weights, k, d,
-                                                         (uint4*)dy, dweights);
+  combine_bwd_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const uint4*)dout, (const uint4*)y, inv_perm, weights,
+                                                         valid_rows_mask, k, d, (uint4*)dy, dweights);
   return check_launch("combine_bwd_kernel");
 }
 

@@ -51,6 +51,9 @@ def route_topk(gate_logits, pre_bias_logits=None, *, k, mode="softmax_topk", nor
   return w, idx
 
 
+_SCORE_FUNC_CODE = {"": 0, "sigmoid": 1, "sqrtsoftplus": 2}
+
+
 def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_round_bf16=False, mode="softmax_topk",
                norm_topk_prob=False, weights_round_bf16=True, routed_scaling_factor=1.0, n_routing_groups=-1,
                topk_routing_group=-1, return_logits=False):
@@ -66,7 +69,7 @@ def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_r
     _need(gate_bias, "gate_bias", torch.float32, 1)
     if gate_bias.numel() != e:
       raise ValueError("gate_bias must have E elements")
-  if score_func not in ("", "sigmoid"):
+  if score_func not in _SCORE_FUNC_CODE:
     raise NotImplementedError(f"score_func {score_func!r}")
   if mode not in _lib.ROUTE_BY_NAME:
     raise ValueError(f"unknown routing mode {mode!r}")
@@ -78,7 +81,7 @@ def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_r
   lib = _lib.load()
   ws = torch.empty((max(lib.moe_gate_route_workspace_bytes(t, d, e), 16),), dtype=torch.uint8, device=dev)
   st = lib.moe_gate_route(_lib.ptr(x), _lib.ptr(gate_kernel_terms), s_, _lib.ptr(gate_bias), t, d, e, k,
-                          1 if score_func == "sigmoid" else 0, int(bool(gate_round_bf16)),
+                          _SCORE_FUNC_CODE[score_func], int(bool(gate_round_bf16)),
                           _lib.ROUTE_BY_NAME[mode], int(bool(norm_topk_prob)),
                           int(bool(weights_round_bf16)), float(routed_scaling_factor), int(n_routing_groups),
                           int(topk_routing_group), _lib.ptr(w), _lib.ptr(idx), _lib.ptr(logits), _lib.ptr(pre), _lib.ptr(ws),
@@ -151,13 +154,23 @@ def gather_rows(x, row_idx=None, idx_div=1, *, out_dtype=torch.bfloat16, block_k
   return out, (static_scale if static_scale is not None else scale)
 
 
-def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None):
-  """out[t] = sum_s weights[t,s] * y[inv_perm[t*k+s]]  (f32 accumulate, bf16 out)."""
+def _valid_mask(valid_rows_mask, m):
+  if valid_rows_mask is None:
+    return None
+  _need(valid_rows_mask, "valid_rows_mask", None, None)
+  if valid_rows_mask.dtype not in (torch.bool, torch.uint8) or valid_rows_mask.numel() != m:
+    raise ValueError("valid_rows_mask must hold T*k bool or uint8 entries")
+  return valid_rows_mask.view(torch.uint8)
+
+
+def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None, valid_rows_mask=None):
+  """out[t] = sum over the valid s of weights[t,s] * y[inv_perm[t*k+s]]  (f32 accumulate, bf16 out)."""
   _need(y, "y", torch.bfloat16, 2)
   m, d = y.shape
   if m % k:
     raise ValueError("rows of y must be a multiple of k")
   t = m // k
+  valid = _valid_mask(valid_rows_mask, m)
   if weights is not None:
     _need(weights, "weights", torch.float32)
     if weights.numel() != m:
@@ -174,18 +187,19 @@ def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None):
       raise ValueError("inv_perm must have T*k elements")
   out = torch.empty((t, d), dtype=torch.bfloat16, device=y.device)
   lib = _lib.load()
-  st = lib.moe_unpermute_combine(_lib.ptr(y), _lib.ptr(perm), _lib.ptr(inv_perm), _lib.ptr(weights), t, k, d, _lib.ptr(out),
+  st = lib.moe_unpermute_combine(_lib.ptr(y), _lib.ptr(perm), _lib.ptr(inv_perm), _lib.ptr(weights), _lib.ptr(valid), t, k, d, _lib.ptr(out),
                                  _lib.ptr(ws), 0 if ws is None else ws.numel() * 4, _lib.current_stream())
   _lib.check(st, "moe_unpermute_combine")
   return out
 
 
-def unpermute_combine_bwd(dout, y, weights, *, k, inv_perm, need_dweights=True):
+def unpermute_combine_bwd(dout, y, weights, *, k, inv_perm, need_dweights=True, valid_rows_mask=None):
   """Gradient of unpermute_combine: -> (dy [M, d] bf16, dweights [T, k] f32 or None)."""
   _need(dout, "dout", torch.bfloat16, 2)
   _need(inv_perm, "inv_perm", torch.int32, 1)
   t, d = dout.shape
   m = t * k
+  valid = _valid_mask(valid_rows_mask, m)
   if inv_perm.numel() != m:
     raise ValueError("inv_perm must have T*k elements")
   if weights is not None:
@@ -201,7 +215,7 @@ def unpermute_combine_bwd(dout, y, weights, *, k, inv_perm, need_dweights=True):
   dy = torch.empty((m, d), dtype=torch.bfloat16, device=dout.device)
   lib = _lib.load()
   st = lib.moe_unpermute_combine_bwd(_lib.ptr(dout), _lib.ptr(y) if need_dweights else None, _lib.ptr(inv_perm), _lib.ptr(weights),
-                                     t, k, d, _lib.ptr(dy), _lib.ptr(dw), _lib.current_stream())
+                                     _lib.ptr(valid), t, k, d, _lib.ptr(dy), _lib.ptr(dw), _lib.current_stream())
   _lib.check(st, "moe_unpermute_combine_bwd")
   return dy, dw
 

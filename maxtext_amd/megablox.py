@@ -478,11 +478,15 @@ class _BiasFn(torch.autograd.Function):
   @staticmethod
   def backward(ctx, dout):
     (group_sizes,) = ctx.saved_tensors
-    m = dout.shape[0]
-    # segment sums over the rows of each group (the remainder past the last group is one more segment), in a fixed order
-    lengths = torch.cat([group_sizes.long(), (m - group_sizes.sum()).reshape(1).long()])
-    sums = torch.segment_reduce(dout.float(), "sum", lengths=lengths, axis=0, unsafe=True)
-    dbias = sums[ctx.offset : ctx.offset + ctx.g_local].to(ctx.bias_dtype)
+    m, n = dout.shape
+    # per-group column sums of dout = the weight gradient of a matmul with a column of ones: the transposed grouped
+    # matmul clips group sizes that run past the last row exactly as the forward kernels do, in a fixed order
+    if n % 8:
+      raise NotImplementedError("the bias gradient needs a multiple of 8 output channels")
+    ones = torch.ones((m, 8), dtype=torch.bfloat16, device=dout.device)
+    sums = kernels.tgmm(ones, dout.to(torch.bfloat16).contiguous(), group_sizes, num_groups_local=ctx.g_local, group_offset=ctx.offset,
+                        out_dtype=torch.float32)  # [G_local, N, 8], every one of the 8 columns holds the sum
+    dbias = sums[:, :, 0].to(ctx.bias_dtype)
     return dout, dbias, None, None
 
 

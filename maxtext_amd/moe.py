@@ -35,7 +35,7 @@ class MoEConfig:
   topk_routing_group: int = -1
   mlp_activations_limit: float = -1.0
   float32_weight_sum: bool = True
-  float32_gate_logits: bool = True
+  float32_gate_logits: bool = False  # configs/base.yml:198
   shared_experts: int = 0
   # activation quantisation for the grouped GEMMs: None | "int8" | "fp8"
   act_quant: Optional[str] = None
@@ -146,7 +146,7 @@ class RoutedMoE:
   def gate_and_route(self, inputs_2d: torch.Tensor, return_logits: bool = False):
     """-> (weights [T,k] f32, indices [T,k] int32[, gate_logits, pre_bias_logits])."""
     cfg = self.config
-    if cfg.routed_score_func not in ("", "sigmoid"):
+    if cfg.routed_score_func not in ("", "sigmoid", "sqrtsoftplus"):
       raise NotImplementedError(cfg.routed_score_func)
     if self._gate_terms is None or self._gate_terms.device != inputs_2d.device:
       from maxtext_amd.quantizations import split_gate_kernel
@@ -161,7 +161,8 @@ class RoutedMoE:
                                 norm_topk_prob=cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"),
                                 routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups,
                                 topk_routing_group=cfg.topk_routing_group, **common)
-    r = kernels.gate_route(x, self._gate_terms, bias, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob, **common)
+    r = kernels.gate_route(x, self._gate_terms, bias, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob,
+                           weights_round_bf16=cfg.route_mode != "topk_raw", **common)
     return (self._scale_per_expert(r[0], r[1]),) + tuple(r[1:])
 
   def _scale_per_expert(self, w, idx):
@@ -207,7 +208,9 @@ class RoutedMoE:
           routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups,
           topk_routing_group=cfg.topk_routing_group)
     else:
-      w, idx = kernels.route_topk(g2, k=self.num_experts_per_tok, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob)
+      # Llama4's raw logits skip the cast to the layer dtype (moe.py:752-753): they keep the gate's dtype
+      w, idx = kernels.route_topk(g2, k=self.num_experts_per_tok, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob,
+                                  weights_round_bf16=cfg.route_mode != "topk_raw")
       w = self._scale_per_expert(w, idx)
     k = self.num_experts_per_tok
     if torch.is_grad_enabled() and (gate_logits.requires_grad or (pre_bias_logits is not None and pre_bias_logits.requires_grad)):
@@ -244,7 +247,7 @@ class RoutedMoE:
         w = w / (w.sum(-1, keepdim=True) + 1e-20)
       return w * cfg.routed_scaling_factor
     if cfg.route_mode == "topk_raw":
-      w = torch.gather(gate_logits.float(), -1, gi).to(torch.bfloat16)
+      w = torch.gather(gate_logits.float(), -1, gi)  # no cast to the layer dtype for Llama4 (moe.py:752-753)
     elif cfg.route_mode == "softmax_all":
       w = torch.gather(torch.softmax(gate_logits.float(), -1), -1, gi).to(torch.bfloat16)
     else:
@@ -288,10 +291,12 @@ class RoutedMoE:
   # -- unpermute (moe.py:1004-1063), non-ragged branch --------------------------------------
   def unpermute(self, intermediate, sorted_selected_experts, weights, batch_size, sequence_length,
                 use_custom_sort_vjp=True, group_sizes=None, inv_perm=None):
-    if not self.config.float32_weight_sum:
-      raise NotImplementedError("only float32_weight_sum=True is implemented")
     k = self.num_experts_per_tok
     w = weights.reshape(-1, k).float().contiguous()
+    if not self.config.float32_weight_sum:
+      # moe.py:1053-1061 without the casts: a bf16 x bf16 einsum, whose products are exact in the f32 accumulator and whose
+      # result is rounded once -- the same kernel, fed with the weights as the layer dtype holds them
+      w = w.to(torch.bfloat16).float()
     if self.config.decoder_block == "llama4":
       w = torch.ones_like(w)  # the router score already scaled the inputs (moe.py:1051-1052)
     if torch.is_grad_enabled() and (intermediate.requires_grad or w.requires_grad):
@@ -377,7 +382,7 @@ class RoutedMoE:
     routing_inputs = inputs if gate_inputs is None else gate_inputs
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (routing_inputs, self.gate_kernel, self.gate_bias))
-    fused_router = self.tid2eid is None and self.config.routed_score_func in ("", "sigmoid")
+    fused_router = self.tid2eid is None and self.config.routed_score_func in ("", "sigmoid", "sqrtsoftplus")
     if fused_router and not needs_grad and routing_inputs.dtype == torch.bfloat16 and routing_inputs.shape[-1] % 64 == 0 and self.num_experts % 4 == 0:
       want_logits = self.config.load_balance_loss_weight > 0.0  # the auxiliary loss needs the full distribution
       r = self.gate_and_route(routing_inputs.reshape(b * s, -1), return_logits=want_logits)
@@ -404,9 +409,11 @@ def _quantize_tokens(x2d, act_quant):
 class RoutedAndSharedMoE:
   """Routed experts plus always-on shared experts (moe.py:3259-3371).
 
-  The shared expert is one more group that owns every token: its weights are stored as expert
-  index E of the stacked [E+1, N, K] tensors, every token gets it as a (k+1)-th selection with
-  combine weight 1, and the whole layer runs through the same three grouped-GEMM launches.
+  The reference's shared block is one gated MLP of width shared_experts * mlp_dim (moe.py:3317-3321).  Such an MLP is
+  the sum of shared_experts MLPs of width mlp_dim (the activation acts per intermediate channel, `wo` sums over them),
+  so each slice is one more group that owns every token: the stacked [E + S, N, K] tensors hold the routed experts
+  followed by the S slices, every token gets them as selections k .. k + S - 1 with combine weight 1, and the whole
+  layer runs through the same three grouped-GEMM launches.
   """
 
   def __init__(self, config: MoEConfig, wi_0, wi_1, wo, gate_kernel=None, gate_bias=None):
@@ -415,31 +422,48 @@ class RoutedAndSharedMoE:
     self.config = config
     self.routed = RoutedMoE(config, wi_0, wi_1, wo, gate_kernel, gate_bias)
     n_stacked = (wi_0.qvalue if isinstance(wi_0, QArray) else wi_0).shape[0]
-    if n_stacked != config.num_experts + 1:
-      raise ValueError("expert tensors must hold num_experts routed experts followed by the shared expert")
+    if n_stacked != config.num_experts + config.shared_experts:
+      raise ValueError("expert tensors must hold num_experts routed experts followed by shared_experts slices of the shared MLP")
 
-  def sparse_matmul(self, inputs, gate_logits, pre_bias_logits, routing=None):
+  @property
+  def routed_moe(self):
+    return self.routed
+
+  def sparse_matmul(self, inputs, gate_logits, pre_bias_logits, routing=None, input_ids=None):
+    """-> (routed + shared output [B,S,d], lb_loss, bias_updates); the last two are the routed block's (moe.py:3355-3370)."""
     cfg, r = self.config, self.routed
     b, s, d = inputs.shape
-    t, k, e = b * s, cfg.num_experts_per_tok, cfg.num_experts
+    t, k, e, sh = b * s, cfg.num_experts_per_tok, cfg.num_experts, cfg.shared_experts
     x2d = inputs.reshape(t, d).contiguous()
-    w, sel = routing if routing is not None else r.get_topk(gate_logits, pre_bias_logits)
-    sel = torch.cat([sel.reshape(t, k), torch.full((t, 1), e, dtype=torch.int32, device=sel.device)], 1).contiguous()
-    w = torch.cat([w.reshape(t, k), torch.ones((t, 1), dtype=torch.float32, device=w.device)], 1).contiguous()
-    perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + 1, want_sorted_experts=False)
-    inter = r._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, r.wi_0, r.wi_1, r.wo, row_idx=perm, row_idx_div=k + 1)
-    out = kernels.unpermute_combine(inter, w, k=k + 1, inv_perm=inv)
-    return out.reshape(b, s, d), None, None
+    w, sel = routing if routing is not None else r.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
+    routed_sel = sel.reshape(b, s, k)
+    shared_ids = torch.arange(e, e + sh, dtype=torch.int32, device=sel.device).expand(t, sh)
+    sel = torch.cat([sel.reshape(t, k), shared_ids], 1).contiguous()
+    w = torch.cat([w.reshape(t, k).float(), torch.ones((t, sh), dtype=torch.float32, device=w.device)], 1).contiguous()
+    perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + sh, want_sorted_experts=False)
+    inter = r._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, r.wi_0, r.wi_1, r.wo, row_idx=perm, row_idx_div=k + sh)
+    out = kernels.unpermute_combine(inter, w, k=k + sh, inv_perm=inv)
+    lb_loss, bias_updates = r._aux_outputs(gate_logits, routed_sel)
+    return out.reshape(b, s, d), lb_loss, bias_updates
 
-  def __call__(self, inputs, input_ids=None, gate_inputs=None, out_sharding=None):
+  def __call__(self, inputs, original_inputs=None, gate_inputs=None, intermediate_sharding=None, out_sharding=None, input_ids=None):
+    """-> (output, lb_loss, bias_updates), as moe.py:3338-3371: the gate reads gate_inputs when given, hash routing
+    (a RoutedMoE with tid2eid set) reads input_ids."""
+    del original_inputs, intermediate_sharding, out_sharding
+    r = self.routed
     b, s, d = inputs.shape
-    if inputs.dtype == torch.bfloat16 and d % 64 == 0 and cfg_ok(self.config):
-      return self.sparse_matmul(inputs, None, None, routing=self.routed.gate_and_route(inputs.reshape(b * s, -1)))
-    gate_logits, pre_bias = self.routed.gate(inputs.reshape(b * s, -1))
+    routing_inputs = inputs if gate_inputs is None else gate_inputs
+    fused = r.tid2eid is None and routing_inputs.dtype == torch.bfloat16 and routing_inputs.shape[-1] % 64 == 0 and cfg_ok(self.config)
+    if fused:
+      want_logits = self.config.load_balance_loss_weight > 0.0  # the auxiliary loss needs the full distribution
+      g = r.gate_and_route(routing_inputs.reshape(b * s, -1), return_logits=want_logits)
+      logits = g[2].reshape(b, s, -1) if want_logits else None
+      return self.sparse_matmul(inputs, logits, None, routing=(g[0], g[1]))
+    gate_logits, pre_bias = r.gate(routing_inputs.reshape(b * s, -1))
     pre_bias = None if pre_bias is None else pre_bias.reshape(b, s, -1)
-    return self.sparse_matmul(inputs, gate_logits.reshape(b, s, -1), pre_bias)
+    return self.sparse_matmul(inputs, gate_logits.reshape(b, s, -1), pre_bias, input_ids=input_ids)
 
 
 def cfg_ok(cfg: MoEConfig) -> bool:
   """Whether moe_gate_route covers this configuration's router."""
-  return cfg.num_experts % 4 == 0 and cfg.routed_score_func in ("", "sigmoid")
+  return cfg.num_experts % 4 == 0 and cfg.routed_score_func in ("", "sigmoid", "sqrtsoftplus")

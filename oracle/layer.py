@@ -17,6 +17,8 @@ from oracle import moe_oracle as O
 def oracle_rhs(qvalue: torch.Tensor, scale: torch.Tensor, qtype: str, n: int):
   """Weights in the kernels' HBM layout ([G,N,K] K-contiguous; scales [G,N] / [G,N/128,K/128] /
   [G,N,K/128]) -> (rhs [g,k,n], rhs_scale in the reference's v2 layout [g,nb,1,n], quant_block)."""
+  if qtype == "bf16":  # unquantised weights [G, N, K]
+    return qvalue.cpu().transpose(1, 2), None, None
   qv, sc = qvalue.cpu(), scale.cpu()
   if qtype == "int8":
     return qv.transpose(1, 2), sc, None
@@ -46,10 +48,12 @@ def oracle_layer(x, gate_logits, pre_bias_logits, wi_0, wi_1, wo, *, num_experts
     w, idx = O.get_topk(logits, k=k, norm_topk_prob=norm_topk_prob)
   n_exp = e
   if shared_experts:
-    # the shared expert (moe.py:3360-3371) as one more group owning every token with weight 1
-    idx = np.concatenate([idx, np.full((idx.shape[0], 1), e, np.int32)], 1)
-    w = np.concatenate([w, np.ones((w.shape[0], 1), np.float32)], 1)
-    n_exp, k = e + 1, k + 1
+    # the shared MLP (moe.py:3317-3321, :3360-3371), width shared_experts * mlp_dim, as shared_experts slices of width
+    # mlp_dim: each is one more group owning every token with weight 1
+    t_ = idx.shape[0]
+    idx = np.concatenate([idx, np.broadcast_to(np.arange(e, e + shared_experts, dtype=np.int32), (t_, shared_experts))], 1)
+    w = np.concatenate([w, np.ones((t_, shared_experts), np.float32)], 1)
+    n_exp, k = e + shared_experts, k + shared_experts
   r0, s0, qb = oracle_rhs(*wi_0, f)
   r1, s1, _ = oracle_rhs(*wi_1, f)
   ro, so, _ = oracle_rhs(*wo, d)

@@ -35,6 +35,12 @@ How each function is pinned (see tests/test_oracle_*.py):
       nibble order and 2^(s-127) scaling on hand-made blocks; quantize_mxfp4 (a test-data generator only) by
       dequantize(quantize(x)) == x on representable inputs.
 
+  ragged_gather / ragged_gather_reduce / weighted_intermediate
+      hand-made rows: a NaN row behind a cleared mask bit stays out of the sum, a group with every row masked
+      gives zeros, the f32 sum rounds once (a case where rounding each term first gives another result), equality
+      with unpermute when every row is valid, double rounding of the weighted activation on a value that
+      separates it from a single rounding.
+
   quantize_lhs_v2 / manual_quantize (the quantisers whose source IS in the reference tree)
       hand cases worked out in exact rational arithmetic (python Fractions with an explicit round-to-nearest-even
       to the 8-bit / 24-bit significand) that separate truncation from round-half-even and round-half-away,
@@ -121,6 +127,8 @@ def gate_logits(x: torch.Tensor, kernel: torch.Tensor, bias=None, *, score_func:
     out = (x.to(torch.bfloat16).double() @ kernel.to(torch.bfloat16).double()).to(torch.bfloat16).float()
   if score_func == "sigmoid":
     out = torch.sigmoid(out)
+  elif score_func == "sqrtsoftplus":  # linears.py:51-53: jnp.sqrt(jax.nn.softplus(x)), softplus = logaddexp(x, 0)
+    out = torch.from_numpy(np.sqrt(np.logaddexp(out.numpy(), np.float32(0))).astype(np.float32))
   elif score_func:
     raise ValueError(score_func)
   pre = out.clone() if deepseek else None
@@ -172,8 +180,11 @@ def get_topk(
   if mode not in ("softmax_topk", "topk_raw", "softmax_all"):
     raise ValueError(f"unknown routing mode {mode}")
   vals, idx = top_k(gate_logits, k)
-  if mode == "topk_raw":  # Llama4: no softmax over the selected logits (moe.py:753 is skipped for LLAMA4)
+  if mode == "topk_raw":
+    # Llama4: the selected logits themselves; the softmax and its cast to the layer dtype (moe.py:753) are skipped, so
+    # the weights keep the gate's dtype, i.e. the values handed in stay as they are
     w = vals.astype(np.float32)
+    weight_dtype = "gate"
   elif mode == "softmax_all":  # Gemma4: softmax over all experts, gathered at the indices (moe.py:742-745)
     w = np.take_along_axis(_softmax_f32(gate_logits), idx, axis=-1)
   else:
@@ -249,6 +260,38 @@ def unroute_sum(tokens: torch.Tensor, selected_experts: np.ndarray):
   inds = np.argsort(np.argsort(selected_experts.reshape(-1), kind="stable"), kind="stable")
   g = tokens[torch.from_numpy(inds.astype(np.int64))]
   return g.reshape(t, k, -1).sum(1)
+
+
+def ragged_gather(x: torch.Tensor, indices: np.ndarray, start=None, end=None, weights=None):
+  """kernels/ragged/ragged_gather.py:310-320: out = x[indices], times weights[:, None] when given (the product
+  is formed in the promoted type of the two and returned in it; callers keep bf16 by passing bf16 weights).
+  [start, end) (ragged_gather.py:357-376) names the output rows a caller will use; the reference leaves the
+  others unspecified, this restatement writes zeros there."""
+  out = x[torch.from_numpy(np.asarray(indices, dtype=np.int64))]
+  if weights is not None:
+    out = out * weights[:, None]
+  if start is not None:
+    rows = torch.arange(out.shape[0])
+    out = torch.where(((rows >= int(start)) & (rows < int(end)))[:, None], out, torch.zeros_like(out))
+  return out
+
+
+def ragged_gather_reduce(x: torch.Tensor, indices: np.ndarray, topk_weights: torch.Tensor, valid_rows_mask: np.ndarray,
+                         reduce_group_size: int):
+  """kernels/ragged/ragged_gather_reduce_v2.py:170-182: gather, weight in f32, zero the rows that are not valid,
+  sum each run of reduce_group_size consecutive rows in f32, round once to bf16.  (`where` drops a masked row
+  whatever it holds, NaN included.)"""
+  out = x[torch.from_numpy(np.asarray(indices, dtype=np.int64))].to(torch.float32) * topk_weights.to(torch.float32)[:, None]
+  out = torch.where(torch.from_numpy(np.asarray(valid_rows_mask, dtype=bool))[:, None], out, torch.zeros_like(out))
+  out = out.reshape(-1, reduce_group_size, out.shape[-1])
+  return out.sum(1).to(torch.bfloat16)
+
+
+def weighted_intermediate(h0: torch.Tensor, h1: torch.Tensor, weights: torch.Tensor, kind: str = "silu", limit: float = 7.0):
+  """models/deepseek_batchsplit_fp8.py:1048-1049: the routing weight of each sorted row multiplies the finished
+  bf16 activation before `wo` (the combine after it is then an unweighted sum): bf16(bf16(act(h0, h1)) * w)."""
+  act = apply_ffn_activation(h0, h1, kind, limit, out_dtype=torch.bfloat16)
+  return (act.to(torch.float32) * weights.to(torch.float32)[:, None]).to(torch.bfloat16)
 
 
 # --------------------------------------------------------------------------

@@ -220,6 +220,79 @@ def test_unpermute_combine(K, t, k, d):
   assert relerr(got3, O.unroute_sum(y.float(), sel)) <= 2.0**-8
 
 
+def test_gather_rows_weighted_and_ranged(K):
+  """The weighted ragged gather (ragged_gather.py:310-320) and its [start, end) window, bit for bit."""
+  g = torch.Generator().manual_seed(12)
+  r_in, r_out, d = 300, 700, 1024
+  x = torch.randn(r_in, d, generator=g).to(torch.bfloat16)
+  x[5] = float("nan")
+  idx = torch.randint(0, r_in, (r_out,), generator=g).to(torch.int32)
+  idx[10], idx[650] = 5, 5  # the NaN row: once inside the window, once outside
+  w = torch.rand(r_out, generator=g).to(torch.bfloat16)
+  def same_bits(a, b):  # NaN payloads are not part of the contract: NaN where NaN is expected, identical bits elsewhere
+    return torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a).view(torch.int16), torch.nan_to_num(b).view(torch.int16))
+
+  want = O.ragged_gather(x, idx.numpy(), weights=w)
+  got = K.gather_rows(cuda(x), cuda(idx), 1, row_weight=cuda(w.float())).cpu()
+  assert got.dtype == torch.bfloat16 and same_bits(got, want)
+  rng_ = torch.tensor([9, 600], dtype=torch.int32)
+  want = O.ragged_gather(x, idx.numpy(), 9, 600, weights=w)
+  got = K.gather_rows(cuda(x), cuda(idx), 1, row_weight=cuda(w.float()), row_range=cuda(rng_)).cpu()
+  assert same_bits(got, want)
+  assert got[:9].abs().max() == 0 and got[600:].abs().max() == 0 and torch.isnan(got[10]).all()
+  # the window applies before quantisation too: rows outside it quantise to zeros with a zero scale
+  q, sc = K.gather_rows(cuda(x), cuda(idx), 1, out_dtype=torch.int8, row_range=cuda(rng_))
+  assert q[600:].abs().max() == 0 and sc[600:].abs().max() == 0
+
+
+@pytest.mark.parametrize("t,k,d", [(64, 8, 512), (300, 2, 4096), (33, 9, 64)])
+def test_combine_valid_rows_mask(K, t, k, d):
+  """Gather-reduce with a mask of valid rows (ragged_gather_reduce_v2.py:170-182): masked rows are left out whatever
+  they hold; integer data keeps the f32 sums exact."""
+  rng = np.random.default_rng(t * k)
+  e = 16
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  y = torch.from_numpy(rng.integers(-8, 9, (t * k, d)).astype(np.float32)).to(torch.bfloat16)
+  w = rng.integers(0, 3, (t, k)).astype(np.float32)
+  mask = rng.random((t, k)) < 0.7
+  mask[0] = False  # a token with no valid row at all
+  perm, inv, _, _ = K.sort_by_expert(cuda(sel), e)
+  inv_h = inv.cpu().numpy()
+  y[inv_h[~mask.reshape(-1)]] = float("nan")  # every masked row holds NaN
+  want = O.ragged_gather_reduce(y, inv_h, torch.from_numpy(w).reshape(-1), mask.reshape(-1), k)
+  got = K.unpermute_combine(cuda(y), cuda(w), k=k, inv_perm=inv, valid_rows_mask=cuda(torch.from_numpy(mask)))
+  assert torch.equal(got.cpu(), want) and got[0].abs().max() == 0
+  # gradient: masked rows get zeros, the others w * dout; dweights of masked entries are zero
+  dout = torch.from_numpy(rng.integers(-4, 5, (t, d)).astype(np.float32)).to(torch.bfloat16)
+  dy, dw = K.unpermute_combine_bwd(cuda(dout), cuda(y), cuda(w), k=k, inv_perm=inv, valid_rows_mask=cuda(torch.from_numpy(mask)))
+  rows = torch.from_numpy(inv_h.astype(np.int64))
+  want_dy = torch.zeros(t * k, d)
+  want_dy[rows] = (torch.from_numpy(w * mask).reshape(-1, 1) * dout.float().repeat_interleave(k, 0))
+  assert torch.equal(dy.cpu().float(), want_dy)
+  y0 = torch.nan_to_num(y.float(), nan=0.0)
+  want_dw = (y0[rows].reshape(t, k, d) * dout.float()[:, None, :]).sum(-1) * torch.from_numpy(mask)
+  assert torch.equal(dw.cpu(), want_dw)
+
+
+def test_gmm_weight_before_wo(K):
+  """The batch-split rule (deepseek_batchsplit_fp8.py:1048-1049): the routing weight multiplies the finished bf16
+  activation inside the first matmul's epilogue; against the oracle's gmm + weighted_intermediate."""
+  g = torch.Generator().manual_seed(8)
+  m, k, n = 640, 512, 384
+  gs = np.array([300, 0, 211, 100], np.int32)  # 29 rows in no group
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w0 = (torch.randn(4, n, k, generator=g) * 0.05).to(torch.bfloat16)
+  w1 = (torch.randn(4, n, k, generator=g) * 0.05).to(torch.bfloat16)
+  rw = (torch.rand(m, generator=g) * 2.5).to(torch.bfloat16)
+  h0 = O.gmm(lhs, w0.transpose(1, 2), gs, out_dtype=torch.bfloat16)
+  h1 = O.gmm(lhs, w1.transpose(1, 2), gs, out_dtype=torch.bfloat16)
+  want = O.weighted_intermediate(h0, h1, rw)
+  got = K.gmm_raw(cuda(lhs), cuda(w0), cuda(gs), rhs_up=cuda(w1), act="silu", out_row_scale=cuda(rw.float()))
+  assert relerr(got, want) <= TOL
+  plain = K.gmm_raw(cuda(lhs), cuda(w0), cuda(gs), rhs_up=cuda(w1), act="silu")
+  assert torch.equal(got, (plain.float() * cuda(rw.float())[:, None]).to(torch.bfloat16))
+
+
 def test_combine_exact_on_integers(K):
   # integer-valued bf16 inputs make the f32 accumulation exact (trick of tests/gather_reduce_sc_test.py:68)
   rng = np.random.default_rng(0)
@@ -722,6 +795,26 @@ def test_gate_route_deepseek_sigmoid_bias(K, groups):
   # routing on the kernel's own scores must equal the oracle's routing on the same scores, bit for bit
   ow, oidx = O.get_topk(logits.cpu().numpy(), pre.cpu().numpy(), k=k, mode="deepseek", routed_scaling_factor=2.5,
                         n_routing_groups=groups[0], topk_routing_group=groups[1])
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+  np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=1e-5)
+
+
+def test_gate_route_sqrtsoftplus(K):
+  """The DeepSeek-V4 router's score function sqrt(softplus(x)) (linears.py:51-53) inside moe_gate_route."""
+  from maxtext_amd.quantizations import split_gate_kernel
+
+  g = torch.Generator().manual_seed(35)
+  t, d, e, k = 300, 1024, 64, 6
+  x = torch.randn(t, d, generator=g).to(torch.bfloat16)
+  x[0] *= 40.0  # logits far out on both sides: sqrt(x) above, exp(x / 2) below
+  wg = torch.randn(d, e, generator=g) * 0.05
+  w, idx, logits, pre = K.gate_route(cuda(x), cuda(split_gate_kernel(wg)), k=k, score_func="sqrtsoftplus", mode="deepseek",
+                                     norm_topk_prob=True, routed_scaling_factor=1.5, return_logits=True)
+  want_logits, want_pre = O.gate_logits(x, wg, score_func="sqrtsoftplus", deepseek=True)
+  np.testing.assert_allclose(pre.cpu().numpy(), want_pre, rtol=2e-5, atol=1e-30)
+  assert torch.equal(logits, pre)  # no bias
+  ow, oidx = O.get_topk(logits.cpu().numpy(), pre.cpu().numpy(), k=k, mode="deepseek", routed_score_func="sqrtsoftplus",
+                        routed_scaling_factor=1.5)
   np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
   np.testing.assert_allclose(w.cpu().numpy(), ow, rtol=1e-5)
 

@@ -199,7 +199,7 @@ def test_layer_gradients_match_torch_autograd(norm_topk_prob):
   w1 = (torch.randn(e, f, d, generator=g) * 0.08).to(torch.bfloat16)
   wo = (torch.randn(e, d, f, generator=g) * 0.08).to(torch.bfloat16)
   dout = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, norm_topk_prob=norm_topk_prob)
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, norm_topk_prob=norm_topk_prob)
   leaves = [v.cuda().requires_grad_() for v in (x, wg, w0, w1, wo)]
   xg, wgg, w0g, w1g, wog = leaves
   block = moe.RoutedMoE(cfg, w0g, w1g, wog, gate_kernel=wgg)
@@ -247,7 +247,7 @@ def test_layer_gradients_with_int8_quantised_forward():
   x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
   logits = torch.randn(1, t, e, generator=g)
   ws = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
   grads = {}
   for q in (None, "int8"):
     leaves = [v.cuda().requires_grad_() for v in [x] + ws]
@@ -272,7 +272,7 @@ def test_layer_gradients_with_expert_biases():
   w0, w1, wo = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
   b0, b1, bo = torch.randn(e, f, generator=g) * 0.5, torch.randn(e, f, generator=g) * 0.5, torch.randn(e, d, generator=g) * 0.5
   dout = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
   leaves = [v.cuda().requires_grad_() for v in (x, w0, w1, wo, b0, b1, bo)]
   block = moe.RoutedMoE(cfg, *leaves[1:4])
   out, _, _ = block.sparse_matmul(leaves[0], logits.cuda(), None, *leaves[1:4], *leaves[4:])
@@ -345,12 +345,12 @@ def test_layer_call_routes_through_gate_route(deepseek):
   bias = (torch.randn(e, generator=g) * 0.1).cuda() if deepseek else None
   ws = [(torch.randn(e + (1 if deepseek else 0), n_, k_, generator=g) * 0.05).to(torch.bfloat16).cuda() for n_, k_ in ((f, d), (f, d), (d, f))]
   if deepseek:
-    cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek3-test",
+    cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek3-test",
                         routed_score_func="sigmoid", routed_bias=True, routed_scaling_factor=2.5, shared_experts=1)
     block = moe.RoutedAndSharedMoE(cfg, *ws, gate_kernel=wg, gate_bias=bias)
     routed = block.routed
   else:
-    cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
+    cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f)
     block = routed = moe.RoutedMoE(cfg, *ws, gate_kernel=wg)
   out, _, _ = block(x)
   w, idx, logits, pre = routed.gate_and_route(x.reshape(t, d), return_logits=True)
@@ -375,7 +375,7 @@ def test_gpt_oss_style_layer_with_mlp_bias():
   w0, w1 = [(torch.randn(e, f, d, generator=g) * 0.1).to(torch.bfloat16) for _ in range(2)]
   wo = (torch.randn(e, d, f, generator=g) * 0.1).to(torch.bfloat16)
   b0, b1, bo = torch.randn(e, f, generator=g) * 0.3, torch.randn(e, f, generator=g) * 0.3, torch.randn(e, d, generator=g) * 0.3
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, decoder_block="gpt_oss", mlp_activations_limit=7.0)
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, decoder_block="gpt_oss", mlp_activations_limit=7.0)
   block = moe.RoutedMoE(cfg, w0.cuda(), w1.cuda(), wo.cuda())
   out, _, _ = block.sparse_matmul(x.cuda(), logits.cuda(), None, w0.cuda(), w1.cuda(), wo.cuda(), b0.cuda(), b1.cuda(), bo.cuda())
   w, idx = block.get_topk(logits.cuda())
@@ -408,7 +408,7 @@ def test_auxiliary_outputs_match_reference_formulas():
   x = torch.randn(b, s_, d, generator=g).to(torch.bfloat16).cuda()
   logits = torch.randn(b, s_, e, generator=g).cuda()
   ws = [(torch.randn(e, n_, k_, generator=g) * 0.05).to(torch.bfloat16).cuda() for n_, k_ in ((f, d), (f, d), (d, f))]
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, load_balance_loss_weight=0.01,
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, load_balance_loss_weight=0.01,
                       routed_bias=True, routed_bias_update_rate=0.001)
   block = moe.RoutedMoE(cfg, *ws)
   out, lb, upd = block.sparse_matmul(x, logits, None, *ws)
@@ -448,7 +448,7 @@ def test_llama4_and_gemma4_style_layers():
     return torch.einsum("tf,tdf->td", torch.nn.functional.silu(h0) * h1, ws[2].double()[ex])
 
   # Llama4
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=1, emb_dim=d, moe_mlp_dim=f, decoder_block="llama4")
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=1, emb_dim=d, moe_mlp_dim=f, decoder_block="llama4")
   block = moe.RoutedMoE(cfg, *[w.cuda() for w in ws])
   out, _, _ = block.sparse_matmul(x.cuda(), logits.cuda(), None, *[w.cuda() for w in ws])
   top = logits.reshape(t, e).max(-1)
@@ -457,7 +457,7 @@ def test_llama4_and_gemma4_style_layers():
   assert relerr(out.reshape(t, d), want) <= TOL
   # Gemma4
   k = 2
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, decoder_block="gemma4", norm_topk_prob=True)
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, decoder_block="gemma4", norm_topk_prob=True)
   block = moe.RoutedMoE(cfg, *[w.cuda() for w in ws])
   block.per_expert_scale = scale.cuda()
   out, _, _ = block.sparse_matmul(x.cuda(), logits.cuda(), None, *[w.cuda() for w in ws])
@@ -484,7 +484,7 @@ def test_hash_routed_layer():
   ws = [(torch.randn(e, n_, k_, generator=g) * 0.08).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
   table = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(vocab)]).float()
   ids = torch.randint(0, vocab, (1, t), generator=g)
-  cfg = moe.MoEConfig(num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek4", decoder_block="deepseek4",
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek4", decoder_block="deepseek4",
                       routed_score_func="sqrtsoftplus", routed_scaling_factor=1.5)
   assert cfg.is_deepseek
   block = moe.RoutedMoE(cfg, *[w.cuda() for w in ws], gate_kernel=wg.cuda())
@@ -503,3 +503,44 @@ def test_hash_routed_layer():
     h1 = torch.einsum("td,tfd->tf", x2, ws[1].double()[ex])
     want += torch.as_tensor(ow[:, s_ : s_ + 1]).double() * torch.einsum("tf,tdf->td", torch.nn.functional.silu(h0) * h1, ws[2].double()[ex])
   assert relerr(out.reshape(t, d), want) <= 2e-2
+
+
+def test_routed_and_shared_block_with_two_shared_experts_gate_inputs_and_aux_outputs():
+  """RoutedAndSharedMoE.__call__ (moe.py:3338-3371): the shared MLP of width shared_experts * mlp_dim as that many
+  stacked slices, the gate reading gate_inputs, and the routed block's auxiliary outputs handed through.  Expected
+  value: the routed layer of the oracle plus a dense gated MLP of width 2 f in f64."""
+  from maxtext_amd import moe
+
+  g = torch.Generator().manual_seed(90)
+  t, d, f, e, k, sh = 192, 256, 128, 8, 2, 2
+  x = torch.randn(1, t, d, generator=g).to(torch.bfloat16)
+  gate_in = torch.randn(1, t, d, generator=g).to(torch.bfloat16)  # the router looks at other activations than the experts
+  wg = torch.randn(d, e, generator=g) * 0.1
+  bias = torch.randn(e, generator=g) * 0.1
+  ws = [(torch.randn(e + sh, n_, k_, generator=g) * 0.05).to(torch.bfloat16) for n_, k_ in ((f, d), (f, d), (d, f))]
+  cfg = moe.MoEConfig(float32_gate_logits=True, num_experts=e, num_experts_per_tok=k, emb_dim=d, moe_mlp_dim=f, model_name="deepseek3-test",
+                      routed_score_func="sigmoid", routed_bias=True, routed_scaling_factor=2.5, shared_experts=sh,
+                      load_balance_loss_weight=0.01, routed_bias_update_rate=0.001)
+  block = moe.RoutedAndSharedMoE(cfg, *[w.cuda() for w in ws], gate_kernel=wg.cuda(), gate_bias=bias.cuda())
+  out, lb, upd = block(x.cuda(), gate_inputs=gate_in.cuda())
+  # routing as the block saw it, from gate_inputs
+  w_r, idx, logits, pre = block.routed.gate_and_route(gate_in.cuda().reshape(t, d), return_logits=True)
+  want_logits, want_pre = O.gate_logits(gate_in.reshape(t, d), wg, bias, score_func="sigmoid", deepseek=True)
+  assert np.abs(logits.cpu().numpy() - want_logits).max() <= 1e-5
+  from oracle.layer import oracle_layer as run_oracle
+
+  trip = lambda w: (w[:e], None, "bf16")
+  routed, oidx, _, _ = run_oracle(x, logits.cpu(), pre.cpu(), trip(ws[0]), trip(ws[1]), trip(ws[2]), num_experts=e, k=k, emb_dim=d, mlp_dim=f,
+                                    deepseek=True, routed_scaling_factor=2.5)
+  np.testing.assert_array_equal(idx.cpu().numpy(), oidx)
+  x64 = x.reshape(t, d).double()
+  w0s, w1s, wos = ws[0][e:].double().reshape(sh * f, d), ws[1][e:].double().reshape(sh * f, d), ws[2][e:].double()
+  inter = torch.nn.functional.silu(x64 @ w0s.T) * (x64 @ w1s.T)  # [t, sh * f]: one MLP of width 2 f
+  shared = inter @ torch.cat([wos[i] for i in range(sh)], 1).T
+  want = routed.double() + shared
+  assert relerr(out.reshape(t, d), want) <= 2e-2
+  # auxiliary outputs are the routed block's own
+  _, lb_r, upd_r = block.routed.sparse_matmul(x.cuda(), logits.reshape(1, t, e), pre.reshape(1, t, e), *[w.cuda()[:e].contiguous() for w in ws])
+  assert lb is not None and upd is not None and torch.equal(lb, lb_r) and torch.equal(upd, upd_r)
+  with pytest.raises(ValueError):
+    moe.RoutedAndSharedMoE(cfg, *[w.cuda()[: e + 1] for w in ws])

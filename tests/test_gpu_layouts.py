@@ -258,3 +258,8 @@ def test_gmm_row_index_row_scale_and_f32_out_in_every_kernel_family(K, case):
   scaled = K.gmm_raw(cuda(lhs_t), cuda(args["rhs"]), cuda(gs), lhs_row_idx=cuda(src), lhs_row_idx_div=k, out_row_scale=cuda(rowf), **idx_kw)
   assert relerr(scaled, want_g.float() * rowf[:, None]) <= TOL
   assert torch.all(scaled[int(gs.sum()):] == 0)
+  # the factor multiplies the finished bf16 result (deepseek_batchsplit_fp8.py:1048-1049): two roundings, bit for bit
+  assert torch.equal(scaled, (via_idx.float() * cuda(rowf)[:, None]).to(torch.bfloat16))
+  scaled32 = K.gmm_raw(cuda(lhs_t), cuda(args["rhs"]), cuda(gs), lhs_row_idx=cuda(src), lhs_row_idx_div=k, out_row_scale=cuda(rowf),
+                       out_dtype=torch.float32, **idx_kw)
+  assert relerr(scaled32, want_g.float() * rowf[:, None]) <= 2e-3

@@ -1,6 +1,8 @@
 """Pins the CPU oracle against the reference's own known answers and against
 independent formulations (brute force, closed forms, second code paths)."""
 
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -651,3 +653,49 @@ def test_gmm_with_v2_scale_layouts_equals_dequantised_matmul():
   want[:7] = lq[:7].double() @ rq[0].double()
   want[7:] = lq[7:].double() @ rq[2].double()
   torch.testing.assert_close(got, want * 0.25 * shared[0, 0].double(), rtol=1e-12, atol=1e-9)
+
+
+def test_gate_logits_sqrtsoftplus_closed_forms():
+  """sqrt(softplus(x)) (linears.py:51-53): sqrt(ln 2) at 0, sqrt(x) far above, exp(x / 2) far below."""
+  x = torch.tensor([[1.0, 0.0, 0.0]]).to(torch.bfloat16)
+  kernel = torch.tensor([[0.0, 50.0, -50.0], [0.0, 0.0, 0.0], [0.0, 0.0, 0.0]])
+  out, pre = O.gate_logits(x, kernel, score_func="sqrtsoftplus", deepseek=True)
+  np.testing.assert_allclose(out[0], [math.sqrt(math.log(2.0)), math.sqrt(50.0), math.exp(-25.0)], rtol=1e-6)
+  assert np.array_equal(out, pre)
+
+
+def test_ragged_variants_hand_cases():
+  """ragged_gather (ragged_gather.py:310-320), ragged_gather_reduce (ragged_gather_reduce_v2.py:170-182) and the
+  weight-before-wo rule (deepseek_batchsplit_fp8.py:1048-1049) on rows worked out by hand."""
+  x = torch.tensor([[1.0, 2.0], [10.0, 20.0], [100.0, 200.0], [float("nan"), 7.0]]).to(torch.bfloat16)
+  # gather with weights: row i of the output is x[indices[i]] * weights[i]
+  got = O.ragged_gather(x, np.array([2, 0, 0, 1]), weights=torch.tensor([0.5, 2.0, 1.0, 0.25]).to(torch.bfloat16))
+  assert got.dtype == torch.bfloat16 and got.tolist() == [[50.0, 100.0], [2.0, 4.0], [1.0, 2.0], [2.5, 5.0]]
+  # rows outside [start, end) come back as zeros, NaN source rows included
+  got = O.ragged_gather(x, np.array([3, 1, 2, 3]), start=1, end=3)
+  assert got.tolist() == [[0.0, 0.0], [10.0, 20.0], [100.0, 200.0], [0.0, 0.0]]
+  # gather-reduce: groups of 2; the NaN row sits behind a cleared mask bit; group 2 has no valid row
+  idx = np.array([0, 1, 3, 2, 3, 3])
+  w = torch.tensor([1.0, 0.5, 9.0, 0.25, 1.0, 1.0])
+  mask = np.array([1, 1, 0, 1, 0, 0], bool)
+  got = O.ragged_gather_reduce(x, idx, w, mask, 2)
+  assert got.dtype == torch.bfloat16 and got.tolist() == [[6.0, 12.0], [25.0, 50.0], [0.0, 0.0]]
+  # one rounding at the end: 256 + 1 + 1 = 258 in f32 -> bf16 258, where rounding after every addition would stay at 256
+  x2 = torch.tensor([[256.0], [1.0]]).to(torch.bfloat16)
+  got = O.ragged_gather_reduce(x2, np.array([0, 1, 1]), torch.ones(3), np.ones(3, bool), 3)
+  assert got.tolist() == [[258.0]]
+  # with every row valid it is unpermute (moe.py:1039-1063) under another name
+  g = torch.Generator().manual_seed(3)
+  t, k, d = 7, 3, 16
+  y = torch.randn(t * k, d, generator=g).to(torch.bfloat16)
+  perm = np.random.default_rng(0).permutation(t * k).astype(np.int32)
+  wts = torch.rand(t, k, generator=g)
+  inv = np.argsort(perm, kind="stable")
+  a = O.ragged_gather_reduce(y, inv, wts.reshape(-1), np.ones(t * k, bool), k)
+  assert torch.equal(a, O.unpermute(y, perm, wts.numpy(), k))
+  # weight before wo: silu(33) = 33 in f32, 33 * 1.015625 = 33.515625 -> bf16 33.5; 33.5 * 1.75 = 58.625 is a tie ->
+  # 58.5 (even); a single rounding of 33.515625 * 1.75 = 58.652... would have given 58.75
+  h0 = torch.tensor([[33.0]]).to(torch.bfloat16)
+  h1 = torch.tensor([[1.015625]]).to(torch.bfloat16)
+  got = O.weighted_intermediate(h0, h1, torch.tensor([1.75]))
+  assert got.tolist() == [[58.5]]
