@@ -145,7 +145,7 @@ static int scratch_of(void** ptr) {
 // tile map and for the launch.
 enum TiledKind { K_T64, K_T128, K_T256, K_DL128, K_DL64, K_DLW };
 
-static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N, int G_total, bool wq_kmajor = false) {
+static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N, int G_total, bool wq_kmajor = false, long long indexed_lhs_rows = 0) {
   // full 256-row tiles for prefill, 64 otherwise; a problem with fewer 256 x 256 tiles than half the CUs of the chip also
   // takes the 64-row tiles, which quadruples its blocks
   const long long tiles_big = (long long)max_tiles_for(M, G_total, 256) * cdiv(N, glu ? 128 : 256);
@@ -158,7 +158,7 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
   // weight-only formats on shapes their direct-to-LDS kernel does not take (K % 64 != 0, K-major scales) stay on the
   // register-staged kernel, whose 128-row tiles are ahead of its 256-row tiles up to 200 rows per expert
-  const bool dlw_ok = bsrc != BSRC_SAME && K % 64 == 0 && !wq_kmajor;
+  const bool dlw_ok = bsrc != BSRC_SAME && dlw_takes(K, N, indexed_lhs_rows, wq_kmajor);
   const bool mid_wq = bsrc != BSRC_SAME && !dlw_ok && (long long)M >= 32LL * G_total && (long long)M < 200LL * G_total;
   const int esz = op == OP_I8 ? 1 : 2;
   if (mid || mid_wq) return K_T128;
@@ -459,7 +459,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     map_tiles(256);
     return launch_dl(op, glu, 64, false, p, M, G, s);
   }
-  TiledKind kind = kernel == MOE_GMM_KERNEL_BIG ? K_T256 : pick_tiled_kind(op, bsrc, glu, M, K, N, G, wq_kmajor);
+  TiledKind kind = kernel == MOE_GMM_KERNEL_BIG ? K_T256 : pick_tiled_kind(op, bsrc, glu, M, K, N, G, wq_kmajor, a->lhs_row_idx ? ro.lhs_rows : 0);
   if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64 || kind == K_DLW)) kind = K_T256;
   map_tiles(tiled_kind_bm(kind));
   return launch_tiled_kind(kind, op, bsrc, glu, p, M, G, s);

@@ -409,6 +409,8 @@ int launch_tiled_bm(int op, int bsrc, bool glu, int bm, bool block_scaled, const
 int launch_dl(int op, bool glu, int stage_bytes, bool rhs_kn, const TiledParams& p, int M, int G_total, hipStream_t s);
 // moe_gmm_dlw.hip: the same pipeline for bf16 activations x int8 / int4 / mxfp4 weights (K % 64 == 0, default scale layouts)
 int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
+// whether that kernel takes the shape (indexed_lhs_rows: rows of lhs when a row index is used, else 0)
+bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor);
 // moe_gmm_fp8.hip
 int launch_fp8_tiled(bool big, bool glu, bool vec4, const Fp8TiledParams& P, int M, int G_total, hipStream_t s);
 int launch_fp8_skinny(bool few_rows, const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s);

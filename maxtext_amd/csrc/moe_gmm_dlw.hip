@@ -1,13 +1,20 @@
 // Grouped matmul: the persistent 256 x 256 kernel for bf16 activations x int8 / int4 / mxfp4 weights (prefill).
 //
-// The pipeline of gmm_dl_kernel (moe_gmm_dl.hip) with a weight side of its own.  Activations go global -> LDS without
-// passing through registers (global_load_lds_dwordx4, 8 rows x 128 B per wave instruction, XOR-swizzled unpadded rows, two
-// buffers of 64 KB).  Weights cannot: their bytes have to become bf16 on the way.  Each thread therefore keeps the raw
-// bytes of its share of one stage in registers (int8: 2 x 16 B, 4-bit formats: 16 B): they are requested one stage before
-// they are needed, widened to bf16 (4-bit formats: multiplied by their group scale) and written into the swizzled LDS rows
-// in the shadow of the MFMAs of the k-step in which the activation requests of the same stage go out, i.e. right after the
-// barrier that proves the buffer free.  A weight is widened once per block (by one of 512 threads), not once per wave, and
-// the fragment reads, the MFMA schedule and the epilogue are those of the bf16 x bf16 kernel.
+// Both operands go global -> LDS without passing through registers (buffer_load ... lds, 1 KB per wave instruction):
+// the activations as XOR-swizzled rows of 128 bytes (64 bf16 values of K), the weights as the RAW bytes of the
+// checkpoint format (64 or 32 bytes per row and stage).  A weight becomes bf16 only in the registers of the wave that
+// multiplies it: each of the 8 waves owns 32 of the tile's 256 weight rows for all 256 activation rows (16 x 2 MFMA
+// tiles of 16 x 16 x 32), so every weight is widened exactly once per block, by the wave that needs it, in the shadow
+// of that wave's own MFMAs, and no weight byte is ever written to LDS by a thread.  The fragments of the next k-step are
+// read (and widened) behind the MFMAs of the current one: activations through a ring of eight fragment registers,
+// weights as two raw fragments.
+//
+// The stages of a block's consecutive tiles form ONE stream: the requests run two stages ahead of the MFMAs across tile
+// boundaries, so a tile's first stages arrive while the previous tile is still being multiplied, and the record of the
+// next tile is read a whole tile ahead.  Everything is addressed through buffer descriptors that end where the tile's
+// rows (the expert's weight matrix) end: rows past the end read as zeros, the lane-dependent part of an address is the
+// same for every tile and the tile-dependent part is scalar, so moving the stream on to the next tile costs no vector
+// work (with a row index: one index load per request).  What is left between two tiles is the epilogue.
 
 #include "moe_gmm_common.h"
 
@@ -18,203 +25,272 @@ struct DlwCfg {
   static constexpr int BSRC = BSRC_;
   static constexpr bool GLU = GLU_;
   static constexpr int BM = 256, BN = 256, BKB = 128, BK = 64, MI = 16;
-  static constexpr int WAVES_M = 2, WAVES_N = 4, NWAVES = 8, THREADS = NWAVES * kWave;
-  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / MI, TN = WN / MI;
-  static constexpr int CPR = BKB / 16, RPI = 1024 / BKB;
-  static constexpr int A_IPW = BM / RPI / NWAVES;  // activation requests per wave per stage
-  static constexpr int STAGE = (BM + BN) * BKB, LDS_BYTES = 2 * STAGE;
-  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static constexpr int NWAVES = 8, THREADS = NWAVES * kWave;
+  static constexpr int WN = BN / NWAVES, TM = BM / MI, TN = WN / MI;  // a wave: 256 rows x 32 weight rows
+  static constexpr int RING = 8;                                       // activation fragments in registers
   static constexpr bool NIBBLES = BSRC == BSRC_I4 || BSRC == BSRC_MX4;
-  static constexpr int VPL = NIBBLES ? 32 : 16;          // weights per 16-byte load
-  static constexpr int LPR = BK / VPL;                    // loads per weight row and stage
-  static constexpr int B_LOADS = BN * LPR / THREADS;      // loads per thread and stage: 2 (int8) or 1
-  static constexpr int SRC_STAGE_BYTES = NIBBLES ? BK / 2 : BK;  // bytes of a weight row per stage
-  static constexpr int UNITS = 4;                         // 16-byte LDS chunks a thread writes per stage
-  static_assert(BSRC != BSRC_SAME && B_LOADS * VPL * 2 / 16 == UNITS, "four chunks per thread");
-  __device__ static __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+  static constexpr int W_ROW = NIBBLES ? BK / 2 : BK;  // raw bytes of a weight row per stage: 32 or 64
+  static constexpr int A_STAGE = BM * BKB, B_STAGE = BN * W_ROW, STAGE = A_STAGE + B_STAGE;
+  static constexpr int NSTAGE = 3, LDS_BYTES = NSTAGE * STAGE;
+  static constexpr int A_IPW = A_STAGE / 1024 / NWAVES;  // activation requests per wave and stage: 4
+  static constexpr int B_IPW = B_STAGE / 1024 / NWAVES;  // weight requests per wave and stage: 2 (int8) or 1
+  static constexpr int B_RPI = 1024 / W_ROW;             // weight rows per request: 16 or 32
+  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static_assert(BSRC != BSRC_SAME && TN == 2 && TM == 16 && LDS_BYTES <= 160 * 1024, "shape");
+  // activations: chunk q of row r sits in slot q ^ swz_a(r) of the row's eight 16-byte slots
+  __device__ static __forceinline__ int swz_a(int row) { return (row >> 1) & 7; }
+  // weights: slot q ^ swz_b(r) of the row's four (int8) or two (4-bit) slots, so that the 16 rows a fragment read covers
+  // spread over all banks
+  __device__ static __forceinline__ int swz_b(int row) { return NIBBLES ? (row >> 3) & 1 : (row >> 2) & 3; }
 };
 
+// A raw buffer descriptor over `bytes` bytes at `base`: requests past the end return zeros instead of faulting, which
+// is how rows past a tile's (or a weight matrix's) end are dealt with.
+__device__ __forceinline__ v4i buffer_desc(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  return v4i{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+}
+__device__ __forceinline__ uint32_t clamp_u32(size_t v) { return v > 0xffffffffull ? 0xffffffffu : (uint32_t)v; }
+
+// global -> LDS copy of 16 bytes per lane through a buffer descriptor (1 KB per wave at lds_addr, a wave-uniform LDS byte
+// address), written as asm: the compiler then neither waits for it before LDS accesses that follow nor gives up counting
+// the LDS reads in flight.  Which buffer a copy writes and a read reads is settled by explicit waits and barriers.
+__device__ __forceinline__ void dma16_buffer(const v4i& rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
+}
+// A 2- or 4-byte load of the same kind into a register.  It is not waited for by the compiler either: the value may be
+// used only after an explicit vmcnt wait that covers it.
+__device__ __forceinline__ uint32_t load_u16_untracked(const v4i& rsrc, uint32_t voff, uint32_t soff) {
+  uint32_t v;
+  asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(v) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t load_u32_untracked(const v4i& rsrc, uint32_t voff, uint32_t soff) {
+  uint32_t v;
+  asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(v) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  return v;
+}
+
 template <typename C>
-__global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParams p) {
+__global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParams p0) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  // (bf16 activations carry no scale: saying so here lets the epilogue fold the per-row factor away)
+  TiledParams p = p0;
+  p.lhs_scale = nullptr;
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
   const int N = p.N, K = p.K;
-  const size_t row_bytes = (size_t)K * 2;
-  const size_t w_row_bytes = C::NIBBLES ? (size_t)K / 2 : (size_t)K;
+  const uint32_t row_bytes = (uint32_t)K * 2;
+  const uint32_t w_row_bytes = C::NIBBLES ? (uint32_t)K / 2 : (uint32_t)K;
   const int num_tiles = p.header[0];
   const int total = p.max_m_tiles * p.tiles_n;
   const int nk = K / C::BK;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
 
   struct Tile {
     TileInfo info;
-    int n0;
+    int n0, id;
   };
-  // tile id -> (m-tile, n-tile): ids congruent mod 8 run on one XCD and form an 8 x 4 patch that shares panels in its L2
-  auto locate = [&](int id, Tile& t) -> bool {
-    const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
-    const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+  struct Peek {  // a tile record that has been requested but not looked at yet
+    TileInfo ti;
+    int n0, id;
+    bool valid;
+  };
+  // tile id -> (m-tile, n-tile): ids congruent mod 8 run on one XCD and form an 8 x 4 patch that shares panels in its L2.
+  // The block's first id >= id0 that names an existing m-tile; its record is requested, not waited for.
+  auto peek_from = [&](int id0) -> Peek {
+    Peek pk;
+    pk.valid = false;
+    pk.n0 = 0;
+    pk.id = total;
+    pk.ti = TileInfo{-1, 0, 0, 0};
+    const int q = total / 8, rem = total % 8;
     const int GSM = p.tune > 0 ? p.tune : 8;
     const int width = GSM * p.tiles_n;
-    const int sg = logical / width, first_m = sg * GSM;
-    const int gsz = min(p.max_m_tiles - first_m, GSM);
-    const int m_idx = first_m + (logical % width) % gsz;
-    if (m_idx >= num_tiles) return false;
-    // (uniform values: kept in scalar registers, so that a tile looked up ahead of time costs no vector registers)
-    const TileInfo ti = p.tiles[m_idx];
-    t.info.group = __builtin_amdgcn_readfirstlane(ti.group);
-    t.info.row0 = __builtin_amdgcn_readfirstlane(ti.row0);
-    t.info.nrows = __builtin_amdgcn_readfirstlane(ti.nrows);
-    t.info.pad = 0;
-    t.n0 = __builtin_amdgcn_readfirstlane(((logical % width) / gsz) * C::OUT_BN);
-    return true;
+    for (int id = id0; id < total; id += gridDim.x) {
+      const int xcd = id % 8, loc = id / 8;
+      const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+      const int sg = logical / width, first_m = sg * GSM;
+      const int gsz = min(p.max_m_tiles - first_m, GSM);
+      const int m_idx = first_m + (logical % width) % gsz;
+      if (m_idx >= num_tiles) continue;
+      pk.ti = p.tiles[m_idx];
+      pk.n0 = ((logical % width) / gsz) * C::OUT_BN;
+      pk.id = id;
+      pk.valid = true;
+      break;
+    }
+    return pk;
   };
-  auto next_compute_tile = [&](int& id, Tile& t) -> bool {
-    for (; id < total; id += gridDim.x) {
-      if (!locate(id, t)) continue;
+  // Turns a requested record into the block's next tile that needs the matmul; tiles of rows that belong to no local
+  // group are written as zeros on the way (and the search goes on from there).
+  auto resolve = [&](Peek pk, Tile& t) -> bool {
+    while (pk.valid) {
+      // (uniform values: kept in scalar registers)
+      t.info.group = __builtin_amdgcn_readfirstlane(pk.ti.group);
+      t.info.row0 = __builtin_amdgcn_readfirstlane(pk.ti.row0);
+      t.info.nrows = __builtin_amdgcn_readfirstlane(pk.ti.nrows);
+      t.info.pad = 0;
+      t.n0 = __builtin_amdgcn_readfirstlane(pk.n0);
+      t.id = __builtin_amdgcn_readfirstlane(pk.id);
       if (t.info.group >= 0) return true;
       zero_fill_tile(p.out, p.ro, t.info.row0, t.info.nrows, t.n0, C::OUT_BN, N, tid, C::THREADS);
+      pk = peek_from(t.id + gridDim.x);
     }
     return false;
   };
 
-  // ---- activations: per-lane sources of this wave's requests --------------------------------------------------
-  const uint8_t* a_src[C::A_IPW];
-  // ---- weights: this thread's loads of a stage --------------------------------------------------------------
-  // load l covers VPL consecutive k values of one weight row: row = idx / LPR, part = idx % LPR with idx = tid + l * THREADS
-  const uint8_t* b_src[C::B_LOADS];
-  const void* b_scale_row[C::B_LOADS];  // the row's scales (4-bit formats)
-  int b_lds[C::B_LOADS];                // byte offset of the row inside a stage
-  int b_sw[C::B_LOADS];                 // the row's swizzle
-  int b_part[C::B_LOADS];
-  auto set_sources = [&](const Tile& t) {
-    int a_rows[C::A_IPW];
+  // ---- the loading side of the stream ---------------------------------------------------------------------------
+  // activations: request i of this wave covers rows (wave * A_IPW + i) * 8 .. + 7 of the tile, 128 bytes of each
+  v4i a_desc;
+  uint32_t a_voff[C::A_IPW];
+  auto a_lane_off = [&](int i, int row) {  // the lane's 16 bytes inside the row's 128: global chunk = LDS slot ^ swizzle
+    const int r = (wave * C::A_IPW + i) * 8 + lane / 8;
+    return (uint32_t)row * row_bytes + (uint32_t)(((lane % 8) ^ C::swz_a(r)) << 4);
+  };
+  auto set_a_sources = [&](const Tile& t) {
+    if (p.ro.row_idx) {
+      a_desc = buffer_desc(p.lhs, clamp_u32((size_t)p.ro.lhs_rows * row_bytes));
+      int rows[C::A_IPW];
 #pragma unroll
-    for (int i = 0; i < C::A_IPW; i++) a_rows[i] = t.info.row0 + min((wave * C::A_IPW + i) * C::RPI + lane / C::CPR, t.info.nrows - 1);
-    lhs_rows_of<C::A_IPW>(p.ro, a_rows);
+      for (int i = 0; i < C::A_IPW; i++) rows[i] = min(t.info.row0 + (wave * C::A_IPW + i) * 8 + lane / 8, p.M - 1);
+      lhs_rows_of<C::A_IPW>(p.ro, rows);
 #pragma unroll
-    for (int i = 0; i < C::A_IPW; i++) {
-      const int r = (wave * C::A_IPW + i) * C::RPI + lane / C::CPR;
-      const int q = (lane % C::CPR) ^ C::swz(r);
-      a_src[i] = p.lhs + (size_t)a_rows[i] * row_bytes + q * 16;
-    }
-#pragma unroll
-    for (int l = 0; l < C::B_LOADS; l++) {
-      const int idx = tid + l * C::THREADS;
-      const int row = idx / C::LPR, part = idx % C::LPR;
-      const bool up = C::GLU && row >= C::BN / 2;
-      const int n = min(t.n0 + (up ? row - C::BN / 2 : row), N - 1);
-      const size_t grow = (size_t)t.info.group * N + n;
-      b_src[l] = (up ? p.rhs_up : p.rhs) + grow * w_row_bytes + part * 16;
-      b_lds[l] = (C::BM + row) * C::BKB;
-      b_sw[l] = C::swz(row);
-      b_part[l] = part;
-      if (C::BSRC == BSRC_I4) {
-        const int nkg = (K + p.i4_group - 1) / p.i4_group;
-        b_scale_row[l] = (const uint16_t*)(up ? p.rhs_up_scale : p.rhs_scale) + grow * nkg;
-      } else if (C::BSRC == BSRC_MX4) {
-        b_scale_row[l] = (const uint8_t*)(up ? p.rhs_up_scale : p.rhs_scale) + grow * (K / 32);
-      } else {
-        b_scale_row[l] = nullptr;
-      }
+      for (int i = 0; i < C::A_IPW; i++) a_voff[i] = a_lane_off(i, rows[i]);
+    } else {
+      a_desc = buffer_desc(p.lhs + (size_t)t.info.row0 * row_bytes, clamp_u32((size_t)t.info.nrows * row_bytes));
     }
   };
-
+  if (!p.ro.row_idx) {
+#pragma unroll
+    for (int i = 0; i < C::A_IPW; i++) a_voff[i] = a_lane_off(i, (wave * C::A_IPW + i) * 8 + lane / 8);
+  }
+  // weights: request i of this wave covers the tile's weight rows (wave * B_IPW + i) * B_RPI .. + B_RPI - 1; with GLU the
+  // upper 128 of the 256 rows are the second projection's, whose requests come from waves 4 .. 7
+  const bool load_up = C::GLU && wave >= C::NWAVES / 2;
+  v4i b_desc;
+  uint32_t b_soff = 0;
+  uint32_t b_voff[C::B_IPW];
+#pragma unroll
+  for (int i = 0; i < C::B_IPW; i++) {
+    const int r = (wave * C::B_IPW + i) * C::B_RPI + lane / (C::W_ROW / 16);  // row of the tile
+    const int pr = C::GLU ? r % (C::BN / 2) : r;                                // row of the projection's 128 / 256
+    b_voff[i] = (uint32_t)pr * w_row_bytes + (uint32_t)(((lane % (C::W_ROW / 16)) ^ C::swz_b(r)) << 4);
+  }
+  auto set_b_sources = [&](const Tile& t) {
+    b_desc = buffer_desc((load_up ? p.rhs_up : p.rhs) + (size_t)t.info.group * N * w_row_bytes, clamp_u32((size_t)N * w_row_bytes));
+    b_soff = (uint32_t)t.n0 * w_row_bytes;
+  };
   auto issue_a = [&](int kt, int buf, int i) {
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(a_src[i] + (size_t)kt * C::BKB), (lds_ptr_t)(smem + buf * C::STAGE + (wave * C::A_IPW + i) * 1024), 16,
-                                     0, 0);
+    dma16_buffer(a_desc, a_voff[i], (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + (wave * C::A_IPW + i) * 1024);
+  };
+  auto issue_b = [&](int kt, int buf, int i) {
+    dma16_buffer(b_desc, b_voff[i], b_soff + (uint32_t)kt * C::W_ROW, lds_base + buf * C::STAGE + C::A_STAGE + (wave * C::B_IPW + i) * 1024);
   };
 
-  // raw weight bytes of one stage (and, for the 4-bit formats, the scale of each load's k range)
-  struct WRegs {
-    uint4 w[C::B_LOADS];
-    float s[C::B_LOADS];
-  };
-  auto b_load = [&](WRegs& r, int kt) {
+  // ---- the multiplying side ----------------------------------------------------------------------------------------
+  // weight fragment j of this wave: rows frag_row(j) .. + 15 of the tile; the lane widens row + lane % 16
+  auto frag_row = [&](int j) { return C::GLU ? j * (C::BN / 2) + wave * 16 : wave * C::WN + j * 16; };
+  // scales of the 4-bit formats: per weight row and 32 (mxfp4, int4 group 32) or 128 values of K; the lane needs the ones
+  // of its own row for the stage's two k-steps: one 2- or 4-byte load per fragment and stage
+  v4i s_desc[C::TN];
+  uint32_t s_soff = 0, s_voff = 0;
+  const bool i4g32 = C::BSRC == BSRC_I4 && p.i4_group == 32;
+  const uint32_t nkg = C::BSRC == BSRC_I4 ? (uint32_t)((K + p.i4_group - 1) / p.i4_group) : (uint32_t)(K / 32);
+  const uint32_t s_row_bytes = C::BSRC == BSRC_I4 ? nkg * 2 : nkg;
+  if (C::NIBBLES) s_voff = (uint32_t)((C::GLU ? wave * 16 : wave * C::WN) + lane % 16) * s_row_bytes;
+  auto set_s_sources = [&](const Tile& t) {
+    if (!C::NIBBLES) return;
 #pragma unroll
-    for (int l = 0; l < C::B_LOADS; l++) {
-      r.w[l] = *(const uint4*)(b_src[l] + (size_t)kt * C::SRC_STAGE_BYTES);
-      const int k0 = kt * C::BK + b_part[l] * C::VPL;
-      if (C::BSRC == BSRC_I4) r.s[l] = bf16_bits_to_f32(((const uint16_t*)b_scale_row[l])[p.i4_group == 32 ? k0 >> 5 : k0 >> 7]);
-      else if (C::BSRC == BSRC_MX4) r.s[l] = __uint_as_float((uint32_t)((const uint8_t*)b_scale_row[l])[k0 / 32] << 23);
-      else r.s[l] = 1.0f;
+    for (int j = 0; j < C::TN; j++)
+      s_desc[j] = buffer_desc((const uint8_t*)(C::GLU && j == 1 ? p.rhs_up_scale : p.rhs_scale) + (size_t)t.info.group * N * s_row_bytes,
+                              clamp_u32((size_t)N * s_row_bytes));
+    s_soff = (uint32_t)t.n0 * s_row_bytes;
+  };
+  uint32_t sc_cur[C::TN] = {0, 0}, sc_nxt[C::TN] = {0, 0};  // raw scale bits of the stage being widened / of the one after it
+  auto load_scales = [&](uint32_t (&sc)[C::TN], int kt) {
+    if (!C::NIBBLES) return;
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) {
+      const uint32_t row_off = s_voff + (C::GLU ? 0u : (uint32_t)j * 16 * s_row_bytes);
+      if (C::BSRC == BSRC_MX4) sc[j] = load_u16_untracked(s_desc[j], row_off + (uint32_t)kt * 2, s_soff);  // bytes 2 kt, 2 kt + 1
+      else if (i4g32) sc[j] = load_u32_untracked(s_desc[j], row_off + (uint32_t)kt * 4, s_soff);            // bf16 2 kt, 2 kt + 1
+      else sc[j] = load_u16_untracked(s_desc[j], row_off + (uint32_t)(kt >> 1) * 2, s_soff);                // bf16 kt / 2
     }
   };
-  // unit u of a stage: 8 weights -> one 16-byte chunk of the row in LDS
-  auto b_store_unit = [&](const WRegs& r, int buf, int u) {
-    constexpr int UPL = C::UNITS / C::B_LOADS;  // units per load: 2 (int8: 8 bytes each) or 4 (4-bit: one word each)
-    const int l = u / UPL, h = u % UPL;
-    const uint32_t w4[4] = {r.w[l].x, r.w[l].y, r.w[l].z, r.w[l].w};
-    uint4 o;
-    if (C::BSRC == BSRC_I8) {
-      const int v0 = (int)w4[2 * h], v1 = (int)w4[2 * h + 1];
-      o = make_uint4(i8x2_to_bf16x2((v0 << 24) >> 24, (v0 << 16) >> 24), i8x2_to_bf16x2((v0 << 8) >> 24, v0 >> 24),
-                     i8x2_to_bf16x2((v1 << 24) >> 24, (v1 << 16) >> 24), i8x2_to_bf16x2((v1 << 8) >> 24, v1 >> 24));
-    } else if (C::BSRC == BSRC_MX4) {
-      const uint32_t w = w4[h];
-      const float sc = r.s[l];
-      o = make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 0)),
-                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 1)),
-                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 2)),
-                     __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, sc, 3)));
-    } else {  // int4: (nibble - 8) * scale rounded to bf16, as the reference dequantises
-      const uint32_t w = w4[h];
-      const float sc = r.s[l];
-      uint32_t x[4];
-#pragma unroll
-      for (int b = 0; b < 4; b++) {
-        const int lo = (int)((w >> (8 * b)) & 0xf) - 8, hi = (int)((w >> (8 * b + 4)) & 0xf) - 8;
-        x[b] = pack_bf16x2((float)lo * sc, (float)hi * sc);
-      }
-      o = make_uint4(x[0], x[1], x[2], x[3]);
-    }
-    const int q = b_part[l] * UPL + h;  // chunk of the 128-byte row
-    *(uint4*)(smem + buf * C::STAGE + b_lds[l] + ((q ^ b_sw[l]) << 4)) = o;
+  auto scale_of = [&](const uint32_t (&sc)[C::TN], int j, int ks) -> float {
+    if (C::BSRC == BSRC_MX4) return __uint_as_float(((sc[j] >> (8 * ks)) & 0xffu) << 23);
+    if (i4g32) return __uint_as_float(ks ? sc[j] & 0xffff0000u : sc[j] << 16);
+    return __uint_as_float(sc[j] << 16);
   };
 
   typedef v4f acc_t;
   acc_t acc[C::TN][C::TM];
-  int b_row[C::TN];
-#pragma unroll
-  for (int j = 0; j < C::TN; j++) {
-    if (C::GLU) {
-      constexpr int H = C::TN / 2;
-      b_row[j] = (j < H ? 0 : C::BN / 2) + wn * (C::WN / 2) + (j < H ? j : j - H) * C::MI;
-    } else {
-      b_row[j] = wn * C::WN + j * C::MI;
-    }
-  }
-  // fragment of k-step ks: row (lane % 16), chunk q = 4 * ks + lane / 16, stored at slot q ^ swz(row)
-  const int t16m = ((lane / 16) ^ C::swz(lane % 16)) * 16;
-  const int row_off_m = (lane % 16) * C::BKB;
-  v4i ga[C::TM], gb[2][C::TN];
-  auto read_a16 = [&](int buf, int ks, int i) {
-    ga[i] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
+  // activation fragment of row tile i, k-step ks: row 16 i + lane % 16, chunk q = 4 ks + lane / 16, at slot q ^ swz_a(row)
+  const int a_lane = (lane % 16) * C::BKB + (((lane / 16) ^ C::swz_a(lane % 16)) << 4);
+  v4i ga[C::RING];
+  auto read_a = [&](int buf, int ks, int i) {
+    ga[i % C::RING] = *(const v4i*)(smem + buf * C::STAGE + i * 16 * C::BKB + (a_lane ^ (ks * 64)));
   };
-  auto read_b16 = [&](int buf, int ks, int set, int j) {
-    gb[set][j] = *(const v4i*)(smem + buf * C::STAGE + (C::BM + b_row[j]) * C::BKB + row_off_m + (t16m ^ (ks * 64)));
+  // raw weight fragment j, k-step ks: row frag_row(j) + lane % 16, the 8 values of K from 32 ks + 8 (lane / 16) on
+  const int b_lane = C::NIBBLES ? (lane % 16) * C::W_ROW + (lane / 16) * 4 : (lane % 16) * C::W_ROW + ((lane / 16) & 1) * 8;
+  const int b_sw = C::swz_b(lane % 16);
+  typedef typename std::conditional<C::NIBBLES, uint32_t, uint2>::type raw_t;
+  raw_t braw[C::TN];
+  auto read_braw = [&](int buf, int ks, int j) {
+    const int slot = C::NIBBLES ? ks : 2 * ks + (lane / 32);  // 16-byte slot of the row that holds the lane's bytes
+    braw[j] = *(const raw_t*)(smem + buf * C::STAGE + C::A_STAGE + frag_row(j) * C::W_ROW + b_lane + ((slot ^ b_sw) << 4));
+  };
+  // widened weight fragments: the set of the current k-step and the one being built for the next
+  v4i gb[2][C::TN];
+  // piece pc (0 .. 3) of fragment j: two of its eight values -> one register of gb[set][j]
+  auto widen_piece = [&](int set, int j, int pc, float sc) {
+    uint32_t o;
+    if constexpr (C::BSRC == BSRC_I8) {
+      const int w = (int)(pc < 2 ? braw[j].x : braw[j].y);
+      const int sh = (pc & 1) * 16;
+      o = pack_bf16x2((float)((w << (24 - sh)) >> 24), (float)((w << (16 - sh)) >> 24));
+    } else if constexpr (C::BSRC == BSRC_MX4) {
+      // (the byte selector is an immediate)
+      o = pc == 0   ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(braw[j], sc, 0))
+          : pc == 1 ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(braw[j], sc, 1))
+          : pc == 2 ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(braw[j], sc, 2))
+                    : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(braw[j], sc, 3));
+    } else {  // int4: (nibble - 8) * scale rounded to bf16, as the reference dequantises
+      const uint32_t b = (braw[j] >> (8 * pc)) & 0xffu;
+      o = pack_bf16x2((float)((int)(b & 0xf) - 8) * sc, (float)((int)(b >> 4) - 8) * sc);
+    }
+    gb[set][j][pc] = (int)o;
   };
 
-  WRegs wr;  // the stage after next (while the loop runs)
-  // One k-step of 32 MFMAs.  RD: the fragments of the next k-step are read behind them.  LD: the k-step after the
-  // barrier: the activation requests of stage ld_kt go out, the weights held in `wr` (the same stage) are widened and
-  // written into the freed buffer, and the raw bytes of the stage after that are requested.
-  auto kstep16 = [&](auto set_c, auto rd_c, auto ld_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
+  // One k-step of 32 MFMAs on the fragments of (cur_buf, cur_ks): row tiles 0 .. 7 sit in the ring, 8 .. 15 are read
+  // behind the first half.  ZC: a tile's first k-step starts from zero.  RD: the next k-step (rd_buf, rd_ks) is prepared
+  // behind the MFMAs: its raw weight fragments are read at the start and widened piece by piece into the other set (with
+  // the scales in sc_rd), its row tiles 0 .. 7 are read behind the second half.  LD: the requests of stage ld_kt of the
+  // loading tile go out into buffer ld_buf.
+  auto kstep = [&](auto set_c, auto rd_c, auto ld_c, auto zc_c, int cur_buf, int cur_ks, int rd_buf, int rd_ks, const uint32_t (&sc_rd)[C::TN],
+                   int ld_kt, int ld_buf) {
     constexpr int SET = decltype(set_c)::value;
-    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value, ZC = decltype(zc_c)::value;
+    float sc[C::TN] = {1.0f, 1.0f};
+    if (RD && C::NIBBLES) {
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) sc[j] = scale_of(sc_rd, j, rd_ks);
+    }
 #pragma unroll
     for (int i = 0; i < C::TM; i++) {
 #pragma unroll
       for (int j = 0; j < C::TN; j++) {
-        acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, gb[SET][j]), __builtin_bit_cast(v8bf, ga[i]), acc[j][i], 0, 0, 0);
+        acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, gb[SET][j]), __builtin_bit_cast(v8bf, ga[i % C::RING]),
+                                                            ZC ? v4f{0.f, 0.f, 0.f, 0.f} : acc[j][i], 0, 0, 0);
         const int slot = i * C::TN + j;
-        if (LD && slot < C::A_IPW) issue_a(ld_kt, ld_buf, slot);
-        // the four chunks of the weight stage, one every fourth MFMA from slot 6 on; then the next stage's raw bytes
-        if (LD && slot >= 6 && slot < 6 + 4 * C::UNITS && (slot - 6) % 4 == 0) b_store_unit(wr, ld_buf, (slot - 6) / 4);
-        if (LD && slot == 6 + 4 * C::UNITS) b_load(wr, min(ld_kt + 1, nk - 1));
-        if (RD && j == 1 && i < C::TN) read_b16(rd_buf, rd_ks, SET ^ 1, i);
-        if (RD && j == C::TN - 1) read_a16(rd_buf, rd_ks, i);
+        if (RD && slot < C::TN) read_braw(rd_buf, rd_ks, slot);
+        // the eight pieces of the two fragments, one every second MFMA from slot 8 on
+        if (RD && slot >= 8 && slot < 8 + 2 * 4 * C::TN && slot % 2 == 0) widen_piece(SET ^ 1, (slot - 8) / 8, ((slot - 8) / 2) % 4, sc[(slot - 8) / 8]);
+        if (LD && slot % 2 == 1 && slot / 2 < C::A_IPW) issue_a(ld_kt, ld_buf, slot / 2);
+        if (LD && slot % 2 == 1 && slot / 2 >= C::A_IPW && slot / 2 < C::A_IPW + C::B_IPW) issue_b(ld_kt, ld_buf, slot / 2 - C::A_IPW);
+        if (j == C::TN - 1 && i < C::TM - C::RING) read_a(cur_buf, cur_ks, i + C::RING);
+        if (RD && j == C::TN - 1 && i >= C::TM - C::RING) read_a(rd_buf, rd_ks, i - (C::TM - C::RING));
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -225,76 +301,90 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   using S1 = std::integral_constant<int, 1>;
   constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
 
-  // A tile's first two stages: activation requests, and the weights of both stages as raw bytes.
-  WRegs w0, w1;
-  auto issue_prologue = [&]() {
+  // The fragments of a tile's first k-step (stage 0 in buffer `buf`), read and widened with nothing to hide behind.
+  auto first_fragments = [&](int buf) {
 #pragma unroll
-    for (int s = 0; s < 2; s++)
+    for (int i = 0; i < C::RING; i++) read_a(buf, 0, i);
 #pragma unroll
-      for (int i = 0; i < C::A_IPW; i++) issue_a(min(s, nk - 1), s, i);
-    b_load(w0, 0);
-    b_load(w1, min(1, nk - 1));
-  };
-  // ... widened into the two buffers once they have arrived (and everything the previous tile read is done)
-  auto finish_prologue = [&]() {
-    wait_vmcnt<0>();
-#pragma unroll
-    for (int u = 0; u < C::UNITS; u++) b_store_unit(w0, 0, u);
-#pragma unroll
-    for (int u = 0; u < C::UNITS; u++) b_store_unit(w1, 1, u);
-    b_load(wr, min(2, nk - 1));
-  };
-
-  int id = blockIdx.x;
-  Tile cur;
-  bool have = next_compute_tile(id, cur);
-  if (have) {
-    set_sources(cur);
-    issue_prologue();
-  }
-  while (have) {
+    for (int j = 0; j < C::TN; j++) read_braw(buf, 0, j);
 #pragma unroll
     for (int j = 0; j < C::TN; j++)
 #pragma unroll
-      for (int i = 0; i < C::TM; i++) acc[j][i] = v4f{0.f, 0.f, 0.f, 0.f};
-    finish_prologue();
-    // every activation request of the prologue has landed, every wave's weight chunks are written
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    asm volatile("s_barrier" ::: "memory");
+      for (int pc = 0; pc < 4; pc++) widen_piece(0, j, pc, C::NIBBLES ? scale_of(sc_cur, j, 0) : 1.0f);
+  };
+
+  Tile cur, nxt;
+  if (!resolve(peek_from(blockIdx.x), cur)) return;
+  // ---- head of the stream: the first tile's stages 0 and 1 (scales: both into registers) ----
+  set_a_sources(cur);
+  set_b_sources(cur);
+  set_s_sources(cur);
+  load_scales(sc_cur, 0);
+  load_scales(sc_nxt, 1);
 #pragma unroll
-    for (int i = 0; i < C::TM; i++) read_a16(0, 0, i);
+  for (int s = 0; s < 2; s++) {
 #pragma unroll
-    for (int j = 0; j < C::TN; j++) read_b16(0, 0, 0, j);
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+    for (int i = 0; i < C::A_IPW; i++) issue_a(s, s, i);
+#pragma unroll
+    for (int i = 0; i < C::B_IPW; i++) issue_b(s, s, i);
+  }
+  wait_vmcnt<0>();
+  asm volatile("s_barrier" ::: "memory");
+  first_fragments(0);
+
+  int base = 0;  // the buffer that holds stage 0 of the current tile
+  while (true) {
+    // the record of the block's next tile is requested now and looked at two stages before this tile ends
+    Peek pk = peek_from(cur.id + gridDim.x);
+    bool have_n = false;
+    const int n_out0 = cur.n0 + (C::GLU ? wave * 16 : wave * C::WN);
     EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
-    int kt = 0;
-    kstep16(S0{}, T_{}, F_{}, 0, 1, 0, 0);
-    for (; kt + 1 < nk; kt++) {
-      const int buf = kt % 2;
-      // own fragment reads of this stage done, own requests (activations of stage kt+1, raw weights of stage kt+2) landed,
-      // own weight chunks of stage kt+1 written: then everybody's
-      __builtin_amdgcn_s_waitcnt(0xC07F);
+    // first half of stage 0; its second half is prepared behind it
+    kstep(S0{}, T_{}, F_{}, T_{}, base, 0, base, 1, sc_cur, 0, 0);
+    // Iteration `it`: the second half of stage it, then the first half of stage it + 1.  At its barrier stage it + 1 has
+    // landed and nobody reads stage it - 1 any more: that buffer takes stage it + 2 of the stream (from nk on: the next
+    // tile's).  The 4-bit formats' scales of stage it + 2 are requested with it; those of stage it + 1 become current.
+    auto stream_kt = [&](int s) { return s < nk ? s : (have_n ? s - nk : nk - 1); };
+    int cb = base;  // buffer of stage `it`
+    auto iteration = [&](int it, auto last_c) {
+      constexpr bool LAST = decltype(last_c)::value;  // the tile's last half stage: nothing is prepared behind it
+      const int nb = cb == C::NSTAGE - 1 ? 0 : cb + 1, lb = nb == C::NSTAGE - 1 ? 0 : nb + 1;
+      // own fragment reads done, own requests landed: then everybody's
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
       wait_vmcnt<0>();
       asm volatile("s_barrier" ::: "memory");
-      kstep16(S1{}, T_{}, T_{}, buf ^ 1, 0, min(kt + 2, nk - 1), buf);
-      kstep16(S0{}, T_{}, F_{}, buf ^ 1, 1, 0, 0);
+      if (C::NIBBLES) {
+#pragma unroll
+        for (int j = 0; j < C::TN; j++) sc_cur[j] = sc_nxt[j];
+        load_scales(sc_nxt, stream_kt(it + 2));
+      }
+      if (LAST) {
+        kstep(S1{}, F_{}, T_{}, F_{}, cb, 1, 0, 0, sc_cur, stream_kt(it + 2), lb);
+      } else {
+        kstep(S1{}, T_{}, T_{}, F_{}, cb, 1, nb, 0, sc_cur, stream_kt(it + 2), lb);
+        kstep(S0{}, T_{}, F_{}, F_{}, nb, 0, nb, 1, sc_cur, 0, 0);
+      }
+      cb = nb;
+    };
+    for (int it = 0; it < nk - 2; it++) iteration(it, F_{});
+    // the stream crosses into the next tile
+    have_n = resolve(pk, nxt);
+    if (have_n) {
+      set_a_sources(nxt);
+      set_b_sources(nxt);
+      set_s_sources(nxt);
     }
-    load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC == BSRC_I8, C::MI>(esc, p, cur.info, wm * C::WM, n_out0, lane);
-    kstep16(S1{}, F_{}, F_{}, 0, 0, 0, 0);
-    // all LDS reads of this tile are done in every wave and nothing is still writing LDS: the buffers can take the next tile
-    // results first (the accumulators are then dead across the tile-boundary code), then the next tile
-    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, cur.info, wm * C::WM, n_out0, lane);
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    wait_vmcnt<0>();
-    asm volatile("s_barrier" ::: "memory");
-    id += gridDim.x;
-    have = next_compute_tile(id, cur);
-    if (have) {
-      set_sources(cur);
-      issue_prologue();
-    }
+    iteration(nk - 2, F_{});
+    load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC == BSRC_I8, C::MI>(esc, p, cur.info, 0, n_out0, lane);
+    iteration(nk - 1, T_{});
+    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, cur.info, 0, n_out0, lane);
+    if (!have_n) break;
+    cur = nxt;
+    base = cb;  // (after the last iteration: the buffer of stage nk = the next tile's stage 0, landed before the last barrier)
+    first_fragments(base);
   }
+  // nothing may still be writing LDS when the block ends
+  __builtin_amdgcn_s_waitcnt(0xC07F);
   wait_vmcnt<0>();
 }
 
@@ -333,8 +423,15 @@ static int launch_dlw_cfg(const TiledParams& p0, int M, int G_total, hipStream_t
   return check_launch("gmm_dlw_kernel");
 }
 
+bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor) {
+  // whole 64-value stages, at least three of them (the stream looks two stages ahead, into the next tile at most); byte
+  // offsets inside one expert's weight matrix and inside the activations that a row index may address fit 32 bits
+  return K % 64 == 0 && K >= 192 && !wq_kmajor && (long long)N * K < (1LL << 32) && indexed_lhs_rows * K * 2 < (1LL << 32);
+}
+
 int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
-  if (p.K % 64 != 0 || p.wq_kmajor) return fail(MOE_ERR_UNSUPPORTED, "gmm: the weight-only direct-to-LDS kernel needs K %% 64 == 0 and scales in the default layout");
+  if (!dlw_takes(p.K, p.N, p.ro.row_idx ? p.ro.lhs_rows : 0, p.wq_kmajor != 0))
+    return fail(MOE_ERR_UNSUPPORTED, "gmm: the weight-only direct-to-LDS kernel needs K %% 64 == 0, K >= 192, scales in the default layout and 32-bit byte offsets");
 #define MOE_DLW_CASE(BSRC) \
   if (bsrc == BSRC) return glu ? launch_dlw_cfg<DlwCfg<BSRC, true>>(p, M, G_total, s) : launch_dlw_cfg<DlwCfg<BSRC, false>>(p, M, G_total, s);
   MOE_DLW_CASE(BSRC_I8)
