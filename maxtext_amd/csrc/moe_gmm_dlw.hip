@@ -58,19 +58,6 @@ __device__ __forceinline__ uint32_t clamp_u32(size_t v) { return v > 0xffffffffu
 __device__ __forceinline__ void dma16_buffer(const v4i& rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
 }
-// A 2- or 4-byte load of the same kind into a register.  It is not waited for by the compiler either: the value may be
-// used only after an explicit vmcnt wait that covers it.
-__device__ __forceinline__ uint32_t load_u16_untracked(const v4i& rsrc, uint32_t voff, uint32_t soff) {
-  uint32_t v;
-  asm volatile("buffer_load_ushort %0, %1, %2, %3 offen" : "=v"(v) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-  return v;
-}
-__device__ __forceinline__ uint32_t load_u32_untracked(const v4i& rsrc, uint32_t voff, uint32_t soff) {
-  uint32_t v;
-  asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(v) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-  return v;
-}
-
 template <typename C>
 __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParams p0) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -193,7 +180,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   auto frag_row = [&](int j) { return C::GLU ? j * (C::BN / 2) + wave * 16 : wave * C::WN + j * 16; };
   // scales of the 4-bit formats: per weight row and 32 (mxfp4, int4 group 32) or 128 values of K; the lane needs the ones
   // of its own row for the stage's two k-steps: one 2- or 4-byte load per fragment and stage
-  v4i s_desc[C::TN];
+  __amdgpu_buffer_rsrc_t s_desc[C::TN];
   uint32_t s_soff = 0, s_voff = 0;
   const bool i4g32 = C::BSRC == BSRC_I4 && p.i4_group == 32;
   const uint32_t nkg = C::BSRC == BSRC_I4 ? (uint32_t)((K + p.i4_group - 1) / p.i4_group) : (uint32_t)(K / 32);
@@ -203,25 +190,34 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
     if (!C::NIBBLES) return;
 #pragma unroll
     for (int j = 0; j < C::TN; j++)
-      s_desc[j] = buffer_desc((const uint8_t*)(C::GLU && j == 1 ? p.rhs_up_scale : p.rhs_scale) + (size_t)t.info.group * N * s_row_bytes,
-                              clamp_u32((size_t)N * s_row_bytes));
+      s_desc[j] = __builtin_amdgcn_make_buffer_rsrc((void*)((const uint8_t*)(C::GLU && j == 1 ? p.rhs_up_scale : p.rhs_scale) + (size_t)t.info.group * N * s_row_bytes),
+                                                    0, (int)clamp_u32((size_t)N * s_row_bytes), 0x00020000);
     s_soff = (uint32_t)t.n0 * s_row_bytes;
   };
-  uint32_t sc_cur[C::TN] = {0, 0}, sc_nxt[C::TN] = {0, 0};  // raw scale bits of the stage being widened / of the one after it
-  auto load_scales = [&](uint32_t (&sc)[C::TN], int kt) {
+  // The raw scale bits of a stage are requested with its weights (ordinary loads: the compiler waits for them where they
+  // are used) and turned into the factors of its two k-steps right after the barrier that also waits for the stage.
+  uint32_t sc_raw[C::TN] = {0, 0};
+  float sc_cur[C::TN][2] = {{1.0f, 1.0f}, {1.0f, 1.0f}};  // [fragment][k-step] of the stage being widened
+  auto load_scales = [&](int kt) {
     if (!C::NIBBLES) return;
 #pragma unroll
     for (int j = 0; j < C::TN; j++) {
       const uint32_t row_off = s_voff + (C::GLU ? 0u : (uint32_t)j * 16 * s_row_bytes);
-      if (C::BSRC == BSRC_MX4) sc[j] = load_u16_untracked(s_desc[j], row_off + (uint32_t)kt * 2, s_soff);  // bytes 2 kt, 2 kt + 1
-      else if (i4g32) sc[j] = load_u32_untracked(s_desc[j], row_off + (uint32_t)kt * 4, s_soff);            // bf16 2 kt, 2 kt + 1
-      else sc[j] = load_u16_untracked(s_desc[j], row_off + (uint32_t)(kt >> 1) * 2, s_soff);                // bf16 kt / 2
+      if (C::BSRC == BSRC_MX4) sc_raw[j] = __builtin_amdgcn_raw_buffer_load_b16(s_desc[j], row_off + (uint32_t)kt * 2, s_soff, 0);  // bytes 2 kt, 2 kt + 1
+      else if (i4g32) sc_raw[j] = __builtin_amdgcn_raw_buffer_load_b32(s_desc[j], row_off + (uint32_t)kt * 4, s_soff, 0);            // bf16 2 kt, 2 kt + 1
+      else sc_raw[j] = __builtin_amdgcn_raw_buffer_load_b16(s_desc[j], row_off + (uint32_t)(kt >> 1) * 2, s_soff, 0);                // bf16 kt / 2
     }
   };
-  auto scale_of = [&](const uint32_t (&sc)[C::TN], int j, int ks) -> float {
-    if (C::BSRC == BSRC_MX4) return __uint_as_float(((sc[j] >> (8 * ks)) & 0xffu) << 23);
-    if (i4g32) return __uint_as_float(ks ? sc[j] & 0xffff0000u : sc[j] << 16);
-    return __uint_as_float(sc[j] << 16);
+  auto scales_to_current = [&]() {
+    if (!C::NIBBLES) return;
+#pragma unroll
+    for (int j = 0; j < C::TN; j++)
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        if (C::BSRC == BSRC_MX4) sc_cur[j][ks] = __uint_as_float(((sc_raw[j] >> (8 * ks)) & 0xffu) << 23);
+        else if (i4g32) sc_cur[j][ks] = __uint_as_float(ks ? sc_raw[j] & 0xffff0000u : sc_raw[j] << 16);
+        else sc_cur[j][ks] = __uint_as_float(sc_raw[j] << 16);
+      }
   };
 
   typedef v4f acc_t;
@@ -266,16 +262,15 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   // One k-step of 32 MFMAs on the fragments of (cur_buf, cur_ks): row tiles 0 .. 7 sit in the ring, 8 .. 15 are read
   // behind the first half.  ZC: a tile's first k-step starts from zero.  RD: the next k-step (rd_buf, rd_ks) is prepared
   // behind the MFMAs: its raw weight fragments are read at the start and widened piece by piece into the other set (with
-  // the scales in sc_rd), its row tiles 0 .. 7 are read behind the second half.  LD: the requests of stage ld_kt of the
+  // the scales in sc_cur), its row tiles 0 .. 7 are read behind the second half.  LD: the requests of stage ld_kt of the
   // loading tile go out into buffer ld_buf.
-  auto kstep = [&](auto set_c, auto rd_c, auto ld_c, auto zc_c, int cur_buf, int cur_ks, int rd_buf, int rd_ks, const uint32_t (&sc_rd)[C::TN],
-                   int ld_kt, int ld_buf) {
+  auto kstep = [&](auto set_c, auto rd_c, auto ld_c, auto zc_c, int cur_buf, int cur_ks, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
     constexpr int SET = decltype(set_c)::value;
     constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value, ZC = decltype(zc_c)::value;
     float sc[C::TN] = {1.0f, 1.0f};
     if (RD && C::NIBBLES) {
 #pragma unroll
-      for (int j = 0; j < C::TN; j++) sc[j] = scale_of(sc_rd, j, rd_ks);
+      for (int j = 0; j < C::TN; j++) sc[j] = rd_ks ? sc_cur[j][1] : sc_cur[j][0];
     }
 #pragma unroll
     for (int i = 0; i < C::TM; i++) {
@@ -310,7 +305,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
 #pragma unroll
     for (int j = 0; j < C::TN; j++)
 #pragma unroll
-      for (int pc = 0; pc < 4; pc++) widen_piece(0, j, pc, C::NIBBLES ? scale_of(sc_cur, j, 0) : 1.0f);
+      for (int pc = 0; pc < 4; pc++) widen_piece(0, j, pc, sc_cur[j][0]);
   };
 
   Tile cur, nxt;
@@ -319,8 +314,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   set_a_sources(cur);
   set_b_sources(cur);
   set_s_sources(cur);
-  load_scales(sc_cur, 0);
-  load_scales(sc_nxt, 1);
+  load_scales(0);
 #pragma unroll
   for (int s = 0; s < 2; s++) {
 #pragma unroll
@@ -329,6 +323,8 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
     for (int i = 0; i < C::B_IPW; i++) issue_b(s, s, i);
   }
   wait_vmcnt<0>();
+  scales_to_current();
+  load_scales(1);
   asm volatile("s_barrier" ::: "memory");
   first_fragments(0);
 
@@ -340,7 +336,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
     const int n_out0 = cur.n0 + (C::GLU ? wave * 16 : wave * C::WN);
     EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
     // first half of stage 0; its second half is prepared behind it
-    kstep(S0{}, T_{}, F_{}, T_{}, base, 0, base, 1, sc_cur, 0, 0);
+    kstep(S0{}, T_{}, F_{}, T_{}, base, 0, base, 1, 0, 0);
     // Iteration `it`: the second half of stage it, then the first half of stage it + 1.  At its barrier stage it + 1 has
     // landed and nobody reads stage it - 1 any more: that buffer takes stage it + 2 of the stream (from nk on: the next
     // tile's).  The 4-bit formats' scales of stage it + 2 are requested with it; those of stage it + 1 become current.
@@ -353,16 +349,13 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
       wait_vmcnt<0>();
       asm volatile("s_barrier" ::: "memory");
-      if (C::NIBBLES) {
-#pragma unroll
-        for (int j = 0; j < C::TN; j++) sc_cur[j] = sc_nxt[j];
-        load_scales(sc_nxt, stream_kt(it + 2));
-      }
+      scales_to_current();
+      load_scales(stream_kt(it + 2));
       if (LAST) {
-        kstep(S1{}, F_{}, T_{}, F_{}, cb, 1, 0, 0, sc_cur, stream_kt(it + 2), lb);
+        kstep(S1{}, F_{}, T_{}, F_{}, cb, 1, 0, 0, stream_kt(it + 2), lb);
       } else {
-        kstep(S1{}, T_{}, T_{}, F_{}, cb, 1, nb, 0, sc_cur, stream_kt(it + 2), lb);
-        kstep(S0{}, T_{}, F_{}, F_{}, nb, 0, nb, 1, sc_cur, 0, 0);
+        kstep(S1{}, T_{}, T_{}, F_{}, cb, 1, nb, 0, stream_kt(it + 2), lb);
+        kstep(S0{}, T_{}, F_{}, F_{}, nb, 0, nb, 1, 0, 0);
       }
       cb = nb;
     };

@@ -17,7 +17,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
-from tolerances import TOL, relerr
+from tolerances import ELEM_ATOL_RMS_CHAINED, TOL, relerr
 
 pytestmark = pytest.mark.gpu
 
@@ -263,3 +263,57 @@ def test_gmm_row_index_row_scale_and_f32_out_in_every_kernel_family(K, case):
   scaled32 = K.gmm_raw(cuda(lhs_t), cuda(args["rhs"]), cuda(gs), lhs_row_idx=cuda(src), lhs_row_idx_div=k, out_row_scale=cuda(rowf),
                        out_dtype=torch.float32, **idx_kw)
   assert relerr(scaled32, want_g.float() * rowf[:, None]) <= 2e-3
+
+
+@pytest.mark.parametrize("fmt", ["int8", "int4", "int4g32", "mxfp4"])
+@pytest.mark.parametrize("glu", [False, True])
+def test_weight_only_prefill_kernel_against_the_tiled_kernel_at_size(K, fmt, glu):
+  """The persistent weight-only kernel (raw weights through LDS, widened per wave, one request stream across tiles) on
+  a shape with hundreds of tiles per block, ragged groups, a ragged last n-tile and an empty group, against the
+  register-staged tiled kernel on the same operands (which the small-shape tests pin to the oracle), plus sampled rows
+  against the oracle's dequantised matmul."""
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
+
+  g = torch.Generator(device="cuda").manual_seed(17)
+  e, k, n = 16, 1088, 1984  # 17 stages of 64; 15.5 n-tiles of 128
+  gs_h = np.array([700, 1031, 0, 512, 256, 1300, 90, 777, 640, 515, 513, 511, 1024, 300, 999, 1100], np.int32)
+  m = int(gs_h.sum()) + 100  # 100 rows in no group
+  gs = torch.from_numpy(gs_h).cuda()
+  lhs = torch.randn(m, k, device="cuda", generator=g).to(torch.bfloat16)
+  kw, ws = {}, []
+  for _ in range(2 if glu else 1):
+    if fmt == "int8":
+      ws.append((torch.randint(-127, 128, (e, n, k), device="cuda", dtype=torch.int8, generator=g), torch.rand(e, n, device="cuda", generator=g) * 0.01 + 1e-3))
+    elif fmt in ("int4", "int4g32"):
+      grp = 128 if fmt == "int4" else 32
+      ws.append((torch.randint(0, 256, (e, n, k // 2), device="cuda", dtype=torch.uint8, generator=g),
+                 (torch.rand(e, n, (k + grp - 1) // grp, device="cuda", generator=g) * 0.01 + 1e-3).to(torch.bfloat16)))
+      kw.update(rhs_dtype=MOE_INT4, rhs_scale_block_k=grp)
+    else:
+      ws.append((torch.randint(0, 256, (e, n, k // 2), device="cuda", dtype=torch.uint8, generator=g),
+                 torch.randint(118, 126, (e, n, k // 32), device="cuda", dtype=torch.uint8, generator=g)))
+      kw.update(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+  kw["rhs_scale"] = ws[0][1]
+  if glu:
+    kw.update(rhs_up=ws[1][0], rhs_up_scale=ws[1][1], act="silu")
+  got = K.gmm_raw(lhs, ws[0][0], gs, **kw)
+  ref = K.gmm_raw(lhs, ws[0][0], gs, kernel="tiled", **kw)
+  assert relerr(got, ref) <= 1e-3
+  assert torch.all(got[int(gs_h.sum()):] == 0)
+  # a few rows of three groups against the oracle (first / last row of a group, a row next to the empty group)
+  off = np.concatenate([[0], np.cumsum(gs_h)])
+
+  def deq(w, sc):
+    w, sc = w.cpu(), sc.cpu()
+    if fmt == "int8":
+      return w.float() * sc[:, None]
+    if fmt in ("int4", "int4g32"):
+      return O.dequantize_int4(w, sc, 128 if fmt == "int4" else 32).float()
+    return O.dequantize_mxfp4(w.reshape(n, k // 32, 16), sc).float()
+
+  for gi in (0, 3, 15):
+    rows = [int(off[gi]), int(off[gi + 1]) - 1]
+    x = lhs[rows].cpu().double()
+    h0 = x @ deq(ws[0][0][gi], ws[0][1][gi]).double().T
+    want = torch.nn.functional.silu(h0) * (x @ deq(ws[1][0][gi], ws[1][1][gi]).double().T) if glu else h0
+    assert relerr(got[rows], want, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
