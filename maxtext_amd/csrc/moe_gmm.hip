@@ -173,7 +173,11 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
 static int tiled_kind_bm(TiledKind k) { return k == K_T64 ? 64 : k == K_T128 ? 128 : 256; }  // (every direct-to-LDS kernel: 256)
 
 static int launch_tiled_kind(TiledKind kind, int op, int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
-  if (kind == K_DL128) return launch_dl(op, glu, 128, false, p, M, G_total, s);
+  if (kind == K_DL128) {
+    // the stream kernel where its 32-bit offsets reach and K has three stages; the kernel that drains between tiles otherwise
+    if (dls_takes(op, p.K, p.N, p.ro.row_idx ? p.ro.lhs_rows : 0)) return launch_dls(op, glu, p, M, G_total, s);
+    return launch_dl(op, glu, 128, false, p, M, G_total, s);
+  }
   if (kind == K_DL64) return launch_dl(op, glu, 64, false, p, M, G_total, s);
   if (kind == K_DLW) return launch_dlw(bsrc, glu, p, M, G_total, s);
   return launch_tiled_bm(op, bsrc, glu, tiled_kind_bm(kind), false, p, M, G_total, s);
@@ -490,6 +494,7 @@ int moe_init(void) {
   if (int st = prepare_tiled()) return st;
   if (int st = prepare_dl()) return st;
   if (int st = prepare_dlw()) return st;
+  if (int st = prepare_dls()) return st;
   if (int st = prepare_tgmm()) return st;
   return prepare_fp8();
 }

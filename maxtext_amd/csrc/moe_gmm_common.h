@@ -307,6 +307,22 @@ __device__ __forceinline__ void own_channel_pieces(const v4i& a, const v4i& b, v
   }
 }
 
+// ---- buffer descriptors and the untracked global -> LDS copy of the persistent stream kernels ----
+
+// A raw buffer descriptor over `bytes` bytes at `base`: requests past the end return zeros instead of faulting, which
+// is how rows past a tile's (or a weight matrix's) end are dealt with.
+__device__ __forceinline__ v4i buffer_desc(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  return v4i{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+}
+__device__ __forceinline__ uint32_t clamp_u32(size_t v) { return v > 0xffffffffull ? 0xffffffffu : (uint32_t)v; }
+
+// global -> LDS copy of 16 bytes per lane through a buffer descriptor (1 KB per wave at lds_addr, a wave-uniform LDS byte
+// address), written as asm: the compiler then neither waits for it before LDS accesses that follow nor gives up counting
+// the LDS reads in flight.  Which buffer a copy writes and a read reads is settled by explicit waits and barriers.
+__device__ __forceinline__ void dma16_buffer(const v4i& rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
+}
 struct SkinnyParams {
   const uint8_t* lhs;      // [M, K] fp8
   const float* lhs_scale;  // [M, K/128]
@@ -399,6 +415,7 @@ int prepare_tiled();
 int prepare_dl();
 int prepare_fp8();
 int prepare_dlw();
+int prepare_dls();
 int prepare_tgmm();
 
 // ---- launchers (one translation unit per kernel family) ----
@@ -408,6 +425,9 @@ int launch_tiled_bm(int op, int bsrc, bool glu, int bm, bool block_scaled, const
 // moe_gmm_dl.hip: direct-to-LDS persistent kernel, 256 x 256 tiles; stage_bytes 128 or 64; rhs_kn: [G, K, N] bf16 weights
 int launch_dl(int op, bool glu, int stage_bytes, bool rhs_kn, const TiledParams& p, int M, int G_total, hipStream_t s);
 // moe_gmm_dlw.hip: the same pipeline for bf16 activations x int8 / int4 / mxfp4 weights (K % 64 == 0, default scale layouts)
+// moe_gmm_dls.hip: the persistent 256 x 256 kernel for int8 x int8 / bf16 x bf16 with one request stream across tiles
+int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
+bool dls_takes(int op, int K, int N, long long indexed_lhs_rows);
 int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
 // whether that kernel takes the shape (indexed_lhs_rows: rows of lhs when a row index is used, else 0)
 bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor);

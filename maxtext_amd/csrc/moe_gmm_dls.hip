@@ -1,0 +1,321 @@
+// Grouped matmul: the persistent 256 x 256 kernel for operands that need no conversion (int8 x int8, bf16 x bf16
+// prefill) with the stages of a block's consecutive tiles as ONE request stream.
+//
+// Both operands go global -> LDS without passing through registers (buffer_load ... lds, 1 KB = 8 rows of 128 bytes per
+// wave instruction; XOR-swizzled unpadded rows; two buffers of 64 KB; one barrier per stage).  8 waves as 2 x 4, each
+// 128 x 64 of the tile in 16 x 16 MFMAs (16x16x64 i8 / 16x16x32 bf16); weight fragments double-buffered, an activation
+// fragment reloaded for the next k-step right after the four MFMAs that use it.
+//
+// The requests run two stages ahead of the MFMAs ACROSS tile boundaries: a tile's first two stages arrive while the
+// previous tile is still being multiplied, and the record of the next tile is read a whole tile ahead.  Addresses go
+// through buffer descriptors that end where the tile's rows (the expert's weight matrix) end: rows past the end read as
+// zeros, the lane-dependent part of an address is the same for every tile and the tile-dependent part is scalar, so
+// moving the stream on to the next tile costs no vector work (with a row index: one index load per request).  What is
+// left between two tiles is the epilogue.
+
+#include "moe_gmm_common.h"
+
+namespace moe {
+
+template <int OP_, bool GLU_>
+struct DlsCfg {
+  static constexpr int OP = OP_;
+  static constexpr bool GLU = GLU_;
+  static constexpr int BM = 256, BN = 256, BKB = 128, MI = 16;
+  static constexpr int ESZ = OP == OP_I8 ? 1 : 2, BK = BKB / ESZ;
+  static constexpr int WAVES_M = 2, WAVES_N = 4, NWAVES = 8, THREADS = NWAVES * kWave;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / MI, TN = WN / MI;
+  static constexpr int A_STAGE = BM * BKB, STAGE = (BM + BN) * BKB, LDS_BYTES = 2 * STAGE;
+  static constexpr int A_IPW = BM / 8 / NWAVES, B_IPW = BN / 8 / NWAVES;  // requests per wave and stage: 4 + 4
+  static constexpr int OUT_BN = GLU ? BN / 2 : BN;
+  static_assert(OP == OP_I8 || OP == OP_BF16, "operands");
+  __device__ static __forceinline__ int swz(int row) { return (row >> 1) & 7; }
+};
+
+template <typename C>
+__global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int OP = C::OP;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
+  const int N = p.N, K = p.K;
+  const uint32_t row_bytes = (uint32_t)K * C::ESZ;
+  const int num_tiles = p.header[0];
+  const int total = p.max_m_tiles * p.tiles_n;
+  const int nk = K / C::BK;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+
+  struct Tile {
+    TileInfo info;
+    int n0, id;
+  };
+  struct Peek {  // a tile record that has been requested but not looked at yet
+    TileInfo ti;
+    int n0, id;
+    bool valid;
+  };
+  // tile id -> (m-tile, n-tile): ids congruent mod 8 run on one XCD and form an 8 x 4 patch that shares panels in its L2.
+  // The block's first id >= id0 that names an existing m-tile; its record is requested, not waited for.
+  auto peek_from = [&](int id0) -> Peek {
+    Peek pk;
+    pk.valid = false;
+    pk.n0 = 0;
+    pk.id = total;
+    pk.ti = TileInfo{-1, 0, 0, 0};
+    const int q = total / 8, rem = total % 8;
+    const int GSM = p.tune > 0 ? p.tune : 8;
+    const int width = GSM * p.tiles_n;
+    for (int id = id0; id < total; id += gridDim.x) {
+      const int xcd = id % 8, loc = id / 8;
+      const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+      const int sg = logical / width, first_m = sg * GSM;
+      const int gsz = min(p.max_m_tiles - first_m, GSM);
+      const int m_idx = first_m + (logical % width) % gsz;
+      if (m_idx >= num_tiles) continue;
+      pk.ti = p.tiles[m_idx];
+      pk.n0 = ((logical % width) / gsz) * C::OUT_BN;
+      pk.id = id;
+      pk.valid = true;
+      break;
+    }
+    return pk;
+  };
+  // Turns a requested record into the block's next tile that needs the matmul; tiles of rows that belong to no local
+  // group are written as zeros on the way (and the search goes on from there).
+  auto resolve = [&](Peek pk, Tile& t) -> bool {
+    while (pk.valid) {
+      // (uniform values: kept in scalar registers)
+      t.info.group = __builtin_amdgcn_readfirstlane(pk.ti.group);
+      t.info.row0 = __builtin_amdgcn_readfirstlane(pk.ti.row0);
+      t.info.nrows = __builtin_amdgcn_readfirstlane(pk.ti.nrows);
+      t.info.pad = 0;
+      t.n0 = __builtin_amdgcn_readfirstlane(pk.n0);
+      t.id = __builtin_amdgcn_readfirstlane(pk.id);
+      if (t.info.group >= 0) return true;
+      zero_fill_tile(p.out, p.ro, t.info.row0, t.info.nrows, t.n0, C::OUT_BN, N, tid, C::THREADS);
+      pk = peek_from(t.id + gridDim.x);
+    }
+    return false;
+  };
+
+  // ---- the loading side of the stream ---------------------------------------------------------------------------
+  // request i of this wave covers rows (wave * 4 + i) * 8 .. + 7 of the tile's 256 activation (weight) rows, 128 bytes
+  // of each; the lane's 16 bytes: global chunk = LDS slot ^ swizzle of the row
+  auto lane_off = [&](int i, uint32_t row) {
+    const int r = (wave * C::A_IPW + i) * 8 + lane / 8;
+    return row * row_bytes + (uint32_t)(((lane % 8) ^ C::swz(r)) << 4);
+  };
+  v4i a_desc, b_desc;
+  uint32_t a_voff[C::A_IPW], b_voff[C::B_IPW], b_soff = 0;
+  auto set_a_sources = [&](const Tile& t) {
+    if (p.ro.row_idx) {
+      a_desc = buffer_desc(p.lhs, clamp_u32((size_t)p.ro.lhs_rows * row_bytes));
+      int rows[C::A_IPW];
+#pragma unroll
+      for (int i = 0; i < C::A_IPW; i++) rows[i] = min(t.info.row0 + (wave * C::A_IPW + i) * 8 + lane / 8, p.M - 1);
+      lhs_rows_of<C::A_IPW>(p.ro, rows);
+#pragma unroll
+      for (int i = 0; i < C::A_IPW; i++) a_voff[i] = lane_off(i, (uint32_t)rows[i]);
+    } else {
+      a_desc = buffer_desc(p.lhs + (size_t)t.info.row0 * row_bytes, clamp_u32((size_t)t.info.nrows * row_bytes));
+    }
+  };
+  if (!p.ro.row_idx) {
+#pragma unroll
+    for (int i = 0; i < C::A_IPW; i++) a_voff[i] = lane_off(i, (uint32_t)((wave * C::A_IPW + i) * 8 + lane / 8));
+  }
+  // weights: with GLU the upper 128 of the tile's 256 rows are the second projection's, whose requests come from waves 4 .. 7
+  const bool load_up = C::GLU && wave >= C::NWAVES / 2;
+#pragma unroll
+  for (int i = 0; i < C::B_IPW; i++) {
+    const int r = (wave * C::B_IPW + i) * 8 + lane / 8;
+    b_voff[i] = lane_off(i, (uint32_t)(C::GLU ? r % (C::BN / 2) : r));
+  }
+  auto set_b_sources = [&](const Tile& t) {
+    b_desc = buffer_desc((load_up ? p.rhs_up : p.rhs) + (size_t)t.info.group * N * row_bytes, clamp_u32((size_t)N * row_bytes));
+    b_soff = (uint32_t)t.n0 * row_bytes;
+  };
+  // request idx of the stage: 0 .. 3 activations, 4 .. 7 weights
+  auto issue_one = [&](int kt, int buf, int idx) {
+    if (idx < C::A_IPW) dma16_buffer(a_desc, a_voff[idx], (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + (wave * C::A_IPW + idx) * 1024);
+    else dma16_buffer(b_desc, b_voff[idx - C::A_IPW], b_soff + (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + C::A_STAGE + (wave * C::B_IPW + idx - C::A_IPW) * 1024);
+  };
+
+  // ---- the multiplying side ----------------------------------------------------------------------------------------
+  typedef typename std::conditional<OP == OP_I8, v4i, v4f>::type acc_t;
+  acc_t acc[C::TN][C::TM];
+  int b_row[C::TN];
+#pragma unroll
+  for (int j = 0; j < C::TN; j++) {
+    if (C::GLU) {
+      constexpr int H = C::TN / 2;
+      b_row[j] = (j < H ? 0 : C::BN / 2) + wn * (C::WN / 2) + (j < H ? j : j - H) * C::MI;
+    } else {
+      b_row[j] = wn * C::WN + j * C::MI;
+    }
+  }
+  // fragment of k-step ks: row (lane % 16), chunk q = 4 * ks + lane / 16, stored at slot q ^ swz(row)
+  const int frag_lane = (lane % 16) * C::BKB + (((lane / 16) ^ C::swz(lane % 16)) << 4);
+  v4i ga[C::TM], gb[2][C::TN];
+  auto read_a = [&](int buf, int ks, int i) {
+    ga[i] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB + (frag_lane ^ (ks * 64)));
+  };
+  auto read_b = [&](int buf, int ks, int set, int j) {
+    gb[set][j] = *(const v4i*)(smem + buf * C::STAGE + C::A_STAGE + b_row[j] * C::BKB + (frag_lane ^ (ks * 64)));
+  };
+  // One k-step of 32 MFMAs on the fragments in registers.  ZC: a tile's first k-step starts from zero.  RD: the fragments
+  // of the next k-step (rd_buf, rd_ks) are read behind the MFMAs (the weights' into the other set, an activation fragment
+  // in place once its four MFMAs are out).  LD: the eight requests of stage ld_kt of the loading tile go out into ld_buf,
+  // one per MFMA from the start of the k-step.
+  auto kstep = [&](auto set_c, auto rd_c, auto ld_c, auto zc_c, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
+    constexpr int SET = decltype(set_c)::value;
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value, ZC = decltype(zc_c)::value;
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) {
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) {
+        if constexpr (OP == OP_I8) {
+          acc[j][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(gb[SET][j], ga[i], ZC ? v4i{0, 0, 0, 0} : acc[j][i], 0, 0, 0);
+        } else {
+          acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, gb[SET][j]), __builtin_bit_cast(v8bf, ga[i]),
+                                                              ZC ? v4f{0.f, 0.f, 0.f, 0.f} : acc[j][i], 0, 0, 0);
+        }
+        const int slot = i * C::TN + j;
+        if (LD && slot < C::A_IPW + C::B_IPW) issue_one(ld_kt, ld_buf, slot);
+        if (RD && j == 1 && i < C::TN) read_b(rd_buf, rd_ks, SET ^ 1, i);
+        if (RD && j == C::TN - 1) read_a(rd_buf, rd_ks, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
+
+  // The fragments of a tile's first k-step (stage 0 in buffer `buf`), with nothing to hide behind.
+  auto first_fragments = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < C::TM; i++) read_a(buf, 0, i);
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) read_b(buf, 0, 0, j);
+  };
+
+  Tile cur, nxt;
+  if (!resolve(peek_from(blockIdx.x), cur)) return;
+  // ---- head of the stream: the first tile's stages 0 and 1 ----
+  set_a_sources(cur);
+  set_b_sources(cur);
+#pragma unroll
+  for (int s = 0; s < 2; s++)
+#pragma unroll
+    for (int i = 0; i < C::A_IPW + C::B_IPW; i++) issue_one(s, s, i);
+  wait_vmcnt<0>();
+  asm volatile("s_barrier" ::: "memory");
+  first_fragments(0);
+
+  int base = 0;  // the buffer that holds stage 0 of the current tile
+  while (true) {
+    // the record of the block's next tile is requested now and looked at two stages before this tile ends
+    Peek pk = peek_from(cur.id + gridDim.x);
+    bool have_n = false;
+    const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+    EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+    // first half of stage 0; the fragments of its second half are read behind it
+    kstep(S0{}, T_{}, F_{}, T_{}, base, 1, 0, 0);
+    // Iteration `it`: the second half of stage it, then the first half of stage it + 1.  Every fragment of stage it is in
+    // registers before the barrier, and stage it + 1 has landed at it: the buffer of stage it takes stage it + 2 of the
+    // stream (from nk on: the next tile's).
+    auto stream_kt = [&](int s) { return s < nk ? s : (have_n ? s - nk : nk - 1); };
+    int cb = base;  // buffer of stage `it`
+    auto iteration = [&](int it, auto last_c) {
+      constexpr bool LAST = decltype(last_c)::value;  // the tile's last half stage: nothing is read behind it
+      // own fragment reads done, own requests landed: then everybody's
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      wait_vmcnt<0>();
+      asm volatile("s_barrier" ::: "memory");
+      if (LAST) {
+        kstep(S1{}, F_{}, T_{}, F_{}, 0, 0, stream_kt(it + 2), cb);
+      } else {
+        kstep(S1{}, T_{}, T_{}, F_{}, cb ^ 1, 0, stream_kt(it + 2), cb);
+        kstep(S0{}, T_{}, F_{}, F_{}, cb ^ 1, 1, 0, 0);
+      }
+      cb ^= 1;
+    };
+    for (int it = 0; it < nk - 2; it++) iteration(it, F_{});
+    // the stream crosses into the next tile
+    have_n = resolve(pk, nxt);
+    if (have_n) {
+      set_a_sources(nxt);
+      set_b_sources(nxt);
+    }
+    iteration(nk - 2, F_{});
+    iteration(nk - 1, T_{});
+    // (requested only now: ahead of the last k-step the scales would push request offsets out to scratch memory, and
+    // every reload between two requests waits for all requests in flight)
+    load_epilogue_scales<C::TM, NT_OUT, C::GLU, true, C::MI>(esc, p, cur.info, wm * C::WM, n_out0, lane);
+    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, cur.info, wm * C::WM, n_out0, lane);
+    if (!have_n) break;
+    cur = nxt;
+    base = cb;  // the buffer of stage nk = the next tile's stage 0, landed before the last barrier
+    first_fragments(base);
+  }
+  // nothing may still be writing LDS when the block ends
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  wait_vmcnt<0>();
+}
+
+// ---------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------
+
+template <typename C>
+static int prepare_dls_cfg() {
+  return reserve_lds(gmm_dls_kernel<C>, C::LDS_BYTES, lds_flags<C>());
+}
+
+int prepare_dls() {
+  int st = MOE_OK;
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_I8, false>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_I8, true>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_BF16, false>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_BF16, true>>();
+  return st;
+}
+
+template <typename C>
+static int launch_dls_cfg(const TiledParams& p0, int M, int G_total, hipStream_t s) {
+  if (int st = prepare_dls_cfg<C>()) return st;
+  TiledParams p = p0;
+  p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
+  p.tiles_n = cdiv(p.N, C::OUT_BN);
+  const long long tiles = (long long)p.max_m_tiles * p.tiles_n;
+  if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  // one persistent block per CU (the LDS footprint allows no more); a multiple of 8 keeps "tile id mod 8"
+  // equal to the XCD a block runs on
+  int num_cus = 0;
+  if (int st = device_cu_count(&num_cus)) return st;
+  long long blocks = tiles < num_cus ? tiles : num_cus;
+  if (blocks >= 8) blocks -= blocks % 8;
+  gmm_dls_kernel<C><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
+  return check_launch("gmm_dls_kernel");
+}
+
+bool dls_takes(int op, int K, int N, long long indexed_lhs_rows) {
+  // whole 128-byte stages, at least three of them (the stream looks two stages ahead, into the next tile at most); byte
+  // offsets inside one expert's weight matrix and inside the activations that a row index may address fit 32 bits
+  const long long esz = op == OP_I8 ? 1 : 2;
+  return (op == OP_I8 || op == OP_BF16) && (K * esz) % 128 == 0 && K * esz >= 384 && (long long)N * K * esz < (1LL << 32) &&
+         indexed_lhs_rows * K * esz < (1LL << 32);
+}
+
+int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
+  if (!dls_takes(op, p.K, p.N, p.ro.row_idx ? p.ro.lhs_rows : 0))
+    return fail(MOE_ERR_UNSUPPORTED, "gmm: the stream kernel needs int8 or bf16 operands, whole 128-byte stages (three or more) and 32-bit byte offsets");
+  if (op == OP_I8) return glu ? launch_dls_cfg<DlsCfg<OP_I8, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_I8, false>>(p, M, G_total, s);
+  return glu ? launch_dls_cfg<DlsCfg<OP_BF16, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_BF16, false>>(p, M, G_total, s);
+}
+
+}  // namespace moe

@@ -44,20 +44,6 @@ struct DlwCfg {
   __device__ static __forceinline__ int swz_b(int row) { return NIBBLES ? (row >> 3) & 1 : (row >> 2) & 3; }
 };
 
-// A raw buffer descriptor over `bytes` bytes at `base`: requests past the end return zeros instead of faulting, which
-// is how rows past a tile's (or a weight matrix's) end are dealt with.
-__device__ __forceinline__ v4i buffer_desc(const void* base, uint32_t bytes) {
-  const uint64_t a = (uint64_t)base;
-  return v4i{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
-}
-__device__ __forceinline__ uint32_t clamp_u32(size_t v) { return v > 0xffffffffull ? 0xffffffffu : (uint32_t)v; }
-
-// global -> LDS copy of 16 bytes per lane through a buffer descriptor (1 KB per wave at lds_addr, a wave-uniform LDS byte
-// address), written as asm: the compiler then neither waits for it before LDS accesses that follow nor gives up counting
-// the LDS reads in flight.  Which buffer a copy writes and a read reads is settled by explicit waits and barriers.
-__device__ __forceinline__ void dma16_buffer(const v4i& rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
-}
 template <typename C>
 __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParams p0) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
