@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # and the figure is reported only while the sources still hash to that value: a kernel that changed since has no
 # measured traffic until its profile is refreshed.
 PROFILE_OF = {
-    "c2": ("profiles/gmm_dl_kernel_int8_mixtral_prefill_c2.md", ["moe_gmm_dl.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c2": ("profiles/gmm_dls_kernel_int8_mixtral_prefill_c2.md", ["moe_gmm_dls.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c3": ("profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md", ["moe_gmm_fp8.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c4": ("profiles/gmm_dlw_kernel_int8w_qwen3_prefill_c4.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c5": ("profiles/gmm_dlw_kernel_int4w_gptoss_prefill_c5_t4096.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
@@ -123,7 +123,7 @@ def dominant_kernel_model(wl, group_sizes):
   op = "int8" if cfg.act_quant == "int8" else "bf16"
   big = rows >= 128 * len(group_sizes)  # the dispatch rule of moe_gmm for its persistent 256 x 256 kernels
   if cfg.act_quant == "int8" or wl.weight_quant in (None, "bf16"):
-    kernel = "gmm_dl_kernel" if big else "gmm_tiled_kernel"
+    kernel = "gmm_dls_kernel" if big else "gmm_tiled_kernel"
   else:
     kernel = "gmm_dlw_kernel" if big and d % 64 == 0 else "gmm_tiled_kernel"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
