@@ -10,7 +10,8 @@ import ctypes
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libmoe_mi355x.so")
+# MOE_MI355X_LIB points the loader at another build of the same library (a tuning variant, an installed copy)
+LIB_PATH = os.environ.get("MOE_MI355X_LIB") or os.path.join(_PKG, "lib", "libmoe_mi355x.so")
 
 # enums of include/moe_mi355x.h
 MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32, MOE_MXFP4 = 0, 1, 2, 3, 4, 5

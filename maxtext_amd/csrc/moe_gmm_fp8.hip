@@ -21,11 +21,16 @@ __device__ __forceinline__ v8i load_a128(const uint8_t* p) {
   return r;
 }
 
+// The two whole-line requests of a 128-byte weight k-block as they arrive (channels i%8 and i%8 + 8), and the
+// fragment made of them once they are there.
+struct RawW128 { v4i lo, hi; };
 template <bool STREAM>
-__device__ __forceinline__ v8i load_w128(const uint8_t* lo_rows, const uint8_t* hi_rows) {
-  const v4i a = load_w16<STREAM>(lo_rows), b = load_w16<STREAM>(hi_rows);
+__device__ __forceinline__ RawW128 request_w128(const uint8_t* lo_rows, const uint8_t* hi_rows) {
+  return RawW128{load_w16<STREAM>(lo_rows), load_w16<STREAM>(hi_rows)};
+}
+__device__ __forceinline__ v8i fragment_w128(const RawW128& w) {
   v4i x, y;
-  own_channel_pieces(a, b, x, y);
+  own_channel_pieces(w.lo, w.hi, x, y);
   v8i r;
 #pragma unroll
   for (int c = 0; c < 4; c++) {
@@ -36,7 +41,8 @@ __device__ __forceinline__ v8i load_w128(const uint8_t* lo_rows, const uint8_t* 
 }
 
 // One wave owns NT tiles of 16 output channels (x2 with GLU) and MT tiles of 16 rows, and walks K in
-// steps of U 128-byte blocks whose loads are all issued before the first MFMA of the step.
+// steps of U 128-byte blocks whose loads are all issued before the first MFMA of the step (the compiler unrolls the
+// loop and moves the next steps' requests ahead of the current step's MFMAs as far as the registers allow).
 template <int MT, int NT, int U, bool GLU>
 __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams p) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -93,17 +99,17 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
     }
   const v4f zero = {0.f, 0.f, 0.f, 0.f};
 
-  auto step = [&](int kb0, auto ucount) {
+  // operands of one step of UC k-blocks, as requested
+  auto request = [&](int kb0, auto ucount, RawW128 (&wf)[U][NT], RawW128 (&uf)[U][GLU ? NT : 1], v8i (&af)[U][MT],
+                     float (&ws)[U][NT], float (&us)[U][NT], float (&as)[U][MT]) {
     constexpr int UC = decltype(ucount)::value;
-    v8i wf[UC][NT], uf[UC][NT], af[UC][MT];
-    float ws[UC][NT], us[UC][NT], as[UC][MT];
 #pragma unroll
     for (int u = 0; u < UC; u++) {
       const size_t off = (size_t)(kb0 + u) * 128;
 #pragma unroll
       for (int t = 0; t < NT; t++) {
-        wf[u][t] = load_w128<MT == 1>(wbase + wlo[t] + off, wbase + whi[t] + off);
-        if (GLU) uf[u][t] = load_w128<MT == 1>(ubase + wlo[t] + off, ubase + whi[t] + off);
+        wf[u][t] = request_w128<MT == 1>(wbase + wlo[t] + off, wbase + whi[t] + off);
+        if (GLU) uf[u][t] = request_w128<MT == 1>(ubase + wlo[t] + off, ubase + whi[t] + off);
       }
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) af[u][mt] = load_a128(ap[mt] + off);
@@ -119,28 +125,47 @@ __global__ __launch_bounds__(256) void gmm_fp8_skinny_kernel(const SkinnyParams 
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) as[u][mt] = asp[mt] ? asp[mt][kb0 + u] : 1.0f;
     }
+  };
+  auto multiply = [&](auto ucount, const RawW128 (&wf)[U][NT], const RawW128 (&uf)[U][GLU ? NT : 1], const v8i (&af)[U][MT],
+                      const float (&ws)[U][NT], const float (&us)[U][NT], const float (&as)[U][MT]) {
+    constexpr int UC = decltype(ucount)::value;
 #pragma unroll
     for (int u = 0; u < UC; u++)
 #pragma unroll
-      for (int t = 0; t < NT; t++)
+      for (int t = 0; t < NT; t++) {
+        const v8i w = fragment_w128(wf[u][t]);
+        v8i wu = w;
+        if (GLU) wu = fragment_w128(uf[u][t]);
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-          const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[u][t], af[u][mt], zero, 0, 0, 0, 127, 0, 127);
+          const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, af[u][mt], zero, 0, 0, 0, 127, 0, 127);
           const float sg = as[u][mt] * ws[u][t];
 #pragma unroll
           for (int r = 0; r < 4; r++) acc_g[t][mt][r] = fmaf(pg[r], sg, acc_g[t][mt][r]);
           if (GLU) {
-            const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf[u][t], af[u][mt], zero, 0, 0, 0, 127, 0, 127);
+            const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wu, af[u][mt], zero, 0, 0, 0, 127, 0, 127);
             const float su = as[u][mt] * us[u][t];
 #pragma unroll
             for (int r = 0; r < 4; r++) acc_u[t][mt][r] = fmaf(pu[r], su, acc_u[t][mt][r]);
           }
         }
+      }
   };
 
-  int kb = 0;
-  for (; kb + U <= nkb; kb += U) step(kb, std::integral_constant<int, U>{});
-  for (; kb < nkb; kb++) step(kb, std::integral_constant<int, 1>{});
+  RawW128 wf0[U][NT], uf0[U][GLU ? NT : 1];
+  v8i af0[U][MT];
+  float ws0[U][NT], us0[U][NT], as0[U][MT];
+  constexpr std::integral_constant<int, U> full{};
+  constexpr std::integral_constant<int, 1> one{};
+  const int nfull = nkb / U;
+  for (int s = 0; s < nfull; s++) {
+    request(s * U, full, wf0, uf0, af0, ws0, us0, as0);
+    multiply(full, wf0, uf0, af0, ws0, us0, as0);
+  }
+  for (int kb = nfull * U; kb < nkb; kb++) {
+    request(kb, one, wf0, uf0, af0, ws0, us0, as0);
+    multiply(one, wf0, uf0, af0, ws0, us0, as0);
+  }
 
   dispatch_act(GLU ? p.act : MOE_ACT_NONE, [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
@@ -738,12 +763,13 @@ static int launch_skinny(SkinnyParams p, bool glu, int max_tiles, hipStream_t s)
   return check_launch("gmm_fp8_skinny_kernel");
 }
 
-// (NT, U) of the fp8 streaming kernel, from sweeps over NT in {1, 2, 4} and U in {1, 2, 4} on the DeepSeek-V3 shapes:
-// 16-row tiles take 4 channel tiles per wave and one K block per step with fused GLU, 2 tiles and 4 blocks without;
-// 64-row tiles take 2 tiles and one block.
+// (NT, U) of the fp8 streaming kernel, from sweeps over NT in {1, 2, 4, 8} and U in {1, 2, 4, 8} on the DeepSeek-V3 shapes
+// (257 experts, 8 rows each): 16-row tiles take one K block per step, 2 channel tiles per wave with fused GLU (7168 -> 2048:
+// 1.22 ms against 1.33 ms with 4 tiles, 1.28 ms with 1) and 4 tiles without (2048 -> 7168: 0.65 ms against 0.67 ms with
+// 2 tiles and 4 blocks, 0.69 ms with 8 tiles); 64-row tiles take 2 tiles and one block.
 int launch_fp8_skinny(bool few_rows, const SkinnyParams& p, bool glu, int max_tiles, hipStream_t s) {
   if (!few_rows) return launch_skinny<4, 2, 1>(p, glu, max_tiles, s);
-  return glu ? launch_skinny<1, 4, 1>(p, glu, max_tiles, s) : launch_skinny<1, 2, 4>(p, glu, max_tiles, s);
+  return glu ? launch_skinny<1, 2, 1>(p, glu, max_tiles, s) : launch_skinny<1, 4, 1>(p, glu, max_tiles, s);
 }
 
 }  // namespace moe
