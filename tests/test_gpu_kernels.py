@@ -993,18 +993,24 @@ def _random_case(rng, k_mult):
   e = int(rng.integers(1, 9))
   k = int(rng.integers(1, 9)) * k_mult
   n = int(rng.integers(1, 40)) * 8
-  regime = rng.integers(0, 3)  # few rows per expert (streaming kernels), medium, many (256-row tiles)
-  hi = (12, 90, 400)[regime]
-  gs = rng.integers(0, hi, e)
-  gs[rng.integers(0, e)] = 0 if e > 1 and rng.random() < 0.5 else gs[rng.integers(0, e)]
+  # few rows per expert (streaming kernels), medium, many (256-row tiles), skewed (one hot expert among cold ones: the
+  # tile height follows the average, so the hot expert spans many small tiles or the cold ones sit in big tiles)
+  regime = rng.integers(0, 4)
+  if regime == 3:
+    gs = rng.integers(0, 7, e)
+    gs[rng.integers(0, e)] = rng.integers(150, 700)
+  else:
+    hi = (12, 90, 400)[regime]
+    gs = rng.integers(0, hi, e)
+    gs[rng.integers(0, e)] = 0 if e > 1 and rng.random() < 0.5 else gs[rng.integers(0, e)]
   m = int(gs.sum()) + int(rng.integers(0, 20))  # trailing rows that belong to no group
   return max(m, 1), k, n, gs.astype(np.int32)
 
 
 @pytest.mark.parametrize("family", ["bf16", "w8", "i8", "int4", "mxfp4", "fp8"])
 def test_gmm_random_shapes(K, family):
-  """20 random (M, K, N, group_sizes) per operand family against the oracle: ragged groups, empty groups, rows
-  past the last group, K and N at every supported granularity, with and without the fused activation and bias."""
+  """20 random (M, K, N, group_sizes) per operand family against the oracle: ragged groups, empty groups, skewed
+  groups, rows past the last group, K and N at every supported granularity, with and without the fused activation and bias."""
   from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
 
   rng = np.random.default_rng({"bf16": 1, "w8": 2, "i8": 3, "int4": 4, "mxfp4": 5, "fp8": 6}[family])
