@@ -308,7 +308,8 @@ typedef enum {
   MOE_GMM_KERNEL_AUTO = 0,
   MOE_GMM_KERNEL_STREAM = 1,    /* streaming kernels without LDS tiles (fp8 block-scaled, weight-only formats)        */
   MOE_GMM_KERNEL_TILED = 2,     /* LDS-tiled kernels with the m-tile chosen by rows per expert (fp8: 128 x 128)       */
-  MOE_GMM_KERNEL_BIG = 3,       /* 256 x 256 tiles: fp8 block-scaled big kernel; int8 x int8 register-staged kernel   */
+  MOE_GMM_KERNEL_BIG = 3,       /* 256 x 256 tiles: fp8 block-scaled (the persistent stream kernel when K % 512 == 0,
+                                   what AUTO picks for prefill-sized groups); int8 x int8 register-staged kernel       */
   MOE_GMM_KERNEL_DL64 = 4,      /* direct-to-LDS persistent kernel with 64-byte stages (int8 x int8, bf16 x bf16)     */
   MOE_GMM_KERNEL_STREAM_NOSPLIT = 5 /* weight-only streaming kernel with every wave walking all of K                   */
 } moe_gmm_kernel;

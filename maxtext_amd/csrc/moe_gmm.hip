@@ -299,7 +299,11 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     if (tiled) {
       const bool big = kernel == MOE_GMM_KERNEL_BIG;
       if (big && !fp8_blocks) return fail(MOE_ERR_UNSUPPORTED, "gmm: the 256 x 256 fp8 kernel takes block-scaled operands only");
-      map_tiles(big ? 256 : 128);
+      // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
+      const bool chip_full = (long long)max_tiles_for(M, G, 256) * cdiv(N, glu ? 128 : 256) >= 128;
+      const bool stream = fp8_blocks && f8s_takes(K, N, M, ro.row_idx ? ro.lhs_rows : 0) &&
+                          (big || (kernel == MOE_GMM_KERNEL_AUTO && (long long)M >= 128LL * G && chip_full));
+      map_tiles(big || stream ? 256 : 128);
       Fp8TiledParams P = {};
       TiledParams& q = P.base;
       q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
@@ -314,6 +318,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
         q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
         q.rhs_scale_gstride = sp.rhs_gstride; q.rhs_scale_nstride = sp.rhs_nstride;
       }
+      if (stream) return launch_f8s(glu, P, M, G, s);
       const bool vec4 = fp8_blocks && (K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
       return launch_fp8_tiled(big, glu, vec4, P, M, G, s);
     }
@@ -496,6 +501,7 @@ int moe_init(void) {
   if (int st = prepare_dlw()) return st;
   if (int st = prepare_dls()) return st;
   if (int st = prepare_tgmm()) return st;
+  if (int st = prepare_f8s()) return st;
   return prepare_fp8();
 }
 

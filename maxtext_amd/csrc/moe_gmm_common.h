@@ -321,6 +321,7 @@ __device__ __forceinline__ uint32_t clamp_u32(size_t v) { return v > 0xffffffffu
 // address), written as asm: the compiler then neither waits for it before LDS accesses that follow nor gives up counting
 // the LDS reads in flight.  Which buffer a copy writes and a read reads is settled by explicit waits and barriers.
 __device__ __forceinline__ void dma16_buffer(const v4i& rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
+  asm volatile("" : "+s"(soff));  // (a literal offset is not an operand the instruction takes)
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
 }
 struct SkinnyParams {
@@ -428,6 +429,11 @@ int launch_dl(int op, bool glu, int stage_bytes, bool rhs_kn, const TiledParams&
 // moe_gmm_dls.hip: the persistent 256 x 256 kernel for int8 x int8 / bf16 x bf16 with one request stream across tiles
 int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
 bool dls_takes(int op, int K, int N, long long indexed_lhs_rows);
+// moe_gmm_f8s.hip: the same stream for block-scaled fp8 (1 x 128 activation scales, 128 x 128 weight scales)
+struct Fp8TiledParams;
+int launch_f8s(bool glu, const Fp8TiledParams& P, int M, int G_total, hipStream_t s);
+bool f8s_takes(int K, int N, long long M, long long indexed_lhs_rows);
+int prepare_f8s();
 int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
 // whether that kernel takes the shape (indexed_lhs_rows: rows of lhs when a row index is used, else 0)
 bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor);

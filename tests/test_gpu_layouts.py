@@ -317,3 +317,47 @@ def test_weight_only_prefill_kernel_against_the_tiled_kernel_at_size(K, fmt, glu
     h0 = x @ deq(ws[0][0][gi], ws[0][1][gi]).double().T
     want = torch.nn.functional.silu(h0) * (x @ deq(ws[1][0][gi], ws[1][1][gi]).double().T) if glu else h0
     assert relerr(got[rows], want, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
+
+
+@pytest.mark.parametrize("glu", [False, True])
+@pytest.mark.parametrize("indexed", [False, True])
+def test_fp8_prefill_stream_kernel_against_the_tiled_kernel_at_size(K, glu, indexed):
+  """The persistent block-scaled fp8 kernel (256 x 256 tiles, scales staged through LDS four stages at a time, one
+  request stream across tiles) on a shape with many tiles per block, ragged and empty groups, a ragged last n-tile and
+  rows in no group, against the 128 x 128 kernel on the same operands (pinned to the oracle by the small-shape tests):
+  both add scale * partial sum per 128-wide block in the same order, so the results agree bit for bit.  Sampled rows
+  are checked against a float64 restatement of the block-scaled product."""
+  g = torch.Generator(device="cuda").manual_seed(23)
+  e, k, n = 12, 1536, 1664  # 12 stages (3 scale groups of 4); 6.5 n-tiles of 256
+  gs_h = np.array([700, 1031, 0, 512, 256, 1300, 90, 777, 640, 515, 513, 260], np.int32)
+  m = int(gs_h.sum()) + 60
+  gs = torch.from_numpy(gs_h).cuda()
+  lhs = (torch.randn(m, k, device="cuda", generator=g) * 2).to(torch.float8_e4m3fn)
+  asc = torch.rand(m, k // 128, device="cuda", generator=g) * 0.02 + 1e-3
+  ws = [((torch.randn(e, n, k, device="cuda", generator=g) * 2).to(torch.float8_e4m3fn),
+         torch.rand(e, n // 128, k // 128, device="cuda", generator=g) * 0.02 + 1e-3) for _ in range(2)]
+  kw = dict(lhs_scale=asc, rhs_scale=ws[0][1], lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128)
+  if glu:
+    kw.update(rhs_up=ws[1][0], rhs_up_scale=ws[1][1], act="silu")
+  src = torch.arange(m, device="cuda", dtype=torch.int32)
+  if indexed:  # every activation row is read through an index, from half as many rows
+    src = torch.randperm(m, device="cuda", generator=g).to(torch.int32)
+    lhs, asc = lhs[: (m + 1) // 2].contiguous(), asc[: (m + 1) // 2].contiguous()
+    kw.update(lhs_scale=asc, lhs_row_idx=src, lhs_row_idx_div=2, num_rows=m)
+  got = K.gmm_raw(lhs, ws[0][0], gs, kernel="big", **kw)
+  ref = K.gmm_raw(lhs, ws[0][0], gs, kernel="tiled", **kw)
+  assert torch.equal(got, ref)
+  assert torch.all(got[int(gs_h.sum()):] == 0)
+  off = np.concatenate([[0], np.cumsum(gs_h)])
+
+  def product(rows, w, sc):  # sum over the blocks of (a_scale * w_scale) * (a_block @ w_block^T)
+    idx = (src[rows] // 2).long() if indexed else torch.tensor(rows)
+    a = lhs[idx].cpu().double().reshape(len(rows), k // 128, 128) * asc[idx].cpu().double()[:, :, None]
+    wd = w.cpu().double().reshape(n, k // 128, 128) * torch.repeat_interleave(sc.cpu().double(), 128, dim=0)[:, :, None]
+    return torch.einsum("rbk,nbk->rn", a, wd)
+
+  for gi in (0, 5, 11):
+    rows = [int(off[gi]), int(off[gi + 1]) - 1]
+    h0 = product(rows, ws[0][0][gi], ws[0][1][gi])
+    want = torch.nn.functional.silu(h0) * product(rows, ws[1][0][gi], ws[1][1][gi]) if glu else h0
+    assert relerr(got[rows], want, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
