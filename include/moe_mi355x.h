@@ -397,6 +397,27 @@ MOE_API int moe_glu_act(const void* h0, const void* h1, size_t n, int act, float
 MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, size_t n, int act, float act_limit,
                             void* dh0, void* dh1, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Gradient preparation of the quantised backward pass (int8 x int8 forward with channelwise scales): the incoming
+ * gradient times the scale of the axis that the gradient product contracts away (_bwd_prepare_inputs,
+ * kernels/megablox/ops.py:530-580), optionally quantised to float8_e5m2 (_bwd_quantize_gradient, ops.py:583-604;
+ * symmetric absmax scale = absmax / 57344, values rounded to nearest even, a zero scale gives zeros).
+ *
+ *   MOE_BWD_FOR_DLHS  d[m, n] = bf16(dout[m, n] * bf16(factor[g(m), n]));  factor = rhs scales [G_local, N] f32, g(m) the
+ *                     expert of row m relative to group_offset, clamped to the local experts; quantised per row:
+ *                     scale_out [M]
+ *   MOE_BWD_FOR_DRHS  d[m, n] = bf16(dout[m, n] * bf16(factor[m]));  factor = lhs scales [M] f32; quantised per column:
+ *                     scale_out [N] (group_sizes is not used)
+ *
+ *   dout [M, N] bf16;  out [M, N] bf16: d itself (quantize == 0; scale_out is not touched), or d / scale on the e5m2
+ *   grid, whose values are exact in bf16 (quantize != 0), so that moe_gmm / moe_tgmm take it as a bf16 operand.
+ * Limits: N % 8 == 0, N <= 16384, at most 1024 groups.
+ */
+typedef enum { MOE_BWD_FOR_DLHS = 0, MOE_BWD_FOR_DRHS = 1 } moe_bwd_mode;
+MOE_API int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, const float* factor,
+                               const int32_t* group_sizes, int num_groups_total, int num_groups_local, int group_offset,
+                               void* out, float* scale_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

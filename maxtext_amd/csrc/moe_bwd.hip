@@ -1,0 +1,213 @@
+// Gradient preparation of the quantised backward pass: the incoming gradient times the scale of the axis the product
+// contracts away (_bwd_prepare_inputs, kernels/megablox/ops.py:530-580), optionally quantised to float8_e5m2 per row or
+// per column (_bwd_quantize_gradient, ops.py:583-604).  The e5m2 values are written as bf16, in which they are exact, so
+// both gradient products run on the bf16 kernels.
+
+#include "moe_common.h"
+
+namespace moe {
+
+constexpr float kE5m2Max = 57344.0f;
+
+// absmax / 57344 rounded once (the quotient is formed in f64: one ulp of the scale moves values across e5m2 rounding
+// boundaries)
+__device__ __forceinline__ float e5m2_scale(float amax) { return (float)((double)amax / (double)kE5m2Max); }
+
+// x / scale rounded to the float8_e5m2 grid, to nearest even (2 mantissa bits; subnormals are multiples of 2^-16); a
+// zero scale gives zero
+__device__ __forceinline__ float to_e5m2_grid(float x, float scale) {
+  if (scale == 0.f) return 0.f;
+  const float q = x / scale;
+  const float a = fabsf(q);
+  if (!(a < INFINITY)) return q;  // inf / nan as they are
+  float r;
+  if (a < 6.103515625e-05f) {  // below 2^-14
+    r = rintf(a * 65536.0f) * (1.0f / 65536.0f);
+  } else {
+    uint32_t b = __float_as_uint(a);
+    b += 0x000FFFFFu + ((b >> 21) & 1u);
+    b &= 0xFFE00000u;
+    r = __uint_as_float(b);
+    if (r > kE5m2Max) r = INFINITY;  // what the cast gives beyond the largest finite value
+  }
+  return copysignf(r, q);
+}
+
+// expert of row m as the reference's backward sees it: the number of group ends <= m, taken relative to the first
+// local group and clamped to the local range (rows of other shards and rows past the last group take the nearest
+// local expert: their gradient rows do not reach the result)
+__device__ __forceinline__ int local_group_of(const int* ends, int G_total, int m, int group_offset, int G_local) {
+  int lo = 0, hi = G_total;  // first index with ends[i] > m
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (ends[mid] > m) hi = mid;
+    else lo = mid + 1;
+  }
+  return min(max(lo - group_offset, 0), G_local - 1);
+}
+
+constexpr int kBwdThreads = 256;
+constexpr int kBwdMaxChunks = 8;  // 8 bf16 per lane and chunk: rows of up to 16384 values
+constexpr int kBwdMaxGroups = 1024;
+
+// One block per row: d = bf16(dout * bf16(factor)), factor = rhs_scale[group(row), n] (BY_CHANNEL) or lhs_scale[row];
+// ROW_QUANT: the row's absmax, then the e5m2 values and the row's scale.
+template <bool BY_CHANNEL, bool ROW_QUANT>
+__global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4* dout, int N, const float* factor, const int* group_sizes,
+                                                                     int G_total, int G_local, int group_offset, uint4* out,
+                                                                     float* scale_out) {
+  __shared__ int ends[BY_CHANNEL ? kBwdMaxGroups : 1];
+  __shared__ uint32_t wmax[kBwdThreads / kWave];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  const float* f = factor;
+  float row_f = 1.0f;
+  if (BY_CHANNEL) {
+    if (tid == 0) {
+      int run = 0;
+      for (int g = 0; g < G_total; g++) {
+        run += group_sizes[g];
+        ends[g] = run;
+      }
+    }
+    __syncthreads();
+    f = factor + (size_t)local_group_of(ends, G_total, m, group_offset, G_local) * N;
+  } else {
+    row_f = round_bf16_fn(factor[m]);
+  }
+  const int nvec = N / 8;
+  float v[kBwdMaxChunks][8];
+  uint32_t amax_bits = 0u;  // max of the bit patterns of |d|: orders like the values, and a NaN's pattern beats every number's
+#pragma unroll
+  for (int c = 0; c < kBwdMaxChunks; c++) {
+    const int i = c * kBwdThreads + tid;
+    if (i < nvec) {
+      const uint4 x = dout[(size_t)m * nvec + i];
+      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float xe = bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu);
+        const float fe = BY_CHANNEL ? round_bf16_fn(f[i * 8 + e]) : row_f;
+        v[c][e] = round_bf16_fn(xe * fe);
+        amax_bits = max(amax_bits, __float_as_uint(fabsf(v[c][e])));
+      }
+    }
+  }
+  float s = 1.0f;
+  if (ROW_QUANT) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, o, kWave));
+    if (tid % kWave == 0) wmax[tid / kWave] = amax_bits;
+    __syncthreads();
+    const float amax = __uint_as_float(max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+    s = e5m2_scale(amax);
+    if (tid == 0) scale_out[m] = s;
+  }
+#pragma unroll
+  for (int c = 0; c < kBwdMaxChunks; c++) {
+    const int i = c * kBwdThreads + tid;
+    if (i < nvec) {
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = ROW_QUANT ? to_e5m2_grid(v[c][e], s) : v[c][e];
+      out[(size_t)m * nvec + i] = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+    }
+  }
+}
+
+// Column maxima of |d|, d = bf16(dout * bf16(lhs_scale[m])): a block walks a band of rows, a lane owns 8 columns; the
+// bands meet in an atomic max on the bit patterns (non-negative floats order like integers; a NaN's pattern is larger
+// than every number's and so survives, as it does in the reference's amax).
+constexpr int kColBand = 64;
+__global__ __launch_bounds__(kBwdThreads) void bwd_col_absmax_kernel(const uint4* dout, int M, int N, const float* lhs_scale, uint32_t* colmax) {
+  const int nvec = N / 8;
+  const int i = blockIdx.x * kBwdThreads + threadIdx.x;
+  if (i >= nvec) return;
+  const int m0 = blockIdx.y * kColBand, m1 = min(m0 + kColBand, M);
+  float mx[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  bool bad[8] = {false, false, false, false, false, false, false, false};
+  for (int m = m0; m < m1; m++) {
+    const uint4 x = dout[(size_t)m * nvec + i];
+    const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+    const float fm = round_bf16_fn(lhs_scale[m]);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float d = fabsf(round_bf16_fn(bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu) * fm));
+      bad[e] = bad[e] || d != d;
+      mx[e] = fmaxf(mx[e], d);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) atomicMax(colmax + i * 8 + e, bad[e] ? 0x7fc00000u : __float_as_uint(mx[e]));
+}
+
+__global__ void bwd_clear_kernel(uint32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// d on the e5m2 grid of its column's scale; `colmax` still holds the maxima
+__global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4* dout, int M, int N, const float* lhs_scale, const float* colmax, uint4* out) {
+  const int nvec = N / 8;
+  const int i = blockIdx.x * kBwdThreads + threadIdx.x;
+  if (i >= nvec) return;
+  const int m0 = blockIdx.y * kColBand, m1 = min(m0 + kColBand, M);
+  float s[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) s[e] = e5m2_scale(colmax[i * 8 + e]);
+  for (int m = m0; m < m1; m++) {
+    const uint4 x = dout[(size_t)m * nvec + i];
+    const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+    const float fm = round_bf16_fn(lhs_scale[m]);
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = to_e5m2_grid(round_bf16_fn(bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu) * fm), s[e]);
+    out[(size_t)m * nvec + i] = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+  }
+}
+
+__global__ void bwd_col_scale_kernel(float* colmax, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) colmax[i] = e5m2_scale(colmax[i]);
+}
+
+}  // namespace moe
+
+using namespace moe;
+
+extern "C" {
+
+int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, const float* factor, const int32_t* group_sizes,
+                       int num_groups_total, int num_groups_local, int group_offset, void* out, float* scale_out, void* stream) {
+  if (!dout || !factor || !out) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: NULL pointer");
+  if (M < 0 || N <= 0) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad sizes");
+  if (mode != MOE_BWD_FOR_DLHS && mode != MOE_BWD_FOR_DRHS) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad mode %d", mode);
+  if (quantize && !scale_out) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: the quantised gradient needs a scale buffer");
+  if (N % 8 != 0 || N > kBwdThreads * kBwdMaxChunks * 8) return fail(MOE_ERR_UNSUPPORTED, "bwd_scale_grad: need N%%8==0 and N<=16384 (N=%d)", N);
+  if (M == 0) return MOE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const uint4* x = (const uint4*)dout;
+  if (mode == MOE_BWD_FOR_DLHS) {
+    if (!group_sizes || num_groups_total <= 0 || num_groups_total > kBwdMaxGroups || num_groups_local <= 0 || group_offset < 0)
+      return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad groups (at most %d)", kBwdMaxGroups);
+    if (quantize)
+      bwd_scale_rows_kernel<true, true><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, (uint4*)out, scale_out);
+    else
+      bwd_scale_rows_kernel<true, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, (uint4*)out, scale_out);
+    return check_launch("bwd_scale_rows_kernel");
+  }
+  if (!quantize) {
+    bwd_scale_rows_kernel<false, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, nullptr, 0, 0, 0, (uint4*)out, scale_out);
+    return check_launch("bwd_scale_rows_kernel");
+  }
+  // per column: clear the maxima, take them, quantise with them, turn them into the scales
+  const int nvec = N / 8;
+  const dim3 grid(cdiv(nvec, kBwdThreads), cdiv(M, kColBand));
+  if (grid.y > 65535) return fail(MOE_ERR_UNSUPPORTED, "bwd_scale_grad: too many rows (%d)", M);
+  bwd_clear_kernel<<<cdiv(N, 256), 256, 0, s>>>((uint32_t*)scale_out, N);
+  bwd_col_absmax_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, (uint32_t*)scale_out);
+  bwd_col_quant_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, (uint4*)out);
+  bwd_col_scale_kernel<<<cdiv(N, 256), 256, 0, s>>>(scale_out, N);
+  return check_launch("bwd_col_quant_kernel");
+}
+
+}  // extern "C"

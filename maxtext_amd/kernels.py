@@ -246,6 +246,36 @@ def glu_act_bwd(h0, h1, dout, act="silu", act_limit=7.0):
   return dh0, dh1
 
 
+def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups_local=None, group_offset=0):
+  """Gradient preparation of the quantised backward (ops.py:530-604): `dout` [m, n] bf16 times the scale of the axis the
+  gradient product contracts away, optionally quantised to float8_e5m2.
+
+  mode "dlhs": factor = rhs scales [g_local, n] f32, picked per row by its expert (group_sizes); quantised per row.
+  mode "drhs": factor = lhs scales [m] f32; quantised per column.
+  -> (d [m, n] bf16, scale): the e5m2 values (exact in bf16) and their f32 scales ([m] or [n]), or (dout * factor, None).
+  """
+  _need(dout, "dout", torch.bfloat16, 2)
+  _need(factor, "factor", torch.float32)
+  m, n = dout.shape
+  code = {"dlhs": 0, "drhs": 1}[mode]
+  if code == 0:
+    _need(group_sizes, "group_sizes", torch.int32, 1)
+    g_local = int(num_groups_local if num_groups_local is not None else factor.shape[0])
+    if factor.numel() != g_local * n:
+      raise ValueError(f"factor must hold [{g_local}, {n}] scales, got {tuple(factor.shape)}")
+    g_total = group_sizes.numel()
+  else:
+    if factor.numel() != m:
+      raise ValueError(f"factor must hold one scale per row ({m}), got {tuple(factor.shape)}")
+    g_total, g_local = 0, 0
+  out = torch.empty_like(dout)
+  scale = torch.empty((m if code == 0 else n,), dtype=torch.float32, device=dout.device) if quantize else None
+  st = _lib.load().moe_bwd_scale_grad(_lib.ptr(dout), m, n, code, 1 if quantize else 0, _lib.ptr(factor), _lib.ptr(group_sizes), g_total,
+                                      g_local, int(group_offset), _lib.ptr(out), _lib.ptr(scale), _lib.current_stream())
+  _lib.check(st, "moe_bwd_scale_grad")
+  return out, scale
+
+
 def transpose_rhs(rhs_gkn):
   """[G, K, N] -> [G, N, K] for 1- or 2-byte element types."""
   _need(rhs_gkn, "rhs", None, 3)

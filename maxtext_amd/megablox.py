@@ -331,20 +331,6 @@ def tgmm(
   return out.transpose(1, 2)
 
 
-E5M2_MAX = 57344.0  # largest finite float8_e5m2
-
-
-def _quantize_e5m2(x: torch.Tensor, dim: int):
-  """Symmetric absmax float8_e5m2 along `dim` (the gradient quantiser of ops.py:583-604): returns the values on the
-  e5m2 grid as bf16 (exact) and the f32 scale with `dim` kept."""
-  xf = x.float()
-  # the quotient is taken in f64 and rounded once: the device's f32 division is not correctly rounded, and one ulp of
-  # scale moves values across e5m2 rounding boundaries
-  scale = (xf.abs().amax(dim=dim, keepdim=True).double() / E5M2_MAX).float()
-  q = torch.where(scale == 0, torch.zeros_like(xf), xf / scale).to(torch.float8_e5m2).to(torch.bfloat16)
-  return q, scale
-
-
 class _GmmFn(torch.autograd.Function):
   """Differentiable gmm for bf16 operands (custom VJP of ops.py:137-230 / :438-527).
 
@@ -355,8 +341,9 @@ class _GmmFn(torch.autograd.Function):
   int8 x int8 forward (channelwise scales): the residuals are the quantised operands and the backward is the
   reference's (_bwd_prepare_inputs ops.py:530-580): the scale of the axis that disappears goes onto the gradient,
   dlhs = gmm(dout * rhs_scale[n], rhs_q^T), drhs = tgmm(lhs_q^T, dout * lhs_scale[m]); with bwd_q the two scaled
-  gradients are first quantised to float8_e5m2 per row / per column (_bwd_quantize_gradient ops.py:583-604).  The
-  int8 and e5m2 values are exact in bf16, so both products run on the bf16 MFMA kernels.
+  gradients are first quantised to float8_e5m2 per row / per column (_bwd_quantize_gradient ops.py:583-604); scaling
+  and quantisation are one kernel each (kernels.bwd_scale_grad).  The int8 and e5m2 values are exact in bf16, so both
+  products run on the bf16 MFMA kernels (int8 is not an operand type of the fp8 MFMA instructions).
   """
 
   @staticmethod
@@ -383,26 +370,19 @@ class _GmmFn(torch.autograd.Function):
     m, n = dout.shape
     g_local = rq.shape[0]
     dlhs = drhs = None
+    quant = ctx.bwd_q is not None
     if ctx.needs_input_grad[0]:
-      # expert of every row (rows past the last group take the last expert; their gradient rows are zero anyway)
-      ends = torch.cumsum(group_sizes, 0)
-      row_group = torch.searchsorted(ends, torch.arange(m, device=dout.device, dtype=ends.dtype), right=True)
-      local = (row_group - ctx.offset).clamp_(0, g_local - 1)
-      d = dout * rs.to(dout.dtype)[local]
-      s_row = None
-      if ctx.bwd_q is not None:
-        d, s_row = _quantize_e5m2(d, dim=1)
+      # dout times the weights' channel scales of each row's expert, e5m2 per row (one kernel); the row scales go back on
+      # in the product's epilogue (rounded bf16 result times scale, rounded again: what the reference's two steps give)
+      d, s_row = kernels.bwd_scale_grad(dout, rs, mode="dlhs", quantize=quant, group_sizes=group_sizes, num_groups_local=g_local,
+                                        group_offset=ctx.offset)
       w_t = kernels.transpose_rhs(rq)  # [g, n, k] -> [g, k, n]: the layout with k as the output axis
       ones = torch.ones((g_local, w_t.shape[1]), dtype=torch.float32, device=dout.device)
-      dlhs = kernels.gmm_raw(d.contiguous(), w_t, group_sizes, rhs_scale=ones, rhs_scale_block_n=1, group_offset=ctx.offset)
-      if s_row is not None:
-        dlhs = (dlhs.float() * s_row).to(torch.bfloat16)
+      dlhs = kernels.gmm_raw(d, w_t, group_sizes, rhs_scale=ones, rhs_scale_block_n=1, group_offset=ctx.offset, out_row_scale=s_row)
     if ctx.needs_input_grad[1]:
-      d = dout * ls.to(dout.dtype)[:, None]
-      s_col = None
-      if ctx.bwd_q is not None:
-        d, s_col = _quantize_e5m2(d, dim=0)
-      w = kernels.tgmm(lq.to(torch.bfloat16), d.contiguous(), group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
+      # dout times the activations' row scales, e5m2 per column
+      d, s_col = kernels.bwd_scale_grad(dout, ls, mode="drhs", quantize=quant)
+      w = kernels.tgmm(lq.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
                        out_dtype=torch.float32)  # [g, n, k]
       if s_col is not None:
         w = w * s_col.reshape(1, n, 1)

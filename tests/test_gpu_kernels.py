@@ -1350,6 +1350,40 @@ def test_gmm_quantized_backward(transpose_rhs, bwd_q):
     megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, bwd_quantize_dtype="float8_e5m2")
 
 
+@pytest.mark.parametrize("quantize", [False, True])
+@pytest.mark.parametrize("n", [192, 2056])
+def test_bwd_scale_grad_bit_exact(K, n, quantize):
+  """The gradient preparation of the quantised backward (ops.py:530-604) against the oracle's e5m2 quantiser on the
+  same scaled gradient: per row with the weights' channel scales of each row's expert (an empty group, rows past the
+  last group, a group offset), per column with the activations' row scales; values and scales bit for bit."""
+  g = torch.Generator().manual_seed(31)
+  m = 333
+  gs = np.array([40, 100, 0, 70, 93], np.int32)  # 30 trailing rows in no group
+  offset, g_local = 1, 3
+  dout = (torch.randn(m, n, generator=g) * torch.rand(m, 1, generator=g) * 8).to(torch.bfloat16)
+  dout[5, 7] = 0.0
+  dout[17] = 0.0  # a zero row: scale 0, values 0
+  dout[:, 11] = 0.0  # a zero column
+  rs = torch.rand(g_local, n, generator=g) * 0.02 + 1e-4
+  ls = torch.rand(m, generator=g) * 0.05 + 1e-4
+  ends = np.cumsum(gs)
+  local = np.clip(np.searchsorted(ends, np.arange(m), side="right") - offset, 0, g_local - 1)
+  d_rows = dout * rs.to(torch.bfloat16)[torch.from_numpy(local)]
+  d_cols = dout * ls.to(torch.bfloat16)[:, None]
+  got_r, s_r = K.bwd_scale_grad(cuda(dout), cuda(rs), mode="dlhs", quantize=quantize, group_sizes=cuda(gs), num_groups_local=g_local,
+                                group_offset=offset)
+  got_c, s_c = K.bwd_scale_grad(cuda(dout), cuda(ls), mode="drhs", quantize=quantize)
+  if not quantize:
+    assert s_r is None and s_c is None
+    assert torch.equal(got_r.cpu(), d_rows) and torch.equal(got_c.cpu(), d_cols)
+    return
+  want_r, want_sr = O.quantize_e5m2(d_rows, dim=1)
+  want_c, want_sc = O.quantize_e5m2(d_cols, dim=0)
+  assert torch.equal(s_r.cpu(), want_sr[:, 0]) and torch.equal(s_c.cpu(), want_sc[0])
+  assert torch.equal(got_r.cpu().float(), want_r) and torch.equal(got_c.cpu().float(), want_c)
+  assert float(s_r[17]) == 0.0 and torch.all(got_r[17] == 0) and float(s_c[11]) == 0.0
+
+
 def test_gmm_autograd_with_expert_bias():
   """Per-expert mlp_bias on the differentiable path (moe.py:1952-1957): forward equals the epilogue bias of the
   inference path; gradients of lhs, both weights and both biases against torch autograd in f64."""
