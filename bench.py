@@ -103,9 +103,11 @@ def dominant_kernel_model(wl, group_sizes):
   nonempty = int((group_sizes > 0).sum())
   flops = 4.0 * rows * d * f
   if wl.weight_quant == "fp8" and rows > 14 * len(group_sizes):
-    # many rows per expert (prefill): the LDS-tiled kernel, bound by the fp8 MFMA rate
+    # many rows per expert (prefill): the LDS kernels, bound by the fp8 MFMA rate (the persistent 256 x 256 stream from
+    # 128 rows per expert on, the dispatch rule of moe_gmm; 128 x 128 tiles below)
+    kernel = "gmm_f8s_kernel" if rows >= 128 * len(group_sizes) and d % 512 == 0 else "gmm_fp8_tiled_kernel"
     return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS["fp8"], scale=1e12,
-                name="gmm_fp8_tiled_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")
+                name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
   if wl.weight_quant == "fp8":
     # HBM bound (decode): weights of the non-empty experts + block scales + activations in + out
     w_bytes = nonempty * 2.0 * d * f
