@@ -228,6 +228,8 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   };
   // widened weight fragments: the set of the current k-step and the one being built for the next
   v4i gb[2][C::TN];
+  // int4: the fragment's low and high nibbles as bytes (values 0, 2, 4, 6 and 1, 3, 5, 7), taken apart once per fragment
+  uint32_t nib_lo[C::TN], nib_hi[C::TN];
   // piece pc (0 .. 3) of fragment j: two of its eight values -> one register of gb[set][j]
   auto widen_piece = [&](int set, int j, int pc, float sc) {
     uint32_t o;
@@ -242,8 +244,14 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
           : pc == 2 ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(braw[j], sc, 2))
                     : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(braw[j], sc, 3));
     } else {  // int4: (nibble - 8) * scale rounded to bf16, as the reference dequantises
-      const uint32_t b = (braw[j] >> (8 * pc)) & 0xffu;
-      o = pack_bf16x2((float)((int)(b & 0xf) - 8) * sc, (float)((int)(b >> 4) - 8) * sc);
+      // byte -> float is one instruction per value, and nibble * scale - 8 * scale is exact in f32 (12 significant bits),
+      // so the fused multiply-add gives (nibble - 8) * scale bit for bit
+      if (pc == 0) {
+        nib_lo[j] = braw[j] & 0x0f0f0f0fu;
+        nib_hi[j] = (braw[j] >> 4) & 0x0f0f0f0fu;
+      }
+      const float c8 = -8.0f * sc;
+      o = pack_bf16x2(fmaf((float)((nib_lo[j] >> (8 * pc)) & 0xffu), sc, c8), fmaf((float)((nib_hi[j] >> (8 * pc)) & 0xffu), sc, c8));
     }
     gb[set][j][pc] = (int)o;
   };
