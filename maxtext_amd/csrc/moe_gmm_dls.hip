@@ -293,6 +293,7 @@ static int launch_dls_cfg(const TiledParams& p0, int M, int G_total, hipStream_t
   p.tiles_n = cdiv(p.N, C::OUT_BN);
   const long long tiles = (long long)p.max_m_tiles * p.tiles_n;
   if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  if (p.tune <= 0) p.tune = default_super_row(M, G_total, C::BM);
   // one persistent block per CU (the LDS footprint allows no more); a multiple of 8 keeps "tile id mod 8"
   // equal to the XCD a block runs on
   int num_cus = 0;

@@ -405,6 +405,7 @@ static int launch_dlw_cfg(const TiledParams& p0, int M, int G_total, hipStream_t
   p.tiles_n = cdiv(p.N, C::OUT_BN);
   const long long tiles = (long long)p.max_m_tiles * p.tiles_n;
   if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
+  if (p.tune <= 0) p.tune = default_super_row(M, G_total, C::BM);
   int num_cus = 0;
   if (int st = device_cu_count(&num_cus)) return st;
   long long blocks = tiles < num_cus ? tiles : num_cus;
