@@ -1454,3 +1454,45 @@ def test_gmm_direct_to_lds_pipelines_bf16(K, m, k, n):
   assert relerr(got, want) <= TOL and torch.all(got[4096:] == 0)
   got = K.gmm_raw(cuda(lhs), cuda(native(wb)), cuda(gs))
   assert relerr(got, O.gmm(lhs, wb, gs, acc_dtype=torch.float32)) <= TOL
+
+
+# ---------------------------------------------------------------- degenerate sizes
+
+
+def test_gmm_degenerate_group_sizes(K):
+  """All groups empty (every row is written as zero), a single row, group sizes that overrun the rows (clipped to m as
+  reference_gmm does, tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:139-141), the smallest K and N the kernels take."""
+  g = torch.Generator().manual_seed(41)
+  lhs = torch.randn(37, 64, generator=g).to(torch.bfloat16)
+  w = (torch.randn(3, 24, 64, generator=g) * 0.1).to(torch.bfloat16)  # [g, n, k]
+  out = K.gmm_raw(cuda(lhs), cuda(w), cuda(np.array([0, 0, 0], np.int32)))
+  assert out.shape == (37, 24) and torch.all(out == 0)
+  one = K.gmm_raw(cuda(lhs[:1]), cuda(w), cuda(np.array([0, 1, 0], np.int32)))
+  assert relerr(one, lhs[:1].float() @ w[1].float().T) <= TOL
+  over = K.gmm_raw(cuda(lhs), cuda(w), cuda(np.array([20, 30, 50], np.int32)))  # 100 rows announced, 37 exist
+  want = torch.cat([lhs[:20].float() @ w[0].float().T, lhs[20:].float() @ w[1].float().T])
+  assert relerr(over, want) <= TOL
+  tiny = K.gmm_raw(cuda(lhs[:, :16].contiguous()), cuda(w[:, :8, :16].contiguous()), cuda(np.array([10, 20, 7], np.int32)))
+  gs = [10, 20, 7]
+  off = np.concatenate([[0], np.cumsum(gs)])
+  want = torch.cat([lhs[off[i]:off[i + 1], :16].float() @ w[i, :8, :16].float().T for i in range(3)])
+  assert relerr(tiny, want) <= TOL
+
+
+def test_route_sort_combine_single_token(K):
+  """One token: routing, sort, gather and combine on the smallest input (k of E selections, all in different groups)."""
+  g = torch.Generator().manual_seed(42)
+  logits = torch.randn(1, 8, generator=g)
+  w, idx = K.route_topk(cuda(logits), k=2)
+  want_w, want_idx = O.get_topk(logits, k=2)
+  assert torch.equal(idx.cpu(), torch.from_numpy(np.asarray(want_idx)).to(torch.int32))
+  assert torch.equal(w.cpu(), torch.from_numpy(np.asarray(want_w, np.float32)))
+  perm, inv, gs, _ = K.sort_by_expert(idx, 8)
+  assert int(gs.sum()) == 2 and sorted(perm.cpu().tolist()) == [0, 1]
+  x = torch.randn(1, 32, generator=g).to(torch.bfloat16)
+  rows = K.gather_rows(cuda(x), perm, 2)
+  rows = rows[0] if isinstance(rows, tuple) else rows
+  assert torch.equal(rows.cpu(), x.expand(2, 32))
+  y = K.unpermute_combine(rows, w, k=2, perm=perm, inv_perm=inv)
+  want = (x.float() * float(w.sum())).to(torch.bfloat16)
+  assert relerr(y, want) <= TOL
