@@ -335,6 +335,65 @@ __device__ __forceinline__ void dma16_buffer(const v4i& rsrc, uint32_t voff, uin
   asm volatile("" : "+s"(soff));  // (a literal offset is not an operand the instruction takes)
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
 }
+// ---- the tile cursor of the persistent stream kernels -------------------------------------------------------------
+// tile id -> (m-tile, n-tile): ids congruent mod 8 run on one XCD (persistent blocks are dealt round-robin to the XCDs
+// and a block's ids advance by the grid size, a multiple of 8); each XCD owns a contiguous range of the order, which
+// runs in super-rows of p.tune m-tiles with the m-tile index fastest, so that the 32 blocks of an XCD work on a patch
+// of a super-row's m-tiles x a few n-tiles that shares activation and weight panels in that XCD's L2.
+struct StreamTile {
+  TileInfo info;
+  int n0, id;
+};
+struct TilePeek {  // a tile record that has been requested but not looked at yet
+  TileInfo ti;
+  int n0, id;
+  bool valid;
+};
+// The block's first id >= id0 that names an existing m-tile; its record is requested, not waited for.
+template <int OUT_BN>
+__device__ __forceinline__ TilePeek peek_tile(const TiledParams& p, int num_tiles, int id0) {
+  const int total = p.max_m_tiles * p.tiles_n;
+  TilePeek pk;
+  pk.valid = false;
+  pk.n0 = 0;
+  pk.id = total;
+  pk.ti = TileInfo{-1, 0, 0, 0};
+  const int q = total / 8, rem = total % 8;
+  const int GSM = p.tune > 0 ? p.tune : 8;
+  const int width = GSM * p.tiles_n;
+  for (int id = id0; id < total; id += gridDim.x) {
+    const int xcd = id % 8, loc = id / 8;
+    const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
+    const int sg = logical / width, first_m = sg * GSM;
+    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int m_idx = first_m + (logical % width) % gsz;
+    if (m_idx >= num_tiles) continue;
+    pk.ti = p.tiles[m_idx];
+    pk.n0 = ((logical % width) / gsz) * OUT_BN;
+    pk.id = id;
+    pk.valid = true;
+    break;
+  }
+  return pk;
+}
+// Turns a requested record into the block's next tile that needs the matmul (its fields uniform, in scalar registers);
+// tiles of rows that belong to no local group are written as zeros on the way, and the search goes on from there.
+template <int OUT_BN, int THREADS>
+__device__ __forceinline__ bool resolve_tile(const TiledParams& p, int num_tiles, TilePeek pk, StreamTile& t, int tid) {
+  while (pk.valid) {
+    t.info.group = __builtin_amdgcn_readfirstlane(pk.ti.group);
+    t.info.row0 = __builtin_amdgcn_readfirstlane(pk.ti.row0);
+    t.info.nrows = __builtin_amdgcn_readfirstlane(pk.ti.nrows);
+    t.info.pad = 0;
+    t.n0 = __builtin_amdgcn_readfirstlane(pk.n0);
+    t.id = __builtin_amdgcn_readfirstlane(pk.id);
+    if (t.info.group >= 0) return true;
+    zero_fill_tile(p.out, p.ro, t.info.row0, t.info.nrows, t.n0, OUT_BN, p.N, tid, THREADS);
+    pk = peek_tile<OUT_BN>(p, num_tiles, t.id + gridDim.x);
+  }
+  return false;
+}
+
 struct SkinnyParams {
   const uint8_t* lhs;      // [M, K] fp8
   const float* lhs_scale;  // [M, K/128]

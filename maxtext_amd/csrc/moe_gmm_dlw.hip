@@ -59,62 +59,13 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   const uint32_t row_bytes = (uint32_t)K * 2;
   const uint32_t w_row_bytes = C::NIBBLES ? (uint32_t)K / 2 : (uint32_t)K;
   const int num_tiles = p.header[0];
-  const int total = p.max_m_tiles * p.tiles_n;
   const int nk = K / C::BK;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
 
-  struct Tile {
-    TileInfo info;
-    int n0, id;
-  };
-  struct Peek {  // a tile record that has been requested but not looked at yet
-    TileInfo ti;
-    int n0, id;
-    bool valid;
-  };
-  // tile id -> (m-tile, n-tile): ids congruent mod 8 run on one XCD and form an 8 x 4 patch that shares panels in its L2.
-  // The block's first id >= id0 that names an existing m-tile; its record is requested, not waited for.
-  auto peek_from = [&](int id0) -> Peek {
-    Peek pk;
-    pk.valid = false;
-    pk.n0 = 0;
-    pk.id = total;
-    pk.ti = TileInfo{-1, 0, 0, 0};
-    const int q = total / 8, rem = total % 8;
-    const int GSM = p.tune > 0 ? p.tune : 8;
-    const int width = GSM * p.tiles_n;
-    for (int id = id0; id < total; id += gridDim.x) {
-      const int xcd = id % 8, loc = id / 8;
-      const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
-      const int sg = logical / width, first_m = sg * GSM;
-      const int gsz = min(p.max_m_tiles - first_m, GSM);
-      const int m_idx = first_m + (logical % width) % gsz;
-      if (m_idx >= num_tiles) continue;
-      pk.ti = p.tiles[m_idx];
-      pk.n0 = ((logical % width) / gsz) * C::OUT_BN;
-      pk.id = id;
-      pk.valid = true;
-      break;
-    }
-    return pk;
-  };
-  // Turns a requested record into the block's next tile that needs the matmul; tiles of rows that belong to no local
-  // group are written as zeros on the way (and the search goes on from there).
-  auto resolve = [&](Peek pk, Tile& t) -> bool {
-    while (pk.valid) {
-      // (uniform values: kept in scalar registers)
-      t.info.group = __builtin_amdgcn_readfirstlane(pk.ti.group);
-      t.info.row0 = __builtin_amdgcn_readfirstlane(pk.ti.row0);
-      t.info.nrows = __builtin_amdgcn_readfirstlane(pk.ti.nrows);
-      t.info.pad = 0;
-      t.n0 = __builtin_amdgcn_readfirstlane(pk.n0);
-      t.id = __builtin_amdgcn_readfirstlane(pk.id);
-      if (t.info.group >= 0) return true;
-      zero_fill_tile(p.out, p.ro, t.info.row0, t.info.nrows, t.n0, C::OUT_BN, N, tid, C::THREADS);
-      pk = peek_from(t.id + gridDim.x);
-    }
-    return false;
-  };
+  using Tile = StreamTile;
+  using Peek = TilePeek;
+  auto peek_from = [&](int id0) { return peek_tile<C::OUT_BN>(p, num_tiles, id0); };
+  auto resolve = [&](Peek pk, Tile& t) { return resolve_tile<C::OUT_BN, C::THREADS>(p, num_tiles, pk, t, tid); };
 
   // ---- the loading side of the stream ---------------------------------------------------------------------------
   // activations: request i of this wave covers rows (wave * A_IPW + i) * 8 .. + 7 of the tile, 128 bytes of each
