@@ -685,7 +685,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint4* __restrict__ 
   }
   __syncthreads();
   const int nch = d / 8;
-  for (int ci = threadIdx.x; ci < nch; ci += blockDim.x) {
+  // (few tokens: gridDim.y blocks share a token's row, so that a decode-sized call still fills the chip)
+  for (int ci = blockIdx.y * blockDim.x + threadIdx.x; ci < nch; ci += blockDim.x * gridDim.y) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < k; s++) {
       if (s_row[s] < 0) continue;
@@ -1040,7 +1041,8 @@ int moe_unpermute_combine(const void* y, const int32_t* perm, const int32_t* inv
     invert_perm_kernel<<<cdiv(M, 256), 256, 0, s>>>(perm, M, (int32_t*)workspace);
     inv_perm = (const int32_t*)workspace;
   }
-  combine_kernel<<<T, 256, 0, s>>>((const uint4*)y, inv_perm, weights, valid_rows_mask, k, d, (uint4*)out);
+  const int splits = T < 2048 ? std::min(cdiv(d / 8, 256), 8) : 1;
+  combine_kernel<<<dim3(T, splits), 256, 0, s>>>((const uint4*)y, inv_perm, weights, valid_rows_mask, k, d, (uint4*)out);
   return check_launch("combine_kernel");
 }
 
