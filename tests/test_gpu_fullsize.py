@@ -140,12 +140,14 @@ def test_fullsize_int_weight_layers(name):
     assert float((out[tok].float().cpu() - want.float()).abs().max()) <= 2.0**-7 * float(want.float().abs().max()) + 1e-6
 
 
-def test_fullsize_deepseek_fp8_decode():
-  """C3 at full size: 256 routed experts + shared expert resident, fp8 128x128 weights."""
+@pytest.mark.parametrize("tokens", [None, 4096])
+def test_fullsize_deepseek_fp8(tokens):
+  """C3 at full size: 256 routed experts + shared expert resident, fp8 128x128 weights; at its own 256 tokens (9 rows per
+  expert: the streaming kernel) and at 4096 tokens (143 rows per expert: the persistent 256 x 256 stream kernel)."""
   from maxtext_amd import kernels, megablox, synthetic
   from maxtext_amd.quantizations import QArray
 
-  wl = synthetic.workload("c3")
+  wl = synthetic.workload("c3", tokens)
   cfg = wl.cfg
   L = synthetic.make_layer(wl, device="cuda")
   r, w, idx, oidx = _routing(wl, L)
