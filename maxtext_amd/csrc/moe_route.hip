@@ -417,15 +417,18 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
   }
 }
 
-// All three passes in one block for at most kSortChunk entries (decode: a launch costs as much as a pass): per-wave
-// histograms in LDS, the prefixes over the four segments and over the experts, then the same in-order ranking.
-__global__ __launch_bounds__(kSortWaves* kWave) void sort_small_kernel(
+// All three passes in one block of NW waves for at most NW * kSortSeg entries (decode and small prefill: a launch costs
+// as much as a pass; NW = 4 up to 1024 entries, 16 up to 4096): per-wave histograms in LDS, the prefixes over the
+// segments and over the experts, then the same in-order ranking.
+template <int NW>
+__global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
     const int32_t* __restrict__ flat, int M, int E, int ebits, int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts) {
-  __shared__ int run[kSortWaves][kSortMaxE];
+  __shared__ int run[NW][kSortMaxE];
   __shared__ int off[kSortMaxE];
+  constexpr int NT = NW * kWave;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  for (int e = threadIdx.x; e < kSortWaves * kSortMaxE; e += kSortWaves * kWave) run[e / kSortMaxE][e % kSortMaxE] = 0;
+  for (int e = threadIdx.x; e < NW * kSortMaxE; e += NT) run[e / kSortMaxE][e % kSortMaxE] = 0;
   __syncthreads();
   const int base = wave * kSortSeg;
 #pragma unroll
@@ -435,10 +438,10 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_small_kernel(
   }
   __syncthreads();
   // counts of the segments -> exclusive prefixes over the segments; the expert's total goes to group_sizes and to off
-  for (int e = threadIdx.x; e < kSortMaxE; e += kSortWaves * kWave) {
+  for (int e = threadIdx.x; e < kSortMaxE; e += NT) {
     int running = 0;
 #pragma unroll
-    for (int w = 0; w < kSortWaves; w++) {
+    for (int w = 0; w < NW; w++) {
       const int c = run[w][e];
       run[w][e] = running;
       running += c;
@@ -448,15 +451,17 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_small_kernel(
   }
   __syncthreads();
   for (int o = 1; o < kSortMaxE; o <<= 1) {  // inclusive scan of the totals
-    int add[kSortMaxE / (kSortWaves * kWave)];
+    constexpr int Q = (kSortMaxE + NT - 1) / NT;
+    int add[Q];
 #pragma unroll
-    for (int q = 0; q < kSortMaxE / (kSortWaves * kWave); q++) {
-      const int e = threadIdx.x + q * kSortWaves * kWave;
-      add[q] = e >= o ? off[e - o] : 0;
+    for (int q = 0; q < Q; q++) {
+      const int e = threadIdx.x + q * NT;
+      add[q] = e >= o && e < kSortMaxE ? off[e - o] : 0;
     }
     __syncthreads();
 #pragma unroll
-    for (int q = 0; q < kSortMaxE / (kSortWaves * kWave); q++) off[threadIdx.x + q * kSortWaves * kWave] += add[q];
+    for (int q = 0; q < Q; q++)
+      if (threadIdx.x + q * NT < kSortMaxE) off[threadIdx.x + q * NT] += add[q];
     __syncthreads();
   }
   for (int e = lane; e < E; e += kWave) run[wave][e] += e > 0 ? off[e - 1] : 0;
@@ -982,7 +987,11 @@ int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* pe
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
   if (nblk <= 1) {  // also M == 0: group_sizes are all zero
-    sort_small_kernel<<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    return check_launch("sort_by_expert");
+  }
+  if (nblk <= 4) {  // up to 4096 entries: still one launch, with 16 waves
+    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, group_sizes, perm, inv_perm, sorted_experts);
     return check_launch("sort_by_expert");
   }
   if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, seg_hist);
