@@ -78,7 +78,7 @@ def parse():
   ap.add_argument("--steps", type=int, default=20)
   ap.add_argument("--warmup", type=int, default=5)
   ap.add_argument("--workload", default=None, choices=["c1", "c2", "c3", "c4", "c5", "c5mx"],
-                  help="one workload; by default c2 (the headline line) and then c3 (reported under \"secondary\")")
+                  help="one workload; by default c2 (the headline line), then c3 (reported under \"secondary\") and c1, c4, c5 (\"other_configs\")")
   ap.add_argument("--source-hash", action="store_true", help="print the kernel source hash that a profile summary of --workload records")
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
   ap.add_argument("--cpu-sample-tokens", type=int, default=None)
@@ -515,6 +515,17 @@ def main():
         "ms_per_step": sec["ms_per_step"], "steps": args.steps, "warmup": args.warmup, "dtype": sec["dtype"],
         "config": sec["config"], "roofline": sec["roofline"], "stage_ms": sec["stage_ms"], "layer_gbps": sec["layer_gbps"],
     }
+    # the remaining configurations of the baseline (parity-test cases, not the headline), each timed the same way so
+    # that one run records all five
+    result["other_configs"] = []
+    for name in ("c1", "c4", "c5"):
+      torch.cuda.empty_cache()
+      o, _, olayer, _, _ = run_workload(args, name)
+      del olayer
+      result["other_configs"].append({
+          "workload": o["config"]["workload"], "value": o["value"], "unit": o["unit"], "ms_per_step": o["ms_per_step"], "dtype": o["dtype"],
+          "config": o["config"], "roofline": o["roofline"], "stage_ms": o["stage_ms"], "layer_gbps": o["layer_gbps"],
+      })
   print(json.dumps(result))
 
 
