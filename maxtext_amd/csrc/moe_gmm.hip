@@ -9,8 +9,13 @@
 //                     weights run on v_mfma_f32_32x32x16_bf16 (weights are widened to bf16 while
 //                     they are copied into LDS), int8 x int8 on v_mfma_i32_32x32x32_i8.
 //                     Used for weight-only formats, small problems and K tails.
-//   gmm_dl_kernel     the prefill kernel for int8 x int8 and bf16 x bf16: persistent blocks, operands
-//                     copied global -> LDS without passing through registers, 4 stages in flight.
+//   gmm_dls_kernel    the prefill kernel for int8 x int8 and bf16 x bf16 (moe_gmm_dls.hip): persistent blocks, 256 x 256
+//                     tiles, operands copied global -> LDS without passing through registers, the requests of a block's
+//                     consecutive tiles as one stream.  gmm_dl_kernel (moe_gmm_dl.hip) is its predecessor, kept for the
+//                     shapes the stream kernel does not take and for [G, K, N] weights.
+//   gmm_dlw_kernel    the same stream for bf16 activations x int8 / int4 / mxfp4 weights (moe_gmm_dlw.hip): raw weight
+//                     bytes through LDS, widened by the wave that multiplies them.
+//   gmm_f8s_kernel    the same stream for block-scaled fp8 (moe_gmm_f8s.hip): scales staged through LDS.
 //   gmm_fp8_skinny_kernel  block-scaled fp8 for few rows per expert (decode): no LDS, every wave
 //                     streams 16 weight rows through v_mfma_f32_16x16x128_f8f6f4 and applies the
 //                     per-128 K-block scales to the f32 partial sums.
