@@ -352,7 +352,10 @@ struct TilePeek {  // a tile record that has been requested but not looked at ye
 // The block's first id >= id0 that names an existing m-tile; its record is requested, not waited for.
 template <int OUT_BN>
 __device__ __forceinline__ TilePeek peek_tile(const TiledParams& p, int num_tiles, int id0) {
-  const int total = p.max_m_tiles * p.tiles_n;
+  // the order covers the tiles that exist (the count the tile map left on the device), not the host's upper bound: with
+  // the bound, the ids of tiles that do not exist all fall into the last XCD's range and leave its blocks idle while the
+  // other seven work through full ranges (GPT-OSS at 4096 tokens: 97 slots for 80 m-tiles, 8.7 rounds instead of 7.2)
+  const int total = num_tiles * p.tiles_n;
   TilePeek pk;
   pk.valid = false;
   pk.n0 = 0;
@@ -365,9 +368,8 @@ __device__ __forceinline__ TilePeek peek_tile(const TiledParams& p, int num_tile
     const int xcd = id % 8, loc = id / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
     const int sg = logical / width, first_m = sg * GSM;
-    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int gsz = min(num_tiles - first_m, GSM);
     const int m_idx = first_m + (logical % width) % gsz;
-    if (m_idx >= num_tiles) continue;
     pk.ti = p.tiles[m_idx];
     pk.n0 = ((logical % width) / gsz) * OUT_BN;
     pk.id = id;

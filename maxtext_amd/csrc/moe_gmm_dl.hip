@@ -59,7 +59,7 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
   const int N = p.N, K = p.K;
   const size_t row_bytes = (size_t)K * C::ESZ;
   const int num_tiles = p.header[0];
-  const int total = p.max_m_tiles * p.tiles_n;
+  const int total = num_tiles * p.tiles_n;  // the tiles that exist, not the host's upper bound (see peek_tile)
 
   // Persistent blocks: block b works on tile ids b, b + gridDim.x, ...  A tile id is turned into (m-tile,
   // n-tile) so that ids that run at the same time on one XCD (ids congruent mod 8 go to the same XCD) form
@@ -74,9 +74,8 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
     const int GSM = p.tune > 0 ? p.tune : 8;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
-    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int gsz = min(num_tiles - first_m, GSM);
     const int m_idx = first_m + (logical % width) % gsz;
-    if (m_idx >= num_tiles) return false;
     // (uniform values: kept in scalar registers, so that a tile looked up ahead of time costs no vector registers)
     const TileInfo ti = p.tiles[m_idx];
     t.info.group = __builtin_amdgcn_readfirstlane(ti.group);

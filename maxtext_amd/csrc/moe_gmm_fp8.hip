@@ -250,21 +250,23 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_tiled_kernel(const Fp8T
 
   // block -> (m-tile, n-tile): ids that run at the same time on one XCD (ids congruent mod 8) form a patch of
   // 4 m-tiles x 8 n-tiles that shares activation and weight panels in that XCD's L2
-  const int total = p.max_m_tiles * p.tiles_n;
+  // (the order covers the tiles that exist, not the host's upper bound: see gmm_tiled_kernel)
+  const int num_tiles = p.header[0];
+  const int total = num_tiles * p.tiles_n;
   TileInfo tile;
   int n0;
   {
     const int id = blockIdx.x;
+    if (id >= total) return;
     const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
     const int GSM = p.tune > 0 ? p.tune : 4;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
-    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int gsz = min(num_tiles - first_m, GSM);
     const int m_idx = first_m + (logical % width) % gsz;
     n0 = ((logical % width) / gsz) * C::OUT_BN;
-    tile = p.tiles[m_idx];  // the slot exists even when the tile does not
-    if (m_idx >= p.header[0]) return;
+    tile = p.tiles[m_idx];
   }
   if (tile.group < 0) {
     zero_fill_tile(p.out, p.ro, tile.row0, tile.nrows, n0, C::OUT_BN, N, tid, C::THREADS);
@@ -492,21 +494,23 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_fp8_big_kernel(const Fp8Til
   const int nkb = K / 128, nst = K / C::BKB;
 
   // block -> (m-tile, n-tile): contiguous ids per XCD, super-rows of GSM m-tiles
-  const int total = p.max_m_tiles * p.tiles_n;
+  // (the order covers the tiles that exist, not the host's upper bound: see gmm_tiled_kernel)
+  const int num_tiles = p.header[0];
+  const int total = num_tiles * p.tiles_n;
   TileInfo tile;
   int n0;
   {
     const int id = blockIdx.x;
+    if (id >= total) return;
     const int q = total / 8, rem = total % 8, xcd = id % 8, loc = id / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
     const int GSM = p.tune > 0 ? p.tune : 4;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
-    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int gsz = min(num_tiles - first_m, GSM);
     const int m_idx = first_m + (logical % width) % gsz;
     n0 = ((logical % width) / gsz) * C::OUT_BN;
     tile = p.tiles[m_idx];
-    if (m_idx >= p.header[0]) return;
   }
   if (tile.group < 0) {
     zero_fill_tile(p.out, p.ro, tile.row0, tile.nrows, n0, C::OUT_BN, N, tid, C::THREADS);

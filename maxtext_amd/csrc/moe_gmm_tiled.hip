@@ -44,22 +44,23 @@ __global__ __launch_bounds__(C::THREADS) void gmm_tiled_kernel(const TiledParams
   const int wm = wave % C::WAVES_M, wn = wave / C::WAVES_M;
 
   // ---- block -> (m-tile, n-tile): contiguous ids per XCD, then GSM x tiles_n super-rows ----
+  // (over the tiles that exist, whose count the tile map left on the device: split over the grid, the host's upper
+  // bound, the ids of tiles that do not exist would all fall to the last XCDs and leave them idle)
+  const int num_tiles = p.header[0];
   int m_idx, n_idx;
   {
-    const int nb = gridDim.x, pid = blockIdx.x;
+    const int nb = num_tiles * p.tiles_n, pid = blockIdx.x;
+    if (pid >= nb) return;
     const int q = nb / 8, rem = nb % 8, xcd = pid % 8, loc = pid / 8;
     const int logical = xcd < rem ? xcd * (q + 1) + loc : rem * (q + 1) + (xcd - rem) * q + loc;
     constexpr int GSM = 4;
     const int width = GSM * p.tiles_n;
     const int sg = logical / width, first_m = sg * GSM;
-    const int gsz = min(p.max_m_tiles - first_m, GSM);
+    const int gsz = min(num_tiles - first_m, GSM);
     m_idx = first_m + (logical % width) % gsz;
     n_idx = (logical % width) / gsz;
   }
-  // the slot exists even when the tile does not (the list is sized for the worst case): both loads go out
-  // together instead of one after the other
   const TileInfo tile = p.tiles[m_idx];
-  if (m_idx >= p.header[0]) return;
   const int n0 = n_idx * C::OUT_BN;
   const int N = p.N, K = p.K;
 
