@@ -155,18 +155,16 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // takes the 64-row tiles, which quadruples its blocks
   const long long tiles_big = (long long)max_tiles_for(M, G_total, 256) * cdiv(N, glu ? 128 : 256);
   const bool big = (long long)M >= 128LL * G_total && tiles_big >= 128;
-  // 32 to 128 rows per expert on average (200 for the weight-only formats, whose big kernel is the register-staged one:
-  // level with the 256-row tiles at 192 rows per expert on the GPT-OSS shape, 12 % ahead at 256 on the skewed Qwen3 one):
-  // 128-row tiles.  Measured against the 64-row tiles on the Mixtral, Qwen3 and GPT-OSS shapes they are 15-35 % faster
-  // from 32 rows per expert on (one weight conversion / tile fetch serves twice the rows), and 256-row tiles would be
-  // half empty; below 32 rows per expert the 64-row tiles stay.
+  // 32 to 128 rows per expert on average: 128-row tiles; below 32, 64-row tiles.  With routed groups of near-equal size
+  // the 64-row tiles are 5-10 % ahead up to 56 rows per expert (GPT-OSS shape, 384 tokens: 0.38 against 0.41 ms for the
+  // layer) and collapse at 64, where half of the groups need a second tile (0.57 against 0.41 ms); with skewed routing
+  // (Qwen3 shape, Zipf 1.2) the 128-row tiles are ahead from 12 rows per expert on (0.18 against 0.21 ms at 40, 0.20
+  // against 0.26 ms at 56).  The weight-only shapes whose direct-to-LDS kernel does not apply follow the same rule:
+  // their 256-row register-staged tiles pass the 128-row ones at 128 rows per expert as well.
   const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
-  // weight-only formats on shapes their direct-to-LDS kernel does not take (K % 64 != 0, K-major scales) stay on the
-  // register-staged kernel, whose 128-row tiles are ahead of its 256-row tiles up to 200 rows per expert
   const bool dlw_ok = bsrc != BSRC_SAME && dlw_takes(K, N, indexed_lhs_rows, wq_kmajor);
-  const bool mid_wq = bsrc != BSRC_SAME && !dlw_ok && (long long)M >= 32LL * G_total && (long long)M < 200LL * G_total;
   const int esz = op == OP_I8 ? 1 : 2;
-  if (mid || mid_wq) return K_T128;
+  if (mid) return K_T128;
   if (big && dlw_ok) return K_DLW;
   // operands that need no conversion stream straight into LDS when every stage is a full row slice
   if (big && bsrc == BSRC_SAME && (K * esz) % 128 == 0) return K_DL128;
@@ -295,9 +293,10 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     // Up to 14 rows per expert on average (decode): the streaming kernel with 16-row tiles, one MFMA row tile per
     // wave; a group with more rows simply gets several tiles, which are adjacent in the grid, run at the same time
     // and share the group's weights through L2.  Beyond that the LDS-tiled kernel with 128 x 128 tiles (measured on
-    // 256 experts of 7168 x 2048: at 12 rows per expert 1.27 against 1.52 ms, at 16, where half of the experts need a
-    // second 16-row tile, 1.66 against 1.54 ms; the 256 x 256 kernel is within 5 % of it from 128
-    // rows per expert on and behind it below, so it is not picked by default).
+    // 256 experts of 7168 x 2048: at 12 rows per expert 1.26 against 1.44 ms, at 16, where half of the experts need a
+    // second 16-row tile, 1.66 against 1.43 ms), and from 128 rows per expert on the persistent 256 x 256 stream (with
+    // groups of exactly 128 rows 1.94 against 1.70 ms, at 160 rows 2.05 against 2.54 ms; routed groups scatter around
+    // their mean, and those over 128 rows cost the 128 x 128 kernel a second tile).
     const bool few_rows = (long long)M <= 16LL * G;
     const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > 14LL * G : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
@@ -437,10 +436,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   }
   const int bsrc = variant == V_BF16 ? BSRC_SAME : variant == V_W8 ? BSRC_I8 : variant == V_W4 ? BSRC_I4 : BSRC_MX4;
   const bool int4_g128 = variant == V_W4 && rbk != 32;
-  // rows per expert up to which the streaming kernel beats the register-staged one (measured on the GPT-OSS and Qwen3
-  // shapes): 56 for group-128 int4, 64 for MXFP4 (0.38 / 0.41 / 0.49 ms at 320 / 384 / 512 tokens against 0.46 / 0.51 /
-  // 0.53 ms), 32 for int8 and group-32 int4
-  const long long stream_rows_hi = int4_g128 ? 56 : variant == V_MX4 ? 64 : 32;
+  // rows per expert up to which the streaming kernel beats the register-staged one (layer times on the GPT-OSS shape with
+  // uniform routing): 36 for group-128 int4 (0.36 / 0.42 ms at 32 / 40 rows against 0.40 / 0.40 ms), 32 for MXFP4 (0.31 /
+  // 0.38 against 0.34 / 0.35 ms).  Int8 and group-32 int4: 16, between the crossover with equal groups (30 on the Qwen3
+  // shape, where both kernels then wait for the weights of all experts) and the one with Zipf-skewed routing (10: few
+  // experts hold most rows and the tiled kernel converts their weights once per 128 rows instead of once per 32).
+  const long long stream_rows_hi = int4_g128 ? 36 : variant == V_MX4 ? 32 : 16;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
   const bool stream_ok = variant != V_BF16 && !wq_kmajor && K % 32 == 0 && (long long)N * K < (1LL << 31);
@@ -451,8 +452,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   if (want_stream && stream_ok) {
     // 16-row tiles up to 16 rows per expert on average, 32-row tiles above; group-128 int4 keeps the 16-row tiles over the
     // whole range (its 32-row variant runs at two waves per SIMD: 0.36 against 0.44 ms on the GPT-OSS shape at 256 tokens)
-    // and stays on this kernel up to 56 rows per expert (0.43 / 0.48 ms at 320 / 384 tokens against 0.52 / 0.58 ms on
-    // the 128-row tiles of the register-staged kernel; level at 512 tokens)
+    // and stays on this kernel up to 36 rows per expert
     const bool one = int4_g128 || (long long)M <= 16LL * G;
     const int bm = one ? 16 : 32;
     map_tiles(bm);
