@@ -134,6 +134,47 @@ MOE_API int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Expert-parallel dispatch bookkeeping on one expert shard (integer work on device-resident sizes; the exchange
+ * itself is a collective and no part of this library).
+ *
+ * moe_local_expert_keys replaces the index half of RoutedMoE.local_permute (moe.py:1091-1200) up to its argsort:
+ *   global_group_sizes     [num_batch_shards, num_experts] i32: rows batch shard s holds for global expert e
+ *   local_expert_size      experts per expert shard; this shard owns experts shard_index * local_expert_size ...
+ *   num_rows               rows of the buffer local_permute is given (inputs.shape[0])
+ *   global_sorted_experts  NULL (is_offset=False): the buffer holds the received rows grouped by (batch shard, local
+ *                          expert), moe.py:1176-1178; key of row r = local expert of its segment, rows past the received
+ *                          total take the last segment's expert (jnp.repeat's total_repeat_length padding).
+ *                          [num_rows] i32 (is_offset=True): the buffer holds every routed row sorted by global expert,
+ *                          moe.py:1166-1172; rows of this shard get e % local_expert_size, all others the key
+ *                          local_expert_size.
+ *   truncate               ragged_buffer_factor > 0: the per-(batch shard, local expert) sizes are cut at num_rows in
+ *                          that order before they are summed (_maybe_truncate_local_group_size, moe.py:1066-1089)
+ *   expert_keys            [num_rows] i32 out: expert_indices of local_permute; sort them with
+ *                          moe_sort_by_expert(expert_keys, T = num_rows, k = 1, E = local_expert_size + 1): perm is
+ *                          sorted_indices, sorted_experts is sorted_experts_ids; moe_gather_rows(inputs, perm) moves the rows
+ *   local_group_size       [local_expert_size] i32 out
+ *   workspace              moe_local_expert_keys_workspace_bytes(num_batch_shards, local_expert_size) bytes
+ * Limits: num_batch_shards * local_expert_size <= 2^24.
+ *
+ * moe_all_to_all_params replaces RoutedMoE.get_all_to_all_params (moe.py:1202-1349): the input offsets, send sizes,
+ * output offsets and receive sizes ([num_expert_parallelism] i32 each) that shard_id hands to ragged_all_to_all.
+ *   all_shards_group_sizes  is_batch_sharded: [P, P] i32, entry (i, j) = rows batch shard i sends to expert shard j;
+ *                           otherwise [P]: rows each expert shard is responsible for (replicated batch)
+ *   buffer_size             >= 0: capacity of a receiver (ragged_buffer_factor > 0): the matrix is cut per receiver in
+ *                           sender order (_truncate_matrix, moe.py:103-120); < 0: no capacity.  Batch-sharded only.
+ *   is_dispatch             1: tokens to experts; 0: the way back (transposed roles, moe.py:1296-1330)
+ * Limits: num_expert_parallelism <= 1024.
+ */
+MOE_API size_t moe_local_expert_keys_workspace_bytes(int num_batch_shards, int local_expert_size);
+MOE_API int moe_local_expert_keys(const int32_t* global_group_sizes, int num_batch_shards, int num_experts,
+                          int local_expert_size, int shard_index, int num_rows, const int32_t* global_sorted_experts,
+                          int truncate, int32_t* expert_keys, int32_t* local_group_size, void* workspace,
+                          size_t workspace_bytes, void* stream);
+MOE_API int moe_all_to_all_params(const int32_t* all_shards_group_sizes, int num_expert_parallelism, int shard_id,
+                          int is_batch_sharded, long long buffer_size, int is_dispatch, int32_t* input_offsets,
+                          int32_t* send_sizes, int32_t* output_offsets, int32_t* recv_sizes, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Row gather with optional quantisation.  Replaces the data half of permute
  * (moe.py:956-959: repeat(x, k)[perm]) fused with the activation quantiser of
  * the grouped GEMM.  Two quantisation rules (moe_quant_rule):

@@ -154,6 +154,43 @@ def gather_rows(x, row_idx=None, idx_div=1, *, out_dtype=torch.bfloat16, block_k
   return out, (static_scale if static_scale is not None else scale)
 
 
+def local_expert_keys(global_group_sizes, local_expert_size, shard_index, num_rows, *, global_sorted_experts=None, truncate=False):
+  """Index half of RoutedMoE.local_permute (moe.py:1091-1200) before its argsort.
+  global_group_sizes [batch shards, E] int32 -> (expert_keys [num_rows] int32, local_group_size [local_expert_size] int32)."""
+  _need(global_group_sizes, "global_group_sizes", torch.int32, 2)
+  s, e = global_group_sizes.shape
+  if global_sorted_experts is not None:
+    _need(global_sorted_experts, "global_sorted_experts", torch.int32, 1)
+    if global_sorted_experts.shape[0] != num_rows:
+      raise ValueError("global_sorted_experts must name the expert of every row")
+  dev = global_group_sizes.device
+  lib = _lib.load()
+  keys = torch.empty((num_rows,), dtype=torch.int32, device=dev)
+  sizes = torch.empty((local_expert_size,), dtype=torch.int32, device=dev)
+  ws = torch.empty((max(lib.moe_local_expert_keys_workspace_bytes(s, local_expert_size), 16),), dtype=torch.uint8, device=dev)
+  st = lib.moe_local_expert_keys(_lib.ptr(global_group_sizes), s, e, int(local_expert_size), int(shard_index), int(num_rows),
+                                 _lib.ptr(global_sorted_experts), int(bool(truncate)), _lib.ptr(keys), _lib.ptr(sizes), _lib.ptr(ws),
+                                 ws.numel(), _lib.current_stream())
+  _lib.check(st, "moe_local_expert_keys")
+  return keys, sizes
+
+
+def all_to_all_params(all_shards_group_sizes, shard_id, num_expert_parallelism, *, is_batch_sharded=True, buffer_size=None,
+                      is_dispatch=True):
+  """RoutedMoE.get_all_to_all_params (moe.py:1202-1349) -> (input_offsets, send_sizes, output_offsets, recv_sizes),
+  int32 [num_expert_parallelism] each, on the device.  buffer_size: a receiver's capacity, or None."""
+  _need(all_shards_group_sizes, "all_shards_group_sizes", torch.int32, 2 if is_batch_sharded else 1)
+  p = int(num_expert_parallelism)
+  if tuple(all_shards_group_sizes.shape) != ((p, p) if is_batch_sharded else (p,)):
+    raise ValueError(f"all_shards_group_sizes has shape {tuple(all_shards_group_sizes.shape)} for {p} shards")
+  out = torch.empty((4, p), dtype=torch.int32, device=all_shards_group_sizes.device)
+  st = _lib.load().moe_all_to_all_params(_lib.ptr(all_shards_group_sizes), p, int(shard_id), int(bool(is_batch_sharded)),
+                                         -1 if buffer_size is None else int(buffer_size), int(bool(is_dispatch)), _lib.ptr(out[0]),
+                                         _lib.ptr(out[1]), _lib.ptr(out[2]), _lib.ptr(out[3]), _lib.current_stream())
+  _lib.check(st, "moe_all_to_all_params")
+  return out[0], out[1], out[2], out[3]
+
+
 def _valid_mask(valid_rows_mask, m):
   if valid_rows_mask is None:
     return None

@@ -288,6 +288,49 @@ class RoutedMoE:
     lb_loss, bias_updates = self._aux_outputs(gate_logits, selected)
     return sorted_inputs, perm, weights, group_size, sorted_experts, lb_loss, bias_updates, None
 
+  # -- expert-parallel dispatch bookkeeping on one shard (moe.py:1066-1401): the exchange itself is a collective ----
+  @staticmethod
+  def local_permute(inputs, global_group_sizes, local_expert_size, shard_index, is_offset=False, global_sorted_experts=None,
+                    use_custom_sort_vjp=True, use_ragged_sort=False, ragged_buffer_factor=-1.0, use_single_sparsecore=False):
+    """-> (sorted_inputs, sorted_indices, local_group_size, sorted_experts_ids), as moe.py:1091-1200.
+    inputs [rows, emb_dim] bf16; global_group_sizes [batch shards, num_experts] int32 on the device.
+    use_ragged_sort moves only the rows that carry tokens (the first sum(local_group_size)); the rest of
+    sorted_inputs is zeros (a2a_ragged_sort leaves it unspecified)."""
+    rows = inputs.shape[0]
+    if is_offset and global_sorted_experts is None:
+      raise ValueError("is_offset=True needs global_sorted_experts")
+    keys, local_group_size = kernels.local_expert_keys(
+        global_group_sizes, local_expert_size, shard_index, rows,
+        global_sorted_experts=global_sorted_experts if is_offset else None, truncate=ragged_buffer_factor > 0.0)
+    sorted_indices, inv, _, sorted_experts_ids = kernels.sort_by_expert(keys.reshape(rows, 1), local_expert_size + 1)
+    row_range = None
+    if use_ragged_sort:
+      row_range = torch.stack([torch.zeros((), dtype=torch.int32, device=inputs.device), local_group_size.sum().to(torch.int32)])
+    if torch.is_grad_enabled() and inputs.requires_grad:
+      if row_range is not None:
+        raise NotImplementedError("gradients through the ragged sort are not implemented")
+      sorted_inputs = _GatherRowsFn.apply(inputs, sorted_indices, inv, 1)
+    else:
+      sorted_inputs = kernels.gather_rows(inputs.contiguous(), sorted_indices, 1, row_range=row_range)
+    return sorted_inputs, sorted_indices, local_group_size, sorted_experts_ids
+
+  @staticmethod
+  def get_all_to_all_params(all_shards_group_sizes, shard_id, num_expert_parallelism, is_batch_sharded=True,
+                            ragged_buffer_factor=-1.0, buffer_size=None, is_dispatch=True):
+    """-> (input_offsets, send_sizes, output_offsets, recv_sizes) for ragged_all_to_all, as moe.py:1202-1349."""
+    if ragged_buffer_factor > 0.0 and buffer_size is None:
+      raise ValueError("ragged_buffer_factor > 0 needs buffer_size")
+    return kernels.all_to_all_params(all_shards_group_sizes, shard_id, num_expert_parallelism, is_batch_sharded=is_batch_sharded,
+                                     buffer_size=buffer_size if ragged_buffer_factor > 0.0 else None, is_dispatch=is_dispatch)
+
+  @staticmethod
+  def get_ragged_buffer_size(local_batch, ep_degree, global_experts, top_k, ragged_buffer_factor):
+    """Rows of the ragged receive buffer (moe.py:1368-1401): the balanced share times the factor (tokens beyond it are
+    dropped), or the worst case: min(ep_degree, global_experts / top_k) times the share."""
+    if ragged_buffer_factor > 0.0:
+      return int(local_batch * ragged_buffer_factor)
+    return int(local_batch * min(ep_degree, global_experts / top_k))
+
   # -- unpermute (moe.py:1004-1063), non-ragged branch --------------------------------------
   def unpermute(self, intermediate, sorted_selected_experts, weights, batch_size, sequence_length,
                 use_custom_sort_vjp=True, group_sizes=None, inv_perm=None):

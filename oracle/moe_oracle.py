@@ -47,6 +47,16 @@ How each function is pinned (see tests/test_oracle_*.py):
       x * (1 / scale) from x / scale, and bf16 from f32 intermediate arithmetic; the closed forms
       q * scale == x on inputs that are exact multiples of the scale; zero rows.
 
+  truncate_matrix / maybe_truncate_local_group_size / local_permute / get_all_to_all_params / get_ragged_buffer_size
+      (the bookkeeping of the expert-parallel dispatch, all integer): the expected arrays of
+      tests/unit/moe_test.py:1174-1336 (local_permute with and without offset), :1338-1442 (the four parameter
+      vectors, batch sharded and replicated), :1444-1494 (buffer sizes); conservation laws for the truncation
+      (column sums never exceed the buffer, rows are cut in shard order, nothing changes below the capacity);
+      brute-force loops over rows for the keys.  The fill of rows past the received total follows
+      jax.numpy.repeat(total_repeat_length=...), which pads with the last value; moe_test.py:1174-1261 reaches it (its
+      slices are longer than the shards' rows) with jnp.repeat on both sides, so it pins the use of that rule, and the
+      rule itself is jax's documented one (those rows carry no tokens and no result depends on them).
+
 PARITY UNPINNED (third-party arithmetic whose source is not in the reference
 tree, and which no reference test pins):
   * quantize_rows_int8 / quantize_weight_int8 / quantize_fp8_blocks / quantize_e5m2: rounding mode and
@@ -251,6 +261,103 @@ def unpermute(intermediate: torch.Tensor, perm: np.ndarray, weights: np.ndarray,
   un = un.reshape(w.shape[0], k, -1)
   out = torch.einsum("bke,bk->be", un, w)
   return out.to(out_dtype)
+
+
+# --------------------------------------------------------------------------
+# Expert-parallel dispatch bookkeeping  (moe.py:103-120, :1066-1349, :1368-1401)
+# --------------------------------------------------------------------------
+
+
+def truncate_matrix(all_shards_group_sizes: np.ndarray, buffer_size: int) -> np.ndarray:
+  """moe.py:103-120: the traffic matrix [sender, receiver] cut so that no receiver gets more than buffer_size rows;
+  senders are served in order (prefix sum over axis 0, clamped, differenced)."""
+  a = np.asarray(all_shards_group_sizes)
+  c = np.minimum(np.cumsum(a, axis=0), buffer_size)
+  return np.diff(np.concatenate([np.zeros((1, a.shape[1]), dtype=c.dtype), c], axis=0), axis=0).astype(a.dtype)
+
+
+def maybe_truncate_local_group_size(all_shard_local_sizes: np.ndarray, buffer_size: int, ragged_buffer_factor: float) -> np.ndarray:
+  """moe.py:1066-1089: rows per local expert summed over the batch shards; with ragged_buffer_factor > 0 the flattened
+  [shard, local expert] sizes are first cut at buffer_size in that order."""
+  a = np.asarray(all_shard_local_sizes)
+  if ragged_buffer_factor > 0.0:
+    flat = a.reshape(-1)
+    c = np.minimum(np.cumsum(flat), buffer_size)
+    a = np.diff(np.concatenate([np.zeros((1,), dtype=c.dtype), c])).reshape(a.shape)
+  return a.sum(axis=0).astype(np.int32)
+
+
+def _repeat_total(values: np.ndarray, repeats: np.ndarray, total: int) -> np.ndarray:
+  """jax.numpy.repeat(values, repeats, total_repeat_length=total): output position p takes values[i] for the largest
+  i whose start (exclusive prefix sum of repeats) is <= p, so a short sum is padded with the last value and a long
+  one is cut."""
+  starts = np.concatenate([[0], np.cumsum(repeats)[:-1]])
+  idx = np.searchsorted(starts, np.arange(total), side="right") - 1
+  return np.asarray(values)[idx]
+
+
+def local_permute(inputs: torch.Tensor, global_group_sizes: np.ndarray, local_expert_size: int, shard_index: int,
+                  is_offset: bool = False, global_sorted_experts=None, ragged_buffer_factor: float = -1.0):
+  """moe.py:1091-1200 -> (sorted_inputs, sorted_indices, local_group_size, sorted_experts_ids).
+
+  global_group_sizes [batch shards, E].  Without offset the rows arrive grouped by (batch shard, local expert) and the
+  key of a row is its local expert; with offset the rows are all routed rows sorted by global expert and rows of other
+  shards get the key local_expert_size, which sorts them behind this shard's."""
+  g = np.asarray(global_group_sizes)
+  all_shard_local = g[:, shard_index * local_expert_size:(shard_index + 1) * local_expert_size]
+  local_sizes = all_shard_local.reshape(-1)
+  rows = inputs.shape[0]
+  local_group_size = maybe_truncate_local_group_size(all_shard_local, rows, ragged_buffer_factor)
+  if is_offset:
+    gse = np.asarray(global_sorted_experts)
+    keys = np.where(gse // local_expert_size == shard_index, gse % local_expert_size, local_expert_size)
+  else:
+    base = np.arange(local_sizes.shape[0]) % local_expert_size
+    keys = _repeat_total(base, local_sizes, rows)
+  sorted_indices = np.argsort(keys, kind="stable").astype(np.int32)
+  sorted_inputs = inputs[torch.from_numpy(sorted_indices.astype(np.int64))]
+  return sorted_inputs, sorted_indices, local_group_size, keys[sorted_indices].astype(np.int32)
+
+
+def get_all_to_all_params(all_shards_group_sizes: np.ndarray, shard_id: int, num_expert_parallelism: int,
+                          is_batch_sharded: bool = True, ragged_buffer_factor: float = -1.0, buffer_size=None,
+                          is_dispatch: bool = True):
+  """moe.py:1202-1349 -> (input_offsets, send_sizes, output_offsets, recv_sizes) of ragged_all_to_all."""
+  a = np.asarray(all_shards_group_sizes)
+
+  def input_offset(m):
+    if is_batch_sharded:
+      return np.concatenate([[0], np.cumsum(m[shard_id])[:-1]]).astype(m.dtype)
+    return np.zeros(num_expert_parallelism, dtype=m.dtype)
+
+  def send_size(m):
+    return m[shard_id] if is_batch_sharded else np.repeat(m[shard_id], num_expert_parallelism)
+
+  def output_offset(m):
+    if is_batch_sharded:
+      return np.cumsum(np.concatenate([np.zeros((1,) + m.shape[1:], dtype=m.dtype), m], axis=0), axis=0, dtype=m.dtype)[shard_id]
+    return np.repeat(np.concatenate([[0], np.cumsum(m[:-1])])[shard_id], num_expert_parallelism).astype(m.dtype)
+
+  def recv_size(m):
+    return m[:, shard_id] if is_batch_sharded else m
+
+  if ragged_buffer_factor > 0.0:
+    assert buffer_size is not None
+    t = truncate_matrix(a, buffer_size)
+    if is_dispatch:  # the sender still holds every row; sizes and receive offsets follow the cut matrix
+      return input_offset(a), send_size(t), output_offset(t), recv_size(t)
+    at, tt = a.T, t.T  # combine: the packed (cut) buffer is sent back to the rows' original positions
+    return input_offset(tt), send_size(tt), output_offset(at), recv_size(tt)
+  m = a if is_dispatch else a.T
+  return input_offset(m), send_size(m), output_offset(m), recv_size(m)
+
+
+def get_ragged_buffer_size(local_batch: int, ep_degree: int, global_experts: int, top_k: int, ragged_buffer_factor: float) -> int:
+  """moe.py:1368-1401: rows of the receive buffer: the balanced share times the factor, or the worst case
+  min(ep_degree, global_experts / top_k) times the share."""
+  if ragged_buffer_factor > 0.0:
+    return int(local_batch * ragged_buffer_factor)
+  return int(local_batch * min(ep_degree, global_experts / top_k))
 
 
 def unroute_sum(tokens: torch.Tensor, selected_experts: np.ndarray):
