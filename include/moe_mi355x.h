@@ -132,6 +132,12 @@ MOE_API size_t moe_sort_workspace_bytes(int T, int k, int E);
 MOE_API int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,
                        int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                        void* workspace, size_t workspace_bytes, void* stream);
+/* The same with the ids rolled first: key = (id - roll_to_expert_id) mod E (permute's roll_to_expert_id,
+ * moe.py:953-954, by which a shard of the ring-of-experts strategy brings its own experts to the front);
+ * group_sizes and sorted_experts are those of the rolled ids.  0 <= roll_to_expert_id < E. */
+MOE_API int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+                       int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Expert-parallel dispatch bookkeeping on one expert shard (integer work on device-resident sizes; the exchange

@@ -323,9 +323,14 @@ constexpr int kSortChunk = kSortSeg * kSortWaves;  // entries per block
 constexpr int kSortMaxE = 512;
 
 __device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
+// sort key of expert id e: (e - roll) mod E (permute's roll_to_expert_id, moe.py:953-954; roll = 0: the id itself)
+__device__ __forceinline__ int sort_key(int e, int E, int roll) {
+  e = clamp_expert(e, E) - roll;
+  return e < 0 ? e + E : e;
+}
 
 __global__ __launch_bounds__(kSortWaves* kWave) void sort_hist_kernel(
-    const int32_t* __restrict__ flat, int M, int E, int32_t* __restrict__ seg_hist) {
+    const int32_t* __restrict__ flat, int M, int E, int roll, int32_t* __restrict__ seg_hist) {
   __shared__ int cnt[kSortWaves][kSortMaxE];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   for (int e = lane; e < E; e += kWave) cnt[wave][e] = 0;
@@ -334,7 +339,7 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_hist_kernel(
 #pragma unroll
   for (int r = 0; r < kSortRounds; r++) {
     int i = base + r * kWave + lane;
-    if (i < M) atomicAdd(&cnt[wave][clamp_expert(flat[i], E)], 1);
+    if (i < M) atomicAdd(&cnt[wave][sort_key(flat[i], E, roll)], 1);
   }
   __syncthreads();
   int32_t* dst = seg_hist + (size_t)(blockIdx.x * kSortWaves + wave) * E;
@@ -365,7 +370,7 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scan_kernel(int32_t* _
 }
 
 __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
-    const int32_t* __restrict__ flat, int M, int E, int ebits,
+    const int32_t* __restrict__ flat, int M, int E, int roll, int ebits,
     const int32_t* __restrict__ seg_hist, const int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
     int32_t* __restrict__ sorted_experts) {
@@ -395,7 +400,7 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
   for (int r = 0; r < kSortRounds; r++) {
     const int i = base + r * kWave + lane;
     const bool valid = i < M;
-    const int e = valid ? clamp_expert(flat[i], E) : 0;
+    const int e = valid ? sort_key(flat[i], E, roll) : 0;
     unsigned long long mask = __ballot(valid);
     for (int b = 0; b < ebits; b++) {
       const bool bit = (e >> b) & 1;
@@ -422,7 +427,7 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
 // segments and over the experts, then the same in-order ranking.
 template <int NW>
 __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
-    const int32_t* __restrict__ flat, int M, int E, int ebits, int32_t* __restrict__ group_sizes,
+    const int32_t* __restrict__ flat, int M, int E, int roll, int ebits, int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts) {
   __shared__ int run[NW][kSortMaxE];
   __shared__ int off[kSortMaxE];
@@ -434,7 +439,7 @@ __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
 #pragma unroll
   for (int r = 0; r < kSortRounds; r++) {
     const int i = base + r * kWave + lane;
-    if (i < M) atomicAdd(&run[wave][clamp_expert(flat[i], E)], 1);
+    if (i < M) atomicAdd(&run[wave][sort_key(flat[i], E, roll)], 1);
   }
   __syncthreads();
   // counts of the segments -> exclusive prefixes over the segments; the expert's total goes to group_sizes and to off
@@ -470,7 +475,7 @@ __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
   for (int r = 0; r < kSortRounds; r++) {
     const int i = base + r * kWave + lane;
     const bool valid = i < M;
-    const int e = valid ? clamp_expert(flat[i], E) : 0;
+    const int e = valid ? sort_key(flat[i], E, roll) : 0;
     unsigned long long mask = __ballot(valid);
     for (int b = 0; b < ebits; b++) {
       const bool bit = (e >> b) & 1;
@@ -971,12 +976,14 @@ size_t moe_sort_workspace_bytes(int T, int k, int E) {
   return (nseg * E + E) * sizeof(int32_t) + 256;
 }
 
-int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,
-                       int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
-                       void* workspace, size_t workspace_bytes, void* stream) {
+int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+                              int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                              void* workspace, size_t workspace_bytes, void* stream) {
   if (!topk_idx || !perm || !group_sizes || !workspace) return fail(MOE_ERR_INVALID_ARG, "sort: NULL pointer");
   if (T < 0 || k <= 0 || E <= 0) return fail(MOE_ERR_INVALID_ARG, "sort: bad sizes");
   if (E > kSortMaxE) return fail(MOE_ERR_UNSUPPORTED, "sort: E=%d > %d", E, kSortMaxE);
+  if (roll_to_expert_id < 0 || roll_to_expert_id >= E) return fail(MOE_ERR_INVALID_ARG, "sort: roll_to_expert_id %d outside [0, %d)", roll_to_expert_id, E);
+  const int roll = roll_to_expert_id;
   if ((long long)T * k > INT_MAX / 2) return fail(MOE_ERR_UNSUPPORTED, "sort: T*k too large");
   if (workspace_bytes < moe_sort_workspace_bytes(T, k, E)) return fail(MOE_ERR_WORKSPACE, "sort: workspace too small");
   const int M = T * k;
@@ -987,19 +994,25 @@ int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* pe
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
   if (nblk <= 1) {  // also M == 0: group_sizes are all zero
-    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts);
     return check_launch("sort_by_expert");
   }
   if (nblk <= 4) {  // up to 4096 entries: still one launch, with 16 waves
-    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts);
     return check_launch("sort_by_expert");
   }
-  if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, seg_hist);
+  if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, seg_hist);
   sort_scan_kernel<<<cdiv(E, kSortWaves), kSortWaves * kWave, 0, s>>>(seg_hist, nseg, E, group_sizes);
   if (nblk > 0)
-    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, ebits, seg_hist, group_sizes,
+    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, seg_hist, group_sizes,
                                                           perm, inv_perm, sorted_experts);
   return check_launch("sort_by_expert");
+}
+
+int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,
+                       int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  return moe_sort_by_expert_rolled(topk_idx, T, k, E, 0, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes, stream);
 }
 
 int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, int R_in, int R_out, int d,

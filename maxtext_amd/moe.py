@@ -272,14 +272,15 @@ class RoutedMoE:
               roll_to_expert_id=None, input_ids=None):
     """-> (sorted_inputs, sorted_selected_experts, weights, group_size, sorted_experts,
     lb_loss, bias_updates, local_group_size), as moe.py:993-1002."""
-    if roll_to_expert_id is not None:
-      raise NotImplementedError("the ring-of-experts roll is a multi-device feature")
     b, s, d = inputs.shape
     x2d = inputs.reshape(b * s, d).contiguous()
     weights, selected = self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
     x2d = self._scale_inputs_by_router_score(x2d, weights)
     sel2d = selected.reshape(b * s, -1).contiguous()
-    perm, inv, group_size, sorted_experts = kernels.sort_by_expert(sel2d, self.num_experts)
+    # roll_to_expert_id (a host integer here; the reference passes shard index * experts per shard): ids are sorted as
+    # (id - roll) mod E, so that the calling shard's experts come first (moe.py:953-954)
+    roll = 0 if roll_to_expert_id is None else int(roll_to_expert_id) % self.num_experts
+    perm, inv, group_size, sorted_experts = kernels.sort_by_expert(sel2d, self.num_experts, roll_to_expert_id=roll)
     if torch.is_grad_enabled() and x2d.requires_grad:
       sorted_inputs = _GatherRowsFn.apply(x2d, perm, inv, self.num_experts_per_tok)
     else:

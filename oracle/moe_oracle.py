@@ -237,14 +237,16 @@ def calculate_load_balance_updates(top_k_indices, num_experts: int, rate: float)
 # --------------------------------------------------------------------------
 
 
-def permute(inputs_2d: torch.Tensor, selected_experts: np.ndarray, num_experts: int):
-  """moe.py:950-960, :986-991 (non-ragged branch).
+def permute(inputs_2d: torch.Tensor, selected_experts: np.ndarray, num_experts: int, roll_to_expert_id=None):
+  """moe.py:950-960, :986-991 (non-ragged branch); roll_to_expert_id: ids become (id - roll) % E first (:953-954).
 
   Returns (sorted_inputs [M,d], sorted_selected_experts [M] int32 -- the stable
   argsort of the flattened expert ids, group_size [E] int32, sorted_experts [M]).
   Row i of sorted_inputs is token perm[i] // k (repeat(x, k)[perm])."""
   t, k = selected_experts.shape
   flat = np.asarray(selected_experts).reshape(-1)
+  if roll_to_expert_id is not None:
+    flat = (flat - roll_to_expert_id) % num_experts
   perm = np.argsort(flat, kind="stable").astype(np.int32)
   sorted_inputs = inputs_2d[torch.from_numpy((perm // k).astype(np.int64))]
   group_size = np.bincount(flat, minlength=num_experts).astype(np.int32)

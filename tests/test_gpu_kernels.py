@@ -112,6 +112,25 @@ def test_sort_by_expert_bit_exact(K, t, e, k):
     assert (ogs == 0).any()  # the skewed selection leaves experts empty
 
 
+@pytest.mark.parametrize("t,e,k,roll", [(7, 8, 2, 2), (128, 8, 2, 6), (1000, 128, 8, 96), (4099, 256, 8, 32), (2048, 32, 4, 31), (513, 512, 3, 64)])
+def test_sort_by_expert_rolled_bit_exact(K, t, e, k, roll):
+  # permute(roll_to_expert_id=...) (moe.py:953-954): the ids are sorted as (id - roll) % E
+  rng = np.random.default_rng(e + t + roll)
+  sel = _zipf_selection(rng, t, e, k) if e >= 32 else np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  perm, inv, gs, se = K.sort_by_expert(cuda(sel), e, roll_to_expert_id=roll)
+  _, operm, ogs, ose = O.permute(torch.zeros(t, 8, dtype=torch.bfloat16), sel, e, roll_to_expert_id=roll)
+  np.testing.assert_array_equal(perm.cpu().numpy(), operm)
+  np.testing.assert_array_equal(gs.cpu().numpy(), ogs)
+  np.testing.assert_array_equal(se.cpu().numpy(), ose)
+  np.testing.assert_array_equal(inv.cpu().numpy(), np.argsort(operm, kind="stable").astype(np.int32))
+  # the rolled order is the plain order of the ids rotated by the rows of the first `roll` experts
+  plain = K.sort_by_expert(cuda(sel), e)
+  ahead = int(plain[2][:roll].sum())
+  np.testing.assert_array_equal(perm.cpu().numpy(), np.roll(plain[0].cpu().numpy(), -ahead))
+  with pytest.raises(RuntimeError):
+    K.sort_by_expert(cuda(sel), e, roll_to_expert_id=e)
+
+
 @pytest.mark.parametrize("d", [8, 512, 2048, 4096, 7168, 14336])
 def test_gather_rows_copy_bit_exact(K, d):
   rng = np.random.default_rng(d)

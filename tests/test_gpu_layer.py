@@ -120,6 +120,27 @@ def test_permute_unpermute_api_roundtrip():
   assert torch.equal(out, (x.float() * k).to(torch.bfloat16))
 
 
+def test_permute_roll_to_expert_id():
+  # permute(roll_to_expert_id=r) (moe.py:953-954): rows of experts r, r+1, ... come first; against the oracle's permute
+  from maxtext_amd import moe
+
+  t, d, e, k, roll = 257, 64, 16, 2, 12
+  cfg = moe.MoEConfig(e, k, d, 128)
+  block = moe.RoutedMoE(cfg, None, None, None)
+  g = torch.Generator(device="cuda").manual_seed(4)
+  x = torch.randn((1, t, d), generator=g, device="cuda").to(torch.bfloat16)
+  logits = torch.randn((1, t, e), generator=g, device="cuda")
+  sorted_inputs, perm, weights, group_size, sorted_experts, _, _, _ = block.permute(x, logits, roll_to_expert_id=roll)
+  _, sel = block.get_topk(logits)
+  want = O.permute(x[0].cpu(), sel.reshape(t, k).cpu().numpy(), e, roll_to_expert_id=roll)
+  assert torch.equal(sorted_inputs.cpu(), want[0])
+  np.testing.assert_array_equal(perm.cpu().numpy(), want[1])
+  np.testing.assert_array_equal(group_size.cpu().numpy(), want[2])
+  np.testing.assert_array_equal(sorted_experts.cpu().numpy(), want[3])
+  out = block.unpermute(sorted_inputs, perm, torch.ones_like(weights), 1, t)
+  assert torch.equal(out, (x.float() * k).to(torch.bfloat16))
+
+
 def test_megablox_gmm_api():
   from maxtext_amd import megablox
 

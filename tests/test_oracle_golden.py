@@ -699,3 +699,21 @@ def test_ragged_variants_hand_cases():
   h1 = torch.tensor([[1.015625]]).to(torch.bfloat16)
   got = O.weighted_intermediate(h0, h1, torch.tensor([1.75]))
   assert got.tolist() == [[58.5]]
+
+
+def test_permute_roll_is_a_rotation_of_the_plain_order():
+  # (id - roll) % E keeps the order inside an expert and moves the experts below `roll` behind all others (moe.py:953-954)
+  rng = np.random.default_rng(5)
+  t, k, e, roll = 37, 3, 8, 3
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  x = torch.arange(t, dtype=torch.float32).reshape(t, 1).to(torch.bfloat16)
+  _, perm0, gs0, _ = O.permute(x, sel, e)
+  si, perm, gs, se = O.permute(x, sel, e, roll_to_expert_id=roll)
+  ahead = int(gs0[:roll].sum())
+  np.testing.assert_array_equal(perm, np.roll(perm0, -ahead))
+  np.testing.assert_array_equal(gs, np.roll(gs0, -roll))
+  np.testing.assert_array_equal(se, np.repeat(np.arange(e), np.roll(gs0, -roll)))
+  # brute force: rows listed expert by expert starting at expert `roll`, tokens in order
+  want = [i for ex in list(range(roll, e)) + list(range(roll)) for i in range(t * k) if sel.reshape(-1)[i] == ex]
+  np.testing.assert_array_equal(perm, want)
+  assert torch.equal(si, x[torch.tensor(want) // k])
