@@ -136,3 +136,93 @@ def test_dispatch_argument_errors(M):
     M.local_permute(torch.zeros((4, 8), dtype=torch.bfloat16, device="cuda"), g, 4, 0, is_offset=True)
   with pytest.raises(RuntimeError):
     kernels.all_to_all_params(cuda_i32(np.ones(4)), 0, 4, is_batch_sharded=False, buffer_size=8)
+
+
+def _shard_layer(moe, cfg, ws, x, logits):
+  return moe.RoutedMoE(cfg, *ws).sparse_matmul(x, logits, None, *ws)[0]
+
+
+def test_ragged_all_to_all_flow_on_one_gpu_matches_the_single_device_layer():
+  # ra2a_and_route + unsort_output_and_ra2a (moe.py:1757-1856, :2022-2087) with 4 batch shards and 4 expert shards played
+  # one after the other on this GPU; the collective is copied by hand from the offsets and sizes this library computes
+  # (ragged_all_to_all: piece j of the sender's operand goes to peer j at the output offset the sender names).
+  from maxtext_amd import kernels, megablox, moe
+  from tolerances import relerr
+
+  p, e, k, d, f, tb = 4, 16, 2, 128, 256, 96
+  l = e // p
+  cfg = moe.MoEConfig(e, k, d, f)
+  g = torch.Generator(device="cuda").manual_seed(11)
+  w0, w1 = [(torch.randn((e, f, d), generator=g, device="cuda") * 0.05).to(torch.bfloat16) for _ in range(2)]
+  wo = (torch.randn((e, d, f), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  block = moe.RoutedMoE(cfg, w0, w1, wo)
+  xs = [torch.randn((1, tb, d), generator=g, device="cuda").to(torch.bfloat16) for _ in range(p)]
+  # skewed logits: expert shards receive different loads, some experts nothing
+  lg = [torch.randn((1, tb, e), generator=g, device="cuda") - 0.4 * torch.arange(e, device="cuda") for _ in range(p)]
+
+  routed = [block.permute(xs[b], lg[b]) for b in range(p)]  # (sorted x, perm, weights, group_size, ...)
+  group_sizes = torch.stack([r[3] for r in routed]).contiguous()            # all_gather(group_sizes): [P, E]
+  traffic = group_sizes.reshape(p, p, l).sum(-1).to(torch.int32).contiguous()  # all_shards_group_sizes [P, P]
+  rows = tb * k
+  buffer_size = moe.RoutedMoE.get_ragged_buffer_size(rows, p, e, k, -1.0)
+  assert buffer_size == rows * p
+
+  # dispatch
+  buffers = [torch.full((buffer_size, d), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(p)]
+  for s in range(p):
+    in_off, send, out_off, recv = [v.cpu().numpy() for v in moe.RoutedMoE.get_all_to_all_params(traffic, s, p)]
+    np.testing.assert_array_equal(recv, traffic[:, s].cpu().numpy())
+    for j in range(p):
+      buffers[j][out_off[j]:out_off[j] + send[j]] = routed[s][0][in_off[j]:in_off[j] + send[j]]
+
+  # every expert shard: local permute, its own experts' three matmuls, local unsort
+  returned = []
+  for j in range(p):
+    xj, local_idx, local_sizes, ids = moe.RoutedMoE.local_permute(buffers[j], group_sizes, l, j, use_ragged_sort=True)
+    n = int(local_sizes.sum())
+    assert n == int(traffic[:, j].sum()) and not torch.isnan(xj[:n].float()).any()
+    np.testing.assert_array_equal(ids[:n].cpu().numpy(), np.repeat(np.arange(l), local_sizes.cpu().numpy()))
+    sl = slice(j * l, (j + 1) * l)
+    h = megablox.gmm(xj, w0[sl].contiguous(), local_sizes, transpose_rhs=True, rhs_up=w1[sl].contiguous(), fuse_act="silu")
+    y = megablox.gmm(h, wo[sl].contiguous(), local_sizes, transpose_rhs=True)
+    returned.append(kernels.unpermute_combine(y.contiguous(), None, k=1, perm=local_idx))  # rows back in arrival order
+
+  # the way back, then each batch shard's unpermute with its routing weights
+  for b in range(p):
+    got_rows = torch.zeros((rows, d), dtype=torch.bfloat16, device="cuda")
+    for j in range(p):
+      in_off, send, out_off, recv = [v.cpu().numpy() for v in moe.RoutedMoE.get_all_to_all_params(traffic, j, p, is_dispatch=False)]
+      got_rows[out_off[b]:out_off[b] + send[b]] = returned[j][in_off[b]:in_off[b] + send[b]]
+    out = block.unpermute(got_rows, routed[b][1], routed[b][2], 1, tb)
+    want = _shard_layer(moe, cfg, (w0, w1, wo), xs[b], lg[b])
+    assert relerr(out.float().cpu(), want.float().cpu()) <= 1e-2
+
+
+def test_ring_of_experts_flow_on_one_gpu_matches_the_single_device_layer():
+  # roe_ag_and_route (moe.py:1709-1755): every expert shard sees all tokens, sorts them with its own experts first
+  # (roll_to_expert_id), multiplies only its experts' rows (group_offset 0, the local experts' weights) and the shards'
+  # partial outputs add up (the reduce-scatter of moe.py:2266) to the single-device layer
+  from maxtext_amd import megablox, moe
+  from tolerances import relerr
+
+  p, e, k, d, f, t = 4, 16, 2, 128, 256, 200
+  l = e // p
+  cfg = moe.MoEConfig(e, k, d, f)
+  g = torch.Generator(device="cuda").manual_seed(12)
+  w0, w1 = [(torch.randn((e, f, d), generator=g, device="cuda") * 0.05).to(torch.bfloat16) for _ in range(2)]
+  wo = (torch.randn((e, d, f), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  block = moe.RoutedMoE(cfg, w0, w1, wo)
+  x = torch.randn((1, t, d), generator=g, device="cuda").to(torch.bfloat16)
+  logits = torch.randn((1, t, e), generator=g, device="cuda")
+  total = torch.zeros((t, d), dtype=torch.float32, device="cuda")
+  for j in range(p):
+    sx, perm, weights, group_size, sorted_experts, _, _, _ = block.permute(x, logits, roll_to_expert_id=j * l)
+    sl = slice(j * l, (j + 1) * l)
+    # rolled ids: this shard's experts are groups 0 .. l-1 of the rolled order; rows of the other groups come back as zeros
+    h = megablox.gmm(sx, w0[sl].contiguous(), group_size, transpose_rhs=True, rhs_up=w1[sl].contiguous(), fuse_act="silu", group_offset=0)
+    y = megablox.gmm(h, wo[sl].contiguous(), group_size, transpose_rhs=True, group_offset=0)
+    n = int(group_size[:l].sum())
+    assert not y[n:].any()
+    total += block.unpermute(y, perm, weights, 1, t).reshape(t, d).float()
+  want = _shard_layer(moe, cfg, (w0, w1, wo), x, logits)
+  assert relerr(total.cpu(), want.reshape(t, d).float().cpu()) <= 1e-2
