@@ -170,8 +170,23 @@ MOE_API int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int
  *                           sender order (_truncate_matrix, moe.py:103-120); < 0: no capacity.  Batch-sharded only.
  *   is_dispatch             1: tokens to experts; 0: the way back (transposed roles, moe.py:1296-1330)
  * Limits: num_expert_parallelism <= 1024.
+ *
+ * moe_ring_ragged_indices derives the index arrays of ring_ragged_sort / ring_ragged_unsort
+ * (kernels/ragged/ragged_sort.py:102-151, :300-350) from the sort's permutation, so that the row movement is one
+ * moe_gather_rows (sort) or one moe_unpermute_combine (unsort) and nothing is read back by the host.  The rows of the
+ * shard's experts [experts_start, experts_start + local_experts) are positions [start, end) of the sorted order.
+ *   unsort = 0  indices = perm [num_rows]; indices_out [min(buffer_size, num_rows)]; row_range [2]:
+ *               buffer_size >= num_rows: indices_out = perm, row_range = (start, end); smaller: indices_out[i] =
+ *               perm[start + i] (0 past the end), row_range = (0, min(end - start, buffer_size)).  Gather with
+ *               idx_div = k and this row_range.
+ *   unsort = 1  indices = inv_perm [num_rows]; indices_out, valid_rows_mask [num_rows]: the inverse permutation
+ *               (shifted by -start into the packed buffer when buffer_size < num_rows) and which of its entries
+ *               point at a row of this shard; the others are 0 with mask 0.
  */
 MOE_API size_t moe_local_expert_keys_workspace_bytes(int num_batch_shards, int local_expert_size);
+MOE_API int moe_ring_ragged_indices(const int32_t* indices, const int32_t* group_sizes, int num_experts, int experts_start,
+                            int local_experts, int num_rows, int buffer_size, int unsort, int32_t* indices_out,
+                            uint8_t* valid_rows_mask, int32_t* row_range, void* stream);
 MOE_API int moe_local_expert_keys(const int32_t* global_group_sizes, int num_batch_shards, int num_experts,
                           int local_expert_size, int shard_index, int num_rows, const int32_t* global_sorted_experts,
                           int truncate, int32_t* expert_keys, int32_t* local_group_size, void* workspace,

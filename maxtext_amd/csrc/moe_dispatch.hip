@@ -142,6 +142,60 @@ __global__ __launch_bounds__(kDispThreads) void all_to_all_params_kernel(const i
   }
 }
 
+// Index arrays of the ring-of-experts ragged sort (kernels/ragged/ragged_sort.py:23-226, :229-365).  The rows of this
+// shard's experts are positions [start, end) of the globally sorted order (start / end = sums of group_sizes before /
+// through the shard's experts); with a buffer smaller than the n sorted rows they are packed at its front.
+//   SORT:   idx_in = the sort permutation.  Unbuffered: idx_out = idx_in, range = [start, end).  Buffered: idx_out[i] =
+//           idx_in[start + i] (0 past the end), range = [0, min(end - start, buffer)).
+//   UNSORT: idx_in = the inverse permutation.  Unbuffered: idx_out = idx_in, mask[i] = start <= idx_in[i] < end.
+//           Buffered: idx_out[i] = idx_in[i] - start where 0 <= that < min(end - start, buffer), else 0 with mask 0.
+__global__ __launch_bounds__(256) void ring_ragged_indices_kernel(const int32_t* __restrict__ idx_in, const int32_t* __restrict__ group_sizes,
+                                                                  int E, int experts_start, int local_experts, int n, int buffer,
+                                                                  int unsort, int32_t* __restrict__ idx_out, uint8_t* __restrict__ mask_out,
+                                                                  int32_t* __restrict__ range_out) {
+  __shared__ long long s_before[256], s_local[256];
+  long long before = 0, local = 0;
+  for (int e = threadIdx.x; e < experts_start + local_experts && e < E; e += 256) {
+    const long long g = max(group_sizes[e], 0);
+    if (e < experts_start) before += g;
+    else local += g;
+  }
+  s_before[threadIdx.x] = before;
+  s_local[threadIdx.x] = local;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) {
+      s_before[threadIdx.x] += s_before[threadIdx.x + o];
+      s_local[threadIdx.x] += s_local[threadIdx.x + o];
+    }
+    __syncthreads();
+  }
+  const long long start = min(s_before[0], (long long)n), end = min(s_before[0] + s_local[0], (long long)n);
+  const bool buffered = buffer < n;
+  const long long limit = min(end - start, (long long)buffer);
+  if (blockIdx.x == 0 && threadIdx.x == 0 && range_out) {
+    range_out[0] = buffered ? 0 : (int32_t)start;
+    range_out[1] = buffered ? (int32_t)limit : (int32_t)end;
+  }
+  const int out_n = unsort ? n : (buffered ? buffer : n);
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= out_n) return;
+  if (!unsort) {
+    idx_out[i] = buffered ? (start + i < n ? idx_in[start + i] : 0) : idx_in[i];
+  } else {
+    const long long v = idx_in[i];
+    if (!buffered) {
+      idx_out[i] = (int32_t)v;
+      mask_out[i] = v >= start && v < end;
+    } else {
+      const long long sh = v - start;
+      const bool ok = sh >= 0 && sh < limit;
+      idx_out[i] = ok ? (int32_t)sh : 0;
+      mask_out[i] = ok;
+    }
+  }
+}
+
 }  // namespace moe
 
 using namespace moe;
@@ -190,6 +244,21 @@ int moe_all_to_all_params(const int32_t* all_shards_group_sizes, int num_expert_
   all_to_all_params_kernel<<<1, kDispThreads, 0, (hipStream_t)stream>>>(all_shards_group_sizes, num_expert_parallelism, shard_id, is_batch_sharded,
                                                                         buffer_size, is_dispatch, input_offsets, send_sizes, output_offsets, recv_sizes);
   return check_launch("all_to_all_params");
+}
+
+int moe_ring_ragged_indices(const int32_t* indices, const int32_t* group_sizes, int num_experts, int experts_start,
+                            int local_experts, int num_rows, int buffer_size, int unsort, int32_t* indices_out,
+                            uint8_t* valid_rows_mask, int32_t* row_range, void* stream) {
+  if (!indices || !group_sizes || !indices_out) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: NULL pointer");
+  if (unsort ? !valid_rows_mask : !row_range) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: NULL output");
+  if (num_experts <= 0 || experts_start < 0 || local_experts <= 0 || experts_start + local_experts > num_experts || num_rows < 0)
+    return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: experts %d .. +%d of %d, %d rows", experts_start, local_experts, num_experts, num_rows);
+  if (buffer_size < 0) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: buffer_size %d", buffer_size);
+  const int out_n = unsort ? num_rows : (buffer_size < num_rows ? buffer_size : num_rows);
+  const int blocks = out_n > 0 ? cdiv(out_n, 256) : 1;
+  ring_ragged_indices_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(indices, group_sizes, num_experts, experts_start, local_experts, num_rows,
+                                                                        buffer_size, unsort, indices_out, valid_rows_mask, row_range);
+  return check_launch("ring_ragged_indices");
 }
 
 }  // extern "C"

@@ -192,6 +192,24 @@ def all_to_all_params(all_shards_group_sizes, shard_id, num_expert_parallelism, 
   return out[0], out[1], out[2], out[3]
 
 
+def ring_ragged_indices(indices, group_sizes, experts_start, local_experts, *, buffer_size=None, unsort=False):
+  """Index arrays of ring_ragged_sort / ring_ragged_unsort (kernels/ragged/ragged_sort.py:102-151, :300-350).
+  unsort=False: indices = perm -> (row_idx [min(buffer, n)], row_range [2]); unsort=True: indices = inv_perm ->
+  (inv_perm into the shard's buffer [n], valid_rows_mask [n] uint8)."""
+  _need(indices, "indices", torch.int32, 1)
+  _need(group_sizes, "group_sizes", torch.int32, 1)
+  n = indices.shape[0]
+  buf = n if buffer_size is None else int(buffer_size)
+  dev = indices.device
+  out = torch.empty((n if unsort else min(buf, n),), dtype=torch.int32, device=dev)
+  mask = torch.empty((n,), dtype=torch.uint8, device=dev) if unsort else None
+  rng = None if unsort else torch.empty((2,), dtype=torch.int32, device=dev)
+  st = _lib.load().moe_ring_ragged_indices(_lib.ptr(indices), _lib.ptr(group_sizes), group_sizes.shape[0], int(experts_start), int(local_experts),
+                                           n, buf, int(bool(unsort)), _lib.ptr(out), _lib.ptr(mask), _lib.ptr(rng), _lib.current_stream())
+  _lib.check(st, "moe_ring_ragged_indices")
+  return (out, mask) if unsort else (out, rng)
+
+
 def _valid_mask(valid_rows_mask, m):
   if valid_rows_mask is None:
     return None
@@ -201,10 +219,15 @@ def _valid_mask(valid_rows_mask, m):
   return valid_rows_mask.view(torch.uint8)
 
 
-def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None, valid_rows_mask=None):
-  """out[t] = sum over the valid s of weights[t,s] * y[inv_perm[t*k+s]]  (f32 accumulate, bf16 out)."""
+def unpermute_combine(y, weights, *, k, perm=None, inv_perm=None, valid_rows_mask=None, num_tokens=None):
+  """out[t] = sum over the valid s of weights[t,s] * y[inv_perm[t*k+s]]  (f32 accumulate, bf16 out).
+  num_tokens: T when y is a packed buffer with other than T*k rows (needs inv_perm, whose valid entries index y)."""
   _need(y, "y", torch.bfloat16, 2)
   m, d = y.shape
+  if num_tokens is not None:
+    if inv_perm is None:
+      raise ValueError("num_tokens needs inv_perm")
+    m = int(num_tokens) * k
   if m % k:
     raise ValueError("rows of y must be a multiple of k")
   t = m // k

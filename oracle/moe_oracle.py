@@ -35,6 +35,11 @@ How each function is pinned (see tests/test_oracle_*.py):
       nibble order and 2^(s-127) scaling on hand-made blocks; quantize_mxfp4 (a test-data generator only) by
       dequantize(quantize(x)) == x on representable inputs.
 
+  ring_ragged_sort / ring_ragged_unsort / a2a_ragged_sort
+      compositions of ragged_gather / ragged_gather_reduce (pinned below) with index arithmetic; checked against
+      row-by-row loops (which sorted positions belong to the shard, where they sit in a packed buffer) and by the
+      identity sum over shards of unsort(sort(x)) == sum of the routing weights times x.
+
   ragged_gather / ragged_gather_reduce / weighted_intermediate
       hand-made rows: a NaN row behind a cleared mask bit stays out of the sum, a group with every row masked
       gives zeros, the f32 sum rounds once (a case where rounding each term first gives another result), equality
@@ -394,6 +399,54 @@ def ragged_gather_reduce(x: torch.Tensor, indices: np.ndarray, topk_weights: tor
   out = torch.where(torch.from_numpy(np.asarray(valid_rows_mask, dtype=bool))[:, None], out, torch.zeros_like(out))
   out = out.reshape(-1, reduce_group_size, out.shape[-1])
   return out.sum(1).to(torch.bfloat16)
+
+
+def _shard_rows(group_sizes: np.ndarray, num_experts: int, shard_idx: int, ep_size: int):
+  """Positions [start, end) of a shard's experts in the order sorted by expert (ragged_sort.py:102-107)."""
+  offs = np.concatenate([[0], np.cumsum(group_sizes)])
+  local = num_experts // ep_size
+  return int(offs[shard_idx * local]), int(offs[(shard_idx + 1) * local])
+
+
+def ring_ragged_sort(hidden: torch.Tensor, topk_indices: np.ndarray, num_experts: int, topk: int, shard_idx: int, ep_size: int,
+                     buffer_size=None):
+  """kernels/ragged/ragged_sort.py:84-151 (forward) -> (x, group_sizes [E], topk_argsort_revert_indices [T*k])."""
+  t = hidden.shape[0]
+  flat = np.asarray(topk_indices).reshape(-1)
+  order = np.argsort(flat, kind="stable")
+  token_sorted = np.repeat(np.arange(t), topk)[order]
+  group_sizes = np.bincount(flat, minlength=num_experts).astype(np.int32)
+  revert = np.argsort(order, kind="stable").astype(np.int32)
+  start, end = _shard_rows(group_sizes, num_experts, shard_idx, ep_size)
+  n = t * topk
+  if buffer_size is None or buffer_size >= n:
+    x = ragged_gather(hidden, token_sorted, start, end)
+  else:
+    sliced = np.pad(token_sorted, (0, buffer_size))[start:start + buffer_size]
+    x = ragged_gather(hidden, sliced, 0, min(end - start, buffer_size))
+  return x, group_sizes, revert
+
+
+def ring_ragged_unsort(sorted_tokens: torch.Tensor, group_sizes: np.ndarray, revert: np.ndarray, topk: int, local_num_experts: int,
+                       shard_idx: int, topk_weights: torch.Tensor):
+  """kernels/ragged/ragged_sort.py:294-351 (forward) -> [T, hidden]."""
+  offs = np.concatenate([[0], np.cumsum(group_sizes)])
+  start, end = int(offs[shard_idx * local_num_experts]), int(offs[(shard_idx + 1) * local_num_experts])
+  revert = np.asarray(revert, dtype=np.int64)
+  buffer_size, n = sorted_tokens.shape[0], revert.shape[0]
+  w = topk_weights.reshape(-1).to(torch.float32)
+  if buffer_size >= n:
+    mask = (revert >= start) & (revert < end)
+    return ragged_gather_reduce(sorted_tokens, revert, w, mask, topk)
+  shifted = revert - start
+  mask = (shifted >= 0) & (shifted < min(end - start, buffer_size))
+  return ragged_gather_reduce(sorted_tokens, np.where(mask, shifted, 0), w, mask, topk)
+
+
+def a2a_ragged_sort(inputs: torch.Tensor, sort_indices: np.ndarray, valid_end: int):
+  """kernels/ragged/ragged_sort.py:497-512 (and, with revert indices, :592-606): rows below valid_end are gathered,
+  the rest are zeros."""
+  return ragged_gather(inputs, sort_indices, 0, int(valid_end))
 
 
 def weighted_intermediate(h0: torch.Tensor, h1: torch.Tensor, weights: torch.Tensor, kind: str = "silu", limit: float = 7.0):

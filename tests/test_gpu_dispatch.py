@@ -226,3 +226,57 @@ def test_ring_of_experts_flow_on_one_gpu_matches_the_single_device_layer():
     total += block.unpermute(y, perm, weights, 1, t).reshape(t, d).float()
   want = _shard_layer(moe, cfg, (w0, w1, wo), x, logits)
   assert relerr(total.cpu(), want.reshape(t, d).float().cpu()) <= 1e-2
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_ring_ragged_sort_unsort(seed):
+  # kernels/ragged/ragged_sort.py:23-451 (forward passes) against the oracle: indices bit-exact, rows are copies, the
+  # weighted sum within the output tolerance
+  from maxtext_amd import ragged_sort
+  from tolerances import relerr
+
+  rng = np.random.default_rng(300 + seed)
+  ep = int(rng.choice([1, 2, 4, 8]))
+  e = ep * int(rng.choice([1, 2, 4, 16]))
+  k = int(rng.integers(1, min(e, 8) + 1))
+  t = int(rng.choice([1, 5, 64, 700]))
+  d = int(rng.choice([8, 64, 512]))
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(torch.bfloat16)
+  w = torch.from_numpy(rng.random((t, k)).astype(np.float32))
+  n = t * k
+  for shard in sorted({0, ep - 1, ep // 2}):
+    for buf in (None, n + 3, max(n // (2 * ep), 1)):
+      want_x, want_gs, want_rev = O.ring_ragged_sort(x, sel, e, k, shard, ep, buffer_size=buf)
+      got_x, got_gs, got_rev = ragged_sort.ring_ragged_sort(x.cuda(), cuda_i32(sel), e, k, shard, ep, buffer_size=buf)
+      np.testing.assert_array_equal(got_gs.cpu().numpy(), want_gs)
+      np.testing.assert_array_equal(got_rev.cpu().numpy(), want_rev)
+      # the reference returns T*k rows when the buffer is larger; this library returns min(buffer, T*k) rows likewise
+      assert got_x.shape == want_x.shape
+      assert torch.equal(got_x.cpu().view(torch.int16), want_x.view(torch.int16))
+      y = torch.from_numpy(rng.standard_normal(tuple(want_x.shape)).astype(np.float32)).to(torch.bfloat16)
+      want_o = O.ring_ragged_unsort(y, want_gs, want_rev, k, e // ep, shard, w)
+      got_o = ragged_sort.ring_ragged_unsort(y.cuda(), got_gs, got_rev, k, e // ep, shard, w.cuda())
+      assert got_o.shape == want_o.shape
+      if want_o.abs().max() > 0:
+        assert relerr(got_o.float().cpu(), want_o.float()) <= 1e-2
+      else:
+        assert not got_o.any()
+
+
+def test_a2a_ragged_sort_unsort():
+  from maxtext_amd import ragged_sort
+
+  rng = np.random.default_rng(9)
+  n, d = 1000, 256
+  x = torch.from_numpy(rng.standard_normal((n, d)).astype(np.float32)).to(torch.bfloat16)
+  idx = rng.permutation(n).astype(np.int32)
+  for valid in (0, 1, 617, n):
+    want = O.a2a_ragged_sort(x, idx, valid)
+    assert torch.equal(ragged_sort.a2a_ragged_sort(x.cuda(), cuda_i32(idx), valid).cpu(), want)
+    assert torch.equal(ragged_sort.a2a_ragged_unsort(x.cuda(), cuda_i32(idx), torch.tensor(valid, device="cuda")).cpu(), want)
+  # unsort(sort(x)) restores the valid prefix when the permutation keeps it in place
+  keep = np.concatenate([rng.permutation(600), np.arange(600, n)]).astype(np.int32)
+  s = ragged_sort.a2a_ragged_sort(x.cuda(), cuda_i32(keep), 600)
+  back = ragged_sort.a2a_ragged_unsort(s, cuda_i32(np.argsort(keep).astype(np.int32)), 600)
+  assert torch.equal(back[:600].cpu(), x[:600]) and not back[600:].any()

@@ -153,3 +153,45 @@ def test_local_keys_brute_force_and_padding():
     np.testing.assert_array_equal(idx, want)
     np.testing.assert_array_equal(ids, keys[want])
     np.testing.assert_array_equal(lgs, local.sum(0))
+
+
+@pytest.mark.parametrize("buffered", [False, True])
+def test_ring_ragged_sort_unsort_row_by_row(buffered):
+  # kernels/ragged/ragged_sort.py:23-451 (forward): every sorted position that belongs to the shard's experts holds its
+  # token's row (at the same position, or packed from 0 in a small buffer, where rows beyond the buffer are dropped)
+  rng = np.random.default_rng(3)
+  t, k, e, ep, d = 23, 3, 8, 4, 4
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  x = torch.arange(t * d, dtype=torch.float32).reshape(t, d).to(torch.bfloat16) + 1
+  w = torch.from_numpy(rng.random((t, k)).astype(np.float32))
+  flat = sel.reshape(-1)
+  order = sorted(range(t * k), key=lambda i: (flat[i], i))
+  total = torch.zeros(t, d)
+  for shard in range(ep):
+    buf = 7 if buffered else None
+    xs, gs, revert = O.ring_ragged_sort(x, sel, e, k, shard, ep, buffer_size=buf)
+    np.testing.assert_array_equal(gs, np.bincount(flat, minlength=e))
+    np.testing.assert_array_equal(revert, np.argsort(np.array(order), kind="stable"))
+    mine = [p for p, i in enumerate(order) if flat[i] // (e // ep) == shard]
+    want = torch.zeros((buf if buffered else t * k, d), dtype=torch.bfloat16)
+    for slot, p in enumerate(mine):
+      if buffered and slot < buf:
+        want[slot] = x[order[p] // k]
+      elif not buffered:
+        want[p] = x[order[p] // k]
+    assert torch.equal(xs, want)
+    out = O.ring_ragged_unsort(xs, gs, revert, k, e // ep, shard, w)
+    kept = mine[:buf] if buffered else mine
+    want_out = torch.zeros(t, d)
+    for p in kept:
+      want_out[order[p] // k] += w.reshape(-1)[order[p]] * x[order[p] // k].float()
+    assert torch.allclose(out.float(), want_out.to(torch.bfloat16).float(), rtol=1e-2, atol=1e-2)
+    total += out.float()
+  if not buffered:  # nothing dropped: the shards' outputs add up to (sum of a token's weights) * x
+    assert torch.allclose(total, w.sum(1, keepdim=True) * x.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_a2a_ragged_sort_by_hand():
+  x = torch.arange(12, dtype=torch.float32).reshape(6, 2).to(torch.bfloat16)
+  out = O.a2a_ragged_sort(x, np.array([2, 0, 1, 5, 4, 3]), 3)
+  assert torch.equal(out, torch.tensor([[4, 5], [0, 1], [2, 3], [0, 0], [0, 0], [0, 0]], dtype=torch.bfloat16))
