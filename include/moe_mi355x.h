@@ -339,6 +339,12 @@ typedef struct {
 /* flags: layout of rhs_scale / rhs_up_scale, see "Operand layouts" above. */
 #define MOE_GMM_RHS_SCALE_KMAJOR 4
 #define MOE_GMM_RHS_SCALE_SHARED 8
+/* flags: the caller's promise that group_sizes holds what it held at the previous moe_gmm call on this device, that the
+ * workspace is the same buffer, untouched since, and that this call is ordered behind that one.  When that call mapped
+ * the same M, groups and tile height, its tile list is used again and the mapping launch is skipped (the second and
+ * third product of an expert layer: one launch less in a chain of dependent launches, about 4 us at decode sizes);
+ * when anything differs the list is rebuilt as usual.  The library keeps one record per device, the last call's. */
+#define MOE_GMM_SAME_GROUPS 16
 
 /* 1 when moe_gmm takes MOE_GMM_RHS_KN for this shape (K % 64 == 0, N % 256 == 0, 128 rows per group on average and
  * enough 256 x 256 tiles to fill the chip), else 0. */

@@ -22,6 +22,7 @@ MOE_GMM_KEEP_OTHER_ROWS = 1
 MOE_GMM_RHS_KN = 2
 MOE_GMM_RHS_SCALE_KMAJOR = 4
 MOE_GMM_RHS_SCALE_SHARED = 8
+MOE_GMM_SAME_GROUPS = 16
 MOE_SCALE_PER_TENSOR = -1
 GMM_KERNEL_BY_NAME = {None: 0, "auto": 0, "stream": 1, "tiled": 2, "big": 3, "dl64": 4, "stream_nosplit": 5}
 MOE_QUANT_RINT_DIV, MOE_QUANT_V2 = 0, 1

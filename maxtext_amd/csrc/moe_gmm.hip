@@ -29,6 +29,9 @@
 
 #include "moe_gmm_common.h"
 
+#include <cstring>
+#include <mutex>
+
 namespace moe {
 
 constexpr int kMapThreads = 256;
@@ -250,7 +253,22 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   const bool kmajor = (a->flags & MOE_GMM_RHS_SCALE_KMAJOR) != 0, shared = (a->flags & MOE_GMM_RHS_SCALE_SHARED) != 0;
   const int bn = a->rhs_scale_block_n, rbk = a->rhs_scale_block_k, lbk = a->lhs_scale_block_k;
   auto map_tiles = [&](int bm) {
-    tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
+    // what the last call on this device mapped, and into which buffer (MOE_GMM_SAME_GROUPS)
+    struct Mapped {
+      const void* ws; const int32_t* gs; int M, G, offset, local, bm, zero_fill;
+    };
+    static Mapped last[kMaxDevices] = {};
+    static std::mutex lock;
+    int dev = 0;
+    const bool known = current_device(&dev) == MOE_OK;
+    const Mapped now = {workspace, a->group_sizes, M, G, a->group_offset, a->num_groups_local, bm, zero_fill ? 1 : 0};
+    bool reuse = false;
+    if (known) {
+      std::lock_guard<std::mutex> hold(lock);
+      reuse = (a->flags & MOE_GMM_SAME_GROUPS) && memcmp(&last[dev], &now, sizeof(Mapped)) == 0;
+      last[dev] = now;
+    }
+    if (!reuse) tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
   };
   RowOpts ro;
   ro.row_idx = a->lhs_row_idx; ro.idx_div = a->lhs_row_idx_div < 1 ? 1 : a->lhs_row_idx_div;

@@ -352,14 +352,16 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
             group_offset=0, out=None, kernel=None, raster=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None,
             keep_other_rows=False, rhs_kn=False, rhs_scale_kmajor=False, rhs_scale_shared=False, out_dtype=torch.bfloat16,
-            lhs_row_idx=None, lhs_row_idx_div=1, out_row_scale=None, num_rows=None, workspace=None):
+            lhs_row_idx=None, lhs_row_idx_div=1, out_row_scale=None, num_rows=None, workspace=None, same_groups=False):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2]).
   rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 without rhs_up, on shapes `gmm_rhs_kn_supported` accepts).
   Scale layouts follow include/moe_mi355x.h: lhs_scale_block_k 0 = [M], -1 = [1] (per tensor), b = [M, ceil(K/b)];
   rhs scales [G, ceil(N/bn), ceil(K/bk)], or [G, ceil(K/bk), N] with rhs_scale_kmajor, without the leading G with
   rhs_scale_shared; bn = -1: one scale for all channels.
   lhs_row_idx [M] int32: row i of the product reads lhs row lhs_row_idx[i] // lhs_row_idx_div (lhs then has any number of
-  rows); out_row_scale [M] f32 multiplies the result rows.  kernel / raster select a kernel family (moe_gmm_tuned)."""
+  rows); out_row_scale [M] f32 multiplies the result rows.  kernel / raster select a kernel family (moe_gmm_tuned).
+  workspace: a caller-held uint8 buffer of moe_gmm_workspace_bytes; same_groups: MOE_GMM_SAME_GROUPS (group_sizes and the
+  workspace are those of the previous call, untouched: its tile list is used again when the tile height agrees)."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
   _need(group_sizes, "group_sizes", torch.int32, 1)
@@ -463,7 +465,8 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.partial_sum = partial_sum.data_ptr() if partial_sum is not None else None
   a.partial_sum_up = partial_sum_up.data_ptr() if partial_sum_up is not None else None
   a.flags = ((_lib.MOE_GMM_KEEP_OTHER_ROWS if keep_other_rows else 0) | (_lib.MOE_GMM_RHS_KN if rhs_kn else 0)
-             | (_lib.MOE_GMM_RHS_SCALE_KMAJOR if rhs_scale_kmajor else 0) | (_lib.MOE_GMM_RHS_SCALE_SHARED if rhs_scale_shared else 0))
+             | (_lib.MOE_GMM_RHS_SCALE_KMAJOR if rhs_scale_kmajor else 0) | (_lib.MOE_GMM_RHS_SCALE_SHARED if rhs_scale_shared else 0)
+             | (_lib.MOE_GMM_SAME_GROUPS if same_groups and workspace is not None else 0))
   code = _lib.GMM_KERNEL_BY_NAME[kernel]
   if code or raster:
     st = lib.moe_gmm_tuned(ctypes.byref(a), code, int(raster), _lib.current_stream())
@@ -471,6 +474,11 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
     st = lib.moe_gmm(ctypes.byref(a), _lib.current_stream())
   _lib.check(st, "moe_gmm")
   return out
+
+
+def gmm_workspace(m, num_groups_total, device):
+  """A tile-list buffer for moe_gmm calls on m rows and num_groups_total groups (uint8)."""
+  return torch.empty((max(_lib.load().moe_gmm_workspace_bytes(int(m), int(num_groups_total)), 16),), dtype=torch.uint8, device=device)
 
 
 def gmm_rhs_kn_supported(m, k, n, num_groups_total):

@@ -159,6 +159,8 @@ def gmm(
     bwd_quantize_dtype=None,
     lhs_row_idx=None,
     lhs_row_idx_div=1,
+    workspace=None,
+    same_groups=False,
     out_row_scale=None,
 ):
   """Grouped matmul: out[rows of group g] = lhs[rows] @ rhs[g] (ops.py:46).
@@ -220,7 +222,7 @@ def gmm(
                           rhs_bias, rhs_up_bias)
 
   common = dict(group_offset=offset, out_dtype=preferred_element_type, lhs_row_idx=lhs_row_idx, lhs_row_idx_div=lhs_row_idx_div,
-                out_row_scale=out_row_scale)
+                out_row_scale=out_row_scale, workspace=workspace, same_groups=same_groups)
   if rhs_bias is not None:
     common["rhs_bias"] = rhs_bias.float().contiguous()  # [G, N] (rhs_bias [G, 1, N] of the v2 kernel, :573)
   if partial_sum is not None:  # [m, n], added to the product before the activation (ops.py:77)

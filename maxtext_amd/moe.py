@@ -376,8 +376,11 @@ class RoutedMoE:
       inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit, lhs_quantize_dtype=q,
                            rhs_quantize_dtype=q, rhs_bias=w0_bias, rhs_up_bias=w1_bias)
       return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q, rhs_bias=wo_bias)
+    # one tile-list buffer for both products: the second reuses the first one's list when its tile height agrees
+    rows = row_idx.shape[0] if row_idx is not None else (sorted_inputs.qvalue if isinstance(sorted_inputs, QArray) else sorted_inputs).shape[0]
+    ws = kernels.gmm_workspace(rows, group_size.numel(), group_size.device)
     inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
-                         rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div)
+                         rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div, workspace=ws)
     if marks:
       marks[1].record()
     if cfg.act_quant is not None:
@@ -385,7 +388,7 @@ class RoutedMoE:
       inter = megablox.quantize_lhs(inter, cfg.act_quant, blocks=128 if cfg.act_quant == "fp8" else None)
     if marks:
       marks[2].record()
-    out = megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias)
+    out = megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias, workspace=ws, same_groups=True)
     if marks:
       marks[3].record()
       ev.append(("wi_glu", marks[0], marks[1]))

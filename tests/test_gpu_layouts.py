@@ -361,3 +361,37 @@ def test_fp8_prefill_stream_kernel_against_the_tiled_kernel_at_size(K, glu, inde
     h0 = product(rows, ws[0][0][gi], ws[0][1][gi])
     want = torch.nn.functional.silu(h0) * product(rows, ws[1][0][gi], ws[1][1][gi]) if glu else h0
     assert relerr(got[rows], want, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
+
+
+def test_same_groups_flag_reuses_or_rebuilds_the_tile_list():
+  # MOE_GMM_SAME_GROUPS: the second product of a layer runs on the first one's tile list when the tile height agrees and
+  # rebuilds it when it does not; either way the result equals that of a call with a workspace of its own, bit for bit
+  from maxtext_amd import kernels as K
+
+  g = torch.Generator(device="cuda").manual_seed(21)
+  e, d, f = 16, 256, 512
+  w_up = (torch.randn((e, f, d), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  w_gate = (torch.randn((e, f, d), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  w_down = (torch.randn((e, d, f), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  w_down_q = torch.randint(-127, 128, (e, d, f), generator=g, device="cuda", dtype=torch.int8)
+  w_down_s = torch.rand((e, d), generator=g, device="cuda") * 0.01
+  for m, sizes in ((40, [7, 0, 12, 1, 20] + [0] * 11), (4096, [256] * 16), (1500, [100, 0, 300, 37, 63] + [100] * 10)):
+    gs = torch.tensor(sizes, dtype=torch.int32, device="cuda")
+    x = torch.randn((m, d), generator=g, device="cuda").to(torch.bfloat16)
+    ws = K.gmm_workspace(m, e, "cuda")
+    h = K.gmm_raw(x, w_gate, gs, rhs_up=w_up, act="silu", workspace=ws)
+    # same tile height (bf16 x bf16 twice)
+    y = K.gmm_raw(h, w_down, gs, workspace=ws, same_groups=True)
+    assert torch.equal(y, K.gmm_raw(h, w_down, gs))
+    # the weight-only format may take another tile height (streaming kernel below 16 rows per expert): list rebuilt
+    yq = K.gmm_raw(h, w_down_q, gs, rhs_scale=w_down_s, workspace=ws, same_groups=True)
+    assert torch.equal(yq, K.gmm_raw(h, w_down_q, gs, rhs_scale=w_down_s))
+    # and back, still promising the same groups
+    y2 = K.gmm_raw(h, w_down, gs, workspace=ws, same_groups=True)
+    assert torch.equal(y2, y)
+    # new group sizes in the same tensor: a call without the flag maps them, the flagged call behind it may reuse that
+    gs.copy_(torch.tensor(list(reversed(sizes)), dtype=torch.int32))
+    h2 = K.gmm_raw(x, w_gate, gs, rhs_up=w_up, act="silu", workspace=ws)
+    y3 = K.gmm_raw(h2, w_down, gs, workspace=ws, same_groups=True)
+    assert torch.equal(h2, K.gmm_raw(x, w_gate, gs, rhs_up=w_up, act="silu"))
+    assert torch.equal(y3, K.gmm_raw(h2, w_down, gs))
