@@ -138,6 +138,16 @@ MOE_API int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int
 MOE_API int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
                        int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                        void* workspace, size_t workspace_bytes, void* stream);
+/* The same, and for up to 4096 routed rows (one launch) the block that sorted also builds the m-tile list of the
+ * grouped matmuls that follow: gmm_workspace (moe_gmm_workspace_bytes(T * k, E) bytes) then holds the list for tiles of
+ * tile_rows rows over these group_sizes with the given num_groups_local / group_offset / MOE_GMM_KEEP_OTHER_ROWS setting,
+ * and a moe_gmm call on that workspace and the group_sizes buffer written here, flagged MOE_GMM_SAME_GROUPS, skips its
+ * own mapping launch when it picks that tile height (16 for the streaming kernels of decode-sized calls; any other
+ * choice rebuilds the list).  Above 4096 rows nothing is mapped and moe_gmm maps as usual. */
+MOE_API int moe_sort_by_expert_mapped(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+                       int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, int tile_rows, int num_groups_local, int group_offset,
+                       int keep_other_rows, void* gmm_workspace, size_t gmm_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Expert-parallel dispatch bookkeeping on one expert shard (integer work on device-resident sizes; the exchange

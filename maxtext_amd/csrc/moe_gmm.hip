@@ -36,78 +36,33 @@ namespace moe {
 
 constexpr int kMapThreads = 256;
 
-__device__ __forceinline__ int block_exclusive_scan(int v, int* s_buf, int* total) {
-  const int tid = threadIdx.x;
-  s_buf[tid] = v;
-  __syncthreads();
-  for (int o = 1; o < kMapThreads; o <<= 1) {
-    int add = tid >= o ? s_buf[tid - o] : 0;
-    __syncthreads();
-    s_buf[tid] += add;
-    __syncthreads();
-  }
-  int incl = s_buf[tid];
-  *total = s_buf[kMapThreads - 1];
-  __syncthreads();
-  return incl - v;
-}
-
 __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
     const int32_t* __restrict__ group_sizes, int G_total, int group_offset, int G_local, int M,
     int BM, int zero_fill, int32_t* __restrict__ header, TileInfo* __restrict__ tiles) {
   __shared__ int s_buf[kMapThreads];
-  const int tid = threadIdx.x;
-  const int per = (G_total + kMapThreads - 1) / kMapThreads;
-  const int g0 = min(tid * per, G_total), g1 = min(g0 + per, G_total);
-  long long rows = 0;
-  for (int g = g0; g < g1; g++) rows += max(group_sizes[g], 0);
-  int total_rows;
-  int row_prefix = block_exclusive_scan((int)min(rows, (long long)M), s_buf, &total_rows);
-  // clipped extents (reference_gmm: end = min(start + size, m)) and tile counts
-  int ntiles = 0;
-  {
-    long long start = row_prefix;
-    for (int g = g0; g < g1; g++) {
-      long long end = start + max(group_sizes[g], 0);
-      int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
-      const int local = g - group_offset;
-      // rows of groups held elsewhere get zero-fill tiles, or none at all when the caller keeps what `out` holds
-      if (zero_fill || (local >= 0 && local < G_local)) ntiles += (e - s + BM - 1) / BM;
-      start = end;
-    }
-  }
-  int total_tiles;
-  int tile_prefix = block_exclusive_scan(ntiles, s_buf, &total_tiles);
-  {
-    long long start = row_prefix;
-    int ti = tile_prefix;
-    for (int g = g0; g < g1; g++) {
-      long long end = start + max(group_sizes[g], 0);
-      int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
-      int local = g - group_offset;
-      int kind = (local >= 0 && local < G_local) ? local : -1;
-      for (int r = s; r < e && (zero_fill || kind >= 0); r += BM) {
-        TileInfo t;
-        t.group = kind;
-        t.row0 = r;
-        t.nrows = min(BM, e - r);
-        t.pad = 0;
-        tiles[ti++] = t;
-      }
-      start = end;
-    }
-  }
-  const int covered = min(total_rows, M);
-  const int tail = zero_fill ? (M - covered + BM - 1) / BM : 0;
-  for (int i = tid; i < tail; i += kMapThreads) {
-    TileInfo t;
-    t.group = -1;
-    t.row0 = covered + i * BM;
-    t.nrows = min(BM, M - t.row0);
-    t.pad = 0;
-    tiles[total_tiles + i] = t;
-  }
-  if (tid == 0) header[0] = total_tiles + tail;
+  build_tile_map<kMapThreads>(group_sizes, G_total, group_offset, G_local, M, BM, zero_fill, header, tiles, s_buf);
+}
+
+// What the last call on a device mapped, and into which buffer (MOE_GMM_SAME_GROUPS).
+struct Mapped {
+  const void* ws; const int32_t* gs; int M, G, offset, local, bm, zero_fill;
+};
+static Mapped g_last_map[kMaxDevices] = {};
+static std::mutex g_last_map_lock;
+
+// Records `now` as the device's current tile list; returns whether the list it replaces was the same one.
+static bool note_tile_map(const Mapped& now) {
+  int dev = 0;
+  if (current_device(&dev) != MOE_OK) return false;
+  std::lock_guard<std::mutex> hold(g_last_map_lock);
+  const bool same = memcmp(&g_last_map[dev], &now, sizeof(Mapped)) == 0;
+  g_last_map[dev] = now;
+  return same;
+}
+
+void note_tile_map_built(const void* workspace, const int32_t* group_sizes, int M, int G_total, int group_offset, int G_local, int bm,
+                         int zero_fill) {
+  note_tile_map(Mapped{workspace, group_sizes, M, G_total, group_offset, G_local, bm, zero_fill ? 1 : 0});
 }
 
 // Tile list of moe_gmm_static_ws: one array per device, held until the process ends.  Its name is a host-side handle,
@@ -253,22 +208,9 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   const bool kmajor = (a->flags & MOE_GMM_RHS_SCALE_KMAJOR) != 0, shared = (a->flags & MOE_GMM_RHS_SCALE_SHARED) != 0;
   const int bn = a->rhs_scale_block_n, rbk = a->rhs_scale_block_k, lbk = a->lhs_scale_block_k;
   auto map_tiles = [&](int bm) {
-    // what the last call on this device mapped, and into which buffer (MOE_GMM_SAME_GROUPS)
-    struct Mapped {
-      const void* ws; const int32_t* gs; int M, G, offset, local, bm, zero_fill;
-    };
-    static Mapped last[kMaxDevices] = {};
-    static std::mutex lock;
-    int dev = 0;
-    const bool known = current_device(&dev) == MOE_OK;
-    const Mapped now = {workspace, a->group_sizes, M, G, a->group_offset, a->num_groups_local, bm, zero_fill ? 1 : 0};
-    bool reuse = false;
-    if (known) {
-      std::lock_guard<std::mutex> hold(lock);
-      reuse = (a->flags & MOE_GMM_SAME_GROUPS) && memcmp(&last[dev], &now, sizeof(Mapped)) == 0;
-      last[dev] = now;
-    }
-    if (!reuse) tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
+    const bool same = note_tile_map(Mapped{workspace, a->group_sizes, M, G, a->group_offset, a->num_groups_local, bm, zero_fill ? 1 : 0});
+    if (!(same && (a->flags & MOE_GMM_SAME_GROUPS)))
+      tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
   };
   RowOpts ro;
   ro.row_idx = a->lhs_row_idx; ro.idx_div = a->lhs_row_idx_div < 1 ? 1 : a->lhs_row_idx_div;

@@ -18,6 +18,89 @@ struct TileInfo {
 // workspace: int32 header[4] (header[0] = number of tiles) | TileInfo tiles[max_tiles]
 static inline int max_tiles_for(int M, int G, int bm) { return cdiv(M, bm) + G + 1; }
 
+// Exclusive prefix sum over one value per thread of a THREADS-wide block; *total = the block's sum.
+template <int THREADS>
+__device__ __forceinline__ int block_exclusive_scan(int v, int* s_buf, int* total) {
+  const int tid = threadIdx.x;
+  s_buf[tid] = v;
+  __syncthreads();
+  for (int o = 1; o < THREADS; o <<= 1) {
+    int add = tid >= o ? s_buf[tid - o] : 0;
+    __syncthreads();
+    s_buf[tid] += add;
+    __syncthreads();
+  }
+  int incl = s_buf[tid];
+  *total = s_buf[THREADS - 1];
+  __syncthreads();
+  return incl - v;
+}
+
+// group_sizes (device) -> the list of (group, first row, rows) m-tiles of height BM that never straddle a group boundary,
+// plus zero-fill tiles for the rows of groups held elsewhere and the rows past the groups' total; header[0] = tile count.
+// One block of THREADS threads; s_buf holds THREADS ints.
+template <int THREADS>
+__device__ __forceinline__ void build_tile_map(const int32_t* __restrict__ group_sizes, int G_total, int group_offset, int G_local, int M,
+                                               int BM, int zero_fill, int32_t* __restrict__ header, TileInfo* __restrict__ tiles, int* s_buf) {
+  const int tid = threadIdx.x;
+  const int per = (G_total + THREADS - 1) / THREADS;
+  const int g0 = min(tid * per, G_total), g1 = min(g0 + per, G_total);
+  long long rows = 0;
+  for (int g = g0; g < g1; g++) rows += max(group_sizes[g], 0);
+  int total_rows;
+  int row_prefix = block_exclusive_scan<THREADS>((int)min(rows, (long long)M), s_buf, &total_rows);
+  // clipped extents (reference_gmm: end = min(start + size, m)) and tile counts
+  int ntiles = 0;
+  {
+    long long start = row_prefix;
+    for (int g = g0; g < g1; g++) {
+      long long end = start + max(group_sizes[g], 0);
+      int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
+      const int local = g - group_offset;
+      // rows of groups held elsewhere get zero-fill tiles, or none at all when the caller keeps what `out` holds
+      if (zero_fill || (local >= 0 && local < G_local)) ntiles += (e - s + BM - 1) / BM;
+      start = end;
+    }
+  }
+  int total_tiles;
+  int tile_prefix = block_exclusive_scan<THREADS>(ntiles, s_buf, &total_tiles);
+  {
+    long long start = row_prefix;
+    int ti = tile_prefix;
+    for (int g = g0; g < g1; g++) {
+      long long end = start + max(group_sizes[g], 0);
+      int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
+      int local = g - group_offset;
+      int kind = (local >= 0 && local < G_local) ? local : -1;
+      for (int r = s; r < e && (zero_fill || kind >= 0); r += BM) {
+        TileInfo t;
+        t.group = kind;
+        t.row0 = r;
+        t.nrows = min(BM, e - r);
+        t.pad = 0;
+        tiles[ti++] = t;
+      }
+      start = end;
+    }
+  }
+  const int covered = min(total_rows, M);
+  const int tail = zero_fill ? (M - covered + BM - 1) / BM : 0;
+  for (int i = tid; i < tail; i += THREADS) {
+    TileInfo t;
+    t.group = -1;
+    t.row0 = covered + i * BM;
+    t.nrows = min(BM, M - t.row0);
+    t.pad = 0;
+    tiles[total_tiles + i] = t;
+  }
+  if (tid == 0) header[0] = total_tiles + tail;
+}
+
+// Tells moe_gmm that `workspace` holds the tile list of these groups at height bm (built by another entry point of the
+// library), so that a call flagged MOE_GMM_SAME_GROUPS can use it.
+void note_tile_map_built(const void* workspace, const int32_t* group_sizes, int M, int G_total, int group_offset, int G_local, int bm,
+                         int zero_fill);
+
 // m-tiles per super-row of the persistent kernels' tile order (the tiles an XCD works on at a time are a patch of one
 // super-row's m-tiles x a few n-tiles): as many as a group of average size plus three standard deviations of a
 // multinomial draw has, so that a patch mostly stays inside one group and shares its weight panels; 8 for larger groups.

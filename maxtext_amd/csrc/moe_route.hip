@@ -8,7 +8,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 
-#include "moe_common.h"
+#include "moe_gmm_common.h"
 
 namespace moe {
 
@@ -425,10 +425,17 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
 // All three passes in one block of NW waves for at most NW * kSortSeg entries (decode and small prefill: a launch costs
 // as much as a pass; NW = 4 up to 1024 entries, 16 up to 4096): per-wave histograms in LDS, the prefixes over the
 // segments and over the experts, then the same in-order ranking.
+// The m-tile list of the grouped matmuls that follow, built behind the sort by the same block (tiles == NULL: not wanted).
+struct SortMapArgs {
+  TileInfo* tiles;
+  int32_t* header;
+  int G_local, group_offset, BM, zero_fill;
+};
+
 template <int NW>
 __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
     const int32_t* __restrict__ flat, int M, int E, int roll, int ebits, int32_t* __restrict__ group_sizes,
-    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts) {
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts, const SortMapArgs mp) {
   __shared__ int run[NW][kSortMaxE];
   __shared__ int off[kSortMaxE];
   constexpr int NT = NW * kWave;
@@ -494,6 +501,10 @@ __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
       if (inv_perm) inv_perm[i] = dest;
       if (sorted_experts) sorted_experts[dest] = e;
     }
+  }
+  if (mp.tiles) {
+    __syncthreads();  // group_sizes, written above by this block, are read back from memory
+    build_tile_map<NT>(group_sizes, E, mp.group_offset, mp.G_local, M, mp.BM, mp.zero_fill, mp.header, mp.tiles, &run[0][0]);
   }
 }
 
@@ -976,9 +987,9 @@ size_t moe_sort_workspace_bytes(int T, int k, int E) {
   return (nseg * E + E) * sizeof(int32_t) + 256;
 }
 
-int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
-                              int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
-                              void* workspace, size_t workspace_bytes, void* stream) {
+static int sort_impl(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+                     int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                     void* workspace, size_t workspace_bytes, const SortMapArgs& mp, bool* mapped, void* stream) {
   if (!topk_idx || !perm || !group_sizes || !workspace) return fail(MOE_ERR_INVALID_ARG, "sort: NULL pointer");
   if (T < 0 || k <= 0 || E <= 0) return fail(MOE_ERR_INVALID_ARG, "sort: bad sizes");
   if (E > kSortMaxE) return fail(MOE_ERR_UNSUPPORTED, "sort: E=%d > %d", E, kSortMaxE);
@@ -994,11 +1005,13 @@ int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int 
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
   if (nblk <= 1) {  // also M == 0: group_sizes are all zero
-    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
+    *mapped = mp.tiles != nullptr;
     return check_launch("sort_by_expert");
   }
   if (nblk <= 4) {  // up to 4096 entries: still one launch, with 16 waves
-    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts);
+    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
+    *mapped = mp.tiles != nullptr;
     return check_launch("sort_by_expert");
   }
   if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, seg_hist);
@@ -1007,6 +1020,32 @@ int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int 
     sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, seg_hist, group_sizes,
                                                           perm, inv_perm, sorted_experts);
   return check_launch("sort_by_expert");
+}
+
+int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+                              int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  bool mapped = false;
+  return sort_impl(topk_idx, T, k, E, roll_to_expert_id, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes,
+                   SortMapArgs{nullptr, nullptr, 0, 0, 0, 0}, &mapped, stream);
+}
+
+int moe_sort_by_expert_mapped(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+                              int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                              void* workspace, size_t workspace_bytes, int tile_rows, int num_groups_local, int group_offset,
+                              int keep_other_rows, void* gmm_workspace, size_t gmm_workspace_bytes, void* stream) {
+  if (!gmm_workspace) return fail(MOE_ERR_INVALID_ARG, "sort: NULL gmm_workspace");
+  if (tile_rows <= 0 || num_groups_local <= 0 || group_offset < 0) return fail(MOE_ERR_INVALID_ARG, "sort: bad tile list arguments");
+  const long long M = (long long)T * k;
+  if (T >= 0 && k > 0 && M <= INT_MAX / 2 && gmm_workspace_bytes < moe_gmm_workspace_bytes((int)M, E))
+    return fail(MOE_ERR_WORKSPACE, "sort: gmm_workspace too small");
+  const int zero_fill = keep_other_rows ? 0 : 1;
+  const SortMapArgs mp = {(TileInfo*)((uint8_t*)gmm_workspace + 16), (int32_t*)gmm_workspace, num_groups_local, group_offset, tile_rows, zero_fill};
+  bool mapped = false;
+  const int st = sort_impl(topk_idx, T, k, E, roll_to_expert_id, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes, mp,
+                           &mapped, stream);
+  if (st == MOE_OK && mapped) note_tile_map_built(gmm_workspace, group_sizes, (int)M, E, group_offset, num_groups_local, tile_rows, zero_fill);
+  return st;
 }
 
 int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,

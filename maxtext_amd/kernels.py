@@ -90,9 +90,11 @@ def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_r
   return (w, idx, logits, pre) if return_logits else (w, idx)
 
 
-def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True, roll_to_expert_id=0):
+def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True, roll_to_expert_id=0, gmm_workspace=None, tile_rows=16):
   """-> (perm [M], inv_perm [M], group_sizes [E], sorted_experts [M] or None), all int32.
-  roll_to_expert_id: the ids are sorted as (id - roll_to_expert_id) mod num_experts (moe.py:953-954)."""
+  roll_to_expert_id: the ids are sorted as (id - roll_to_expert_id) mod num_experts (moe.py:953-954).
+  gmm_workspace (from gmm_workspace(M, num_experts)): up to 4096 routed rows the sort also leaves the grouped matmuls'
+  tile list of height tile_rows there, which gmm_raw(..., workspace=gmm_workspace, same_groups=True) then uses."""
   _need(topk_idx, "topk_idx", torch.int32, 2)
   t, k = topk_idx.shape
   m = t * k
@@ -104,6 +106,12 @@ def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True, roll_to_e
   se = torch.empty((m,), dtype=torch.int32, device=dev) if want_sorted_experts else None
   nbytes = lib.moe_sort_workspace_bytes(t, k, num_experts)
   ws = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=dev)
+  if gmm_workspace is not None:
+    st = lib.moe_sort_by_expert_mapped(_lib.ptr(topk_idx), t, k, num_experts, int(roll_to_expert_id), _lib.ptr(perm), _lib.ptr(inv),
+                                       _lib.ptr(gs), _lib.ptr(se), _lib.ptr(ws), ws.numel(), int(tile_rows), num_experts, 0, 0,
+                                       _lib.ptr(gmm_workspace), gmm_workspace.numel(), _lib.current_stream())
+    _lib.check(st, "moe_sort_by_expert_mapped")
+    return perm, inv, gs, se
   st = lib.moe_sort_by_expert_rolled(_lib.ptr(topk_idx), t, k, num_experts, int(roll_to_expert_id), _lib.ptr(perm), _lib.ptr(inv),
                                      _lib.ptr(gs), _lib.ptr(se), _lib.ptr(ws), ws.numel(), _lib.current_stream())
   _lib.check(st, "moe_sort_by_expert_rolled")

@@ -355,7 +355,8 @@ class RoutedMoE:
     return out.reshape(batch_size, sequence_length, -1)
 
   # -- the three grouped GEMMs: gmm_up + apply_ffn_activation + wo (moe.py:1932-1986, :841, :2226)
-  def _experts(self, sorted_inputs, group_size, w0, w1, wo, w0_bias=None, w1_bias=None, wo_bias=None, row_idx=None, row_idx_div=1):
+  def _experts(self, sorted_inputs, group_size, w0, w1, wo, w0_bias=None, w1_bias=None, wo_bias=None, row_idx=None, row_idx_div=1,
+               workspace=None):
     """row_idx / row_idx_div: `sorted_inputs` holds the T token rows (plain or quantised) and row i of the first product
     reads row row_idx[i] // row_idx_div of it: the permute fused into the matmul, no [M, d] copy."""
     cfg = self.config
@@ -378,9 +379,11 @@ class RoutedMoE:
       return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q, rhs_bias=wo_bias)
     # one tile-list buffer for both products: the second reuses the first one's list when its tile height agrees
     rows = row_idx.shape[0] if row_idx is not None else (sorted_inputs.qvalue if isinstance(sorted_inputs, QArray) else sorted_inputs).shape[0]
-    ws = kernels.gmm_workspace(rows, group_size.numel(), group_size.device)
+    # (`workspace`: one the sort already left a tile list in, for these group sizes)
+    ws = workspace if workspace is not None else kernels.gmm_workspace(rows, group_size.numel(), group_size.device)
     inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
-                         rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div, workspace=ws)
+                         rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div, workspace=ws,
+                         same_groups=workspace is not None)
     if marks:
       marks[1].record()
     if cfg.act_quant is not None:
@@ -407,8 +410,10 @@ class RoutedMoE:
     x2d = inputs.reshape(b * s, d).contiguous()
     weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
     x2d = self._scale_inputs_by_router_score(x2d, weights)
+    # decode-sized calls: the sort leaves the tile list of the streaming matmul kernels (16-row tiles) behind, one launch less
+    ws = kernels.gmm_workspace(b * s * k, self.num_experts, x2d.device) if b * s * k <= 4096 else None
     perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
-                                                      want_sorted_experts=False)
+                                                      want_sorted_experts=False, gmm_workspace=ws)
     training = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (x2d, weights, w0_kernel, w1_kernel, wo_kernel))
     if training:
@@ -418,7 +423,7 @@ class RoutedMoE:
       # the permute is fused into the first grouped matmul: the T token rows are quantised once (not their M = T * k
       # copies) and the matmul reads row perm[i] // k for its row i, so the [M, d] gathered copy is never written
       inter = self._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias,
-                            row_idx=perm, row_idx_div=k)
+                            row_idx=perm, row_idx_div=k, workspace=ws)
     out = self.unpermute(inter, perm, weights, b, s, inv_perm=inv)
     lb_loss, bias_updates = self._aux_outputs(gate_logits, selected.reshape(b, s, k))
     return out, lb_loss, bias_updates
@@ -487,8 +492,9 @@ class RoutedAndSharedMoE:
     shared_ids = torch.arange(e, e + sh, dtype=torch.int32, device=sel.device).expand(t, sh)
     sel = torch.cat([sel.reshape(t, k), shared_ids], 1).contiguous()
     w = torch.cat([w.reshape(t, k).float(), torch.ones((t, sh), dtype=torch.float32, device=w.device)], 1).contiguous()
-    perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + sh, want_sorted_experts=False)
-    inter = r._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, r.wi_0, r.wi_1, r.wo, row_idx=perm, row_idx_div=k + sh)
+    ws = kernels.gmm_workspace(t * (k + sh), e + sh, x2d.device) if t * (k + sh) <= 4096 else None
+    perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + sh, want_sorted_experts=False, gmm_workspace=ws)
+    inter = r._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, r.wi_0, r.wi_1, r.wo, row_idx=perm, row_idx_div=k + sh, workspace=ws)
     out = kernels.unpermute_combine(inter, w, k=k + sh, inv_perm=inv)
     lb_loss, bias_updates = r._aux_outputs(gate_logits, routed_sel)
     return out.reshape(b, s, d), lb_loss, bias_updates

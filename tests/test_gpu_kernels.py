@@ -1515,3 +1515,30 @@ def test_route_sort_combine_single_token(K):
   y = K.unpermute_combine(rows, w, k=2, perm=perm, inv_perm=inv)
   want = (x.float() * float(w.sum())).to(torch.bfloat16)
   assert relerr(y, want) <= TOL
+
+
+@pytest.mark.parametrize("t,e,k", [(1, 32, 4), (16, 32, 4), (128, 32, 4), (256, 256, 8), (1024, 8, 2), (1025, 8, 4)])
+def test_sort_leaves_the_tile_list_for_the_matmuls(K, t, e, k):
+  # moe_sort_by_expert_mapped: same sort results; the grouped matmul that follows on the same workspace, flagged
+  # MOE_GMM_SAME_GROUPS, gives the result of a call that maps for itself (bit for bit), whether it picks 16-row tiles
+  # (weight-only int8 at decode sizes) or another height (bf16: list rebuilt); above 4096 rows nothing is mapped
+  rng = np.random.default_rng(t + e)
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  m = t * k
+  ws = K.gmm_workspace(m, e, "cuda")
+  perm, inv, gs, se = K.sort_by_expert(cuda(sel), e, gmm_workspace=ws)
+  perm0, inv0, gs0, se0 = K.sort_by_expert(cuda(sel), e)
+  for a, b in ((perm, perm0), (inv, inv0), (gs, gs0), (se, se0)):
+    assert torch.equal(a, b)
+  g = torch.Generator(device="cuda").manual_seed(t)
+  d, f = 128, 256
+  x = torch.randn((m, d), generator=g, device="cuda").to(torch.bfloat16)
+  wq = torch.randint(-127, 128, (e, f, d), generator=g, device="cuda", dtype=torch.int8)
+  sc = torch.rand((e, f), generator=g, device="cuda") * 0.01
+  wb = (torch.randn((e, f, d), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  y = K.gmm_raw(x, wq, gs, rhs_scale=sc, workspace=ws, same_groups=True)
+  assert torch.equal(y, K.gmm_raw(x, wq, gs0, rhs_scale=sc))
+  yb = K.gmm_raw(x, wb, gs, workspace=ws, same_groups=True)
+  assert torch.equal(yb, K.gmm_raw(x, wb, gs0))
+  y2 = K.gmm_raw(x, wq, gs, rhs_scale=sc, workspace=ws, same_groups=True)
+  assert torch.equal(y2, y)
