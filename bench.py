@@ -124,11 +124,11 @@ def dominant_kernel_model(wl, group_sizes):
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name="gmm_wq_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="bf16")
   op = "int8" if cfg.act_quant == "int8" else "bf16"
-  big = rows >= 128 * len(group_sizes)  # the dispatch rule of moe_gmm for its persistent 256 x 256 kernels
+  # the dispatch rule of moe_gmm for its persistent 256 x 256 kernels: 128 rows per expert on average (104 weight-only)
   if cfg.act_quant == "int8" or wl.weight_quant in (None, "bf16"):
-    kernel = "gmm_dls_kernel" if big else "gmm_tiled_kernel"
+    kernel = "gmm_dls_kernel" if rows >= 128 * len(group_sizes) else "gmm_tiled_kernel"
   else:
-    kernel = "gmm_dlw_kernel" if big and d % 64 == 0 else "gmm_tiled_kernel"
+    kernel = "gmm_dlw_kernel" if rows >= 104 * len(group_sizes) and d % 64 == 0 else "gmm_tiled_kernel"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
               name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype=op)
 

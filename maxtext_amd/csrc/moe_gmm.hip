@@ -112,7 +112,12 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // full 256-row tiles for prefill, 64 otherwise; a problem with fewer 256 x 256 tiles than half the CUs of the chip also
   // takes the 64-row tiles, which quadruples its blocks
   const long long tiles_big = (long long)max_tiles_for(M, G_total, 256) * cdiv(N, glu ? 128 : 256);
-  const bool big = (long long)M >= 128LL * G_total && tiles_big >= 128;
+  const bool dlw_ok = bsrc != BSRC_SAME && dlw_takes(K, N, indexed_lhs_rows, wq_kmajor);
+  // 256-row tiles from 128 rows per expert on average, where half of the routed groups no longer fit a 128-row tile (int8
+  // x int8 on the Qwen3 shape: 0.106 against 0.126 ms at 112 rows, 0.133 against 0.131 at 128); the weight-only stream
+  // kernel already from 104, its alternative being the register-staged 128-row tiles (GPT-OSS layer at 96 / 112 rows per
+  // expert: 0.42 / 0.49 ms on 128-row tiles, 0.44 / 0.44 on the stream kernel; with Zipf routing it leads from 70 on)
+  const bool big = (long long)M >= (dlw_ok ? 104LL : 128LL) * G_total && tiles_big >= 128;
   // 32 to 128 rows per expert on average: 128-row tiles; below 32, 64-row tiles.  With routed groups of near-equal size
   // the 64-row tiles are 5-10 % ahead up to 56 rows per expert (GPT-OSS shape, 384 tokens: 0.38 against 0.41 ms for the
   // layer) and collapse at 64, where half of the groups need a second tile (0.57 against 0.41 ms); with skewed routing
@@ -120,7 +125,6 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // against 0.26 ms at 56).  The weight-only shapes whose direct-to-LDS kernel does not apply follow the same rule:
   // their 256-row register-staged tiles pass the 128-row ones at 128 rows per expert as well.
   const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
-  const bool dlw_ok = bsrc != BSRC_SAME && dlw_takes(K, N, indexed_lhs_rows, wq_kmajor);
   const int esz = op == OP_I8 ? 1 : 2;
   if (mid) return K_T128;
   if (big && dlw_ok) return K_DLW;
