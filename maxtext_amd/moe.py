@@ -411,7 +411,8 @@ class RoutedMoE:
     weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
     x2d = self._scale_inputs_by_router_score(x2d, weights)
     # decode-sized calls: the sort leaves the tile list of the streaming matmul kernels (16-row tiles) behind, one launch less
-    ws = kernels.gmm_workspace(b * s * k, self.num_experts, x2d.device) if b * s * k <= 4096 else None
+    # (up to 16 rows per expert on average, where moe_gmm takes those kernels, and 4096 rows, the sort's one-launch limit)
+    ws = kernels.gmm_workspace(b * s * k, self.num_experts, x2d.device) if b * s * k <= min(4096, 16 * self.num_experts) else None
     perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
                                                       want_sorted_experts=False, gmm_workspace=ws)
     training = torch.is_grad_enabled() and any(
@@ -492,7 +493,7 @@ class RoutedAndSharedMoE:
     shared_ids = torch.arange(e, e + sh, dtype=torch.int32, device=sel.device).expand(t, sh)
     sel = torch.cat([sel.reshape(t, k), shared_ids], 1).contiguous()
     w = torch.cat([w.reshape(t, k).float(), torch.ones((t, sh), dtype=torch.float32, device=w.device)], 1).contiguous()
-    ws = kernels.gmm_workspace(t * (k + sh), e + sh, x2d.device) if t * (k + sh) <= 4096 else None
+    ws = kernels.gmm_workspace(t * (k + sh), e + sh, x2d.device) if t * (k + sh) <= min(4096, 16 * (e + sh)) else None
     perm, inv, group_size, _ = kernels.sort_by_expert(sel, e + sh, want_sorted_experts=False, gmm_workspace=ws)
     inter = r._experts(_quantize_tokens(x2d, cfg.act_quant), group_size, r.wi_0, r.wi_1, r.wo, row_idx=perm, row_idx_div=k + sh, workspace=ws)
     out = kernels.unpermute_combine(inter, w, k=k + sh, inv_perm=inv)
