@@ -115,7 +115,7 @@ def dominant_kernel_model(wl, group_sizes):
     io_bytes = rows * d * 1.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name="gmm_fp8_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")
-  if wl.weight_quant in ("int4", "mxfp4") and rows <= (36 if wl.weight_quant == "int4" else 32) * cfg.num_experts:
+  if wl.weight_quant in ("int4", "mxfp4") and rows <= 32 * cfg.num_experts:
     # weight-only 4-bit decode (the dispatch rule of moe_gmm for its streaming kernel): bound by streaming the weights of
     # the experts that were hit
     w_bytes = nonempty * 2.0 * d * f * 0.5
@@ -128,7 +128,9 @@ def dominant_kernel_model(wl, group_sizes):
   if cfg.act_quant == "int8" or wl.weight_quant in (None, "bf16"):
     kernel = "gmm_dls_kernel" if rows >= 128 * len(group_sizes) else "gmm_tiled_kernel"
   else:
-    kernel = "gmm_dlw_kernel" if rows >= 104 * len(group_sizes) and d % 64 == 0 else "gmm_tiled_kernel"
+    # (int8 / int4 also below, on 128-row tiles, down to 16 rows per expert; MXFP4 stays on the register-staged tiles there)
+    on_stream = rows >= (104 if wl.weight_quant == "mxfp4" else 16) * len(group_sizes)
+    kernel = "gmm_dlw_kernel" if on_stream and d % 64 == 0 else "gmm_tiled_kernel"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
               name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype=op)
 

@@ -14,7 +14,8 @@
 //                     consecutive tiles as one stream.  gmm_dl_kernel (moe_gmm_dl.hip) is its predecessor, kept for the
 //                     shapes the stream kernel does not take and for [G, K, N] weights.
 //   gmm_dlw_kernel    the same stream for bf16 activations x int8 / int4 / mxfp4 weights (moe_gmm_dlw.hip): raw weight
-//                     bytes through LDS, widened by the wave that multiplies them.
+//                     bytes through LDS, widened by the wave that multiplies them; on 128-row tiles (half of the row tiles
+//                     multiplied) for int8 / int4 between the streaming kernel's range and prefill-sized groups.
 //   gmm_f8s_kernel    the same stream for block-scaled fp8 (moe_gmm_f8s.hip): scales staged through LDS.
 //   gmm_fp8_skinny_kernel  block-scaled fp8 for few rows per expert (decode): no LDS, every wave
 //                     streams 16 weight rows through v_mfma_f32_16x16x128_f8f6f4 and applies the
@@ -106,7 +107,7 @@ static int scratch_of(void** ptr) {
 
 // Which kernel family takes a shape (rows per expert on average decide the m-tile) and its m-tile: one decision for the
 // tile map and for the launch.
-enum TiledKind { K_T64, K_T128, K_T256, K_DL128, K_DL64, K_DLW };
+enum TiledKind { K_T64, K_T128, K_T256, K_DL128, K_DL64, K_DLW, K_DLW128 };
 
 static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N, int G_total, bool wq_kmajor = false, long long indexed_lhs_rows = 0) {
   // full 256-row tiles for prefill, 64 otherwise; a problem with fewer 256 x 256 tiles than half the CUs of the chip also
@@ -117,7 +118,9 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // x int8 on the Qwen3 shape: 0.106 against 0.126 ms at 112 rows, 0.133 against 0.131 at 128); the weight-only stream
   // kernel already from 104, its alternative being the register-staged 128-row tiles (GPT-OSS layer at 96 / 112 rows per
   // expert: 0.42 / 0.49 ms on 128-row tiles, 0.44 / 0.44 on the stream kernel; with Zipf routing it leads from 70 on)
-  const bool big = (long long)M >= (dlw_ok ? 104LL : 128LL) * G_total && tiles_big >= 128;
+  // (int8 / int4 weights: from 112, their 128-row alternative being the same stream kernel on half-height tiles, see below:
+  // GPT-OSS int4 layer at 104 / 112 rows per expert 0.38 / 0.45 ms on those, 0.44 / 0.44 on 256-row tiles)
+  const bool big = (long long)M >= (dlw_ok ? (bsrc == BSRC_MX4 ? 104LL : 112LL) : 128LL) * G_total && tiles_big >= 128;
   // 32 to 128 rows per expert on average: 128-row tiles; below 32, 64-row tiles.  With routed groups of near-equal size
   // the 64-row tiles are 5-10 % ahead up to 56 rows per expert (GPT-OSS shape, 384 tokens: 0.38 against 0.41 ms for the
   // layer) and collapse at 64, where half of the groups need a second tile (0.57 against 0.41 ms); with skewed routing
@@ -126,6 +129,14 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // their 256-row register-staged tiles pass the 128-row ones at 128 rows per expert as well.
   const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
   const int esz = op == OP_I8 ? 1 : 2;
+  // weight-only int8 / int4 between the streaming kernel's range and the 256-row tiles: the stream kernel on 128-row tiles
+  // (half of its row tiles multiplied, nothing fetched for the other half) is 10-15 % ahead of the register-staged 128-row
+  // tiles (GPT-OSS int4 layer at 40 to 96 rows per expert 0.36-0.37 against 0.40-0.42 ms, Qwen3 int8 with Zipf routing at
+  // 20 to 80 rows 0.14-0.21 against 0.15-0.25 ms) and level with the 64-row ones at 16 to 32; MXFP4 stays on the
+  // register-staged tiles, which are 4 % ahead there (its widening is one instruction either way)
+  if (dlw_ok && bsrc != BSRC_MX4 && !big && (long long)M >= 16LL * G_total && (long long)M < 128LL * G_total &&
+      (long long)max_tiles_for(M, G_total, 128) * cdiv(N, glu ? 128 : 256) >= 128)
+    return K_DLW128;
   if (mid) return K_T128;
   if (big && dlw_ok) return K_DLW;
   // operands that need no conversion stream straight into LDS when every stage is a full row slice
@@ -135,7 +146,7 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   return K_T64;
 }
 
-static int tiled_kind_bm(TiledKind k) { return k == K_T64 ? 64 : k == K_T128 ? 128 : 256; }  // (every direct-to-LDS kernel: 256)
+static int tiled_kind_bm(TiledKind k) { return k == K_T64 ? 64 : k == K_T128 || k == K_DLW128 ? 128 : 256; }  // (every direct-to-LDS kernel: 256)
 
 static int launch_tiled_kind(TiledKind kind, int op, int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
   if (kind == K_DL128) {
@@ -144,7 +155,7 @@ static int launch_tiled_kind(TiledKind kind, int op, int bsrc, bool glu, const T
     return launch_dl(op, glu, 128, false, p, M, G_total, s);
   }
   if (kind == K_DL64) return launch_dl(op, glu, 64, false, p, M, G_total, s);
-  if (kind == K_DLW) return launch_dlw(bsrc, glu, p, M, G_total, s);
+  if (kind == K_DLW || kind == K_DLW128) return launch_dlw(bsrc, glu, kind == K_DLW128, p, M, G_total, s);
   return launch_tiled_bm(op, bsrc, glu, tiled_kind_bm(kind), false, p, M, G_total, s);
 }
 
@@ -401,11 +412,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   const int bsrc = variant == V_BF16 ? BSRC_SAME : variant == V_W8 ? BSRC_I8 : variant == V_W4 ? BSRC_I4 : BSRC_MX4;
   const bool int4_g128 = variant == V_W4 && rbk != 32;
   // rows per expert up to which the streaming kernel beats the register-staged one (layer times on the GPT-OSS shape with
-  // uniform routing): 36 for group-128 int4 (0.36 / 0.42 ms at 32 / 40 rows against 0.40 / 0.40 ms), 32 for MXFP4 (0.31 /
+  // uniform routing): 32 for group-128 int4 (0.36 / 0.42 ms at 32 / 40 rows against 0.36 / 0.36 ms on the stream kernel's 128-row
+  // tiles), 32 for MXFP4 (0.31 /
   // 0.38 against 0.34 / 0.35 ms).  Int8 and group-32 int4: 16, between the crossover with equal groups (30 on the Qwen3
   // shape, where both kernels then wait for the weights of all experts) and the one with Zipf-skewed routing (10: few
   // experts hold most rows and the tiled kernel converts their weights once per 128 rows instead of once per 32).
-  const long long stream_rows_hi = int4_g128 ? 36 : variant == V_MX4 ? 32 : 16;
+  const long long stream_rows_hi = int4_g128 ? 32 : variant == V_MX4 ? 32 : 16;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
   const bool stream_ok = variant != V_BF16 && !wq_kmajor && K % 32 == 0 && (long long)N * K < (1LL << 31);
@@ -416,7 +428,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   if (want_stream && stream_ok) {
     // 16-row tiles up to 16 rows per expert on average, 32-row tiles above; group-128 int4 keeps the 16-row tiles over the
     // whole range (its 32-row variant runs at two waves per SIMD: 0.36 against 0.44 ms on the GPT-OSS shape at 256 tokens)
-    // and stays on this kernel up to 36 rows per expert
+    // and stays on this kernel up to 32 rows per expert
     const bool one = int4_g128 || (long long)M <= 16LL * G;
     const int bm = one ? 16 : 32;
     map_tiles(bm);
@@ -438,7 +450,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     return launch_dl(op, glu, 64, false, p, M, G, s);
   }
   TiledKind kind = kernel == MOE_GMM_KERNEL_BIG ? K_T256 : pick_tiled_kind(op, bsrc, glu, M, K, N, G, wq_kmajor, a->lhs_row_idx ? ro.lhs_rows : 0);
-  if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64 || kind == K_DLW)) kind = K_T256;
+  if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64 || kind == K_DLW || kind == K_DLW128)) kind = kind == K_DLW128 ? K_T128 : K_T256;
   map_tiles(tiled_kind_bm(kind));
   return launch_tiled_kind(kind, op, bsrc, glu, p, M, G, s);
 }

@@ -305,7 +305,8 @@ __device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, 
 // Writes a wave's results.  The MFMA leaves lane l with 4 consecutive channels of row l % MI: 8-byte stores, neighbouring
 // lanes in different rows.  (Passing each row tile through LDS so that consecutive lanes store consecutive 16 bytes was
 // measured and is slower: the epilogue is bound by what stands between the stores, not by the stores.)
-template <int TM, int TN, int NT_OUT, bool GLU, typename acc_t>
+// (I_END < TM: only the wave's first I_END row tiles hold rows of this tile.)
+template <int TM, int TN, int NT_OUT, bool GLU, int I_END = TM, typename acc_t>
 __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
                                                const TiledParams& p, const TileInfo& tile, int row_base, int n_base, int lane) {
   constexpr int MI = sizeof(acc_t) == 16 ? 16 : 32;  // 4 accumulator registers per tile: the 16 x 16 instructions
@@ -319,7 +320,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
   for (int i = 0; i < TM; i++) rw[i] = 1.0f;
   if (p.ro.row_scale) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+    for (int i = 0; i < I_END; i++) {
       const int lr = row_base + i * MI + (lane % MI);
       rw[i] = p.ro.row_scale[tile.row0 + (lr < tile.nrows ? lr : 0)];
     }
@@ -329,7 +330,7 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
     constexpr int ACT = decltype(act_c)::value;
     constexpr bool GENERAL = decltype(general_c)::value;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+    for (int i = 0; i < I_END; i++) {
       const int lr = row_base + i * MI + (lane % MI);
       const bool row_ok = lr < tile.nrows;
 #pragma unroll
@@ -589,7 +590,7 @@ struct Fp8TiledParams;
 int launch_f8s(bool glu, const Fp8TiledParams& P, int M, int G_total, hipStream_t s);
 bool f8s_takes(int K, int N, long long M, long long indexed_lhs_rows);
 int prepare_f8s();
-int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s);
+int launch_dlw(int bsrc, bool glu, bool half, const TiledParams& p, int M, int G_total, hipStream_t s);
 // whether that kernel takes the shape (indexed_lhs_rows: rows of lhs when a row index is used, else 0)
 bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor);
 // moe_gmm_fp8.hip

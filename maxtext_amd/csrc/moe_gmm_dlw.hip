@@ -47,7 +47,10 @@ struct DlwCfg {
   __device__ static __forceinline__ int swz_b(int row) { return NIBBLES ? (row >> 3) & 1 : (row >> 2) & 3; }
 };
 
-template <typename C>
+// HALF: the tile list holds tiles of at most 128 rows (32 to 104 rows per expert on average): 8 row tiles per wave are
+// multiplied instead of 16, with the work behind the MFMAs packed into half as many slots; the upper half of a stage's
+// activation rows lies past the end of the tile's buffer descriptor and is neither fetched nor read.
+template <typename C, bool HALF>
 __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParams p0) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   // (bf16 activations carry no scale: saying so here lets the epilogue fold the per-row factor away)
@@ -215,25 +218,31 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
   auto kstep = [&](auto set_c, auto rd_c, auto ld_c, auto zc_c, int cur_buf, int cur_ks, int rd_buf, int rd_ks, int ld_kt, int ld_buf) {
     constexpr int SET = decltype(set_c)::value;
     constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value, ZC = decltype(zc_c)::value;
+    constexpr int TMX = HALF ? C::TM / 2 : C::TM;           // row tiles that are multiplied
+    constexpr int W0 = HALF ? 4 : 8, WSTEP = HALF ? 1 : 2;  // slots of the eight widening pieces: W0, W0 + WSTEP, ...
+    static_assert(2 * (C::A_IPW + C::B_IPW) <= TMX * C::TN && W0 + WSTEP * 4 * C::TN <= TMX * C::TN, "slots");
     float sc[C::TN] = {1.0f, 1.0f};
     if (RD && C::NIBBLES) {
 #pragma unroll
       for (int j = 0; j < C::TN; j++) sc[j] = rd_ks ? sc_cur[j][1] : sc_cur[j][0];
     }
 #pragma unroll
-    for (int i = 0; i < C::TM; i++) {
+    for (int i = 0; i < TMX; i++) {
 #pragma unroll
       for (int j = 0; j < C::TN; j++) {
         acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, gb[SET][j]), __builtin_bit_cast(v8bf, ga[i % C::RING]),
                                                             ZC ? v4f{0.f, 0.f, 0.f, 0.f} : acc[j][i], 0, 0, 0);
         const int slot = i * C::TN + j;
         if (RD && slot < C::TN) read_braw(rd_buf, rd_ks, slot);
-        // the eight pieces of the two fragments, one every second MFMA from slot 8 on
-        if (RD && slot >= 8 && slot < 8 + 2 * 4 * C::TN && slot % 2 == 0) widen_piece(SET ^ 1, (slot - 8) / 8, ((slot - 8) / 2) % 4, sc[(slot - 8) / 8]);
+        // the eight pieces of the two fragments
+        if (RD && slot >= W0 && slot < W0 + WSTEP * 4 * C::TN && (slot - W0) % WSTEP == 0) {
+          const int q = (slot - W0) / WSTEP;
+          widen_piece(SET ^ 1, q / 4, q % 4, sc[q / 4]);
+        }
         if (LD && slot % 2 == 1 && slot / 2 < C::A_IPW) issue_a(ld_kt, ld_buf, slot / 2);
         if (LD && slot % 2 == 1 && slot / 2 >= C::A_IPW && slot / 2 < C::A_IPW + C::B_IPW) issue_b(ld_kt, ld_buf, slot / 2 - C::A_IPW);
-        if (j == C::TN - 1 && i < C::TM - C::RING) read_a(cur_buf, cur_ks, i + C::RING);
-        if (RD && j == C::TN - 1 && i >= C::TM - C::RING) read_a(rd_buf, rd_ks, i - (C::TM - C::RING));
+        if (j == C::TN - 1 && i < TMX - C::RING) read_a(cur_buf, cur_ks, i + C::RING);
+        if (RD && j == C::TN - 1 && i >= TMX - C::RING) read_a(rd_buf, rd_ks, i - (TMX - C::RING));
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -318,7 +327,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
     iteration(nk - 2, F_{});
     load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC == BSRC_I8, C::MI>(esc, p, cur.info, 0, n_out0, lane);
     iteration(nk - 1, T_{});
-    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, cur.info, 0, n_out0, lane);
+    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU, HALF ? C::TM / 2 : C::TM>(acc, esc, p, cur.info, 0, n_out0, lane);
     if (!have_n) break;
     cur = nxt;
     base = cb;  // (after the last iteration: the buffer of stage nk = the next tile's stage 0, landed before the last barrier)
@@ -334,8 +343,12 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
 // ---------------------------------------------------------------------------------------
 
 template <typename C>
+struct HalfTiles {};  // (a key for the second kernel's per-device set-up flags)
+
+template <typename C>
 static int prepare_dlw_cfg() {
-  return reserve_lds(gmm_dlw_kernel<C>, C::LDS_BYTES, lds_flags<C>());
+  if (int st = reserve_lds(gmm_dlw_kernel<C, false>, C::LDS_BYTES, lds_flags<C>())) return st;
+  return reserve_lds(gmm_dlw_kernel<C, true>, C::LDS_BYTES, lds_flags<HalfTiles<C>>());
 }
 
 int prepare_dlw() {
@@ -348,20 +361,22 @@ int prepare_dlw() {
   return st;
 }
 
+// half: the tile list was built with 128-row tiles
 template <typename C>
-static int launch_dlw_cfg(const TiledParams& p0, int M, int G_total, hipStream_t s) {
+static int launch_dlw_cfg(bool half, const TiledParams& p0, int M, int G_total, hipStream_t s) {
   if (int st = prepare_dlw_cfg<C>()) return st;
   TiledParams p = p0;
-  p.max_m_tiles = max_tiles_for(M, G_total, C::BM);
+  p.max_m_tiles = max_tiles_for(M, G_total, half ? C::BM / 2 : C::BM);
   p.tiles_n = cdiv(p.N, C::OUT_BN);
   const long long tiles = (long long)p.max_m_tiles * p.tiles_n;
   if (tiles > 0x7fffffffLL) return fail(MOE_ERR_UNSUPPORTED, "gmm: grid too large");
-  if (p.tune <= 0) p.tune = default_super_row(M, G_total, C::BM);
+  if (p.tune <= 0) p.tune = default_super_row(M, G_total, half ? C::BM / 2 : C::BM);
   int num_cus = 0;
   if (int st = device_cu_count(&num_cus)) return st;
   long long blocks = tiles < num_cus ? tiles : num_cus;
   if (blocks >= 8) blocks -= blocks % 8;
-  gmm_dlw_kernel<C><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
+  if (half) gmm_dlw_kernel<C, true><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
+  else gmm_dlw_kernel<C, false><<<(unsigned)blocks, C::THREADS, C::LDS_BYTES, s>>>(p);
   return check_launch("gmm_dlw_kernel");
 }
 
@@ -371,11 +386,11 @@ bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor) {
   return K % 64 == 0 && K >= 192 && !wq_kmajor && (long long)N * K < (1LL << 32) && indexed_lhs_rows * K * 2 < (1LL << 32);
 }
 
-int launch_dlw(int bsrc, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
+int launch_dlw(int bsrc, bool glu, bool half, const TiledParams& p, int M, int G_total, hipStream_t s) {
   if (!dlw_takes(p.K, p.N, p.ro.row_idx ? p.ro.lhs_rows : 0, p.wq_kmajor != 0))
     return fail(MOE_ERR_UNSUPPORTED, "gmm: the weight-only direct-to-LDS kernel needs K %% 64 == 0, K >= 192, scales in the default layout and 32-bit byte offsets");
 #define MOE_DLW_CASE(BSRC) \
-  if (bsrc == BSRC) return glu ? launch_dlw_cfg<DlwCfg<BSRC, true>>(p, M, G_total, s) : launch_dlw_cfg<DlwCfg<BSRC, false>>(p, M, G_total, s);
+  if (bsrc == BSRC) return glu ? launch_dlw_cfg<DlwCfg<BSRC, true>>(half, p, M, G_total, s) : launch_dlw_cfg<DlwCfg<BSRC, false>>(half, p, M, G_total, s);
   MOE_DLW_CASE(BSRC_I8)
   MOE_DLW_CASE(BSRC_I4)
   MOE_DLW_CASE(BSRC_MX4)

@@ -267,7 +267,8 @@ def test_gmm_row_index_row_scale_and_f32_out_in_every_kernel_family(K, case):
 
 @pytest.mark.parametrize("fmt", ["int8", "int4", "int4g32", "mxfp4"])
 @pytest.mark.parametrize("glu", [False, True])
-def test_weight_only_prefill_kernel_against_the_tiled_kernel_at_size(K, fmt, glu):
+@pytest.mark.parametrize("regime", ["prefill", "mid"])
+def test_weight_only_prefill_kernel_against_the_tiled_kernel_at_size(K, fmt, glu, regime):
   """The persistent weight-only kernel (raw weights through LDS, widened per wave, one request stream across tiles) on
   a shape with hundreds of tiles per block, ragged groups, a ragged last n-tile and an empty group, against the
   register-staged tiled kernel on the same operands (which the small-shape tests pin to the oracle), plus sampled rows
@@ -277,6 +278,8 @@ def test_weight_only_prefill_kernel_against_the_tiled_kernel_at_size(K, fmt, glu
   g = torch.Generator(device="cuda").manual_seed(17)
   e, k, n = 16, 1088, 1984  # 17 stages of 64; 15.5 n-tiles of 128
   gs_h = np.array([700, 1031, 0, 512, 256, 1300, 90, 777, 640, 515, 513, 511, 1024, 300, 999, 1100], np.int32)
+  if regime == "mid":  # 60 rows per expert on average: int8 / int4 run the same kernel on 128-row tiles (half of the row tiles multiplied)
+    gs_h = np.array([70, 103, 0, 51, 25, 130, 9, 77, 64, 129, 128, 127, 1, 30, 99, 17], np.int32)
   m = int(gs_h.sum()) + 100  # 100 rows in no group
   gs = torch.from_numpy(gs_h).cuda()
   lhs = torch.randn(m, k, device="cuda", generator=g).to(torch.bfloat16)
