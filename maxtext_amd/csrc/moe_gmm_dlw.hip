@@ -111,8 +111,10 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
     b_desc = buffer_desc((load_up ? p.rhs_up : p.rhs) + (size_t)t.info.group * N * w_row_bytes, clamp_u32((size_t)N * w_row_bytes));
     b_soff = (uint32_t)t.n0 * w_row_bytes;
   };
+  // (HALF: rows 128 .. 255 of a stage, the requests of waves 4 .. 7, are never read)
+  const bool a_wanted = !HALF || wave < C::NWAVES / 2;
   auto issue_a = [&](int kt, int buf, int i) {
-    dma16_buffer(a_desc, a_voff[i], (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + (wave * C::A_IPW + i) * 1024);
+    if (a_wanted) dma16_buffer(a_desc, a_voff[i], (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + (wave * C::A_IPW + i) * 1024);
   };
   auto issue_b = [&](int kt, int buf, int i) {
     dma16_buffer(b_desc, b_voff[i], b_soff + (uint32_t)kt * C::W_ROW, lds_base + buf * C::STAGE + C::A_STAGE + (wave * C::B_IPW + i) * 1024);
