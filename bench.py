@@ -128,9 +128,8 @@ def dominant_kernel_model(wl, group_sizes):
   if cfg.act_quant == "int8" or wl.weight_quant in (None, "bf16"):
     kernel = "gmm_dls_kernel" if rows >= 128 * len(group_sizes) else "gmm_tiled_kernel"
   else:
-    # (int8 / int4 also below, on 128-row tiles, down to 16 rows per expert; MXFP4 stays on the register-staged tiles there)
-    on_stream = rows >= (104 if wl.weight_quant == "mxfp4" else 16) * len(group_sizes)
-    kernel = "gmm_dlw_kernel" if on_stream and d % 64 == 0 else "gmm_tiled_kernel"
+    # (from 16 rows per expert on: on 128-row tiles up to 112, on 256-row tiles above)
+    kernel = "gmm_dlw_kernel" if rows >= 16 * len(group_sizes) and d % 64 == 0 else "gmm_tiled_kernel"
   return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS[op], scale=1e12,
               name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype=op)
 

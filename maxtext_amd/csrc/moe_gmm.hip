@@ -116,11 +116,9 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   const bool dlw_ok = bsrc != BSRC_SAME && dlw_takes(K, N, indexed_lhs_rows, wq_kmajor);
   // 256-row tiles from 128 rows per expert on average, where half of the routed groups no longer fit a 128-row tile (int8
   // x int8 on the Qwen3 shape: 0.106 against 0.126 ms at 112 rows, 0.133 against 0.131 at 128); the weight-only stream
-  // kernel already from 104, its alternative being the register-staged 128-row tiles (GPT-OSS layer at 96 / 112 rows per
-  // expert: 0.42 / 0.49 ms on 128-row tiles, 0.44 / 0.44 on the stream kernel; with Zipf routing it leads from 70 on)
-  // (int8 / int4 weights: from 112, their 128-row alternative being the same stream kernel on half-height tiles, see below:
-  // GPT-OSS int4 layer at 104 / 112 rows per expert 0.38 / 0.45 ms on those, 0.44 / 0.44 on 256-row tiles)
-  const bool big = (long long)M >= (dlw_ok ? (bsrc == BSRC_MX4 ? 104LL : 112LL) : 128LL) * G_total && tiles_big >= 128;
+  // kernel from 112: below, the same kernel runs on 128-row tiles (GPT-OSS int4 layer at 104 / 112 rows per expert 0.38 /
+  // 0.45 ms on those, 0.44 / 0.44 on 256-row tiles)
+  const bool big = (long long)M >= (dlw_ok ? 112LL : 128LL) * G_total && tiles_big >= 128;
   // 32 to 128 rows per expert on average: 128-row tiles; below 32, 64-row tiles.  With routed groups of near-equal size
   // the 64-row tiles are 5-10 % ahead up to 56 rows per expert (GPT-OSS shape, 384 tokens: 0.38 against 0.41 ms for the
   // layer) and collapse at 64, where half of the groups need a second tile (0.57 against 0.41 ms); with skewed routing
@@ -129,12 +127,12 @@ static TiledKind pick_tiled_kind(int op, int bsrc, bool glu, int M, int K, int N
   // their 256-row register-staged tiles pass the 128-row ones at 128 rows per expert as well.
   const bool mid = !big && (long long)M >= 32LL * G_total && (long long)M < 128LL * G_total;
   const int esz = op == OP_I8 ? 1 : 2;
-  // weight-only int8 / int4 between the streaming kernel's range and the 256-row tiles: the stream kernel on 128-row tiles
-  // (half of its row tiles multiplied, nothing fetched for the other half) is 10-15 % ahead of the register-staged 128-row
-  // tiles (GPT-OSS int4 layer at 40 to 96 rows per expert 0.36-0.37 against 0.40-0.42 ms, Qwen3 int8 with Zipf routing at
-  // 20 to 80 rows 0.14-0.21 against 0.15-0.25 ms) and level with the 64-row ones at 16 to 32; MXFP4 stays on the
-  // register-staged tiles, which are 4 % ahead there (its widening is one instruction either way)
-  if (dlw_ok && bsrc != BSRC_MX4 && !big && (long long)M >= 16LL * G_total && (long long)M < 128LL * G_total &&
+  // weight-only formats between the streaming kernel's range and the 256-row tiles: the stream kernel on 128-row tiles
+  // (half of its row tiles multiplied, nothing requested for the other half) is 10-15 % ahead of the register-staged
+  // 128-row tiles for int8 and int4 (GPT-OSS int4 layer at 40 to 96 rows per expert 0.34-0.35 against 0.40-0.42 ms, Qwen3
+  // int8 with Zipf routing at 20 to 80 rows 0.14-0.20 against 0.15-0.25 ms), 1-2 % for MXFP4 (0.338-0.352 against
+  // 0.344-0.358 ms), and level with the 64-row tiles at 16 to 32 rows
+  if (dlw_ok && !big && (long long)M >= 16LL * G_total && (long long)M < 128LL * G_total &&
       (long long)max_tiles_for(M, G_total, 128) * cdiv(N, glu ? 128 : 256) >= 128)
     return K_DLW128;
   if (mid) return K_T128;
