@@ -223,3 +223,32 @@ def test_fullsize_whole_layer_output_against_oracle(name):
   # wherever the bf16 intermediates differ by an ulp: a noise of about 0.6 % of the output's rms per element, whose
   # maximum over 33 million elements reaches 3.3 %
   assert relerr(got, want, atol_rms=4e-2 if cfg.act_quant else ELEM_ATOL_RMS_CHAINED) <= TOL
+
+
+@pytest.mark.parametrize("name,tokens", [("c4", 768), ("c5", 384), ("c5", 880), ("c5mx", 512)])
+def test_mid_sized_weight_only_layers_against_oracle(name, tokens):
+  """The token counts between decode and prefill (20 to 104 rows per expert), where the weight-only formats run the stream
+  kernel on 128-row tiles with the permute fused in through the row index: every element against the CPU oracle."""
+  from maxtext_amd import moe, synthetic
+  from maxtext_amd.quantizations import QArray
+  from oracle.layer import oracle_layer
+
+  wl = synthetic.workload(name, tokens)
+  cfg = wl.cfg
+  layer = synthetic.make_layer(wl, device="cpu")
+  trip = lambda qa: (qa.qvalue, qa.scale, qa.qtype)
+  want, _, operm, ogs = oracle_layer(
+      layer["x"], layer["gate_logits"], layer["pre_bias_logits"], trip(layer["wi_0"]), trip(layer["wi_1"]), trip(layer["wo"]),
+      num_experts=cfg.num_experts, k=cfg.num_experts_per_tok, emb_dim=cfg.emb_dim, mlp_dim=cfg.moe_mlp_dim,
+      norm_topk_prob=cfg.norm_topk_prob, act_quant=cfg.act_quant, activation=cfg.activation, acc_dtype=torch.float32)
+  rows_per_expert = tokens * cfg.num_experts_per_tok / cfg.num_experts
+  assert 16 < rows_per_expert < 112  # the regime
+  if name == "c4":
+    assert ogs.max() > 128  # skewed routing: groups that need a second tile
+  dev = lambda v: QArray(v.qvalue.cuda(), v.scale.cuda(), v.qtype) if isinstance(v, QArray) else v.cuda()
+  wi_0, wi_1, wo = dev(layer["wi_0"]), dev(layer["wi_1"]), dev(layer["wo"])
+  block = moe.RoutedMoE(cfg, wi_0, wi_1, wo)
+  out, _, _ = block.sparse_matmul(layer["x"].cuda(), layer["gate_logits"].cuda(), None, wi_0, wi_1, wo)
+  got = out.reshape(want.shape)
+  assert torch.isfinite(got.float()).all()
+  assert relerr(got, want, atol_rms=ELEM_ATOL_RMS_CHAINED) <= TOL
