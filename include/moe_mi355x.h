@@ -11,9 +11,10 @@
  *   - `group_sizes` stays on the device: no entry point reads it on the host;
  *   - inputs are never written; outputs are fully defined (rows that belong to no
  *     local group are written as zeros), so buffers need no pre-clearing;
- *   - calls on different streams with disjoint buffers may overlap; the only state the library keeps is per device
- *     and written once (the CU count and "this kernel may use more than 64 KB of LDS"), set up on the first call
- *     that needs it or ahead of time by moe_init().
+ *   - calls on different streams with disjoint buffers may overlap; the state the library keeps is per device: values
+ *     written once (the CU count, "this kernel may use more than 64 KB of LDS", the address of the static workspace),
+ *     set up on the first call that needs them or ahead of time by moe_init(), and one host-side record, under a lock,
+ *     of what the last moe_gmm call on the device mapped and where, which only calls flagged MOE_GMM_SAME_GROUPS consult.
  *
  * Paths in the citations are relative to the reference (AI-Hypercomputer/maxtext).
  */
