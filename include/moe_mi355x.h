@@ -477,6 +477,18 @@ MOE_API int moe_glu_act_bwd(const void* h0, const void* h1, const void* dout, si
                             void* dh0, void* dh1, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Per-expert bias on finished bf16 rows: out[m, :] = bf16(h[m, :] + bias[g(m), :]) for the rows of the local groups
+ * (g(m) = the row's group minus group_offset), all other rows copied.  This is the separate add of the reference's
+ * layer (layer_w0 + w0_bias after the matmul has rounded to the activation dtype, moe.py:1952-1957, :2239-2242), which
+ * the differentiable path keeps so that its forward rounds twice like the reference's; inference calls pass the bias to
+ * moe_gmm (rhs_bias), whose epilogue adds it before the one rounding.
+ *   h, out [M, N] bf16 (may be the same buffer);  bias [num_groups_local, N] f32
+ * Limits: N % 8 == 0, at most 1024 groups.
+ */
+MOE_API int moe_add_group_bias(const void* h, int M, int N, const float* bias, const int32_t* group_sizes, int num_groups_total,
+                       int num_groups_local, int group_offset, void* out, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Gradient preparation of the quantised backward pass (int8 x int8 forward with channelwise scales): the incoming
  * gradient times the scale of the axis that the gradient product contracts away (_bwd_prepare_inputs,
  * kernels/megablox/ops.py:530-580), optionally quantised to float8_e5m2 (_bwd_quantize_gradient, ops.py:583-604;

@@ -170,6 +170,43 @@ __global__ void bwd_col_scale_kernel(float* colmax, int n) {
   if (i < n) colmax[i] = e5m2_scale(colmax[i]);
 }
 
+// h + bias[expert of the row] for the rows of local groups, the others copied as they are: one block per row.
+__global__ __launch_bounds__(kBwdThreads) void add_group_bias_kernel(const uint4* h, int N, const float* bias, const int* group_sizes, int G_total,
+                                                                     int G_local, int group_offset, uint4* out) {
+  __shared__ int ends[kBwdMaxGroups];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  if (tid == 0) {
+    int run = 0;
+    for (int g = 0; g < G_total; g++) {
+      run += max(group_sizes[g], 0);
+      ends[g] = run;
+    }
+  }
+  __syncthreads();
+  int lo = 0, hi = G_total;  // first group whose end lies past the row (G_total: the row is in no group)
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (ends[mid] > m) hi = mid;
+    else lo = mid + 1;
+  }
+  const int local = lo - group_offset;
+  const bool owned = lo < G_total && local >= 0 && local < G_local;
+  const float* b = bias + (size_t)(owned ? local : 0) * N;
+  const int nvec = N / 8;
+  for (int i = tid; i < nvec; i += kBwdThreads) {
+    const uint4 x = h[(size_t)m * nvec + i];
+    uint4 y = x;
+    if (owned) {
+      const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu) + b[i * 8 + e];
+      y = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+    }
+    out[(size_t)m * nvec + i] = y;
+  }
+}
+
 }  // namespace moe
 
 using namespace moe;
@@ -208,6 +245,18 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
   bwd_col_quant_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, (uint4*)out);
   bwd_col_scale_kernel<<<cdiv(N, 256), 256, 0, s>>>(scale_out, N);
   return check_launch("bwd_col_quant_kernel");
+}
+
+int moe_add_group_bias(const void* h, int M, int N, const float* bias, const int32_t* group_sizes, int num_groups_total,
+                       int num_groups_local, int group_offset, void* out, void* stream) {
+  if (!h || !bias || !group_sizes || !out) return fail(MOE_ERR_INVALID_ARG, "add_group_bias: NULL pointer");
+  if (M < 0 || N <= 0 || N % 8 != 0) return fail(MOE_ERR_UNSUPPORTED, "add_group_bias: need N %% 8 == 0 (N=%d)", N);
+  if (num_groups_total <= 0 || num_groups_total > kBwdMaxGroups || num_groups_local <= 0 || group_offset < 0)
+    return fail(MOE_ERR_INVALID_ARG, "add_group_bias: bad groups (at most %d)", kBwdMaxGroups);
+  if (M == 0) return MOE_OK;
+  add_group_bias_kernel<<<M, kBwdThreads, 0, (hipStream_t)stream>>>((const uint4*)h, N, bias, group_sizes, num_groups_total, num_groups_local,
+                                                                     group_offset, (uint4*)out);
+  return check_launch("add_group_bias_kernel");
 }
 
 }  // extern "C"

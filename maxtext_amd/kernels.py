@@ -345,6 +345,21 @@ def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups
   return out, scale
 
 
+def add_group_bias(h, bias, group_sizes, *, group_offset=0):
+  """bf16(h + bias[expert of the row]) for the rows of the local groups (bias [G_local, N] f32), other rows copied."""
+  _need(h, "h", torch.bfloat16, 2)
+  _need(bias, "bias", torch.float32, 2)
+  _need(group_sizes, "group_sizes", torch.int32, 1)
+  m, n = h.shape
+  if bias.shape[1] != n:
+    raise ValueError(f"bias has {bias.shape[1]} channels for {n}")
+  out = torch.empty_like(h)
+  st = _lib.load().moe_add_group_bias(_lib.ptr(h), m, n, _lib.ptr(bias), _lib.ptr(group_sizes), group_sizes.numel(), bias.shape[0],
+                                      int(group_offset), _lib.ptr(out), _lib.current_stream())
+  _lib.check(st, "moe_add_group_bias")
+  return out
+
+
 def transpose_rhs(rhs_gkn):
   """[G, K, N] -> [G, N, K] for 1- or 2-byte element types."""
   _need(rhs_gkn, "rhs", None, 3)

@@ -446,16 +446,10 @@ class _BiasFn(torch.autograd.Function):
 
   @staticmethod
   def forward(ctx, h, bias, group_sizes, offset):
-    m = h.shape[0]
     g_local = bias.shape[0]
-    ends = torch.cumsum(group_sizes, 0)
-    row_group = torch.searchsorted(ends, torch.arange(m, device=h.device, dtype=ends.dtype), right=True)
-    local = row_group - offset
-    owned = (local >= 0) & (local < g_local) & (row_group < group_sizes.numel())
     ctx.save_for_backward(group_sizes)
     ctx.offset, ctx.g_local, ctx.bias_dtype = offset, g_local, bias.dtype
-    add = bias.float()[local.clamp(0, g_local - 1)] * owned[:, None]
-    return (h.float() + add).to(h.dtype)
+    return kernels.add_group_bias(h.contiguous(), bias.float().contiguous(), group_sizes, group_offset=offset)
 
   @staticmethod
   def backward(ctx, dout):

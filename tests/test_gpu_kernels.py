@@ -1542,3 +1542,22 @@ def test_sort_leaves_the_tile_list_for_the_matmuls(K, t, e, k):
   assert torch.equal(yb, K.gmm_raw(x, wb, gs0))
   y2 = K.gmm_raw(x, wq, gs, rhs_scale=sc, workspace=ws, same_groups=True)
   assert torch.equal(y2, y)
+
+
+@pytest.mark.parametrize("m,n,sizes,offset,g_local", [(40, 64, [7, 0, 12, 1, 20], 0, 5), (300, 2880, [100, 0, 37, 63, 50], 1, 3), (64, 8, [70], 0, 1),
+                                                     (513, 512, [3] * 100 + [0] * 28, 64, 64)])
+def test_add_group_bias_bit_exact(K, m, n, sizes, offset, g_local):
+  # bf16(h + bias[group of the row - offset]) on the rows of the local groups; rows of other groups and rows in no
+  # group are copied (moe.py:1952-1957 as the differentiable path applies it)
+  g = torch.Generator().manual_seed(m + n)
+  h = torch.randn((m, n), generator=g).to(torch.bfloat16)
+  bias = torch.randn((g_local, n), generator=g)
+  gs = np.array(sizes, np.int32)
+  ends = np.cumsum(gs)
+  want = h.clone()
+  for r in range(m):
+    grp = int(np.searchsorted(ends, r, side="right"))
+    if grp < len(sizes) and 0 <= grp - offset < g_local:
+      want[r] = (h[r].float() + bias[grp - offset]).to(torch.bfloat16)
+  got = K.add_group_bias(h.cuda(), bias.cuda(), cuda(gs), group_offset=offset)
+  assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
