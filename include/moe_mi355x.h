@@ -419,6 +419,12 @@ MOE_API int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem
 MOE_API int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
                      int num_groups_total, int num_groups_local, int group_offset, const void* existing_out,
                      int existing_dtype, int out_dtype, void* out, void* stream);
+/* The same with the products of output row n (the channel of dout) multiplied by out_row_scale[n] ([N] f32) before
+ * existing_out is added and the result is rounded: the column scales of a float8_e5m2 gradient (ops.py:590-603) go
+ * back onto the weight gradient here instead of in a pass over [G, N, K]. */
+MOE_API int moe_tgmm_scaled(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
+                    int num_groups_total, int num_groups_local, int group_offset, const float* out_row_scale,
+                    const void* existing_out, int existing_dtype, int out_dtype, void* out, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Unpermute + top-k weighted combine.  Replaces RoutedMoE.unpermute

@@ -21,14 +21,19 @@ struct TgmmParams {
   const int32_t* group_sizes;
   void* out;  // [G_local, N, K] bf16 or f32
   const void* existing;  // NULL, or [G_local, N, K] values added to the products before the store (may be `out` itself)
+  const float* n_scale;  // NULL, or [N]: the products of output row n are multiplied by n_scale[n] first
   int M, K, N;
   int G_total, G_local, group_offset;
   int out_f32, existing_f32;
 };
 
-// out[off .. off+3] = v + existing[off .. off+3].  A lane reads the four values it is about to overwrite, so `existing`
-// may be the output buffer.
-__device__ __forceinline__ void tgmm_store4(const TgmmParams& p, size_t off, float v0, float v1, float v2, float v3) {
+// out[off .. off+3] = v * n_scale[n] + existing[off .. off+3]: four values along K of output row n.  A lane reads the
+// four values it is about to overwrite, so `existing` may be the output buffer.
+__device__ __forceinline__ void tgmm_store4(const TgmmParams& p, size_t off, int n, float v0, float v1, float v2, float v3) {
+  if (p.n_scale) {
+    const float sc = p.n_scale[n];
+    v0 *= sc; v1 *= sc; v2 *= sc; v3 *= sc;
+  }
   if (p.existing) {
     if (p.existing_f32) {
       const float4 e = *(const float4*)((const float*)p.existing + off);
@@ -151,7 +156,7 @@ __global__ __launch_bounds__(kTgThreads) void tgmm_kernel(const TgmmParams p) {
         const int k = k0 + wk * 64 + i * 32 + 8 * q + 4 * (lane / 32);
         if (k >= K) continue;
         const size_t off = ((size_t)g_local * N + n) * K + k;
-        tgmm_store4(p, off, acc[j][i][4 * q], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]);
+        tgmm_store4(p, off, n, acc[j][i][4 * q], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]);
       }
   }
 }
@@ -218,7 +223,7 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
   if (size == 0) {  // an empty group's gradient is zero
     for (int i = tid; i < kTdTile * (kTdTile / 4); i += kTdThreads) {
       const size_t off = ((size_t)g_local * N + n0 + i / (kTdTile / 4)) * K + k0 + (i % (kTdTile / 4)) * 4;
-      tgmm_store4(p, off, 0.f, 0.f, 0.f, 0.f);
+      tgmm_store4(p, off, n0 + i / (kTdTile / 4), 0.f, 0.f, 0.f, 0.f);
     }
     return;
   }
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
     for (int j = 0; j < 4; j++) {
       const int k = k0 + wk * 64 + j * 16 + 4 * gq;
       const size_t off = ((size_t)g_local * N + n) * K + k;
-      tgmm_store4(p, off, acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]);
+      tgmm_store4(p, off, n, acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]);
     }
   }
 }
@@ -369,9 +374,9 @@ namespace moe {
 int prepare_tgmm() { return reserve_lds(tgmm_dl_kernel, kTdLds, lds_flags<TgmmParams>()); }
 }  // namespace moe
 
-extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
-                        int num_groups_total, int num_groups_local, int group_offset, const void* existing_out,
-                        int existing_dtype, int out_dtype, void* out, void* stream) {
+extern "C" int moe_tgmm_scaled(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
+                               int num_groups_total, int num_groups_local, int group_offset, const float* out_row_scale,
+                               const void* existing_out, int existing_dtype, int out_dtype, void* out, void* stream) {
   if (!lhs || !dout || !group_sizes || !out) return fail(MOE_ERR_INVALID_ARG, "tgmm: NULL pointer");
   if (M < 0 || K <= 0 || N <= 0 || num_groups_total <= 0 || num_groups_local <= 0 || group_offset < 0)
     return fail(MOE_ERR_INVALID_ARG, "tgmm: bad sizes");
@@ -389,6 +394,7 @@ extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_
   if (existing_out == out && existing_dtype != out_dtype)
     return fail(MOE_ERR_INVALID_ARG, "tgmm: existing_out aliases out with another element type");
   p.existing = existing_out; p.existing_f32 = existing_dtype == MOE_F32;
+  p.n_scale = out_row_scale;
   // groups of 128 rows and more on average take the 256 x 256 tiles when the shape allows it
   const long long tiles = (long long)(K / kTdTile) * (N / kTdTile) * num_groups_local;
   if (K % kTdTile == 0 && N % kTdTile == 0 && K < (1 << 24) && N < (1 << 24) && (long long)M >= 128LL * num_groups_total && tiles >= 128 && tiles <= 0x7fffffffLL) {
@@ -399,4 +405,11 @@ extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_
   dim3 grid(cdiv(K, kTgBK), cdiv(N, kTgBN), num_groups_local);
   tgmm_kernel<<<grid, kTgThreads, 0, (hipStream_t)stream>>>(p);
   return check_launch("tgmm_kernel");
+}
+
+extern "C" int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
+                        int num_groups_total, int num_groups_local, int group_offset, const void* existing_out,
+                        int existing_dtype, int out_dtype, void* out, void* stream) {
+  return moe_tgmm_scaled(lhs, dout, group_sizes, M, K, N, num_groups_total, num_groups_local, group_offset, nullptr, existing_out,
+                         existing_dtype, out_dtype, out, stream);
 }

@@ -509,9 +509,11 @@ def gmm_rhs_kn_supported(m, k, n, num_groups_total):
   return bool(_lib.load().moe_gmm_rhs_kn_supported(int(m), int(k), int(n), int(num_groups_total)))
 
 
-def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16, existing_out=None):
+def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16, existing_out=None,
+         out_row_scale=None):
   """Weight gradient: out[g, n, k] = sum over rows m of group g of dout[m, n] * lhs[m, k]  ->  [G_local, N, K].
 
+  out_row_scale: [N] f32; the f32 products of output row n are multiplied by out_row_scale[n] first.
   existing_out: [G_local, N, K] bf16 or f32, added to the f32 products before the rounding to out_dtype."""
   _need(lhs, "lhs", torch.bfloat16, 2)
   _need(dout, "dout", torch.bfloat16, 2)
@@ -532,9 +534,15 @@ def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_d
     _need(existing_out, "existing_out", existing_out.dtype, 3)
     if tuple(existing_out.shape) != (g_local, n, k):
       raise ValueError(f"existing_out must be [{g_local}, {n}, {k}], got {tuple(existing_out.shape)}")
+  if out_row_scale is not None:
+    _need(out_row_scale, "out_row_scale", torch.float32, 1)
+    if out_row_scale.numel() != n:
+      raise ValueError(f"out_row_scale must have {n} entries, got {out_row_scale.numel()}")
   lib = _lib.load()
-  st = lib.moe_tgmm(_lib.ptr(lhs), _lib.ptr(dout), _lib.ptr(group_sizes), m, k, n, g_total, g_local, int(group_offset),
-                    None if existing_out is None else _lib.ptr(existing_out), 0 if existing_out is None else code[existing_out.dtype],
-                    code[out_dtype], _lib.ptr(out), _lib.current_stream())
-  _lib.check(st, "moe_tgmm")
+  st = lib.moe_tgmm_scaled(_lib.ptr(lhs), _lib.ptr(dout), _lib.ptr(group_sizes), m, k, n, g_total, g_local, int(group_offset),
+                           None if out_row_scale is None else _lib.ptr(out_row_scale),
+                           None if existing_out is None else _lib.ptr(existing_out),
+                           0 if existing_out is None else code[existing_out.dtype], code[out_dtype], _lib.ptr(out),
+                           _lib.current_stream())
+  _lib.check(st, "moe_tgmm_scaled")
   return out

@@ -384,10 +384,10 @@ class _GmmFn(torch.autograd.Function):
     if ctx.needs_input_grad[1]:
       # dout times the activations' row scales, e5m2 per column
       d, s_col = kernels.bwd_scale_grad(dout, ls, mode="drhs", quantize=quant)
+      # the column scales go back onto the f32 products in the kernel's epilogue, which rounds once to the weights' type
+      direct = ctx.rhs_dtype in (torch.bfloat16, torch.float32)
       w = kernels.tgmm(lq.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
-                       out_dtype=torch.float32)  # [g, n, k]
-      if s_col is not None:
-        w = w * s_col.reshape(1, n, 1)
+                       out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
       w = w.to(ctx.rhs_dtype)
       drhs = w if ctx.transpose_rhs else w.transpose(1, 2)
     return dlhs, drhs

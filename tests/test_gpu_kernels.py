@@ -675,6 +675,31 @@ def test_tgmm_existing_out_is_added_before_rounding(K, m, k, n, gs, existing_dty
     megablox.tgmm(cuda(lhs).t(), cuda(dout), cuda(gs), existing_out=cuda(existing))  # 3 groups given, 5 expected
 
 
+@pytest.mark.parametrize("m,k,n,gs", [(333, 136, 264, [40, 0, 100, 93, 100]), (700, 1024, 3072, [140, 0, 199, 193, 100])])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_tgmm_row_scale_goes_on_before_existing_out_and_rounding(K, m, k, n, gs, out_dtype):
+  """out[g, n, :] = f32 products * out_row_scale[n] (+ existing_out), rounded once (the column scales of an e5m2 gradient,
+  ops.py:590-603): integer data keeps the sums exact, odd multiples of 1/8 as scales make the bf16 result round, so
+  the comparison with the oracle's unscaled f32 product, scaled and rounded here, is bit for bit."""
+  rng = np.random.default_rng(47)
+  gs = np.array(gs, np.int32)
+  lhs = torch.from_numpy(rng.integers(-3, 4, (m, k)).astype(np.float32)).to(torch.bfloat16)
+  dout = torch.from_numpy(rng.integers(-31, 32, (m, n)).astype(np.float32)).to(torch.bfloat16)  # sums beyond bf16's 8 bits
+  scale = torch.from_numpy((2 * rng.integers(1, 40, n) + 1).astype(np.float32) / 8)
+  existing = torch.from_numpy(rng.integers(-9, 10, (3, n, k)).astype(np.float32) * 0.5)
+  plain = O.tgmm(lhs, dout, gs, num_actual_groups=3, group_offset=1, out_dtype=torch.float32).transpose(1, 2)  # [g, n, k] f32, exact
+  want = plain * scale.reshape(1, n, 1)
+  got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), num_groups_local=3, group_offset=1, out_dtype=out_dtype, out_row_scale=cuda(scale))
+  assert got.dtype == out_dtype and torch.equal(got.cpu(), want.to(out_dtype))
+  if out_dtype == torch.bfloat16:  # (rounding the products before the scaling would give other bits)
+    assert not torch.equal(want.to(out_dtype), (plain.to(out_dtype) * scale.reshape(1, n, 1)).to(out_dtype))
+  got = K.tgmm(cuda(lhs), cuda(dout), cuda(gs), num_groups_local=3, group_offset=1, out_dtype=out_dtype, out_row_scale=cuda(scale),
+               existing_out=cuda(existing))
+  assert torch.equal(got.cpu(), (want + existing).to(out_dtype))
+  with pytest.raises(ValueError):
+    K.tgmm(cuda(lhs), cuda(dout), cuda(gs), out_row_scale=cuda(scale[:-1]))
+
+
 def test_tgmm_argument_errors(K):
   a = torch.zeros(16, 64, dtype=torch.bfloat16, device="cuda")
   gs = torch.tensor([16], dtype=torch.int32, device="cuda")
