@@ -398,3 +398,91 @@ def test_same_groups_flag_reuses_or_rebuilds_the_tile_list():
     y3 = K.gmm_raw(h2, w_down, gs, workspace=ws, same_groups=True)
     assert torch.equal(h2, K.gmm_raw(x, w_gate, gs, rhs_up=w_up, act="silu"))
     assert torch.equal(y3, K.gmm_raw(h2, w_down, gs))
+
+
+@pytest.mark.parametrize("family", ["bf16", "int8w", "int4", "int4g32", "mxfp4", "int8", "fp8"])
+def test_picked_kernel_against_the_tiled_kernel_on_random_large_shapes(K, family):
+  """12 random shapes per operand family at sizes where the library picks among all of its kernels (2 to 48 groups, 20
+  to 300 rows per group on average, uniform or Zipf-skewed with an empty group, rows in no group, K and N at the
+  direct-to-LDS kernels' granularity and off it, with and without the fused activation, rows read through an index, a
+  factor per result row, a window of the groups) against the register-staged tiled kernel on the same operands (which
+  the small-shape tests pin to the oracle).  The kernels add in the same order and agree bit for bit, except the
+  streaming kernel of the 4-bit formats, which sums per scale group first: there one bf16 step of the largest value."""
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
+
+  rng = np.random.default_rng(900 + sum(map(ord, family)))
+  g = torch.Generator(device="cuda").manual_seed(5)
+  rand = lambda *shape: torch.rand(*shape, device="cuda", generator=g)
+  randn = lambda *shape: torch.randn(*shape, device="cuda", generator=g)
+  bytes_ = lambda lo, hi, shape, dt: torch.randint(lo, hi, shape, device="cuda", dtype=dt, generator=g)
+  for case in range(12):
+    e = int(rng.integers(2, 49))
+    k = int(rng.integers(2, 20)) * 128 if family == "fp8" else int(rng.integers(4, 40)) * 64
+    n = int(rng.integers(2, 22)) * 128 if family == "fp8" else int(rng.integers(32, 360)) * 8
+    avg = int(rng.choice([20, 40, 60, 100, 120, 140, 300]))
+    if rng.random() < 0.4:
+      p = 1.0 / np.arange(1, e + 1) ** 1.2
+      gs = rng.multinomial(avg * e, p / p.sum())
+      rng.shuffle(gs)
+    else:
+      gs = rng.integers(0, 2 * avg + 1, e)
+    if e > 2:
+      gs[rng.integers(0, e)] = 0
+    m = max(int(gs.sum()) + int(rng.integers(0, 50)), 1)
+    glu = bool(rng.integers(0, 2))
+    kw = {}
+    lhs = randn(m, k).to(torch.bfloat16)
+    if family in ("int8w", "int8"):
+      ws = [(bytes_(-127, 128, (e, n, k), torch.int8), rand(e, n) * 0.01 + 1e-3) for _ in range(2)]
+      if family == "int8":
+        lhs = bytes_(-127, 128, (m, k), torch.int8)
+        kw["lhs_scale"] = rand(m) * 0.01 + 1e-3
+    elif family in ("int4", "int4g32"):
+      grp = 128 if family == "int4" else 32
+      ws = [(bytes_(0, 256, (e, n, k // 2), torch.uint8), (rand(e, n, (k + grp - 1) // grp) * 0.01 + 1e-3).to(torch.bfloat16)) for _ in range(2)]
+      kw.update(rhs_dtype=MOE_INT4, rhs_scale_block_k=grp)
+    elif family == "mxfp4":
+      ws = [(bytes_(0, 256, (e, n, k // 2), torch.uint8), bytes_(118, 126, (e, n, k // 32), torch.uint8)) for _ in range(2)]
+      kw.update(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+    elif family == "fp8":
+      lhs = (randn(m, k) * 2).to(torch.float8_e4m3fn)
+      kw.update(lhs_scale=rand(m, k // 128) * 0.02 + 1e-3, lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128)
+      ws = [((randn(e, n, k) * 2).to(torch.float8_e4m3fn), rand(e, n // 128, k // 128) * 0.02 + 1e-3) for _ in range(2)]
+    else:
+      ws = [((randn(e, n, k) * 0.05).to(torch.bfloat16), None) for _ in range(2)]
+    opts = []
+    if rng.random() < 0.5:  # rows read through an index: a source with fewer rows, each read several times or never
+      div = int(rng.integers(1, 4))
+      src = torch.randperm(m, device="cuda", generator=g)[: m // div + 1]
+      lhs = lhs[src].contiguous()
+      if "lhs_scale" in kw:
+        kw["lhs_scale"] = kw["lhs_scale"][src].contiguous()
+      kw.update(lhs_row_idx=cuda(rng.integers(0, (m // div + 1) * div, m).astype(np.int32)), lhs_row_idx_div=div, num_rows=m)
+      opts.append(f"index / {div}")
+    if rng.random() < 0.5:
+      kw["out_row_scale"] = rand(m) + 0.5
+      opts.append("row factor")
+    lo, hi = 0, int(gs.sum())
+    if rng.random() < 0.4 and e > 3:
+      off = int(rng.integers(0, e // 2))
+      loc = int(rng.integers(1, e - off + 1))
+      ws = [(w[off:off + loc].clone(), None if sc is None else sc[off:off + loc].clone()) for w, sc in ws]
+      kw["group_offset"] = off
+      lo, hi = int(gs[:off].sum()), int(gs[:off + loc].sum())
+      opts.append(f"groups {off} .. {off + loc - 1}")
+    if ws[0][1] is not None:
+      kw["rhs_scale"] = ws[0][1]
+    if glu:
+      kw.update(rhs_up=ws[1][0], act="silu")
+      if ws[1][1] is not None:
+        kw["rhs_up_scale"] = ws[1][1]
+    tag = f"{family} case {case}: m={m} k={k} n={n} glu={glu} {opts} group_sizes={gs.tolist()}"
+    got = K.gmm_raw(lhs, ws[0][0], cuda(gs.astype(np.int32)), **kw)
+    ref = K.gmm_raw(lhs, ws[0][0], cuda(gs.astype(np.int32)), kernel="tiled", **kw)
+    assert torch.all(got[:lo] == 0) and torch.all(got[hi:] == 0), tag  # rows of no group and of groups outside the window
+    if family in ("int4", "int4g32", "mxfp4"):
+      worst, top = float((got.float() - ref.float()).abs().max()), float(ref.float().abs().max())
+      # (a factor per row multiplies the rounded result and rounds again: one step before it can be two after it)
+      assert worst <= 2.0 ** (-6 if "out_row_scale" in kw else -7) * top, f"{tag}: {worst} of {top}"
+    else:
+      assert torch.equal(got, ref), tag
