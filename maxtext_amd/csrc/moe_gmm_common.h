@@ -303,8 +303,8 @@ __device__ __forceinline__ void load_epilogue_scales(EpilogueScales<TM, NT_OUT, 
 }
 
 // Writes a wave's results.  The MFMA leaves lane l with 4 consecutive channels of row l % MI: 8-byte stores, neighbouring
-// lanes in different rows.  (Passing each row tile through LDS so that consecutive lanes store consecutive 16 bytes was
-// measured and is slower: the epilogue is bound by what stands between the stores, not by the stores.)
+// lanes in different rows; the plain bf16 case pairs tiles and stores 16 bytes per lane (below).  (Passing each row tile
+// through LDS so that consecutive lanes store consecutive 16 bytes was measured and is slower.)
 // (I_END < TM: only the wave's first I_END row tiles hold rows of this tile.)
 template <int TM, int TN, int NT_OUT, bool GLU, int I_END = TM, typename acc_t>
 __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const EpilogueScales<TM, NT_OUT, GLU>& e,
@@ -329,6 +329,41 @@ __device__ __forceinline__ void store_epilogue(const acc_t (&acc)[TN][TM], const
   auto body = [&](auto act_c, auto general_c) {
     constexpr int ACT = decltype(act_c)::value;
     constexpr bool GENERAL = decltype(general_c)::value;
+    if constexpr (!GENERAL && MI == 16 && NT_OUT % 2 == 0) {
+      // Two neighbouring 16-channel tiles at a time: lanes 16 apart trade halves (lane (row, q) gives its 4 channels of the
+      // tile it does not keep and receives the neighbour's 4 of the one it keeps), so that every lane stores 16 bytes and a
+      // row's 64 bytes of the pair leave in one instruction: half the store instructions and half the write requests
+      // (256 x 256 int8 tiles, 14336-long K: 0.929 against 0.947 ms).
+#pragma unroll
+      for (int i = 0; i < I_END; i++) {
+        const int lr = row_base + i * MI + (lane % MI);
+        const bool row_ok = lr < tile.nrows;
+#pragma unroll
+        for (int j = 0; j < NT_OUT; j += 2) {
+          uint32_t pk[2][2];
+#pragma unroll
+          for (int t = 0; t < 2; t++) {
+            const float sg[4] = {e.sg[j + t][0].x, e.sg[j + t][0].y, e.sg[j + t][0].z, e.sg[j + t][0].w};
+            const float su[4] = {e.su[j + t][0].x, e.su[j + t][0].y, e.su[j + t][0].z, e.su[j + t][0].w};
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              const float g = fmaf((float)acc[j + t][i][r], e.sa[i] * sg[r], 0.f);
+              v[r] = GLU ? glu_act<ACT>(g, fmaf((float)acc[j + t + NT_OUT][i][r], e.sa[i] * su[r], 0.f), p.act_limit) : g;
+            }
+            pk[t][0] = pack_bf16x2(v[0], v[1]);
+            pk[t][1] = pack_bf16x2(v[2], v[3]);
+          }
+          const auto s0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
+          const auto s1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
+          const int qq = lane / 16;
+          const int n8 = n_base + (j + (qq & 1)) * 16 + 4 * (qq & ~1);
+          if (row_ok && n8 < p.N)
+            *(uint4*)((uint16_t*)p.out + (size_t)(tile.row0 + lr) * p.N + n8) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < I_END; i++) {
       const int lr = row_base + i * MI + (lane % MI);
