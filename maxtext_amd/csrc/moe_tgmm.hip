@@ -354,6 +354,25 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
   wait_vmcnt<0>();  // no request may still be writing LDS when the block ends
 
   // D[k][n]: the lane holds n = s16 and k = 4 * gq + r of each 16 x 16 tile
+  if (!p.out_f32 && !p.existing) {
+    // plain bf16 results: neighbouring k-tiles trade halves between lanes 16 apart, so that a lane stores 16 bytes and
+    // the 64 bytes of a row n leave in one instruction
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int n = n0 + wn * 128 + i * 16 + s16;
+      const float sc = p.n_scale ? p.n_scale[n] : 1.0f;
+#pragma unroll
+      for (int j = 0; j < 4; j += 2) {
+        const auto s0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(acc[j][i][0] * sc, acc[j][i][1] * sc),
+                                                         pack_bf16x2(acc[j + 1][i][0] * sc, acc[j + 1][i][1] * sc), false, false);
+        const auto s1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(acc[j][i][2] * sc, acc[j][i][3] * sc),
+                                                         pack_bf16x2(acc[j + 1][i][2] * sc, acc[j + 1][i][3] * sc), false, false);
+        const int k = k0 + wk * 64 + (j + (gq & 1)) * 16 + 4 * (gq & ~1);
+        *(uint4*)((uint16_t*)p.out + ((size_t)g_local * N + n) * K + k) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const int n = n0 + wn * 128 + i * 16 + s16;
