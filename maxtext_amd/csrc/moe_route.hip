@@ -570,7 +570,7 @@ __device__ __forceinline__ void quant_scale(float m, int rule, float& sc, float&
     inv = sc == 0.f ? 0.f : round_bf16_fn(1.0f / sc);
   } else {
     sc = m / qmax;
-    inv = 0.f;  // unused: this rule divides
+    inv = sc == 0.f ? 0.f : 1.0f / sc;  // this rule divides; the int8 path uses the reciprocal to find the values that need it
   }
 }
 
@@ -585,8 +585,15 @@ __device__ __forceinline__ float quant_value(float f, float sc, float inv, int r
     (void)is_static;
     return MODE == GQ_INT8 ? truncf(y) : y;
   }
-  float q = sc == 0.f ? 0.f : f / sc;
-  if (MODE == GQ_INT8) q = rintf(q);
+  if (MODE == GQ_INT8) {
+    // rint(f / sc) without dividing: f * (1 / sc) is off the rounded quotient by at most 1.2e-7 of its value, 2.4e-5
+    // for |q| < 200, so unless it lies within 1e-4 of k + 1/2 both round to the same integer; the few values that do lie
+    // there (and those beyond 200, NaN included) take the division.  sc == 0 has inv == 0 and gives 0.
+    float q = f * inv;
+    if (fabsf(__builtin_amdgcn_fractf(q) - 0.5f) < 1e-4f || !(fabsf(q) < 200.0f)) q = sc == 0.f ? 0.f : f / sc;
+    return fminf(fmaxf(rintf(q), -qmax), qmax);
+  }
+  const float q = sc == 0.f ? 0.f : f / sc;
   return fminf(fmaxf(q, -qmax), qmax);
 }
 
@@ -636,7 +643,7 @@ __global__ __launch_bounds__(kGqThreads) void gather_rows_kernel(
     // one scale for the whole tensor: bf16(scale) and its bf16 inverse for the v2 rule (:528-529), the value itself otherwise
     const float s = *qc.static_scale;
     row_sc = qc.rule == MOE_QUANT_V2 ? round_bf16_fn(s) : s;
-    row_inv = qc.rule == MOE_QUANT_V2 ? round_bf16_fn(1.0f / row_sc) : 0.f;
+    row_inv = qc.rule == MOE_QUANT_V2 ? round_bf16_fn(1.0f / row_sc) : row_sc == 0.f ? 0.f : 1.0f / row_sc;
   } else if (qc.block_lanes == 0) {
     float m = 0.f;
 #pragma unroll
