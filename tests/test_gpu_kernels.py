@@ -155,6 +155,35 @@ def test_gather_rows_int8_quant(K, d):
   assert torch.equal(q.cpu(), oq)
 
 
+def test_gather_rows_int8_quant_next_to_rounding_boundaries(K):
+  """Rows whose quotients x / scale sit on and right beside k + 1/2: the values are bf16((k + 1/2) * scale) for random k
+  and row maxima, so the quotients scatter within 2^-9 of the boundaries, thousands exactly on them, hundreds beside them
+  by less than 1e-4; the quantised values must equal the oracle's rint(x / scale) on every one
+  (the kernel multiplies by 1 / scale and divides only next to a boundary), also with a per-tensor static scale and
+  with a scale per 128-wide block."""
+  rng = np.random.default_rng(73)
+  rows, d = 96, 1024
+  amax = torch.from_numpy(np.concatenate([[127.0, 254.0, 63.5, 1e-3, 3e4], rng.uniform(0.01, 300.0, rows - 5)]).astype(np.float32)).to(torch.bfloat16).float()
+  scale = amax / 127.0
+  k = torch.from_numpy(rng.integers(-127, 127, (rows, d)).astype(np.float32)) + 0.5
+  x = (k * scale[:, None]).to(torch.bfloat16)
+  x[:, 0] = amax.to(torch.bfloat16)  # the row maximum itself, so that the scale is the intended one
+  oq, os_ = O.quantize_rows_int8(x)
+  assert torch.equal(os_, scale)
+  frac = (x.float() / os_[:, None]).double() % 1.0
+  assert int(((frac - 0.5).abs() < 1e-4).sum()) > 1000 and int((frac == 0.5).sum()) > 100  # the cases meant are there
+  q, s = K.gather_rows(cuda(x), None, 1, out_dtype=torch.int8)
+  assert torch.equal(s.cpu(), os_) and torch.equal(q.cpu(), oq)
+  qb, sb = K.gather_rows(cuda(x), None, 1, out_dtype=torch.int8, block_k=128)
+  ob, osb = O.quantize_rows_int8(x.reshape(rows * (d // 128), 128))
+  assert torch.equal(sb.cpu().reshape(-1), osb) and torch.equal(qb.cpu().reshape(-1, 128), ob)
+  static = torch.tensor([0.37], dtype=torch.float32)
+  xs = ((k[:8] * 0.37).clamp(-60, 60)).to(torch.bfloat16)
+  qs, _ = K.gather_rows(cuda(xs), None, 1, out_dtype=torch.int8, static_scale=cuda(static))
+  want = torch.clamp(torch.round(xs.float() / static), -127, 127).to(torch.int8)
+  assert torch.equal(qs.cpu(), want)
+
+
 @pytest.mark.parametrize("d", [128, 2048, 7168, 2880])
 def test_gather_rows_fp8_block_quant(K, d):
   g = torch.Generator().manual_seed(d + 2)
