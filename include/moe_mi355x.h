@@ -45,8 +45,10 @@ typedef enum {
   MOE_FP8_E4M3 = 2, /* OCP float8_e4m3fn (max 448), layers/quantizations.py:237      */
   MOE_INT4 = 3,     /* 2 per byte along K, first value in the low nibble, stored +8  */
   MOE_F32 = 4,
-  MOE_MXFP4 = 5    /* OCP MX fp4: e2m1 values, 2 per byte along K (first in the low nibble), one e8m0 scale
+  MOE_MXFP4 = 5,   /* OCP MX fp4: e2m1 values, 2 per byte along K (first in the low nibble), one e8m0 scale
                       byte 2^(s-127) per 32 values (dequantize_mxfp4.py:46-72) */
+  MOE_FP8_E5M2 = 6 /* OCP float8_e5m2 (max 57344): the gradient type of the fp8_full recipe's backward
+                      (bwd_qtype, layers/quantizations.py:234-250, kernels/megablox/ops.py:583-604); lhs of moe_gmm only */
 } moe_dtype;
 
 typedef enum {
@@ -252,7 +254,7 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  * (reference_gmm, tests/unit/pallas_mosaic_tpu_v2_kernel_test.py:139-141).
  *
  * Operand layouts in HBM
- *   lhs        [M, K] row-major ([lhs_rows, K] with lhs_row_idx), lhs_dtype in {BF16, INT8, FP8_E4M3}
+ *   lhs        [M, K] row-major ([lhs_rows, K] with lhs_row_idx), lhs_dtype in {BF16, INT8, FP8_E4M3, FP8_E5M2}
  *   lhs_scale  f32: NULL (bf16 lhs) | [M] one per row (lhs_scale_block_k == 0; qpl.quantize channelwise_axes=[0],
  *              ops.py:241-248) | [1] one for the tensor (lhs_scale_block_k == MOE_SCALE_PER_TENSOR; the static (1, 1)
  *              lhs_scale of gmm_v2, ops.py:333-360) | [M, ceil(K / b)] one per row and b values of K
@@ -285,6 +287,8 @@ MOE_API int moe_gather_rows(const void* x, const int32_t* row_idx, int idx_div, 
  *     lhs per row or per tensor  x  rhs per channel or per tensor over all of K (what gmm() quantises to, ops.py:232-267)
  *     lhs per row / per tensor / [M, K/b]  x  rhs KMAJOR per channel [G, nkb, N] (gmm_v2's layouts; K % 128 == 0)
  *     FP8 only: lhs [M, K/128]  x  rhs 128 x 128 blocks [G, N/128, K/128] (DeepSeek-V3 checkpoints)
+ *   FP8_E5M2 x FP8 (the quantised gradient against the forward's e4m3 weights, ops.py:583-642): lhs per row or per
+ *     tensor x rhs per channel or per tensor, without rhs_up, on shapes moe_gmm_lhs_e5m2_supported() accepts
  * Alignment: K % 32 == 0 (INT4, MXFP4), K % 16 == 0 otherwise; N % 8 == 0; pointers 16-byte aligned.
  */
 #define MOE_SCALE_PER_TENSOR (-1)
@@ -360,6 +364,10 @@ typedef struct {
 /* 1 when moe_gmm takes MOE_GMM_RHS_KN for this shape (K % 64 == 0, N % 256 == 0, 128 rows per group on average and
  * enough 256 x 256 tiles to fill the chip), else 0. */
 MOE_API int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total);
+/* 1 when moe_gmm takes MOE_FP8_E5M2 activations for this shape (the persistent 256 x 256 kernel: K % 128 == 0, K >= 384,
+ * N * K < 2^32, 128 rows per group on average and enough tiles to fill the chip), else 0: widen the gradient to bf16
+ * (moe_bwd_scale_grad with quantize == 1) and the weights with it. */
+MOE_API int moe_gmm_lhs_e5m2_supported(int M, int K, int N, int num_groups_total);
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
 MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);
 
@@ -495,7 +503,7 @@ MOE_API int moe_add_group_bias(const void* h, int M, int N, const float* bias, c
                        int num_groups_local, int group_offset, void* out, void* stream);
 
 /* ---------------------------------------------------------------------------
- * Gradient preparation of the quantised backward pass (int8 x int8 forward with channelwise scales): the incoming
+ * Gradient preparation of the quantised backward pass (int8 x int8 or fp8 x fp8 forward with channelwise scales): the incoming
  * gradient times the scale of the axis that the gradient product contracts away (_bwd_prepare_inputs,
  * kernels/megablox/ops.py:530-580), optionally quantised to float8_e5m2 (_bwd_quantize_gradient, ops.py:583-604;
  * symmetric absmax scale = absmax / 57344, values rounded to nearest even, a zero scale gives zeros).
@@ -507,7 +515,8 @@ MOE_API int moe_add_group_bias(const void* h, int M, int N, const float* bias, c
  *                     scale_out [N] (group_sizes is not used)
  *
  *   dout [M, N] bf16;  out [M, N] bf16: d itself (quantize == 0; scale_out is not touched), or d / scale on the e5m2
- *   grid, whose values are exact in bf16 (quantize != 0), so that moe_gmm / moe_tgmm take it as a bf16 operand.
+ *   grid, whose values are exact in bf16 (quantize == 1), so that moe_gmm / moe_tgmm take it as a bf16 operand;
+ *   quantize == 2: out [M, N] holds the same values as float8_e5m2 bytes, the MOE_FP8_E5M2 lhs of moe_gmm.
  * Limits: N % 8 == 0, N <= 16384, at most 1024 groups.
  */
 typedef enum { MOE_BWD_FOR_DLHS = 0, MOE_BWD_FOR_DRHS = 1 } moe_bwd_mode;

@@ -14,7 +14,7 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MOE_MI355X_LIB") or os.path.join(_PKG, "lib", "libmoe_mi355x.so")
 
 # enums of include/moe_mi355x.h
-MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32, MOE_MXFP4 = 0, 1, 2, 3, 4, 5
+MOE_BF16, MOE_INT8, MOE_FP8_E4M3, MOE_INT4, MOE_F32, MOE_MXFP4, MOE_FP8_E5M2 = 0, 1, 2, 3, 4, 5, 6
 MOE_ROUTE_SOFTMAX_TOPK, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_TOPK_RAW, MOE_ROUTE_SOFTMAX_ALL = 0, 1, 2, 3
 ROUTE_BY_NAME = {"softmax_topk": 0, "deepseek": 1, "topk_raw": 2, "softmax_all": 3}
 MOE_ACT_NONE, MOE_ACT_SILU, MOE_ACT_SWIGLUOAI, MOE_ACT_SILU_CLIP = 0, 1, 2, 3
@@ -92,6 +92,7 @@ SIGNATURES = {
                                 c_void_p]),
     "moe_gmm_workspace_bytes": (c_size_t, [c_int, c_int]),
     "moe_gmm_rhs_kn_supported": (c_int, [c_int, c_int, c_int, c_int]),
+    "moe_gmm_lhs_e5m2_supported": (c_int, [c_int, c_int, c_int, c_int]),
     "moe_gmm": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
     "moe_gmm_tuned": (c_int, [ctypes.POINTER(GmmArgs), c_int, c_int, c_void_p]),
     "moe_gmm_static_ws": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),

@@ -1,7 +1,8 @@
 // Gradient preparation of the quantised backward pass: the incoming gradient times the scale of the axis the product
 // contracts away (_bwd_prepare_inputs, kernels/megablox/ops.py:530-580), optionally quantised to float8_e5m2 per row or
 // per column (_bwd_quantize_gradient, ops.py:583-604).  The e5m2 values are written as bf16, in which they are exact, so
-// both gradient products run on the bf16 kernels.
+// that both gradient products can run on the bf16 kernels, or as float8_e5m2 bytes for the fp8 MFMA (e5m2 gradient x
+// e4m3 weights).
 
 #include "moe_common.h"
 
@@ -33,6 +34,29 @@ __device__ __forceinline__ float to_e5m2_grid(float x, float scale) {
   return copysignf(r, q);
 }
 
+// A value on the e5m2 grid as its float8_e5m2 byte: the upper byte of the IEEE half of the same value (e5m2 is a half
+// with 8 mantissa bits dropped; every grid value, inf and nan included, converts exactly).
+__device__ __forceinline__ uint32_t e5m2_byte(float on_grid) {
+  const _Float16 h = (_Float16)on_grid;
+  return (uint32_t)(__builtin_bit_cast(uint16_t, h) >> 8);
+}
+
+// 8 results of one lane: bf16 (16 bytes at `out` + 16 * idx) or, BYTES, float8_e5m2 (8 bytes at `out` + 8 * idx)
+template <bool BYTES>
+__device__ __forceinline__ void store8(void* out, size_t idx, const float (&o)[8]) {
+  if (BYTES) {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      lo |= e5m2_byte(o[e]) << (8 * e);
+      hi |= e5m2_byte(o[4 + e]) << (8 * e);
+    }
+    ((uint2*)out)[idx] = make_uint2(lo, hi);
+  } else {
+    ((uint4*)out)[idx] = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+  }
+}
+
 // expert of row m as the reference's backward sees it: the number of group ends <= m, taken relative to the first
 // local group and clamped to the local range (rows of other shards and rows past the last group take the nearest
 // local expert: their gradient rows do not reach the result)
@@ -52,9 +76,9 @@ constexpr int kBwdMaxGroups = 1024;
 
 // One block per row: d = bf16(dout * bf16(factor)), factor = rhs_scale[group(row), n] (BY_CHANNEL) or lhs_scale[row];
 // ROW_QUANT: the row's absmax, then the e5m2 values and the row's scale.
-template <bool BY_CHANNEL, bool ROW_QUANT>
+template <bool BY_CHANNEL, bool ROW_QUANT, bool BYTES = false>
 __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4* dout, int N, const float* factor, const int* group_sizes,
-                                                                     int G_total, int G_local, int group_offset, uint4* out,
+                                                                     int G_total, int G_local, int group_offset, void* out,
                                                                      float* scale_out) {
   __shared__ int ends[BY_CHANNEL ? kBwdMaxGroups : 1];
   __shared__ uint32_t wmax[kBwdThreads / kWave];
@@ -65,7 +89,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4
     if (tid == 0) {
       int run = 0;
       for (int g = 0; g < G_total; g++) {
-        run += group_sizes[g];
+        run += max(group_sizes[g], 0);
         ends[g] = run;
       }
     }
@@ -109,7 +133,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4
       float o[8];
 #pragma unroll
       for (int e = 0; e < 8; e++) o[e] = ROW_QUANT ? to_e5m2_grid(v[c][e], s) : v[c][e];
-      out[(size_t)m * nvec + i] = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+      store8<BYTES>(out, (size_t)m * nvec + i, o);
     }
   }
 }
@@ -146,7 +170,8 @@ __global__ void bwd_clear_kernel(uint32_t* p, int n) {
 }
 
 // d on the e5m2 grid of its column's scale; `colmax` still holds the maxima
-__global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4* dout, int M, int N, const float* lhs_scale, const float* colmax, uint4* out) {
+template <bool BYTES>
+__global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4* dout, int M, int N, const float* lhs_scale, const float* colmax, void* out) {
   const int nvec = N / 8;
   const int i = blockIdx.x * kBwdThreads + threadIdx.x;
   if (i >= nvec) return;
@@ -161,7 +186,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4*
     float o[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) o[e] = to_e5m2_grid(round_bf16_fn(bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu) * fm), s[e]);
-    out[(size_t)m * nvec + i] = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]), pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+    store8<BYTES>(out, (size_t)m * nvec + i, o);
   }
 }
 
@@ -218,7 +243,9 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
   if (!dout || !factor || !out) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: NULL pointer");
   if (M < 0 || N <= 0) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad sizes");
   if (mode != MOE_BWD_FOR_DLHS && mode != MOE_BWD_FOR_DRHS) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad mode %d", mode);
+  if (quantize < 0 || quantize > 2) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: quantize must be 0, 1 (e5m2 values as bf16) or 2 (float8_e5m2 bytes)");
   if (quantize && !scale_out) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: the quantised gradient needs a scale buffer");
+  const bool bytes = quantize == 2;
   if (N % 8 != 0 || N > kBwdThreads * kBwdMaxChunks * 8) return fail(MOE_ERR_UNSUPPORTED, "bwd_scale_grad: need N%%8==0 and N<=16384 (N=%d)", N);
   if (M == 0) return MOE_OK;
   hipStream_t s = (hipStream_t)stream;
@@ -226,14 +253,16 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
   if (mode == MOE_BWD_FOR_DLHS) {
     if (!group_sizes || num_groups_total <= 0 || num_groups_total > kBwdMaxGroups || num_groups_local <= 0 || group_offset < 0)
       return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad groups (at most %d)", kBwdMaxGroups);
-    if (quantize)
-      bwd_scale_rows_kernel<true, true><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, (uint4*)out, scale_out);
+    if (bytes)
+      bwd_scale_rows_kernel<true, true, true><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, out, scale_out);
+    else if (quantize)
+      bwd_scale_rows_kernel<true, true><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, out, scale_out);
     else
-      bwd_scale_rows_kernel<true, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, (uint4*)out, scale_out);
+      bwd_scale_rows_kernel<true, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, out, scale_out);
     return check_launch("bwd_scale_rows_kernel");
   }
   if (!quantize) {
-    bwd_scale_rows_kernel<false, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, nullptr, 0, 0, 0, (uint4*)out, scale_out);
+    bwd_scale_rows_kernel<false, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, nullptr, 0, 0, 0, out, scale_out);
     return check_launch("bwd_scale_rows_kernel");
   }
   // per column: clear the maxima, take them, quantise with them, turn them into the scales
@@ -242,7 +271,8 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
   if (grid.y > 65535) return fail(MOE_ERR_UNSUPPORTED, "bwd_scale_grad: too many rows (%d)", M);
   bwd_clear_kernel<<<cdiv(N, 256), 256, 0, s>>>((uint32_t*)scale_out, N);
   bwd_col_absmax_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, (uint32_t*)scale_out);
-  bwd_col_quant_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, (uint4*)out);
+  if (bytes) bwd_col_quant_kernel<true><<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, out);
+  else bwd_col_quant_kernel<false><<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, out);
   bwd_col_scale_kernel<<<cdiv(N, 256), 256, 0, s>>>(scale_out, N);
   return check_launch("bwd_col_quant_kernel");
 }

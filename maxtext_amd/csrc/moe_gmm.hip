@@ -171,6 +171,13 @@ int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total) {
   return (long long)max_tiles_for(M, num_groups_total, 256) * (N / 256) >= 128 ? 1 : 0;
 }
 
+int moe_gmm_lhs_e5m2_supported(int M, int K, int N, int num_groups_total) {
+  // the rule by which moe_gmm sends fp8 operands with epilogue scales to the persistent stream kernel
+  if (M <= 0 || K <= 0 || N <= 0 || num_groups_total <= 0 || N % 8 != 0) return 0;
+  if (!dls_takes(OP_F8, K, N, 0) || (long long)N * K >= (1LL << 31) || (long long)M < 128LL * num_groups_total) return 0;
+  return (long long)max_tiles_for(M, num_groups_total, 256) * cdiv(N, 256) >= 128 ? 1 : 0;
+}
+
 size_t moe_gmm_workspace_bytes(int M, int num_groups_total) {
   if (M < 0 || num_groups_total <= 0) return 0;
   return 16 + (size_t)max_tiles_for(M, num_groups_total, 16) * sizeof(TileInfo);
@@ -217,7 +224,10 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   int32_t* header = (int32_t*)workspace;
   TileInfo* tiles = (TileInfo*)((uint8_t*)workspace + 16);
   const int M = a->M, K = a->K, N = a->N, G = a->num_groups_total;
-  const int L = a->lhs_dtype, R = a->rhs_dtype;
+  // float8_e5m2 activations (the quantised gradient of the backward, ops.py:583-604) against e4m3 weights: the fp8 path
+  // with the other format selector on the MFMA's activation operand; only the persistent stream kernel carries it
+  const bool lhs_e5m2 = a->lhs_dtype == MOE_FP8_E5M2;
+  const int L = lhs_e5m2 ? MOE_FP8_E4M3 : a->lhs_dtype, R = a->rhs_dtype;
   const bool kmajor = (a->flags & MOE_GMM_RHS_SCALE_KMAJOR) != 0, shared = (a->flags & MOE_GMM_RHS_SCALE_SHARED) != 0;
   const int bn = a->rhs_scale_block_n, rbk = a->rhs_scale_block_k, lbk = a->lhs_scale_block_k;
   auto map_tiles = [&](int bm) {
@@ -234,7 +244,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   const bool quant_pair = (L == MOE_INT8 && R == MOE_INT8) || (L == MOE_FP8_E4M3 && R == MOE_FP8_E4M3);
   ScalePlan sp = {};
   // DeepSeek block scales: fp8 with [M, K/128] x [G, N/128, K/128]
-  const bool fp8_blocks = L == MOE_FP8_E4M3 && R == MOE_FP8_E4M3 && lbk == 128 && bn == 128 && rbk == 128 && !kmajor && !shared;
+  const bool fp8_blocks = !lhs_e5m2 && L == MOE_FP8_E4M3 && R == MOE_FP8_E4M3 && lbk == 128 && bn == 128 && rbk == 128 && !kmajor && !shared;
   if (quant_pair && !fp8_blocks) {
     if (!a->lhs_scale || !a->rhs_scale || (glu && !a->rhs_up_scale)) return fail(MOE_ERR_INVALID_ARG, "gmm: quantised operands need their scales");
     if (lbk == 0) { sp.lhs_epi = a->lhs_scale; sp.lhs_epi_stride = 1; }
@@ -273,13 +283,32 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     const bool few_rows = (long long)M <= 16LL * G;
     const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > 14LL * G : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
+    // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
+    const bool chip_full = (long long)max_tiles_for(M, G, 256) * cdiv(N, glu ? 128 : 256) >= 128;
+    const bool prefill = kernel == MOE_GMM_KERNEL_BIG || (kernel == MOE_GMM_KERNEL_AUTO && (long long)M >= 128LL * G && chip_full);
+    // scales in the epilogue only (per row / per tensor x per channel / per tensor): the int8 x int8 problem on another MFMA
+    const bool stream_epi = !fp8_blocks && prefill && dls_takes(OP_F8, K, N, ro.row_idx ? ro.lhs_rows : 0);
+    if (lhs_e5m2 && !stream_epi)
+      return fail(MOE_ERR_UNSUPPORTED, "gmm: float8_e5m2 activations run on the persistent 256 x 256 kernel only (128 rows per group on average, "
+                  "K %% 128 == 0, K >= 384, no rhs_up, no K-block scales); widen them to bf16 for other shapes");
+    if (stream_epi) {
+      if (lhs_e5m2 && glu) return fail(MOE_ERR_UNSUPPORTED, "gmm: float8_e5m2 activations take no rhs_up");
+      map_tiles(256);
+      TiledParams q = {};
+      q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
+      q.rhs_bias = a->rhs_bias; q.rhs_up_bias = a->rhs_up_bias;
+      q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
+      q.header = header; q.tiles = tiles; q.out = a->out;
+      q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.tune = raster; q.ro = ro;
+      q.lhs_scale = sp.lhs_epi; q.lhs_scale_stride = sp.lhs_epi_stride;
+      q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
+      q.rhs_scale_gstride = sp.rhs_gstride; q.rhs_scale_nstride = sp.rhs_nstride;
+      return launch_dls(OP_F8, glu, q, M, G, s, lhs_e5m2 ? 1 : 0);
+    }
     if (tiled) {
       const bool big = kernel == MOE_GMM_KERNEL_BIG;
       if (big && !fp8_blocks) return fail(MOE_ERR_UNSUPPORTED, "gmm: the 256 x 256 fp8 kernel takes block-scaled operands only");
-      // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
-      const bool chip_full = (long long)max_tiles_for(M, G, 256) * cdiv(N, glu ? 128 : 256) >= 128;
-      const bool stream = fp8_blocks && f8s_takes(K, N, M, ro.row_idx ? ro.lhs_rows : 0) &&
-                          (big || (kernel == MOE_GMM_KERNEL_AUTO && (long long)M >= 128LL * G && chip_full));
+      const bool stream = fp8_blocks && f8s_takes(K, N, M, ro.row_idx ? ro.lhs_rows : 0) && prefill;
       map_tiles(big || stream ? 256 : 128);
       Fp8TiledParams P = {};
       TiledParams& q = P.base;

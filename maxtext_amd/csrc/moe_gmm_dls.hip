@@ -1,5 +1,6 @@
-// Grouped matmul: the persistent 256 x 256 kernel for operands that need no conversion (int8 x int8, bf16 x bf16
-// prefill) with the stages of a block's consecutive tiles as ONE request stream.
+// Grouped matmul: the persistent 256 x 256 kernel for operands that need no conversion (int8 x int8, bf16 x bf16 and
+// fp8 x fp8 with per-row x per-channel scales, prefill) with the stages of a block's consecutive tiles as ONE request
+// stream.
 //
 // Both operands go global -> LDS without passing through registers (buffer_load ... lds, 1 KB = 8 rows of 128 bytes per
 // wave instruction; XOR-swizzled unpadded rows; two buffers of 64 KB; one barrier per stage).  8 waves as 2 x 4, each
@@ -12,23 +13,34 @@
 // zeros, the lane-dependent part of an address is the same for every tile and the tile-dependent part is scalar, so
 // moving the stream on to the next tile costs no vector work (with a row index: one index load per request).  What is
 // left between two tiles is the epilogue.
+//
+// fp8 (e4m3 weights, e4m3 or e5m2 activations; scales per row / per tensor x per channel / per tensor, applied in the
+// epilogue: what gmm() quantises to, kernels/megablox/ops.py:232-267, and the e5m2 gradient times e4m3 weights of its
+// backward, ops.py:583-604) runs the same stream on v_mfma_f32_16x16x128_f8f6f4: a 128-byte stage is ONE instruction per
+// 16 x 16 tile.  An operand fragment of that instruction is 8 registers, so only 4 of a wave's 8 activation fragments
+// and its 4 weight fragments are live beside the 128 accumulators, and a stage is multiplied in two halves of 16 MFMAs:
+// row tiles 0 .. 3 fragment by fragment (each slot reloaded with row tile + 4 after its four MFMAs), then row tiles
+// 4 .. 7 weight fragment by weight fragment (each reloaded with the next stage's after its four MFMAs, the activation
+// slots during the last four).  The stage barrier sits between the halves.
 
 #include "moe_gmm_common.h"
 
 namespace moe {
 
-template <int OP_, bool GLU_>
+template <int OP_, bool GLU_, int LF_ = 0>
 struct DlsCfg {
   static constexpr int OP = OP_;
   static constexpr bool GLU = GLU_;
+  static constexpr int LF = LF_;  // fp8 activations: 0 = e4m3, 1 = e5m2 (format selector of the MFMA's second operand)
   static constexpr int BM = 256, BN = 256, BKB = 128, MI = 16;
-  static constexpr int ESZ = OP == OP_I8 ? 1 : 2, BK = BKB / ESZ;
+  static constexpr int ESZ = OP == OP_BF16 ? 2 : 1, BK = BKB / ESZ;
   static constexpr int WAVES_M = 2, WAVES_N = 4, NWAVES = 8, THREADS = NWAVES * kWave;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / MI, TN = WN / MI;
   static constexpr int A_STAGE = BM * BKB, STAGE = (BM + BN) * BKB, LDS_BYTES = 2 * STAGE;
   static constexpr int A_IPW = BM / 8 / NWAVES, B_IPW = BN / 8 / NWAVES;  // requests per wave and stage: 4 + 4
   static constexpr int OUT_BN = GLU ? BN / 2 : BN;
-  static_assert(OP == OP_I8 || OP == OP_BF16, "operands");
+  static_assert(OP == OP_I8 || OP == OP_BF16 || OP == OP_F8, "operands");
+  static_assert(LF == 0 || OP == OP_F8, "only fp8 activations come in two formats");
   __device__ static __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 };
 
@@ -93,9 +105,10 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParam
     else dma16_buffer(b_desc, b_voff[idx - C::A_IPW], b_soff + (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + C::A_STAGE + (wave * C::B_IPW + idx - C::A_IPW) * 1024);
   };
 
-  // ---- the multiplying side ----------------------------------------------------------------------------------------
-  typedef typename std::conditional<OP == OP_I8, v4i, v4f>::type acc_t;
-  acc_t acc[C::TN][C::TM];
+
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
   int b_row[C::TN];
 #pragma unroll
   for (int j = 0; j < C::TN; j++) {
@@ -106,8 +119,124 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParam
       b_row[j] = wn * C::WN + j * C::MI;
     }
   }
-  // fragment of k-step ks: row (lane % 16), chunk q = 4 * ks + lane / 16, stored at slot q ^ swz(row)
+  // fragment of a 64-byte k-step ks: row (lane % 16), chunk q = 4 * ks + lane / 16, stored at slot q ^ swz(row)
   const int frag_lane = (lane % 16) * C::BKB + (((lane / 16) ^ C::swz(lane % 16)) << 4);
+
+  if constexpr (OP == OP_F8) {
+    // ---- the multiplying side, fp8 ---------------------------------------------------------------------------------
+    constexpr int RING = C::TM / 2;
+    static_assert(C::TM == 8 && C::TN == 4, "the two halves of a stage");
+    v4f acc[C::TN][C::TM];
+    // fragment: row (lane % 16), K bytes 16 q .. and 64 + 16 q .. with q = lane / 16 (both operands alike, so the order
+    // of K inside the instruction does not matter)
+    v8i ga[RING], gb[C::TN];
+    auto read_frag = [&](v8i& f, const uint8_t* src) {
+      const v4i lo = *(const v4i*)(src + frag_lane), hi = *(const v4i*)(src + (frag_lane ^ 64));
+      f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
+      f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
+    };
+    auto read_a = [&](int buf, int i, int slot) { read_frag(ga[slot], smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB); };
+    auto read_b = [&](int buf, int j) { read_frag(gb[j], smem + buf * C::STAGE + C::A_STAGE + b_row[j] * C::BKB); };
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    // First half of a stage (in buffer buf): row tiles 0 .. 3 from the ring, each slot reloaded with row tile + 4.
+    // ZC: the tile's first stage starts from zero.
+    auto half_lo = [&](auto zc_c, int buf) {
+      constexpr bool ZC = decltype(zc_c)::value;
+#pragma unroll
+      for (int t = 0; t < 16; t++) {
+        const int i = t / 4, j = t % 4;
+        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(gb[j], ga[i], ZC ? zero : acc[j][i], 0, C::LF, 0, 127, 0, 127);
+        if (j == 3) read_a(buf, i + RING, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // Second half: row tiles 4 .. 7 (in the ring), weight fragment by weight fragment.  RD: the next stage (buffer
+    // rd_buf) is prepared behind it, its weight fragments and its row tiles 0 .. 3.  The eight requests of stage ld_kt go
+    // out into ld_buf, one per MFMA from the start.
+    auto half_hi = [&](auto rd_c, auto zc_c, int rd_buf, int ld_kt, int ld_buf) {
+      constexpr bool RD = decltype(rd_c)::value, ZC = decltype(zc_c)::value;
+#pragma unroll
+      for (int t = 0; t < 16; t++) {
+        const int j = t / 4, ii = t % 4;
+        acc[j][RING + ii] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(gb[j], ga[ii], ZC ? zero : acc[j][RING + ii], 0, C::LF, 0, 127, 0, 127);
+        if (t < C::A_IPW + C::B_IPW) issue_one(ld_kt, ld_buf, t);
+        if (RD && ii == 3) read_b(rd_buf, j);
+        if (RD && j == 3) read_a(rd_buf, ii, ii);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    auto first_fragments = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < RING; i++) read_a(buf, i, i);
+#pragma unroll
+      for (int j = 0; j < C::TN; j++) read_b(buf, j);
+    };
+
+    Tile cur, nxt;
+    if (!resolve(peek_from(blockIdx.x), cur)) return;
+    set_a_sources(cur);
+    set_b_sources(cur);
+#pragma unroll
+    for (int s = 0; s < 2; s++)
+#pragma unroll
+      for (int i = 0; i < C::A_IPW + C::B_IPW; i++) issue_one(s, s, i);
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    first_fragments(0);
+
+    int base = 0;  // the buffer that holds stage 0 of the current tile
+    while (true) {
+      Peek pk = peek_from(cur.id + gridDim.x);
+      bool have_n = false;
+      const int n_out0 = cur.n0 + (C::GLU ? wn * (C::WN / 2) : wn * C::WN);
+      EpilogueScales<C::TM, NT_OUT, C::GLU> esc;
+      half_lo(T_{}, base);
+      // Iteration `it`: the second half of stage it, then the first half of stage it + 1 (the schedule of the int8 / bf16
+      // loop below with halves of a stage in place of its k-steps).
+      auto stream_kt = [&](int s) { return s < nk ? s : (have_n ? s - nk : nk - 1); };
+      int cb = base;
+      auto iteration = [&](int it, auto last_c, auto zc_c) {
+        constexpr bool LAST = decltype(last_c)::value;
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        wait_vmcnt<0>();
+        asm volatile("s_barrier" ::: "memory");
+        if (LAST) {
+          half_hi(F_{}, zc_c, 0, stream_kt(it + 2), cb);
+        } else {
+          half_hi(T_{}, zc_c, cb ^ 1, stream_kt(it + 2), cb);
+          half_lo(F_{}, cb ^ 1);
+        }
+        cb ^= 1;
+      };
+      iteration(0, F_{}, T_{});
+      for (int it = 1; it < nk - 2; it++) iteration(it, F_{}, F_{});
+      have_n = resolve(pk, nxt);
+      if (have_n) {
+        set_a_sources(nxt);
+        set_b_sources(nxt);
+      }
+      iteration(nk - 2, F_{}, F_{});
+      iteration(nk - 1, T_{}, F_{});
+      // (the sums are pinned to this point: their only readers sit behind the branches of the epilogue, and the compiler
+      // otherwise moves the last MFMAs of every chain down there, away from the requests and reads they overlap, parking
+      // the fragments in scratch memory on the way)
+#pragma unroll
+      for (int j = 0; j < C::TN; j++)
+#pragma unroll
+        for (int i = 0; i < C::TM; i++) asm volatile("" : "+v"(acc[j][i]));
+      load_epilogue_scales<C::TM, NT_OUT, C::GLU, true, C::MI>(esc, p, cur.info, wm * C::WM, n_out0, lane);
+      store_epilogue<C::TM, C::TN, NT_OUT, C::GLU>(acc, esc, p, cur.info, wm * C::WM, n_out0, lane);
+      if (!have_n) break;
+      cur = nxt;
+      base = cb;
+      first_fragments(base);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    wait_vmcnt<0>();
+  } else {
+  // ---- the multiplying side, int8 / bf16 ------------------------------------------------------------------------
+  typedef typename std::conditional<OP == OP_I8, v4i, v4f>::type acc_t;
+  acc_t acc[C::TN][C::TM];
   v4i ga[C::TM], gb[2][C::TN];
   auto read_a = [&](int buf, int ks, int i) {
     ga[i] = *(const v4i*)(smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB + (frag_lane ^ (ks * 64)));
@@ -140,11 +269,8 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParam
       }
     }
   };
-  using T_ = std::true_type;
-  using F_ = std::false_type;
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
-  constexpr int NT_OUT = C::GLU ? C::TN / 2 : C::TN;
 
   // The fragments of a tile's first k-step (stage 0 in buffer `buf`), with nothing to hide behind.
   auto first_fragments = [&](int buf) {
@@ -216,6 +342,7 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParam
   // nothing may still be writing LDS when the block ends
   __builtin_amdgcn_s_waitcnt(0xC07F);
   wait_vmcnt<0>();
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -233,6 +360,9 @@ int prepare_dls() {
   if (!st) st = prepare_dls_cfg<DlsCfg<OP_I8, true>>();
   if (!st) st = prepare_dls_cfg<DlsCfg<OP_BF16, false>>();
   if (!st) st = prepare_dls_cfg<DlsCfg<OP_BF16, true>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, false>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, true>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, false, 1>>();
   return st;
 }
 
@@ -258,14 +388,19 @@ static int launch_dls_cfg(const TiledParams& p0, int M, int G_total, hipStream_t
 bool dls_takes(int op, int K, int N, long long indexed_lhs_rows) {
   // whole 128-byte stages, at least three of them (the stream looks two stages ahead, into the next tile at most); byte
   // offsets inside one expert's weight matrix and inside the activations that a row index may address fit 32 bits
-  const long long esz = op == OP_I8 ? 1 : 2;
-  return (op == OP_I8 || op == OP_BF16) && (K * esz) % 128 == 0 && K * esz >= 384 && (long long)N * K * esz < (1LL << 32) &&
+  const long long esz = op == OP_BF16 ? 2 : 1;
+  return (op == OP_I8 || op == OP_BF16 || op == OP_F8) && (K * esz) % 128 == 0 && K * esz >= 384 && (long long)N * K * esz < (1LL << 32) &&
          indexed_lhs_rows * K * esz < (1LL << 32);
 }
 
-int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s) {
+int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s, int lhs_e5m2) {
   if (!dls_takes(op, p.K, p.N, p.ro.row_idx ? p.ro.lhs_rows : 0))
-    return fail(MOE_ERR_UNSUPPORTED, "gmm: the stream kernel needs int8 or bf16 operands, whole 128-byte stages (three or more) and 32-bit byte offsets");
+    return fail(MOE_ERR_UNSUPPORTED, "gmm: the stream kernel needs int8, bf16 or fp8 operands, whole 128-byte stages (three or more) and 32-bit byte offsets");
+  if (lhs_e5m2 && (op != OP_F8 || glu)) return fail(MOE_ERR_UNSUPPORTED, "gmm: e5m2 activations run against e4m3 weights without rhs_up");
+  if (op == OP_F8) {
+    if (lhs_e5m2) return launch_dls_cfg<DlsCfg<OP_F8, false, 1>>(p, M, G_total, s);
+    return glu ? launch_dls_cfg<DlsCfg<OP_F8, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_F8, false>>(p, M, G_total, s);
+  }
   if (op == OP_I8) return glu ? launch_dls_cfg<DlsCfg<OP_I8, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_I8, false>>(p, M, G_total, s);
   return glu ? launch_dls_cfg<DlsCfg<OP_BF16, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_BF16, false>>(p, M, G_total, s);
 }

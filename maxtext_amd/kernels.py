@@ -11,9 +11,11 @@ import ctypes
 import torch
 
 from maxtext_amd import _lib
-from maxtext_amd._lib import (MOE_BF16, MOE_FP8_E4M3, MOE_INT4, MOE_INT8, MOE_MXFP4, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_SOFTMAX_TOPK)
+from maxtext_amd._lib import (MOE_BF16, MOE_FP8_E4M3, MOE_FP8_E5M2, MOE_INT4, MOE_INT8, MOE_MXFP4, MOE_ROUTE_DEEPSEEK, MOE_ROUTE_SOFTMAX_TOPK)
 
 _DTYPE_CODE = {torch.bfloat16: MOE_BF16, torch.int8: MOE_INT8, torch.float8_e4m3fn: MOE_FP8_E4M3}
+_LHS_DTYPE_CODE = dict(_DTYPE_CODE)
+_LHS_DTYPE_CODE[torch.float8_e5m2] = MOE_FP8_E5M2  # the quantised gradient of the backward; activations only
 
 
 def _need(t: torch.Tensor, name: str, dtype=None, ndim=None):
@@ -315,13 +317,14 @@ def glu_act_bwd(h0, h1, dout, act="silu", act_limit=7.0):
   return dh0, dh1
 
 
-def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups_local=None, group_offset=0):
+def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups_local=None, group_offset=0, as_fp8=False):
   """Gradient preparation of the quantised backward (ops.py:530-604): `dout` [m, n] bf16 times the scale of the axis the
   gradient product contracts away, optionally quantised to float8_e5m2.
 
   mode "dlhs": factor = rhs scales [g_local, n] f32, picked per row by its expert (group_sizes); quantised per row.
   mode "drhs": factor = lhs scales [m] f32; quantised per column.
   -> (d [m, n] bf16, scale): the e5m2 values (exact in bf16) and their f32 scales ([m] or [n]), or (dout * factor, None).
+  as_fp8 (with quantize): d is returned as a float8_e5m2 tensor instead, the lhs of gmm_raw against e4m3 weights.
   """
   _need(dout, "dout", torch.bfloat16, 2)
   _need(factor, "factor", torch.float32)
@@ -337,9 +340,11 @@ def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups
     if factor.numel() != m:
       raise ValueError(f"factor must hold one scale per row ({m}), got {tuple(factor.shape)}")
     g_total, g_local = 0, 0
-  out = torch.empty_like(dout)
+  if as_fp8 and not quantize:
+    raise ValueError("as_fp8 needs quantize")
+  out = torch.empty((m, n), dtype=torch.float8_e5m2, device=dout.device) if as_fp8 else torch.empty_like(dout)
   scale = torch.empty((m if code == 0 else n,), dtype=torch.float32, device=dout.device) if quantize else None
-  st = _lib.load().moe_bwd_scale_grad(_lib.ptr(dout), m, n, code, 1 if quantize else 0, _lib.ptr(factor), _lib.ptr(group_sizes), g_total,
+  st = _lib.load().moe_bwd_scale_grad(_lib.ptr(dout), m, n, code, (2 if as_fp8 else 1) if quantize else 0, _lib.ptr(factor), _lib.ptr(group_sizes), g_total,
                                       g_local, int(group_offset), _lib.ptr(out), _lib.ptr(scale), _lib.current_stream())
   _lib.check(st, "moe_bwd_scale_grad")
   return out, scale
@@ -400,7 +405,7 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
     g_local, kr, n = rhs.shape
   else:
     g_local, n, kr = rhs.shape
-  if lhs.dtype not in _DTYPE_CODE:
+  if lhs.dtype not in _LHS_DTYPE_CODE:
     raise TypeError(f"lhs dtype {lhs.dtype} not supported")
   if rhs_dtype is None:
     if rhs.dtype not in _DTYPE_CODE:
@@ -475,7 +480,7 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
   a.M, a.K, a.N = m, kdim, n
   a.num_groups_total, a.num_groups_local, a.group_offset = g_total, g_local, int(group_offset)
-  a.lhs_dtype, a.rhs_dtype = _DTYPE_CODE[lhs.dtype], rhs_dtype
+  a.lhs_dtype, a.rhs_dtype = _LHS_DTYPE_CODE[lhs.dtype], rhs_dtype
   a.lhs_scale_block_k, a.rhs_scale_block_n, a.rhs_scale_block_k = int(lhs_scale_block_k), int(rhs_scale_block_n), int(rhs_scale_block_k)
   a.act = _lib.ACT_BY_NAME[act]
   a.act_limit = float(act_limit)
@@ -502,6 +507,11 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
 def gmm_workspace(m, num_groups_total, device):
   """A tile-list buffer for moe_gmm calls on m rows and num_groups_total groups (uint8)."""
   return torch.empty((max(_lib.load().moe_gmm_workspace_bytes(int(m), int(num_groups_total)), 16),), dtype=torch.uint8, device=device)
+
+
+def gmm_lhs_e5m2_supported(m, k, n, num_groups_total):
+  """True when `gmm_raw` takes float8_e5m2 activations (against e4m3 weights) for this shape."""
+  return bool(_lib.load().moe_gmm_lhs_e5m2_supported(int(m), int(k), int(n), int(num_groups_total)))
 
 
 def gmm_rhs_kn_supported(m, k, n, num_groups_total):

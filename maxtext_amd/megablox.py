@@ -88,7 +88,9 @@ def quantize_rhs(rhs_gnk: torch.Tensor, qdtype, share_across_experts=True, *, ca
   quantizations.manual_quantize (per tensor, static, ops.py:262-266); fp8_blocks=True the 128 x 128 blocks of DeepSeek
   checkpoints."""
   qname = _qname(qdtype)
-  if manual:
+  # a "fixed,-max,max" range gives qpl.quantize the same constant scale for every channel, i.e. the static per-tensor
+  # quantiser; its exact arithmetic is third-party, manual_quantize's (layers/quantizations.py:961-991) is used for both
+  if manual or (calibration_method is not None and calibration_method.lower().startswith("fixed")):
     return quantizations.manual_quantize_weight(rhs_gnk, qname, calibration_method)
   if qname == "int8":
     return quantizations.quantize_weight_int8(rhs_gnk, share_across_experts=share_across_experts)
@@ -215,10 +217,13 @@ def gmm(
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
     if partial_sum is not None or partial_sum_up is not None or existing_out is not None or lhs_row_idx is not None or out_row_scale is not None:
       raise NotImplementedError("gradients with partial_sum / existing_out / lhs_row_idx / out_row_scale are not implemented")
-    if preferred_element_type != torch.bfloat16 or use_gmm_v2 or use_manual_quantization or (rule and rule.act_calibration_method != "absmax"):
-      raise NotImplementedError("the differentiable path takes bfloat16 outputs and dynamic (absmax) v1 quantisation")
-    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule.act_qtype if rule else None,
-                          rule.weight_qtype if rule else None, fuse_act, act_limit, rule.bwd_qtype if rule else bwd_quantize_dtype,
+    if preferred_element_type != torch.bfloat16 or use_gmm_v2:
+      raise NotImplementedError("the differentiable path takes bfloat16 outputs and the v1 quantisation of ops.py:232-267")
+    if rule is not None and rule.disable_channelwise_axes:
+      raise NotImplementedError("dynamic per-tensor scales (disable_channelwise_axes) are not implemented")
+    if rule is not None and (rule.bwd_calibration_method or "absmax") != "absmax":
+      raise NotImplementedError("the gradient is quantised with absmax calibration")
+    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, use_manual_quantization, fuse_act, act_limit,
                           rhs_bias, rhs_up_bias)
 
   common = dict(group_offset=offset, out_dtype=preferred_element_type, lhs_row_idx=lhs_row_idx, lhs_row_idx_div=lhs_row_idx_div,
@@ -336,60 +341,97 @@ def tgmm(
 class _GmmFn(torch.autograd.Function):
   """Differentiable gmm for bf16 operands (custom VJP of ops.py:137-230 / :438-527).
 
-  Unquantised or fp8 forward: backward uses the bf16 residuals, dlhs = gmm(dout, rhs^T) (ops.py:612-642) and
-  drhs = tgmm(lhs^T, dout) (ops.py:766-796); fp8 block scales run along the contracted axis of both products and
-  cannot be folded into the gradient, so the fp8 quantisers are differentiated as identities.
+  Unquantised forward, or a forward that quantises one side only: backward uses the bf16 residuals,
+  dlhs = gmm(dout, rhs^T) (ops.py:612-642) and drhs = tgmm(lhs^T, dout) (ops.py:766-796).
 
-  int8 x int8 forward (channelwise scales): the residuals are the quantised operands and the backward is the
-  reference's (_bwd_prepare_inputs ops.py:530-580): the scale of the axis that disappears goes onto the gradient,
-  dlhs = gmm(dout * rhs_scale[n], rhs_q^T), drhs = tgmm(lhs_q^T, dout * lhs_scale[m]); with bwd_q the two scaled
-  gradients are first quantised to float8_e5m2 per row / per column (_bwd_quantize_gradient ops.py:583-604); scaling
-  and quantisation are one kernel each (kernels.bwd_scale_grad).  The int8 and e5m2 values are exact in bf16, so both
-  products run on the bf16 MFMA kernels (int8 is not an operand type of the fp8 MFMA instructions).
+  int8 x int8 and fp8 x fp8 forward (e4m3 both sides: the fp8_full recipe, layers/quantizations.py:234-250, :798-855;
+  per-row x per-channel absmax scales, or the static per-tensor scales of "fixed,-max,max" calibration and of
+  manual_quantize): the residuals are the quantised operands and the backward is the reference's (_bwd_prepare_inputs
+  ops.py:530-580): the scale of the axis that disappears goes onto the gradient, dlhs = gmm(dout * rhs_scale[n], rhs_q^T),
+  drhs = tgmm(lhs_q^T, dout * lhs_scale[m]); with bwd_q the two scaled gradients are first quantised to float8_e5m2 per
+  row / per column (_bwd_quantize_gradient ops.py:583-604); scaling and quantisation are one kernel each
+  (kernels.bwd_scale_grad).  Where the operands are exact in bf16 (int8, e4m3, e5m2 all are) the products run on the
+  bf16 MFMA kernels; dlhs of an fp8 forward with a quantised gradient runs as e5m2 x e4m3 on the fp8 MFMA where the
+  persistent kernel takes the shape (kernels.gmm_lhs_e5m2_supported).
   """
 
   @staticmethod
-  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q):
+  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual):
+    lhs_q, rhs_q = (rule.act_qtype, rule.weight_qtype) if rule is not None else (None, None)
+    bwd_q = rule.bwd_qtype if rule is not None else None
     ctx.offset, ctx.transpose_rhs, ctx.bwd_q = offset, transpose_rhs, bwd_q
-    ctx.quantized = lhs_q in _INT8_NAMES and rhs_q in _INT8_NAMES
+    both_int8 = lhs_q in _INT8_NAMES and rhs_q in _INT8_NAMES
+    both_fp8 = lhs_q in _FP8_NAMES and rhs_q in _FP8_NAMES
+    ctx.quantized = both_int8 or both_fp8
     if bwd_q is not None and not ctx.quantized:
-      raise NotImplementedError("bwd_quantize_dtype needs the int8 x int8 forward (channelwise scales)")
+      raise NotImplementedError("bwd_quantize_dtype needs an int8 x int8 or fp8 x fp8 forward (channelwise or static scales)")
     if bwd_q is not None and bwd_q not in _E5M2_NAMES:
       raise ValueError(f"unsupported bwd_quantize_dtype {bwd_q}")
     with torch.no_grad():
       if ctx.quantized:
-        lq = quantize_lhs(lhs.contiguous(), lhs_q)
-        rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q)
+        lq = quantize_lhs(lhs.contiguous(), lhs_q, calibration_method=rule.act_calibration_method)
+        rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q, calibration_method=rule.weight_calibration_method, manual=manual)
         ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes)
         ctx.rhs_dtype = rhs.dtype
         return gmm(lq, rq, group_sizes, group_offset=offset, transpose_rhs=True)
       ctx.save_for_backward(lhs, rhs, group_sizes)
-      return gmm(lhs, rhs, group_sizes, group_offset=offset, transpose_rhs=transpose_rhs, lhs_quantize_dtype=lhs_q, rhs_quantize_dtype=rhs_q)
+      kw = {}
+      if rule is not None:
+        kw = dict(use_qwix_quantization=True, qwix_rule=rule, use_manual_quantization=manual)
+      return gmm(lhs, rhs, group_sizes, group_offset=offset, transpose_rhs=transpose_rhs, **kw)
 
   @staticmethod
   def _backward_quantized(ctx, dout):
-    lq, ls, rq, rs, group_sizes = ctx.saved_tensors  # lq [m,k] i8, ls [m], rq [g,n,k] i8, rs [g,n]
+    lq, ls, rq, rs, group_sizes = ctx.saved_tensors  # lq [m,k], ls [m] or [1]; rq [g,n,k], rs [g,n], [1,n] or [1]
     m, n = dout.shape
+    k = lq.shape[1]
     g_local = rq.shape[0]
+    fp8 = lq.dtype == torch.float8_e4m3fn
     dlhs = drhs = None
     quant = ctx.bwd_q is not None
+    ev = PROFILE_EVENTS
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(3)] if ev is not None else None
+    if marks:
+      marks[0].record()
     if ctx.needs_input_grad[0]:
-      # dout times the weights' channel scales of each row's expert, e5m2 per row (one kernel); the row scales go back on
-      # in the product's epilogue (rounded bf16 result times scale, rounded again: what the reference's two steps give)
-      d, s_row = kernels.bwd_scale_grad(dout, rs, mode="dlhs", quantize=quant, group_sizes=group_sizes, num_groups_local=g_local,
-                                        group_offset=ctx.offset)
+      # dout times the weights' channel scales of each row's expert, e5m2 per row (one kernel)
+      rs_gn = rs.reshape(-1, n) if rs.numel() % n == 0 else rs.reshape(1, 1).expand(1, n)
+      rs_gn = (rs_gn if rs_gn.shape[0] == g_local else rs_gn[:1].expand(g_local, n)).contiguous()
       w_t = kernels.transpose_rhs(rq)  # [g, n, k] -> [g, k, n]: the layout with k as the output axis
-      ones = torch.ones((g_local, w_t.shape[1]), dtype=torch.float32, device=dout.device)
-      dlhs = kernels.gmm_raw(d, w_t, group_sizes, rhs_scale=ones, rhs_scale_block_n=1, group_offset=ctx.offset, out_row_scale=s_row)
+      as_fp8 = fp8 and quant and kernels.gmm_lhs_e5m2_supported(m, n, k, group_sizes.numel())
+      d, s_row = kernels.bwd_scale_grad(dout, rs_gn, mode="dlhs", quantize=quant, group_sizes=group_sizes, num_groups_local=g_local,
+                                        group_offset=ctx.offset, as_fp8=as_fp8)
+      one = torch.ones((1,), dtype=torch.float32, device=dout.device)
+      if as_fp8:
+        # e5m2 x e4m3 on the fp8 MFMA; the rows' scales are the activations' epilogue scales
+        dlhs = kernels.gmm_raw(d, w_t, group_sizes, lhs_scale=s_row, rhs_scale=one, rhs_scale_block_n=_lib_per_tensor(),
+                               rhs_scale_shared=True, group_offset=ctx.offset)
+      else:
+        # the row scales go back on in the product's epilogue (rounded bf16 result times scale, rounded again: what the
+        # reference's two steps give)
+        w_b = w_t if w_t.dtype == torch.int8 else w_t.to(torch.bfloat16)
+        if w_b.dtype == torch.int8:
+          dlhs = kernels.gmm_raw(d, w_b, group_sizes, rhs_scale=one, rhs_scale_block_n=_lib_per_tensor(), rhs_scale_shared=True,
+                                 group_offset=ctx.offset, out_row_scale=s_row)
+        else:
+          dlhs = kernels.gmm_raw(d, w_b, group_sizes, group_offset=ctx.offset, out_row_scale=s_row)
+    if marks:
+      marks[1].record()
     if ctx.needs_input_grad[1]:
       # dout times the activations' row scales, e5m2 per column
-      d, s_col = kernels.bwd_scale_grad(dout, ls, mode="drhs", quantize=quant)
+      ls_m = ls if ls.numel() == m else ls.reshape(1).expand(m).contiguous()
+      d, s_col = kernels.bwd_scale_grad(dout, ls_m, mode="drhs", quantize=quant)
       # the column scales go back onto the f32 products in the kernel's epilogue, which rounds once to the weights' type
       direct = ctx.rhs_dtype in (torch.bfloat16, torch.float32)
       w = kernels.tgmm(lq.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
                        out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
       w = w.to(ctx.rhs_dtype)
       drhs = w if ctx.transpose_rhs else w.transpose(1, 2)
+    if marks:
+      marks[2].record()
+      shape = f"k{k}_n{n}"
+      ev.append(("dlhs_q_" + shape, marks[0], marks[1]))
+      ev.append(("tgmm_q_" + shape, marks[1], marks[2]))
     return dlhs, drhs
 
   @staticmethod
@@ -398,7 +440,7 @@ class _GmmFn(torch.autograd.Function):
     if ctx.quantized:
       with torch.no_grad():
         dlhs, drhs = _GmmFn._backward_quantized(ctx, dout)
-      return dlhs, drhs, None, None, None, None, None, None
+      return dlhs, drhs, None, None, None, None, None
     lhs, rhs, group_sizes = ctx.saved_tensors
     dlhs = drhs = None
     ev = PROFILE_EVENTS
@@ -420,7 +462,13 @@ class _GmmFn(torch.autograd.Function):
         shape = f"k{lhs.shape[1]}_n{dout.shape[1]}"
         ev.append(("dlhs_" + shape, marks[0], marks[1]))
         ev.append(("tgmm_" + shape, marks[1], marks[2]))
-    return dlhs, drhs, None, None, None, None, None, None
+    return dlhs, drhs, None, None, None, None, None
+
+
+def _lib_per_tensor():
+  from maxtext_amd import _lib
+
+  return _lib.MOE_SCALE_PER_TENSOR
 
 
 class _GluFn(torch.autograd.Function):
@@ -466,19 +514,19 @@ class _BiasFn(torch.autograd.Function):
     return dout, dbias, None, None
 
 
-def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, fuse_act, act_limit, bwd_q=None,
-                   rhs_bias=None, rhs_up_bias=None):
+def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual, fuse_act, act_limit, rhs_bias=None,
+                   rhs_up_bias=None):
   for name, t in (("lhs", lhs), ("rhs", rhs), ("rhs_up", rhs_up)):
     if t is not None and not isinstance(t, torch.Tensor):
       raise NotImplementedError(f"gradients need bf16 tensors; {name} is already quantised")
-  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q)
+  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual)
   if rhs_bias is not None:
     h0 = _BiasFn.apply(h0, rhs_bias, group_sizes, offset)
   if rhs_up is None:
     if fuse_act is not None:
       raise ValueError("fuse_act needs rhs_up")
     return h0
-  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, lhs_q, rhs_q, bwd_q)
+  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual)
   if rhs_up_bias is not None:
     h1 = _BiasFn.apply(h1, rhs_up_bias, group_sizes, offset)
   if fuse_act is None:

@@ -61,6 +61,7 @@ class QtRule:
   bwd_qtype: object = None
   weight_calibration_method: str = "absmax"
   act_calibration_method: str = "absmax"
+  bwd_calibration_method: str = "absmax"
   disable_channelwise_axes: bool = False
 
 
