@@ -77,7 +77,7 @@ def parse():
   ap.add_argument("--gpus", type=int, default=1)
   ap.add_argument("--steps", type=int, default=20)
   ap.add_argument("--warmup", type=int, default=5)
-  ap.add_argument("--workload", default=None, choices=["c1", "c2", "c3", "c4", "c5", "c5mx"],
+  ap.add_argument("--workload", default=None, choices=["c1", "c2", "c3", "c4", "c5", "c5mx", "c2f8"],
                   help="one workload; by default c2 (the headline line), then c3 (reported under \"secondary\") and c1, c4, c5 (\"other_configs\")")
   ap.add_argument("--source-hash", action="store_true", help="print the kernel source hash that a profile summary of --workload records")
   ap.add_argument("--tokens", type=int, default=None, help="override the token count (c5 sweep)")
@@ -90,6 +90,11 @@ def parse():
                   help="overwrite 1 GiB between steps so that no weights survive in the last-level cache (decode sizes)")
   ap.add_argument("--train", action="store_true",
                   help="forward + backward of the layer with bf16 weights of the workload's shape (weight and input gradients)")
+  ap.add_argument("--quant", default="none", choices=["none", "int8", "fp8_full"],
+                  help="--train: quantisation of the grouped matmuls: int8 x int8 forward with the quantised backward, or the "
+                       "reference's fp8_full recipe (e4m3 operands, e5m2 gradients, layers/quantizations.py:798-855)")
+  ap.add_argument("--calibration", default="absmax", help="--train --quant fp8_full: calibration of weights and activations, "
+                  "\"absmax\" or \"fixed,-max,max\" (tests/integration/tokamax_test.py:99-101 uses fixed,-224,224)")
   ap.add_argument("--calibrate-copy", action="store_true",
                   help="also run one plain 1 GiB device copy (reference dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   return ap.parse_args()
@@ -123,9 +128,9 @@ def dominant_kernel_model(wl, group_sizes):
     io_bytes = rows * d * 2.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name="gmm_wq_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="bf16")
-  op = "int8" if cfg.act_quant == "int8" else "bf16"
+  op = "int8" if cfg.act_quant == "int8" else "fp8" if cfg.act_quant == "fp8_row" else "bf16"
   # the dispatch rule of moe_gmm for its persistent 256 x 256 kernels: 128 rows per expert on average (104 weight-only)
-  if cfg.act_quant == "int8" or wl.weight_quant in (None, "bf16"):
+  if cfg.act_quant in ("int8", "fp8_row") or wl.weight_quant in (None, "bf16"):
     kernel = "gmm_dls_kernel" if rows >= 128 * len(group_sizes) else "gmm_tiled_kernel"
   else:
     # (from 16 rows per expert on: on 128-row tiles up to 112, on 256-row tiles above)
@@ -144,7 +149,7 @@ def cpu_baseline(wl, layer, sample_tokens):
 
   cfg = wl.cfg
   t = min(sample_tokens, wl.tokens)
-  trip = lambda qa: (qa.qvalue.cpu(), qa.scale.cpu(), qa.qtype)
+  trip = lambda qa: tuple(v.cpu() if hasattr(v, "cpu") else v for v in synthetic.as_triple(qa))
   x = layer["x"][:, :t].cpu()
   logits = layer["gate_logits"][:, :t].cpu()
   pre = None if layer["pre_bias_logits"] is None else layer["pre_bias_logits"][:, :t].cpu()
@@ -278,7 +283,11 @@ def train_main(args):
   wl = synthetic.workload(args.workload, args.tokens)
   import dataclasses
 
-  cfg = dataclasses.replace(wl.cfg, act_quant=None, shared_experts=0)
+  cfg = dataclasses.replace(wl.cfg, act_quant="int8" if args.quant == "int8" else None, shared_experts=0)
+  if args.quant == "fp8_full":
+    cfg = dataclasses.replace(cfg, quantization="fp8_full", use_qwix_quantization=True,
+                              weight_quantization_calibration_method=args.calibration,
+                              act_quantization_calibration_method=args.calibration)
   e, d, f, k, t = cfg.num_experts, cfg.emb_dim, cfg.moe_mlp_dim, cfg.num_experts_per_tok, wl.tokens
   g = torch.Generator(device="cuda").manual_seed(0)
   mk = lambda *shape: (torch.randn(*shape, device="cuda", generator=g) * 0.02).to(torch.bfloat16).requires_grad_()
@@ -310,7 +319,8 @@ def train_main(args):
     ts = [a.elapsed_time(b) for n, a, b in events if n == name]
     stage_ms[name] = sum(ts) / len(ts)
   m = t * k
-  dom = f"tgmm_k{d}_n{f}"  # weight gradient of wi_0 / wi_1: [E, f, d] from x [M, d] and d h [M, f]
+  # weight gradient of wi_0 / wi_1: [E, f, d] from x [M, d] and d h [M, f] (the quantised backward records its own names)
+  dom = f"tgmm_k{d}_n{f}" if args.quant == "none" else f"tgmm_q_k{d}_n{f}"
   dom_ms = stage_ms[dom]
   achieved = 2.0 * m * d * f / (dom_ms * 1e-3) / 1e12
   flops = 18.0 * m * d * f
@@ -320,7 +330,8 @@ def train_main(args):
       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
       "config": {"workload": f"{wl.name} shape, training: forward + backward of the MoE expert layer, {t} tokens, d_model {d}, "
-                             f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU",
+                             f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU"
+                             + ("" if args.quant == "none" else f", grouped matmuls quantised ({args.quant}, {args.calibration})"),
                  "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
       "roofline": dict(bound="mfma", achieved=achieved, peak=PEAK_TFLOPS["bf16"], unit="TFLOP/s", frac=achieved / PEAK_TFLOPS["bf16"],
                        traffic=traffic, traffic_source=traffic_source,
@@ -505,7 +516,7 @@ def main():
   torch.cuda.empty_cache()
   result["calibration"] = calibration(model["dtype"], vendor_shape)
   if not args.no_cpu_baseline:
-    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048, "c5mx": 2048}[wl.name]
+    sample = args.cpu_sample_tokens or {"c1": 2048, "c2": 8192, "c3": 64, "c4": 8192, "c5": 2048, "c5mx": 2048, "c2f8": 8192}[wl.name]
     result["cpu_baseline"] = cpu_baseline(wl, layer, sample)
   del layer
   torch.cuda.empty_cache()

@@ -524,6 +524,25 @@ MOE_API int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int qua
                                const int32_t* group_sizes, int num_groups_total, int num_groups_local, int group_offset,
                                void* out, float* scale_out, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Weight quantiser of the training path: what gmm() applies to bf16 weights on every step
+ * (_fwd_quantize_activation_and_weight, kernels/megablox/ops.py:250-266).
+ *
+ *   w       [G, N, K] bf16, K contiguous
+ *   q       [G, N, K] out_dtype: MOE_INT8 or MOE_FP8_E4M3
+ *   dynamic (static_scale == NULL): qpl.quantize(rhs, qtype, channelwise_axes=[2]) (ops.py:250-260): one scale per output
+ *           channel over all of K, shared by the experts (shared != 0: scale [N], the [1, 1, n] of the reference) or per
+ *           expert (shared == 0: scale [G, N]); scale = absmax / qmax, q = rint(w / scale) (int8) or the nearest-even
+ *           float8 cast of w / scale, zero channels give q = 0 and scale 0.  The third-party quantiser's rounding is not
+ *           in the reference tree: this is the library's MOE_QUANT_RINT_DIV rule.
+ *   static  (static_scale [1] f32 on the device): manual_quantize (layers/quantizations.py:961-991) for bf16 weights:
+ *           q = clip(bf16(w / bf16(scale)), +-qmax) cast as `.astype` does (int8 truncates toward zero, float8 rounds to
+ *           nearest even); `scale` is not written.
+ * Limits: K % 8 == 0.
+ */
+MOE_API int moe_quantize_rhs(const void* w, int G, int N, int K, int out_dtype, int shared, const float* static_scale,
+                             void* q, float* scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -105,6 +105,7 @@ SIGNATURES = {
     "moe_glu_act": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_float, c_void_p, c_void_p]),
     "moe_glu_act_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "moe_bwd_scale_grad": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "moe_quantize_rhs": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe_add_group_bias": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moe_unpermute_combine_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "moe_local_expert_keys_workspace_bytes": (c_size_t, [c_int, c_int]),

@@ -350,6 +350,28 @@ def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups
   return out, scale
 
 
+def quantize_rhs(w_gnk, out_dtype, *, shared=True, static_scale=None):
+  """Weight quantiser of the training path (ops.py:250-266): w [G, N, K] bf16 -> (q [G, N, K] int8 / float8_e4m3fn, scale).
+  Dynamic: one absmax scale per output channel, shared by the experts (scale [1, N]) or per expert ([G, N]);
+  static_scale ([1] f32 on the device): manual_quantize's per-tensor rule, scale returned as given."""
+  _need(w_gnk, "w", torch.bfloat16, 3)
+  if out_dtype not in (torch.int8, torch.float8_e4m3fn):
+    raise TypeError(f"out_dtype {out_dtype} not supported")
+  g, n, k = w_gnk.shape
+  q = torch.empty((g, n, k), dtype=out_dtype, device=w_gnk.device)
+  scale = None
+  if static_scale is not None:
+    _need(static_scale, "static_scale", torch.float32)
+    if static_scale.numel() != 1:
+      raise ValueError("static_scale must hold one value")
+  else:
+    scale = torch.empty((1, n) if shared else (g, n), dtype=torch.float32, device=w_gnk.device)
+  st = _lib.load().moe_quantize_rhs(_lib.ptr(w_gnk), g, n, k, _DTYPE_CODE[out_dtype], 1 if shared else 0, _lib.ptr(static_scale), _lib.ptr(q),
+                                    _lib.ptr(scale), _lib.current_stream())
+  _lib.check(st, "moe_quantize_rhs")
+  return q, (static_scale if static_scale is not None else scale)
+
+
 def add_group_bias(h, bias, group_sizes, *, group_offset=0):
   """bf16(h + bias[expert of the row]) for the rows of the local groups (bias [G_local, N] f32), other rows copied."""
   _need(h, "h", torch.bfloat16, 2)

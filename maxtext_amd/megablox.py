@@ -90,8 +90,18 @@ def quantize_rhs(rhs_gnk: torch.Tensor, qdtype, share_across_experts=True, *, ca
   qname = _qname(qdtype)
   # a "fixed,-max,max" range gives qpl.quantize the same constant scale for every channel, i.e. the static per-tensor
   # quantiser; its exact arithmetic is third-party, manual_quantize's (layers/quantizations.py:961-991) is used for both
-  if manual or (calibration_method is not None and calibration_method.lower().startswith("fixed")):
+  static = manual or (calibration_method is not None and calibration_method.lower().startswith("fixed"))
+  on_kernel = (qname in _TORCH_Q and not fp8_blocks and rhs_gnk.is_cuda and rhs_gnk.dtype == torch.bfloat16 and rhs_gnk.shape[2] % 8 == 0)
+  if static:
+    if on_kernel:
+      st = _static_scale_tensor(qname, calibration_method, rhs_gnk.device)
+      q, _ = kernels.quantize_rhs(rhs_gnk.contiguous(), _TORCH_Q[qname], static_scale=st)
+      # (the QArray's scale is the python float in the weights' dtype, layers/quantizations.py:985-989)
+      return QArray(q, st.to(rhs_gnk.dtype).float(), qname, block_n=-1, block_k=0, shared=True)
     return quantizations.manual_quantize_weight(rhs_gnk, qname, calibration_method)
+  if on_kernel:
+    q, sc = kernels.quantize_rhs(rhs_gnk.contiguous(), _TORCH_Q[qname], shared=share_across_experts)
+    return QArray(q, sc, qname, block_n=1, block_k=0, shared=share_across_experts)
   if qname == "int8":
     return quantizations.quantize_weight_int8(rhs_gnk, share_across_experts=share_across_experts)
   if qname == "fp8":

@@ -37,10 +37,33 @@ class MoEConfig:
   float32_weight_sum: bool = True
   float32_gate_logits: bool = False  # configs/base.yml:198
   shared_experts: int = 0
-  # activation quantisation for the grouped GEMMs: None | "int8" | "fp8"
+  # activation quantisation for the grouped GEMMs: None | "int8" (one scale per row) | "fp8" (the DeepSeek recipe: one
+  # scale per row and 128 values of K, against 128 x 128 weight blocks) | "fp8_row" (one scale per row, against per-channel
+  # weight scales: what gmm() quantises to, kernels/megablox/ops.py:241-260)
   act_quant: Optional[str] = None
+  # the reference's quantisation keys that reach the grouped matmuls (configs/base.yml; moe.py:1554-1556): only
+  # quantization == "fp8_full" together with use_qwix_quantization quantises them, by the rule of
+  # layers/quantizations.py:798-855 (e4m3 weights and activations, e5m2 gradients, the three calibration methods)
+  quantization: str = ""
+  use_qwix_quantization: bool = False
+  weight_quantization_calibration_method: str = "absmax"
+  act_quantization_calibration_method: str = "absmax"
+  bwd_quantization_calibration_method: str = "absmax"
   load_balance_loss_weight: float = 0.0  # > 0: permute / sparse_matmul return the auxiliary loss (moe.py:888-891)
   routed_bias_update_rate: float = 0.0  # > 0 with routed_bias: return the loss-free balancing update (moe.py:893-898)
+
+  @property
+  def gmm_quantization_rule(self):
+    """The QtRule the grouped matmuls run under, or None (get_fp8_full_qwix_rule_w_sparsity,
+    layers/quantizations.py:798-821; only "fp8_full" names "gmm" among its op_names)."""
+    if self.quantization != "fp8_full" or not self.use_qwix_quantization:
+      return None
+    from maxtext_amd.quantizations import QtRule
+
+    return QtRule(weight_qtype="float8_e4m3fn", act_qtype="float8_e4m3fn", bwd_qtype="float8_e5m2",
+                  weight_calibration_method=self.weight_quantization_calibration_method,
+                  act_calibration_method=self.act_quantization_calibration_method,
+                  bwd_calibration_method=self.bwd_quantization_calibration_method)
 
   @property
   def is_deepseek(self) -> bool:
@@ -373,10 +396,15 @@ class RoutedMoE:
       # inputs are kept for the backward pass; per-expert biases are added (and differentiated) after each GEMM
       if any(isinstance(t, QArray) for t in (sorted_inputs, w0, w1, wo)):
         raise NotImplementedError("gradients need bf16 weights; QArray weights are an inference format")
-      q = cfg.act_quant
-      inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit, lhs_quantize_dtype=q,
-                           rhs_quantize_dtype=q, rhs_bias=w0_bias, rhs_up_bias=w1_bias)
-      return megablox.gmm(inter, wo, group_size, transpose_rhs=True, lhs_quantize_dtype=q, rhs_quantize_dtype=q, rhs_bias=wo_bias)
+      rule = cfg.gmm_quantization_rule
+      if rule is not None:  # fp8_full: the qwix rule decides types and calibration (moe.py:1554-1556)
+        qkw = dict(use_qwix_quantization=True, qwix_rule=rule)
+      else:
+        q = "fp8" if cfg.act_quant == "fp8_row" else cfg.act_quant
+        qkw = dict(lhs_quantize_dtype=q, rhs_quantize_dtype=q)
+      inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
+                           rhs_bias=w0_bias, rhs_up_bias=w1_bias, **qkw)
+      return megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias, **qkw)
     # one tile-list buffer for both products: the second reuses the first one's list when its tile height agrees
     rows = row_idx.shape[0] if row_idx is not None else (sorted_inputs.qvalue if isinstance(sorted_inputs, QArray) else sorted_inputs).shape[0]
     # (`workspace`: one the sort already left a tile list in, for these group sizes)
@@ -387,8 +415,8 @@ class RoutedMoE:
     if marks:
       marks[1].record()
     if cfg.act_quant is not None:
-      # the layer's fp8 configuration is the DeepSeek recipe: 128 x 128 weight blocks with 1 x 128 activation scales
-      inter = megablox.quantize_lhs(inter, cfg.act_quant, blocks=128 if cfg.act_quant == "fp8" else None)
+      # "fp8" is the DeepSeek recipe: 128 x 128 weight blocks with 1 x 128 activation scales
+      inter = megablox.quantize_lhs(inter, "fp8" if cfg.act_quant == "fp8_row" else cfg.act_quant, blocks=128 if cfg.act_quant == "fp8" else None)
     if marks:
       marks[2].record()
     out = megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias, workspace=ws, same_groups=True)
@@ -448,14 +476,17 @@ class RoutedMoE:
 
 
 def _quantize_tokens(x2d, act_quant):
-  """The activation quantiser of the first grouped matmul on the token rows: int8 with one scale per row, or fp8 with
-  one scale per row and 128 values (the DeepSeek recipe); None leaves the bf16 rows as they are."""
+  """The activation quantiser of the first grouped matmul on the token rows: int8 with one scale per row, fp8 with
+  one scale per row and 128 values (the DeepSeek recipe) or per row; None leaves the bf16 rows as they are."""
   if act_quant == "int8":
     q, sc = kernels.gather_rows(x2d, out_dtype=torch.int8)
     return QArray(q, sc, "int8")
   if act_quant == "fp8":
     q, sc = kernels.gather_rows(x2d, out_dtype=torch.float8_e4m3fn, block_k=128)
     return QArray(q, sc, "fp8")
+  if act_quant == "fp8_row":
+    q, sc = kernels.gather_rows(x2d, out_dtype=torch.float8_e4m3fn)
+    return QArray(q, sc, "fp8", block_k=0)
   return x2d
 
 

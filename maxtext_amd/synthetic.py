@@ -12,6 +12,8 @@ tests that compare bit-for-bit build on the CPU and copy.
   c4  qwen3:     T 16384, d 2048, f 768,   E 128, k 8, int8 weights, bf16 activations, router
                  logits biased by -1.2*log(rank) (Zipf popularity, some experts empty)
   c5  gpt-oss:   d 2880,  f 2880, E 32,    k 4, int4 group-128 weights, T in {1,16,128,1024,4096}
+  c2f8           the c2 shape with float8_e4m3fn weights (one scale per output channel) and activations (one scale per
+                 token): the operand layout of the fp8_full recipe (kernels/megablox/ops.py:232-267)
 """
 
 from __future__ import annotations
@@ -31,7 +33,7 @@ class Workload:
   name: str
   tokens: int
   cfg: MoEConfig
-  weight_quant: str  # "int8" | "fp8" | "int4" | "mxfp4"
+  weight_quant: str  # "int8" | "fp8" (128 x 128 blocks) | "fp8c" (per channel) | "int4" | "mxfp4"
   seed: int
   zipf_s: float = 0.0
   router_from_weights: bool = False
@@ -45,6 +47,9 @@ def workload(name: str, tokens: Optional[int] = None) -> Workload:
   if name == "c2":
     cfg = MoEConfig(8, 2, 4096, 14336, model_name="mixtral-8x7b", act_quant="int8")
     return Workload("c2", tokens or 8192, cfg, "int8", 1236)
+  if name == "c2f8":
+    cfg = MoEConfig(8, 2, 4096, 14336, model_name="mixtral-8x7b", act_quant="fp8_row")
+    return Workload("c2f8", tokens or 8192, cfg, "fp8c", 1241)
   if name == "c3":
     cfg = MoEConfig(256, 8, 7168, 2048, model_name="deepseek3-671b", decoder_block="deepseek", routed_scaling_factor=2.5,
                     routed_score_func="sigmoid", routed_bias=True, shared_experts=1, act_quant="fp8")
@@ -66,6 +71,8 @@ def _quantize(w_gnk: torch.Tensor, kind: str) -> Q.QArray:
     return Q.quantize_weight_int8(w_gnk)
   if kind == "fp8":
     return Q.quantize_weight_fp8_blocks(w_gnk)
+  if kind == "fp8c":
+    return Q.quantize_weight_fp8_channel(w_gnk, share_across_experts=False)
   if kind == "int4":
     return Q.quantize_weight_int4(w_gnk)
   if kind == "mxfp4":
@@ -83,6 +90,8 @@ def _expert_weights(gen, n_experts, n, k, kind, device, chunk=8) -> Q.QArray:
     qs.append(qa.qvalue)
     ss.append(qa.scale)
     del w
+  if kind == "fp8c":
+    return Q.QArray(torch.cat(qs), torch.cat(ss), "fp8", block_n=1, block_k=0)
   return Q.QArray(torch.cat(qs), torch.cat(ss), kind)
 
 
@@ -116,6 +125,13 @@ def make_layer(wl: Workload, device="cuda"):
               wi_0=wi_0, wi_1=wi_1, wo=wo)
 
 
+def as_triple(qa: Q.QArray):
+  """(qvalue, scale, kind) of a weight QArray, `kind` naming the scale layout as well: "fp8c" for float8 values with one
+  scale per output channel ("fp8" alone means 128 x 128 blocks)."""
+  kind = "fp8c" if qa.qtype == "fp8" and qa.block_n == 1 else qa.qtype
+  return qa.qvalue, qa.scale, kind
+
+
 def layer_flops(wl: Workload) -> float:
   """2*M*d*f per projection, three projections (+ the shared expert over all T rows)."""
   cfg = wl.cfg
@@ -124,5 +140,5 @@ def layer_flops(wl: Workload) -> float:
 
 
 def weight_bytes_per_expert(wl: Workload) -> float:
-  per = {"int8": 1.0, "fp8": 1.0, "int4": 0.5, "mxfp4": 0.5}[wl.weight_quant]
+  per = {"int8": 1.0, "fp8": 1.0, "fp8c": 1.0, "int4": 0.5, "mxfp4": 0.5}[wl.weight_quant]
   return 3.0 * wl.cfg.emb_dim * wl.cfg.moe_mlp_dim * per

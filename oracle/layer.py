@@ -20,7 +20,7 @@ def oracle_rhs(qvalue: torch.Tensor, scale: torch.Tensor, qtype: str, n: int):
   if qtype == "bf16":  # unquantised weights [G, N, K]
     return qvalue.cpu().transpose(1, 2), None, None
   qv, sc = qvalue.cpu(), scale.cpu()
-  if qtype == "int8":
+  if qtype in ("int8", "fp8c"):  # one scale per output channel [G, N] (fp8c: float8_e4m3fn values)
     return qv.transpose(1, 2), sc, None
   if qtype == "fp8":
     s = torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]
@@ -63,6 +63,8 @@ def oracle_layer(x, gate_logits, pre_bias_logits, wi_0, wi_1, wo, *, num_experts
       return O.quantize_rows_int8(rows)
     if act_quant == "fp8":
       return O.quantize_fp8_blocks(rows, 1, 128)
+    if act_quant == "fp8_row":
+      return O.quantize_rows_fp8(rows)
     return rows, None
 
   def expert_fn(rows, gs):

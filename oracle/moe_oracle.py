@@ -745,6 +745,16 @@ def quantize_rows_int8(x: torch.Tensor):
   return q, scale.squeeze(-1)
 
 
+def quantize_rows_fp8(x: torch.Tensor):
+  """Per-row float8_e4m3fn quantisation of activations [m, k]: the [m, 1] scale of qpl.quantize(lhs, float8_e4m3fn,
+  channelwise_axes=[0]) (ops.py:241-248) under this build's v1 rule: scale = absmax / 448, q = e4m3(x / scale) rounded
+  to nearest even, zero rows give q = 0 and scale 0.  -> (q float8_e4m3fn, scale f32 [m])."""
+  x = x.to(torch.float32)
+  scale = _absmax_scale(x, 1, 448.0)
+  q = torch.where(scale == 0, torch.zeros_like(x), x / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+  return q, scale.squeeze(1)
+
+
 def quantize_weight_int8(w: torch.Tensor, per_expert: bool = True):
   """w [g, k, n] -> int8 [g,k,n], scale [g, n] f32.  per_expert=True is the
   serve-mode layout gathered per row at moe.py:1450-1459; per_expert=False

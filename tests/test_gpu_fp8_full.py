@@ -143,6 +143,46 @@ def test_gmm_e5m2_gradient_times_e4m3_weights(K):
               rhs_scale_block_n=-1, rhs_scale_shared=True)
 
 
+@pytest.mark.parametrize("qdt", [torch.int8, E4M3], ids=["int8", "fp8"])
+@pytest.mark.parametrize("shared", [True, False])
+def test_quantize_rhs_bit_exact(K, qdt, shared):
+  """The per-step weight quantiser (ops.py:250-260) against the host statement of the same rule: scale = absmax / qmax
+  over each output channel (of all experts, or per expert), q = rint(w / scale) / the nearest-even float8 cast; values and
+  scales bit for bit, incl. an all-zero channel and bf16 / bf16 quotients that are exact ties."""
+  g = torch.Generator().manual_seed(41)
+  G, N, Kd = 3, 72, 264
+  w = (torch.randn(G, N, Kd, generator=g) * 0.05).to(torch.bfloat16)
+  w[:, 5] = 0.0
+  w[1, 9] = 0.0
+  w[0, 7, :8] = torch.tensor([1.0, 0.5, 0.25, 0.75, -1.0, 0.375, 0.4375, 0.03125]).to(torch.bfloat16)
+  w[:, 7, 8:] *= 0.1  # channel 7's absmax is the exact 1.0: its quotients are short binary fractions, many of them ties
+  qmax = 127.0 if qdt == torch.int8 else 448.0
+  wf = w.float()
+  amax = wf.abs().amax(dim=(0, 2), keepdim=True) if shared else wf.abs().amax(dim=2, keepdim=True)
+  sc = amax / qmax
+  y = torch.where(sc == 0, torch.zeros_like(wf), wf / sc)
+  want_q = torch.round(y).clamp(-qmax, qmax).to(qdt) if qdt == torch.int8 else y.clamp(-qmax, qmax).to(qdt)
+  q, s = K.quantize_rhs(cuda(w), qdt, shared=shared)
+  assert tuple(s.shape) == ((1, N) if shared else (G, N))
+  assert torch.equal(s.cpu().reshape(-1), sc.reshape(-1))
+  assert torch.equal(q.cpu().float(), want_q.float())
+  assert float(s.cpu().reshape(-1, N)[0, 5]) == 0.0 and torch.all(q[:, 5].float() == 0)
+
+
+@pytest.mark.parametrize("qdt,cal", [(torch.int8, "fixed,-4,4"), (E4M3, "fixed,-224,224"), (E4M3, "fixed,3")])
+def test_quantize_rhs_static_equals_manual_quantize(K, qdt, cal):
+  """The static per-tensor rule against the oracle's restatement of manual_quantize (layers/quantizations.py:961-991),
+  pinned by exact rational arithmetic in the CPU tests: values bit for bit, out-of-range values clipped."""
+  g = torch.Generator().manual_seed(42)
+  w = (torch.randn(2, 40, 136, generator=g) * 2.0).to(torch.bfloat16)
+  w[0, 0, :4] = torch.tensor([1000.0, -1000.0, 0.0, 3.0]).to(torch.bfloat16)
+  qmax = 127.0 if qdt == torch.int8 else 448.0
+  st = torch.tensor([O.get_static_scale(qmax, cal)], dtype=torch.float32)
+  want_q, _ = O.manual_quantize(w, qdt, cal)
+  q, s = K.quantize_rhs(cuda(w), qdt, static_scale=cuda(st))
+  assert torch.equal(q.cpu().float(), want_q.float())
+
+
 @pytest.mark.parametrize("n", [192, 2056])
 def test_bwd_scale_grad_emits_e5m2_bytes(K, n):
   """quantize == 2 writes the float8_e5m2 bytes of exactly the values quantize == 1 writes as bf16, same scales."""
@@ -190,10 +230,7 @@ def test_gmm_quantized_backward_fwd_dtypes_and_calibrations(shape, calibration, 
   lhs_g = cuda(lhs).requires_grad_()
   rhs_g = cuda(w).requires_grad_()
   out = megablox.gmm(lhs_g, rhs_g, cuda(gs), use_qwix_quantization=True, qwix_rule=rule)
-  # the operands the forward quantised to: activations restated on the host (bit-equal to the kernel's, checked); weights
-  # taken from the library's quantiser, whose torch division on the GPU may differ from the host's by one ulp of the
-  # scale, which tips the many exact ties of bf16 / bf16 quotients the other way, and checked against the host rule
-  # up to that
+  # the operands the forward quantised to, restated on the host and checked bit for bit against the library's quantisers
   qdt = torch.int8 if fwd == "int8" else E4M3
   qmax = 127.0 if fwd == "int8" else 448.0
   dev_l = megablox.quantize_lhs(cuda(lhs), fwd, calibration_method=calibration)
@@ -204,12 +241,10 @@ def test_gmm_quantized_backward_fwd_dtypes_and_calibrations(shape, calibration, 
     y = torch.where(ls[:, None] == 0, torch.zeros_like(lhs.float()), lhs.float() / ls[:, None])
     want_lq = torch.round(y).clamp(-qmax, qmax).to(qdt) if fwd == "int8" else y.clamp(-qmax, qmax).to(qdt)
     assert torch.equal(dev_l.scale.cpu(), ls) and torch.equal(lq.float(), want_lq.float())
-    rs = dev_r.scale.cpu().reshape(-1, n)[0]  # [n], shared by the experts
-    host_rs = w.float().abs().amax(dim=(0, 1)) / qmax
-    assert torch.allclose(rs, host_rs, rtol=2.0**-22, atol=0)
-    deq = rq.float() * rs
-    step = (2.0**-3 if fwd == "fp8" else 1.0 / 127) * host_rs * qmax  # one grid step at the top of the range
-    assert float(((deq - w.float()).abs() / step).max()) <= 0.51
+    rs = w.float().abs().amax(dim=(0, 1)) / qmax  # [n], shared by the experts
+    y = torch.where(rs == 0, torch.zeros_like(w.float()), w.float() / rs)
+    want_rq = torch.round(y).clamp(-qmax, qmax).to(qdt) if fwd == "int8" else y.clamp(-qmax, qmax).to(qdt)
+    assert torch.equal(dev_r.scale.cpu().reshape(-1), rs) and torch.equal(rq.float(), want_rq.float())
   else:
     s = O.get_static_scale(qmax, calibration)
     ls = torch.full((m,), s)

@@ -295,6 +295,53 @@ def test_activation_closed_forms():
   g = torch.tensor([-3.0, 0.0, 2.0, 7.0])
   u = torch.tensor([1.0, 2.0, -7.0, 0.5])
   np.testing.assert_allclose(b, g / (1 + torch.exp(-1.702 * g)) * (u + 1), rtol=1e-6)
+  # DeepSeek-V4 clipped SwiGLU (moe.py:854-866): gate clipped from above only, up clipped on both sides, plain silu, no
+  # "+ 1" and no 1.702: each of these would fail one of the four columns (9 -> 7; -8 -> -7; -3 stays; factor 1)
+  c = O.apply_ffn_activation(h0, h1, "silu_clip", out_dtype=torch.float32)
+  np.testing.assert_allclose(c, (g / (1 + torch.exp(-g))) * u, rtol=1e-6)
+  assert float(c[0]) == pytest.approx(-3.0 / (1 + np.exp(3.0)) * 1.0, rel=1e-6)  # a gate below -limit is NOT clipped
+  assert float(O.apply_ffn_activation(torch.tensor([2.0]), torch.tensor([3.0]), "silu_clip", limit=1.0, out_dtype=torch.float32)) == pytest.approx(
+      1.0 / (1 + np.exp(-1.0)) * 1.0, rel=1e-6)  # the limit is the argument, not a constant
+
+
+def test_quantize_int4_groups_hand_case():
+  """_quantize_per_group of tests/unit/dequantize_pack_quantized_int4_test.py:46-53 restated: scale = absmax / 7 clamped
+  at 1e-12, q = round(w / scale) clamped to [-8, 7]; values on and between grid points, an all-zero group (the clamp),
+  and the ragged 64-wide last group of K = 2880."""
+  w = torch.zeros(2, 8)
+  w[0] = torch.tensor([7.0, -7.0, 3.0, 3.5, 2.5, -0.4, 0.6, 0.0])  # scale 1: 3.5 -> 4, 2.5 -> 2 (half to even), -0.4 -> 0, 0.6 -> 1
+  w[1, :4] = torch.tensor([14.0, -16.0, 1.0, 15.0])  # group of 4: scale 16/7; -16 -> -7, 14 -> round(6.125) = 6, 15 -> round(6.5625) = 7
+  q, s = O.quantize_int4_groups(w, group=4)
+  assert s.shape == (2, 2)
+  assert s[0].tolist() == [1.0, pytest.approx(2.5 / 7)]
+  assert q[0, :4].tolist() == [7, -7, 3, 4]
+  assert q[0, 4:].tolist() == [7, -1, 2, 0]  # second group of row 0: scale 2.5/7: 2.5 -> 7, -0.4 -> -1.12 -> -1, 0.6 -> 1.68 -> 2
+  assert float(s[1, 0]) == pytest.approx(16.0 / 7) and q[1, :4].tolist() == [6, -7, 0, 7]
+  assert float(s[1, 1]) == pytest.approx(1e-12) and q[1, 4:].tolist() == [0, 0, 0, 0]  # zero group: clamped scale, zeros
+  # K = 2880 with groups of 128: 22 full groups and one of 64; the tail's scale comes from its 64 values only
+  g = torch.Generator().manual_seed(3)
+  big = torch.randn(3, 2880, generator=g)
+  big[:, 2816:] *= 0.01
+  qb, sb = O.quantize_int4_groups(big, group=128)
+  assert qb.shape == (3, 2880) and sb.shape == (3, 23)
+  np.testing.assert_allclose(sb[:, 22], big[:, 2816:].abs().amax(1) / 7, rtol=1e-6)
+  np.testing.assert_allclose(sb[:, 5], big[:, 640:768].abs().amax(1) / 7, rtol=1e-6)
+  assert int(qb[:, 2816:].abs().max()) == 7  # the small tail still uses the full grid
+  deq = O.dequantize_int4(O.pack_int4(qb), sb.to(torch.bfloat16), 128).float()
+  assert float((deq - big).abs().max()) <= float(sb.max()) * 0.51 + 0.02
+
+
+def test_quantize_rows_fp8_hand_case():
+  """Per-row float8_e4m3fn under this build's v1 rule: scale = absmax / 448, values divided by it and rounded to nearest
+  even on the e4m3 grid (3 mantissa bits: between 16 and 32 the grid step is 2, between 256 and 448 it is 32)."""
+  x = torch.tensor([[448.0, -224.0, 17.0, 19.0, 1.0, 0.0],  # scale 1: 17 -> 16 (tie to even mantissa), 19 -> 20 (tie to even)
+                    [896.0, 100.0, -34.0, 38.0, 2.0, 600.0],  # scale 2: 50 -> 48 (tie: 48 even, 52 odd), -17 -> -16, 19 -> 20, 300 -> 288 (nearer than 320)
+                    [0.0, 0.0, 0.0, 0.0, 0.0, 0.0]])
+  q, s = O.quantize_rows_fp8(x)
+  assert q.dtype == torch.float8_e4m3fn and s.tolist() == [1.0, 2.0, 0.0]
+  assert q.float()[0].tolist() == [448.0, -224.0, 16.0, 20.0, 1.0, 0.0]
+  assert q.float()[1].tolist() == [448.0, 48.0, -16.0, 20.0, 1.0, 288.0]
+  assert q.float()[2].tolist() == [0.0] * 6
 
 
 def _layer_fixture(seed=8, t=60, d=32, f=48, e=6, k=2):
