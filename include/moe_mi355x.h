@@ -13,8 +13,9 @@
  *     local group are written as zeros), so buffers need no pre-clearing;
  *   - calls on different streams with disjoint buffers may overlap; the state the library keeps is per device: values
  *     written once (the CU count, "this kernel may use more than 64 KB of LDS", the address of the static workspace),
- *     set up on the first call that needs them or ahead of time by moe_init(), and one host-side record, under a lock,
- *     of what the last moe_gmm call on the device mapped and where, which only calls flagged MOE_GMM_SAME_GROUPS consult.
+ *     set up on the first call that needs them or ahead of time by moe_init() (two host threads that race there repeat
+ *     an idempotent query and store the same value), and one host-side record, under a lock, of what the last moe_gmm
+ *     call on the device mapped and where, which only calls flagged MOE_GMM_SAME_GROUPS consult.
  *
  * Paths in the citations are relative to the reference (AI-Hypercomputer/maxtext).
  */
@@ -146,7 +147,9 @@ MOE_API int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int
  * tile_rows rows over these group_sizes with the given num_groups_local / group_offset / MOE_GMM_KEEP_OTHER_ROWS setting,
  * and a moe_gmm call on that workspace and the group_sizes buffer written here, flagged MOE_GMM_SAME_GROUPS, skips its
  * own mapping launch when it picks that tile height (16 for the streaming kernels of decode-sized calls; any other
- * choice rebuilds the list).  Above 4096 rows nothing is mapped and moe_gmm maps as usual. */
+ * choice rebuilds the list).  Above 4096 rows nothing is mapped: the sort then drops whatever record the library held
+ * of a tile list over this group_sizes buffer (as every entry point does that writes group sizes without mapping), so a
+ * following moe_gmm maps as usual, flagged or not. */
 MOE_API int moe_sort_by_expert_mapped(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
                        int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                        void* workspace, size_t workspace_bytes, int tile_rows, int num_groups_local, int group_offset,
@@ -354,11 +357,14 @@ typedef struct {
 /* flags: layout of rhs_scale / rhs_up_scale, see "Operand layouts" above. */
 #define MOE_GMM_RHS_SCALE_KMAJOR 4
 #define MOE_GMM_RHS_SCALE_SHARED 8
-/* flags: the caller's promise that group_sizes holds what it held at the previous moe_gmm call on this device, that the
- * workspace is the same buffer, untouched since, and that this call is ordered behind that one.  When that call mapped
- * the same M, groups and tile height, its tile list is used again and the mapping launch is skipped (the second and
- * third product of an expert layer: one launch less in a chain of dependent launches, about 4 us at decode sizes);
- * when anything differs the list is rebuilt as usual.  The library keeps one record per device, the last call's. */
+/* flags: the caller's promise that group_sizes holds what it held at the previous moe_gmm call on this device (or at
+ * the moe_sort_by_expert_mapped call that built the list), that the workspace is the same buffer, untouched since, and
+ * that this call is ordered behind that one.  When that call mapped the same M, groups and tile height, its tile list is
+ * used again and the mapping launch is skipped (the second and third product of an expert layer: one launch less in a
+ * chain of dependent launches, about 4 us at decode sizes); when anything differs the list is rebuilt as usual.  The
+ * library keeps one record per device, the last call's, and drops it when one of its own entry points (the sorts,
+ * moe_local_expert_keys) writes that group_sizes buffer again without mapping; what the library cannot see is a buffer
+ * the caller overwrites itself, or frees and gets back at the same address: that is the promise. */
 #define MOE_GMM_SAME_GROUPS 16
 
 /* 1 when moe_gmm takes MOE_GMM_RHS_KN for this shape (K % 64 == 0, N % 256 == 0, 128 rows per group on average and
@@ -368,6 +374,10 @@ MOE_API int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total);
  * N * K < 2^32, 128 rows per group on average and enough tiles to fill the chip), else 0: widen the gradient to bf16
  * (moe_bwd_scale_grad with quantize == 1) and the weights with it. */
 MOE_API int moe_gmm_lhs_e5m2_supported(int M, int K, int N, int num_groups_total);
+/* 1 when the persistent stream kernels take this operand pair at this K and N (whole stages, at least three of them,
+ * and every 32-bit byte offset a request can form stays below 2^32), with indexed_lhs_rows = lhs_rows when lhs_row_idx is
+ * used, else 0.  moe_gmm falls back to its other kernels otherwise; no counterpart in the reference. */
+MOE_API int moe_gmm_stream_kernel_takes(int lhs_dtype, int rhs_dtype, int K, int N, long long indexed_lhs_rows);
 MOE_API size_t moe_gmm_workspace_bytes(int M, int num_groups_total);
 MOE_API int moe_gmm(const moe_gmm_args* args, void* stream);
 

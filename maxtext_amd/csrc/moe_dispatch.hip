@@ -5,6 +5,10 @@
 
 #include "moe_common.h"
 
+namespace moe {
+void note_group_sizes_rewritten(const int32_t* group_sizes);  // moe_gmm.hip: drops a tile list recorded over this buffer
+}
+
 #include <climits>
 
 namespace moe {
@@ -228,6 +232,7 @@ int moe_local_expert_keys(const int32_t* global_group_sizes, int num_batch_shard
     if (global_sorted_experts) offset_keys_kernel<<<blocks, 256, 0, s>>>(global_sorted_experts, local_expert_size, shard_index, num_rows, expert_keys);
     else local_keys_kernel<<<blocks, 256, 0, s>>>(starts, n, local_expert_size, num_rows, expert_keys);
   }
+  note_group_sizes_rewritten(local_group_size);
   return check_launch("local_expert_keys");
 }
 

@@ -66,6 +66,13 @@ void note_tile_map_built(const void* workspace, const int32_t* group_sizes, int 
   note_tile_map(Mapped{workspace, group_sizes, M, G_total, group_offset, G_local, bm, zero_fill ? 1 : 0});
 }
 
+void note_group_sizes_rewritten(const int32_t* group_sizes) {
+  int dev = 0;
+  if (current_device(&dev) != MOE_OK) return;
+  std::lock_guard<std::mutex> hold(g_last_map_lock);
+  if (g_last_map[dev].gs == group_sizes) g_last_map[dev] = Mapped{};
+}
+
 // Tile list of moe_gmm_static_ws: one array per device, held until the process ends.  Its name is a host-side handle,
 // not a device address: the address is looked up once per device (scratch_of) and passed to the kernels like any
 // caller-supplied workspace.
@@ -95,6 +102,7 @@ static int scratch_of(void** ptr) {
   static void* ptr_of[kMaxDevices] = {};
   int dev = 0;
   if (int st = current_device(&dev)) return st;
+  std::lock_guard<std::mutex> hold(g_last_map_lock);
   if (!ptr_of[dev]) {
     void* p = nullptr;
     hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_ws));
@@ -176,6 +184,17 @@ int moe_gmm_lhs_e5m2_supported(int M, int K, int N, int num_groups_total) {
   if (M <= 0 || K <= 0 || N <= 0 || num_groups_total <= 0 || N % 8 != 0) return 0;
   if (!dls_takes(OP_F8, K, N, 0) || (long long)N * K >= (1LL << 31) || (long long)M < 128LL * num_groups_total) return 0;
   return (long long)max_tiles_for(M, num_groups_total, 256) * cdiv(N, 256) >= 128 ? 1 : 0;
+}
+
+int moe_gmm_stream_kernel_takes(int lhs_dtype, int rhs_dtype, int K, int N, long long indexed_lhs_rows) {
+  // which operand families the persistent stream kernels accept at this K, N (and number of indexed activation rows): the
+  // shape half of moe_gmm's dispatch, exposed so that the 32-bit offset guards can be checked on the host
+  if (K <= 0 || N <= 0 || indexed_lhs_rows < 0) return 0;
+  if (lhs_dtype == MOE_INT8 && rhs_dtype == MOE_INT8) return dls_takes(OP_I8, K, N, indexed_lhs_rows) ? 1 : 0;
+  if (lhs_dtype == MOE_BF16 && rhs_dtype == MOE_BF16) return dls_takes(OP_BF16, K, N, indexed_lhs_rows) ? 1 : 0;
+  if ((lhs_dtype == MOE_FP8_E4M3 || lhs_dtype == MOE_FP8_E5M2) && rhs_dtype == MOE_FP8_E4M3) return dls_takes(OP_F8, K, N, indexed_lhs_rows) ? 1 : 0;
+  if (lhs_dtype == MOE_BF16 && (rhs_dtype == MOE_INT8 || rhs_dtype == MOE_INT4 || rhs_dtype == MOE_MXFP4)) return dlw_takes(K, N, indexed_lhs_rows, false) ? 1 : 0;
+  return 0;
 }
 
 size_t moe_gmm_workspace_bytes(int M, int num_groups_total) {

@@ -101,6 +101,11 @@ __device__ __forceinline__ void build_tile_map(const int32_t* __restrict__ group
 void note_tile_map_built(const void* workspace, const int32_t* group_sizes, int M, int G_total, int group_offset, int G_local, int bm,
                          int zero_fill);
 
+// Tells moe_gmm that a library entry has written new values into `group_sizes` without building a tile list: the
+// record of a list over that buffer's old contents is dropped, so that a following call flagged MOE_GMM_SAME_GROUPS
+// maps again instead of multiplying the new rows with the old group boundaries.
+void note_group_sizes_rewritten(const int32_t* group_sizes);
+
 // m-tiles per super-row of the persistent kernels' tile order (the tiles an XCD works on at a time are a patch of one
 // super-row's m-tiles x a few n-tiles): as many as a group of average size plus three standard deviations of a
 // multinomial draw has, so that a patch mostly stays inside one group and shares its weight panels; 8 for larger groups.

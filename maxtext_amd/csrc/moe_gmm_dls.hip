@@ -386,11 +386,14 @@ static int launch_dls_cfg(const TiledParams& p0, int M, int G_total, hipStream_t
 }
 
 bool dls_takes(int op, int K, int N, long long indexed_lhs_rows) {
-  // whole 128-byte stages, at least three of them (the stream looks two stages ahead, into the next tile at most); byte
-  // offsets inside one expert's weight matrix and inside the activations that a row index may address fit 32 bits
-  const long long esz = op == OP_BF16 ? 2 : 1;
-  return (op == OP_I8 || op == OP_BF16 || op == OP_F8) && (K * esz) % 128 == 0 && K * esz >= 384 && (long long)N * K * esz < (1LL << 32) &&
-         indexed_lhs_rows * K * esz < (1LL << 32);
+  // whole 128-byte stages, at least three of them (the stream looks two stages ahead, into the next tile at most).  Byte
+  // offsets are 32-bit: a weight request adds the lane's row (up to 255 rows past the last n-tile's first row, i.e. up to
+  // N + 255 in all) times the row pitch to the descriptor's base, an activation request the lane's row of the 256-row
+  // tile (or, with a row index, any of the indexed rows); each sum must stay below 2^32 so that a row past the end lands
+  // beyond the descriptor's range and reads as zeros instead of wrapping around into it
+  const long long esz = op == OP_BF16 ? 2 : 1, pitch = K * esz;
+  return (op == OP_I8 || op == OP_BF16 || op == OP_F8) && pitch % 128 == 0 && pitch >= 384 && ((long long)N + 256) * pitch < (1LL << 32) &&
+         (indexed_lhs_rows + 256) * pitch < (1LL << 32);
 }
 
 int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s, int lhs_e5m2) {

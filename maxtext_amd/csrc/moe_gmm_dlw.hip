@@ -383,9 +383,10 @@ static int launch_dlw_cfg(bool half, const TiledParams& p0, int M, int G_total, 
 }
 
 bool dlw_takes(int K, int N, long long indexed_lhs_rows, bool wq_kmajor) {
-  // whole 64-value stages, at least three of them (the stream looks two stages ahead, into the next tile at most); byte
-  // offsets inside one expert's weight matrix and inside the activations that a row index may address fit 32 bits
-  return K % 64 == 0 && K >= 192 && !wq_kmajor && (long long)N * K < (1LL << 32) && indexed_lhs_rows * K * 2 < (1LL << 32);
+  // whole 64-value stages, at least three of them (the stream looks two stages ahead, into the next tile at most); 32-bit
+  // byte offsets: a request adds its lane's row (up to 255 rows past the last n-tile's first row; any indexed activation
+  // row) times the row pitch to the descriptor's base, and the sum must not wrap around into the descriptor's range
+  return K % 64 == 0 && K >= 192 && !wq_kmajor && ((long long)N + 256) * K < (1LL << 32) && (indexed_lhs_rows + 256) * K * 2 < (1LL << 32);
 }
 
 int launch_dlw(int bsrc, bool glu, bool half, const TiledParams& p, int M, int G_total, hipStream_t s) {

@@ -381,7 +381,8 @@ bool f8s_takes(int K, int N, long long M, long long indexed_lhs_rows) {
   // stages in groups of four (the scales travel four stages at a time); byte offsets inside one expert's weight matrix,
   // inside the activations and inside their scales fit 32 bits
   const long long rows = indexed_lhs_rows > 0 ? indexed_lhs_rows : M;
-  return K % 512 == 0 && K >= 512 && (long long)N * K < (1LL << 32) && rows * K < (1LL << 32);
+  // (a request's lane row reaches up to 255 rows past the last n-tile's first row / the last indexed row: see dls_takes)
+  return K % 512 == 0 && K >= 512 && ((long long)N + 256) * K < (1LL << 32) && (rows + 256) * K < (1LL << 32);
 }
 
 int launch_f8s(bool glu, const Fp8TiledParams& P, int M, int G_total, hipStream_t s) {

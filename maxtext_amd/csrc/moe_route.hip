@@ -1014,13 +1014,17 @@ static int sort_impl(const int32_t* topk_idx, int T, int k, int E, int roll_to_e
   if (nblk <= 1) {  // also M == 0: group_sizes are all zero
     sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
     *mapped = mp.tiles != nullptr;
+    if (!*mapped) note_group_sizes_rewritten(group_sizes);
     return check_launch("sort_by_expert");
   }
   if (nblk <= 4) {  // up to 4096 entries: still one launch, with 16 waves
     sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
     *mapped = mp.tiles != nullptr;
+    if (!*mapped) note_group_sizes_rewritten(group_sizes);
     return check_launch("sort_by_expert");
   }
+  // (nothing is mapped from here on: a tile list recorded over this group_sizes buffer no longer describes it)
+  note_group_sizes_rewritten(group_sizes);
   if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, seg_hist);
   sort_scan_kernel<<<cdiv(E, kSortWaves), kSortWaves * kWave, 0, s>>>(seg_hist, nseg, E, group_sizes);
   if (nblk > 0)

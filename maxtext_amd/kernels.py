@@ -92,20 +92,31 @@ def gate_route(x, gate_kernel_terms, gate_bias=None, *, k, score_func="", gate_r
   return (w, idx, logits, pre) if return_logits else (w, idx)
 
 
-def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True, roll_to_expert_id=0, gmm_workspace=None, tile_rows=16):
+def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True, roll_to_expert_id=0, gmm_workspace=None, tile_rows=16, out=None):
   """-> (perm [M], inv_perm [M], group_sizes [E], sorted_experts [M] or None), all int32.
   roll_to_expert_id: the ids are sorted as (id - roll_to_expert_id) mod num_experts (moe.py:953-954).
   gmm_workspace (from gmm_workspace(M, num_experts)): up to 4096 routed rows the sort also leaves the grouped matmuls'
-  tile list of height tile_rows there, which gmm_raw(..., workspace=gmm_workspace, same_groups=True) then uses."""
+  tile list of height tile_rows there, which gmm_raw(..., workspace=gmm_workspace, same_groups=True) then uses.
+  out: (perm, inv_perm, group_sizes, sorted_experts) buffers of an earlier call, written again (a caller with
+  persistent buffers)."""
   _need(topk_idx, "topk_idx", torch.int32, 2)
   t, k = topk_idx.shape
   m = t * k
   dev = topk_idx.device
   lib = _lib.load()
-  perm = torch.empty((m,), dtype=torch.int32, device=dev)
-  inv = torch.empty((m,), dtype=torch.int32, device=dev)
-  gs = torch.empty((num_experts,), dtype=torch.int32, device=dev)
-  se = torch.empty((m,), dtype=torch.int32, device=dev) if want_sorted_experts else None
+  if out is not None:
+    perm, inv, gs, se = out
+    for name, buf, size in (("perm", perm, m), ("inv_perm", inv, m), ("group_sizes", gs, num_experts)):
+      _need(buf, name, torch.int32, 1)
+      if buf.numel() != size:
+        raise ValueError(f"out: {name} must hold {size} entries")
+    if se is not None and se.numel() != m:
+      raise ValueError(f"out: sorted_experts must hold {m} entries")
+  else:
+    perm = torch.empty((m,), dtype=torch.int32, device=dev)
+    inv = torch.empty((m,), dtype=torch.int32, device=dev)
+    gs = torch.empty((num_experts,), dtype=torch.int32, device=dev)
+    se = torch.empty((m,), dtype=torch.int32, device=dev) if want_sorted_experts else None
   nbytes = lib.moe_sort_workspace_bytes(t, k, num_experts)
   ws = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=dev)
   if gmm_workspace is not None:

@@ -221,7 +221,7 @@ def gmm(
     rule = qwix_rule
     if not isinstance(rule, quantizations.QtRule):
       raise ValueError(f"Expect a QtRule for quantized training. But get quantization_rule={rule} for gmm.")
-  elif lhs_quantize_dtype or rhs_quantize_dtype:
+  elif lhs_quantize_dtype or rhs_quantize_dtype or bwd_quantize_dtype:
     rule = quantizations.QtRule(weight_qtype=rhs_quantize_dtype, act_qtype=lhs_quantize_dtype, bwd_qtype=bwd_quantize_dtype)
 
   if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):

@@ -62,3 +62,25 @@ def test_argument_errors_are_reported_not_launched():
   a = _lib.GmmArgs()
   a.struct_size = 3
   assert lib.moe_gmm(ctypes.byref(a), None) == -1
+
+
+def test_stream_kernel_offset_guards():
+  """The persistent stream kernels form 32-bit byte offsets (lane row x row pitch, up to 255 rows past the last n-tile's
+  first row); the shape predicate must refuse every shape in which such a sum could reach 2^32 and wrap around."""
+  lib = _lib.load()
+  takes = lib.moe_gmm_stream_kernel_takes
+  I8, BF16, F8, E5M2, I4 = _lib.MOE_INT8, _lib.MOE_BF16, _lib.MOE_FP8_E4M3, _lib.MOE_FP8_E5M2, _lib.MOE_INT4
+  assert takes(I8, I8, 4096, 28672, 0) == 1 and takes(BF16, BF16, 4096, 14336, 0) == 1 and takes(F8, F8, 4096, 14336, 0) == 1
+  assert takes(E5M2, F8, 14336, 4096, 0) == 1 and takes(BF16, I4, 2880, 2880, 0) == 1
+  # whole stages, three or more
+  assert takes(I8, I8, 4096 + 64, 1024, 0) == 0 and takes(I8, I8, 256, 1024, 0) == 0 and takes(BF16, BF16, 128, 1024, 0) == 0
+  # weights: (N + 256) * pitch must stay below 2^32
+  k = 16384
+  n_ok = (1 << 32) // k - 257
+  assert takes(I8, I8, k, n_ok, 0) == 1 and takes(I8, I8, k, n_ok + 1, 0) == 0
+  assert takes(BF16, BF16, k, n_ok // 2 - 128, 0) == 1 and takes(BF16, BF16, k, n_ok // 2 + 1, 0) == 0
+  # indexed activations: (rows + 256) * pitch likewise
+  rows_ok = (1 << 32) // 4096 - 257
+  assert takes(I8, I8, 4096, 1024, rows_ok) == 1 and takes(I8, I8, 4096, 1024, rows_ok + 1) == 0
+  assert takes(BF16, I4, 4096, 1024, (1 << 32) // 8192 - 257) == 1 and takes(BF16, I4, 4096, 1024, (1 << 32) // 8192 - 256) == 0
+  assert takes(I8, BF16, 4096, 1024, 0) == 0

@@ -1598,6 +1598,33 @@ def test_sort_leaves_the_tile_list_for_the_matmuls(K, t, e, k):
   assert torch.equal(y2, y)
 
 
+def test_flagged_matmuls_after_a_sort_that_maps_nothing_use_the_new_groups(K):
+  """Two steps on the SAME group_sizes / workspace buffers above 4096 routed rows (where the sort maps nothing), each a
+  sort followed by two grouped matmuls flagged MOE_GMM_SAME_GROUPS, as a serving loop with persistent buffers issues
+  them: the second step's first matmul finds a record that matches in every field (same workspace, same group_sizes
+  pointer, same sizes and tile height) and must still map the new routing."""
+  e, k, t, d, f = 8, 2, 4096, 256, 512
+  m = t * k
+  ws = K.gmm_workspace(m, e, "cuda")
+  g = torch.Generator(device="cuda").manual_seed(7)
+  x = torch.randn((m, d), generator=g, device="cuda").to(torch.bfloat16)
+  w1 = (torch.randn((e, f, d), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  w2 = (torch.randn((e, d, f), generator=g, device="cuda") * 0.05).to(torch.bfloat16)
+  bufs = None
+  for step, skew in enumerate((0.0, 3.0)):
+    rng = np.random.default_rng(100 + step)
+    p = np.exp(-skew * np.arange(e) / e)
+    sel = np.stack([rng.choice(e, size=k, replace=False, p=p / p.sum()) for _ in range(t)]).astype(np.int32)
+    bufs = K.sort_by_expert(cuda(sel), e, gmm_workspace=ws, out=bufs)
+    gs = bufs[2]
+    h = K.gmm_raw(x, w1, gs, workspace=ws, same_groups=True)
+    y = K.gmm_raw(h, w2, gs, workspace=ws, same_groups=True)
+    fresh = gs.clone()
+    h0 = K.gmm_raw(x, w1, fresh)
+    assert torch.equal(h, h0) and torch.equal(y, K.gmm_raw(h0, w2, fresh))
+    assert torch.equal(gs.cpu(), torch.from_numpy(np.bincount(sel.reshape(-1), minlength=e).astype(np.int32)))
+
+
 @pytest.mark.parametrize("m,n,sizes,offset,g_local", [(40, 64, [7, 0, 12, 1, 20], 0, 5), (300, 2880, [100, 0, 37, 63, 50], 1, 3), (64, 8, [70], 0, 1),
                                                      (513, 512, [3] * 100 + [0] * 28, 64, 64)])
 def test_add_group_bias_bit_exact(K, m, n, sizes, offset, g_local):

@@ -57,6 +57,39 @@ def test_static_workspace_entry_point_matches_moe_gmm_on_two_calls():
     assert torch.all(got[sum(sizes):] == 0) and float(got[: sum(sizes)].float().abs().max()) > 0
 
 
+def test_static_workspace_with_the_same_groups_flag():
+  """MOE_GMM_SAME_GROUPS on the library's own array: a flagged second product of the same tile height reuses the list, one
+  of another height or of another problem in between rebuilds it; every result bit for bit moe_gmm's."""
+  lib = _lib.load()
+  stream = _lib.current_stream()
+  m, k, n, sizes = 2100, 512, 512, [700, 0, 800, 500]
+  lhs, ls, rhs, rs, gs = _operands(m, k, n, sizes, 3)
+  ws = torch.empty((lib.moe_gmm_workspace_bytes(m, len(sizes)),), dtype=torch.uint8, device="cuda")
+
+  def both(lhs_, ls_, rhs_, rs_, gs_, flagged):
+    rows, nn = lhs_.shape[0], rhs_.shape[1]
+    want = torch.full((rows, nn), 7.0, dtype=torch.bfloat16, device="cuda")
+    got = torch.full((rows, nn), -3.0, dtype=torch.bfloat16, device="cuda")
+    w2 = torch.empty((lib.moe_gmm_workspace_bytes(rows, gs_.numel()),), dtype=torch.uint8, device="cuda")
+    _lib.check(lib.moe_gmm(ctypes.byref(_args(lhs_, ls_, rhs_, rs_, gs_, want, w2)), stream), "moe_gmm")
+    b = _args(lhs_, ls_, rhs_, rs_, gs_, got, None)
+    b.flags = _lib.MOE_GMM_SAME_GROUPS if flagged else 0
+    _lib.check(lib.moe_gmm_static_ws(ctypes.byref(b), stream), "moe_gmm_static_ws")
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+  both(lhs, ls, rhs, rs, gs, False)          # maps 256-row tiles
+  both(lhs, ls, rhs, rs, gs, True)           # same height: the list is used again
+  # the same groups at 40 rows: a 64-row tile list; flagged, it must not read the 256-row list left above
+  small = torch.tensor([12, 0, 20, 8], dtype=torch.int32).cuda()
+  both(lhs[:40].contiguous(), ls[:40].contiguous(), rhs, rs, small, True)
+  # back to the first problem, flagged: the record now names another problem, so the list is rebuilt
+  both(lhs, ls, rhs, rs, gs, True)
+  # another group_sizes buffer with other contents at the same sizes, flagged: rebuilt again
+  other = torch.tensor([100, 900, 600, 500], dtype=torch.int32).cuda()
+  both(lhs, ls, rhs, rs, other, True)
+
+
 def test_static_workspace_entry_point_rejects_what_does_not_fit():
   lib = _lib.load()
   cap = lib.moe_gmm_static_ws_capacity()
