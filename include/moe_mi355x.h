@@ -142,6 +142,11 @@ MOE_API int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int
 MOE_API int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
                        int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                        void* workspace, size_t workspace_bytes, void* stream);
+/* The same with the roll read from the device: roll_to_expert_id_dev [1] i32 (taken mod E).  In the reference it is
+ * expert_shard_id * local_experts with expert_shard_id = jax.lax.axis_index (moe.py:2014-2019), a device value. */
+MOE_API int moe_sort_by_expert_rolled_dev(const int32_t* topk_idx, int T, int k, int E, const int32_t* roll_to_expert_id_dev,
+                       int32_t* perm, int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, void* stream);
 /* The same, and for up to 4096 routed rows (one launch) the block that sorted also builds the m-tile list of the
  * grouped matmuls that follow: gmm_workspace (moe_gmm_workspace_bytes(T * k, E) bytes) then holds the list for tiles of
  * tile_rows rows over these group_sizes with the given num_groups_local / group_offset / MOE_GMM_KEEP_OTHER_ROWS setting,
@@ -342,6 +347,11 @@ typedef struct {
    * to out_dtype: the routing weights applied between the activation and wo
    * (models/deepseek_batchsplit_fp8.py:1049, intermediate_layer *= weights[:, None]). */
   const float* out_row_scale;
+  /* [1] i32 on the device, or NULL: when given it replaces group_offset (negative values are read as 0).  Inside
+   * shard_map the reference's group_offset is a ()-shaped device array derived from jax.lax.axis_index
+   * (backend.py:340-345, moe.py:2014-2019), which a custom call receives as a buffer, not as an attribute: the tile-map
+   * kernel reads it, so the host never needs the value. */
+  const int32_t* group_offset_dev;
 } moe_gmm_args;
 
 /* flags: rows that belong to no local group are left as `out` holds them instead of being written as zeros:
@@ -548,8 +558,15 @@ MOE_API int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int qua
  *   static  (static_scale [1] f32 on the device): manual_quantize (layers/quantizations.py:961-991) for bf16 weights:
  *           q = clip(bf16(w / bf16(scale)), +-qmax) cast as `.astype` does (int8 truncates toward zero, float8 rounds to
  *           nearest even); `scale` is not written.
+ *           shared == 2: one scale for the whole tensor (scale [1]): disable_channelwise_axes of the qwix rule
+ *           (channelwise_axes=[], ops.py:258).
  * Limits: K % 8 == 0.
+ *
+ * moe_tensor_scale: scale[0] = max|x| / qmax over x [rows, K] bf16: the dynamic per-tensor activation scale of
+ * disable_channelwise_axes (ops.py:245); feed it to moe_gather_rows as static_scale.  `scale` doubles as the
+ * reduction's scratch word.
  */
+MOE_API int moe_tensor_scale(const void* x, long long rows, int K, float qmax, float* scale, void* stream);
 MOE_API int moe_quantize_rhs(const void* w, int G, int N, int K, int out_dtype, int shared, const float* static_scale,
                              void* q, float* scale, void* stream);
 

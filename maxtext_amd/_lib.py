@@ -73,6 +73,7 @@ class GmmArgs(ctypes.Structure):
       ("pad_", ctypes.c_int32),
       ("lhs_row_idx", c_void_p),
       ("out_row_scale", c_void_p),
+      ("group_offset_dev", c_void_p),
   ]
 
 
@@ -106,6 +107,8 @@ SIGNATURES = {
     "moe_glu_act": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_float, c_void_p, c_void_p]),
     "moe_glu_act_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "moe_bwd_scale_grad": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "moe_tensor_scale": (c_int, [c_void_p, ctypes.c_longlong, c_int, c_float, c_void_p, c_void_p]),
+    "moe_sort_by_expert_rolled_dev": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_quantize_rhs": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe_add_group_bias": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moe_unpermute_combine_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),

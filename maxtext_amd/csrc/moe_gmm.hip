@@ -38,15 +38,16 @@ namespace moe {
 constexpr int kMapThreads = 256;
 
 __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
-    const int32_t* __restrict__ group_sizes, int G_total, int group_offset, int G_local, int M,
+    const int32_t* __restrict__ group_sizes, int G_total, int group_offset, const int32_t* __restrict__ group_offset_dev, int G_local, int M,
     int BM, int zero_fill, int32_t* __restrict__ header, TileInfo* __restrict__ tiles) {
   __shared__ int s_buf[kMapThreads];
+  if (group_offset_dev) group_offset = max(*group_offset_dev, 0);  // the shard's first group, held on the device
   build_tile_map<kMapThreads>(group_sizes, G_total, group_offset, G_local, M, BM, zero_fill, header, tiles, s_buf);
 }
 
 // What the last call on a device mapped, and into which buffer (MOE_GMM_SAME_GROUPS).
 struct Mapped {
-  const void* ws; const int32_t* gs; int M, G, offset, local, bm, zero_fill;
+  const void* ws; const int32_t* gs; const int32_t* offset_dev; int M, G, offset, local, bm, zero_fill;
 };
 static Mapped g_last_map[kMaxDevices] = {};
 static std::mutex g_last_map_lock;
@@ -63,7 +64,7 @@ static bool note_tile_map(const Mapped& now) {
 
 void note_tile_map_built(const void* workspace, const int32_t* group_sizes, int M, int G_total, int group_offset, int G_local, int bm,
                          int zero_fill) {
-  note_tile_map(Mapped{workspace, group_sizes, M, G_total, group_offset, G_local, bm, zero_fill ? 1 : 0});
+  note_tile_map(Mapped{workspace, group_sizes, nullptr, M, G_total, group_offset, G_local, bm, zero_fill ? 1 : 0});
 }
 
 void note_group_sizes_rewritten(const int32_t* group_sizes) {
@@ -250,9 +251,11 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   const bool kmajor = (a->flags & MOE_GMM_RHS_SCALE_KMAJOR) != 0, shared = (a->flags & MOE_GMM_RHS_SCALE_SHARED) != 0;
   const int bn = a->rhs_scale_block_n, rbk = a->rhs_scale_block_k, lbk = a->lhs_scale_block_k;
   auto map_tiles = [&](int bm) {
-    const bool same = note_tile_map(Mapped{workspace, a->group_sizes, M, G, a->group_offset, a->num_groups_local, bm, zero_fill ? 1 : 0});
+    // (a device-held offset is part of the caller's promise like group_sizes: the record keeps its address)
+    const bool same = note_tile_map(Mapped{workspace, a->group_sizes, a->group_offset_dev, M, G, a->group_offset_dev ? 0 : a->group_offset,
+                                           a->num_groups_local, bm, zero_fill ? 1 : 0});
     if (!(same && (a->flags & MOE_GMM_SAME_GROUPS)))
-      tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->num_groups_local, M, bm, zero_fill, header, tiles);
+      tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->group_offset_dev, a->num_groups_local, M, bm, zero_fill, header, tiles);
   };
   RowOpts ro;
   ro.row_idx = a->lhs_row_idx; ro.idx_div = a->lhs_row_idx_div < 1 ? 1 : a->lhs_row_idx_div;

@@ -20,7 +20,9 @@ __device__ __forceinline__ void unpack_bf16x8(const uint4& u, float (&f)[8]) {
   for (int e = 0; e < 8; e++) f[e] = bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu);
 }
 
-// maxima[slot of the row] = max |w| over the row; slot = n (scales shared by the experts) or g * N + n
+__device__ __forceinline__ int scale_slot(int row, int N, int shared) { return shared == 2 ? 0 : shared ? row % N : row; }
+
+// maxima[slot of the row] = max |w| over the row; slot = n (scales shared by the experts), g * N + n, or 0 (per tensor)
 __global__ __launch_bounds__(kQThreads) void rhs_absmax_kernel(const uint4* __restrict__ w, int N, int K, int shared, uint32_t* __restrict__ maxima) {
   __shared__ uint32_t wmax[kQThreads / kWave];
   const int row = blockIdx.x, tid = threadIdx.x;
@@ -36,7 +38,7 @@ __global__ __launch_bounds__(kQThreads) void rhs_absmax_kernel(const uint4* __re
   for (int o = kWave / 2; o > 0; o >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, o, kWave));
   if (tid % kWave == 0) wmax[tid / kWave] = m;
   __syncthreads();
-  if (tid == 0) atomicMax(maxima + (shared ? row % N : row), max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+  if (tid == 0) atomicMax(maxima + scale_slot(row, N, shared), max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
 }
 
 // MODE 0: int8, 1: float8_e4m3fn.  STATIC: q = clip(bf16(w / bf16(scale)), +-bf16(qmax)) cast as `.astype` does (int8
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(kQThreads) void rhs_quant_kernel(const uint4* __res
   const float qmax = MODE == 0 ? 127.0f : 448.0f;
   float sc;
   if (STATIC) sc = round_bf16_fn(*static_scale);
-  else sc = maxima[shared ? row % N : row] / qmax;
+  else sc = maxima[scale_slot(row, N, shared)] / qmax;
   for (int i = tid; i < nvec; i += kQThreads) {
     float f[8];
     unpack_bf16x8(w[(size_t)row * nvec + i], f);
@@ -118,11 +120,22 @@ extern "C" int moe_quantize_rhs(const void* w, int G, int N, int K, int out_dtyp
     else rhs_quant_kernel<1, true><<<rows, kQThreads, 0, s>>>(x, N, K, 0, nullptr, static_scale, (uint2*)q);
     return check_launch("rhs_quant_kernel");
   }
-  const int ns = shared ? N : rows;
+  if (shared < 0 || shared > 2) return fail(MOE_ERR_INVALID_ARG, "quantize_rhs: shared must be 0 (per expert), 1 (shared by the experts) or 2 (per tensor)");
+  const int ns = shared == 2 ? 1 : shared ? N : rows;
   rhs_clear_kernel<<<cdiv(ns, 256), 256, 0, s>>>((uint32_t*)scale, ns);
-  rhs_absmax_kernel<<<rows, kQThreads, 0, s>>>(x, N, K, shared ? 1 : 0, (uint32_t*)scale);
-  if (out_dtype == MOE_INT8) rhs_quant_kernel<0, false><<<rows, kQThreads, 0, s>>>(x, N, K, shared ? 1 : 0, scale, nullptr, (uint2*)q);
-  else rhs_quant_kernel<1, false><<<rows, kQThreads, 0, s>>>(x, N, K, shared ? 1 : 0, scale, nullptr, (uint2*)q);
+  rhs_absmax_kernel<<<rows, kQThreads, 0, s>>>(x, N, K, shared, (uint32_t*)scale);
+  if (out_dtype == MOE_INT8) rhs_quant_kernel<0, false><<<rows, kQThreads, 0, s>>>(x, N, K, shared, scale, nullptr, (uint2*)q);
+  else rhs_quant_kernel<1, false><<<rows, kQThreads, 0, s>>>(x, N, K, shared, scale, nullptr, (uint2*)q);
   rhs_scale_kernel<<<cdiv(ns, 256), 256, 0, s>>>(scale, ns, out_dtype == MOE_INT8 ? 127.0f : 448.0f);
   return check_launch("rhs_quant_kernel");
+}
+
+extern "C" int moe_tensor_scale(const void* x, long long rows, int K, float qmax, float* scale, void* stream) {
+  if (!x || !scale) return fail(MOE_ERR_INVALID_ARG, "tensor_scale: NULL pointer");
+  if (rows < 0 || rows > 0x7fffffffLL || K <= 0 || K % 8 != 0 || !(qmax > 0.f)) return fail(MOE_ERR_INVALID_ARG, "tensor_scale: bad sizes (K %% 8 == 0)");
+  hipStream_t s = (hipStream_t)stream;
+  rhs_clear_kernel<<<1, 64, 0, s>>>((uint32_t*)scale, 1);
+  if (rows > 0) rhs_absmax_kernel<<<(unsigned)rows, kQThreads, 0, s>>>((const uint4*)x, 1, K, 2, (uint32_t*)scale);
+  rhs_scale_kernel<<<1, 64, 0, s>>>(scale, 1, qmax);
+  return check_launch("tensor_scale");
 }

@@ -324,13 +324,20 @@ constexpr int kSortMaxE = 512;
 
 __device__ __forceinline__ int clamp_expert(int e, int E) { return e < 0 ? 0 : (e >= E ? E - 1 : e); }
 // sort key of expert id e: (e - roll) mod E (permute's roll_to_expert_id, moe.py:953-954; roll = 0: the id itself)
+// the roll as given, or read from the device and taken mod E
+__device__ __forceinline__ int resolve_roll(int roll, const int32_t* roll_dev, int E) {
+  if (!roll_dev) return roll;
+  const int r = *roll_dev % E;
+  return r < 0 ? r + E : r;
+}
 __device__ __forceinline__ int sort_key(int e, int E, int roll) {
   e = clamp_expert(e, E) - roll;
   return e < 0 ? e + E : e;
 }
 
 __global__ __launch_bounds__(kSortWaves* kWave) void sort_hist_kernel(
-    const int32_t* __restrict__ flat, int M, int E, int roll, int32_t* __restrict__ seg_hist) {
+    const int32_t* __restrict__ flat, int M, int E, int roll, const int32_t* __restrict__ roll_dev, int32_t* __restrict__ seg_hist) {
+  roll = resolve_roll(roll, roll_dev, E);
   __shared__ int cnt[kSortWaves][kSortMaxE];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   for (int e = lane; e < E; e += kWave) cnt[wave][e] = 0;
@@ -370,12 +377,13 @@ __global__ __launch_bounds__(kSortWaves* kWave) void sort_scan_kernel(int32_t* _
 }
 
 __global__ __launch_bounds__(kSortWaves* kWave) void sort_scatter_kernel(
-    const int32_t* __restrict__ flat, int M, int E, int roll, int ebits,
+    const int32_t* __restrict__ flat, int M, int E, int roll, const int32_t* __restrict__ roll_dev, int ebits,
     const int32_t* __restrict__ seg_hist, const int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
     int32_t* __restrict__ sorted_experts) {
   __shared__ int run[kSortWaves][kSortMaxE];
   __shared__ int off[kSortMaxE];
+  roll = resolve_roll(roll, roll_dev, E);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   // first row of every expert = exclusive scan of group_sizes, rebuilt by each block (E <= 512 values)
   for (int e = threadIdx.x; e < kSortMaxE; e += kSortWaves * kWave) off[e] = e < E ? group_sizes[e] : 0;
@@ -434,11 +442,12 @@ struct SortMapArgs {
 
 template <int NW>
 __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
-    const int32_t* __restrict__ flat, int M, int E, int roll, int ebits, int32_t* __restrict__ group_sizes,
+    const int32_t* __restrict__ flat, int M, int E, int roll, const int32_t* __restrict__ roll_dev, int ebits, int32_t* __restrict__ group_sizes,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts, const SortMapArgs mp) {
   __shared__ int run[NW][kSortMaxE];
   __shared__ int off[kSortMaxE];
   constexpr int NT = NW * kWave;
+  roll = resolve_roll(roll, roll_dev, E);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   for (int e = threadIdx.x; e < NW * kSortMaxE; e += NT) run[e / kSortMaxE][e % kSortMaxE] = 0;
   __syncthreads();
@@ -909,7 +918,7 @@ using namespace moe;
 extern "C" {
 
 const char* moe_last_error(void) { return g_err; }
-int moe_abi_version(void) { return 2; }
+int moe_abi_version(void) { return 3; }
 
 int moe_route_topk(const float* gate_logits, const float* pre_bias_logits, int T, int E, int k,
                    int mode, int norm_topk_prob, int weights_round_bf16,
@@ -994,7 +1003,7 @@ size_t moe_sort_workspace_bytes(int T, int k, int E) {
   return (nseg * E + E) * sizeof(int32_t) + 256;
 }
 
-static int sort_impl(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, int32_t* perm,
+static int sort_impl(const int32_t* topk_idx, int T, int k, int E, int roll_to_expert_id, const int32_t* roll_dev, int32_t* perm,
                      int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                      void* workspace, size_t workspace_bytes, const SortMapArgs& mp, bool* mapped, void* stream) {
   if (!topk_idx || !perm || !group_sizes || !workspace) return fail(MOE_ERR_INVALID_ARG, "sort: NULL pointer");
@@ -1012,23 +1021,23 @@ static int sort_impl(const int32_t* topk_idx, int T, int k, int E, int roll_to_e
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
   if (nblk <= 1) {  // also M == 0: group_sizes are all zero
-    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
+    sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, roll_dev, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
     *mapped = mp.tiles != nullptr;
     if (!*mapped) note_group_sizes_rewritten(group_sizes);
     return check_launch("sort_by_expert");
   }
   if (nblk <= 4) {  // up to 4096 entries: still one launch, with 16 waves
-    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
+    sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, roll_dev, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
     *mapped = mp.tiles != nullptr;
     if (!*mapped) note_group_sizes_rewritten(group_sizes);
     return check_launch("sort_by_expert");
   }
   // (nothing is mapped from here on: a tile list recorded over this group_sizes buffer no longer describes it)
   note_group_sizes_rewritten(group_sizes);
-  if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, seg_hist);
+  if (nblk > 0) sort_hist_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, roll_dev, seg_hist);
   sort_scan_kernel<<<cdiv(E, kSortWaves), kSortWaves * kWave, 0, s>>>(seg_hist, nseg, E, group_sizes);
   if (nblk > 0)
-    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, ebits, seg_hist, group_sizes,
+    sort_scatter_kernel<<<nblk, kSortWaves * kWave, 0, s>>>(topk_idx, M, E, roll, roll_dev, ebits, seg_hist, group_sizes,
                                                           perm, inv_perm, sorted_experts);
   return check_launch("sort_by_expert");
 }
@@ -1037,7 +1046,16 @@ int moe_sort_by_expert_rolled(const int32_t* topk_idx, int T, int k, int E, int 
                               int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                               void* workspace, size_t workspace_bytes, void* stream) {
   bool mapped = false;
-  return sort_impl(topk_idx, T, k, E, roll_to_expert_id, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes,
+  return sort_impl(topk_idx, T, k, E, roll_to_expert_id, nullptr, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes,
+                   SortMapArgs{nullptr, nullptr, 0, 0, 0, 0}, &mapped, stream);
+}
+
+int moe_sort_by_expert_rolled_dev(const int32_t* topk_idx, int T, int k, int E, const int32_t* roll_to_expert_id_dev, int32_t* perm,
+                                  int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+  if (!roll_to_expert_id_dev) return fail(MOE_ERR_INVALID_ARG, "sort: NULL roll_to_expert_id_dev");
+  bool mapped = false;
+  return sort_impl(topk_idx, T, k, E, 0, roll_to_expert_id_dev, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes,
                    SortMapArgs{nullptr, nullptr, 0, 0, 0, 0}, &mapped, stream);
 }
 
@@ -1053,7 +1071,7 @@ int moe_sort_by_expert_mapped(const int32_t* topk_idx, int T, int k, int E, int 
   const int zero_fill = keep_other_rows ? 0 : 1;
   const SortMapArgs mp = {(TileInfo*)((uint8_t*)gmm_workspace + 16), (int32_t*)gmm_workspace, num_groups_local, group_offset, tile_rows, zero_fill};
   bool mapped = false;
-  const int st = sort_impl(topk_idx, T, k, E, roll_to_expert_id, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes, mp,
+  const int st = sort_impl(topk_idx, T, k, E, roll_to_expert_id, nullptr, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes, mp,
                            &mapped, stream);
   if (st == MOE_OK && mapped) note_tile_map_built(gmm_workspace, group_sizes, (int)M, E, group_offset, num_groups_local, tile_rows, zero_fill);
   return st;

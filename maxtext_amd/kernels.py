@@ -125,6 +125,14 @@ def sort_by_expert(topk_idx, num_experts, *, want_sorted_experts=True, roll_to_e
                                        _lib.ptr(gmm_workspace), gmm_workspace.numel(), _lib.current_stream())
     _lib.check(st, "moe_sort_by_expert_mapped")
     return perm, inv, gs, se
+  if isinstance(roll_to_expert_id, torch.Tensor):  # a device scalar (the reference's comes from jax.lax.axis_index): never read here
+    _need(roll_to_expert_id, "roll_to_expert_id", torch.int32)
+    if roll_to_expert_id.numel() != 1:
+      raise ValueError("roll_to_expert_id must hold one value")
+    st = lib.moe_sort_by_expert_rolled_dev(_lib.ptr(topk_idx), t, k, num_experts, _lib.ptr(roll_to_expert_id), _lib.ptr(perm), _lib.ptr(inv),
+                                           _lib.ptr(gs), _lib.ptr(se), _lib.ptr(ws), ws.numel(), _lib.current_stream())
+    _lib.check(st, "moe_sort_by_expert_rolled_dev")
+    return perm, inv, gs, se
   st = lib.moe_sort_by_expert_rolled(_lib.ptr(topk_idx), t, k, num_experts, int(roll_to_expert_id), _lib.ptr(perm), _lib.ptr(inv),
                                      _lib.ptr(gs), _lib.ptr(se), _lib.ptr(ws), ws.numel(), _lib.current_stream())
   _lib.check(st, "moe_sort_by_expert_rolled")
@@ -361,9 +369,20 @@ def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups
   return out, scale
 
 
-def quantize_rhs(w_gnk, out_dtype, *, shared=True, static_scale=None):
+def tensor_scale(x, qmax):
+  """absmax(x) / qmax of a bf16 matrix as a [1] f32 device tensor: the dynamic per-tensor scale of
+  disable_channelwise_axes (ops.py:245), usable as gather_rows' static_scale."""
+  _need(x, "x", torch.bfloat16, 2)
+  scale = torch.empty((1,), dtype=torch.float32, device=x.device)
+  st = _lib.load().moe_tensor_scale(_lib.ptr(x), x.shape[0], x.shape[1], float(qmax), _lib.ptr(scale), _lib.current_stream())
+  _lib.check(st, "moe_tensor_scale")
+  return scale
+
+
+def quantize_rhs(w_gnk, out_dtype, *, shared=True, static_scale=None, per_tensor=False):
   """Weight quantiser of the training path (ops.py:250-266): w [G, N, K] bf16 -> (q [G, N, K] int8 / float8_e4m3fn, scale).
-  Dynamic: one absmax scale per output channel, shared by the experts (scale [1, N]) or per expert ([G, N]);
+  Dynamic: one absmax scale per output channel, shared by the experts (scale [1, N]) or per expert ([G, N]), or one for
+  the tensor (per_tensor: scale [1], disable_channelwise_axes);
   static_scale ([1] f32 on the device): manual_quantize's per-tensor rule, scale returned as given."""
   _need(w_gnk, "w", torch.bfloat16, 3)
   if out_dtype not in (torch.int8, torch.float8_e4m3fn):
@@ -376,8 +395,8 @@ def quantize_rhs(w_gnk, out_dtype, *, shared=True, static_scale=None):
     if static_scale.numel() != 1:
       raise ValueError("static_scale must hold one value")
   else:
-    scale = torch.empty((1, n) if shared else (g, n), dtype=torch.float32, device=w_gnk.device)
-  st = _lib.load().moe_quantize_rhs(_lib.ptr(w_gnk), g, n, k, _DTYPE_CODE[out_dtype], 1 if shared else 0, _lib.ptr(static_scale), _lib.ptr(q),
+    scale = torch.empty((1,) if per_tensor else (1, n) if shared else (g, n), dtype=torch.float32, device=w_gnk.device)
+  st = _lib.load().moe_quantize_rhs(_lib.ptr(w_gnk), g, n, k, _DTYPE_CODE[out_dtype], 2 if per_tensor else 1 if shared else 0, _lib.ptr(static_scale), _lib.ptr(q),
                                     _lib.ptr(scale), _lib.current_stream())
   _lib.check(st, "moe_quantize_rhs")
   return q, (static_scale if static_scale is not None else scale)
@@ -413,7 +432,8 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
             rhs_dtype=None, lhs_scale_block_k=0, rhs_scale_block_n=1, rhs_scale_block_k=0, act=None, act_limit=7.0,
             group_offset=0, out=None, kernel=None, raster=0, rhs_bias=None, rhs_up_bias=None, partial_sum=None, partial_sum_up=None,
             keep_other_rows=False, rhs_kn=False, rhs_scale_kmajor=False, rhs_scale_shared=False, out_dtype=torch.bfloat16,
-            lhs_row_idx=None, lhs_row_idx_div=1, out_row_scale=None, num_rows=None, workspace=None, same_groups=False):
+            lhs_row_idx=None, lhs_row_idx_div=1, out_row_scale=None, num_rows=None, workspace=None, same_groups=False,
+            group_offset_dev=None):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2]).
   rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 without rhs_up, on shapes `gmm_rhs_kn_supported` accepts).
   Scale layouts follow include/moe_mi355x.h: lhs_scale_block_k 0 = [M], -1 = [1] (per tensor), b = [M, ceil(K/b)];
@@ -422,7 +442,8 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   lhs_row_idx [M] int32: row i of the product reads lhs row lhs_row_idx[i] // lhs_row_idx_div (lhs then has any number of
   rows); out_row_scale [M] f32 multiplies the result rows.  kernel / raster select a kernel family (moe_gmm_tuned).
   workspace: a caller-held uint8 buffer of moe_gmm_workspace_bytes; same_groups: MOE_GMM_SAME_GROUPS (group_sizes and the
-  workspace are those of the previous call, untouched: its tile list is used again when the tile height agrees)."""
+  workspace are those of the previous call, untouched: its tile list is used again when the tile height agrees).
+  group_offset_dev: int32 [1] on the device; replaces group_offset without the host ever reading it."""
   _need(lhs, "lhs", None, 2)
   _need(rhs, "rhs", None, 3)
   _need(group_sizes, "group_sizes", torch.int32, 1)
@@ -521,6 +542,11 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
   a.lhs_row_idx = lhs_row_idx.data_ptr() if lhs_row_idx is not None else None
   a.lhs_row_idx_div, a.lhs_rows = int(lhs_row_idx_div), lhs_rows
   a.out_row_scale = out_row_scale.data_ptr() if out_row_scale is not None else None
+  if group_offset_dev is not None:
+    _need(group_offset_dev, "group_offset_dev", torch.int32)
+    if group_offset_dev.numel() != 1:
+      raise ValueError("group_offset_dev must hold one value")
+    a.group_offset_dev = group_offset_dev.data_ptr()
   a.rhs_bias = rhs_bias.data_ptr() if rhs_bias is not None else None
   a.rhs_up_bias = rhs_up_bias.data_ptr() if rhs_up_bias is not None else None
   a.partial_sum = partial_sum.data_ptr() if partial_sum is not None else None

@@ -60,12 +60,12 @@ def _static_scale_tensor(qname, calibration_method, device):
   return torch.tensor([quantizations.get_static_scale(_QMAX[qname], calibration_method)], dtype=torch.float32, device=device)
 
 
-def quantize_lhs(lhs: torch.Tensor, qdtype, *, calibration_method="absmax", blocks=None, v2=False) -> QArray:
+def quantize_lhs(lhs: torch.Tensor, qdtype, *, calibration_method="absmax", blocks=None, v2=False, per_tensor=False) -> QArray:
   """Activation quantiser.
 
   v2=False: the v1 path, qpl.quantize(lhs, act_qtype, channelwise_axes=[0], calibration_method) (ops.py:241-248):
-  one scale per row, for int8 and for fp8; "fixed,..." gives one static scale for the tensor.  blocks=128 keeps the
-  DeepSeek recipe's one scale per row and 128 values of K.
+  one scale per row, for int8 and for fp8; "fixed,..." gives one static scale for the tensor, per_tensor one dynamic
+  scale for it (channelwise_axes=[]).  blocks=128 keeps the DeepSeek recipe's one scale per row and 128 values of K.
   v2=True: the quantiser inside gmm_v2 (pallas_mosaic_tpu_v2_gmm_kernel.py:528-542): one scale per row and 512 values
   of K (:1231), or the static (1, 1) scale of ops.py:333-360."""
   qname = _qname(qdtype)
@@ -76,13 +76,19 @@ def quantize_lhs(lhs: torch.Tensor, qdtype, *, calibration_method="absmax", bloc
     st = _static_scale_tensor(qname, calibration_method, lhs.device)
     q, s = kernels.gather_rows(lhs, out_dtype=_TORCH_Q[qname], rule=rule, static_scale=st)
     return QArray(q, s, qname, block_k=-1)
+  if per_tensor:
+    # channelwise_axes=[] (disable_channelwise_axes, ops.py:245): one absmax scale for the tensor, found on the device and
+    # then used like a static one
+    st = kernels.tensor_scale(lhs, _QMAX[qname])
+    q, s = kernels.gather_rows(lhs, out_dtype=_TORCH_Q[qname], rule=rule, static_scale=st)
+    return QArray(q, s, qname, block_k=-1)
   block_k = 512 if v2 and blocks is None else (blocks or 0)
   q, s = kernels.gather_rows(lhs, out_dtype=_TORCH_Q[qname], block_k=block_k, rule=rule)
   return QArray(q, s, qname, block_k=block_k)
 
 
 def quantize_rhs(rhs_gnk: torch.Tensor, qdtype, share_across_experts=True, *, calibration_method="absmax", manual=False,
-                 fp8_blocks=False) -> QArray:
+                 fp8_blocks=False, per_tensor=False) -> QArray:
   """Weight quantiser for rhs in [G, N, K] layout: one scale per output channel shared by the experts, the [1, 1, n]
   scale of qpl.quantize(rhs, channelwise_axes=[2]) (ops.py:250-260), for int8 and fp8; manual=True is
   quantizations.manual_quantize (per tensor, static, ops.py:262-266); fp8_blocks=True the 128 x 128 blocks of DeepSeek
@@ -99,6 +105,11 @@ def quantize_rhs(rhs_gnk: torch.Tensor, qdtype, share_across_experts=True, *, ca
       # (the QArray's scale is the python float in the weights' dtype, layers/quantizations.py:985-989)
       return QArray(q, st.to(rhs_gnk.dtype).float(), qname, block_n=-1, block_k=0, shared=True)
     return quantizations.manual_quantize_weight(rhs_gnk, qname, calibration_method)
+  if per_tensor:
+    if not on_kernel:
+      raise NotImplementedError("per-tensor dynamic weight scales need bf16 weights on the GPU (K % 8 == 0)")
+    q, sc = kernels.quantize_rhs(rhs_gnk.contiguous(), _TORCH_Q[qname], per_tensor=True)
+    return QArray(q, sc, qname, block_n=-1, block_k=0, shared=True)
   if on_kernel:
     q, sc = kernels.quantize_rhs(rhs_gnk.contiguous(), _TORCH_Q[qname], shared=share_across_experts)
     return QArray(q, sc, qname, block_n=1, block_k=0, shared=share_across_experts)
@@ -144,7 +155,7 @@ def gmm(
     lhs,
     rhs,
     group_sizes,
-    preferred_element_type=torch.bfloat16,
+    preferred_element_type=torch.float32,
     tiling=(128,) * 9,
     group_offset=None,
     existing_out=None,
@@ -192,7 +203,7 @@ def gmm(
   calibration gives static per-tensor scales.  With use_gmm_v2 the activations are quantised by gmm_v2's own rule
   (per row and 512 values of K, or the static (1, 1) scale, ops.py:333-360) to the type the weights ask for
   (pallas_mosaic_tpu_v2_gmm_kernel.py:1208-1223: int8 weights -> int8, fp8 weights -> fp8; int4 weights stay
-  weight-only here).  preferred_element_type: bfloat16 or float32.
+  weight-only here).  preferred_element_type: float32 (the reference's default, ops.py:50) or bfloat16.
   lhs_row_idx / lhs_row_idx_div / out_row_scale: see kernels.gmm_raw (the permute and the routing weights fused in).
   """
   del tiling, interpret, lhs_vma_axes, rhs_vma_axes, use_tokamax_backend
@@ -205,13 +216,18 @@ def gmm(
       raise ValueError("existing_out must be a contiguous tensor of preferred_element_type")
   if weight_gather_axes:
     raise NotImplementedError("weight all-gather belongs to the multi-device path")
-  if group_offset is None:
-    offset = 0
-  else:
+  offset, offset_dev = 0, None
+  needs_grad = torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias))
+  if group_offset is not None:
     if isinstance(group_offset, torch.Tensor):
       if group_offset.dim() != 0:
         raise ValueError(f"group_offset must be a ()-shaped array. Got: {tuple(group_offset.shape)}.")
-      offset = int(group_offset.item())
+      if group_offset.is_cuda and not needs_grad:
+        # a device scalar (inside shard_map the reference derives it from jax.lax.axis_index, moe.py:2014-2019): handed to
+        # the tile-map kernel as it is, the host never reads it
+        offset_dev = group_offset.reshape(1).to(torch.int32)
+      else:
+        offset = int(group_offset.item())  # (the backward's kernels take the offset by value: one host read per call)
     else:
       offset = int(group_offset)
 
@@ -224,20 +240,22 @@ def gmm(
   elif lhs_quantize_dtype or rhs_quantize_dtype or bwd_quantize_dtype:
     rule = quantizations.QtRule(weight_qtype=rhs_quantize_dtype, act_qtype=lhs_quantize_dtype, bwd_qtype=bwd_quantize_dtype)
 
-  if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (lhs, rhs, rhs_up, rhs_bias, rhs_up_bias)):
+  if needs_grad:
     if partial_sum is not None or partial_sum_up is not None or existing_out is not None or lhs_row_idx is not None or out_row_scale is not None:
       raise NotImplementedError("gradients with partial_sum / existing_out / lhs_row_idx / out_row_scale are not implemented")
-    if preferred_element_type != torch.bfloat16 or use_gmm_v2:
-      raise NotImplementedError("the differentiable path takes bfloat16 outputs and the v1 quantisation of ops.py:232-267")
+    if use_gmm_v2:
+      raise NotImplementedError("the differentiable path takes the v1 quantisation of ops.py:232-267")
     if rule is not None and rule.disable_channelwise_axes:
       raise NotImplementedError("dynamic per-tensor scales (disable_channelwise_axes) are not implemented")
     if rule is not None and (rule.bwd_calibration_method or "absmax") != "absmax":
       raise NotImplementedError("the gradient is quantised with absmax calibration")
-    return _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, use_manual_quantization, fuse_act, act_limit,
-                          rhs_bias, rhs_up_bias)
+    out = _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, use_manual_quantization, fuse_act, act_limit,
+                         rhs_bias, rhs_up_bias)
+    # (the differentiable kernels produce bf16; a float32 result is that value widened, and its gradient arrives rounded to bf16)
+    return out if preferred_element_type == torch.bfloat16 else out.to(preferred_element_type)
 
-  common = dict(group_offset=offset, out_dtype=preferred_element_type, lhs_row_idx=lhs_row_idx, lhs_row_idx_div=lhs_row_idx_div,
-                out_row_scale=out_row_scale, workspace=workspace, same_groups=same_groups)
+  common = dict(group_offset=offset, group_offset_dev=offset_dev, out_dtype=preferred_element_type, lhs_row_idx=lhs_row_idx,
+                lhs_row_idx_div=lhs_row_idx_div, out_row_scale=out_row_scale, workspace=workspace, same_groups=same_groups)
   if rhs_bias is not None:
     common["rhs_bias"] = rhs_bias.float().contiguous()  # [G, N] (rhs_bias [G, 1, N] of the v2 kernel, :573)
   if partial_sum is not None:  # [m, n], added to the product before the activation (ops.py:77)
@@ -255,17 +273,16 @@ def gmm(
   rhs_n = _native_rhs(rhs, transpose_rhs)
   up_n = _native_rhs(rhs_up, transpose_rhs) if rhs_up is not None else None
   if rule is not None and rule.weight_qtype and not isinstance(rhs_n, QArray):
-    if rule.disable_channelwise_axes and not use_manual_quantization:
-      raise NotImplementedError("dynamic per-tensor weight scales (disable_channelwise_axes) are not implemented")
-    qkw = dict(calibration_method=rule.weight_calibration_method, manual=use_manual_quantization)
+    # disable_channelwise_axes: channelwise_axes=[] (ops.py:258), one dynamic scale for the whole tensor
+    qkw = dict(calibration_method=rule.weight_calibration_method, manual=use_manual_quantization,
+               per_tensor=bool(rule.disable_channelwise_axes))
     rhs_n = quantize_rhs(rhs_n, rule.weight_qtype, **qkw)
     if up_n is not None:
       up_n = quantize_rhs(up_n, rule.weight_qtype, **qkw)
   if rule is not None and rule.act_qtype and not isinstance(lhs, QArray):
-    if rule.disable_channelwise_axes and not (rule.act_calibration_method or "").lower().startswith("fixed"):
-      raise NotImplementedError("dynamic per-tensor activation scales (disable_channelwise_axes) are not implemented")
     if not use_gmm_v2:
-      lhs = quantize_lhs(lhs.contiguous(), rule.act_qtype, calibration_method=rule.act_calibration_method)
+      lhs = quantize_lhs(lhs.contiguous(), rule.act_qtype, calibration_method=rule.act_calibration_method,
+                         per_tensor=bool(rule.disable_channelwise_axes))
   if use_gmm_v2 and isinstance(rhs_n, QArray) and not isinstance(lhs, QArray) and rhs_n.qtype in ("int8", "fp8"):
     # gmm_v2 quantises the activations itself, to the type the weights ask for (:1208-1223), statically when the rule
     # carries a fixed range (ops.py:333-360)
@@ -383,12 +400,12 @@ class _GmmFn(torch.autograd.Function):
         rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q, calibration_method=rule.weight_calibration_method, manual=manual)
         ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes)
         ctx.rhs_dtype = rhs.dtype
-        return gmm(lq, rq, group_sizes, group_offset=offset, transpose_rhs=True)
+        return gmm(lq, rq, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=True)
       ctx.save_for_backward(lhs, rhs, group_sizes)
       kw = {}
       if rule is not None:
         kw = dict(use_qwix_quantization=True, qwix_rule=rule, use_manual_quantization=manual)
-      return gmm(lhs, rhs, group_sizes, group_offset=offset, transpose_rhs=transpose_rhs, **kw)
+      return gmm(lhs, rhs, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=transpose_rhs, **kw)
 
   @staticmethod
   def _backward_quantized(ctx, dout):
@@ -446,7 +463,7 @@ class _GmmFn(torch.autograd.Function):
 
   @staticmethod
   def backward(ctx, dout):
-    dout = dout.contiguous()
+    dout = dout.to(torch.bfloat16).contiguous()
     if ctx.quantized:
       with torch.no_grad():
         dlhs, drhs = _GmmFn._backward_quantized(ctx, dout)
@@ -460,7 +477,7 @@ class _GmmFn(torch.autograd.Function):
         marks[0].record()
       if ctx.needs_input_grad[0]:
         # dout [m, n] @ rhs[g]^T: the kernel's weight layout [G, out, in] is here [G, k, n]
-        dlhs = gmm(dout, rhs, group_sizes, group_offset=ctx.offset, transpose_rhs=not ctx.transpose_rhs)
+        dlhs = gmm(dout, rhs, group_sizes, torch.bfloat16, group_offset=ctx.offset, transpose_rhs=not ctx.transpose_rhs)
         # rows of groups outside [offset, offset + G_local) are zero in the forward output
       if marks:
         marks[1].record()

@@ -384,6 +384,7 @@ class RoutedMoE:
     reads row row_idx[i] // row_idx_div of it: the permute fused into the matmul, no [M, d] copy."""
     cfg = self.config
     act, limit = cfg.activation, (cfg.mlp_activations_limit if cfg.mlp_activations_limit > 0 else 7.0)
+    bf16 = torch.bfloat16  # preferred_element_type=self.dtype of the reference's calls (moe.py:1549)
     ev = self.profile_events
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)] if ev is not None else None
     if marks:
@@ -402,14 +403,14 @@ class RoutedMoE:
       else:
         q = "fp8" if cfg.act_quant == "fp8_row" else cfg.act_quant
         qkw = dict(lhs_quantize_dtype=q, rhs_quantize_dtype=q)
-      inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
+      inter = megablox.gmm(sorted_inputs, w0, group_size, bf16, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
                            rhs_bias=w0_bias, rhs_up_bias=w1_bias, **qkw)
-      return megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias, **qkw)
+      return megablox.gmm(inter, wo, group_size, bf16, transpose_rhs=True, rhs_bias=wo_bias, **qkw)
     # one tile-list buffer for both products: the second reuses the first one's list when its tile height agrees
     rows = row_idx.shape[0] if row_idx is not None else (sorted_inputs.qvalue if isinstance(sorted_inputs, QArray) else sorted_inputs).shape[0]
     # (`workspace`: one the sort already left a tile list in, for these group sizes)
     ws = workspace if workspace is not None else kernels.gmm_workspace(rows, group_size.numel(), group_size.device)
-    inter = megablox.gmm(sorted_inputs, w0, group_size, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
+    inter = megablox.gmm(sorted_inputs, w0, group_size, bf16, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
                          rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div, workspace=ws,
                          same_groups=workspace is not None)
     if marks:
@@ -419,7 +420,7 @@ class RoutedMoE:
       inter = megablox.quantize_lhs(inter, "fp8" if cfg.act_quant == "fp8_row" else cfg.act_quant, blocks=128 if cfg.act_quant == "fp8" else None)
     if marks:
       marks[2].record()
-    out = megablox.gmm(inter, wo, group_size, transpose_rhs=True, rhs_bias=wo_bias, workspace=ws, same_groups=True)
+    out = megablox.gmm(inter, wo, group_size, bf16, transpose_rhs=True, rhs_bias=wo_bias, workspace=ws, same_groups=True)
     if marks:
       marks[3].record()
       ev.append(("wi_glu", marks[0], marks[1]))

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_size_queries_and_struct_layout_without_gpu():
   lib = _lib.load()
-  assert lib.moe_abi_version() == 2
+  assert lib.moe_abi_version() == 3
   assert lib.moe_sort_workspace_bytes(2048, 2, 8) >= (4 * 4 * 8 + 8) * 4
   assert lib.moe_gmm_workspace_bytes(4096, 8) >= 16 + (4096 // 16 + 9) * 16
 

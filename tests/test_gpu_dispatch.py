@@ -10,6 +10,14 @@ from oracle import moe_oracle as O
 pytestmark = pytest.mark.gpu
 
 
+def gmm_bf16(*args, **kwargs):
+  """megablox.gmm with the layer dtype as preferred_element_type, as the reference's layer calls it (moe.py:1549)."""
+  from maxtext_amd import megablox
+
+  kwargs.setdefault("preferred_element_type", torch.bfloat16)
+  return megablox.gmm(*args, **kwargs)
+
+
 @pytest.fixture(scope="module")
 def M():
   from maxtext_amd import moe
@@ -183,8 +191,8 @@ def test_ragged_all_to_all_flow_on_one_gpu_matches_the_single_device_layer():
     assert n == int(traffic[:, j].sum()) and not torch.isnan(xj[:n].float()).any()
     np.testing.assert_array_equal(ids[:n].cpu().numpy(), np.repeat(np.arange(l), local_sizes.cpu().numpy()))
     sl = slice(j * l, (j + 1) * l)
-    h = megablox.gmm(xj, w0[sl].contiguous(), local_sizes, transpose_rhs=True, rhs_up=w1[sl].contiguous(), fuse_act="silu")
-    y = megablox.gmm(h, wo[sl].contiguous(), local_sizes, transpose_rhs=True)
+    h = gmm_bf16(xj, w0[sl].contiguous(), local_sizes, transpose_rhs=True, rhs_up=w1[sl].contiguous(), fuse_act="silu")
+    y = gmm_bf16(h, wo[sl].contiguous(), local_sizes, transpose_rhs=True)
     returned.append(kernels.unpermute_combine(y.contiguous(), None, k=1, perm=local_idx))  # rows back in arrival order
 
   # the way back, then each batch shard's unpermute with its routing weights
@@ -219,8 +227,8 @@ def test_ring_of_experts_flow_on_one_gpu_matches_the_single_device_layer():
     sx, perm, weights, group_size, sorted_experts, _, _, _ = block.permute(x, logits, roll_to_expert_id=j * l)
     sl = slice(j * l, (j + 1) * l)
     # rolled ids: this shard's experts are groups 0 .. l-1 of the rolled order; rows of the other groups come back as zeros
-    h = megablox.gmm(sx, w0[sl].contiguous(), group_size, transpose_rhs=True, rhs_up=w1[sl].contiguous(), fuse_act="silu", group_offset=0)
-    y = megablox.gmm(h, wo[sl].contiguous(), group_size, transpose_rhs=True, group_offset=0)
+    h = gmm_bf16(sx, w0[sl].contiguous(), group_size, transpose_rhs=True, rhs_up=w1[sl].contiguous(), fuse_act="silu", group_offset=0)
+    y = gmm_bf16(h, wo[sl].contiguous(), group_size, transpose_rhs=True, group_offset=0)
     n = int(group_size[:l].sum())
     assert not y[n:].any()
     total += block.unpermute(y, perm, weights, 1, t).reshape(t, d).float()

@@ -12,6 +12,12 @@ from tolerances import ELEM_ATOL_RMS_CHAINED, TOL, relerr
 pytestmark = pytest.mark.gpu
 
 
+def gmm_bf16(M, *args, **kwargs):
+  """megablox.gmm with the layer dtype as preferred_element_type, as the reference's layer calls it (moe.py:1549)."""
+  kwargs.setdefault("preferred_element_type", torch.bfloat16)
+  return M.gmm(*args, **kwargs)
+
+
 @pytest.fixture(scope="module")
 def M():
   from maxtext_amd import _lib, megablox
@@ -60,7 +66,7 @@ def test_deepseek_fp8_state_dict_through_gmm(M, gs):
   x = torch.randn(m, k, generator=g).to(torch.bfloat16)
   xq = M.quantize_lhs(x.cuda(), "fp8", blocks=128)
   gsz = np.array(gs, np.int32)
-  got = M.gmm(xq, dev(w0), torch.from_numpy(gsz).cuda(), transpose_rhs=True)
+  got = gmm_bf16(M, xq, dev(w0), torch.from_numpy(gsz).cuda(), transpose_rhs=True)
   xs = xq.scale.cpu().reshape(m, k // 128)
   x_deq = (xq.qvalue.cpu().float().reshape(m, k // 128, 128) * xs[..., None]).reshape(m, k)
   w_deq = torch.stack([O.dequantize_fp8_blocks(w0.qvalue[i], w0.scale[i], 128).float() for i in range(e)])
@@ -68,7 +74,7 @@ def test_deepseek_fp8_state_dict_through_gmm(M, gs):
   want = grouped(x_deq, w_deq, gs)
   assert relerr(got, want) <= TOL
   # fused gate/up + SiLU as the layer runs it
-  got_glu = M.gmm(xq, dev(w0), torch.from_numpy(gsz).cuda(), transpose_rhs=True, rhs_up=dev(w1), fuse_act="silu")
+  got_glu = gmm_bf16(M, xq, dev(w0), torch.from_numpy(gsz).cuda(), transpose_rhs=True, rhs_up=dev(w1), fuse_act="silu")
   w1_deq = torch.stack([O.dequantize_fp8_blocks(w1.qvalue[i], w1.scale[i], 128).float() for i in range(e)])
   h0, h1 = want, grouped(x_deq, w1_deq, gs)
   # a product of two matmul results: the error of either factor scales with the other, not with the product
@@ -97,7 +103,7 @@ def test_compressed_int4_through_gmm(M, gs, group_size):
     w_deq.append((torch.from_numpy(w).float().reshape(n, k // group_size, group_size) * sc.float()[..., None]).reshape(n, k))
   qa = formats.compressed_int4_experts(packed, scales, [(n, k)] * e, group_size=group_size)
   x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(torch.bfloat16)
-  got = M.gmm(x.cuda(), dev(qa), torch.tensor(gs, dtype=torch.int32).cuda(), transpose_rhs=True)
+  got = gmm_bf16(M, x.cuda(), dev(qa), torch.tensor(gs, dtype=torch.int32).cuda(), transpose_rhs=True)
   assert relerr(got, grouped(x, torch.stack(w_deq), gs)) <= TOL
 
 
@@ -120,7 +126,7 @@ def test_gpt_oss_mxfp4_through_gmm(M, gs):
   wi_0, wi_1, wo, (b0, b1, bo) = formats.gpt_oss_mxfp4_layer(blocks, scales, dblocks, dscales, bias, dbias)
   x = (torch.randn(m, d, generator=g)).to(torch.bfloat16)
   gsz = torch.tensor(gs, dtype=torch.int32).cuda()
-  inter = M.gmm(x.cuda(), dev(wi_0), gsz, transpose_rhs=True, rhs_up=dev(wi_1), fuse_act="swigluoai", act_limit=7.0,
+  inter = gmm_bf16(M, x.cuda(), dev(wi_0), gsz, transpose_rhs=True, rhs_up=dev(wi_1), fuse_act="swigluoai", act_limit=7.0,
                 rhs_bias=b0.cuda(), rhs_up_bias=b1.cuda())
   full = O.dequantize_mxfp4(blocks, scales).float()  # [e, 2f, d]
   row_e = np.repeat(np.arange(e), gs)
@@ -132,7 +138,7 @@ def test_gpt_oss_mxfp4_through_gmm(M, gs):
   want_inter = O.apply_ffn_activation(h0.float(), h1.float(), "swigluoai", 7.0, out_dtype=torch.float32)
   want_inter[nrow:] = 0
   assert relerr(inter, want_inter, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
-  out = M.gmm(inter, dev(wo), gsz, transpose_rhs=True, rhs_bias=bo.cuda())
+  out = gmm_bf16(M, inter, dev(wo), gsz, transpose_rhs=True, rhs_bias=bo.cuda())
   want = grouped(inter.cpu(), O.dequantize_mxfp4(dblocks, dscales).float(), gs)
   want[:nrow] += dbias.double()[row_e]
   assert relerr(out, want) <= TOL
@@ -151,6 +157,6 @@ def test_aqt_int8_serve_kernel_through_gmm(M, gs):
   s = torch.rand(e, 1, n, generator=g) * 0.01 + 1e-3
   qa = formats.aqt_int8_experts(q, s)
   x = torch.randn(m, k, generator=g).to(torch.bfloat16)
-  got = M.gmm(x.cuda(), dev(qa), torch.tensor(gs, dtype=torch.int32).cuda(), transpose_rhs=True)
+  got = gmm_bf16(M, x.cuda(), dev(qa), torch.tensor(gs, dtype=torch.int32).cuda(), transpose_rhs=True)
   want = grouped(x, q.transpose(1, 2).float(), gs) * s[:, 0].double()[np.repeat(np.arange(e), gs)]
   assert relerr(got, want) <= TOL

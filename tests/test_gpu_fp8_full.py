@@ -13,6 +13,14 @@ from tolerances import ELEM_ATOL_RMS_CHAINED, relerr
 
 pytestmark = pytest.mark.gpu
 
+
+def gmm_bf16(*args, **kwargs):
+  """megablox.gmm with the layer dtype as preferred_element_type, as the reference's layer calls it (moe.py:1549)."""
+  from maxtext_amd import megablox
+
+  kwargs.setdefault("preferred_element_type", torch.bfloat16)
+  return megablox.gmm(*args, **kwargs)
+
 TOL = 1e-2
 E4M3 = torch.float8_e4m3fn
 
@@ -229,7 +237,7 @@ def test_gmm_quantized_backward_fwd_dtypes_and_calibrations(shape, calibration, 
 
   lhs_g = cuda(lhs).requires_grad_()
   rhs_g = cuda(w).requires_grad_()
-  out = megablox.gmm(lhs_g, rhs_g, cuda(gs), use_qwix_quantization=True, qwix_rule=rule)
+  out = gmm_bf16(lhs_g, rhs_g, cuda(gs), use_qwix_quantization=True, qwix_rule=rule)
   # the operands the forward quantised to, restated on the host and checked bit for bit against the library's quantisers
   qdt = torch.int8 if fwd == "int8" else E4M3
   qmax = 127.0 if fwd == "int8" else 448.0
@@ -292,14 +300,14 @@ def test_fp8_full_layer_gradients_tokamax_configuration():
   xs, p0, p1, po = [cuda(v).requires_grad_() for v in (x, w0, w1, wo)]
   kw = dict(use_qwix_quantization=True, qwix_rule=rule)
   # the fused call's own composition, spelled out so that every stage's gradient can be read back
-  g0 = megablox.gmm(xs, p0, cuda(gs), **kw)
-  g1 = megablox.gmm(xs, p1, cuda(gs), **kw)
+  g0 = gmm_bf16(xs, p0, cuda(gs), **kw)
+  g1 = gmm_bf16(xs, p1, cuda(gs), **kw)
   h = megablox._GluFn.apply(g0, g1, "silu", 7.0)
   for v in (g0, g1, h):
     v.retain_grad()
-  y = megablox.gmm(h, po, cuda(gs), **kw)
+  y = gmm_bf16(h, po, cuda(gs), **kw)
   y.backward(cuda(dy))
-  fused = megablox.gmm(xs.detach().requires_grad_(), p0, cuda(gs), rhs_up=p1, fuse_act="silu", **kw)
+  fused = gmm_bf16(xs.detach().requires_grad_(), p0, cuda(gs), rhs_up=p1, fuse_act="silu", **kw)
   assert torch.equal(fused, h)
 
   # oracle: each stage on the operands the stage before it produced on the GPU (a bf16 rounding that differs between the

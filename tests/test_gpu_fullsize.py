@@ -18,6 +18,14 @@ from oracle import moe_oracle as O
 from tolerances import ELEM_ATOL_RMS_CHAINED, relerr
 
 pytestmark = pytest.mark.gpu
+
+
+def gmm_bf16(*args, **kwargs):
+  """megablox.gmm with the layer dtype as preferred_element_type, as the reference's layer calls it (moe.py:1549)."""
+  from maxtext_amd import megablox
+
+  kwargs.setdefault("preferred_element_type", torch.bfloat16)
+  return megablox.gmm(*args, **kwargs)
 TOL = 1e-2
 N_SAMPLE = 40
 
@@ -122,9 +130,9 @@ def test_fullsize_int_weight_layers(name):
     rows = kernels.gather_rows(x2d, perm, k)
     assert torch.equal(rows[:4096].cpu(), x2d.cpu()[torch.from_numpy(operm[:4096].astype(np.int64) // k)])
     rows_q, rows_scale = rows, None
-  inter = megablox.gmm(rows, L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act=cfg.activation)
+  inter = gmm_bf16(rows, L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act=cfg.activation)
   inter_in = megablox.quantize_lhs(inter, "int8") if cfg.act_quant == "int8" else inter
-  y = megablox.gmm(inter_in, L["wo"], gs, transpose_rhs=True)
+  y = gmm_bf16(inter_in, L["wo"], gs, transpose_rhs=True)
   assert torch.isfinite(inter.float()).all() and torch.isfinite(y.float()).all()
   n = _check_sampled_rows(wl, L, rows_q, rows_scale, inter, y, gs, cfg.act_quant)
   assert n >= 16
@@ -162,8 +170,8 @@ def test_fullsize_deepseek_fp8(tokens):
   q, sc = kernels.gather_rows(x2d, perm, k + 1, out_dtype=torch.float8_e4m3fn, block_k=128)
   oq, osc = O.quantize_fp8_blocks(x2d.cpu()[torch.from_numpy(operm.astype(np.int64) // (k + 1))], 1, 128)
   assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(sc.cpu(), osc)
-  inter = megablox.gmm(QArray(q, sc, "fp8"), L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act="silu")
-  y = megablox.gmm(megablox.quantize_lhs(inter, "fp8", blocks=128), L["wo"], gs, transpose_rhs=True)
+  inter = gmm_bf16(QArray(q, sc, "fp8"), L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act="silu")
+  y = gmm_bf16(megablox.quantize_lhs(inter, "fp8", blocks=128), L["wo"], gs, transpose_rhs=True)
   assert torch.isfinite(y.float()).all()
   # sampled rows against the oracle's block-scaled formula (including rows of the shared expert)
   gsn = gs.cpu().numpy()

@@ -13,6 +13,14 @@ from oracle import moe_oracle as O
 
 pytestmark = pytest.mark.gpu
 
+
+def gmm_bf16(*args, **kwargs):
+  """megablox.gmm with the layer dtype as preferred_element_type, as the reference's layer calls it (moe.py:1549)."""
+  from maxtext_amd import megablox
+
+  kwargs.setdefault("preferred_element_type", torch.bfloat16)
+  return megablox.gmm(*args, **kwargs)
+
 TOL = 1e-2
 # kernel families of moe_gmm_tuned the block-scaled fp8 tests run: picked by shape / streaming / 128 x 128 tiles / 256 x 256 tiles
 FP8_KERNELS = {0: None, 1: "stream", 2: "tiled", 3: "big"}
@@ -763,7 +771,7 @@ def test_gmm_autograd_matches_torch_autograd(transpose_rhs, m, k, n, gs):
 
   lhs_g = cuda(lhs).requires_grad_()
   rhs_g = cuda(w.transpose(1, 2) if transpose_rhs else w).requires_grad_()
-  out = megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs)
+  out = gmm_bf16(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs)
   assert relerr(out, ref) <= TOL
   out.backward(cuda(dout))
   assert lhs_g.grad.shape == lhs.shape and rhs_g.grad.shape == rhs_g.shape
@@ -790,7 +798,7 @@ def test_gmm_autograd_through_fused_activation():
   h1 = torch.cat([a[off[i] : off[i + 1]] @ b1[i].T for i in range(2)])
   (torch.nn.functional.silu(h0) * h1 * dout.double()).sum().backward()
   la, r0, r1 = cuda(lhs).requires_grad_(), cuda(w0).requires_grad_(), cuda(w1).requires_grad_()
-  out = megablox.gmm(la, r0, cuda(gs), transpose_rhs=True, rhs_up=r1, fuse_act="silu")
+  out = gmm_bf16(la, r0, cuda(gs), transpose_rhs=True, rhs_up=r1, fuse_act="silu")
   out.backward(cuda(dout))
   # bf16 intermediates (h0, h1 and their gradients are rounded to bf16) -> 2e-2 on the gradients
   assert relerr(la.grad, a.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
@@ -1314,8 +1322,8 @@ def test_megablox_gmm_partial_sum_accumulates_k_chunks():
   acc = None
   for c in range(4):
     sl = slice(c * 128, (c + 1) * 128)
-    acc = megablox.gmm(lhs_d[:, sl].contiguous(), wb[:, sl].contiguous(), gs_d, partial_sum=acc)
-  full = megablox.gmm(lhs_d, wb, gs_d)
+    acc = gmm_bf16(lhs_d[:, sl].contiguous(), wb[:, sl].contiguous(), gs_d, partial_sum=acc)
+  full = gmm_bf16(lhs_d, wb, gs_d)
   assert relerr(acc, full, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2  # three extra bf16 roundings of the running sum
 
 
@@ -1328,13 +1336,13 @@ def test_gmm_existing_out_keeps_rows_of_other_groups():
   wb = w.to(torch.bfloat16)
   full = O.gmm(lhs, wb, gs)
   buf = torch.full((700, 128), 7.0, dtype=torch.bfloat16, device="cuda")
-  out = megablox.gmm(cuda(lhs), cuda(wb[:2]), cuda(gs), existing_out=buf, group_offset=0)
+  out = gmm_bf16(cuda(lhs), cuda(wb[:2]), cuda(gs), existing_out=buf, group_offset=0)
   assert out.data_ptr() == buf.data_ptr()
   assert torch.all(buf[150:] == 7.0) and relerr(buf[:150], full[:150]) <= TOL
-  megablox.gmm(cuda(lhs), cuda(wb[2:]), cuda(gs), existing_out=buf, group_offset=2)
+  gmm_bf16(cuda(lhs), cuda(wb[2:]), cuda(gs), existing_out=buf, group_offset=2)
   assert relerr(buf[:620], full[:620]) <= TOL and torch.all(buf[620:] == 7.0)
   # without existing_out the same call zeroes the rows it does not own
-  plain = megablox.gmm(cuda(lhs), cuda(wb[2:]), cuda(gs), group_offset=2)
+  plain = gmm_bf16(cuda(lhs), cuda(wb[2:]), cuda(gs), group_offset=2)
   assert torch.all(plain[:150] == 0) and torch.all(plain[620:] == 0)
   # the few-rows (streaming) kernels take the same tile list
   lhs2, w2, _, gs2 = _gmm_inputs(60, 256, 128, [10, 20, 5, 15], 96)
@@ -1409,7 +1417,7 @@ def test_gmm_quantized_backward(transpose_rhs, bwd_q):
 
   lhs_g = cuda(lhs).requires_grad_()
   rhs_g = cuda(w.transpose(1, 2).contiguous() if transpose_rhs else w).requires_grad_()
-  out = megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, lhs_quantize_dtype="int8", rhs_quantize_dtype="int8",
+  out = gmm_bf16(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, lhs_quantize_dtype="int8", rhs_quantize_dtype="int8",
                      bwd_quantize_dtype=bwd_q)
   assert relerr(out, want_out) <= TOL
   out.backward(cuda(dout))
@@ -1420,7 +1428,7 @@ def test_gmm_quantized_backward(transpose_rhs, bwd_q):
   assert got_dr.shape == want_dr.shape and relerr(got_dr, want_dr) <= tol
   assert torch.all(got_dr[1] == 0)
   with pytest.raises(NotImplementedError):
-    megablox.gmm(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, bwd_quantize_dtype="float8_e5m2")
+    gmm_bf16(lhs_g, rhs_g, cuda(gs), transpose_rhs=transpose_rhs, bwd_quantize_dtype="float8_e5m2")
 
 
 @pytest.mark.parametrize("quantize", [False, True])
@@ -1477,9 +1485,9 @@ def test_gmm_autograd_with_expert_bias():
   ref = torch.cat([torch.nn.functional.silu(h0) * h1, torch.zeros(44, n, dtype=torch.float64)])
   (ref * dout.double()).sum().backward()
   la, q0, q1, d0, d1 = (cuda(t).requires_grad_() for t in (lhs, w0, w1, b0, b1))
-  out = megablox.gmm(la, q0, cuda(gs), transpose_rhs=True, rhs_up=q1, fuse_act="silu", rhs_bias=d0, rhs_up_bias=d1)
+  out = gmm_bf16(la, q0, cuda(gs), transpose_rhs=True, rhs_up=q1, fuse_act="silu", rhs_bias=d0, rhs_up_bias=d1)
   with torch.no_grad():
-    fused = megablox.gmm(cuda(lhs), cuda(w0), cuda(gs), transpose_rhs=True, rhs_up=cuda(w1), fuse_act="silu", rhs_bias=cuda(b0), rhs_up_bias=cuda(b1))
+    fused = gmm_bf16(cuda(lhs), cuda(w0), cuda(gs), transpose_rhs=True, rhs_up=cuda(w1), fuse_act="silu", rhs_bias=cuda(b0), rhs_up_bias=cuda(b1))
   assert relerr(out, ref, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2 and relerr(out, fused, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2 and torch.all(out[256:] == 0)
   out.backward(cuda(dout))
   assert relerr(la.grad, a.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2

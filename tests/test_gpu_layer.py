@@ -15,6 +15,14 @@ import torch
 from oracle import moe_oracle as O
 
 pytestmark = pytest.mark.gpu
+
+
+def gmm_bf16(*args, **kwargs):
+  """megablox.gmm with the layer dtype as preferred_element_type, as the reference's layer calls it (moe.py:1549)."""
+  from maxtext_amd import megablox
+
+  kwargs.setdefault("preferred_element_type", torch.bfloat16)
+  return megablox.gmm(*args, **kwargs)
 TOL = 1e-2
 
 
@@ -150,17 +158,25 @@ def test_megablox_gmm_api():
   rhs = (torch.randn(e, kd, n, generator=g) * 0.05).to(torch.bfloat16)  # reference default layout [g, k, n]
   gs = np.array([100, 0, 312, 100], np.int32)
   want = O.gmm(lhs, rhs, gs)
-  got = megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda())
+  got = gmm_bf16(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda())
   assert relerr(got, want) <= TOL
-  got_t = megablox.gmm(lhs.cuda(), rhs.transpose(1, 2).contiguous().cuda(), torch.from_numpy(gs).cuda(), transpose_rhs=True)
+  got_t = gmm_bf16(lhs.cuda(), rhs.transpose(1, 2).contiguous().cuda(), torch.from_numpy(gs).cuda(), transpose_rhs=True)
   assert torch.equal(got, got_t)
+  # the default result type is the reference's float32 (ops.py:50), with and without gradients
+  dflt = megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda())
+  assert dflt.dtype == torch.float32 and relerr(dflt, O.gmm(lhs, rhs, gs, out_dtype=torch.float32)) <= 1e-3
+  lg = lhs.cuda().requires_grad_()
+  dg = megablox.gmm(lg, rhs.cuda(), torch.from_numpy(gs).cuda())
+  assert dg.dtype == torch.float32
+  dg.sum().backward()
+  assert lg.grad is not None and lg.grad.dtype == torch.bfloat16
   # dynamic int8 on both sides (ops.py:232-267): close to the unquantised product (quantizations_test.py:653: < 0.2)
-  got_q = megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda(), lhs_quantize_dtype="int8", rhs_quantize_dtype="int8")
+  got_q = gmm_bf16(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs).cuda(), lhs_quantize_dtype="int8", rhs_quantize_dtype="int8")
   assert (got_q.float().cpu() - want.float()).abs().mean() / want.float().abs().mean() < 0.2
   with pytest.raises(ValueError):
-    megablox.gmm(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs.astype(np.int64)).cuda())
+    gmm_bf16(lhs.cuda(), rhs.cuda(), torch.from_numpy(gs.astype(np.int64)).cuda())
   with pytest.raises(ValueError):
-    megablox.gmm(lhs.cuda()[None], rhs.cuda(), torch.from_numpy(gs).cuda())
+    gmm_bf16(lhs.cuda()[None], rhs.cuda(), torch.from_numpy(gs).cuda())
 
 
 def test_layer_linearity_at_benchmark_width():
