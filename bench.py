@@ -522,11 +522,13 @@ def main():
   torch.cuda.empty_cache()
   if both:
     sec, swl, slayer, smodel, _ = run_workload(args, "c3")
+    sec_cpu = None if args.no_cpu_baseline else cpu_baseline(swl, slayer, args.cpu_sample_tokens or 64)
     del slayer
     result["secondary"] = {
         "workload": sec["config"]["workload"], "metric": "moe_quant_gmm_layer_tflops", "value": sec["value"], "unit": sec["unit"],
         "ms_per_step": sec["ms_per_step"], "steps": args.steps, "warmup": args.warmup, "dtype": sec["dtype"],
         "config": sec["config"], "roofline": sec["roofline"], "stage_ms": sec["stage_ms"], "layer_gbps": sec["layer_gbps"],
+        "cpu_baseline": sec_cpu,
     }
     # the remaining configurations of the baseline (parity-test cases, not the headline), each timed the same way so
     # that one run records all five
@@ -539,6 +541,23 @@ def main():
           "workload": o["config"]["workload"], "value": o["value"], "unit": o["unit"], "ms_per_step": o["ms_per_step"], "dtype": o["dtype"],
           "config": o["config"], "roofline": o["roofline"], "stage_ms": o["stage_ms"], "layer_gbps": o["layer_gbps"],
       })
+    # the decode half of the GPT-OSS token sweep (BASELINE's fifth configuration: 1, 16, 128, 1024 tokens; 4096 is the
+    # line above): launch-bound sizes, so each is replayed as one captured HIP graph, once as it comes (the 0.4 GB of
+    # weights partly live in the last-level cache from one replay to the next) and once with 1 GiB overwritten between
+    # steps
+    sweep = []
+    for tokens in (1, 16, 128, 1024):
+      entry = {"tokens": tokens}
+      for key, cold in (("graph", False), ("graph_cold", True)):
+        torch.cuda.empty_cache()
+        sub = argparse.Namespace(**{**vars(args), "graph": True, "cold": cold, "gate": False})
+        o, _, olayer, _, _ = run_workload(sub, "c5", tokens)
+        del olayer
+        entry[key] = {"ms_per_step": o["ms_per_step"], "layer_gbps": o["layer_gbps"], "value": o["value"], "unit": o["unit"],
+                      "roofline": o["roofline"], "stage_ms": o["stage_ms"]}
+        entry["workload"] = o["config"]["workload"]
+      sweep.append(entry)
+    result["c5_token_sweep"] = sweep
   print(json.dumps(result))
 
 
