@@ -185,6 +185,7 @@ def gmm(
     workspace=None,
     same_groups=False,
     out_row_scale=None,
+    lhs_row_inv=None,
 ):
   """Grouped matmul: out[rows of group g] = lhs[rows] @ rhs[g] (ops.py:46).
 
@@ -204,7 +205,10 @@ def gmm(
   (per row and 512 values of K, or the static (1, 1) scale, ops.py:333-360) to the type the weights ask for
   (pallas_mosaic_tpu_v2_gmm_kernel.py:1208-1223: int8 weights -> int8, fp8 weights -> fp8; int4 weights stay
   weight-only here).  preferred_element_type: float32 (the reference's default, ops.py:50) or bfloat16.
-  lhs_row_idx / lhs_row_idx_div / out_row_scale: see kernels.gmm_raw (the permute and the routing weights fused in).
+  lhs_row_idx / lhs_row_idx_div / out_row_scale: see kernels.gmm_raw (the permute and the routing weights fused in);
+  lhs_row_inv: the inverse permutation of lhs_row_idx when it is one, used by the gradient of lhs (a deterministic sum over
+  each token's copies).  Every argument is differentiable where the reference's is: lhs, rhs, rhs_up, the biases,
+  partial_sum and existing_out (both receive the incoming gradient, ops.py:524-527), out_row_scale.
   """
   del tiling, interpret, lhs_vma_axes, rhs_vma_axes, use_tokamax_backend
   _validate_args(lhs, rhs, group_sizes)
@@ -240,17 +244,23 @@ def gmm(
   elif lhs_quantize_dtype or rhs_quantize_dtype or bwd_quantize_dtype:
     rule = quantizations.QtRule(weight_qtype=rhs_quantize_dtype, act_qtype=lhs_quantize_dtype, bwd_qtype=bwd_quantize_dtype)
 
+  needs_grad = needs_grad or (torch.is_grad_enabled() and any(
+      isinstance(t, torch.Tensor) and t.requires_grad for t in (partial_sum, partial_sum_up, existing_out, out_row_scale)))
   if needs_grad:
-    if partial_sum is not None or partial_sum_up is not None or existing_out is not None or lhs_row_idx is not None or out_row_scale is not None:
-      raise NotImplementedError("gradients with partial_sum / existing_out / lhs_row_idx / out_row_scale are not implemented")
     if use_gmm_v2:
       raise NotImplementedError("the differentiable path takes the v1 quantisation of ops.py:232-267")
     if rule is not None and rule.disable_channelwise_axes:
       raise NotImplementedError("dynamic per-tensor scales (disable_channelwise_axes) are not implemented")
     if rule is not None and (rule.bwd_calibration_method or "absmax") != "absmax":
       raise NotImplementedError("the gradient is quantised with absmax calibration")
+    if existing_out is not None and existing_out.dtype != torch.bfloat16:
+      raise NotImplementedError("existing_out is bfloat16 on the differentiable path")
     out = _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, use_manual_quantization, fuse_act, act_limit,
-                         rhs_bias, rhs_up_bias)
+                         rhs_bias, rhs_up_bias, partial_sum, partial_sum_up, existing_out, lhs_row_idx, lhs_row_idx_div, lhs_row_inv)
+    if out_row_scale is not None:
+      # the routing weights between the activation and wo (models/deepseek_batchsplit_fp8.py:1048-1049): the finished
+      # bf16 result times the row's factor, rounded again; autograd gives both gradients
+      out = (out.float() * out_row_scale.reshape(-1, 1).float()).to(torch.bfloat16)
     # (the differentiable kernels produce bf16; a float32 result is that value widened, and its gradient arrives rounded to bf16)
     return out if preferred_element_type == torch.bfloat16 else out.to(preferred_element_type)
 
@@ -383,10 +393,18 @@ class _GmmFn(torch.autograd.Function):
   """
 
   @staticmethod
-  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual):
+  def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual, partial_sum=None, existing_out=None, row_idx=None, row_div=1,
+              row_inv=None):
+    """partial_sum [m, n] is added to the product, existing_out [m, n] receives the rows of the local groups (both get
+    the incoming gradient as theirs, ops.py:524-527); row_idx / row_div: row i of the product reads lhs row
+    row_idx[i] // row_div (the fused permute: lhs holds the T token rows and no [m, k] copy is kept for the backward),
+    row_inv: the inverse permutation of row_idx when it is one (the gradient of lhs is then a deterministic sum over each
+    token's row_div copies instead of an atomic scatter)."""
     lhs_q, rhs_q = (rule.act_qtype, rule.weight_qtype) if rule is not None else (None, None)
     bwd_q = rule.bwd_qtype if rule is not None else None
     ctx.offset, ctx.transpose_rhs, ctx.bwd_q = offset, transpose_rhs, bwd_q
+    ctx.row_div, ctx.has_ps, ctx.has_eo = int(row_div), partial_sum is not None, existing_out is not None
+    ctx.lhs_rows = lhs.shape[0]
     both_int8 = lhs_q in _INT8_NAMES and rhs_q in _INT8_NAMES
     both_fp8 = lhs_q in _FP8_NAMES and rhs_q in _FP8_NAMES
     ctx.quantized = both_int8 or both_fp8
@@ -394,22 +412,39 @@ class _GmmFn(torch.autograd.Function):
       raise NotImplementedError("bwd_quantize_dtype needs an int8 x int8 or fp8 x fp8 forward (channelwise or static scales)")
     if bwd_q is not None and bwd_q not in _E5M2_NAMES:
       raise ValueError(f"unsupported bwd_quantize_dtype {bwd_q}")
+    extra = dict(partial_sum=partial_sum, existing_out=existing_out, lhs_row_idx=row_idx, lhs_row_idx_div=int(row_div))
+    if existing_out is not None:
+      ctx.mark_dirty(existing_out)
+    none = torch.empty(0, device=lhs.device)
+    idx_t = (row_idx if row_idx is not None else none, row_inv if row_inv is not None else none)
+    ctx.has_idx, ctx.has_inv = row_idx is not None, row_inv is not None
     with torch.no_grad():
       if ctx.quantized:
         lq = quantize_lhs(lhs.contiguous(), lhs_q, calibration_method=rule.act_calibration_method)
         rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q, calibration_method=rule.weight_calibration_method, manual=manual)
-        ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes)
+        ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes, *idx_t)
         ctx.rhs_dtype = rhs.dtype
-        return gmm(lq, rq, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=True)
-      ctx.save_for_backward(lhs, rhs, group_sizes)
+        return gmm(lq, rq, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=True, **extra)
+      ctx.save_for_backward(lhs, rhs, group_sizes, *idx_t)
       kw = {}
       if rule is not None:
         kw = dict(use_qwix_quantization=True, qwix_rule=rule, use_manual_quantization=manual)
-      return gmm(lhs, rhs, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=transpose_rhs, **kw)
+      return gmm(lhs, rhs, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=transpose_rhs, **kw, **extra)
+
+  @staticmethod
+  def _rows_to_tokens(ctx, d_rows, row_idx, row_inv):
+    """Gradient of the rows read through the index -> gradient of the lhs rows themselves."""
+    if not ctx.has_idx:
+      return d_rows
+    if ctx.has_inv:  # a permutation: token t's copies are the rows row_inv[t * div .. + div - 1], summed in f32 in that order
+      return kernels.unpermute_combine(d_rows.contiguous(), None, k=ctx.row_div, inv_perm=row_inv)
+    acc = torch.zeros((ctx.lhs_rows, d_rows.shape[1]), dtype=torch.float32, device=d_rows.device)
+    acc.index_add_(0, torch.div(row_idx, ctx.row_div, rounding_mode="floor").long().clamp_(0, ctx.lhs_rows - 1), d_rows.float())
+    return acc.to(d_rows.dtype)
 
   @staticmethod
   def _backward_quantized(ctx, dout):
-    lq, ls, rq, rs, group_sizes = ctx.saved_tensors  # lq [m,k], ls [m] or [1]; rq [g,n,k], rs [g,n], [1,n] or [1]
+    lq, ls, rq, rs, group_sizes, row_idx, row_inv = ctx.saved_tensors  # lq [m,k], ls [m] or [1]; rq [g,n,k], rs [g,n], [1,n] or [1]
     m, n = dout.shape
     k = lq.shape[1]
     g_local = rq.shape[0]
@@ -442,15 +477,21 @@ class _GmmFn(torch.autograd.Function):
                                  group_offset=ctx.offset, out_row_scale=s_row)
         else:
           dlhs = kernels.gmm_raw(d, w_b, group_sizes, group_offset=ctx.offset, out_row_scale=s_row)
+      dlhs = _GmmFn._rows_to_tokens(ctx, dlhs, row_idx, row_inv)
     if marks:
       marks[1].record()
     if ctx.needs_input_grad[1]:
       # dout times the activations' row scales, e5m2 per column
+      lq_rows = lq
+      if ctx.has_idx:  # the quantised token rows, gathered for this product only (int8 / fp8 rows: half of a bf16 copy)
+        tok = torch.div(row_idx, ctx.row_div, rounding_mode="floor").long().clamp_(0, lq.shape[0] - 1)
+        lq_rows = lq[tok]
+        ls = ls if ls.numel() == 1 else ls[tok].contiguous()
       ls_m = ls if ls.numel() == m else ls.reshape(1).expand(m).contiguous()
       d, s_col = kernels.bwd_scale_grad(dout, ls_m, mode="drhs", quantize=quant)
       # the column scales go back onto the f32 products in the kernel's epilogue, which rounds once to the weights' type
       direct = ctx.rhs_dtype in (torch.bfloat16, torch.float32)
-      w = kernels.tgmm(lq.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
+      w = kernels.tgmm(lq_rows.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
                        out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
       w = w.to(ctx.rhs_dtype)
       drhs = w if ctx.transpose_rhs else w.transpose(1, 2)
@@ -463,12 +504,15 @@ class _GmmFn(torch.autograd.Function):
 
   @staticmethod
   def backward(ctx, dout):
+    g_in = dout
     dout = dout.to(torch.bfloat16).contiguous()
+    # the gradients of partial_sum and existing_out are the incoming gradient itself (ops.py:524-527)
+    tail = (None, None, None, None, None, g_in if ctx.has_ps else None, g_in if ctx.has_eo else None, None, None, None)
     if ctx.quantized:
       with torch.no_grad():
         dlhs, drhs = _GmmFn._backward_quantized(ctx, dout)
-      return dlhs, drhs, None, None, None, None, None
-    lhs, rhs, group_sizes = ctx.saved_tensors
+      return (dlhs, drhs) + tail
+    lhs, rhs, group_sizes, row_idx, row_inv = ctx.saved_tensors
     dlhs = drhs = None
     ev = PROFILE_EVENTS
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(3)] if ev is not None else None
@@ -479,17 +523,20 @@ class _GmmFn(torch.autograd.Function):
         # dout [m, n] @ rhs[g]^T: the kernel's weight layout [G, out, in] is here [G, k, n]
         dlhs = gmm(dout, rhs, group_sizes, torch.bfloat16, group_offset=ctx.offset, transpose_rhs=not ctx.transpose_rhs)
         # rows of groups outside [offset, offset + G_local) are zero in the forward output
+        dlhs = _GmmFn._rows_to_tokens(ctx, dlhs, row_idx, row_inv)
       if marks:
         marks[1].record()
       if ctx.needs_input_grad[1]:
-        d = tgmm(lhs.t(), dout, group_sizes, rhs.dtype, group_offset=ctx.offset, num_actual_groups=rhs.shape[0])
+        # with a row index the gathered copy exists for this product only (it is not kept from the forward pass)
+        rows = kernels.gather_rows(lhs.contiguous(), row_idx, ctx.row_div) if ctx.has_idx else lhs
+        d = tgmm(rows.t(), dout, group_sizes, rhs.dtype, group_offset=ctx.offset, num_actual_groups=rhs.shape[0])
         drhs = d.transpose(1, 2) if ctx.transpose_rhs else d.contiguous()
       if marks:
         marks[2].record()
         shape = f"k{lhs.shape[1]}_n{dout.shape[1]}"
         ev.append(("dlhs_" + shape, marks[0], marks[1]))
         ev.append(("tgmm_" + shape, marks[1], marks[2]))
-    return dlhs, drhs, None, None, None, None, None
+    return (dlhs, drhs) + tail
 
 
 def _lib_per_tensor():
@@ -542,18 +589,24 @@ class _BiasFn(torch.autograd.Function):
 
 
 def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual, fuse_act, act_limit, rhs_bias=None,
-                   rhs_up_bias=None):
+                   rhs_up_bias=None, partial_sum=None, partial_sum_up=None, existing_out=None, lhs_row_idx=None, lhs_row_idx_div=1,
+                   lhs_row_inv=None):
   for name, t in (("lhs", lhs), ("rhs", rhs), ("rhs_up", rhs_up)):
     if t is not None and not isinstance(t, torch.Tensor):
       raise NotImplementedError(f"gradients need bf16 tensors; {name} is already quantised")
-  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual)
+  if existing_out is not None and (rhs_up is not None or rhs_bias is not None):
+    raise NotImplementedError("existing_out takes the plain product (no rhs_up, no bias) on the differentiable path")
+  ps = None if partial_sum is None else partial_sum.to(torch.bfloat16).contiguous()
+  ps_up = None if partial_sum_up is None else partial_sum_up.to(torch.bfloat16).contiguous()
+  idx = (lhs_row_idx, lhs_row_idx_div, lhs_row_inv)
+  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual, ps, existing_out, *idx)
   if rhs_bias is not None:
     h0 = _BiasFn.apply(h0, rhs_bias, group_sizes, offset)
   if rhs_up is None:
     if fuse_act is not None:
       raise ValueError("fuse_act needs rhs_up")
     return h0
-  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual)
+  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual, ps_up, None, *idx)
   if rhs_up_bias is not None:
     h1 = _BiasFn.apply(h1, rhs_up_bias, group_sizes, offset)
   if fuse_act is None:

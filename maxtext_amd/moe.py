@@ -331,9 +331,12 @@ class RoutedMoE:
     if use_ragged_sort:
       row_range = torch.stack([torch.zeros((), dtype=torch.int32, device=inputs.device), local_group_size.sum().to(torch.int32)])
     if torch.is_grad_enabled() and inputs.requires_grad:
-      if row_range is not None:
-        raise NotImplementedError("gradients through the ragged sort are not implemented")
-      sorted_inputs = _GatherRowsFn.apply(inputs, sorted_indices, inv, 1)
+      if row_range is not None:  # a2a_ragged_sort with its custom VJP (kernels/ragged/ragged_sort.py:454-537)
+        from maxtext_amd import ragged_sort
+
+        sorted_inputs = ragged_sort._A2aSortFn.apply(inputs, sorted_indices, row_range)
+      else:
+        sorted_inputs = _GatherRowsFn.apply(inputs, sorted_indices, inv, 1)
     else:
       sorted_inputs = kernels.gather_rows(inputs.contiguous(), sorted_indices, 1, row_range=row_range)
     return sorted_inputs, sorted_indices, local_group_size, sorted_experts_ids
@@ -379,7 +382,7 @@ class RoutedMoE:
 
   # -- the three grouped GEMMs: gmm_up + apply_ffn_activation + wo (moe.py:1932-1986, :841, :2226)
   def _experts(self, sorted_inputs, group_size, w0, w1, wo, w0_bias=None, w1_bias=None, wo_bias=None, row_idx=None, row_idx_div=1,
-               workspace=None):
+               workspace=None, row_inv=None):
     """row_idx / row_idx_div: `sorted_inputs` holds the T token rows (plain or quantised) and row i of the first product
     reads row row_idx[i] // row_idx_div of it: the permute fused into the matmul, no [M, d] copy."""
     cfg = self.config
@@ -404,7 +407,7 @@ class RoutedMoE:
         q = "fp8" if cfg.act_quant == "fp8_row" else cfg.act_quant
         qkw = dict(lhs_quantize_dtype=q, rhs_quantize_dtype=q)
       inter = megablox.gmm(sorted_inputs, w0, group_size, bf16, transpose_rhs=True, rhs_up=w1, fuse_act=act, act_limit=limit,
-                           rhs_bias=w0_bias, rhs_up_bias=w1_bias, **qkw)
+                           rhs_bias=w0_bias, rhs_up_bias=w1_bias, lhs_row_idx=row_idx, lhs_row_idx_div=row_idx_div, lhs_row_inv=row_inv, **qkw)
       return megablox.gmm(inter, wo, group_size, bf16, transpose_rhs=True, rhs_bias=wo_bias, **qkw)
     # one tile-list buffer for both products: the second reuses the first one's list when its tile height agrees
     rows = row_idx.shape[0] if row_idx is not None else (sorted_inputs.qvalue if isinstance(sorted_inputs, QArray) else sorted_inputs).shape[0]
@@ -447,8 +450,10 @@ class RoutedMoE:
     training = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (x2d, weights, w0_kernel, w1_kernel, wo_kernel))
     if training:
-      sorted_inputs = _GatherRowsFn.apply(x2d, perm, inv, k) if x2d.requires_grad else kernels.gather_rows(x2d, perm, k)
-      inter = self._experts(sorted_inputs, group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias)
+      # the permute stays fused under grad: the first products read the token rows through perm, their input gradient is
+      # summed over each token's k copies through inv (the custom VJP of moe.py:154-171), and no [M, d] copy is kept
+      inter = self._experts(x2d, group_size, w0_kernel, w1_kernel, wo_kernel, w0_bias, w1_bias, wo_bias, row_idx=perm, row_idx_div=k,
+                            row_inv=inv)
     else:
       # the permute is fused into the first grouped matmul: the T token rows are quantised once (not their M = T * k
       # copies) and the matmul reads row perm[i] // k for its row i, so the [M, d] gathered copy is never written

@@ -288,3 +288,112 @@ def test_a2a_ragged_sort_unsort():
   s = ragged_sort.a2a_ragged_sort(x.cuda(), cuda_i32(keep), 600)
   back = ragged_sort.a2a_ragged_unsort(s, cuda_i32(np.argsort(keep).astype(np.int32)), 600)
   assert torch.equal(back[:600].cpu(), x[:600]) and not back[600:].any()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_ring_ragged_sort_unsort_gradients(seed):
+  """The custom VJPs of ring_ragged_sort / ring_ragged_unsort (kernels/ragged/ragged_sort.py:155-224, :364-441) against
+  torch autograd through a plain restatement of the forward passes (index_select + mask), full and packed buffers."""
+  from maxtext_amd import ragged_sort
+  from tolerances import relerr
+
+  rng = np.random.default_rng(500 + seed)
+  ep = int(rng.choice([1, 2, 4]))
+  e = ep * int(rng.choice([2, 4, 16]))
+  k = int(rng.integers(1, min(e, 6) + 1))
+  t = int(rng.choice([5, 64, 300]))
+  d = int(rng.choice([8, 64, 256]))
+  sel = np.stack([rng.permutation(e)[:k] for _ in range(t)]).astype(np.int32)
+  n = t * k
+  flat = sel.reshape(-1)
+  perm = np.argsort(flat, kind="stable")
+  gs = np.bincount(flat, minlength=e)
+  local = e // ep
+  x = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(torch.bfloat16)
+  w = torch.from_numpy(rng.random((t, k)).astype(np.float32))
+  for shard in sorted({0, ep - 1}):
+    start = int(gs[: shard * local].sum())
+    end = start + int(gs[shard * local:(shard + 1) * local].sum())
+    for buf in (None, max(n // (2 * ep), 1)):
+      rows = n if buf is None or buf >= n else buf
+      # positions of the buffer that hold a row, and the flat slot each of them copies
+      if rows == n:
+        pos = np.arange(start, end)
+        slots = perm[start:end]
+      else:
+        cnt = min(end - start, rows)
+        pos = np.arange(cnt)
+        slots = perm[start:start + cnt]
+      pos_t, tok_t = torch.from_numpy(pos).long(), torch.from_numpy(slots // k).long()
+      # sort: x_sorted[pos] = hidden[token of the slot]
+      g_x = torch.from_numpy(rng.standard_normal((rows, d)).astype(np.float32)).to(torch.bfloat16)
+      h = x.double().requires_grad_()
+      ref = torch.zeros((rows, d), dtype=torch.float64).index_put((pos_t,), h[tok_t])
+      (ref * g_x.double()).sum().backward()
+      hg = x.cuda().requires_grad_()
+      got_x, got_gs, got_rev = ragged_sort.ring_ragged_sort(hg, cuda_i32(sel), e, k, shard, ep, buffer_size=buf)
+      assert torch.equal(got_x.detach().cpu().float(), ref.detach().float())
+      got_x.backward(g_x.cuda())
+      if h.grad.abs().max() > 0:
+        assert relerr(hg.grad, h.grad) <= 1e-2
+      else:
+        assert not hg.grad.any()
+      # unsort: out[token] = sum over its slots in the buffer of w[slot] * y[pos]
+      y = torch.from_numpy(rng.standard_normal((rows, d)).astype(np.float32)).to(torch.bfloat16)
+      g_o = torch.from_numpy(rng.standard_normal((t, d)).astype(np.float32)).to(torch.bfloat16)
+      yd = y.double().requires_grad_()
+      contrib = yd[pos_t] * w.reshape(-1).double()[torch.from_numpy(slots).long()][:, None]
+      ref_o = torch.zeros((t, d), dtype=torch.float64).index_add(0, tok_t, contrib)
+      (ref_o * g_o.double()).sum().backward()
+      yg = y.cuda().requires_grad_()
+      got_o = ragged_sort.ring_ragged_unsort(yg, got_gs, got_rev, k, local, shard, w.cuda())
+      if ref_o.abs().max() > 0:
+        assert relerr(got_o, ref_o) <= 1e-2
+      got_o.backward(g_o.cuda())
+      if yd.grad.abs().max() > 0:
+        assert relerr(yg.grad, yd.grad) <= 1e-2
+      else:
+        assert not yg.grad.any()
+
+
+def test_a2a_ragged_sort_unsort_gradients():
+  """The custom VJPs of a2a_ragged_sort / a2a_ragged_unsort (ragged_sort.py:515-537, :596-616) and of
+  local_permute(use_ragged_sort=True) against torch autograd through out = where(i < end, x[idx[i]], 0)."""
+  from maxtext_amd import moe, ragged_sort
+
+  rng = np.random.default_rng(11)
+  n, d = 700, 128
+  x = torch.from_numpy(rng.standard_normal((n, d)).astype(np.float32)).to(torch.bfloat16)
+  g = torch.from_numpy(rng.standard_normal((n, d)).astype(np.float32)).to(torch.bfloat16)
+  for valid in (0, 1, 400, n):
+    # a permutation that keeps the valid prefix in place as a set (the case the reference's unsort rule is exact for)
+    idx = np.concatenate([rng.permutation(valid), valid + rng.permutation(n - valid)]).astype(np.int32)
+    mask = (torch.arange(n) < valid)[:, None]
+    xd = x.double().requires_grad_()
+    (torch.where(mask, xd[torch.from_numpy(idx).long()], torch.zeros((), dtype=torch.float64)) * g.double()).sum().backward()
+    for fn in (ragged_sort.a2a_ragged_sort, ragged_sort.a2a_ragged_unsort):
+      xg = x.cuda().requires_grad_()
+      out = fn(xg, cuda_i32(idx), valid)
+      out.backward(g.cuda())
+      assert torch.equal(xg.grad.cpu().double(), xd.grad)  # a permutation of rows: exact
+  # a2a_ragged_sort alone is exact for any permutation
+  idx = rng.permutation(n).astype(np.int32)
+  xd = x.double().requires_grad_()
+  (torch.where((torch.arange(n) < 250)[:, None], xd[torch.from_numpy(idx).long()], torch.zeros((), dtype=torch.float64)) * g.double()).sum().backward()
+  xg = x.cuda().requires_grad_()
+  ragged_sort.a2a_ragged_sort(xg, cuda_i32(idx), 250).backward(g.cuda())
+  assert torch.equal(xg.grad.cpu().double(), xd.grad)
+  # local_permute with the ragged sort, under grad: rows past the received total get no gradient
+  sizes = np.array([[3, 0, 5, 2], [1, 4, 0, 6]], np.int32)  # 2 batch shards x 4 experts; this shard owns experts 2, 3
+  rows = 20
+  buf = torch.from_numpy(rng.standard_normal((rows, d)).astype(np.float32)).to(torch.bfloat16)
+  bg = buf.cuda().requires_grad_()
+  sorted_inputs, sorted_indices, local_sizes, _ = moe.RoutedMoE.local_permute(bg, cuda_i32(sizes), 2, 1, use_ragged_sort=True)
+  total = int(local_sizes.sum())
+  assert total == 5 + 2 + 0 + 6
+  gg = torch.ones_like(sorted_inputs)
+  sorted_inputs.backward(gg)
+  got = bg.grad.cpu().float()
+  want = torch.zeros(rows, d)
+  want[sorted_indices.cpu().long()[:total]] = 1.0
+  assert torch.equal(got, want)

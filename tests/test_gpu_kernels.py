@@ -806,6 +806,100 @@ def test_gmm_autograd_through_fused_activation():
   assert relerr(r1.grad, b1.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
 
 
+@pytest.mark.parametrize("quant", [None, "int8", "fp8"])
+@pytest.mark.parametrize("with_inverse", [True, False])
+def test_gmm_autograd_with_row_index(quant, with_inverse):
+  """The fused permute under grad: lhs holds the T token rows, row i of the product reads row perm[i] // k.  dlhs is the sum
+  of each token's k row gradients (a deterministic sum through the inverse permutation, or a scatter-add when the index
+  is not a permutation), drhs reads the rows through the index again; against torch autograd in f64 (unquantised) or the
+  same call on the gathered copy (quantised forward with its quantised backward)."""
+  from maxtext_amd import megablox
+  from maxtext_amd.quantizations import QtRule
+
+  g = torch.Generator().manual_seed(15)
+  t, k, kd, n = 300, 2, 256, 192
+  m = t * k
+  gs = np.array([250, 0, 200, 120], np.int32)  # 30 trailing rows in no group
+  x = torch.randn(t, kd, generator=g).to(torch.bfloat16)
+  w = (torch.randn(4, kd, n, generator=g) * 0.05).to(torch.bfloat16)
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  if with_inverse:
+    perm = torch.randperm(m, generator=g).to(torch.int32)
+    inv = torch.empty_like(perm)
+    inv[perm.long()] = torch.arange(m, dtype=torch.int32)
+  else:
+    perm = torch.randint(0, m, (m,), generator=g).to(torch.int32)  # tokens read any number of times
+    inv = None
+  rows = (perm // k).long()
+  kw = {}
+  if quant is not None:
+    kw = dict(use_qwix_quantization=True, qwix_rule=QtRule(weight_qtype=quant, act_qtype=quant, bwd_qtype="float8_e5m2"))
+  xg, wg = cuda(x).requires_grad_(), cuda(w).requires_grad_()
+  out = gmm_bf16(xg, wg, cuda(gs), lhs_row_idx=cuda(perm), lhs_row_idx_div=k, lhs_row_inv=None if inv is None else cuda(inv), **kw)
+  out.backward(cuda(dout))
+  if quant is None:
+    x64, w64 = x.double().requires_grad_(), w.double().requires_grad_()
+    lhs64 = x64[rows]
+    off = np.concatenate([[0], np.cumsum(gs)])
+    ref = torch.cat([lhs64[off[i]:off[i + 1]] @ w64[i] for i in range(4)] + [torch.zeros(m - off[-1], n, dtype=torch.float64)])
+    (ref * dout.double()).sum().backward()
+    assert relerr(out, ref) <= TOL
+    assert relerr(xg.grad, x64.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= TOL and relerr(wg.grad, w64.grad) <= TOL
+  else:
+    # the same products on the gathered copy: per-row quantisation commutes with the gather, so forward and weight
+    # gradient are bit-equal and the token gradient is the sum of the copy's row gradients
+    x2 = cuda(x).requires_grad_()
+    w2 = cuda(w).requires_grad_()
+    gathered = x2[cuda(rows)]
+    out2 = gmm_bf16(gathered, w2, cuda(gs), **kw)
+    assert torch.equal(out, out2)
+    out2.backward(cuda(dout))
+    assert torch.equal(wg.grad, w2.grad)
+    assert relerr(xg.grad, x2.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= TOL
+
+
+def test_gmm_autograd_partial_sum_existing_out_and_row_scale():
+  """The remaining differentiable arguments: partial_sum and existing_out receive the incoming gradient (ops.py:524-527),
+  out_row_scale multiplies the finished rows (its gradient is the row's inner product with the incoming gradient)."""
+  from maxtext_amd import megablox
+
+  g = torch.Generator().manual_seed(16)
+  m, kd, n = 420, 128, 136
+  gs = np.array([200, 0, 220], np.int32)
+  lhs = torch.randn(m, kd, generator=g).to(torch.bfloat16)
+  w = (torch.randn(3, kd, n, generator=g) * 0.05).to(torch.bfloat16)
+  ps = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  scale = torch.rand(m, generator=g) + 0.5
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  a, b, p64, s64 = lhs.double().requires_grad_(), w.double().requires_grad_(), ps.double().requires_grad_(), scale.double().requires_grad_()
+  off = [0, 200, 200, 420]
+  ref = (torch.cat([a[off[i]:off[i + 1]] @ b[i] for i in range(3)]) + p64) * s64[:, None]
+  (ref * dout.double()).sum().backward()
+  la, wa, pa, sa = cuda(lhs).requires_grad_(), cuda(w).requires_grad_(), cuda(ps).requires_grad_(), cuda(scale).requires_grad_()
+  out = gmm_bf16(la, wa, cuda(gs), partial_sum=pa, out_row_scale=sa)
+  assert relerr(out, ref) <= TOL
+  out.backward(cuda(dout))
+  assert relerr(la.grad, a.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= TOL and relerr(wa.grad, b.grad, atol_rms=ELEM_ATOL_RMS_CHAINED) <= TOL
+  assert relerr(pa.grad, p64.grad) <= TOL and relerr(sa.grad, s64.grad) <= TOL
+  # existing_out: two shards of the experts write their rows into one buffer; its gradient is the incoming gradient
+  gs5 = np.array([100, 60, 0, 160, 100], np.int32)
+  w5 = (torch.randn(5, kd, n, generator=g) * 0.05).to(torch.bfloat16)
+  la = cuda(lhs).requires_grad_()
+  w_lo, w_hi = cuda(w5[:2]).requires_grad_(), cuda(w5[2:]).requires_grad_()
+  buf = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda").requires_grad_()
+  first = gmm_bf16(la, w_lo, cuda(gs5), existing_out=buf.clone(), group_offset=0)
+  both = gmm_bf16(la, w_hi, cuda(gs5), existing_out=first, group_offset=2)
+  both.backward(cuda(dout))
+  a, b = lhs.double().requires_grad_(), w5.double().requires_grad_()
+  off = np.concatenate([[0], np.cumsum(gs5)])
+  ref = torch.cat([a[off[i]:off[i + 1]] @ b[i] for i in range(5)])
+  (ref * dout.double()).sum().backward()
+  assert relerr(both, ref) <= TOL
+  assert relerr(la.grad, a.grad) <= TOL
+  assert relerr(torch.cat([w_lo.grad, w_hi.grad]), b.grad) <= TOL
+  assert torch.equal(buf.grad, cuda(dout))
+
+
 # ---------------------------------------------------------------- router: gate matmul + top-k in one call
 
 
