@@ -873,6 +873,42 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in
   }
 }
 
+// 1-byte elements with K % 16 == 0 and N % 16 == 0 (the int8 / fp8 weights the quantised backward re-lays out on every
+// step): a 128 x 128 tile goes through LDS with 16-byte loads along N and 16-byte stores along K, so that every request
+// covers whole 128-byte lines on both sides; a lane gathers the 16 bytes of its output chunk with byte reads.  The chunk c
+// of row k sits at slot c ^ (k / 16 % 8), which spreads the eight rows a store instruction's lanes read over the banks.
+__global__ __launch_bounds__(256) void transpose8_kernel(const uint8_t* __restrict__ in, int K, int N, uint8_t* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[128 * 128];
+  const size_t g = blockIdx.z;
+  const int k0 = blockIdx.y * 128, n0 = blockIdx.x * 128;
+  const int tid = threadIdx.x;
+  {
+    const int c = tid % 8, r = tid / 8;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+      const int k = it * 32 + r;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (k0 + k < K && n0 + c * 16 < N) v = *(const uint4*)(in + (g * K + k0 + k) * N + n0 + c * 16);
+      *(uint4*)(tile + k * 128 + ((c ^ ((k >> 4) & 7)) << 4)) = v;
+    }
+  }
+  __syncthreads();
+  const int kc = tid % 8, nr = tid / 8;
+  if (k0 + kc * 16 >= K) return;
+#pragma unroll
+  for (int it = 0; it < 4; it++) {
+    const int n = it * 32 + nr;
+    if (n0 + n >= N) continue;
+    const uint8_t* src = tile + kc * 16 * 128 + (((n >> 4) ^ kc) << 4) + (n & 15);
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+      w[q] = (uint32_t)src[(4 * q) * 128] | ((uint32_t)src[(4 * q + 1) * 128] << 8) | ((uint32_t)src[(4 * q + 2) * 128] << 16) |
+             ((uint32_t)src[(4 * q + 3) * 128] << 24);
+    *(uint4*)(out + (g * N + n0 + n) * K + k0 + kc * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
 // 2-byte elements with K % 8 == 0 and N % 8 == 0: 16-byte loads along N into LDS, then ds_read_b64_tr_b16 (the
 // transposing LDS load: 16 lanes read a 4 x 16 block and lane L receives column L) twice per lane, which yields 8
 // consecutive K values of one output row as one 16-byte store.
@@ -1186,7 +1222,9 @@ int moe_transpose_rhs(const void* rhs_gkn, int G, int K, int N, int elem_bytes, 
   if (G > 65535 || cdiv(K, 64) > 65535) return fail(MOE_ERR_UNSUPPORTED, "transpose: grid too large");
   dim3 grid(cdiv(N, 64), cdiv(K, 64), G);
   hipStream_t s = (hipStream_t)stream;
-  if (elem_bytes == 1)
+  if (elem_bytes == 1 && K % 16 == 0 && N % 16 == 0 && (((uintptr_t)rhs_gkn | (uintptr_t)rhs_gnk) & 15) == 0)
+    transpose8_kernel<<<dim3(cdiv(N, 128), cdiv(K, 128), G), 256, 0, s>>>((const uint8_t*)rhs_gkn, K, N, (uint8_t*)rhs_gnk);
+  else if (elem_bytes == 1)
     transpose_kernel<uint8_t><<<grid, 256, 0, s>>>((const uint8_t*)rhs_gkn, K, N, (uint8_t*)rhs_gnk);
   else if (elem_bytes == 2 && K % 8 == 0 && N % 8 == 0 && (((uintptr_t)rhs_gkn | (uintptr_t)rhs_gnk) & 15) == 0)
     transpose16_kernel<<<grid, 256, 0, s>>>((const uint16_t*)rhs_gkn, K, N, (uint16_t*)rhs_gnk);

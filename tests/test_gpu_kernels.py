@@ -364,6 +364,11 @@ def test_combine_exact_on_integers(K):
 def test_transpose_rhs(K):
   w = torch.randint(-128, 128, (3, 200, 136), dtype=torch.int8)
   assert torch.equal(K.transpose_rhs(cuda(w)).cpu(), w.transpose(1, 2).contiguous())
+  for shape in ((2, 208, 144), (3, 128, 128), (1, 16, 16), (2, 1040, 400), (2, 128, 2064)):  # 1-byte, 16-byte path, ragged 128 x 128 tiles
+    w8 = torch.randint(-128, 128, shape, dtype=torch.int8)
+    assert torch.equal(K.transpose_rhs(cuda(w8)).cpu(), w8.transpose(1, 2).contiguous()), shape
+    f8 = torch.randn(*shape).to(torch.float8_e4m3fn)
+    assert torch.equal(K.transpose_rhs(cuda(f8)).cpu().view(torch.uint8), f8.transpose(1, 2).contiguous().view(torch.uint8)), shape
   wb = torch.randn(2, 70, 264).to(torch.bfloat16)  # K % 8 != 0: element-wise kernel
   assert torch.equal(K.transpose_rhs(cuda(wb)).cpu(), wb.transpose(1, 2).contiguous())
   for shape in ((2, 72, 264), (3, 128, 64), (1, 200, 136), (2, 8, 8), (1, 1024, 520)):  # 16-byte path, ragged tiles
