@@ -252,9 +252,10 @@ __global__ __launch_bounds__(C::THREADS, C::NWAVES >= 8 ? 2 : 1) void gmm_dl_ker
             acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                 __builtin_bit_cast(v8bf, gb[SET][j]), __builtin_bit_cast(v8bf, ga[i]), acc[j][i], 0, 0, 0);
           }
-          // the stage's requests go out one per MFMA from the start of the k-step: they have until the middle of the
-          // next stage to land, and spreading them over the whole k-step measured 5 % slower
-          if (LD && i * C::TN + j < C::LPS) issue_one(ld_kt, ld_buf, i * C::TN + j);
+          // the stage's requests go out behind every third MFMA from the start of the k-step: one per MFMA fills the
+          // address unit's queue, and the MFMAs behind a request that waits for a free entry wait with it (dlhs of the
+          // Mixtral shape 1.71 -> 1.60 and 1.91 -> 1.83 ms); over the whole k-step they land too late (1.66 / 1.85 ms)
+          if (LD && (i * C::TN + j) % 3 == 0 && (i * C::TN + j) / 3 < C::LPS) issue_one(ld_kt, ld_buf, (i * C::TN + j) / 3);
           if (RD && j == 1 && i < C::TN) read_b16(rd_buf, rd_ks, SET ^ 1, i);
           if (RD && j == C::TN - 1) read_a16(rd_buf, rd_ks, i);
           __builtin_amdgcn_sched_barrier(0);
