@@ -215,6 +215,21 @@ MOE_API int moe_local_expert_keys(const int32_t* global_group_sizes, int num_bat
 MOE_API int moe_all_to_all_params(const int32_t* all_shards_group_sizes, int num_expert_parallelism, int shard_id,
                           int is_batch_sharded, long long buffer_size, int is_dispatch, int32_t* input_offsets,
                           int32_t* send_sizes, int32_t* output_offsets, int32_t* recv_sizes, void* stream);
+/* The same three calls with the shard's index in device memory (an int32 the kernels read; the host never does): inside
+ * shard_map the reference takes it from jax.lax.axis_index (moe.py:1134, :1709-1712, :2014-2019), a traced device value that
+ * a custom call receives as a buffer.  Values outside the shards that exist are clamped into them.  In
+ * moe_ring_ragged_indices_dev the shard owns experts [shard * local_experts, (shard + 1) * local_experts), so num_experts
+ * must be a multiple of local_experts. */
+MOE_API int moe_ring_ragged_indices_dev(const int32_t* indices, const int32_t* group_sizes, int num_experts,
+                            const int32_t* shard_index_dev, int local_experts, int num_rows, int buffer_size, int unsort,
+                            int32_t* indices_out, uint8_t* valid_rows_mask, int32_t* row_range, void* stream);
+MOE_API int moe_local_expert_keys_dev(const int32_t* global_group_sizes, int num_batch_shards, int num_experts,
+                          int local_expert_size, const int32_t* shard_index_dev, int num_rows,
+                          const int32_t* global_sorted_experts, int truncate, int32_t* expert_keys, int32_t* local_group_size,
+                          void* workspace, size_t workspace_bytes, void* stream);
+MOE_API int moe_all_to_all_params_dev(const int32_t* all_shards_group_sizes, int num_expert_parallelism,
+                          const int32_t* shard_id_dev, int is_batch_sharded, long long buffer_size, int is_dispatch,
+                          int32_t* input_offsets, int32_t* send_sizes, int32_t* output_offsets, int32_t* recv_sizes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Row gather with optional quantisation.  Replaces the data half of permute

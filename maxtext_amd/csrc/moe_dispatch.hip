@@ -33,13 +33,20 @@ __device__ __forceinline__ long long block_inclusive_scan(long long v, long long
   return incl;
 }
 
+// A shard's index as the caller holds it: by value, or in device memory (inside shard_map it is jax.lax.axis_index, which
+// only exists on the device); a device value is clamped into [0, hi] so that no table is indexed outside its rows.
+__device__ __forceinline__ int resolve_shard(int by_value, const int32_t* dev, int hi) {
+  return dev ? min(max(*dev, 0), hi) : by_value;
+}
+
 // starts[i], i < S * L: rows that precede segment i = (batch shard i / L, local expert i % L) in the received buffer;
 // starts[S * L] = rows received.  local_group_size[l] = sum over the batch shards of segment (s, l), each segment cut
 // to what is left of `capacity` rows when the prefix sum reaches it (capacity < 0: no cut).
 __global__ __launch_bounds__(kDispThreads) void local_sizes_kernel(const int32_t* __restrict__ global_group_sizes, int S, int E, int L,
-                                                                   int shard_index, long long capacity, int32_t* __restrict__ starts,
-                                                                   int32_t* __restrict__ local_group_size) {
+                                                                   int shard_index, const int32_t* __restrict__ shard_dev, long long capacity,
+                                                                   int32_t* __restrict__ starts, int32_t* __restrict__ local_group_size) {
   __shared__ long long s_buf[kDispThreads];
+  shard_index = resolve_shard(shard_index, shard_dev, E / L - 1);
   const int tid = threadIdx.x;
   const int n = S * L;
   long long carry = 0;
@@ -88,10 +95,11 @@ __global__ void local_keys_kernel(const int32_t* __restrict__ starts, int n, int
 
 // Rows sorted by global expert (every routed row of the replicated batch): this shard's rows keep their local expert,
 // all others get the key L, which sorts them behind (moe.py:1166-1172).
-__global__ void offset_keys_kernel(const int32_t* __restrict__ global_sorted_experts, int L, int shard_index, int R,
-                                   int32_t* __restrict__ keys) {
+__global__ void offset_keys_kernel(const int32_t* __restrict__ global_sorted_experts, int L, int shard_index, const int32_t* __restrict__ shard_dev,
+                                   int max_shard, int R, int32_t* __restrict__ keys) {
   const int r = blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= R) return;
+  shard_index = resolve_shard(shard_index, shard_dev, max_shard);
   const int e = global_sorted_experts[r];
   // floor division and modulus as jnp.floor_divide / jnp.mod define them (a negative id belongs to no shard)
   const int q = e >= 0 ? e / L : -((-e + L - 1) / L);
@@ -102,12 +110,13 @@ __global__ void offset_keys_kernel(const int32_t* __restrict__ global_sorted_exp
 // a[i][j] = rows batch shard i sends to expert shard j, or [P] when the batch is replicated.  With a capacity the
 // matrix is cut per receiver in sender order (_truncate_matrix, moe.py:103-120); the sum of the cut entries of a
 // column up to sender n is min(column prefix, capacity), which is all the sums below need.
-__global__ __launch_bounds__(kDispThreads) void all_to_all_params_kernel(const int32_t* __restrict__ a, int P, int shard, int batch_sharded,
-                                                                         long long capacity, int dispatch, int32_t* __restrict__ input_offsets,
+__global__ __launch_bounds__(kDispThreads) void all_to_all_params_kernel(const int32_t* __restrict__ a, int P, int shard, const int32_t* __restrict__ shard_dev,
+                                                                         int batch_sharded, long long capacity, int dispatch, int32_t* __restrict__ input_offsets,
                                                                          int32_t* __restrict__ send_sizes, int32_t* __restrict__ output_offsets,
                                                                          int32_t* __restrict__ recv_sizes) {
   const int j = threadIdx.x;
   if (j >= P) return;
+  shard = resolve_shard(shard, shard_dev, P - 1);
   if (!batch_sharded) {
     long long before = 0;
     for (int i = 0; i < shard; i++) before += a[i];
@@ -154,10 +163,11 @@ __global__ __launch_bounds__(kDispThreads) void all_to_all_params_kernel(const i
 //   UNSORT: idx_in = the inverse permutation.  Unbuffered: idx_out = idx_in, mask[i] = start <= idx_in[i] < end.
 //           Buffered: idx_out[i] = idx_in[i] - start where 0 <= that < min(end - start, buffer), else 0 with mask 0.
 __global__ __launch_bounds__(256) void ring_ragged_indices_kernel(const int32_t* __restrict__ idx_in, const int32_t* __restrict__ group_sizes,
-                                                                  int E, int experts_start, int local_experts, int n, int buffer,
-                                                                  int unsort, int32_t* __restrict__ idx_out, uint8_t* __restrict__ mask_out,
-                                                                  int32_t* __restrict__ range_out) {
+                                                                  int E, int experts_start, const int32_t* __restrict__ shard_dev, int local_experts,
+                                                                  int n, int buffer, int unsort, int32_t* __restrict__ idx_out,
+                                                                  uint8_t* __restrict__ mask_out, int32_t* __restrict__ range_out) {
   __shared__ long long s_before[256], s_local[256];
+  if (shard_dev) experts_start = resolve_shard(0, shard_dev, E / local_experts - 1) * local_experts;
   long long before = 0, local = 0;
   for (int e = threadIdx.x; e < experts_start + local_experts && e < E; e += 256) {
     const long long g = max(group_sizes[e], 0);
@@ -211,9 +221,9 @@ size_t moe_local_expert_keys_workspace_bytes(int num_batch_shards, int local_exp
   return ((size_t)num_batch_shards * local_expert_size + 1) * sizeof(int32_t);
 }
 
-int moe_local_expert_keys(const int32_t* global_group_sizes, int num_batch_shards, int num_experts, int local_expert_size,
-                          int shard_index, int num_rows, const int32_t* global_sorted_experts, int truncate,
-                          int32_t* expert_keys, int32_t* local_group_size, void* workspace, size_t workspace_bytes, void* stream) {
+static int local_expert_keys_impl(const int32_t* global_group_sizes, int num_batch_shards, int num_experts, int local_expert_size,
+                                  int shard_index, const int32_t* shard_dev, int num_rows, const int32_t* global_sorted_experts, int truncate,
+                                  int32_t* expert_keys, int32_t* local_group_size, void* workspace, size_t workspace_bytes, void* stream) {
   if (!global_group_sizes || !expert_keys || !local_group_size || !workspace) return fail(MOE_ERR_INVALID_ARG, "local_expert_keys: NULL pointer");
   if (num_batch_shards <= 0 || num_experts <= 0 || local_expert_size <= 0 || shard_index < 0 || num_rows < 0)
     return fail(MOE_ERR_INVALID_ARG, "local_expert_keys: bad sizes");
@@ -225,20 +235,35 @@ int moe_local_expert_keys(const int32_t* global_group_sizes, int num_batch_shard
   hipStream_t s = (hipStream_t)stream;
   int32_t* starts = (int32_t*)workspace;
   const int n = num_batch_shards * local_expert_size;
-  local_sizes_kernel<<<1, kDispThreads, 0, s>>>(global_group_sizes, num_batch_shards, num_experts, local_expert_size, shard_index,
+  local_sizes_kernel<<<1, kDispThreads, 0, s>>>(global_group_sizes, num_batch_shards, num_experts, local_expert_size, shard_index, shard_dev,
                                                 truncate ? (long long)num_rows : -1LL, starts, local_group_size);
   if (num_rows > 0) {
     const int blocks = cdiv(num_rows, 256);
-    if (global_sorted_experts) offset_keys_kernel<<<blocks, 256, 0, s>>>(global_sorted_experts, local_expert_size, shard_index, num_rows, expert_keys);
+    if (global_sorted_experts) offset_keys_kernel<<<blocks, 256, 0, s>>>(global_sorted_experts, local_expert_size, shard_index, shard_dev, num_experts / local_expert_size - 1, num_rows, expert_keys);
     else local_keys_kernel<<<blocks, 256, 0, s>>>(starts, n, local_expert_size, num_rows, expert_keys);
   }
   note_group_sizes_rewritten(local_group_size);
   return check_launch("local_expert_keys");
 }
 
-int moe_all_to_all_params(const int32_t* all_shards_group_sizes, int num_expert_parallelism, int shard_id, int is_batch_sharded,
-                          long long buffer_size, int is_dispatch, int32_t* input_offsets, int32_t* send_sizes,
-                          int32_t* output_offsets, int32_t* recv_sizes, void* stream) {
+int moe_local_expert_keys(const int32_t* global_group_sizes, int num_batch_shards, int num_experts, int local_expert_size,
+                          int shard_index, int num_rows, const int32_t* global_sorted_experts, int truncate,
+                          int32_t* expert_keys, int32_t* local_group_size, void* workspace, size_t workspace_bytes, void* stream) {
+  return local_expert_keys_impl(global_group_sizes, num_batch_shards, num_experts, local_expert_size, shard_index, nullptr, num_rows,
+                                global_sorted_experts, truncate, expert_keys, local_group_size, workspace, workspace_bytes, stream);
+}
+
+int moe_local_expert_keys_dev(const int32_t* global_group_sizes, int num_batch_shards, int num_experts, int local_expert_size,
+                              const int32_t* shard_index_dev, int num_rows, const int32_t* global_sorted_experts, int truncate,
+                              int32_t* expert_keys, int32_t* local_group_size, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!shard_index_dev) return fail(MOE_ERR_INVALID_ARG, "local_expert_keys_dev: NULL shard index");
+  return local_expert_keys_impl(global_group_sizes, num_batch_shards, num_experts, local_expert_size, 0, shard_index_dev, num_rows,
+                                global_sorted_experts, truncate, expert_keys, local_group_size, workspace, workspace_bytes, stream);
+}
+
+static int all_to_all_params_impl(const int32_t* all_shards_group_sizes, int num_expert_parallelism, int shard_id, const int32_t* shard_dev,
+                                  int is_batch_sharded, long long buffer_size, int is_dispatch, int32_t* input_offsets, int32_t* send_sizes,
+                                  int32_t* output_offsets, int32_t* recv_sizes, void* stream) {
   if (!all_shards_group_sizes || !input_offsets || !send_sizes || !output_offsets || !recv_sizes)
     return fail(MOE_ERR_INVALID_ARG, "all_to_all_params: NULL pointer");
   if (num_expert_parallelism <= 0 || shard_id < 0 || shard_id >= num_expert_parallelism)
@@ -246,14 +271,29 @@ int moe_all_to_all_params(const int32_t* all_shards_group_sizes, int num_expert_
   if (num_expert_parallelism > kDispMaxParallelism) return fail(MOE_ERR_UNSUPPORTED, "all_to_all_params: more than %d shards", kDispMaxParallelism);
   if (!is_batch_sharded && buffer_size >= 0)
     return fail(MOE_ERR_UNSUPPORTED, "all_to_all_params: a receive capacity needs the batch-sharded traffic matrix");
-  all_to_all_params_kernel<<<1, kDispThreads, 0, (hipStream_t)stream>>>(all_shards_group_sizes, num_expert_parallelism, shard_id, is_batch_sharded,
+  all_to_all_params_kernel<<<1, kDispThreads, 0, (hipStream_t)stream>>>(all_shards_group_sizes, num_expert_parallelism, shard_id, shard_dev, is_batch_sharded,
                                                                         buffer_size, is_dispatch, input_offsets, send_sizes, output_offsets, recv_sizes);
   return check_launch("all_to_all_params");
 }
 
-int moe_ring_ragged_indices(const int32_t* indices, const int32_t* group_sizes, int num_experts, int experts_start,
-                            int local_experts, int num_rows, int buffer_size, int unsort, int32_t* indices_out,
-                            uint8_t* valid_rows_mask, int32_t* row_range, void* stream) {
+int moe_all_to_all_params(const int32_t* all_shards_group_sizes, int num_expert_parallelism, int shard_id, int is_batch_sharded,
+                          long long buffer_size, int is_dispatch, int32_t* input_offsets, int32_t* send_sizes,
+                          int32_t* output_offsets, int32_t* recv_sizes, void* stream) {
+  return all_to_all_params_impl(all_shards_group_sizes, num_expert_parallelism, shard_id, nullptr, is_batch_sharded, buffer_size, is_dispatch,
+                                input_offsets, send_sizes, output_offsets, recv_sizes, stream);
+}
+
+int moe_all_to_all_params_dev(const int32_t* all_shards_group_sizes, int num_expert_parallelism, const int32_t* shard_id_dev, int is_batch_sharded,
+                              long long buffer_size, int is_dispatch, int32_t* input_offsets, int32_t* send_sizes,
+                              int32_t* output_offsets, int32_t* recv_sizes, void* stream) {
+  if (!shard_id_dev) return fail(MOE_ERR_INVALID_ARG, "all_to_all_params_dev: NULL shard id");
+  return all_to_all_params_impl(all_shards_group_sizes, num_expert_parallelism, 0, shard_id_dev, is_batch_sharded, buffer_size, is_dispatch,
+                                input_offsets, send_sizes, output_offsets, recv_sizes, stream);
+}
+
+static int ring_ragged_indices_impl(const int32_t* indices, const int32_t* group_sizes, int num_experts, int experts_start, const int32_t* shard_dev,
+                                    int local_experts, int num_rows, int buffer_size, int unsort, int32_t* indices_out,
+                                    uint8_t* valid_rows_mask, int32_t* row_range, void* stream) {
   if (!indices || !group_sizes || !indices_out) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: NULL pointer");
   if (unsort ? !valid_rows_mask : !row_range) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: NULL output");
   if (num_experts <= 0 || experts_start < 0 || local_experts <= 0 || experts_start + local_experts > num_experts || num_rows < 0)
@@ -261,9 +301,26 @@ int moe_ring_ragged_indices(const int32_t* indices, const int32_t* group_sizes, 
   if (buffer_size < 0) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices: buffer_size %d", buffer_size);
   const int out_n = unsort ? num_rows : (buffer_size < num_rows ? buffer_size : num_rows);
   const int blocks = out_n > 0 ? cdiv(out_n, 256) : 1;
-  ring_ragged_indices_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(indices, group_sizes, num_experts, experts_start, local_experts, num_rows,
+  ring_ragged_indices_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>(indices, group_sizes, num_experts, experts_start, shard_dev, local_experts, num_rows,
                                                                         buffer_size, unsort, indices_out, valid_rows_mask, row_range);
   return check_launch("ring_ragged_indices");
+}
+
+int moe_ring_ragged_indices(const int32_t* indices, const int32_t* group_sizes, int num_experts, int experts_start,
+                            int local_experts, int num_rows, int buffer_size, int unsort, int32_t* indices_out,
+                            uint8_t* valid_rows_mask, int32_t* row_range, void* stream) {
+  return ring_ragged_indices_impl(indices, group_sizes, num_experts, experts_start, nullptr, local_experts, num_rows, buffer_size, unsort,
+                                  indices_out, valid_rows_mask, row_range, stream);
+}
+
+int moe_ring_ragged_indices_dev(const int32_t* indices, const int32_t* group_sizes, int num_experts, const int32_t* shard_index_dev,
+                                int local_experts, int num_rows, int buffer_size, int unsort, int32_t* indices_out,
+                                uint8_t* valid_rows_mask, int32_t* row_range, void* stream) {
+  if (!shard_index_dev) return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices_dev: NULL shard index");
+  if (local_experts <= 0 || num_experts % local_experts != 0)
+    return fail(MOE_ERR_INVALID_ARG, "ring_ragged_indices_dev: %d experts do not divide into shards of %d", num_experts, local_experts);
+  return ring_ragged_indices_impl(indices, group_sizes, num_experts, 0, shard_index_dev, local_experts, num_rows, buffer_size, unsort,
+                                  indices_out, valid_rows_mask, row_range, stream);
 }
 
 }  // extern "C"

@@ -184,9 +184,19 @@ def gather_rows(x, row_idx=None, idx_div=1, *, out_dtype=torch.bfloat16, block_k
   return out, (static_scale if static_scale is not None else scale)
 
 
+def _shard_on_device(shard, name, device):
+  """A shard index given as a tensor stays on the device (int32, one element): the `_dev` entry points read it there."""
+  if not isinstance(shard, torch.Tensor):
+    return None
+  if shard.numel() != 1:
+    raise ValueError(f"{name} must hold one value")
+  return shard.to(device=device, dtype=torch.int32).reshape(1).contiguous()
+
+
 def local_expert_keys(global_group_sizes, local_expert_size, shard_index, num_rows, *, global_sorted_experts=None, truncate=False):
   """Index half of RoutedMoE.local_permute (moe.py:1091-1200) before its argsort.
-  global_group_sizes [batch shards, E] int32 -> (expert_keys [num_rows] int32, local_group_size [local_expert_size] int32)."""
+  global_group_sizes [batch shards, E] int32 -> (expert_keys [num_rows] int32, local_group_size [local_expert_size] int32).
+  shard_index: an int, or a one-element tensor (jax.lax.axis_index of the reference) that is read on the device."""
   _need(global_group_sizes, "global_group_sizes", torch.int32, 2)
   s, e = global_group_sizes.shape
   if global_sorted_experts is not None:
@@ -198,9 +208,15 @@ def local_expert_keys(global_group_sizes, local_expert_size, shard_index, num_ro
   keys = torch.empty((num_rows,), dtype=torch.int32, device=dev)
   sizes = torch.empty((local_expert_size,), dtype=torch.int32, device=dev)
   ws = torch.empty((max(lib.moe_local_expert_keys_workspace_bytes(s, local_expert_size), 16),), dtype=torch.uint8, device=dev)
-  st = lib.moe_local_expert_keys(_lib.ptr(global_group_sizes), s, e, int(local_expert_size), int(shard_index), int(num_rows),
-                                 _lib.ptr(global_sorted_experts), int(bool(truncate)), _lib.ptr(keys), _lib.ptr(sizes), _lib.ptr(ws),
-                                 ws.numel(), _lib.current_stream())
+  shard_dev = _shard_on_device(shard_index, "shard_index", dev)
+  if shard_dev is not None:
+    st = lib.moe_local_expert_keys_dev(_lib.ptr(global_group_sizes), s, e, int(local_expert_size), _lib.ptr(shard_dev), int(num_rows),
+                                       _lib.ptr(global_sorted_experts), int(bool(truncate)), _lib.ptr(keys), _lib.ptr(sizes), _lib.ptr(ws),
+                                       ws.numel(), _lib.current_stream())
+  else:
+    st = lib.moe_local_expert_keys(_lib.ptr(global_group_sizes), s, e, int(local_expert_size), int(shard_index), int(num_rows),
+                                   _lib.ptr(global_sorted_experts), int(bool(truncate)), _lib.ptr(keys), _lib.ptr(sizes), _lib.ptr(ws),
+                                   ws.numel(), _lib.current_stream())
   _lib.check(st, "moe_local_expert_keys")
   return keys, sizes
 
@@ -214,17 +230,23 @@ def all_to_all_params(all_shards_group_sizes, shard_id, num_expert_parallelism, 
   if tuple(all_shards_group_sizes.shape) != ((p, p) if is_batch_sharded else (p,)):
     raise ValueError(f"all_shards_group_sizes has shape {tuple(all_shards_group_sizes.shape)} for {p} shards")
   out = torch.empty((4, p), dtype=torch.int32, device=all_shards_group_sizes.device)
-  st = _lib.load().moe_all_to_all_params(_lib.ptr(all_shards_group_sizes), p, int(shard_id), int(bool(is_batch_sharded)),
-                                         -1 if buffer_size is None else int(buffer_size), int(bool(is_dispatch)), _lib.ptr(out[0]),
-                                         _lib.ptr(out[1]), _lib.ptr(out[2]), _lib.ptr(out[3]), _lib.current_stream())
+  shard_dev = _shard_on_device(shard_id, "shard_id", all_shards_group_sizes.device)
+  tail = (int(bool(is_batch_sharded)), -1 if buffer_size is None else int(buffer_size), int(bool(is_dispatch)), _lib.ptr(out[0]),
+          _lib.ptr(out[1]), _lib.ptr(out[2]), _lib.ptr(out[3]), _lib.current_stream())
+  if shard_dev is not None:
+    st = _lib.load().moe_all_to_all_params_dev(_lib.ptr(all_shards_group_sizes), p, _lib.ptr(shard_dev), *tail)
+  else:
+    st = _lib.load().moe_all_to_all_params(_lib.ptr(all_shards_group_sizes), p, int(shard_id), *tail)
   _lib.check(st, "moe_all_to_all_params")
   return out[0], out[1], out[2], out[3]
 
 
-def ring_ragged_indices(indices, group_sizes, experts_start, local_experts, *, buffer_size=None, unsort=False):
+def ring_ragged_indices(indices, group_sizes, experts_start, local_experts, *, buffer_size=None, unsort=False, shard_index=None):
   """Index arrays of ring_ragged_sort / ring_ragged_unsort (kernels/ragged/ragged_sort.py:102-151, :300-350).
   unsort=False: indices = perm -> (row_idx [min(buffer, n)], row_range [2]); unsort=True: indices = inv_perm ->
-  (inv_perm into the shard's buffer [n], valid_rows_mask [n] uint8)."""
+  (inv_perm into the shard's buffer [n], valid_rows_mask [n] uint8).
+  shard_index: a one-element tensor read on the device; the shard then owns experts [shard * local_experts, + local_experts)
+  and experts_start is ignored."""
   _need(indices, "indices", torch.int32, 1)
   _need(group_sizes, "group_sizes", torch.int32, 1)
   n = indices.shape[0]
@@ -233,8 +255,12 @@ def ring_ragged_indices(indices, group_sizes, experts_start, local_experts, *, b
   out = torch.empty((n if unsort else min(buf, n),), dtype=torch.int32, device=dev)
   mask = torch.empty((n,), dtype=torch.uint8, device=dev) if unsort else None
   rng = None if unsort else torch.empty((2,), dtype=torch.int32, device=dev)
-  st = _lib.load().moe_ring_ragged_indices(_lib.ptr(indices), _lib.ptr(group_sizes), group_sizes.shape[0], int(experts_start), int(local_experts),
-                                           n, buf, int(bool(unsort)), _lib.ptr(out), _lib.ptr(mask), _lib.ptr(rng), _lib.current_stream())
+  shard_dev = _shard_on_device(shard_index, "shard_index", dev)
+  tail = (int(local_experts), n, buf, int(bool(unsort)), _lib.ptr(out), _lib.ptr(mask), _lib.ptr(rng), _lib.current_stream())
+  if shard_dev is not None:
+    st = _lib.load().moe_ring_ragged_indices_dev(_lib.ptr(indices), _lib.ptr(group_sizes), group_sizes.shape[0], _lib.ptr(shard_dev), *tail)
+  else:
+    st = _lib.load().moe_ring_ragged_indices(_lib.ptr(indices), _lib.ptr(group_sizes), group_sizes.shape[0], int(experts_start), *tail)
   _lib.check(st, "moe_ring_ragged_indices")
   return (out, mask) if unsort else (out, rng)
 

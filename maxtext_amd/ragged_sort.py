@@ -1,7 +1,7 @@
 """Host-side mirror of src/maxtext/kernels/ragged/ragged_sort.py: the sorts of the expert-parallel strategies that move
 only the rows a shard owns, with the custom VJPs of the reference (:155-224, :364-441, :515-537, :596-616).  Each pass,
 forward or backward, is one index kernel plus one row-moving kernel of the library; no size is read back by the host.
-`shard_idx` replaces jax.lax.axis_index(ep_name): a plain integer here."""
+`shard_idx` replaces jax.lax.axis_index(ep_name): an integer, or a one-element tensor that only the kernels read."""
 
 from __future__ import annotations
 
@@ -18,6 +18,12 @@ def _row_range(valid_end, device):
   return torch.stack([torch.zeros((), dtype=torch.int32, device=device), end])
 
 
+def _ring_indices(indices, group_sizes, shard_idx, local_experts, **kw):
+  if isinstance(shard_idx, torch.Tensor):
+    return kernels.ring_ragged_indices(indices, group_sizes, 0, local_experts, shard_index=shard_idx, **kw)
+  return kernels.ring_ragged_indices(indices, group_sizes, int(shard_idx) * local_experts, local_experts, **kw)
+
+
 def _inverse_permutation(p):
   """argsort of a permutation, on the device."""
   inv = torch.empty_like(p)
@@ -31,16 +37,16 @@ class _RingSortFn(torch.autograd.Function):
   masked; indices shifted into the packed buffer when it is smaller than T * k)."""
 
   @staticmethod
-  def forward(ctx, hidden, row_idx, row_range, inv, group_sizes, topk, start_expert, local_experts, buffer_rows):
+  def forward(ctx, hidden, row_idx, row_range, inv, group_sizes, topk, shard_idx, local_experts, buffer_rows):
     ctx.save_for_backward(inv, group_sizes)
-    ctx.meta = (topk, start_expert, local_experts, buffer_rows, hidden.shape[0])
+    ctx.meta = (topk, shard_idx, local_experts, buffer_rows, hidden.shape[0])
     return kernels.gather_rows(hidden.contiguous(), row_idx, topk, row_range=row_range)
 
   @staticmethod
   def backward(ctx, g_x):
     inv, group_sizes = ctx.saved_tensors
-    topk, start_expert, local_experts, buffer_rows, tokens = ctx.meta
-    idx, mask = kernels.ring_ragged_indices(inv, group_sizes, start_expert, local_experts, buffer_size=buffer_rows, unsort=True)
+    topk, shard_idx, local_experts, buffer_rows, tokens = ctx.meta
+    idx, mask = _ring_indices(inv, group_sizes, shard_idx, local_experts, buffer_size=buffer_rows, unsort=True)
     g = kernels.unpermute_combine(g_x.contiguous(), None, k=topk, inv_perm=idx, valid_rows_mask=mask, num_tokens=tokens)
     return g, None, None, None, None, None, None, None, None
 
@@ -54,9 +60,9 @@ def ring_ragged_sort(hidden_states_local, topk_indices_local, num_experts, topk,
     raise ValueError(f"topk_indices_local has {k} columns for topk={topk}")
   perm, inv, group_sizes, _ = kernels.sort_by_expert(topk_indices_local.contiguous(), num_experts, want_sorted_experts=False)
   local = num_experts // ep_size
-  row_idx, row_range = kernels.ring_ragged_indices(perm, group_sizes, shard_idx * local, local, buffer_size=buffer_size)
+  row_idx, row_range = _ring_indices(perm, group_sizes, shard_idx, local, buffer_size=buffer_size)
   if torch.is_grad_enabled() and hidden_states_local.requires_grad:
-    x = _RingSortFn.apply(hidden_states_local, row_idx, row_range, inv, group_sizes, topk, shard_idx * local, local, row_idx.shape[0])
+    x = _RingSortFn.apply(hidden_states_local, row_idx, row_range, inv, group_sizes, topk, shard_idx, local, row_idx.shape[0])
   else:
     x = kernels.gather_rows(hidden_states_local.contiguous(), row_idx, topk, row_range=row_range)
   return x, group_sizes, inv
@@ -69,17 +75,17 @@ class _RingUnsortFn(torch.autograd.Function):
   here, as in the reference (:441)."""
 
   @staticmethod
-  def forward(ctx, sorted_tokens, idx, mask, w, revert, group_sizes, topk, start_expert, local_experts):
+  def forward(ctx, sorted_tokens, idx, mask, w, revert, group_sizes, topk, shard_idx, local_experts):
     ctx.save_for_backward(w, revert, group_sizes)
-    ctx.meta = (topk, start_expert, local_experts, sorted_tokens.shape[0])
+    ctx.meta = (topk, shard_idx, local_experts, sorted_tokens.shape[0])
     return kernels.unpermute_combine(sorted_tokens.contiguous(), w, k=topk, inv_perm=idx, valid_rows_mask=mask, num_tokens=revert.shape[0] // topk)
 
   @staticmethod
   def backward(ctx, g_out):
     w, revert, group_sizes = ctx.saved_tensors
-    topk, start_expert, local_experts, buffer_rows = ctx.meta
+    topk, shard_idx, local_experts, buffer_rows = ctx.meta
     perm = _inverse_permutation(revert)  # sorted position -> flat slot t * topk + s
-    row_idx, row_range = kernels.ring_ragged_indices(perm, group_sizes, start_expert, local_experts, buffer_size=buffer_rows)
+    row_idx, row_range = _ring_indices(perm, group_sizes, shard_idx, local_experts, buffer_size=buffer_rows)
     w_rows = w[row_idx.long().clamp_(0, w.numel() - 1)].contiguous()  # the slot's weight, row by row of the (packed) buffer
     g = kernels.gather_rows(g_out.contiguous(), row_idx, topk, row_weight=w_rows, row_range=row_range)
     return g, None, None, None, None, None, None, None, None
@@ -91,11 +97,10 @@ def ring_ragged_unsort(sorted_tokens_local, group_sizes_local, topk_argsort_reve
   n = topk_argsort_revert_indices.shape[0]
   revert = topk_argsort_revert_indices.contiguous()
   gs = group_sizes_local.contiguous()
-  idx, mask = kernels.ring_ragged_indices(revert, gs, shard_idx * local_num_experts, local_num_experts,
-                                          buffer_size=sorted_tokens_local.shape[0], unsort=True)
+  idx, mask = _ring_indices(revert, gs, shard_idx, local_num_experts, buffer_size=sorted_tokens_local.shape[0], unsort=True)
   w = topk_weights.reshape(-1).float().contiguous()
   if torch.is_grad_enabled() and sorted_tokens_local.requires_grad:
-    return _RingUnsortFn.apply(sorted_tokens_local, idx, mask, w.detach(), revert, gs, topk, shard_idx * local_num_experts, local_num_experts)
+    return _RingUnsortFn.apply(sorted_tokens_local, idx, mask, w.detach(), revert, gs, topk, shard_idx, local_num_experts)
   return kernels.unpermute_combine(sorted_tokens_local.contiguous(), w, k=topk, inv_perm=idx, valid_rows_mask=mask, num_tokens=n // topk)
 
 

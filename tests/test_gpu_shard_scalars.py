@@ -105,3 +105,56 @@ def test_dynamic_per_tensor_scales(K, qname):
   want = O.gmm(want_l.float(), want_r.float(), sizes, lhs_scale=ls.reshape(1, 1), rhs_scale=rs.reshape(1, 1).expand(1, n))
   assert relerr(out, want) <= TOL
   assert float(K.tensor_scale(torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda"), qmax)) == 0.0
+
+
+def test_dispatch_bookkeeping_with_the_shard_index_on_the_device(K):
+  """moe_local_expert_keys / moe_all_to_all_params / moe_ring_ragged_indices with the shard's index in a device buffer
+  (jax.lax.axis_index of moe.py:1134, :1709-1712): bit-equal to the by-value calls for every shard, and a value past the
+  last shard is clamped to it."""
+  rng = np.random.default_rng(5)
+  shards, experts, local = 4, 16, 4
+  ggs = rng.integers(0, 40, size=(shards, experts)).astype(np.int32)
+  rows = int(ggs.sum()) + 7
+  sorted_experts = np.sort(rng.integers(0, experts, size=rows)).astype(np.int32)
+  traffic = rng.integers(0, 50, size=(shards, shards)).astype(np.int32)
+  topk_idx = rng.integers(0, experts, size=(96, 2)).astype(np.int32)
+  perm, inv, gs, _ = K.sort_by_expert(cuda(topk_idx), experts, want_sorted_experts=False)
+  for shard in range(shards + 1):
+    ref = min(shard, shards - 1)
+    dev = torch.tensor([shard], dtype=torch.int32, device="cuda")
+    for offset_mode in (False, True):
+      kw = dict(global_sorted_experts=cuda(sorted_experts) if offset_mode else None, truncate=not offset_mode)
+      a = K.local_expert_keys(cuda(ggs), local, ref, rows, **kw)
+      b = K.local_expert_keys(cuda(ggs), local, dev, rows, **kw)
+      assert all(torch.equal(x, y) for x, y in zip(a, b))
+    for dispatch in (True, False):
+      a = K.all_to_all_params(cuda(traffic), ref, shards, buffer_size=60, is_dispatch=dispatch)
+      b = K.all_to_all_params(cuda(traffic), dev, shards, buffer_size=60, is_dispatch=dispatch)
+      assert all(torch.equal(x, y) for x, y in zip(a, b))
+    a = K.all_to_all_params(cuda(traffic[0]), ref, shards, is_batch_sharded=False)
+    b = K.all_to_all_params(cuda(traffic[0]), dev, shards, is_batch_sharded=False)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    for unsort, idx, buf in ((False, perm, None), (False, perm, 40), (True, inv, None), (True, inv, 40)):
+      a = K.ring_ragged_indices(idx, gs, ref * local, local, buffer_size=buf, unsort=unsort)
+      b = K.ring_ragged_indices(idx, gs, 0, local, buffer_size=buf, unsort=unsort, shard_index=dev)
+      assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
+def test_ring_ragged_sort_with_a_device_shard_index():
+  """ring_ragged_sort / _unsort with the shard index as a tensor: same rows, sizes and gradient as with the integer."""
+  from maxtext_amd import ragged_sort
+
+  g = torch.Generator().manual_seed(11)
+  t, d, e, k, ep = 64, 128, 8, 2, 4
+  x = torch.randn(t, d, generator=g).to(torch.bfloat16).cuda()
+  idx = torch.randint(0, e, (t, k), generator=g, dtype=torch.int32).cuda()
+  w = torch.rand(t, k, generator=g).cuda()
+  for shard in range(ep):
+    outs = []
+    for s in (shard, torch.tensor(shard, device="cuda")):
+      xi = x.clone().requires_grad_(True)
+      rows, gs, inv = ragged_sort.ring_ragged_sort(xi, idx, e, k, s, ep)
+      y = ragged_sort.ring_ragged_unsort(rows * 2, gs, inv, k, e // ep, s, w)
+      y.float().square().sum().backward()
+      outs.append((rows.detach(), gs, inv, y.detach(), xi.grad))
+    assert all(torch.equal(a, b) for a, b in zip(*outs))
