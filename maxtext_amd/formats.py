@@ -105,3 +105,95 @@ def aqt_int8_experts(qvalue: torch.Tensor, scale: torch.Tensor) -> QArray:
   if scale.numel() != e * n:
     raise ValueError(f"scale must have E*N = {e * n} elements, got {tuple(scale.shape)}")
   return QArray(qvalue.transpose(1, 2).contiguous(), scale.reshape(e, n).float().contiguous(), "int8")
+
+
+# ---- readers of checkpoint directories ------------------------------------------------------------------------------
+
+
+class SafetensorsDir(Mapping):
+  """The tensors of a Hugging Face checkpoint directory by name, read one at a time as they are asked for (`safe_open`:
+  a memory-mapped read of the tensor's bytes, nothing is unpickled and no shard is loaded whole).  The name -> file map is
+  `model.safetensors.index.json` when the directory has one (deepseek_dequantize.py:121-140, dequantize_mxfp4.py:84-100)
+  and the key lists of every `*.safetensors` file otherwise (convert_deepseek_family_ckpt.py:315-331,
+  convert_gpt_oss_ckpt.py:79-90).  `key_prefix` is stripped from the names (the text branch of a multimodal checkpoint,
+  convert_deepseek_family_ckpt.py:320-327)."""
+
+  INDEX = "model.safetensors.index.json"
+
+  def __init__(self, path, key_prefix: str = "", device="cpu"):
+    import glob
+    import json
+    import os
+
+    self.path, self.device, self._prefix = path, str(device), key_prefix
+    index = os.path.join(path, self.INDEX)
+    if os.path.exists(index):
+      with open(index, "r", encoding="utf8") as f:
+        raw = json.load(f)["weight_map"]
+    else:
+      from safetensors import safe_open
+
+      raw = {}
+      for file in sorted(glob.glob(os.path.join(path, "[!.]*.safetensors"))):
+        with safe_open(file, framework="pt", device="cpu") as f:
+          for key in f.keys():
+            raw[key] = os.path.basename(file)
+      if not raw:
+        raise FileNotFoundError(f"no {self.INDEX} and no *.safetensors file in {path}")
+    self._files = {k[len(key_prefix):]: (k, v) for k, v in raw.items() if k.startswith(key_prefix)}
+
+  def __getitem__(self, name):
+    import os
+
+    from safetensors import safe_open
+
+    raw, file = self._files[name]
+    with safe_open(os.path.join(self.path, file), framework="pt", device=self.device) as f:
+      return f.get_tensor(raw)
+
+  def __iter__(self):
+    return iter(self._files)
+
+  def __len__(self):
+    return len(self._files)
+
+
+def read_deepseek_fp8_layer(path, layer: int, num_experts: int, prefix: str = "model.layers", key_prefix: str = "", device="cpu"):
+  """(wi_0, wi_1, wo) of one MoE layer straight from a DeepSeek fp8 checkpoint directory.  The block scales are looked up
+  under both names the reference's reader tries: `<name>.weight_scale_inv` (V3) and `<name>.scale` (V4),
+  deepseek_dequantize.py:155-175."""
+  state = path if isinstance(path, Mapping) else SafetensorsDir(path, key_prefix, device)
+  out = []
+  for proj in ("gate_proj", "up_proj", "down_proj"):
+    ws, ss = [], []
+    for e in range(num_experts):
+      name = f"{prefix}.{layer}.mlp.experts.{e}.{proj}"
+      ws.append(state[name + ".weight"])
+      ss.append(state[name + ".weight_scale_inv"] if name + ".weight_scale_inv" in state else state[name + ".scale"])
+    out.append(deepseek_fp8_experts(ws, ss))
+  return tuple(out)
+
+
+def read_compressed_int4_layer(path, layer: int, num_experts: int, group_size: int = 32, prefix: str = "model.layers",
+                               key_prefix: str = "", device="cpu"):
+  """(wi_0, wi_1, wo) of one MoE layer from a compressed-tensors int4 checkpoint directory (Kimi-K2 family):
+  `<name>.weight_packed`, `.weight_scale`, `.weight_shape` per expert and projection, the three tensors
+  convert_deepseek_family_ckpt.py:343-361 hands to its dequantiser."""
+  state = path if isinstance(path, Mapping) else SafetensorsDir(path, key_prefix, device)
+  out = []
+  for proj in ("gate_proj", "up_proj", "down_proj"):
+    names = [f"{prefix}.{layer}.mlp.experts.{e}.{proj}" for e in range(num_experts)]
+    out.append(compressed_int4_experts([state[n + ".weight_packed"] for n in names], [state[n + ".weight_scale"] for n in names],
+                                       [state[n + ".weight_shape"].tolist() for n in names], group_size))
+  return tuple(out)
+
+
+def read_gpt_oss_mxfp4_layer(path, layer: int, experts: str = "model.layers.{layer}.mlp.experts", key_prefix: str = "", device="cpu"):
+  """(wi_0, wi_1, wo, biases) of one GPT-OSS layer from its checkpoint directory: `gate_up_proj_blocks` / `_scales` /
+  `_bias` and `down_proj_blocks` / `_scales` / `_bias` under `experts` (the `_blocks` / `_scales` pairs of
+  dequantize_mxfp4.py:92-131)."""
+  state = path if isinstance(path, Mapping) else SafetensorsDir(path, key_prefix, device)
+  base = experts.format(layer=layer)
+  get = lambda n: state[f"{base}.{n}"] if f"{base}.{n}" in state else None  # noqa: E731
+  return gpt_oss_mxfp4_layer(state[f"{base}.gate_up_proj_blocks"], state[f"{base}.gate_up_proj_scales"], state[f"{base}.down_proj_blocks"],
+                             state[f"{base}.down_proj_scales"], get("gate_up_proj_bias"), get("down_proj_bias"))

@@ -93,3 +93,97 @@ def test_aqt_int8_relayout():
     want = (x @ q[ex].float()) * s[ex, 0]
     got = (x @ qa.qvalue[ex].float().T) * qa.scale[ex]
     assert torch.allclose(got, want)
+
+
+def _write_shards(tmp_path, tensors, shards, with_index):
+  """Splits `tensors` over `shards` safetensors files the way a Hugging Face checkpoint directory does."""
+  import json
+
+  from safetensors.torch import save_file
+
+  names = sorted(tensors)
+  weight_map = {}
+  for i in range(shards):
+    part = {n: tensors[n].contiguous() for n in names[i::shards]}
+    file = f"model-{i + 1:05d}-of-{shards:05d}.safetensors"
+    save_file(part, str(tmp_path / file))
+    weight_map.update({n: file for n in part})
+  if with_index:
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}))
+
+
+@pytest.mark.parametrize("with_index", [True, False])
+@pytest.mark.parametrize("v4_names", [False, True])
+def test_read_deepseek_fp8_layer_from_a_checkpoint_directory(tmp_path, with_index, v4_names):
+  """A sharded fp8 checkpoint directory (index file or bare shards; `weight_scale_inv` or the V4 `scale` name,
+  deepseek_dequantize.py:155-175) read tensor by tensor gives the operands the in-memory adapter gives, and they
+  dequantise to what deepseek_dequantize.py:42-68 computes."""
+  g = torch.Generator().manual_seed(3)
+  n, k, e, layer = 256, 128, 4, 5
+  tensors, per_proj = {"model.embed_tokens.weight": torch.zeros(8, 4, dtype=torch.bfloat16)}, {}
+  for proj in ("gate_proj", "up_proj", "down_proj"):
+    for i in range(e):
+      w = torch.randn(n, k, generator=g).to(torch.float8_e4m3fn)
+      s = torch.rand(n // 128, k // 128, generator=g) * 0.01 + 1e-3
+      base = f"model.layers.{layer}.mlp.experts.{i}.{proj}"
+      tensors[base + ".weight"] = w
+      tensors[base + (".scale" if v4_names else ".weight_scale_inv")] = s
+      per_proj.setdefault(proj, []).append((w, s))
+  _write_shards(tmp_path, tensors, 3, with_index)
+  got = formats.read_deepseek_fp8_layer(str(tmp_path), layer, e)
+  for qa, proj in zip(got, ("gate_proj", "up_proj", "down_proj")):
+    want = formats.deepseek_fp8_experts([w for w, _ in per_proj[proj]], [s for _, s in per_proj[proj]])
+    assert torch.equal(qa.qvalue.view(torch.uint8), want.qvalue.view(torch.uint8)) and torch.equal(qa.scale, want.scale)
+    w, s = per_proj[proj][2]
+    dense = (w.float().reshape(n // 128, 128, k // 128, 128) * s.reshape(n // 128, 1, k // 128, 1)).reshape(n, k).to(torch.bfloat16)
+    assert torch.equal(O.dequantize_fp8_blocks(qa.qvalue[2], qa.scale[2], 128), dense)
+  d = formats.SafetensorsDir(str(tmp_path))
+  assert len(d) == len(tensors) and "model.embed_tokens.weight" in d and "nope" not in d
+  with pytest.raises(KeyError):
+    formats.read_deepseek_fp8_layer(str(tmp_path), layer + 1, e)
+
+
+def test_read_compressed_int4_and_gpt_oss_layers_from_checkpoint_directories(tmp_path):
+  """compressed-tensors int4 (weight_packed / weight_scale / weight_shape, convert_deepseek_family_ckpt.py:343-361, under a
+  multimodal key prefix) and GPT-OSS blocks / scales / biases (dequantize_mxfp4.py:92-131) read from files equal the
+  in-memory adapters on the same tensors."""
+  rng = np.random.default_rng(1)
+  n, k, e, layer = 8, 64, 2, 3
+  i4, packed, scales = {}, {}, {}
+  for proj in ("gate_proj", "up_proj", "down_proj"):
+    for i in range(e):
+      base = f"language_model.model.layers.{layer}.mlp.experts.{i}.{proj}"
+      p = torch.from_numpy(rng.integers(-2**31, 2**31, (n, k // 8), dtype=np.int64).astype(np.int32))
+      s = torch.tensor(rng.random((n, k // 32)) + 0.5, dtype=torch.bfloat16)
+      i4[base + ".weight_packed"], i4[base + ".weight_scale"] = p, s
+      i4[base + ".weight_shape"] = torch.tensor([n, k], dtype=torch.int32)
+      packed.setdefault(proj, []).append(p)
+      scales.setdefault(proj, []).append(s)
+  i4["vision_tower.patch_embed.weight"] = torch.zeros(2, 2)
+  d4 = tmp_path / "int4"
+  d4.mkdir()
+  _write_shards(d4, i4, 2, with_index=False)
+  got = formats.read_compressed_int4_layer(str(d4), layer, e, group_size=32, key_prefix="language_model.")
+  for qa, proj in zip(got, ("gate_proj", "up_proj", "down_proj")):
+    want = formats.compressed_int4_experts(packed[proj], scales[proj], [(n, k)] * e, 32)
+    assert qa.qtype == "int4g32" and torch.equal(qa.qvalue, want.qvalue) and torch.equal(qa.scale, want.scale)
+
+  ne, f2, d = 3, 16, 64
+  oss = {
+      f"model.layers.{layer}.mlp.experts.gate_up_proj_blocks": torch.from_numpy(rng.integers(0, 256, (ne, 2 * f2, d // 32, 16), dtype=np.uint8)),
+      f"model.layers.{layer}.mlp.experts.gate_up_proj_scales": torch.from_numpy(rng.integers(120, 130, (ne, 2 * f2, d // 32), dtype=np.uint8)),
+      f"model.layers.{layer}.mlp.experts.gate_up_proj_bias": torch.randn(ne, 2 * f2).to(torch.bfloat16),
+      f"model.layers.{layer}.mlp.experts.down_proj_blocks": torch.from_numpy(rng.integers(0, 256, (ne, d, f2 * 2 // 32, 16), dtype=np.uint8)),
+      f"model.layers.{layer}.mlp.experts.down_proj_scales": torch.from_numpy(rng.integers(120, 130, (ne, d, f2 * 2 // 32), dtype=np.uint8)),
+      f"model.layers.{layer}.mlp.experts.down_proj_bias": torch.randn(ne, d).to(torch.bfloat16),
+  }
+  do = tmp_path / "oss"
+  do.mkdir()
+  _write_shards(do, oss, 2, with_index=True)
+  w0, w1, wo, biases = formats.read_gpt_oss_mxfp4_layer(str(do), layer)
+  base = f"model.layers.{layer}.mlp.experts."
+  x0, x1, xo, xb = formats.gpt_oss_mxfp4_layer(oss[base + "gate_up_proj_blocks"], oss[base + "gate_up_proj_scales"], oss[base + "down_proj_blocks"],
+                                               oss[base + "down_proj_scales"], oss[base + "gate_up_proj_bias"], oss[base + "down_proj_bias"])
+  for a, b in ((w0, x0), (w1, x1), (wo, xo)):
+    assert torch.equal(a.qvalue, b.qvalue) and torch.equal(a.scale, b.scale)
+  assert all(torch.equal(a, b) for a, b in zip(biases, xb))
