@@ -468,6 +468,16 @@ MOE_API int moe_tgmm(const void* lhs, const void* dout, const int32_t* group_siz
 MOE_API int moe_tgmm_scaled(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
                     int num_groups_total, int num_groups_local, int group_offset, const float* out_row_scale,
                     const void* existing_out, int existing_dtype, int out_dtype, void* out, void* stream);
+/* moe_tgmm_scaled on 1-byte operands as they are stored: lhs [M, K] float8_e4m3fn (the quantised activations kept from the
+ * forward) and dout [M, N] float8_e5m2 or float8_e4m3fn (dout_dtype; the gradient quantised per column by
+ * moe_bwd_scale_grad with quantize = 2), the drhs product of the fp8_full backward (kernels/megablox/ops.py:590-604) on the
+ * fp8 MFMA with f32 accumulation.  Same output, out_row_scale and existing_out as above.  Runs on 256 x 256 output tiles only:
+ * K % 256 == 0, N % 256 == 0, M >= 128 * num_groups_total, at least 128 tiles (moe_tgmm_fp8_supported says so; other shapes
+ * return MOE_ERR_UNSUPPORTED and take the operands widened to bf16, in which fp8 values are exact, through moe_tgmm_scaled). */
+MOE_API int moe_tgmm_fp8_supported(int M, int K, int N, int num_groups_total, int num_groups_local);
+MOE_API int moe_tgmm_fp8(const void* lhs, const void* dout, int dout_dtype, const int32_t* group_sizes, int M, int K, int N,
+                 int num_groups_total, int num_groups_local, int group_offset, const float* out_row_scale,
+                 const void* existing_out, int existing_dtype, int out_dtype, void* out, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Unpermute + top-k weighted combine.  Replaces RoutedMoE.unpermute

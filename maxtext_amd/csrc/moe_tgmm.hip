@@ -387,13 +387,294 @@ __global__ __launch_bounds__(kTdThreads, 2) void tgmm_dl_kernel(const TgmmParams
   }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// The same 256 x 256 tiles for 1-byte operands: the drhs product of the fp8_full backward (kernels/megablox/ops.py:590-604:
+// float8_e4m3fn activations x float8_e5m2 gradient, the contraction running over the rows of both) on
+// v_mfma_scale_f32_16x16x128_f8f6f4, without widening either operand.  A stage is 128 contraction rows of both operands
+// (128 x 256 bytes each, a wave instruction copies four rows), two buffers of 64 KB.  Fragments come out of the row-major
+// stage through ds_read_b64_tr_b8: 16 lanes address an 8-row x 16-byte block (lane l: row l / 2, half l % 2) and lane l
+// receives column l of the 8 rows; four such reads give a lane the 32 contraction values of its column that one
+// 16 x 16 x 128 fragment holds.  Lane group q takes stage rows 32 q .. 32 q + 31 for BOTH operands, which is all the
+// instruction needs (any order of the contraction index, as long as the two fragments agree).  A fragment is 8
+// registers, so a wave (64 k x 128 n) keeps its 4 lhs fragments and a ring of 4 of its 8 dout fragments beside the 128
+// accumulators and multiplies a stage in two halves of 16 MFMAs: dout fragments 0 .. 3 from the ring (each slot reloaded
+// with fragment + 4 after its four MFMAs), then fragments 4 .. 7, lhs fragment by lhs fragment, with the next stage's
+// fragments read behind them.  The 16-byte chunk c of stage row r sits at slot c ^ (r % 8) ^ 8 * ((r / 32) % 2): the 8 rows
+// of a read and those of the next lane group fall into 16 different 16-byte bank groups.
+// ---------------------------------------------------------------------------------------
+
+constexpr int kT8BM = 128;                            // contraction rows per stage
+constexpr int kT8Row = kTdTile;                       // bytes of one operand row in a stage
+constexpr int kT8Operand = kT8BM * kT8Row;            // 32 KB
+constexpr int kT8Stage = 2 * kT8Operand;              // lhs rows | dout rows
+constexpr int kT8Lds = 2 * kT8Stage;                  // two buffers
+constexpr int kT8Ipw = kT8Operand / 1024 / kTdWaves;  // requests per wave, operand and stage
+constexpr int kT8Lps = 2 * kT8Ipw;
+constexpr int kT8ReqStride = 2;                       // a stage's requests go out behind every second MFMA of a half
+
+__device__ __forceinline__ int t8_swz(int row) { return (row & 7) ^ (((row >> 5) & 1) << 3); }
+
+typedef int v2i_t8 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2i_t8* lds_v2i_t8;
+__device__ __forceinline__ void tr8_read_frag(v8i& f, const uint8_t* p) {
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const v2i_t8 x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_t8)(p + t * 8 * kT8Row));
+    f[2 * t] = x[0];
+    f[2 * t + 1] = x[1];
+  }
+}
+
+template <int DF>  // element format of dout: 0 = e4m3, 1 = e5m2 (lhs is e4m3)
+__global__ __launch_bounds__(kTdThreads, 2) void tgmm_f8_kernel(const TgmmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t t8_smem[];
+  __shared__ int s_red[kTdWaves];
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wk = wave % 4, wn = wave / 4;  // wave tile: 64 k x 128 n
+  const int N = p.N, K = p.K;
+
+  // tile of this block: the order of tgmm_dl_kernel (XCD ranges, patches of 8 n-tiles x 4 k-tiles of one group)
+  const int tiles_k = K / kTdTile, tiles_n = N / kTdTile, per_group = tiles_k * tiles_n;
+  const int total = per_group * p.G_local;
+  const int q8 = total / 8, rem = total % 8, xcd = blockIdx.x % 8, loc = blockIdx.x / 8;
+  const int logical = xcd < rem ? xcd * (q8 + 1) + loc : rem * (q8 + 1) + (xcd - rem) * q8 + loc;
+  const int g_local = logical / per_group, t = logical % per_group, g = g_local + p.group_offset;
+  constexpr int GSM = 8;
+  const int width = GSM * tiles_k, first_n = (t / width) * GSM, gsz = min(tiles_n - first_n, GSM);
+  const int n0 = (first_n + (t % width) % gsz) * kTdTile, k0 = ((t % width) / gsz) * kTdTile;
+
+  long long part = 0;
+  for (int i = tid; i < min(g, p.G_total); i += kTdThreads) part += max(p.group_sizes[i], 0);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o);
+  if (lane == 0) s_red[wave] = (int)min(part, (long long)p.M);
+  __syncthreads();
+  long long start_ll = 0;
+  for (int w = 0; w < kTdWaves; w++) start_ll += s_red[w];
+  const int start = __builtin_amdgcn_readfirstlane((int)min(start_ll, (long long)p.M));
+  const int size = __builtin_amdgcn_readfirstlane(g < p.G_total ? min(max(p.group_sizes[g], 0), p.M - start) : 0);
+
+  const int s16 = lane % 16, gq = lane / 16;
+  if (size == 0) {  // an empty group's gradient is zero
+    for (int i = tid; i < kTdTile * (kTdTile / 4); i += kTdThreads) {
+      const size_t off = ((size_t)g_local * N + n0 + i / (kTdTile / 4)) * K + k0 + (i % (kTdTile / 4)) * 4;
+      tgmm_store4(p, off, n0 + i / (kTdTile / 4), 0.f, 0.f, 0.f, 0.f);
+    }
+    return;
+  }
+
+  // ---- requests: request i of an operand covers stage rows 4 * (4 * wave + i) + {0 .. 3}, lane l the 16 bytes of LDS
+  // slot l % 16 of row l / 16.  Requests i and i + 2 of a wave are 8 rows apart inside one block of 32 rows, which leaves
+  // the swizzle as it is: two per-lane offsets per operand.  Rows past the group's end come from a row of zeros.
+  uint32_t a_off[2], b_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = 4 * (wave * kT8Ipw + i) + lane / 16;
+    const int chunk = (lane % 16) ^ t8_swz(r);
+    a_off[i] = (uint32_t)r * K + chunk * 16;
+    b_off[i] = (uint32_t)r * N + chunk * 16;
+  }
+  static_assert(kT8Ipw == 4, "request i + 2 is request i eight rows further down");
+  const uint8_t* const a_base = (const uint8_t*)p.lhs + ((size_t)start * K + k0);
+  const uint8_t* const b_base = (const uint8_t*)p.dout + ((size_t)start * N + n0);
+  const size_t a_step = (size_t)kT8BM * K, b_step = (size_t)kT8BM * N;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)t8_smem;
+  auto issue_one = [&](auto full_c, int kt, int buf, int idx) {
+    constexpr bool FULL = decltype(full_c)::value;
+    const int i = idx % kT8Ipw;
+    const bool is_a = idx < kT8Ipw;
+    const uint8_t* src = is_a ? a_base + (kt * a_step + (size_t)(i / 2) * 8 * K) + a_off[i % 2]
+                              : b_base + (kt * b_step + (size_t)(i / 2) * 8 * N) + b_off[i % 2];
+    if constexpr (!FULL) {
+      int l = lane;
+      asm volatile("" : "+v"(l));
+      const int r = 4 * (wave * kT8Ipw + i) + l / 16;
+      const uint64_t keep = kt * kT8BM + r < size ? ~0ull : 0ull;
+      const uint64_t zero = (uint64_t)(tg_zero_row + (l % 16) * 16);
+      src = (const uint8_t*)(((uint64_t)src & keep) | (zero & ~keep));
+    }
+    dma16_untracked(src, lds_base + buf * kT8Stage + (is_a ? 0 : kT8Operand) + (wave * kT8Ipw + i) * 1024);
+  };
+
+  // ---- fragments: lane (group gq, s16) addresses row 32 * gq + s16 / 2 (+ 8, 16, 24) of the stage and the 8 bytes
+  // s16 % 2 of the fragment's 16-byte column block c, stored at slot c ^ (s16 / 2) ^ 8 * (gq % 2); fragment f of an operand
+  // is block c0 + f with c0 a multiple of 4 (lhs) or 8 (dout), so the step is an XOR of address bits 4 .. 6.
+  const int xmask = (s16 / 2) ^ ((gq & 1) << 3);
+  const int row_part = (32 * gq + s16 / 2) * kT8Row + (s16 % 2) * 8;
+  const int k_base = row_part + (((4 * wk) ^ xmask) << 4);
+  const int n_base = row_part + (((8 * wn) ^ xmask) << 4);
+  constexpr int RING = 4;
+  v8i fk[4], fn[RING];
+  auto read_k = [&](int buf, int f) {
+    int base = k_base;
+    asm volatile("" : "+v"(base));
+    tr8_read_frag(fk[f], t8_smem + buf * kT8Stage + (base ^ (16 * f)));
+  };
+  auto read_n = [&](int buf, int f, int slot) {
+    int base = n_base;
+    asm volatile("" : "+v"(base));
+    tr8_read_frag(fn[slot], t8_smem + buf * kT8Stage + kT8Operand + (base ^ (16 * f)));
+  };
+
+  v4f acc[4][8];  // [k fragment][n fragment]
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[j][i][r] = 0.f;
+
+  // first half of a stage (buffer buf): dout fragments 0 .. 3 from the ring, each slot reloaded with fragment + 4
+  auto half_lo = [&](int buf) {
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      const int i = t / 4, j = t % 4;
+      acc[j][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fk[j], fn[i], acc[j][i], 0, DF, 0, 127, 0, 127);
+      if (j == 3) read_n(buf, i + RING, i);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // second half: dout fragments 4 .. 7, lhs fragment by lhs fragment.  RD: the next stage (rd_buf) is prepared behind it.
+  // LD: the requests of stage ld_kt go out into ld_buf.
+  auto half_hi = [&](auto rd_c, auto ld_c, auto full_c, int rd_buf, int ld_kt, int ld_buf) {
+    constexpr bool RD = decltype(rd_c)::value, LD = decltype(ld_c)::value;
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      const int j = t / 4, ii = t % 4;
+      acc[j][RING + ii] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fk[j], fn[ii], acc[j][RING + ii], 0, DF, 0, 127, 0, 127);
+      if (LD && t % kT8ReqStride == 0 && t / kT8ReqStride < kT8Lps) issue_one(full_c, ld_kt, ld_buf, t / kT8ReqStride);
+      if (RD && ii == 3) read_k(rd_buf, j);
+      if (RD && j == 3) read_n(rd_buf, ii, ii);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+
+  // Stage kt sits in buffer kt % 2.  After a stage's first half every fragment of it is in registers: the block meets
+  // (own reads returned, own requests of stage kt + 1 landed), and during the second half the fragments of stage kt + 1
+  // are read from the other buffer while stage kt + 2 is requested into this one.
+  const int nk = (size + kT8BM - 1) / kT8BM;
+#pragma unroll
+  for (int s = 0; s < 2; s++)
+#pragma unroll
+    for (int i = 0; i < kT8Lps; i++) issue_one(F_{}, min(s, nk - 1), s, i);
+  wait_vmcnt<0>();
+  __syncthreads();
+#pragma unroll
+  for (int f = 0; f < RING; f++) read_n(0, f, f);
+#pragma unroll
+  for (int f = 0; f < 4; f++) read_k(0, f);
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  half_lo(0);
+  int kt = 0;
+  const int nfull = size / kT8BM;  // stages 0 .. nfull-1 hold 128 rows of the group
+  for (; kt + 2 < nfull; kt++) {   // steady state: the stage requested is a full one
+    const int buf = kt % 2;
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    half_hi(T_{}, T_{}, T_{}, buf ^ 1, kt + 2, buf);
+    half_lo(buf ^ 1);
+  }
+  for (; kt + 1 < nk; kt++) {
+    const int buf = kt % 2;
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    wait_vmcnt<0>();
+    asm volatile("s_barrier" ::: "memory");
+    half_hi(T_{}, T_{}, F_{}, buf ^ 1, min(kt + 2, nk - 1), buf);
+    half_lo(buf ^ 1);
+  }
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  half_hi(F_{}, F_{}, F_{}, 0, 0, 0);
+  wait_vmcnt<0>();  // no request may still be writing LDS when the block ends
+  // (the sums are pinned to this point: their only readers sit behind the branches below)
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int i = 0; i < 8; i++) asm volatile("" : "+v"(acc[j][i]));
+
+  // D[k][n]: the lane holds n = s16 and k = 4 * gq + r of each 16 x 16 tile
+  if (!p.out_f32 && !p.existing) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int n = n0 + wn * 128 + i * 16 + s16;
+      const float sc = p.n_scale ? p.n_scale[n] : 1.0f;
+#pragma unroll
+      for (int j = 0; j < 4; j += 2) {
+        const auto s0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(acc[j][i][0] * sc, acc[j][i][1] * sc),
+                                                         pack_bf16x2(acc[j + 1][i][0] * sc, acc[j + 1][i][1] * sc), false, false);
+        const auto s1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(acc[j][i][2] * sc, acc[j][i][3] * sc),
+                                                         pack_bf16x2(acc[j + 1][i][2] * sc, acc[j + 1][i][3] * sc), false, false);
+        const int k = k0 + wk * 64 + (j + (gq & 1)) * 16 + 4 * (gq & ~1);
+        *(uint4*)((uint16_t*)p.out + ((size_t)g_local * N + n) * K + k) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int n = n0 + wn * 128 + i * 16 + s16;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int k = k0 + wk * 64 + j * 16 + 4 * gq;
+      const size_t off = ((size_t)g_local * N + n) * K + k;
+      tgmm_store4(p, off, n, acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]);
+    }
+  }
+}
+
 }  // namespace moe
 
 using namespace moe;
 
 namespace moe {
 int prepare_tgmm() { return reserve_lds(tgmm_dl_kernel, kTdLds, lds_flags<TgmmParams>()); }
+struct TgmmF8Tag0 {};
+struct TgmmF8Tag1 {};
+static int prepare_tgmm_f8(int df) {
+  return df ? reserve_lds(tgmm_f8_kernel<1>, kT8Lds, lds_flags<TgmmF8Tag1>()) : reserve_lds(tgmm_f8_kernel<0>, kT8Lds, lds_flags<TgmmF8Tag0>());
+}
 }  // namespace moe
+
+static bool tgmm_f8_takes(long long M, int K, int N, int G_total, int G_local) {
+  const long long tiles = (long long)(K / kTdTile) * (N / kTdTile) * G_local;
+  return K % kTdTile == 0 && N % kTdTile == 0 && K < (1 << 24) && N < (1 << 24) && M >= 128LL * G_total && tiles >= 128 && tiles <= 0x7fffffffLL;
+}
+
+extern "C" int moe_tgmm_fp8_supported(int M, int K, int N, int num_groups_total, int num_groups_local) {
+  return M >= 0 && K > 0 && N > 0 && num_groups_total > 0 && num_groups_local > 0 && tgmm_f8_takes(M, K, N, num_groups_total, num_groups_local);
+}
+
+extern "C" int moe_tgmm_fp8(const void* lhs, const void* dout, int dout_dtype, const int32_t* group_sizes, int M, int K, int N,
+                            int num_groups_total, int num_groups_local, int group_offset, const float* out_row_scale,
+                            const void* existing_out, int existing_dtype, int out_dtype, void* out, void* stream) {
+  if (!lhs || !dout || !group_sizes || !out) return fail(MOE_ERR_INVALID_ARG, "tgmm_fp8: NULL pointer");
+  if (M < 0 || K <= 0 || N <= 0 || num_groups_total <= 0 || num_groups_local <= 0 || group_offset < 0)
+    return fail(MOE_ERR_INVALID_ARG, "tgmm_fp8: bad sizes");
+  if (dout_dtype != MOE_FP8_E4M3 && dout_dtype != MOE_FP8_E5M2) return fail(MOE_ERR_UNSUPPORTED, "tgmm_fp8: dout_dtype %d", dout_dtype);
+  if (out_dtype != MOE_BF16 && out_dtype != MOE_F32) return fail(MOE_ERR_UNSUPPORTED, "tgmm_fp8: out_dtype %d", out_dtype);
+  if (!tgmm_f8_takes(M, K, N, num_groups_total, num_groups_local))
+    return fail(MOE_ERR_UNSUPPORTED, "tgmm_fp8: needs K and N multiples of 256, 128 rows per group on average and 128 output tiles "
+                "(M=%d K=%d N=%d groups=%d); widen the operands to bf16 for moe_tgmm_scaled otherwise", M, K, N, num_groups_total);
+  if (((uintptr_t)lhs | (uintptr_t)dout | (uintptr_t)out | (uintptr_t)existing_out) & 15) return fail(MOE_ERR_UNSUPPORTED, "tgmm_fp8: pointers must be 16-byte aligned");
+  if (existing_out && existing_dtype != MOE_BF16 && existing_dtype != MOE_F32) return fail(MOE_ERR_UNSUPPORTED, "tgmm_fp8: existing_dtype %d", existing_dtype);
+  if (existing_out == out && existing_dtype != out_dtype) return fail(MOE_ERR_INVALID_ARG, "tgmm_fp8: existing_out aliases out with another element type");
+  TgmmParams p;
+  p.lhs = (const uint16_t*)lhs; p.dout = (const uint16_t*)dout; p.group_sizes = group_sizes; p.out = out;
+  p.M = M; p.K = K; p.N = N; p.G_total = num_groups_total; p.G_local = num_groups_local; p.group_offset = group_offset;
+  p.out_f32 = out_dtype == MOE_F32;
+  p.existing = existing_out; p.existing_f32 = existing_dtype == MOE_F32;
+  p.n_scale = out_row_scale;
+  const int df = dout_dtype == MOE_FP8_E5M2;
+  if (int st = prepare_tgmm_f8(df)) return st;
+  const unsigned tiles = (unsigned)((K / kTdTile) * (N / kTdTile) * num_groups_local);
+  if (df) tgmm_f8_kernel<1><<<tiles, kTdThreads, kT8Lds, (hipStream_t)stream>>>(p);
+  else tgmm_f8_kernel<0><<<tiles, kTdThreads, kT8Lds, (hipStream_t)stream>>>(p);
+  return check_launch("tgmm_f8_kernel");
+}
 
 extern "C" int moe_tgmm_scaled(const void* lhs, const void* dout, const int32_t* group_sizes, int M, int K, int N,
                                int num_groups_total, int num_groups_local, int group_offset, const float* out_row_scale,

@@ -641,3 +641,48 @@ def tgmm(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_d
                            _lib.current_stream())
   _lib.check(st, "moe_tgmm_scaled")
   return out
+
+
+def tgmm_fp8_supported(m, k, n, num_groups_total, num_groups_local=None):
+  """Whether tgmm_fp8 takes this shape (256 x 256 output tiles, 128 rows per group on average)."""
+  g_local = num_groups_total if num_groups_local is None else num_groups_local
+  return bool(_lib.load().moe_tgmm_fp8_supported(int(m), int(k), int(n), int(num_groups_total), int(g_local)))
+
+
+def tgmm_fp8(lhs, dout, group_sizes, *, num_groups_local=None, group_offset=0, out_dtype=torch.bfloat16, existing_out=None,
+             out_row_scale=None):
+  """tgmm on 1-byte operands as stored: lhs [M, K] float8_e4m3fn, dout [M, N] float8_e5m2 or float8_e4m3fn (the drhs
+  product of the fp8_full backward, kernels/megablox/ops.py:590-604) -> [G_local, N, K]."""
+  _need(lhs, "lhs", torch.float8_e4m3fn, 2)
+  _need(dout, "dout", None, 2)
+  if dout.dtype not in (torch.float8_e5m2, torch.float8_e4m3fn):
+    raise TypeError("dout must be float8_e5m2 or float8_e4m3fn")
+  _need(group_sizes, "group_sizes", torch.int32, 1)
+  m, k = lhs.shape
+  if dout.shape[0] != m:
+    raise ValueError("lhs and dout must have the same number of rows")
+  n = dout.shape[1]
+  g_total = group_sizes.numel()
+  g_local = g_total - int(group_offset) if num_groups_local is None else int(num_groups_local)
+  code = {torch.bfloat16: _lib.MOE_BF16, torch.float32: _lib.MOE_F32}
+  if out_dtype not in code:
+    raise TypeError("out_dtype must be bfloat16 or float32")
+  out = torch.empty((g_local, n, k), dtype=out_dtype, device=lhs.device)
+  if existing_out is not None:
+    if existing_out.dtype not in code:
+      raise TypeError("existing_out must be bfloat16 or float32")
+    _need(existing_out, "existing_out", existing_out.dtype, 3)
+    if tuple(existing_out.shape) != (g_local, n, k):
+      raise ValueError(f"existing_out must be [{g_local}, {n}, {k}], got {tuple(existing_out.shape)}")
+  if out_row_scale is not None:
+    _need(out_row_scale, "out_row_scale", torch.float32, 1)
+    if out_row_scale.numel() != n:
+      raise ValueError(f"out_row_scale must have {n} entries, got {out_row_scale.numel()}")
+  st = _lib.load().moe_tgmm_fp8(_lib.ptr(lhs), _lib.ptr(dout), _lib.MOE_FP8_E5M2 if dout.dtype == torch.float8_e5m2 else _lib.MOE_FP8_E4M3,
+                                _lib.ptr(group_sizes), m, k, n, g_total, g_local, int(group_offset),
+                                None if out_row_scale is None else _lib.ptr(out_row_scale),
+                                None if existing_out is None else _lib.ptr(existing_out),
+                                0 if existing_out is None else code[existing_out.dtype], code[out_dtype], _lib.ptr(out),
+                                _lib.current_stream())
+  _lib.check(st, "moe_tgmm_fp8")
+  return out

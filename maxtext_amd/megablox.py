@@ -488,11 +488,17 @@ class _GmmFn(torch.autograd.Function):
         lq_rows = lq[tok]
         ls = ls if ls.numel() == 1 else ls[tok].contiguous()
       ls_m = ls if ls.numel() == m else ls.reshape(1).expand(m).contiguous()
-      d, s_col = kernels.bwd_scale_grad(dout, ls_m, mode="drhs", quantize=quant)
+      # fp8 residuals and an e5m2 gradient multiply as they are stored on shapes the fp8 weight-gradient kernel takes
+      bytes_in = fp8 and quant and kernels.tgmm_fp8_supported(m, k, n, group_sizes.numel(), g_local)
+      d, s_col = kernels.bwd_scale_grad(dout, ls_m, mode="drhs", quantize=quant, as_fp8=bytes_in)
       # the column scales go back onto the f32 products in the kernel's epilogue, which rounds once to the weights' type
       direct = ctx.rhs_dtype in (torch.bfloat16, torch.float32)
-      w = kernels.tgmm(lq_rows.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
-                       out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
+      if bytes_in:
+        w = kernels.tgmm_fp8(lq_rows.contiguous(), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
+                             out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
+      else:
+        w = kernels.tgmm(lq_rows.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
+                         out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
       w = w.to(ctx.rhs_dtype)
       drhs = w if ctx.transpose_rhs else w.transpose(1, 2)
     if marks:

@@ -151,6 +151,39 @@ def test_gmm_e5m2_gradient_times_e4m3_weights(K):
               rhs_scale_block_n=-1, rhs_scale_shared=True)
 
 
+@pytest.mark.parametrize("dout_dtype", [torch.float8_e5m2, E4M3], ids=["e5m2", "e4m3"])
+@pytest.mark.parametrize("offset,g_local", [(0, 4), (1, 2)])
+def test_tgmm_on_fp8_operands_as_stored(K, dout_dtype, offset, g_local):
+  """The drhs product of the fp8_full backward (ops.py:590-604) on 1-byte operands: e4m3 activations x e5m2 (or e4m3)
+  gradient over the whole value range incl. subnormals, ragged groups (a group of 77 rows, an empty one, rows in no
+  group), column scales, existing_out and f32 output, against the exact product of the same bytes; and equal, up to
+  the order of the f32 additions, to the bf16 kernel on the widened operands."""
+  m, k, n, gs = 4300, 2048, 2048, np.asarray([1500, 0, 77, 2600], np.int32)
+  assert K.tgmm_fp8_supported(m, k, n, 4, g_local) and not K.tgmm_fp8_supported(m, 512, 1024, 4, g_local)
+  g = torch.Generator().manual_seed(31 + offset)
+  lhs = (torch.randn(m, k, generator=g) * torch.exp2(torch.randint(-8, 6, (m, 1), generator=g).float())).to(E4M3)
+  spread = (-16, 12) if dout_dtype == torch.float8_e5m2 else (-8, 6)
+  d = (torch.randn(m, n, generator=g) * torch.exp2(torch.randint(*spread, (1, n), generator=g).float())).to(dout_dtype)
+  s_col = torch.rand(n, generator=g) * 1e-2 + 1e-4
+  prev = (torch.randn(g_local, n, k, generator=g) * 4).to(torch.bfloat16)
+  # oracle: [groups, k, n] from the dequantised bytes in f64, scaled per output row n, laid out [groups, n, k]
+  want = O.tgmm(lhs.float(), d.float(), gs, num_actual_groups=g_local, group_offset=offset, out_dtype=torch.float64)
+  want = want.transpose(1, 2) * s_col.double()[None, :, None]
+  kw = dict(num_groups_local=g_local, group_offset=offset)
+  got = K.tgmm_fp8(cuda(lhs), cuda(d), cuda(gs), out_row_scale=cuda(s_col), out_dtype=torch.float32, **kw)
+  assert relerr(got, want.float()) <= 2e-4  # exact products; what is left is the order (and the MFMA's internal alignment) of the f32 additions
+  wide = K.tgmm(cuda(lhs).to(torch.bfloat16), cuda(d).to(torch.bfloat16), cuda(gs), out_row_scale=cuda(s_col), out_dtype=torch.float32, **kw)
+  assert relerr(got, wide) <= 2e-4
+  # bf16 result (the paired-store epilogue), and existing_out joining the accumulator before the one rounding
+  got16 = K.tgmm_fp8(cuda(lhs), cuda(d), cuda(gs), out_row_scale=cuda(s_col), **kw)
+  assert torch.equal(got16, got.to(torch.bfloat16)) or relerr(got16, want.float()) <= 4e-3
+  got_e = K.tgmm_fp8(cuda(lhs), cuda(d), cuda(gs), out_row_scale=cuda(s_col), existing_out=cuda(prev), **kw)
+  assert relerr(got_e, (want + prev.double()).float()) <= 4e-3
+  assert torch.all(got[1 - offset] == 0) if offset == 0 else True  # the empty group's gradient is zero
+  with pytest.raises(RuntimeError):  # shapes without 256 x 256 tiles are refused, not mis-run
+    K.tgmm_fp8(cuda(lhs[:, :384].contiguous()), cuda(d), cuda(gs), **kw)
+
+
 @pytest.mark.parametrize("qdt", [torch.int8, E4M3], ids=["int8", "fp8"])
 @pytest.mark.parametrize("shared", [True, False])
 def test_quantize_rhs_bit_exact(K, qdt, shared):
