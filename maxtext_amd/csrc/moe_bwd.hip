@@ -41,6 +41,59 @@ __device__ __forceinline__ uint32_t e5m2_byte(float on_grid) {
   return (uint32_t)(__builtin_bit_cast(uint16_t, h) >> 8);
 }
 
+// What the quantiser needs of a scale: the scale, its reciprocal rounded once, and whether every value takes the exact
+// route (a zero or non-finite scale).
+struct E5m2Scale {
+  float s, inv;
+  bool exact;
+};
+__device__ __forceinline__ E5m2Scale e5m2_prepare(float amax) {
+  E5m2Scale r;
+  r.s = e5m2_scale(amax);
+  r.exact = !(r.s > 0.f && r.s < INFINITY);
+  r.inv = 1.0f / r.s;
+  return r;
+}
+
+// float8_e5m2 bytes of x0 / s0 and x1 / s1 (bits 0-7 and 8-15), equal to e5m2_byte(to_e5m2_grid(x, s)) bit for bit at a
+// fraction of its instructions: the quotient is formed as x * (1 / s), which lies within 2 ulps of x / s, and rounded by
+// v_cvt_pk_bf8_f32 (nearest even, OCP e5m2 on gfx950); only a product within 4 ulps of a tie of the grid, in the grid's
+// subnormal range (below 2^-14, zero excepted) or not finite goes through the exact division and the rounding spelled
+// out above, lane by lane.
+__device__ __forceinline__ uint32_t e5m2_bytes2(float x0, float x1, const E5m2Scale& a, const E5m2Scale& b) {
+  const float q0 = x0 * a.inv, q1 = x1 * b.inv;
+  uint32_t pk = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(q0, q1, 0, false) & 0xffffu;
+  const uint32_t b0 = __float_as_uint(q0) & 0x7fffffffu, b1 = __float_as_uint(q1) & 0x7fffffffu;
+  const bool n0 = a.exact || ((b0 & 0x1fffffu) - 0xffffcu) <= 8u || (b0 - 1u) < 0x387fffffu || b0 >= 0x7f800000u;
+  const bool n1 = b.exact || ((b1 & 0x1fffffu) - 0xffffcu) <= 8u || (b1 - 1u) < 0x387fffffu || b1 >= 0x7f800000u;
+  if (n0) pk = (pk & 0xff00u) | e5m2_byte(to_e5m2_grid(x0, a.s));
+  if (n1) pk = (pk & 0x00ffu) | (e5m2_byte(to_e5m2_grid(x1, b.s)) << 8);
+  return pk;
+}
+
+// the value of a float8_e5m2 byte (the half whose upper byte it is)
+__device__ __forceinline__ float e5m2_value(uint32_t byte) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(byte << 8)); }
+
+// 8 quantised results of one lane from their bytes (two per entry of pk): bf16 values or the bytes themselves
+template <bool BYTES>
+__device__ __forceinline__ void store8_e5m2(void* out, size_t idx, const uint32_t (&pk)[4]) {
+  if (BYTES) {
+    ((uint2*)out)[idx] = make_uint2(pk[0] | (pk[1] << 16), pk[2] | (pk[3] << 16));
+  } else {
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) w[e] = pack_bf16x2(e5m2_value(pk[e] & 0xffu), e5m2_value(pk[e] >> 8));
+    ((uint4*)out)[idx] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+// bf16(a), bf16(b) as floats: one v_cvt_pk_bf16_f32 for the pair
+__device__ __forceinline__ void round_bf16_pair(float a, float b, float& ra, float& rb) {
+  const uint32_t p = pack_bf16x2(a, b);
+  ra = __uint_as_float(p << 16);
+  rb = __uint_as_float(p & 0xffff0000u);
+}
+
 // 8 results of one lane: bf16 (16 bytes at `out` + 16 * idx) or, BYTES, float8_e5m2 (8 bytes at `out` + 8 * idx)
 template <bool BYTES>
 __device__ __forceinline__ void store8(void* out, size_t idx, const float (&o)[8]) {
@@ -74,6 +127,38 @@ constexpr int kBwdThreads = 256;
 constexpr int kBwdMaxChunks = 8;  // 8 bf16 per lane and chunk: rows of up to 16384 values
 constexpr int kBwdMaxGroups = 1024;
 
+// ends[g] = rows up to and including group g (negative sizes count as empty), built by the whole block: every thread
+// loads up to four sizes at once and the partial sums meet in a scan, so a block pays one memory latency for the table
+// instead of one per group.  Ends with a barrier.
+__device__ __forceinline__ void block_group_ends(const int* __restrict__ group_sizes, int G_total, int* ends) {
+  __shared__ int wave_sum[kBwdThreads / kWave];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  constexpr int PER = kBwdMaxGroups / kBwdThreads;
+  int loc[PER], sum = 0;
+#pragma unroll
+  for (int j = 0; j < PER; j++) {
+    const int g = tid * PER + j;
+    sum += g < G_total ? max(group_sizes[g], 0) : 0;
+    loc[j] = sum;
+  }
+  int incl = sum;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int t = __shfl_up(incl, o, kWave);
+    if (lane >= o) incl += t;
+  }
+  if (lane == kWave - 1) wave_sum[wave] = incl;
+  __syncthreads();
+  int base = incl - sum;
+  for (int w = 0; w < wave; w++) base += wave_sum[w];
+#pragma unroll
+  for (int j = 0; j < PER; j++) {
+    const int g = tid * PER + j;
+    if (g < G_total) ends[g] = base + loc[j];
+  }
+  __syncthreads();
+}
+
 // One block per row: d = bf16(dout * bf16(factor)), factor = rhs_scale[group(row), n] (BY_CHANNEL) or lhs_scale[row];
 // ROW_QUANT: the row's absmax, then the e5m2 values and the row's scale.
 template <bool BY_CHANNEL, bool ROW_QUANT, bool BYTES = false>
@@ -86,14 +171,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4
   const float* f = factor;
   float row_f = 1.0f;
   if (BY_CHANNEL) {
-    if (tid == 0) {
-      int run = 0;
-      for (int g = 0; g < G_total; g++) {
-        run += max(group_sizes[g], 0);
-        ends[g] = run;
-      }
-    }
-    __syncthreads();
+    block_group_ends(group_sizes, G_total, ends);
     f = factor + (size_t)local_group_of(ends, G_total, m, group_offset, G_local) * N;
   } else {
     row_f = round_bf16_fn(factor[m]);
@@ -108,32 +186,37 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4
       const uint4 x = dout[(size_t)m * nvec + i];
       const uint32_t w[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const float xe = bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu);
-        const float fe = BY_CHANNEL ? round_bf16_fn(f[i * 8 + e]) : row_f;
-        v[c][e] = round_bf16_fn(xe * fe);
-        amax_bits = max(amax_bits, __float_as_uint(fabsf(v[c][e])));
+      for (int e = 0; e < 8; e += 2) {
+        const float x0 = __uint_as_float(w[e / 2] << 16), x1 = __uint_as_float(w[e / 2] & 0xffff0000u);
+        float f0 = row_f, f1 = row_f;
+        if (BY_CHANNEL) round_bf16_pair(f[i * 8 + e], f[i * 8 + e + 1], f0, f1);
+        round_bf16_pair(x0 * f0, x1 * f1, v[c][e], v[c][e + 1]);
+        amax_bits = max(amax_bits, max(__float_as_uint(v[c][e]) & 0x7fffffffu, __float_as_uint(v[c][e + 1]) & 0x7fffffffu));
       }
     }
   }
-  float s = 1.0f;
+  E5m2Scale sc = {1.0f, 1.0f, false};
   if (ROW_QUANT) {
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, o, kWave));
     if (tid % kWave == 0) wmax[tid / kWave] = amax_bits;
     __syncthreads();
     const float amax = __uint_as_float(max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
-    s = e5m2_scale(amax);
-    if (tid == 0) scale_out[m] = s;
+    sc = e5m2_prepare(amax);
+    if (tid == 0) scale_out[m] = sc.s;
   }
 #pragma unroll
   for (int c = 0; c < kBwdMaxChunks; c++) {
     const int i = c * kBwdThreads + tid;
     if (i < nvec) {
-      float o[8];
+      if (ROW_QUANT) {
+        uint32_t pk[4];
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = ROW_QUANT ? to_e5m2_grid(v[c][e], s) : v[c][e];
-      store8<BYTES>(out, (size_t)m * nvec + i, o);
+        for (int e = 0; e < 4; e++) pk[e] = e5m2_bytes2(v[c][2 * e], v[c][2 * e + 1], sc, sc);
+        store8_e5m2<BYTES>(out, (size_t)m * nvec + i, pk);
+      } else {
+        store8<false>(out, (size_t)m * nvec + i, v[c]);
+      }
     }
   }
 }
@@ -147,21 +230,22 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_absmax_kernel(const uint4
   const int i = blockIdx.x * kBwdThreads + threadIdx.x;
   if (i >= nvec) return;
   const int m0 = blockIdx.y * kColBand, m1 = min(m0 + kColBand, M);
-  float mx[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  bool bad[8] = {false, false, false, false, false, false, false, false};
+  uint32_t mx[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
   for (int m = m0; m < m1; m++) {
     const uint4 x = dout[(size_t)m * nvec + i];
     const uint32_t w[4] = {x.x, x.y, x.z, x.w};
     const float fm = round_bf16_fn(lhs_scale[m]);
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-      const float d = fabsf(round_bf16_fn(bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu) * fm));
-      bad[e] = bad[e] || d != d;
-      mx[e] = fmaxf(mx[e], d);
+    for (int e = 0; e < 8; e += 2) {
+      float d0, d1;
+      round_bf16_pair(__uint_as_float(w[e / 2] << 16) * fm, __uint_as_float(w[e / 2] & 0xffff0000u) * fm, d0, d1);
+      // (the bit patterns of |d| order like the values, and a NaN's pattern beats every number's)
+      mx[e] = max(mx[e], __float_as_uint(d0) & 0x7fffffffu);
+      mx[e + 1] = max(mx[e + 1], __float_as_uint(d1) & 0x7fffffffu);
     }
   }
 #pragma unroll
-  for (int e = 0; e < 8; e++) atomicMax(colmax + i * 8 + e, bad[e] ? 0x7fc00000u : __float_as_uint(mx[e]));
+  for (int e = 0; e < 8; e++) atomicMax(colmax + i * 8 + e, mx[e] > 0x7f800000u ? 0x7fc00000u : mx[e]);
 }
 
 __global__ void bwd_clear_kernel(uint32_t* p, int n) {
@@ -176,17 +260,21 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4*
   const int i = blockIdx.x * kBwdThreads + threadIdx.x;
   if (i >= nvec) return;
   const int m0 = blockIdx.y * kColBand, m1 = min(m0 + kColBand, M);
-  float s[8];
+  E5m2Scale s[8];
 #pragma unroll
-  for (int e = 0; e < 8; e++) s[e] = e5m2_scale(colmax[i * 8 + e]);
+  for (int e = 0; e < 8; e++) s[e] = e5m2_prepare(colmax[i * 8 + e]);
   for (int m = m0; m < m1; m++) {
     const uint4 x = dout[(size_t)m * nvec + i];
     const uint32_t w[4] = {x.x, x.y, x.z, x.w};
     const float fm = round_bf16_fn(lhs_scale[m]);
-    float o[8];
+    uint32_t pk[4];
 #pragma unroll
-    for (int e = 0; e < 8; e++) o[e] = to_e5m2_grid(round_bf16_fn(bf16_bits_to_f32((w[e / 2] >> (16 * (e & 1))) & 0xffffu) * fm), s[e]);
-    store8<BYTES>(out, (size_t)m * nvec + i, o);
+    for (int e = 0; e < 4; e++) {
+      float d0, d1;
+      round_bf16_pair(__uint_as_float(w[e] << 16) * fm, __uint_as_float(w[e] & 0xffff0000u) * fm, d0, d1);
+      pk[e] = e5m2_bytes2(d0, d1, s[2 * e], s[2 * e + 1]);
+    }
+    store8_e5m2<BYTES>(out, (size_t)m * nvec + i, pk);
   }
 }
 
@@ -200,14 +288,7 @@ __global__ __launch_bounds__(kBwdThreads) void add_group_bias_kernel(const uint4
                                                                      int G_local, int group_offset, uint4* out) {
   __shared__ int ends[kBwdMaxGroups];
   const int m = blockIdx.x, tid = threadIdx.x;
-  if (tid == 0) {
-    int run = 0;
-    for (int g = 0; g < G_total; g++) {
-      run += max(group_sizes[g], 0);
-      ends[g] = run;
-    }
-  }
-  __syncthreads();
+  block_group_ends(group_sizes, G_total, ends);
   int lo = 0, hi = G_total;  // first group whose end lies past the row (G_total: the row is in no group)
   while (lo < hi) {
     const int mid = (lo + hi) >> 1;
