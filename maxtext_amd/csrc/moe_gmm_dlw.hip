@@ -327,9 +327,14 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dlw_kernel(const TiledParam
       set_s_sources(nxt);
     }
     iteration(nk - 2, F_{});
-    load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC == BSRC_I8, C::MI>(esc, p, cur.info, 0, n_out0, lane);
+    // (the epilogue's lane constants are made per tile: hoisted out of the tile loop they are spilled over the main loop
+    // and reloaded between the requests of a tile's last iterations, where every reload waits for the requests in flight;
+    // Qwen3 second projection 0.437 -> 0.411 ms)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    load_epilogue_scales<C::TM, NT_OUT, C::GLU, C::BSRC == BSRC_I8, C::MI>(esc, p, cur.info, 0, n_out0, lane_e);
     iteration(nk - 1, T_{});
-    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU, HALF ? C::TM / 2 : C::TM>(acc, esc, p, cur.info, 0, n_out0, lane);
+    store_epilogue<C::TM, C::TN, NT_OUT, C::GLU, HALF ? C::TM / 2 : C::TM>(acc, esc, p, cur.info, 0, n_out0, lane_e);
     if (!have_n) break;
     cur = nxt;
     base = cb;  // (after the last iteration: the buffer of stage nk = the next tile's stage 0, landed before the last barrier)
