@@ -376,8 +376,9 @@ typedef struct {
 /* flags: rhs is [G_local, K, N] with N contiguous, the reference's default layout (transpose_rhs=False, ops.py:47-52),
  * read as it is: no re-layout pass.  This is how the backward computes dlhs = gmm(dout, rhs, transpose_rhs=True)
  * (ops.py:470-485) from the forward's [G, N, K] weights, whose roles of K and N are then swapped.  BF16 x BF16 without
- * rhs_up, on shapes moe_gmm_rhs_kn_supported() accepts (others return MOE_ERR_UNSUPPORTED: re-lay the weights out with
- * moe_transpose_rhs and call without the flag). */
+ * rhs_up, on shapes moe_gmm_rhs_kn_supported() accepts, and fp8 x fp8 (e4m3 weights, e4m3 or e5m2 activations, scales
+ * per row / tensor x per channel / tensor, no row index) on shapes moe_gmm_fp8_rhs_kn_supported() accepts; others return
+ * MOE_ERR_UNSUPPORTED: re-lay the weights out with moe_transpose_rhs and call without the flag. */
 #define MOE_GMM_RHS_KN 2
 /* flags: layout of rhs_scale / rhs_up_scale, see "Operand layouts" above. */
 #define MOE_GMM_RHS_SCALE_KMAJOR 4
@@ -399,6 +400,9 @@ MOE_API int moe_gmm_rhs_kn_supported(int M, int K, int N, int num_groups_total);
  * N * K < 2^32, 128 rows per group on average and enough tiles to fill the chip), else 0: widen the gradient to bf16
  * (moe_bwd_scale_grad with quantize == 1) and the weights with it. */
 MOE_API int moe_gmm_lhs_e5m2_supported(int M, int K, int N, int num_groups_total);
+/* 1 when moe_gmm takes MOE_GMM_RHS_KN with fp8 operands for this shape (what moe_gmm_lhs_e5m2_supported asks, and
+ * N % 256 == 0), else 0. */
+MOE_API int moe_gmm_fp8_rhs_kn_supported(int M, int K, int N, int num_groups_total);
 /* 1 when the persistent stream kernels take this operand pair at this K and N (whole stages, at least three of them,
  * and every 32-bit byte offset a request can form stays below 2^32), with indexed_lhs_rows = lhs_rows when lhs_row_idx is
  * used, else 0.  moe_gmm falls back to its other kernels otherwise; no counterpart in the reference. */

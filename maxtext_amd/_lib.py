@@ -94,6 +94,7 @@ SIGNATURES = {
     "moe_gmm_workspace_bytes": (c_size_t, [c_int, c_int]),
     "moe_gmm_rhs_kn_supported": (c_int, [c_int, c_int, c_int, c_int]),
     "moe_gmm_lhs_e5m2_supported": (c_int, [c_int, c_int, c_int, c_int]),
+    "moe_gmm_fp8_rhs_kn_supported": (c_int, [c_int, c_int, c_int, c_int]),
     "moe_gmm_stream_kernel_takes": (c_int, [c_int, c_int, c_int, c_int, ctypes.c_longlong]),
     "moe_gmm": (c_int, [ctypes.POINTER(GmmArgs), c_void_p]),
     "moe_gmm_tuned": (c_int, [ctypes.POINTER(GmmArgs), c_int, c_int, c_void_p]),

@@ -187,6 +187,11 @@ int moe_gmm_lhs_e5m2_supported(int M, int K, int N, int num_groups_total) {
   return (long long)max_tiles_for(M, num_groups_total, 256) * cdiv(N, 256) >= 128 ? 1 : 0;
 }
 
+int moe_gmm_fp8_rhs_kn_supported(int M, int K, int N, int num_groups_total) {
+  // fp8 weights as [G, K, N]: the persistent stream kernel reads them through the transposing 8-bit LDS load, 256 channels at a time
+  return moe_gmm_lhs_e5m2_supported(M, K, N, num_groups_total) && N % 256 == 0 ? 1 : 0;
+}
+
 int moe_gmm_stream_kernel_takes(int lhs_dtype, int rhs_dtype, int K, int N, long long indexed_lhs_rows) {
   // which operand families the persistent stream kernels accept at this K, N (and number of indexed activation rows): the
   // shape half of moe_gmm's dispatch, exposed so that the 32-bit offset guards can be checked on the host
@@ -261,8 +266,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   ro.row_idx = a->lhs_row_idx; ro.idx_div = a->lhs_row_idx_div < 1 ? 1 : a->lhs_row_idx_div;
   ro.lhs_rows = a->lhs_row_idx ? a->lhs_rows : M; ro.out_f32 = a->out_dtype == MOE_F32; ro.row_scale = a->out_row_scale;
 
-  if ((a->flags & MOE_GMM_RHS_KN) && (L != MOE_BF16 || R != MOE_BF16 || glu || !moe_gmm_rhs_kn_supported(M, K, N, G)))
-    return fail(MOE_ERR_UNSUPPORTED, "gmm: [G, K, N] weights need bf16 x bf16 without rhs_up and a shape moe_gmm_rhs_kn_supported accepts");
+  const bool rhs_kn = (a->flags & MOE_GMM_RHS_KN) != 0;
+  const bool kn_fp8 = rhs_kn && L == MOE_FP8_E4M3 && R == MOE_FP8_E4M3;
+  if (rhs_kn && !kn_fp8 && (L != MOE_BF16 || R != MOE_BF16 || glu || !moe_gmm_rhs_kn_supported(M, K, N, G)))
+    return fail(MOE_ERR_UNSUPPORTED, "gmm: [G, K, N] weights need bf16 x bf16 (or fp8 x fp8) without rhs_up and a shape moe_gmm_rhs_kn_supported accepts");
+  if (kn_fp8 && (glu || !moe_gmm_fp8_rhs_kn_supported(M, K, N, G) || a->lhs_row_idx))
+    return fail(MOE_ERR_UNSUPPORTED, "gmm: [G, K, N] fp8 weights need a shape moe_gmm_fp8_rhs_kn_supported accepts, no rhs_up and no row index");
   const bool quant_pair = (L == MOE_INT8 && R == MOE_INT8) || (L == MOE_FP8_E4M3 && R == MOE_FP8_E4M3);
   ScalePlan sp = {};
   // DeepSeek block scales: fp8 with [M, K/128] x [G, N/128, K/128]
@@ -310,6 +319,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     const bool prefill = kernel == MOE_GMM_KERNEL_BIG || (kernel == MOE_GMM_KERNEL_AUTO && (long long)M >= 128LL * G && chip_full);
     // scales in the epilogue only (per row / per tensor x per channel / per tensor): the int8 x int8 problem on another MFMA
     const bool stream_epi = !fp8_blocks && prefill && dls_takes(OP_F8, K, N, ro.row_idx ? ro.lhs_rows : 0);
+    if (kn_fp8 && !stream_epi) return fail(MOE_ERR_UNSUPPORTED, "gmm: [G, K, N] fp8 weights run on the persistent 256 x 256 kernel only (no K-block scales)");
     if (lhs_e5m2 && !stream_epi)
       return fail(MOE_ERR_UNSUPPORTED, "gmm: float8_e5m2 activations run on the persistent 256 x 256 kernel only (128 rows per group on average, "
                   "K %% 128 == 0, K >= 384, no rhs_up, no K-block scales); widen them to bf16 for other shapes");
@@ -325,7 +335,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       q.lhs_scale = sp.lhs_epi; q.lhs_scale_stride = sp.lhs_epi_stride;
       q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
       q.rhs_scale_gstride = sp.rhs_gstride; q.rhs_scale_nstride = sp.rhs_nstride;
-      return launch_dls(OP_F8, glu, q, M, G, s, lhs_e5m2 ? 1 : 0);
+      return launch_dls(OP_F8, glu, q, M, G, s, lhs_e5m2 ? 1 : 0, kn_fp8 ? 1 : 0);
     }
     if (tiled) {
       const bool big = kernel == MOE_GMM_KERNEL_BIG;

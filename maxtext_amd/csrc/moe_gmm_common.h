@@ -624,7 +624,7 @@ int launch_dl(int op, bool glu, int stage_bytes, bool rhs_kn, const TiledParams&
 // moe_gmm_dlw.hip: the same pipeline for bf16 activations x int8 / int4 / mxfp4 weights (K % 64 == 0, default scale layouts)
 // moe_gmm_dls.hip: the persistent 256 x 256 kernel for int8 x int8 / bf16 x bf16 with one request stream across tiles
 // (fp8 x fp8 with epilogue scales too; lhs_e5m2: the activations are float8_e5m2, the weights e4m3)
-int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s, int lhs_e5m2 = 0);
+int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s, int lhs_e5m2 = 0, int rhs_kn = 0);
 bool dls_takes(int op, int K, int N, long long indexed_lhs_rows);
 // moe_gmm_f8s.hip: the same stream for block-scaled fp8 (1 x 128 activation scales, 128 x 128 weight scales)
 struct Fp8TiledParams;

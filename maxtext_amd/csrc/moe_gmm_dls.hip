@@ -27,11 +27,15 @@
 
 namespace moe {
 
-template <int OP_, bool GLU_, int LF_ = 0>
+template <int OP_, bool GLU_, int LF_ = 0, bool KN_ = false>
 struct DlsCfg {
   static constexpr int OP = OP_;
   static constexpr bool GLU = GLU_;
   static constexpr int LF = LF_;  // fp8 activations: 0 = e4m3, 1 = e5m2 (format selector of the MFMA's second operand)
+  // fp8 weights given as [G, K, N] (the contraction index as the row: dlhs of a layer whose weights are [G, N, K], read as
+  // they are).  The weight half of a stage then holds 128 contraction rows x 256 output channels (128 x 256 B, four rows per
+  // wave instruction) and the weight fragments come out of it through ds_read_b64_tr_b8.
+  static constexpr bool KN = KN_;
   static constexpr int BM = 256, BN = 256, BKB = 128, MI = 16;
   static constexpr int ESZ = OP == OP_BF16 ? 2 : 1, BK = BKB / ESZ;
   static constexpr int WAVES_M = 2, WAVES_N = 4, NWAVES = 8, THREADS = NWAVES * kWave;
@@ -45,6 +49,10 @@ struct DlsCfg {
   static constexpr int REQ_STRIDE = 3, REQ_STRIDE_F8 = 1;
   static_assert(OP == OP_I8 || OP == OP_BF16 || OP == OP_F8, "operands");
   static_assert(LF == 0 || OP == OP_F8, "only fp8 activations come in two formats");
+  static_assert(!KN || (OP == OP_F8 && !GLU), "[G, K, N] weights: fp8 without rhs_up");
+  // slot of the 16-byte chunk c of contraction row r in a [G, K, N] weight stage: c ^ kn_swz(r); the 8 rows of a transposing
+  // read and those of the next lane group (16 rows further) then fall into 16 different 16-byte bank groups
+  __device__ static __forceinline__ int kn_swz(int row) { return (row & 7) ^ (((row >> 4) & 1) << 3); }
   __device__ static __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 };
 
@@ -96,17 +104,28 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParam
   const bool load_up = C::GLU && wave >= C::NWAVES / 2;
 #pragma unroll
   for (int i = 0; i < C::B_IPW; i++) {
-    const int r = (wave * C::B_IPW + i) * 8 + lane / 8;
-    b_voff[i] = lane_off(i, (uint32_t)(C::GLU ? r % (C::BN / 2) : r));
+    if constexpr (C::KN) {
+      // request i covers contraction rows (wave * 4 + i) * 4 + lane / 16 of the stage, the lane LDS slot lane % 16 of its row
+      const int r = (wave * C::B_IPW + i) * 4 + lane / 16;
+      b_voff[i] = (uint32_t)r * (uint32_t)N + (uint32_t)(((lane % 16) ^ C::kn_swz(r)) << 4);
+    } else {
+      const int r = (wave * C::B_IPW + i) * 8 + lane / 8;
+      b_voff[i] = lane_off(i, (uint32_t)(C::GLU ? r % (C::BN / 2) : r));
+    }
   }
   auto set_b_sources = [&](const Tile& t) {
-    b_desc = buffer_desc((load_up ? p.rhs_up : p.rhs) + (size_t)t.info.group * N * row_bytes, clamp_u32((size_t)N * row_bytes));
-    b_soff = (uint32_t)t.n0 * row_bytes;
+    if constexpr (C::KN) {
+      b_desc = buffer_desc(p.rhs + (size_t)t.info.group * N * row_bytes, clamp_u32((size_t)N * row_bytes));
+      b_soff = (uint32_t)t.n0;  // the tile's first output channel: a byte offset inside every contraction row
+    } else {
+      b_desc = buffer_desc((load_up ? p.rhs_up : p.rhs) + (size_t)t.info.group * N * row_bytes, clamp_u32((size_t)N * row_bytes));
+      b_soff = (uint32_t)t.n0 * row_bytes;
+    }
   };
   // request idx of the stage: 0 .. 3 activations, 4 .. 7 weights
   auto issue_one = [&](int kt, int buf, int idx) {
     if (idx < C::A_IPW) dma16_buffer(a_desc, a_voff[idx], (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + (wave * C::A_IPW + idx) * 1024);
-    else dma16_buffer(b_desc, b_voff[idx - C::A_IPW], b_soff + (uint32_t)kt * C::BKB, lds_base + buf * C::STAGE + C::A_STAGE + (wave * C::B_IPW + idx - C::A_IPW) * 1024);
+    else dma16_buffer(b_desc, b_voff[idx - C::A_IPW], b_soff + (uint32_t)kt * C::BKB * (C::KN ? (uint32_t)N : 1u), lds_base + buf * C::STAGE + C::A_STAGE + (wave * C::B_IPW + idx - C::A_IPW) * 1024);
   };
 
 
@@ -140,7 +159,26 @@ __global__ __launch_bounds__(C::THREADS, 2) void gmm_dls_kernel(const TiledParam
       f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
     };
     auto read_a = [&](int buf, int i, int slot) { read_frag(ga[slot], smem + buf * C::STAGE + (wm * C::WM + i * 16) * C::BKB); };
-    auto read_b = [&](int buf, int j) { read_frag(gb[j], smem + buf * C::STAGE + C::A_STAGE + b_row[j] * C::BKB); };
+    // [G, K, N] weights: lane (s, q) addresses row 16 q + s / 2 (+ 8, 64, 72) of the stage's 128 contraction rows, i.e. the K
+    // bytes 16 q .. and 64 + 16 q .. its activation fragment holds, and the 8 bytes s % 2 of the fragment's 16-byte channel block
+    const int kn_base = C::A_STAGE + (16 * (lane / 16) + (lane % 16) / 2) * C::BN + ((((wn * C::TN) ^ ((lane % 16) / 2) ^ (((lane / 16) & 1) << 3))) << 4) + (lane % 2) * 8;
+    auto read_b = [&](int buf, int j) {
+      if constexpr (C::KN) {
+        typedef int v2i_kn __attribute__((ext_vector_type(2)));
+        typedef __attribute__((address_space(3))) v2i_kn* lds_v2i_kn;
+        int base = kn_base;
+        asm volatile("" : "+v"(base));
+        const uint8_t* src = smem + buf * C::STAGE + (base ^ (j << 4));
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          const v2i_kn x = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_kn)(src + ((t & 1) * 8 + (t >> 1) * 64) * C::BN));
+          gb[j][2 * t] = x[0];
+          gb[j][2 * t + 1] = x[1];
+        }
+      } else {
+        read_frag(gb[j], smem + buf * C::STAGE + C::A_STAGE + b_row[j] * C::BKB);
+      }
+    };
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     // First half of a stage (in buffer buf): row tiles 0 .. 3 from the ring, each slot reloaded with row tile + 4.
     // ZC: the tile's first stage starts from zero.
@@ -372,6 +410,8 @@ int prepare_dls() {
   if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, false>>();
   if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, true>>();
   if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, false, 1>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, false, 0, true>>();
+  if (!st) st = prepare_dls_cfg<DlsCfg<OP_F8, false, 1, true>>();
   return st;
 }
 
@@ -405,11 +445,13 @@ bool dls_takes(int op, int K, int N, long long indexed_lhs_rows) {
          (indexed_lhs_rows + 256) * pitch < (1LL << 32);
 }
 
-int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s, int lhs_e5m2) {
+int launch_dls(int op, bool glu, const TiledParams& p, int M, int G_total, hipStream_t s, int lhs_e5m2, int rhs_kn) {
   if (!dls_takes(op, p.K, p.N, p.ro.row_idx ? p.ro.lhs_rows : 0))
     return fail(MOE_ERR_UNSUPPORTED, "gmm: the stream kernel needs int8, bf16 or fp8 operands, whole 128-byte stages (three or more) and 32-bit byte offsets");
   if (lhs_e5m2 && (op != OP_F8 || glu)) return fail(MOE_ERR_UNSUPPORTED, "gmm: e5m2 activations run against e4m3 weights without rhs_up");
+  if (rhs_kn && (op != OP_F8 || glu || p.N % 256 != 0)) return fail(MOE_ERR_UNSUPPORTED, "gmm: [G, K, N] weights on the stream kernel need fp8 operands, no rhs_up and N %% 256 == 0");
   if (op == OP_F8) {
+    if (rhs_kn) return lhs_e5m2 ? launch_dls_cfg<DlsCfg<OP_F8, false, 1, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_F8, false, 0, true>>(p, M, G_total, s);
     if (lhs_e5m2) return launch_dls_cfg<DlsCfg<OP_F8, false, 1>>(p, M, G_total, s);
     return glu ? launch_dls_cfg<DlsCfg<OP_F8, true>>(p, M, G_total, s) : launch_dls_cfg<DlsCfg<OP_F8, false>>(p, M, G_total, s);
   }

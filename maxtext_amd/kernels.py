@@ -461,7 +461,8 @@ def gmm_raw(lhs, rhs, group_sizes, *, lhs_scale=None, rhs_scale=None, rhs_up=Non
             lhs_row_idx=None, lhs_row_idx_div=1, out_row_scale=None, num_rows=None, workspace=None, same_groups=False,
             group_offset_dev=None):
   """Grouped matmul on native layouts: lhs [M,K], rhs [G,N,K] (INT4 / MXFP4: uint8 [G,N,K/2]).
-  rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 without rhs_up, on shapes `gmm_rhs_kn_supported` accepts).
+  rhs_kn: rhs is [G,K,N] instead (bf16 x bf16 on shapes `gmm_rhs_kn_supported` accepts, fp8 x fp8 on shapes
+  `gmm_fp8_rhs_kn_supported` accepts; no rhs_up).
   Scale layouts follow include/moe_mi355x.h: lhs_scale_block_k 0 = [M], -1 = [1] (per tensor), b = [M, ceil(K/b)];
   rhs scales [G, ceil(N/bn), ceil(K/bk)], or [G, ceil(K/bk), N] with rhs_scale_kmajor, without the leading G with
   rhs_scale_shared; bn = -1: one scale for all channels.
@@ -597,6 +598,11 @@ def gmm_workspace(m, num_groups_total, device):
 def gmm_lhs_e5m2_supported(m, k, n, num_groups_total):
   """True when `gmm_raw` takes float8_e5m2 activations (against e4m3 weights) for this shape."""
   return bool(_lib.load().moe_gmm_lhs_e5m2_supported(int(m), int(k), int(n), int(num_groups_total)))
+
+
+def gmm_fp8_rhs_kn_supported(m, k, n, num_groups_total):
+  """True when `gmm_raw(..., rhs_kn=True)` takes [G, K, N] float8_e4m3fn weights of this shape as they are (fp8 activations)."""
+  return bool(_lib.load().moe_gmm_fp8_rhs_kn_supported(int(m), int(k), int(n), int(num_groups_total)))
 
 
 def gmm_rhs_kn_supported(m, k, n, num_groups_total):

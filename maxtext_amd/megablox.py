@@ -459,15 +459,18 @@ class _GmmFn(torch.autograd.Function):
       # dout times the weights' channel scales of each row's expert, e5m2 per row (one kernel)
       rs_gn = rs.reshape(-1, n) if rs.numel() % n == 0 else rs.reshape(1, 1).expand(1, n)
       rs_gn = (rs_gn if rs_gn.shape[0] == g_local else rs_gn[:1].expand(g_local, n)).contiguous()
-      w_t = kernels.transpose_rhs(rq)  # [g, n, k] -> [g, k, n]: the layout with k as the output axis
       as_fp8 = fp8 and quant and kernels.gmm_lhs_e5m2_supported(m, n, k, group_sizes.numel())
+      # the forward's [g, n, k] weights are the [G, K, N] layout of this product (n contracted, k the output axis): the fp8
+      # stream kernel reads them as they are; the other routes take a re-laid-out copy [g, k, n]
+      as_kn = as_fp8 and kernels.gmm_fp8_rhs_kn_supported(m, n, k, group_sizes.numel())
+      w_t = None if as_kn else kernels.transpose_rhs(rq)
       d, s_row = kernels.bwd_scale_grad(dout, rs_gn, mode="dlhs", quantize=quant, group_sizes=group_sizes, num_groups_local=g_local,
                                         group_offset=ctx.offset, as_fp8=as_fp8)
       one = torch.ones((1,), dtype=torch.float32, device=dout.device)
       if as_fp8:
         # e5m2 x e4m3 on the fp8 MFMA; the rows' scales are the activations' epilogue scales
-        dlhs = kernels.gmm_raw(d, w_t, group_sizes, lhs_scale=s_row, rhs_scale=one, rhs_scale_block_n=_lib_per_tensor(),
-                               rhs_scale_shared=True, group_offset=ctx.offset)
+        dlhs = kernels.gmm_raw(d, rq if as_kn else w_t, group_sizes, lhs_scale=s_row, rhs_scale=one, rhs_scale_block_n=_lib_per_tensor(),
+                               rhs_scale_shared=True, group_offset=ctx.offset, rhs_kn=as_kn)
       else:
         # the row scales go back on in the product's epilogue (rounded bf16 result times scale, rounded again: what the
         # reference's two steps give)

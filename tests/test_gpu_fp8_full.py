@@ -151,6 +151,36 @@ def test_gmm_e5m2_gradient_times_e4m3_weights(K):
               rhs_scale_block_n=-1, rhs_scale_shared=True)
 
 
+@pytest.mark.parametrize("lhs_dtype", [torch.float8_e5m2, E4M3], ids=["e5m2", "e4m3"])
+def test_gmm_fp8_weights_read_as_gkn(K, lhs_dtype):
+  """MOE_GMM_RHS_KN with fp8 operands (dlhs of the fp8_full backward from the forward's [G, N, K] weights, ops.py:470-485,
+  without the re-layout): bit-equal to the same product on the transposed copy, ragged groups, an empty group, rows in no
+  group, a group window, per-row scales and a row factor."""
+  m, kc, n, gs = 4200, 640, 2048, np.asarray([1500, 0, 700, 1900], np.int32)  # contraction kc, n output channels
+  assert K.gmm_fp8_rhs_kn_supported(m, kc, n, 4) and not K.gmm_fp8_rhs_kn_supported(m, kc, n + 128, 4)
+  g = torch.Generator().manual_seed(23)
+  d = (torch.randn(m, kc, generator=g) * torch.exp2(torch.randint(-10, 8, (m, 1), generator=g).float())).clamp(-448, 448).to(lhs_dtype)
+  w_kn = (torch.randn(4, kc, n, generator=g) * 3).to(E4M3)  # [G, K, N]
+  w_nk = w_kn.float().transpose(1, 2).contiguous().to(E4M3)  # the re-laid-out copy, [G, N, K]
+  s_row = torch.rand(m, generator=g) * 1e-3 + 1e-5
+  fac = torch.rand(m, generator=g) + 0.5
+  one = torch.ones(1)
+  kw = dict(lhs_scale=cuda(s_row), rhs_scale=cuda(one), rhs_scale_block_n=-1, rhs_scale_shared=True, out_dtype=torch.float32)
+  for extra in (dict(), dict(out_row_scale=cuda(fac))):
+    ref = K.gmm_raw(cuda(d), cuda(w_nk), cuda(gs), **kw, **extra)
+    got = K.gmm_raw(cuda(d), cuda(w_kn), cuda(gs), rhs_kn=True, **kw, **extra)
+    assert torch.equal(got, ref)
+  want = O.gmm(d.float(), w_nk.float(), gs, lhs_scale=s_row, transpose_rhs=True, out_dtype=torch.float32)
+  assert relerr(got / cuda(fac)[:, None], want) <= 1e-4
+  # a window of two local groups
+  ref = K.gmm_raw(cuda(d), cuda(w_nk[2:4]), cuda(gs), group_offset=2, **kw)
+  got = K.gmm_raw(cuda(d), cuda(w_kn[2:4]), cuda(gs), group_offset=2, rhs_kn=True, **kw)
+  assert torch.equal(got, ref)
+  with pytest.raises(RuntimeError):  # K-block scales do not run there
+    K.gmm_raw(cuda(d.to(E4M3)), cuda(w_kn), cuda(gs), rhs_kn=True, lhs_scale=cuda(torch.ones(m, kc // 128)), lhs_scale_block_k=128,
+              rhs_scale=cuda(torch.ones(4, n // 128, kc // 128)), rhs_scale_block_n=128, rhs_scale_block_k=128)
+
+
 @pytest.mark.parametrize("dout_dtype", [torch.float8_e5m2, E4M3], ids=["e5m2", "e4m3"])
 @pytest.mark.parametrize("offset,g_local", [(0, 4), (1, 2)])
 def test_tgmm_on_fp8_operands_as_stored(K, dout_dtype, offset, g_local):
