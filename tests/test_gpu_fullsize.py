@@ -231,8 +231,8 @@ def test_fullsize_deepseek_whole_layer_output_against_oracle():
 
 @pytest.mark.parametrize("name", ["c2", "c4", "c5"])
 def test_fullsize_whole_layer_output_against_oracle(name):
-  """Every element of the layer output at BASELINE's full size (C2: 8192 x 4096, C4: 16384 x 2048, C5: 4096 x 2880)
-  against the CPU oracle run on the identical quantised weights, plus the integer half of the path over all rows."""
+  """Every element of the layer output at BASELINE's full size (C2: 8192 x 4096, C4: 16384 x 2048, C5: 4096 x 2880) against
+  the CPU oracle run on the identical quantised weights, plus the integer half of the path over all rows."""
   from maxtext_amd import moe, synthetic
   from maxtext_amd.quantizations import QArray
   from oracle.layer import oracle_layer
@@ -240,12 +240,14 @@ def test_fullsize_whole_layer_output_against_oracle(name):
   wl = synthetic.workload(name)
   cfg = wl.cfg
   layer = synthetic.make_layer(wl, device="cpu")
-  trip = lambda qa: (qa.qvalue, qa.scale, qa.qtype)
+  trip = synthetic.as_triple
   want, oidx, operm, ogs = oracle_layer(
       layer["x"], layer["gate_logits"], layer["pre_bias_logits"], trip(layer["wi_0"]), trip(layer["wi_1"]), trip(layer["wo"]),
       num_experts=cfg.num_experts, k=cfg.num_experts_per_tok, emb_dim=cfg.emb_dim, mlp_dim=cfg.moe_mlp_dim,
       norm_topk_prob=cfg.norm_topk_prob, act_quant=cfg.act_quant, activation=cfg.activation, acc_dtype=torch.float32)
-  dev = lambda v: QArray(v.qvalue.cuda(), v.scale.cuda(), v.qtype) if isinstance(v, QArray) else v.cuda()
+  import dataclasses
+
+  dev = lambda v: dataclasses.replace(v, qvalue=v.qvalue.cuda(), scale=v.scale.cuda()) if isinstance(v, QArray) else v.cuda()
   wi_0, wi_1, wo = dev(layer["wi_0"]), dev(layer["wi_1"]), dev(layer["wo"])
   block = moe.RoutedMoE(cfg, wi_0, wi_1, wo)
   x, logits = layer["x"].cuda(), layer["gate_logits"].cuda()
@@ -259,6 +261,54 @@ def test_fullsize_whole_layer_output_against_oracle(name):
   # wherever the bf16 intermediates differ by an ulp: a noise of about 0.6 % of the output's rms per element, whose
   # maximum over 33 million elements reaches 3.3 %
   assert relerr(got, want, atol_rms=4e-2 if cfg.act_quant else ELEM_ATOL_RMS_CHAINED) <= TOL
+
+
+def test_fullsize_fp8_row_by_channel_layer_stage_by_stage():
+  """The forward of the fp8_full recipe at the Mixtral shape (8192 tokens, e4m3 rows x e4m3 channels on the stream kernel),
+  every element of every stage against the CPU oracle.  An e4m3 re-quantisation in the middle of the chain makes two
+  pipelines diverge by whole fp8 steps wherever their bf16 intermediates differ by an ulp (about 70 of a row's 14336
+  values, 7 % of the output's rms at the worst of 33 million), so each oracle stage is fed the GPU's previous stage and the
+  quantisers are compared bit for bit; the end-to-end output is then held to the max-norm bound only."""
+  from maxtext_amd import kernels, megablox, synthetic
+
+  wl = synthetic.workload("c2f8")
+  cfg = wl.cfg
+  L = synthetic.make_layer(wl, device="cuda")
+  t, k, e, d = wl.tokens, cfg.num_experts_per_tok, cfg.num_experts, cfg.emb_dim
+  w, idx = kernels.route_topk(L["gate_logits"].reshape(t, e).float().contiguous(), k=k, norm_topk_prob=cfg.norm_topk_prob)
+  perm, inv, gs, _ = kernels.sort_by_expert(idx, e)
+  x2d = L["x"].reshape(t, d)
+  # stage 0: the activation quantiser, one scale per token row, bit for bit
+  xq = megablox.quantize_lhs(x2d, "fp8")
+  oq, osc = O.quantize_rows_fp8(x2d.cpu())
+  assert torch.equal(xq.qvalue.cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(xq.scale.cpu(), osc)
+  # stage 1: both first projections + SwiGLU, the rows read through the permutation
+  inter = gmm_bf16(xq, L["wi_0"], gs, transpose_rhs=True, rhs_up=L["wi_1"], fuse_act=cfg.activation, lhs_row_idx=perm, lhs_row_idx_div=k)
+  rows = torch.from_numpy(perm.cpu().numpy().astype(np.int64) // k)
+  ogs = gs.cpu().numpy()
+  kw = dict(lhs_scale=osc[rows], out_dtype=torch.float32, acc_dtype=torch.float32)
+  tr = lambda qa: qa.qvalue.cpu().transpose(1, 2)
+  h0 = O.gmm(oq[rows], tr(L["wi_0"]), ogs, rhs_scale=L["wi_0"].scale.cpu(), **kw)
+  h1 = O.gmm(oq[rows], tr(L["wi_1"]), ogs, rhs_scale=L["wi_1"].scale.cpu(), **kw)
+  assert relerr(inter, O.apply_ffn_activation(h0, h1, cfg.activation)) <= TOL
+  del h0, h1
+  # stage 2: the intermediate's quantiser bit for bit, then the second projection on the GPU's own intermediate
+  iq = megablox.quantize_lhs(inter, "fp8")
+  oiq, oisc = O.quantize_rows_fp8(inter.cpu())
+  assert torch.equal(iq.qvalue.cpu().view(torch.uint8), oiq.view(torch.uint8)) and torch.equal(iq.scale.cpu(), oisc)
+  y = gmm_bf16(iq, L["wo"], gs, transpose_rhs=True)
+  want_y = O.gmm(oiq, tr(L["wo"]), ogs, rhs_scale=L["wo"].scale.cpu(), lhs_scale=oisc, acc_dtype=torch.float32)
+  assert relerr(y, want_y) <= TOL
+  # stage 3: the combine on the GPU's rows
+  out = kernels.unpermute_combine(y, w, k=k, inv_perm=inv)
+  want_out = O.unpermute(y.cpu(), perm.cpu().numpy(), w.cpu().numpy(), k)
+  assert relerr(out, want_out) <= TOL
+  # and the layer mirror gives these very values end to end
+  from maxtext_amd import moe
+
+  block = moe.RoutedMoE(cfg, L["wi_0"], L["wi_1"], L["wo"])
+  full, _, _ = block.sparse_matmul(L["x"], L["gate_logits"], None, L["wi_0"], L["wi_1"], L["wo"])
+  assert torch.equal(full.reshape(t, d), out)
 
 
 @pytest.mark.parametrize("name,tokens", [("c4", 768), ("c5", 384), ("c5", 880), ("c5mx", 512)])
