@@ -2,10 +2,12 @@
 // qpl.quantize(rhs, weight_qtype, channelwise_axes=[2]) (kernels/megablox/ops.py:250-260: one scale per output channel,
 // shared by the experts and by K) or manual_quantize (layers/quantizations.py:961-991: one static scale for the tensor).
 //
-// Weights are [G, N, K] with K contiguous, so a channel's values are G rows of K.  Dynamic scales take two passes over
-// the weights (bf16 in, 1 byte out: 5 bytes per value in all): every block reduces one row to its absmax and merges it
-// into the channel's maximum with an atomic max on the bit pattern; the second pass divides by absmax / qmax and rounds.
-// A static scale needs the second pass only.
+// Weights are [G, N, K] with K contiguous, so a channel's values are G rows of K.  Dynamic scales per channel are made
+// and applied by one block per channel that sweeps its rows twice, the second time out of the caches (bf16 in once, 1 byte
+// out: 3 bytes per value from HBM); a scale over more than a million values (per tensor, or hundreds of experts sharing
+// long rows) takes two launches (5 bytes per value): every block reduces one row to its absmax and merges it into the
+// scale's maximum with an atomic max on the bit pattern, the second pass divides by absmax / qmax and rounds.  A static
+// scale needs the second pass only.
 
 #include "moe_common.h"
 
@@ -88,6 +90,64 @@ __global__ __launch_bounds__(kQThreads) void rhs_quant_kernel(const uint4* __res
   }
 }
 
+// Dynamic scales per channel in one launch: a block owns one scale (a channel's G rows of K when the experts share it,
+// one row otherwise), sweeps its rows once for the absmax and a second time, while they still sit in the caches (64 to
+// 230 KB per block on the Mixtral shapes), to quantise them: the weights come from HBM once instead of twice.  Same
+// arithmetic as the two kernels above.
+template <int MODE>
+__global__ __launch_bounds__(kQThreads) void rhs_quant_slot_kernel(const uint4* __restrict__ w, int G, int N, int K, int shared, uint2* __restrict__ q,
+                                                                    float* __restrict__ scale) {
+  __shared__ uint32_t wmax[kQThreads / kWave];
+  const int slot = blockIdx.x, tid = threadIdx.x;
+  const int nvec = K / 8, nrows = shared ? G : 1;
+  const float qmax = MODE == 0 ? 127.0f : 448.0f;
+  uint32_t m = 0u;
+  for (int r = 0; r < nrows; r++) {
+    const uint4* row = w + ((size_t)(shared ? r * N + slot : slot)) * nvec;
+    for (int i = tid; i < nvec; i += kQThreads) {
+      float f[8];
+      unpack_bf16x8(row[i], f);
+#pragma unroll
+      for (int e = 0; e < 8; e++) m = max(m, __float_as_uint(fabsf(f[e])));
+    }
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, o, kWave));
+  if (tid % kWave == 0) wmax[tid / kWave] = m;
+  __syncthreads();
+  const float sc = __uint_as_float(max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]))) / qmax;
+  if (tid == 0) scale[slot] = sc;
+  for (int r = 0; r < nrows; r++) {
+    const size_t base = ((size_t)(shared ? r * N + slot : slot)) * nvec;
+    for (int i = tid; i < nvec; i += kQThreads) {
+      float f[8];
+      unpack_bf16x8(w[base + i], f);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float y = sc == 0.f ? 0.f : f[e] / sc;
+        f[e] = fminf(fmaxf(MODE == 0 ? rintf(y) : y, -qmax), qmax);
+      }
+      uint32_t lo, hi;
+      if (MODE == 0) {
+        uint32_t b[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) b[e] = (uint32_t)((int)f[e]) & 0xffu;
+        lo = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        hi = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+      } else {
+        int l = 0, h = 0;
+        l = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], l, false);
+        l = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], l, true);
+        h = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], h, false);
+        h = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], h, true);
+        lo = (uint32_t)l;
+        hi = (uint32_t)h;
+      }
+      q[base + i] = make_uint2(lo, hi);
+    }
+  }
+}
+
 __global__ void rhs_clear_kernel(uint32_t* p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0u;
@@ -122,6 +182,13 @@ extern "C" int moe_quantize_rhs(const void* w, int G, int N, int K, int out_dtyp
   }
   if (shared < 0 || shared > 2) return fail(MOE_ERR_INVALID_ARG, "quantize_rhs: shared must be 0 (per expert), 1 (shared by the experts) or 2 (per tensor)");
   const int ns = shared == 2 ? 1 : shared ? N : rows;
+  // a scale whose values fit the caches between two sweeps of one block (2 MB: 128 experts of 8192) is made and applied in
+  // one launch
+  if (shared != 2 && (long long)(shared ? G : 1) * K <= (1LL << 20)) {
+    if (out_dtype == MOE_INT8) rhs_quant_slot_kernel<0><<<ns, kQThreads, 0, s>>>(x, G, N, K, shared, (uint2*)q, scale);
+    else rhs_quant_slot_kernel<1><<<ns, kQThreads, 0, s>>>(x, G, N, K, shared, (uint2*)q, scale);
+    return check_launch("rhs_quant_slot_kernel");
+  }
   rhs_clear_kernel<<<cdiv(ns, 256), 256, 0, s>>>((uint32_t*)scale, ns);
   rhs_absmax_kernel<<<rows, kQThreads, 0, s>>>(x, N, K, shared, (uint32_t*)scale);
   if (out_dtype == MOE_INT8) rhs_quant_kernel<0, false><<<rows, kQThreads, 0, s>>>(x, N, K, shared, scale, nullptr, (uint2*)q);

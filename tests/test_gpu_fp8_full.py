@@ -216,12 +216,14 @@ def test_tgmm_on_fp8_operands_as_stored(K, dout_dtype, offset, g_local):
 
 @pytest.mark.parametrize("qdt", [torch.int8, E4M3], ids=["int8", "fp8"])
 @pytest.mark.parametrize("shared", [True, False])
-def test_quantize_rhs_bit_exact(K, qdt, shared):
+@pytest.mark.parametrize("G,N,Kd", [(3, 72, 264), (300, 16, 4096), (2, 24, 16384)], ids=["small", "two-pass", "long-rows"])
+def test_quantize_rhs_bit_exact(K, qdt, shared, G, N, Kd):
   """The per-step weight quantiser (ops.py:250-260) against the host statement of the same rule: scale = absmax / qmax
   over each output channel (of all experts, or per expert), q = rint(w / scale) / the nearest-even float8 cast; values and
-  scales bit for bit, incl. an all-zero channel and bf16 / bf16 quotients that are exact ties."""
+  scales bit for bit, incl. an all-zero channel and bf16 / bf16 quotients that are exact ties.  The shapes reach both
+  routes: a channel that fits one block's registers (one pass) and, with 36 experts of 4096 values sharing a scale, one
+  that does not (two passes)."""
   g = torch.Generator().manual_seed(41)
-  G, N, Kd = 3, 72, 264
   w = (torch.randn(G, N, Kd, generator=g) * 0.05).to(torch.bfloat16)
   w[:, 5] = 0.0
   w[1, 9] = 0.0
