@@ -231,6 +231,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_absmax_kernel(const uint4
   if (i >= nvec) return;
   const int m0 = blockIdx.y * kColBand, m1 = min(m0 + kColBand, M);
   uint32_t mx[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+#pragma unroll 8
   for (int m = m0; m < m1; m++) {
     const uint4 x = dout[(size_t)m * nvec + i];
     const uint32_t w[4] = {x.x, x.y, x.z, x.w};
@@ -263,6 +264,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4*
   E5m2Scale s[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) s[e] = e5m2_prepare(colmax[i * 8 + e]);
+#pragma unroll 4
   for (int m = m0; m < m1; m++) {
     const uint4 x = dout[(size_t)m * nvec + i];
     const uint32_t w[4] = {x.x, x.y, x.z, x.w};
