@@ -172,6 +172,9 @@ def test_gmm_fp8_weights_read_as_gkn(K, lhs_dtype):
     assert torch.equal(got, ref)
   want = O.gmm(d.float(), w_nk.float(), gs, lhs_scale=s_row, transpose_rhs=True, out_dtype=torch.float32)
   assert relerr(got / cuda(fac)[:, None], want) <= 1e-4
+  # bf16 results (the paired 16-byte stores), as the backward asks for them
+  kw16 = dict(kw, out_dtype=torch.bfloat16)
+  assert torch.equal(K.gmm_raw(cuda(d), cuda(w_kn), cuda(gs), rhs_kn=True, **kw16), K.gmm_raw(cuda(d), cuda(w_nk), cuda(gs), **kw16))
   # a window of two local groups
   ref = K.gmm_raw(cuda(d), cuda(w_nk[2:4]), cuda(gs), group_offset=2, **kw)
   got = K.gmm_raw(cuda(d), cuda(w_kn[2:4]), cuda(gs), group_offset=2, rhs_kn=True, **kw)
