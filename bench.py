@@ -36,6 +36,7 @@ PROFILE_OF = {
     "c4": ("profiles/gmm_dlw_kernel_int8w_qwen3_prefill_c4.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c5": ("profiles/gmm_dlw_kernel_int4w_gptoss_prefill_c5_t4096.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c2_train": ("profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md", ["moe_tgmm.hip", "moe_common.h"]),
+    "c2_train_fp8_full": ("profiles/fp8_full_train_step_mixtral_shape.md", ["moe_tgmm.hip", "moe_common.h"]),
 }
 
 
@@ -321,11 +322,16 @@ def train_main(args):
     stage_ms[name] = sum(ts) / len(ts)
   m = t * k
   # weight gradient of wi_0 / wi_1: [E, f, d] from x [M, d] and d h [M, f] (the quantised backward records its own names)
-  dom = f"tgmm_k{d}_n{f}" if args.quant == "none" else f"tgmm_q_k{d}_n{f}"
+  # of the quantised backward the launch alone, on the MFMA rate of the operands it multiplies
+  dom, dom_kernel, dom_peak = f"tgmm_k{d}_n{f}", "tgmm_dl_kernel", PEAK_TFLOPS["bf16"]
+  if args.quant != "none":
+    dom = f"tgmm_kernel_k{d}_n{f}"
+    if f"tgmm_f8_kernel_k{d}_n{f}" in stage_ms:
+      dom, dom_kernel, dom_peak = f"tgmm_f8_kernel_k{d}_n{f}", "tgmm_f8_kernel", PEAK_TFLOPS["fp8"]
   dom_ms = stage_ms[dom]
   achieved = 2.0 * m * d * f / (dom_ms * 1e-3) / 1e12
   flops = 18.0 * m * d * f
-  traffic, traffic_source = measured_traffic(wl.name + "_train") if args.tokens is None else (None, None)
+  traffic, traffic_source = measured_traffic(wl.name + "_train" + ("_fp8_full" if args.quant == "fp8_full" else "")) if args.tokens is None else (None, None)
   result = {
       "metric": "moe_bf16_layer_fwd_bwd_tflops", "value": flops / (elapsed / args.steps) / 1e12, "unit": "TFLOP/s",
       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps,
@@ -334,9 +340,9 @@ def train_main(args):
                              f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU"
                              + ("" if args.quant == "none" else f", grouped matmuls quantised ({args.quant}, {args.calibration})"),
                  "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
-      "roofline": dict(bound="mfma", achieved=achieved, peak=PEAK_TFLOPS["bf16"], unit="TFLOP/s", frac=achieved / PEAK_TFLOPS["bf16"],
+      "roofline": dict(bound="mfma", achieved=achieved, peak=dom_peak, unit="TFLOP/s", frac=achieved / dom_peak,
                        traffic=traffic, traffic_source=traffic_source,
-                       kernel="tgmm_dl_kernel (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
+                       kernel=dom_kernel + " (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
       "stage_ms": stage_ms,
   }
   result["calibration"] = calibration("bf16")
@@ -460,7 +466,7 @@ def run_workload(args, name, tokens=None):
 def main():
   args = parse()
   if args.source_hash:
-    key = (args.workload or "c2") + ("_train" if args.train else "")
+    key = (args.workload or "c2") + ("_train" if args.train else "") + ("_fp8_full" if args.train and args.quant == "fp8_full" else "")
     print(kernel_source_hash(PROFILE_OF[key][1]))
     return
   if args.gpus != 1:

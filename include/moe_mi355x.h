@@ -562,13 +562,17 @@ MOE_API int moe_add_group_bias(const void* h, int M, int N, const float* bias, c
  *                     scale_out [M]
  *   MOE_BWD_FOR_DRHS  d[m, n] = bf16(dout[m, n] * bf16(factor[m]));  factor = lhs scales [M] f32; quantised per column:
  *                     scale_out [N] (group_sizes is not used)
+ *   MOE_BWD_PER_TENSOR  d[m, n] = bf16(dout[m, n] * bf16(factor[0]));  factor = the one scale [1] f32 of a tensor quantised
+ *                     with channelwise_axes=[] (disable_channelwise_axes, ops.py:568, :594, :601), either operand's; one
+ *                     scale for the whole gradient: scale_out [N], every entry holding that scale (the buffer carries the
+ *                     column maxima on the way; group_sizes is not used)
  *
  *   dout [M, N] bf16;  out [M, N] bf16: d itself (quantize == 0; scale_out is not touched), or d / scale on the e5m2
  *   grid, whose values are exact in bf16 (quantize == 1), so that moe_gmm / moe_tgmm take it as a bf16 operand;
  *   quantize == 2: out [M, N] holds the same values as float8_e5m2 bytes, the MOE_FP8_E5M2 lhs of moe_gmm.
  * Limits: N % 8 == 0, N <= 16384, at most 1024 groups.
  */
-typedef enum { MOE_BWD_FOR_DLHS = 0, MOE_BWD_FOR_DRHS = 1 } moe_bwd_mode;
+typedef enum { MOE_BWD_FOR_DLHS = 0, MOE_BWD_FOR_DRHS = 1, MOE_BWD_PER_TENSOR = 2 } moe_bwd_mode;
 MOE_API int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, const float* factor,
                                const int32_t* group_sizes, int num_groups_total, int num_groups_local, int group_offset,
                                void* out, float* scale_out, void* stream);

@@ -164,7 +164,7 @@ __device__ __forceinline__ void block_group_ends(const int* __restrict__ group_s
 template <bool BY_CHANNEL, bool ROW_QUANT, bool BYTES = false>
 __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4* dout, int N, const float* factor, const int* group_sizes,
                                                                      int G_total, int G_local, int group_offset, void* out,
-                                                                     float* scale_out) {
+                                                                     float* scale_out, int factor_stride = 1) {
   __shared__ int ends[BY_CHANNEL ? kBwdMaxGroups : 1];
   __shared__ uint32_t wmax[kBwdThreads / kWave];
   const int m = blockIdx.x, tid = threadIdx.x;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4
     block_group_ends(group_sizes, G_total, ends);
     f = factor + (size_t)local_group_of(ends, G_total, m, group_offset, G_local) * N;
   } else {
-    row_f = round_bf16_fn(factor[m]);
+    row_f = round_bf16_fn(factor[(size_t)m * factor_stride]);  // (stride 0: one factor for the tensor)
   }
   const int nvec = N / 8;
   float v[kBwdMaxChunks][8];
@@ -225,7 +225,8 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_scale_rows_kernel(const uint4
 // bands meet in an atomic max on the bit patterns (non-negative floats order like integers; a NaN's pattern is larger
 // than every number's and so survives, as it does in the reference's amax).
 constexpr int kColBand = 64;
-__global__ __launch_bounds__(kBwdThreads) void bwd_col_absmax_kernel(const uint4* dout, int M, int N, const float* lhs_scale, uint32_t* colmax) {
+__global__ __launch_bounds__(kBwdThreads) void bwd_col_absmax_kernel(const uint4* dout, int M, int N, const float* lhs_scale, int scale_stride,
+                                                                     uint32_t* colmax) {
   const int nvec = N / 8;
   const int i = blockIdx.x * kBwdThreads + threadIdx.x;
   if (i >= nvec) return;
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_absmax_kernel(const uint4
   for (int m = m0; m < m1; m++) {
     const uint4 x = dout[(size_t)m * nvec + i];
     const uint32_t w[4] = {x.x, x.y, x.z, x.w};
-    const float fm = round_bf16_fn(lhs_scale[m]);
+    const float fm = round_bf16_fn(lhs_scale[(size_t)m * scale_stride]);
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
       float d0, d1;
@@ -256,7 +257,8 @@ __global__ void bwd_clear_kernel(uint32_t* p, int n) {
 
 // d on the e5m2 grid of its column's scale; `colmax` still holds the maxima
 template <bool BYTES>
-__global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4* dout, int M, int N, const float* lhs_scale, const float* colmax, void* out) {
+__global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4* dout, int M, int N, const float* lhs_scale, int scale_stride,
+                                                                    const float* colmax, void* out) {
   const int nvec = N / 8;
   const int i = blockIdx.x * kBwdThreads + threadIdx.x;
   if (i >= nvec) return;
@@ -268,7 +270,7 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4*
   for (int m = m0; m < m1; m++) {
     const uint4 x = dout[(size_t)m * nvec + i];
     const uint32_t w[4] = {x.x, x.y, x.z, x.w};
-    const float fm = round_bf16_fn(lhs_scale[m]);
+    const float fm = round_bf16_fn(lhs_scale[(size_t)m * scale_stride]);
     uint32_t pk[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -278,6 +280,20 @@ __global__ __launch_bounds__(kBwdThreads) void bwd_col_quant_kernel(const uint4*
     }
     store8_e5m2<BYTES>(out, (size_t)m * nvec + i, pk);
   }
+}
+
+// Per-tensor quantisation: every column's maximum becomes the maximum of them all (one block; the patterns order like the
+// values and a NaN's beats every number's, as above).
+__global__ __launch_bounds__(kBwdThreads) void bwd_col_merge_kernel(uint32_t* colmax, int n) {
+  __shared__ uint32_t wmax[kBwdThreads / kWave];
+  uint32_t mx = 0u;
+  for (int i = threadIdx.x; i < n; i += kBwdThreads) mx = max(mx, colmax[i]);
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, kWave));
+  if (threadIdx.x % kWave == 0) wmax[threadIdx.x / kWave] = mx;
+  __syncthreads();
+  mx = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+  for (int i = threadIdx.x; i < n; i += kBwdThreads) colmax[i] = mx;
 }
 
 __global__ void bwd_col_scale_kernel(float* colmax, int n) {
@@ -325,7 +341,7 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
                        int num_groups_total, int num_groups_local, int group_offset, void* out, float* scale_out, void* stream) {
   if (!dout || !factor || !out) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: NULL pointer");
   if (M < 0 || N <= 0) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad sizes");
-  if (mode != MOE_BWD_FOR_DLHS && mode != MOE_BWD_FOR_DRHS) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad mode %d", mode);
+  if (mode != MOE_BWD_FOR_DLHS && mode != MOE_BWD_FOR_DRHS && mode != MOE_BWD_PER_TENSOR) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: bad mode %d", mode);
   if (quantize < 0 || quantize > 2) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: quantize must be 0, 1 (e5m2 values as bf16) or 2 (float8_e5m2 bytes)");
   if (quantize && !scale_out) return fail(MOE_ERR_INVALID_ARG, "bwd_scale_grad: the quantised gradient needs a scale buffer");
   const bool bytes = quantize == 2;
@@ -344,8 +360,11 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
       bwd_scale_rows_kernel<true, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, group_sizes, num_groups_total, num_groups_local, group_offset, out, scale_out);
     return check_launch("bwd_scale_rows_kernel");
   }
+  // per tensor: one factor for every row, and the columns' maxima merged into one before they are used
+  const bool tensor = mode == MOE_BWD_PER_TENSOR;
+  const int fstride = tensor ? 0 : 1;
   if (!quantize) {
-    bwd_scale_rows_kernel<false, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, nullptr, 0, 0, 0, out, scale_out);
+    bwd_scale_rows_kernel<false, false><<<M, kBwdThreads, 0, s>>>(x, N, factor, nullptr, 0, 0, 0, out, scale_out, fstride);
     return check_launch("bwd_scale_rows_kernel");
   }
   // per column: clear the maxima, take them, quantise with them, turn them into the scales
@@ -353,9 +372,10 @@ int moe_bwd_scale_grad(const void* dout, int M, int N, int mode, int quantize, c
   const dim3 grid(cdiv(nvec, kBwdThreads), cdiv(M, kColBand));
   if (grid.y > 65535) return fail(MOE_ERR_UNSUPPORTED, "bwd_scale_grad: too many rows (%d)", M);
   bwd_clear_kernel<<<cdiv(N, 256), 256, 0, s>>>((uint32_t*)scale_out, N);
-  bwd_col_absmax_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, (uint32_t*)scale_out);
-  if (bytes) bwd_col_quant_kernel<true><<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, out);
-  else bwd_col_quant_kernel<false><<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, scale_out, out);
+  bwd_col_absmax_kernel<<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, fstride, (uint32_t*)scale_out);
+  if (tensor) bwd_col_merge_kernel<<<1, kBwdThreads, 0, s>>>((uint32_t*)scale_out, N);
+  if (bytes) bwd_col_quant_kernel<true><<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, fstride, scale_out, out);
+  else bwd_col_quant_kernel<false><<<grid, kBwdThreads, 0, s>>>(x, M, N, factor, fstride, scale_out, out);
   bwd_col_scale_kernel<<<cdiv(N, 256), 256, 0, s>>>(scale_out, N);
   return check_launch("bwd_col_quant_kernel");
 }

@@ -368,13 +368,15 @@ def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups
 
   mode "dlhs": factor = rhs scales [g_local, n] f32, picked per row by its expert (group_sizes); quantised per row.
   mode "drhs": factor = lhs scales [m] f32; quantised per column.
+  mode "tensor": factor = the one scale [1] of an operand quantised per tensor (disable_channelwise_axes, ops.py:568-601);
+  one scale for the whole gradient, returned as [n] equal entries (a column scale like any other; [:1] is the scalar).
   -> (d [m, n] bf16, scale): the e5m2 values (exact in bf16) and their f32 scales ([m] or [n]), or (dout * factor, None).
   as_fp8 (with quantize): d is returned as a float8_e5m2 tensor instead, the lhs of gmm_raw against e4m3 weights.
   """
   _need(dout, "dout", torch.bfloat16, 2)
   _need(factor, "factor", torch.float32)
   m, n = dout.shape
-  code = {"dlhs": 0, "drhs": 1}[mode]
+  code = {"dlhs": 0, "drhs": 1, "tensor": 2}[mode]
   if code == 0:
     _need(group_sizes, "group_sizes", torch.int32, 1)
     g_local = int(num_groups_local if num_groups_local is not None else factor.shape[0])
@@ -382,8 +384,8 @@ def bwd_scale_grad(dout, factor, *, mode, quantize, group_sizes=None, num_groups
       raise ValueError(f"factor must hold [{g_local}, {n}] scales, got {tuple(factor.shape)}")
     g_total = group_sizes.numel()
   else:
-    if factor.numel() != m:
-      raise ValueError(f"factor must hold one scale per row ({m}), got {tuple(factor.shape)}")
+    if factor.numel() != (m if code == 1 else 1):
+      raise ValueError(f"factor must hold one scale {'per row (%d)' % m if code == 1 else 'for the tensor'}, got {tuple(factor.shape)}")
     g_total, g_local = 0, 0
   if as_fp8 and not quantize:
     raise ValueError("as_fp8 needs quantize")

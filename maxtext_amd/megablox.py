@@ -249,8 +249,6 @@ def gmm(
   if needs_grad:
     if use_gmm_v2:
       raise NotImplementedError("the differentiable path takes the v1 quantisation of ops.py:232-267")
-    if rule is not None and rule.disable_channelwise_axes:
-      raise NotImplementedError("dynamic per-tensor scales (disable_channelwise_axes) are not implemented")
     if rule is not None and (rule.bwd_calibration_method or "absmax") != "absmax":
       raise NotImplementedError("the gradient is quantised with absmax calibration")
     if existing_out is not None and existing_out.dtype != torch.bfloat16:
@@ -420,8 +418,11 @@ class _GmmFn(torch.autograd.Function):
     ctx.has_idx, ctx.has_inv = row_idx is not None, row_inv is not None
     with torch.no_grad():
       if ctx.quantized:
-        lq = quantize_lhs(lhs.contiguous(), lhs_q, calibration_method=rule.act_calibration_method)
-        rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q, calibration_method=rule.weight_calibration_method, manual=manual)
+        # disable_channelwise_axes: one dynamic scale per tensor (channelwise_axes=[], ops.py:245, :258), for the gradients too
+        ctx.per_tensor = bool(rule.disable_channelwise_axes)
+        lq = quantize_lhs(lhs.contiguous(), lhs_q, calibration_method=rule.act_calibration_method, per_tensor=ctx.per_tensor)
+        rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q, calibration_method=rule.weight_calibration_method, manual=manual,
+                          per_tensor=ctx.per_tensor)
         ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes, *idx_t)
         ctx.rhs_dtype = rhs.dtype
         return gmm(lq, rq, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=True, **extra)
@@ -451,6 +452,7 @@ class _GmmFn(torch.autograd.Function):
     fp8 = lq.dtype == torch.float8_e4m3fn
     dlhs = drhs = None
     quant = ctx.bwd_q is not None
+    per_tensor = getattr(ctx, "per_tensor", False)
     ev = PROFILE_EVENTS
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(3)] if ev is not None else None
     if marks:
@@ -464,8 +466,14 @@ class _GmmFn(torch.autograd.Function):
       # stream kernel reads them as they are; the other routes take a re-laid-out copy [g, k, n]
       as_kn = as_fp8 and kernels.gmm_fp8_rhs_kn_supported(m, n, k, group_sizes.numel())
       w_t = None if as_kn else kernels.transpose_rhs(rq)
-      d, s_row = kernels.bwd_scale_grad(dout, rs_gn, mode="dlhs", quantize=quant, group_sizes=group_sizes, num_groups_local=g_local,
-                                        group_offset=ctx.offset, as_fp8=as_fp8)
+      if per_tensor:
+        # one weight scale and ONE scale for the whole gradient (channelwise_axes=[], ops.py:594): it comes back as a
+        # vector of equal entries, of which the products take the first (fp8 route) or one per row
+        d, s_all = kernels.bwd_scale_grad(dout, rs.reshape(-1)[:1].contiguous(), mode="tensor", quantize=quant, as_fp8=as_fp8)
+        s_row = None if s_all is None else s_all[:1].expand(m).contiguous()
+      else:
+        d, s_row = kernels.bwd_scale_grad(dout, rs_gn, mode="dlhs", quantize=quant, group_sizes=group_sizes, num_groups_local=g_local,
+                                          group_offset=ctx.offset, as_fp8=as_fp8)
       one = torch.ones((1,), dtype=torch.float32, device=dout.device)
       if as_fp8:
         # e5m2 x e4m3 on the fp8 MFMA; the rows' scales are the activations' epilogue scales
@@ -493,15 +501,24 @@ class _GmmFn(torch.autograd.Function):
       ls_m = ls if ls.numel() == m else ls.reshape(1).expand(m).contiguous()
       # fp8 residuals and an e5m2 gradient multiply as they are stored on shapes the fp8 weight-gradient kernel takes
       bytes_in = fp8 and quant and kernels.tgmm_fp8_supported(m, k, n, group_sizes.numel(), g_local)
-      d, s_col = kernels.bwd_scale_grad(dout, ls_m, mode="drhs", quantize=quant, as_fp8=bytes_in)
+      if per_tensor:  # (ops.py:568, :601: one activation scale, one gradient scale; [n] equal entries serve as column scales)
+        d, s_col = kernels.bwd_scale_grad(dout, ls.reshape(-1)[:1].contiguous(), mode="tensor", quantize=quant, as_fp8=bytes_in)
+      else:
+        d, s_col = kernels.bwd_scale_grad(dout, ls_m, mode="drhs", quantize=quant, as_fp8=bytes_in)
       # the column scales go back onto the f32 products in the kernel's epilogue, which rounds once to the weights' type
       direct = ctx.rhs_dtype in (torch.bfloat16, torch.float32)
+      if marks:  # the weight-gradient launch alone, beside the stage that includes its quantiser passes
+        marks += [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        marks[3].record()
       if bytes_in:
         w = kernels.tgmm_fp8(lq_rows.contiguous(), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
                              out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
       else:
         w = kernels.tgmm(lq_rows.to(torch.bfloat16), d, group_sizes, num_groups_local=g_local, group_offset=ctx.offset,
                          out_dtype=ctx.rhs_dtype if direct else torch.float32, out_row_scale=s_col)  # [g, n, k]
+      if marks:
+        marks[4].record()
+        ev.append((("tgmm_f8_kernel_" if bytes_in else "tgmm_kernel_") + f"k{k}_n{n}", marks[3], marks[4]))
       w = w.to(ctx.rhs_dtype)
       drhs = w if ctx.transpose_rhs else w.transpose(1, 2)
     if marks:

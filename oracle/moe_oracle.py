@@ -588,9 +588,10 @@ def tgmm(lhs: torch.Tensor, dout: torch.Tensor, group_sizes, *, num_actual_group
 E5M2_MAX = 57344.0  # largest finite float8_e5m2
 
 
-def quantize_e5m2(x: torch.Tensor, dim: int):
+def quantize_e5m2(x: torch.Tensor, dim):
   """Gradient quantiser of the backward pass (ops.py:583-604): symmetric absmax scale along `dim`
-  (channelwise_axes=[0] keeps one scale per row -> dim=1; [1] one per column -> dim=0), values cast to
+  (channelwise_axes=[0] keeps one scale per row -> dim=1; [1] one per column -> dim=0; [] one for the tensor, the
+  rule's disable_channelwise_axes -> dim=(0, 1)), values cast to
   float8_e5m2.  Returns (values as f32 on the e5m2 grid, scale f32 with `dim` kept).  Rounding mode and the
   zero-scale rule of qwix are not in the reference tree (see module docstring): round-to-nearest-even of the
   torch cast, zero scale -> zeros."""
@@ -601,7 +602,8 @@ def quantize_e5m2(x: torch.Tensor, dim: int):
 
 
 def gmm_bwd_quantized(grad: torch.Tensor, lhs_q: torch.Tensor, lhs_scale: torch.Tensor, rhs_q: torch.Tensor,
-                      rhs_scale: torch.Tensor, group_sizes, *, bwd_qtype: str | None = None, grad_dtype=torch.bfloat16):
+                      rhs_scale: torch.Tensor, group_sizes, *, bwd_qtype: str | None = None, grad_dtype=torch.bfloat16,
+                      per_tensor: bool = False):
   """Backward of a quantised gmm as the reference runs it (ops.py:438-527 with _bwd_prepare_inputs :530-580 and
   _bwd_quantize_gradient :583-604), for channelwise scales: lhs_q [m,k] with lhs_scale [m]; rhs_q [g,k,n] with
   rhs_scale [n] (shared, ops.py:250-260) or [g,n] (per expert).
@@ -610,6 +612,9 @@ def gmm_bwd_quantized(grad: torch.Tensor, lhs_q: torch.Tensor, lhs_scale: torch.
     drhs_dout = grad * lhs_scale[m]      (:575-578)
     both optionally quantised to e5m2, per row / per column (:590-603)
     dlhs = gmm(dlhs_dout, rhs_q^T)       (:612-642)      drhs = tgmm(lhs_q^T, drhs_dout)   (:766-796)
+
+  per_tensor: the rule's disable_channelwise_axes (channelwise_axes=[] at :568, :594, :601): lhs_scale and rhs_scale hold one
+  value each (any shape that broadcasts as given above), and each scaled gradient is quantised with ONE absmax scale.
 
   Scaled gradients are rounded to grad_dtype (the reference multiplies in grad.dtype).  Returns (dlhs [m,k] f64,
   drhs [g,k,n] f64)."""
@@ -625,8 +630,8 @@ def gmm_bwd_quantized(grad: torch.Tensor, lhs_q: torch.Tensor, lhs_scale: torch.
   s_col = torch.ones((1, n))
   if bwd_qtype is not None:
     assert bwd_qtype in ("e5m2", "float8_e5m2")
-    dlhs_dout, s_row = quantize_e5m2(dlhs_dout, dim=1)
-    drhs_dout, s_col = quantize_e5m2(drhs_dout, dim=0)
+    dlhs_dout, s_row = quantize_e5m2(dlhs_dout, dim=(0, 1) if per_tensor else 1)
+    drhs_dout, s_col = quantize_e5m2(drhs_dout, dim=(0, 1) if per_tensor else 0)
   dlhs = gmm(dlhs_dout, rhs_q.to(torch.float32).transpose(1, 2), group_sizes, out_dtype=torch.float64) * s_row.double()
   drhs = tgmm(lhs_q.to(torch.float32), drhs_dout, group_sizes, out_dtype=torch.float64) * s_col.double()[None]
   return dlhs, drhs

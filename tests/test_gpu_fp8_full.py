@@ -344,6 +344,50 @@ def test_gmm_quantized_backward_fwd_dtypes_and_calibrations(shape, calibration, 
   assert torch.all(rhs_g.grad[1] == 0)
 
 
+@pytest.mark.parametrize("bwd_q", [None, "float8_e5m2"], ids=["bf16grad", "e5m2grad"])
+@pytest.mark.parametrize("fwd", ["int8", "float8_e4m3fn"], ids=["int8", "fp8"])
+@pytest.mark.parametrize("shape", [dict(m=450, k=256, n=192, gs=[200, 0, 70, 150]), dict(m=1100, k=512, n=768, gs=[500, 0, 300, 260])],
+                         ids=["small", "stream"])
+def test_gmm_quantized_backward_per_tensor_scales(shape, fwd, bwd_q):
+  """A rule with disable_channelwise_axes (channelwise_axes=[] at ops.py:245, :258, :568, :594, :601): one dynamic absmax
+  scale for the activations, one for the weights and one for each of the two scaled gradients.  Forward operands bit for
+  bit against the host statement of the rule, output and both gradients against the oracle's quantised backward."""
+  from maxtext_amd import megablox
+  from maxtext_amd.quantizations import QtRule
+
+  m, k, n, gs = shape["m"], shape["k"], shape["n"], np.asarray(shape["gs"], np.int32)
+  g = torch.Generator().manual_seed(13)
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w = (torch.randn(4, k, n, generator=g) * 0.05).to(torch.bfloat16)  # [g, k, n]
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  rule = QtRule(weight_qtype=fwd, act_qtype=fwd, bwd_qtype=bwd_q, disable_channelwise_axes=True)
+  lhs_g = cuda(lhs).requires_grad_()
+  rhs_g = cuda(w).requires_grad_()
+  out = gmm_bf16(lhs_g, rhs_g, cuda(gs), use_qwix_quantization=True, qwix_rule=rule)
+  qdt = torch.int8 if fwd == "int8" else E4M3
+  qmax = 127.0 if fwd == "int8" else 448.0
+  ls = lhs.float().abs().max() / qmax
+  rs = w.float().abs().max() / qmax
+  cast = (lambda y: torch.round(y).clamp(-qmax, qmax).to(qdt)) if fwd == "int8" else (lambda y: y.clamp(-qmax, qmax).to(qdt))
+  lq, rq = cast(lhs.float() / ls), cast(w.float() / rs)
+  dev_l = megablox.quantize_lhs(cuda(lhs), fwd, per_tensor=True)
+  dev_r = megablox.quantize_rhs(cuda(w.transpose(1, 2).contiguous()), fwd, per_tensor=True)
+  assert torch.equal(dev_l.scale.cpu().reshape(()), ls) and torch.equal(dev_l.qvalue.cpu().float(), lq.float())
+  assert torch.equal(dev_r.scale.cpu().reshape(()), rs) and torch.equal(dev_r.qvalue.cpu().transpose(1, 2).float(), rq.float())
+  ls_m, rs_n = ls.expand(m).contiguous(), rs.expand(n).contiguous()
+  want_out = O.gmm(lq.float(), rq.float(), gs, lhs_scale=ls_m, rhs_scale=rs_n[None])
+  assert relerr(out, want_out) <= TOL
+  want_dl, want_dr = O.gmm_bwd_quantized(dout, lq.float(), ls_m, rq.float(), rs_n, gs, bwd_qtype=None if bwd_q is None else "e5m2",
+                                         per_tensor=True)
+  out.backward(cuda(dout))
+  tol = TOL if bwd_q is None else 2e-2  # a gradient value next to an e5m2 rounding boundary may land on either side
+  total = int(gs.sum())
+  assert relerr(lhs_g.grad, want_dl, atol_rms=ELEM_ATOL_RMS_CHAINED) <= tol
+  assert torch.all(lhs_g.grad[total:] == 0)
+  assert rhs_g.grad.shape == want_dr.shape and relerr(rhs_g.grad, want_dr, atol_rms=ELEM_ATOL_RMS_CHAINED) <= tol
+  assert torch.all(rhs_g.grad[1] == 0)
+
+
 def test_fp8_full_layer_gradients_tokamax_configuration():
   """The configuration of the reference's fp8_full training smoke test (tests/integration/tokamax_test.py:53-114:
   emb 256, moe_mlp 256, 2 experts + 1 shared, weights and activations "fixed,-224,224", gradients absmax e5m2): one

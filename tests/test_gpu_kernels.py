@@ -1564,6 +1564,34 @@ def test_bwd_scale_grad_bit_exact(K, n, quantize):
   assert float(s_r[17]) == 0.0 and torch.all(got_r[17] == 0) and float(s_c[11]) == 0.0
 
 
+@pytest.mark.parametrize("as_fp8", [False, True])
+@pytest.mark.parametrize("n", [192, 2056])
+def test_bwd_scale_grad_per_tensor_bit_exact(K, n, as_fp8):
+  """disable_channelwise_axes in the backward (ops.py:568, :594, :601: channelwise_axes=[]): the gradient times the one
+  scale of an operand quantised per tensor, then ONE absmax scale for the whole gradient; values and scale bit for bit
+  against the oracle's e5m2 quantiser over both axes, as bf16 values and as float8_e5m2 bytes; a NaN-free all-zero
+  gradient gives scale 0 and zeros."""
+  g = torch.Generator().manual_seed(33)
+  m = 333
+  dout = (torch.randn(m, n, generator=g) * torch.rand(m, 1, generator=g) * 8).to(torch.bfloat16)
+  dout[17] = 0.0
+  dout[:, 11] = 0.0
+  f = torch.tensor([0.0173])
+  d = dout * f.to(torch.bfloat16)
+  plain, none = K.bwd_scale_grad(cuda(dout), cuda(f), mode="tensor", quantize=False)
+  assert none is None and torch.equal(plain.cpu(), d)
+  want, want_s = O.quantize_e5m2(d, dim=(0, 1))
+  got, s = K.bwd_scale_grad(cuda(dout), cuda(f), mode="tensor", quantize=True, as_fp8=as_fp8)
+  assert got.dtype == (torch.float8_e5m2 if as_fp8 else torch.bfloat16)
+  assert tuple(s.shape) == (n,) and torch.all(s.cpu() == want_s.reshape(())) and float(want_s) == float(np.float32(float(d.float().abs().max())) / np.float32(57344.0))
+  assert torch.equal(got.cpu().float(), want)
+  assert float(got.float().abs().max()) == 57344.0  # the tensor's largest value sits on the format's largest
+  zero, s0 = K.bwd_scale_grad(cuda(torch.zeros_like(dout)), cuda(f), mode="tensor", quantize=True, as_fp8=as_fp8)
+  assert torch.all(s0 == 0) and torch.all(zero.float() == 0)
+  with pytest.raises(ValueError):
+    K.bwd_scale_grad(cuda(dout), cuda(torch.ones(m)), mode="tensor", quantize=True)
+
+
 def test_gmm_autograd_with_expert_bias():
   """Per-expert mlp_bias on the differentiable path (moe.py:1952-1957): forward equals the epilogue bias of the
   inference path; gradients of lhs, both weights and both biases against torch autograd in f64."""

@@ -507,6 +507,36 @@ def test_quantized_backward_equals_autograd_through_dequantised_operands():
   assert float((dlq - dl).abs().max() / dl.abs().max()) <= 0.1 and float((drq - dr).abs().max() / dr.abs().max()) <= 0.1
 
 
+def test_quantized_backward_with_per_tensor_scales():
+  """ops.py:568-601 with disable_channelwise_axes: scalar operand scales and one e5m2 scale per gradient.  Without
+  gradient quantisation the result is the channelwise backward on constant scale vectors (the same algebra); with it, a
+  hand case: the tensor's largest magnitude lands on 57344, a value at a quarter of it on 14336, and one scale serves
+  rows whose own maxima differ by 2^10 (per row each would reach 57344)."""
+  g = torch.Generator().manual_seed(6)
+  m, k, n, gs = 30, 8, 16, [10, 0, 20]
+  lhs_q = torch.randint(-127, 128, (m, k), generator=g).to(torch.int8)
+  rhs_q = torch.randint(-127, 128, (3, k, n), generator=g).to(torch.int8)
+  ls, rs = torch.full((m,), 0.75), torch.full((n,), 1.5)
+  grad = torch.randn(m, n, generator=g)
+  a = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs, gs, grad_dtype=torch.float64, per_tensor=True)
+  b = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs, gs, grad_dtype=torch.float64)
+  assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+  x = torch.tensor([[8.0, -2.0, 0.5], [2.0**-7, 2.0**-8, 0.0]])
+  q, s = O.quantize_e5m2(x, dim=(0, 1))
+  assert tuple(s.shape) == (1, 1) and float(s) == float(np.float32(8.0) / np.float32(57344.0))
+  np.testing.assert_array_equal(q.numpy(), [[57344.0, -14336.0, 3584.0], [56.0, 28.0, 0.0]])
+  q_row, s_row = O.quantize_e5m2(x, dim=1)
+  assert float(q_row[1, 0]) == 57344.0 and float(s_row[1, 0]) == float(np.float32(2.0**-7) / np.float32(57344.0))
+  # the quantised backward with ONE scale equals the products of the dequantised gradients
+  dlq, drq = O.gmm_bwd_quantized(grad, lhs_q, ls, rhs_q, rs, gs, bwd_qtype="e5m2", grad_dtype=torch.float64, per_tensor=True)
+  q1, s1 = O.quantize_e5m2(grad * 1.5, dim=(0, 1))
+  q2, s2 = O.quantize_e5m2(grad * 0.75, dim=(0, 1))
+  want_dl = O.gmm(q1 * s1, rhs_q.float().transpose(1, 2), gs, out_dtype=torch.float64)
+  want_dr = O.tgmm(lhs_q.float(), q2 * s2, gs, out_dtype=torch.float64)
+  assert float((dlq - want_dl).abs().max()) <= 1e-3 * float(want_dl.abs().max())
+  assert float((drq - want_dr).abs().max()) <= 1e-3 * float(want_dr.abs().max())
+
+
 def test_hash_routing_is_a_table_lookup():
   """moe.py:729-738: a hand case (two tokens, k = 2) and the invariants of the scaling (moe.py:767-773)."""
   scores = np.array([[0.1, 0.2, 0.3, 0.4], [0.4, 0.3, 0.2, 0.1]], np.float32)
