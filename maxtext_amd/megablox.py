@@ -247,14 +247,13 @@ def gmm(
   needs_grad = needs_grad or (torch.is_grad_enabled() and any(
       isinstance(t, torch.Tensor) and t.requires_grad for t in (partial_sum, partial_sum_up, existing_out, out_row_scale)))
   if needs_grad:
-    if use_gmm_v2:
-      raise NotImplementedError("the differentiable path takes the v1 quantisation of ops.py:232-267")
     if rule is not None and (rule.bwd_calibration_method or "absmax") != "absmax":
       raise NotImplementedError("the gradient is quantised with absmax calibration")
     if existing_out is not None and existing_out.dtype != torch.bfloat16:
       raise NotImplementedError("existing_out is bfloat16 on the differentiable path")
     out = _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, use_manual_quantization, fuse_act, act_limit,
-                         rhs_bias, rhs_up_bias, partial_sum, partial_sum_up, existing_out, lhs_row_idx, lhs_row_idx_div, lhs_row_inv)
+                         rhs_bias, rhs_up_bias, partial_sum, partial_sum_up, existing_out, lhs_row_idx, lhs_row_idx_div, lhs_row_inv,
+                         v2=bool(use_gmm_v2))
     if out_row_scale is not None:
       # the routing weights between the activation and wo (models/deepseek_batchsplit_fp8.py:1048-1049): the finished
       # bf16 result times the row's factor, rounded again; autograd gives both gradients
@@ -392,12 +391,15 @@ class _GmmFn(torch.autograd.Function):
 
   @staticmethod
   def forward(ctx, lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual, partial_sum=None, existing_out=None, row_idx=None, row_div=1,
-              row_inv=None):
+              row_inv=None, v2=False):
     """partial_sum [m, n] is added to the product, existing_out [m, n] receives the rows of the local groups (both get
     the incoming gradient as theirs, ops.py:524-527); row_idx / row_div: row i of the product reads lhs row
     row_idx[i] // row_div (the fused permute: lhs holds the T token rows and no [m, k] copy is kept for the backward),
     row_inv: the inverse permutation of row_idx when it is one (the gradient of lhs is then a deterministic sum over each
-    token's row_div copies instead of an atomic scatter)."""
+    token's row_div copies instead of an atomic scatter).
+    v2 (use_gmm_v2): the forward leaves the activations to the product, which quantises them itself per row and 512 values
+    of K or with the static (1, 1) scale (ops.py:241, :333-360); the residual is the bf16 lhs, which the backward quantises
+    per row by the v1 rule before it proceeds as above (_bwd_prepare_inputs, ops.py:561-572)."""
     lhs_q, rhs_q = (rule.act_qtype, rule.weight_qtype) if rule is not None else (None, None)
     bwd_q = rule.bwd_qtype if rule is not None else None
     ctx.offset, ctx.transpose_rhs, ctx.bwd_q = offset, transpose_rhs, bwd_q
@@ -420,16 +422,21 @@ class _GmmFn(torch.autograd.Function):
       if ctx.quantized:
         # disable_channelwise_axes: one dynamic scale per tensor (channelwise_axes=[], ops.py:245, :258), for the gradients too
         ctx.per_tensor = bool(rule.disable_channelwise_axes)
-        lq = quantize_lhs(lhs.contiguous(), lhs_q, calibration_method=rule.act_calibration_method, per_tensor=ctx.per_tensor)
         rq = quantize_rhs(_native_rhs(rhs, transpose_rhs), rhs_q, calibration_method=rule.weight_calibration_method, manual=manual,
                           per_tensor=ctx.per_tensor)
-        ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes, *idx_t)
         ctx.rhs_dtype = rhs.dtype
+        ctx.v2_act = (lhs_q, rule.act_calibration_method) if v2 else None
+        if v2:
+          ctx.save_for_backward(lhs, none, rq.qvalue, rq.scale, group_sizes, *idx_t)
+          return gmm(lhs, rq, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=True, use_gmm_v2=True,
+                     use_qwix_quantization=True, qwix_rule=rule, **extra)
+        lq = quantize_lhs(lhs.contiguous(), lhs_q, calibration_method=rule.act_calibration_method, per_tensor=ctx.per_tensor)
+        ctx.save_for_backward(lq.qvalue, lq.scale, rq.qvalue, rq.scale, group_sizes, *idx_t)
         return gmm(lq, rq, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=True, **extra)
       ctx.save_for_backward(lhs, rhs, group_sizes, *idx_t)
       kw = {}
       if rule is not None:
-        kw = dict(use_qwix_quantization=True, qwix_rule=rule, use_manual_quantization=manual)
+        kw = dict(use_qwix_quantization=True, qwix_rule=rule, use_manual_quantization=manual, use_gmm_v2=v2)
       return gmm(lhs, rhs, group_sizes, torch.bfloat16, group_offset=offset, transpose_rhs=transpose_rhs, **kw, **extra)
 
   @staticmethod
@@ -446,6 +453,11 @@ class _GmmFn(torch.autograd.Function):
   @staticmethod
   def _backward_quantized(ctx, dout):
     lq, ls, rq, rs, group_sizes, row_idx, row_inv = ctx.saved_tensors  # lq [m,k], ls [m] or [1]; rq [g,n,k], rs [g,n], [1,n] or [1]
+    if getattr(ctx, "v2_act", None) is not None:
+      # the residual is the bf16 activation: quantised here per row by the v1 rule (ops.py:561-572), not by the product's
+      # own K-block rule
+      q = quantize_lhs(lq.contiguous(), ctx.v2_act[0], calibration_method=ctx.v2_act[1], per_tensor=getattr(ctx, "per_tensor", False))
+      lq, ls = q.qvalue, q.scale
     m, n = dout.shape
     k = lq.shape[1]
     g_local = rq.shape[0]
@@ -533,7 +545,7 @@ class _GmmFn(torch.autograd.Function):
     g_in = dout
     dout = dout.to(torch.bfloat16).contiguous()
     # the gradients of partial_sum and existing_out are the incoming gradient itself (ops.py:524-527)
-    tail = (None, None, None, None, None, g_in if ctx.has_ps else None, g_in if ctx.has_eo else None, None, None, None)
+    tail = (None, None, None, None, None, g_in if ctx.has_ps else None, g_in if ctx.has_eo else None, None, None, None, None)
     if ctx.quantized:
       with torch.no_grad():
         dlhs, drhs = _GmmFn._backward_quantized(ctx, dout)
@@ -616,7 +628,7 @@ class _BiasFn(torch.autograd.Function):
 
 def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual, fuse_act, act_limit, rhs_bias=None,
                    rhs_up_bias=None, partial_sum=None, partial_sum_up=None, existing_out=None, lhs_row_idx=None, lhs_row_idx_div=1,
-                   lhs_row_inv=None):
+                   lhs_row_inv=None, v2=False):
   for name, t in (("lhs", lhs), ("rhs", rhs), ("rhs_up", rhs_up)):
     if t is not None and not isinstance(t, torch.Tensor):
       raise NotImplementedError(f"gradients need bf16 tensors; {name} is already quantised")
@@ -625,14 +637,14 @@ def _gmm_with_grad(lhs, rhs, rhs_up, group_sizes, offset, transpose_rhs, rule, m
   ps = None if partial_sum is None else partial_sum.to(torch.bfloat16).contiguous()
   ps_up = None if partial_sum_up is None else partial_sum_up.to(torch.bfloat16).contiguous()
   idx = (lhs_row_idx, lhs_row_idx_div, lhs_row_inv)
-  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual, ps, existing_out, *idx)
+  h0 = _GmmFn.apply(lhs, rhs, group_sizes, offset, transpose_rhs, rule, manual, ps, existing_out, *idx, v2)
   if rhs_bias is not None:
     h0 = _BiasFn.apply(h0, rhs_bias, group_sizes, offset)
   if rhs_up is None:
     if fuse_act is not None:
       raise ValueError("fuse_act needs rhs_up")
     return h0
-  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual, ps_up, None, *idx)
+  h1 = _GmmFn.apply(lhs, rhs_up, group_sizes, offset, transpose_rhs, rule, manual, ps_up, None, *idx, v2)
   if rhs_up_bias is not None:
     h1 = _BiasFn.apply(h1, rhs_up_bias, group_sizes, offset)
   if fuse_act is None:

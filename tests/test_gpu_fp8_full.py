@@ -388,6 +388,58 @@ def test_gmm_quantized_backward_per_tensor_scales(shape, fwd, bwd_q):
   assert torch.all(rhs_g.grad[1] == 0)
 
 
+@pytest.mark.parametrize("calibration", ["absmax", "fixed,-224,224"], ids=["absmax", "static"])
+@pytest.mark.parametrize("fwd", ["int8", "float8_e4m3fn"], ids=["int8", "fp8"])
+def test_gmm_v2_forward_and_its_quantized_backward(fwd, calibration):
+  """use_gmm_v2 on the differentiable path (ops.py:203-215, :241, :561-572, :636, :785): the forward leaves the bf16
+  activations to the product, which quantises them by its own rule (per row and 512 values of K, or the static (1, 1)
+  scale: the oracle's op-by-op restatement of pallas_mosaic_tpu_v2_gmm_kernel.py:489-542, bit-exact on the GPU in
+  test_gpu_layouts); the backward quantises the kept bf16 activations per row by the v1 rule and then runs the
+  reference's quantised backward with e5m2 gradients."""
+  from maxtext_amd import megablox
+  from maxtext_amd.quantizations import QtRule
+
+  if fwd == "int8" and calibration != "absmax":
+    calibration = "fixed,-4,4"
+  m, k, n, gs = 450, 1024, 192, np.asarray([200, 0, 70, 150], np.int32)
+  g = torch.Generator().manual_seed(14)
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  lhs[:, 512:] *= 0.125  # the two K blocks of a row get different scales
+  w = (torch.randn(4, k, n, generator=g) * (0.05 if calibration == "absmax" else 1.0)).to(torch.bfloat16)  # [g, k, n]
+  dout = torch.randn(m, n, generator=g).to(torch.bfloat16)
+  rule = QtRule(weight_qtype=fwd, act_qtype=fwd, bwd_qtype="float8_e5m2", weight_calibration_method=calibration,
+                act_calibration_method=calibration)
+  lhs_g = cuda(lhs).requires_grad_()
+  rhs_g = cuda(w).requires_grad_()
+  out = gmm_bf16(lhs_g, rhs_g, cuda(gs), use_qwix_quantization=True, qwix_rule=rule, use_gmm_v2=True)
+  qdt = torch.int8 if fwd == "int8" else E4M3
+  qmax = 127.0 if fwd == "int8" else 448.0
+  static = None if calibration == "absmax" else O.get_static_scale(qmax, calibration)
+  # weights: the library's quantiser (bit for bit against the host rule in the tests above)
+  dev_r = megablox.quantize_rhs(cuda(w.transpose(1, 2).contiguous()), fwd, calibration_method=calibration)
+  rq = dev_r.qvalue.cpu().transpose(1, 2)
+  rs = dev_r.scale.cpu().reshape(-1).expand(n).contiguous() if dev_r.scale.numel() == 1 else dev_r.scale.cpu().reshape(-1)
+  # forward: the product's own quantiser
+  lq2, ls2 = O.quantize_lhs_v2(lhs, qdt, quant_block=512, static_scale=static)
+  want_out = O.gmm(lq2, rq, gs, lhs_scale=ls2, rhs_scale=rs[None], quant_block=(512, k))
+  assert relerr(out, want_out) <= TOL
+  # backward: the v1 rule on the kept activations
+  dev_l = megablox.quantize_lhs(cuda(lhs), fwd, calibration_method=calibration)
+  lq = dev_l.qvalue.cpu()
+  ls = dev_l.scale.cpu().reshape(-1)
+  ls = ls.expand(m).contiguous() if ls.numel() == 1 else ls
+  if static is None:
+    assert torch.equal(ls, lhs.float().abs().amax(1) / qmax)
+    assert not torch.equal(lq.float(), lq2.float())  # (the two rules differ on these rows: the test tells them apart)
+  want_dl, want_dr = O.gmm_bwd_quantized(dout, lq.float(), ls, rq.float(), rs, gs, bwd_qtype="e5m2")
+  out.backward(cuda(dout))
+  total = int(gs.sum())
+  assert relerr(lhs_g.grad, want_dl, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
+  assert torch.all(lhs_g.grad[total:] == 0)
+  assert rhs_g.grad.shape == want_dr.shape and relerr(rhs_g.grad, want_dr, atol_rms=ELEM_ATOL_RMS_CHAINED) <= 2e-2
+  assert torch.all(rhs_g.grad[1] == 0)
+
+
 def test_fp8_full_layer_gradients_tokamax_configuration():
   """The configuration of the reference's fp8_full training smoke test (tests/integration/tokamax_test.py:53-114:
   emb 256, moe_mlp 256, 2 experts + 1 shared, weights and activations "fixed,-224,224", gradients absmax e5m2): one
