@@ -274,8 +274,19 @@ def train_cpu_baseline(wl, sample_tokens):
 
 
 def train_main(args):
+  result = train_result(args, args.quant, args.calibration, args.steps, args.warmup)
+  result["calibration"] = calibration("bf16")
+  if not args.no_cpu_baseline:
+    from maxtext_amd import synthetic
+
+    result["cpu_baseline"] = train_cpu_baseline(synthetic.workload(args.workload, args.tokens), args.cpu_sample_tokens or 1024)
+  print(json.dumps(result))
+
+
+def train_result(args, quant, calibration_method, steps, warmup):
   """Forward + backward of the routed layer with bf16 weights: 3 forward GEMMs, 3 input-gradient GEMMs
-  (moe_gmm on re-laid-out weights) and 3 weight-gradient launches (moe_tgmm) per step."""
+  (moe_gmm on re-laid-out weights) and 3 weight-gradient launches (moe_tgmm) per step; quant "fp8_full" / "int8": the
+  reference's quantised recipe for all nine products.  Returns the fields of the result line."""
   import torch
 
   from maxtext_amd import _lib, megablox, moe, synthetic
@@ -285,11 +296,11 @@ def train_main(args):
   wl = synthetic.workload(args.workload, args.tokens)
   import dataclasses
 
-  cfg = dataclasses.replace(wl.cfg, act_quant="int8" if args.quant == "int8" else None, shared_experts=0)
-  if args.quant == "fp8_full":
+  cfg = dataclasses.replace(wl.cfg, act_quant="int8" if quant == "int8" else None, shared_experts=0)
+  if quant == "fp8_full":
     cfg = dataclasses.replace(cfg, quantization="fp8_full", use_qwix_quantization=True,
-                              weight_quantization_calibration_method=args.calibration,
-                              act_quantization_calibration_method=args.calibration)
+                              weight_quantization_calibration_method=calibration_method,
+                              act_quantization_calibration_method=calibration_method)
   e, d, f, k, t = cfg.num_experts, cfg.emb_dim, cfg.moe_mlp_dim, cfg.num_experts_per_tok, wl.tokens
   g = torch.Generator(device="cuda").manual_seed(0)
   mk = lambda *shape: (torch.randn(*shape, device="cuda", generator=g) * 0.02).to(torch.bfloat16).requires_grad_()
@@ -306,12 +317,12 @@ def train_main(args):
     out = block.sparse_matmul(x, logits, pre, w0, w1, wo)[0]
     out.backward(dout)
 
-  for _ in range(args.warmup):
+  for _ in range(warmup):
     step()
   torch.cuda.synchronize()
   megablox.PROFILE_EVENTS = []
   t0 = time.perf_counter()
-  for _ in range(args.steps):
+  for _ in range(steps):
     step()
   torch.cuda.synchronize()
   elapsed = time.perf_counter() - t0
@@ -321,34 +332,33 @@ def train_main(args):
     ts = [a.elapsed_time(b) for n, a, b in events if n == name]
     stage_ms[name] = sum(ts) / len(ts)
   m = t * k
-  # weight gradient of wi_0 / wi_1: [E, f, d] from x [M, d] and d h [M, f] (the quantised backward records its own names)
-  # of the quantised backward the launch alone, on the MFMA rate of the operands it multiplies
+  # weight gradient of wi_0 / wi_1: [E, f, d] from x [M, d] and d h [M, f]; of the quantised backward the launch alone (it
+  # records its own names), on the MFMA rate of the operands it multiplies
   dom, dom_kernel, dom_peak = f"tgmm_k{d}_n{f}", "tgmm_dl_kernel", PEAK_TFLOPS["bf16"]
-  if args.quant != "none":
+  if quant != "none":
     dom = f"tgmm_kernel_k{d}_n{f}"
     if f"tgmm_f8_kernel_k{d}_n{f}" in stage_ms:
       dom, dom_kernel, dom_peak = f"tgmm_f8_kernel_k{d}_n{f}", "tgmm_f8_kernel", PEAK_TFLOPS["fp8"]
   dom_ms = stage_ms[dom]
   achieved = 2.0 * m * d * f / (dom_ms * 1e-3) / 1e12
   flops = 18.0 * m * d * f
-  traffic, traffic_source = measured_traffic(wl.name + "_train" + ("_fp8_full" if args.quant == "fp8_full" else "")) if args.tokens is None else (None, None)
+  traffic, traffic_source = measured_traffic(wl.name + "_train" + ("_fp8_full" if quant == "fp8_full" else "")) if args.tokens is None else (None, None)
   result = {
-      "metric": "moe_bf16_layer_fwd_bwd_tflops", "value": flops / (elapsed / args.steps) / 1e12, "unit": "TFLOP/s",
-      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3 / args.steps,
+      "metric": "moe_bf16_layer_fwd_bwd_tflops", "value": flops / (elapsed / steps) / 1e12, "unit": "TFLOP/s",
+      "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": elapsed * 1e3 / steps,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
       "config": {"workload": f"{wl.name} shape, training: forward + backward of the MoE expert layer, {t} tokens, d_model {d}, "
                              f"d_ff {f}, {e} experts top-{k}, bf16 weights and activations, SwiGLU"
-                             + ("" if args.quant == "none" else f", grouped matmuls quantised ({args.quant}, {args.calibration})"),
+                             + ("" if quant == "none" else f", grouped matmuls quantised ({quant}, {calibration_method})"),
                  "tokens": t, "d_model": d, "d_ff": f, "experts": e, "top_k": k, "parallelism": "single GPU"},
       "roofline": dict(bound="mfma", achieved=achieved, peak=dom_peak, unit="TFLOP/s", frac=achieved / dom_peak,
                        traffic=traffic, traffic_source=traffic_source,
                        kernel=dom_kernel + " (weight gradient of wi_0 / wi_1)", kernel_ms=dom_ms),
       "stage_ms": stage_ms,
   }
-  result["calibration"] = calibration("bf16")
-  if not args.no_cpu_baseline:
-    result["cpu_baseline"] = train_cpu_baseline(wl, args.cpu_sample_tokens or 1024)
-  print(json.dumps(result))
+  del block, w0, w1, wo, x
+  torch.cuda.empty_cache()
+  return result
 
 
 def run_workload(args, name, tokens=None):
@@ -540,7 +550,8 @@ def main():
     # the remaining configurations of the baseline (parity-test cases, not the headline), each timed the same way so
     # that one run records all five
     result["other_configs"] = []
-    for name in ("c1", "c4", "c5"):
+    # (c2f8: the first configuration's shape with the fp8 operands of the fp8_full recipe, per row x per channel scales)
+    for name in ("c1", "c4", "c5", "c2f8"):
       torch.cuda.empty_cache()
       o, _, olayer, _, _ = run_workload(args, name)
       del olayer
@@ -565,6 +576,14 @@ def main():
         entry["workload"] = o["config"]["workload"]
       sweep.append(entry)
     result["c5_token_sweep"] = sweep
+    # forward + backward of the expert layer at the first configuration's shape, bf16 and the fp8_full recipe (a few steps
+    # each; `python bench.py --train [--quant fp8_full]` is the full line with its calibration and CPU baseline)
+    result["training"] = []
+    for quant in ("none", "fp8_full"):
+      torch.cuda.empty_cache()
+      sub = argparse.Namespace(**{**vars(args), "workload": "c2", "tokens": None})
+      tr = train_result(sub, quant, "absmax", min(args.steps, 5), min(args.warmup, 2))
+      result["training"].append({k: tr[k] for k in ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "config", "roofline", "stage_ms")})
   print(json.dumps(result))
 
 
