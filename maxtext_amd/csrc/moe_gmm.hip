@@ -29,6 +29,7 @@
 
 
 #include "moe_gmm_common.h"
+#include "moe_gmm_wqs.h"
 
 #include <cstring>
 #include <mutex>
@@ -476,7 +477,10 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   // 0.38 against 0.34 / 0.35 ms).  Int8 and group-32 int4: 16, between the crossover with equal groups (30 on the Qwen3
   // shape, where both kernels then wait for the weights of all experts) and the one with Zipf-skewed routing (10: few
   // experts hold most rows and the tiled kernel converts their weights once per 128 rows instead of once per 32).
-  const long long stream_rows_hi = int4_g128 ? 32 : variant == V_MX4 ? 32 : 16;
+  // Group-128 int4 on shapes the LDS-streamed kernel takes: 48 (GPT-OSS shape, layer times at 40 / 48 / 64 rows per expert:
+  // 0.28 / 0.32 / 0.38 ms against 0.33 ms on the 128-row tiles throughout).
+  const bool wqs_ok = int4_g128 && kernel == MOE_GMM_KERNEL_AUTO && wqs_takes(WQ_I4, K, N, a->num_groups_local, glu);
+  const long long stream_rows_hi = int4_g128 ? (wqs_ok ? 48 : 32) : variant == V_MX4 ? 32 : 16;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
   const bool stream_ok = variant != V_BF16 && !wq_kmajor && K % 32 == 0 && (long long)N * K < (1LL << 31);
@@ -500,6 +504,9 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
     q.ch_gstride = p.rhs_scale_gstride; q.ch_nstride = p.rhs_scale_nstride;
     const int fmt = variant == V_W8 ? WQ_I8 : variant == V_MX4 ? WQ_MX4 : (rbk == 32 ? WQ_I4G32 : WQ_I4);
+    // group-128 int4: the LDS-streamed persistent kernel where it takes the shape (MOE_GMM_KERNEL_STREAM keeps the
+    // register-staged one)
+    if (wqs_ok) return launch_wqs(q, glu, a->num_groups_local, s);
     return launch_wq(fmt, one, q, glu, max_tiles_for(M, G, bm), kernel == MOE_GMM_KERNEL_STREAM_NOSPLIT ? 1 : 0, s);
   }
   const int op = OP_BF16;
@@ -540,6 +547,7 @@ int moe_init(void) {
   if (int st = prepare_dl()) return st;
   if (int st = prepare_dlw()) return st;
   if (int st = prepare_dls()) return st;
+  if (int st = prepare_wqs()) return st;
   if (int st = prepare_tgmm()) return st;
   if (int st = prepare_f8s()) return st;
   return prepare_fp8();

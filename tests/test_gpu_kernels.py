@@ -559,6 +559,65 @@ def test_gmm_decode_int4_weight_only(K, m, k, n, gs):
   assert relerr(got, want) <= TOL
 
 
+WQS_SHAPES = [
+    # m, k, n, group sizes, first local group, local groups
+    (40, 256, 128, [7, 0, 12, 1, 20], 0, 5),          # one segment of K; four channel groups with SwiGLU (the minimum)
+    (150, 1536, 264, [16, 3, 33, 0, 50, 48], 0, 6),    # two segments; a channel tail (264 = 8 x 32 + 8); groups of 1..4 tiles
+    (90, 2880, 320, [10, 25, 1, 16, 17, 9, 12], 2, 3),  # three segments with a ragged last k-block; a shard of the experts
+    (700, 3072, 160, [40] * 16 + [60], 0, 17),        # many tiles per block: runs that cross tiles; 40 rows per expert
+]
+
+
+@pytest.mark.parametrize("m,k,n,gs,off,g_local", WQS_SHAPES)
+def test_gmm_int4_lds_streamed_kernel(K, m, k, n, gs, off, g_local):
+  """The persistent decode kernel for group-128 int4 (weights copied global -> LDS three segments ahead, activations
+  resident in registers): both projections with SwiGLU and the plain product, against the oracle and against the
+  register-staged streaming kernel on the same operands; per-expert biases, partial sums, f32 output, activation rows
+  read through an index, and rows of experts outside the local shard (zeros)."""
+  from maxtext_amd._lib import MOE_INT4
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 23)
+  q, s = O.quantize_int4_groups(native(w), 128)
+  qu, su = O.quantize_int4_groups(native(w_up), 128)
+  s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
+  lo, hi = off, off + g_local
+  v2 = lambda sc: sc.float().permute(0, 2, 1)[:, :, None, :]
+  pk, pku = O.pack_int4(q), O.pack_int4(qu)
+  kw = dict(rhs_dtype=MOE_INT4, rhs_scale_block_k=128, group_offset=off)
+  # plain product
+  got = K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), **kw)
+  want = O.gmm(lhs, q.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(s[lo:hi]), quant_block=128, group_offset=off)
+  assert relerr(got, want) <= TOL
+  old = K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), kernel="stream", **kw)
+  assert relerr(got, old.cpu()) <= 8e-3  # the same products summed over K in another order: at most one bf16 step of the result
+  ends = np.cumsum(gs)
+  first, last = (int(ends[lo - 1]) if lo else 0), int(ends[hi - 1])
+  assert torch.all(got[:first] == 0) and torch.all(got[last:] == 0)
+  # SwiGLU with biases, partial sums and f32 output
+  g = torch.Generator().manual_seed(24)
+  b0, b1 = torch.randn(len(gs), n, generator=g), torch.randn(len(gs), n, generator=g)
+  p0, p1 = (torch.randn(m, n, generator=g) * 0.5).to(torch.bfloat16), (torch.randn(m, n, generator=g) * 0.5).to(torch.bfloat16)
+  got = K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), rhs_up=cuda(pku[lo:hi]), rhs_up_scale=cuda(su[lo:hi]),
+                  rhs_bias=cuda(b0[lo:hi]), rhs_up_bias=cuda(b1[lo:hi]), partial_sum=cuda(p0), partial_sum_up=cuda(p1), act="swigluoai",
+                  act_limit=7.0, out_dtype=torch.float32, **kw)
+  okw = dict(quant_block=128, out_dtype=torch.float32, group_offset=off)
+  h0 = O.gmm(lhs, q.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(s[lo:hi]), rhs_bias=b0[lo:hi, None, :], **okw) + p0.float()
+  h1 = O.gmm(lhs, qu.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(su[lo:hi]), rhs_bias=b1[lo:hi, None, :], **okw) + p1.float()
+  want = O.apply_ffn_activation(h0, h1, "swigluoai", 7.0, out_dtype=torch.float32)
+  want[:first] = 0
+  want[last:] = 0
+  assert got.dtype == torch.float32 and relerr(got, want) <= TOL
+  # the fused permute: m product rows read the rows of a shorter activation matrix through an index
+  t_rows = max(m // 3, 1)
+  idx = torch.randint(0, t_rows * 3, (m,), generator=g, dtype=torch.int32)
+  x = lhs[:t_rows].contiguous()
+  got = K.gmm_raw(cuda(x), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), rhs_up=cuda(pku[lo:hi]), rhs_up_scale=cuda(su[lo:hi]),
+                  act="silu", lhs_row_idx=cuda(idx), lhs_row_idx_div=3, **kw)
+  rows = x[(idx // 3).long()]
+  want = O.apply_ffn_activation(O.gmm(rows, q.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(s[lo:hi]), **okw),
+                                O.gmm(rows, qu.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(su[lo:hi]), **okw))
+  assert relerr(got, want) <= TOL
+
+
 FP8_SHAPES = [
     (40, 256, 128, [7, 0, 12, 1, 20]),
     (256, 1024, 384, [8] * 32),

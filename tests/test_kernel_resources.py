@@ -58,3 +58,25 @@ def test_stream_kernels_keep_their_main_loops_free_of_scratch_accesses(tmp_path)
   assert len(kernels) >= 12, sorted(kernels)  # 4 + 6 + 2 instantiations
   bad = {k: v for k, v in kernels.items() if v}
   assert not bad, f"scratch accesses inside the main loop: {bad}"
+
+
+@pytest.mark.skipif(not (shutil.which("hipcc") or os.path.exists("/opt/rocm/bin/hipcc")), reason="needs hipcc")
+def test_lds_streamed_decode_kernel_uses_no_scratch_and_waits_only_where_written(tmp_path):
+  """The persistent int4 decode kernel keeps a tile's activations in registers across work items: every instantiation must
+  fit its registers (no scratch at all: a reload would wait for the copies in flight), and inside its item loop the only
+  waits on the vector-memory counter are the three explicit ones per segment (8, 4 or 0 copies of younger segments
+  outstanding) and those of the side block that loads a new tile's state; a wait the compiler added for a load of its own
+  would drain the copies on every item."""
+  asm = _assembly("moe_gmm_wqs.hip", str(tmp_path))
+  sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_wqs_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
+  assert len(sizes) == 6, sizes  # 3 segment counts x with / without the second projection
+  assert all(int(b) == 0 for _, b in sizes), sizes
+  parts = re.split(r"\n(_ZN3moe14gmm_wqs_kernel\w+):", asm)
+  for i in range(1, len(parts), 2):
+    body = parts[i + 1].split(".end_amdhsa_kernel")[0]
+    barriers = [m.start() for m in re.finditer(r"s_barrier", body)]
+    assert len(barriers) >= 2
+    # between the first segment barrier and the last barrier of the loop body: waits are vmcnt(8/4/0) chosen by branches
+    loop = body[barriers[0]:barriers[-1]]
+    waits = re.findall(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", loop)
+    assert set(waits) <= {"8", "4", "0"}, (parts[i], waits)
