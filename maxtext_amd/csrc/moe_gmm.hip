@@ -479,8 +479,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   // experts hold most rows and the tiled kernel converts their weights once per 128 rows instead of once per 32).
   // Group-128 int4 on shapes the LDS-streamed kernel takes: 48 (GPT-OSS shape, layer times at 40 / 48 / 64 rows per expert:
   // 0.28 / 0.32 / 0.38 ms against 0.33 ms on the 128-row tiles throughout).
-  const bool wqs_ok = int4_g128 && kernel == MOE_GMM_KERNEL_AUTO && wqs_takes(WQ_I4, K, N, a->num_groups_local, glu);
-  const long long stream_rows_hi = int4_g128 ? (wqs_ok ? 48 : 32) : variant == V_MX4 ? 32 : 16;
+  const int wq_fmt = variant == V_W8 ? WQ_I8 : variant == V_MX4 ? WQ_MX4 : (rbk == 32 ? WQ_I4G32 : WQ_I4);
+  const bool wqs_ok = (int4_g128 || variant == V_MX4) && kernel == MOE_GMM_KERNEL_AUTO && wqs_takes(wq_fmt, K, N, a->num_groups_local, glu);
+#ifndef MOE_WQS_MX_ROWS_HI
+#define MOE_WQS_MX_ROWS_HI 48
+#endif
+  const long long stream_rows_hi = int4_g128 ? (wqs_ok ? 48 : 32) : variant == V_MX4 ? (wqs_ok ? MOE_WQS_MX_ROWS_HI : 32) : 16;
   // few rows per expert with weight-only int8 / int4: the streaming kernel (decode is bound by weight bytes)
   // (a lane of that kernel owns 32 consecutive k values, so K must be a multiple of 32; other K take the tiled kernel)
   const bool stream_ok = variant != V_BF16 && !wq_kmajor && K % 32 == 0 && (long long)N * K < (1LL << 31);
@@ -492,7 +496,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     // 16-row tiles up to 16 rows per expert on average, 32-row tiles above; group-128 int4 keeps the 16-row tiles over the
     // whole range (its 32-row variant runs at two waves per SIMD: 0.36 against 0.44 ms on the GPT-OSS shape at 256 tokens)
     // and stays on this kernel up to 32 rows per expert
-    const bool one = int4_g128 || (long long)M <= 16LL * G;
+    const bool one = int4_g128 || wqs_ok || (long long)M <= 16LL * G;
     const int bm = one ? 16 : 32;
     map_tiles(bm);
     WqSkinnyParams q = {};
@@ -503,10 +507,10 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     q.header = header; q.tiles = tiles; q.out = a->out;
     q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
     q.ch_gstride = p.rhs_scale_gstride; q.ch_nstride = p.rhs_scale_nstride;
-    const int fmt = variant == V_W8 ? WQ_I8 : variant == V_MX4 ? WQ_MX4 : (rbk == 32 ? WQ_I4G32 : WQ_I4);
+    const int fmt = wq_fmt;
     // group-128 int4: the LDS-streamed persistent kernel where it takes the shape (MOE_GMM_KERNEL_STREAM keeps the
     // register-staged one)
-    if (wqs_ok) return launch_wqs(q, glu, a->num_groups_local, s);
+    if (wqs_ok) return launch_wqs(fmt, q, glu, a->num_groups_local, s);
     return launch_wq(fmt, one, q, glu, max_tiles_for(M, G, bm), kernel == MOE_GMM_KERNEL_STREAM_NOSPLIT ? 1 : 0, s);
   }
   const int op = OP_BF16;

@@ -24,16 +24,21 @@ namespace moe {
 //
 // int4 values are widened as in the register-staged kernel: a nibble n (value + 8) is OR-ed into the mantissa of 128.0,
 // the MFMA yields P = sum (128 + n_k) a_k, and the block's contribution is scale * (P - 136 * sum a_k) in f32.
+// MXFP4 (e2m1 pairs, one e8m0 scale per 32 values = per lane and k-block) is widened by v_cvt_scalef32_pk_bf16_fp4, scale
+// included, so its MFMAs add straight into the item's sums; its scales are the 32 x K/32 bytes of each half.
 // ---------------------------------------------------------------------------------------
 
 constexpr int kWqsThreads = 512;
 constexpr int kWqsRing = 4;                           // segment slots: one multiplied, three in flight
 constexpr int kWqsSegBytes = 64 * 512;                // 64 rows x 8 k-blocks x 64 B
-constexpr int kWqsScaleBytes = 4096;                  // per item: two regions (32 rows x nkb bf16, nkb <= 32) at +0 and +2048
-constexpr int kWqsScaleRing = 4;                      // an item's scales arrive up to three items ahead
+// Scales of an item: two regions (one per half) of NSEG KB each (int4: 32 rows x nkb bf16 <= NSEG/2 KB; MXFP4: 32 rows x K/32
+// bytes <= NSEG KB).  They arrive with the item's first segment, i.e. up to ceil(3 / NSEG) items ahead: 4, 3, 2 buffers
+// for 1, 2, 3 segments per item, at most 12 KB.
+constexpr int kWqsScaleArea = 16384;
+constexpr int wqs_scale_ring(int nseg) { return nseg == 1 ? 4 : nseg == 2 ? 3 : 2; }
 constexpr int kWqsRedBytes = 2 * 3 * 8 * kWave * 4;   // partial sums of the waves ksub = 1..3 of both channel halves
 constexpr int kWqsScale0 = kWqsRing * kWqsSegBytes;
-constexpr int kWqsRed0 = kWqsScale0 + kWqsScaleRing * kWqsScaleBytes;
+constexpr int kWqsRed0 = kWqsScale0 + kWqsScaleArea;
 constexpr int kWqsLds = kWqsRed0 + kWqsRedBytes;      // 159744 bytes
 constexpr int kWqsMaxKBlocks = 24;  // K <= 3072: eight k-blocks per wave (K up to 4096) do not fit the registers
 
@@ -42,10 +47,15 @@ constexpr int kWqsMaxKBlocks = 24;  // K <= 3072: eight k-blocks per wave (K up 
 // instructions do not look inside asm statements.
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t c) { return (x & mask) | c; }
 
-template <int NSEG, bool GLU>
+template <int FMT, int NSEG, bool GLU>
 __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyParams p, int num_groups) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  static_assert(FMT == WQ_I4 || FMT == WQ_MX4, "group-128 int4 or MXFP4");
+  constexpr bool MX = FMT == WQ_MX4;
   constexpr int KBW = 2 * NSEG;  // k-blocks a wave owns
+  constexpr int SRING = wqs_scale_ring(NSEG);
+  constexpr int SHALF = NSEG * 1024;  // bytes of one half's scale region in LDS
+  static_assert(SRING * 2 * SHALF <= kWqsScaleArea, "scale buffers");
   constexpr int CH = GLU ? 32 : 64;
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -64,7 +74,8 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
 
   // weights and scales through buffer descriptors: a request past the end of a tensor returns zeros
   const uint32_t w_bytes = clamp_u32((size_t)num_groups * N * row_bytes);
-  const uint32_t s_bytes = clamp_u32((size_t)num_groups * N * nkb * 2);
+  const uint32_t srow_bytes = MX ? (uint32_t)K / 32 : (uint32_t)nkb * 2;  // scale bytes of one channel
+  const uint32_t s_bytes = clamp_u32((size_t)num_groups * N * srow_bytes);
   const v4i desc_w = buffer_desc(p.rhs, w_bytes);
   const v4i desc_u = buffer_desc(GLU ? p.rhs_up : p.rhs, w_bytes);
   const v4i sdesc_w = buffer_desc(p.rhs_scale, s_bytes);
@@ -105,10 +116,14 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
 #pragma unroll
       for (int s = 0; s < 4; s++) {
         const uint4 x = ok ? raw[i][s] : make_uint4(0, 0, 0, 0);
-        // k order (k0,k4,k1,k5,k2,k6,k3,k7): the order the nibbles of a word come out in
-        act[i][s] = make_uint4(__builtin_amdgcn_perm(x.z, x.x, 0x05040100u), __builtin_amdgcn_perm(x.z, x.x, 0x07060302u),
-                               __builtin_amdgcn_perm(x.w, x.y, 0x05040100u), __builtin_amdgcn_perm(x.w, x.y, 0x07060302u));
-        t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(v8bf, act[i][s]), t, 0, 0, 0);
+        if (MX) {
+          act[i][s] = x;  // (the conversion hands out a word's values in their own order)
+        } else {
+          // k order (k0,k4,k1,k5,k2,k6,k3,k7): the order the nibbles of a word come out in
+          act[i][s] = make_uint4(__builtin_amdgcn_perm(x.z, x.x, 0x05040100u), __builtin_amdgcn_perm(x.z, x.x, 0x07060302u),
+                                 __builtin_amdgcn_perm(x.w, x.y, 0x05040100u), __builtin_amdgcn_perm(x.w, x.y, 0x07060302u));
+          t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(v8bf, act[i][s]), t, 0, 0, 0);
+        }
       }
       sa[i] = t[0];
     }
@@ -120,12 +135,13 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
     const int q = q0 + it;
     const int m = q / ncg, cg = q - m * ncg;
     const int group = m == m_cur ? g_cur : g_next;  // (three positions ahead never leave the next tile: ncg >= 4)
-    if (s == 0 && (uint32_t)(wave % 4) * 1024u < 64u * (uint32_t)nkb) {
-      // the item's scales: 32 channels x nkb bf16 of each half, contiguous in the [G, N, nkb] tensor
+    if (s == 0 && (uint32_t)(wave % 4) * 1024u < 32u * srow_bytes) {
+      // the item's scales: the rows of 32 channels of each half, contiguous in the [G, N, nkb] / [G, N, K/32] tensor (a
+      // copy's last KB may run past them: what it brings is other channels' scales, or zeros past the tensor)
       const int ch0 = GLU ? cg * 32 : cg * 64 + (up_half ? 32 : 0);
-      const uint32_t voff = ((uint32_t)(group * N + ch0) * (uint32_t)nkb) * 2u + (uint32_t)(wave % 4) * 1024u + (uint32_t)lane * 16u;
+      const uint32_t voff = (uint32_t)(group * N + ch0) * srow_bytes + (uint32_t)(wave % 4) * 1024u + (uint32_t)lane * 16u;
       dma16_buffer(up_half ? sdesc_u : sdesc_w, voff, 0u,
-                   lds_base + kWqsScale0 + (uint32_t)(it % kWqsScaleRing) * kWqsScaleBytes + (up_half ? 2048u : 0u) + (uint32_t)(wave % 4) * 1024u);
+                   lds_base + kWqsScale0 + (uint32_t)(it % SRING) * (2u * SHALF) + (up_half ? (uint32_t)SHALF : 0u) + (uint32_t)(wave % 4) * 1024u);
     }
     const uint32_t slot = lds_base + (uint32_t)(pos % kWqsRing) * kWqsSegBytes;
 #pragma unroll
@@ -144,7 +160,6 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
     if (pos < nstream) issue(pos);
   load_acts();
 
-  const uint16_t* const scale_lds = (const uint16_t*)(smem + kWqsScale0);
   float* const red = (float*)(smem + kWqsRed0);
   uint32_t M4 = 0x000f000fu, cbase = 0x43004300u;  // nibbles of a pair; two bf16 128.0: both opaque, i.e. in registers
   asm volatile("" : "+s"(M4));
@@ -158,9 +173,12 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
       load_tile(m);
       load_acts();
     }
-    float acc_g[4] = {0.f, 0.f, 0.f, 0.f}, acc_u[4] = {0.f, 0.f, 0.f, 0.f};
-    // this lane's four channels of each half, at the wave's first k-block: the k-blocks that follow are 4 entries apart
-    const uint16_t* sc = scale_lds + (it % kWqsScaleRing) * (kWqsScaleBytes / 2) + (a * 16 + 4 * kq) * nkb + ksub;
+    v4f acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t* const sbuf = smem + kWqsScale0 + (it % SRING) * (2 * SHALF);
+    // int4: this lane's four channels (accumulator layout) of each half, at the wave's first k-block: the k-blocks that
+    // follow are 4 entries apart.  MXFP4: the lane's own channel (operand layout), one byte per 32 values.
+    const uint16_t* sc = (const uint16_t*)sbuf + (a * 16 + 4 * kq) * nkb + ksub;
+    const uint8_t* scb = sbuf + (a * 16 + j) * (K / 32) + ksub * 4 + kq;
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
       const int pos = it * NSEG + s;
@@ -182,30 +200,50 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
         const int c = ((ksub + 4 * b) * 4 + kq) ^ j;
         const uint4 wq = *(const uint4*)(slot + (a * 16 + j) * 512 + c * 16);
         const uint4 uq = *(const uint4*)(slot + (32 + a * 16 + j) * 512 + c * 16);
-        float sg[4], su[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          sg[r] = bf16_bits_to_f32(sc[r * nkb + 4 * i]);
-          su[r] = bf16_bits_to_f32(sc[1024 + r * nkb + 4 * i]);
-        }
         const uint32_t xw[4] = {wq.x, wq.y, wq.z, wq.w};
         const uint32_t xu[4] = {uq.x, uq.y, uq.z, uq.w};
-        v4f pg = {0.f, 0.f, 0.f, 0.f}, pu = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (MX) {
+          // (a scale byte read past a row's end, for a k-block past the last, belongs to another channel: finite, and the
+          // activations it meets are zeros)
+          const float sg = __uint_as_float((uint32_t)scb[16 * i] << 23), su = __uint_as_float((uint32_t)scb[SHALF + 16 * i] << 23);
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
-          const v8bf wf = __builtin_bit_cast(v8bf, make_uint4(and_or(xw[w], M4, cbase), and_or(xw[w] >> 4, M4, cbase), and_or(xw[w] >> 8, M4, cbase),
-                                                              and_or(xw[w] >> 12, M4, cbase)));
-          const v8bf uf = __builtin_bit_cast(v8bf, make_uint4(and_or(xu[w], M4, cbase), and_or(xu[w] >> 4, M4, cbase), and_or(xu[w] >> 8, M4, cbase),
-                                                              and_or(xu[w] >> 12, M4, cbase)));
-          const v8bf af = __builtin_bit_cast(v8bf, act[i][w]);
-          pg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, pg, 0, 0, 0);
-          pu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf, af, pu, 0, 0, 0);
-        }
-        const float off = 136.0f * sa[i];
+          for (int w = 0; w < 4; w++) {
+            const v8bf wf = __builtin_bit_cast(v8bf, make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xw[w], sg, 0)),
+                                                                __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xw[w], sg, 1)),
+                                                                __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xw[w], sg, 2)),
+                                                                __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xw[w], sg, 3))));
+            const v8bf uf = __builtin_bit_cast(v8bf, make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xu[w], su, 0)),
+                                                                __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xu[w], su, 1)),
+                                                                __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xu[w], su, 2)),
+                                                                __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(xu[w], su, 3))));
+            const v8bf af = __builtin_bit_cast(v8bf, act[i][w]);
+            acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, acc_g, 0, 0, 0);
+            acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf, af, acc_u, 0, 0, 0);
+          }
+        } else {
+          float sg[4], su[4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          acc_g[r] = fmaf(sg[r], pg[r] - off, acc_g[r]);
-          acc_u[r] = fmaf(su[r], pu[r] - off, acc_u[r]);
+          for (int r = 0; r < 4; r++) {
+            sg[r] = bf16_bits_to_f32(sc[r * nkb + 4 * i]);
+            su[r] = bf16_bits_to_f32(sc[SHALF / 2 + r * nkb + 4 * i]);
+          }
+          v4f pg = {0.f, 0.f, 0.f, 0.f}, pu = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            const v8bf wf = __builtin_bit_cast(v8bf, make_uint4(and_or(xw[w], M4, cbase), and_or(xw[w] >> 4, M4, cbase), and_or(xw[w] >> 8, M4, cbase),
+                                                                and_or(xw[w] >> 12, M4, cbase)));
+            const v8bf uf = __builtin_bit_cast(v8bf, make_uint4(and_or(xu[w], M4, cbase), and_or(xu[w] >> 4, M4, cbase), and_or(xu[w] >> 8, M4, cbase),
+                                                                and_or(xu[w] >> 12, M4, cbase)));
+            const v8bf af = __builtin_bit_cast(v8bf, act[i][w]);
+            pg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, pg, 0, 0, 0);
+            pu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf, af, pu, 0, 0, 0);
+          }
+          const float off = 136.0f * sa[i];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            acc_g[r] = fmaf(sg[r], pg[r] - off, acc_g[r]);
+            acc_u[r] = fmaf(su[r], pu[r] - off, acc_u[r]);
+          }
         }
       }
     }
@@ -276,46 +314,54 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
 // Host side
 // ---------------------------------------------------------------------------------------
 
-// group-128 int4 with K up to 3072, at least four channel groups per tile (a copy issued three positions ahead then
-// never looks past the next tile) and tensors within 32-bit offsets
+// group-128 int4 or MXFP4 with K up to 3072, at least four channel groups per tile (a copy issued three positions ahead
+// then never looks past the next tile), scale rows that start on 16-byte boundaries and tensors within 32-bit offsets
 bool wqs_takes(int fmt, int K, int N, int G_local, bool glu) {
   const int nkb = (K + 127) / 128;
   const int ncg = cdiv(N, glu ? 32 : 64);
-  return fmt == WQ_I4 && K % 32 == 0 && nkb <= kWqsMaxKBlocks && N % 8 == 0 && ncg >= 4 &&
+  if (fmt != WQ_I4 && fmt != WQ_MX4) return false;
+  const long long srow = fmt == WQ_MX4 ? K / 32 : nkb * 2;
+  return K % 32 == 0 && nkb <= kWqsMaxKBlocks && N % 8 == 0 && ncg >= 4 && ((long long)N * srow) % 16 == 0 && (32 * srow) % 16 == 0 &&
          (long long)G_local * N * (K / 2) + (1 << 16) < (1LL << 32);
 }
 
-template <int NSEG>
-static int launch_wqs_n(const WqSkinnyParams& p, bool glu, int num_groups, int blocks, hipStream_t s) {
-  if (glu) {
-    if (int st = reserve_lds(gmm_wqs_kernel<NSEG, true>, kWqsLds, lds_flags<std::integral_constant<int, 7000 + NSEG>>())) return st;
-    gmm_wqs_kernel<NSEG, true><<<blocks, kWqsThreads, kWqsLds, s>>>(p, num_groups);
-  } else {
-    if (int st = reserve_lds(gmm_wqs_kernel<NSEG, false>, kWqsLds, lds_flags<std::integral_constant<int, 7100 + NSEG>>())) return st;
-    gmm_wqs_kernel<NSEG, false><<<blocks, kWqsThreads, kWqsLds, s>>>(p, num_groups);
-  }
+template <int FMT, int NSEG, bool GLU>
+static int launch_wqs_one(const WqSkinnyParams& p, int num_groups, int blocks, hipStream_t s) {
+  if (int st = reserve_lds(gmm_wqs_kernel<FMT, NSEG, GLU>, kWqsLds, lds_flags<std::integral_constant<int, 7000 + FMT * 100 + NSEG * 2 + (GLU ? 1 : 0)>>()))
+    return st;
+  gmm_wqs_kernel<FMT, NSEG, GLU><<<blocks, kWqsThreads, kWqsLds, s>>>(p, num_groups);
   return check_launch("gmm_wqs_kernel");
 }
 
-int launch_wqs(const WqSkinnyParams& p, bool glu, int num_groups, hipStream_t s) {
+template <int FMT>
+static int launch_wqs_fmt(const WqSkinnyParams& p, bool glu, int num_groups, int blocks, hipStream_t s) {
+  switch (cdiv(cdiv(p.K, 128), 8)) {
+    case 1: return glu ? launch_wqs_one<FMT, 1, true>(p, num_groups, blocks, s) : launch_wqs_one<FMT, 1, false>(p, num_groups, blocks, s);
+    case 2: return glu ? launch_wqs_one<FMT, 2, true>(p, num_groups, blocks, s) : launch_wqs_one<FMT, 2, false>(p, num_groups, blocks, s);
+    case 3: return glu ? launch_wqs_one<FMT, 3, true>(p, num_groups, blocks, s) : launch_wqs_one<FMT, 3, false>(p, num_groups, blocks, s);
+  }
+  return fail(MOE_ERR_UNSUPPORTED, "gmm: K = %d is past the LDS-streamed decode kernel", p.K);
+}
+
+int launch_wqs(int fmt, const WqSkinnyParams& p, bool glu, int num_groups, hipStream_t s) {
   int cus = 0;
   if (int st = device_cu_count(&cus)) return st;
-  const int nseg = cdiv(cdiv(p.K, 128), 8);
-  switch (nseg) {
-    case 1: return launch_wqs_n<1>(p, glu, num_groups, cus, s);
-    case 2: return launch_wqs_n<2>(p, glu, num_groups, cus, s);
-    case 3: return launch_wqs_n<3>(p, glu, num_groups, cus, s);
-  }
-  return fail(MOE_ERR_UNSUPPORTED, "gmm: K = %d is past the LDS-streamed int4 kernel", p.K);
+  return fmt == WQ_MX4 ? launch_wqs_fmt<WQ_MX4>(p, glu, num_groups, cus, s) : launch_wqs_fmt<WQ_I4>(p, glu, num_groups, cus, s);
+}
+
+template <int FMT, int NSEG>
+static int prepare_wqs_pair() {
+  if (int st = reserve_lds(gmm_wqs_kernel<FMT, NSEG, true>, kWqsLds, lds_flags<std::integral_constant<int, 7000 + FMT * 100 + NSEG * 2 + 1>>())) return st;
+  return reserve_lds(gmm_wqs_kernel<FMT, NSEG, false>, kWqsLds, lds_flags<std::integral_constant<int, 7000 + FMT * 100 + NSEG * 2>>());
 }
 
 int prepare_wqs() {
-  if (int st = reserve_lds(gmm_wqs_kernel<1, true>, kWqsLds, lds_flags<std::integral_constant<int, 7001>>())) return st;
-  if (int st = reserve_lds(gmm_wqs_kernel<2, true>, kWqsLds, lds_flags<std::integral_constant<int, 7002>>())) return st;
-  if (int st = reserve_lds(gmm_wqs_kernel<3, true>, kWqsLds, lds_flags<std::integral_constant<int, 7003>>())) return st;
-  if (int st = reserve_lds(gmm_wqs_kernel<1, false>, kWqsLds, lds_flags<std::integral_constant<int, 7101>>())) return st;
-  if (int st = reserve_lds(gmm_wqs_kernel<2, false>, kWqsLds, lds_flags<std::integral_constant<int, 7102>>())) return st;
-  return reserve_lds(gmm_wqs_kernel<3, false>, kWqsLds, lds_flags<std::integral_constant<int, 7103>>());
+  if (int st = prepare_wqs_pair<WQ_I4, 1>()) return st;
+  if (int st = prepare_wqs_pair<WQ_I4, 2>()) return st;
+  if (int st = prepare_wqs_pair<WQ_I4, 3>()) return st;
+  if (int st = prepare_wqs_pair<WQ_MX4, 1>()) return st;
+  if (int st = prepare_wqs_pair<WQ_MX4, 2>()) return st;
+  return prepare_wqs_pair<WQ_MX4, 3>();
 }
 
 }  // namespace moe

@@ -568,25 +568,35 @@ WQS_SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("fmt", ["int4", "mxfp4"])
 @pytest.mark.parametrize("m,k,n,gs,off,g_local", WQS_SHAPES)
-def test_gmm_int4_lds_streamed_kernel(K, m, k, n, gs, off, g_local):
-  """The persistent decode kernel for group-128 int4 (weights copied global -> LDS three segments ahead, activations
-  resident in registers): both projections with SwiGLU and the plain product, against the oracle and against the
-  register-staged streaming kernel on the same operands; per-expert biases, partial sums, f32 output, activation rows
+def test_gmm_4bit_lds_streamed_kernel(K, m, k, n, gs, off, g_local, fmt):
+  """The persistent decode kernel for group-128 int4 and MXFP4 (weights copied global -> LDS three segments ahead,
+  activations resident in registers): both projections with SwiGLU and the plain product, against the oracle and against
+  the register-staged streaming kernel on the same operands; per-expert biases, partial sums, f32 output, activation rows
   read through an index, and rows of experts outside the local shard (zeros)."""
-  from maxtext_amd._lib import MOE_INT4
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
   lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 23)
-  q, s = O.quantize_int4_groups(native(w), 128)
-  qu, su = O.quantize_int4_groups(native(w_up), 128)
-  s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
   lo, hi = off, off + g_local
-  v2 = lambda sc: sc.float().permute(0, 2, 1)[:, :, None, :]
-  pk, pku = O.pack_int4(q), O.pack_int4(qu)
-  kw = dict(rhs_dtype=MOE_INT4, rhs_scale_block_k=128, group_offset=off)
+  if fmt == "int4":
+    q, s = O.quantize_int4_groups(native(w), 128)
+    qu, su = O.quantize_int4_groups(native(w_up), 128)
+    s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
+    v2 = lambda sc: sc.float().permute(0, 2, 1)[:, :, None, :]
+    pk, pku = O.pack_int4(q), O.pack_int4(qu)
+    kw = dict(rhs_dtype=MOE_INT4, rhs_scale_block_k=128, group_offset=off)
+    ogmm = lambda x, up, **o: O.gmm(x, (qu if up else q).transpose(1, 2)[lo:hi], gs, rhs_scale=v2((su if up else s)[lo:hi]), quant_block=128,
+                                    group_offset=off, **o)
+  else:
+    blocks, s = O.quantize_mxfp4(native(w))  # [g, n, k/32, 16], [g, n, k/32]
+    ublocks, su = O.quantize_mxfp4(native(w_up))
+    deq, udeq = O.dequantize_mxfp4(blocks, s).to(torch.bfloat16), O.dequantize_mxfp4(ublocks, su).to(torch.bfloat16)
+    pk, pku = blocks.reshape(len(gs), n, k // 2), ublocks.reshape(len(gs), n, k // 2)
+    kw = dict(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32, group_offset=off)
+    ogmm = lambda x, up, **o: O.gmm(x, (udeq if up else deq)[lo:hi], gs, transpose_rhs=True, group_offset=off, **o)
   # plain product
   got = K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), **kw)
-  want = O.gmm(lhs, q.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(s[lo:hi]), quant_block=128, group_offset=off)
-  assert relerr(got, want) <= TOL
+  assert relerr(got, ogmm(lhs, False)) <= TOL
   old = K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), kernel="stream", **kw)
   assert relerr(got, old.cpu()) <= 8e-3  # the same products summed over K in another order: at most one bf16 step of the result
   ends = np.cumsum(gs)
@@ -599,9 +609,8 @@ def test_gmm_int4_lds_streamed_kernel(K, m, k, n, gs, off, g_local):
   got = K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), rhs_up=cuda(pku[lo:hi]), rhs_up_scale=cuda(su[lo:hi]),
                   rhs_bias=cuda(b0[lo:hi]), rhs_up_bias=cuda(b1[lo:hi]), partial_sum=cuda(p0), partial_sum_up=cuda(p1), act="swigluoai",
                   act_limit=7.0, out_dtype=torch.float32, **kw)
-  okw = dict(quant_block=128, out_dtype=torch.float32, group_offset=off)
-  h0 = O.gmm(lhs, q.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(s[lo:hi]), rhs_bias=b0[lo:hi, None, :], **okw) + p0.float()
-  h1 = O.gmm(lhs, qu.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(su[lo:hi]), rhs_bias=b1[lo:hi, None, :], **okw) + p1.float()
+  h0 = ogmm(lhs, False, rhs_bias=b0[lo:hi, None, :], out_dtype=torch.float32) + p0.float()
+  h1 = ogmm(lhs, True, rhs_bias=b1[lo:hi, None, :], out_dtype=torch.float32) + p1.float()
   want = O.apply_ffn_activation(h0, h1, "swigluoai", 7.0, out_dtype=torch.float32)
   want[:first] = 0
   want[last:] = 0
@@ -613,8 +622,7 @@ def test_gmm_int4_lds_streamed_kernel(K, m, k, n, gs, off, g_local):
   got = K.gmm_raw(cuda(x), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), rhs_up=cuda(pku[lo:hi]), rhs_up_scale=cuda(su[lo:hi]),
                   act="silu", lhs_row_idx=cuda(idx), lhs_row_idx_div=3, **kw)
   rows = x[(idx // 3).long()]
-  want = O.apply_ffn_activation(O.gmm(rows, q.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(s[lo:hi]), **okw),
-                                O.gmm(rows, qu.transpose(1, 2)[lo:hi], gs, rhs_scale=v2(su[lo:hi]), **okw))
+  want = O.apply_ffn_activation(ogmm(rows, False, out_dtype=torch.float32), ogmm(rows, True, out_dtype=torch.float32))
   assert relerr(got, want) <= TOL
 
 

@@ -69,7 +69,7 @@ def test_lds_streamed_decode_kernel_uses_no_scratch_and_waits_only_where_written
   would drain the copies on every item."""
   asm = _assembly("moe_gmm_wqs.hip", str(tmp_path))
   sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_wqs_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
-  assert len(sizes) == 6, sizes  # 3 segment counts x with / without the second projection
+  assert len(sizes) == 12, sizes  # 2 formats x 3 segment counts x with / without the second projection
   assert all(int(b) == 0 for _, b in sizes), sizes
   parts = re.split(r"\n(_ZN3moe14gmm_wqs_kernel\w+):", asm)
   for i in range(1, len(parts), 2):
