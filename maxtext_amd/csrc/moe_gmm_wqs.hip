@@ -127,6 +127,11 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
       }
       sa[i] = t[0];
     }
+    // the loads complete here (an empty statement that "uses" every register), not at their first use behind the copies
+#pragma unroll
+    for (int i = 0; i < KBW; i++)
+#pragma unroll
+      for (int s = 0; s < 4; s++) asm volatile("" : "+v"(act[i][s].x), "+v"(act[i][s].y), "+v"(act[i][s].z), "+v"(act[i][s].w));
   };
 
   // ---- copies of one stream position: segment s of item q into ring slot `slot` ----
