@@ -1754,6 +1754,35 @@ def test_gmm_degenerate_group_sizes(K):
   assert relerr(tiny, want) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["int4", "mxfp4"])
+def test_gmm_4bit_decode_degenerate_group_sizes(K, fmt):
+  """The LDS-streamed decode kernel on all-empty groups (every row zero), a single row, and group sizes that overrun the
+  rows (clipped to m): the cases of test_gmm_degenerate_group_sizes on 4-bit weights."""
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
+  g = torch.Generator().manual_seed(43)
+  m, k, n = 37, 256, 128
+  lhs = torch.randn(m, k, generator=g).to(torch.bfloat16)
+  w = torch.randn(3, n, k, generator=g) * 0.1  # [g, n, k]
+  if fmt == "int4":
+    q, s = O.quantize_int4_groups(w, 128)
+    s = s.to(torch.bfloat16)
+    deq = (q.float().reshape(3, n, k // 128, 128) * s.float()[..., None]).reshape(3, n, k)
+    pk, kw = O.pack_int4(q), dict(rhs_dtype=MOE_INT4, rhs_scale_block_k=128)
+  else:
+    blocks, s = O.quantize_mxfp4(w)
+    deq = O.dequantize_mxfp4(blocks, s)
+    pk, kw = blocks.reshape(3, n, k // 2), dict(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+  up = dict(rhs_up=cuda(pk), rhs_up_scale=cuda(s), act="silu")  # (with the second projection the kernel takes 128 channels)
+  out = K.gmm_raw(cuda(lhs), cuda(pk), cuda(np.array([0, 0, 0], np.int32)), rhs_scale=cuda(s), **up, **kw)
+  assert out.shape == (m, n) and torch.all(out == 0)
+  h = lambda x, e: x.float() @ deq[e].float().T
+  act = lambda y: torch.nn.functional.silu(y) * y
+  one = K.gmm_raw(cuda(lhs[:1]), cuda(pk), cuda(np.array([0, 1, 0], np.int32)), rhs_scale=cuda(s), **up, **kw)
+  assert relerr(one, act(h(lhs[:1], 1))) <= TOL
+  over = K.gmm_raw(cuda(lhs), cuda(pk), cuda(np.array([20, 30, 50], np.int32)), rhs_scale=cuda(s), **up, **kw)  # 100 rows announced, 37 exist
+  assert relerr(over, torch.cat([act(h(lhs[:20], 0)), act(h(lhs[20:], 1))])) <= TOL
+
+
 def test_route_sort_combine_single_token(K):
   """One token: routing, sort, gather and combine on the smallest input (k of E selections, all in different groups)."""
   g = torch.Generator().manual_seed(42)
