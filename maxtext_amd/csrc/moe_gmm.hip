@@ -480,6 +480,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   // Group-128 int4 on shapes the LDS-streamed kernel takes: 48 (GPT-OSS shape, layer times at 40 / 48 / 64 rows per expert:
   // 0.28 / 0.32 / 0.38 ms against 0.33 ms on the 128-row tiles throughout).
   const int wq_fmt = variant == V_W8 ? WQ_I8 : variant == V_MX4 ? WQ_MX4 : (rbk == 32 ? WQ_I4G32 : WQ_I4);
+  // (its copies move 16 bytes per lane; every pointer of the call has been checked for 16-byte alignment above)
   const bool wqs_ok = (int4_g128 || variant == V_MX4) && kernel == MOE_GMM_KERNEL_AUTO && wqs_takes(wq_fmt, K, N, a->num_groups_local, glu);
 #ifndef MOE_WQS_MX_ROWS_HI
 #define MOE_WQS_MX_ROWS_HI 48
