@@ -18,22 +18,31 @@ struct TileInfo {
 // workspace: int32 header[4] (header[0] = number of tiles) | TileInfo tiles[max_tiles]
 static inline int max_tiles_for(int M, int G, int bm) { return cdiv(M, bm) + G + 1; }
 
-// Exclusive prefix sum over one value per thread of a THREADS-wide block; *total = the block's sum.
+// Exclusive prefix sum over one value per thread of a THREADS-wide block; *total = the block's sum.  Each wave scans its
+// values with lane shuffles, the waves' totals meet in s_buf: three barriers whatever the block's width.
 template <int THREADS>
 __device__ __forceinline__ int block_exclusive_scan(int v, int* s_buf, int* total) {
-  const int tid = threadIdx.x;
-  s_buf[tid] = v;
-  __syncthreads();
-  for (int o = 1; o < THREADS; o <<= 1) {
-    int add = tid >= o ? s_buf[tid - o] : 0;
-    __syncthreads();
-    s_buf[tid] += add;
-    __syncthreads();
+  static_assert(THREADS % kWave == 0, "whole waves");
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  int incl = v;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int t = __shfl_up(incl, o, kWave);
+    if (lane >= o) incl += t;
   }
-  int incl = s_buf[tid];
-  *total = s_buf[THREADS - 1];
+  __syncthreads();  // (s_buf may still be read by the caller's previous use)
+  if (lane == kWave - 1) s_buf[wave] = incl;
   __syncthreads();
-  return incl - v;
+  int base = 0, sum = 0;
+#pragma unroll
+  for (int w = 0; w < THREADS / kWave; w++) {
+    const int c = s_buf[w];
+    base += w < wave ? c : 0;
+    sum += c;
+  }
+  *total = sum;
+  __syncthreads();
+  return base + incl - v;
 }
 
 // group_sizes (device) -> the list of (group, first row, rows) m-tiles of height BM that never straddle a group boundary,
