@@ -46,6 +46,83 @@ __global__ __launch_bounds__(kMapThreads) void tile_map_kernel(
   build_tile_map<kMapThreads>(group_sizes, G_total, group_offset, G_local, M, BM, zero_fill, header, tiles, s_buf);
 }
 
+// The same list for a launch that hands the short last tiles of its groups to the decode kernel: a local group's rows
+// are cut into tiles of BM rows as above, but a remainder of at most tail_rows rows becomes 16-row tiles of a second list
+// (header[1] = their number, records from tiles + tail_base on).  A 256-row tile costs the persistent kernels the same
+// whether it holds 256 rows or 5; the decode kernel streams the expert's weights once per 16 rows, about a quarter of
+// that.  Zero-fill tiles (rows of groups held elsewhere, rows past the groups) stay in the first list.
+constexpr int kTailTile = 16;
+constexpr int kTailRows = 48;  // remainders up to three decode tiles (the two routes cost the same at about 58 rows on the GPT-OSS shape)
+__global__ __launch_bounds__(kMapThreads) void tile_map_split_kernel(
+    const int32_t* __restrict__ group_sizes, int G_total, int group_offset, const int32_t* __restrict__ group_offset_dev, int G_local, int M,
+    int BM, int tail_rows, int tail_base, int zero_fill, int32_t* __restrict__ header, TileInfo* __restrict__ tiles) {
+  __shared__ int s_buf[kMapThreads];
+  if (group_offset_dev) group_offset = max(*group_offset_dev, 0);
+  const int tid = threadIdx.x;
+  const int per = (G_total + kMapThreads - 1) / kMapThreads;
+  const int g0 = min(tid * per, G_total), g1 = min(g0 + per, G_total);
+  long long rows = 0;
+  for (int g = g0; g < g1; g++) rows += max(group_sizes[g], 0);
+  int total_rows;
+  const int row_prefix = block_exclusive_scan<kMapThreads>((int)min(rows, (long long)M), s_buf, &total_rows);
+  // a group's clipped extent [s, e) -> (tiles of BM rows, 16-row tail tiles)
+  auto split = [&](int s, int e, bool local, int& nmain, int& ntail) {
+    const int n = e - s, rem = n % BM;
+    nmain = n / BM;
+    ntail = 0;
+    if (rem > 0) {
+      if (local && rem <= tail_rows) ntail = (rem + kTailTile - 1) / kTailTile;
+      else nmain += 1;
+    }
+  };
+  int my_main = 0, my_tail = 0;
+  {
+    long long start = row_prefix;
+    for (int g = g0; g < g1; g++) {
+      const long long end = start + max(group_sizes[g], 0);
+      const int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
+      const int local = g - group_offset;
+      const bool is_local = local >= 0 && local < G_local;
+      if (zero_fill || is_local) {
+        int a, b;
+        split(s, e, is_local, a, b);
+        my_main += a;
+        my_tail += b;
+      }
+      start = end;
+    }
+  }
+  int total_main, total_tail;
+  const int main_prefix = block_exclusive_scan<kMapThreads>(my_main, s_buf, &total_main);
+  const int tail_prefix = block_exclusive_scan<kMapThreads>(my_tail, s_buf, &total_tail);
+  {
+    long long start = row_prefix;
+    int ti = main_prefix, tj = tail_base + tail_prefix;
+    for (int g = g0; g < g1; g++) {
+      const long long end = start + max(group_sizes[g], 0);
+      const int s = (int)min(start, (long long)M), e = (int)min(end, (long long)M);
+      const int local = g - group_offset;
+      const bool is_local = local >= 0 && local < G_local;
+      if (zero_fill || is_local) {
+        int a, b;
+        split(s, e, is_local, a, b);
+        const int kind = is_local ? local : -1;
+        for (int t = 0; t < a; t++) tiles[ti++] = TileInfo{kind, s + t * BM, min(BM, e - (s + t * BM)), 0};
+        const int tail0 = e - (e - s) % BM;  // (b > 0 only with a remainder that went to the second list)
+        for (int t = 0; t < b; t++) tiles[tj++] = TileInfo{kind, tail0 + t * kTailTile, min(kTailTile, e - (tail0 + t * kTailTile)), 0};
+      }
+      start = end;
+    }
+  }
+  const int covered = min(total_rows, M);
+  const int tail = zero_fill ? (M - covered + BM - 1) / BM : 0;
+  for (int i = tid; i < tail; i += kMapThreads) tiles[total_main + i] = TileInfo{-1, covered + i * BM, min(BM, M - (covered + i * BM)), 0};
+  if (tid == 0) {
+    header[0] = total_main + tail;
+    header[1] = total_tail;
+  }
+}
+
 // What the last call on a device mapped, and into which buffer (MOE_GMM_SAME_GROUPS).
 struct Mapped {
   const void* ws; const int32_t* gs; const int32_t* offset_dev; int M, G, offset, local, bm, zero_fill;
@@ -262,6 +339,14 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
                                            a->num_groups_local, bm, zero_fill ? 1 : 0});
     if (!(same && (a->flags & MOE_GMM_SAME_GROUPS)))
       tile_map_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->group_offset_dev, a->num_groups_local, M, bm, zero_fill, header, tiles);
+  };
+  // (the split list is recorded under its own tile-height code: a plain list of the same height is another list)
+  auto map_tiles_split = [&](int bm, int tail_rows, int tail_base) {
+    const bool same = note_tile_map(Mapped{workspace, a->group_sizes, a->group_offset_dev, M, G, a->group_offset_dev ? 0 : a->group_offset,
+                                           a->num_groups_local, bm | (tail_rows << 16), zero_fill ? 1 : 0});
+    if (!(same && (a->flags & MOE_GMM_SAME_GROUPS)))
+      tile_map_split_kernel<<<1, kMapThreads, 0, s>>>(a->group_sizes, G, a->group_offset, a->group_offset_dev, a->num_groups_local, M, bm, tail_rows,
+                                                      tail_base, zero_fill, header, tiles);
   };
   RowOpts ro;
   ro.row_idx = a->lhs_row_idx; ro.idx_div = a->lhs_row_idx_div < 1 ? 1 : a->lhs_row_idx_div;
@@ -522,6 +607,26 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
   }
   TiledKind kind = kernel == MOE_GMM_KERNEL_BIG ? K_T256 : pick_tiled_kind(op, bsrc, glu, M, K, N, G, wq_kmajor, a->lhs_row_idx ? ro.lhs_rows : 0);
   if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64 || kind == K_DLW || kind == K_DLW128)) kind = kind == K_DLW128 ? K_T128 : K_T256;
+  // 4-bit weights on the persistent kernel: a group's last rows, when they are few, go to the decode kernel in a second
+  // launch (16-row tiles of a second list) instead of filling a corner of one more 128- or 256-row tile
+  const bool split_tails = (kind == K_DLW || kind == K_DLW128) && kernel == MOE_GMM_KERNEL_AUTO && (bsrc == BSRC_I4 || bsrc == BSRC_MX4) && !wq_kmajor &&
+                           wqs_takes(wq_fmt, K, N, a->num_groups_local, glu);
+  if (split_tails) {
+    const int bm = tiled_kind_bm(kind);
+    const int tail_base = max_tiles_for(M, G, bm);  // past every record the first list can hold
+    if ((size_t)16 + ((size_t)tail_base + (size_t)G * cdiv(kTailRows, kTailTile)) * sizeof(TileInfo) <= workspace_bytes) {
+      map_tiles_split(bm, kTailRows, tail_base);
+      if (int st = launch_tiled_kind(kind, op, bsrc, glu, p, M, G, s)) return st;
+      WqSkinnyParams q = {};
+      q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
+      q.rhs_scale = a->rhs_scale; q.rhs_up_scale = a->rhs_up_scale;
+      q.rhs_bias = a->rhs_bias; q.rhs_up_bias = a->rhs_up_bias;
+      q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
+      q.header = header + 1; q.tiles = tiles + tail_base; q.out = a->out;
+      q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
+      return launch_wqs(wq_fmt, q, glu, a->num_groups_local, s);
+    }
+  }
   map_tiles(tiled_kind_bm(kind));
   return launch_tiled_kind(kind, op, bsrc, glu, p, M, G, s);
 }

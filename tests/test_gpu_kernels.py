@@ -626,6 +626,53 @@ def test_gmm_4bit_lds_streamed_kernel(K, m, k, n, gs, off, g_local, fmt):
   assert relerr(got, want) <= TOL
 
 
+@pytest.mark.parametrize("fmt", ["int4", "mxfp4"])
+@pytest.mark.parametrize("regime", ["tiles256", "tiles128"])
+def test_gmm_4bit_prefill_hands_short_group_tails_to_the_decode_kernel(K, fmt, regime):
+  """4-bit weights at prefill sizes: a group's remainder of at most 48 rows past its 256- (or 128-) row tiles runs as
+  16-row tiles on the decode kernel in a second launch, everything else on the persistent kernel.  Remainders on both
+  sides of every boundary (0, 1, 16, 17, 48, 49, a full tile less one), an empty group, rows in no group, a shard of
+  the experts with the other rows kept; against the oracle, and every row written exactly once."""
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
+  bm = 256 if regime == "tiles256" else 128
+  rem = [0, 1, 16, 17, 48, 49, bm - 1, 5]
+  gs = np.asarray([bm * (1 + i % 2) + r for i, r in enumerate(rem)] + [0, 33], np.int32)  # the last group: a tail and nothing else
+  if regime == "tiles128":
+    gs = np.asarray([(bm if i % 3 == 0 else 0) + r for i, r in enumerate(rem)] + [0, 33, 130, 128], np.int32)  # 50-odd rows per expert
+  e = len(gs)
+  m, k, n = int(gs.sum()) + 40, 320, 160
+  lhs, w, w_up, _ = _gmm_inputs(m, k, n, gs.tolist(), 31)
+  if fmt == "int4":
+    q, s = O.quantize_int4_groups(native(w), 128)
+    qu, su = O.quantize_int4_groups(native(w_up), 128)
+    s, su = s.to(torch.bfloat16), su.to(torch.bfloat16)
+    v2 = lambda sc: sc.float().permute(0, 2, 1)[:, :, None, :]
+    pk, pku, kw = O.pack_int4(q), O.pack_int4(qu), dict(rhs_dtype=MOE_INT4, rhs_scale_block_k=128)
+    ogmm = lambda up, lo, hi, **o: O.gmm(lhs, (qu if up else q).transpose(1, 2)[lo:hi], gs, rhs_scale=v2((su if up else s)[lo:hi]), quant_block=128, **o)
+  else:
+    blocks, s = O.quantize_mxfp4(native(w))
+    ublocks, su = O.quantize_mxfp4(native(w_up))
+    deq, udeq = O.dequantize_mxfp4(blocks, s).to(torch.bfloat16), O.dequantize_mxfp4(ublocks, su).to(torch.bfloat16)
+    pk, pku, kw = blocks.reshape(e, n, k // 2), ublocks.reshape(e, n, k // 2), dict(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+    ogmm = lambda up, lo, hi, **o: O.gmm(lhs, (udeq if up else deq)[lo:hi], gs, transpose_rhs=True, **o)
+  total = int(gs.sum())
+  got = K.gmm_raw(cuda(lhs), cuda(pk), cuda(gs), rhs_scale=cuda(s), **kw)
+  assert relerr(got, ogmm(False, 0, e)) <= TOL and torch.all(got[total:] == 0)
+  got = K.gmm_raw(cuda(lhs), cuda(pk), cuda(gs), rhs_scale=cuda(s), rhs_up=cuda(pku), rhs_up_scale=cuda(su), act="silu", **kw)
+  want = O.apply_ffn_activation(ogmm(False, 0, e, out_dtype=torch.float32), ogmm(True, 0, e, out_dtype=torch.float32))
+  # (the persistent kernel multiplies int4 weights dequantised to bf16, as the reference's converter stores them; the oracle
+  # keeps q * scale exact: the chained tolerance of test_gmm_int4_weight_only)
+  assert relerr(got, want, atol_rms=ELEM_ATOL_RMS_CHAINED) <= TOL
+  # experts 2 .. 6 only, into a buffer whose other rows stay as they are
+  lo, hi = 2, 7
+  ends = np.cumsum(gs)
+  first, last = int(ends[lo - 1]), int(ends[hi - 1])
+  buf = torch.full((m, n), 3.0, dtype=torch.bfloat16, device="cuda")
+  K.gmm_raw(cuda(lhs), cuda(pk[lo:hi]), cuda(gs), rhs_scale=cuda(s[lo:hi]), group_offset=lo, out=buf, keep_other_rows=True, **kw)
+  assert torch.all(buf[:first] == 3.0) and torch.all(buf[last:] == 3.0)
+  assert relerr(buf[first:last], ogmm(False, lo, hi, group_offset=lo)[first:last]) <= TOL
+
+
 FP8_SHAPES = [
     (40, 256, 128, [7, 0, 12, 1, 20]),
     (256, 1024, 384, [8] * 32),

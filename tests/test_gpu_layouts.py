@@ -301,7 +301,12 @@ def test_weight_only_prefill_kernel_against_the_tiled_kernel_at_size(K, fmt, glu
     kw.update(rhs_up=ws[1][0], rhs_up_scale=ws[1][1], act="silu")
   got = K.gmm_raw(lhs, ws[0][0], gs, **kw)
   ref = K.gmm_raw(lhs, ws[0][0], gs, kernel="tiled", **kw)
-  assert relerr(got, ref) <= 1e-3
+  # (group-128 int4 and MXFP4: the short last tiles of the groups run on the decode kernel, which sums over K in another
+  # order and, for int4, keeps nibble * scale in f32 where the other two multiply weights rounded to bf16: up to one bf16
+  # step of the result apart)
+  # (for int4 the two arithmetic routes are compared in the max norm only: behind SwiGLU an element of small magnitude may
+  # differ by a few per cent of the tensor's rms between them; the rows sampled below are held to the oracle elementwise)
+  assert relerr(got, ref, elementwise=fmt != "int4") <= (8e-3 if fmt in ("int4", "mxfp4") else 1e-3)
   assert torch.all(got[int(gs_h.sum()):] == 0)
   # a few rows of three groups against the oracle (first / last row of a group, a row next to the empty group)
   off = np.concatenate([[0], np.cumsum(gs_h)])
