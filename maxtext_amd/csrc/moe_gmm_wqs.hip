@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
           t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, __builtin_bit_cast(v8bf, act[i][s]), t, 0, 0, 0);
         }
       }
-      sa[i] = t[0];
+      sa[i] = -136.0f * t[0];  // what the sums of the k-block start at: the widened nibbles are 128 + 8 too large
     }
     // the loads complete here (an empty statement that "uses" every register), not at their first use behind the copies
 #pragma unroll
@@ -135,6 +135,14 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
   };
 
   // ---- copies of one stream position: segment s of item q into ring slot `slot` ----
+  // the lane's part of a copy's offset: row 8 * wave + 2 * i + lane / 32 of the segment (rows 0..31 the first half, 32..63
+  // the second: the other projection, or channels 32..63), the 16-byte chunk XOR-ed with row % 16
+  uint32_t lane_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int row = 8 * wave + 2 * i + lane / 32;
+    lane_off[i] = (uint32_t)(GLU ? row % 32 : row) * row_bytes + (uint32_t)((lane % 32) ^ (row & 15)) * 16u;
+  }
   auto issue = [&](int pos) {
     const int it = pos / NSEG, s = pos - it * NSEG;
     const int q = q0 + it;
@@ -148,15 +156,11 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
       dma16_buffer(up_half ? sdesc_u : sdesc_w, voff, 0u,
                    lds_base + kWqsScale0 + (uint32_t)(it % SRING) * (2u * SHALF) + (up_half ? (uint32_t)SHALF : 0u) + (uint32_t)(wave % 4) * 1024u);
     }
+    // (channels past N in an item's last rows are the next expert's first rows, or zeros past the tensor: never stored)
     const uint32_t slot = lds_base + (uint32_t)(pos % kWqsRing) * kWqsSegBytes;
+    const uint32_t base = (uint32_t)(group * N + cg * CH) * row_bytes + (uint32_t)s * 512u;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int row = 8 * wave + 2 * i + lane / 32;  // row of the segment: 0..31 first half, 32..63 second
-      const int ch = min(GLU ? cg * 32 + row % 32 : cg * 64 + row, N - 1);
-      const uint32_t c = (uint32_t)((lane % 32) ^ (row & 15));
-      const uint32_t voff = (uint32_t)(group * N + ch) * row_bytes + ((uint32_t)s * 32u + c) * 16u;
-      dma16_buffer(up_half ? desc_u : desc_w, voff, 0u, slot + (uint32_t)(8 * wave + 2 * i) * 512u);
-    }
+    for (int i = 0; i < 4; i++) dma16_buffer(up_half ? desc_u : desc_w, base + lane_off[i], 0u, slot + (uint32_t)(8 * wave + 2 * i) * 512u);
   };
 
   load_tile(m_cur);
@@ -232,7 +236,7 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
             sg[r] = bf16_bits_to_f32(sc[r * nkb + 4 * i]);
             su[r] = bf16_bits_to_f32(sc[SHALF / 2 + r * nkb + 4 * i]);
           }
-          v4f pg = {0.f, 0.f, 0.f, 0.f}, pu = {0.f, 0.f, 0.f, 0.f};
+          v4f pg = {sa[i], sa[i], sa[i], sa[i]}, pu = pg;
 #pragma unroll
           for (int w = 0; w < 4; w++) {
             const v8bf wf = __builtin_bit_cast(v8bf, make_uint4(and_or(xw[w], M4, cbase), and_or(xw[w] >> 4, M4, cbase), and_or(xw[w] >> 8, M4, cbase),
@@ -243,11 +247,10 @@ __global__ __launch_bounds__(kWqsThreads) void gmm_wqs_kernel(const WqSkinnyPara
             pg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, pg, 0, 0, 0);
             pu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf, af, pu, 0, 0, 0);
           }
-          const float off = 136.0f * sa[i];
 #pragma unroll
           for (int r = 0; r < 4; r++) {
-            acc_g[r] = fmaf(sg[r], pg[r] - off, acc_g[r]);
-            acc_u[r] = fmaf(su[r], pu[r] - off, acc_u[r]);
+            acc_g[r] = fmaf(sg[r], pg[r], acc_g[r]);
+            acc_u[r] = fmaf(su[r], pu[r], acc_u[r]);
           }
         }
       }
