@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0
 PROFILE_OF = {
     "c2": ("profiles/gmm_dls_kernel_int8_mixtral_prefill_c2.md", ["moe_gmm_dls.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c2f8": ("profiles/gmm_dls_kernel_fp8_mixtral_shape_prefill_c2f8.md", ["moe_gmm_dls.hip", "moe_gmm_common.h", "moe_common.h"]),
-    "c3": ("profiles/gmm_fp8_skinny_kernel_deepseek_decode_c3.md", ["moe_gmm_fp8.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c3": ("profiles/gmm_f8d_kernel_deepseek_decode_c3.md", ["moe_gmm_f8d.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c4": ("profiles/gmm_dlw_kernel_int8w_qwen3_prefill_c4.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c5": ("profiles/gmm_dlw_kernel_int4w_gptoss_prefill_c5_t4096.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c2_train": ("profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md", ["moe_tgmm.hip", "moe_common.h"]),
@@ -116,12 +116,13 @@ def dominant_kernel_model(wl, group_sizes):
     return dict(bound="mfma", work=flops, unit="TFLOP/s", peak=PEAK_TFLOPS["fp8"], scale=1e12,
                 name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
   if wl.weight_quant == "fp8":
-    # HBM bound (decode): weights of the non-empty experts + block scales + activations in + out
+    # HBM bound (decode): weights of the non-empty experts + block scales + activations in + out (the LDS-streamed persistent
+    # kernel where moe_gmm gives it the shape: rows of a multiple of 1024 values up to 7168)
     w_bytes = nonempty * 2.0 * d * f
     s_bytes = nonempty * 2.0 * (d / 128) * (f / 128) * 4 + rows * (d / 128) * 4
     io_bytes = rows * d * 1.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
-                name="gmm_fp8_skinny_kernel (wi_0|wi_1 + SwiGLU)", dtype="fp8")
+                name=("gmm_f8d_kernel" if d % 1024 == 0 and d <= 7168 else "gmm_fp8_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
   if wl.weight_quant in ("int4", "mxfp4") and rows <= (48 if wl.weight_quant == "int4" else 32) * cfg.num_experts:
     # weight-only 4-bit decode (the dispatch rule of moe_gmm for its streaming kernels: group-128 int4 on the LDS-streamed
     # persistent kernel, MXFP4 on the register-staged one): bound by streaming the weights of the experts that were hit

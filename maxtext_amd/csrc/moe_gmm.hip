@@ -30,6 +30,7 @@
 
 #include "moe_gmm_common.h"
 #include "moe_gmm_wqs.h"
+#include "moe_gmm_f8d.h"
 
 #include <cstring>
 #include <mutex>
@@ -398,7 +399,13 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     // groups of exactly 128 rows 1.94 against 1.70 ms, at 160 rows 2.05 against 2.54 ms; routed groups scatter around
     // their mean, and those over 128 rows cost the 128 x 128 kernel a second tile).
     const bool few_rows = (long long)M <= 16LL * G;
-    const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > 14LL * G : kernel != MOE_GMM_KERNEL_STREAM;
+    // block-scaled operands at decode sizes: the LDS-streamed persistent kernel where it takes the shape
+    // (MOE_GMM_KERNEL_STREAM keeps the register-staged one)
+#ifndef MOE_F8D_ROWS_HI
+#define MOE_F8D_ROWS_HI 14
+#endif
+    const bool f8d_ok = fp8_blocks && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
+    const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8d_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
     // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
     const bool chip_full = (long long)max_tiles_for(M, G, 256) * cdiv(N, glu ? 128 : 256) >= 128;
@@ -446,7 +453,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       const bool vec4 = fp8_blocks && (K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
       return launch_fp8_tiled(big, glu, vec4, P, M, G, s);
     }
-    const int bm = few_rows ? 16 : 64;
+    const int bm = few_rows || f8d_ok ? 16 : 64;
     map_tiles(bm);
     SkinnyParams p = {};
     p.lhs = (const uint8_t*)a->lhs; p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
@@ -462,6 +469,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     p.header = header; p.tiles = tiles; p.out = a->out;
     p.M = M; p.K = K; p.N = N; p.act = a->act; p.act_limit = a->act_limit; p.ro = ro;
     p.min_rows = 1; p.max_rows = bm;
+    if (f8d_ok) return launch_f8d(p, glu, a->num_groups_local, s);
     return launch_fp8_skinny(few_rows, p, glu, max_tiles_for(M, G, bm), s);
   }
 
@@ -658,6 +666,7 @@ int moe_init(void) {
   if (int st = prepare_dlw()) return st;
   if (int st = prepare_dls()) return st;
   if (int st = prepare_wqs()) return st;
+  if (int st = prepare_f8d()) return st;
   if (int st = prepare_tgmm()) return st;
   if (int st = prepare_f8s()) return st;
   return prepare_fp8();

@@ -707,6 +707,67 @@ def test_gmm_fp8_block_scaled(K, m, k, n, gs, variant):
   assert relerr(got, want) <= TOL
 
 
+F8D_SHAPES = [
+    # m, k, n, group sizes, first local group, local groups (the library takes this kernel up to 14 rows per group on average)
+    (40, 1024, 128, [7, 0, 12, 1, 20], 0, 5),            # two segments of K; four channel groups with SwiGLU (the minimum)
+    (80, 2048, 264, [16, 3, 33, 0, 2, 17], 0, 6),        # four segments; a channel tail (264 = 8 x 32 + 8); groups of 1..3 tiles
+    (90, 7168, 320, [10, 25, 1, 16, 17, 9, 12], 2, 3),   # the longest rows the kernel takes; a shard of the experts
+    (450, 3072, 160, [12] * 32 + [52], 0, 33),           # many tiles per block: runs that cross tiles
+]
+
+
+@pytest.mark.parametrize("m,k,n,gs,off,g_local", F8D_SHAPES)
+def test_gmm_fp8_lds_streamed_decode_kernel(K, m, k, n, gs, off, g_local):
+  """The persistent decode kernel for block-scaled fp8 (e4m3 activations with 1 x 128 scales, e4m3 weights with 128 x 128
+  scales; weights copied global -> LDS three segments ahead, activations resident in registers): both projections with
+  SwiGLU and the plain product, against the oracle and against the register-staged streaming kernel on the same
+  operands; per-expert biases, partial sums, f32 output, activation rows read through an index, and rows of experts
+  outside the local shard (zeros)."""
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 29)
+  lo, hi = off, off + g_local
+  aq, asc = O.quantize_fp8_blocks(lhs, 1, 128)
+  wq, wsc = O.quantize_fp8_blocks(native(w), 128, 128)  # [g, n, k], scale [g, n/128, k/128]
+  uq, usc = O.quantize_fp8_blocks(native(w_up), 128, 128)
+  v2 = lambda sc: torch.repeat_interleave(sc.permute(0, 2, 1), 128, dim=2)[:, :, None, :n]  # -> [g, nb, 1, n]
+  kw = dict(lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128, group_offset=off)
+  ogmm = lambda x, xs, up, **o: O.gmm(x, (uq if up else wq)[lo:hi], gs, lhs_scale=xs, rhs_scale=v2((usc if up else wsc)[lo:hi]), transpose_rhs=True,
+                                      quant_block=128, group_offset=off, **o)
+  # plain product
+  got = K.gmm_raw(cuda(aq), cuda(wq[lo:hi]), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc[lo:hi]), **kw)
+  assert relerr(got, ogmm(aq, asc, False)) <= TOL
+  old = K.gmm_raw(cuda(aq), cuda(wq[lo:hi]), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc[lo:hi]), kernel="stream", **kw)
+  assert relerr(got, old.cpu()) <= 8e-3  # the same products summed over K in another order: at most one bf16 step of the result
+  ends = np.cumsum(gs)
+  first, last = (int(ends[lo - 1]) if lo else 0), int(ends[hi - 1])
+  assert torch.all(got[:first] == 0) and torch.all(got[last:] == 0)
+  # SwiGLU with biases, partial sums and f32 output
+  g = torch.Generator().manual_seed(30)
+  b0, b1 = torch.randn(len(gs), n, generator=g), torch.randn(len(gs), n, generator=g)
+  p0, p1 = (torch.randn(m, n, generator=g) * 0.5).to(torch.bfloat16), (torch.randn(m, n, generator=g) * 0.5).to(torch.bfloat16)
+  got = K.gmm_raw(cuda(aq), cuda(wq[lo:hi]), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc[lo:hi]), rhs_up=cuda(uq[lo:hi]),
+                  rhs_up_scale=cuda(usc[lo:hi]), rhs_bias=cuda(b0[lo:hi]), rhs_up_bias=cuda(b1[lo:hi]), partial_sum=cuda(p0), partial_sum_up=cuda(p1),
+                  act="swigluoai", act_limit=7.0, out_dtype=torch.float32, **kw)
+  h0 = ogmm(aq, asc, False, rhs_bias=b0[lo:hi, None, :], out_dtype=torch.float32) + p0.float()
+  h1 = ogmm(aq, asc, True, rhs_bias=b1[lo:hi, None, :], out_dtype=torch.float32) + p1.float()
+  want = O.apply_ffn_activation(h0, h1, "swigluoai", 7.0, out_dtype=torch.float32)
+  want[:first] = 0
+  want[last:] = 0
+  assert got.dtype == torch.float32 and relerr(got, want) <= TOL
+  same = K.gmm_raw(cuda(aq), cuda(wq[lo:hi]), cuda(gs), lhs_scale=cuda(asc), rhs_scale=cuda(wsc[lo:hi]), rhs_up=cuda(uq[lo:hi]),
+                   rhs_up_scale=cuda(usc[lo:hi]), rhs_bias=cuda(b0[lo:hi]), rhs_up_bias=cuda(b1[lo:hi]), partial_sum=cuda(p0), partial_sum_up=cuda(p1),
+                   act="swigluoai", act_limit=7.0, out_dtype=torch.float32, kernel="stream", **kw)
+  assert relerr(got, same.cpu()) <= 1e-4  # f32 results of the two kernels: only the order of the K sum differs
+  # the fused permute: m product rows read the rows of a shorter activation matrix (and its scales) through an index
+  t_rows = max(m // 3, 1)
+  idx = torch.randint(0, t_rows * 3, (m,), generator=g, dtype=torch.int32)
+  x, xs = aq[:t_rows].contiguous(), asc[:t_rows].contiguous()
+  got = K.gmm_raw(cuda(x), cuda(wq[lo:hi]), cuda(gs), lhs_scale=cuda(xs), rhs_scale=cuda(wsc[lo:hi]), rhs_up=cuda(uq[lo:hi]),
+                  rhs_up_scale=cuda(usc[lo:hi]), act="silu", lhs_row_idx=cuda(idx), lhs_row_idx_div=3, **kw)
+  rows, rscales = x[(idx // 3).long()], xs[(idx // 3).long()]
+  want = O.apply_ffn_activation(ogmm(rows, rscales, False, out_dtype=torch.float32), ogmm(rows, rscales, True, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
 def test_gmm_group_offset_and_nan_isolation(K):
   # non-local groups produce zeros (v2 kernel test :939); a NaN row must not leak into other experts' rows (:592)
   lhs, w, _, gs = _gmm_inputs(600, 256, 128, [100, 200, 150, 100], 8)

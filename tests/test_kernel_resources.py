@@ -80,3 +80,25 @@ def test_lds_streamed_decode_kernel_uses_no_scratch_and_waits_only_where_written
     loop = body[barriers[0]:barriers[-1]]
     waits = re.findall(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", loop)
     assert set(waits) <= {"8", "4", "0"}, (parts[i], waits)
+
+
+@pytest.mark.skipif(not (shutil.which("hipcc") or os.path.exists("/opt/rocm/bin/hipcc")), reason="needs hipcc")
+def test_lds_streamed_fp8_decode_kernel_uses_no_scratch_and_waits_only_where_written(tmp_path):
+  """The persistent fp8 decode kernel follows the same rules: up to 112 registers of activations stay resident per lane, so
+  every instantiation must fit its registers, and between the barriers of its item loop the only waits on the
+  vector-memory counter are the explicit ones per segment."""
+  asm = _assembly("moe_gmm_f8d.hip", str(tmp_path))
+  sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_f8d_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
+  assert len(sizes) == 14, sizes  # 7 row lengths (K = 1024 .. 7168) x with / without the second projection
+  assert all(int(b) == 0 for _, b in sizes), sizes
+  parts = re.split(r"\n(_ZN3moe14gmm_f8d_kernel\w+):", asm)
+  assert len(parts) == 29
+  for i in range(1, len(parts), 2):
+    body = parts[i + 1].split(".end_amdhsa_kernel")[0]
+    barriers = [m.start() for m in re.finditer(r"s_barrier", body)]
+    assert len(barriers) >= 2
+    loop = body[barriers[0]:barriers[-1]]
+    waits = re.findall(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", loop)
+    assert set(waits) <= {"8", "4", "0"}, (parts[i], waits)
+    assert "nt lds" in loop and re.search(r"offen lds", loop)  # weights read once stream past the caches, shared ones do not
+
