@@ -62,7 +62,35 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
   const int nnb = (N + 127) / 128;
   const int ntiles = __builtin_amdgcn_readfirstlane(p.header[0]);
   const long long total = (long long)ntiles * ncg;
-  const int q0 = (int)(total * blockIdx.x / gridDim.x), q1 = (int)(total * (blockIdx.x + 1) / gridDim.x);
+  // ---- the run of items this block takes: an even split of the list, except ... ----
+  // ... when the last expert has several tiles (the shared expert of a DeepSeek layer: every token's rows) and a tile is
+  // about one block's share of the work.  Then its tiles go one each to blocks of one XCD (blocks are dealt round-robin to
+  // the 8 XCDs: those with index 8k + 7), which walk the same channel groups side by side and find each item's weights in
+  // that XCD's L2 after the first of them has read it; the other blocks split the other tiles' items evenly.
+  const int nb = (int)gridDim.x, b = (int)blockIdx.x;
+  int nsh = 0;
+  if (ntiles >= 2 && nb % 8 == 0) {
+    const int last = ntiles - 1;
+    const int gl = __builtin_amdgcn_readfirstlane(p.tiles[last].group);
+    const int gk = last - 1 - lane >= 0 ? p.tiles[last - 1 - lane].group : -3;  // lane k: the tile k + 1 before the last
+    const unsigned long long same = __ballot(gk == gl && gl >= 0);
+    const int run = same == ~0ull ? 64 : __builtin_ctzll(~same);  // tiles right before the last one that belong to its expert
+    const long long share = total / nb;
+    if (run >= 1 && run < 64 && run + 1 <= nb / 8 && 2LL * ncg >= share && 4LL * ncg <= 5 * share) nsh = run + 1;
+  }
+  int q0, q1;
+  if (nsh && b % 8 == 7 && b / 8 < nsh) {
+    q0 = (ntiles - nsh + b / 8) * ncg;
+    q1 = q0 + ncg;
+  } else if (nsh) {
+    const int r = b - min(nsh, b / 8), nbo = nb - nsh;  // rank among the other blocks
+    const long long others = (long long)(ntiles - nsh) * ncg;
+    q0 = (int)(others * r / nbo);
+    q1 = (int)(others * (r + 1) / nbo);
+  } else {
+    q0 = (int)(total * b / nb);
+    q1 = (int)(total * (b + 1) / nb);
+  }
   if (q0 >= q1) return;
   const int nitems = q1 - q0, nstream = nitems * NSEG;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
@@ -273,7 +301,7 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
 // scale rows (K % 512 == 0 gives that) and tensors within 32-bit offsets
 bool f8d_takes(int K, int N, int G_local, bool glu) {
   const int ncg = cdiv(N, glu ? 32 : 64);
-  return K % 1024 == 0 && K / 512 <= kF8dMaxSeg && N % 8 == 0 && ncg >= 4 && (long long)G_local * N * K + (1 << 16) < (1LL << 32);
+  return K % 1024 == 0 && K / 512 <= kF8dMaxSeg && N % 8 == 0 && ncg >= 4 && (long long)G_local * N * K + 65LL * K + 1024 < (1LL << 32);  // (an item's last rows may lie up to 63 rows past N)
 }
 
 #ifndef MOE_F8D_NT

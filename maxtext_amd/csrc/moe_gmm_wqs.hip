@@ -330,7 +330,7 @@ bool wqs_takes(int fmt, int K, int N, int G_local, bool glu) {
   if (fmt != WQ_I4 && fmt != WQ_MX4) return false;
   const long long srow = fmt == WQ_MX4 ? K / 32 : nkb * 2;
   return K % 32 == 0 && nkb <= kWqsMaxKBlocks && N % 8 == 0 && ncg >= 4 && ((long long)N * srow) % 16 == 0 && (32 * srow) % 16 == 0 &&
-         (long long)G_local * N * (K / 2) + (1 << 16) < (1LL << 32);
+         (long long)G_local * N * (K / 2) + 65LL * (K / 2) + 1024 < (1LL << 32);  // (an item's last rows may lie up to 63 rows past N)
 }
 
 template <int FMT, int NSEG, bool GLU>
