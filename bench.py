@@ -117,12 +117,12 @@ def dominant_kernel_model(wl, group_sizes):
                 name=kernel + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
   if wl.weight_quant == "fp8":
     # HBM bound (decode): weights of the non-empty experts + block scales + activations in + out (the LDS-streamed persistent
-    # kernel where moe_gmm gives it the shape: rows of a multiple of 1024 values up to 7168)
+    # kernel where moe_gmm gives it the shape: rows of a multiple of 512 values up to 7168)
     w_bytes = nonempty * 2.0 * d * f
     s_bytes = nonempty * 2.0 * (d / 128) * (f / 128) * 4 + rows * (d / 128) * 4
     io_bytes = rows * d * 1.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
-                name=("gmm_f8d_kernel" if d % 1024 == 0 and d <= 7168 else "gmm_fp8_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
+                name=("gmm_f8d_kernel" if d % 512 == 0 and d <= 7168 else "gmm_fp8_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
   if wl.weight_quant in ("int4", "mxfp4") and rows <= (48 if wl.weight_quant == "int4" else 32) * cfg.num_experts:
     # weight-only 4-bit decode (the dispatch rule of moe_gmm for its streaming kernels: group-128 int4 on the LDS-streamed
     # persistent kernel, MXFP4 on the register-staged one): bound by streaming the weights of the experts that were hit

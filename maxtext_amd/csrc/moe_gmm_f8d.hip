@@ -296,12 +296,12 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
 // Host side
 // ---------------------------------------------------------------------------------------
 
-// K a multiple of 1024 up to 7168 (whole segments, an even number of them: the instantiations that exist), at least four
+// K a multiple of 512 up to 7168 (whole segments), at least four
 // channel groups per tile (a copy issued three positions ahead then never looks past the next tile), 16-byte aligned
 // scale rows (K % 512 == 0 gives that) and tensors within 32-bit offsets
 bool f8d_takes(int K, int N, int G_local, bool glu) {
   const int ncg = cdiv(N, glu ? 32 : 64);
-  return K % 1024 == 0 && K / 512 <= kF8dMaxSeg && N % 8 == 0 && ncg >= 4 && (long long)G_local * N * K + 65LL * K + 1024 < (1LL << 32);  // (an item's last rows may lie up to 63 rows past N)
+  return K % 512 == 0 && K / 512 <= kF8dMaxSeg && N % 8 == 0 && ncg >= 4 && (long long)G_local * N * K + 65LL * K + 1024 < (1LL << 32);  // (an item's last rows may lie up to 63 rows past N)
 }
 
 #ifndef MOE_F8D_NT
@@ -325,12 +325,19 @@ int launch_f8d(const SkinnyParams& p, bool glu, int num_groups, hipStream_t s) {
   int cus = 0;
   if (int st = device_cu_count(&cus)) return st;
   switch (p.K / 512) {
+    case 1: return launch_f8d_seg<1>(p, glu, num_groups, cus, s);
     case 2: return launch_f8d_seg<2>(p, glu, num_groups, cus, s);
+    case 3: return launch_f8d_seg<3>(p, glu, num_groups, cus, s);
     case 4: return launch_f8d_seg<4>(p, glu, num_groups, cus, s);
+    case 5: return launch_f8d_seg<5>(p, glu, num_groups, cus, s);
     case 6: return launch_f8d_seg<6>(p, glu, num_groups, cus, s);
+    case 7: return launch_f8d_seg<7>(p, glu, num_groups, cus, s);
     case 8: return launch_f8d_seg<8>(p, glu, num_groups, cus, s);
+    case 9: return launch_f8d_seg<9>(p, glu, num_groups, cus, s);
     case 10: return launch_f8d_seg<10>(p, glu, num_groups, cus, s);
+    case 11: return launch_f8d_seg<11>(p, glu, num_groups, cus, s);
     case 12: return launch_f8d_seg<12>(p, glu, num_groups, cus, s);
+    case 13: return launch_f8d_seg<13>(p, glu, num_groups, cus, s);
     case 14: return launch_f8d_seg<14>(p, glu, num_groups, cus, s);
   }
   return fail(MOE_ERR_UNSUPPORTED, "gmm: K = %d is not a shape of the LDS-streamed fp8 decode kernel", p.K);
@@ -344,12 +351,19 @@ static int prepare_f8d_pair() {
 }
 
 int prepare_f8d() {
+  if (int st = prepare_f8d_pair<1>()) return st;
   if (int st = prepare_f8d_pair<2>()) return st;
+  if (int st = prepare_f8d_pair<3>()) return st;
   if (int st = prepare_f8d_pair<4>()) return st;
+  if (int st = prepare_f8d_pair<5>()) return st;
   if (int st = prepare_f8d_pair<6>()) return st;
+  if (int st = prepare_f8d_pair<7>()) return st;
   if (int st = prepare_f8d_pair<8>()) return st;
+  if (int st = prepare_f8d_pair<9>()) return st;
   if (int st = prepare_f8d_pair<10>()) return st;
+  if (int st = prepare_f8d_pair<11>()) return st;
   if (int st = prepare_f8d_pair<12>()) return st;
+  if (int st = prepare_f8d_pair<13>()) return st;
   return prepare_f8d_pair<14>();
 }
 

@@ -710,9 +710,10 @@ def test_gmm_fp8_block_scaled(K, m, k, n, gs, variant):
 F8D_SHAPES = [
     # m, k, n, group sizes, first local group, local groups (the library takes this kernel up to 14 rows per group on average)
     (40, 1024, 128, [7, 0, 12, 1, 20], 0, 5),            # two segments of K; four channel groups with SwiGLU (the minimum)
+    (30, 512, 256, [3, 16, 0, 11], 0, 4),                # one segment: the scales of four items in flight
     (80, 2048, 264, [16, 3, 33, 0, 2, 17], 0, 6),        # four segments; a channel tail (264 = 8 x 32 + 8); groups of 1..3 tiles
     (90, 7168, 320, [10, 25, 1, 16, 17, 9, 12], 2, 3),   # the longest rows the kernel takes; a shard of the experts
-    (450, 3072, 160, [12] * 32 + [52], 0, 33),           # many tiles per block: runs that cross tiles
+    (450, 3584, 160, [12] * 32 + [52], 0, 33),           # an odd number of segments; many tiles per block: runs that cross tiles
     # a last expert of several tiles where a tile is about one block's share of the work (the shared expert of a
     # DeepSeek layer): its tiles go one each to blocks of one XCD, the other blocks split the rest
     (420, 1024, 192, [1] * 300 + [100], 0, 301),
