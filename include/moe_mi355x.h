@@ -159,6 +159,16 @@ MOE_API int moe_sort_by_expert_mapped(const int32_t* topk_idx, int T, int k, int
                        int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
                        void* workspace, size_t workspace_bytes, int tile_rows, int num_groups_local, int group_offset,
                        int keep_other_rows, void* gmm_workspace, size_t gmm_workspace_bytes, void* stream);
+/* moe_route_topk followed by moe_sort_by_expert_mapped on the indices it wrote (get_topk, moe.py:717-765, then the
+ * argsort / bincount of permute, moe.py:950-960), with the arguments and results of both.  Up to 16 tokens (and 1024 routed
+ * rows) without routing groups the two run as ONE launch (such a decode step spends as long on a launch as on either piece of work);
+ * otherwise this is the two calls one after the other.  topk_idx is both a result and the sort's input. */
+MOE_API int moe_route_sort_mapped(const float* gate_logits, const float* pre_bias_logits, int T, int E, int k,
+                       int mode, int norm_topk_prob, int weights_round_bf16, float routed_scaling_factor,
+                       int n_routing_groups, int topk_routing_group, float* topk_weights, int32_t* topk_idx,
+                       int roll_to_expert_id, int32_t* perm, int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                       void* workspace, size_t workspace_bytes, int tile_rows, int num_groups_local, int group_offset,
+                       int keep_other_rows, void* gmm_workspace, size_t gmm_workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Expert-parallel dispatch bookkeeping on one expert shard (integer work on device-resident sizes; the exchange

@@ -67,15 +67,13 @@ struct GateEpilogue {
   int round_bf16;         // round the matmul result to bf16 first
 };
 
+// One token per wave: token t_raw of T (a wave past the end repeats the last token and writes nothing; every wave of the
+// block must make the call, there is a block barrier inside).  s_row_w / s_pre_w: this wave's kRouteMaxE floats of LDS.
 template <bool GATE>
-__global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
+__device__ __forceinline__ void route_token(
     const float* __restrict__ logits, const float* __restrict__ pre_bias, int T, int E, int k,
     int mode, int norm, int round_bf16, float scaling, int n_groups, int topk_groups,
-    float* __restrict__ w_out, int32_t* __restrict__ idx_out, const GateEpilogue g) {
-  __shared__ float s_row[kRouteWaves][kRouteMaxE];
-  __shared__ float s_pre[GATE ? kRouteWaves : 1][GATE ? kRouteMaxE : 1];
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int t_raw = blockIdx.x * kRouteWaves + wave;
+    float* __restrict__ w_out, int32_t* __restrict__ idx_out, const GateEpilogue& g, int t_raw, int lane, float* s_row_w, float* s_pre_w) {
   const bool active = t_raw < T;
   const int t = active ? t_raw : T - 1;
   const float* row = logits + (size_t)t * E;
@@ -94,7 +92,7 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
         if (g.score_func == 1) x = 1.0f / (1.0f + expf(-x));
         // sqrt(softplus(x)), softplus as logaddexp(x, 0) = max(x, 0) + log1p(exp(-|x|)) (linears.py:51-53)
         if (g.score_func == 2) x = sqrtf(fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))));
-        s_pre[wave][e] = x;
+        s_pre_w[e] = x;
         if (active && g.pre_bias_out) g.pre_bias_out[(size_t)t * E + e] = x;
         if (g.bias) x += g.bias[e];
         if (active && g.logits_out) g.logits_out[(size_t)t * E + e] = x;
@@ -113,7 +111,7 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
 #pragma unroll
     for (int j = 0; j < kRouteVpl; j++) {
       int e = lane + kWave * j;
-      if (e < E) s_row[wave][e] = v[j];
+      if (e < E) s_row_w[e] = v[j];
     }
     __syncthreads();
     float score = -INFINITY;
@@ -121,7 +119,7 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
     if (lane < n_groups) {
       float b1 = -INFINITY, b2 = -INFINITY;
       for (int i = 0; i < gs; i++) {
-        float x = s_row[wave][lane * gs + i];
+        float x = s_row_w[lane * gs + i];
         if (x > b1) {
           b2 = b1;
           b1 = x;
@@ -175,7 +173,7 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
   float w;
   if (mode == MOE_ROUTE_DEEPSEEK) {
     if (GATE)
-      w = lane < k ? s_pre[wave][myi] : 0.f;  // written by this wave's own lanes above
+      w = lane < k ? s_pre_w[myi] : 0.f;  // written by this wave's own lanes above
     else
       w = lane < k ? pre_bias[(size_t)t * E + myi] : 0.f;
     if (norm) {
@@ -212,6 +210,18 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
     w_out[(size_t)t * k + lane] = w;
     idx_out[(size_t)t * k + lane] = myi;
   }
+}
+
+template <bool GATE>
+__global__ __launch_bounds__(kRouteWaves* kWave) void route_topk_kernel(
+    const float* __restrict__ logits, const float* __restrict__ pre_bias, int T, int E, int k,
+    int mode, int norm, int round_bf16, float scaling, int n_groups, int topk_groups,
+    float* __restrict__ w_out, int32_t* __restrict__ idx_out, const GateEpilogue g) {
+  __shared__ float s_row[kRouteWaves][kRouteMaxE];
+  __shared__ float s_pre[GATE ? kRouteWaves : 1][GATE ? kRouteMaxE : 1];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  route_token<GATE>(logits, pre_bias, T, E, k, mode, norm, round_bf16, scaling, n_groups, topk_groups, w_out, idx_out, g,
+                    blockIdx.x * kRouteWaves + wave, lane, s_row[wave], s_pre[GATE ? wave : 0]);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -441,9 +451,9 @@ struct SortMapArgs {
 };
 
 template <int NW>
-__global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
+__device__ __forceinline__ void sort_small_block(
     const int32_t* __restrict__ flat, int M, int E, int roll, const int32_t* __restrict__ roll_dev, int ebits, int32_t* __restrict__ group_sizes,
-    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts, const SortMapArgs mp) {
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts, const SortMapArgs& mp) {
   __shared__ int run[NW][kSortMaxE];
   __shared__ int off[kSortMaxE];
   constexpr int NT = NW * kWave;
@@ -517,6 +527,39 @@ __global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
     __syncthreads();  // group_sizes, written above by this block, are read back from memory
     build_tile_map<NT>(group_sizes, E, mp.group_offset, mp.G_local, M, mp.BM, mp.zero_fill, mp.header, mp.tiles, &run[0][0]);
   }
+}
+
+template <int NW>
+__global__ __launch_bounds__(NW* kWave) void sort_small_kernel(
+    const int32_t* __restrict__ flat, int M, int E, int roll, const int32_t* __restrict__ roll_dev, int ebits, int32_t* __restrict__ group_sizes,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm, int32_t* __restrict__ sorted_experts, const SortMapArgs mp) {
+  sort_small_block<NW>(flat, M, E, roll, roll_dev, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
+}
+
+// Routing and the sort behind it in one block, for at most NW tokens (the smallest decode steps): every wave routes one
+// token, the indices they wrote are read back by the block as the sort's keys.  One launch instead of two where a launch
+// costs as much as the work; with more tokens than waves the routing of one block would take turns and lose to the
+// many blocks of the kernel of its own.
+struct RouteArgs {
+  const float* logits;
+  const float* pre_bias;
+  int T, E, k, mode, norm, round_bf16;
+  float scaling;
+  int n_groups, topk_groups;
+  float* w_out;
+  int32_t* idx_out;
+};
+
+template <int NW>
+__global__ __launch_bounds__(NW* kWave) void route_sort_small_kernel(
+    const RouteArgs r, int roll, int ebits, int32_t* __restrict__ group_sizes, int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm,
+    int32_t* __restrict__ sorted_experts, const SortMapArgs mp) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  // (one token per wave, all at once: r.T <= NW, no routing groups)
+  route_token<false>(r.logits, r.pre_bias, r.T, r.E, r.k, r.mode, r.norm, r.round_bf16, r.scaling, 0, 0, r.w_out, r.idx_out, GateEpilogue{}, wave, lane,
+                     nullptr, nullptr);
+  __syncthreads();  // the indices, written above by this block, are read back from memory
+  sort_small_block<NW>(r.idx_out, r.T * r.k, r.E, roll, nullptr, ebits, group_sizes, perm, inv_perm, sorted_experts, mp);
 }
 
 __global__ void invert_perm_kernel(const int32_t* __restrict__ perm, int M,
@@ -1113,6 +1156,42 @@ int moe_sort_by_expert_mapped(const int32_t* topk_idx, int T, int k, int E, int 
                            &mapped, stream);
   if (st == MOE_OK && mapped) note_tile_map_built(gmm_workspace, group_sizes, (int)M, E, group_offset, num_groups_local, tile_rows, zero_fill);
   return st;
+}
+
+int moe_route_sort_mapped(const float* gate_logits, const float* pre_bias_logits, int T, int E, int k,
+                          int mode, int norm_topk_prob, int weights_round_bf16, float routed_scaling_factor,
+                          int n_routing_groups, int topk_routing_group, float* topk_weights, int32_t* topk_idx,
+                          int roll_to_expert_id, int32_t* perm, int32_t* inv_perm, int32_t* group_sizes, int32_t* sorted_experts,
+                          void* workspace, size_t workspace_bytes, int tile_rows, int num_groups_local, int group_offset,
+                          int keep_other_rows, void* gmm_workspace, size_t gmm_workspace_bytes, void* stream) {
+  const long long M = (long long)T * k;
+  // one launch for both when one block has a wave per token; two launches otherwise (the arguments are checked there)
+  const bool one = T > 0 && T <= 4 * kSortWaves && k > 0 && E > 0 && E <= kSortMaxE && E <= kRouteMaxE && k <= 16 && k <= E && M <= kSortChunk && gate_logits && topk_weights &&
+                   topk_idx && perm && group_sizes && workspace && gmm_workspace && roll_to_expert_id >= 0 && roll_to_expert_id < E &&
+                   mode >= MOE_ROUTE_SOFTMAX_TOPK && mode <= MOE_ROUTE_SOFTMAX_ALL && (mode != MOE_ROUTE_DEEPSEEK || pre_bias_logits) &&
+                   n_routing_groups <= 0 && tile_rows > 0 && num_groups_local > 0 && group_offset >= 0 &&
+                   workspace_bytes >= moe_sort_workspace_bytes(T, k, E) && gmm_workspace_bytes >= moe_gmm_workspace_bytes((int)M, E);
+  if (!one) {
+    if (int st = moe_route_topk(gate_logits, pre_bias_logits, T, E, k, mode, norm_topk_prob, weights_round_bf16, routed_scaling_factor,
+                                n_routing_groups, topk_routing_group, topk_weights, topk_idx, stream))
+      return st;
+    return moe_sort_by_expert_mapped(topk_idx, T, k, E, roll_to_expert_id, perm, inv_perm, group_sizes, sorted_experts, workspace, workspace_bytes,
+                                     tile_rows, num_groups_local, group_offset, keep_other_rows, gmm_workspace, gmm_workspace_bytes, stream);
+  }
+  int ebits = 0;
+  while ((1 << ebits) < E) ebits++;
+  const int zero_fill = keep_other_rows ? 0 : 1;
+  const SortMapArgs mp = {(TileInfo*)((uint8_t*)gmm_workspace + 16), (int32_t*)gmm_workspace, num_groups_local, group_offset, tile_rows, zero_fill};
+  const RouteArgs r = {gate_logits, pre_bias_logits, T, E, k, mode, norm_topk_prob, weights_round_bf16, routed_scaling_factor, 0, 0, topk_weights, topk_idx};
+  if (T <= kSortWaves)
+    route_sort_small_kernel<kSortWaves><<<1, kSortWaves * kWave, 0, (hipStream_t)stream>>>(r, roll_to_expert_id, ebits, group_sizes, perm, inv_perm,
+                                                                                            sorted_experts, mp);
+  else
+    route_sort_small_kernel<4 * kSortWaves><<<1, 4 * kSortWaves * kWave, 0, (hipStream_t)stream>>>(r, roll_to_expert_id, ebits, group_sizes, perm,
+                                                                                                    inv_perm, sorted_experts, mp);
+  if (int st = check_launch("route_sort_small_kernel")) return st;
+  note_tile_map_built(gmm_workspace, group_sizes, (int)M, E, group_offset, num_groups_local, tile_rows, zero_fill);
+  return MOE_OK;
 }
 
 int moe_sort_by_expert(const int32_t* topk_idx, int T, int k, int E, int32_t* perm,

@@ -53,6 +53,37 @@ def route_topk(gate_logits, pre_bias_logits=None, *, k, mode="softmax_topk", nor
   return w, idx
 
 
+def route_sort(gate_logits, pre_bias_logits=None, *, k, gmm_workspace, mode="softmax_topk", norm_topk_prob=False, weights_round_bf16=True,
+               routed_scaling_factor=1.0, n_routing_groups=-1, topk_routing_group=-1, roll_to_expert_id=0, tile_rows=16):
+  """route_topk and sort_by_expert(..., gmm_workspace=...) through one call (one launch up to 16 tokens):
+  -> (weights [T,k] f32, indices [T,k] int32, perm [M], inv_perm [M], group_sizes [E]), as those two return them."""
+  _need(gate_logits, "gate_logits", torch.float32, 2)
+  t, e = gate_logits.shape
+  if mode not in _lib.ROUTE_BY_NAME:
+    raise ValueError(f"unknown routing mode {mode!r}")
+  if mode == "deepseek":
+    _need(pre_bias_logits, "pre_bias_logits", torch.float32, 2)
+    if pre_bias_logits.shape != gate_logits.shape:
+      raise ValueError("pre_bias_logits must match gate_logits")
+  _need(gmm_workspace, "gmm_workspace", torch.uint8)
+  dev = gate_logits.device
+  m = t * k
+  w = torch.empty((t, k), dtype=torch.float32, device=dev)
+  idx = torch.empty((t, k), dtype=torch.int32, device=dev)
+  perm = torch.empty((m,), dtype=torch.int32, device=dev)
+  inv = torch.empty((m,), dtype=torch.int32, device=dev)
+  gs = torch.empty((e,), dtype=torch.int32, device=dev)
+  lib = _lib.load()
+  ws = torch.empty((max(lib.moe_sort_workspace_bytes(t, k, e), 16),), dtype=torch.uint8, device=dev)
+  st = lib.moe_route_sort_mapped(_lib.ptr(gate_logits), _lib.ptr(pre_bias_logits) if mode == "deepseek" else None, t, e, k, _lib.ROUTE_BY_NAME[mode],
+                                 int(bool(norm_topk_prob)), int(bool(weights_round_bf16)), float(routed_scaling_factor), int(n_routing_groups),
+                                 int(topk_routing_group), _lib.ptr(w), _lib.ptr(idx), int(roll_to_expert_id), _lib.ptr(perm), _lib.ptr(inv),
+                                 _lib.ptr(gs), None, _lib.ptr(ws), ws.numel(), int(tile_rows), e, 0, 0, _lib.ptr(gmm_workspace),
+                                 gmm_workspace.numel(), _lib.current_stream())
+  _lib.check(st, "moe_route_sort_mapped")
+  return w, idx, perm, inv, gs
+
+
 _SCORE_FUNC_CODE = {"": 0, "sigmoid": 1, "sqrtsoftplus": 2}
 
 

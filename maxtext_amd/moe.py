@@ -240,6 +240,23 @@ class RoutedMoE:
       w = self._weights_with_grad(gate_logits, pre_bias_logits, idx.reshape(*shape, k))
     return w.reshape(*shape, k), idx.reshape(*shape, k)
 
+  def _get_topk_sorted(self, gate_logits, pre_bias_logits, ws):
+    """get_topk and the sort of permute through one library call (one launch at decode sizes): -> (weights [..., k],
+    indices [..., k], perm, inv_perm, group_sizes).  For calls without hash routing and without gradients."""
+    cfg = self.config
+    shape, k = gate_logits.shape[:-1], self.num_experts_per_tok
+    g2 = gate_logits.reshape(-1, gate_logits.shape[-1]).float().contiguous()
+    if cfg.is_deepseek:
+      p2 = pre_bias_logits.reshape(g2.shape).float().contiguous()
+      w, idx, perm, inv, gs = kernels.route_sort(
+          g2, p2, k=k, gmm_workspace=ws, mode="deepseek", norm_topk_prob=cfg.routed_score_func in ("sigmoid", "sqrtsoftplus"),
+          routed_scaling_factor=cfg.routed_scaling_factor, n_routing_groups=cfg.n_routing_groups, topk_routing_group=cfg.topk_routing_group)
+    else:
+      w, idx, perm, inv, gs = kernels.route_sort(g2, k=k, gmm_workspace=ws, mode=cfg.route_mode, norm_topk_prob=cfg.norm_topk_prob,
+                                                 weights_round_bf16=cfg.route_mode != "topk_raw")
+      w = self._scale_per_expert(w, idx)
+    return w.reshape(*shape, k), idx.reshape(*shape, k), perm, inv, gs
+
   def _hash_routing(self, scores, input_ids):
     """Hash routing (moe.py:729-738): the experts of a token are read from a table indexed by its id, the weights are
     the scores at those experts, scaled as for DeepSeek (moe.py:767-773).  A table lookup and a gather: torch ops,
@@ -440,13 +457,19 @@ class RoutedMoE:
     b, s, d = inputs.shape
     k = self.num_experts_per_tok
     x2d = inputs.reshape(b * s, d).contiguous()
-    weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
-    x2d = self._scale_inputs_by_router_score(x2d, weights)
     # decode-sized calls: the sort leaves the tile list of the streaming matmul kernels (16-row tiles) behind, one launch less
     # (up to 16 rows per expert on average, where moe_gmm takes those kernels, and 4096 rows, the sort's one-launch limit)
     ws = kernels.gmm_workspace(b * s * k, self.num_experts, x2d.device) if b * s * k <= min(4096, 16 * self.num_experts) else None
-    perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
-                                                      want_sorted_experts=False, gmm_workspace=ws)
+    no_grad = not (torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (gate_logits, pre_bias_logits)))
+    if routing is None and ws is not None and self.tid2eid is None and no_grad and gate_logits is not None:
+      # ... and the routing runs in the sort's launch (one block does both up to 16 tokens)
+      weights, selected, perm, inv, group_size = self._get_topk_sorted(gate_logits, pre_bias_logits, ws)
+      x2d = self._scale_inputs_by_router_score(x2d, weights)
+    else:
+      weights, selected = routing if routing is not None else self.get_topk(gate_logits, pre_bias_logits, input_ids=input_ids)
+      x2d = self._scale_inputs_by_router_score(x2d, weights)
+      perm, inv, group_size, _ = kernels.sort_by_expert(selected.reshape(b * s, k).contiguous(), self.num_experts,
+                                                        want_sorted_experts=False, gmm_workspace=ws)
     training = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (x2d, weights, w0_kernel, w1_kernel, wo_kernel))
     if training:

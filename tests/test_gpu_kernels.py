@@ -1941,6 +1941,30 @@ def test_sort_leaves_the_tile_list_for_the_matmuls(K, t, e, k):
   assert torch.equal(y2, y)
 
 
+@pytest.mark.parametrize("t,e,k,mode", [(1, 32, 4, "softmax_topk"), (16, 32, 4, "softmax_topk"), (3, 128, 5, "topk_raw"), (13, 256, 8, "deepseek"),
+                                        (4, 8, 2, "softmax_all"), (5, 8, 2, "softmax_all"), (17, 32, 4, "softmax_topk"), (300, 32, 4, "softmax_topk")])
+def test_route_and_sort_in_one_call(K, t, e, k, mode):
+  """moe_route_sort_mapped: the weights and indices of moe_route_topk and the permutation, group sizes and tile list of
+  moe_sort_by_expert_mapped on those indices, bit for bit, as one launch (up to 16 tokens, with 4 or 16 waves) or as the
+  two calls (the last two cases); the flagged grouped matmul that follows equals one that maps for itself."""
+  g = torch.Generator(device="cuda").manual_seed(t * e + k)
+  logits = torch.randn((t, e), generator=g, device="cuda")
+  pre = torch.sigmoid(logits) if mode == "deepseek" else None
+  kw = dict(k=k, mode=mode, norm_topk_prob=mode != "topk_raw", routed_scaling_factor=2.5 if mode == "deepseek" else 1.0)
+  w0, idx0 = K.route_topk(logits, pre, **kw)
+  perm0, inv0, gs0, _ = K.sort_by_expert(idx0, e, want_sorted_experts=False)
+  ws = K.gmm_workspace(t * k, e, "cuda")
+  w, idx, perm, inv, gs = K.route_sort(logits, pre, gmm_workspace=ws, **kw)
+  for a, b in ((w, w0), (idx, idx0), (perm, perm0), (inv, inv0), (gs, gs0)):
+    assert torch.equal(a, b)
+  d, f = 128, 256
+  x = torch.randn((t * k, d), generator=g, device="cuda").to(torch.bfloat16)
+  wq = torch.randint(-127, 128, (e, f, d), generator=g, device="cuda", dtype=torch.int8)
+  sc = torch.rand((e, f), generator=g, device="cuda") * 0.01
+  y = K.gmm_raw(x, wq, gs, rhs_scale=sc, workspace=ws, same_groups=True)
+  assert torch.equal(y, K.gmm_raw(x, wq, gs0, rhs_scale=sc))
+
+
 def test_flagged_matmuls_after_a_sort_that_maps_nothing_use_the_new_groups(K):
   """Two steps on the SAME group_sizes / workspace buffers above 4096 routed rows (where the sort maps nothing), each a
   sort followed by two grouped matmuls flagged MOE_GMM_SAME_GROUPS, as a serving loop with persistent buffers issues
