@@ -404,7 +404,10 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
 #ifndef MOE_F8D_ROWS_HI
 #define MOE_F8D_ROWS_HI 14
 #endif
-    const bool f8d_ok = fp8_blocks && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
+    // (without block scales: per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
+    const bool f8d_epi = !fp8_blocks && !lhs_e5m2 && !kn_fp8 && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
+                         ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0);
+    const bool f8d_ok = (fp8_blocks || f8d_epi) && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
     const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8d_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
     // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
@@ -469,7 +472,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     p.header = header; p.tiles = tiles; p.out = a->out;
     p.M = M; p.K = K; p.N = N; p.act = a->act; p.act_limit = a->act_limit; p.ro = ro;
     p.min_rows = 1; p.max_rows = bm;
-    if (f8d_ok) return launch_f8d(p, glu, a->num_groups_local, s);
+    if (f8d_ok) return launch_f8d(p, glu, fp8_blocks ? 0 : 1, a->num_groups_local, s);
     return launch_fp8_skinny(few_rows, p, glu, max_tiles_for(M, G, bm), s);
   }
 
@@ -511,6 +514,23 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       return launch_dl(op, glu, 64, false, p, M, G, s);
     }
     if (kernel == MOE_GMM_KERNEL_STREAM || kernel == MOE_GMM_KERNEL_STREAM_NOSPLIT) return fail(MOE_ERR_UNSUPPORTED, "gmm: no streaming kernel for int8 x int8");
+    // int8 x int8 at decode sizes (up to 14 rows per expert on average): the LDS-streamed persistent kernel where it takes the
+    // shape (per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
+    if (op == OP_I8 && kernel == MOE_GMM_KERNEL_AUTO && (long long)M <= 14LL * G && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
+        ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0) && f8d_takes(K, N, a->num_groups_local, glu)) {
+      map_tiles(16);
+      SkinnyParams q = {};
+      q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
+      q.row_scale_lhs = sp.lhs_epi; q.row_scale_lhs_stride = sp.lhs_epi_stride;
+      q.ch_scale = (const float*)a->rhs_scale; q.ch_scale_up = (const float*)a->rhs_up_scale;
+      q.ch_gstride = sp.rhs_gstride; q.ch_nstride = sp.rhs_nstride;
+      q.rhs_bias = a->rhs_bias; q.rhs_up_bias = a->rhs_up_bias;
+      q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
+      q.header = header; q.tiles = tiles; q.out = a->out;
+      q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
+      q.min_rows = 1; q.max_rows = 16;
+      return launch_f8d(q, glu, 2, a->num_groups_local, s);
+    }
     TiledKind kind = pick_tiled_kind(op, BSRC_SAME, glu, M, K, N, G);
     if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64)) kind = K_T256;
     map_tiles(tiled_kind_bm(kind));

@@ -85,6 +85,37 @@ def test_gmm_fp8_row_by_channel_scales(K, shape, shared):
     assert relerr(got, other.cpu()) <= 2e-3  # the same products in another order of summation, rounded to bf16
 
 
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("m,k,n,gs", [(40, 1024, 128, [7, 0, 12, 1, 20]), (90, 3584, 328, [10, 25, 1, 16, 17, 9, 12]), (420, 512, 256, [1] * 300 + [100])])
+def test_gmm_fp8_row_by_channel_scales_at_decode_sizes(K, m, k, n, gs, shared):
+  """e4m3 x e4m3 with [m] x [n] scales at a handful of rows per expert: the LDS-streamed persistent kernel (row and channel
+  scales applied to the finished sums) against the oracle and against the register-staged kernel; both projections with
+  an activation, biases, f32 output and rows read through an index."""
+  lhs, w, gs = _problem(m, k, n, gs, 41)
+  g = torch.Generator().manual_seed(42)
+  w_up = torch.randn(len(gs), n, k, generator=g) * 0.05
+  lq, ls = _rows_fp8(lhs)
+  rq, rs = _channels_fp8(w, shared)
+  uq, us = _channels_fp8(w_up, shared)
+  kw = dict(lhs_scale=cuda(ls), rhs_scale=cuda(rs), rhs_scale_block_n=1, rhs_scale_block_k=0, rhs_scale_shared=shared)
+  got = K.gmm_raw(cuda(lq), cuda(rq), cuda(gs), **kw)
+  assert relerr(got, O.gmm(lq, rq, gs, lhs_scale=ls, rhs_scale=rs, transpose_rhs=True)) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  old = K.gmm_raw(cuda(lq), cuda(rq), cuda(gs), kernel="stream", **kw)
+  assert relerr(got, old.cpu()) <= 8e-3  # the same products in another order of summation, rounded to bf16
+  b0, b1 = torch.randn(len(gs), n, generator=g) * 0.1, torch.randn(len(gs), n, generator=g) * 0.1
+  t_rows = max(m // 3, 1)
+  idx = torch.randint(0, t_rows * 3, (m,), generator=g, dtype=torch.int32)
+  rows = (idx // 3).long()
+  got = K.gmm_raw(cuda(lq[:t_rows]), cuda(rq), cuda(gs), lhs_scale=cuda(ls[:t_rows]), rhs_scale=cuda(rs), rhs_up=cuda(uq), rhs_up_scale=cuda(us),
+                  rhs_scale_block_n=1, rhs_scale_block_k=0, rhs_scale_shared=shared, act="swigluoai", act_limit=7.0, rhs_bias=cuda(b0),
+                  rhs_up_bias=cuda(b1), lhs_row_idx=cuda(idx), lhs_row_idx_div=3, out_dtype=torch.float32)
+  h0 = O.gmm(lq[rows], rq, gs, lhs_scale=ls[rows], rhs_scale=rs, transpose_rhs=True, rhs_bias=b0[:, None, :], out_dtype=torch.float32)
+  h1 = O.gmm(lq[rows], uq, gs, lhs_scale=ls[rows], rhs_scale=us, transpose_rhs=True, rhs_bias=b1[:, None, :], out_dtype=torch.float32)
+  want = O.apply_ffn_activation(h0, h1, "swigluoai", 7.0, out_dtype=torch.float32)
+  assert got.dtype == torch.float32 and relerr(got, want) <= TOL
+
+
 @pytest.mark.parametrize("act", ["silu", "swigluoai"])
 def test_gmm_fp8_channel_scales_fused_glu_bias_and_row_index(K, act):
   """The persistent fp8 kernel with rhs_up + activation, per-expert biases, f32 output and activation rows read through

@@ -483,6 +483,42 @@ def test_gmm_int8_int8(K, m, k, n, gs):
   assert relerr(got, want) <= TOL
 
 
+@pytest.mark.parametrize("m,k,n,gs", [(40, 1024, 128, [7, 0, 12, 1, 20]), (90, 3584, 328, [10, 25, 1, 16, 17, 9, 12]), (420, 512, 256, [1] * 300 + [100]),
+                                      (60, 4096, 256, [5, 0, 9, 14, 3, 11, 2, 16])])
+def test_gmm_int8_int8_at_decode_sizes(K, m, k, n, gs):
+  """int8 x int8 with per-row x per-channel scales at a handful of rows per expert: the LDS-streamed persistent kernel
+  (int32 sums, scales applied once) against the oracle and against the LDS-tiled kernel on the same operands; both
+  projections with an activation, biases, partial sums, f32 output and rows read through an index."""
+  lhs, w, w_up, gs = _gmm_inputs(m, k, n, gs, 33)
+  q, s = O.quantize_weight_int8(w)
+  qu, su = O.quantize_weight_int8(w_up)
+  lq, ls = O.quantize_rows_int8(lhs)
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s))
+  assert relerr(got, O.gmm(lq, q, gs, lhs_scale=ls, rhs_scale=s)) <= TOL
+  assert torch.all(got[int(gs.sum()):] == 0)
+  other = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s), kernel="tiled")
+  assert relerr(got, other.cpu()) <= 4e-3  # the same exact integer sums: at most the scale product's rounding apart, in bf16
+  g = torch.Generator().manual_seed(34)
+  b0, b1 = torch.randn(len(gs), n, generator=g), torch.randn(len(gs), n, generator=g)
+  p0, p1 = (torch.randn(m, n, generator=g) * 0.5).to(torch.bfloat16), (torch.randn(m, n, generator=g) * 0.5).to(torch.bfloat16)
+  got = K.gmm_raw(cuda(lq), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls), rhs_scale=cuda(s), rhs_up=cuda(native(qu)), rhs_up_scale=cuda(su),
+                  rhs_bias=cuda(b0), rhs_up_bias=cuda(b1), partial_sum=cuda(p0), partial_sum_up=cuda(p1), act="swigluoai", act_limit=7.0,
+                  out_dtype=torch.float32)
+  h0 = O.gmm(lq, q, gs, lhs_scale=ls, rhs_scale=s, rhs_bias=b0[:, None, :], out_dtype=torch.float32) + p0.float()
+  h1 = O.gmm(lq, qu, gs, lhs_scale=ls, rhs_scale=su, rhs_bias=b1[:, None, :], out_dtype=torch.float32) + p1.float()
+  want = O.apply_ffn_activation(h0, h1, "swigluoai", 7.0, out_dtype=torch.float32)
+  want[int(gs.sum()):] = 0
+  assert got.dtype == torch.float32 and relerr(got, want) <= TOL
+  t_rows = max(m // 3, 1)
+  idx = torch.randint(0, t_rows * 3, (m,), generator=g, dtype=torch.int32)
+  rows = (idx // 3).long()
+  got = K.gmm_raw(cuda(lq[:t_rows]), cuda(native(q)), cuda(gs), lhs_scale=cuda(ls[:t_rows]), rhs_scale=cuda(s), rhs_up=cuda(native(qu)),
+                  rhs_up_scale=cuda(su), act="silu", lhs_row_idx=cuda(idx), lhs_row_idx_div=3)
+  want = O.apply_ffn_activation(O.gmm(lq[rows], q, gs, lhs_scale=ls[rows], rhs_scale=s, out_dtype=torch.float32),
+                                O.gmm(lq[rows], qu, gs, lhs_scale=ls[rows], rhs_scale=su, out_dtype=torch.float32))
+  assert relerr(got, want) <= TOL
+
+
 def test_gmm_int8_exact_with_unit_scales(K):
   # integer operands, unit scales, |sum| < 256: the bf16 output must equal the integer product exactly
   g = torch.Generator().manual_seed(4)

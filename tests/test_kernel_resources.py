@@ -89,10 +89,10 @@ def test_lds_streamed_fp8_decode_kernel_uses_no_scratch_and_waits_only_where_wri
   vector-memory counter are the explicit ones per segment."""
   asm = _assembly("moe_gmm_f8d.hip", str(tmp_path))
   sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_f8d_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
-  assert len(sizes) == 28, sizes  # 14 row lengths (K = 512 .. 7168) x with / without the second projection
+  assert len(sizes) == 84, sizes  # 14 row lengths (K = 512 .. 7168) x with / without the second projection x three operand kinds
   assert all(int(b) == 0 for _, b in sizes), sizes
   parts = re.split(r"\n(_ZN3moe14gmm_f8d_kernel\w+):", asm)
-  assert len(parts) == 57
+  assert len(parts) == 169
   for i in range(1, len(parts), 2):
     body = parts[i + 1].split(".end_amdhsa_kernel")[0]
     barriers = [m.start() for m in re.finditer(r"s_barrier", body)]
