@@ -565,6 +565,14 @@ def main():
           "workload": o["config"]["workload"], "value": o["value"], "unit": o["unit"], "ms_per_step": o["ms_per_step"], "dtype": o["dtype"],
           "config": o["config"], "roofline": o["roofline"], "stage_ms": o["stage_ms"], "layer_gbps": o["layer_gbps"],
       })
+      if name == "c1":
+        # (a layer of 0.07 ms of kernels: issued call by call it is bound by the host's launches, so the same steps are also
+        # timed as replays of one captured HIP graph)
+        torch.cuda.empty_cache()
+        sub = argparse.Namespace(**{**vars(args), "graph": True, "gate": False})
+        o, _, olayer, _, _ = run_workload(sub, name)
+        del olayer
+        result["other_configs"][-1]["graph"] = {"ms_per_step": o["ms_per_step"], "value": o["value"], "unit": o["unit"], "roofline": o["roofline"]}
     # the decode half of the GPT-OSS token sweep (BASELINE's fifth configuration: 1, 16, 128, 1024 tokens; 4096 is the
     # line above): launch-bound sizes, so each is replayed as one captured HIP graph, once as it comes (the 0.4 GB of
     # weights partly live in the last-level cache from one replay to the next) and once with 1 GiB overwritten between
