@@ -491,3 +491,88 @@ def test_picked_kernel_against_the_tiled_kernel_on_random_large_shapes(K, family
       assert worst <= 2.0 ** (-6 if "out_row_scale" in kw else -7) * top, f"{tag}: {worst} of {top}"
     else:
       assert torch.equal(got, ref), tag
+
+
+@pytest.mark.parametrize("family", ["int4", "mxfp4", "fp8", "fp8c", "int8"])
+def test_lds_streamed_decode_kernels_against_the_other_kernels_on_random_shapes(K, family):
+  """10 random decode-sized shapes per operand family the persistent LDS-streamed kernels take (4 to 40 groups of 0 to 16
+  rows, now and then a group of several tiles, or ~300 groups of a row or two with a last group of several tiles: the
+  shape of a layer with a shared expert, whose tiles the fp8 kernel hands to blocks of their own; rows in no group; K over
+  the kernels' whole range, N with a channel tail; with and without the fused activation, rows read through an index, a
+  window of the groups) against another kernel of the library on the same operands: the register-staged streaming kernel
+  (4-bit, fp8 with block scales) or the LDS-tiled one (fp8 / int8 with row and channel scales), which the small-shape
+  tests pin to the oracle.  The sums over K are formed in another order: one bf16 step of the largest value."""
+  from maxtext_amd._lib import MOE_INT4, MOE_MXFP4
+
+  rng = np.random.default_rng(1700 + sum(map(ord, family)))
+  g = torch.Generator(device="cuda").manual_seed(6)
+  rand = lambda *shape: torch.rand(*shape, device="cuda", generator=g)
+  randn = lambda *shape: torch.randn(*shape, device="cuda", generator=g)
+  bytes_ = lambda lo, hi, shape, dt: torch.randint(lo, hi, shape, device="cuda", dtype=dt, generator=g)
+  four_bit = family in ("int4", "mxfp4")
+  for case in range(10):
+    many = case % 5 == 4  # the shared-expert shape
+    e = int(rng.integers(260, 330)) if many else int(rng.integers(4, 41))
+    if four_bit:
+      k = int(rng.integers(1, 25)) * 128 if family == "int4" else int(rng.integers(4, 97)) * 32
+      if family == "int4" and rng.random() < 0.3:
+        k = 2880
+    else:
+      k = 512 if many else int(rng.integers(1, 15)) * 512
+    n = int(rng.integers(16, 48)) * 8 if many else int(rng.integers(32, 80)) * 8
+    gs = rng.integers(0, 3, e) if many else rng.integers(0, 17, e)
+    if many:
+      gs[-1] = int(rng.integers(20, 200))
+    elif rng.random() < 0.5:
+      gs[rng.integers(0, e)] = int(rng.integers(17, 60))
+    if int(gs.sum()) > 13 * e:  # stay where the library takes the decode kernels
+      gs = gs // 2
+    m = max(int(gs.sum()) + int(rng.integers(0, 20)), 1)
+    glu = bool(rng.integers(0, 2))
+    kw = {}
+    lhs = randn(m, k).to(torch.bfloat16)
+    if family == "int4":
+      ws = [(bytes_(0, 256, (e, n, k // 2), torch.uint8), (rand(e, n, (k + 127) // 128) * 0.01 + 1e-3).to(torch.bfloat16)) for _ in range(2)]
+      kw.update(rhs_dtype=MOE_INT4, rhs_scale_block_k=128)
+    elif family == "mxfp4":
+      ws = [(bytes_(0, 256, (e, n, k // 2), torch.uint8), bytes_(118, 126, (e, n, k // 32), torch.uint8)) for _ in range(2)]
+      kw.update(rhs_dtype=MOE_MXFP4, rhs_scale_block_k=32)
+    elif family == "fp8":
+      lhs = (randn(m, k) * 2).to(torch.float8_e4m3fn)
+      kw.update(lhs_scale=rand(m, k // 128) * 0.02 + 1e-3, lhs_scale_block_k=128, rhs_scale_block_n=128, rhs_scale_block_k=128)
+      ws = [((randn(e, n, k) * 2).to(torch.float8_e4m3fn), rand(e, (n + 127) // 128, k // 128) * 0.02 + 1e-3) for _ in range(2)]
+    elif family == "fp8c":
+      lhs = (randn(m, k) * 2).to(torch.float8_e4m3fn)
+      kw.update(lhs_scale=rand(m) * 0.02 + 1e-3, rhs_scale_block_n=1, rhs_scale_block_k=0)
+      ws = [((randn(e, n, k) * 2).to(torch.float8_e4m3fn), rand(e, n) * 0.02 + 1e-3) for _ in range(2)]
+    else:
+      lhs = bytes_(-127, 128, (m, k), torch.int8)
+      kw["lhs_scale"] = rand(m) * 0.01 + 1e-3
+      ws = [(bytes_(-127, 128, (e, n, k), torch.int8), rand(e, n) * 0.01 + 1e-3) for _ in range(2)]
+    opts = []
+    if rng.random() < 0.5:
+      div = int(rng.integers(1, 4))
+      src = torch.randperm(m, device="cuda", generator=g)[: m // div + 1]
+      lhs = lhs[src].contiguous()
+      if "lhs_scale" in kw:
+        kw["lhs_scale"] = kw["lhs_scale"][src].contiguous()
+      kw.update(lhs_row_idx=cuda(rng.integers(0, (m // div + 1) * div, m).astype(np.int32)), lhs_row_idx_div=div, num_rows=m)
+      opts.append(f"index / {div}")
+    lo, hi = 0, int(gs.sum())
+    if rng.random() < 0.3 and not many:
+      off = int(rng.integers(0, e // 2))
+      loc = int(rng.integers(1, e - off + 1))
+      ws = [(w[off:off + loc].clone(), sc[off:off + loc].clone()) for w, sc in ws]
+      kw["group_offset"] = off
+      lo, hi = int(gs[:off].sum()), int(gs[:off + loc].sum())
+      opts.append(f"groups {off} .. {off + loc - 1}")
+    kw["rhs_scale"] = ws[0][1]
+    if glu:
+      kw.update(rhs_up=ws[1][0], rhs_up_scale=ws[1][1], act="silu")
+    tag = f"{family} case {case}: m={m} k={k} n={n} glu={glu} {opts} group_sizes={gs.tolist()}"
+    got = K.gmm_raw(lhs, ws[0][0], cuda(gs.astype(np.int32)), **kw)
+    ref = K.gmm_raw(lhs, ws[0][0], cuda(gs.astype(np.int32)), kernel="stream" if four_bit or family == "fp8" else "tiled", **kw)
+    assert torch.all(got[:lo] == 0) and torch.all(got[hi:] == 0), tag
+    assert not torch.isnan(got.float()).any(), tag
+    worst, top = float((got.float() - ref.float()).abs().max()), float(ref.float().abs().max())
+    assert worst <= 2.0 ** -7 * top, f"{tag}: {worst} of {top}"
