@@ -444,7 +444,7 @@ typedef enum {
   MOE_GMM_KERNEL_AUTO = 0,
   MOE_GMM_KERNEL_STREAM = 1,    /* register-staged streaming kernels (fp8 block-scaled, weight-only formats); AUTO
                                    prefers the persistent kernels that stream the weights through LDS where they take
-                                   the shape (group-128 int4, MXFP4, block-scaled fp8 with K % 512 == 0, K <= 7168)   */
+                                   the shape (group-128 int4, MXFP4, 8-bit x 8-bit operands with K % 512 == 0)        */
   MOE_GMM_KERNEL_TILED = 2,     /* LDS-tiled kernels with the m-tile chosen by rows per expert (fp8: 128 x 128)       */
   MOE_GMM_KERNEL_BIG = 3,       /* 256 x 256 tiles: fp8 block-scaled (the persistent stream kernel when K % 512 == 0,
                                    what AUTO picks for prefill-sized groups); int8 x int8 register-staged kernel       */

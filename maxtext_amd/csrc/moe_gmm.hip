@@ -408,7 +408,9 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     const bool f8d_epi = !fp8_blocks && !lhs_e5m2 && !kn_fp8 && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
                          ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0);
     const bool f8d_ok = (fp8_blocks || f8d_epi) && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
-    const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8d_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G : kernel != MOE_GMM_KERNEL_STREAM;
+    // (rows past that kernel's length: its variant with the activations beside the weights)
+    const bool f8l_ok = !f8d_ok && f8d_epi && kernel == MOE_GMM_KERNEL_AUTO && f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows);
+    const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8d_ok || f8l_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
     // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
     const bool chip_full = (long long)max_tiles_for(M, G, 256) * cdiv(N, glu ? 128 : 256) >= 128;
@@ -456,7 +458,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       const bool vec4 = fp8_blocks && (K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
       return launch_fp8_tiled(big, glu, vec4, P, M, G, s);
     }
-    const int bm = few_rows || f8d_ok ? 16 : 64;
+    const int bm = few_rows || f8d_ok || f8l_ok ? 16 : 64;
     map_tiles(bm);
     SkinnyParams p = {};
     p.lhs = (const uint8_t*)a->lhs; p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
@@ -473,6 +475,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     p.M = M; p.K = K; p.N = N; p.act = a->act; p.act_limit = a->act_limit; p.ro = ro;
     p.min_rows = 1; p.max_rows = bm;
     if (f8d_ok) return launch_f8d(p, glu, fp8_blocks ? 0 : 1, a->num_groups_local, s);
+    if (f8l_ok) return launch_f8l(p, glu, false, a->num_groups_local, s);
     return launch_fp8_skinny(few_rows, p, glu, max_tiles_for(M, G, bm), s);
   }
 
@@ -517,7 +520,8 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     // int8 x int8 at decode sizes (up to 14 rows per expert on average): the LDS-streamed persistent kernel where it takes the
     // shape (per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
     if (op == OP_I8 && kernel == MOE_GMM_KERNEL_AUTO && (long long)M <= 14LL * G && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
-        ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0) && f8d_takes(K, N, a->num_groups_local, glu)) {
+        ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0) &&
+        (f8d_takes(K, N, a->num_groups_local, glu) || f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows))) {
       map_tiles(16);
       SkinnyParams q = {};
       q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
@@ -529,6 +533,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       q.header = header; q.tiles = tiles; q.out = a->out;
       q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
       q.min_rows = 1; q.max_rows = 16;
+      if (!f8d_takes(K, N, a->num_groups_local, glu)) return launch_f8l(q, glu, true, a->num_groups_local, s);  // (rows past 7168 values)
       return launch_f8d(q, glu, 2, a->num_groups_local, s);
     }
     TiledKind kind = pick_tiled_kind(op, BSRC_SAME, glu, M, K, N, G);

@@ -10,6 +10,9 @@ namespace moe {
 bool f8d_takes(int K, int N, int G_local, bool glu);
 // kind: 0 = fp8 with block scales, 1 = fp8, 2 = int8 with per-row x per-channel scales (row_scale_lhs / ch_scale of the parameters)
 int launch_f8d(const SkinnyParams& p, bool glu, int kind, int num_groups_local, hipStream_t s);
+// The same operands (kinds 1 and 2) with rows of any multiple of 512 values: the activations travel beside the weights.
+bool f8l_takes(int K, int N, int G_local, bool glu, long long lhs_rows);
+int launch_f8l(const SkinnyParams& p, bool glu, bool int8, int num_groups_local, hipStream_t s);
 int prepare_f8d();
 
 }  // namespace moe
