@@ -399,17 +399,16 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     // groups of exactly 128 rows 1.94 against 1.70 ms, at 160 rows 2.05 against 2.54 ms; routed groups scatter around
     // their mean, and those over 128 rows cost the 128 x 128 kernel a second tile).
     const bool few_rows = (long long)M <= 16LL * G;
-    // block-scaled operands at decode sizes: the LDS-streamed persistent kernel where it takes the shape
-    // (MOE_GMM_KERNEL_STREAM keeps the register-staged one)
+    // decode sizes: the LDS-streamed persistent kernels where they take the shape, one for block-scaled operands, one for
+    // per-row x per-channel scales (MOE_GMM_KERNEL_STREAM keeps the register-staged kernel)
 #ifndef MOE_F8D_ROWS_HI
 #define MOE_F8D_ROWS_HI 14
 #endif
     // (without block scales: per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
     const bool f8d_epi = !fp8_blocks && !lhs_e5m2 && !kn_fp8 && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
                          ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0);
-    const bool f8d_ok = (fp8_blocks || f8d_epi) && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
-    // (rows past that kernel's length: its variant with the activations beside the weights)
-    const bool f8l_ok = !f8d_ok && f8d_epi && kernel == MOE_GMM_KERNEL_AUTO && f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows);
+    const bool f8d_ok = fp8_blocks && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
+    const bool f8l_ok = f8d_epi && kernel == MOE_GMM_KERNEL_AUTO && f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows);
     const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8d_ok || f8l_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
     // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
@@ -474,7 +473,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     p.header = header; p.tiles = tiles; p.out = a->out;
     p.M = M; p.K = K; p.N = N; p.act = a->act; p.act_limit = a->act_limit; p.ro = ro;
     p.min_rows = 1; p.max_rows = bm;
-    if (f8d_ok) return launch_f8d(p, glu, fp8_blocks ? 0 : 1, a->num_groups_local, s);
+    if (f8d_ok) return launch_f8d(p, glu, a->num_groups_local, s);
     if (f8l_ok) return launch_f8l(p, glu, false, a->num_groups_local, s);
     return launch_fp8_skinny(few_rows, p, glu, max_tiles_for(M, G, bm), s);
   }
@@ -521,7 +520,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     // shape (per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
     if (op == OP_I8 && kernel == MOE_GMM_KERNEL_AUTO && (long long)M <= 14LL * G && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
         ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0) &&
-        (f8d_takes(K, N, a->num_groups_local, glu) || f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows))) {
+        f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows)) {
       map_tiles(16);
       SkinnyParams q = {};
       q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
@@ -533,8 +532,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       q.header = header; q.tiles = tiles; q.out = a->out;
       q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
       q.min_rows = 1; q.max_rows = 16;
-      if (!f8d_takes(K, N, a->num_groups_local, glu)) return launch_f8l(q, glu, true, a->num_groups_local, s);  // (rows past 7168 values)
-      return launch_f8d(q, glu, 2, a->num_groups_local, s);
+      return launch_f8l(q, glu, true, a->num_groups_local, s);
     }
     TiledKind kind = pick_tiled_kind(op, BSRC_SAME, glu, M, K, N, G);
     if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64)) kind = K_T256;

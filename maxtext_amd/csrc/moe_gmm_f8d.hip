@@ -24,7 +24,6 @@ namespace moe {
 // ---------------------------------------------------------------------------------------
 
 constexpr int kF8dThreads = 512;
-enum { kF8dBlocks = 0, kF8dEpi = 1, kF8dI8 = 2 };  // operand kinds (launch_f8d's `kind`)
 constexpr int kF8dRing = 4;               // segment slots: one multiplied, three in flight
 constexpr int kF8dSegBytes = 64 * 512;    // 64 rows x 4 k-blocks x 128 B
 constexpr int kF8dMaxSeg = 14;            // K <= 7168: the activations of 14 k-blocks per wave fill 112 registers
@@ -46,14 +45,8 @@ __device__ __forceinline__ void f8d_copy(const v4i& rsrc, uint32_t voff, uint32_
     asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr) : "memory", "m0");
 }
 
-// OPK = kF8dBlocks: the scales above.  kF8dEpi: without them the operands carry one scale per activation row and one per output channel
-// (ops.py:241-260), applied to the finished sums: the MFMAs of all k-blocks add straight into the item's sums, the row's
-// scale is read with its activations, and the item's channel scales take the place of the block scales in LDS.
-// OPK = kF8dI8: int8 x int8 with the same per-row and per-channel scales: two v_mfma_i32_16x16x64_i8 per k-block, sums in
-// int32 until the four waves' parts are added.
-template <int NSEG, bool GLU, bool NT, int OPK>
+template <int NSEG, bool GLU, bool NT>
 __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams p, int num_groups) {
-  constexpr bool BLOCKS = OPK == kF8dBlocks, I8 = OPK == kF8dI8;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   static_assert(NSEG >= 1 && NSEG <= kF8dMaxSeg, "segments per item");
   constexpr int SRING = f8d_scale_ring(NSEG);
@@ -104,11 +97,11 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
 
   // weights and scales through buffer descriptors: a request past the end of a tensor returns zeros
   const uint32_t w_bytes = clamp_u32((size_t)num_groups * N * row_bytes);
-  const uint32_t s_bytes = BLOCKS ? clamp_u32((size_t)num_groups * nnb * nkb * 4) : clamp_u32(((size_t)(num_groups - 1) * p.ch_gstride + N) * 4);
+  const uint32_t s_bytes = clamp_u32((size_t)num_groups * nnb * nkb * 4);
   const v4i desc_w = buffer_desc(p.rhs, w_bytes);
   const v4i desc_u = buffer_desc(GLU ? p.rhs_up : p.rhs, w_bytes);
-  const v4i sdesc_w = buffer_desc(BLOCKS ? p.rhs_scale : p.ch_scale, s_bytes);
-  const v4i sdesc_u = buffer_desc(BLOCKS ? (GLU ? p.rhs_up_scale : p.rhs_scale) : (GLU ? p.ch_scale_up : p.ch_scale), s_bytes);
+  const v4i sdesc_w = buffer_desc(p.rhs_scale, s_bytes);
+  const v4i sdesc_u = buffer_desc(GLU ? p.rhs_up_scale : p.rhs_scale, s_bytes);
   const bool up_half = wave >= 4;  // this wave copies rows 32..63 of a segment: the second projection / channels 32..63
 
   // ---- the tile the run is in: record, expert of the next tile, activations and scales of this wave's k-blocks ----
@@ -116,7 +109,7 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
   TileInfo tile;
   int g_cur = 0, g_next = 0, shared_cur = 0, shared_next = 0;
   v8i act[NSEG];
-  float as[BLOCKS ? NSEG : 1];  // BLOCKS: the row's scale of each of this wave's k-blocks; else the row's one scale
+  float as[NSEG];
   auto load_tile = [&](int m) {
     // (read into scalar registers here: a load left pending would be waited for at its first use, behind the copies)
     const TileInfo t = p.tiles[m];
@@ -135,23 +128,21 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
     // lane (j, kq) takes bytes kq*16.. and 64 + kq*16.. of its row's k-block: the order the weight fragments are read in
     const int gr = lhs_row_of(p.ro, tile.row0 + min(j, tile.nrows - 1));
     const uint8_t* arow = p.lhs + (size_t)gr * K + kq * 16;
-    const float* asr = BLOCKS ? p.lhs_scale + (size_t)gr * nkb : nullptr;
+    const float* asr = p.lhs_scale + (size_t)gr * nkb;
 #pragma unroll
     for (int i = 0; i < NSEG; i++) {
       const int kb = 4 * i + ksub;
       const uint4 x = *(const uint4*)(arow + kb * 128), y = *(const uint4*)(arow + kb * 128 + 64);
       act[i][0] = x.x; act[i][1] = x.y; act[i][2] = x.z; act[i][3] = x.w;
       act[i][4] = y.x; act[i][5] = y.y; act[i][6] = y.z; act[i][7] = y.w;
-      if (BLOCKS) as[i] = asr[kb];
+      as[i] = asr[kb];
     }
-    if (!BLOCKS) as[0] = p.row_scale_lhs ? p.row_scale_lhs[(size_t)gr * p.row_scale_lhs_stride] : 1.0f;
     // the loads complete here (an empty statement that "uses" every register), not at their first use behind the copies
 #pragma unroll
     for (int i = 0; i < NSEG; i++) {
       asm volatile("" : "+v"(act[i]));
-      if (BLOCKS) asm volatile("" : "+v"(as[i]));
+      asm volatile("" : "+v"(as[i]));
     }
-    if (!BLOCKS) asm volatile("" : "+v"(as[0]));
   };
 
   // ---- copies of one stream position: segment s of item q into ring slot `slot` ----
@@ -172,8 +163,7 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
     if (s == 0 && wave % 4 == 0) {
       // the item's weight scales: the K/128 floats of its 128-channel block (a copy brings a whole KB: what follows
       // them is other blocks' scales, or zeros past the tensor)
-      // (without block scales: the scales of the item's channels, [g, n] f32 with n contiguous)
-      const uint32_t voff = (BLOCKS ? (uint32_t)((group * nnb + cg * CH / 128) * nkb) : (uint32_t)(group * p.ch_gstride + cg * CH)) * 4u + (uint32_t)lane * 16u;
+      const uint32_t voff = (uint32_t)((group * nnb + cg * CH / 128) * nkb) * 4u + (uint32_t)lane * 16u;
       f8d_copy<false>(up_half ? sdesc_u : sdesc_w, voff, lds_base + kF8dScale0 + (uint32_t)(it % SRING) * kF8dScaleBuf + (up_half ? 1024u : 0u));
     }
     // (channels past N in an item's last rows are the next expert's first rows, or zeros past the tensor: never stored)
@@ -206,7 +196,6 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
       load_acts();
     }
     v4f acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
-    v4i ig = {0, 0, 0, 0}, iu = {0, 0, 0, 0};  // (int8)
     const float* const sbuf = (const float*)(smem + kF8dScale0 + (it % SRING) * kF8dScaleBuf);
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
@@ -229,28 +218,16 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
       v8i wf, uf;
       wf[0] = w0.x; wf[1] = w0.y; wf[2] = w0.z; wf[3] = w0.w; wf[4] = w1.x; wf[5] = w1.y; wf[6] = w1.z; wf[7] = w1.w;
       uf[0] = u0.x; uf[1] = u0.y; uf[2] = u0.z; uf[3] = u0.w; uf[4] = u1.x; uf[5] = u1.y; uf[6] = u1.z; uf[7] = u1.w;
-      if constexpr (BLOCKS) {
-        const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, act[s], zero, 0, 0, 0, 127, 0, 127);
-        const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf, act[s], zero, 0, 0, 0, 127, 0, 127);
-        const float fg = as[s] * sbuf[kb], fu = as[s] * sbuf[256 + kb];
+      const v4f pg = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, act[s], zero, 0, 0, 0, 127, 0, 127);
+      const v4f pu = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf, act[s], zero, 0, 0, 0, 127, 0, 127);
+      const float fg = as[s] * sbuf[kb], fu = as[s] * sbuf[256 + kb];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          acc_g[r] = fmaf(pg[r], fg, acc_g[r]);
-          acc_u[r] = fmaf(pu[r], fu, acc_u[r]);
-        }
-        // (the sums are final here: left alone, the compiler keeps every segment's products to add them at the item's end)
-        asm volatile("" : "+v"(acc_g), "+v"(acc_u));
-      } else if constexpr (I8) {
-        // (each half of the lane's 32 bytes is one MFMA's 16: bytes kq*16.. of the k-block's first 64, then of its second 64)
-        const v4i a0 = {act[s][0], act[s][1], act[s][2], act[s][3]}, a1 = {act[s][4], act[s][5], act[s][6], act[s][7]};
-        ig = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{wf[0], wf[1], wf[2], wf[3]}, a0, ig, 0, 0, 0);
-        iu = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{uf[0], uf[1], uf[2], uf[3]}, a0, iu, 0, 0, 0);
-        ig = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{wf[4], wf[5], wf[6], wf[7]}, a1, ig, 0, 0, 0);
-        iu = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{uf[4], uf[5], uf[6], uf[7]}, a1, iu, 0, 0, 0);
-      } else {
-        acc_g = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, act[s], acc_g, 0, 0, 0, 127, 0, 127);
-        acc_u = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(uf, act[s], acc_u, 0, 0, 0, 127, 0, 127);
+      for (int r = 0; r < 4; r++) {
+        acc_g[r] = fmaf(pg[r], fg, acc_g[r]);
+        acc_u[r] = fmaf(pu[r], fu, acc_u[r]);
       }
+      // (the sums are final here: left alone, the compiler keeps every segment's products to add them at the item's end)
+      asm volatile("" : "+v"(acc_g), "+v"(acc_u));
     }
 
     // ---- sums of the waves ksub = 1..3 -> LDS -> wave (a, 0) ----
@@ -258,8 +235,8 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
       float* r = red + (size_t)((a * 3 + ksub - 1) * 8) * kWave + lane;
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        r[e * kWave] = I8 ? __int_as_float(ig[e]) : acc_g[e];
-        r[(4 + e) * kWave] = I8 ? __int_as_float(iu[e]) : acc_u[e];
+        r[e * kWave] = acc_g[e];
+        r[(4 + e) * kWave] = acc_u[e];
       }
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the sums are in LDS
@@ -270,27 +247,8 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
         const float* r = red + (size_t)((a * 3 + w) * 8) * kWave + lane;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          if (I8) {
-            ig[e] += __float_as_int(r[e * kWave]);
-            iu[e] += __float_as_int(r[(4 + e) * kWave]);
-          } else {
-            acc_g[e] += r[e * kWave];
-            acc_u[e] += r[(4 + e) * kWave];
-          }
-        }
-      }
-      if constexpr (I8) {  // the exact integer sums, converted once
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          acc_g[e] = (float)ig[e];
-          acc_u[e] = (float)iu[e];
-        }
-      }
-      if constexpr (!BLOCKS) {  // row scale x channel scale on the finished sums
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          acc_g[r] *= as[0] * sbuf[a * 16 + 4 * kq + r];
-          acc_u[r] *= as[0] * sbuf[(GLU ? 256 : 32) + a * 16 + 4 * kq + r];
+          acc_g[e] += r[e * kWave];
+          acc_u[e] += r[(4 + e) * kWave];
         }
       }
       const int n = cg * CH + a * 16 + 4 * kq;
@@ -335,11 +293,13 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8d_kernel(const SkinnyParams
 }
 
 // ---------------------------------------------------------------------------------------
-// Rows too long for resident activations (K > 7168: 14 k-blocks per wave are 112 registers): the same persistent stream with
-// the tile's activations travelling beside the weights.  A segment is 64 weight rows + the tile's 16 activation rows, 512 B
+// Operands with one scale per activation row and one per output channel (ops.py:241-260; float8_e4m3 or int8), applied to the
+// finished sums: the same persistent stream with the tile's activations travelling beside the weights instead of staying
+// in registers (rows of any length: 14 k-blocks per wave would be 112 registers at K = 7168 already).  A segment is 64 weight rows + the tile's 16 activation rows, 512 B
 // of each (40 KB), in a ring of three (two in flight); an item re-reads its tile's activation rows, which come from L2.
-// Nothing is kept per k-block, so the segment loop is an ordinary one and K is any multiple of 512.  Operands with one
-// scale per row and one per channel only (fp8 or int8).
+// Nothing is kept per k-block, so the segment loop is an ordinary one and K is any multiple of 512; the sums form in the
+// MFMA accumulators (int32 for int8: two v_mfma_i32_16x16x64_i8 per k-block), the row's scale is read with the tile, the
+// item's channel scales are copied to LDS with its first segment.  Measured level with resident activations where both apply.
 // ---------------------------------------------------------------------------------------
 
 constexpr int kF8lRing = 3;
@@ -562,64 +522,51 @@ bool f8d_takes(int K, int N, int G_local, bool glu) {
 #define MOE_F8D_NT 1
 #endif
 
-template <int NSEG, bool GLU, int OPK>
+template <int NSEG, bool GLU>
 static int launch_f8d_one(const SkinnyParams& p, int num_groups, int blocks, hipStream_t s) {
   constexpr bool NT = MOE_F8D_NT != 0;
-  if (int st = reserve_lds(gmm_f8d_kernel<NSEG, GLU, NT, OPK>, kF8dLds, lds_flags<std::integral_constant<int, 7500 + NSEG * 8 + (GLU ? 1 : 0) + OPK * 2>>()))
-    return st;
-  gmm_f8d_kernel<NSEG, GLU, NT, OPK><<<blocks, kF8dThreads, kF8dLds, s>>>(p, num_groups);
+  if (int st = reserve_lds(gmm_f8d_kernel<NSEG, GLU, NT>, kF8dLds, lds_flags<std::integral_constant<int, 7500 + NSEG * 2 + (GLU ? 1 : 0)>>())) return st;
+  gmm_f8d_kernel<NSEG, GLU, NT><<<blocks, kF8dThreads, kF8dLds, s>>>(p, num_groups);
   return check_launch("gmm_f8d_kernel");
 }
 
 template <int NSEG>
-static int launch_f8d_seg(const SkinnyParams& p, bool glu, int kind, int num_groups, int blocks, hipStream_t s) {
-  if (kind == kF8dBlocks) return glu ? launch_f8d_one<NSEG, true, kF8dBlocks>(p, num_groups, blocks, s) : launch_f8d_one<NSEG, false, kF8dBlocks>(p, num_groups, blocks, s);
-  if (kind == kF8dEpi) return glu ? launch_f8d_one<NSEG, true, kF8dEpi>(p, num_groups, blocks, s) : launch_f8d_one<NSEG, false, kF8dEpi>(p, num_groups, blocks, s);
-  return glu ? launch_f8d_one<NSEG, true, kF8dI8>(p, num_groups, blocks, s) : launch_f8d_one<NSEG, false, kF8dI8>(p, num_groups, blocks, s);
+static int launch_f8d_seg(const SkinnyParams& p, bool glu, int num_groups, int blocks, hipStream_t s) {
+  return glu ? launch_f8d_one<NSEG, true>(p, num_groups, blocks, s) : launch_f8d_one<NSEG, false>(p, num_groups, blocks, s);
 }
 
-// kind 0: fp8 with lhs_scale / rhs_scale as [M, K/128] / [G, N/128, K/128]; 1: fp8, 2: int8 with row_scale_lhs / ch_scale
-// (per channel, n contiguous, the experts' rows a multiple of 4 floats apart or shared, 16-byte aligned)
-int launch_f8d(const SkinnyParams& p, bool glu, int kind, int num_groups, hipStream_t s) {
-  if (kind < kF8dBlocks || kind > kF8dI8) return fail(MOE_ERR_INVALID_ARG, "gmm: operand kind %d of the LDS-streamed decode kernel", kind);
+int launch_f8d(const SkinnyParams& p, bool glu, int num_groups, hipStream_t s) {
   int cus = 0;
   if (int st = device_cu_count(&cus)) return st;
   switch (p.K / 512) {
-    case 1: return launch_f8d_seg<1>(p, glu, kind, num_groups, cus, s);
-    case 2: return launch_f8d_seg<2>(p, glu, kind, num_groups, cus, s);
-    case 3: return launch_f8d_seg<3>(p, glu, kind, num_groups, cus, s);
-    case 4: return launch_f8d_seg<4>(p, glu, kind, num_groups, cus, s);
-    case 5: return launch_f8d_seg<5>(p, glu, kind, num_groups, cus, s);
-    case 6: return launch_f8d_seg<6>(p, glu, kind, num_groups, cus, s);
-    case 7: return launch_f8d_seg<7>(p, glu, kind, num_groups, cus, s);
-    case 8: return launch_f8d_seg<8>(p, glu, kind, num_groups, cus, s);
-    case 9: return launch_f8d_seg<9>(p, glu, kind, num_groups, cus, s);
-    case 10: return launch_f8d_seg<10>(p, glu, kind, num_groups, cus, s);
-    case 11: return launch_f8d_seg<11>(p, glu, kind, num_groups, cus, s);
-    case 12: return launch_f8d_seg<12>(p, glu, kind, num_groups, cus, s);
-    case 13: return launch_f8d_seg<13>(p, glu, kind, num_groups, cus, s);
-    case 14: return launch_f8d_seg<14>(p, glu, kind, num_groups, cus, s);
+    case 1: return launch_f8d_seg<1>(p, glu, num_groups, cus, s);
+    case 2: return launch_f8d_seg<2>(p, glu, num_groups, cus, s);
+    case 3: return launch_f8d_seg<3>(p, glu, num_groups, cus, s);
+    case 4: return launch_f8d_seg<4>(p, glu, num_groups, cus, s);
+    case 5: return launch_f8d_seg<5>(p, glu, num_groups, cus, s);
+    case 6: return launch_f8d_seg<6>(p, glu, num_groups, cus, s);
+    case 7: return launch_f8d_seg<7>(p, glu, num_groups, cus, s);
+    case 8: return launch_f8d_seg<8>(p, glu, num_groups, cus, s);
+    case 9: return launch_f8d_seg<9>(p, glu, num_groups, cus, s);
+    case 10: return launch_f8d_seg<10>(p, glu, num_groups, cus, s);
+    case 11: return launch_f8d_seg<11>(p, glu, num_groups, cus, s);
+    case 12: return launch_f8d_seg<12>(p, glu, num_groups, cus, s);
+    case 13: return launch_f8d_seg<13>(p, glu, num_groups, cus, s);
+    case 14: return launch_f8d_seg<14>(p, glu, num_groups, cus, s);
   }
   return fail(MOE_ERR_UNSUPPORTED, "gmm: K = %d is not a shape of the LDS-streamed fp8 decode kernel", p.K);
 }
 
-template <int NSEG, int OPK>
+template <int NSEG>
 static int prepare_f8d_pair() {
   constexpr bool NT = MOE_F8D_NT != 0;
-  if (int st = reserve_lds(gmm_f8d_kernel<NSEG, true, NT, OPK>, kF8dLds, lds_flags<std::integral_constant<int, 7500 + NSEG * 8 + 1 + OPK * 2>>())) return st;
-  return reserve_lds(gmm_f8d_kernel<NSEG, false, NT, OPK>, kF8dLds, lds_flags<std::integral_constant<int, 7500 + NSEG * 8 + OPK * 2>>());
-}
-
-template <int NSEG>
-static int prepare_f8d_set() {
-  if (int st = prepare_f8d_pair<NSEG, kF8dBlocks>()) return st;
-  if (int st = prepare_f8d_pair<NSEG, kF8dEpi>()) return st;
-  return prepare_f8d_pair<NSEG, kF8dI8>();
+  if (int st = reserve_lds(gmm_f8d_kernel<NSEG, true, NT>, kF8dLds, lds_flags<std::integral_constant<int, 7500 + NSEG * 2 + 1>>())) return st;
+  return reserve_lds(gmm_f8d_kernel<NSEG, false, NT>, kF8dLds, lds_flags<std::integral_constant<int, 7500 + NSEG * 2>>());
 }
 
 
-// The long-row variant: K any multiple of 512 (used past 7168), per-row x per-channel scales; the activation matrix
-// within 32-bit offsets as well
+// The per-row x per-channel kernel: K any multiple of 512, at least four channel groups per tile, weights and activations
+// within 32-bit offsets
 bool f8l_takes(int K, int N, int G_local, bool glu, long long lhs_rows) {
   const int ncg = cdiv(N, glu ? 32 : 64);
   return K % 512 == 0 && K >= 512 && N % 8 == 0 && ncg >= 4 && (long long)G_local * N * K + 65LL * K + 1024 < (1LL << 32) &&
@@ -651,20 +598,20 @@ static int prepare_f8l() {
 
 int prepare_f8d() {
   if (int st = prepare_f8l()) return st;
-  if (int st = prepare_f8d_set<1>()) return st;
-  if (int st = prepare_f8d_set<2>()) return st;
-  if (int st = prepare_f8d_set<3>()) return st;
-  if (int st = prepare_f8d_set<4>()) return st;
-  if (int st = prepare_f8d_set<5>()) return st;
-  if (int st = prepare_f8d_set<6>()) return st;
-  if (int st = prepare_f8d_set<7>()) return st;
-  if (int st = prepare_f8d_set<8>()) return st;
-  if (int st = prepare_f8d_set<9>()) return st;
-  if (int st = prepare_f8d_set<10>()) return st;
-  if (int st = prepare_f8d_set<11>()) return st;
-  if (int st = prepare_f8d_set<12>()) return st;
-  if (int st = prepare_f8d_set<13>()) return st;
-  return prepare_f8d_set<14>();
+  if (int st = prepare_f8d_pair<1>()) return st;
+  if (int st = prepare_f8d_pair<2>()) return st;
+  if (int st = prepare_f8d_pair<3>()) return st;
+  if (int st = prepare_f8d_pair<4>()) return st;
+  if (int st = prepare_f8d_pair<5>()) return st;
+  if (int st = prepare_f8d_pair<6>()) return st;
+  if (int st = prepare_f8d_pair<7>()) return st;
+  if (int st = prepare_f8d_pair<8>()) return st;
+  if (int st = prepare_f8d_pair<9>()) return st;
+  if (int st = prepare_f8d_pair<10>()) return st;
+  if (int st = prepare_f8d_pair<11>()) return st;
+  if (int st = prepare_f8d_pair<12>()) return st;
+  if (int st = prepare_f8d_pair<13>()) return st;
+  return prepare_f8d_pair<14>();
 }
 
 }  // namespace moe

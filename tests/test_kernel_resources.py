@@ -89,10 +89,10 @@ def test_lds_streamed_fp8_decode_kernel_uses_no_scratch_and_waits_only_where_wri
   vector-memory counter are the explicit ones per segment."""
   asm = _assembly("moe_gmm_f8d.hip", str(tmp_path))
   sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_f8d_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
-  assert len(sizes) == 84, sizes  # 14 row lengths (K = 512 .. 7168) x with / without the second projection x three operand kinds
+  assert len(sizes) == 28, sizes  # 14 row lengths (K = 512 .. 7168) x with / without the second projection
   assert all(int(b) == 0 for _, b in sizes), sizes
   parts = re.split(r"\n(_ZN3moe14gmm_f8d_kernel\w+):", asm)
-  assert len(parts) == 169
+  assert len(parts) == 57
   for i in range(1, len(parts), 2):
     body = parts[i + 1].split(".end_amdhsa_kernel")[0]
     barriers = [m.start() for m in re.finditer(r"s_barrier", body)]
@@ -101,7 +101,7 @@ def test_lds_streamed_fp8_decode_kernel_uses_no_scratch_and_waits_only_where_wri
     waits = re.findall(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", loop)
     assert set(waits) <= {"8", "4", "0"}, (parts[i], waits)
     assert "nt lds" in loop and re.search(r"offen lds", loop)  # weights read once stream past the caches, shared ones do not
-  # the long-row variant (activations beside the weights): four instantiations, no scratch, waits of 5 (the next segment's
+  # the kernel of the per-row x per-channel scales (activations copied beside the weights): four instantiations, no scratch, waits of 5 (the next segment's
   # copies may be outstanding) or 0 between its barriers
   sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_f8l_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
   assert len(sizes) == 4 and all(int(b) == 0 for _, b in sizes), sizes
