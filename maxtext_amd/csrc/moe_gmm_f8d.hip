@@ -1,4 +1,5 @@
-// Grouped matmul, decode sizes: block-scaled fp8 x fp8 with the weights streamed through LDS.
+// Grouped matmul, decode sizes: 8-bit x 8-bit operands with the weights streamed through LDS (gmm_f8d_kernel: block-scaled
+// fp8; gmm_f8l_kernel: fp8 or int8 with per-row x per-channel scales).
 
 #include "moe_gmm_f8d.h"
 
