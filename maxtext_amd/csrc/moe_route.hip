@@ -459,6 +459,48 @@ __device__ __forceinline__ void sort_small_block(
   constexpr int NT = NW * kWave;
   roll = resolve_roll(roll, roll_dev, E);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (M <= kWave && E <= kWave) {
+    // The smallest decode steps (at most 64 routed rows over at most 64 experts): one wave holds an entry and an expert per
+    // lane and sorts without a block barrier or a trip through memory: equal keys found by ballots, their count left in LDS
+    // by the first of them, the experts' first rows by a scan over the lanes.  The tile list is then built from the counts in LDS.
+    __shared__ int t_cnt[kWave], t_off[kWave];
+    if (wave == 0) {
+      const bool valid = lane < M;
+      const int e = valid ? sort_key(flat[lane], E, roll) : 0;
+      unsigned long long mask = __ballot(valid);
+      for (int b = 0; b < ebits; b++) {
+        const bool bit = (e >> b) & 1;
+        const unsigned long long bal = __ballot(valid && bit);
+        mask &= bit ? bal : ~bal;
+      }
+      const int rank = __popcll(mask & ((1ull << lane) - 1ull)), cnt = __popcll(mask);
+      t_cnt[lane] = 0;
+      __builtin_amdgcn_wave_barrier();
+      if (valid && rank == 0) t_cnt[e] = cnt;
+      __builtin_amdgcn_wave_barrier();
+      const int c = lane < E ? t_cnt[lane] : 0;
+      int incl = c;
+#pragma unroll
+      for (int o = 1; o < kWave; o <<= 1) {
+        const int t = __shfl_up(incl, o);
+        if (lane >= o) incl += t;
+      }
+      t_off[lane] = incl - c;
+      if (lane < E) group_sizes[lane] = c;
+      __builtin_amdgcn_wave_barrier();
+      if (valid) {
+        const int dest = t_off[e] + rank;
+        perm[dest] = lane;
+        if (inv_perm) inv_perm[lane] = dest;
+        if (sorted_experts) sorted_experts[dest] = e;
+      }
+    }
+    if (mp.tiles) {
+      __syncthreads();
+      build_tile_map<NT>(t_cnt, E, mp.group_offset, mp.G_local, M, mp.BM, mp.zero_fill, mp.header, mp.tiles, &run[0][0]);
+    }
+    return;
+  }
   // (only the E counters that exist are cleared, scanned and offset: with 32 experts of at most 1024 that is 5 scan steps
   // instead of 10, each between two barriers)
   for (int e = threadIdx.x; e < NW * E; e += NT) run[e / E][e % E] = 0;
