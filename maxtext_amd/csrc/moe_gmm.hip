@@ -409,7 +409,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
                          ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0);
     const bool f8d_ok = fp8_blocks && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
     const bool f8l_ok = f8d_epi && kernel == MOE_GMM_KERNEL_AUTO && f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows);
-    const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8d_ok || f8l_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G : kernel != MOE_GMM_KERNEL_STREAM;
+    // (the second of them also runs on 32-row tiles, two row tiles per weight segment)
+#ifndef MOE_F8L_ROWS_HI
+#define MOE_F8L_ROWS_HI 24
+#endif
+    const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8l_ok ? (long long)MOE_F8L_ROWS_HI : f8d_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G
+                                                     : kernel != MOE_GMM_KERNEL_STREAM;
     if (kernel > MOE_GMM_KERNEL_BIG) return fail(MOE_ERR_UNSUPPORTED, "gmm: kernel family %d does not take fp8 operands", kernel);
     // prefill-sized groups: the persistent 256 x 256 stream, where it takes the shape
     const bool chip_full = (long long)max_tiles_for(M, G, 256) * cdiv(N, glu ? 128 : 256) >= 128;
@@ -457,7 +462,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       const bool vec4 = fp8_blocks && (K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
       return launch_fp8_tiled(big, glu, vec4, P, M, G, s);
     }
-    const int bm = few_rows || f8d_ok || f8l_ok ? 16 : 64;
+    const int bm = f8l_ok ? ((long long)M <= 14LL * G ? 16 : 32) : few_rows || f8d_ok ? 16 : 64;
     map_tiles(bm);
     SkinnyParams p = {};
     p.lhs = (const uint8_t*)a->lhs; p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
@@ -474,7 +479,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
     p.M = M; p.K = K; p.N = N; p.act = a->act; p.act_limit = a->act_limit; p.ro = ro;
     p.min_rows = 1; p.max_rows = bm;
     if (f8d_ok) return launch_f8d(p, glu, a->num_groups_local, s);
-    if (f8l_ok) return launch_f8l(p, glu, false, a->num_groups_local, s);
+    if (f8l_ok) return launch_f8l(p, glu, false, bm, a->num_groups_local, s);
     return launch_fp8_skinny(few_rows, p, glu, max_tiles_for(M, G, bm), s);
   }
 
@@ -516,12 +521,13 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       return launch_dl(op, glu, 64, false, p, M, G, s);
     }
     if (kernel == MOE_GMM_KERNEL_STREAM || kernel == MOE_GMM_KERNEL_STREAM_NOSPLIT) return fail(MOE_ERR_UNSUPPORTED, "gmm: no streaming kernel for int8 x int8");
-    // int8 x int8 at decode sizes (up to 14 rows per expert on average): the LDS-streamed persistent kernel where it takes the
+    // int8 x int8 at decode sizes (16-row tiles up to 14 rows per expert on average, 32-row tiles above): the LDS-streamed persistent kernel where it takes the
     // shape (per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
-    if (op == OP_I8 && kernel == MOE_GMM_KERNEL_AUTO && (long long)M <= 14LL * G && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
+    if (op == OP_I8 && kernel == MOE_GMM_KERNEL_AUTO && (long long)M <= (long long)MOE_F8L_ROWS_HI * G && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
         ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0) &&
         f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows)) {
-      map_tiles(16);
+      const int bm = (long long)M <= 14LL * G ? 16 : 32;
+      map_tiles(bm);
       SkinnyParams q = {};
       q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;
       q.row_scale_lhs = sp.lhs_epi; q.row_scale_lhs_stride = sp.lhs_epi_stride;
@@ -531,8 +537,8 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       q.partial_sum = (const uint16_t*)a->partial_sum; q.partial_sum_up = (const uint16_t*)a->partial_sum_up;
       q.header = header; q.tiles = tiles; q.out = a->out;
       q.M = M; q.K = K; q.N = N; q.act = a->act; q.act_limit = a->act_limit; q.ro = ro;
-      q.min_rows = 1; q.max_rows = 16;
-      return launch_f8l(q, glu, true, a->num_groups_local, s);
+      q.min_rows = 1; q.max_rows = bm;
+      return launch_f8l(q, glu, true, bm, a->num_groups_local, s);
     }
     TiledKind kind = pick_tiled_kind(op, BSRC_SAME, glu, M, K, N, G);
     if (kernel == MOE_GMM_KERNEL_TILED && (kind == K_DL128 || kind == K_DL64)) kind = K_T256;

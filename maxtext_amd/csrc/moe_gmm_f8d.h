@@ -14,7 +14,7 @@ namespace moe {
 bool f8d_takes(int K, int N, int G_local, bool glu);
 int launch_f8d(const SkinnyParams& p, bool glu, int num_groups_local, hipStream_t s);
 bool f8l_takes(int K, int N, int G_local, bool glu, long long lhs_rows);
-int launch_f8l(const SkinnyParams& p, bool glu, bool int8, int num_groups_local, hipStream_t s);
+int launch_f8l(const SkinnyParams& p, bool glu, bool int8, int tile_rows, int num_groups_local, hipStream_t s);  // tiles of 16 or 32 rows
 int prepare_f8d();  // (both kernels)
 
 }  // namespace moe

@@ -486,7 +486,9 @@ def test_gmm_int8_int8(K, m, k, n, gs):
 @pytest.mark.parametrize("m,k,n,gs", [(40, 1024, 128, [7, 0, 12, 1, 20]), (90, 3584, 328, [10, 25, 1, 16, 17, 9, 12]), (420, 512, 256, [1] * 300 + [100]),
                                       (60, 4096, 256, [5, 0, 9, 14, 3, 11, 2, 16]),
                                       # rows past 7168 values: the variant whose activations travel beside the weights
-                                      (45, 7680, 136, [7, 0, 12, 1, 20]), (70, 14336, 256, [5, 0, 9, 14, 3, 11, 2, 16, 1])])
+                                      (45, 7680, 136, [7, 0, 12, 1, 20]), (70, 14336, 256, [5, 0, 9, 14, 3, 11, 2, 16, 1]),
+                                      # 15 to 28 rows per expert on average: 32-row tiles, two row tiles per weight segment
+                                      (100, 2048, 200, [32, 0, 17, 5, 31, 1]), (310, 1024, 128, [25] * 12), (130, 8192, 264, [33, 20, 64, 1, 0])])
 def test_gmm_int8_int8_at_decode_sizes(K, m, k, n, gs):
   """int8 x int8 with per-row x per-channel scales at a handful of rows per expert: the LDS-streamed persistent kernel
   (int32 sums, scales applied once) against the oracle and against the LDS-tiled kernel on the same operands; both
