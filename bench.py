@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0
 PROFILE_OF = {
     "c2": ("profiles/gmm_dls_kernel_int8_mixtral_prefill_c2.md", ["moe_gmm_dls.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c2f8": ("profiles/gmm_dls_kernel_fp8_mixtral_shape_prefill_c2f8.md", ["moe_gmm_dls.hip", "moe_gmm_common.h", "moe_common.h"]),
-    "c3": ("profiles/gmm_f8d_kernel_deepseek_decode_c3.md", ["moe_gmm_f8d.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c3": ("profiles/gmm_f8d_kernel_deepseek_decode_c3.md", ["moe_gmm_f8d.hip", "moe_gmm_f8d.h", "moe_gmm_common.h", "moe_common.h"]),
     "c4": ("profiles/gmm_dlw_kernel_int8w_qwen3_prefill_c4.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c5": ("profiles/gmm_dlw_kernel_int4w_gptoss_prefill_c5_t4096.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c2_train": ("profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md", ["moe_tgmm.hip", "moe_common.h"]),

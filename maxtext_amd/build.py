@@ -11,7 +11,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "lib", "libmoe_mi355x.so")
-SOURCES = ["moe_route.hip", "moe_gmm.hip", "moe_gmm_tiled.hip", "moe_gmm_dl.hip", "moe_gmm_dls.hip", "moe_gmm_dlw.hip", "moe_gmm_fp8.hip", "moe_gmm_f8s.hip", "moe_gmm_wq.hip", "moe_gmm_wqs.hip", "moe_gmm_f8d.hip", "moe_tgmm.hip", "moe_bwd.hip", "moe_dispatch.hip", "moe_quant.hip"]
+SOURCES = ["moe_route.hip", "moe_gmm.hip", "moe_gmm_tiled.hip", "moe_gmm_dl.hip", "moe_gmm_dls.hip", "moe_gmm_dlw.hip", "moe_gmm_fp8.hip", "moe_gmm_f8s.hip", "moe_gmm_wq.hip", "moe_gmm_wqs.hip", "moe_gmm_f8d.hip", "moe_gmm_f8l.hip", "moe_tgmm.hip", "moe_bwd.hip", "moe_dispatch.hip", "moe_quant.hip"]
 # benchmark-only helpers (machine calibration loops), linked into a library of their own
 CALIB_LIB_PATH = os.path.join(PKG_DIR, "lib", "libbench_calib.so")
 CALIB_SOURCE = "bench_calib.hip"

@@ -696,6 +696,7 @@ int moe_init(void) {
   if (int st = prepare_dls()) return st;
   if (int st = prepare_wqs()) return st;
   if (int st = prepare_f8d()) return st;
+  if (int st = prepare_f8l()) return st;
   if (int st = prepare_tgmm()) return st;
   if (int st = prepare_f8s()) return st;
   return prepare_fp8();

@@ -103,6 +103,7 @@ def test_lds_streamed_fp8_decode_kernel_uses_no_scratch_and_waits_only_where_wri
     assert "nt lds" in loop and re.search(r"offen lds", loop)  # weights read once stream past the caches, shared ones do not
   # the kernel of the per-row x per-channel scales (activations copied beside the weights): eight instantiations (16- and
   # 32-row tiles), no scratch, waits of 5 or 6 (the next segment's copies may be outstanding) or 0 between its barriers
+  asm = _assembly("moe_gmm_f8l.hip", str(tmp_path))
   sizes = re.findall(r"\.name:\s+(_ZN3moe14gmm_f8l_kernel\w+)\n\s+\.private_segment_fixed_size:\s+(\d+)", asm)
   assert len(sizes) == 8 and all(int(b) == 0 for _, b in sizes), sizes
   parts = re.split(r"\n(_ZN3moe14gmm_f8l_kernel\w+):", asm)
