@@ -132,8 +132,9 @@ def dominant_kernel_model(wl, group_sizes):
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name=("gmm_wqs_kernel" if wl.weight_quant == "int4" else "gmm_wq_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="bf16")
   op = "int8" if cfg.act_quant == "int8" else "fp8" if cfg.act_quant == "fp8_row" else "bf16"
-  if cfg.act_quant in ("int8", "fp8_row") and rows <= 14 * len(group_sizes) and d % 512 == 0:
-    # 8-bit x 8-bit with per-row x per-channel scales at decode sizes: the LDS-streamed persistent kernel, bound by the weights
+  if cfg.act_quant in ("int8", "fp8_row") and rows <= 48 * len(group_sizes) and d % 512 == 0:
+    # 8-bit x 8-bit with per-row x per-channel scales up to 48 rows per expert (the dispatch rule of moe_gmm): the LDS-streamed
+    # persistent kernel, bound by the weights
     w_bytes = nonempty * 2.0 * d * f
     return dict(bound="hbm", work=w_bytes + nonempty * 2.0 * f * 4 + rows * d * 1.0 + rows * f * 2.0, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name="gmm_f8l_kernel (wi_0|wi_1 + SwiGLU)", dtype=op)

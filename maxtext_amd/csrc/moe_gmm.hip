@@ -409,9 +409,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
                          ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0);
     const bool f8d_ok = fp8_blocks && kernel == MOE_GMM_KERNEL_AUTO && f8d_takes(K, N, a->num_groups_local, glu);
     const bool f8l_ok = f8d_epi && kernel == MOE_GMM_KERNEL_AUTO && f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows);
-    // (the second of them also runs on 32-row tiles, two row tiles per weight segment)
+    // (the second of them also runs on 32- and 64-row tiles, several row tiles per weight segment)
 #ifndef MOE_F8L_ROWS_HI
-#define MOE_F8L_ROWS_HI 24
+#define MOE_F8L_ROWS_HI 48  // 16-row tiles to 14 rows per expert on average, 32-row tiles to MOE_F8L_ROWS_32, 64-row tiles above
+#endif
+#ifndef MOE_F8L_ROWS_32
+#define MOE_F8L_ROWS_32 24
 #endif
     const bool tiled = kernel == MOE_GMM_KERNEL_AUTO ? (long long)M > (f8l_ok ? (long long)MOE_F8L_ROWS_HI : f8d_ok ? (long long)MOE_F8D_ROWS_HI : 14LL) * G
                                                      : kernel != MOE_GMM_KERNEL_STREAM;
@@ -462,7 +465,7 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       const bool vec4 = fp8_blocks && (K / 128) % 4 == 0 && ((uintptr_t)a->lhs_scale & 15) == 0;
       return launch_fp8_tiled(big, glu, vec4, P, M, G, s);
     }
-    const int bm = f8l_ok ? ((long long)M <= 14LL * G ? 16 : 32) : few_rows || f8d_ok ? 16 : 64;
+    const int bm = f8l_ok ? ((long long)M <= 14LL * G ? 16 : (long long)M <= (long long)MOE_F8L_ROWS_32 * G ? 32 : 64) : few_rows || f8d_ok ? 16 : 64;
     map_tiles(bm);
     SkinnyParams p = {};
     p.lhs = (const uint8_t*)a->lhs; p.rhs = (const uint8_t*)a->rhs; p.rhs_up = (const uint8_t*)a->rhs_up;
@@ -521,12 +524,12 @@ static int gmm_impl(const moe_gmm_args* a, void* workspace, size_t workspace_byt
       return launch_dl(op, glu, 64, false, p, M, G, s);
     }
     if (kernel == MOE_GMM_KERNEL_STREAM || kernel == MOE_GMM_KERNEL_STREAM_NOSPLIT) return fail(MOE_ERR_UNSUPPORTED, "gmm: no streaming kernel for int8 x int8");
-    // int8 x int8 at decode sizes (16-row tiles up to 14 rows per expert on average, 32-row tiles above): the LDS-streamed persistent kernel where it takes the
+    // int8 x int8 at decode sizes (16-row tiles up to 14 rows per expert on average, 32- and 64-row tiles above): the LDS-streamed persistent kernel where it takes the
     // shape (per-channel weight scales with n contiguous, the experts' rows whole 16-byte units apart)
     if (op == OP_I8 && kernel == MOE_GMM_KERNEL_AUTO && (long long)M <= (long long)MOE_F8L_ROWS_HI * G && sp.rhs_epi && sp.rhs_nstride == 1 && sp.rhs_gstride % 4 == 0 &&
         ((uintptr_t)a->rhs_scale & 15) == 0 && (!glu || ((uintptr_t)a->rhs_up_scale & 15) == 0) &&
         f8l_takes(K, N, a->num_groups_local, glu, ro.lhs_rows)) {
-      const int bm = (long long)M <= 14LL * G ? 16 : 32;
+      const int bm = (long long)M <= 14LL * G ? 16 : (long long)M <= (long long)MOE_F8L_ROWS_32 * G ? 32 : 64;
       map_tiles(bm);
       SkinnyParams q = {};
       q.lhs = (const uint8_t*)a->lhs; q.rhs = (const uint8_t*)a->rhs; q.rhs_up = (const uint8_t*)a->rhs_up;

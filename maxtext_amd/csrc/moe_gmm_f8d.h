@@ -5,7 +5,7 @@
 //   gmm_f8l_kernel (moe_gmm_f8l.hip): float8_e4m3 or int8 operands with one scale per row and one per output channel
 //                   (row_scale_lhs / ch_scale of the parameters: per channel, n contiguous, the experts' rows a multiple of
 //                   4 floats apart or shared, 16-byte aligned), the tile's activations copied beside the weights (K any
-//                   multiple of 512, tiles of 16 or 32 rows).
+//                   multiple of 512, tiles of 16, 32 or 64 rows).
 #pragma once
 
 #include "moe_gmm_common.h"
@@ -33,7 +33,7 @@ bool f8d_takes(int K, int N, int G_local, bool glu);
 int launch_f8d(const SkinnyParams& p, bool glu, int num_groups_local, hipStream_t s);
 int prepare_f8d();
 bool f8l_takes(int K, int N, int G_local, bool glu, long long lhs_rows);
-int launch_f8l(const SkinnyParams& p, bool glu, bool int8, int tile_rows, int num_groups_local, hipStream_t s);  // tiles of 16 or 32 rows
+int launch_f8l(const SkinnyParams& p, bool glu, bool int8, int tile_rows, int num_groups_local, hipStream_t s);  // tiles of 16, 32 or 64 rows
 int prepare_f8l();
 
 }  // namespace moe

@@ -15,37 +15,47 @@ namespace moe {
 // come from L2.  Nothing is kept per k-block, so the segment loop is an ordinary one, K is any multiple of 512, and a
 // second row tile costs 8 KB per segment and 16 accumulator registers.  The sums form in the MFMA accumulators (int32
 // for int8: two v_mfma_i32_16x16x64_i8 per k-block), the row's scale is read with the tile, the item's channel scales
-// are copied to LDS with its first segment.  Measured level with resident activations where both apply.
+// are copied to LDS with its first segment.  Measured level with resident activations where both apply.  64-row tiles
+// (25 to 48 rows per expert) run on segments half as wide, so that weights and activations of three segments in flight fit.
 // ---------------------------------------------------------------------------------------
 
-constexpr int kF8lRing = 3;
-// MT row tiles of 16 per item (tiles of 16 or 32 rows): a segment is 64 weight rows, then 16 * MT activation rows
+// MT row tiles of 16 per item (tiles of 16, 32 or 64 rows): a segment is 64 weight rows, then 16 * MT activation rows, KB
+// k-blocks of 128 bytes of each.  16- and 32-row tiles: four k-blocks, one per wave of a channel tile, ring of three.  64-row
+// tiles: two k-blocks (the rows would not fit otherwise), the four waves of a channel tile are two k-blocks x two pairs of row
+// tiles, ring of four, so that the same 96 KB are in flight.
 template <int MT>
 struct F8lLds {
-  static constexpr int kSegBytes = (64 + 16 * MT) * 512;
-  static constexpr int kHalfFloats = MT == 1 ? 256 : 64;  // an item's channel scales per half: the KB a copy brings, or (32-row tiles:
+  static constexpr int kKb = MT == 4 ? 2 : 4;
+  static constexpr int kRing = MT == 4 ? 4 : 3;
+  static constexpr int kSegWidth = kKb * 128;
+  static constexpr int kSegBytes = (64 + 16 * MT) * kSegWidth;
+  static constexpr int kHalfFloats = MT == 2 ? 64 : 256;  // an item's channel scales per half: the KB a copy brings, or (32-row tiles:
                                                           // LDS is full) the 256 B that 16 lanes bring
   static constexpr int kScaleBuf = 2 * kHalfFloats * 4;
-  static constexpr int kScale0 = kF8lRing * kSegBytes;
+  static constexpr int kScale0 = kRing * kSegBytes;
   static constexpr int kRed0 = kScale0 + 3 * kScaleBuf;
-  static constexpr int kBytes = kRed0 + kF8dRedBytes;  // 141312 / 161280 bytes
+  static constexpr int kBytes = kRed0 + kF8dRedBytes;  // 141312 / 161280 / 149504 bytes
   static_assert(kBytes <= 160 * 1024, "LDS");
 };
 
 template <bool GLU, bool NT, bool I8, int MT>
 __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams p, int num_groups) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  static_assert(MT == 1 || MT == 2, "16- or 32-row tiles");
+  static_assert(MT == 1 || MT == 2 || MT == 4, "16-, 32- or 64-row tiles");
   using L = F8lLds<MT>;
+  constexpr int KB = L::kKb, RING = L::kRing, AHEAD = RING - 1, SEGW = L::kSegWidth;
+  constexpr int NRP = 4 / KB, MTW = MT / NRP;  // groups of row tiles among the waves of a channel tile, row tiles per wave
+  constexpr int LPR = 8 * KB, RPI = kWave / LPR;  // lanes per segment row, rows per copy instruction
+  constexpr int WCOP = 8 / RPI, ACOP = 2 * MT / RPI;  // a wave's copy instructions per segment: weights, activations
   constexpr int CH = GLU ? 32 : 64;
   constexpr int SRING = 3;  // scale buffers: a copy two positions ahead is at most two items ahead
   constexpr int HF = L::kHalfFloats;
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int a = wave / 4, ksub = wave % 4;
+  const int a = wave / 4, ksub = wave % KB, rp = (wave % 4) / KB;
   const int j = lane % 16, kq = lane / 16;
   const int N = p.N, K = p.K;
-  const int nseg = K / 512;
+  const int nseg = K / SEGW;
   const uint32_t row_bytes = (uint32_t)K;
   const int ncg = (N + CH - 1) / CH;
   const int ntiles = __builtin_amdgcn_readfirstlane(p.header[0]);
@@ -65,14 +75,15 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams
   const bool up_half = wave >= 4;
 
   // ---- the tile the run is in and the one after it: experts, and where this lane's activation rows of each start ----
-  // (lane: row 16 t + 2 * wave + lane / 32 of the tile for copy t, row 16 t + lane % 16 for the scale of the finished sums)
+  // (lane: row 8 RPI t + RPI wave + lane / LPR of the tile for copy t, row 16 (MTW rp + t) + lane % 16 for the scale of the
+  // finished sums)
   int m_cur = q0 / ncg;
   TileInfo tile;
   int g_cur = 0, g_next = 0;
-  uint32_t aoff_cur[MT], aoff_next[MT];
-  float rs[MT];
-  const int crow = 2 * wave + lane / 32;
-  const uint32_t achunk = (uint32_t)((lane % 32) ^ (crow & 15)) * 16u;
+  uint32_t aoff_cur[ACOP], aoff_next[ACOP];
+  float rs[MTW];
+  const int crow = RPI * wave + lane / LPR;
+  const uint32_t achunk = (uint32_t)((lane % LPR) ^ (crow & 15)) * 16u;
   auto load_tile = [&](int m) {
     // (everything is read here, into registers that are used here: a load left pending would be waited for behind the copies)
     const TileInfo t = p.tiles[m];
@@ -84,49 +95,55 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams
     g_cur = max(tile.group, 0);
     g_next = m + 1 < ntiles ? max(__builtin_amdgcn_readfirstlane(tn.group), 0) : 0;
 #pragma unroll
-    for (int t2 = 0; t2 < MT; t2++) {
-      aoff_cur[t2] = (uint32_t)lhs_row_of(p.ro, tile.row0 + min(16 * t2 + crow, tile.nrows - 1)) * row_bytes + achunk;
-      aoff_next[t2] = (uint32_t)lhs_row_of(p.ro, n_row0 + min(16 * t2 + crow, n_nrows - 1)) * row_bytes + achunk;
-      const int gr = lhs_row_of(p.ro, tile.row0 + min(16 * t2 + j, tile.nrows - 1));
+    for (int t2 = 0; t2 < ACOP; t2++) {
+      aoff_cur[t2] = (uint32_t)lhs_row_of(p.ro, tile.row0 + min(8 * RPI * t2 + crow, tile.nrows - 1)) * row_bytes + achunk;
+      aoff_next[t2] = (uint32_t)lhs_row_of(p.ro, n_row0 + min(8 * RPI * t2 + crow, n_nrows - 1)) * row_bytes + achunk;
+      asm volatile("" : "+v"(aoff_cur[t2]), "+v"(aoff_next[t2]));
+    }
+#pragma unroll
+    for (int t2 = 0; t2 < MTW; t2++) {
+      const int gr = lhs_row_of(p.ro, tile.row0 + min(16 * (MTW * rp + t2) + j, tile.nrows - 1));
       rs[t2] = p.row_scale_lhs ? p.row_scale_lhs[(size_t)gr * p.row_scale_lhs_stride] : 1.0f;
-      asm volatile("" : "+v"(aoff_cur[t2]), "+v"(aoff_next[t2]), "+v"(rs[t2]));
+      asm volatile("" : "+v"(rs[t2]));
     }
   };
 
-  uint32_t lane_off[4];
+  uint32_t lane_off[WCOP];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int row = 8 * wave + 2 * i + lane / 32;
-    lane_off[i] = (uint32_t)(GLU ? row % 32 : row) * row_bytes + (uint32_t)((lane % 32) ^ (row & 15)) * 16u;
+  for (int i = 0; i < WCOP; i++) {
+    const int row = 8 * wave + RPI * i + lane / LPR;
+    lane_off[i] = (uint32_t)(GLU ? row % 32 : row) * row_bytes + (uint32_t)((lane % LPR) ^ (row & 15)) * 16u;
   }
   auto issue = [&](int pos) {
     const int it = pos / nseg, s = pos - it * nseg;
     const int q = q0 + it;
     const int m = q / ncg, cg = q - m * ncg;
-    const bool cur = m == m_cur;  // (two positions ahead never leave the next tile: ncg >= 4)
+    const bool cur = m == m_cur;  // (the positions ahead, at most two items on, never leave the next tile: ncg >= 4)
     const int group = cur ? g_cur : g_next;
     if (s == 0 && wave % 4 == 0) {
       const uint32_t voff = (uint32_t)(group * p.ch_gstride + cg * CH) * 4u + (uint32_t)lane * 16u;
       const uint32_t dst = lds_base + L::kScale0 + (uint32_t)(it % SRING) * L::kScaleBuf + (up_half ? (uint32_t)HF * 4u : 0u);
-      if (MT == 1) {
+      if (MT != 2) {
         f8d_copy<false>(up_half ? sdesc_u : sdesc_w, voff, dst);
       } else if (lane < 16) {  // (64 floats: the lanes that are switched off copy nothing)
         f8d_copy<false>(up_half ? sdesc_u : sdesc_w, voff, dst);
       }
     }
-    const uint32_t slot = lds_base + (uint32_t)(pos % kF8lRing) * L::kSegBytes;
-    const uint32_t base = (uint32_t)(group * N + cg * CH) * row_bytes + (uint32_t)s * 512u;
+    const uint32_t slot = lds_base + (uint32_t)(pos % RING) * L::kSegBytes;
+    const uint32_t base = (uint32_t)(group * N + cg * CH) * row_bytes + (uint32_t)(s * SEGW);
 #pragma unroll
-    for (int i = 0; i < 4; i++) f8d_copy<NT>(up_half ? desc_u : desc_w, base + lane_off[i], slot + (uint32_t)(8 * wave + 2 * i) * 512u);
-    // the tile's activation rows 16 t + 2 * wave and the one after it (read again by every item of the tile: temporal)
+    for (int i = 0; i < WCOP; i++)
+      f8d_copy<NT>(up_half ? desc_u : desc_w, base + lane_off[i], slot + (uint32_t)((8 * wave + RPI * i) * SEGW));
+    // the tile's activation rows 8 RPI t + RPI wave and the RPI - 1 after it (read again by every item of the tile: temporal)
 #pragma unroll
-    for (int t2 = 0; t2 < MT; t2++)
-      f8d_copy<false>(desc_a, (cur ? aoff_cur[t2] : aoff_next[t2]) + (uint32_t)s * 512u, slot + (uint32_t)(64 + 16 * t2 + 2 * wave) * 512u);
+    for (int t2 = 0; t2 < ACOP; t2++)
+      f8d_copy<false>(desc_a, (cur ? aoff_cur[t2] : aoff_next[t2]) + (uint32_t)(s * SEGW),
+                      slot + (uint32_t)((64 + 8 * RPI * t2 + RPI * wave) * SEGW));
   };
 
   load_tile(m_cur);
 #pragma unroll
-  for (int pos = 0; pos < 2; pos++)
+  for (int pos = 0; pos < AHEAD; pos++)
     if (pos < nstream) issue(pos);
 
   float* const red = (float*)(smem + L::kRed0);
@@ -137,31 +154,31 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams
       m_cur = m;
       load_tile(m);
     }
-    v4f acc_g[MT], acc_u[MT];
-    v4i ig[MT], iu[MT];
+    v4f acc_g[MTW], acc_u[MTW];
+    v4i ig[MTW], iu[MTW];
 #pragma unroll
-    for (int t2 = 0; t2 < MT; t2++) {
+    for (int t2 = 0; t2 < MTW; t2++) {
       acc_g[t2] = acc_u[t2] = v4f{0.f, 0.f, 0.f, 0.f};
       ig[t2] = iu[t2] = v4i{0, 0, 0, 0};
     }
     const float* const sbuf = (const float*)(smem + L::kScale0 + (it % SRING) * L::kScaleBuf);
     for (int s = 0; s < nseg; s++) {
       const int pos = it * nseg + s;
-      // this wave's copies of the segment (4 + MT, one more with the scales) have landed once at most those of the next
-      // segment are outstanding
-      if (pos + 1 < nstream) wait_vmcnt<4 + MT>();
+      // this wave's copies of the segment (WCOP + ACOP, one more, ahead of them, with the scales) have landed once at most
+      // those of the segments after it are outstanding
+      if (pos + AHEAD - 1 < nstream) wait_vmcnt<(AHEAD - 1) * (WCOP + ACOP)>();
       else wait_vmcnt<0>();
       asm volatile("s_barrier" ::: "memory");
-      if (pos + 2 < nstream) issue(pos + 2);
-      const uint8_t* slot = smem + (pos % kF8lRing) * L::kSegBytes;
+      if (pos + AHEAD < nstream) issue(pos + AHEAD);
+      const uint8_t* slot = smem + (pos % RING) * L::kSegBytes;
       const int c0 = (ksub * 8 + kq) ^ j, c1 = (ksub * 8 + 4 + kq) ^ j;
-      const uint8_t* wrow = slot + (a * 16 + j) * 512;
-      const uint8_t* urow = slot + (32 + a * 16 + j) * 512;
+      const uint8_t* wrow = slot + (a * 16 + j) * SEGW;
+      const uint8_t* urow = slot + (32 + a * 16 + j) * SEGW;
       const uint4 w0 = *(const uint4*)(wrow + c0 * 16), w1 = *(const uint4*)(wrow + c1 * 16);
       const uint4 u0 = *(const uint4*)(urow + c0 * 16), u1 = *(const uint4*)(urow + c1 * 16);
 #pragma unroll
-      for (int t2 = 0; t2 < MT; t2++) {
-        const uint8_t* arow = slot + (64 + 16 * t2 + j) * 512;
+      for (int t2 = 0; t2 < MTW; t2++) {
+        const uint8_t* arow = slot + (64 + 16 * (MTW * rp + t2) + j) * SEGW;
         const uint4 x0 = *(const uint4*)(arow + c0 * 16), x1 = *(const uint4*)(arow + c1 * 16);
         if constexpr (I8) {
           const v4i a0 = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w}, a1 = {(int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
@@ -180,12 +197,12 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams
       }
     }
 
-    // ---- per row tile: sums of the waves ksub = 1..3 -> LDS -> wave (a, 0), which runs the epilogue ----
+    // ---- per row tile: sums of the waves ksub > 0 -> LDS -> wave (a, rp, 0), which runs the epilogue ----
 #pragma unroll
-    for (int t2 = 0; t2 < MT; t2++) {
+    for (int t2 = 0; t2 < MTW; t2++) {
       if (t2 > 0) asm volatile("s_barrier" ::: "memory");  // the sums of the tile before have been read
       if (ksub > 0) {
-        float* r = red + (size_t)((a * 3 + ksub - 1) * 8) * kWave + lane;
+        float* r = red + (size_t)(((a * NRP + rp) * (KB - 1) + ksub - 1) * 8) * kWave + lane;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           r[e * kWave] = I8 ? __int_as_float(ig[t2][e]) : acc_g[t2][e];
@@ -198,8 +215,8 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams
         v4f sg = acc_g[t2], su = acc_u[t2];
         v4i jg = ig[t2], ju = iu[t2];
 #pragma unroll
-        for (int w = 0; w < 3; w++) {
-          const float* r = red + (size_t)((a * 3 + w) * 8) * kWave + lane;
+        for (int w = 0; w < KB - 1; w++) {
+          const float* r = red + (size_t)(((a * NRP + rp) * (KB - 1) + w) * 8) * kWave + lane;
 #pragma unroll
           for (int e = 0; e < 4; e++) {
             if (I8) {
@@ -217,7 +234,7 @@ __global__ __launch_bounds__(kF8dThreads) void gmm_f8l_kernel(const SkinnyParams
           su[r] = (I8 ? (float)ju[r] : su[r]) * (rs[t2] * sbuf[(GLU ? HF : 32) + a * 16 + 4 * kq + r]);
         }
         const int n = cg * CH + a * 16 + 4 * kq;
-        const int jr = 16 * t2 + j;
+        const int jr = 16 * (MTW * rp + t2) + j;
         const size_t row = (size_t)(tile.row0 + jr);
         if (jr < tile.nrows && tile.group < 0) {  // rows of no local group: zeros
           float z[4] = {0.f, 0.f, 0.f, 0.f};
@@ -287,12 +304,13 @@ static int launch_f8l_mt(const SkinnyParams& p, bool glu, bool int8, int num_gro
   return glu ? launch_f8l_one<true, false, MT>(p, num_groups, blocks, s) : launch_f8l_one<false, false, MT>(p, num_groups, blocks, s);
 }
 
-// tile_rows: the height of the tile list's tiles, 16 or 32
+// tile_rows: the height of the tile list's tiles, 16, 32 or 64
 int launch_f8l(const SkinnyParams& p, bool glu, bool int8, int tile_rows, int num_groups, hipStream_t s) {
   int cus = 0;
   if (int st = device_cu_count(&cus)) return st;
   if (tile_rows == 16) return launch_f8l_mt<1>(p, glu, int8, num_groups, cus, s);
   if (tile_rows == 32) return launch_f8l_mt<2>(p, glu, int8, num_groups, cus, s);
+  if (tile_rows == 64) return launch_f8l_mt<4>(p, glu, int8, num_groups, cus, s);
   return fail(MOE_ERR_INVALID_ARG, "gmm: tiles of %d rows for the 8-bit decode kernel", tile_rows);
 }
 
@@ -307,7 +325,8 @@ static int prepare_f8l_mt() {
 
 int prepare_f8l() {
   if (int st = prepare_f8l_mt<1>()) return st;
-  return prepare_f8l_mt<2>();
+  if (int st = prepare_f8l_mt<2>()) return st;
+  return prepare_f8l_mt<4>();
 }
 
 }  // namespace moe

@@ -88,7 +88,8 @@ def test_gmm_fp8_row_by_channel_scales(K, shape, shared):
 @pytest.mark.parametrize("shared", [True, False])
 @pytest.mark.parametrize("m,k,n,gs", [(40, 1024, 128, [7, 0, 12, 1, 20]), (90, 3584, 328, [10, 25, 1, 16, 17, 9, 12]), (420, 512, 256, [1] * 300 + [100]),
                                       (45, 7680, 136, [7, 0, 12, 1, 20]), (70, 14336, 256, [5, 0, 9, 14, 3, 11, 2, 16, 1]),  # (rows past 7168 values)
-                                      (100, 2048, 200, [32, 0, 17, 5, 31, 1]), (310, 1024, 128, [25] * 12)])  # (32-row tiles)
+                                      (100, 2048, 200, [32, 0, 17, 5, 31, 1]), (310, 1024, 128, [25] * 12),  # (32-row tiles)
+                                      (160, 2048, 200, [64, 0, 17, 5, 63, 1]), (200, 512, 256, [40] * 5), (200, 8192, 264, [65, 30, 64, 1, 0, 30])])  # (64-row)
 def test_gmm_fp8_row_by_channel_scales_at_decode_sizes(K, m, k, n, gs, shared):
   """e4m3 x e4m3 with [m] x [n] scales at a handful of rows per expert: the LDS-streamed persistent kernel (row and channel
   scales applied to the finished sums) against the oracle and against the register-staged kernel; both projections with

@@ -488,7 +488,10 @@ def test_gmm_int8_int8(K, m, k, n, gs):
                                       # rows past 7168 values: the variant whose activations travel beside the weights
                                       (45, 7680, 136, [7, 0, 12, 1, 20]), (70, 14336, 256, [5, 0, 9, 14, 3, 11, 2, 16, 1]),
                                       # 15 to 28 rows per expert on average: 32-row tiles, two row tiles per weight segment
-                                      (100, 2048, 200, [32, 0, 17, 5, 31, 1]), (310, 1024, 128, [25] * 12), (130, 8192, 264, [33, 20, 64, 1, 0])])
+                                      (100, 2048, 200, [32, 0, 17, 5, 31, 1]), (310, 1024, 128, [25] * 12), (130, 8192, 264, [33, 20, 64, 1, 0]),
+                                      # 25 to 48: 64-row tiles on segments of two k-blocks
+                                      (160, 2048, 200, [64, 0, 17, 5, 63, 1]), (380, 1024, 128, [37] * 10), (200, 512, 256, [40] * 5),
+                                      (200, 8192, 264, [65, 30, 64, 1, 0, 30])])
 def test_gmm_int8_int8_at_decode_sizes(K, m, k, n, gs):
   """int8 x int8 with per-row x per-channel scales at a handful of rows per expert: the LDS-streamed persistent kernel
   (int32 sums, scales applied once) against the oracle and against the LDS-tiled kernel on the same operands; both

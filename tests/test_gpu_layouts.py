@@ -496,7 +496,7 @@ def test_picked_kernel_against_the_tiled_kernel_on_random_large_shapes(K, family
 @pytest.mark.parametrize("family", ["int4", "mxfp4", "fp8", "fp8c", "int8"])
 def test_lds_streamed_decode_kernels_against_the_other_kernels_on_random_shapes(K, family):
   """10 random decode-sized shapes per operand family the persistent LDS-streamed kernels take (4 to 40 groups of 0 to 16
-  rows, now and then a group of several tiles, or ~300 groups of a row or two with a last group of several tiles: the
+  rows, now and then a group of several tiles, for the row and channel scales also groups of up to 70 rows, or ~300 groups of a row or two with a last group of several tiles: the
   shape of a layer with a shared expert, whose tiles the fp8 kernel hands to blocks of their own; rows in no group; K over
   the kernels' whole range, N with a channel tail; with and without the fused activation, rows read through an index, a
   window of the groups) against another kernel of the library on the same operands: the register-staged streaming kernel
@@ -528,6 +528,10 @@ def test_lds_streamed_decode_kernels_against_the_other_kernels_on_random_shapes(
       gs[rng.integers(0, e)] = int(rng.integers(17, 60))
     if int(gs.sum()) > 13 * e:  # stay where the library takes the decode kernels
       gs = gs // 2
+    if family in ("fp8c", "int8") and case % 3 == 1:  # 15 to 47 rows per group on average: the 32- and 64-row tiles of this kind's kernel
+      gs = rng.integers(8, 72, e) if case % 2 else rng.integers(0, 40, e)
+      while int(gs.sum()) > 47 * e:
+        gs = gs * 3 // 4
     m = max(int(gs.sum()) + int(rng.integers(0, 20)), 1)
     glu = bool(rng.integers(0, 2))
     kw = {}
