@@ -123,14 +123,15 @@ def dominant_kernel_model(wl, group_sizes):
     io_bytes = rows * d * 1.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
                 name=("gmm_f8d_kernel" if d % 512 == 0 and d <= 7168 else "gmm_fp8_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="fp8")
-  if wl.weight_quant in ("int4", "mxfp4") and rows <= (48 if wl.weight_quant == "int4" else 32) * cfg.num_experts:
-    # weight-only 4-bit decode (the dispatch rule of moe_gmm for its streaming kernels: group-128 int4 on the LDS-streamed
-    # persistent kernel, MXFP4 on the register-staged one): bound by streaming the weights of the experts that were hit
+  if wl.weight_quant in ("int4", "mxfp4") and rows <= 48 * cfg.num_experts:
+    # weight-only 4-bit decode (the dispatch rule of moe_gmm for its streaming kernels: group-128 int4 and MXFP4 with rows of
+    # up to 3072 values on the LDS-streamed persistent kernel, longer rows on the register-staged one): bound by streaming
+    # the weights of the experts that were hit
     w_bytes = nonempty * 2.0 * d * f * 0.5
     s_bytes = nonempty * 2.0 * f * (math.ceil(d / 128) * 2 if wl.weight_quant == "int4" else d / 32)
     io_bytes = rows * d * 2.0 + rows * f * 2.0
     return dict(bound="hbm", work=w_bytes + s_bytes + io_bytes, unit="GB/s", peak=PEAK_HBM_GBS, scale=1e9,
-                name=("gmm_wqs_kernel" if wl.weight_quant == "int4" else "gmm_wq_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="bf16")
+                name=("gmm_wqs_kernel" if d <= 3072 and d % 32 == 0 else "gmm_wq_skinny_kernel") + " (wi_0|wi_1 + SwiGLU)", dtype="bf16")
   op = "int8" if cfg.act_quant == "int8" else "fp8" if cfg.act_quant == "fp8_row" else "bf16"
   if cfg.act_quant in ("int8", "fp8_row") and rows <= 48 * len(group_sizes) and d % 512 == 0:
     # 8-bit x 8-bit with per-row x per-channel scales up to 48 rows per expert (the dispatch rule of moe_gmm): the LDS-streamed
