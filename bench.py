@@ -35,6 +35,8 @@ PROFILE_OF = {
     "c3": ("profiles/gmm_f8d_kernel_deepseek_decode_c3.md", ["moe_gmm_f8d.hip", "moe_gmm_f8d.h", "moe_gmm_common.h", "moe_common.h"]),
     "c4": ("profiles/gmm_dlw_kernel_int8w_qwen3_prefill_c4.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
     "c5": ("profiles/gmm_dlw_kernel_int4w_gptoss_prefill_c5_t4096.md", ["moe_gmm_dlw.hip", "moe_gmm_common.h", "moe_common.h"]),
+    "c2_t16": ("profiles/gmm_f8l_kernel_int8_mixtral_decode_c2_t16.md", ["moe_gmm_f8l.hip", "moe_gmm_f8d.h", "moe_gmm_common.h", "moe_common.h"]),
+    "c2_t128": ("profiles/gmm_f8l_kernel_int8_mixtral_decode_c2_t128.md", ["moe_gmm_f8l.hip", "moe_gmm_f8d.h", "moe_gmm_common.h", "moe_common.h"]),
     "c2_train": ("profiles/tgmm_dl_kernel_bf16_mixtral_shape_train.md", ["moe_tgmm.hip", "moe_common.h"]),
     "c2_train_fp8_full": ("profiles/fp8_full_train_step_mixtral_shape.md", ["moe_tgmm.hip", "moe_common.h"]),
 }
@@ -452,7 +454,8 @@ def run_workload(args, name, tokens=None):
       stage_ms[stage] = sum(ts) / len(ts)
   dom_ms = stage_ms.get("wi_glu")
   achieved = model["work"] / (dom_ms * 1e-3) / model["scale"] if dom_ms else None
-  traffic, traffic_source = measured_traffic(wl.name) if tokens is None else (None, None)
+  # (a token count other than the configuration's own has counters where a profile of that size is committed)
+  traffic, traffic_source = measured_traffic(wl.name if tokens is None else f"{wl.name}_t{tokens}")
   roofline = dict(bound=model["bound"], achieved=achieved, peak=model["peak"], unit=model["unit"],
                   frac=(achieved / model["peak"]) if achieved else None, traffic=traffic, traffic_source=traffic_source,
                   kernel=model["name"], kernel_ms=dom_ms)
@@ -592,6 +595,15 @@ def main():
         entry["workload"] = o["config"]["workload"]
       sweep.append(entry)
     result["c5_token_sweep"] = sweep
+    # the first configuration at decode sizes (16 and 128 tokens: 4 and 32 rows per expert): 1.4 GB of int8 weights, bound by
+    # reading them; issued call by call like the configurations above
+    result["c2_decode"] = []
+    for tokens in (16, 128):
+      torch.cuda.empty_cache()
+      o, _, olayer, _, _ = run_workload(args, "c2", tokens)
+      del olayer
+      result["c2_decode"].append({"tokens": tokens, "workload": o["config"]["workload"], "ms_per_step": o["ms_per_step"], "layer_gbps": o["layer_gbps"],
+                                  "value": o["value"], "unit": o["unit"], "roofline": o["roofline"], "stage_ms": o["stage_ms"]})
     # forward + backward of the expert layer at the first configuration's shape, bf16 and the fp8_full recipe (a few steps
     # each; `python bench.py --train [--quant fp8_full]` is the full line with its calibration and CPU baseline)
     result["training"] = []
