@@ -46,7 +46,8 @@ def oracle_layer(wl, layer):
   from oracle.layer import oracle_layer as run
 
   cfg = wl.cfg
-  trip = lambda qa: (qa.qvalue, qa.scale, qa.qtype)
+  # (the oracle names fp8 weights with one scale per output channel "fp8c"; "fp8" there is the 128 x 128 block layout)
+  trip = lambda qa: (qa.qvalue, qa.scale, "fp8c" if qa.qtype == "fp8" and qa.scale.dim() == 2 else qa.qtype)
   return run(layer["x"], layer["gate_logits"], layer["pre_bias_logits"], trip(layer["wi_0"]), trip(layer["wi_1"]), trip(layer["wo"]),
              num_experts=cfg.num_experts, k=cfg.num_experts_per_tok, emb_dim=cfg.emb_dim, mlp_dim=cfg.moe_mlp_dim,
              deepseek=cfg.is_deepseek, routed_scaling_factor=cfg.routed_scaling_factor, norm_topk_prob=cfg.norm_topk_prob,
@@ -59,7 +60,7 @@ def run_gpu(wl, layer_cpu):
 
   def dev(v):
     if isinstance(v, QArray):
-      return QArray(v.qvalue.cuda(), v.scale.cuda(), v.qtype)
+      return dataclasses.replace(v, qvalue=v.qvalue.cuda(), scale=v.scale.cuda())
     return None if v is None else v.cuda()
 
   L = {k: dev(v) for k, v in layer_cpu.items()}
@@ -75,7 +76,14 @@ def run_gpu(wl, layer_cpu):
 CASES = {
     "c1_full": lambda: _small("c1", 2048),
     "c2_small": lambda: _small("c2", 1024, emb_dim=1024, moe_mlp_dim=2048),
+    # decode sizes of the 8-bit x 8-bit layers: 4, 24 and 40 rows per expert (the LDS-streamed kernel on 16-, 32- and 64-row tiles)
+    "c2_t16": lambda: _small("c2", 16, emb_dim=1024, moe_mlp_dim=2048),
+    "c2_t96": lambda: _small("c2", 96, emb_dim=1024, moe_mlp_dim=2048),
+    "c2_t160": lambda: _small("c2", 160, emb_dim=1024, moe_mlp_dim=2048),
+    "c2f8_t16": lambda: _small("c2f8", 16, emb_dim=1024, moe_mlp_dim=2048),
+    "c2f8_t160": lambda: _small("c2f8", 160, emb_dim=1024, moe_mlp_dim=2048),
     "c3_small": lambda: _small("c3", 64, emb_dim=1024, moe_mlp_dim=512, num_experts=32),
+    "c3_t32": lambda: _small("c3", 32, emb_dim=1024, moe_mlp_dim=512, num_experts=32),  # (8 rows per expert: the block-scaled decode kernel)
     "c4_small": lambda: _small("c4", 2048, emb_dim=512, moe_mlp_dim=256),
     # the GPT-OSS shape at its full dimensions (32 experts, d = f = 2880) over the token sweep; 4096 tokens run in
     # tests/test_gpu_fullsize.py
