@@ -345,7 +345,7 @@ def test_layer_gradients_with_expert_biases():
 # ---------------------------------------------------------------- graph replay
 
 
-@pytest.mark.parametrize("case", ["c1_full", "c3_small", "c5_t16"])
+@pytest.mark.parametrize("case", ["c1_full", "c3_small", "c5_t16", "c2_t16", "c2_t160", "c2f8_t16", "c3_t32"])
 def test_graph_replay_equals_eager(case):
   """A captured layer call replayed several times, with eager work and synchronisations in between and new
   inputs each time, must reproduce the eager result bit for bit."""
