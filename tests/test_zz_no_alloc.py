@@ -41,7 +41,9 @@ def test_static_workspace_entry_point_matches_moe_gmm_on_two_calls():
   stream = _lib.current_stream()
   # first call: a prefill-sized problem (persistent 256 x 256 kernel); second: a smaller, ragged one (64-row tiles), so
   # that the second tile list is shorter than what the first call left in the array
-  for m, k, n, sizes, seed in ((2100, 512, 512, [700, 0, 800, 500], 1), (90, 256, 128, [30, 0, 45, 10], 2)):
+  # then two decode-sized ones that the LDS-streamed persistent kernel takes (16-row tiles, 64-row tiles)
+  for m, k, n, sizes, seed in ((2100, 512, 512, [700, 0, 800, 500], 1), (90, 256, 128, [30, 0, 45, 10], 2),
+                               (70, 1024, 256, [5, 0, 9, 14, 3, 11, 2, 16], 3), (210, 512, 256, [40] * 5, 4)):
     lhs, ls, rhs, rs, gs = _operands(m, k, n, sizes, seed)
     ws = torch.empty((lib.moe_gmm_workspace_bytes(m, len(sizes)),), dtype=torch.uint8, device="cuda")
     want = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
